@@ -1,0 +1,251 @@
+/*
+ * sarek_hip.h - C ABI of libsarek_hip.so, the native half of the `sarek-hip`
+ * backend plugin for Sarek/SPOC on AMD Instinct MI355X (gfx950).
+ *
+ * The OCaml side of the plugin (Hip_bindings / Hip_api / Hip_plugin) binds
+ * these symbols with ctypes-foreign, exactly as sarek-cuda binds libcuda and
+ * libnvrtc (sarek-cuda/Cuda_bindings.ml:39-81, sarek-cuda/Cuda_nvrtc.ml:99-137).
+ *
+ * Conventions (same as the CUDA driver symbols the reference binds,
+ * sarek-cuda/Cuda_types.ml:249): every function returns an `int` status,
+ * 0 = success; results come back through caller-allocated out-pointers;
+ * strings are NUL terminated; handles are opaque pointers; device pointers
+ * are plain `void*`; no callbacks into the caller.  Positive status values
+ * are hipError_t / hiprtcResult+1000 codes, negative values are
+ * SAREK_HIP_E_* below.  `sarek_hip_last_error()` returns a thread-local
+ * human-readable message for the last non-zero status.
+ *
+ * All launches are asynchronous on the given stream (NULL = the default
+ * stream); copies are synchronous, as in the reference
+ * (sarek-cuda/Cuda_api.ml:224-243).
+ */
+#ifndef SAREK_HIP_H
+#define SAREK_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define SAREK_HIP_ABI_VERSION 1
+
+/* Library-level status codes (negative; HIP codes are positive). */
+#define SAREK_HIP_OK 0
+#define SAREK_HIP_E_INVALID_ARG (-1)    /* NULL pointer, negative size, ... */
+#define SAREK_HIP_E_UNSUPPORTED (-2)    /* source language / shape not supported */
+#define SAREK_HIP_E_COMPILE (-3)        /* hiprtc compilation failed; see log */
+#define SAREK_HIP_E_NO_DEVICE (-4)      /* no gfx950-class device selected */
+#define SAREK_HIP_E_WORKSPACE (-5)      /* caller workspace too small */
+#define SAREK_HIP_E_PARSE (-6)          /* malformed IR text */
+#define SAREK_HIP_E_CODEGEN (-7)        /* IR construct the lowering rejects */
+#define SAREK_HIP_E_BUFFER_TOO_SMALL (-8)
+
+typedef void *sarek_hip_stream;  /* hipStream_t */
+typedef void *sarek_hip_event;   /* hipEvent_t */
+typedef struct sarek_hip_kernel_s *sarek_hip_kernel; /* compiled module+function */
+
+int sarek_hip_abi_version(void);
+const char *sarek_hip_last_error(void);
+const char *sarek_hip_status_name(int status);
+
+/* ---------------------------------------------------------------------- */
+/* Device  (replaces the cuInit, cuDeviceGet.. and cuCtx.. groups,
+ * sarek-cuda/Cuda_api.ml:35-179)                                            */
+
+typedef struct {
+  char name[256];
+  char gcn_arch[64];            /* e.g. "gfx950:sramecc+:xnack-" */
+  uint64_t total_global_mem;    /* bytes */
+  int max_threads_per_block;
+  int max_block_dim[3];
+  int max_grid_dim[3];
+  int shared_mem_per_block;     /* LDS bytes usable by one workgroup */
+  int warp_size;                /* 64 on CDNA */
+  int multiprocessor_count;     /* compute units */
+  int clock_rate_khz;
+  int memory_clock_rate_khz;
+  int memory_bus_width_bits;
+  int l2_cache_size;
+  int compute_major, compute_minor;
+} sarek_hip_device_info;
+
+int sarek_hip_init(void);                       /* hipInit(0); idempotent */
+int sarek_hip_is_available(void);               /* 1/0, never fails (Framework_registry.ml:77-87) */
+int sarek_hip_device_count(int *count);
+int sarek_hip_device_get_info(int device, sarek_hip_device_info *out);
+int sarek_hip_device_set_current(int device);
+int sarek_hip_device_get_current(int *device);
+int sarek_hip_device_synchronize(void);         /* Transfer.flush -> Device.synchronize */
+int sarek_hip_mem_get_info(size_t *free_bytes, size_t *total_bytes);
+int sarek_hip_driver_version(int *version);
+
+/* ---------------------------------------------------------------------- */
+/* Memory  (replaces cuMemAlloc/Free/Memcpy.., sarek-cuda/Cuda_api.ml:183-244).
+ * `sarek_hip_mem_free(NULL)` and a double free of the same pointer are
+ * accepted: the reference frees buffers both explicitly and from a GC
+ * finaliser that may run late (sarek/core/Gpu_memory.ml:163-178).          */
+int sarek_hip_mem_alloc(void **dptr, size_t bytes);
+int sarek_hip_mem_free(void *dptr);
+int sarek_hip_memcpy_htod(void *dst_device, const void *src_host, size_t bytes);
+int sarek_hip_memcpy_dtoh(void *dst_host, const void *src_device, size_t bytes);
+int sarek_hip_memcpy_dtod(void *dst_device, const void *src_device, size_t bytes);
+int sarek_hip_memset_d8(void *dst_device, unsigned char value, size_t bytes);
+
+/* ---------------------------------------------------------------------- */
+/* Stream / Event  (sarek-cuda/Cuda_api.ml:248-293).  Default priority only. */
+int sarek_hip_stream_create(sarek_hip_stream *out);
+int sarek_hip_stream_destroy(sarek_hip_stream s);
+int sarek_hip_stream_synchronize(sarek_hip_stream s);
+int sarek_hip_event_create(sarek_hip_event *out);
+int sarek_hip_event_destroy(sarek_hip_event e);
+int sarek_hip_event_record(sarek_hip_event e, sarek_hip_stream s);
+int sarek_hip_event_synchronize(sarek_hip_event e);
+int sarek_hip_event_elapsed_ms(sarek_hip_event start, sarek_hip_event stop, float *ms);
+
+/* ---------------------------------------------------------------------- */
+/* Kernel JIT + launch  (replaces the nvrtc.., cuModule.. groups and cuLaunchKernel,
+ * sarek-cuda/Cuda_nvrtc.ml:263-389, sarek-cuda/Cuda_api.ml:315-486).
+ * `source` is HIP C++ text; it is compiled by hiprtc for the current
+ * device's architecture (--offload-arch=<gcnArchName>).  On failure the
+ * compiler log is copied into `log` (truncated to log_len-1 bytes).        */
+int sarek_hip_kernel_compile(const char *source, const char *kernel_name,
+                             sarek_hip_kernel *out, char *log, size_t log_len);
+/* Same, memoised on (device, hash(source), kernel_name)
+ * (Kernel.compile_cached, sarek-cuda/Cuda_api.ml:399-412).                 */
+int sarek_hip_kernel_compile_cached(const char *source, const char *kernel_name,
+                                    sarek_hip_kernel *out, char *log, size_t log_len);
+int sarek_hip_kernel_clear_cache(void);
+int sarek_hip_kernel_destroy(sarek_hip_kernel k);
+/* params: array of n_params pointers to the argument values, the
+ * cuLaunchKernel convention (sarek-cuda/Cuda_api.ml:473-486).              */
+int sarek_hip_kernel_launch(sarek_hip_kernel k, const unsigned grid[3], const unsigned block[3],
+                            unsigned shared_mem_bytes, sarek_hip_stream stream, void **params,
+                            int n_params);
+
+/* ---------------------------------------------------------------------- */
+/* Plugin level: what Hip_plugin.generate_source / Hip_plugin.run_source call
+ * (sarek-cuda/Cuda_plugin.ml:155-157,174-220).                             */
+
+/* Source language tags, numbered like Framework_sig.source_lang
+ * (spoc/framework/Framework_sig.ml:72-77) with HIP_Source appended.        */
+enum {
+  SAREK_HIP_LANG_CUDA_SOURCE = 0,
+  SAREK_HIP_LANG_OPENCL_SOURCE = 1,
+  SAREK_HIP_LANG_PTX = 2,
+  SAREK_HIP_LANG_SPIR_V = 3,
+  SAREK_HIP_LANG_GLSL_SOURCE = 4,
+  SAREK_HIP_LANG_HIP_SOURCE = 5
+};
+
+/* One element of Framework_sig.run_source_arg list
+ * (spoc/framework/Framework_sig.ml:88-96).                                 */
+enum {
+  SAREK_HIP_ARG_BUFFER = 0,
+  SAREK_HIP_ARG_INT32 = 1,
+  SAREK_HIP_ARG_INT64 = 2,
+  SAREK_HIP_ARG_FLOAT32 = 3,
+  SAREK_HIP_ARG_FLOAT64 = 4
+};
+typedef struct {
+  int kind;
+  void *buffer;     /* SAREK_HIP_ARG_BUFFER: device pointer */
+  int64_t length;   /* SAREK_HIP_ARG_BUFFER: vector length in elements */
+  int32_t i32;
+  int64_t i64;
+  float f32;
+  double f64;
+} sarek_hip_arg;
+
+/* IR text (the s-expression form written by the plugin's IR serialiser) ->
+ * HIP source for gfx950.  When the IR is one of the recognised hot kernels
+ * (tiled matmul, stream triad, block-256 tree sum / dot product) and
+ * specialisation is enabled, the source carries a leading
+ * `// sarek-hip-specialise: <tag>` line that run_source honours; the plain
+ * lowering always follows, so the text is valid HIP either way.
+ * block: launch block dims or NULL.  Writes at most out_len bytes incl. NUL;
+ * *needed gets the full size.                                              */
+int sarek_hip_generate_source(const char *ir_text, const int block[3], char *out, size_t out_len,
+                              size_t *needed);
+
+/* Compile (cached) + bind + launch on the default stream.  Only
+ * SAREK_HIP_LANG_HIP_SOURCE and SAREK_HIP_LANG_CUDA_SOURCE (treated as HIP
+ * text) are accepted; others return SAREK_HIP_E_UNSUPPORTED.  A specialise
+ * tag in the source reroutes the call to the matching hand-written kernel
+ * below, ignoring block/grid.                                              */
+int sarek_hip_run_source(const char *source, int lang, const char *kernel_name,
+                         const int block[3], const int grid[3], int shared_mem_bytes,
+                         const sarek_hip_arg *args, int n_args);
+
+/* 1 (default) / 0: honour specialise tags.  Also read once from the
+ * environment variable SAREK_HIP_SPECIALISE (0 disables).                  */
+int sarek_hip_set_specialisation(int enabled);
+/* Name of the code path the last sarek_hip_run_source call took on this
+ * thread: "jit" or the specialise tag.                                     */
+const char *sarek_hip_last_run_path(void);
+
+/* ---------------------------------------------------------------------- */
+/* Hand-written CDNA4 kernels.  All pointers are device pointers.  These have
+ * no counterpart symbol in the reference: they replace the JIT-compiled
+ * generated kernels named in each comment.                                 */
+
+/* Stream triad  a[i] = b[i] + c[i]*s, i < n   (generated kernel
+ * benchmarks/descriptions/generated/stream_triad_generated.md:9-17; source
+ * benchmarks/bench_stream_triad.ml:22-32).                                 */
+int sarek_hip_triad_f32(float *a, const float *b, const float *c, float s, int64_t n,
+                        sarek_hip_stream stream);
+
+/* Fused triad + sum: writes a as above and *sum_out = sum_i a[i] (double,
+ * device memory).  `partials` is caller workspace of at least
+ * sarek_hip_triad_sum_workspace_floats(n) floats.                          */
+int64_t sarek_hip_triad_sum_workspace_floats(int64_t n);
+int sarek_hip_triad_sum_f32(float *a, const float *b, const float *c, float s, int64_t n,
+                            float *partials, int64_t partials_len, double *sum_out,
+                            sarek_hip_stream stream);
+
+/* Block-256 tree reductions: out[j] = sum of in[256j .. 256j+255] (zero
+ * padded), j < ceil(n/256)  (benchmarks/bench_reduction.ml:62-96;
+ * generated kernel reduction_generated.md:9-75).  dot: sum of a[i]*b[i]
+ * (benchmarks/bench_dot_product.ml:16-54).                                 */
+int sarek_hip_reduce_sum_block256_f32(const float *in, float *out, int64_t n,
+                                      sarek_hip_stream stream);
+int sarek_hip_dot_block256_f32(const float *a, const float *b, float *out, int64_t n,
+                               sarek_hip_stream stream);
+/* *sum_out = left-to-right double fold of partials[0..count)
+ * (host fold of benchmarks/bench_reduction.ml:154-160, kept on device).    */
+int sarek_hip_fold_partials_f64(const float *partials, int64_t count, double *sum_out,
+                                sarek_hip_stream stream);
+
+/* Row-major GEMM  C[m x n] = A[m x k] . B[k x n]  (replaces the generated
+ * 16x16 tiled kernel, matrix_mul_tiled_generated.md:9-50; source
+ * benchmarks/bench_matrix_mul_tiled.ml:55-95).  Any m,n,k >= 1.            */
+int sarek_hip_gemm_f32(const float *a, const float *b, float *c, int m, int n, int k,
+                       sarek_hip_stream stream);
+
+/* 16-bit-input, f32-accumulate GEMMs.  a, b hold bf16 / IEEE fp16 bit
+ * patterns, row-major [m x k] and [k x n]; c is f32 row-major.             */
+int sarek_hip_gemm_bf16(const uint16_t *a, const uint16_t *b, float *c, int m, int n, int k,
+                        sarek_hip_stream stream);
+int sarek_hip_gemm_f16(const uint16_t *a, const uint16_t *b, float *c, int m, int n, int k,
+                       sarek_hip_stream stream);
+
+/* Fused epilogue chain: y = relu(A.B + bias[col]) (f32, [m x n]) and
+ * rowsum[r] = sum_c y[r,c] (f32, [m]).  fp16 inputs.                        */
+int sarek_hip_gemm_f16_bias_relu_rowsum(const uint16_t *a, const uint16_t *b, const float *bias,
+                                        float *y, float *rowsum, int m, int n, int k,
+                                        sarek_hip_stream stream);
+
+/* Round-to-nearest-even narrowing of an f32 vector to bf16 / fp16 bit
+ * patterns (the input cast of the 16-bit GEMM path).                       */
+int sarek_hip_cast_f32_to_bf16(const float *in, uint16_t *out, int64_t n, sarek_hip_stream stream);
+int sarek_hip_cast_f32_to_f16(const float *in, uint16_t *out, int64_t n, sarek_hip_stream stream);
+
+/* Integer tuning knob (launch shapes, tile variants), for sweeps without a
+ * rebuild.  Unknown names are stored and ignored.                           */
+int sarek_hip_set_tunable(const char *name, int64_t value);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* SAREK_HIP_H */

@@ -1,0 +1,207 @@
+// Plugin-level entry points: what Hip_plugin.run_source does for an external or
+// generated kernel (compile cached, bind the run_source_arg list, launch on the
+// default stream; sarek-cuda/Cuda_plugin.ml:174-220), plus the hand-kernel dispatch:
+// a source that starts with "// sarek-hip-specialise: <tag>" is served by the matching
+// hand-written kernel when the caller's launch geometry covers the whole problem the
+// way the generated kernel assumes; otherwise the text is JIT-compiled as it stands.
+#include <cstdlib>
+#include <cstring>
+#include <string>
+#include <vector>
+
+#include "common.hpp"
+#include "plugin.hpp"
+
+namespace sarek_hip {
+
+const char *const kSpecialiseMarker = "// sarek-hip-specialise: ";
+
+namespace {
+
+int g_specialise = -1;  // -1: read the environment on first use
+thread_local std::string t_last_path = "none";
+
+bool specialisation_enabled() {
+  if (g_specialise < 0) {
+    const char *e = std::getenv("SAREK_HIP_SPECIALISE");
+    g_specialise = (e && e[0] == '0') ? 0 : 1;
+  }
+  return g_specialise == 1;
+}
+
+std::string read_tag(const char *source) {
+  const size_t ml = std::strlen(kSpecialiseMarker);
+  // skip leading whitespace / blank lines
+  while (*source == ' ' || *source == '\n' || *source == '\r' || *source == '\t') ++source;
+  if (std::strncmp(source, kSpecialiseMarker, ml) != 0) return "";
+  const char *p = source + ml;
+  const char *e = p;
+  while (*e && *e != '\n' && *e != '\r' && *e != ' ') ++e;
+  return std::string(p, e);
+}
+
+bool is_buf(const sarek_hip_arg &a) { return a.kind == SAREK_HIP_ARG_BUFFER; }
+bool is_i32(const sarek_hip_arg &a) { return a.kind == SAREK_HIP_ARG_INT32; }
+bool is_f32(const sarek_hip_arg &a) { return a.kind == SAREK_HIP_ARG_FLOAT32; }
+
+// Argument shape of a generated kernel: each vector parameter is a buffer followed by
+// its int32 length (Execute.expand_to_run_source_args, sarek/sarek/Execute.ml:197-216).
+bool vec_at(const sarek_hip_arg *args, int n_args, int i) {
+  return i + 1 < n_args && is_buf(args[i]) && is_i32(args[i + 1]) && args[i].buffer != nullptr;
+}
+
+int64_t cdiv(int64_t a, int64_t b) { return (a + b - 1) / b; }
+
+// Returns 1 when the call was served by a hand kernel (status in *rc), 0 to fall back.
+int try_specialised(const std::string &tag, const int block[3], const int grid[3],
+                    const sarek_hip_arg *args, int n_args, int *rc) {
+  if (tag == "matmul_tiled_f32") {
+    // (a, len, b, len, c, len, m, n, k); block 16x16, grid covering the whole C.
+    if (n_args != 9 || !vec_at(args, n_args, 0) || !vec_at(args, n_args, 2) ||
+        !vec_at(args, n_args, 4) || !is_i32(args[6]) || !is_i32(args[7]) || !is_i32(args[8]))
+      return 0;
+    const int64_t m = args[6].i32, n = args[7].i32, k = args[8].i32;
+    if (m <= 0 || n <= 0 || k <= 0) return 0;
+    if (block[0] != 16 || block[1] != 16 || block[2] != 1) return 0;
+    if (grid[0] < cdiv(n, 16) || grid[1] < cdiv(m, 16) || grid[2] != 1) return 0;
+    if (args[0].length < m * k || args[2].length < k * n || args[4].length < m * n) return 0;
+    *rc = sarek_hip_gemm_f32(static_cast<const float *>(args[0].buffer),
+                             static_cast<const float *>(args[2].buffer),
+                             static_cast<float *>(args[4].buffer), (int)m, (int)n, (int)k, nullptr);
+    return 1;
+  }
+  if (tag == "stream_triad_f32") {
+    // (a, len, b, len, c, len, scalar, n); 1-D launch with at least n threads.
+    if (n_args != 8 || !vec_at(args, n_args, 0) || !vec_at(args, n_args, 2) ||
+        !vec_at(args, n_args, 4) || !is_f32(args[6]) || !is_i32(args[7]))
+      return 0;
+    const int64_t n = args[7].i32;
+    if (n < 0) return 0;
+    if (block[1] != 1 || block[2] != 1 || grid[1] != 1 || grid[2] != 1) return 0;
+    if (static_cast<int64_t>(block[0]) * grid[0] < n) return 0;
+    if (args[0].length < n || args[2].length < n || args[4].length < n) return 0;
+    *rc = sarek_hip_triad_f32(static_cast<float *>(args[0].buffer),
+                              static_cast<const float *>(args[2].buffer),
+                              static_cast<const float *>(args[4].buffer), args[6].f32, n, nullptr);
+    return 1;
+  }
+  if (tag == "reduce_sum_block256_f32" || tag == "dot_block256_f32") {
+    const bool dot = tag[0] == 'd';
+    const int nv = dot ? 3 : 2;
+    if (n_args != 2 * nv + 1) return 0;
+    for (int v = 0; v < nv; ++v)
+      if (!vec_at(args, n_args, 2 * v)) return 0;
+    if (!is_i32(args[2 * nv])) return 0;
+    const int64_t n = args[2 * nv].i32;
+    if (n < 0) return 0;
+    // the generated kernel's tree is written for exactly 256 threads per block
+    if (block[0] != 256 || block[1] != 1 || block[2] != 1 || grid[1] != 1 || grid[2] != 1) return 0;
+    const int64_t nblocks = cdiv(n, 256);
+    // blocks past ceil(n/256) would store zeros; only take over when the grid is exact
+    if (grid[0] != nblocks) return 0;
+    if (args[2 * (nv - 1)].length < nblocks) return 0;
+    for (int v = 0; v < nv - 1; ++v) {
+      if (args[2 * v].length < n) return 0;
+      if (reinterpret_cast<uintptr_t>(args[2 * v].buffer) % 16 != 0) return 0;
+    }
+    if (dot)
+      *rc = sarek_hip_dot_block256_f32(static_cast<const float *>(args[0].buffer),
+                                       static_cast<const float *>(args[2].buffer),
+                                       static_cast<float *>(args[4].buffer), n, nullptr);
+    else
+      *rc = sarek_hip_reduce_sum_block256_f32(static_cast<const float *>(args[0].buffer),
+                                              static_cast<float *>(args[2].buffer), n, nullptr);
+    return 1;
+  }
+  return 0;
+}
+
+}  // namespace
+}  // namespace sarek_hip
+
+using namespace sarek_hip;
+
+extern "C" {
+
+int sarek_hip_set_specialisation(int enabled) {
+  g_specialise = enabled ? 1 : 0;
+  return SAREK_HIP_OK;
+}
+
+const char *sarek_hip_last_run_path(void) { return t_last_path.c_str(); }
+
+int sarek_hip_run_source(const char *source, int lang, const char *kernel_name, const int block[3],
+                         const int grid[3], int shared_mem_bytes, const sarek_hip_arg *args,
+                         int n_args) {
+  t_last_path = "none";
+  if (!source || !kernel_name || !block || !grid || n_args < 0 || (n_args > 0 && !args))
+    return fail(SAREK_HIP_E_INVALID_ARG, "run_source: NULL or negative argument");
+  switch (lang) {
+    case SAREK_HIP_LANG_HIP_SOURCE:
+    case SAREK_HIP_LANG_CUDA_SOURCE:
+      break;
+    case SAREK_HIP_LANG_OPENCL_SOURCE:
+      return fail(SAREK_HIP_E_UNSUPPORTED, "HIP backend does not support OpenCL_Source");
+    case SAREK_HIP_LANG_PTX:
+      return fail(SAREK_HIP_E_UNSUPPORTED, "HIP backend does not support PTX");
+    case SAREK_HIP_LANG_SPIR_V:
+      return fail(SAREK_HIP_E_UNSUPPORTED, "HIP backend does not support SPIR_V");
+    case SAREK_HIP_LANG_GLSL_SOURCE:
+      return fail(SAREK_HIP_E_UNSUPPORTED, "HIP backend does not support GLSL_Source");
+    default:
+      return fail(SAREK_HIP_E_INVALID_ARG, "run_source: unknown source language %d", lang);
+  }
+  for (int i = 0; i < 3; ++i)
+    if (block[i] <= 0 || grid[i] <= 0)
+      return fail(SAREK_HIP_E_INVALID_ARG, "run_source: block and grid dimensions must be positive");
+  if (shared_mem_bytes < 0)
+    return fail(SAREK_HIP_E_INVALID_ARG, "run_source: negative shared memory size");
+
+  if (specialisation_enabled()) {
+    std::string tag = read_tag(source);
+    if (!tag.empty()) {
+      int rc = SAREK_HIP_OK;
+      if (try_specialised(tag, block, grid, args, n_args, &rc)) {
+        t_last_path = tag;
+        return rc;
+      }
+    }
+  }
+
+  sarek_hip_kernel k = nullptr;
+  std::vector<char> log(16384);
+  int rc = sarek_hip_kernel_compile_cached(source, kernel_name, &k, log.data(), log.size());
+  if (rc != SAREK_HIP_OK) return rc;
+
+  // Parameter block: one slot per argument, kept alive until the launch call returns.
+  struct Slot {
+    union {
+      void *p;
+      int32_t i32;
+      int64_t i64;
+      float f32;
+      double f64;
+    };
+  };
+  std::vector<Slot> slots(n_args);
+  std::vector<void *> params(n_args);
+  for (int i = 0; i < n_args; ++i) {
+    switch (args[i].kind) {
+      case SAREK_HIP_ARG_BUFFER: slots[i].p = args[i].buffer; break;
+      case SAREK_HIP_ARG_INT32: slots[i].i32 = args[i].i32; break;
+      case SAREK_HIP_ARG_INT64: slots[i].i64 = args[i].i64; break;
+      case SAREK_HIP_ARG_FLOAT32: slots[i].f32 = args[i].f32; break;
+      case SAREK_HIP_ARG_FLOAT64: slots[i].f64 = args[i].f64; break;
+      default:
+        return fail(SAREK_HIP_E_INVALID_ARG, "run_source: argument %d has unknown kind %d", i,
+                    args[i].kind);
+    }
+    params[i] = &slots[i];
+  }
+  const unsigned g[3] = {(unsigned)grid[0], (unsigned)grid[1], (unsigned)grid[2]};
+  const unsigned b[3] = {(unsigned)block[0], (unsigned)block[1], (unsigned)block[2]};
+  rc = sarek_hip_kernel_launch(k, g, b, (unsigned)shared_mem_bytes, nullptr, params.data(), n_args);
+  if (rc == SAREK_HIP_OK) t_last_path = "jit";
+  return rc;
+}
+}

@@ -1,0 +1,365 @@
+// Device / Memory / Stream / Event / Kernel layer of libsarek_hip: the HIP and hiprtc
+// calls the plugin's Hip_api module needs, behind the library's status convention.
+// Mirrors the responsibilities of sarek-cuda/Cuda_api.ml:35-512 and
+// sarek-cuda/Cuda_nvrtc.ml:263-389 (compile with log capture, cached kernels,
+// parameter-pointer launch).
+#include <hip/hiprtc.h>
+
+#include <cstring>
+#include <map>
+#include <mutex>
+#include <set>
+#include <string>
+#include <vector>
+
+#include "common.hpp"
+
+struct sarek_hip_kernel_s {
+  hipModule_t module = nullptr;
+  hipFunction_t function = nullptr;
+  std::string name;
+  int device = -1;
+  bool cached = false;
+};
+
+namespace sarek_hip {
+namespace {
+
+std::mutex g_mu;
+bool g_inited = false;
+std::set<void *> g_live_allocs;  // device pointers handed out and not yet freed
+std::map<std::string, sarek_hip_kernel> g_kernel_cache;
+
+int rtc_fail(hiprtcResult r, const char *what) {
+  return fail(1000 + static_cast<int>(r), "%s: %s", what, hiprtcGetErrorString(r));
+}
+
+// FNV-1a 64-bit of the source text, for the kernel cache key.
+uint64_t fnv1a(const char *s) {
+  uint64_t h = 1469598103934665603ull;
+  for (; *s; ++s) {
+    h ^= static_cast<unsigned char>(*s);
+    h *= 1099511628211ull;
+  }
+  return h;
+}
+
+void copy_log(const std::string &text, char *log, size_t log_len) {
+  if (!log || log_len == 0) return;
+  size_t n = text.size() < log_len - 1 ? text.size() : log_len - 1;
+  std::memcpy(log, text.data(), n);
+  log[n] = '\0';
+}
+
+int compile_impl(const char *source, const char *kernel_name, sarek_hip_kernel *out, char *log,
+                 size_t log_len) {
+  if (!source || !kernel_name || !out)
+    return fail(SAREK_HIP_E_INVALID_ARG, "kernel_compile: NULL argument");
+  if (log && log_len) log[0] = '\0';
+  int dev = 0;
+  SAREK_HIP_TRY(hipGetDevice(&dev));
+  hipDeviceProp_t prop;
+  SAREK_HIP_TRY(hipGetDeviceProperties(&prop, dev));
+  std::string arch = std::string("--offload-arch=") + prop.gcnArchName;
+
+  hiprtcProgram prog;
+  hiprtcResult r = hiprtcCreateProgram(&prog, source, "sarek_kernel.hip", 0, nullptr, nullptr);
+  if (r != HIPRTC_SUCCESS) return rtc_fail(r, "hiprtcCreateProgram");
+  const char *opts[] = {arch.c_str(), "-O3", "-std=c++17"};
+  r = hiprtcCompileProgram(prog, 3, opts);
+  std::string build_log;
+  size_t log_size = 0;
+  if (hiprtcGetProgramLogSize(prog, &log_size) == HIPRTC_SUCCESS && log_size > 1) {
+    build_log.resize(log_size);
+    hiprtcGetProgramLog(prog, &build_log[0]);
+  }
+  copy_log(build_log, log, log_len);
+  if (r != HIPRTC_SUCCESS) {
+    hiprtcDestroyProgram(&prog);
+    return fail(SAREK_HIP_E_COMPILE, "hiprtc compilation of kernel '%s' failed: %s\n%s", kernel_name,
+                hiprtcGetErrorString(r), build_log.c_str());
+  }
+  size_t code_size = 0;
+  r = hiprtcGetCodeSize(prog, &code_size);
+  if (r != HIPRTC_SUCCESS) {
+    hiprtcDestroyProgram(&prog);
+    return rtc_fail(r, "hiprtcGetCodeSize");
+  }
+  std::vector<char> code(code_size);
+  r = hiprtcGetCode(prog, code.data());
+  hiprtcDestroyProgram(&prog);
+  if (r != HIPRTC_SUCCESS) return rtc_fail(r, "hiprtcGetCode");
+
+  auto *k = new sarek_hip_kernel_s();
+  k->name = kernel_name;
+  k->device = dev;
+  hipError_t e = hipModuleLoadData(&k->module, code.data());
+  if (e != hipSuccess) {
+    delete k;
+    return check_hip(e, "hipModuleLoadData");
+  }
+  e = hipModuleGetFunction(&k->function, k->module, kernel_name);
+  if (e != hipSuccess) {
+    (void)hipModuleUnload(k->module);
+    delete k;
+    return check_hip(e, "hipModuleGetFunction");
+  }
+  *out = k;
+  return SAREK_HIP_OK;
+}
+
+}  // namespace
+}  // namespace sarek_hip
+
+using namespace sarek_hip;
+
+extern "C" {
+
+int sarek_hip_init(void) {
+  std::lock_guard<std::mutex> lock(g_mu);
+  if (g_inited) return SAREK_HIP_OK;
+  SAREK_HIP_TRY(hipInit(0));
+  g_inited = true;
+  return SAREK_HIP_OK;
+}
+
+int sarek_hip_is_available(void) {
+  int n = 0;
+  if (hipInit(0) != hipSuccess) return 0;
+  if (hipGetDeviceCount(&n) != hipSuccess) {
+    (void)hipGetLastError();
+    return 0;
+  }
+  return n > 0 ? 1 : 0;
+}
+
+int sarek_hip_device_count(int *count) {
+  if (!count) return fail(SAREK_HIP_E_INVALID_ARG, "device_count: NULL out pointer");
+  SAREK_HIP_TRY(hipGetDeviceCount(count));
+  return SAREK_HIP_OK;
+}
+
+int sarek_hip_device_get_info(int device, sarek_hip_device_info *out) {
+  if (!out) return fail(SAREK_HIP_E_INVALID_ARG, "device_get_info: NULL out pointer");
+  hipDeviceProp_t p;
+  SAREK_HIP_TRY(hipGetDeviceProperties(&p, device));
+  std::memset(out, 0, sizeof(*out));
+  std::strncpy(out->name, p.name, sizeof(out->name) - 1);
+  std::strncpy(out->gcn_arch, p.gcnArchName, sizeof(out->gcn_arch) - 1);
+  out->total_global_mem = p.totalGlobalMem;
+  out->max_threads_per_block = p.maxThreadsPerBlock;
+  for (int i = 0; i < 3; ++i) {
+    out->max_block_dim[i] = p.maxThreadsDim[i];
+    out->max_grid_dim[i] = p.maxGridSize[i];
+  }
+  out->shared_mem_per_block = static_cast<int>(p.sharedMemPerBlock);
+  out->warp_size = p.warpSize;
+  out->multiprocessor_count = p.multiProcessorCount;
+  out->clock_rate_khz = p.clockRate;
+  out->memory_clock_rate_khz = p.memoryClockRate;
+  out->memory_bus_width_bits = p.memoryBusWidth;
+  out->l2_cache_size = p.l2CacheSize;
+  out->compute_major = p.major;
+  out->compute_minor = p.minor;
+  return SAREK_HIP_OK;
+}
+
+int sarek_hip_device_set_current(int device) {
+  SAREK_HIP_TRY(hipSetDevice(device));
+  return SAREK_HIP_OK;
+}
+
+int sarek_hip_device_get_current(int *device) {
+  if (!device) return fail(SAREK_HIP_E_INVALID_ARG, "device_get_current: NULL out pointer");
+  SAREK_HIP_TRY(hipGetDevice(device));
+  return SAREK_HIP_OK;
+}
+
+int sarek_hip_device_synchronize(void) {
+  SAREK_HIP_TRY(hipDeviceSynchronize());
+  return SAREK_HIP_OK;
+}
+
+int sarek_hip_mem_get_info(size_t *free_bytes, size_t *total_bytes) {
+  if (!free_bytes || !total_bytes) return fail(SAREK_HIP_E_INVALID_ARG, "mem_get_info: NULL out pointer");
+  SAREK_HIP_TRY(hipMemGetInfo(free_bytes, total_bytes));
+  return SAREK_HIP_OK;
+}
+
+int sarek_hip_driver_version(int *version) {
+  if (!version) return fail(SAREK_HIP_E_INVALID_ARG, "driver_version: NULL out pointer");
+  SAREK_HIP_TRY(hipDriverGetVersion(version));
+  return SAREK_HIP_OK;
+}
+
+int sarek_hip_mem_alloc(void **dptr, size_t bytes) {
+  if (!dptr) return fail(SAREK_HIP_E_INVALID_ARG, "mem_alloc: NULL out pointer");
+  *dptr = nullptr;
+  // A zero-length vector still needs a distinct, freeable handle.
+  SAREK_HIP_TRY(hipMalloc(dptr, bytes ? bytes : 1));
+  std::lock_guard<std::mutex> lock(g_mu);
+  g_live_allocs.insert(*dptr);
+  return SAREK_HIP_OK;
+}
+
+int sarek_hip_mem_free(void *dptr) {
+  if (!dptr) return SAREK_HIP_OK;
+  {
+    std::lock_guard<std::mutex> lock(g_mu);
+    auto it = g_live_allocs.find(dptr);
+    if (it == g_live_allocs.end()) return SAREK_HIP_OK;  // already freed (or not ours): no-op
+    g_live_allocs.erase(it);
+  }
+  SAREK_HIP_TRY(hipFree(dptr));
+  return SAREK_HIP_OK;
+}
+
+int sarek_hip_memcpy_htod(void *dst_device, const void *src_host, size_t bytes) {
+  if (bytes == 0) return SAREK_HIP_OK;
+  if (!dst_device || !src_host) return fail(SAREK_HIP_E_INVALID_ARG, "memcpy_htod: NULL pointer");
+  SAREK_HIP_TRY(hipMemcpy(dst_device, src_host, bytes, hipMemcpyHostToDevice));
+  return SAREK_HIP_OK;
+}
+
+int sarek_hip_memcpy_dtoh(void *dst_host, const void *src_device, size_t bytes) {
+  if (bytes == 0) return SAREK_HIP_OK;
+  if (!dst_host || !src_device) return fail(SAREK_HIP_E_INVALID_ARG, "memcpy_dtoh: NULL pointer");
+  SAREK_HIP_TRY(hipMemcpy(dst_host, src_device, bytes, hipMemcpyDeviceToHost));
+  return SAREK_HIP_OK;
+}
+
+int sarek_hip_memcpy_dtod(void *dst_device, const void *src_device, size_t bytes) {
+  if (bytes == 0) return SAREK_HIP_OK;
+  if (!dst_device || !src_device) return fail(SAREK_HIP_E_INVALID_ARG, "memcpy_dtod: NULL pointer");
+  SAREK_HIP_TRY(hipMemcpy(dst_device, src_device, bytes, hipMemcpyDeviceToDevice));
+  return SAREK_HIP_OK;
+}
+
+int sarek_hip_memset_d8(void *dst_device, unsigned char value, size_t bytes) {
+  if (bytes == 0) return SAREK_HIP_OK;
+  if (!dst_device) return fail(SAREK_HIP_E_INVALID_ARG, "memset_d8: NULL pointer");
+  SAREK_HIP_TRY(hipMemset(dst_device, value, bytes));
+  return SAREK_HIP_OK;
+}
+
+int sarek_hip_stream_create(sarek_hip_stream *out) {
+  if (!out) return fail(SAREK_HIP_E_INVALID_ARG, "stream_create: NULL out pointer");
+  hipStream_t s;
+  SAREK_HIP_TRY(hipStreamCreateWithFlags(&s, hipStreamNonBlocking));
+  *out = s;
+  return SAREK_HIP_OK;
+}
+
+int sarek_hip_stream_destroy(sarek_hip_stream s) {
+  if (!s) return SAREK_HIP_OK;
+  SAREK_HIP_TRY(hipStreamDestroy(as_stream(s)));
+  return SAREK_HIP_OK;
+}
+
+int sarek_hip_stream_synchronize(sarek_hip_stream s) {
+  SAREK_HIP_TRY(hipStreamSynchronize(as_stream(s)));
+  return SAREK_HIP_OK;
+}
+
+int sarek_hip_event_create(sarek_hip_event *out) {
+  if (!out) return fail(SAREK_HIP_E_INVALID_ARG, "event_create: NULL out pointer");
+  hipEvent_t e;
+  SAREK_HIP_TRY(hipEventCreate(&e));
+  *out = e;
+  return SAREK_HIP_OK;
+}
+
+int sarek_hip_event_destroy(sarek_hip_event e) {
+  if (!e) return SAREK_HIP_OK;
+  SAREK_HIP_TRY(hipEventDestroy(reinterpret_cast<hipEvent_t>(e)));
+  return SAREK_HIP_OK;
+}
+
+int sarek_hip_event_record(sarek_hip_event e, sarek_hip_stream s) {
+  if (!e) return fail(SAREK_HIP_E_INVALID_ARG, "event_record: NULL event");
+  SAREK_HIP_TRY(hipEventRecord(reinterpret_cast<hipEvent_t>(e), as_stream(s)));
+  return SAREK_HIP_OK;
+}
+
+int sarek_hip_event_synchronize(sarek_hip_event e) {
+  if (!e) return fail(SAREK_HIP_E_INVALID_ARG, "event_synchronize: NULL event");
+  SAREK_HIP_TRY(hipEventSynchronize(reinterpret_cast<hipEvent_t>(e)));
+  return SAREK_HIP_OK;
+}
+
+int sarek_hip_event_elapsed_ms(sarek_hip_event start, sarek_hip_event stop, float *ms) {
+  if (!start || !stop || !ms) return fail(SAREK_HIP_E_INVALID_ARG, "event_elapsed_ms: NULL argument");
+  SAREK_HIP_TRY(hipEventElapsedTime(ms, reinterpret_cast<hipEvent_t>(start),
+                                    reinterpret_cast<hipEvent_t>(stop)));
+  return SAREK_HIP_OK;
+}
+
+int sarek_hip_kernel_compile(const char *source, const char *kernel_name, sarek_hip_kernel *out,
+                             char *log, size_t log_len) {
+  return compile_impl(source, kernel_name, out, log, log_len);
+}
+
+int sarek_hip_kernel_compile_cached(const char *source, const char *kernel_name,
+                                    sarek_hip_kernel *out, char *log, size_t log_len) {
+  if (!source || !kernel_name || !out)
+    return fail(SAREK_HIP_E_INVALID_ARG, "kernel_compile_cached: NULL argument");
+  int dev = 0;
+  SAREK_HIP_TRY(hipGetDevice(&dev));
+  char key_buf[64];
+  std::snprintf(key_buf, sizeof(key_buf), "%d:%016llx:%zu:", dev,
+                static_cast<unsigned long long>(fnv1a(source)), std::strlen(source));
+  std::string key = std::string(key_buf) + kernel_name;
+  {
+    std::lock_guard<std::mutex> lock(g_mu);
+    auto it = g_kernel_cache.find(key);
+    if (it != g_kernel_cache.end()) {
+      *out = it->second;
+      if (log && log_len) log[0] = '\0';
+      return SAREK_HIP_OK;
+    }
+  }
+  sarek_hip_kernel k = nullptr;
+  int rc = compile_impl(source, kernel_name, &k, log, log_len);
+  if (rc != SAREK_HIP_OK) return rc;
+  k->cached = true;
+  std::lock_guard<std::mutex> lock(g_mu);
+  auto ins = g_kernel_cache.emplace(key, k);
+  if (!ins.second) {  // another thread compiled the same source meanwhile
+    (void)hipModuleUnload(k->module);
+    delete k;
+  }
+  *out = ins.first->second;
+  return SAREK_HIP_OK;
+}
+
+int sarek_hip_kernel_clear_cache(void) {
+  std::lock_guard<std::mutex> lock(g_mu);
+  for (auto &kv : g_kernel_cache) {
+    (void)hipModuleUnload(kv.second->module);
+    delete kv.second;
+  }
+  g_kernel_cache.clear();
+  return SAREK_HIP_OK;
+}
+
+int sarek_hip_kernel_destroy(sarek_hip_kernel k) {
+  if (!k || k->cached) return SAREK_HIP_OK;  // cached kernels live until clear_cache
+  hipError_t e = hipModuleUnload(k->module);
+  delete k;
+  return check_hip(e, "hipModuleUnload");
+}
+
+int sarek_hip_kernel_launch(sarek_hip_kernel k, const unsigned grid[3], const unsigned block[3],
+                            unsigned shared_mem_bytes, sarek_hip_stream stream, void **params,
+                            int n_params) {
+  if (!k || !grid || !block) return fail(SAREK_HIP_E_INVALID_ARG, "kernel_launch: NULL argument");
+  if (n_params > 0 && !params) return fail(SAREK_HIP_E_INVALID_ARG, "kernel_launch: NULL params");
+  for (int i = 0; i < 3; ++i)
+    if (grid[i] == 0 || block[i] == 0)
+      return fail(SAREK_HIP_E_INVALID_ARG, "kernel_launch: zero grid or block dimension");
+  SAREK_HIP_TRY(hipModuleLaunchKernel(k->function, grid[0], grid[1], grid[2], block[0], block[1],
+                                      block[2], shared_mem_bytes, as_stream(stream), params,
+                                      nullptr));
+  return SAREK_HIP_OK;
+}
+}

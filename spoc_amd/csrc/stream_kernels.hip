@@ -1,0 +1,345 @@
+// Bandwidth-bound kernels of the sarek-hip hot path for gfx950 (wave64):
+// stream triad, fused triad+sum, block-256 sum / dot product, the double fold of
+// partials and the f32 -> bf16/fp16 input casts.
+//
+// Design: every global access is a 128-bit (float4) coalesced load or store, each
+// thread keeps several independent 128-bit loads in flight, `a` is written with
+// non-temporal stores (it is never re-read by these kernels), and sums go
+// lane -> DPP wave reduction -> LDS across the waves of a block -> one f32 partial
+// per block -> a one-block fold in double.
+#include "common.hpp"
+#include "tunables.hpp"
+
+namespace sarek_hip {
+namespace {
+
+constexpr int kBlock = 256;   // threads per workgroup (4 waves)
+constexpr int kUnroll = 4;    // float4 per thread per grid-stride step
+
+// ---- wave64 sum by DPP -------------------------------------------------------
+template <int Ctrl>
+__device__ __forceinline__ float dpp_add(float v) {
+  int iv = __builtin_bit_cast(int, v);
+  int sh = __builtin_amdgcn_update_dpp(0, iv, Ctrl, 0xF, 0xF, true);
+  return v + __builtin_bit_cast(float, sh);
+}
+
+// Sum over the 64 lanes of a wave; the result is valid in every lane.
+__device__ __forceinline__ float wave_sum(float v) {
+  v = dpp_add<0xB1>(v);   // quad_perm [1,0,3,2]
+  v = dpp_add<0x4E>(v);   // quad_perm [2,3,0,1]
+  v = dpp_add<0x141>(v);  // row_half_mirror: lane i <-> 7-i within each 8 lanes: sums of 8
+  v = dpp_add<0x140>(v);  // row_mirror: sums of 16, valid in all 16 lanes of a row
+  int iv = __builtin_bit_cast(int, v);
+  float r0 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(iv, 0));
+  float r1 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(iv, 16));
+  float r2 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(iv, 32));
+  float r3 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(iv, 48));
+  return (r0 + r1) + (r2 + r3);
+}
+
+// Sum over a 256-thread block; valid in thread 0.
+__device__ __forceinline__ float block_sum(float v) {
+  __shared__ float wave_part[kBlock / 64];
+  v = wave_sum(v);
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  if (lane == 0) wave_part[wave] = v;
+  __syncthreads();
+  float r = 0.f;
+  if (threadIdx.x == 0) r = (wave_part[0] + wave_part[1]) + (wave_part[2] + wave_part[3]);
+  return r;
+}
+
+// One triad element with the Native backend's rounding: operands widen to double,
+// the product of two binary32 values is exact in double, one double addition, one
+// rounding to binary32.
+__device__ __forceinline__ float triad1(float b, float c, double s) {
+  return static_cast<float>(static_cast<double>(b) + static_cast<double>(c) * s);
+}
+
+__device__ __forceinline__ float4 triad4(float4 b, float4 c, double s) {
+  return make_float4(triad1(b.x, c.x, s), triad1(b.y, c.y, s), triad1(b.z, c.z, s),
+                     triad1(b.w, c.w, s));
+}
+
+typedef float f32x4_t __attribute__((ext_vector_type(4)));
+__device__ __forceinline__ float4 ldg_nt(const float4 *p) {
+  f32x4_t v = __builtin_nontemporal_load(reinterpret_cast<const f32x4_t *>(p));
+  return make_float4(v.x, v.y, v.z, v.w);
+}
+__device__ __forceinline__ void stg_nt(float4 *p, float4 v) {
+  f32x4_t w = {v.x, v.y, v.z, v.w};
+  __builtin_nontemporal_store(w, reinterpret_cast<f32x4_t *>(p));
+}
+
+// a = b + c*s over n4 float4 plus the (n & 3) scalar tail; when WithSum, one f32
+// partial per block is written to partials[blockIdx.x].
+template <bool WithSum>
+__global__ __launch_bounds__(kBlock) void triad_kernel(float *__restrict__ a,
+                                                       const float *__restrict__ b,
+                                                       const float *__restrict__ c, float s,
+                                                       int64_t n, float *__restrict__ partials) {
+  const double sd = static_cast<double>(s);
+  const int64_t n4 = n >> 2;
+  float4 *a4 = reinterpret_cast<float4 *>(a);
+  const float4 *b4 = reinterpret_cast<const float4 *>(b);
+  const float4 *c4 = reinterpret_cast<const float4 *>(c);
+  float4 acc = make_float4(0.f, 0.f, 0.f, 0.f);
+  const int64_t step = static_cast<int64_t>(gridDim.x) * (kBlock * kUnroll);
+  for (int64_t base = static_cast<int64_t>(blockIdx.x) * (kBlock * kUnroll) + threadIdx.x;
+       base < n4; base += step) {
+    float4 bv[kUnroll], cv[kUnroll];
+    if (base + (kUnroll - 1) * kBlock < n4) {
+#pragma unroll
+      for (int u = 0; u < kUnroll; ++u) bv[u] = ldg_nt(b4 + base + u * kBlock);
+#pragma unroll
+      for (int u = 0; u < kUnroll; ++u) cv[u] = ldg_nt(c4 + base + u * kBlock);
+#pragma unroll
+      for (int u = 0; u < kUnroll; ++u) {
+        float4 r = triad4(bv[u], cv[u], sd);
+        stg_nt(a4 + base + u * kBlock, r);
+        if (WithSum) {
+          acc.x += r.x; acc.y += r.y; acc.z += r.z; acc.w += r.w;
+        }
+      }
+    } else {
+#pragma unroll
+      for (int u = 0; u < kUnroll; ++u) {
+        const int64_t i = base + u * kBlock;
+        if (i < n4) {
+          float4 r = triad4(b4[i], c4[i], sd);
+          a4[i] = r;
+          if (WithSum) {
+            acc.x += r.x; acc.y += r.y; acc.z += r.z; acc.w += r.w;
+          }
+        }
+      }
+    }
+  }
+  // scalar tail: at most three elements, taken by the first threads of block 0
+  if (blockIdx.x == 0) {
+    const int64_t i = (n4 << 2) + threadIdx.x;
+    if (i < n) {
+      float r = triad1(b[i], c[i], sd);
+      a[i] = r;
+      if (WithSum) acc.x += r;
+    }
+  }
+  if (WithSum) {
+    float t = block_sum((acc.x + acc.y) + (acc.z + acc.w));
+    if (threadIdx.x == 0) partials[blockIdx.x] = t;
+  }
+}
+
+// Unaligned-pointer fallback: one element per thread, grid-stride.
+template <bool WithSum>
+__global__ __launch_bounds__(kBlock) void triad_scalar_kernel(float *__restrict__ a,
+                                                              const float *__restrict__ b,
+                                                              const float *__restrict__ c,
+                                                              float s, int64_t n,
+                                                              float *__restrict__ partials) {
+  const double sd = static_cast<double>(s);
+  float acc = 0.f;
+  const int64_t step = static_cast<int64_t>(gridDim.x) * kBlock;
+  for (int64_t i = static_cast<int64_t>(blockIdx.x) * kBlock + threadIdx.x; i < n; i += step) {
+    float r = triad1(b[i], c[i], sd);
+    a[i] = r;
+    acc += r;
+  }
+  if (WithSum) {
+    float t = block_sum(acc);
+    if (threadIdx.x == 0) partials[blockIdx.x] = t;
+  }
+}
+
+// *out = sum of partials[0..count) accumulated in double by one block.
+__global__ __launch_bounds__(1024) void fold_kernel(const float *__restrict__ partials,
+                                                    int64_t count, double *__restrict__ out) {
+  __shared__ double sh[1024];
+  double acc = 0.0;
+  for (int64_t i = threadIdx.x; i < count; i += 1024) acc += static_cast<double>(partials[i]);
+  sh[threadIdx.x] = acc;
+  __syncthreads();
+  for (int half = 512; half >= 1; half >>= 1) {
+    if (static_cast<int>(threadIdx.x) < half) sh[threadIdx.x] += sh[threadIdx.x + half];
+    __syncthreads();
+  }
+  if (threadIdx.x == 0) *out = sh[0];
+}
+
+// One wave per 256-element block of the input: out[j] = sum(in[256j..256j+255]),
+// zero padded past n.  Dot sums x[i]*y[i].  Each lane folds its four elements, the
+// wave sum is f32; the summation order differs from the reference's halving tree,
+// which its own checks allow for (1e-3 relative on the folded total).
+template <bool Dot>
+__global__ __launch_bounds__(kBlock) void block256_kernel(const float *__restrict__ x,
+                                                          const float *__restrict__ y,
+                                                          float *__restrict__ out, int64_t n,
+                                                          int64_t nblocks) {
+  const int lane = threadIdx.x & 63;
+  const int64_t wave = static_cast<int64_t>(blockIdx.x) * (kBlock / 64) + (threadIdx.x >> 6);
+  const int64_t wstep = static_cast<int64_t>(gridDim.x) * (kBlock / 64);
+  for (int64_t j = wave; j < nblocks; j += wstep) {
+    const int64_t i = j * 256 + lane * 4;
+    float v;
+    if (i + 3 < n) {
+      float4 xv = *reinterpret_cast<const float4 *>(x + i);
+      if (Dot) {
+        float4 yv = *reinterpret_cast<const float4 *>(y + i);
+        v = (xv.x * yv.x + xv.y * yv.y) + (xv.z * yv.z + xv.w * yv.w);
+      } else {
+        v = (xv.x + xv.y) + (xv.z + xv.w);
+      }
+    } else {
+      v = 0.f;
+      for (int e = 0; e < 4; ++e)
+        if (i + e < n) v += Dot ? x[i + e] * y[i + e] : x[i + e];
+    }
+    v = wave_sum(v);
+    if (lane == 0) out[j] = v;
+  }
+}
+
+// f32 -> bf16 bits, round to nearest even; NaN stays a quiet NaN.
+__device__ __forceinline__ uint16_t f32_to_bf16_rne(float f) {
+  uint32_t u = __builtin_bit_cast(uint32_t, f);
+  if ((u & 0x7F800000u) == 0x7F800000u) {
+    if (u & 0x007FFFFFu) u |= 0x00400000u;
+    return static_cast<uint16_t>(u >> 16);
+  }
+  u += 0x7FFFu + ((u >> 16) & 1u);
+  return static_cast<uint16_t>(u >> 16);
+}
+
+__device__ __forceinline__ uint16_t f32_to_f16_rne(float f) {
+  _Float16 h = static_cast<_Float16>(f);  // v_cvt_f16_f32: round to nearest even
+  return __builtin_bit_cast(uint16_t, h);
+}
+
+template <bool Bf16>
+__global__ __launch_bounds__(kBlock) void cast16_kernel(const float *__restrict__ in,
+                                                        uint16_t *__restrict__ out, int64_t n) {
+  const int64_t step = static_cast<int64_t>(gridDim.x) * kBlock;
+  for (int64_t i = static_cast<int64_t>(blockIdx.x) * kBlock + threadIdx.x; i < n; i += step)
+    out[i] = Bf16 ? f32_to_bf16_rne(in[i]) : f32_to_f16_rne(in[i]);
+}
+
+inline bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+
+// Number of workgroups the triad kernels are launched with for n elements.
+inline int64_t triad_blocks(int64_t n) {
+  const int64_t per_block = static_cast<int64_t>(kBlock) * kUnroll * 4;  // elements per step
+  int64_t need = ceil_div(n > 0 ? n : 1, per_block);
+  int64_t cap = static_cast<int64_t>(tunable("triad.max_blocks", 256 * 16));
+  return need < cap ? need : cap;
+}
+
+int launch_triad(float *a, const float *b, const float *c, float s, int64_t n, float *partials,
+                 bool with_sum, hipStream_t st) {
+  if (n == 0) return SAREK_HIP_OK;
+  const bool vec = aligned16(a) && aligned16(b) && aligned16(c);
+  const unsigned blocks = static_cast<unsigned>(triad_blocks(n));
+  if (vec) {
+    if (with_sum)
+      hipLaunchKernelGGL(triad_kernel<true>, dim3(blocks), dim3(kBlock), 0, st, a, b, c, s, n, partials);
+    else
+      hipLaunchKernelGGL(triad_kernel<false>, dim3(blocks), dim3(kBlock), 0, st, a, b, c, s, n, partials);
+  } else {
+    if (with_sum)
+      hipLaunchKernelGGL(triad_scalar_kernel<true>, dim3(blocks), dim3(kBlock), 0, st, a, b, c, s, n, partials);
+    else
+      hipLaunchKernelGGL(triad_scalar_kernel<false>, dim3(blocks), dim3(kBlock), 0, st, a, b, c, s, n, partials);
+  }
+  return check_launch("triad kernel launch");
+}
+
+}  // namespace
+}  // namespace sarek_hip
+
+using namespace sarek_hip;
+
+extern "C" {
+
+int sarek_hip_triad_f32(float *a, const float *b, const float *c, float s, int64_t n,
+                        sarek_hip_stream stream) {
+  if (n < 0) return fail(SAREK_HIP_E_INVALID_ARG, "triad: negative length %lld", (long long)n);
+  if (n > 0 && (!a || !b || !c)) return fail(SAREK_HIP_E_INVALID_ARG, "triad: NULL vector");
+  return launch_triad(a, b, c, s, n, nullptr, false, as_stream(stream));
+}
+
+int64_t sarek_hip_triad_sum_workspace_floats(int64_t n) { return n <= 0 ? 1 : triad_blocks(n); }
+
+int sarek_hip_triad_sum_f32(float *a, const float *b, const float *c, float s, int64_t n,
+                            float *partials, int64_t partials_len, double *sum_out,
+                            sarek_hip_stream stream) {
+  if (n < 0) return fail(SAREK_HIP_E_INVALID_ARG, "triad_sum: negative length %lld", (long long)n);
+  if (!sum_out) return fail(SAREK_HIP_E_INVALID_ARG, "triad_sum: NULL sum_out");
+  if (n > 0 && (!a || !b || !c || !partials))
+    return fail(SAREK_HIP_E_INVALID_ARG, "triad_sum: NULL vector or workspace");
+  const int64_t blocks = n == 0 ? 0 : triad_blocks(n);
+  if (partials_len < blocks)
+    return fail(SAREK_HIP_E_WORKSPACE, "triad_sum: workspace holds %lld floats, %lld needed",
+                (long long)partials_len, (long long)blocks);
+  hipStream_t st = as_stream(stream);
+  int rc = launch_triad(a, b, c, s, n, partials, true, st);
+  if (rc != SAREK_HIP_OK) return rc;
+  hipLaunchKernelGGL(fold_kernel, dim3(1), dim3(1024), 0, st, partials, blocks, sum_out);
+  return check_launch("fold kernel launch");
+}
+
+int sarek_hip_fold_partials_f64(const float *partials, int64_t count, double *sum_out,
+                                sarek_hip_stream stream) {
+  if (count < 0 || !sum_out || (count > 0 && !partials))
+    return fail(SAREK_HIP_E_INVALID_ARG, "fold_partials: bad arguments");
+  hipLaunchKernelGGL(fold_kernel, dim3(1), dim3(1024), 0, as_stream(stream), partials, count, sum_out);
+  return check_launch("fold kernel launch");
+}
+
+static int launch_block256(const float *x, const float *y, float *out, int64_t n, bool dot,
+                           hipStream_t st) {
+  if (n < 0) return fail(SAREK_HIP_E_INVALID_ARG, "block256: negative length");
+  if (n == 0) return SAREK_HIP_OK;
+  if (!x || !out || (dot && !y)) return fail(SAREK_HIP_E_INVALID_ARG, "block256: NULL vector");
+  if (!aligned16(x) || (dot && !aligned16(y)))
+    return fail(SAREK_HIP_E_INVALID_ARG, "block256: input vectors must be 16-byte aligned");
+  const int64_t nblocks = ceil_div(n, 256);
+  int64_t wg = ceil_div(nblocks, kBlock / 64);
+  const int64_t cap = tunable("block256.max_blocks", 256 * 32);
+  if (wg > cap) wg = cap;
+  if (dot)
+    hipLaunchKernelGGL(block256_kernel<true>, dim3((unsigned)wg), dim3(kBlock), 0, st, x, y, out, n, nblocks);
+  else
+    hipLaunchKernelGGL(block256_kernel<false>, dim3((unsigned)wg), dim3(kBlock), 0, st, x, y, out, n, nblocks);
+  return check_launch("block256 kernel launch");
+}
+
+int sarek_hip_reduce_sum_block256_f32(const float *in, float *out, int64_t n,
+                                      sarek_hip_stream stream) {
+  return launch_block256(in, nullptr, out, n, false, as_stream(stream));
+}
+
+int sarek_hip_dot_block256_f32(const float *a, const float *b, float *out, int64_t n,
+                               sarek_hip_stream stream) {
+  return launch_block256(a, b, out, n, true, as_stream(stream));
+}
+
+static int launch_cast(const float *in, uint16_t *out, int64_t n, bool bf16, hipStream_t st) {
+  if (n < 0 || (n > 0 && (!in || !out))) return fail(SAREK_HIP_E_INVALID_ARG, "cast: bad arguments");
+  if (n == 0) return SAREK_HIP_OK;
+  int64_t wg = ceil_div(n, kBlock);
+  if (wg > 256 * 32) wg = 256 * 32;
+  if (bf16)
+    hipLaunchKernelGGL(cast16_kernel<true>, dim3((unsigned)wg), dim3(kBlock), 0, st, in, out, n);
+  else
+    hipLaunchKernelGGL(cast16_kernel<false>, dim3((unsigned)wg), dim3(kBlock), 0, st, in, out, n);
+  return check_launch("cast kernel launch");
+}
+
+int sarek_hip_cast_f32_to_bf16(const float *in, uint16_t *out, int64_t n, sarek_hip_stream stream) {
+  return launch_cast(in, out, n, true, as_stream(stream));
+}
+
+int sarek_hip_cast_f32_to_f16(const float *in, uint16_t *out, int64_t n, sarek_hip_stream stream) {
+  return launch_cast(in, out, n, false, as_stream(stream));
+}
+}

@@ -1,0 +1,337 @@
+"""ctypes binding of libsarek_hip.so plus tensor-level helpers.
+
+Mirrors the surface a plugin's ``Hip_bindings``/``Hip_api`` pair would expose
+(sarek-cuda/Cuda_bindings.ml, sarek-cuda/Cuda_api.ml in the reference): raw symbols
+in :data:`lib`, checked wrappers below.  torch is used for device memory and the
+current stream only.
+"""
+import ctypes as C
+import os
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "libsarek_hip.so")
+
+
+class SarekHipError(RuntimeError):
+    """Non-zero status from libsarek_hip (cf. Backend_error in the reference)."""
+
+    def __init__(self, status, name, message):
+        super().__init__(f"{name} ({status}): {message}")
+        self.status = status
+        self.name = name
+        self.message = message
+
+
+# Status codes of include/sarek_hip.h
+OK = 0
+E_INVALID_ARG = -1
+E_UNSUPPORTED = -2
+E_COMPILE = -3
+E_NO_DEVICE = -4
+E_WORKSPACE = -5
+E_PARSE = -6
+E_CODEGEN = -7
+E_BUFFER_TOO_SMALL = -8
+
+LANG_CUDA, LANG_OPENCL, LANG_PTX, LANG_SPIRV, LANG_GLSL, LANG_HIP = range(6)
+ARG_BUFFER, ARG_INT32, ARG_INT64, ARG_FLOAT32, ARG_FLOAT64 = range(5)
+
+
+class DeviceInfo(C.Structure):
+    _fields_ = [
+        ("name", C.c_char * 256), ("gcn_arch", C.c_char * 64),
+        ("total_global_mem", C.c_uint64), ("max_threads_per_block", C.c_int),
+        ("max_block_dim", C.c_int * 3), ("max_grid_dim", C.c_int * 3),
+        ("shared_mem_per_block", C.c_int), ("warp_size", C.c_int),
+        ("multiprocessor_count", C.c_int), ("clock_rate_khz", C.c_int),
+        ("memory_clock_rate_khz", C.c_int), ("memory_bus_width_bits", C.c_int),
+        ("l2_cache_size", C.c_int), ("compute_major", C.c_int), ("compute_minor", C.c_int),
+    ]
+
+
+class Arg(C.Structure):
+    _fields_ = [("kind", C.c_int), ("buffer", C.c_void_p), ("length", C.c_int64),
+                ("i32", C.c_int32), ("i64", C.c_int64), ("f32", C.c_float), ("f64", C.c_double)]
+
+
+_vp, _i, _i64, _sz, _f = C.c_void_p, C.c_int, C.c_int64, C.c_size_t, C.c_float
+_int3 = C.POINTER(C.c_int)
+_uint3 = C.POINTER(C.c_uint)
+
+# Every symbol include/sarek_hip.h declares: (restype, argtypes).
+SYMBOLS = {
+    "sarek_hip_abi_version": (_i, []),
+    "sarek_hip_last_error": (C.c_char_p, []),
+    "sarek_hip_status_name": (C.c_char_p, [_i]),
+    "sarek_hip_init": (_i, []),
+    "sarek_hip_is_available": (_i, []),
+    "sarek_hip_device_count": (_i, [C.POINTER(_i)]),
+    "sarek_hip_device_get_info": (_i, [_i, C.POINTER(DeviceInfo)]),
+    "sarek_hip_device_set_current": (_i, [_i]),
+    "sarek_hip_device_get_current": (_i, [C.POINTER(_i)]),
+    "sarek_hip_device_synchronize": (_i, []),
+    "sarek_hip_mem_get_info": (_i, [C.POINTER(_sz), C.POINTER(_sz)]),
+    "sarek_hip_driver_version": (_i, [C.POINTER(_i)]),
+    "sarek_hip_mem_alloc": (_i, [C.POINTER(_vp), _sz]),
+    "sarek_hip_mem_free": (_i, [_vp]),
+    "sarek_hip_memcpy_htod": (_i, [_vp, _vp, _sz]),
+    "sarek_hip_memcpy_dtoh": (_i, [_vp, _vp, _sz]),
+    "sarek_hip_memcpy_dtod": (_i, [_vp, _vp, _sz]),
+    "sarek_hip_memset_d8": (_i, [_vp, C.c_ubyte, _sz]),
+    "sarek_hip_stream_create": (_i, [C.POINTER(_vp)]),
+    "sarek_hip_stream_destroy": (_i, [_vp]),
+    "sarek_hip_stream_synchronize": (_i, [_vp]),
+    "sarek_hip_event_create": (_i, [C.POINTER(_vp)]),
+    "sarek_hip_event_destroy": (_i, [_vp]),
+    "sarek_hip_event_record": (_i, [_vp, _vp]),
+    "sarek_hip_event_synchronize": (_i, [_vp]),
+    "sarek_hip_event_elapsed_ms": (_i, [_vp, _vp, C.POINTER(_f)]),
+    "sarek_hip_kernel_compile": (_i, [C.c_char_p, C.c_char_p, C.POINTER(_vp), C.c_char_p, _sz]),
+    "sarek_hip_kernel_compile_cached": (_i, [C.c_char_p, C.c_char_p, C.POINTER(_vp), C.c_char_p, _sz]),
+    "sarek_hip_kernel_clear_cache": (_i, []),
+    "sarek_hip_kernel_destroy": (_i, [_vp]),
+    "sarek_hip_kernel_launch": (_i, [_vp, _uint3, _uint3, C.c_uint, _vp, C.POINTER(_vp), _i]),
+    "sarek_hip_generate_source": (_i, [C.c_char_p, _int3, C.c_char_p, _sz, C.POINTER(_sz)]),
+    "sarek_hip_run_source": (_i, [C.c_char_p, _i, C.c_char_p, _int3, _int3, _i, C.POINTER(Arg), _i]),
+    "sarek_hip_set_specialisation": (_i, [_i]),
+    "sarek_hip_last_run_path": (C.c_char_p, []),
+    "sarek_hip_triad_f32": (_i, [_vp, _vp, _vp, _f, _i64, _vp]),
+    "sarek_hip_triad_sum_workspace_floats": (_i64, [_i64]),
+    "sarek_hip_triad_sum_f32": (_i, [_vp, _vp, _vp, _f, _i64, _vp, _i64, _vp, _vp]),
+    "sarek_hip_reduce_sum_block256_f32": (_i, [_vp, _vp, _i64, _vp]),
+    "sarek_hip_dot_block256_f32": (_i, [_vp, _vp, _vp, _i64, _vp]),
+    "sarek_hip_fold_partials_f64": (_i, [_vp, _i64, _vp, _vp]),
+    "sarek_hip_gemm_f32": (_i, [_vp, _vp, _vp, _i, _i, _i, _vp]),
+    "sarek_hip_gemm_bf16": (_i, [_vp, _vp, _vp, _i, _i, _i, _vp]),
+    "sarek_hip_gemm_f16": (_i, [_vp, _vp, _vp, _i, _i, _i, _vp]),
+    "sarek_hip_gemm_f16_bias_relu_rowsum": (_i, [_vp, _vp, _vp, _vp, _vp, _i, _i, _i, _vp]),
+    "sarek_hip_cast_f32_to_bf16": (_i, [_vp, _vp, _i64, _vp]),
+    "sarek_hip_cast_f32_to_f16": (_i, [_vp, _vp, _i64, _vp]),
+    "sarek_hip_set_tunable": (_i, [C.c_char_p, _i64]),
+}
+
+
+def _load():
+    if not os.path.exists(LIB_PATH):
+        raise ImportError(
+            f"{LIB_PATH} is not built: run `python -c 'import __graft_entry__ as g; g.build()'` "
+            "(or `make -C spoc_amd/csrc`).  There is no CPU fallback.")
+    lib = C.CDLL(LIB_PATH)
+    for name, (res, args) in SYMBOLS.items():
+        fn = getattr(lib, name)  # AttributeError if the library lacks a declared symbol
+        fn.restype = res
+        fn.argtypes = args
+    return lib
+
+
+lib = _load()
+
+
+def check(status):
+    if status != OK:
+        raise SarekHipError(status, lib.sarek_hip_status_name(status).decode(),
+                            lib.sarek_hip_last_error().decode(errors="replace"))
+
+
+def set_tunable(name, value):
+    check(lib.sarek_hip_set_tunable(name.encode(), int(value)))
+
+
+# ---------------------------------------------------------------------------
+# Tensor-level helpers (torch = device memory + stream plumbing only)
+
+def _torch():
+    import torch
+    return torch
+
+
+def _stream():
+    return C.c_void_p(_torch().cuda.current_stream().cuda_stream)
+
+
+def _ptr(t):
+    return C.c_void_p(t.data_ptr())
+
+
+def _need(t, dtype, name):
+    torch = _torch()
+    if not (isinstance(t, torch.Tensor) and t.is_cuda and t.dtype == dtype and t.is_contiguous()):
+        raise TypeError(f"{name}: expected a contiguous device tensor of {dtype}")
+
+
+def device_info(device=0):
+    info = DeviceInfo()
+    check(lib.sarek_hip_device_get_info(device, C.byref(info)))
+    return info
+
+
+def triad(b, c, s, out=None):
+    """a = b + c*s (f32 vectors).  Returns a."""
+    torch = _torch()
+    _need(b, torch.float32, "b")
+    _need(c, torch.float32, "c")
+    a = torch.empty_like(b) if out is None else out
+    check(lib.sarek_hip_triad_f32(_ptr(a), _ptr(b), _ptr(c), float(s), b.numel(), _stream()))
+    return a
+
+
+def triad_sum_workspace(n, device="cuda"):
+    torch = _torch()
+    cnt = int(lib.sarek_hip_triad_sum_workspace_floats(int(n)))
+    return (torch.empty(cnt, dtype=torch.float32, device=device),
+            torch.empty(1, dtype=torch.float64, device=device))
+
+
+def triad_sum(b, c, s, out=None, workspace=None):
+    """Fused a = b + c*s and sum(a).  Returns (a, sum_tensor[1] f64 on device)."""
+    torch = _torch()
+    _need(b, torch.float32, "b")
+    _need(c, torch.float32, "c")
+    a = torch.empty_like(b) if out is None else out
+    partials, total = workspace if workspace is not None else triad_sum_workspace(b.numel(), b.device)
+    check(lib.sarek_hip_triad_sum_f32(_ptr(a), _ptr(b), _ptr(c), float(s), b.numel(),
+                                      _ptr(partials), partials.numel(), _ptr(total), _stream()))
+    return a, total
+
+
+def reduce_sum_block256(x):
+    torch = _torch()
+    _need(x, torch.float32, "x")
+    out = torch.empty((x.numel() + 255) // 256, dtype=torch.float32, device=x.device)
+    check(lib.sarek_hip_reduce_sum_block256_f32(_ptr(x), _ptr(out), x.numel(), _stream()))
+    return out
+
+
+def dot_block256(a, b):
+    torch = _torch()
+    _need(a, torch.float32, "a")
+    _need(b, torch.float32, "b")
+    out = torch.empty((a.numel() + 255) // 256, dtype=torch.float32, device=a.device)
+    check(lib.sarek_hip_dot_block256_f32(_ptr(a), _ptr(b), _ptr(out), a.numel(), _stream()))
+    return out
+
+
+def fold_partials(p):
+    torch = _torch()
+    _need(p, torch.float32, "partials")
+    out = torch.empty(1, dtype=torch.float64, device=p.device)
+    check(lib.sarek_hip_fold_partials_f64(_ptr(p), p.numel(), _ptr(out), _stream()))
+    return out
+
+
+def gemm_f32(a, b, out=None):
+    torch = _torch()
+    _need(a, torch.float32, "a")
+    _need(b, torch.float32, "b")
+    m, k = a.shape
+    k2, n = b.shape
+    if k != k2:
+        raise ValueError("gemm_f32: inner dimensions differ")
+    c = torch.empty((m, n), dtype=torch.float32, device=a.device) if out is None else out
+    check(lib.sarek_hip_gemm_f32(_ptr(a), _ptr(b), _ptr(c), m, n, k, _stream()))
+    return c
+
+
+def _gemm16(fn, dtype, a, b, out):
+    torch = _torch()
+    _need(a, dtype, "a")
+    _need(b, dtype, "b")
+    m, k = a.shape
+    k2, n = b.shape
+    if k != k2:
+        raise ValueError("gemm16: inner dimensions differ")
+    c = torch.empty((m, n), dtype=torch.float32, device=a.device) if out is None else out
+    check(fn(_ptr(a), _ptr(b), _ptr(c), m, n, k, _stream()))
+    return c
+
+
+def gemm_bf16(a, b, out=None):
+    return _gemm16(lib.sarek_hip_gemm_bf16, _torch().bfloat16, a, b, out)
+
+
+def gemm_f16(a, b, out=None):
+    return _gemm16(lib.sarek_hip_gemm_f16, _torch().float16, a, b, out)
+
+
+def gemm_f16_bias_relu_rowsum(a, b, bias, out=None, rowsum=None):
+    torch = _torch()
+    _need(a, torch.float16, "a")
+    _need(b, torch.float16, "b")
+    _need(bias, torch.float32, "bias")
+    m, k = a.shape
+    k2, n = b.shape
+    if k != k2 or bias.numel() != n:
+        raise ValueError("gemm_f16_bias_relu_rowsum: shape mismatch")
+    y = torch.empty((m, n), dtype=torch.float32, device=a.device) if out is None else out
+    rs = torch.empty(m, dtype=torch.float32, device=a.device) if rowsum is None else rowsum
+    check(lib.sarek_hip_gemm_f16_bias_relu_rowsum(_ptr(a), _ptr(b), _ptr(bias), _ptr(y), _ptr(rs),
+                                                  m, n, k, _stream()))
+    return y, rs
+
+
+def cast_bf16(x):
+    torch = _torch()
+    _need(x, torch.float32, "x")
+    out = torch.empty(x.shape, dtype=torch.bfloat16, device=x.device)
+    check(lib.sarek_hip_cast_f32_to_bf16(_ptr(x), _ptr(out), x.numel(), _stream()))
+    return out
+
+
+def cast_f16(x):
+    torch = _torch()
+    _need(x, torch.float32, "x")
+    out = torch.empty(x.shape, dtype=torch.float16, device=x.device)
+    check(lib.sarek_hip_cast_f32_to_f16(_ptr(x), _ptr(out), x.numel(), _stream()))
+    return out
+
+
+def make_args(items):
+    """Build a run_source argument array.
+
+    items: device tensors (expanded to buffer + int32 length, as the reference's
+    dispatcher does for vectors), ("i32", v), ("i64", v), ("f32", v), ("f64", v),
+    or ("buf", tensor) for a bare buffer without the injected length.
+    """
+    torch = _torch()
+    out = []
+    for it in items:
+        if isinstance(it, torch.Tensor):
+            out.append(Arg(kind=ARG_BUFFER, buffer=it.data_ptr(), length=it.numel()))
+            out.append(Arg(kind=ARG_INT32, i32=it.numel()))
+        else:
+            kind, v = it
+            if kind == "buf":
+                out.append(Arg(kind=ARG_BUFFER, buffer=v.data_ptr(), length=v.numel()))
+            elif kind == "i32":
+                out.append(Arg(kind=ARG_INT32, i32=int(v)))
+            elif kind == "i64":
+                out.append(Arg(kind=ARG_INT64, i64=int(v)))
+            elif kind == "f32":
+                out.append(Arg(kind=ARG_FLOAT32, f32=float(v)))
+            elif kind == "f64":
+                out.append(Arg(kind=ARG_FLOAT64, f64=float(v)))
+            else:
+                raise ValueError(f"unknown argument kind {kind!r}")
+    return (Arg * len(out))(*out), len(out)
+
+
+def run_source(source, kernel_name, block, grid, items, shared_mem=0, lang=LANG_HIP):
+    """Plugin-level run_source on the default stream."""
+    args, n = make_args(items)
+    blk = (C.c_int * 3)(*block)
+    grd = (C.c_int * 3)(*grid)
+    check(lib.sarek_hip_run_source(source.encode(), lang, kernel_name.encode(), blk, grd,
+                                   int(shared_mem), args, n))
+    return lib.sarek_hip_last_run_path().decode()
+
+
+def generate_source(ir_text, block=None):
+    blk = (C.c_int * 3)(*block) if block is not None else None
+    needed = C.c_size_t(0)
+    buf = C.create_string_buffer(1 << 16)
+    rc = lib.sarek_hip_generate_source(ir_text.encode(), blk, buf, len(buf), C.byref(needed))
+    if rc == E_BUFFER_TOO_SMALL:
+        buf = C.create_string_buffer(needed.value + 1)
+        rc = lib.sarek_hip_generate_source(ir_text.encode(), blk, buf, len(buf), C.byref(needed))
+    check(rc)
+    return buf.value.decode()

@@ -1,0 +1,68 @@
+"""The C-ABI library loads and exports every symbol include/sarek_hip.h declares.
+No compute call is made here (this file runs without a GPU)."""
+import ctypes
+import os
+import re
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def declared_symbols():
+    text = open(os.path.join(ROOT, "include", "sarek_hip.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(sarek_hip_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_header_symbols_are_exported(hip):
+    names = declared_symbols()
+    assert len(names) >= 45
+    raw = ctypes.CDLL(hip.LIB_PATH)
+    missing = [n for n in names if not hasattr(raw, n)]
+    assert missing == []
+
+
+def test_python_binding_covers_the_header(hip):
+    assert sorted(hip.SYMBOLS) == declared_symbols()
+
+
+def test_abi_version_and_status_names(hip):
+    assert hip.lib.sarek_hip_abi_version() == 1
+    assert hip.lib.sarek_hip_status_name(0) == b"SAREK_HIP_OK"
+    assert hip.lib.sarek_hip_status_name(-2) == b"SAREK_HIP_E_UNSUPPORTED"
+    assert hip.lib.sarek_hip_status_name(-5) == b"SAREK_HIP_E_WORKSPACE"
+
+
+def test_is_available_never_raises(hip):
+    # Framework_registry wraps is_available in try (sarek/framework/Framework_registry.ml:77-87)
+    assert hip.lib.sarek_hip_is_available() in (0, 1)
+
+
+def test_argument_validation_needs_no_gpu(hip):
+    # invalid arguments are rejected before any HIP call is made
+    assert hip.lib.sarek_hip_gemm_f32(None, None, None, 0, 4, 4, None) == hip.E_INVALID_ARG
+    assert b"positive" in hip.lib.sarek_hip_last_error()
+    assert hip.lib.sarek_hip_triad_f32(None, None, None, 3.0, -1, None) == hip.E_INVALID_ARG
+    assert hip.lib.sarek_hip_triad_sum_f32(None, None, None, 3.0, 8, None, 0, None, None) == hip.E_INVALID_ARG
+    blk = (ctypes.c_int * 3)(16, 16, 1)
+    # unsupported source languages, error text in the reference's wording
+    # (sarek-cuda/Cuda_plugin.ml:211-220)
+    for lang, word in ((hip.LANG_OPENCL, b"OpenCL_Source"), (hip.LANG_PTX, b"PTX"),
+                       (hip.LANG_SPIRV, b"SPIR_V"), (hip.LANG_GLSL, b"GLSL_Source")):
+        rc = hip.lib.sarek_hip_run_source(b"x", lang, b"k", blk, blk, 0, None, 0)
+        assert rc == hip.E_UNSUPPORTED
+        assert word in hip.lib.sarek_hip_last_error()
+    assert hip.lib.sarek_hip_mem_free(None) == 0
+    assert hip.lib.sarek_hip_triad_sum_workspace_floats(1 << 28) >= 1
+
+
+def test_missing_library_fails_loudly(monkeypatch, tmp_path):
+    import importlib
+    from spoc_amd import hip as real
+    monkeypatch.setattr(real, "LIB_PATH", str(tmp_path / "nope.so"))
+    try:
+        real._load()
+    except ImportError as e:
+        assert "no CPU fallback" in str(e) or "not built" in str(e)
+    else:
+        raise AssertionError("loading a missing library must raise")
+    importlib.reload(real)

@@ -1,0 +1,192 @@
+"""GPU parity: f32 / bf16 / fp16 GEMMs and the fused bias+ReLU+row-sum epilogue through
+the C ABI against the CPU oracle (Native-backend semantics: double accumulation in
+increasing k, one rounding at the store).
+
+Tolerances (stated by the task for this path):
+  f32 GEMM      max|err| <= 1e-4 * |A|_inf-elem * |B|_inf-elem * sqrt(K)
+  bf16/fp16-in  <= 2e-2 relative, measured as max|err| / max|C_ref|
+The 16-bit inputs are rounded once (RNE) and both sides consume the same rounded values,
+so the observed error is f32-accumulation error only and is asserted much tighter."""
+import numpy as np
+import pytest
+
+pytestmark = pytest.mark.gpu
+
+
+def dev(torch, x):
+    return torch.from_numpy(np.ascontiguousarray(x)).cuda()
+
+
+def f32_tol(a, b, k):
+    return 1e-4 * float(np.abs(a).max()) * float(np.abs(b).max()) * np.sqrt(k)
+
+
+F32_SHAPES = [(1, 1, 1), (16, 16, 16), (17, 33, 19), (128, 128, 128), (256, 256, 64),
+              (257, 255, 100), (300, 520, 36), (512, 512, 512), (1024, 1024, 1024)]
+
+
+@pytest.mark.parametrize("m,n,k", F32_SHAPES)
+def test_gemm_f32_vs_oracle(hip, oracle, torch_cuda, m, n, k):
+    torch = torch_cuda
+    a = oracle.fill_uniform(m * k, seed=0xA11CE, lo=-1.0, hi=1.0).reshape(m, k)
+    b = oracle.fill_uniform(k * n, seed=0xB0B, lo=-1.0, hi=1.0).reshape(k, n)
+    c = hip.gemm_f32(dev(torch, a), dev(torch, b)).cpu().numpy()
+    ref = oracle.gemm(a, b)
+    err = float(np.abs(c - ref).max())
+    assert err <= f32_tol(a, b, k), (err, f32_tol(a, b, k))
+    assert err <= 4e-6 * np.sqrt(k) + 1e-6  # what f32 accumulation actually gives
+
+
+def test_gemm_f32_reference_bench_inputs(hip, oracle, torch_cuda):
+    """bench_matrix_mul_tiled.ml:109-112 inputs, its 1e-3 absolute check (:194)."""
+    torch = torch_cuda
+    m = n = k = 256
+    a = ((np.arange(m * k) % 10) / 10.0).astype(np.float32).reshape(m, k)
+    b = (((np.arange(k * n) + 1) % 10) / 10.0).astype(np.float32).reshape(k, n)
+    c = hip.gemm_f32(dev(torch, a), dev(torch, b)).cpu().numpy()
+    expected = ((np.arange(m * k) % 10) / 10.0).reshape(m, k) @ (((np.arange(k * n) + 1) % 10) / 10.0).reshape(k, n)
+    assert np.abs(c - expected).max() <= 1e-3
+    assert np.abs(c - oracle.gemm(a, b)).max() <= 1e-4
+
+
+def test_gemm_f32_identity_and_selector(hip, torch_cuda):
+    torch = torch_cuda
+    torch.manual_seed(0)
+    a = torch.rand(300, 260, device="cuda") * 2 - 1
+    eye = torch.eye(260, device="cuda")
+    assert torch.equal(hip.gemm_f32(a, eye), a)       # exact: one nonzero product per sum
+    e = torch.zeros(260, 40, device="cuda")
+    e[7, 3] = 1.0
+    c = hip.gemm_f32(a, e)
+    assert torch.equal(c[:, 3], a[:, 7]) and float(c.abs().sum()) == float(a[:, 7].abs().sum())
+
+
+def test_gemm_f32_full_size_rows(hip, oracle, torch_cuda):
+    """8192^3: sampled rows against the oracle + linearity."""
+    torch = torch_cuda
+    m = n = k = 8192
+    a = oracle.fill_uniform(m * k, seed=0xA11CE, lo=-1.0, hi=1.0).reshape(m, k)
+    b = oracle.fill_uniform(k * n, seed=0xB0B, lo=-1.0, hi=1.0).reshape(k, n)
+    da, db = dev(torch, a), dev(torch, b)
+    c = hip.gemm_f32(da, db)
+    rows = np.array([0, 1, 255, 256, 4095, 4096, 8191], np.int32)
+    ref = oracle.gemm_rows(a, b, rows)
+    got = c[torch.from_numpy(rows).long().cuda()].cpu().numpy()
+    err = float(np.abs(got - ref).max())
+    assert err <= f32_tol(a, b, k), err
+    c2 = hip.gemm_f32(da * 2.0, db)           # scaling by 2 is exact in binary
+    assert torch.equal(c2, c * 2.0)
+
+
+BF_SHAPES = [(8, 8, 8), (32, 32, 16), (256, 256, 64), (256, 256, 128), (264, 520, 72),
+             (1, 8, 8), (100, 64, 200), (512, 768, 256), (1024, 1024, 1024)]
+
+
+def normal16(oracle, shape, seed, kind):
+    rng = np.random.default_rng(seed)
+    x = rng.normal(0.0, 0.02, shape).astype(np.float32)
+    return oracle.round_bf16(x) if kind == "bf16" else oracle.round_f16(x)
+
+
+@pytest.mark.parametrize("kind", ["bf16", "f16"])
+@pytest.mark.parametrize("m,n,k", BF_SHAPES)
+def test_gemm16_vs_oracle(hip, oracle, torch_cuda, kind, m, n, k):
+    torch = torch_cuda
+    a = normal16(oracle, (m, k), 0xA4, kind)
+    b = normal16(oracle, (k, n), 0xB4, kind)
+    tdt = torch.bfloat16 if kind == "bf16" else torch.float16
+    da, db = dev(torch, a).to(tdt), dev(torch, b).to(tdt)   # exact: values already representable
+    assert torch.equal(da.float().cpu(), torch.from_numpy(a))
+    fn = hip.gemm_bf16 if kind == "bf16" else hip.gemm_f16
+    c = fn(da, db).cpu().numpy()
+    ref = oracle.gemm(a, b)
+    scale = float(np.abs(ref).max())
+    rel = float(np.abs(c - ref).max()) / scale
+    assert rel <= 2e-2, rel
+    assert rel <= 1e-4, rel
+
+
+@pytest.mark.parametrize("kind", ["bf16", "f16"])
+def test_gemm16_unaligned_shapes_use_fallback(hip, oracle, torch_cuda, kind):
+    torch = torch_cuda
+    m, n, k = 37, 51, 29   # n, k not multiples of 8
+    a = normal16(oracle, (m, k), 1, kind)
+    b = normal16(oracle, (k, n), 2, kind)
+    tdt = torch.bfloat16 if kind == "bf16" else torch.float16
+    fn = hip.gemm_bf16 if kind == "bf16" else hip.gemm_f16
+    c = fn(dev(torch, a).to(tdt), dev(torch, b).to(tdt)).cpu().numpy()
+    ref = oracle.gemm(a, b)
+    assert np.abs(c - ref).max() <= 1e-4 * np.abs(ref).max()
+
+
+def test_gemm16_integer_inputs_exact(hip, torch_cuda):
+    """Small integers: every product and partial sum is exact in f32, so any indexing or
+    k-permutation mistake shows up as a wrong integer."""
+    torch = torch_cuda
+    torch.manual_seed(3)
+    m, n, k = 320, 384, 192
+    a = torch.randint(-3, 4, (m, k), device="cuda").float()
+    b = torch.randint(-3, 4, (k, n), device="cuda").float()
+    want = (a.double() @ b.double()).float()
+    assert torch.equal(hip.gemm_bf16(a.bfloat16(), b.bfloat16()), want)
+    assert torch.equal(hip.gemm_f16(a.half(), b.half()), want)
+    assert torch.equal(hip.gemm_f32(a, b), want)
+
+
+@pytest.mark.parametrize("m,n,k", [(64, 256, 64), (255, 512, 128), (300, 264, 72), (33, 40, 24)])
+def test_epilogue_vs_oracle(hip, oracle, torch_cuda, m, n, k):
+    torch = torch_cuda
+    a = normal16(oracle, (m, k), 0xA5, "f16")
+    b = normal16(oracle, (k, n), 0xB5, "f16")
+    bias = oracle.fill_uniform(n, seed=0xB1A5, lo=-0.1, hi=0.1)
+    y, rs = hip.gemm_f16_bias_relu_rowsum(dev(torch, a).half(), dev(torch, b).half(), dev(torch, bias))
+    y_ref, rs_ref = oracle.gemm_bias_relu_rowsum(a, b, bias)
+    y = y.cpu().numpy()
+    rs = rs.cpu().numpy()
+    assert np.abs(y - y_ref).max() <= 2e-2 * np.abs(y_ref).max()
+    assert np.abs(y - y_ref).max() <= 1e-5 * max(1.0, np.abs(y_ref).max())
+    assert (y >= 0).all()
+    assert np.abs(rs - rs_ref).max() <= 1e-4 * np.abs(rs_ref).max()
+
+
+def test_epilogue_full_size_config(hip, oracle, torch_cuda):
+    """M=4095 (non tile multiple), N=11008, K=4096: sampled rows vs oracle, row sums vs Y."""
+    torch = torch_cuda
+    m, n, k = 4095, 11008, 4096
+    rng = np.random.default_rng(0xC5)
+    a = oracle.round_f16(rng.normal(0, 0.02, (m, k)).astype(np.float32))
+    b = oracle.round_f16(rng.normal(0, 0.02, (k, n)).astype(np.float32))
+    bias = oracle.fill_uniform(n, seed=0xB1A5, lo=-0.1, hi=0.1)
+    y, rs = hip.gemm_f16_bias_relu_rowsum(dev(torch, a).half(), dev(torch, b).half(), dev(torch, bias))
+    rows = np.array([0, 127, 128, 2047, 3968, 4094], np.int32)
+    y_ref, rs_ref = oracle.gemm_bias_relu_rowsum(a, b, bias, rows=rows)
+    idx = torch.from_numpy(rows).long().cuda()
+    got = y[idx].cpu().numpy()
+    assert np.abs(got - y_ref).max() <= 2e-2 * np.abs(y_ref).max()
+    assert np.abs(rs[idx].cpu().numpy() - rs_ref).max() <= 1e-4 * np.abs(rs_ref).max()
+    # size-independent: the fused row sums equal the row sums of the stored Y
+    assert torch.allclose(rs, y.double().sum(dim=1).float(), rtol=1e-4, atol=1e-3)
+
+
+def test_gemm_bf16_full_size_rows(hip, oracle, torch_cuda):
+    torch = torch_cuda
+    m = n = k = 8192
+    torch.manual_seed(0xA4)
+    a = (torch.randn(m, k, device="cuda") * 0.02).bfloat16()
+    b = (torch.randn(k, n, device="cuda") * 0.02).bfloat16()
+    c = hip.gemm_bf16(a, b)
+    rows = np.array([0, 255, 256, 5000, 8191], np.int32)
+    ref = oracle.gemm_rows(a.float().cpu().numpy(), b.float().cpu().numpy(), rows)
+    got = c[torch.from_numpy(rows).long().cuda()].cpu().numpy()
+    assert np.abs(got - ref).max() <= 2e-2 * np.abs(ref).max()
+    assert np.abs(got - ref).max() <= 1e-4 * np.abs(ref).max()
+    # exact power-of-two scaling commutes with the kernel
+    assert torch.equal(hip.gemm_bf16(a * 2, b), c * 2)
+
+
+def test_gemm_rejects_bad_arguments(hip, torch_cuda):
+    torch = torch_cuda
+    a = torch.zeros(4, 4, device="cuda")
+    with pytest.raises(hip.SarekHipError) as e:
+        hip.check(hip.lib.sarek_hip_gemm_f32(a.data_ptr(), a.data_ptr(), a.data_ptr(), 4, -1, 4, None))
+    assert e.value.status == hip.E_INVALID_ARG

@@ -1,0 +1,136 @@
+"""GPU parity: stream triad, fused triad+sum, block-256 reductions, casts — HIP kernels
+through the C ABI against the CPU oracle on the same seeded inputs.
+
+Bars: `a` bit-exact (the kernel evaluates b + c*s in double and rounds once, as the
+Native backend does); sums within 1e-5 relative (f32 reductions); block partials within
+the reference's own tolerance (1e-3 relative, bench_reduction.ml:161-163) and in practice
+~1e-6."""
+import numpy as np
+import pytest
+
+pytestmark = pytest.mark.gpu
+
+SIZES = [0, 1, 3, 4, 5, 255, 256, 257, 1023, 4096, 65537, 1 << 20, (1 << 22) + 3]
+
+
+def dev(torch, x):
+    return torch.from_numpy(np.ascontiguousarray(x)).cuda()
+
+
+@pytest.mark.parametrize("n", SIZES)
+def test_triad_bit_exact(hip, oracle, torch_cuda, n):
+    torch = torch_cuda
+    b = oracle.fill_uniform(n, seed=0xB)
+    c = oracle.fill_uniform(n, seed=0xC)
+    a = hip.triad(dev(torch, b), dev(torch, c), 3.0)
+    torch.cuda.synchronize()
+    assert np.array_equal(a.cpu().numpy(), oracle.triad(b, c, 3.0))
+
+
+def test_triad_reference_inputs(hip, oracle, torch_cuda):
+    torch = torch_cuda
+    n = 100000
+    b = ((np.arange(n) % 100) / 100.0).astype(np.float32)
+    c = (((np.arange(n) + 1) % 100) / 100.0).astype(np.float32)
+    a = hip.triad(dev(torch, b), dev(torch, c), 3.0).cpu().numpy()
+    expected = (np.arange(n) % 100) / 100.0 + ((np.arange(n) + 1) % 100) / 100.0 * 3.0
+    assert np.abs(a - expected).max() <= 1e-5  # bench_stream_triad.ml:122
+    assert np.array_equal(a, oracle.triad(b, c, 3.0))
+
+
+@pytest.mark.parametrize("n", SIZES)
+def test_triad_sum(hip, oracle, torch_cuda, n):
+    torch = torch_cuda
+    b = oracle.fill_uniform(n, seed=0xB)
+    c = oracle.fill_uniform(n, seed=0xC)
+    a, total = hip.triad_sum(dev(torch, b), dev(torch, c), 3.0)
+    torch.cuda.synchronize()
+    a_ref, _, sum_ref = oracle.triad_sum(b, c, 3.0)
+    assert np.array_equal(a.cpu().numpy(), a_ref)
+    got = float(total.item())
+    assert abs(got - sum_ref) <= 1e-5 * abs(sum_ref) + 0.0 if n else got == 0.0
+
+
+def test_triad_sum_unaligned_pointers(hip, oracle, torch_cuda):
+    torch = torch_cuda
+    n = 10001
+    b = oracle.fill_uniform(n + 1, seed=1)
+    c = oracle.fill_uniform(n + 1, seed=2)
+    db, dc = dev(torch, b)[1:], dev(torch, c)[1:]   # 4-byte aligned only
+    out = torch.empty(n + 1, dtype=torch.float32, device="cuda")[1:]
+    a, total = hip.triad_sum(db, dc, 3.0, out=out)
+    a_ref, _, sum_ref = oracle.triad_sum(b[1:], c[1:], 3.0)
+    assert np.array_equal(a.cpu().numpy(), a_ref)
+    assert abs(float(total.item()) - sum_ref) <= 1e-5 * sum_ref
+
+
+def test_triad_sum_workspace_too_small_is_an_error(hip, torch_cuda):
+    torch = torch_cuda
+    n = 1 << 20
+    b = torch.zeros(n, device="cuda")
+    ws = (torch.empty(1, device="cuda"), torch.empty(1, dtype=torch.float64, device="cuda"))
+    with pytest.raises(hip.SarekHipError) as e:
+        hip.triad_sum(b, b, 3.0, workspace=ws)
+    assert e.value.status == hip.E_WORKSPACE
+
+
+def test_triad_sum_full_size_properties(hip, torch_cuda):
+    """n = 2^28 (the benchmark size): properties that need no CPU pass.
+    b = c = 1 -> every a is exactly 4 and the sum is exactly 4n; linearity in s."""
+    torch = torch_cuda
+    n = 1 << 28
+    b = torch.ones(n, device="cuda")
+    c = torch.ones(n, device="cuda")
+    a, total = hip.triad_sum(b, c, 3.0)
+    assert float(total.item()) == 4.0 * n
+    assert bool((a == 4.0).all())
+    a2, total2 = hip.triad_sum(b, c, 0.0, out=a)
+    assert float(total2.item()) == float(n)
+    # pseudo-random input: compare the fused sum with a float64 device sum of a
+    torch.manual_seed(7)
+    b.uniform_(0, 1)
+    c.uniform_(0, 1)
+    a, total = hip.triad_sum(b, c, 3.0, out=a)
+    ref = float(a.double().sum().item())
+    assert abs(float(total.item()) - ref) <= 1e-5 * ref
+    want = (b.double() + c.double() * 3.0).float()
+    assert torch.equal(a, want)
+
+
+@pytest.mark.parametrize("n", [1, 255, 256, 257, 1000, 65536, 1000003])
+def test_reduce_sum_block256(hip, oracle, torch_cuda, n):
+    torch = torch_cuda
+    ones = torch.ones(n, device="cuda")
+    p = hip.reduce_sum_block256(ones)
+    assert p.numel() == (n + 255) // 256
+    assert float(hip.fold_partials(p).item()) == float(n)  # bench_reduction.ml:110-111
+    x = oracle.fill_uniform(n, seed=0x5)
+    p = hip.reduce_sum_block256(dev(torch, x)).cpu().numpy()
+    p_ref = oracle.reduce_sum_block256(x)
+    assert np.allclose(p, p_ref, rtol=1e-5, atol=1e-6)
+    got = float(hip.fold_partials(dev(torch, p)).item())
+    assert abs(got - oracle.fold_partials(p_ref)) <= 1e-5 * oracle.fold_partials(p_ref)
+
+
+@pytest.mark.parametrize("n", [1, 256, 1000, 100000])
+def test_dot_block256(hip, oracle, torch_cuda, n):
+    torch = torch_cuda
+    a = ((np.arange(n) % 100) / 100.0).astype(np.float32)
+    b = (((np.arange(n) + 1) % 100) / 100.0).astype(np.float32)
+    p = hip.dot_block256(dev(torch, a), dev(torch, b)).cpu().numpy()
+    p_ref = oracle.dot_block256(a, b)
+    assert np.allclose(p, p_ref, rtol=1e-5, atol=1e-6)
+    expected = oracle.fold_partials(p_ref)
+    assert abs(float(p.astype(np.float64).sum()) - expected) <= 1e-3 * max(expected, 1e-30)
+
+
+def test_casts_bit_exact(hip, oracle, torch_cuda):
+    torch = torch_cuda
+    rng = np.random.default_rng(11)
+    x = (rng.standard_normal(100003) * np.exp(rng.uniform(-30, 12, 100003))).astype(np.float32)
+    x[:6] = [0.0, -0.0, 65504.0, 65520.0, 2.0 ** -24, 2.0 ** -25]
+    d = dev(torch, x)
+    assert np.array_equal(hip.cast_bf16(d).view(torch.int16).cpu().numpy().view(np.uint16),
+                          oracle.bf16_bits(x))
+    assert np.array_equal(hip.cast_f16(d).view(torch.int16).cpu().numpy().view(np.uint16),
+                          oracle.f16_bits(x))

@@ -1,0 +1,248 @@
+"""Pins the CPU oracle (oracle/sarek_native_oracle.c) without running the reference.
+
+Each check is chosen so that a plausible mistake in the restatement (a transposed
+operand, k order reversed, a missing rounding step, f32 instead of double
+accumulation, wrong tree order) fails at least one of them.  Known answers come from
+the reference's own deterministic inputs and tolerances:
+  benchmarks/bench_matrix_mul_tiled.ml:43-52,109-112,194  (inputs, double loop, 1e-3)
+  benchmarks/bench_stream_triad.ml:44-49,122              (inputs, 1e-5)
+  benchmarks/descriptions/stream_triad.md:143-148         (2 + 1*3 = 5)
+  benchmarks/bench_reduction.ml:110-111,154-163           (all ones -> n, 1e-3 rel)
+  sarek/tests/e2e/test_reduce.ml:54-58,386-389            (tol max(1, 1e-4*expected))
+  benchmarks/bench_dot_product.ml                         (inputs, 1e-3 rel)
+"""
+import numpy as np
+import pytest
+
+
+def ref_inputs_matmul(m, n, k):
+    a = (np.arange(m * k) % 10) / 10.0
+    b = ((np.arange(k * n) + 1) % 10) / 10.0
+    return a.reshape(m, k), b.reshape(k, n)
+
+
+def python_double_loop(a, b):
+    """ocaml_matmul of the reference bench: sequential double accumulation."""
+    m, k = a.shape
+    n = b.shape[1]
+    c = np.zeros((m, n))
+    for r in range(m):
+        for cc in range(n):
+            s = 0.0
+            for i in range(k):
+                s = s + a[r, i] * b[i, cc]
+            c[r, cc] = s
+    return c
+
+
+def test_gemm_reference_inputs_match_double_loop(oracle):
+    m, n, k = 24, 20, 37
+    a64, b64 = ref_inputs_matmul(m, n, k)
+    a32, b32 = a64.astype(np.float32), b64.astype(np.float32)
+    got = oracle.gemm(a32, b32)
+    # the bench's expected values use the unrounded double inputs; its tolerance is 1e-3
+    assert np.abs(got - python_double_loop(a64, b64)).max() <= 1e-3
+    # exact statement: double loop over the f32-rounded inputs, one rounding at the store
+    want = python_double_loop(a32.astype(np.float64), b32.astype(np.float64)).astype(np.float32)
+    assert np.array_equal(got, want)
+
+
+def test_gemm_sequential_k_order_is_what_is_restated(oracle):
+    # values whose double sum depends on the order: increasing k must be used
+    rng = np.random.default_rng(1)
+    k = 4096
+    a = (rng.standard_normal((1, k)) * 10.0 ** rng.integers(-6, 6, (1, k))).astype(np.float32)
+    b = (rng.standard_normal((k, 1)) * 10.0 ** rng.integers(-6, 6, (k, 1))).astype(np.float32)
+    fwd = 0.0
+    for i in range(k):
+        fwd = fwd + float(a[0, i]) * float(b[i, 0])
+    rev = 0.0
+    for i in reversed(range(k)):
+        rev = rev + float(a[0, i]) * float(b[i, 0])
+    got = oracle.gemm(a, b)[0, 0]
+    assert got == np.float32(fwd)
+    # sanity of the test itself: the order matters at double precision for these inputs
+    assert fwd != rev
+
+
+def test_gemm_not_transposed_and_nonsquare(oracle):
+    rng = np.random.default_rng(2)
+    a = rng.uniform(-1, 1, (7, 13)).astype(np.float32)
+    b = rng.uniform(-1, 1, (13, 5)).astype(np.float32)
+    want = (a.astype(np.float64) @ b.astype(np.float64))
+    got = oracle.gemm(a, b)
+    assert got.shape == (7, 5)
+    assert np.abs(got - want).max() <= 1e-6
+    e = np.zeros((13, 5), np.float32)
+    e[3, 2] = 1.0  # picks column 3 of A into column 2 of C
+    assert np.array_equal(oracle.gemm(a, e)[:, 2], a[:, 3])
+
+
+def test_gemm_double_accumulation_not_f32(oracle):
+    # 1 + 2^-30 * 4096 terms: lost entirely in f32 accumulation, kept in double
+    k = 4097
+    a = np.full((1, k), 2.0 ** -15, np.float32)
+    b = np.full((k, 1), 2.0 ** -15, np.float32)
+    a[0, 0] = 1.0
+    b[0, 0] = 1.0
+    want = np.float32(1.0 + 4096 * 2.0 ** -30)
+    assert want != np.float32(1.0)
+    assert oracle.gemm(a, b)[0, 0] == want
+
+
+@pytest.mark.parametrize("m,n,k", [(16, 16, 16), (17, 33, 19), (1, 1, 1), (5, 40, 48), (32, 15, 1)])
+def test_tiled_bsp_restatement_equals_closed_form(oracle, m, n, k):
+    """Zero-padded 16x16 tiles + supersteps give exactly the plain product."""
+    rng = np.random.default_rng(m * 1000 + n * 10 + k)
+    a = rng.uniform(-1, 1, (m, k)).astype(np.float32)
+    b = rng.uniform(-1, 1, (k, n)).astype(np.float32)
+    assert np.array_equal(oracle.matmul_tiled_bsp(a, b), oracle.gemm(a, b))
+
+
+def test_gemm_rows_subset(oracle):
+    rng = np.random.default_rng(3)
+    a = rng.uniform(-1, 1, (50, 64)).astype(np.float32)
+    b = rng.uniform(-1, 1, (64, 30)).astype(np.float32)
+    rows = np.array([49, 0, 17], np.int32)
+    assert np.array_equal(oracle.gemm_rows(a, b, rows), oracle.gemm(a, b)[rows])
+
+
+def test_gemm_thread_count_does_not_change_result(oracle):
+    rng = np.random.default_rng(4)
+    a = rng.uniform(-1, 1, (33, 100)).astype(np.float32)
+    b = rng.uniform(-1, 1, (100, 21)).astype(np.float32)
+    assert np.array_equal(oracle.gemm(a, b, threads=1), oracle.gemm(a, b, threads=7))
+
+
+def test_triad_reference_inputs(oracle):
+    n = 1000
+    b = ((np.arange(n) % 100) / 100.0).astype(np.float32)
+    c = (((np.arange(n) + 1) % 100) / 100.0).astype(np.float32)
+    got = oracle.triad(b, c, 3.0)
+    expected = (np.arange(n) % 100) / 100.0 + ((np.arange(n) + 1) % 100) / 100.0 * 3.0
+    assert np.abs(got - expected).max() <= 1e-5
+    # exact: double arithmetic on the f32 inputs, one rounding
+    assert np.array_equal(got, (b.astype(np.float64) + c.astype(np.float64) * 3.0).astype(np.float32))
+    assert oracle.triad(np.float32([2.0]), np.float32([1.0]), 3.0)[0] == np.float32(5.0)
+
+
+def test_triad_is_single_rounding_not_two(oracle):
+    # c*s rounded to f32 first would lose the low bits: 1 + 2^-24 * 3
+    b = np.float32([1.0])
+    c = np.float32([1.0 + 2.0 ** -23])
+    s = 3.0
+    two_roundings = np.float32(np.float32(c[0] * np.float32(s)) + b[0])
+    one_rounding = np.float32(float(b[0]) + float(c[0]) * s)
+    got = oracle.triad(b, c, s)[0]
+    assert got == one_rounding
+    # operands are not swapped: b + c*s, not c + b*s
+    assert oracle.triad(np.float32([10.0]), np.float32([1.0]), 3.0)[0] == np.float32(13.0)
+    del two_roundings
+
+
+@pytest.mark.parametrize("n", [1, 255, 256, 257, 1000, 4096, 100000])
+def test_reduce_all_ones_is_exactly_n(oracle, n):
+    p = oracle.reduce_sum_block256(np.ones(n, np.float32))
+    assert p.size == (n + 255) // 256
+    assert oracle.fold_partials(p) == float(n)
+    # full blocks hold 256, the ragged last block holds the remainder
+    assert all(p[:-1] == 256.0)
+    assert p[-1] == (n - 256 * (p.size - 1))
+
+
+def test_reduce_tree_order_and_rounding(oracle):
+    """Brute-force halving tree in Python doubles, partial rounded to f32."""
+    rng = np.random.default_rng(5)
+    n = 700
+    x = (rng.standard_normal(n) * 10.0 ** rng.integers(-4, 8, n)).astype(np.float32)
+    want = []
+    for blk in range((n + 255) // 256):
+        s = [float(x[blk * 256 + t]) if blk * 256 + t < n else 0.0 for t in range(256)]
+        half = 128
+        while half >= 1:
+            for t in range(half):
+                s[t] = s[t] + s[t + half]
+            half //= 2
+        want.append(np.float32(s[0]))
+    got = oracle.reduce_sum_block256(x)
+    assert np.array_equal(got, np.array(want, np.float32))
+    fold = 0.0
+    for v in got:
+        fold = fold + float(v)
+    assert oracle.fold_partials(got) == fold
+
+
+def test_reduce_index_sum_reference_vectors(oracle):
+    # test_reduce.ml inputs: a[i] = i, b[i] = 1 (dot) and the sum tolerance rule
+    n = 4096
+    a = np.arange(n, dtype=np.float32)
+    ones = np.ones(n, np.float32)
+    expected = float(n * (n - 1) // 2)
+    got = oracle.fold_partials(oracle.dot_block256(a, ones))
+    assert abs(got - expected) <= max(1.0, 1e-4 * expected)
+    assert got == expected  # all partials are exact integers below 2^24
+
+
+def test_dot_reference_inputs(oracle):
+    n = 100000
+    a = ((np.arange(n) % 100) / 100.0).astype(np.float32)
+    b = (((np.arange(n) + 1) % 100) / 100.0).astype(np.float32)
+    expected = float(np.sum(((np.arange(n) % 100) / 100.0) * (((np.arange(n) + 1) % 100) / 100.0)))
+    got = oracle.fold_partials(oracle.dot_block256(a, b))
+    assert abs(got - expected) < 1e-3 * expected
+    # product is formed in double (exact), not rounded to f32 before the tree
+    x = np.float32([1.0 + 2.0 ** -12]); y = np.float32([1.0 + 2.0 ** -12])
+    exact = float(x[0]) * float(y[0])
+    assert oracle.dot_block256(x, y)[0] == np.float32(exact)
+
+
+def test_triad_sum_is_the_unfused_pair(oracle):
+    rng = np.random.default_rng(6)
+    n = 3000
+    b = rng.random(n, dtype=np.float32)
+    c = rng.random(n, dtype=np.float32)
+    a, partials, total = oracle.triad_sum(b, c, 3.0)
+    assert np.array_equal(a, oracle.triad(b, c, 3.0))
+    assert np.array_equal(partials, oracle.reduce_sum_block256(a))
+    assert total == oracle.fold_partials(partials)
+    assert abs(total - float(np.sum(a.astype(np.float64)))) <= 1e-6 * total
+
+
+def test_rounding_to_bf16_and_f16_match_library_casts(oracle):
+    import torch
+    rng = np.random.default_rng(7)
+    x = (rng.standard_normal(200000) * np.exp(rng.uniform(-30, 12, 200000))).astype(np.float32)
+    x[:8] = [0.0, -0.0, 65504.0, 65519.0, 65520.0, 2.0 ** -24, 2.0 ** -25, 3 * 2.0 ** -25]
+    with np.errstate(over="ignore"):
+        assert np.array_equal(oracle.f16_bits(x), x.astype(np.float16).view(np.uint16))
+    t = torch.from_numpy(x)
+    assert torch.equal(torch.from_numpy(oracle.round_bf16(x)), t.bfloat16().float())
+    assert np.array_equal(oracle.bf16_bits(x), t.bfloat16().view(torch.int16).numpy().view(np.uint16))
+    assert torch.equal(torch.from_numpy(oracle.round_f16(x[np.abs(x) < 6e4])),
+                       t[t.abs() < 6e4].half().float())
+
+
+def test_epilogue_definition(oracle):
+    """relu(A.B + bias) and its row sums, against numpy float64 (no reference counterpart)."""
+    rng = np.random.default_rng(8)
+    a = oracle.round_f16(rng.normal(0, 0.02, (9, 64)).astype(np.float32))
+    b = oracle.round_f16(rng.normal(0, 0.02, (64, 24)).astype(np.float32))
+    bias = rng.uniform(-0.1, 0.1, 24).astype(np.float32)
+    y, rs = oracle.gemm_bias_relu_rowsum(a, b, bias)
+    want = np.maximum(a.astype(np.float64) @ b.astype(np.float64) + bias.astype(np.float64), 0.0)
+    assert np.abs(y - want).max() <= 1e-7
+    assert (y >= 0).all() and (y == 0).any() and (y > 0).any()
+    assert np.abs(rs - want.sum(axis=1)).max() <= 1e-6
+    rows = np.array([8, 2], np.int32)
+    y2, rs2 = oracle.gemm_bias_relu_rowsum(a, b, bias, rows=rows)
+    assert np.array_equal(y2, y[rows]) and np.array_equal(rs2, rs[rows])
+
+
+def test_fill_uniform_is_counter_based_and_in_range(oracle):
+    x = oracle.fill_uniform(100000, seed=0xB, lo=0.0, hi=1.0)
+    assert x.min() >= 0.0 and x.max() < 1.0
+    assert abs(float(x.mean()) - 0.5) < 0.01
+    assert np.array_equal(x, oracle.fill_uniform(100000, seed=0xB, threads=3))
+    assert not np.array_equal(x, oracle.fill_uniform(100000, seed=0xC))
+    y = oracle.fill_uniform(1000, seed=0xA11CE, lo=-1.0, hi=1.0)
+    assert y.min() >= -1.0 and y.max() < 1.0
