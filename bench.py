@@ -1,0 +1,241 @@
+#!/usr/bin/env python3
+"""Benchmark of the sarek-hip hot path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload NAME] [--no-also]
+
+Prints ONE JSON line.  A "step" is one pass of the workload's hot-path entry point over
+one batch of synthetic input that is already resident in HBM.  The headline workload is
+the bf16-in / f32-accumulate 8192^3 GEMM; the other configurations of the hot path
+(fused triad+sum n=2^28, f32 GEMM 8192^3 and 1024^3, fp16 fused-epilogue GEMM) are
+measured the same way and reported under "also", each with its own roofline object.
+
+Timing mirrors the reference's benches (warmup, then timed iterations with the device
+synchronised; benchmarks/bench_stream_triad.ml:76-116) with one difference: the K timed
+steps are bracketed by one synchronise on each side, and the kernel time used for the
+roofline comes from HIP events recorded on the launch stream.
+"""
+import argparse
+import ctypes as C
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+PEAK_HBM_GBS = 8000.0          # MI355X HBM3E
+PEAK_MFMA_TFLOPS = {"bf16": 2500.0, "f16": 2500.0, "f32": 157.3}
+
+
+def parse():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--workload", default="gemm_bf16_8192",
+                    choices=["gemm_bf16_8192", "triad_sum_2p28", "gemm_f32_8192", "gemm_f32_1024",
+                             "gemm_f16_epilogue"])
+    ap.add_argument("--no-also", action="store_true", help="measure only the headline workload")
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    return ap.parse_args()
+
+
+class Events:
+    """HIP events of the library, recorded on the stream the kernels are launched on."""
+
+    def __init__(self, hip, stream):
+        self.hip, self.stream = hip, stream
+        self.e0, self.e1 = C.c_void_p(), C.c_void_p()
+        hip.check(hip.lib.sarek_hip_event_create(C.byref(self.e0)))
+        hip.check(hip.lib.sarek_hip_event_create(C.byref(self.e1)))
+
+    def start(self):
+        self.hip.check(self.hip.lib.sarek_hip_event_record(self.e0, self.stream))
+
+    def stop_ms(self):
+        self.hip.check(self.hip.lib.sarek_hip_event_record(self.e1, self.stream))
+        self.hip.check(self.hip.lib.sarek_hip_event_synchronize(self.e1))
+        ms = C.c_float(0)
+        self.hip.check(self.hip.lib.sarek_hip_event_elapsed_ms(self.e0, self.e1, C.byref(ms)))
+        return float(ms.value)
+
+
+def make_workload(name, torch, hip):
+    """Returns (step_fn, info) with inputs resident on the GPU."""
+    g = torch.Generator(device="cuda")
+    if name == "triad_sum_2p28":
+        n = 1 << 28
+        g.manual_seed(0xB)
+        b = torch.rand(n, device="cuda", generator=g)
+        g.manual_seed(0xC)
+        c = torch.rand(n, device="cuda", generator=g)
+        a = torch.empty_like(b)
+        ws = hip.triad_sum_workspace(n)
+        info = dict(metric="fused triad+sum GB/s", unit="GB/s", dtype="f32",
+                    work=12.0 * n, work_unit=1e9, bound="hbm", peak=PEAK_HBM_GBS,
+                    kernel="triad_kernel<true>",
+                    config={"workload": "fused stream triad + sum, a=b+3c, sum(a)", "n": n,
+                            "algorithmic_bytes": 12 * n})
+        return (lambda: hip.triad_sum(b, c, 3.0, out=a, workspace=ws)), info
+    if name in ("gemm_f32_8192", "gemm_f32_1024"):
+        s = 8192 if name.endswith("8192") else 1024
+        g.manual_seed(0xA11CE)
+        a = torch.rand(s, s, device="cuda", generator=g) * 2 - 1
+        g.manual_seed(0xB0B)
+        b = torch.rand(s, s, device="cuda", generator=g) * 2 - 1
+        c = torch.empty(s, s, device="cuda")
+        info = dict(metric=f"f32 GEMM {s}^3 TFLOP/s", unit="TFLOP/s", dtype="f32",
+                    work=2.0 * s ** 3, work_unit=1e12, bound="mfma", peak=PEAK_MFMA_TFLOPS["f32"],
+                    kernel="gemm_f32_kernel",
+                    config={"workload": f"f32 GEMM C=A.B row-major, U[-1,1)", "m": s, "n": s, "k": s})
+        return (lambda: hip.gemm_f32(a, b, out=c)), info
+    if name == "gemm_bf16_8192":
+        s = 8192
+        g.manual_seed(0xA4)
+        a = (torch.randn(s, s, device="cuda", generator=g) * 0.02).bfloat16()
+        g.manual_seed(0xB4)
+        b = (torch.randn(s, s, device="cuda", generator=g) * 0.02).bfloat16()
+        c = torch.empty(s, s, device="cuda")
+        info = dict(metric="GEMM TFLOP/s at 8192^3 (bf16-in, f32-accumulate)", unit="TFLOP/s",
+                    dtype="bf16", work=2.0 * s ** 3, work_unit=1e12, bound="mfma",
+                    peak=PEAK_MFMA_TFLOPS["bf16"], kernel="gemm16_kernel<bf16>",
+                    config={"workload": "bf16-in f32-acc GEMM C=A.B row-major, N(0,0.02)",
+                            "m": s, "n": s, "k": s})
+        return (lambda: hip.gemm_bf16(a, b, out=c)), info
+    if name == "gemm_f16_epilogue":
+        m, n, k = 4095, 11008, 4096
+        g.manual_seed(0xA5)
+        a = (torch.randn(m, k, device="cuda", generator=g) * 0.02).half()
+        g.manual_seed(0xB5)
+        b = (torch.randn(k, n, device="cuda", generator=g) * 0.02).half()
+        bias = torch.rand(n, device="cuda", generator=g) * 0.2 - 0.1
+        y = torch.empty(m, n, device="cuda")
+        rs = torch.empty(m, device="cuda")
+        info = dict(metric="fp16 GEMM + bias + ReLU + row-sum TFLOP/s", unit="TFLOP/s", dtype="f16",
+                    work=2.0 * m * n * k, work_unit=1e12, bound="mfma",
+                    peak=PEAK_MFMA_TFLOPS["f16"], kernel="gemm16_kernel<f16, bias_relu_rowsum>",
+                    config={"workload": "fp16-in f32-acc Y=relu(A.B+bias), rowsum(Y)",
+                            "m": m, "n": n, "k": k})
+        return (lambda: hip.gemm_f16_bias_relu_rowsum(a, b, bias, out=y, rowsum=rs)), info
+    raise ValueError(name)
+
+
+def measure(name, torch, hip, steps, warmup):
+    step, info = make_workload(name, torch, hip)
+    stream = C.c_void_p(torch.cuda.current_stream().cuda_stream)
+    ev = Events(hip, stream)
+    for _ in range(warmup):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    ev.start()
+    for _ in range(steps):
+        step()
+    gpu_ms = ev.stop_ms()
+    torch.cuda.synchronize()
+    wall_ms = (time.perf_counter() - t0) * 1e3
+    # per-launch kernel time: each step bracketed by its own event pair, median
+    per = []
+    for _ in range(min(steps, 20)):
+        ev.start()
+        step()
+        per.append(ev.stop_ms())
+    per.sort()
+    kernel_ms = per[len(per) // 2]
+    ms_per_step = wall_ms / steps
+    value = info["work"] / (ms_per_step * 1e-3) / info["work_unit"]
+    achieved = info["work"] / (kernel_ms * 1e-3) / info["work_unit"]
+    res = {
+        "metric": info["metric"], "value": round(value, 2), "unit": info["unit"],
+        "ms_per_step": round(ms_per_step, 5), "gpu_ms_per_step_events": round(gpu_ms / steps, 5),
+        "dtype": info["dtype"], "config": info["config"],
+        "roofline": {"bound": info["bound"], "achieved": round(achieved, 2), "peak": info["peak"],
+                     "unit": "GB/s" if info["bound"] == "hbm" else "TFLOP/s",
+                     "frac": round(achieved / info["peak"], 4), "traffic": None,
+                     "kernel": info["kernel"], "kernel_ms": round(kernel_ms, 5)},
+    }
+    return res
+
+
+def cpu_baseline(name):
+    """The CPU oracle (a C restatement of the reference's Native backend arithmetic) timed
+    on this host's cores on a bounded sample of the same workload."""
+    import numpy as np
+
+    import oracle
+    cores = os.cpu_count() or 1
+    cores = min(cores, 16) if "GRAFT_REPO_ROOT" in os.environ else cores
+    rng = np.random.default_rng(0)
+    if name == "triad_sum_2p28":
+        n = 1 << 26
+        b = rng.random(n, dtype=np.float32)
+        c = rng.random(n, dtype=np.float32)
+        oracle.triad_sum(b[:1 << 20], c[:1 << 20], 3.0, threads=cores)
+        t0 = time.perf_counter()
+        oracle.triad_sum(b, c, 3.0, threads=cores)
+        dt = time.perf_counter() - t0
+        return {"value": round(12.0 * n / dt / 1e9, 2), "unit": "GB/s", "cores": cores, "kind": "port",
+                "sample": f"n=2^26 of 2^28 elements, one pass (triad, block-256 tree sum, double fold), {dt:.2f} s"}
+    if name == "gemm_f16_epilogue":
+        rows, n, k = 256, 11008, 4096
+    elif name == "gemm_f32_1024":
+        rows, n, k = 1024, 1024, 1024
+    else:
+        rows, n, k = 256, 8192, 8192
+    a = rng.normal(0, 0.02, (rows, k)).astype(np.float32)
+    b = rng.normal(0, 0.02, (k, n)).astype(np.float32)
+    idx = np.arange(rows, dtype=np.int32)
+    oracle.gemm_rows(a[:8], b, idx[:8], threads=cores)
+    t0 = time.perf_counter()
+    oracle.gemm_rows(a, b, idx, threads=cores)
+    dt = time.perf_counter() - t0
+    return {"value": round(2.0 * rows * n * k / dt / 1e12, 4), "unit": "TFLOP/s", "cores": cores,
+            "kind": "port",
+            "sample": f"{rows} of the output rows (n={n}, k={k}), double accumulation in k order, {dt:.2f} s"}
+
+
+def main():
+    args = parse()
+    if args.gpus != 1:
+        print("bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1)",
+              file=sys.stderr)
+        sys.exit(2)
+    import torch
+    from spoc_amd import hip
+    if not torch.cuda.is_available():
+        print("bench.py needs a GPU", file=sys.stderr)
+        sys.exit(2)
+    torch.cuda.set_device(0)
+
+    head = measure(args.workload, torch, hip, args.steps, args.warmup)
+    out = {
+        "metric": head["metric"], "value": head["value"], "unit": head["unit"], "n_gpus": 1,
+        "steps": args.steps, "warmup": args.warmup, "ms_per_step": head["ms_per_step"],
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": head["dtype"],
+        "data": "synthetic", "config": head["config"], "roofline": head["roofline"],
+        "gpu_ms_per_step_events": head["gpu_ms_per_step_events"],
+    }
+    if not args.no_cpu_baseline:
+        out["cpu_baseline"] = cpu_baseline(args.workload)
+    if not args.no_also:
+        also = []
+        for name in ["triad_sum_2p28", "gemm_f32_8192", "gemm_f16_epilogue", "gemm_f32_1024",
+                     "gemm_bf16_8192"]:
+            if name == args.workload:
+                continue
+            torch.cuda.empty_cache()
+            r = measure(name, torch, hip, args.steps, args.warmup)
+            if not args.no_cpu_baseline and name == "triad_sum_2p28":
+                r["cpu_baseline"] = cpu_baseline(name)
+            also.append(r)
+        out["also"] = also
+    info = hip.device_info(0)
+    out["device"] = {"name": info.name.decode(), "arch": info.gcn_arch.decode(),
+                     "cus": info.multiprocessor_count, "clock_mhz": info.clock_rate_khz // 1000}
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()

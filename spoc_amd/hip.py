@@ -116,6 +116,11 @@ def _load():
         raise ImportError(
             f"{LIB_PATH} is not built: run `python -c 'import __graft_entry__ as g; g.build()'` "
             "(or `make -C spoc_amd/csrc`).  There is no CPU fallback.")
+    # One HIP runtime per process: the torch wheel ships its own libamdhip64 /
+    # libhsa-runtime64 and loads them by path, so if this library pulled in the system
+    # copies first the process would hold two runtimes and the second sees no device.
+    # Loading torch first makes both sides share torch's copy (same sonames).
+    import torch  # noqa: F401
     lib = C.CDLL(LIB_PATH)
     for name, (res, args) in SYMBOLS.items():
         fn = getattr(lib, name)  # AttributeError if the library lacks a declared symbol
