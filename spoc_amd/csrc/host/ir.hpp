@@ -145,10 +145,7 @@ std::string generate(const Kernel &k);   // records + variants + helpers + kerne
 
 // specialise.cpp: "" or the tag of the hand-written kernel that computes the same thing
 std::string recognise(const Kernel &k);
-
-// fusion.cpp: map -> reduce fusion (Sarek_fusion.fuse_reduction)
-bool can_fuse_reduction(const Kernel &producer, const Kernel &consumer, const std::string &array);
-Kernel fuse_reduction(const Kernel &producer, const Kernel &consumer, const std::string &array);
+std::string canonical_form(const Kernel &k);   // the normal form recognise() compares
 
 }  // namespace ir
 }  // namespace sarek_hip

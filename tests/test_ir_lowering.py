@@ -1,0 +1,238 @@
+"""IR -> HIP lowering and hot-kernel recognition (host logic; no GPU needed).
+
+Golden parity: for the reference's benchmark kernels the HIP text must equal the text the
+reference's own lowering produces for CUDA-dialect targets, which its CI keeps in
+benchmarks/descriptions/generated/*_generated.md (fixtures: tests/golden/generated/).
+Unit cases mirror sarek-cuda/test/test_sarek_ir_cuda.ml:27-251 with HIP spellings.
+"""
+import ctypes as C
+import glob
+import os
+
+import pytest
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+IR_DIR = os.path.join(HERE, "golden", "ir")
+GEN_DIR = os.path.join(HERE, "golden", "generated")
+MARK = "// sarek-hip-specialise: "
+
+KERNELS = sorted(os.path.basename(p)[:-3] for p in glob.glob(os.path.join(IR_DIR, "*.ir")))
+EXPECTED_TAGS = {
+    "matrix_mul_tiled": "matmul_tiled_f32", "stream_triad": "stream_triad_f32",
+    "reduction": "reduce_sum_block256_f32", "dot_product": "dot_block256_f32",
+}
+
+
+def split_tag(src):
+    if src.startswith(MARK):
+        first, rest = src.split("\n", 1)
+        return first[len(MARK):], rest
+    return "", src
+
+
+def kernel_with_body(body, params=""):
+    return f"(kernel sarek_kern (params {params}) (locals) (body {body}) (native_fn true))"
+
+
+def body_text(hip, stmt, params=""):
+    """Lowered text of one statement, without the kernel wrapper."""
+    src = hip.generate_source(kernel_with_body(stmt, params))
+    tag, src = split_tag(src)
+    start = src.index(") {\n") + 4
+    end = src.rindex("}\n}\n")
+    return src[start:end]
+
+
+def expr_text(hip, expr):
+    out = body_text(hip, f"(expr {expr})")
+    assert out.startswith("  ") and out.endswith(";\n")
+    return out[2:-2]
+
+
+def test_fixture_list():
+    assert set(EXPECTED_TAGS) <= set(KERNELS) and len(KERNELS) >= 10
+
+
+@pytest.mark.parametrize("name", KERNELS)
+def test_lowering_reproduces_golden_text(hip, name):
+    ir = open(os.path.join(IR_DIR, name + ".ir")).read()
+    expected = open(os.path.join(GEN_DIR, name + ".cuda.txt")).read()
+    tag, src = split_tag(hip.generate_source(ir, block=(256, 1, 1)))
+    assert src == expected
+    assert tag == EXPECTED_TAGS.get(name, "")
+
+
+def test_literals(hip):
+    assert expr_text(hip, "(i32 42)") == "42"
+    assert expr_text(hip, "(i64 42)") == "42LL"
+    assert "." in expr_text(hip, "(f64 3.14)")
+    assert expr_text(hip, "(bool true)") == "1"
+    assert expr_text(hip, "(bool false)") == "0"
+    assert expr_text(hip, "(f32 0.0)") == "0.0f"
+    assert expr_text(hip, "(f32 2.5)") == "2.5f"
+    assert expr_text(hip, "(f32 0.1)") == "0.10000000000000001f"   # "%.17g" + f
+    assert expr_text(hip, "(f32 1e30)") == "1e+30f"
+
+
+def test_operations(hip):
+    assert expr_text(hip, "(var x 1 i32)") == "x"
+    assert expr_text(hip, "(add (i32 1) (i32 2))") == "(1 + 2)"
+    assert expr_text(hip, "(mul (var x 1 i32) (i32 3))") == "(x * 3)"
+    assert expr_text(hip, "(neg (var x 1 i32))") == "(-x)"
+    assert expr_text(hip, "(shl (var x 1 i32) (i32 2))") == "(x << 2)"
+    assert expr_text(hip, "(if (lt (var x 1 i32) (i32 0)) (i32 1) (i32 2))") == "((x < 0) ? 1 : 2)"
+    assert expr_text(hip, "(cast f32 (var x 1 i32))") == "(float)x"
+    assert expr_text(hip, "(len v)") == "sarek_v_length"
+    assert expr_text(hip, "(read v (var x 1 i32))") == "v[x]"
+
+
+def test_statements(hip):
+    assert body_text(hip, "(empty)") == ""
+    assert body_text(hip, "(seq (empty) (empty))") == ""
+    out = body_text(hip, "(assign (lvar (var result 1 i32 mut)) (i32 42))")
+    assert out == "  result = 42;\n"
+    out = body_text(hip, "(if (bool true) (empty))")
+    assert out == "  if (1) {\n  }\n"
+    out = body_text(hip, "(if (bool true) (empty) (empty))")
+    assert "} else {" in out
+    out = body_text(hip, "(while (lt (var i 1 i32) (i32 10)) (empty))")
+    assert out.startswith("  while ((i < 10)) {")
+    up = body_text(hip, "(for (var i 1 i32 mut) (i32 0) (i32 9) upto (empty))")
+    assert up == "  for (int i = 0; i <= 9; i++) {\n  }\n"          # inclusive bound
+    down = body_text(hip, "(for (var i 1 i32 mut) (i32 9) (i32 0) downto (empty))")
+    assert down == "  for (int i = 9; i >= 0; i--) {\n  }\n"
+    assert body_text(hip, "(let (var x 1 i32) (i32 42) (empty))") == "  int x = 42;\n"
+    assert "double y = 3.14" in body_text(hip, "(letmut (var y 1 f64 mut) (f64 3.14) (empty))")
+    assert body_text(hip, "(block (empty))") == "  {\n  }\n"
+    assert body_text(hip, "(pragma (unroll) (empty))") == "  #pragma unroll\n"
+    assert body_text(hip, '(native "asm volatile(\\"\\");")') == '  asm volatile("");\n'
+
+
+def test_barriers_use_hip_spellings(hip):
+    assert body_text(hip, "(barrier)") == "  __syncthreads();\n"
+    assert body_text(hip, "(memfence)") == "  __threadfence();\n"
+    warp = body_text(hip, "(warpbarrier)")
+    assert "__syncwarp" not in warp and "__builtin_amdgcn_wave_barrier()" in warp
+
+
+def test_intrinsics(hip):
+    assert expr_text(hip, "(intr (Gpu) thread_idx_x)") == "threadIdx.x"
+    assert expr_text(hip, "(intr (Gpu) block_dim_y)") == "blockDim.y"
+    assert expr_text(hip, "(intr (Std) global_thread_id)") == "(threadIdx.x + blockIdx.x * blockDim.x)"
+    assert expr_text(hip, "(intr (Std) global_size)") == "(blockDim.x * gridDim.x)"
+    assert expr_text(hip, "(intr (Float32) sqrt (var x 1 f32))") == "sqrt(x)"
+    assert expr_text(hip, "(intr (Float32) of_int (var x 1 i32))") == "(float)(x)"
+    assert expr_text(hip, "(intr (Float32) add (var x 1 f32) (var y 2 f32))") == "(x + y)"
+    # template resolved by the caller's registry wins over the built-in table
+    assert expr_text(hip, '(intr (My) twice (template "(2 * %s)") (var x 1 i32))') == "(2 * x)"
+    assert expr_text(hip, '(intr (My) f (template "my_f") (var x 1 i32) (i32 1))') == "my_f(x, 1)"
+    assert expr_text(hip, "(intr (Mod Sub) unknown_fn (i32 1))") == "Mod.Sub.unknown_fn(1)"
+    assert expr_text(hip, "(intr (Gpu) atomic_add (read h (i32 0)) (i32 1))") == "atomicAdd(&h[0], 1)"
+    assert expr_text(hip, "(intr (Gpu) atomic_add (var h 1 (vec i32)) (i32 3) (i32 1))") == "atomicAdd(&h[3], 1)"
+
+
+def test_vector_params_get_length_arguments(hip):
+    src = hip.generate_source(kernel_with_body(
+        "(empty)", "(param (var v 1 (vec f64))) (param (var k 2 i64)) (param (var flag 3 bool))"))
+    assert "__global__ void sarek_kern(double* __restrict__ v, int sarek_v_length, long long k, int flag) {" in src
+    assert src.startswith('\nextern "C" {\n') and src.endswith("}\n}\n")
+
+
+def test_records_variants_and_helpers(hip):
+    ir = """
+    (kernel k (params (param (var ps 1 (vec (record Geo.point (x f32) (y f32))))))
+      (locals (shared tile f32 (i32 64)) (local (var acc 2 f32 mut) (f32 0.0)))
+      (body (match (var s 3 (variant shape (Circle f32) (Rect f32 f32) (Empty)))
+              (case (Circle r) (assign (lvar (var acc 2 f32 mut)) (var r 4 f32)))
+              (case (Rect w h) (assign (lvar (var acc 2 f32 mut)) (mul (var w 5 f32) (var h 6 f32))))
+              (case _ (empty))))
+      (types (Geo.point (x f32) (y f32)))
+      (variants (shape (Circle f32) (Rect f32 f32) (Empty)))
+      (funcs (func sq (params (var a 7 f32)) f32 (return (mul (var a 7 f32) (var a 7 f32)))))
+      (native_fn false))"""
+    src = hip.generate_source(ir)
+    assert "enum { Circle = 0, Rect = 1, Empty = 2 };" in src
+    assert "typedef struct {\n  int tag;\n  union {\n    float Circle_v;\n    struct { float _0; float _1; } Rect_v;\n  } data;\n} shape;" in src
+    assert "__device__ __host__ inline shape make_shape_Rect(float v0, float v1) {" in src
+    assert "typedef struct {\n  float x;\n  float y;\n} Geo_point;" in src
+    assert "__device__ float sq(float a) {\n  return (a * a);\n}" in src
+    assert "Geo_point* __restrict__ ps, int sarek_ps_length" in src
+    assert "  __shared__ float tile[64];\n  float acc = 0.0f;\n" in src
+    assert "switch (s.tag) {" in src and "case Circle: {" in src and "float r = s.data.Circle_v;" in src
+    assert "float w = s.data.Rect_v._0;" in src and "default: {" in src
+
+
+@pytest.mark.parametrize("text,needle", [
+    ("(kernel k (params) (locals) (body (frobnicate)))", "unknown statement form"),
+    ("(kernel k (params) (locals) (body (empty))", "unbalanced"),
+    ("(kernel k (params) (locals))", "without a (body"),
+    ("(kernel k (params (param (var x 1 q8))) (locals) (body (empty)))", "unknown type"),
+])
+def test_parse_errors(hip, text, needle):
+    with pytest.raises(hip.SarekHipError) as e:
+        hip.generate_source(text)
+    assert e.value.status == hip.E_PARSE and needle in e.value.message
+
+
+def test_codegen_error_for_array_creation_outside_let(hip):
+    with pytest.raises(hip.SarekHipError) as e:
+        hip.generate_source(kernel_with_body("(expr (newarray f32 (i32 4) shared))"))
+    assert e.value.status == hip.E_CODEGEN
+
+
+def test_output_buffer_protocol(hip):
+    ir = open(os.path.join(IR_DIR, "stream_triad.ir")).read().encode()
+    needed = C.c_size_t(0)
+    rc = hip.lib.sarek_hip_generate_source(ir, None, None, 0, C.byref(needed))
+    assert rc == hip.E_BUFFER_TOO_SMALL and needed.value > 100
+    buf = C.create_string_buffer(needed.value)
+    assert hip.lib.sarek_hip_generate_source(ir, None, buf, len(buf), C.byref(needed)) == 0
+    assert buf.value.decode().startswith(MARK + "stream_triad_f32\n")
+
+
+# ---- recognition is strict: near misses are NOT taken over --------------------------
+
+def triad_ir(expr):
+    return kernel_with_body(
+        "(let (var tid 6 i32) (intr (Std) global_thread_id) (if (lt (var tid 6 i32) (var n 5 i32)) "
+        f"(assign (lelem a (var tid 6 i32)) {expr})))",
+        "(param (var a 1 (vec f32))) (param (var b 2 (vec f32))) (param (var c 3 (vec f32))) "
+        "(param (var scalar 4 f32)) (param (var n 5 i32))")
+
+
+B, Cc, S = "(read b (var tid 6 i32))", "(read c (var tid 6 i32))", "(var scalar 4 f32)"
+
+
+@pytest.mark.parametrize("expr,tag", [
+    (f"(add {B} (mul {Cc} {S}))", "stream_triad_f32"),
+    (f"(add (mul {S} {Cc}) {B})", "stream_triad_f32"),            # commuted operands: same value
+    (f"(add {Cc} (mul {B} {S}))", ""),                             # b and c swapped: different kernel
+    (f"(sub {B} (mul {Cc} {S}))", ""),
+    (f"(add {B} (mul {Cc} (f32 3.0)))", ""),
+    (f"(add {B} (mul (read c (add (var tid 6 i32) (i32 1))) {S}))", ""),
+])
+def test_triad_recognition_is_exact(hip, expr, tag):
+    assert split_tag(hip.generate_source(triad_ir(expr)))[0] == tag
+
+
+def test_recognition_survives_renaming_and_nesting(hip):
+    ir = open(os.path.join(IR_DIR, "matrix_mul_tiled.ir")).read()
+    renamed = (ir.replace("tile_a", "sh_one").replace("tile_b", "sh_two").replace("sum", "accum")
+               .replace("(block ", "(seq ").replace("thread_idx_", "thread_id_"))
+    assert split_tag(hip.generate_source(renamed))[0] == "matmul_tiled_f32"
+
+
+def test_tiled_matmul_near_misses_fall_back(hip):
+    ir = open(os.path.join(IR_DIR, "matrix_mul_tiled.ir")).read()
+    assert split_tag(hip.generate_source(ir.replace("(i32 16)", "(i32 8)")))[0] == ""
+    # a barrier removed: no longer the same program
+    assert split_tag(hip.generate_source(ir.replace("(barrier)", "(empty)", 1)))[0] == ""
+    # transposed B access
+    swapped = ir.replace("(read b (add (mul (var b_row", "(read b (add (mul (var col", 1)
+    assert split_tag(hip.generate_source(swapped))[0] == ""
+
+
+def test_reduction_with_other_operator_is_not_taken(hip):
+    ir = open(os.path.join(IR_DIR, "reduction.ir")).read()
+    assert split_tag(hip.generate_source(ir.replace("(add (read sdata", "(mul (read sdata", 1)))[0] == ""
+    assert split_tag(hip.generate_source(ir.replace("(i32 64)", "(i32 65)", 1)))[0] == ""
