@@ -20,9 +20,17 @@
 //      n-offset 4*(i%4), and receives column i of that 4 x 16 block (its 4 rows).
 //      Two such reads (rows 0-3 and 4-7 of the lane's k range) give the 8 k values.
 //
-// Global -> LDS goes through registers with 16-byte loads; the next slab's loads are
-// issued before the MFMA work of the current slab and written to the other LDS stage
-// after it (one barrier per slab).
+// Two kernels share this tiling:
+//   gemm16_dma_kernel (K % 64 == 0): global -> LDS by global_load_lds_dwordx4, which
+//     writes the 64 lanes' 16-byte pieces to 1 KiB of consecutive LDS with no register
+//     staging and no ds_write.  Rows cannot be padded that way, so bank conflicts are
+//     avoided by an XOR swizzle applied on the global-address side: LDS 16-byte slot p of
+//     row r holds global chunk p ^ (r & 7) for A (128-byte rows) and p ^ ((r & 3) << 1)
+//     for B (512-byte rows); readers apply the same XOR.  The next slab streams into the
+//     other stage while the MFMAs of the current slab run; operand fragments for k-step
+//     kk+1 are fetched from LDS while the MFMAs of k-step kk issue.
+//   gemm16_staged_kernel (any K % 8 == 0): global -> registers -> LDS with zero fill for
+//     the K tail, rows padded instead of swizzled.
 #include "common.hpp"
 #include "tunables.hpp"
 
@@ -41,6 +49,8 @@ typedef __attribute__((ext_vector_type(2))) unsigned int u32x2;
 
 constexpr int BM = 256, BN = 256, BK = 64;
 constexpr int THREADS = 512;
+constexpr int NUM_XCD = 8;   // XCDs of an MI355X; workgroup ids are dealt to them round-robin
+constexpr int GROUP = 8;     // tile-rows per raster band
 constexpr int A_STRIDE = BK * 2 + 16;   // bytes per A row in LDS (144)
 constexpr int B_STRIDE = BN * 2 + 32;   // bytes per B row in LDS (544)
 constexpr int A_BYTES = BM * A_STRIDE;  // 36864
@@ -73,29 +83,199 @@ __device__ __forceinline__ float half_wave_sum(float v) {
   return v;
 }
 
+// Writes one wave's 128 x 64 accumulator block.  Accumulator layout of the 32x32 MFMA:
+// register r of lane l holds row 8*(r/4) + 4*(l/32) + r%4, column l%32 of its tile.
+template <int Epi>
+__device__ __forceinline__ void epilogue(f32x16 (&acc)[4][2], float *__restrict__ C,
+                                         const float *__restrict__ bias,
+                                         float *__restrict__ rowsum, int M, int N, int row0,
+                                         int col0, int lm, int lh) {
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+      const int row = row0 + i * 32 + 8 * (r >> 2) + 4 * lh + (r & 3);
+      float rs = 0.f;
+#pragma unroll
+      for (int j = 0; j < 2; ++j) {
+        const int col = col0 + j * 32 + lm;
+        float v = acc[i][j][r];
+        if (Epi == EPI_BIAS_RELU_ROWSUM) {
+          v += (col < N) ? bias[col] : 0.f;
+          v = v > 0.f ? v : 0.f;
+          if (col < N) rs += v;
+        }
+        if (row < M && col < N) C[static_cast<int64_t>(row) * N + col] = v;
+      }
+      if (Epi == EPI_BIAS_RELU_ROWSUM) {
+        rs = half_wave_sum(rs);
+        if (lm == 0 && row < M) atomicAdd(rowsum + row, rs);
+      }
+    }
+  }
+}
+
+// Workgroup -> tile.  The hardware deals consecutive workgroup ids round-robin to the
+// 8 XCDs (each with its own L2), so ids are first regrouped to give every XCD one
+// contiguous run of tiles, and the run is walked in bands of GROUP tile-rows, column by
+// column: the ~32 tiles an XCD has in flight then form a compact GROUP x 4 patch that
+// moves through K together and shares A row-panels and B column-panels in that L2.
+__device__ __forceinline__ void tile_of_block(int tiles_m, int tiles_n, int xcd_remap, int &tm,
+                                              int &tn) {
+  const int nblocks = tiles_m * tiles_n;
+  const int xcd = blockIdx.x % NUM_XCD, slot = blockIdx.x / NUM_XCD;
+  int tile = xcd * (nblocks / NUM_XCD) + min(xcd, nblocks % NUM_XCD) + slot;
+  if (xcd_remap == 0) tile = blockIdx.x;
+  const int per_group = GROUP * tiles_n;
+  const int g = tile / per_group;
+  const int rows_in_group = min(GROUP, tiles_m - g * GROUP);
+  const int in_g = tile - g * per_group;
+  tm = g * GROUP + in_g % rows_in_group;
+  tn = in_g / rows_in_group;
+}
+
+// ---- direct-to-LDS kernel ---------------------------------------------------------
+// One static array per stage and operand: distinct objects, so the compiler can tell
+// that the DMA into one stage does not alias the ds_reads of the other and need not
+// wait for it.
+constexpr int DMA_A_BYTES = BM * BK * 2;  // 32768, rows of 128 bytes
+constexpr int DMA_B_BYTES = BK * BN * 2;  // 32768, rows of 512 bytes
+__shared__ __attribute__((aligned(1024))) char dma_a0[DMA_A_BYTES];
+__shared__ __attribute__((aligned(1024))) char dma_b0[DMA_B_BYTES];
+__shared__ __attribute__((aligned(1024))) char dma_a1[DMA_A_BYTES];
+__shared__ __attribute__((aligned(1024))) char dma_b1[DMA_B_BYTES];
+
+typedef const __attribute__((address_space(1))) void *gptr_t;
+
+// 64 lanes x 16 bytes from per-lane global addresses to lds_dst[0..1023].
+__device__ __forceinline__ void dma16(const void *src, char *lds_dst) {
+  __builtin_amdgcn_global_load_lds((gptr_t)src, (LDS_PTR void *)lds_dst, 16, 0, 0);
+}
+
 template <bool Bf16, int Epi>
-__global__ __launch_bounds__(THREADS) void gemm16_kernel(const uint16_t *__restrict__ A,
+__global__ __launch_bounds__(THREADS) void gemm16_dma_kernel(const uint16_t *__restrict__ A,
+                                                             const uint16_t *__restrict__ B,
+                                                             float *__restrict__ C,
+                                                             const float *__restrict__ bias,
+                                                             float *__restrict__ rowsum, int M,
+                                                             int N, int K, int tiles_m,
+                                                             int tiles_n, int xcd_remap) {
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int wm = wave >> 2, wn = wave & 3;
+  const int lm = lane & 31, lh = lane >> 5;
+  int tm, tn;
+  tile_of_block(tiles_m, tiles_n, xcd_remap, tm, tn);
+  const int m0 = tm * BM, n0 = tn * BN;
+
+  // ---- DMA source addresses -----------------------------------------------------
+  // A: wave-instruction q = wave + 8*i (i < 4) fills rows 8q..8q+7; lane l -> row 8q + l/8,
+  //    LDS slot l%8, global chunk (l%8) ^ (l/8)   [(row & 7) == l/8].
+  // B: instruction q fills rows 2q, 2q+1; lane l -> row 2q + l/32, LDS slot l%32,
+  //    global chunk (l%32) ^ ((row & 3) << 1).
+  // Rows past M and columns past N are clamped to valid addresses: what they produce is
+  // never stored.
+  const uint16_t *a_src[4];
+  const uint16_t *b_src[4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int q = wave + 8 * i;
+    const int arow = min(m0 + 8 * q + (lane >> 3), M - 1);
+    a_src[i] = A + static_cast<int64_t>(arow) * K + (((lane & 7) ^ (lane >> 3)) << 3);
+    const int brow = 2 * q + (lane >> 5);
+    const int bchunk = (lane & 31) ^ ((brow & 3) << 1);
+    const int bcol = min(n0 + bchunk * 8, N - 8);
+    b_src[i] = B + static_cast<int64_t>(brow) * N + bcol;
+  }
+  const int64_t b_slab_step = static_cast<int64_t>(BK) * N;  // elements per K slab in B
+
+  f32x16 acc[4][2];
+#pragma unroll
+  for (int i = 0; i < 4; ++i)
+#pragma unroll
+    for (int j = 0; j < 2; ++j)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
+
+  // ---- fragment read offsets ------------------------------------------------------
+  // A: row = wm*128 + i*32 + lm, chunk = 2*kk + lh, slot = chunk ^ (lm & 7).
+  const int a_row_off = (wm * 128 + lm) * 128;
+  // B (transposing read): 16-lane group g16 = lane/16: n half = g16 & 1, k half = lh;
+  // lane li supplies row (li>>2) of its 4-row block and the 8 bytes at n offset 4*(li&3).
+  const int li = lane & 15;
+  const int b_r = li >> 2;                                     // row within the 4-row block
+  const int b_nbyte = (wn * 64 + ((lane >> 4) & 1) * 16) * 2 + (li & 3) * 8;  // + j*64
+
+  auto issue = [&](char *sa, char *sb, int slab) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int q = wave + 8 * i;
+      dma16(a_src[i] + slab * BK, sa + q * 1024);
+      dma16(b_src[i] + slab * b_slab_step, sb + q * 1024);
+    }
+  };
+  auto load_frags = [&](const char *sa, const char *sb, int kk, u32x4 (&af)[4], u32x4 (&bf)[2]) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int slot = (2 * kk + lh) ^ (lm & 7);
+      af[i] = *reinterpret_cast<const u32x4 *>(sa + a_row_off + i * 32 * 128 + slot * 16);
+    }
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+      // rows kk*16 + lh*8 + {0..3} and {4..7}; (row & 3) == b_r in both
+      const int row_lo = kk * 16 + lh * 8 + b_r;
+      const int nbyte = (b_nbyte + j * 64) ^ (b_r << 5);   // XOR on the 32-byte unit bits
+      u32x2 lo = lds_read_tr16(sb, row_lo * 512 + nbyte);
+      u32x2 hi = lds_read_tr16(sb, (row_lo + 4) * 512 + nbyte);
+      bf[j] = u32x4{lo.x, lo.y, hi.x, hi.y};
+    }
+  };
+  auto compute_slab = [&](const char *sa, const char *sb) {
+    u32x4 af[2][4], bf[2][2];
+    load_frags(sa, sb, 0, af[0], bf[0]);
+#pragma unroll
+    for (int kk = 0; kk < BK / 16; ++kk) {
+      const int cur = kk & 1;
+      if (kk + 1 < BK / 16) load_frags(sa, sb, kk + 1, af[cur ^ 1], bf[cur ^ 1]);
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int j = 0; j < 2; ++j) acc[i][j] = mfma<Bf16>(af[cur][i], bf[cur][j], acc[i][j]);
+    }
+  };
+
+  const int nslabs = K / BK;
+  issue(dma_a0, dma_b0, 0);
+  __syncthreads();   // waits for this wave's DMA (vmcnt) and for everyone else's
+  for (int s = 0; s < nslabs; s += 2) {
+    if (s + 1 < nslabs) issue(dma_a1, dma_b1, s + 1);
+    compute_slab(dma_a0, dma_b0);
+    __syncthreads();
+    if (s + 1 < nslabs) {
+      if (s + 2 < nslabs) issue(dma_a0, dma_b0, s + 2);
+      compute_slab(dma_a1, dma_b1);
+      __syncthreads();
+    }
+  }
+  epilogue<Epi>(acc, C, bias, rowsum, M, N, m0 + wm * 128, n0 + wn * 64, lm, lh);
+}
+
+template <bool Bf16, int Epi>
+__global__ __launch_bounds__(THREADS) void gemm16_staged_kernel(const uint16_t *__restrict__ A,
                                                          const uint16_t *__restrict__ B,
                                                          float *__restrict__ C,
                                                          const float *__restrict__ bias,
                                                          float *__restrict__ rowsum, int M, int N,
-                                                         int K, int tiles_m, int tiles_n) {
+                                                         int K, int tiles_m, int tiles_n, int xcd_remap) {
   extern __shared__ __attribute__((aligned(16))) char lds[];
   const int tid = threadIdx.x;
   const int lane = tid & 63, wave = tid >> 6;
   const int wm = wave >> 2, wn = wave & 3;  // 2 x 4 waves
   const int lm = lane & 31, lh = lane >> 5;
 
-  // Tile raster: groups of 8 tile-rows walk the N direction together so the tiles
-  // resident at one time share A row-panels and B column-panels in L2.
-  int tile = blockIdx.x;
-  constexpr int GROUP = 8;
-  const int per_group = GROUP * tiles_n;
-  const int g = tile / per_group;
-  const int rows_in_group = min(GROUP, tiles_m - g * GROUP);
-  const int in_g = tile - g * per_group;
-  const int tm = g * GROUP + in_g % rows_in_group;
-  const int tn = in_g / rows_in_group;
+  int tm, tn;
+  tile_of_block(tiles_m, tiles_n, xcd_remap, tm, tn);
   const int m0 = tm * BM, n0 = tn * BN;
 
   // ---- global -> register staging --------------------------------------------
@@ -186,32 +366,7 @@ __global__ __launch_bounds__(THREADS) void gemm16_kernel(const uint16_t *__restr
     __syncthreads();
   }
 
-  // ---- epilogue ----------------------------------------------------------------
-  // Accumulator layout of the 32x32 MFMA: register r of lane l holds
-  // row 8*(r/4) + 4*(l/32) + r%4, column l%32 of the tile.
-#pragma unroll
-  for (int i = 0; i < 4; ++i) {
-#pragma unroll
-    for (int r = 0; r < 16; ++r) {
-      const int row = m0 + wm * 128 + i * 32 + 8 * (r >> 2) + 4 * lh + (r & 3);
-      float rs = 0.f;
-#pragma unroll
-      for (int j = 0; j < 2; ++j) {
-        const int col = n0 + wn * 64 + j * 32 + lm;
-        float v = acc[i][j][r];
-        if (Epi == EPI_BIAS_RELU_ROWSUM) {
-          v += (col < N) ? bias[col] : 0.f;
-          v = v > 0.f ? v : 0.f;
-          if (col < N) rs += v;
-        }
-        if (row < M && col < N) C[static_cast<int64_t>(row) * N + col] = v;
-      }
-      if (Epi == EPI_BIAS_RELU_ROWSUM) {
-        rs = half_wave_sum(rs);
-        if (lm == 0 && row < M) atomicAdd(rowsum + row, rs);
-      }
-    }
-  }
+  epilogue<Epi>(acc, C, bias, rowsum, M, N, m0 + wm * 128, n0 + wn * 64, lm, lh);
 }
 
 // Any shape, any alignment: one thread per C element, f32 accumulate in k order.
@@ -274,16 +429,22 @@ int launch_gemm16(const uint16_t *a, const uint16_t *b, float *c, const float *b
                       (reinterpret_cast<uintptr_t>(a) % 16 == 0) &&
                       (reinterpret_cast<uintptr_t>(b) % 16 == 0);
   if (vec_ok && tunable("gemm16.force_simple", 0) == 0) {
+    const int tiles_m = (m + BM - 1) / BM, tiles_n = (n + BN - 1) / BN;
+    const int remap = (int)tunable("gemm.xcd_remap", 1);
+    if (k % BK == 0 && tunable("gemm16.force_staged", 0) == 0) {
+      hipLaunchKernelGGL((gemm16_dma_kernel<Bf16, Epi>), dim3(tiles_m * tiles_n), dim3(THREADS), 0, st,
+                         a, b, c, bias, rowsum, m, n, k, tiles_m, tiles_n, remap);
+      return check_launch("gemm16 kernel launch");
+    }
     static bool attr_done[2][2] = {{false, false}, {false, false}};
-    auto kern = gemm16_kernel<Bf16, Epi>;
+    auto kern = gemm16_staged_kernel<Bf16, Epi>;
     if (!attr_done[Bf16][Epi]) {
       SAREK_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
                                         hipFuncAttributeMaxDynamicSharedMemorySize, LDS_BYTES));
       attr_done[Bf16][Epi] = true;
     }
-    const int tiles_m = (m + BM - 1) / BM, tiles_n = (n + BN - 1) / BN;
     hipLaunchKernelGGL(kern, dim3(tiles_m * tiles_n), dim3(THREADS), LDS_BYTES, st, a, b, c, bias,
-                       rowsum, m, n, k, tiles_m, tiles_n);
+                       rowsum, m, n, k, tiles_m, tiles_n, remap);
   } else {
     auto kern = gemm16_simple_kernel<Bf16, Epi>;
     hipLaunchKernelGGL(kern, dim3((n + 63) / 64, (m + 3) / 4), dim3(256), 0, st, a, b, c, bias,

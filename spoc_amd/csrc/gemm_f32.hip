@@ -26,6 +26,8 @@ typedef __attribute__((ext_vector_type(4))) float f32x4;
 
 constexpr int BM = 256, BN = 256, BK = 32;
 constexpr int THREADS = 512;
+constexpr int NUM_XCD = 8;   // XCDs of an MI355X; workgroup ids are dealt to them round-robin
+constexpr int GROUP = 8;     // tile-rows per raster band
 constexpr int A_STRIDE = BK + 4;            // floats per A row in LDS (36)
 constexpr int B_STRIDE = BN;                // floats per B row in LDS
 constexpr int A_FLOATS = BM * A_STRIDE;     // 9216
@@ -36,15 +38,22 @@ constexpr int LDS_BYTES = 2 * STAGE_FLOATS * 4;  // 139264
 __global__ __launch_bounds__(THREADS) void gemm_f32_kernel(const float *__restrict__ A,
                                                            const float *__restrict__ B,
                                                            float *__restrict__ C, int M, int N,
-                                                           int K, int tiles_m, int tiles_n) {
+                                                           int K, int tiles_m, int tiles_n, int xcd_remap) {
   extern __shared__ __attribute__((aligned(16))) float lds_f[];
   const int tid = threadIdx.x;
   const int lane = tid & 63, wave = tid >> 6;
   const int wm = wave >> 2, wn = wave & 3;
   const int lm = lane & 31, lh = lane >> 5;
 
-  int tile = blockIdx.x;
-  constexpr int GROUP = 8;
+  // Workgroup -> tile.  The hardware deals consecutive workgroup ids round-robin to the
+  // 8 XCDs (each with its own L2), so ids are first regrouped to give every XCD one
+  // contiguous run of tiles, and the run is walked in bands of GROUP tile-rows, column by
+  // column: the ~32 tiles an XCD has in flight then form a compact GROUP x 4 patch that
+  // moves through K together and shares A row-panels and B column-panels in that L2.
+  const int nblocks = tiles_m * tiles_n;
+  const int xcd = blockIdx.x % NUM_XCD, slot = blockIdx.x / NUM_XCD;
+  int tile = xcd * (nblocks / NUM_XCD) + min(xcd, nblocks % NUM_XCD) + slot;
+  if (xcd_remap == 0) tile = blockIdx.x;
   const int per_group = GROUP * tiles_n;
   const int g = tile / per_group;
   const int rows_in_group = min(GROUP, tiles_m - g * GROUP);
@@ -186,7 +195,7 @@ extern "C" int sarek_hip_gemm_f32(const float *a, const float *b, float *c, int 
     }
     const int tiles_m = (m + BM - 1) / BM, tiles_n = (n + BN - 1) / BN;
     hipLaunchKernelGGL(gemm_f32_kernel, dim3(tiles_m * tiles_n), dim3(THREADS), LDS_BYTES, st, a, b,
-                       c, m, n, k, tiles_m, tiles_n);
+                       c, m, n, k, tiles_m, tiles_n, (int)tunable("gemm.xcd_remap", 1));
   } else {
     hipLaunchKernelGGL(gemm_f32_simple_kernel, dim3((n + 63) / 64, (m + 3) / 4), dim3(256), 0, st,
                        a, b, c, m, n, k);
