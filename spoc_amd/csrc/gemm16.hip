@@ -135,15 +135,11 @@ __device__ __forceinline__ void tile_of_block(int tiles_m, int tiles_n, int xcd_
 }
 
 // ---- direct-to-LDS kernel ---------------------------------------------------------
-// One static array per stage and operand: distinct objects, so the compiler can tell
-// that the DMA into one stage does not alias the ds_reads of the other and need not
+// One static LDS array per ring stage and operand: distinct objects, so the compiler can
+// tell that the DMA into one stage does not alias the ds_reads of another and need not
 // wait for it.
-constexpr int DMA_A_BYTES = BM * BK * 2;  // 32768, rows of 128 bytes
-constexpr int DMA_B_BYTES = BK * BN * 2;  // 32768, rows of 512 bytes
-__shared__ __attribute__((aligned(1024))) char dma_a0[DMA_A_BYTES];
-__shared__ __attribute__((aligned(1024))) char dma_b0[DMA_B_BYTES];
-__shared__ __attribute__((aligned(1024))) char dma_a1[DMA_A_BYTES];
-__shared__ __attribute__((aligned(1024))) char dma_b1[DMA_B_BYTES];
+template <int Id, int Bytes>
+__shared__ __attribute__((aligned(1024))) char lds_ring[Bytes];
 
 typedef const __attribute__((address_space(1))) void *gptr_t;
 
@@ -152,7 +148,20 @@ __device__ __forceinline__ void dma16(const void *src, char *lds_dst) {
   __builtin_amdgcn_global_load_lds((gptr_t)src, (LDS_PTR void *)lds_dst, 16, 0, 0);
 }
 
-template <bool Bf16, int Epi>
+// s_waitcnt immediate (gfx9 encoding) that waits for vmcnt <= n and lgkmcnt <= 0.
+constexpr int waitcnt_vm_lgkm0(int n) { return (n & 15) | ((n >> 4) << 14) | (7 << 4) | (0 << 8); }
+
+// Workgroup barrier without the fence __syncthreads() carries (which would drain every
+// outstanding DMA): callers wait for exactly the DMA they need first.
+__device__ __forceinline__ void barrier_no_fence() {
+  asm volatile("" ::: "memory");
+  __builtin_amdgcn_s_barrier();
+  asm volatile("" ::: "memory");
+}
+
+// BKT: K extent of one slab (32 or 64); NS: ring stages.  The DMA of slab s+NS is issued
+// after the barrier inside slab s, so NS-1 slabs of MFMA work cover its latency.
+template <bool Bf16, int Epi, int BKT, int NS>
 __global__ __launch_bounds__(THREADS) void gemm16_dma_kernel(const uint16_t *__restrict__ A,
                                                              const uint16_t *__restrict__ B,
                                                              float *__restrict__ C,
@@ -160,6 +169,14 @@ __global__ __launch_bounds__(THREADS) void gemm16_dma_kernel(const uint16_t *__r
                                                              float *__restrict__ rowsum, int M,
                                                              int N, int K, int tiles_m,
                                                              int tiles_n, int xcd_remap) {
+  constexpr int KK = BKT / 16;                 // MFMA k-steps per slab
+  constexpr int A_ROW = BKT * 2;               // bytes per A row in LDS (unpadded)
+  constexpr int A_ROWS_PER_DMA = 1024 / A_ROW; // rows one wave-wide DMA fills
+  constexpr int A_CHUNKS = A_ROW / 16;
+  constexpr int A_BYTES_S = BM * A_ROW, B_BYTES_S = BKT * BN * 2;
+  constexpr int DMA_PER_WAVE = A_BYTES_S / 1024 / 8;   // per operand, per slab (2 or 4)
+  static_assert(NS * (A_BYTES_S + B_BYTES_S) <= 160 * 1024, "LDS ring too large");
+
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -169,26 +186,36 @@ __global__ __launch_bounds__(THREADS) void gemm16_dma_kernel(const uint16_t *__r
   tile_of_block(tiles_m, tiles_n, xcd_remap, tm, tn);
   const int m0 = tm * BM, n0 = tn * BN;
 
-  // ---- DMA source addresses -----------------------------------------------------
-  // A: wave-instruction q = wave + 8*i (i < 4) fills rows 8q..8q+7; lane l -> row 8q + l/8,
-  //    LDS slot l%8, global chunk (l%8) ^ (l/8)   [(row & 7) == l/8].
-  // B: instruction q fills rows 2q, 2q+1; lane l -> row 2q + l/32, LDS slot l%32,
-  //    global chunk (l%32) ^ ((row & 3) << 1).
+  // Swizzles (applied to the 16-byte slot index within a row):
+  //   A, 128-byte rows: slot ^ (row & 7);  A, 64-byte rows: slot ^ ((row >> 1) & 3)
+  //   B, 512-byte rows: slot ^ ((row & 3) << 1)
+  auto a_swz = [](int row) { return A_CHUNKS == 8 ? (row & 7) : ((row >> 1) & 3); };
+
+  // ---- DMA source addresses (slab 0) ---------------------------------------------
+  // A: wave-instruction q = wave + 8*i fills rows q*R .. q*R+R-1 (R = A_ROWS_PER_DMA);
+  //    lane l -> row q*R + l/A_CHUNKS, LDS slot l%A_CHUNKS, global chunk slot ^ a_swz(row).
+  // B: instruction q fills rows 2q, 2q+1; lane l -> row 2q + l/32, slot l%32,
+  //    global chunk slot ^ ((row & 3) << 1).
   // Rows past M and columns past N are clamped to valid addresses: what they produce is
   // never stored.
-  const uint16_t *a_src[4];
-  const uint16_t *b_src[4];
+  // Addresses are (uniform 64-bit base) + (per-lane 32-bit byte offset), the form the
+  // hardware takes as scalar base + vector offset, so only one register per DMA is kept.
+  uint32_t a_off[DMA_PER_WAVE], b_off[DMA_PER_WAVE];
 #pragma unroll
-  for (int i = 0; i < 4; ++i) {
+  for (int i = 0; i < DMA_PER_WAVE; ++i) {
     const int q = wave + 8 * i;
-    const int arow = min(m0 + 8 * q + (lane >> 3), M - 1);
-    a_src[i] = A + static_cast<int64_t>(arow) * K + (((lane & 7) ^ (lane >> 3)) << 3);
+    const int arow_t = q * A_ROWS_PER_DMA + lane / A_CHUNKS;
+    const int arow = min(arow_t, M - 1 - m0);
+    a_off[i] = (static_cast<uint32_t>(arow) * K + (((lane % A_CHUNKS) ^ a_swz(arow_t)) << 3)) * 2u;
     const int brow = 2 * q + (lane >> 5);
     const int bchunk = (lane & 31) ^ ((brow & 3) << 1);
     const int bcol = min(n0 + bchunk * 8, N - 8);
-    b_src[i] = B + static_cast<int64_t>(brow) * N + bcol;
+    b_off[i] = (static_cast<uint32_t>(brow) * N + bcol) * 2u;
   }
-  const int64_t b_slab_step = static_cast<int64_t>(BK) * N;  // elements per K slab in B
+  const char *a_base = reinterpret_cast<const char *>(A + static_cast<int64_t>(m0) * K);
+  const char *b_base = reinterpret_cast<const char *>(B);
+  const int64_t b_slab_bytes = static_cast<int64_t>(BKT) * N * 2;
+  const int nslabs = K / BKT;
 
   f32x16 acc[4][2];
 #pragma unroll
@@ -199,65 +226,128 @@ __global__ __launch_bounds__(THREADS) void gemm16_dma_kernel(const uint16_t *__r
       for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
 
   // ---- fragment read offsets ------------------------------------------------------
-  // A: row = wm*128 + i*32 + lm, chunk = 2*kk + lh, slot = chunk ^ (lm & 7).
-  const int a_row_off = (wm * 128 + lm) * 128;
-  // B (transposing read): 16-lane group g16 = lane/16: n half = g16 & 1, k half = lh;
-  // lane li supplies row (li>>2) of its 4-row block and the 8 bytes at n offset 4*(li&3).
+  // A: row = wm*128 + i*32 + lm, chunk = 2*kk + lh, slot = chunk ^ a_swz(row).  Since
+  //    2*kk and lh occupy different bits, slot = (lh ^ a_swz) ^ 2*kk: the address for
+  //    k-step kk is one base XOR (kk << 5), and i*32 rows is a constant offset.
+  // B (transposing read): 16-lane group g16 = lane/16: n half = g16 & 1, k half = lh; lane li
+  //    supplies row (li>>2) of its 4-row block and the 8 bytes at n offset 4*(li&3).  Rows
+  //    kk*16 + lh*8 + {0..3} and +4 share (row & 3) = li>>2, so the swizzle XOR is the same
+  //    for both reads; j*64 bytes only touches bit 6, i.e. another XOR.
+  const int a_row = wm * 128 + lm;
+  int a_addr0 = a_row * A_ROW + ((lh ^ a_swz(a_row)) << 4);
   const int li = lane & 15;
-  const int b_r = li >> 2;                                     // row within the 4-row block
-  const int b_nbyte = (wn * 64 + ((lane >> 4) & 1) * 16) * 2 + (li & 3) * 8;  // + j*64
+  const int b_r = li >> 2;
+  int b_addr0 = (lh * 8 + b_r) * 512 +
+                (((wn * 64 + ((lane >> 4) & 1) * 16) * 2 + (li & 3) * 8) ^ (b_r << 5));
 
+  // Slab index past the end is clamped: the tail keeps issuing (redundant) DMA so that the
+  // number of outstanding transfers per wave stays the same in every iteration.
   auto issue = [&](char *sa, char *sb, int slab) {
+    const int sl = min(slab, nslabs - 1);
+    const char *ab = a_base + sl * (BKT * 2);
+    const char *bb = b_base + sl * b_slab_bytes;
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
+    for (int i = 0; i < DMA_PER_WAVE; ++i) {
       const int q = wave + 8 * i;
-      dma16(a_src[i] + slab * BK, sa + q * 1024);
-      dma16(b_src[i] + slab * b_slab_step, sb + q * 1024);
+      dma16(ab + a_off[i], sa + q * 1024);
+      dma16(bb + b_off[i], sb + q * 1024);
     }
   };
   auto load_frags = [&](const char *sa, const char *sb, int kk, u32x4 (&af)[4], u32x4 (&bf)[2]) {
+    const char *pa = sa + (a_addr0 ^ (kk << 5));
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      const int slot = (2 * kk + lh) ^ (lm & 7);
-      af[i] = *reinterpret_cast<const u32x4 *>(sa + a_row_off + i * 32 * 128 + slot * 16);
-    }
+    for (int i = 0; i < 4; ++i)
+      af[i] = *reinterpret_cast<const u32x4 *>(pa + i * 32 * A_ROW);
 #pragma unroll
     for (int j = 0; j < 2; ++j) {
-      // rows kk*16 + lh*8 + {0..3} and {4..7}; (row & 3) == b_r in both
-      const int row_lo = kk * 16 + lh * 8 + b_r;
-      const int nbyte = (b_nbyte + j * 64) ^ (b_r << 5);   // XOR on the 32-byte unit bits
-      u32x2 lo = lds_read_tr16(sb, row_lo * 512 + nbyte);
-      u32x2 hi = lds_read_tr16(sb, (row_lo + 4) * 512 + nbyte);
+      const int off = (b_addr0 ^ (j << 6)) + kk * 16 * 512;
+      u32x2 lo = lds_read_tr16(sb, off);
+      u32x2 hi = lds_read_tr16(sb, off + 4 * 512);
       bf[j] = u32x4{lo.x, lo.y, hi.x, hi.y};
     }
   };
-  auto compute_slab = [&](const char *sa, const char *sb) {
-    u32x4 af[2][4], bf[2][2];
-    load_frags(sa, sb, 0, af[0], bf[0]);
+  auto mfma_step = [&](u32x4 (&af)[4], u32x4 (&bf)[2]) {
 #pragma unroll
-    for (int kk = 0; kk < BK / 16; ++kk) {
-      const int cur = kk & 1;
-      if (kk + 1 < BK / 16) load_frags(sa, sb, kk + 1, af[cur ^ 1], bf[cur ^ 1]);
+    for (int i = 0; i < 4; ++i)
 #pragma unroll
-      for (int i = 0; i < 4; ++i)
+      for (int j = 0; j < 2; ++j) acc[i][j] = mfma<Bf16>(af[i], bf[j], acc[i][j]);
+  };
+  // Issue order inside one k-step: the 8 LDS reads of the next step's fragments go out in
+  // pairs behind the first four MFMAs; the last four MFMAs cover their latency.
+  auto interleave = [] {
 #pragma unroll
-        for (int j = 0; j < 2; ++j) acc[i][j] = mfma<Bf16>(af[cur][i], bf[cur][j], acc[i][j]);
+    for (int g = 0; g < 4; ++g) {
+      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);  // 1 MFMA
+      __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);  // 2 DS reads
     }
+    __builtin_amdgcn_sched_group_barrier(0x008, 4, 0);
+    __builtin_amdgcn_sched_barrier(0);
   };
 
-  const int nslabs = K / BK;
-  issue(dma_a0, dma_b0, 0);
-  __syncthreads();   // waits for this wave's DMA (vmcnt) and for everyone else's
-  for (int s = 0; s < nslabs; s += 2) {
-    if (s + 1 < nslabs) issue(dma_a1, dma_b1, s + 1);
-    compute_slab(dma_a0, dma_b0);
-    __syncthreads();
-    if (s + 1 < nslabs) {
-      if (s + 2 < nslabs) issue(dma_a0, dma_b0, s + 2);
-      compute_slab(dma_a1, dma_b1);
-      __syncthreads();
+  u32x4 af[2][4], bf[2][2];
+
+  // One slab: stage `cur` is consumed, `nxt` is the stage of slab s+1; after the barrier
+  // every wave is done reading `cur`, so it is refilled with slab s+NS.
+  auto slab = [&](char *ca, char *cb, const char *na, const char *nb, int s) {
+    // Keep the per-stage LDS addresses from being hoisted out of the K loop (they would
+    // occupy a register per stage and k-step): the bases are made opaque once per slab.
+    asm volatile("" : "+v"(a_addr0), "+v"(b_addr0));
+#pragma unroll
+    for (int kk = 0; kk + 1 < KK; ++kk) {
+      load_frags(ca, cb, kk + 1, af[(kk + 1) & 1], bf[(kk + 1) & 1]);
+      mfma_step(af[kk & 1], bf[kk & 1]);
+      interleave();
     }
+    // own DMA of slab s+1 landed (NS-2 later slabs may still be in flight), own reads done
+    __builtin_amdgcn_s_waitcnt(waitcnt_vm_lgkm0((NS - 2) * 2 * DMA_PER_WAVE));
+    barrier_no_fence();
+    issue(ca, cb, s + NS);
+    load_frags(na, nb, 0, af[0], bf[0]);
+    mfma_step(af[(KK - 1) & 1], bf[(KK - 1) & 1]);
+    interleave();
+  };
+
+  // prologue: fill the ring, wait for slab 0, fetch its first fragments
+#pragma unroll
+  for (int d = 0; d < NS; ++d) {
+    if (d == 0) issue(lds_ring<0, A_BYTES_S>, lds_ring<1, B_BYTES_S>, 0);
+    if (d == 1) issue(lds_ring<2, A_BYTES_S>, lds_ring<3, B_BYTES_S>, 1);
+    if (d == 2) issue(lds_ring<4, A_BYTES_S>, lds_ring<5, B_BYTES_S>, 2);
+    if (d == 3) issue(lds_ring<6, A_BYTES_S>, lds_ring<7, B_BYTES_S>, 3);
   }
+  __builtin_amdgcn_s_waitcnt(waitcnt_vm_lgkm0((NS - 1) * 2 * DMA_PER_WAVE));
+  barrier_no_fence();
+  load_frags(lds_ring<0, A_BYTES_S>, lds_ring<1, B_BYTES_S>, 0, af[0], bf[0]);
+  __builtin_amdgcn_sched_barrier(0);
+
+  // The ring is unrolled so that every stage is a compile-time array: whole rounds first
+  // (no exits inside the round, which keeps the accumulators in place), then the
+  // remaining nslabs % NS slabs.
+  auto ring_slab = [&](int st, int s) {
+    if (st == 0)
+      slab(lds_ring<0, A_BYTES_S>, lds_ring<1, B_BYTES_S>, lds_ring<2, A_BYTES_S>, lds_ring<3, B_BYTES_S>, s);
+    if constexpr (NS == 2) {
+      if (st == 1)
+        slab(lds_ring<2, A_BYTES_S>, lds_ring<3, B_BYTES_S>, lds_ring<0, A_BYTES_S>, lds_ring<1, B_BYTES_S>, s);
+    } else {
+      if (st == 1)
+        slab(lds_ring<2, A_BYTES_S>, lds_ring<3, B_BYTES_S>, lds_ring<4, A_BYTES_S>, lds_ring<5, B_BYTES_S>, s);
+      if (st == 2)
+        slab(lds_ring<4, A_BYTES_S>, lds_ring<5, B_BYTES_S>, lds_ring<6, A_BYTES_S>, lds_ring<7, B_BYTES_S>, s);
+      if (st == 3)
+        slab(lds_ring<6, A_BYTES_S>, lds_ring<7, B_BYTES_S>, lds_ring<0, A_BYTES_S>, lds_ring<1, B_BYTES_S>, s);
+    }
+  };
+  const int full = nslabs - nslabs % NS;
+  for (int s = 0; s < full; s += NS) {
+#pragma unroll
+    for (int st = 0; st < NS; ++st) ring_slab(st, s + st);
+  }
+#pragma unroll
+  for (int st = 0; st < NS - 1; ++st)
+    if (full + st < nslabs) ring_slab(st, full + st);
+  // drain the (redundant) tail DMA before the LDS is released
+  __builtin_amdgcn_s_waitcnt(waitcnt_vm_lgkm0(0));
   epilogue<Epi>(acc, C, bias, rowsum, M, N, m0 + wm * 128, n0 + wn * 64, lm, lh);
 }
 
@@ -432,8 +522,12 @@ int launch_gemm16(const uint16_t *a, const uint16_t *b, float *c, const float *b
     const int tiles_m = (m + BM - 1) / BM, tiles_n = (n + BN - 1) / BN;
     const int remap = (int)tunable("gemm.xcd_remap", 1);
     if (k % BK == 0 && tunable("gemm16.force_staged", 0) == 0) {
-      hipLaunchKernelGGL((gemm16_dma_kernel<Bf16, Epi>), dim3(tiles_m * tiles_n), dim3(THREADS), 0, st,
-                         a, b, c, bias, rowsum, m, n, k, tiles_m, tiles_n, remap);
+      if (tunable("gemm16.ring", 4) == 4)
+        hipLaunchKernelGGL((gemm16_dma_kernel<Bf16, Epi, 32, 4>), dim3(tiles_m * tiles_n),
+                           dim3(THREADS), 0, st, a, b, c, bias, rowsum, m, n, k, tiles_m, tiles_n, remap);
+      else
+        hipLaunchKernelGGL((gemm16_dma_kernel<Bf16, Epi, 64, 2>), dim3(tiles_m * tiles_n),
+                           dim3(THREADS), 0, st, a, b, c, bias, rowsum, m, n, k, tiles_m, tiles_n, remap);
       return check_launch("gemm16 kernel launch");
     }
     static bool attr_done[2][2] = {{false, false}, {false, false}};
