@@ -186,16 +186,22 @@ __global__ __launch_bounds__(THREADS) void gemm16_dma_kernel(const uint16_t *__r
   tile_of_block(tiles_m, tiles_n, xcd_remap, tm, tn);
   const int m0 = tm * BM, n0 = tn * BN;
 
-  // Swizzles (applied to the 16-byte slot index within a row):
-  //   A, 128-byte rows: slot ^ (row & 7);  A, 64-byte rows: slot ^ ((row >> 1) & 3)
-  //   B, 512-byte rows: slot ^ ((row & 3) << 1)
-  auto a_swz = [](int row) { return A_CHUNKS == 8 ? (row & 7) : ((row >> 1) & 3); };
+  // Swizzles (XOR on the 16-byte slot index within a row).  The LDS of this chip serves
+  // 256 bytes per clock (64 banks x 4 bytes): a ds_read_b128 is served 16 lanes at a time
+  // and a ds_read_b64_tr_b16 32 lanes at a time, and a phase is conflict free when its
+  // pieces fall on distinct positions modulo 256 bytes.
+  //   A, 128-byte rows: 16 consecutive rows read the same chunk c; row parity picks the
+  //      128-byte half, so the slot must differ over rows of equal parity:
+  //      slot = c ^ ((row >> 1) & 7).   A, 64-byte rows: slot = c ^ ((row >> 2) & 3).
+  //   B, 512-byte rows: a phase reads 4 rows x two 32-byte pieces (n halves); rows are
+  //      spread 64 bytes apart: slot = c ^ ((row & 3) << 2).
+  auto a_swz = [](int row) { return A_CHUNKS == 8 ? ((row >> 1) & 7) : ((row >> 2) & 3); };
 
   // ---- DMA source addresses (slab 0) ---------------------------------------------
   // A: wave-instruction q = wave + 8*i fills rows q*R .. q*R+R-1 (R = A_ROWS_PER_DMA);
   //    lane l -> row q*R + l/A_CHUNKS, LDS slot l%A_CHUNKS, global chunk slot ^ a_swz(row).
   // B: instruction q fills rows 2q, 2q+1; lane l -> row 2q + l/32, slot l%32,
-  //    global chunk slot ^ ((row & 3) << 1).
+  //    global chunk slot ^ ((row & 3) << 2).
   // Rows past M and columns past N are clamped to valid addresses: what they produce is
   // never stored.
   // Addresses are (uniform 64-bit base) + (per-lane 32-bit byte offset), the form the
@@ -208,7 +214,7 @@ __global__ __launch_bounds__(THREADS) void gemm16_dma_kernel(const uint16_t *__r
     const int arow = min(arow_t, M - 1 - m0);
     a_off[i] = (static_cast<uint32_t>(arow) * K + (((lane % A_CHUNKS) ^ a_swz(arow_t)) << 3)) * 2u;
     const int brow = 2 * q + (lane >> 5);
-    const int bchunk = (lane & 31) ^ ((brow & 3) << 1);
+    const int bchunk = (lane & 31) ^ ((brow & 3) << 2);
     const int bcol = min(n0 + bchunk * 8, N - 8);
     b_off[i] = (static_cast<uint32_t>(brow) * N + bcol) * 2u;
   }
@@ -238,7 +244,7 @@ __global__ __launch_bounds__(THREADS) void gemm16_dma_kernel(const uint16_t *__r
   const int li = lane & 15;
   const int b_r = li >> 2;
   int b_addr0 = (lh * 8 + b_r) * 512 +
-                (((wn * 64 + ((lane >> 4) & 1) * 16) * 2 + (li & 3) * 8) ^ (b_r << 5));
+                (((wn * 64 + ((lane >> 4) & 1) * 16) * 2 + (li & 3) * 8) ^ (b_r << 6));
 
   // Slab index past the end is clamped: the tail keeps issuing (redundant) DMA so that the
   // number of outstanding transfers per wave stays the same in every iteration.
