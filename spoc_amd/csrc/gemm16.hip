@@ -31,6 +31,8 @@
 //     kk+1 are fetched from LDS while the MFMAs of k-step kk issue.
 //   gemm16_staged_kernel (any K % 8 == 0): global -> registers -> LDS with zero fill for
 //     the K tail, rows padded instead of swizzled.
+#include <type_traits>
+
 #include "common.hpp"
 #include "tunables.hpp"
 
@@ -50,7 +52,6 @@ typedef __attribute__((ext_vector_type(2))) unsigned int u32x2;
 constexpr int BM = 256, BN = 256, BK = 64;
 constexpr int THREADS = 512;
 constexpr int NUM_XCD = 8;   // XCDs of an MI355X; workgroup ids are dealt to them round-robin
-constexpr int GROUP = 8;     // tile-rows per raster band
 constexpr int A_STRIDE = BK * 2 + 16;   // bytes per A row in LDS (144)
 constexpr int B_STRIDE = BN * 2 + 32;   // bytes per B row in LDS (544)
 constexpr int A_BYTES = BM * A_STRIDE;  // 36864
@@ -83,10 +84,10 @@ __device__ __forceinline__ float half_wave_sum(float v) {
   return v;
 }
 
-// Writes one wave's 128 x 64 accumulator block.  Accumulator layout of the 32x32 MFMA:
+// Writes one wave's 128 x (32*TJ) accumulator block.  Accumulator layout of the 32x32 MFMA:
 // register r of lane l holds row 8*(r/4) + 4*(l/32) + r%4, column l%32 of its tile.
-template <int Epi>
-__device__ __forceinline__ void epilogue(f32x16 (&acc)[4][2], float *__restrict__ C,
+template <int Epi, int TJ>
+__device__ __forceinline__ void epilogue(f32x16 (&acc)[4][TJ], float *__restrict__ C,
                                          const float *__restrict__ bias,
                                          float *__restrict__ rowsum, int M, int N, int row0,
                                          int col0, int lm, int lh) {
@@ -97,7 +98,7 @@ __device__ __forceinline__ void epilogue(f32x16 (&acc)[4][2], float *__restrict_
       const int row = row0 + i * 32 + 8 * (r >> 2) + 4 * lh + (r & 3);
       float rs = 0.f;
 #pragma unroll
-      for (int j = 0; j < 2; ++j) {
+      for (int j = 0; j < TJ; ++j) {
         const int col = col0 + j * 32 + lm;
         float v = acc[i][j][r];
         if (Epi == EPI_BIAS_RELU_ROWSUM) {
@@ -122,6 +123,7 @@ __device__ __forceinline__ void epilogue(f32x16 (&acc)[4][2], float *__restrict_
 // moves through K together and shares A row-panels and B column-panels in that L2.
 __device__ __forceinline__ void tile_of_block(int tiles_m, int tiles_n, int xcd_remap, int &tm,
                                               int &tn) {
+  const int GROUP = xcd_remap > 1 ? xcd_remap : 8;   // tile-rows per raster band
   const int nblocks = tiles_m * tiles_n;
   const int xcd = blockIdx.x % NUM_XCD, slot = blockIdx.x / NUM_XCD;
   int tile = xcd * (nblocks / NUM_XCD) + min(xcd, nblocks % NUM_XCD) + slot;
@@ -161,8 +163,11 @@ __device__ __forceinline__ void barrier_no_fence() {
 
 // BKT: K extent of one slab (32 or 64); NS: ring stages.  The DMA of slab s+NS is issued
 // after the barrier inside slab s, so NS-1 slabs of MFMA work cover its latency.
-template <bool Bf16, int Epi, int BKT, int NS>
-__global__ __launch_bounds__(THREADS) void gemm16_dma_kernel(const uint16_t *__restrict__ A,
+// TJ: 32-column MFMA tiles per wave along N.  TJ = 2: 8 waves (2 x 4) of 128 x 64, two
+// per SIMD; TJ = 4: 4 waves (2 x 2) of 128 x 128, one per SIMD with the 256 accumulator
+// registers in the AGPR half of the register file (fewer LDS bytes read per flop).
+template <bool Bf16, int Epi, int BKT, int NS, int TJ>
+__global__ __launch_bounds__(64 * 2 * (8 / TJ)) void gemm16_dma_kernel(const uint16_t *__restrict__ A,
                                                              const uint16_t *__restrict__ B,
                                                              float *__restrict__ C,
                                                              const float *__restrict__ bias,
@@ -174,13 +179,15 @@ __global__ __launch_bounds__(THREADS) void gemm16_dma_kernel(const uint16_t *__r
   constexpr int A_ROWS_PER_DMA = 1024 / A_ROW; // rows one wave-wide DMA fills
   constexpr int A_CHUNKS = A_ROW / 16;
   constexpr int A_BYTES_S = BM * A_ROW, B_BYTES_S = BKT * BN * 2;
-  constexpr int DMA_PER_WAVE = A_BYTES_S / 1024 / 8;   // per operand, per slab (2 or 4)
+  constexpr int WN = 8 / TJ;                   // waves along N (4 or 2); 2 along M
+  constexpr int NWAVES = 2 * WN;
+  constexpr int DMA_PER_WAVE = A_BYTES_S / 1024 / NWAVES;   // per operand, per slab
   static_assert(NS * (A_BYTES_S + B_BYTES_S) <= 160 * 1024, "LDS ring too large");
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-  const int wm = wave >> 2, wn = wave & 3;
+  const int wm = wave / WN, wn = wave % WN;
   const int lm = lane & 31, lh = lane >> 5;
   int tm, tn;
   tile_of_block(tiles_m, tiles_n, xcd_remap, tm, tn);
@@ -198,7 +205,7 @@ __global__ __launch_bounds__(THREADS) void gemm16_dma_kernel(const uint16_t *__r
   auto a_swz = [](int row) { return A_CHUNKS == 8 ? ((row >> 1) & 7) : ((row >> 2) & 3); };
 
   // ---- DMA source addresses (slab 0) ---------------------------------------------
-  // A: wave-instruction q = wave + 8*i fills rows q*R .. q*R+R-1 (R = A_ROWS_PER_DMA);
+  // A: wave-instruction q = wave + NWAVES*i fills rows q*R .. q*R+R-1 (R = A_ROWS_PER_DMA);
   //    lane l -> row q*R + l/A_CHUNKS, LDS slot l%A_CHUNKS, global chunk slot ^ a_swz(row).
   // B: instruction q fills rows 2q, 2q+1; lane l -> row 2q + l/32, slot l%32,
   //    global chunk slot ^ ((row & 3) << 2).
@@ -209,7 +216,7 @@ __global__ __launch_bounds__(THREADS) void gemm16_dma_kernel(const uint16_t *__r
   uint32_t a_off[DMA_PER_WAVE], b_off[DMA_PER_WAVE];
 #pragma unroll
   for (int i = 0; i < DMA_PER_WAVE; ++i) {
-    const int q = wave + 8 * i;
+    const int q = wave + NWAVES * i;
     const int arow_t = q * A_ROWS_PER_DMA + lane / A_CHUNKS;
     const int arow = min(arow_t, M - 1 - m0);
     a_off[i] = (static_cast<uint32_t>(arow) * K + (((lane % A_CHUNKS) ^ a_swz(arow_t)) << 3)) * 2u;
@@ -223,11 +230,11 @@ __global__ __launch_bounds__(THREADS) void gemm16_dma_kernel(const uint16_t *__r
   const int64_t b_slab_bytes = static_cast<int64_t>(BKT) * N * 2;
   const int nslabs = K / BKT;
 
-  f32x16 acc[4][2];
+  f32x16 acc[4][TJ];
 #pragma unroll
   for (int i = 0; i < 4; ++i)
 #pragma unroll
-    for (int j = 0; j < 2; ++j)
+    for (int j = 0; j < TJ; ++j)
 #pragma unroll
       for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
 
@@ -244,7 +251,7 @@ __global__ __launch_bounds__(THREADS) void gemm16_dma_kernel(const uint16_t *__r
   const int li = lane & 15;
   const int b_r = li >> 2;
   int b_addr0 = (lh * 8 + b_r) * 512 +
-                (((wn * 64 + ((lane >> 4) & 1) * 16) * 2 + (li & 3) * 8) ^ (b_r << 6));
+                (((wn * (32 * TJ) + ((lane >> 4) & 1) * 16) * 2 + (li & 3) * 8) ^ (b_r << 6));
 
   // Slab index past the end is clamped: the tail keeps issuing (redundant) DMA so that the
   // number of outstanding transfers per wave stays the same in every iteration.
@@ -254,43 +261,46 @@ __global__ __launch_bounds__(THREADS) void gemm16_dma_kernel(const uint16_t *__r
     const char *bb = b_base + sl * b_slab_bytes;
 #pragma unroll
     for (int i = 0; i < DMA_PER_WAVE; ++i) {
-      const int q = wave + 8 * i;
+      const int q = wave + NWAVES * i;
       dma16(ab + a_off[i], sa + q * 1024);
       dma16(bb + b_off[i], sb + q * 1024);
     }
   };
-  auto load_frags = [&](const char *sa, const char *sb, int kk, u32x4 (&af)[4], u32x4 (&bf)[2]) {
+  auto load_frags = [&](const char *sa, const char *sb, int kk, u32x4 (&af)[4], u32x4 (&bf)[TJ]) {
     const char *pa = sa + (a_addr0 ^ (kk << 5));
 #pragma unroll
     for (int i = 0; i < 4; ++i)
       af[i] = *reinterpret_cast<const u32x4 *>(pa + i * 32 * A_ROW);
 #pragma unroll
-    for (int j = 0; j < 2; ++j) {
+    for (int j = 0; j < TJ; ++j) {
+      // j*64 bytes: with TJ = 4 the wave's 256-byte column span is 256-byte aligned, so
+      // adding j*64 never carries into the bits the swizzle touches differently
       const int off = (b_addr0 ^ (j << 6)) + kk * 16 * 512;
       u32x2 lo = lds_read_tr16(sb, off);
       u32x2 hi = lds_read_tr16(sb, off + 4 * 512);
       bf[j] = u32x4{lo.x, lo.y, hi.x, hi.y};
     }
   };
-  auto mfma_step = [&](u32x4 (&af)[4], u32x4 (&bf)[2]) {
+  auto mfma_step = [&](u32x4 (&af)[4], u32x4 (&bf)[TJ]) {
 #pragma unroll
     for (int i = 0; i < 4; ++i)
 #pragma unroll
-      for (int j = 0; j < 2; ++j) acc[i][j] = mfma<Bf16>(af[i], bf[j], acc[i][j]);
+      for (int j = 0; j < TJ; ++j) acc[i][j] = mfma<Bf16>(af[i], bf[j], acc[i][j]);
   };
   // Issue order inside one k-step: the 8 LDS reads of the next step's fragments go out in
   // pairs behind the first four MFMAs; the last four MFMAs cover their latency.
   auto interleave = [] {
+    constexpr int READS = 4 + 2 * TJ, MFMAS = 4 * TJ;
 #pragma unroll
-    for (int g = 0; g < 4; ++g) {
+    for (int g = 0; g < READS / 2; ++g) {
       __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);  // 1 MFMA
       __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);  // 2 DS reads
     }
-    __builtin_amdgcn_sched_group_barrier(0x008, 4, 0);
+    __builtin_amdgcn_sched_group_barrier(0x008, MFMAS - READS / 2, 0);
     __builtin_amdgcn_sched_barrier(0);
   };
 
-  u32x4 af[2][4], bf[2][2];
+  u32x4 af[2][4], bf[2][TJ];
 
   // One slab: stage `cur` is consumed, `nxt` is the stage of slab s+1; after the barrier
   // every wave is done reading `cur`, so it is refilled with slab s+NS.
@@ -314,12 +324,11 @@ __global__ __launch_bounds__(THREADS) void gemm16_dma_kernel(const uint16_t *__r
   };
 
   // prologue: fill the ring, wait for slab 0, fetch its first fragments
-#pragma unroll
-  for (int d = 0; d < NS; ++d) {
-    if (d == 0) issue(lds_ring<0, A_BYTES_S>, lds_ring<1, B_BYTES_S>, 0);
-    if (d == 1) issue(lds_ring<2, A_BYTES_S>, lds_ring<3, B_BYTES_S>, 1);
-    if (d == 2) issue(lds_ring<4, A_BYTES_S>, lds_ring<5, B_BYTES_S>, 2);
-    if (d == 3) issue(lds_ring<6, A_BYTES_S>, lds_ring<7, B_BYTES_S>, 3);
+  issue(lds_ring<0, A_BYTES_S>, lds_ring<1, B_BYTES_S>, 0);
+  issue(lds_ring<2, A_BYTES_S>, lds_ring<3, B_BYTES_S>, 1);
+  if constexpr (NS == 4) {
+    issue(lds_ring<4, A_BYTES_S>, lds_ring<5, B_BYTES_S>, 2);
+    issue(lds_ring<6, A_BYTES_S>, lds_ring<7, B_BYTES_S>, 3);
   }
   __builtin_amdgcn_s_waitcnt(waitcnt_vm_lgkm0((NS - 1) * 2 * DMA_PER_WAVE));
   barrier_no_fence();
@@ -329,32 +338,33 @@ __global__ __launch_bounds__(THREADS) void gemm16_dma_kernel(const uint16_t *__r
   // The ring is unrolled so that every stage is a compile-time array: whole rounds first
   // (no exits inside the round, which keeps the accumulators in place), then the
   // remaining nslabs % NS slabs.
-  auto ring_slab = [&](int st, int s) {
-    if (st == 0)
-      slab(lds_ring<0, A_BYTES_S>, lds_ring<1, B_BYTES_S>, lds_ring<2, A_BYTES_S>, lds_ring<3, B_BYTES_S>, s);
-    if constexpr (NS == 2) {
-      if (st == 1)
-        slab(lds_ring<2, A_BYTES_S>, lds_ring<3, B_BYTES_S>, lds_ring<0, A_BYTES_S>, lds_ring<1, B_BYTES_S>, s);
-    } else {
-      if (st == 1)
-        slab(lds_ring<2, A_BYTES_S>, lds_ring<3, B_BYTES_S>, lds_ring<4, A_BYTES_S>, lds_ring<5, B_BYTES_S>, s);
-      if (st == 2)
-        slab(lds_ring<4, A_BYTES_S>, lds_ring<5, B_BYTES_S>, lds_ring<6, A_BYTES_S>, lds_ring<7, B_BYTES_S>, s);
-      if (st == 3)
-        slab(lds_ring<6, A_BYTES_S>, lds_ring<7, B_BYTES_S>, lds_ring<0, A_BYTES_S>, lds_ring<1, B_BYTES_S>, s);
-    }
+  auto ring_slab = [&](auto st_c, int s) {
+    constexpr int st = decltype(st_c)::value;
+    constexpr int nx = (st + 1) % NS;
+    slab(lds_ring<2 * st, A_BYTES_S>, lds_ring<2 * st + 1, B_BYTES_S>, lds_ring<2 * nx, A_BYTES_S>,
+         lds_ring<2 * nx + 1, B_BYTES_S>, s);
   };
+  using I0 = std::integral_constant<int, 0>;
+  using I1 = std::integral_constant<int, 1>;
+  using I2 = std::integral_constant<int, 2>;
+  using I3 = std::integral_constant<int, 3>;
   const int full = nslabs - nslabs % NS;
   for (int s = 0; s < full; s += NS) {
-#pragma unroll
-    for (int st = 0; st < NS; ++st) ring_slab(st, s + st);
+    ring_slab(I0{}, s);
+    ring_slab(I1{}, s + 1);
+    if constexpr (NS == 4) {
+      ring_slab(I2{}, s + 2);
+      ring_slab(I3{}, s + 3);
+    }
   }
-#pragma unroll
-  for (int st = 0; st < NS - 1; ++st)
-    if (full + st < nslabs) ring_slab(st, full + st);
+  if (full < nslabs) ring_slab(I0{}, full);
+  if constexpr (NS == 4) {
+    if (full + 1 < nslabs) ring_slab(I1{}, full + 1);
+    if (full + 2 < nslabs) ring_slab(I2{}, full + 2);
+  }
   // drain the (redundant) tail DMA before the LDS is released
   __builtin_amdgcn_s_waitcnt(waitcnt_vm_lgkm0(0));
-  epilogue<Epi>(acc, C, bias, rowsum, M, N, m0 + wm * 128, n0 + wn * 64, lm, lh);
+  epilogue<Epi, TJ>(acc, C, bias, rowsum, M, N, m0 + wm * 128, n0 + wn * (32 * TJ), lm, lh);
 }
 
 template <bool Bf16, int Epi>
@@ -462,7 +472,7 @@ __global__ __launch_bounds__(THREADS) void gemm16_staged_kernel(const uint16_t *
     __syncthreads();
   }
 
-  epilogue<Epi>(acc, C, bias, rowsum, M, N, m0 + wm * 128, n0 + wn * 64, lm, lh);
+  epilogue<Epi, 2>(acc, C, bias, rowsum, M, N, m0 + wm * 128, n0 + wn * 64, lm, lh);
 }
 
 // Any shape, any alignment: one thread per C element, f32 accumulate in k order.
@@ -528,12 +538,16 @@ int launch_gemm16(const uint16_t *a, const uint16_t *b, float *c, const float *b
     const int tiles_m = (m + BM - 1) / BM, tiles_n = (n + BN - 1) / BN;
     const int remap = (int)tunable("gemm.xcd_remap", 1);
     if (k % BK == 0 && tunable("gemm16.force_staged", 0) == 0) {
-      if (tunable("gemm16.ring", 4) == 4)
-        hipLaunchKernelGGL((gemm16_dma_kernel<Bf16, Epi, 32, 4>), dim3(tiles_m * tiles_n),
-                           dim3(THREADS), 0, st, a, b, c, bias, rowsum, m, n, k, tiles_m, tiles_n, remap);
-      else
-        hipLaunchKernelGGL((gemm16_dma_kernel<Bf16, Epi, 64, 2>), dim3(tiles_m * tiles_n),
-                           dim3(THREADS), 0, st, a, b, c, bias, rowsum, m, n, k, tiles_m, tiles_n, remap);
+      const int ring = (int)tunable("gemm16.ring", 4), tj = (int)tunable("gemm16.tj", 2);
+      const dim3 grid(tiles_m * tiles_n);
+#define SAREK_LAUNCH_DMA(BKT, NS, TJ)                                                             \
+  hipLaunchKernelGGL((gemm16_dma_kernel<Bf16, Epi, BKT, NS, TJ>), grid, dim3(64 * 2 * (8 / TJ)), 0, \
+                     st, a, b, c, bias, rowsum, m, n, k, tiles_m, tiles_n, remap)
+      if (ring == 4 && tj == 2) SAREK_LAUNCH_DMA(32, 4, 2);
+      else if (ring == 4) SAREK_LAUNCH_DMA(32, 4, 4);
+      else if (tj == 2) SAREK_LAUNCH_DMA(64, 2, 2);
+      else SAREK_LAUNCH_DMA(64, 2, 4);
+#undef SAREK_LAUNCH_DMA
       return check_launch("gemm16 kernel launch");
     }
     static bool attr_done[2][2] = {{false, false}, {false, false}};

@@ -27,7 +27,6 @@ typedef __attribute__((ext_vector_type(4))) float f32x4;
 constexpr int BM = 256, BN = 256, BK = 32;
 constexpr int THREADS = 512;
 constexpr int NUM_XCD = 8;   // XCDs of an MI355X; workgroup ids are dealt to them round-robin
-constexpr int GROUP = 8;     // tile-rows per raster band
 constexpr int A_STRIDE = BK + 4;            // floats per A row in LDS (36)
 constexpr int B_STRIDE = BN;                // floats per B row in LDS
 constexpr int A_FLOATS = BM * A_STRIDE;     // 9216
@@ -54,6 +53,7 @@ __global__ __launch_bounds__(THREADS) void gemm_f32_kernel(const float *__restri
   const int xcd = blockIdx.x % NUM_XCD, slot = blockIdx.x / NUM_XCD;
   int tile = xcd * (nblocks / NUM_XCD) + min(xcd, nblocks % NUM_XCD) + slot;
   if (xcd_remap == 0) tile = blockIdx.x;
+  const int GROUP = xcd_remap > 1 ? xcd_remap : 8;   // tile-rows per raster band
   const int per_group = GROUP * tiles_n;
   const int g = tile / per_group;
   const int rows_in_group = min(GROUP, tiles_m - g * GROUP);
