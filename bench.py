@@ -26,6 +26,14 @@ if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
 
 PEAK_HBM_GBS = 8000.0          # MI355X HBM3E
+# HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (KiB per dispatch,
+# FETCH_SIZE scaled by 2.0 and WRITE_SIZE by 1.0 after calibration against a plain 1 GiB copy).
+MEASURED_TRAFFIC_BYTES = {
+    "triad_sum_2p28": (1048600 * 2 + 1048700) * 1024,
+    "gemm_bf16_8192": (817384 * 2 + 262144) * 1024,
+    "gemm_f32_8192": (1579270 * 2 + 262144) * 1024,
+    "gemm_f16_epilogue": (313832 * 2 + 187093) * 1024,
+}
 PEAK_MFMA_TFLOPS = {"bf16": 2500.0, "f16": 2500.0, "f32": 157.3}
 
 
@@ -36,7 +44,7 @@ def parse():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--workload", default="gemm_bf16_8192",
                     choices=["gemm_bf16_8192", "triad_sum_2p28", "gemm_f32_8192", "gemm_f32_1024",
-                             "gemm_f16_epilogue"])
+                             "gemm_f16_epilogue", "copy_1gib"])
     ap.add_argument("--no-also", action="store_true", help="measure only the headline workload")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     return ap.parse_args()
@@ -65,6 +73,16 @@ class Events:
 def make_workload(name, torch, hip):
     """Returns (step_fn, info) with inputs resident on the GPU."""
     g = torch.Generator(device="cuda")
+    if name == "copy_1gib":
+        # plain device copy of known size: calibrates the FETCH_SIZE / WRITE_SIZE counters
+        n = 1 << 28
+        src = torch.rand(n, device="cuda", generator=g)
+        dst = torch.empty_like(src)
+        info = dict(metric="plain copy GB/s (counter calibration)", unit="GB/s", dtype="f32",
+                    work=8.0 * n, work_unit=1e9, bound="hbm", peak=PEAK_HBM_GBS,
+                    kernel="at::native copy kernel",
+                    config={"workload": "dst.copy_(src), 1 GiB read + 1 GiB written", "n": n})
+        return (lambda: dst.copy_(src)), info
     if name == "triad_sum_2p28":
         n = 1 << 28
         g.manual_seed(0xB)
@@ -100,7 +118,7 @@ def make_workload(name, torch, hip):
         c = torch.empty(s, s, device="cuda")
         info = dict(metric="GEMM TFLOP/s at 8192^3 (bf16-in, f32-accumulate)", unit="TFLOP/s",
                     dtype="bf16", work=2.0 * s ** 3, work_unit=1e12, bound="mfma",
-                    peak=PEAK_MFMA_TFLOPS["bf16"], kernel="gemm16_kernel<bf16>",
+                    peak=PEAK_MFMA_TFLOPS["bf16"], kernel="gemm16_dma_kernel<bf16, store, 32, 4, 2>",
                     config={"workload": "bf16-in f32-acc GEMM C=A.B row-major, N(0,0.02)",
                             "m": s, "n": s, "k": s})
         return (lambda: hip.gemm_bf16(a, b, out=c)), info
@@ -115,7 +133,7 @@ def make_workload(name, torch, hip):
         rs = torch.empty(m, device="cuda")
         info = dict(metric="fp16 GEMM + bias + ReLU + row-sum TFLOP/s", unit="TFLOP/s", dtype="f16",
                     work=2.0 * m * n * k, work_unit=1e12, bound="mfma",
-                    peak=PEAK_MFMA_TFLOPS["f16"], kernel="gemm16_kernel<f16, bias_relu_rowsum>",
+                    peak=PEAK_MFMA_TFLOPS["f16"], kernel="gemm16_dma_kernel<f16, bias_relu_rowsum, 32, 4, 2>",
                     config={"workload": "fp16-in f32-acc Y=relu(A.B+bias), rowsum(Y)",
                             "m": m, "n": n, "k": k})
         return (lambda: hip.gemm_f16_bias_relu_rowsum(a, b, bias, out=y, rowsum=rs)), info
@@ -153,7 +171,8 @@ def measure(name, torch, hip, steps, warmup):
         "dtype": info["dtype"], "config": info["config"],
         "roofline": {"bound": info["bound"], "achieved": round(achieved, 2), "peak": info["peak"],
                      "unit": "GB/s" if info["bound"] == "hbm" else "TFLOP/s",
-                     "frac": round(achieved / info["peak"], 4), "traffic": None,
+                     "frac": round(achieved / info["peak"], 4),
+                     "traffic": MEASURED_TRAFFIC_BYTES.get(name),
                      "kernel": info["kernel"], "kernel_ms": round(kernel_ms, 5)},
     }
     return res
@@ -217,7 +236,7 @@ def main():
         "data": "synthetic", "config": head["config"], "roofline": head["roofline"],
         "gpu_ms_per_step_events": head["gpu_ms_per_step_events"],
     }
-    if not args.no_cpu_baseline:
+    if not args.no_cpu_baseline and args.workload != "copy_1gib":
         out["cpu_baseline"] = cpu_baseline(args.workload)
     if not args.no_also:
         also = []

@@ -3,34 +3,34 @@
 //
 // C[M x N] = A[M x K] . B[K x N], all row-major.
 //
-// Tiling: one workgroup (512 threads = 8 waves, 2 along M x 4 along N) owns a
-// 256 x 256 tile of C and walks K in slabs of 64.  Each wave owns 128 x 64 of the
-// tile = 4 x 2 MFMA tiles of 32 x 32 (128 accumulator registers).
+// Tiling: one workgroup owns a 256 x 256 tile of C and walks K in slabs.  Default: 8 waves
+// (2 along M x 4 along N, two per SIMD), each owning 128 x 64 = 4 x 2 MFMA tiles of 32 x 32
+// (128 accumulator registers).  One workgroup per CU (LDS bound), 8192^3 = 1024 tiles =
+// 4 per CU.
 //
-// LDS holds two stages of (A slab [256][64], B slab [64][256]).  A rows are padded
-// to 144 bytes so the eight 16-byte reads of consecutive rows fall in distinct
-// banks; B rows are padded to 544 bytes so the four rows touched by one transposing
-// read fall in distinct banks.
-//
-// Operand fetch:
+// Operand fetch from LDS:
 //   A: lane (m = lane%32, h = lane/32) needs k = 8h..8h+7 of row m: one ds_read_b128.
-//   B: lane (n = lane%32, h) needs k = 8h..8h+7 of column n.  B is n-contiguous in
-//      LDS, so the column is gathered by ds_read_b64_tr_b16: within each group of
-//      16 lanes, lane i supplies the address of 4 consecutive n of row (i/4) at
-//      n-offset 4*(i%4), and receives column i of that 4 x 16 block (its 4 rows).
-//      Two such reads (rows 0-3 and 4-7 of the lane's k range) give the 8 k values.
+//   B: lane (n = lane%32, h) needs k = 8h..8h+7 of column n.  B is n-contiguous in LDS (as in
+//      global memory), so the column is gathered by ds_read_b64_tr_b16: within each group of
+//      16 lanes, lane i supplies the address of 4 consecutive n of row (i/4) at n-offset
+//      4*(i%4), and receives column i of that 4 x 16 block (its 4 rows).  Two such reads
+//      (rows 0-3 and 4-7 of the lane's k range) give the 8 k values.
 //
-// Two kernels share this tiling:
-//   gemm16_dma_kernel (K % 64 == 0): global -> LDS by global_load_lds_dwordx4, which
-//     writes the 64 lanes' 16-byte pieces to 1 KiB of consecutive LDS with no register
-//     staging and no ds_write.  Rows cannot be padded that way, so bank conflicts are
-//     avoided by an XOR swizzle applied on the global-address side: LDS 16-byte slot p of
-//     row r holds global chunk p ^ (r & 7) for A (128-byte rows) and p ^ ((r & 3) << 1)
-//     for B (512-byte rows); readers apply the same XOR.  The next slab streams into the
-//     other stage while the MFMAs of the current slab run; operand fragments for k-step
-//     kk+1 are fetched from LDS while the MFMAs of k-step kk issue.
-//   gemm16_staged_kernel (any K % 8 == 0): global -> registers -> LDS with zero fill for
-//     the K tail, rows padded instead of swizzled.
+// Three kernels:
+//   gemm16_dma_kernel (K % 64 == 0, the fast path): global -> LDS by
+//     global_load_lds_dwordx4, which writes the 64 lanes' 16-byte pieces to 1 KiB of
+//     consecutive LDS with no register staging and no ds_write.  Rows cannot be padded that
+//     way, so bank conflicts are removed by an XOR swizzle applied on the global-address
+//     side (which chunk a lane fetches) and again by the readers.  K slabs of 32 stream
+//     through a ring of 4 LDS stages (128 KiB): the DMA of slab s+4 is issued right after
+//     the barrier inside slab s, so three slabs of MFMA work cover its latency; the barrier
+//     sits before the LAST k-step of a slab, and the first fragments of the next slab are
+//     fetched under that step's MFMAs, so no LDS latency is exposed at slab boundaries.
+//     Inside a k-step the LDS reads of the next step's fragments are interleaved behind the
+//     first MFMAs (sched_group_barrier).
+//   gemm16_staged_kernel (any K % 8 == 0): global -> registers -> LDS with zero fill for the
+//     K tail, rows padded (144 / 544 bytes) instead of swizzled, two LDS stages of K = 64.
+//   gemm16_simple_kernel: any shape and alignment, one thread per C element.
 #include <type_traits>
 
 #include "common.hpp"
