@@ -197,8 +197,11 @@ int sarek_hip_triad_f32(float *a, const float *b, const float *c, float s, int64
                         sarek_hip_stream stream);
 
 /* Fused triad + sum: writes a as above and *sum_out = sum_i a[i] (double,
- * device memory).  `partials` is caller workspace of at least
- * sarek_hip_triad_sum_workspace_floats(n) floats.                          */
+ * device memory).  Every workgroup leaves an f32 partial in `partials`
+ * (caller workspace of at least sarek_hip_triad_sum_workspace_floats(n)
+ * floats; contents on entry are irrelevant) and a one-workgroup kernel on
+ * the same stream folds them in double, in index order: the result does
+ * not depend on scheduling.                                                */
 int64_t sarek_hip_triad_sum_workspace_floats(int64_t n);
 int sarek_hip_triad_sum_f32(float *a, const float *b, const float *c, float s, int64_t n,
                             float *partials, int64_t partials_len, double *sum_out,
