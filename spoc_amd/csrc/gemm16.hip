@@ -34,6 +34,7 @@
 #include <type_traits>
 
 #include "common.hpp"
+#include "gemm_common.hpp"
 #include "tunables.hpp"
 
 namespace sarek_hip {
@@ -47,11 +48,8 @@ typedef __attribute__((ext_vector_type(16))) float f32x16;
 typedef __attribute__((ext_vector_type(4))) unsigned int u32x4;
 typedef __attribute__((ext_vector_type(2))) unsigned int u32x2;
 
-#define LDS_PTR __attribute__((address_space(3)))
-
 constexpr int BM = 256, BN = 256, BK = 64;
 constexpr int THREADS = 512;
-constexpr int NUM_XCD = 8;   // XCDs of an MI355X; workgroup ids are dealt to them round-robin
 constexpr int A_STRIDE = BK * 2 + 16;   // bytes per A row in LDS (144)
 constexpr int B_STRIDE = BN * 2 + 32;   // bytes per B row in LDS (544)
 constexpr int A_BYTES = BM * A_STRIDE;  // 36864
@@ -116,51 +114,7 @@ __device__ __forceinline__ void epilogue(f32x16 (&acc)[4][TJ], float *__restrict
   }
 }
 
-// Workgroup -> tile.  The hardware deals consecutive workgroup ids round-robin to the
-// 8 XCDs (each with its own L2), so ids are first regrouped to give every XCD one
-// contiguous run of tiles, and the run is walked in bands of GROUP tile-rows, column by
-// column: the ~32 tiles an XCD has in flight then form a compact GROUP x 4 patch that
-// moves through K together and shares A row-panels and B column-panels in that L2.
-__device__ __forceinline__ void tile_of_block(int tiles_m, int tiles_n, int xcd_remap, int &tm,
-                                              int &tn) {
-  const int GROUP = xcd_remap > 1 ? xcd_remap : 8;   // tile-rows per raster band
-  const int nblocks = tiles_m * tiles_n;
-  const int xcd = blockIdx.x % NUM_XCD, slot = blockIdx.x / NUM_XCD;
-  int tile = xcd * (nblocks / NUM_XCD) + min(xcd, nblocks % NUM_XCD) + slot;
-  if (xcd_remap == 0) tile = blockIdx.x;
-  const int per_group = GROUP * tiles_n;
-  const int g = tile / per_group;
-  const int rows_in_group = min(GROUP, tiles_m - g * GROUP);
-  const int in_g = tile - g * per_group;
-  tm = g * GROUP + in_g % rows_in_group;
-  tn = in_g / rows_in_group;
-}
-
 // ---- direct-to-LDS kernel ---------------------------------------------------------
-// One static LDS array per ring stage and operand: distinct objects, so the compiler can
-// tell that the DMA into one stage does not alias the ds_reads of another and need not
-// wait for it.
-template <int Id, int Bytes>
-__shared__ __attribute__((aligned(1024))) char lds_ring[Bytes];
-
-typedef const __attribute__((address_space(1))) void *gptr_t;
-
-// 64 lanes x 16 bytes from per-lane global addresses to lds_dst[0..1023].
-__device__ __forceinline__ void dma16(const void *src, char *lds_dst) {
-  __builtin_amdgcn_global_load_lds((gptr_t)src, (LDS_PTR void *)lds_dst, 16, 0, 0);
-}
-
-// s_waitcnt immediate (gfx9 encoding) that waits for vmcnt <= n and lgkmcnt <= 0.
-constexpr int waitcnt_vm_lgkm0(int n) { return (n & 15) | ((n >> 4) << 14) | (7 << 4) | (0 << 8); }
-
-// Workgroup barrier without the fence __syncthreads() carries (which would drain every
-// outstanding DMA): callers wait for exactly the DMA they need first.
-__device__ __forceinline__ void barrier_no_fence() {
-  asm volatile("" ::: "memory");
-  __builtin_amdgcn_s_barrier();
-  asm volatile("" ::: "memory");
-}
-
 // BKT: K extent of one slab (32 or 64); NS: ring stages.  The DMA of slab s+NS is issued
 // after the barrier inside slab s, so NS-1 slabs of MFMA work cover its latency.
 // TJ: 32-column MFMA tiles per wave along N.  TJ = 2: 8 waves (2 x 4) of 128 x 64, two
@@ -255,15 +209,18 @@ __global__ __launch_bounds__(64 * 2 * (8 / TJ)) void gemm16_dma_kernel(const uin
 
   // Slab index past the end is clamped: the tail keeps issuing (redundant) DMA so that the
   // number of outstanding transfers per wave stays the same in every iteration.
+  // A: one resource for the tile's row panel, the slab selects a scalar byte offset.
+  // B: the resource is rebased to the slab's first row (keeps every offset below 2^31).
+  const __amdgpu_buffer_rsrc_t a_rsrc = make_rsrc(a_base, 0x80000000u);
   auto issue = [&](char *sa, char *sb, int slab) {
     const int sl = min(slab, nslabs - 1);
-    const char *ab = a_base + sl * (BKT * 2);
-    const char *bb = b_base + sl * b_slab_bytes;
+    const __amdgpu_buffer_rsrc_t b_rsrc = make_rsrc(b_base + sl * b_slab_bytes, 0x80000000u);
+    const uint32_t a_so = static_cast<uint32_t>(sl) * (BKT * 2);
 #pragma unroll
     for (int i = 0; i < DMA_PER_WAVE; ++i) {
       const int q = wave + NWAVES * i;
-      dma16(ab + a_off[i], sa + q * 1024);
-      dma16(bb + b_off[i], sb + q * 1024);
+      dma16(a_rsrc, a_off[i], a_so, sa + q * 1024);
+      dma16(b_rsrc, b_off[i], 0u, sb + q * 1024);
     }
   };
   auto load_frags = [&](const char *sa, const char *sb, int kk, u32x4 (&af)[4], u32x4 (&bf)[TJ]) {
@@ -537,7 +494,10 @@ int launch_gemm16(const uint16_t *a, const uint16_t *b, float *c, const float *b
   if (vec_ok && tunable("gemm16.force_simple", 0) == 0) {
     const int tiles_m = (m + BM - 1) / BM, tiles_n = (n + BN - 1) / BN;
     const int remap = (int)tunable("gemm.xcd_remap", 1);
-    if (k % BK == 0 && tunable("gemm16.force_staged", 0) == 0) {
+    // DMA offsets are 32-bit: 256 rows of A and 64 rows of B must span less than 2 GiB
+    const bool offsets_ok = static_cast<int64_t>(k) * 256 * 2 < 0x7FFFFFFF &&
+                            static_cast<int64_t>(n) * 64 * 2 < 0x7FFFFFFF;
+    if (k % BK == 0 && offsets_ok && tunable("gemm16.force_staged", 0) == 0) {
       const int ring = (int)tunable("gemm16.ring", 4), tj = (int)tunable("gemm16.tj", 2);
       const dim3 grid(tiles_m * tiles_n);
 #define SAREK_LAUNCH_DMA(BKT, NS, TJ)                                                             \

@@ -15,7 +15,10 @@
 // its A row with one ds_read_b128 (k = 8*kk + 4h + j, j = 0..3) and uses them over
 // four MFMA steps; the matching B values are row 8*kk + 4h + j, column n (ds_read_b32,
 // bank-conflict free because n is contiguous).
+#include <type_traits>
+
 #include "common.hpp"
+#include "gemm_common.hpp"
 #include "tunables.hpp"
 
 namespace sarek_hip {
@@ -26,7 +29,6 @@ typedef __attribute__((ext_vector_type(4))) float f32x4;
 
 constexpr int BM = 256, BN = 256, BK = 32;
 constexpr int THREADS = 512;
-constexpr int NUM_XCD = 8;   // XCDs of an MI355X; workgroup ids are dealt to them round-robin
 constexpr int A_STRIDE = BK + 4;            // floats per A row in LDS (36)
 constexpr int B_STRIDE = BN;                // floats per B row in LDS
 constexpr int A_FLOATS = BM * A_STRIDE;     // 9216
@@ -34,7 +36,7 @@ constexpr int B_FLOATS = BK * B_STRIDE;     // 8192
 constexpr int STAGE_FLOATS = A_FLOATS + B_FLOATS;
 constexpr int LDS_BYTES = 2 * STAGE_FLOATS * 4;  // 139264
 
-__global__ __launch_bounds__(THREADS) void gemm_f32_kernel(const float *__restrict__ A,
+__global__ __launch_bounds__(THREADS) void gemm_f32_staged_kernel(const float *__restrict__ A,
                                                            const float *__restrict__ B,
                                                            float *__restrict__ C, int M, int N,
                                                            int K, int tiles_m, int tiles_n, int xcd_remap) {
@@ -44,22 +46,8 @@ __global__ __launch_bounds__(THREADS) void gemm_f32_kernel(const float *__restri
   const int wm = wave >> 2, wn = wave & 3;
   const int lm = lane & 31, lh = lane >> 5;
 
-  // Workgroup -> tile.  The hardware deals consecutive workgroup ids round-robin to the
-  // 8 XCDs (each with its own L2), so ids are first regrouped to give every XCD one
-  // contiguous run of tiles, and the run is walked in bands of GROUP tile-rows, column by
-  // column: the ~32 tiles an XCD has in flight then form a compact GROUP x 4 patch that
-  // moves through K together and shares A row-panels and B column-panels in that L2.
-  const int nblocks = tiles_m * tiles_n;
-  const int xcd = blockIdx.x % NUM_XCD, slot = blockIdx.x / NUM_XCD;
-  int tile = xcd * (nblocks / NUM_XCD) + min(xcd, nblocks % NUM_XCD) + slot;
-  if (xcd_remap == 0) tile = blockIdx.x;
-  const int GROUP = xcd_remap > 1 ? xcd_remap : 8;   // tile-rows per raster band
-  const int per_group = GROUP * tiles_n;
-  const int g = tile / per_group;
-  const int rows_in_group = min(GROUP, tiles_m - g * GROUP);
-  const int in_g = tile - g * per_group;
-  const int tm = g * GROUP + in_g % rows_in_group;
-  const int tn = in_g / rows_in_group;
+  int tm, tn;
+  tile_of_block(tiles_m, tiles_n, xcd_remap, tm, tn);
   const int m0 = tm * BM, n0 = tn * BN;
 
   f32x4 ra[4], rb[4];
@@ -158,6 +146,203 @@ __global__ __launch_bounds__(THREADS) void gemm_f32_kernel(const float *__restri
     }
 }
 
+// ---- direct-to-LDS ring kernel ------------------------------------------------------
+// Tile = (32*TI*WMW) x (32*TJ*WNW), WMW x WNW waves, each wave TI x TJ MFMA tiles of 32 x 32.
+// K slabs of BKT stream through NS LDS stages by global_load_lds_dwordx4 (no staging
+// registers, no ds_write); the pipeline is the one of the 16-bit GEMM: DMA of slab s+NS
+// issued after the barrier inside slab s, barrier before the last k-step of a slab, next
+// slab's first fragments fetched under that step's MFMAs.
+//
+// k-step = 8 k.  A: lane (m, h) reads k = 8kk+4h .. +3 of its row with one ds_read_b128 and
+// feeds them to four MFMA steps j; B: for step j the lane reads row 8kk+4h+j at columns
+// TJ*lane .. TJ*lane+TJ-1 of the wave's span (one ds_read of TJ floats): MFMA tile jn of the
+// wave therefore holds columns {TJ*l + jn}, and in the epilogue every lane owns TJ adjacent
+// columns of C, stored as one vector.
+//
+// LDS (64 banks x 4 B): A rows of 64 B: slot ^= (row>>2)&3, rows of 128 B: slot ^= (row>>1)&7
+// (16-lane phases of ds_read_b128).  B reads are contiguous across lanes; only for TJ = 1
+// the two half-waves (rows r, r+4) would meet modulo 256 B, so rows with bit 2 set are
+// stored with their 128-byte halves swapped.
+template <int TI, int TJ, int WMW, int WNW, int BKT, int NS>
+__global__ __launch_bounds__(64 * WMW * WNW) void gemm_f32_dma_kernel(
+    const float *__restrict__ A, const float *__restrict__ B, float *__restrict__ C, int M, int N,
+    int K, int tiles_m, int tiles_n, int xcd_remap) {
+  typedef __attribute__((ext_vector_type(TJ))) float bvec_t;
+  constexpr int BMT = 32 * TI * WMW, BNT = 32 * TJ * WNW, NWAVES = WMW * WNW;
+  constexpr int KK = BKT / 8;
+  constexpr int A_ROW = BKT * 4, A_CHUNKS = A_ROW / 16, A_ROWS_PER_DMA = 1024 / A_ROW;
+  constexpr int B_ROW = BNT * 4, B_CHUNKS = B_ROW / 16, B_ROWS_PER_DMA = 1024 / B_ROW;
+  constexpr int A_BYTES_S = BMT * A_ROW, B_BYTES_S = BKT * B_ROW;
+  constexpr int A_DMA = A_BYTES_S / 1024 / NWAVES, B_DMA = B_BYTES_S / 1024 / NWAVES;
+  static_assert(A_DMA >= 1 && B_DMA >= 1 && A_DMA * 1024 * NWAVES == A_BYTES_S &&
+                    B_DMA * 1024 * NWAVES == B_BYTES_S, "slab does not split over the waves");
+  static_assert(A_ROW == 64 || A_ROW == 128, "BKT must be 16 or 32");
+  static_assert(B_ROW <= 1024 && NS * (A_BYTES_S + B_BYTES_S) <= 160 * 1024, "LDS layout");
+  static_assert((NS - 1) * (A_DMA + B_DMA) < 64, "vmcnt range");
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int wm = wave / WNW, wn = wave % WNW;
+  const int lm = lane & 31, lh = lane >> 5;
+  int tm, tn;
+  tile_of_block(tiles_m, tiles_n, xcd_remap, tm, tn);
+  const int m0 = tm * BMT, n0 = tn * BNT;
+
+  auto a_swz = [](int row) { return A_CHUNKS == 8 ? ((row >> 1) & 7) : ((row >> 2) & 3); };
+  auto b_swz = [](int row) { return TJ == 1 ? (((row >> 2) & 1) << 3) : 0; };
+
+  // DMA sources: uniform 64-bit base + per-lane 32-bit byte offset.  Rows past M and columns
+  // past N are clamped to valid addresses; what they produce is never stored.
+  uint32_t a_off[A_DMA], b_off[B_DMA];
+#pragma unroll
+  for (int i = 0; i < A_DMA; ++i) {
+    const int q = wave + NWAVES * i;
+    const int row_t = q * A_ROWS_PER_DMA + lane / A_CHUNKS;
+    const int row = min(row_t, M - 1 - m0);
+    a_off[i] = (static_cast<uint32_t>(row) * K + (((lane % A_CHUNKS) ^ a_swz(row_t)) << 2)) * 4u;
+  }
+#pragma unroll
+  for (int i = 0; i < B_DMA; ++i) {
+    const int q = wave + NWAVES * i;
+    const int brow = q * B_ROWS_PER_DMA + lane / B_CHUNKS;
+    const int chunk = (lane % B_CHUNKS) ^ b_swz(brow);
+    const int col = min(n0 + chunk * 4, N - 4);
+    b_off[i] = (static_cast<uint32_t>(brow) * N + col) * 4u;
+  }
+  const char *a_base = reinterpret_cast<const char *>(A + static_cast<int64_t>(m0) * K);
+  const char *b_base = reinterpret_cast<const char *>(B);
+  const int64_t b_slab_bytes = static_cast<int64_t>(BKT) * N * 4;
+  const int nslabs = K / BKT;
+
+  f32x16 acc[TI][TJ];
+#pragma unroll
+  for (int i = 0; i < TI; ++i)
+#pragma unroll
+    for (int j = 0; j < TJ; ++j)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
+
+  const int a_row = wm * 32 * TI + lm;
+  int a_addr0 = a_row * A_ROW + ((lh ^ a_swz(a_row)) << 4);           // ^ (kk << 5), + i*32*A_ROW
+  int b_addr0 = (4 * lh) * B_ROW + (((wn * 32 * TJ + TJ * lm) * 4) ^ (TJ == 1 ? (lh << 7) : 0));
+
+  // A: one resource for the tile's row panel, the slab selects a scalar byte offset.
+  // B: the resource is rebased to the slab's first row (keeps every offset below 2^31).
+  const __amdgpu_buffer_rsrc_t a_rsrc = make_rsrc(a_base, 0x80000000u);
+  auto issue = [&](char *sa, char *sb, int slab) {
+    const int sl = min(slab, nslabs - 1);   // the tail re-issues the last slab: constant vmcnt
+    const __amdgpu_buffer_rsrc_t b_rsrc = make_rsrc(b_base + sl * b_slab_bytes, 0x80000000u);
+    const uint32_t a_so = static_cast<uint32_t>(sl) * (BKT * 4);
+#pragma unroll
+    for (int i = 0; i < A_DMA; ++i) dma16(a_rsrc, a_off[i], a_so, sa + (wave + NWAVES * i) * 1024);
+#pragma unroll
+    for (int i = 0; i < B_DMA; ++i) dma16(b_rsrc, b_off[i], 0u, sb + (wave + NWAVES * i) * 1024);
+  };
+  auto load_frags = [&](const char *sa, const char *sb, int kk, f32x4 (&af)[TI], bvec_t (&bf)[4]) {
+    const char *pa = sa + (a_addr0 ^ (kk << 5));
+#pragma unroll
+    for (int i = 0; i < TI; ++i) af[i] = *reinterpret_cast<const f32x4 *>(pa + i * 32 * A_ROW);
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+      bf[j] = *reinterpret_cast<const bvec_t *>(sb + b_addr0 + (kk * 8 + j) * B_ROW);
+  };
+  auto mfma_step = [&](f32x4 (&af)[TI], bvec_t (&bf)[4]) {
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+#pragma unroll
+      for (int i = 0; i < TI; ++i)
+#pragma unroll
+        for (int jn = 0; jn < TJ; ++jn) {
+          acc[i][jn] = __builtin_amdgcn_mfma_f32_32x32x2f32(af[i][j], bf[j][jn], acc[i][jn], 0, 0, 0);
+        }
+  };
+  auto interleave = [] {
+    constexpr int READS = TI + 4, MFMAS = 4 * TI * TJ;
+    constexpr int GROUPS = READS < MFMAS ? READS : MFMAS;
+    constexpr int PER = (READS + GROUPS - 1) / GROUPS;
+#pragma unroll
+    for (int g = 0; g < GROUPS; ++g) {
+      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);    // 1 MFMA
+      __builtin_amdgcn_sched_group_barrier(0x100, PER, 0);  // DS reads
+    }
+    if (MFMAS > GROUPS) __builtin_amdgcn_sched_group_barrier(0x008, MFMAS - GROUPS, 0);
+    __builtin_amdgcn_sched_barrier(0);
+  };
+
+  f32x4 af[2][TI];
+  bvec_t bf[2][4];
+
+  auto slab = [&](char *ca, char *cb, const char *na, const char *nb, int s) {
+    asm volatile("" : "+v"(a_addr0), "+v"(b_addr0));   // keep per-stage addresses out of registers
+#pragma unroll
+    for (int kk = 0; kk + 1 < KK; ++kk) {
+      load_frags(ca, cb, kk + 1, af[(kk + 1) & 1], bf[(kk + 1) & 1]);
+      mfma_step(af[kk & 1], bf[kk & 1]);
+      interleave();
+    }
+    __builtin_amdgcn_s_waitcnt(waitcnt_vm_lgkm0((NS - 2) * (A_DMA + B_DMA)));
+    barrier_no_fence();
+    issue(ca, cb, s + NS);
+    load_frags(na, nb, 0, af[0], bf[0]);
+    mfma_step(af[(KK - 1) & 1], bf[(KK - 1) & 1]);
+    interleave();
+  };
+
+  issue(lds_ring<0, A_BYTES_S>, lds_ring<1, B_BYTES_S>, 0);
+  issue(lds_ring<2, A_BYTES_S>, lds_ring<3, B_BYTES_S>, 1);
+  if constexpr (NS == 4) {
+    issue(lds_ring<4, A_BYTES_S>, lds_ring<5, B_BYTES_S>, 2);
+    issue(lds_ring<6, A_BYTES_S>, lds_ring<7, B_BYTES_S>, 3);
+  }
+  __builtin_amdgcn_s_waitcnt(waitcnt_vm_lgkm0((NS - 1) * (A_DMA + B_DMA)));
+  barrier_no_fence();
+  load_frags(lds_ring<0, A_BYTES_S>, lds_ring<1, B_BYTES_S>, 0, af[0], bf[0]);
+  __builtin_amdgcn_sched_barrier(0);
+
+  auto ring_slab = [&](auto st_c, int s) {
+    constexpr int st = decltype(st_c)::value;
+    constexpr int nx = (st + 1) % NS;
+    slab(lds_ring<2 * st, A_BYTES_S>, lds_ring<2 * st + 1, B_BYTES_S>, lds_ring<2 * nx, A_BYTES_S>,
+         lds_ring<2 * nx + 1, B_BYTES_S>, s);
+  };
+  using I0 = std::integral_constant<int, 0>;
+  using I1 = std::integral_constant<int, 1>;
+  using I2 = std::integral_constant<int, 2>;
+  using I3 = std::integral_constant<int, 3>;
+  const int full = nslabs - nslabs % NS;
+  for (int s = 0; s < full; s += NS) {
+    ring_slab(I0{}, s);
+    ring_slab(I1{}, s + 1);
+    if constexpr (NS == 4) {
+      ring_slab(I2{}, s + 2);
+      ring_slab(I3{}, s + 3);
+    }
+  }
+  if (full < nslabs) ring_slab(I0{}, full);
+  if constexpr (NS == 4) {
+    if (full + 1 < nslabs) ring_slab(I1{}, full + 1);
+    if (full + 2 < nslabs) ring_slab(I2{}, full + 2);
+  }
+  __builtin_amdgcn_s_waitcnt(waitcnt_vm_lgkm0(0));   // drain the redundant tail DMA
+
+  // Epilogue: register r of lane l holds row 8*(r/4) + 4*(l/32) + r%4 of its 32-row tile and
+  // columns TJ*(l%32) .. +TJ-1 of the wave's span (one per MFMA tile jn).
+#pragma unroll
+  for (int i = 0; i < TI; ++i)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+      const int row = m0 + wm * 32 * TI + i * 32 + 8 * (r >> 2) + 4 * lh + (r & 3);
+      const int col = n0 + wn * 32 * TJ + TJ * lm;
+      if (row < M && col < N) {
+        bvec_t v;
+#pragma unroll
+        for (int jn = 0; jn < TJ; ++jn) v[jn] = acc[i][jn][r];
+        *reinterpret_cast<bvec_t *>(C + static_cast<int64_t>(row) * N + col) = v;
+      }
+    }
+}
+
 // Any shape, any alignment: one thread per C element, f32 FMA in k order.
 __global__ __launch_bounds__(256) void gemm_f32_simple_kernel(const float *__restrict__ A,
                                                               const float *__restrict__ B,
@@ -187,15 +372,35 @@ extern "C" int sarek_hip_gemm_f32(const float *a, const float *b, float *c, int 
                       (reinterpret_cast<uintptr_t>(a) % 16 == 0) &&
                       (reinterpret_cast<uintptr_t>(b) % 16 == 0);
   if (vec_ok && tunable("gemm_f32.force_simple", 0) == 0) {
+    const int remap = (int)tunable("gemm.xcd_remap", 1);
+    // DMA offsets are 32-bit: 256 rows of A and 32 rows of B must span less than 2 GiB
+    const bool offsets_ok = static_cast<int64_t>(k) * 256 * 4 < 0x7FFFFFFF &&
+                            static_cast<int64_t>(n) * 32 * 4 < 0x7FFFFFFF;
+    if (k % 32 == 0 && offsets_ok && reinterpret_cast<uintptr_t>(c) % 16 == 0 &&
+        tunable("gemm_f32.force_staged", 0) == 0) {
+      // Tile choice: the largest tile that still gives every CU at least two workgroups.
+      auto ntiles = [&](int t) { return static_cast<int64_t>((m + t - 1) / t) * ((n + t - 1) / t); };
+      int tile = (int)tunable("gemm_f32.tile", 0);
+      if (tile == 0) tile = ntiles(256) >= 512 ? 256 : ntiles(128) >= 512 ? 128 : 64;
+#define SAREK_LAUNCH_F32(T, TI, TJ, WMW, WNW, BKT)                                               \
+  hipLaunchKernelGGL((gemm_f32_dma_kernel<TI, TJ, WMW, WNW, BKT, 4>),                             \
+                     dim3((unsigned)ntiles(T)), dim3(64 * WMW * WNW), 0, st, a, b, c, m, n, k,    \
+                     (m + T - 1) / T, (n + T - 1) / T, remap)
+      if (tile == 256) SAREK_LAUNCH_F32(256, 4, 2, 2, 4, 16);
+      else if (tile == 128) SAREK_LAUNCH_F32(128, 2, 2, 2, 2, 16);
+      else SAREK_LAUNCH_F32(64, 1, 1, 2, 2, 32);
+#undef SAREK_LAUNCH_F32
+      return check_launch("gemm_f32 kernel launch");
+    }
     static bool attr_done = false;
     if (!attr_done) {
-      SAREK_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(gemm_f32_kernel),
+      SAREK_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(gemm_f32_staged_kernel),
                                         hipFuncAttributeMaxDynamicSharedMemorySize, LDS_BYTES));
       attr_done = true;
     }
     const int tiles_m = (m + BM - 1) / BM, tiles_n = (n + BN - 1) / BN;
-    hipLaunchKernelGGL(gemm_f32_kernel, dim3(tiles_m * tiles_n), dim3(THREADS), LDS_BYTES, st, a, b,
-                       c, m, n, k, tiles_m, tiles_n, (int)tunable("gemm.xcd_remap", 1));
+    hipLaunchKernelGGL(gemm_f32_staged_kernel, dim3(tiles_m * tiles_n), dim3(THREADS), LDS_BYTES, st, a, b,
+                       c, m, n, k, tiles_m, tiles_n, remap);
   } else {
     hipLaunchKernelGGL(gemm_f32_simple_kernel, dim3((n + 63) / 64, (m + 3) / 4), dim3(256), 0, st,
                        a, b, c, m, n, k);
