@@ -29,10 +29,10 @@ PEAK_HBM_GBS = 8000.0          # MI355X HBM3E
 # HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (KiB per dispatch,
 # FETCH_SIZE scaled by 2.0 and WRITE_SIZE by 1.0 after calibration against a plain 1 GiB copy).
 MEASURED_TRAFFIC_BYTES = {
-    "triad_sum_2p28": (1048600 * 2 + 1048700) * 1024,
-    "gemm_bf16_8192": (817384 * 2 + 262144) * 1024,
-    "gemm_f32_8192": (1579270 * 2 + 262144) * 1024,
-    "gemm_f16_epilogue": (313832 * 2 + 187093) * 1024,
+    "triad_sum_2p28": (1048592 * 2 + 1050631) * 1024,
+    "gemm_bf16_8192": (800150 * 2 + 262144) * 1024,
+    "gemm_f32_8192": (1747126 * 2 + 262144) * 1024,
+    "gemm_f16_epilogue": (308713 * 2 + 187093) * 1024,
 }
 PEAK_MFMA_TFLOPS = {"bf16": 2500.0, "f16": 2500.0, "f32": 157.3}
 
@@ -106,7 +106,7 @@ def make_workload(name, torch, hip):
         c = torch.empty(s, s, device="cuda")
         info = dict(metric=f"f32 GEMM {s}^3 TFLOP/s", unit="TFLOP/s", dtype="f32",
                     work=2.0 * s ** 3, work_unit=1e12, bound="mfma", peak=PEAK_MFMA_TFLOPS["f32"],
-                    kernel="gemm_f32_kernel",
+                    kernel="gemm_f32_dma_kernel",
                     config={"workload": f"f32 GEMM C=A.B row-major, U[-1,1)", "m": s, "n": s, "k": s})
         return (lambda: hip.gemm_f32(a, b, out=c)), info
     if name == "gemm_bf16_8192":
