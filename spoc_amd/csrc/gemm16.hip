@@ -18,8 +18,9 @@
 //
 // Three kernels:
 //   gemm16_dma_kernel (K % 64 == 0, the fast path): global -> LDS by
-//     global_load_lds_dwordx4, which writes the 64 lanes' 16-byte pieces to 1 KiB of
-//     consecutive LDS with no register staging and no ds_write.  Rows cannot be padded that
+//     buffer_load_dwordx4 ... lds, which writes the 64 lanes' 16-byte pieces to 1 KiB of
+//     consecutive LDS with no register staging and no ds_write (the buffer form: the
+//     global_load form of the same transfer slows MFMA issue down).  Rows cannot be padded that
 //     way, so bank conflicts are removed by an XOR swizzle applied on the global-address
 //     side (which chunk a lane fetches) and again by the readers.  K slabs of 32 stream
 //     through a ring of 4 LDS stages (128 KiB): the DMA of slab s+4 is issued right after
@@ -59,6 +60,7 @@ constexpr int LDS_BYTES = 2 * STAGE_BYTES;  // 143360
 
 enum { EPI_STORE = 0, EPI_BIAS_RELU_ROWSUM = 1 };
 
+
 template <bool Bf16>
 __device__ __forceinline__ f32x16 mfma(u32x4 a, u32x4 b, f32x16 c) {
   if constexpr (Bf16)
@@ -76,40 +78,81 @@ __device__ __forceinline__ u32x2 lds_read_tr16(const char *lds, int off) {
   return __builtin_bit_cast(u32x2, v);
 }
 
-// Sum over the 32 lanes of each half-wave; valid in every lane of the half.
-__device__ __forceinline__ float half_wave_sum(float v) {
-  for (int off = 16; off >= 1; off >>= 1) v += __shfl_xor(v, off, 64);
-  return v;
-}
-
 // Writes one wave's 128 x (32*TJ) accumulator block.  Accumulator layout of the 32x32 MFMA:
 // register r of lane l holds row 8*(r/4) + 4*(l/32) + r%4, column l%32 of its tile.
+//
+// Fused form: y = relu(acc + bias[col]) is stored, and the row sums of the workgroup's
+// 256 x 256 tile are formed before anything goes to memory:
+//   1. per lane: sum over its TJ columns -> 64 values, one per row the lane touches
+//      (index q = 16*i + r);
+//   2. across the 32 lanes of a half-wave (which share those 64 rows) by a halving
+//      butterfly: at the step with lane mask m a lane keeps one half of its values and
+//      receives the partner's sums for that half, so 32+16+8+4+2 exchanges leave lane lm
+//      with the sums of rows q = 2*lm and 2*lm+1;
+//   3. across the WN waves that share the rows through `scratch` (LDS, WN x 256 floats; all
+//      waves must be done with the LDS ring: barriers inside), then one atomicAdd per row.
 template <int Epi, int TJ>
 __device__ __forceinline__ void epilogue(f32x16 (&acc)[4][TJ], float *__restrict__ C,
                                          const float *__restrict__ bias,
-                                         float *__restrict__ rowsum, int M, int N, int row0,
-                                         int col0, int lm, int lh) {
+                                         float *__restrict__ rowsum, int M, int N, int m0,
+                                         int wm, int wn, int col0, int lm, int lh,
+                                         float *scratch) {
+  constexpr int WN = 8 / TJ;
+  const int row0 = m0 + wm * 128;
+  float bj[TJ];
+  bool cok[TJ];
+#pragma unroll
+  for (int j = 0; j < TJ; ++j) {
+    const int col = col0 + j * 32 + lm;
+    cok[j] = col < N;
+    bj[j] = (Epi == EPI_BIAS_RELU_ROWSUM && cok[j]) ? bias[col] : 0.f;
+  }
+  float rs[64];
 #pragma unroll
   for (int i = 0; i < 4; ++i) {
 #pragma unroll
     for (int r = 0; r < 16; ++r) {
       const int row = row0 + i * 32 + 8 * (r >> 2) + 4 * lh + (r & 3);
-      float rs = 0.f;
+      float sum = 0.f;
 #pragma unroll
       for (int j = 0; j < TJ; ++j) {
-        const int col = col0 + j * 32 + lm;
         float v = acc[i][j][r];
         if (Epi == EPI_BIAS_RELU_ROWSUM) {
-          v += (col < N) ? bias[col] : 0.f;
+          v += bj[j];
           v = v > 0.f ? v : 0.f;
-          if (col < N) rs += v;
+          sum += cok[j] ? v : 0.f;
         }
-        if (row < M && col < N) C[static_cast<int64_t>(row) * N + col] = v;
+        if (row < M && cok[j]) C[static_cast<int64_t>(row) * N + col0 + j * 32 + lm] = v;
       }
-      if (Epi == EPI_BIAS_RELU_ROWSUM) {
-        rs = half_wave_sum(rs);
-        if (lm == 0 && row < M) atomicAdd(rowsum + row, rs);
+      rs[i * 16 + r] = sum;
+    }
+  }
+  if constexpr (Epi == EPI_BIAS_RELU_ROWSUM) {
+#pragma unroll
+    for (int step = 0; step < 5; ++step) {
+      const int m = 16 >> step, half = 32 >> step;
+      const bool up = (lm & m) != 0;
+#pragma unroll
+      for (int q = 0; q < half; ++q) {
+        const float send = up ? rs[q] : rs[q + half];
+        const float keep = up ? rs[q + half] : rs[q];
+        rs[q] = keep + __shfl_xor(send, m, 64);
       }
+    }
+    // lane lm now holds rows q = 2*lm + e (e = 0, 1) of its half-wave's row set
+    __syncthreads();  // every wave has left the K loop: the LDS ring is free
+#pragma unroll
+    for (int e = 0; e < 2; ++e) {
+      const int q = 2 * lm + e, i = q >> 4, r = q & 15;
+      scratch[wn * 256 + wm * 128 + i * 32 + 8 * (r >> 2) + 4 * lh + (r & 3)] = rs[e];
+    }
+    __syncthreads();
+    const int t = threadIdx.x;
+    if (t < 256 && m0 + t < M) {
+      float total = 0.f;
+#pragma unroll
+      for (int w = 0; w < WN; ++w) total += scratch[w * 256 + t];
+      atomicAdd(rowsum + m0 + t, total);
     }
   }
 }
@@ -212,16 +255,21 @@ __global__ __launch_bounds__(64 * 2 * (8 / TJ)) void gemm16_dma_kernel(const uin
   // A: one resource for the tile's row panel, the slab selects a scalar byte offset.
   // B: the resource is rebased to the slab's first row (keeps every offset below 2^31).
   const __amdgpu_buffer_rsrc_t a_rsrc = make_rsrc(a_base, 0x80000000u);
-  auto issue = [&](char *sa, char *sb, int slab) {
+  auto issue_a = [&](char *sa, int slab) {
     const int sl = min(slab, nslabs - 1);
-    const __amdgpu_buffer_rsrc_t b_rsrc = make_rsrc(b_base + sl * b_slab_bytes, 0x80000000u);
     const uint32_t a_so = static_cast<uint32_t>(sl) * (BKT * 2);
 #pragma unroll
-    for (int i = 0; i < DMA_PER_WAVE; ++i) {
-      const int q = wave + NWAVES * i;
-      dma16(a_rsrc, a_off[i], a_so, sa + q * 1024);
-      dma16(b_rsrc, b_off[i], 0u, sb + q * 1024);
-    }
+    for (int i = 0; i < DMA_PER_WAVE; ++i) dma16(a_rsrc, a_off[i], a_so, sa + (wave + NWAVES * i) * 1024);
+  };
+  auto issue_b = [&](char *sb, int slab) {
+    const int sl = min(slab, nslabs - 1);
+    const __amdgpu_buffer_rsrc_t b_rsrc = make_rsrc(b_base + sl * b_slab_bytes, 0x80000000u);
+#pragma unroll
+    for (int i = 0; i < DMA_PER_WAVE; ++i) dma16(b_rsrc, b_off[i], 0u, sb + (wave + NWAVES * i) * 1024);
+  };
+  auto issue = [&](char *sa, char *sb, int slab) {
+    issue_a(sa, slab);
+    issue_b(sb, slab);
   };
   auto load_frags = [&](const char *sa, const char *sb, int kk, u32x4 (&af)[4], u32x4 (&bf)[TJ]) {
     const char *pa = sa + (a_addr0 ^ (kk << 5));
@@ -260,13 +308,16 @@ __global__ __launch_bounds__(64 * 2 * (8 / TJ)) void gemm16_dma_kernel(const uin
   u32x4 af[2][4], bf[2][TJ];
 
   // One slab: stage `cur` is consumed, `nxt` is the stage of slab s+1; after the barrier
-  // every wave is done reading `cur`, so it is refilled with slab s+NS.
-  auto slab = [&](char *ca, char *cb, const char *na, const char *nb, int s) {
+  // every wave is done reading `cur`, so it is refilled with slab s+NS: the A half right
+  // away, the B half one k-step later (at the top of the next slab, into `pb`, the stage
+  // consumed before this one), which spreads the requests over the slab.
+  auto slab = [&](char *ca, char *cb, const char *na, const char *nb, char *pb, int s) {
     // Keep the per-stage LDS addresses from being hoisted out of the K loop (they would
     // occupy a register per stage and k-step): the bases are made opaque once per slab.
     asm volatile("" : "+v"(a_addr0), "+v"(b_addr0));
 #pragma unroll
     for (int kk = 0; kk + 1 < KK; ++kk) {
+      if (kk == 0) issue_b(pb, s - 1 + NS);
       load_frags(ca, cb, kk + 1, af[(kk + 1) & 1], bf[(kk + 1) & 1]);
       mfma_step(af[kk & 1], bf[kk & 1]);
       interleave();
@@ -274,20 +325,21 @@ __global__ __launch_bounds__(64 * 2 * (8 / TJ)) void gemm16_dma_kernel(const uin
     // own DMA of slab s+1 landed (NS-2 later slabs may still be in flight), own reads done
     __builtin_amdgcn_s_waitcnt(waitcnt_vm_lgkm0((NS - 2) * 2 * DMA_PER_WAVE));
     barrier_no_fence();
-    issue(ca, cb, s + NS);
+    issue_a(ca, s + NS);
     load_frags(na, nb, 0, af[0], bf[0]);
     mfma_step(af[(KK - 1) & 1], bf[(KK - 1) & 1]);
     interleave();
   };
 
-  // prologue: fill the ring, wait for slab 0, fetch its first fragments
+  // prologue: fill the ring (the B half of the last stage follows in slab 0), wait for
+  // slab 0, fetch its first fragments
   issue(lds_ring<0, A_BYTES_S>, lds_ring<1, B_BYTES_S>, 0);
-  issue(lds_ring<2, A_BYTES_S>, lds_ring<3, B_BYTES_S>, 1);
   if constexpr (NS == 4) {
+    issue(lds_ring<2, A_BYTES_S>, lds_ring<3, B_BYTES_S>, 1);
     issue(lds_ring<4, A_BYTES_S>, lds_ring<5, B_BYTES_S>, 2);
-    issue(lds_ring<6, A_BYTES_S>, lds_ring<7, B_BYTES_S>, 3);
   }
-  __builtin_amdgcn_s_waitcnt(waitcnt_vm_lgkm0((NS - 1) * 2 * DMA_PER_WAVE));
+  issue_a(lds_ring<2 * (NS - 1), A_BYTES_S>, NS - 1);
+  __builtin_amdgcn_s_waitcnt(waitcnt_vm_lgkm0((NS - 2) * 2 * DMA_PER_WAVE + DMA_PER_WAVE));
   barrier_no_fence();
   load_frags(lds_ring<0, A_BYTES_S>, lds_ring<1, B_BYTES_S>, 0, af[0], bf[0]);
   __builtin_amdgcn_sched_barrier(0);
@@ -297,9 +349,9 @@ __global__ __launch_bounds__(64 * 2 * (8 / TJ)) void gemm16_dma_kernel(const uin
   // remaining nslabs % NS slabs.
   auto ring_slab = [&](auto st_c, int s) {
     constexpr int st = decltype(st_c)::value;
-    constexpr int nx = (st + 1) % NS;
+    constexpr int nx = (st + 1) % NS, pv = (st + NS - 1) % NS;
     slab(lds_ring<2 * st, A_BYTES_S>, lds_ring<2 * st + 1, B_BYTES_S>, lds_ring<2 * nx, A_BYTES_S>,
-         lds_ring<2 * nx + 1, B_BYTES_S>, s);
+         lds_ring<2 * nx + 1, B_BYTES_S>, lds_ring<2 * pv + 1, B_BYTES_S>, s);
   };
   using I0 = std::integral_constant<int, 0>;
   using I1 = std::integral_constant<int, 1>;
@@ -321,7 +373,8 @@ __global__ __launch_bounds__(64 * 2 * (8 / TJ)) void gemm16_dma_kernel(const uin
   }
   // drain the (redundant) tail DMA before the LDS is released
   __builtin_amdgcn_s_waitcnt(waitcnt_vm_lgkm0(0));
-  epilogue<Epi, TJ>(acc, C, bias, rowsum, M, N, m0 + wm * 128, n0 + wn * (32 * TJ), lm, lh);
+  epilogue<Epi, TJ>(acc, C, bias, rowsum, M, N, m0, wm, wn, n0 + wn * (32 * TJ), lm, lh,
+                    reinterpret_cast<float *>(lds_ring<0, A_BYTES_S>));
 }
 
 template <bool Bf16, int Epi>
@@ -429,7 +482,8 @@ __global__ __launch_bounds__(THREADS) void gemm16_staged_kernel(const uint16_t *
     __syncthreads();
   }
 
-  epilogue<Epi, 2>(acc, C, bias, rowsum, M, N, m0 + wm * 128, n0 + wn * 64, lm, lh);
+  epilogue<Epi, 2>(acc, C, bias, rowsum, M, N, m0, wm, wn, n0 + wn * 64, lm, lh,
+                   reinterpret_cast<float *>(lds));
 }
 
 // Any shape, any alignment: one thread per C element, f32 accumulate in k order.
