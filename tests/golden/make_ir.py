@@ -244,11 +244,127 @@ def mandelbrot():
     return kernel(params, body)
 
 
+def reduction_max():
+    fresh()
+    params = [("input", "(vec f32)"), ("output", "(vec f32)"), ("n", "i32")]
+    for p, t in params:
+        var(p, t)
+    n = var("n")
+    sdata = var("sdata", "(array f32 shared)")
+    tid, gid = var("tid"), var("gid")
+    # the golden text was generated from a source that wrote Float.neg_infinity: a global
+    # reference, which lowers to a plain variable of that name (Sarek_lower_ir.ml:378-380)
+    ninf = var("Float.neg_infinity", "f32")
+    steps = [block(if_(lt(gid, n), assign_elem("sdata", tid, read("input", gid)),
+                       assign_elem("sdata", tid, ninf))), BARRIER]
+    half = 128
+    while half >= 1:
+        a, b = var("a%d" % half, "f32"), var("b%d" % half, "f32")
+        a, b = a.replace("a%d" % half, "a", 1), b.replace("b%d" % half, "b", 1)
+        steps += [block(if_(lt(tid, i32(half)),
+                            let(a, read("sdata", tid),
+                                let(b, read("sdata", add(tid, i32(half))),
+                                    if_(gt(b, a), assign_elem("sdata", tid, b)))))), BARRIER]
+        half //= 2
+    steps += [block(if_(eq(tid, i32(0)), assign_elem("output", intr("block_idx_x"), read("sdata", i32(0))))),
+              BARRIER]
+    body = shared(sdata, "f32", 256, lets(
+        [(tid, intr("thread_idx_x")),
+         (gid, add(intr("thread_idx_x"), mul(intr("block_dim_x"), intr("block_idx_x"))))],
+        seq(*steps)))
+    return kernel(params, body)
+
+
+def transpose_tiled():
+    fresh()
+    params = [("input", "(vec f32)"), ("output", "(vec f32)"), ("width", "i32"), ("height", "i32")]
+    for p, t in params:
+        var(p, t)
+    w, h = var("width"), var("height")
+    tile = var("tile", "(array f32 shared)")
+    ts, tx, ty = var("tile_size"), var("tx"), var("ty")
+    bc, br, rc, rr = var("block_col"), var("block_row"), var("read_col"), var("read_row")
+    ri, ti = var("read_idx"), var("tile_idx")
+    wc, wr = var("write_col"), var("write_row")
+    ti2, wi = var("tile_idx2"), var("write_idx")
+    ti2 = ti2.replace("tile_idx2", "tile_idx", 1)
+    load = block(if_(land(lt(rc, w), lt(rr, h)),
+                     let(ri, add(mul(rr, w), rc),
+                         let(ti, add(mul(ty, i32(17)), tx),
+                             assign_elem("tile", ti, read("input", ri))))))
+    store = block(if_(land(lt(wc, h), lt(wr, w)),
+                      let(ti2, add(mul(tx, i32(17)), ty),
+                          let(wi, add(mul(wr, h), wc),
+                              assign_elem("output", wi, read("tile", ti2))))))
+    body = shared(tile, "f32", 272, lets(
+        [(ts, i32(16)), (tx, intr("thread_idx_x")), (ty, intr("thread_idx_y")),
+         (bc, mul(intr("block_idx_x"), ts)), (br, mul(intr("block_idx_y"), ts)),
+         (rc, add(bc, tx)), (rr, add(br, ty))],
+        seq(load, BARRIER, lets([(wc, add(br, tx)), (wr, add(bc, ty))], seq(store, BARRIER)))))
+    return kernel(params, body)
+
+
+def scatter():
+    fresh()
+    params = [("input", "(vec i32)"), ("indices", "(vec i32)"), ("output", "(vec i32)"), ("n", "i32")]
+    for p, t in params:
+        var(p, t)
+    i, idx = var("i"), var("idx")
+    body = let(i, intr("global_thread_id", "Std"),
+               if_(lt(i, var("n")), let(idx, read("indices", i), assign_elem("output", idx, read("input", i)))))
+    return kernel(params, body)
+
+
+def radix_sort_histogram():
+    fresh()
+    params = [("input", "(vec i32)"), ("histogram", "(vec i32)"), ("n", "i32"), ("shift", "i32"), ("mask", "i32")]
+    for p, t in params:
+        var(p, t)
+    n, shift, mask = var("n"), var("shift"), var("mask")
+    lh = var("local_hist", "(array i32 shared)")
+    hist = var("histogram", "(vec i32)")
+    tid, gid, nb = var("tid"), var("gid"), var("num_bins")
+    value, digit = var("value"), var("digit")
+    old1, old2 = var("_old"), var("_old2").replace("_old2", "_old", 1)
+    clear = block(if_(lt(tid, nb), assign_elem("local_hist", tid, i32(0))))
+    count = block(if_(lt(gid, n),
+                      let(value, read("input", gid),
+                          let(digit, op("bitand", op("shr", value, shift), mask),
+                              let(old1, intr("atomic_add_int32", "Gpu", lh, digit, i32(1)), "(empty)")))))
+    flush = block(if_(lt(tid, nb),
+                      let(old2, intr("atomic_add_global_int32", "Gpu", hist, tid, read("local_hist", tid)),
+                          "(empty)")))
+    body = shared(lh, "i32", 256, lets(
+        [(tid, intr("thread_idx_x")), (gid, intr("global_thread_id", "Std")), (nb, i32(256))],
+        seq(clear, BARRIER, count, BARRIER, flush, BARRIER)))
+    return kernel(params, body)
+
+
+def radix_sort_scatter():
+    fresh()
+    params = [("input", "(vec i32)"), ("output", "(vec i32)"), ("counters", "(vec i32)"), ("n", "i32"),
+              ("shift", "i32"), ("mask", "i32")]
+    for p, t in params:
+        var(p, t)
+    n, shift, mask = var("n"), var("shift"), var("mask")
+    counters = var("counters", "(vec i32)")
+    gid, value, digit, pos = var("gid"), var("value"), var("digit"), var("pos")
+    body = let(gid, intr("global_thread_id", "Std"),
+               if_(lt(gid, n),
+                   let(value, read("input", gid),
+                       let(digit, op("bitand", op("shr", value, shift), mask),
+                           let(pos, intr("atomic_add_global_int32", "Gpu", counters, digit, i32(1)),
+                               assign_elem("output", pos, value))))))
+    return kernel(params, body)
+
+
 KERNELS = {
     "stream_triad": stream_triad, "vector_add": vector_add, "vector_copy": vector_copy,
     "matrix_mul": matrix_mul, "matrix_mul_tiled": matrix_mul_tiled,
     "reduction": lambda: tree(False), "dot_product": lambda: tree(True),
     "transpose_naive": transpose_naive, "gather": gather, "mandelbrot": mandelbrot,
+    "reduction_max": reduction_max, "transpose_tiled": transpose_tiled, "scatter": scatter,
+    "radix_sort_histogram": radix_sort_histogram, "radix_sort_scatter": radix_sort_scatter,
 }
 
 

@@ -50,7 +50,7 @@ def expr_text(hip, expr):
 
 
 def test_fixture_list():
-    assert set(EXPECTED_TAGS) <= set(KERNELS) and len(KERNELS) >= 10
+    assert set(EXPECTED_TAGS) <= set(KERNELS) and len(KERNELS) == 15
 
 
 @pytest.mark.parametrize("name", KERNELS)
