@@ -26,6 +26,8 @@ if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
 
 PEAK_HBM_GBS = 8000.0          # MI355X HBM3E
+# MI355X peak engine clock: the published MFMA peaks are quoted at this clock
+NOMINAL_CLOCK_MHZ = 2400.0
 # HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (KiB per dispatch,
 # FETCH_SIZE scaled by 2.0 and WRITE_SIZE by 1.0 after calibration against a plain 1 GiB copy).
 MEASURED_TRAFFIC_BYTES = {
@@ -175,6 +177,17 @@ def measure(name, torch, hip, steps, warmup):
                      "traffic": MEASURED_TRAFFIC_BYTES.get(name),
                      "kernel": info["kernel"], "kernel_ms": round(kernel_ms, 5)},
     }
+    if info["bound"] == "mfma":
+        # shader clock the kernel actually ran at (in-kernel cycle counter against the
+        # constant-rate wall clock), over back-to-back launches as in the timed loop
+        with hip.clock_probe() as probe:
+            for _ in range(min(steps, 10)):
+                step()
+            mhz = probe.mhz()
+        if mhz:
+            res["roofline"]["shader_clock_mhz"] = round(mhz, 1)
+            res["roofline"]["frac_of_peak_at_that_clock"] = round(
+                achieved / (info["peak"] * mhz / NOMINAL_CLOCK_MHZ), 4)
     return res
 
 

@@ -248,6 +248,17 @@ int sarek_hip_cast_f32_to_f16(const float *in, uint16_t *out, int64_t n, sarek_h
  * rebuild.  Unknown names are stored and ignored.                           */
 int sarek_hip_set_tunable(const char *name, int64_t value);
 
+/* Diagnostic (no reference counterpart): while a probe buffer is set, every
+ * workgroup of the MFMA GEMM kernels (sarek_hip_gemm_bf16/_f16/_f16_bias_relu_rowsum,
+ * direct-to-LDS path) writes two 64-bit counts when it retires:
+ * pairs[2*w] = shader-clock cycles it was resident, pairs[2*w+1] = ticks of the
+ * constant-rate wall clock over the same interval (rate in *ticks_per_second).
+ * cycles/ticks gives the shader clock the kernel actually ran at.  A launch
+ * with more workgroups than capacity_pairs records nothing.  Pass NULL to
+ * switch the probe off (the default).                                        */
+int sarek_hip_set_clock_probe(uint64_t *device_pairs, int64_t capacity_pairs,
+                              int64_t *ticks_per_second);
+
 #ifdef __cplusplus
 }
 #endif

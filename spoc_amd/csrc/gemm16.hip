@@ -170,7 +170,8 @@ __global__ __launch_bounds__(64 * 2 * (8 / TJ)) void gemm16_dma_kernel(const uin
                                                              const float *__restrict__ bias,
                                                              float *__restrict__ rowsum, int M,
                                                              int N, int K, int tiles_m,
-                                                             int tiles_n, int xcd_remap) {
+                                                             int tiles_n, int xcd_remap,
+                                                             unsigned long long *probe) {
   constexpr int KK = BKT / 16;                 // MFMA k-steps per slab
   constexpr int A_ROW = BKT * 2;               // bytes per A row in LDS (unpadded)
   constexpr int A_ROWS_PER_DMA = 1024 / A_ROW; // rows one wave-wide DMA fills
@@ -189,6 +190,11 @@ __global__ __launch_bounds__(64 * 2 * (8 / TJ)) void gemm16_dma_kernel(const uin
   int tm, tn;
   tile_of_block(tiles_m, tiles_n, xcd_remap, tm, tn);
   const int m0 = tm * BM, n0 = tn * BN;
+  long long probe_c0 = 0, probe_t0 = 0;
+  if (probe) {
+    probe_c0 = clock64();
+    probe_t0 = wall_clock64();
+  }
 
   // Swizzles (XOR on the 16-byte slot index within a row).  The LDS of this chip serves
   // 256 bytes per clock (64 banks x 4 bytes): a ds_read_b128 is served 16 lanes at a time
@@ -375,6 +381,10 @@ __global__ __launch_bounds__(64 * 2 * (8 / TJ)) void gemm16_dma_kernel(const uin
   __builtin_amdgcn_s_waitcnt(waitcnt_vm_lgkm0(0));
   epilogue<Epi, TJ>(acc, C, bias, rowsum, M, N, m0, wm, wn, n0 + wn * (32 * TJ), lm, lh,
                     reinterpret_cast<float *>(lds_ring<0, A_BYTES_S>));
+  if (probe && tid == 0) {
+    probe[2 * blockIdx.x] = static_cast<unsigned long long>(clock64() - probe_c0);
+    probe[2 * blockIdx.x + 1] = static_cast<unsigned long long>(wall_clock64() - probe_t0);
+  }
 }
 
 template <bool Bf16, int Epi>
@@ -554,9 +564,10 @@ int launch_gemm16(const uint16_t *a, const uint16_t *b, float *c, const float *b
     if (k % BK == 0 && offsets_ok && tunable("gemm16.force_staged", 0) == 0) {
       const int ring = (int)tunable("gemm16.ring", 4), tj = (int)tunable("gemm16.tj", 2);
       const dim3 grid(tiles_m * tiles_n);
+      unsigned long long *probe = clock_probe(static_cast<int64_t>(tiles_m) * tiles_n);
 #define SAREK_LAUNCH_DMA(BKT, NS, TJ)                                                             \
   hipLaunchKernelGGL((gemm16_dma_kernel<Bf16, Epi, BKT, NS, TJ>), grid, dim3(64 * 2 * (8 / TJ)), 0, \
-                     st, a, b, c, bias, rowsum, m, n, k, tiles_m, tiles_n, remap)
+                     st, a, b, c, bias, rowsum, m, n, k, tiles_m, tiles_n, remap, probe)
       if (ring == 4 && tj == 2) SAREK_LAUNCH_DMA(32, 4, 2);
       else if (ring == 4) SAREK_LAUNCH_DMA(32, 4, 4);
       else if (tj == 2) SAREK_LAUNCH_DMA(64, 2, 2);

@@ -166,7 +166,7 @@ __global__ __launch_bounds__(THREADS) void gemm_f32_staged_kernel(const float *_
 template <int TI, int TJ, int WMW, int WNW, int BKT, int NS>
 __global__ __launch_bounds__(64 * WMW * WNW) void gemm_f32_dma_kernel(
     const float *__restrict__ A, const float *__restrict__ B, float *__restrict__ C, int M, int N,
-    int K, int tiles_m, int tiles_n, int xcd_remap) {
+    int K, int tiles_m, int tiles_n, int xcd_remap, unsigned long long *probe) {
   typedef __attribute__((ext_vector_type(TJ))) float bvec_t;
   constexpr int BMT = 32 * TI * WMW, BNT = 32 * TJ * WNW, NWAVES = WMW * WNW;
   constexpr int KK = BKT / 8;
@@ -188,6 +188,11 @@ __global__ __launch_bounds__(64 * WMW * WNW) void gemm_f32_dma_kernel(
   int tm, tn;
   tile_of_block(tiles_m, tiles_n, xcd_remap, tm, tn);
   const int m0 = tm * BMT, n0 = tn * BNT;
+  long long probe_c0 = 0, probe_t0 = 0;
+  if (probe) {
+    probe_c0 = clock64();
+    probe_t0 = wall_clock64();
+  }
 
   auto a_swz = [](int row) { return A_CHUNKS == 8 ? ((row >> 1) & 7) : ((row >> 2) & 3); };
   auto b_swz = [](int row) { return TJ == 1 ? (((row >> 2) & 1) << 3) : 0; };
@@ -341,6 +346,10 @@ __global__ __launch_bounds__(64 * WMW * WNW) void gemm_f32_dma_kernel(
         *reinterpret_cast<bvec_t *>(C + static_cast<int64_t>(row) * N + col) = v;
       }
     }
+  if (probe && tid == 0) {
+    probe[2 * blockIdx.x] = static_cast<unsigned long long>(clock64() - probe_c0);
+    probe[2 * blockIdx.x + 1] = static_cast<unsigned long long>(wall_clock64() - probe_t0);
+  }
 }
 
 // Any shape, any alignment: one thread per C element, f32 FMA in k order.
@@ -385,7 +394,7 @@ extern "C" int sarek_hip_gemm_f32(const float *a, const float *b, float *c, int 
 #define SAREK_LAUNCH_F32(T, TI, TJ, WMW, WNW, BKT)                                               \
   hipLaunchKernelGGL((gemm_f32_dma_kernel<TI, TJ, WMW, WNW, BKT, 4>),                             \
                      dim3((unsigned)ntiles(T)), dim3(64 * WMW * WNW), 0, st, a, b, c, m, n, k,    \
-                     (m + T - 1) / T, (n + T - 1) / T, remap)
+                     (m + T - 1) / T, (n + T - 1) / T, remap, clock_probe(ntiles(T)))
       if (tile == 256) SAREK_LAUNCH_F32(256, 4, 2, 2, 4, 16);
       else if (tile == 128) SAREK_LAUNCH_F32(128, 2, 2, 2, 2, 16);
       else SAREK_LAUNCH_F32(64, 1, 1, 2, 2, 32);

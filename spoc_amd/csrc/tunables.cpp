@@ -5,6 +5,9 @@
 #include <mutex>
 #include <string>
 
+#include <hip/hip_runtime.h>
+
+#include "common.hpp"
 #include "sarek_hip.h"
 
 namespace sarek_hip {
@@ -14,7 +17,14 @@ std::map<std::string, int64_t> &table() {
   static std::map<std::string, int64_t> t;
   return t;
 }
+unsigned long long *g_probe = nullptr;
+int64_t g_probe_pairs = 0;
 }  // namespace
+
+unsigned long long *clock_probe(int64_t workgroups) {
+  std::lock_guard<std::mutex> lock(g_mu);
+  return (g_probe && workgroups <= g_probe_pairs) ? g_probe : nullptr;
+}
 
 int64_t tunable(const char *name, int64_t fallback) {
   std::lock_guard<std::mutex> lock(g_mu);
@@ -38,5 +48,22 @@ void set_tunable(const char *name, int64_t value) {
 extern "C" int sarek_hip_set_tunable(const char *name, int64_t value) {
   if (!name) return SAREK_HIP_E_INVALID_ARG;
   sarek_hip::set_tunable(name, value);
+  return SAREK_HIP_OK;
+}
+
+extern "C" int sarek_hip_set_clock_probe(uint64_t *device_pairs, int64_t capacity_pairs,
+                                         int64_t *ticks_per_second) {
+  using namespace sarek_hip;
+  if (device_pairs && capacity_pairs <= 0)
+    return fail(SAREK_HIP_E_INVALID_ARG, "clock probe: capacity must be positive");
+  if (ticks_per_second) {
+    int dev = 0, khz = 0;
+    SAREK_HIP_TRY(hipGetDevice(&dev));
+    SAREK_HIP_TRY(hipDeviceGetAttribute(&khz, hipDeviceAttributeWallClockRate, dev));
+    *ticks_per_second = static_cast<int64_t>(khz) * 1000;
+  }
+  std::lock_guard<std::mutex> lock(g_mu);
+  g_probe = reinterpret_cast<unsigned long long *>(device_pairs);
+  g_probe_pairs = device_pairs ? capacity_pairs : 0;
   return SAREK_HIP_OK;
 }

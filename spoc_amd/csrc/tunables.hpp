@@ -8,4 +8,6 @@ namespace sarek_hip {
 // variable SAREK_HIP_TUNE_<name with '.' replaced by '_'> seeds the knob on first use.
 int64_t tunable(const char *name, int64_t fallback);
 void set_tunable(const char *name, int64_t value);
+// Clock-probe buffer for a launch of `workgroups` workgroups, or nullptr.
+unsigned long long *clock_probe(int64_t workgroups);
 }  // namespace sarek_hip

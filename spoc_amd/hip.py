@@ -108,6 +108,7 @@ SYMBOLS = {
     "sarek_hip_cast_f32_to_bf16": (_i, [_vp, _vp, _i64, _vp]),
     "sarek_hip_cast_f32_to_f16": (_i, [_vp, _vp, _i64, _vp]),
     "sarek_hip_set_tunable": (_i, [C.c_char_p, _i64]),
+    "sarek_hip_set_clock_probe": (_i, [_vp, _i64, C.POINTER(_i64)]),
 }
 
 
@@ -140,6 +141,37 @@ def check(status):
 
 def set_tunable(name, value):
     check(lib.sarek_hip_set_tunable(name.encode(), int(value)))
+
+
+class clock_probe:
+    """Context manager: MFMA GEMM launches inside it record, per workgroup, the shader-clock
+    cycles and wall-clock ticks it was resident.  `mhz()` is the shader clock those
+    workgroups ran at, averaged over the last launch that fitted the buffer."""
+
+    def __init__(self, workgroups=4096):
+        torch = _torch()
+        self.buf = torch.zeros(2 * workgroups, dtype=torch.int64, device="cuda")
+        self.rate = C.c_int64(0)
+
+    def __enter__(self):
+        check(lib.sarek_hip_set_clock_probe(C.c_void_p(self.buf.data_ptr()), self.buf.numel() // 2,
+                                            C.byref(self.rate)))
+        return self
+
+    def __exit__(self, *exc):
+        check(lib.sarek_hip_set_clock_probe(None, 0, None))
+        return False
+
+    def pairs(self):
+        _torch().cuda.synchronize()
+        p = self.buf.view(-1, 2).cpu().numpy()
+        return p[p[:, 1] > 0]
+
+    def mhz(self):
+        p = self.pairs()
+        if len(p) == 0:
+            return None
+        return float(p[:, 0].sum()) / float(p[:, 1].sum()) * self.rate.value / 1e6
 
 
 # ---------------------------------------------------------------------------

@@ -190,3 +190,30 @@ def test_gemm_rejects_bad_arguments(hip, torch_cuda):
     with pytest.raises(hip.SarekHipError) as e:
         hip.check(hip.lib.sarek_hip_gemm_f32(a.data_ptr(), a.data_ptr(), a.data_ptr(), 4, -1, 4, None))
     assert e.value.status == hip.E_INVALID_ARG
+
+
+def test_clock_probe_records_cycles_and_ticks(hip, torch_cuda):
+    """The diagnostic probe: one (cycles, ticks) pair per workgroup, plausible clock, and
+    nothing written once it is switched off or when the launch has more workgroups than
+    the buffer holds."""
+    torch = torch_cuda
+    m = n = 1024
+    k = 512
+    a = torch.randn(m, k, device="cuda").to(torch.bfloat16)
+    b = torch.randn(k, n, device="cuda").to(torch.bfloat16)
+    with hip.clock_probe(workgroups=64) as probe:
+        hip.gemm_bf16(a, b)                      # 16 workgroups of 256 x 256
+        pairs = probe.pairs()
+        assert len(pairs) == 16
+        assert 500 < probe.mhz() < 2600
+        probe.buf.zero_()
+        hip.gemm_bf16(torch.zeros(4096, 64, device="cuda", dtype=torch.bfloat16),
+                      torch.zeros(64, 8192, device="cuda", dtype=torch.bfloat16))   # 512 > 64
+        assert len(probe.pairs()) == 0
+    probe.buf.zero_()
+    hip.gemm_bf16(a, b)
+    assert len(probe.pairs()) == 0
+    x = torch.randn(512, 256, device="cuda")
+    with hip.clock_probe(workgroups=64) as probe:
+        hip.gemm_f32(x, x[:256, :].contiguous())
+        assert len(probe.pairs()) > 0 and 500 < probe.mhz() < 2600
