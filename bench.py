@@ -177,6 +177,8 @@ def measure(name, torch, hip, steps, warmup):
                      "traffic": MEASURED_TRAFFIC_BYTES.get(name),
                      "kernel": info["kernel"], "kernel_ms": round(kernel_ms, 5)},
     }
+    if name == "triad_sum_2p28":
+        res["roofline"]["probe_kernels_GBs"] = hbm_ceiling(torch, hip)
     if info["bound"] == "mfma":
         # shader clock the kernel actually ran at (in-kernel cycle counter against the
         # constant-rate wall clock), over back-to-back launches as in the timed loop
@@ -189,6 +191,59 @@ def measure(name, torch, hip, steps, warmup):
             res["roofline"]["frac_of_peak_at_that_clock"] = round(
                 achieved / (info["peak"] * mhz / NOMINAL_CLOCK_MHZ), 4)
     return res
+
+
+HBM_PROBE_SRC = r"""
+typedef float f4 __attribute__((ext_vector_type(4)));
+#define LOADS(dst, src) _Pragma("unroll") for (int u = 0; u < 4; ++u) dst[u] = __builtin_nontemporal_load(src + base + u * 256)
+extern "C" __global__ __launch_bounds__(256) void probe_read(const f4* r0, int n0, float* sink, int ns) {
+  const long base = (long)blockIdx.x * 1024 + threadIdx.x;
+  f4 v[4];
+  LOADS(v, r0);
+  const f4 s = v[0] + v[1] + v[2] + v[3];
+  if (s.x + s.y + s.z + s.w == 12345.678f) sink[0] = 1.f;
+}
+extern "C" __global__ __launch_bounds__(256) void probe_write(f4* w, int nw) {
+  const long base = (long)blockIdx.x * 1024 + threadIdx.x;
+  const f4 v = {1.f, 2.f, 3.f, 4.f};
+  _Pragma("unroll") for (int u = 0; u < 4; ++u) __builtin_nontemporal_store(v, w + base + u * 256);
+}
+extern "C" __global__ __launch_bounds__(256) void probe_2r1w(f4* w, int nw, const f4* r0, int n0, const f4* r1, int n1) {
+  const long base = (long)blockIdx.x * 1024 + threadIdx.x;
+  f4 v[4], c[4];
+  LOADS(v, r0);
+  LOADS(c, r1);
+  _Pragma("unroll") for (int u = 0; u < 4; ++u) __builtin_nontemporal_store(v[u] + c[u], w + base + u * 256);
+}
+"""
+
+
+def hbm_ceiling(torch, hip, n=1 << 28):
+    """What this GPU's HBM delivers to the simplest kernels of three traffic shapes (one
+    workgroup per 4096 floats, 128-bit non-temporal accesses), JIT-compiled through the
+    plugin path: context for the triad's fraction of the nominal 8 TB/s."""
+    a = torch.empty(n, device="cuda")
+    b = torch.rand(n, device="cuda")
+    c = torch.rand(n, device="cuda")
+    sink = torch.zeros(1, device="cuda")
+    grid = (n // 4096, 1, 1)
+    stream = C.c_void_p(torch.cuda.current_stream().cuda_stream)
+    ev = Events(hip, stream)
+    out = {}
+    for key, kern, items, nbytes in [
+            ("read_only", "probe_read", [b, sink], 4 * n),
+            ("write_only", "probe_write", [a], 4 * n),
+            ("two_reads_one_write", "probe_2r1w", [a, b, c], 12 * n)]:
+        times = []
+        for i in range(12):
+            ev.start()
+            hip.run_source(HBM_PROBE_SRC, kern, (256, 1, 1), grid, items)
+            ms = ev.stop_ms()
+            if i >= 2:
+                times.append(ms)
+        times.sort()
+        out[key] = round(nbytes / (times[len(times) // 2] * 1e-3) / 1e9, 1)
+    return out
 
 
 def cpu_baseline(name):

@@ -387,10 +387,29 @@ extern "C" int sarek_hip_gemm_f32(const float *a, const float *b, float *c, int 
                             static_cast<int64_t>(n) * 32 * 4 < 0x7FFFFFFF;
     if (k % 32 == 0 && offsets_ok && reinterpret_cast<uintptr_t>(c) % 16 == 0 &&
         tunable("gemm_f32.force_staged", 0) == 0) {
-      // Tile choice: the largest tile that still gives every CU at least two workgroups.
+      // Tile choice by a cost model of the launch: a CU holds `occ` workgroups of a tile
+      // shape at once (LDS ring), tiles run in rounds of cus*occ, a workgroup that shares
+      // its CU takes occ times as long, and the tail round runs unshared when it fits one
+      // workgroup per CU.  `eff` is the MFMA issue efficiency measured for each shape.
       auto ntiles = [&](int t) { return static_cast<int64_t>((m + t - 1) / t) * ((n + t - 1) / t); };
+      static const int cus = [] {
+        int dev = 0, v = 0;
+        if (hipGetDevice(&dev) != hipSuccess ||
+            hipDeviceGetAttribute(&v, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || v <= 0)
+          v = 256;
+        return v;
+      }();
+      auto cost = [&](int t, int occ, double eff) {
+        const int64_t tiles = ntiles(t), slots = static_cast<int64_t>(cus) * occ;
+        const int64_t full = tiles / slots, rest = tiles % slots;
+        const double rounds = static_cast<double>(full) * occ + (rest == 0 ? 0 : rest <= cus ? 1 : occ);
+        return rounds * t * t / eff;
+      };
       int tile = (int)tunable("gemm_f32.tile", 0);
-      if (tile == 0) tile = ntiles(256) >= 512 ? 256 : ntiles(128) >= 512 ? 128 : 64;
+      if (tile == 0) {
+        const double c256 = cost(256, 1, 1.0), c128 = cost(128, 2, 0.95), c64 = cost(64, 2, 0.80);
+        tile = (c256 <= c128 && c256 <= c64) ? 256 : (c128 <= c64 ? 128 : 64);
+      }
 #define SAREK_LAUNCH_F32(T, TI, TJ, WMW, WNW, BKT)                                               \
   hipLaunchKernelGGL((gemm_f32_dma_kernel<TI, TJ, WMW, WNW, BKT, 4>),                             \
                      dim3((unsigned)ntiles(T)), dim3(64 * WMW * WNW), 0, st, a, b, c, m, n, k,    \
