@@ -215,6 +215,11 @@ int sarek_hip_reduce_sum_block256_f32(const float *in, float *out, int64_t n,
                                       sarek_hip_stream stream);
 int sarek_hip_dot_block256_f32(const float *a, const float *b, float *out, int64_t n,
                                sarek_hip_stream stream);
+/* out[j] = what the reference's block-256 "take the greater" tree leaves for block j
+ * (benchmarks/bench_reduction_max.ml:18-100), elements past n read as `pad`
+ * (-1000000.0 in that file); same comparison pairs and order as the tree.   */
+int sarek_hip_reduce_max_block256_f32(const float *in, float *out, int64_t n, float pad,
+                                      sarek_hip_stream stream);
 /* *sum_out = left-to-right double fold of partials[0..count)
  * (host fold of benchmarks/bench_reduction.ml:154-160, kept on device).    */
 int sarek_hip_fold_partials_f64(const float *partials, int64_t count, double *sum_out,

@@ -14,7 +14,7 @@ _SO = os.path.join(_HERE, "liboracle.so")
 
 __all__ = [
     "build", "fill_uniform", "round_bf16", "round_f16", "bf16_bits", "f16_bits",
-    "triad", "reduce_sum_block256", "dot_block256", "fold_partials", "triad_sum",
+    "triad", "reduce_sum_block256", "reduce_max_block256", "dot_block256", "fold_partials", "triad_sum",
     "gemm", "gemm_rows", "gemm_bias_relu_rowsum", "matmul_tiled_bsp",
 ]
 
@@ -46,6 +46,7 @@ def _L():
         lib.oracle_triad_f32.argtypes = [f32p, f32p, f32p, C.c_float, i64, i32]
         lib.oracle_reduce_sum_block256_f32.argtypes = [f32p, i64, f32p, i32]
         lib.oracle_dot_block256_f32.argtypes = [f32p, f32p, i64, f32p, i32]
+        lib.oracle_reduce_max_block256_f32.argtypes = [f32p, i64, C.c_double, f32p]
         lib.oracle_fold_partials_f64.argtypes = [f32p, i64]
         lib.oracle_fold_partials_f64.restype = C.c_double
         lib.oracle_triad_sum_f32.argtypes = [f32p, f32p, f32p, C.c_float, i64, f32p, i32]
@@ -114,6 +115,13 @@ def reduce_sum_block256(x, threads=None):
     p = np.empty((x.size + 255) // 256, dtype=np.float32)
     _L().oracle_reduce_sum_block256_f32(xp, x.size, p.ctypes.data_as(C.POINTER(C.c_float)),
                                         threads or default_threads())
+    return p
+
+
+def reduce_max_block256(x, pad=-1000000.0):
+    x, xp = _f32(x)
+    p = np.empty((x.size + 255) // 256, dtype=np.float32)
+    _L().oracle_reduce_max_block256_f32(xp, x.size, float(pad), p.ctypes.data_as(C.POINTER(C.c_float)))
     return p
 
 

@@ -270,6 +270,28 @@ void oracle_dot_block256_f32(const float *a, const float *b, int64_t n, float *p
   parallel_ranges((n + 255) / 256, threads, reduce_blocks_range, &r);
 }
 
+/* Block-256 "take the greater" tree (benchmarks/bench_reduction_max.ml:18-100):
+ * sdata[tid] = in[gid], or `pad` (-1000000.0 there) when gid >= n; for half =
+ * 128..1, threads tid < half do  a = sdata[tid]; b = sdata[tid+half];
+ * if b > a then sdata[tid] <- b;  output[block] = sdata[0].  Shared values are
+ * doubles holding binary32 values, so the comparisons equal binary32 ones.  */
+void oracle_reduce_max_block256_f32(const float *in, int64_t n, double pad, float *partials) {
+  const int64_t nblocks = (n + 255) / 256;
+  for (int64_t blk = 0; blk < nblocks; ++blk) {
+    double s[256];
+    for (int t = 0; t < 256; ++t) {
+      const int64_t g = blk * 256 + t;
+      s[t] = g < n ? (double)in[g] : pad;
+    }
+    for (int half = 128; half >= 1; half >>= 1)
+      for (int t = 0; t < half; ++t) {
+        const double a = s[t], b = s[t + half];
+        if (b > a) s[t] = b;
+      }
+    partials[blk] = (float)s[0];
+  }
+}
+
 /* Host fold of the partials, left to right in double
  * (benchmarks/bench_reduction.ml:154-160).                               */
 double oracle_fold_partials_f64(const float *partials, int64_t count) {

@@ -2,9 +2,10 @@
 // source and run_source can serve the launch with a hand-written CDNA4 kernel.
 //
 // A kernel is recognised only when, after normalisation, it is the same program as one of
-// the four templates below (the kernels of benchmarks/bench_matrix_mul_tiled.ml:55-95,
-// benchmarks/bench_stream_triad.ml:22-32, benchmarks/bench_reduction.ml:62-96 and
-// benchmarks/bench_dot_product.ml:16-54 in the reference).  Anything else gets the plain
+// the five templates below (the kernels of benchmarks/bench_matrix_mul_tiled.ml:55-95,
+// benchmarks/bench_stream_triad.ml:22-32, benchmarks/bench_reduction.ml:62-96,
+// benchmarks/bench_dot_product.ml:16-54 and benchmarks/bench_reduction_max.ml:18-100 in the
+// reference; the last with any constant as the out-of-range fill).  Anything else gets the plain
 // lowering: a miss costs speed, never correctness.
 //
 // Normalisation removes what the front end is free to vary without changing meaning:
@@ -16,7 +17,10 @@
 //   - thread-index intrinsics use one spelling and `global_thread_id` is expanded to
 //     thread_idx_x + block_idx_x * block_dim_x.
 #include <algorithm>
+#include <cstdint>
 #include <cstdio>
+#include <cstdlib>
+#include <cstring>
 #include <map>
 
 #include "ir.hpp"
@@ -341,6 +345,32 @@ std::string tree_template(bool dot) {
          ") (native_fn true))";
 }
 
+// The "take the greater" tree of benchmarks/bench_reduction_max.ml:18-100; `pad` is what
+// out-of-range slots are filled with.
+std::string max_tree_template(const std::string &pad) {
+  const std::string tid = "(var tid 5 i32)", gid = "(var gid 6 i32)", n = "(var n 4 i32)";
+  const std::string slot = "(lelem sdata " + tid + ")";
+  std::string steps = "(block (if (lt " + gid + " " + n + ") (assign " + slot + " (read input " + gid +
+                      ")) (assign " + slot + " " + pad + "))) (barrier) ";
+  for (int half = 128; half >= 1; half >>= 1) {
+    const std::string h = "(i32 " + std::to_string(half) + ")";
+    const std::string a = "(var a " + std::to_string(100 + half) + " f32)";
+    const std::string b = "(var b " + std::to_string(400 + half) + " f32)";
+    steps += "(block (if (lt " + tid + " " + h + ") (let " + a + " (read sdata " + tid + ") (let " + b +
+             " (read sdata (add " + tid + " " + h + ")) (if (gt " + b + " " + a + ") (assign " + slot +
+             " " + b + ")))))) (barrier) ";
+  }
+  steps += "(block (if (eq " + tid + " (i32 0)) (assign (lelem output (intr (Gpu) block_idx_x)) "
+           "(read sdata (i32 0)))))";
+  const std::string body =
+      "(let (var sdata 7 (array f32 shared)) (newarray f32 (i32 256) shared) "
+      "(let " + tid + " (intr (Gpu) thread_idx_x) "
+      "(let " + gid + " (add (intr (Gpu) thread_idx_x) (mul (intr (Gpu) block_dim_x) (intr (Gpu) block_idx_x))) "
+      "(seq " + steps + "))))";
+  return "(kernel sarek_kern (params (param (var input 1 (vec f32))) (param (var output 3 (vec f32))) "
+         "(param " + n + ")) (locals) (body " + body + ") (native_fn true))";
+}
+
 // The generated text of the tree kernels ends with a barrier after the final store
 // (reduction_generated.md:69-75 in the reference's golden files) when the last statement
 // is itself a superstep; accept both spellings.
@@ -349,6 +379,31 @@ std::string strip_trailing_barrier(std::string s) {
   if (s.size() >= tail.size() && s.compare(s.size() - tail.size(), tail.size(), tail) == 0)
     s = s.substr(0, s.size() - tail.size()) + "]";
   return s;
+}
+
+// Matches `c` against the max-tree template for any finite or infinite f32 pad constant;
+// returns the pad's bits as 8 hex digits, or "" when the kernel is something else.
+std::string match_max_tree(const std::string &c) {
+  static const std::string marker = "f32:-12345.5";
+  static const std::string t = strip_trailing_barrier(canon_kernel(parse_kernel(max_tree_template("(f32 -12345.5)"))));
+  static const size_t at = t.find(marker);
+  if (at == std::string::npos || t.find(marker, at + 1) != std::string::npos) return "";
+  const std::string prefix = t.substr(0, at), suffix = t.substr(at + marker.size());
+  if (c.size() < prefix.size() + suffix.size() + 5) return "";
+  if (c.compare(0, prefix.size(), prefix) != 0) return "";
+  if (c.compare(c.size() - suffix.size(), suffix.size(), suffix) != 0) return "";
+  const std::string mid = c.substr(prefix.size(), c.size() - prefix.size() - suffix.size());
+  if (mid.compare(0, 4, "f32:") != 0) return "";
+  char *end = nullptr;
+  const std::string num = mid.substr(4);
+  const double v = std::strtod(num.c_str(), &end);
+  if (end == num.c_str() || *end != 0 || v != v) return "";
+  const float f = static_cast<float>(v);
+  uint32_t bits;
+  std::memcpy(&bits, &f, 4);
+  char buf[16];
+  std::snprintf(buf, sizeof(buf), "%08x", bits);
+  return buf;
 }
 
 }  // namespace
@@ -364,6 +419,8 @@ std::string recognise(const Kernel &k) {
   const std::string cs = strip_trailing_barrier(c);
   if (cs == t_reduce) return "reduce_sum_block256_f32";
   if (cs == t_dot) return "dot_block256_f32";
+  const std::string pad = match_max_tree(cs);
+  if (!pad.empty()) return "reduce_max_block256_f32:" + pad;
   return "";
 }
 

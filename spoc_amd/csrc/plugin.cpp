@@ -113,6 +113,24 @@ int try_specialised(const std::string &tag, const int block[3], const int grid[3
                                               static_cast<float *>(args[2].buffer), n, nullptr);
     return 1;
   }
+  if (tag.compare(0, 24, "reduce_max_block256_f32:") == 0 && tag.size() == 32) {
+    // (input, len, output, len, n); the fill value travels in the tag as f32 bits
+    char *end = nullptr;
+    const unsigned long bits = std::strtoul(tag.c_str() + 24, &end, 16);
+    if (*end != 0) return 0;
+    const uint32_t b32 = static_cast<uint32_t>(bits);
+    float pad;
+    std::memcpy(&pad, &b32, 4);
+    if (n_args != 5 || !vec_at(args, n_args, 0) || !vec_at(args, n_args, 2) || !is_i32(args[4])) return 0;
+    const int64_t n = args[4].i32;
+    if (n < 0) return 0;
+    if (block[0] != 256 || block[1] != 1 || block[2] != 1 || grid[1] != 1 || grid[2] != 1) return 0;
+    const int64_t nblocks = cdiv(n, 256);
+    if (grid[0] != nblocks || args[2].length < nblocks || args[0].length < n) return 0;
+    *rc = sarek_hip_reduce_max_block256_f32(static_cast<const float *>(args[0].buffer),
+                                            static_cast<float *>(args[2].buffer), n, pad, nullptr);
+    return 1;
+  }
   return 0;
 }
 

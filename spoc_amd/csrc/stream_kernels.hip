@@ -226,6 +226,37 @@ __global__ __launch_bounds__(kBlock) void block256_kernel(const float *__restric
   }
 }
 
+// One wave per 256-element block: out[j] = the value the reference's halving tree
+// (benchmarks/bench_reduction_max.ml:18-100: sdata[tid] = gid < n ? in[gid] : pad, then for
+// half = 128..1 "if sdata[tid+half] > sdata[tid] then sdata[tid] <- sdata[tid+half]")
+// leaves in sdata[0].  The same pairs are compared in the same order with the same
+// strict ">" (lane l holds elements l, l+64, l+128, l+192 of the block), so NaNs and
+// signed zeros come out as from the tree.
+__device__ __forceinline__ float take_greater(float a, float b) { return b > a ? b : a; }
+
+__global__ __launch_bounds__(kBlock) void block256_max_kernel(const float *__restrict__ x,
+                                                              float *__restrict__ out, int64_t n,
+                                                              int64_t nblocks, float pad) {
+  const int lane = threadIdx.x & 63;
+  const int64_t wave = static_cast<int64_t>(blockIdx.x) * (kBlock / 64) + (threadIdx.x >> 6);
+  const int64_t wstep = static_cast<int64_t>(gridDim.x) * (kBlock / 64);
+  for (int64_t j = wave; j < nblocks; j += wstep) {
+    const int64_t i = j * 256 + lane;
+    float v[4];
+#pragma unroll
+    for (int q = 0; q < 4; ++q) v[q] = (i + 64 * q < n) ? x[i + 64 * q] : pad;
+    v[0] = take_greater(v[0], v[2]);   // half = 128: (l, l+128), (l+64, l+192)
+    v[1] = take_greater(v[1], v[3]);
+    float m = take_greater(v[0], v[1]);  // half = 64
+#pragma unroll
+    for (int half = 32; half >= 1; half >>= 1) {
+      const float other = __shfl_down(m, half, 64);
+      m = take_greater(m, other);       // only lanes < half matter from here on
+    }
+    if (lane == 0) out[j] = m;
+  }
+}
+
 // f32 -> bf16 bits, round to nearest even; NaN stays a quiet NaN.
 __device__ __forceinline__ uint16_t f32_to_bf16_rne(float f) {
   uint32_t u = __builtin_bit_cast(uint32_t, f);
@@ -359,6 +390,20 @@ int sarek_hip_reduce_sum_block256_f32(const float *in, float *out, int64_t n,
 int sarek_hip_dot_block256_f32(const float *a, const float *b, float *out, int64_t n,
                                sarek_hip_stream stream) {
   return launch_block256(a, b, out, n, true, as_stream(stream));
+}
+
+int sarek_hip_reduce_max_block256_f32(const float *in, float *out, int64_t n, float pad,
+                                      sarek_hip_stream stream) {
+  if (n < 0) return fail(SAREK_HIP_E_INVALID_ARG, "block256 max: negative length");
+  if (n == 0) return SAREK_HIP_OK;
+  if (!in || !out) return fail(SAREK_HIP_E_INVALID_ARG, "block256 max: NULL vector");
+  const int64_t nblocks = ceil_div(n, 256);
+  int64_t wg = ceil_div(nblocks, kBlock / 64);
+  const int64_t cap = tunable("block256.max_blocks", 256 * 32);
+  if (wg > cap) wg = cap;
+  hipLaunchKernelGGL(block256_max_kernel, dim3((unsigned)wg), dim3(kBlock), 0, as_stream(stream), in,
+                     out, n, nblocks, pad);
+  return check_launch("block256 max kernel launch");
 }
 
 static int launch_cast(const float *in, uint16_t *out, int64_t n, bool bf16, hipStream_t st) {

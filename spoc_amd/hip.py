@@ -100,6 +100,7 @@ SYMBOLS = {
     "sarek_hip_triad_sum_f32": (_i, [_vp, _vp, _vp, _f, _i64, _vp, _i64, _vp, _vp]),
     "sarek_hip_reduce_sum_block256_f32": (_i, [_vp, _vp, _i64, _vp]),
     "sarek_hip_dot_block256_f32": (_i, [_vp, _vp, _vp, _i64, _vp]),
+    "sarek_hip_reduce_max_block256_f32": (_i, [_vp, _vp, _i64, _f, _vp]),
     "sarek_hip_fold_partials_f64": (_i, [_vp, _i64, _vp, _vp]),
     "sarek_hip_gemm_f32": (_i, [_vp, _vp, _vp, _i, _i, _i, _vp]),
     "sarek_hip_gemm_bf16": (_i, [_vp, _vp, _vp, _i, _i, _i, _vp]),
@@ -236,6 +237,14 @@ def reduce_sum_block256(x):
     _need(x, torch.float32, "x")
     out = torch.empty((x.numel() + 255) // 256, dtype=torch.float32, device=x.device)
     check(lib.sarek_hip_reduce_sum_block256_f32(_ptr(x), _ptr(out), x.numel(), _stream()))
+    return out
+
+
+def reduce_max_block256(x, pad=-1000000.0):
+    torch = _torch()
+    _need(x, torch.float32, "x")
+    out = torch.empty((x.numel() + 255) // 256, dtype=torch.float32, device=x.device)
+    check(lib.sarek_hip_reduce_max_block256_f32(_ptr(x), _ptr(out), x.numel(), float(pad), _stream()))
     return out
 
 

@@ -284,3 +284,26 @@ def test_scatter_and_radix_ir_end_to_end(hip, torch_cuda):
     assert np.all(np.diff(gd) >= 0)
     assert np.array_equal(np.sort(got), np.sort(vals))
     assert np.array_equal(counters.cpu().numpy(), starts + counts)
+
+
+@pytest.mark.parametrize("specialise", [1, 0])
+def test_reduction_max_ir_end_to_end(hip, oracle, torch_cuda, specialise):
+    """bench_reduction_max.ml as written today (fill -1000000.0): hand kernel and JIT-compiled
+    lowering give the tree's result bit for bit."""
+    from test_ir_lowering import reduction_max_ir
+    torch = torch_cuda
+    n = 70001
+    nblocks = (n + 255) // 256
+    x = (oracle.fill_uniform(n, seed=0x9) * 2000 - 1000).astype(np.float32)
+    dx = torch.from_numpy(x).cuda()
+    out = torch.zeros(nblocks, device="cuda")
+    hip.check(hip.lib.sarek_hip_set_specialisation(specialise))
+    try:
+        path = hip.run_source(hip.generate_source(reduction_max_ir()), "sarek_kern", (256, 1, 1),
+                              (nblocks, 1, 1), [dx, out, ("i32", n)], shared_mem=1024)
+        hip.check(hip.lib.sarek_hip_device_synchronize())
+    finally:
+        hip.check(hip.lib.sarek_hip_set_specialisation(1))
+    assert path.startswith("reduce_max_block256_f32:") if specialise else path == "jit"
+    assert np.array_equal(out.cpu().numpy(), oracle.reduce_max_block256(x))
+    assert out.max().item() == x.max()     # the bench's own check: max of partials = max of input

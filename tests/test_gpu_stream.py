@@ -134,3 +134,20 @@ def test_casts_bit_exact(hip, oracle, torch_cuda):
                           oracle.bf16_bits(x))
     assert np.array_equal(hip.cast_f16(d).view(torch.int16).cpu().numpy().view(np.uint16),
                           oracle.f16_bits(x))
+
+
+@pytest.mark.parametrize("n", [1, 255, 256, 257, 100000, 1 << 20])
+def test_block256_max_matches_tree_bit_for_bit(hip, oracle, torch_cuda, n):
+    torch = torch_cuda
+    rng = np.random.default_rng(n)
+    x = (rng.standard_normal(n) * 1000).astype(np.float32)
+    if n > 300:
+        x[5] = np.nan
+        x[300] = -0.0
+        x[301] = 0.0
+    got = hip.reduce_max_block256(torch.from_numpy(x).cuda()).cpu().numpy()
+    exp = oracle.reduce_max_block256(x)
+    assert np.array_equal(got.view(np.uint32), exp.view(np.uint32))
+    # another fill value
+    got = hip.reduce_max_block256(torch.from_numpy(x).cuda(), pad=float("-inf")).cpu().numpy()
+    assert np.array_equal(got.view(np.uint32), oracle.reduce_max_block256(x, pad=float("-inf")).view(np.uint32))

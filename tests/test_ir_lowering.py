@@ -236,3 +236,26 @@ def test_reduction_with_other_operator_is_not_taken(hip):
     ir = open(os.path.join(IR_DIR, "reduction.ir")).read()
     assert split_tag(hip.generate_source(ir.replace("(add (read sdata", "(mul (read sdata", 1)))[0] == ""
     assert split_tag(hip.generate_source(ir.replace("(i32 64)", "(i32 65)", 1)))[0] == ""
+
+
+def reduction_max_ir(pad="(f32 -1000000.0)"):
+    """The kernel as benchmarks/bench_reduction_max.ml:18-100 writes it today (the golden
+    text predates it and fills with Float.neg_infinity, a free variable)."""
+    ir = open(os.path.join(IR_DIR, "reduction_max.ir")).read()
+    free = "(var Float.neg_infinity"
+    i = ir.index(free)
+    j = ir.index(")", i) + 1
+    return ir[:i] + pad + ir[j:]
+
+
+def test_reduction_max_recognition_carries_the_fill_value(hip):
+    import struct
+    tag, src = split_tag(hip.generate_source(reduction_max_ir()))
+    assert tag == "reduce_max_block256_f32:" + struct.pack(">f", -1000000.0).hex()
+    assert "sdata[tid] = -1000000.0f;" in src
+    assert split_tag(hip.generate_source(reduction_max_ir("(f32 -inf)")))[0] == "reduce_max_block256_f32:ff800000"
+    # the golden form (free variable as fill) is lowered but not taken over
+    assert split_tag(hip.generate_source(open(os.path.join(IR_DIR, "reduction_max.ir")).read()))[0] == ""
+    # "<" instead of ">" is a min tree: another program
+    assert split_tag(hip.generate_source(reduction_max_ir().replace("(gt ", "(lt ", 1)))[0] == ""
+    assert split_tag(hip.generate_source(reduction_max_ir().replace("(i32 32)", "(i32 33)", 1)))[0] == ""

@@ -246,3 +246,39 @@ def test_fill_uniform_is_counter_based_and_in_range(oracle):
     assert not np.array_equal(x, oracle.fill_uniform(100000, seed=0xC))
     y = oracle.fill_uniform(1000, seed=0xA11CE, lo=-1.0, hi=1.0)
     assert y.min() >= -1.0 and y.max() < 1.0
+
+
+def test_max_tree_equals_plain_max_and_keeps_tree_nan_rules(oracle):
+    """bench_reduction_max.ml:18-100: on NaN-free data the tree is the plain maximum of the
+    block with the fill value for missing slots; with a NaN the strict '>' keeps whatever
+    sits in the left slot, which a literal thread-by-thread replay of the supersteps fixes."""
+    rng = np.random.default_rng(11)
+    n = 256 * 5 + 77
+    x = (rng.standard_normal(n) * 100).astype(np.float32)
+    got = oracle.reduce_max_block256(x)
+    exp = np.array([max(x[i:i + 256].max(), np.float32(-1000000.0)) for i in range(0, n, 256)], np.float32)
+    assert np.array_equal(got, exp)
+    # all values below the fill: the partial block reports the fill, full blocks do not
+    y = np.full(300, -2000000.0, np.float32)
+    assert oracle.reduce_max_block256(y).tolist() == [-2000000.0, -1000000.0]
+    # the reference's own input and check (bench_reduction_max.ml:95-101,159-166):
+    # input[i] = i mod 10000, max over the partials = max over the input, within 1e-5
+    z = (np.arange(25000) % 10000).astype(np.float32)
+    assert abs(float(oracle.reduce_max_block256(z).max()) - 9999.0) < 1e-5
+
+    def replay(block):
+        s = [float(v) for v in block] + [-1000000.0] * (256 - len(block))
+        half = 128
+        while half >= 1:
+            for t in range(half):       # one superstep: reads and writes touch disjoint slots
+                a, b = s[t], s[t + half]
+                if b > a:
+                    s[t] = b
+            half //= 2
+        return np.float32(s[0])
+    w = x[:256].copy()
+    w[3] = np.nan      # left slot of a pair: survives every comparison it takes part in
+    w[200] = np.nan    # right slot: never greater, dropped
+    got = oracle.reduce_max_block256(w)
+    exp = replay(w)
+    assert (np.isnan(got[0]) and np.isnan(exp)) or got[0] == exp
