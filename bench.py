@@ -31,10 +31,10 @@ NOMINAL_CLOCK_MHZ = 2400.0
 # HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (KiB per dispatch,
 # FETCH_SIZE scaled by 2.0 and WRITE_SIZE by 1.0 after calibration against a plain 1 GiB copy).
 MEASURED_TRAFFIC_BYTES = {
-    "triad_sum_2p28": (1048592 * 2 + 1050631) * 1024,
-    "gemm_bf16_8192": (800150 * 2 + 262144) * 1024,
-    "gemm_f32_8192": (1747126 * 2 + 262144) * 1024,
-    "gemm_f16_epilogue": (308713 * 2 + 187093) * 1024,
+    "triad_sum_2p28": (1048600 * 2 + 1050630) * 1024,
+    "gemm_bf16_8192": (791638 * 2 + 262153) * 1024,
+    "gemm_f32_8192": (1747220 * 2 + 262153) * 1024,
+    "gemm_f16_epilogue": (307325 * 2 + 176779) * 1024,
 }
 PEAK_MFMA_TFLOPS = {"bf16": 2500.0, "f16": 2500.0, "f32": 157.3}
 
@@ -181,15 +181,24 @@ def measure(name, torch, hip, steps, warmup):
         res["roofline"]["probe_kernels_GBs"] = hbm_ceiling(torch, hip)
     if info["bound"] == "mfma":
         # shader clock the kernel actually ran at (in-kernel cycle counter against the
-        # constant-rate wall clock), over back-to-back launches as in the timed loop
+        # constant-rate wall clock), and the rate of those very launches against the peak
+        # scaled to that clock
         with hip.clock_probe() as probe:
+            pairs = []
             for _ in range(min(steps, 10)):
+                probe.buf.zero_()
+                ev.start()
                 step()
-            mhz = probe.mhz()
-        if mhz:
+                ms = ev.stop_ms()
+                mhz = probe.mhz()
+                if mhz:
+                    pairs.append((ms, mhz))
+        if pairs:
+            pairs.sort()
+            ms, mhz = pairs[len(pairs) // 2]
             res["roofline"]["shader_clock_mhz"] = round(mhz, 1)
             res["roofline"]["frac_of_peak_at_that_clock"] = round(
-                achieved / (info["peak"] * mhz / NOMINAL_CLOCK_MHZ), 4)
+                info["work"] / (ms * 1e-3) / info["work_unit"] / (info["peak"] * mhz / NOMINAL_CLOCK_MHZ), 4)
     return res
 
 
