@@ -46,7 +46,7 @@ def parse():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--workload", default="gemm_bf16_8192",
                     choices=["gemm_bf16_8192", "triad_sum_2p28", "gemm_f32_8192", "gemm_f32_1024",
-                             "gemm_f16_epilogue", "copy_1gib"])
+                             "gemm_f16_epilogue", "copy_1gib", "vendor_gemm_bf16_8192"])
     ap.add_argument("--no-also", action="store_true", help="measure only the headline workload")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     return ap.parse_args()
@@ -124,6 +124,20 @@ def make_workload(name, torch, hip):
                     config={"workload": "bf16-in f32-acc GEMM C=A.B row-major, N(0,0.02)",
                             "m": s, "n": s, "k": s})
         return (lambda: hip.gemm_bf16(a, b, out=c)), info
+    if name == "vendor_gemm_bf16_8192":
+        # the vendor library's GEMM (torch.matmul -> hipBLASLt) on the headline inputs, for
+        # side-by-side profiles; it writes bf16 C where the kernel here writes f32
+        s = 8192
+        g.manual_seed(0xA4)
+        a = (torch.randn(s, s, device="cuda", generator=g) * 0.02).bfloat16()
+        g.manual_seed(0xB4)
+        b = (torch.randn(s, s, device="cuda", generator=g) * 0.02).bfloat16()
+        c = torch.empty(s, s, device="cuda", dtype=torch.bfloat16)
+        info = dict(metric="vendor library GEMM TFLOP/s at 8192^3 (bf16 in, bf16 out)", unit="TFLOP/s",
+                    dtype="bf16", work=2.0 * s ** 3, work_unit=1e12, bound="mfma",
+                    peak=PEAK_MFMA_TFLOPS["bf16"], kernel="hipBLASLt (torch.matmul)",
+                    config={"workload": "torch.matmul bf16, N(0,0.02)", "m": s, "n": s, "k": s})
+        return (lambda: torch.matmul(a, b, out=c)), info
     if name == "gemm_f16_epilogue":
         m, n, k = 4095, 11008, 4096
         g.manual_seed(0xA5)
@@ -316,7 +330,7 @@ def main():
         "data": "synthetic", "config": head["config"], "roofline": head["roofline"],
         "gpu_ms_per_step_events": head["gpu_ms_per_step_events"],
     }
-    if not args.no_cpu_baseline and args.workload != "copy_1gib":
+    if not args.no_cpu_baseline and args.workload not in ("copy_1gib", "vendor_gemm_bf16_8192"):
         out["cpu_baseline"] = cpu_baseline(args.workload)
     if not args.no_also:
         also = []

@@ -22,17 +22,19 @@
 //     consecutive LDS with no register staging and no ds_write (the buffer form: the
 //     global_load form of the same transfer slows MFMA issue down).  Rows cannot be padded that
 //     way, so bank conflicts are removed by an XOR swizzle applied on the global-address
-//     side (which chunk a lane fetches) and again by the readers.  K slabs of 32 stream
-//     through a ring of 4 LDS stages (128 KiB): the DMA of slab s+4 is issued right after
-//     the barrier inside slab s, so three slabs of MFMA work cover its latency; the barrier
-//     sits before the LAST k-step of a slab, and the first fragments of the next slab are
-//     fetched under that step's MFMAs, so no LDS latency is exposed at slab boundaries.
-//     Inside a k-step the LDS reads of the next step's fragments are interleaved behind the
-//     first MFMAs (sched_group_barrier).
+//     side (which chunk a lane fetches) and again by the readers.  A streams through a ring
+//     of 2 LDS stages of K = 64 (whole 128-byte lines per request), B through a ring of 4
+//     slabs of K = 32 (128 KiB in all): a stage is refilled as soon as the barrier inside
+//     the slab that read it last has passed, so one to three slabs of MFMA work cover the
+//     latency; the barrier sits before the LAST k-step of a slab, and the first fragments of
+//     the next slab are fetched under that step's MFMAs, so no LDS latency is exposed at
+//     slab boundaries.  Inside a k-step the LDS reads of the next step's fragments are
+//     interleaved behind the first MFMAs (sched_group_barrier).
 //   gemm16_staged_kernel (any K % 8 == 0): global -> registers -> LDS with zero fill for the
 //     K tail, rows padded (144 / 544 bytes) instead of swizzled, two LDS stages of K = 64.
 //   gemm16_simple_kernel: any shape and alignment, one thread per C element.
 #include <type_traits>
+#include <utility>
 
 #include "common.hpp"
 #include "gemm_common.hpp"
@@ -158,12 +160,45 @@ __device__ __forceinline__ void epilogue(f32x16 (&acc)[4][TJ], float *__restrict
 }
 
 // ---- direct-to-LDS kernel ---------------------------------------------------------
-// BKT: K extent of one slab (32 or 64); NS: ring stages.  The DMA of slab s+NS is issued
-// after the barrier inside slab s, so NS-1 slabs of MFMA work cover its latency.
+// A moves in stages of BKA k (ring of NA), B in slabs of BKB k (ring of NB); RA = BKA / BKB
+// B slabs consume one A stage.  Default: BKA = 64, NA = 2, BKB = 32, NB = 4.  A rows are
+// K-contiguous in memory, so a 32-wide A slab would touch half of each 128-byte line and
+// the next slab the other half (two L1 -> L2 requests per line: a third more requests
+// over the whole kernel, and the address path stalls on them); with 64-wide A stages
+// every request is a whole line, while B, whose rows are N-contiguous (512 bytes of a row
+// per tile), keeps the finer slabs and the deeper ring.  One barrier per B slab.
 // TJ: 32-column MFMA tiles per wave along N.  TJ = 2: 8 waves (2 x 4) of 128 x 64, two
 // per SIMD; TJ = 4: 4 waves (2 x 2) of 128 x 128, one per SIMD with the 256 accumulator
 // registers in the AGPR half of the register file (fewer LDS bytes read per flop).
-template <bool Bf16, int Epi, int BKT, int NS, int TJ>
+//
+// Order of a wave's transfers (what vmcnt counts): top of slab j: B(j-1+NB), into the stage
+// slab j-1 used; after the barrier of slab j: the A stage that slab j was the last to read.
+constexpr int dma_allowed_in_flight(int I, int RA, int NA, int NB, int DA, int DB) {
+  // Transfers that may still be in flight at the barrier of slab s = I (mod period) once
+  // everything slab s+1 reads has landed: those issued after the later of B(s+1) and the
+  // A stage that slab s+1 starts (if it starts one).  Event 2j = top of slab j, 2j+1 = its
+  // barrier.
+  const int s = I + 64 * RA * NA * NB;
+  int need = 2 * (s + 2 - NB);
+  if ((s + 1) % RA == 0) {
+    const int ev = 2 * (s + RA - RA * NA) + 1;
+    if (ev > need) need = ev;
+  }
+  int count = 0;
+  for (int e = need + 1; e < 2 * s + 1; ++e) {
+    const int j = e / 2;
+    if (e % 2 == 0) count += DB;
+    else if (j % RA == RA - 1) count += DA;
+  }
+  return count;
+}
+constexpr int lcm_int(int a, int b) {
+  int m = a;
+  while (m % b != 0) m += a;
+  return m;
+}
+
+template <bool Bf16, int Epi, int BKA, int BKB, int NA, int NB, int TJ>
 __global__ __launch_bounds__(64 * 2 * (8 / TJ)) void gemm16_dma_kernel(const uint16_t *__restrict__ A,
                                                              const uint16_t *__restrict__ B,
                                                              float *__restrict__ C,
@@ -172,15 +207,21 @@ __global__ __launch_bounds__(64 * 2 * (8 / TJ)) void gemm16_dma_kernel(const uin
                                                              int N, int K, int tiles_m,
                                                              int tiles_n, int xcd_remap,
                                                              unsigned long long *probe) {
-  constexpr int KK = BKT / 16;                 // MFMA k-steps per slab
-  constexpr int A_ROW = BKT * 2;               // bytes per A row in LDS (unpadded)
+  constexpr int KKB = BKB / 16;                // MFMA k-steps per B slab
+  constexpr int RA = BKA / BKB;                // B slabs per A stage
+  constexpr int A_ROW = BKA * 2;               // bytes per A row in LDS (unpadded)
   constexpr int A_ROWS_PER_DMA = 1024 / A_ROW; // rows one wave-wide DMA fills
   constexpr int A_CHUNKS = A_ROW / 16;
-  constexpr int A_BYTES_S = BM * A_ROW, B_BYTES_S = BKT * BN * 2;
+  constexpr int A_BYTES_S = BM * A_ROW, B_BYTES_S = BKB * BN * 2;
   constexpr int WN = 8 / TJ;                   // waves along N (4 or 2); 2 along M
   constexpr int NWAVES = 2 * WN;
-  constexpr int DMA_PER_WAVE = A_BYTES_S / 1024 / NWAVES;   // per operand, per slab
-  static_assert(NS * (A_BYTES_S + B_BYTES_S) <= 160 * 1024, "LDS ring too large");
+  constexpr int DA = A_BYTES_S / 1024 / NWAVES;   // transfers per wave and A stage
+  constexpr int DB = B_BYTES_S / 1024 / NWAVES;   // transfers per wave and B slab
+  constexpr int P = lcm_int(NB, RA * NA);         // slabs after which the stage pattern repeats
+  static_assert(KKB >= 2 && KKB % 2 == 0 && BKA % BKB == 0, "slab shapes");
+  static_assert(NA >= 2 && NB >= 2 && RA * (NA - 1) >= 1, "ring depths");
+  static_assert(NA * A_BYTES_S + NB * B_BYTES_S <= 160 * 1024, "LDS ring too large");
+  static_assert((NB - 1) * DB + NA * DA < 64, "vmcnt range");
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
@@ -207,7 +248,7 @@ __global__ __launch_bounds__(64 * 2 * (8 / TJ)) void gemm16_dma_kernel(const uin
   //      spread 64 bytes apart: slot = c ^ ((row & 3) << 2).
   auto a_swz = [](int row) { return A_CHUNKS == 8 ? ((row >> 1) & 7) : ((row >> 2) & 3); };
 
-  // ---- DMA source addresses (slab 0) ---------------------------------------------
+  // ---- DMA source addresses (stage / slab 0) ---------------------------------------
   // A: wave-instruction q = wave + NWAVES*i fills rows q*R .. q*R+R-1 (R = A_ROWS_PER_DMA);
   //    lane l -> row q*R + l/A_CHUNKS, LDS slot l%A_CHUNKS, global chunk slot ^ a_swz(row).
   // B: instruction q fills rows 2q, 2q+1; lane l -> row 2q + l/32, slot l%32,
@@ -216,13 +257,17 @@ __global__ __launch_bounds__(64 * 2 * (8 / TJ)) void gemm16_dma_kernel(const uin
   // never stored.
   // Addresses are (uniform 64-bit base) + (per-lane 32-bit byte offset), the form the
   // hardware takes as scalar base + vector offset, so only one register per DMA is kept.
-  uint32_t a_off[DMA_PER_WAVE], b_off[DMA_PER_WAVE];
+  uint32_t a_off[DA], b_off[DB];
 #pragma unroll
-  for (int i = 0; i < DMA_PER_WAVE; ++i) {
+  for (int i = 0; i < DA; ++i) {
     const int q = wave + NWAVES * i;
     const int arow_t = q * A_ROWS_PER_DMA + lane / A_CHUNKS;
     const int arow = min(arow_t, M - 1 - m0);
     a_off[i] = (static_cast<uint32_t>(arow) * K + (((lane % A_CHUNKS) ^ a_swz(arow_t)) << 3)) * 2u;
+  }
+#pragma unroll
+  for (int i = 0; i < DB; ++i) {
+    const int q = wave + NWAVES * i;
     const int brow = 2 * q + (lane >> 5);
     const int bchunk = (lane & 31) ^ ((brow & 3) << 2);
     const int bcol = min(n0 + bchunk * 8, N - 8);
@@ -230,8 +275,8 @@ __global__ __launch_bounds__(64 * 2 * (8 / TJ)) void gemm16_dma_kernel(const uin
   }
   const char *a_base = reinterpret_cast<const char *>(A + static_cast<int64_t>(m0) * K);
   const char *b_base = reinterpret_cast<const char *>(B);
-  const int64_t b_slab_bytes = static_cast<int64_t>(BKT) * N * 2;
-  const int nslabs = K / BKT;
+  const int64_t b_slab_bytes = static_cast<int64_t>(BKB) * N * 2;
+  const int nslabs = K / BKB, nstages = K / BKA;
 
   f32x16 acc[4][TJ];
 #pragma unroll
@@ -242,12 +287,13 @@ __global__ __launch_bounds__(64 * 2 * (8 / TJ)) void gemm16_dma_kernel(const uin
       for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
 
   // ---- fragment read offsets ------------------------------------------------------
-  // A: row = wm*128 + i*32 + lm, chunk = 2*kk + lh, slot = chunk ^ a_swz(row).  Since
-  //    2*kk and lh occupy different bits, slot = (lh ^ a_swz) ^ 2*kk: the address for
-  //    k-step kk is one base XOR (kk << 5), and i*32 rows is a constant offset.
+  // A: row = wm*128 + i*32 + lm, chunk = 2*ka + lh (ka = k-step within the stage),
+  //    slot = chunk ^ a_swz(row).  Since 2*ka and lh occupy different bits,
+  //    slot = (lh ^ a_swz) ^ 2*ka: the address for k-step ka is one base XOR (ka << 5),
+  //    and i*32 rows is a constant offset.
   // B (transposing read): 16-lane group g16 = lane/16: n half = g16 & 1, k half = lh; lane li
   //    supplies row (li>>2) of its 4-row block and the 8 bytes at n offset 4*(li&3).  Rows
-  //    kk*16 + lh*8 + {0..3} and +4 share (row & 3) = li>>2, so the swizzle XOR is the same
+  //    kb*16 + lh*8 + {0..3} and +4 share (row & 3) = li>>2, so the swizzle XOR is the same
   //    for both reads; j*64 bytes only touches bit 6, i.e. another XOR.
   const int a_row = wm * 128 + lm;
   int a_addr0 = a_row * A_ROW + ((lh ^ a_swz(a_row)) << 4);
@@ -256,29 +302,26 @@ __global__ __launch_bounds__(64 * 2 * (8 / TJ)) void gemm16_dma_kernel(const uin
   int b_addr0 = (lh * 8 + b_r) * 512 +
                 (((wn * (32 * TJ) + ((lane >> 4) & 1) * 16) * 2 + (li & 3) * 8) ^ (b_r << 6));
 
-  // Slab index past the end is clamped: the tail keeps issuing (redundant) DMA so that the
-  // number of outstanding transfers per wave stays the same in every iteration.
-  // A: one resource for the tile's row panel, the slab selects a scalar byte offset.
+  // Indices past the end are clamped: the tail keeps issuing (redundant) DMA into stages
+  // nobody reads any more, so that the count of outstanding transfers per wave follows the
+  // same pattern in every iteration.
+  // A: one resource for the tile's row panel, the stage selects a scalar byte offset.
   // B: the resource is rebased to the slab's first row (keeps every offset below 2^31).
   const __amdgpu_buffer_rsrc_t a_rsrc = make_rsrc(a_base, 0x80000000u);
-  auto issue_a = [&](char *sa, int slab) {
-    const int sl = min(slab, nslabs - 1);
-    const uint32_t a_so = static_cast<uint32_t>(sl) * (BKT * 2);
+  auto issue_a = [&](char *sa, int stage) {
+    const uint32_t a_so = static_cast<uint32_t>(min(stage, nstages - 1)) * (BKA * 2);
 #pragma unroll
-    for (int i = 0; i < DMA_PER_WAVE; ++i) dma16(a_rsrc, a_off[i], a_so, sa + (wave + NWAVES * i) * 1024);
+    for (int i = 0; i < DA; ++i) dma16(a_rsrc, a_off[i], a_so, sa + (wave + NWAVES * i) * 1024);
   };
   auto issue_b = [&](char *sb, int slab) {
     const int sl = min(slab, nslabs - 1);
     const __amdgpu_buffer_rsrc_t b_rsrc = make_rsrc(b_base + sl * b_slab_bytes, 0x80000000u);
 #pragma unroll
-    for (int i = 0; i < DMA_PER_WAVE; ++i) dma16(b_rsrc, b_off[i], 0u, sb + (wave + NWAVES * i) * 1024);
+    for (int i = 0; i < DB; ++i) dma16(b_rsrc, b_off[i], 0u, sb + (wave + NWAVES * i) * 1024);
   };
-  auto issue = [&](char *sa, char *sb, int slab) {
-    issue_a(sa, slab);
-    issue_b(sb, slab);
-  };
-  auto load_frags = [&](const char *sa, const char *sb, int kk, u32x4 (&af)[4], u32x4 (&bf)[TJ]) {
-    const char *pa = sa + (a_addr0 ^ (kk << 5));
+  // ka: k-step within the A stage, kb: k-step within the B slab
+  auto load_frags = [&](const char *sa, const char *sb, int ka, int kb, u32x4 (&af)[4], u32x4 (&bf)[TJ]) {
+    const char *pa = sa + (a_addr0 ^ (ka << 5));
 #pragma unroll
     for (int i = 0; i < 4; ++i)
       af[i] = *reinterpret_cast<const u32x4 *>(pa + i * 32 * A_ROW);
@@ -286,7 +329,7 @@ __global__ __launch_bounds__(64 * 2 * (8 / TJ)) void gemm16_dma_kernel(const uin
     for (int j = 0; j < TJ; ++j) {
       // j*64 bytes: with TJ = 4 the wave's 256-byte column span is 256-byte aligned, so
       // adding j*64 never carries into the bits the swizzle touches differently
-      const int off = (b_addr0 ^ (j << 6)) + kk * 16 * 512;
+      const int off = (b_addr0 ^ (j << 6)) + kb * 16 * 512;
       u32x2 lo = lds_read_tr16(sb, off);
       u32x2 hi = lds_read_tr16(sb, off + 4 * 512);
       bf[j] = u32x4{lo.x, lo.y, hi.x, hi.y};
@@ -298,8 +341,8 @@ __global__ __launch_bounds__(64 * 2 * (8 / TJ)) void gemm16_dma_kernel(const uin
 #pragma unroll
       for (int j = 0; j < TJ; ++j) acc[i][j] = mfma<Bf16>(af[i], bf[j], acc[i][j]);
   };
-  // Issue order inside one k-step: the 8 LDS reads of the next step's fragments go out in
-  // pairs behind the first four MFMAs; the last four MFMAs cover their latency.
+  // Issue order inside one k-step: the LDS reads of the next step's fragments go out in
+  // pairs behind the first MFMAs; the remaining MFMAs cover their latency.
   auto interleave = [] {
     constexpr int READS = 4 + 2 * TJ, MFMAS = 4 * TJ;
 #pragma unroll
@@ -313,74 +356,66 @@ __global__ __launch_bounds__(64 * 2 * (8 / TJ)) void gemm16_dma_kernel(const uin
 
   u32x4 af[2][4], bf[2][TJ];
 
-  // One slab: stage `cur` is consumed, `nxt` is the stage of slab s+1; after the barrier
-  // every wave is done reading `cur`, so it is refilled with slab s+NS: the A half right
-  // away, the B half one k-step later (at the top of the next slab, into `pb`, the stage
-  // consumed before this one), which spreads the requests over the slab.
-  auto slab = [&](char *ca, char *cb, const char *na, const char *nb, char *pb, int s) {
+  // One B slab; I = its index modulo P fixes every stage at compile time (each stage is
+  // its own array, so the compiler does not order DMA into one stage against reads of
+  // another).  After the barrier every wave is done reading the slab's B stage, which the
+  // next slab's top refills, and, on the last slab of an A stage, that stage, which is
+  // refilled at once.  The barrier sits before the last k-step, whose MFMAs cover the
+  // first fragment reads of the next slab.
+  auto slab = [&](auto ic, int s) {
+    constexpr int I = decltype(ic)::value;
+    constexpr int In = (I + 1) % P;
+    constexpr int ia = (I / RA) % NA, ib = I % NB, ibp = (I + NB - 1) % NB;
+    constexpr int ian = (In / RA) % NA, ibn = In % NB;
+    constexpr int ka0 = (I % RA) * KKB, ka0n = (In % RA) * KKB;
     // Keep the per-stage LDS addresses from being hoisted out of the K loop (they would
     // occupy a register per stage and k-step): the bases are made opaque once per slab.
     asm volatile("" : "+v"(a_addr0), "+v"(b_addr0));
 #pragma unroll
-    for (int kk = 0; kk + 1 < KK; ++kk) {
-      if (kk == 0) issue_b(pb, s - 1 + NS);
-      load_frags(ca, cb, kk + 1, af[(kk + 1) & 1], bf[(kk + 1) & 1]);
+    for (int kk = 0; kk + 1 < KKB; ++kk) {
+      if (kk == 0) issue_b(lds_ring<20 + ibp, B_BYTES_S>, s - 1 + NB);
+      load_frags(lds_ring<10 + ia, A_BYTES_S>, lds_ring<20 + ib, B_BYTES_S>, ka0 + kk + 1, kk + 1,
+                 af[(kk + 1) & 1], bf[(kk + 1) & 1]);
       mfma_step(af[kk & 1], bf[kk & 1]);
       interleave();
     }
-    // own DMA of slab s+1 landed (NS-2 later slabs may still be in flight), own reads done
-    __builtin_amdgcn_s_waitcnt(waitcnt_vm_lgkm0((NS - 2) * 2 * DMA_PER_WAVE));
+    __builtin_amdgcn_s_waitcnt(waitcnt_vm_lgkm0(dma_allowed_in_flight(I, RA, NA, NB, DA, DB)));
     barrier_no_fence();
-    issue_a(ca, s + NS);
-    load_frags(na, nb, 0, af[0], bf[0]);
-    mfma_step(af[(KK - 1) & 1], bf[(KK - 1) & 1]);
+    if constexpr (I % RA == RA - 1) issue_a(lds_ring<10 + ia, A_BYTES_S>, s / RA + NA);
+    load_frags(lds_ring<10 + ian, A_BYTES_S>, lds_ring<20 + ibn, B_BYTES_S>, ka0n, 0, af[0], bf[0]);
+    mfma_step(af[(KKB - 1) & 1], bf[(KKB - 1) & 1]);
     interleave();
   };
 
-  // prologue: fill the ring (the B half of the last stage follows in slab 0), wait for
-  // slab 0, fetch its first fragments
-  issue(lds_ring<0, A_BYTES_S>, lds_ring<1, B_BYTES_S>, 0);
-  if constexpr (NS == 4) {
-    issue(lds_ring<2, A_BYTES_S>, lds_ring<3, B_BYTES_S>, 1);
-    issue(lds_ring<4, A_BYTES_S>, lds_ring<5, B_BYTES_S>, 2);
-  }
-  issue_a(lds_ring<2 * (NS - 1), A_BYTES_S>, NS - 1);
-  __builtin_amdgcn_s_waitcnt(waitcnt_vm_lgkm0((NS - 2) * 2 * DMA_PER_WAVE + DMA_PER_WAVE));
+  // prologue: fill both rings except the last B stage (the top of slab 0 issues it) and
+  // wait for all of it, so that from here on a wave never has more in flight than the
+  // steady-state pattern assumes
+  [&]<int... Is>(std::integer_sequence<int, Is...>) {
+    (issue_a(lds_ring<10 + Is, A_BYTES_S>, Is), ...);
+  }(std::make_integer_sequence<int, NA>{});
+  [&]<int... Is>(std::integer_sequence<int, Is...>) {
+    (issue_b(lds_ring<20 + Is, B_BYTES_S>, Is), ...);
+  }(std::make_integer_sequence<int, NB - 1>{});
+  __builtin_amdgcn_s_waitcnt(waitcnt_vm_lgkm0(0));
   barrier_no_fence();
-  load_frags(lds_ring<0, A_BYTES_S>, lds_ring<1, B_BYTES_S>, 0, af[0], bf[0]);
+  load_frags(lds_ring<10, A_BYTES_S>, lds_ring<20, B_BYTES_S>, 0, 0, af[0], bf[0]);
   __builtin_amdgcn_sched_barrier(0);
 
-  // The ring is unrolled so that every stage is a compile-time array: whole rounds first
-  // (no exits inside the round, which keeps the accumulators in place), then the
-  // remaining nslabs % NS slabs.
-  auto ring_slab = [&](auto st_c, int s) {
-    constexpr int st = decltype(st_c)::value;
-    constexpr int nx = (st + 1) % NS, pv = (st + NS - 1) % NS;
-    slab(lds_ring<2 * st, A_BYTES_S>, lds_ring<2 * st + 1, B_BYTES_S>, lds_ring<2 * nx, A_BYTES_S>,
-         lds_ring<2 * nx + 1, B_BYTES_S>, lds_ring<2 * pv + 1, B_BYTES_S>, s);
-  };
-  using I0 = std::integral_constant<int, 0>;
-  using I1 = std::integral_constant<int, 1>;
-  using I2 = std::integral_constant<int, 2>;
-  using I3 = std::integral_constant<int, 3>;
-  const int full = nslabs - nslabs % NS;
-  for (int s = 0; s < full; s += NS) {
-    ring_slab(I0{}, s);
-    ring_slab(I1{}, s + 1);
-    if constexpr (NS == 4) {
-      ring_slab(I2{}, s + 2);
-      ring_slab(I3{}, s + 3);
-    }
+  // Whole periods first (no exits inside a period, which keeps the accumulators in
+  // place), then the remaining nslabs % P slabs.
+  const int full = nslabs - nslabs % P;
+  for (int s = 0; s < full; s += P) {
+    [&]<int... Is>(std::integer_sequence<int, Is...>) {
+      (slab(std::integral_constant<int, Is>{}, s + Is), ...);
+    }(std::make_integer_sequence<int, P>{});
   }
-  if (full < nslabs) ring_slab(I0{}, full);
-  if constexpr (NS == 4) {
-    if (full + 1 < nslabs) ring_slab(I1{}, full + 1);
-    if (full + 2 < nslabs) ring_slab(I2{}, full + 2);
-  }
+  [&]<int... Is>(std::integer_sequence<int, Is...>) {
+    ((full + Is < nslabs ? slab(std::integral_constant<int, Is>{}, full + Is) : (void)0), ...);
+  }(std::make_integer_sequence<int, P - 1>{});
   // drain the (redundant) tail DMA before the LDS is released
   __builtin_amdgcn_s_waitcnt(waitcnt_vm_lgkm0(0));
   epilogue<Epi, TJ>(acc, C, bias, rowsum, M, N, m0, wm, wn, n0 + wn * (32 * TJ), lm, lh,
-                    reinterpret_cast<float *>(lds_ring<0, A_BYTES_S>));
+                    reinterpret_cast<float *>(lds_ring<10, A_BYTES_S>));
   if (probe && tid == 0) {
     probe[2 * blockIdx.x] = static_cast<unsigned long long>(clock64() - probe_c0);
     probe[2 * blockIdx.x + 1] = static_cast<unsigned long long>(wall_clock64() - probe_t0);
@@ -562,16 +597,21 @@ int launch_gemm16(const uint16_t *a, const uint16_t *b, float *c, const float *b
     const bool offsets_ok = static_cast<int64_t>(k) * 256 * 2 < 0x7FFFFFFF &&
                             static_cast<int64_t>(n) * 64 * 2 < 0x7FFFFFFF;
     if (k % BK == 0 && offsets_ok && tunable("gemm16.force_staged", 0) == 0) {
-      const int ring = (int)tunable("gemm16.ring", 4), tj = (int)tunable("gemm16.tj", 2);
+      // shape knobs for sweeps: gemm16.ring 0 = A in K=64 stages x2 + B in K=32 slabs x4
+      // (default), 4 = both in K=32 slabs x4, 2 = both in K=64 slabs x2; gemm16.tj 2 | 4
+      const int ring = (int)tunable("gemm16.ring", 0), tj = (int)tunable("gemm16.tj", 2);
       const dim3 grid(tiles_m * tiles_n);
       unsigned long long *probe = clock_probe(static_cast<int64_t>(tiles_m) * tiles_n);
-#define SAREK_LAUNCH_DMA(BKT, NS, TJ)                                                             \
-  hipLaunchKernelGGL((gemm16_dma_kernel<Bf16, Epi, BKT, NS, TJ>), grid, dim3(64 * 2 * (8 / TJ)), 0, \
-                     st, a, b, c, bias, rowsum, m, n, k, tiles_m, tiles_n, remap, probe)
-      if (ring == 4 && tj == 2) SAREK_LAUNCH_DMA(32, 4, 2);
-      else if (ring == 4) SAREK_LAUNCH_DMA(32, 4, 4);
-      else if (tj == 2) SAREK_LAUNCH_DMA(64, 2, 2);
-      else SAREK_LAUNCH_DMA(64, 2, 4);
+#define SAREK_LAUNCH_DMA(BKA, BKB, NA, NB, TJ)                                                      \
+  hipLaunchKernelGGL((gemm16_dma_kernel<Bf16, Epi, BKA, BKB, NA, NB, TJ>), grid,                      \
+                     dim3(64 * 2 * (8 / TJ)), 0, st, a, b, c, bias, rowsum, m, n, k, tiles_m,         \
+                     tiles_n, remap, probe)
+      if (ring == 4 && tj == 2) SAREK_LAUNCH_DMA(32, 32, 4, 4, 2);
+      else if (ring == 4) SAREK_LAUNCH_DMA(32, 32, 4, 4, 4);
+      else if (ring == 2 && tj == 2) SAREK_LAUNCH_DMA(64, 64, 2, 2, 2);
+      else if (ring == 2) SAREK_LAUNCH_DMA(64, 64, 2, 2, 4);
+      else if (tj == 4) SAREK_LAUNCH_DMA(64, 32, 2, 4, 4);
+      else SAREK_LAUNCH_DMA(64, 32, 2, 4, 2);
 #undef SAREK_LAUNCH_DMA
       return check_launch("gemm16 kernel launch");
     }
