@@ -217,3 +217,36 @@ def test_clock_probe_records_cycles_and_ticks(hip, torch_cuda):
     with hip.clock_probe(workgroups=64) as probe:
         hip.gemm_f32(x, x[:256, :].contiguous())
         assert len(probe.pairs()) > 0 and 500 < probe.mhz() < 2600
+
+
+@pytest.mark.parametrize("tile", [64, 128, 256])
+@pytest.mark.parametrize("m,n,k", [(300, 520, 32), (257, 132, 96), (512, 768, 160), (70, 1028, 288)])
+def test_gemm_f32_every_tile_shape(hip, oracle, torch_cuda, tile, m, n, k):
+    """The three direct-to-LDS tile shapes on ragged M, N and on K values that end the ring
+    at every position (K/32 = 1, 3, 5, 9 slabs against a ring of 4)."""
+    a = oracle.fill_uniform(m * k, seed=m + tile, lo=-1, hi=1).reshape(m, k)
+    b = oracle.fill_uniform(k * n, seed=n + tile, lo=-1, hi=1).reshape(k, n)
+    hip.set_tunable("gemm_f32.tile", tile)
+    try:
+        c = hip.gemm_f32(dev(torch_cuda, a), dev(torch_cuda, b)).cpu().numpy()
+    finally:
+        hip.set_tunable("gemm_f32.tile", 0)
+    assert np.abs(c - oracle.gemm(a, b)).max() <= f32_tol(a, b, k)
+
+
+@pytest.mark.parametrize("ring,tj", [(0, 2), (0, 4), (4, 2), (4, 4), (2, 2), (2, 4)])
+@pytest.mark.parametrize("m,n,k", [(300, 520, 64), (257, 136, 192), (512, 768, 448), (70, 1032, 1216)])
+def test_gemm16_every_ring_shape(hip, oracle, torch_cuda, ring, tj, m, n, k):
+    """Every instantiation of the direct-to-LDS 16-bit kernel (A/B ring shapes, 8 or 4 waves)
+    on ragged M, N and on K values that end the stage pattern at different positions."""
+    a = normal16(oracle, (m, k), m + ring, "bf16")
+    b = normal16(oracle, (k, n), n + tj, "bf16")
+    ref = oracle.gemm(a, b)
+    hip.set_tunable("gemm16.ring", ring)
+    hip.set_tunable("gemm16.tj", tj)
+    try:
+        c = hip.gemm_bf16(dev(torch_cuda, a).bfloat16(), dev(torch_cuda, b).bfloat16()).cpu().numpy()
+    finally:
+        hip.set_tunable("gemm16.ring", 0)
+        hip.set_tunable("gemm16.tj", 2)
+    assert np.abs(c - ref).max() / np.abs(ref).max() < 1e-4
