@@ -249,6 +249,24 @@ int sarek_hip_gemm_f16_bias_relu_rowsum(const uint16_t *a, const uint16_t *b, co
 int sarek_hip_cast_f32_to_bf16(const float *in, uint16_t *out, int64_t n, sarek_hip_stream stream);
 int sarek_hip_cast_f32_to_f16(const float *in, uint16_t *out, int64_t n, sarek_hip_stream stream);
 
+/* Persistent cache of compiled kernels: the reference's Framework_cache
+ * (sarek/framework/Framework_cache.ml:63-141; used there by the Vulkan plugin,
+ * sarek-vulkan/Vulkan_api.ml:1254-1283).  Directory: $XDG_CACHE_HOME, else
+ * $HOME/.cache, else the temp dir, then "/spoc"; key = MD5 hex of
+ * dev_name ^ driver_version ^ source; one file per key.  A miss or an I/O error
+ * is never an error of the call: `found` says whether an entry was read, the
+ * counters say why not.  sarek_hip_kernel_compile(_cached) stores hiprtc code
+ * objects here and looks there before compiling; SAREK_HIP_DISK_CACHE=0 in the
+ * environment switches that off.
+ * stats: out[0] hits, out[1] misses, out[2] puts, out[3] I/O errors.        */
+int sarek_hip_cache_dir(char *out, size_t out_len);
+int sarek_hip_cache_compute_key(const char *dev_name, const char *driver_version,
+                                const char *source, char out_hex[33]);
+int sarek_hip_cache_get(const char *key, void *out, size_t out_len, size_t *size, int *found);
+int sarek_hip_cache_put(const char *key, const void *data, size_t len);
+int sarek_hip_cache_get_stats(int64_t out[4]);
+int sarek_hip_cache_reset_stats(void);
+
 /* Integer tuning knob (launch shapes, tile variants), for sweeps without a
  * rebuild.  Unknown names are stored and ignored.                           */
 int sarek_hip_set_tunable(const char *name, int64_t value);

@@ -5,6 +5,8 @@
 // parameter-pointer launch).
 #include <hip/hiprtc.h>
 
+#include "code_cache.hpp"
+
 #include <cstring>
 #include <map>
 #include <mutex>
@@ -62,6 +64,34 @@ int compile_impl(const char *source, const char *kernel_name, sarek_hip_kernel *
   SAREK_HIP_TRY(hipGetDeviceProperties(&prop, dev));
   std::string arch = std::string("--offload-arch=") + prop.gcnArchName;
 
+  // Persistent cache: the code object depends on the source, the target and the compiler.
+  std::string cache_key;
+  if (cache_enabled()) {
+    int rtc_major = 0, rtc_minor = 0, runtime_version = 0;
+    (void)hiprtcVersion(&rtc_major, &rtc_minor);
+    (void)hipRuntimeGetVersion(&runtime_version);
+    cache_key = cache_compute_key(std::string(prop.name) + "|" + prop.gcnArchName,
+                                  "hiprtc " + std::to_string(rtc_major) + "." + std::to_string(rtc_minor) +
+                                      " hip " + std::to_string(runtime_version) + " -O3",
+                                  source);
+    std::vector<char> cached;
+    if (cache_get(cache_key, &cached) && !cached.empty()) {
+      auto *k = new sarek_hip_kernel_s();
+      k->name = kernel_name;
+      k->device = dev;
+      if (hipModuleLoadData(&k->module, cached.data()) == hipSuccess) {
+        if (hipModuleGetFunction(&k->function, k->module, kernel_name) == hipSuccess) {
+          *out = k;
+          return SAREK_HIP_OK;
+        }
+        (void)hipModuleUnload(k->module);
+      }
+      delete k;
+      (void)hipGetLastError();
+      cache_note_error();   // unusable entry: compile afresh and overwrite it
+    }
+  }
+
   hiprtcProgram prog;
   hiprtcResult r = hiprtcCreateProgram(&prog, source, "sarek_kernel.hip", 0, nullptr, nullptr);
   if (r != HIPRTC_SUCCESS) return rtc_fail(r, "hiprtcCreateProgram");
@@ -89,6 +119,7 @@ int compile_impl(const char *source, const char *kernel_name, sarek_hip_kernel *
   r = hiprtcGetCode(prog, code.data());
   hiprtcDestroyProgram(&prog);
   if (r != HIPRTC_SUCCESS) return rtc_fail(r, "hiprtcGetCode");
+  if (!cache_key.empty()) cache_put(cache_key, code.data(), code.size());
 
   auto *k = new sarek_hip_kernel_s();
   k->name = kernel_name;

@@ -108,6 +108,12 @@ SYMBOLS = {
     "sarek_hip_gemm_f16_bias_relu_rowsum": (_i, [_vp, _vp, _vp, _vp, _vp, _i, _i, _i, _vp]),
     "sarek_hip_cast_f32_to_bf16": (_i, [_vp, _vp, _i64, _vp]),
     "sarek_hip_cast_f32_to_f16": (_i, [_vp, _vp, _i64, _vp]),
+    "sarek_hip_cache_dir": (_i, [C.c_char_p, _sz]),
+    "sarek_hip_cache_compute_key": (_i, [C.c_char_p, C.c_char_p, C.c_char_p, C.c_char_p]),
+    "sarek_hip_cache_get": (_i, [C.c_char_p, _vp, _sz, C.POINTER(_sz), C.POINTER(_i)]),
+    "sarek_hip_cache_put": (_i, [C.c_char_p, _vp, _sz]),
+    "sarek_hip_cache_get_stats": (_i, [C.POINTER(_i64)]),
+    "sarek_hip_cache_reset_stats": (_i, []),
     "sarek_hip_set_tunable": (_i, [C.c_char_p, _i64]),
     "sarek_hip_set_clock_probe": (_i, [_vp, _i64, C.POINTER(_i64)]),
 }
@@ -142,6 +148,47 @@ def check(status):
 
 def set_tunable(name, value):
     check(lib.sarek_hip_set_tunable(name.encode(), int(value)))
+
+
+# ---------------------------------------------------------------------------
+# Persistent kernel cache (the reference's Framework_cache)
+
+def cache_dir():
+    buf = C.create_string_buffer(4096)
+    check(lib.sarek_hip_cache_dir(buf, len(buf)))
+    return buf.value.decode()
+
+
+def cache_compute_key(dev_name, driver_version, source):
+    out = C.create_string_buffer(33)
+    check(lib.sarek_hip_cache_compute_key(dev_name.encode(), driver_version.encode(), source.encode(), out))
+    return out.value.decode()
+
+
+def cache_put(key, data):
+    check(lib.sarek_hip_cache_put(key.encode(), data, len(data)))
+
+
+def cache_get(key):
+    """bytes of the entry, or None."""
+    size, found = _sz(0), _i(0)
+    buf = C.create_string_buffer(1 << 16)
+    st = lib.sarek_hip_cache_get(key.encode(), buf, len(buf), C.byref(size), C.byref(found))
+    if st == E_BUFFER_TOO_SMALL:
+        buf = C.create_string_buffer(size.value)
+        st = lib.sarek_hip_cache_get(key.encode(), buf, len(buf), C.byref(size), C.byref(found))
+    check(st)
+    return buf.raw[:size.value] if found.value else None
+
+
+def cache_stats():
+    out = (_i64 * 4)()
+    check(lib.sarek_hip_cache_get_stats(out))
+    return dict(hits=out[0], misses=out[1], puts=out[2], errors=out[3])
+
+
+def cache_reset_stats():
+    check(lib.sarek_hip_cache_reset_stats())
 
 
 class clock_probe:
