@@ -341,16 +341,25 @@ __global__ __launch_bounds__(64 * 2 * (8 / TJ)) void gemm16_dma_kernel(const uin
 #pragma unroll
       for (int j = 0; j < TJ; ++j) acc[i][j] = mfma<Bf16>(af[i], bf[j], acc[i][j]);
   };
-  // Issue order inside one k-step: the LDS reads of the next step's fragments go out in
-  // pairs behind the first MFMAs; the remaining MFMAs cover their latency.
-  auto interleave = [] {
+  // Issue order inside one k-step: an MFMA goes first, then behind each following MFMA
+  // one DMA instruction (NV of them belong to this k-step) and two LDS reads of the next
+  // step's fragments; the remaining MFMAs cover the read latency.  Left to itself the
+  // compiler bunches the DMA instructions in front of the first MFMA, where their issue
+  // time (and any back-pressure from the address path) leaves the MFMA pipe idle: pinning
+  // them behind MFMAs took 6 % (8 waves) to 9 % (4 waves) off the cycle count.
+  auto interleave = [](auto nv_c) {
+    constexpr int NV = decltype(nv_c)::value;
     constexpr int READS = 4 + 2 * TJ, MFMAS = 4 * TJ;
+    constexpr int G = READS / 2, SLOTS = NV > G ? NV : G;
+    static_assert(SLOTS + 1 <= MFMAS, "not enough MFMAs to hide the issues behind");
+    __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);                // 1 MFMA
 #pragma unroll
-    for (int g = 0; g < READS / 2; ++g) {
-      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);  // 1 MFMA
-      __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);  // 2 DS reads
+    for (int g = 0; g < SLOTS; ++g) {
+      if (g < NV) __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);  // 1 VMEM read (DMA)
+      if (g < G) __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);   // 2 DS reads
+      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
     }
-    __builtin_amdgcn_sched_group_barrier(0x008, MFMAS - READS / 2, 0);
+    __builtin_amdgcn_sched_group_barrier(0x008, MFMAS - 1 - SLOTS, 0);
     __builtin_amdgcn_sched_barrier(0);
   };
 
@@ -377,14 +386,15 @@ __global__ __launch_bounds__(64 * 2 * (8 / TJ)) void gemm16_dma_kernel(const uin
       load_frags(lds_ring<10 + ia, A_BYTES_S>, lds_ring<20 + ib, B_BYTES_S>, ka0 + kk + 1, kk + 1,
                  af[(kk + 1) & 1], bf[(kk + 1) & 1]);
       mfma_step(af[kk & 1], bf[kk & 1]);
-      interleave();
+      if (kk == 0) interleave(std::integral_constant<int, DB>{});
+      else interleave(std::integral_constant<int, 0>{});
     }
     __builtin_amdgcn_s_waitcnt(waitcnt_vm_lgkm0(dma_allowed_in_flight(I, RA, NA, NB, DA, DB)));
     barrier_no_fence();
     if constexpr (I % RA == RA - 1) issue_a(lds_ring<10 + ia, A_BYTES_S>, s / RA + NA);
     load_frags(lds_ring<10 + ian, A_BYTES_S>, lds_ring<20 + ibn, B_BYTES_S>, ka0n, 0, af[0], bf[0]);
     mfma_step(af[(KKB - 1) & 1], bf[(KKB - 1) & 1]);
-    interleave();
+    interleave(std::integral_constant<int, (I % RA == RA - 1) ? DA : 0>{});
   };
 
   // prologue: fill both rings except the last B stage (the top of slab 0 issues it) and

@@ -16,6 +16,7 @@
 // four MFMA steps; the matching B values are row 8*kk + 4h + j, column n (ds_read_b32,
 // bank-conflict free because n is contiguous).
 #include <type_traits>
+#include <utility>
 
 #include "common.hpp"
 #include "gemm_common.hpp"
@@ -262,15 +263,24 @@ __global__ __launch_bounds__(64 * WMW * WNW) void gemm_f32_dma_kernel(
           acc[i][jn] = __builtin_amdgcn_mfma_f32_32x32x2f32(af[i][j], bf[j][jn], acc[i][jn], 0, 0, 0);
         }
   };
-  auto interleave = [] {
+  // Issue order inside one k-step: behind each of the first MFMAs go the DMA instructions
+  // of this k-step (NV of them; unpinned, the compiler bunches them in front of the first
+  // MFMA, where their issue time leaves the pipe idle) and the LDS reads of the next
+  // step's fragments.
+  auto interleave = [](auto nv_c) {
+    constexpr int NV = decltype(nv_c)::value;
     constexpr int READS = TI + 4, MFMAS = 4 * TI * TJ;
     constexpr int GROUPS = READS < MFMAS ? READS : MFMAS;
-    constexpr int PER = (READS + GROUPS - 1) / GROUPS;
-#pragma unroll
-    for (int g = 0; g < GROUPS; ++g) {
-      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);    // 1 MFMA
-      __builtin_amdgcn_sched_group_barrier(0x100, PER, 0);  // DS reads
-    }
+    constexpr int PER = (READS + GROUPS - 1) / GROUPS, VPER = (NV + GROUPS - 1) / GROUPS;
+    [&]<int... Gs>(std::integer_sequence<int, Gs...>) {
+      (([] {
+         __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);    // 1 MFMA
+         if constexpr (Gs * VPER < NV)                         // DMA instructions
+           __builtin_amdgcn_sched_group_barrier(0x020, (NV - Gs * VPER) < VPER ? (NV - Gs * VPER) : VPER, 0);
+         __builtin_amdgcn_sched_group_barrier(0x100, PER, 0);  // DS reads
+       }()),
+       ...);
+    }(std::make_integer_sequence<int, GROUPS>{});
     if (MFMAS > GROUPS) __builtin_amdgcn_sched_group_barrier(0x008, MFMAS - GROUPS, 0);
     __builtin_amdgcn_sched_barrier(0);
   };
@@ -284,14 +294,14 @@ __global__ __launch_bounds__(64 * WMW * WNW) void gemm_f32_dma_kernel(
     for (int kk = 0; kk + 1 < KK; ++kk) {
       load_frags(ca, cb, kk + 1, af[(kk + 1) & 1], bf[(kk + 1) & 1]);
       mfma_step(af[kk & 1], bf[kk & 1]);
-      interleave();
+      interleave(std::integral_constant<int, 0>{});
     }
     __builtin_amdgcn_s_waitcnt(waitcnt_vm_lgkm0((NS - 2) * (A_DMA + B_DMA)));
     barrier_no_fence();
     issue(ca, cb, s + NS);
     load_frags(na, nb, 0, af[0], bf[0]);
     mfma_step(af[(KK - 1) & 1], bf[(KK - 1) & 1]);
-    interleave();
+    interleave(std::integral_constant<int, A_DMA + B_DMA>{});
   };
 
   issue(lds_ring<0, A_BYTES_S>, lds_ring<1, B_BYTES_S>, 0);
