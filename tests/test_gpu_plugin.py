@@ -307,3 +307,23 @@ def test_reduction_max_ir_end_to_end(hip, oracle, torch_cuda, specialise):
     assert path.startswith("reduce_max_block256_f32:") if specialise else path == "jit"
     assert np.array_equal(out.cpu().numpy(), oracle.reduce_max_block256(x))
     assert out.max().item() == x.max()     # the bench's own check: max of partials = max of input
+
+
+@pytest.mark.parametrize("name,size,path", [
+    ("matrix_mul_tiled", 200, "matmul_tiled_f32"), ("stream_triad", 100003, "stream_triad_f32"),
+    ("reduction", 100003, "reduce_sum_block256_f32"), ("dot_product", 100003, "dot_block256_f32"),
+    ("reduction_max", 100003, "reduce_max_block256_f32:c9742400")])
+def test_reference_benchmarks_run_and_verify(hip, torch_cuda, name, size, path):
+    """The mirrors of benchmarks/bench_*.ml: the reference's inputs, geometry and checks, served
+    by the hand kernels; and the same with the plain JIT lowering."""
+    from spoc_amd import benchmarks
+    fn = benchmarks.BENCHMARKS[name][0]
+    rec = fn(size, warmup=1, iterations=3)
+    assert rec["verified"] and rec["path"] == path and len(rec["iterations"]) == 3
+    assert rec["median_ms"] > 0 and rec["throughput_gflops"] > 0 and rec["framework"] == "HIP"
+    hip.check(hip.lib.sarek_hip_set_specialisation(0))
+    try:
+        rec = fn(size, warmup=1, iterations=2)
+    finally:
+        hip.check(hip.lib.sarek_hip_set_specialisation(1))
+    assert rec["verified"] and rec["path"] == "jit"
