@@ -32,9 +32,9 @@ NOMINAL_CLOCK_MHZ = 2400.0
 # FETCH_SIZE scaled by 2.0 and WRITE_SIZE by 1.0 after calibration against a plain 1 GiB copy).
 MEASURED_TRAFFIC_BYTES = {
     "triad_sum_2p28": (1048600 * 2 + 1050630) * 1024,
-    "gemm_bf16_8192": (791638 * 2 + 262153) * 1024,
-    "gemm_f32_8192": (1747220 * 2 + 262153) * 1024,
-    "gemm_f16_epilogue": (307325 * 2 + 176779) * 1024,
+    "gemm_bf16_8192": (793626 * 2 + 262153) * 1024,
+    "gemm_f32_8192": (1695900 * 2 + 262153) * 1024,
+    "gemm_f16_epilogue": (306687 * 2 + 176779) * 1024,
 }
 PEAK_MFMA_TFLOPS = {"bf16": 2500.0, "f16": 2500.0, "f32": 157.3}
 
