@@ -56,6 +56,7 @@ struct SExp {
 
 class Reader {
  public:
+  static constexpr int kMaxDepth = 2000;
   explicit Reader(const std::string &s) : s_(s) {}
   SExp read_all() {
     SExp e = read();
@@ -83,11 +84,17 @@ class Reader {
     e.pos = i_;
     if (s_[i_] == '(') {
       ++i_;
+      // every later pass recurses over this tree: bound its depth here, far above any
+      // real kernel, so that no input can run the caller's stack out
+      if (++depth_ > kMaxDepth)
+        throw ParseError("IR text: nesting deeper than " + std::to_string(kMaxDepth) + " at offset " +
+                         std::to_string(e.pos));
       for (;;) {
         skip();
         if (i_ >= s_.size()) throw ParseError("IR text: unbalanced '(' opened at offset " + std::to_string(e.pos));
         if (s_[i_] == ')') {
           ++i_;
+          --depth_;
           return e;
         }
         e.items.push_back(read());
@@ -119,6 +126,7 @@ class Reader {
   }
   const std::string &s_;
   size_t i_ = 0;
+  int depth_ = 0;
 };
 
 const std::string &head(const SExp &e) {

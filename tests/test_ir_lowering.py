@@ -259,3 +259,20 @@ def test_reduction_max_recognition_carries_the_fill_value(hip):
     # "<" instead of ">" is a min tree: another program
     assert split_tag(hip.generate_source(reduction_max_ir().replace("(gt ", "(lt ", 1)))[0] == ""
     assert split_tag(hip.generate_source(reduction_max_ir().replace("(i32 32)", "(i32 33)", 1)))[0] == ""
+
+
+def test_nesting_depth_is_bounded(hip):
+    """Every pass recurses over the tree; the reader refuses trees deep enough to endanger the
+    caller's stack instead of crashing, and accepts anything a real kernel could hold."""
+    def nested(d):
+        return "(kernel k (params) (locals) (body " + "(seq " * d + "(empty)" + ")" * d + "))"
+    assert "sarek_kern" not in hip.generate_source(nested(1900))
+    for d in (2100, 200000):
+        with pytest.raises(hip.SarekHipError, match="nesting deeper than 2000"):
+            hip.generate_source(nested(d))
+    lets = 1500
+    ir = ("(kernel k (params (param (var o 1 (vec i32)))) (locals) (body " +
+          "".join(f"(let (var x{i} {i + 2} i32) (add (i32 {i}) "
+                  f"{('(var x%d %d i32)' % (i - 1, i + 1)) if i else '(i32 0)'}) " for i in range(lets)) +
+          f"(assign (lelem o (i32 0)) (var x{lets - 1} {lets + 1} i32))" + ")" * lets + "))")
+    assert f"int x{lets - 1} = " in hip.generate_source(ir)
