@@ -66,3 +66,41 @@ def test_missing_library_fails_loudly(monkeypatch, tmp_path):
     else:
         raise AssertionError("loading a missing library must raise")
     importlib.reload(real)
+
+
+C_CLIENT = r'''
+#include <stdio.h>
+#include <string.h>
+#include "sarek_hip.h"
+int main(void) {
+  char key[33], dir[4096];
+  int64_t stats[4];
+  if (sarek_hip_abi_version() <= 0) return 1;
+  if (sarek_hip_cache_compute_key("Device1", "1.0", "kernel code", key) != SAREK_HIP_OK) return 2;
+  if (strlen(key) != 32) return 3;
+  if (sarek_hip_cache_get_stats(stats) != SAREK_HIP_OK) return 4;
+  if (sarek_hip_gemm_f32(NULL, NULL, NULL, 1, 1, 1, NULL) != SAREK_HIP_E_INVALID_ARG) return 5;
+  if (strstr(sarek_hip_last_error(), "NULL") == NULL) return 6;
+  if (sarek_hip_set_tunable(NULL, 1) != SAREK_HIP_E_INVALID_ARG) return 7;
+  (void)dir;
+  printf("%s\n", key);
+  return 0;
+}
+'''
+
+
+def test_header_is_c_and_a_c_client_links(hip, tmp_path):
+    """include/sarek_hip.h is the boundary a C (or ctypes / cgo-style) client binds: it must
+    compile as plain C99 with warnings on, and the library must link from C."""
+    import subprocess
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    src = tmp_path / "client.c"
+    src.write_text(C_CLIENT)
+    exe = tmp_path / "client"
+    libdir = os.path.join(root, "spoc_amd")
+    subprocess.run(["gcc", "-std=c99", "-Wall", "-Wextra", "-Werror", "-pedantic", "-I", os.path.join(root, "include"),
+                    str(src), "-o", str(exe), "-L", libdir, "-lsarek_hip", f"-Wl,-rpath,{libdir}",
+                    "-Wl,-rpath,/opt/rocm/lib"], check=True)
+    out = subprocess.run([str(exe)], check=True, capture_output=True, text=True).stdout.strip()
+    import hashlib
+    assert out == hashlib.md5(b"Device11.0kernel code").hexdigest()
