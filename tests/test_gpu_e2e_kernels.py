@@ -196,3 +196,90 @@ def test_block_scan_with_two_shared_buffers(hip, torch_cuda):
     launch(hip, ir, n, [ints(torch, v), out, ("i32", n)], shared_mem=4096)
     exp = np.concatenate([np.cumsum(v[i:i + 256]) for i in range(0, n, 256)])
     assert np.array_equal(out.cpu().numpy(), exp)
+
+
+def test_bitonic_sort_many_launches_of_one_cached_kernel(hip, torch_cuda):
+    """test_sort.ml (bitonic step): data.(i) / data.(i lxor j) compare-exchange, launched
+    log^2(n) times with different scalars; boolean logic with `not`, `&&`, `||`."""
+    torch = torch_cuda
+    n = 1 << 12
+    v = np.random.default_rng(7).integers(-10000, 10000, n)
+    fresh()
+    params = [("data", "(vec i32)"), ("j", "i32"), ("k", "i32"), ("n", "i32")]
+    for p, t in params:
+        var(p, t)
+    i, ij, di, dij, asc = var("i"), var("ij"), var("di"), var("dij"), var("ascending", "bool")
+    j, k = var("j"), var("k")
+    cond = op("or", land(asc, op("gt", di, dij)), land(f"(not {asc})", lt(di, dij)))
+    ir = kernel(params, let(i, intr("global_thread_id", "Std"), if_(lt(i, var("n")), let(
+        ij, op("bitxor", i, j), if_(op("gt", ij, i), lets(
+            [(di, read("data", i)), (dij, read("data", ij)), (asc, op("eq", op("bitand", i, k), i32(0)))],
+            if_(cond, seq(assign_elem("data", i, dij), assign_elem("data", ij, di)))))))))
+    src = hip.generate_source(ir, block=(256, 1, 1))
+    d = ints(torch, v)
+    kk = 2
+    while kk <= n:
+        jj = kk // 2
+        while jj >= 1:
+            hip.run_source(src, "sarek_kern", (256, 1, 1), (n // 256, 1, 1),
+                           [d, ("i32", jj), ("i32", kk), ("i32", n)])
+            jj //= 2
+        kk *= 2
+    hip.check(hip.lib.sarek_hip_device_synchronize())
+    assert np.array_equal(d.cpu().numpy(), np.sort(v))
+
+
+def test_nbody_record_constructor_and_inner_loop(hip, torch_cuda):
+    """test_nbody_ppx.ml: a record built by a helper function, an inner for loop over all
+    bodies with mutable accumulators, sqrt and division."""
+    torch = torch_cuda
+    n = 300
+    rng = np.random.default_rng(8)
+    pos = rng.normal(size=(3, n)).astype(np.float32)
+    part = "(record particle (x f32) (y f32) (z f32))"
+    P, Q = f"(var p 20 {part})", f"(var q 21 {part})"
+
+    def mk(idx):
+        return f"(app (var make_p 0 {part}) (read xs {idx}) (read ys {idx}) (read zs {idx}))"
+    tid, jv = "(var tid 8 i32)", "(var j 9 i32 mut)"
+    fx, fy, fz = ("(var f%s %d f32 mut)" % (c, 10 + i) for i, c in enumerate("xyz"))
+    dx, dy, dz = ("(var d%s %d f32)" % (c, 13 + i) for i, c in enumerate("xyz"))
+    dist2, inv = "(var dist2 16 f32)", "(var inv 17 f32)"
+    ir = f"""
+    (kernel sarek_kern
+      (params (param (var xs 1 (vec f32))) (param (var ys 2 (vec f32))) (param (var zs 3 (vec f32)))
+              (param (var ax 4 (vec f32))) (param (var ay 5 (vec f32))) (param (var az 6 (vec f32)))
+              (param (var n 7 i32)))
+      (locals)
+      (body (let {tid} (add (intr (Gpu) thread_idx_x) (mul (intr (Gpu) block_idx_x) (intr (Gpu) block_dim_x)))
+        (if (lt {tid} (var n 7 i32))
+          (let {P} {mk(tid)}
+          (letmut {fx} (f32 0.0) (letmut {fy} (f32 0.0) (letmut {fz} (f32 0.0)
+           (seq
+            (for {jv} (i32 0) (sub (var n 7 i32) (i32 1)) upto
+              (if (ne {jv} {tid})
+                (let {Q} {mk(jv)}
+                (let {dx} (sub (field {Q} x) (field {P} x))
+                (let {dy} (sub (field {Q} y) (field {P} y))
+                (let {dz} (sub (field {Q} z) (field {P} z))
+                (let {dist2} (add (add (add (mul {dx} {dx}) (mul {dy} {dy})) (mul {dz} {dz})) (f32 1e-9))
+                (let {inv} (div (f32 1.0) (mul (intr (Float32) sqrt {dist2}) {dist2}))
+                  (seq (assign (lvar {fx}) (add {fx} (mul {dx} {inv})))
+                       (assign (lvar {fy}) (add {fy} (mul {dy} {inv})))
+                       (assign (lvar {fz}) (add {fz} (mul {dz} {inv}))))))))))))
+            (assign (lelem ax {tid}) {fx}) (assign (lelem ay {tid}) {fy}) (assign (lelem az {tid}) {fz})))))))))
+      (types (particle (x f32) (y f32) (z f32)))
+      (funcs (func make_p (params (var x 30 f32) (var y 31 f32) (var z 32 f32)) {part}
+               (return (record particle (x (var x 30 f32)) (y (var y 31 f32)) (z (var z 32 f32))))))
+      (native_fn false))"""
+    xs, ys, zs = (torch.from_numpy(pos[c].copy()).cuda() for c in range(3))
+    acc = [torch.zeros(n, device="cuda") for _ in range(3)]
+    launch(hip, ir, n, [xs, ys, zs, *acc, ("i32", n)])
+    p64 = pos.astype(np.float64)
+    d = p64[:, None, :] - p64[:, :, None]                 # d[c, i, j] = pos[c, j] - pos[c, i]
+    dist2 = (d ** 2).sum(0) + 1e-9
+    w = 1.0 / (np.sqrt(dist2) * dist2)
+    np.fill_diagonal(w, 0.0)
+    exp = (d * w[None]).sum(2)
+    for c in range(3):
+        assert np.allclose(acc[c].cpu().numpy(), exp[c], rtol=2e-3, atol=2e-3)
