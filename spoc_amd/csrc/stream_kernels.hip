@@ -193,40 +193,56 @@ __global__ __launch_bounds__(1024) void fold_kernel(const float *__restrict__ pa
   if (threadIdx.x == 0) *out = sh[0];
 }
 
-// One wave per 256-element block of the input: out[j] = sum(in[256j..256j+255]),
-// zero padded past n.  Dot sums x[i]*y[i].  Each lane folds its four elements, the
-// wave sum is f32; the summation order differs from the reference's halving tree,
+// Per-256-element-block kernels: out[j] = reduction of in[256j .. 256j+255].  A wave takes
+// kBlocksPerWave consecutive blocks (8 KiB of each input) in one shot, all loads issued
+// before the first use, non-temporal; the grid has one wave per such group, no loop.
+constexpr int kBlocksPerWave = 8;
+
+// Sum (or, Dot, sum of x[i]*y[i]), zero padded past n.  Each lane folds its four elements,
+// the wave sum is f32; the summation order differs from the reference's halving tree,
 // which its own checks allow for (1e-3 relative on the folded total).
 template <bool Dot>
 __global__ __launch_bounds__(kBlock) void block256_kernel(const float *__restrict__ x,
                                                           const float *__restrict__ y,
                                                           float *__restrict__ out, int64_t n,
                                                           int64_t nblocks) {
+  constexpr int U = kBlocksPerWave;
   const int lane = threadIdx.x & 63;
-  const int64_t wave = static_cast<int64_t>(blockIdx.x) * (kBlock / 64) + (threadIdx.x >> 6);
-  const int64_t wstep = static_cast<int64_t>(gridDim.x) * (kBlock / 64);
-  for (int64_t j = wave; j < nblocks; j += wstep) {
-    const int64_t i = j * 256 + lane * 4;
-    float v;
-    if (i + 3 < n) {
-      float4 xv = *reinterpret_cast<const float4 *>(x + i);
-      if (Dot) {
-        float4 yv = *reinterpret_cast<const float4 *>(y + i);
-        v = (xv.x * yv.x + xv.y * yv.y) + (xv.z * yv.z + xv.w * yv.w);
-      } else {
-        v = (xv.x + xv.y) + (xv.z + xv.w);
-      }
-    } else {
-      v = 0.f;
-      for (int e = 0; e < 4; ++e)
-        if (i + e < n) v += Dot ? x[i + e] * y[i + e] : x[i + e];
+  const int64_t j0 = (static_cast<int64_t>(blockIdx.x) * (kBlock / 64) + (threadIdx.x >> 6)) * U;
+  if (j0 >= nblocks) return;
+  float r[U];
+  if ((j0 + U) * 256 <= n) {
+    float4 xv[U], yv[U];
+#pragma unroll
+    for (int u = 0; u < U; ++u) xv[u] = ldg_nt(reinterpret_cast<const float4 *>(x + (j0 + u) * 256) + lane);
+    if (Dot) {
+#pragma unroll
+      for (int u = 0; u < U; ++u) yv[u] = ldg_nt(reinterpret_cast<const float4 *>(y + (j0 + u) * 256) + lane);
     }
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const float v = Dot ? (xv[u].x * yv[u].x + xv[u].y * yv[u].y) + (xv[u].z * yv[u].z + xv[u].w * yv[u].w)
+                          : (xv[u].x + xv[u].y) + (xv[u].z + xv[u].w);
+      r[u] = wave_sum(v);
+    }
+    if (lane == 0) {
+#pragma unroll
+      for (int u = 0; u < U; ++u) out[j0 + u] = r[u];
+    }
+    return;
+  }
+  // the group that holds the end of the input
+  for (int u = 0; u < U && j0 + u < nblocks; ++u) {
+    const int64_t i = (j0 + u) * 256 + lane * 4;
+    float v = 0.f;
+    for (int e = 0; e < 4; ++e)
+      if (i + e < n) v += Dot ? x[i + e] * y[i + e] : x[i + e];
     v = wave_sum(v);
-    if (lane == 0) out[j] = v;
+    if (lane == 0) out[j0 + u] = v;
   }
 }
 
-// One wave per 256-element block: out[j] = the value the reference's halving tree
+// out[j] = the value the reference's halving tree
 // (benchmarks/bench_reduction_max.ml:18-100: sdata[tid] = gid < n ? in[gid] : pad, then for
 // half = 128..1 "if sdata[tid+half] > sdata[tid] then sdata[tid] <- sdata[tid+half]")
 // leaves in sdata[0].  The same pairs are compared in the same order with the same
@@ -234,26 +250,38 @@ __global__ __launch_bounds__(kBlock) void block256_kernel(const float *__restric
 // signed zeros come out as from the tree.
 __device__ __forceinline__ float take_greater(float a, float b) { return b > a ? b : a; }
 
+__device__ __forceinline__ float tree_max_of_block(float v0, float v1, float v2, float v3) {
+  v0 = take_greater(v0, v2);   // half = 128: (l, l+128), (l+64, l+192)
+  v1 = take_greater(v1, v3);
+  float m = take_greater(v0, v1);  // half = 64
+#pragma unroll
+  for (int half = 32; half >= 1; half >>= 1) {
+    const float other = __shfl_down(m, half, 64);
+    m = take_greater(m, other);    // only lanes < half matter from here on
+  }
+  return m;                        // valid in lane 0
+}
+
 __global__ __launch_bounds__(kBlock) void block256_max_kernel(const float *__restrict__ x,
                                                               float *__restrict__ out, int64_t n,
                                                               int64_t nblocks, float pad) {
+  constexpr int U = kBlocksPerWave;
   const int lane = threadIdx.x & 63;
-  const int64_t wave = static_cast<int64_t>(blockIdx.x) * (kBlock / 64) + (threadIdx.x >> 6);
-  const int64_t wstep = static_cast<int64_t>(gridDim.x) * (kBlock / 64);
-  for (int64_t j = wave; j < nblocks; j += wstep) {
-    const int64_t i = j * 256 + lane;
-    float v[4];
+  const int64_t j0 = (static_cast<int64_t>(blockIdx.x) * (kBlock / 64) + (threadIdx.x >> 6)) * U;
+  if (j0 >= nblocks) return;
+  const bool full = (j0 + U) * 256 <= n;
+  float v[U][4];
 #pragma unroll
-    for (int q = 0; q < 4; ++q) v[q] = (i + 64 * q < n) ? x[i + 64 * q] : pad;
-    v[0] = take_greater(v[0], v[2]);   // half = 128: (l, l+128), (l+64, l+192)
-    v[1] = take_greater(v[1], v[3]);
-    float m = take_greater(v[0], v[1]);  // half = 64
+  for (int u = 0; u < U; ++u)
 #pragma unroll
-    for (int half = 32; half >= 1; half >>= 1) {
-      const float other = __shfl_down(m, half, 64);
-      m = take_greater(m, other);       // only lanes < half matter from here on
+    for (int q = 0; q < 4; ++q) {
+      const int64_t i = (j0 + u) * 256 + lane + 64 * q;
+      v[u][q] = (full || i < n) ? __builtin_nontemporal_load(x + (i < n ? i : 0)) : pad;
     }
-    if (lane == 0) out[j] = m;
+#pragma unroll
+  for (int u = 0; u < U; ++u) {
+    const float m = tree_max_of_block(v[u][0], v[u][1], v[u][2], v[u][3]);
+    if (lane == 0 && j0 + u < nblocks) out[j0 + u] = m;
   }
 }
 
@@ -372,9 +400,8 @@ static int launch_block256(const float *x, const float *y, float *out, int64_t n
   if (!aligned16(x) || (dot && !aligned16(y)))
     return fail(SAREK_HIP_E_INVALID_ARG, "block256: input vectors must be 16-byte aligned");
   const int64_t nblocks = ceil_div(n, 256);
-  int64_t wg = ceil_div(nblocks, kBlock / 64);
-  const int64_t cap = tunable("block256.max_blocks", 256 * 32);
-  if (wg > cap) wg = cap;
+  const int64_t wg = ceil_div(nblocks, (kBlock / 64) * kBlocksPerWave);
+  if (wg > 0x7FFFFFFF) return fail(SAREK_HIP_E_INVALID_ARG, "block256: input too long for one launch");
   if (dot)
     hipLaunchKernelGGL(block256_kernel<true>, dim3((unsigned)wg), dim3(kBlock), 0, st, x, y, out, n, nblocks);
   else
@@ -398,9 +425,8 @@ int sarek_hip_reduce_max_block256_f32(const float *in, float *out, int64_t n, fl
   if (n == 0) return SAREK_HIP_OK;
   if (!in || !out) return fail(SAREK_HIP_E_INVALID_ARG, "block256 max: NULL vector");
   const int64_t nblocks = ceil_div(n, 256);
-  int64_t wg = ceil_div(nblocks, kBlock / 64);
-  const int64_t cap = tunable("block256.max_blocks", 256 * 32);
-  if (wg > cap) wg = cap;
+  const int64_t wg = ceil_div(nblocks, (kBlock / 64) * kBlocksPerWave);
+  if (wg > 0x7FFFFFFF) return fail(SAREK_HIP_E_INVALID_ARG, "block256 max: input too long for one launch");
   hipLaunchKernelGGL(block256_max_kernel, dim3((unsigned)wg), dim3(kBlock), 0, as_stream(stream), in,
                      out, n, nblocks, pad);
   return check_launch("block256 max kernel launch");
