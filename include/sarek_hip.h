@@ -88,8 +88,23 @@ int sarek_hip_driver_version(int *version);
  * finaliser that may run late (sarek/core/Gpu_memory.ml:163-178).          */
 int sarek_hip_mem_alloc(void **dptr, size_t bytes);
 int sarek_hip_mem_free(void *dptr);
+/* Memory.host_ptr_to_device / device_to_host_ptr (sarek-cuda/Cuda_api.ml:207-230, called
+ * with a vector's whole host block by sarek/core/Transfer.ml:228-333).  Synchronous:
+ * the copy is complete on return, and it starts only after the device has finished
+ * the work it was given before.  Larger copies from or to ordinary (pageable)
+ * host memory (uploads from 12 MiB, downloads from 2 MiB) are pipelined through
+ * pinned staging slots by 4 host threads, three of them helpers that sleep
+ * between copies (64 MiB of pinned memory per device, kept until the process
+ * ends); tunables "transfer.threads" (0 = always the driver's own copy),
+ * "transfer.chunk_kib" (slot size), "transfer.min_up_kib", "transfer.min_down_kib". */
 int sarek_hip_memcpy_htod(void *dst_device, const void *src_host, size_t bytes);
 int sarek_hip_memcpy_dtoh(void *dst_host, const void *src_device, size_t bytes);
+/* Pinned host memory for a vector's host block (the reference allocates it as an
+ * ordinary Bigarray, sarek/core/Vector_storage.ml:22; wrapping a block from here with
+ * Ctypes.bigarray_of_ptr lets the two copies above run at the full PCIe rate with no
+ * staging).  `sarek_hip_host_free(NULL)` is accepted.                           */
+int sarek_hip_host_alloc(void **host_ptr, size_t bytes);
+int sarek_hip_host_free(void *host_ptr);
 int sarek_hip_memcpy_dtod(void *dst_device, const void *src_device, size_t bytes);
 int sarek_hip_memset_d8(void *dst_device, unsigned char value, size_t bytes);
 

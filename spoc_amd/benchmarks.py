@@ -58,7 +58,19 @@ def _device_record(times, throughput, verified, path, unit):
 
 
 def _upload(torch, array):
-    return torch.from_numpy(np.ascontiguousarray(array, dtype=np.float32)).cuda()
+    """Transfer.to_device (sarek/core/Transfer.ml:228-268): the vector's host block goes up
+    through Memory.host_ptr_to_device; torch only owns the device block."""
+    host = np.ascontiguousarray(array, dtype=np.float32)
+    dev = torch.empty(host.size, dtype=torch.float32, device="cuda")
+    hip.memcpy_htod(dev.data_ptr(), host)
+    return dev
+
+
+def _download(tensor):
+    """Transfer.to_cpu (sarek/core/Transfer.ml:274-333) through Memory.device_to_host_ptr."""
+    host = np.empty(tensor.numel(), dtype=np.float32)
+    hip.memcpy_dtoh(host, tensor.data_ptr())
+    return host
 
 
 def bench_matrix_mul_tiled(size, warmup=5, iterations=20, tile_size=16):
@@ -86,7 +98,7 @@ def bench_matrix_mul_tiled(size, warmup=5, iterations=20, tile_size=16):
         return hip.run_source(src, "sarek_kern", (tile_size, tile_size, 1), grid, args,
                               shared_mem=2 * tile_size * tile_size * 4)
     times, path = _time_launches(launch, warmup, iterations)
-    verified = bool(np.all(np.abs(vc.cpu().numpy().astype(np.float64).reshape(m, n) - expected) <= 1e-3))
+    verified = bool(np.all(np.abs(_download(vc).astype(np.float64).reshape(m, n) - expected) <= 1e-3))
     gflops = 2.0 * m * n * k / (statistics.median(times) * 1e6)
     return _device_record(times, gflops, verified, path, "GFLOPS")
 
@@ -106,7 +118,7 @@ def bench_stream_triad(size, warmup=5, iterations=20, block_size=256):
     args = [va, vb, vc, ("f32", 3.0), ("i32", n)]
     times, path = _time_launches(lambda: hip.run_source(src, "sarek_kern", (block_size, 1, 1), grid, args),
                                  warmup, iterations)
-    verified = bool(np.all(np.abs(va.cpu().numpy().astype(np.float64) - expected) <= 1e-5))
+    verified = bool(np.all(np.abs(_download(va).astype(np.float64) - expected) <= 1e-5))
     gbs = 3.0 * n * 4.0 / (statistics.median(times) / 1e3 * 1e9)
     return _device_record(times, gbs, verified, path, "GB/s")
 
@@ -121,7 +133,7 @@ def _tree_bench(ir, inputs, n, expected, check, bytes_moved, stat, warmup, itera
     times, path = _time_launches(
         lambda: hip.run_source(src, "sarek_kern", (256, 1, 1), (nblocks, 1, 1), args, shared_mem=1024),
         warmup, iterations)
-    result = float(fold(vout.cpu().numpy().astype(np.float64)))   # host fold over the partials
+    result = float(fold(_download(vout).astype(np.float64)))   # host fold over the partials
     verified = check(result, expected)
     t = statistics.mean(times) if stat == "mean" else statistics.median(times)
     return _device_record(times, bytes_moved / (t / 1e3) / 1e9, verified, path, "GB/s")
@@ -154,6 +166,45 @@ def bench_reduction_max(size, warmup=5, iterations=20):
                        lambda r, e: abs(r - e) < 1e-5, 4.0 * n, "median", warmup, iterations, fold=np.max)
 
 
+def bench_transfer(size, warmup=2, iterations=7):
+    """Not one of the reference's programs: the Transfer.to_device / Transfer.to_cpu legs
+    (sarek/core/Transfer.ml:228-333) that its benches run once before and after their timed
+    loops, timed alone for a float32 vector of `size` elements in ordinary (pageable) host
+    memory.  Throughput is the upload rate; the record also carries the download rate and
+    both rates of the driver's own copy."""
+    import torch
+    host = (np.arange(size) % 100 / 100.0).astype(np.float32)
+    back = np.empty_like(host)
+    dev = torch.empty(size, dtype=torch.float32, device="cuda")
+    sync = hip.lib.sarek_hip_device_synchronize
+
+    def timed(fn):
+        for _ in range(warmup):
+            fn()
+        ts = []
+        for _ in range(iterations):
+            t0 = time.perf_counter()
+            fn()
+            hip.check(sync())
+            ts.append((time.perf_counter() - t0) * 1e3)
+        return ts
+    rates = {}
+    for label, threads in (("driver", 0), ("staged", None)):
+        if threads is not None:
+            hip.set_tunable("transfer.threads", threads)
+        up = timed(lambda: hip.memcpy_htod(dev.data_ptr(), host))
+        down = timed(lambda: hip.memcpy_dtoh(back, dev.data_ptr()))
+        hip.set_tunable("transfer.threads", 4)
+        rates[label] = (up, down)
+    gbs = lambda ts: host.nbytes / (statistics.median(ts) / 1e3) / 1e9
+    rec = _device_record(rates["staged"][0], gbs(rates["staged"][0]), np.array_equal(back, host),
+                         "memcpy_htod", "GB/s")
+    rec["download_gbs"] = gbs(rates["staged"][1])
+    rec["driver_copy_upload_gbs"] = gbs(rates["driver"][0])
+    rec["driver_copy_download_gbs"] = gbs(rates["driver"][1])
+    return rec
+
+
 BENCHMARKS = {
     # name: (function, the reference's default sizes)
     "matrix_mul_tiled": (bench_matrix_mul_tiled, [128, 256, 512, 1024, 2048, 4096]),
@@ -161,6 +212,7 @@ BENCHMARKS = {
     "reduction": (bench_reduction, [1_000_000, 10_000_000, 50_000_000, 100_000_000]),   # warmup 10 there
     "dot_product": (bench_dot_product, [1_000_000, 10_000_000, 50_000_000, 100_000_000]),
     "reduction_max": (bench_reduction_max, [1_000_000, 10_000_000, 50_000_000, 100_000_000]),
+    "transfer": (bench_transfer, [1_000_000, 10_000_000, 100_000_000, 268_435_456]),   # no such program there
 }
 
 
@@ -174,6 +226,9 @@ def run(name, sizes=None, warmup=None, iterations=20):
         print(f"  Mean: {rec['mean_ms']:.3f} ms, Median: {rec['median_ms']:.3f} ms, "
               f"StdDev: {rec['stddev_ms']:.3f} ms")
         print(f"  Throughput: {rec['throughput_gflops']:.3f} {rec['throughput_unit']}  [{rec['path']}]")
+        if "download_gbs" in rec:
+            print(f"  Download: {rec['download_gbs']:.3f} GB/s; driver's own copy: "
+                  f"{rec['driver_copy_upload_gbs']:.3f} up, {rec['driver_copy_download_gbs']:.3f} down")
         print(f"  Verified: {'✓' if rec['verified'] else '✗'}", flush=True)
         out.append({"benchmark": {"name": name, "parameters": {"size": size, "iterations": iterations,
                                                                "warmup": warmup}},

@@ -245,20 +245,6 @@ int sarek_hip_mem_free(void *dptr) {
   return SAREK_HIP_OK;
 }
 
-int sarek_hip_memcpy_htod(void *dst_device, const void *src_host, size_t bytes) {
-  if (bytes == 0) return SAREK_HIP_OK;
-  if (!dst_device || !src_host) return fail(SAREK_HIP_E_INVALID_ARG, "memcpy_htod: NULL pointer");
-  SAREK_HIP_TRY(hipMemcpy(dst_device, src_host, bytes, hipMemcpyHostToDevice));
-  return SAREK_HIP_OK;
-}
-
-int sarek_hip_memcpy_dtoh(void *dst_host, const void *src_device, size_t bytes) {
-  if (bytes == 0) return SAREK_HIP_OK;
-  if (!dst_host || !src_device) return fail(SAREK_HIP_E_INVALID_ARG, "memcpy_dtoh: NULL pointer");
-  SAREK_HIP_TRY(hipMemcpy(dst_host, src_device, bytes, hipMemcpyDeviceToHost));
-  return SAREK_HIP_OK;
-}
-
 int sarek_hip_memcpy_dtod(void *dst_device, const void *src_device, size_t bytes) {
   if (bytes == 0) return SAREK_HIP_OK;
   if (!dst_device || !src_device) return fail(SAREK_HIP_E_INVALID_ARG, "memcpy_dtod: NULL pointer");

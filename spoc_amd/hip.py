@@ -77,6 +77,8 @@ SYMBOLS = {
     "sarek_hip_memcpy_htod": (_i, [_vp, _vp, _sz]),
     "sarek_hip_memcpy_dtoh": (_i, [_vp, _vp, _sz]),
     "sarek_hip_memcpy_dtod": (_i, [_vp, _vp, _sz]),
+    "sarek_hip_host_alloc": (_i, [C.POINTER(_vp), _sz]),
+    "sarek_hip_host_free": (_i, [_vp]),
     "sarek_hip_memset_d8": (_i, [_vp, C.c_ubyte, _sz]),
     "sarek_hip_stream_create": (_i, [C.POINTER(_vp)]),
     "sarek_hip_stream_destroy": (_i, [_vp]),
@@ -242,6 +244,53 @@ def _need(t, dtype, name):
     torch = _torch()
     if not (isinstance(t, torch.Tensor) and t.is_cuda and t.dtype == dtype and t.is_contiguous()):
         raise TypeError(f"{name}: expected a contiguous device tensor of {dtype}")
+
+
+def mem_alloc(nbytes):
+    """Memory.alloc: device block, as an integer address."""
+    p = _vp()
+    check(lib.sarek_hip_mem_alloc(C.byref(p), nbytes))
+    return p.value
+
+
+def mem_free(dptr):
+    check(lib.sarek_hip_mem_free(_vp(dptr)))
+
+
+def memcpy_htod(dptr, host):
+    """Memory.host_ptr_to_device from a contiguous numpy array."""
+    check(lib.sarek_hip_memcpy_htod(_vp(dptr), _vp(host.ctypes.data), host.nbytes))
+
+
+def memcpy_dtoh(host, dptr):
+    """Memory.device_to_host_ptr into a contiguous numpy array."""
+    check(lib.sarek_hip_memcpy_dtoh(_vp(host.ctypes.data), _vp(dptr), host.nbytes))
+
+
+class pinned_array:
+    """numpy array over a block from sarek_hip_host_alloc; freed by close() or on exit of
+    a with-block (the array must not be used afterwards)."""
+
+    def __init__(self, count, dtype):
+        import numpy as np
+        dtype = np.dtype(dtype)
+        self._ptr = _vp()
+        nbytes = int(count) * dtype.itemsize
+        check(lib.sarek_hip_host_alloc(C.byref(self._ptr), nbytes))
+        buf = (C.c_char * nbytes).from_address(self._ptr.value)
+        self.array = np.frombuffer(buf, dtype=dtype, count=int(count))
+
+    def close(self):
+        if self._ptr is not None:
+            self.array = None
+            check(lib.sarek_hip_host_free(self._ptr))
+            self._ptr = None
+
+    def __enter__(self):
+        return self.array
+
+    def __exit__(self, *exc):
+        self.close()
 
 
 def device_info(device=0):
