@@ -282,6 +282,63 @@ int sarek_hip_cache_put(const char *key, const void *data, size_t len);
 int sarek_hip_cache_get_stats(int64_t out[4]);
 int sarek_hip_cache_reset_stats(void);
 
+/* ---------------------------------------------------------------------- */
+/* IR fusion: sarek/sarek/Sarek_fusion.ml over IR text (same grammar as
+ * sarek_hip_generate_source reads; results are written in it too), for hosts
+ * that hold kernels as text and have no OCaml.  Results follow the reference
+ * kernel for kernel, its limits included (see sarek_hip_fusion_fuse).  Text
+ * outputs use the generate_source buffer convention (at most out_len bytes
+ * incl. NUL, *needed = full size, SAREK_HIP_E_BUFFER_TOO_SMALL when short).  */
+enum {                                   /* `mode` below                              */
+  SAREK_HIP_FUSION_VERTICAL = 0,         /* can_fuse / fuse                 :401-547   */
+  SAREK_HIP_FUSION_REDUCTION = 1,        /* can_fuse_reduction / fuse_reduction :641-757 */
+  SAREK_HIP_FUSION_STENCIL = 2,          /* can_fuse_stencil / fuse_stencil :795-1019  */
+  SAREK_HIP_FUSION_TRY = 3,              /* try_fuse                        :760-766   */
+  SAREK_HIP_FUSION_TRY_ALL = 4           /* try_fuse_all                    :1022-1030 */
+};
+enum { SAREK_HIP_FUSION_FUSE = 0, SAREK_HIP_FUSION_DONT_FUSE = 1, SAREK_HIP_FUSION_MAYBE_FUSE = 2 };
+
+/* analyze (:340-354).  out: (info (reads (ARRAY pattern)*) (writes (ARRAY pattern)*)
+ * (barriers true|false) (atomics false)), arrays sorted by name,
+ * pattern ::= (one_to_one expr) | (stencil OFFSET*) | (reduction OP) | gather | unknown */
+int sarek_hip_fusion_analyze(const char *kernel_ir, char *out, size_t out_len, size_t *needed);
+/* *result = 1 when the producer can be fused into the consumer through array
+ * `intermediate` under `mode` (TRY modes: when the corresponding try_* returns Some). */
+int sarek_hip_fusion_can_fuse(const char *producer_ir, const char *consumer_ir, const char *intermediate,
+                              int mode, int *result);
+/* The fused kernel as IR text: "<consumer>_fused" ("<consumer>_stencil_fused" for the
+ * stencil rewrite), consumer parameters without the intermediate followed by the
+ * producer's new ones, native_fn false.  As in the reference, the fixed modes return
+ * the consumer unchanged when the producer's store cannot be inlined (conditional store,
+ * no read of the intermediate); the TRY modes set *fused = 0 and write "" when no rewrite
+ * applies.  The reduction rewrite inserts the producer's expression as it stands.      */
+int sarek_hip_fusion_fuse(const char *producer_ir, const char *consumer_ir, const char *intermediate, int mode,
+                          int *fused, char *out, size_t out_len, size_t *needed);
+/* should_fuse (:1068-1098): decision + the reference's reason text.                 */
+int sarek_hip_fusion_should_fuse(const char *producer_ir, const char *consumer_ir, const char *intermediate,
+                                 int *decision, char *reason, size_t reason_len);
+/* fuse_pipeline (automatic = 0, :570-598) / auto_fuse_pipeline (1, :1133-1165).
+ * out: the resulting kernel; report: one line per entry, "eliminated ARRAY" then
+ * "skipped REASON", each list in the reference's order (latest first).  An empty
+ * list is SAREK_HIP_E_INVALID_ARG with Fusion_error's text.                         */
+int sarek_hip_fusion_pipeline(const char *const *kernel_irs, int n_kernels, int automatic, char *out,
+                              size_t out_len, size_t *needed, char *report, size_t report_len,
+                              size_t *report_needed);
+/* analyze_pipeline (:1180-1214): the text it prints.                                */
+int sarek_hip_fusion_analyze_pipeline(const char *const *kernel_irs, int n_kernels, char *out, size_t out_len,
+                                      size_t *needed);
+/* analyze_stencil_fusion (:829-871): radii = {combined, producer, consumer};
+ * inputs = the producer's input arrays, space separated.                            */
+int sarek_hip_fusion_stencil_info(const char *producer_ir, const char *consumer_ir, const char *intermediate,
+                                  int *found, int radii[3], char *inputs, size_t inputs_len, size_t *needed);
+/* The expression-level pieces (:35-48, :77-124, :611-634).
+ * detect_reduction out: (reduction ACC ACC_ID OP ARRAY LOOPVAR LOOPVAR_ID).          */
+int sarek_hip_fusion_expr_equal(const char *expr_a, const char *expr_b, int *equal);
+int sarek_hip_fusion_subst_array_read(const char *array, const char *index_expr, const char *replacement_expr,
+                                      const char *expr, char *out, size_t out_len, size_t *needed);
+int sarek_hip_fusion_detect_reduction(const char *stmt_ir, int *found, char *out, size_t out_len, size_t *needed);
+int sarek_hip_fusion_is_reduction_kernel(const char *kernel_ir, const char *array, int *found, char op[8]);
+
 /* Integer tuning knob (launch shapes, tile variants), for sweeps without a
  * rebuild.  Unknown names are stored and ignored.                           */
 int sarek_hip_set_tunable(const char *name, int64_t value);

@@ -137,6 +137,8 @@ Kernel parse_kernel(const std::string &text);
 StmtP parse_stmt(const std::string &text);
 ExprP parse_expr(const std::string &text);
 std::string print_kernel(const Kernel &k);
+std::string print_expr(const ExprP &e);
+std::string print_stmt(const StmtP &s);
 
 // ir_hip.cpp: IR -> HIP C++ for gfx950
 std::string gen_expr(const ExprP &e);

@@ -534,9 +534,8 @@ Kernel to_kernel(const SExp &e) {
     const std::string &h = head(sec);
     if (h == "params") {
       for (size_t j = 1; j < sec.items.size(); ++j) {
-        Decl d = to_decl(sec.items[j]);
-        if (d.kind != Decl::Param) perr(sec.items[j], "only (param ...) is allowed in (params ...)");
-        k.params.push_back(d);
+        // any declaration, as kern_params : decl list; the lowering rejects what is not a parameter
+        k.params.push_back(to_decl(sec.items[j]));
       }
     } else if (h == "locals") {
       for (size_t j = 1; j < sec.items.size(); ++j) {
@@ -791,6 +790,8 @@ std::string pr_decl(const Decl &d) {
 Kernel parse_kernel(const std::string &text) { return to_kernel(Reader(text).read_all()); }
 StmtP parse_stmt(const std::string &text) { return to_stmt(Reader(text).read_all()); }
 ExprP parse_expr(const std::string &text) { return to_expr(Reader(text).read_all()); }
+std::string print_expr(const ExprP &e) { return pr_expr(e); }
+std::string print_stmt(const StmtP &s) { return pr_stmt(s, ""); }
 
 std::string print_kernel(const Kernel &k) {
   std::string o = "(kernel " + k.name + "\n  (params";

@@ -116,6 +116,21 @@ SYMBOLS = {
     "sarek_hip_cache_put": (_i, [C.c_char_p, _vp, _sz]),
     "sarek_hip_cache_get_stats": (_i, [C.POINTER(_i64)]),
     "sarek_hip_cache_reset_stats": (_i, []),
+    "sarek_hip_fusion_analyze": (_i, [C.c_char_p, C.c_char_p, _sz, C.POINTER(_sz)]),
+    "sarek_hip_fusion_can_fuse": (_i, [C.c_char_p, C.c_char_p, C.c_char_p, _i, C.POINTER(_i)]),
+    "sarek_hip_fusion_fuse": (_i, [C.c_char_p, C.c_char_p, C.c_char_p, _i, C.POINTER(_i), C.c_char_p, _sz,
+                                   C.POINTER(_sz)]),
+    "sarek_hip_fusion_should_fuse": (_i, [C.c_char_p, C.c_char_p, C.c_char_p, C.POINTER(_i), C.c_char_p, _sz]),
+    "sarek_hip_fusion_pipeline": (_i, [C.POINTER(C.c_char_p), _i, _i, C.c_char_p, _sz, C.POINTER(_sz),
+                                       C.c_char_p, _sz, C.POINTER(_sz)]),
+    "sarek_hip_fusion_analyze_pipeline": (_i, [C.POINTER(C.c_char_p), _i, C.c_char_p, _sz, C.POINTER(_sz)]),
+    "sarek_hip_fusion_stencil_info": (_i, [C.c_char_p, C.c_char_p, C.c_char_p, C.POINTER(_i), C.POINTER(_i),
+                                           C.c_char_p, _sz, C.POINTER(_sz)]),
+    "sarek_hip_fusion_expr_equal": (_i, [C.c_char_p, C.c_char_p, C.POINTER(_i)]),
+    "sarek_hip_fusion_subst_array_read": (_i, [C.c_char_p, C.c_char_p, C.c_char_p, C.c_char_p, C.c_char_p, _sz,
+                                               C.POINTER(_sz)]),
+    "sarek_hip_fusion_detect_reduction": (_i, [C.c_char_p, C.POINTER(_i), C.c_char_p, _sz, C.POINTER(_sz)]),
+    "sarek_hip_fusion_is_reduction_kernel": (_i, [C.c_char_p, C.c_char_p, C.POINTER(_i), C.c_char_p]),
     "sarek_hip_set_tunable": (_i, [C.c_char_p, _i64]),
     "sarek_hip_set_clock_probe": (_i, [_vp, _i64, C.POINTER(_i64)]),
 }
