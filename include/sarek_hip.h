@@ -240,6 +240,14 @@ int sarek_hip_reduce_max_block256_f32(const float *in, float *out, int64_t n, fl
 int sarek_hip_fold_partials_f64(const float *partials, int64_t count, double *sum_out,
                                 sarek_hip_stream stream);
 
+/* dst[i] = src[i], i < n: the kernel of benchmarks/bench_vector_copy.ml:21-27
+ * (`if tid < n then b.(tid) <- a.(tid)`); elements past n are not touched.          */
+int sarek_hip_copy_f32(float *dst, const float *src, int64_t n, sarek_hip_stream stream);
+/* out[c * height + r] = in[r * width + c] for r < height, c < width: the kernels of
+ * benchmarks/bench_transpose.ml and bench_transpose_tiled.ml (`in` has `height` rows
+ * of `width` floats).  in and out must not overlap.                                 */
+int sarek_hip_transpose_f32(const float *in, float *out, int width, int height, sarek_hip_stream stream);
+
 /* Row-major GEMM  C[m x n] = A[m x k] . B[k x n]  (replaces the generated
  * 16x16 tiled kernel, matrix_mul_tiled_generated.md:9-50; source
  * benchmarks/bench_matrix_mul_tiled.ml:55-95).  Any m,n,k >= 1.            */

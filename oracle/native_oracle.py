@@ -16,6 +16,7 @@ __all__ = [
     "build", "fill_uniform", "round_bf16", "round_f16", "bf16_bits", "f16_bits",
     "triad", "reduce_sum_block256", "reduce_max_block256", "dot_block256", "fold_partials", "triad_sum",
     "gemm", "gemm_rows", "gemm_bias_relu_rowsum", "matmul_tiled_bsp",
+    "vector_add", "vector_copy", "transpose", "matmul_naive",
 ]
 
 
@@ -56,6 +57,10 @@ def _L():
         lib.oracle_gemm_bias_relu_rowsum.argtypes = [f32p, f32p, f32p, f32p, f32p, i32p,
                                                      i64, i64, i64, i32]
         lib.oracle_matmul_tiled_bsp.argtypes = [f32p, f32p, f32p, i32, i32, i32]
+        lib.oracle_vector_add_f32.argtypes = [f32p, f32p, f32p, i64, i64]
+        lib.oracle_vector_copy_f32.argtypes = [f32p, f32p, i64, i64]
+        lib.oracle_transpose_f32.argtypes = [f32p, f32p, i32, i32, i64]
+        lib.oracle_matmul_naive_f32.argtypes = [f32p, f32p, f32p, i32, i32, i32, i64]
         _lib = lib
     return _lib
 
@@ -200,3 +205,44 @@ def matmul_tiled_bsp(a, b):
     c = np.zeros((m, n), dtype=np.float32)
     _L().oracle_matmul_tiled_bsp(ap, bp, c.ctypes.data_as(C.POINTER(C.c_float)), m, n, k)
     return c
+
+
+def _launch_size(n, threads):
+    return int(threads) if threads is not None else int(n)
+
+
+def vector_add(a, b, out, n, threads=None):
+    """In place on `out` (float32 array): what the vector-add kernel leaves there."""
+    a, ap = _f32(a)
+    b, bp = _f32(b)
+    assert out.dtype == np.float32 and out.flags.c_contiguous
+    _L().oracle_vector_add_f32(ap, bp, out.ctypes.data_as(C.POINTER(C.c_float)), n, _launch_size(n, threads))
+    return out
+
+
+def vector_copy(a, out, n, threads=None):
+    a, ap = _f32(a)
+    assert out.dtype == np.float32 and out.flags.c_contiguous
+    _L().oracle_vector_copy_f32(ap, out.ctypes.data_as(C.POINTER(C.c_float)), n, _launch_size(n, threads))
+    return out
+
+
+def transpose(x, width, height, out=None, threads=None):
+    x, xp = _f32(x)
+    if out is None:
+        out = np.zeros(width * height, dtype=np.float32)
+    assert out.dtype == np.float32 and out.flags.c_contiguous
+    _L().oracle_transpose_f32(xp, out.ctypes.data_as(C.POINTER(C.c_float)), width, height,
+                              _launch_size(width * height, threads))
+    return out
+
+
+def matmul_naive(a, b, m, n, k, out=None, threads=None):
+    a, ap = _f32(a)
+    b, bp = _f32(b)
+    if out is None:
+        out = np.zeros(m * n, dtype=np.float32)
+    assert out.dtype == np.float32 and out.flags.c_contiguous
+    _L().oracle_matmul_naive_f32(ap, bp, out.ctypes.data_as(C.POINTER(C.c_float)), m, n, k,
+                                 _launch_size(m * n, threads))
+    return out

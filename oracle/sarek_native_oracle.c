@@ -422,4 +422,48 @@ void oracle_matmul_tiled_bsp(const float *a, const float *b, float *c, int m, in
     }
 }
 
+/* ------------------------------------------------------------------ */
+/* The reference's other memory-bound kernels, thread by thread as its 1-D
+ * launches run them (one logical thread per global id, `if tid < n`):
+ * vector add (benchmarks/bench_vector_add.ml:53-61; the sum of two binary32
+ * values is formed in double and rounded once at the store, which is the
+ * binary32 sum), vector copy (bench_vector_copy.ml:21-27), the transpose
+ * (bench_transpose.ml: col = tid mod width, row = tid / width,
+ * output[col*height + row] = input[row*width + col]; bench_transpose_tiled.ml
+ * computes the same matrix through a 16x17 shared tile) and the
+ * one-thread-per-element matmul (bench_matrix_mul.ml:55-73: row = tid / n,
+ * col = tid mod n, sum in double in increasing i, one rounding at the store).
+ * `threads` is the launch size (grid * block): ids at or past the guard do
+ * nothing, so elements they would own keep their old value.             */
+void oracle_vector_add_f32(const float *a, const float *b, float *c, int64_t n, int64_t threads) {
+  for (int64_t tid = 0; tid < threads; ++tid)
+    if (tid < n) c[tid] = (float)((double)a[tid] + (double)b[tid]);
+}
+
+void oracle_vector_copy_f32(const float *a, float *b, int64_t n, int64_t threads) {
+  for (int64_t tid = 0; tid < threads; ++tid)
+    if (tid < n) b[tid] = a[tid];
+}
+
+void oracle_transpose_f32(const float *input, float *output, int32_t width, int32_t height, int64_t threads) {
+  const int32_t n = width * height;
+  for (int64_t tid = 0; tid < threads; ++tid)
+    if (tid < n) {
+      const int32_t col = (int32_t)tid % width, row = (int32_t)tid / width;
+      output[col * height + row] = input[row * width + col];
+    }
+}
+
+void oracle_matmul_naive_f32(const float *a, const float *b, float *c, int32_t m, int32_t n, int32_t k,
+                             int64_t threads) {
+  for (int64_t tid = 0; tid < threads; ++tid) {
+    const int32_t row = (int32_t)tid / n, col = (int32_t)tid % n;
+    if (row < m && col < n) {
+      double sum = 0.0;
+      for (int32_t i = 0; i <= k - 1; ++i) sum = sum + (double)a[row * k + i] * (double)b[i * n + col];
+      c[row * n + col] = (float)sum;
+    }
+  }
+}
+
 int oracle_abi_version(void) { return 1; }

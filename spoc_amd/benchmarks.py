@@ -1,7 +1,8 @@
 """The reference's benchmark programs for the hot path, run through the sarek-hip plugin.
 
 Host-side mirror of benchmarks/bench_matrix_mul_tiled.ml, bench_stream_triad.ml,
-bench_reduction.ml, bench_dot_product.ml and bench_reduction_max.ml: same inputs, same
+bench_reduction.ml, bench_dot_product.ml, bench_reduction_max.ml, bench_vector_add.ml,
+bench_vector_copy.ml, bench_matrix_mul.ml, bench_transpose.ml and bench_transpose_tiled.ml: same inputs, same
 launch geometry, same warmup / timed-iteration protocol (wall clock around the launch plus
 the device flush, one sample per iteration), same verification and tolerance, same
 throughput formula and statistic, and the same per-device result record
@@ -166,6 +167,108 @@ def bench_reduction_max(size, warmup=5, iterations=20):
                        lambda r, e: abs(r - e) < 1e-5, 4.0 * n, "median", warmup, iterations, fold=np.max)
 
 
+def _benchmark_gpu(launch, warmup, iterations):
+    """benchmarks/common.ml:200-237 (Common.benchmark_gpu): one launch to compile, `warmup`
+    launches, then `iterations` samples of device-idle -> launch -> device-idle."""
+    sync = hip.lib.sarek_hip_device_synchronize
+    path = launch()
+    hip.check(sync())
+    for _ in range(warmup):
+        launch()
+        hip.check(sync())
+    times = []
+    for _ in range(iterations):
+        hip.check(sync())
+        t0 = time.perf_counter()
+        path = launch()
+        hip.check(sync())
+        times.append((time.perf_counter() - t0) * 1e3)
+    return times, path
+
+
+def bench_vector_add(size, warmup=10, iterations=20):
+    """benchmarks/bench_vector_add.ml:53-150: a[i] = 0.001 i, b[i] = 0.002 i, every element within
+    1e-3 of the double sum, GB/s = 12 n / MINIMUM time."""
+    import torch
+    n = size
+    a, b = np.arange(n) * 0.001, np.arange(n) * 0.002
+    va, vb = _upload(torch, a), _upload(torch, b)
+    vc = torch.empty(n, dtype=torch.float32, device="cuda")
+    src = hip.generate_source(reference_kernels.vector_add(), block=(256, 1, 1))
+    grid = ((n + 255) // 256, 1, 1)
+    args = [va, vb, vc, ("i32", n)]
+    times, path = _benchmark_gpu(lambda: hip.run_source(src, "sarek_kern", (256, 1, 1), grid, args),
+                                 warmup, iterations)
+    verified = bool(np.all(np.abs(_download(vc).astype(np.float64) - (a + b)) <= 1e-3))
+    return _device_record(times, 12.0 * n / (min(times) / 1e3) / 1e9, verified, path, "GB/s")
+
+
+def bench_vector_copy(size, warmup=5, iterations=20, block_size=256):
+    """benchmarks/bench_vector_copy.ml:21-170: a[i] = (i mod 100)/100, every element within 1e-6,
+    GB/s = 8 n / median (launch + flush per sample)."""
+    import torch
+    n = size
+    a = (np.arange(n) % 100) / 100.0
+    va = _upload(torch, a)
+    vb = torch.empty(n, dtype=torch.float32, device="cuda")
+    src = hip.generate_source(reference_kernels.vector_copy(), block=(block_size, 1, 1))
+    grid = ((n + block_size - 1) // block_size, 1, 1)
+    args = [va, vb, ("i32", n)]
+    times, path = _time_launches(lambda: hip.run_source(src, "sarek_kern", (block_size, 1, 1), grid, args),
+                                 warmup, iterations)
+    verified = bool(np.all(np.abs(_download(vb).astype(np.float64) - a) <= 1e-6))
+    return _device_record(times, 8.0 * n / (statistics.median(times) / 1e3) / 1e9, verified, path, "GB/s")
+
+
+def bench_matrix_mul(size, warmup=10, iterations=20, block_size=256):
+    """benchmarks/bench_matrix_mul.ml:43-165: one thread per element of C, inputs as the tiled
+    bench, every element within 1e-3 of the double product, GFLOPS = 2 m n k / MEAN."""
+    import torch
+    m = n = k = size
+    a = (np.arange(m * k) % 10) / 10.0
+    b = ((np.arange(k * n) + 1) % 10) / 10.0
+    expected = a.reshape(m, k) @ b.reshape(k, n)
+    va, vb = _upload(torch, a), _upload(torch, b)
+    vc = torch.empty(m * n, dtype=torch.float32, device="cuda")
+    src = hip.generate_source(reference_kernels.matrix_mul(), block=(block_size, 1, 1))
+    grid = ((m * n + block_size - 1) // block_size, 1, 1)
+    args = [va, vb, vc, ("i32", m), ("i32", n), ("i32", k)]
+    times, path = _benchmark_gpu(lambda: hip.run_source(src, "sarek_kern", (block_size, 1, 1), grid, args),
+                                 warmup, iterations)
+    verified = bool(np.all(np.abs(_download(vc).astype(np.float64).reshape(m, n) - expected) <= 1e-3))
+    return _device_record(times, 2.0 * m * n * k / (statistics.mean(times) * 1e6), verified, path, "GFLOPS")
+
+
+def _bench_transpose(ir, block, grid_of, size, warmup, iterations):
+    """benchmarks/bench_transpose.ml:100-210 / bench_transpose_tiled.ml:120-240: input[i] = i, square
+    size x size, tolerance 1e-3 (10 beyond 2^24 elements), GB/s = 8 n / MEAN."""
+    import torch
+    m = size
+    n = m * m
+    data = np.arange(n, dtype=np.float64)
+    vin = _upload(torch, data)
+    vout = torch.zeros(n, dtype=torch.float32, device="cuda")
+    src = hip.generate_source(ir, block=block)
+    args = [vin, vout, ("i32", m), ("i32", m)]
+    times, path = _benchmark_gpu(lambda: hip.run_source(src, "sarek_kern", block, grid_of(m), args),
+                                 warmup, iterations)
+    tolerance = 10.0 if n > 16_777_216 else 0.001
+    expected = data.reshape(m, m).T.reshape(-1)
+    verified = bool(np.all(np.abs(_download(vout).astype(np.float64) - expected) <= tolerance))
+    return _device_record(times, 8.0 * n / (statistics.mean(times) / 1e3) / 1e9, verified, path, "GB/s")
+
+
+def bench_transpose(size, warmup=10, iterations=20):
+    return _bench_transpose(reference_kernels.transpose_naive(), (256, 1, 1),
+                            lambda m: ((m * m + 255) // 256, 1, 1), size, warmup, iterations)
+
+
+def bench_transpose_tiled(size, warmup=10, iterations=20, tile_size=16):
+    return _bench_transpose(reference_kernels.transpose_tiled(), (tile_size, tile_size, 1),
+                            lambda m: ((m + tile_size - 1) // tile_size, (m + tile_size - 1) // tile_size, 1),
+                            size, warmup, iterations)
+
+
 def bench_transfer(size, warmup=2, iterations=7):
     """Not one of the reference's programs: the Transfer.to_device / Transfer.to_cpu legs
     (sarek/core/Transfer.ml:228-333) that its benches run once before and after their timed
@@ -212,6 +315,11 @@ BENCHMARKS = {
     "reduction": (bench_reduction, [1_000_000, 10_000_000, 50_000_000, 100_000_000]),   # warmup 10 there
     "dot_product": (bench_dot_product, [1_000_000, 10_000_000, 50_000_000, 100_000_000]),
     "reduction_max": (bench_reduction_max, [1_000_000, 10_000_000, 50_000_000, 100_000_000]),
+    "vector_add": (bench_vector_add, [1_000_000, 10_000_000, 50_000_000, 100_000_000]),      # warmup 10
+    "vector_copy": (bench_vector_copy, [1_000_000, 10_000_000, 50_000_000, 100_000_000, 500_000_000]),
+    "matrix_mul": (bench_matrix_mul, [256, 512, 1024, 2048]),                               # warmup 10
+    "transpose": (bench_transpose, [256, 512, 1024, 2048, 4096, 8192]),                     # warmup 10
+    "transpose_tiled": (bench_transpose_tiled, [256, 512, 1024, 2048, 4096, 8192]),         # warmup 10
     "transfer": (bench_transfer, [1_000_000, 10_000_000, 100_000_000, 268_435_456]),   # no such program there
 }
 

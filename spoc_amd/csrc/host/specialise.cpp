@@ -2,10 +2,11 @@
 // source and run_source can serve the launch with a hand-written CDNA4 kernel.
 //
 // A kernel is recognised only when, after normalisation, it is the same program as one of
-// the five templates below (the kernels of benchmarks/bench_matrix_mul_tiled.ml:55-95,
+// the templates below (the kernels of benchmarks/bench_matrix_mul_tiled.ml:55-95,
 // benchmarks/bench_stream_triad.ml:22-32, benchmarks/bench_reduction.ml:62-96,
 // benchmarks/bench_dot_product.ml:16-54 and benchmarks/bench_reduction_max.ml:18-100 in the
-// reference; the last with any constant as the out-of-range fill).  Anything else gets the plain
+// reference, the last with any constant as the out-of-range fill; and the vector add, vector
+// copy, one-thread-per-element matmul and the two transposes).  Anything else gets the plain
 // lowering: a miss costs speed, never correctness.
 //
 // Normalisation removes what the front end is free to vary without changing meaning:
@@ -320,6 +321,87 @@ const char *kStreamTriad = R"IR(
  (native_fn true))
 )IR";
 
+// The reference's other memory-bound bench kernels and its one-thread-per-element matmul
+// (benchmarks/bench_vector_add.ml:53-61, bench_vector_copy.ml:21-27, bench_matrix_mul.ml:55-73,
+// bench_transpose.ml and bench_transpose_tiled.ml).
+const char *kVectorAdd = R"IR(
+(kernel sarek_kern
+ (params (param (var a 1 (vec f32))) (param (var b 2 (vec f32))) (param (var c 3 (vec f32))) (param (var n 4 i32)))
+ (locals)
+ (body
+ (let (var tid 5 i32) (intr (Std) global_thread_id)
+ (if (lt (var tid 5 i32) (var n 4 i32)) (assign (lelem c (var tid 5 i32)) (add (read a (var tid 5 i32)) (read b (var tid 5 i32)))))))
+ (native_fn true))
+)IR";
+
+const char *kVectorCopy = R"IR(
+(kernel sarek_kern
+ (params (param (var a 1 (vec f32))) (param (var b 2 (vec f32))) (param (var n 3 i32)))
+ (locals)
+ (body
+ (let (var tid 4 i32) (intr (Std) global_thread_id)
+ (if (lt (var tid 4 i32) (var n 3 i32)) (assign (lelem b (var tid 4 i32)) (read a (var tid 4 i32))))))
+ (native_fn true))
+)IR";
+
+const char *kMatmulNaive = R"IR(
+(kernel sarek_kern
+ (params (param (var a 1 (vec f32))) (param (var b 2 (vec f32))) (param (var c 3 (vec f32))) (param (var m 4 i32)) (param (var n 5 i32)) (param (var k 6 i32)))
+ (locals)
+ (body
+ (let (var tid 7 i32) (intr (Std) global_thread_id)
+ (let (var row 8 i32) (div (var tid 7 i32) (var n 5 i32))
+ (let (var col 9 i32) (mod (var tid 7 i32) (var n 5 i32))
+ (if (and (lt (var row 8 i32) (var m 4 i32)) (lt (var col 9 i32) (var n 5 i32))) (letmut (var sum 11 f32 mut) (f32 0.0)
+ (seq
+ (for (var i 10 i32 mut) (i32 0) (sub (var k 6 i32) (i32 1)) upto (assign (lvar (var sum 11 f32 mut)) (add (var sum 11 f32 mut) (mul (read a (add (mul (var row 8 i32) (var k 6 i32)) (var i 10 i32 mut))) (read b (add (mul (var i 10 i32 mut) (var n 5 i32)) (var col 9 i32)))))))
+ (assign (lelem c (add (mul (var row 8 i32) (var n 5 i32)) (var col 9 i32))) (var sum 11 f32 mut)))))))))
+ (native_fn true))
+)IR";
+
+const char *kTransposeNaive = R"IR(
+(kernel sarek_kern
+ (params (param (var input 1 (vec f32))) (param (var output 2 (vec f32))) (param (var width 3 i32)) (param (var height 4 i32)))
+ (locals)
+ (body
+ (let (var tid 5 i32) (intr (Std) global_thread_id)
+ (let (var n 6 i32) (mul (var width 3 i32) (var height 4 i32))
+ (if (lt (var tid 5 i32) (var n 6 i32)) (let (var col 7 i32) (mod (var tid 5 i32) (var width 3 i32))
+ (let (var row 8 i32) (div (var tid 5 i32) (var width 3 i32))
+ (let (var in_idx 9 i32) (add (mul (var row 8 i32) (var width 3 i32)) (var col 7 i32))
+ (let (var out_idx 10 i32) (add (mul (var col 7 i32) (var height 4 i32)) (var row 8 i32))
+ (assign (lelem output (var out_idx 10 i32)) (read input (var in_idx 9 i32)))))))))))
+ (native_fn true))
+)IR";
+
+const char *kTransposeTiled = R"IR(
+(kernel sarek_kern
+ (params (param (var input 1 (vec f32))) (param (var output 2 (vec f32))) (param (var width 3 i32)) (param (var height 4 i32)))
+ (locals)
+ (body
+ (let (var tile 5 (array f32 shared)) (newarray f32 (i32 272) shared)
+ (let (var tile_size 6 i32) (i32 16)
+ (let (var tx 7 i32) (intr (Gpu) thread_idx_x)
+ (let (var ty 8 i32) (intr (Gpu) thread_idx_y)
+ (let (var block_col 9 i32) (mul (intr (Gpu) block_idx_x) (var tile_size 6 i32))
+ (let (var block_row 10 i32) (mul (intr (Gpu) block_idx_y) (var tile_size 6 i32))
+ (let (var read_col 11 i32) (add (var block_col 9 i32) (var tx 7 i32))
+ (let (var read_row 12 i32) (add (var block_row 10 i32) (var ty 8 i32))
+ (seq
+ (block (if (and (lt (var read_col 11 i32) (var width 3 i32)) (lt (var read_row 12 i32) (var height 4 i32))) (let (var read_idx 13 i32) (add (mul (var read_row 12 i32) (var width 3 i32)) (var read_col 11 i32))
+ (let (var tile_idx 14 i32) (add (mul (var ty 8 i32) (i32 17)) (var tx 7 i32))
+ (assign (lelem tile (var tile_idx 14 i32)) (read input (var read_idx 13 i32)))))))
+ (barrier)
+ (let (var write_col 15 i32) (add (var block_row 10 i32) (var tx 7 i32))
+ (let (var write_row 16 i32) (add (var block_col 9 i32) (var ty 8 i32))
+ (seq
+ (block (if (and (lt (var write_col 15 i32) (var height 4 i32)) (lt (var write_row 16 i32) (var width 3 i32))) (let (var tile_idx 17 i32) (add (mul (var tx 7 i32) (i32 17)) (var ty 8 i32))
+ (let (var write_idx 18 i32) (add (mul (var write_row 16 i32) (var height 4 i32)) (var write_col 15 i32))
+ (assign (lelem output (var write_idx 18 i32)) (read tile (var tile_idx 17 i32)))))))
+ (barrier))))))))))))))
+ (native_fn true))
+)IR";
+
 std::string tree_template(bool dot) {
   const std::string tid = "(var tid 5 i32)", gid = "(var gid 6 i32)", n = "(var n 4 i32)";
   const std::string slot = "(lelem sdata " + tid + ")";
@@ -413,10 +495,20 @@ std::string recognise(const Kernel &k) {
   static const std::string t_triad = canon_kernel(parse_kernel(kStreamTriad));
   static const std::string t_reduce = strip_trailing_barrier(canon_kernel(parse_kernel(tree_template(false))));
   static const std::string t_dot = strip_trailing_barrier(canon_kernel(parse_kernel(tree_template(true))));
+  static const std::string t_add = canon_kernel(parse_kernel(kVectorAdd));
+  static const std::string t_copy = canon_kernel(parse_kernel(kVectorCopy));
+  static const std::string t_naive = canon_kernel(parse_kernel(kMatmulNaive));
+  static const std::string t_tr_naive = canon_kernel(parse_kernel(kTransposeNaive));
+  static const std::string t_tr_tiled = strip_trailing_barrier(canon_kernel(parse_kernel(kTransposeTiled)));
   const std::string c = canon_kernel(k);
   if (c == t_matmul) return "matmul_tiled_f32";
   if (c == t_triad) return "stream_triad_f32";
+  if (c == t_add) return "vector_add_f32";
+  if (c == t_copy) return "vector_copy_f32";
+  if (c == t_naive) return "matmul_naive_f32";
+  if (c == t_tr_naive) return "transpose_naive_f32";
   const std::string cs = strip_trailing_barrier(c);
+  if (cs == t_tr_tiled) return "transpose_tiled_f32";
   if (cs == t_reduce) return "reduce_sum_block256_f32";
   if (cs == t_dot) return "dot_block256_f32";
   const std::string pad = match_max_tree(cs);

@@ -52,6 +52,21 @@ bool vec_at(const sarek_hip_arg *args, int n_args, int i) {
 
 int64_t cdiv(int64_t a, int64_t b) { return (a + b - 1) / b; }
 
+// [p, p + n) and [q, q + n) (floats) share an element without being the same range.  Element-wise
+// kernels give the same result in place as out of place; a shifted overlap is a race in the
+// generated kernel and is left to it.
+bool shifted_overlap(const void *p, const void *q, int64_t n) {
+  const uintptr_t a = reinterpret_cast<uintptr_t>(p), b = reinterpret_cast<uintptr_t>(q);
+  const uintptr_t bytes = static_cast<uintptr_t>(n) * 4;
+  return a != b && a < b + bytes && b < a + bytes;
+}
+
+// A 1-D launch with at least `threads` threads.
+bool covers_1d(const int block[3], const int grid[3], int64_t threads) {
+  return block[1] == 1 && block[2] == 1 && grid[1] == 1 && grid[2] == 1 &&
+         static_cast<int64_t>(block[0]) * grid[0] >= threads;
+}
+
 // Returns 1 when the call was served by a hand kernel (status in *rc), 0 to fall back.
 int try_specialised(const std::string &tag, const int block[3], const int grid[3],
                     const sarek_hip_arg *args, int n_args, int *rc) {
@@ -83,6 +98,68 @@ int try_specialised(const std::string &tag, const int block[3], const int grid[3
     *rc = sarek_hip_triad_f32(static_cast<float *>(args[0].buffer),
                               static_cast<const float *>(args[2].buffer),
                               static_cast<const float *>(args[4].buffer), args[6].f32, n, nullptr);
+    return 1;
+  }
+  if (tag == "vector_add_f32") {
+    // (a, len, b, len, c, len, n): c[i] = a[i] + b[i], i < n.  The triad kernel with scalar 1:
+    // a + b*1 in double, rounded once, is the f32 sum.
+    if (n_args != 7 || !vec_at(args, n_args, 0) || !vec_at(args, n_args, 2) || !vec_at(args, n_args, 4) ||
+        !is_i32(args[6]))
+      return 0;
+    const int64_t n = args[6].i32;
+    if (n < 0 || !covers_1d(block, grid, n)) return 0;
+    if (args[0].length < n || args[2].length < n || args[4].length < n) return 0;
+    if (shifted_overlap(args[4].buffer, args[0].buffer, n) || shifted_overlap(args[4].buffer, args[2].buffer, n))
+      return 0;
+    *rc = sarek_hip_triad_f32(static_cast<float *>(args[4].buffer), static_cast<const float *>(args[0].buffer),
+                              static_cast<const float *>(args[2].buffer), 1.0f, n, nullptr);
+    return 1;
+  }
+  if (tag == "vector_copy_f32") {
+    // (a, len, b, len, n): b[i] = a[i], i < n
+    if (n_args != 5 || !vec_at(args, n_args, 0) || !vec_at(args, n_args, 2) || !is_i32(args[4])) return 0;
+    const int64_t n = args[4].i32;
+    if (n < 0 || !covers_1d(block, grid, n)) return 0;
+    if (args[0].length < n || args[2].length < n) return 0;
+    if (shifted_overlap(args[2].buffer, args[0].buffer, n)) return 0;
+    *rc = sarek_hip_copy_f32(static_cast<float *>(args[2].buffer), static_cast<const float *>(args[0].buffer), n,
+                             nullptr);
+    return 1;
+  }
+  if (tag == "matmul_naive_f32") {
+    // (a, len, b, len, c, len, m, n, k); one thread per element of C, row = tid / n, col = tid mod n
+    if (n_args != 9 || !vec_at(args, n_args, 0) || !vec_at(args, n_args, 2) ||
+        !vec_at(args, n_args, 4) || !is_i32(args[6]) || !is_i32(args[7]) || !is_i32(args[8]))
+      return 0;
+    const int64_t m = args[6].i32, n = args[7].i32, k = args[8].i32;
+    if (m <= 0 || n <= 0 || k <= 0 || m * n > 0x7FFFFFFF) return 0;
+    if (!covers_1d(block, grid, m * n)) return 0;
+    if (args[0].length < m * k || args[2].length < k * n || args[4].length < m * n) return 0;
+    *rc = sarek_hip_gemm_f32(static_cast<const float *>(args[0].buffer),
+                             static_cast<const float *>(args[2].buffer),
+                             static_cast<float *>(args[4].buffer), (int)m, (int)n, (int)k, nullptr);
+    return 1;
+  }
+  if (tag == "transpose_naive_f32" || tag == "transpose_tiled_f32") {
+    // (input, len, output, len, width, height): output[c * height + r] = input[r * width + c]
+    if (n_args != 6 || !vec_at(args, n_args, 0) || !vec_at(args, n_args, 2) || !is_i32(args[4]) ||
+        !is_i32(args[5]))
+      return 0;
+    const int64_t w = args[4].i32, h = args[5].i32;
+    if (w <= 0 || h <= 0 || w * h > 0x7FFFFFFF) return 0;
+    if (tag == "transpose_naive_f32") {
+      if (!covers_1d(block, grid, w * h)) return 0;
+    } else {
+      // 16 x 16 tiles; block x walks input columns, block y input rows
+      if (block[0] != 16 || block[1] != 16 || block[2] != 1 || grid[2] != 1) return 0;
+      if (grid[0] < cdiv(w, 16) || grid[1] < cdiv(h, 16)) return 0;
+    }
+    if (args[0].length < w * h || args[2].length < w * h) return 0;
+    const uintptr_t in = reinterpret_cast<uintptr_t>(args[0].buffer),
+                    out = reinterpret_cast<uintptr_t>(args[2].buffer), bytes = static_cast<uintptr_t>(w * h) * 4;
+    if (in < out + bytes && out < in + bytes) return 0;   // overlapping matrices: leave it to the generated code
+    *rc = sarek_hip_transpose_f32(static_cast<const float *>(args[0].buffer), static_cast<float *>(args[2].buffer),
+                                  (int)w, (int)h, nullptr);
     return 1;
   }
   if (tag == "reduce_sum_block256_f32" || tag == "dot_block256_f32") {

@@ -104,6 +104,8 @@ SYMBOLS = {
     "sarek_hip_dot_block256_f32": (_i, [_vp, _vp, _vp, _i64, _vp]),
     "sarek_hip_reduce_max_block256_f32": (_i, [_vp, _vp, _i64, _f, _vp]),
     "sarek_hip_fold_partials_f64": (_i, [_vp, _i64, _vp, _vp]),
+    "sarek_hip_copy_f32": (_i, [_vp, _vp, _i64, _vp]),
+    "sarek_hip_transpose_f32": (_i, [_vp, _vp, _i, _i, _vp]),
     "sarek_hip_gemm_f32": (_i, [_vp, _vp, _vp, _i, _i, _i, _vp]),
     "sarek_hip_gemm_bf16": (_i, [_vp, _vp, _vp, _i, _i, _i, _vp]),
     "sarek_hip_gemm_f16": (_i, [_vp, _vp, _vp, _i, _i, _i, _vp]),
@@ -373,6 +375,31 @@ def fold_partials(p):
     _need(p, torch.float32, "partials")
     out = torch.empty(1, dtype=torch.float64, device=p.device)
     check(lib.sarek_hip_fold_partials_f64(_ptr(p), p.numel(), _ptr(out), _stream()))
+    return out
+
+
+def copy(src, out=None):
+    """out[i] = src[i] (bench_vector_copy's kernel)."""
+    torch = _torch()
+    _need(src, torch.float32, "src")
+    out = torch.empty_like(src) if out is None else out
+    _need(out, torch.float32, "out")
+    if out.numel() < src.numel():
+        raise ValueError("copy: out is shorter than src")
+    check(lib.sarek_hip_copy_f32(_ptr(out), _ptr(src), src.numel(), _stream()))
+    return out
+
+
+def transpose(x, out=None):
+    """x: [height, width] row-major -> out: [width, height] (bench_transpose's kernels)."""
+    torch = _torch()
+    _need(x, torch.float32, "x")
+    h, w = x.shape
+    out = torch.empty((w, h), dtype=torch.float32, device=x.device) if out is None else out
+    _need(out, torch.float32, "out")
+    if out.numel() != x.numel():
+        raise ValueError("transpose: out has the wrong size")
+    check(lib.sarek_hip_transpose_f32(_ptr(x), _ptr(out), w, h, _stream()))
     return out
 
 

@@ -240,7 +240,7 @@ def test_transpose_tiled_ir_end_to_end(hip, torch_cuda):
                           (16, 16, 1), ((w + 15) // 16, (h + 15) // 16, 1),
                           [x, out, ("i32", w), ("i32", h)], shared_mem=272 * 4)
     hip.check(hip.lib.sarek_hip_device_synchronize())
-    assert path == "jit"
+    assert path == "transpose_tiled_f32"
     assert torch.equal(out.view(w, h), x.view(h, w).t())
 
 

@@ -20,6 +20,8 @@ KERNELS = sorted(os.path.basename(p)[:-3] for p in glob.glob(os.path.join(IR_DIR
 EXPECTED_TAGS = {
     "matrix_mul_tiled": "matmul_tiled_f32", "stream_triad": "stream_triad_f32",
     "reduction": "reduce_sum_block256_f32", "dot_product": "dot_block256_f32",
+    "vector_add": "vector_add_f32", "vector_copy": "vector_copy_f32", "matrix_mul": "matmul_naive_f32",
+    "transpose_naive": "transpose_naive_f32", "transpose_tiled": "transpose_tiled_f32",
 }
 
 
@@ -236,6 +238,29 @@ def test_reduction_with_other_operator_is_not_taken(hip):
     ir = open(os.path.join(IR_DIR, "reduction.ir")).read()
     assert split_tag(hip.generate_source(ir.replace("(add (read sdata", "(mul (read sdata", 1)))[0] == ""
     assert split_tag(hip.generate_source(ir.replace("(i32 64)", "(i32 65)", 1)))[0] == ""
+
+
+def test_data_movement_and_naive_matmul_near_misses_fall_back(hip):
+    def tag_of(name, old=None, new=None):
+        ir = open(os.path.join(IR_DIR, name + ".ir")).read()
+        if old is not None:
+            assert old in ir
+            ir = ir.replace(old, new, 1)
+        return split_tag(hip.generate_source(ir))[0]
+    assert tag_of("vector_add") == "vector_add_f32"
+    assert tag_of("vector_add", "(add (read a", "(sub (read a") == ""
+    assert tag_of("vector_add", "(lt (var tid 5 i32) (var n 4 i32))", "(le (var tid 5 i32) (var n 4 i32))") == ""
+    assert tag_of("vector_copy", "(read a (var tid 4 i32))", "(read a (i32 0))") == ""
+    # row and column swapped in the store: another matrix
+    assert tag_of("matrix_mul", "(lelem c (add (mul (var row 8 i32) (var n 5 i32)) (var col 9 i32)))",
+                  "(lelem c (add (mul (var col 9 i32) (var n 5 i32)) (var row 8 i32)))") == ""
+    assert tag_of("matrix_mul", "(sub (var k 6 i32) (i32 1))", "(var k 6 i32)") == ""     # one step too many
+    # a "transpose" that does not transpose, and a tile pitch of 16 (same result, other program)
+    assert tag_of("transpose_naive", "(add (mul (var col 7 i32) (var height 4 i32)) (var row 8 i32))",
+                  "(add (mul (var row 8 i32) (var width 3 i32)) (var col 7 i32))") == ""
+    assert tag_of("transpose_tiled", "(i32 17)", "(i32 16)") == ""
+    assert tag_of("transpose_tiled", "(lt (var write_col 15 i32) (var height 4 i32))",
+                  "(lt (var write_col 15 i32) (var width 3 i32))") == ""
 
 
 def reduction_max_ir(pad="(f32 -1000000.0)"):

@@ -282,3 +282,74 @@ def test_max_tree_equals_plain_max_and_keeps_tree_nan_rules(oracle):
     got = oracle.reduce_max_block256(w)
     exp = replay(w)
     assert (np.isnan(got[0]) and np.isnan(exp)) or got[0] == exp
+
+
+# ---- the other memory-bound kernels and the one-thread-per-element matmul ----------------------
+#   benchmarks/bench_vector_add.ml:68-71,108     (a = 0.001 i, b = 0.002 i, 1e-3)
+#   benchmarks/bench_vector_copy.ml:41-43,109    ((i mod 100)/100, 1e-6)
+#   benchmarks/bench_transpose.ml:50-57,103,143-148 (input[i] = i, cpu_transpose, 1e-3)
+#   benchmarks/bench_matrix_mul.ml:43-52,86-90   (inputs and double loop of the tiled bench)
+
+def test_vector_add_reference_inputs_and_single_rounding(oracle):
+    n = 10007
+    a, b = np.arange(n) * 0.001, np.arange(n) * 0.002
+    out = np.full(n, -7.0, dtype=np.float32)
+    oracle.vector_add(a, b, out, n)
+    assert np.all(np.abs(out.astype(np.float64) - (a + b)) <= 1e-3)        # the bench's check
+    # two binary32 values add exactly in double, so one rounding gives the binary32 sum
+    rng = np.random.default_rng(5)
+    x = (rng.standard_normal(4096) * 10.0 ** rng.integers(-20, 20, 4096)).astype(np.float32)
+    y = (rng.standard_normal(4096) * 10.0 ** rng.integers(-20, 20, 4096)).astype(np.float32)
+    out = np.zeros(4096, dtype=np.float32)
+    assert np.array_equal(oracle.vector_add(x, y, out, 4096), x + y)
+    # `if tid < n`: a longer vector keeps its tail, a shorter launch leaves its own tail alone
+    out = np.full(100, -7.0, dtype=np.float32)
+    oracle.vector_add(x[:100], y[:100], out, 60, threads=256)
+    assert np.array_equal(out[:60], (x + y)[:60]) and np.all(out[60:] == -7.0)
+    out = np.full(100, -7.0, dtype=np.float32)
+    oracle.vector_add(x[:100], y[:100], out, 100, threads=64)
+    assert np.array_equal(out[:64], (x + y)[:64]) and np.all(out[64:] == -7.0)
+
+
+def test_vector_copy_reference_inputs(oracle):
+    n = 1000
+    a = (np.arange(n) % 100) / 100.0
+    out = np.full(n + 5, 9.0, dtype=np.float32)
+    oracle.vector_copy(a, out, n)
+    assert np.all(np.abs(out[:n].astype(np.float64) - a) <= 1e-6) and np.all(out[n:] == 9.0)
+    assert np.array_equal(out[:n], a.astype(np.float32))
+
+
+def test_transpose_reference_inputs_and_shapes(oracle):
+    m = 48
+    data = np.arange(m * m, dtype=np.float64)
+    out = oracle.transpose(data, m, m)
+    expected = np.zeros(m * m)
+    for row in range(m):                       # cpu_transpose of the bench
+        for col in range(m):
+            expected[col * m + row] = data[row * m + col]
+    assert np.all(np.abs(out - expected) <= 1e-3)
+    # rectangular: `width` columns in, `height` columns out; a wrong pitch fails this
+    w, h = 7, 5
+    x = np.arange(w * h, dtype=np.float32)
+    assert np.array_equal(oracle.transpose(x, w, h).reshape(w, h), x.reshape(h, w).T)
+    part = oracle.transpose(x, w, h, out=np.full(w * h, -1, dtype=np.float32), threads=w * 2)   # two input rows
+    assert np.array_equal(part.reshape(w, h)[:, :2], x.reshape(h, w).T[:, :2]) and np.all(part.reshape(w, h)[:, 2:] == -1)
+    twice = oracle.transpose(oracle.transpose(x, w, h), h, w)
+    assert np.array_equal(twice, x)
+
+
+def test_naive_matmul_is_the_same_sum_as_the_tiled_kernel(oracle):
+    m, n, k = 19, 23, 41
+    a = oracle.fill_uniform(m * k, seed=3, lo=-1, hi=1)
+    b = oracle.fill_uniform(k * n, seed=4, lo=-1, hi=1)
+    c = oracle.matmul_naive(a, b, m, n, k)
+    # zero padding of the tiles adds exact zeros: both kernels compute the same double sums
+    assert np.array_equal(c.reshape(m, n), oracle.gemm(a.reshape(m, k), b.reshape(k, n)))
+    assert np.array_equal(c.reshape(m, n), oracle.matmul_tiled_bsp(a.reshape(m, k), b.reshape(k, n)))
+    a64, b64 = ref_inputs_matmul(16, 16, 16)
+    c = oracle.matmul_naive(a64.reshape(-1), b64.reshape(-1), 16, 16, 16)
+    assert np.all(np.abs(c.reshape(16, 16) - python_double_loop(a64, b64)) <= 1e-3)
+    # row = tid / n, col = tid mod n: a launch of n + 3 threads fills row 0 and three of row 1
+    part = oracle.matmul_naive(a, b, m, n, k, out=np.full(m * n, -1, dtype=np.float32), threads=n + 3)
+    assert np.array_equal(part[:n + 3], c_full := oracle.matmul_naive(a, b, m, n, k)[:n + 3]) and np.all(part[n + 3:] == -1)
