@@ -95,7 +95,7 @@ def make_workload(name, torch, hip):
         ws = hip.triad_sum_workspace(n)
         info = dict(metric="fused triad+sum GB/s", unit="GB/s", dtype="f32",
                     work=12.0 * n, work_unit=1e9, bound="hbm", peak=PEAK_HBM_GBS,
-                    kernel="triad_kernel<true> (+ fold_kernel, 1 % of the time)",
+                    kernel="triad_kernel<true, true> (+ fold_kernel, 1 % of the time)",
                     config={"workload": "fused stream triad + sum, a=b+3c, sum(a)", "n": n,
                             "algorithmic_bytes": 12 * n})
         return (lambda: hip.triad_sum(b, c, 3.0, out=a, workspace=ws)), info

@@ -80,7 +80,7 @@ __device__ __forceinline__ void stg_nt(float4 *p, float4 v) {
 
 // a = b + c*s.  Workgroup g owns float4 [g*kChunk, (g+1)*kChunk); the last one also takes
 // the (n & 3) scalar tail.  When WithSum, partials[g] gets the workgroup's f32 sum.
-template <bool WithSum>
+template <bool WithSum, bool NtLoad = true>
 __global__ __launch_bounds__(kBlock) void triad_kernel(float *__restrict__ a,
                                                        const float *__restrict__ b,
                                                        const float *__restrict__ c, float s,
@@ -97,9 +97,9 @@ __global__ __launch_bounds__(kBlock) void triad_kernel(float *__restrict__ a,
   if (full) {
     float4 bv[kUnroll], cv[kUnroll];
 #pragma unroll
-    for (int u = 0; u < kUnroll; ++u) bv[u] = ldg_nt(b4 + base + u * kBlock);
+    for (int u = 0; u < kUnroll; ++u) bv[u] = NtLoad ? ldg_nt(b4 + base + u * kBlock) : b4[base + u * kBlock];
 #pragma unroll
-    for (int u = 0; u < kUnroll; ++u) cv[u] = ldg_nt(c4 + base + u * kBlock);
+    for (int u = 0; u < kUnroll; ++u) cv[u] = NtLoad ? ldg_nt(c4 + base + u * kBlock) : c4[base + u * kBlock];
 #pragma unroll
     for (int u = 0; u < kUnroll; ++u) r[u] = triad4(bv[u], cv[u], sd);
   } else {
@@ -311,6 +311,18 @@ __global__ __launch_bounds__(kBlock) void cast16_kernel(const float *__restrict_
 
 inline bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 
+// Load policy for `input_bytes` of input.  Inputs that together fit the 256 MB last-level
+// cache may still be there (the producer's output, the previous launch's input): plain loads
+// hit it, non-temporal ones go round it (measured: triad 7.1 vs 6.6 TB/s at 3 x 120 MB).
+// Larger inputs come from HBM whatever the policy and non-temporal loads keep them out of
+// the way of the stores (6.4 vs 5.8 TB/s at 3 x 1 GiB).  The read-only block-256 kernels have
+// no store stream to protect and measured the same or better with non-temporal loads at
+// every size, so they always use them.  Tunable "stream.nt" forces 0 / 1.
+inline bool streams_from_hbm(int64_t input_bytes) {
+  const int64_t forced = tunable("stream.nt", -1);
+  return forced >= 0 ? forced != 0 : input_bytes > (int64_t{256} << 20);
+}
+
 // Workgroups (= f32 partials) of the triad kernels for n elements.
 inline int64_t triad_blocks(int64_t n) {
   return ceil_div(n > 0 ? n : 1, static_cast<int64_t>(kChunk) * 4);
@@ -323,14 +335,17 @@ int launch_triad(float *a, const float *b, const float *c, float s, int64_t n, f
   if (blocks64 > 0x7FFFFFFF) return fail(SAREK_HIP_E_INVALID_ARG, "triad: vector too long");
   const unsigned blocks = static_cast<unsigned>(blocks64);
   if (vec) {
+    const bool nt = streams_from_hbm(n * 8);
     if (with_sum) {
-      hipLaunchKernelGGL(triad_kernel<true>, dim3(blocks), dim3(kBlock), 0, st, a, b, c, s, n, partials);
+      if (nt) hipLaunchKernelGGL((triad_kernel<true, true>), dim3(blocks), dim3(kBlock), 0, st, a, b, c, s, n, partials);
+      else hipLaunchKernelGGL((triad_kernel<true, false>), dim3(blocks), dim3(kBlock), 0, st, a, b, c, s, n, partials);
       int rc = check_launch("triad kernel launch");
       if (rc != SAREK_HIP_OK) return rc;
       hipLaunchKernelGGL(fold_kernel, dim3(1), dim3(1024), 0, st, partials, blocks64, sum_out);
       return check_launch("fold kernel launch");
     }
-    hipLaunchKernelGGL(triad_kernel<false>, dim3(blocks), dim3(kBlock), 0, st, a, b, c, s, n, partials);
+    if (nt) hipLaunchKernelGGL((triad_kernel<false, true>), dim3(blocks), dim3(kBlock), 0, st, a, b, c, s, n, partials);
+    else hipLaunchKernelGGL((triad_kernel<false, false>), dim3(blocks), dim3(kBlock), 0, st, a, b, c, s, n, partials);
     return check_launch("triad kernel launch");
   }
   // 4-byte aligned vectors: scalar kernel on a capped grid, then a separate fold
