@@ -2,7 +2,8 @@
 
 Host-side mirror of benchmarks/bench_matrix_mul_tiled.ml, bench_stream_triad.ml,
 bench_reduction.ml, bench_dot_product.ml, bench_reduction_max.ml, bench_vector_add.ml,
-bench_vector_copy.ml, bench_matrix_mul.ml, bench_transpose.ml and bench_transpose_tiled.ml: same inputs, same
+bench_vector_copy.ml, bench_matrix_mul.ml, bench_transpose.ml, bench_transpose_tiled.ml and
+bench_scan.ml: same inputs, same
 launch geometry, same warmup / timed-iteration protocol (wall clock around the launch plus
 the device flush, one sample per iteration), same verification and tolerance, same
 throughput formula and statistic, and the same per-device result record
@@ -269,6 +270,25 @@ def bench_transpose_tiled(size, warmup=10, iterations=20, tile_size=16):
                             size, warmup, iterations)
 
 
+def bench_scan(size, warmup=5, iterations=20):
+    """benchmarks/bench_scan.ml:112-221: inclusive prefix sum of [1..n] in one 256-thread block
+    (n = min(size, 256)), every element equal to the serial prefix sum, M elements/s = n / median."""
+    import torch
+    n = min(size, 256)
+    data = np.arange(1, n + 1, dtype=np.int32)
+    vin = torch.empty(n, dtype=torch.int32, device="cuda")
+    hip.memcpy_htod(vin.data_ptr(), data)
+    vout = torch.zeros(n, dtype=torch.int32, device="cuda")
+    src = hip.generate_source(reference_kernels.inclusive_scan(), block=(256, 1, 1))
+    args = [vin, vout, ("i32", n)]
+    times, path = _time_launches(lambda: hip.run_source(src, "sarek_kern", (256, 1, 1), (1, 1, 1), args),
+                                 warmup, iterations)
+    got = np.empty(n, dtype=np.int32)
+    hip.memcpy_dtoh(got, vout.data_ptr())
+    verified = bool(np.array_equal(got, np.cumsum(data, dtype=np.int32)))
+    return _device_record(times, n / (statistics.median(times) / 1e3 * 1e6), verified, path, "Melem/s")
+
+
 def bench_transfer(size, warmup=2, iterations=7):
     """Not one of the reference's programs: the Transfer.to_device / Transfer.to_cpu legs
     (sarek/core/Transfer.ml:228-333) that its benches run once before and after their timed
@@ -320,6 +340,7 @@ BENCHMARKS = {
     "matrix_mul": (bench_matrix_mul, [256, 512, 1024, 2048]),                               # warmup 10
     "transpose": (bench_transpose, [256, 512, 1024, 2048, 4096, 8192]),                     # warmup 10
     "transpose_tiled": (bench_transpose_tiled, [256, 512, 1024, 2048, 4096, 8192]),         # warmup 10
+    "scan": (bench_scan, [64, 128, 256]),
     "transfer": (bench_transfer, [1_000_000, 10_000_000, 100_000_000, 268_435_456]),   # no such program there
 }
 

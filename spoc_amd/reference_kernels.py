@@ -358,6 +358,37 @@ def radix_sort_scatter():
     return kernel(params, body)
 
 
+def inclusive_scan():
+    """benchmarks/bench_scan.ml:48-109: Hillis-Steele inclusive scan of one 256-element block in
+    two shared int32 arrays that swap roles every superstep.  No golden generated text exists
+    for this kernel; the transcription is pinned by its result (a prefix sum, exact in int32)."""
+    fresh()
+    params = [("input", "(vec i32)"), ("output", "(vec i32)"), ("n", "i32")]
+    for p, t in params:
+        var(p, t)
+    n = var("n")
+    temp, temp2 = var("temp", "(array i32 shared)"), var("temp2", "(array i32 shared)")
+    tid, gid = var("tid"), var("gid")
+    steps = [block(if_(lt(gid, n), assign_elem("temp", tid, read("input", gid)), assign_elem("temp", tid, i32(0)))),
+             BARRIER]
+    src, dst = "temp", "temp2"
+    d = 1
+    while d <= 128:
+        v, a = var(f"v{d}"), var(f"add{d}")
+        steps += [block(let(v, read(src, tid),
+                            let(a, f"(if {op('ge', tid, i32(d))} {read(src, sub(tid, i32(d)))} {i32(0)})",
+                                assign_elem(dst, tid, add(v, a))))),
+                  BARRIER]
+        src, dst = dst, src
+        d *= 2
+    steps.append(if_(lt(gid, n), assign_elem("output", gid, read(src, tid))))
+    body = shared(temp, "i32", 512, shared(temp2, "i32", 512, lets(
+        [(tid, intr("thread_idx_x")),
+         (gid, add(intr("thread_idx_x"), mul(intr("block_dim_x"), intr("block_idx_x"))))],
+        seq(*steps))))
+    return kernel(params, body)
+
+
 KERNELS = {
     "stream_triad": stream_triad, "vector_add": vector_add, "vector_copy": vector_copy,
     "matrix_mul": matrix_mul, "matrix_mul_tiled": matrix_mul_tiled,

@@ -187,7 +187,7 @@ def test_naive_matmul_ir(hip, oracle, torch_cuda, specialise, m, n, k):
 @pytest.mark.parametrize("name,size,path", [
     ("vector_add", 100003, "vector_add_f32"), ("vector_copy", 100003, "vector_copy_f32"),
     ("matrix_mul", 200, "matmul_naive_f32"), ("transpose", 200, "transpose_naive_f32"),
-    ("transpose_tiled", 200, "transpose_tiled_f32")])
+    ("transpose_tiled", 200, "transpose_tiled_f32"), ("scan", 256, "jit"), ("scan", 100, "jit")])
 def test_reference_benchmarks_run_and_verify(hip, torch_cuda, name, size, path):
     """The mirrors of the five bench programs: the reference's inputs, geometry and checks, served
     by the hand kernels; and the same with the plain JIT lowering."""
