@@ -119,6 +119,14 @@ int sarek_hip_event_record(sarek_hip_event e, sarek_hip_stream s);
 int sarek_hip_event_synchronize(sarek_hip_event e);
 int sarek_hip_event_elapsed_ms(sarek_hip_event start, sarek_hip_event stop, float *ms);
 
+/* BACKEND.enable_profiling / disable_profiling (cuProfilerStart / cuProfilerStop,
+ * sarek-cuda/Cuda_plugin_base.ml:294-300; optional symbols there,
+ * sarek-cuda/Cuda_bindings.ml:497-525): the range markers an attached profiler
+ * honours.  Like the reference, the result of the underlying call is ignored; both
+ * always return SAREK_HIP_OK.                                                  */
+int sarek_hip_profiler_start(void);
+int sarek_hip_profiler_stop(void);
+
 /* ---------------------------------------------------------------------- */
 /* Kernel JIT + launch  (replaces the nvrtc.., cuModule.. groups and cuLaunchKernel,
  * sarek-cuda/Cuda_nvrtc.ml:263-389, sarek-cuda/Cuda_api.ml:315-486).
@@ -199,6 +207,77 @@ int sarek_hip_set_specialisation(int enabled);
 /* Name of the code path the last sarek_hip_run_source call took on this
  * thread: "jit" or the specialise tag.                                     */
 const char *sarek_hip_last_run_path(void);
+
+/* ---------------------------------------------------------------------- */
+/* The host side of a launch, for callers without the reference's OCaml core:
+ * vectors with a host block, per-device buffers and a location state
+ * (sarek/core/Vector.ml, Vector_types.ml:198-203), the transfers between them
+ * (sarek/core/Transfer.ml:173-388) and the dispatcher (sarek/sarek/Execute.ml:188-216,
+ * 321-335, 520-543, 613-651).  Semantics follow the reference state by state.     */
+typedef struct sarek_hip_vector_s *sarek_hip_vector;
+enum {                                  /* Vector_types.scalar_kind + Custom            */
+  SAREK_HIP_KIND_FLOAT32 = 0, SAREK_HIP_KIND_FLOAT64 = 1, SAREK_HIP_KIND_INT32 = 2,
+  SAREK_HIP_KIND_INT64 = 3, SAREK_HIP_KIND_CHAR = 4, SAREK_HIP_KIND_COMPLEX32 = 5,
+  SAREK_HIP_KIND_CUSTOM = 6
+};
+enum {                                  /* Vector_types.location                         */
+  SAREK_HIP_LOC_CPU = 0, SAREK_HIP_LOC_GPU = 1, SAREK_HIP_LOC_BOTH = 2,
+  SAREK_HIP_LOC_STALE_CPU = 3,          /* the device copy is the good one               */
+  SAREK_HIP_LOC_STALE_GPU = 4           /* the host copy is the good one                 */
+};
+/* Vector.create / create_custom: host block of `length` elements, contents unspecified,
+ * location CPU.  pinned != 0 takes the block from sarek_hip_host_alloc.              */
+int sarek_hip_vector_create(int kind, int64_t length, int64_t custom_elem_size, int pinned,
+                            sarek_hip_vector *out);
+int sarek_hip_vector_destroy(sarek_hip_vector v);          /* host block and device buffers */
+int64_t sarek_hip_vector_length(sarek_hip_vector v);
+int64_t sarek_hip_vector_elem_size(sarek_hip_vector v);
+int sarek_hip_vector_kind(sarek_hip_vector v);
+int sarek_hip_vector_location(sarek_hip_vector v, int *location, int *device /* may be NULL */);
+void *sarek_hip_vector_host_ptr(sarek_hip_vector v);       /* Vector.host_ptr: raw, no sync  */
+int sarek_hip_vector_device_ptr(sarek_hip_vector v, void **dptr);   /* NULL: no buffer yet */
+int sarek_hip_vector_set_auto_sync(sarek_hip_vector v, int enabled);
+/* Vector.get / Vector.set (Vector.ml:80-109): bounds-checked ("Vector.get: index I out
+ * of bounds [0, N)" with SAREK_HIP_E_INVALID_ARG); get first downloads a Stale_CPU
+ * vector when auto-sync is on; set marks a Both / GPU vector Stale_GPU and does not
+ * download first.  read / write are the same for a range of elements (Vector.to_array,
+ * a loop of Vector.set).                                                           */
+int sarek_hip_vector_get(sarek_hip_vector v, int64_t index, void *out_elem);
+int sarek_hip_vector_set(sarek_hip_vector v, int64_t index, const void *elem);
+int sarek_hip_vector_read(sarek_hip_vector v, void *dst, int64_t first, int64_t count);
+int sarek_hip_vector_write(sarek_hip_vector v, const void *src, int64_t first, int64_t count);
+/* Transfer.set_auto, to_device (to the current device), to_cpu ?force, sync,
+ * free_all_buffers, flush.                                                         */
+int sarek_hip_transfer_set_auto(int enabled);
+int sarek_hip_transfer_to_device(sarek_hip_vector v);
+int sarek_hip_transfer_to_cpu(sarek_hip_vector v, int force);
+int sarek_hip_transfer_sync(sarek_hip_vector v);
+int sarek_hip_transfer_free_buffers(sarek_hip_vector v);
+int sarek_hip_transfer_flush(void);
+/* Execute.vector_arg (Execute.ml:28-35; Int goes as INT32, as expand_to_run_source_args sends it). */
+enum { SAREK_HIP_VARG_VEC = 0, SAREK_HIP_VARG_INT32 = 1, SAREK_HIP_VARG_INT64 = 2,
+       SAREK_HIP_VARG_FLOAT32 = 3, SAREK_HIP_VARG_FLOAT64 = 4 };
+typedef struct sarek_hip_varg {
+  int kind;
+  sarek_hip_vector vec;
+  int32_t i32;
+  int64_t i64;
+  float f32;
+  double f64;
+} sarek_hip_varg;
+/* Execute.run_vectors (Execute.ml:520-543): uploads what is not on the device yet,
+ * lowers the IR (one lowering per distinct text is kept), expands vectors to
+ * (buffer, int32 length), launches through sarek_hip_run_source under the kernel's own
+ * name, then marks the Both vectors Stale_CPU.  A kernel the lowering refuses is
+ * "Backend failed to generate source" (Execute.ml:257-263).                        */
+int sarek_hip_execute_run_vectors(const char *ir_text, const int block[3], const int grid[3],
+                                  int shared_mem_bytes, const sarek_hip_varg *args, int n_args);
+/* Execute.run_source (Execute.ml:613-651): an external kernel; inject_lengths = 0 passes
+ * bare buffers (sarek/tests/e2e/test_external_kernel.ml:46-62).                      */
+int sarek_hip_execute_run_source(const char *source, int lang, const char *kernel_name,
+                                 const int block[3], const int grid[3], int shared_mem_bytes,
+                                 int inject_lengths, const sarek_hip_varg *args, int n_args);
+int sarek_hip_execute_sync_vectors_to_cpu(const sarek_hip_varg *args, int n_args);
 
 /* ---------------------------------------------------------------------- */
 /* Hand-written CDNA4 kernels.  All pointers are device pointers.  These have

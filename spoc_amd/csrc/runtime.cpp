@@ -311,6 +311,22 @@ int sarek_hip_event_elapsed_ms(sarek_hip_event start, sarek_hip_event stop, floa
   return SAREK_HIP_OK;
 }
 
+int sarek_hip_profiler_start(void) {
+#pragma clang diagnostic push
+#pragma clang diagnostic ignored "-Wdeprecated-declarations"
+  if (hipProfilerStart() != hipSuccess) (void)hipGetLastError();
+#pragma clang diagnostic pop
+  return SAREK_HIP_OK;
+}
+
+int sarek_hip_profiler_stop(void) {
+#pragma clang diagnostic push
+#pragma clang diagnostic ignored "-Wdeprecated-declarations"
+  if (hipProfilerStop() != hipSuccess) (void)hipGetLastError();
+#pragma clang diagnostic pop
+  return SAREK_HIP_OK;
+}
+
 int sarek_hip_kernel_compile(const char *source, const char *kernel_name, sarek_hip_kernel *out,
                              char *log, size_t log_len) {
   return compile_impl(source, kernel_name, out, log, log_len);

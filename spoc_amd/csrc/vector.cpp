@@ -1,0 +1,434 @@
+// Host side of a launch above the plugin boundary: vectors with a host block, per-device
+// buffers and a location state (sarek/core/Vector.ml, Vector_types.ml:198-203), the
+// transfers that move them (sarek/core/Transfer.ml:173-388) and the dispatcher that turns
+// a kernel's IR plus a list of vectors and scalars into a run_source call
+// (sarek/sarek/Execute.ml:188-216, 231-304, 321-335, 520-543, 613-651).  In the reference
+// these are backend-agnostic OCaml; a host without OCaml gets them here, state machine
+// and corner cases included:
+//   - to_device copies only from CPU / Stale_GPU (or another device) and leaves Both;
+//   - a launch marks only Both vectors Stale_CPU;
+//   - a host write marks Both / GPU vectors Stale_GPU and does NOT first fetch a stale
+//     host copy (a write into a Stale_CPU vector is overwritten by the next download);
+//   - a host read downloads a Stale_CPU vector when auto-sync is on (vector and global).
+#include <cstdlib>
+#include <cstring>
+#include <map>
+#include <mutex>
+#include <string>
+#include <unordered_map>
+#include <vector>
+
+#include "common.hpp"
+#include "host/ir.hpp"
+#include "plugin.hpp"
+
+struct sarek_hip_vector_s {
+  int kind = SAREK_HIP_KIND_FLOAT32;
+  int64_t length = 0, elem_size = 4;
+  void *host = nullptr;
+  bool pinned = false;
+  bool auto_sync = true;                 // Vector_types.t.auto_sync
+  int location = SAREK_HIP_LOC_CPU;
+  int device = -1;                       // the device of a non-CPU location
+  std::map<int, void *> buffers;         // device id -> device block (vec.device_buffers)
+};
+
+namespace sarek_hip {
+namespace {
+
+bool g_auto_mode = true;                 // Transfer.auto_mode (Transfer.ml:20-28)
+
+int64_t kind_elem_size(int kind, int64_t custom) {
+  switch (kind) {                        // Vector_types.scalar_elem_size
+    case SAREK_HIP_KIND_FLOAT32: case SAREK_HIP_KIND_INT32: return 4;
+    case SAREK_HIP_KIND_FLOAT64: case SAREK_HIP_KIND_INT64: case SAREK_HIP_KIND_COMPLEX32: return 8;
+    case SAREK_HIP_KIND_CHAR: return 1;
+    case SAREK_HIP_KIND_CUSTOM: return custom;
+    default: return 0;
+  }
+}
+
+size_t bytes_of(const sarek_hip_vector_s *v) { return static_cast<size_t>(v->length * v->elem_size); }
+
+int current_device(int *dev) {
+  SAREK_HIP_TRY(hipGetDevice(dev));
+  return SAREK_HIP_OK;
+}
+
+// Transfer.ensure_buffer: the vector's block on `dev`, allocated on first use.
+int ensure_buffer(sarek_hip_vector_s *v, int dev, void **out) {
+  auto it = v->buffers.find(dev);
+  if (it != v->buffers.end()) {
+    *out = it->second;
+    return SAREK_HIP_OK;
+  }
+  void *p = nullptr;
+  int st = sarek_hip_mem_alloc(&p, bytes_of(v));
+  if (st != SAREK_HIP_OK) return st;
+  v->buffers[dev] = p;
+  *out = p;
+  return SAREK_HIP_OK;
+}
+
+bool on_device(const sarek_hip_vector_s *v, int loc, int dev) { return v->location == loc && v->device == dev; }
+
+// Transfer.to_device (Transfer.ml:228-268)
+int to_device(sarek_hip_vector_s *v, int dev) {
+  if (on_device(v, SAREK_HIP_LOC_GPU, dev) || on_device(v, SAREK_HIP_LOC_BOTH, dev) ||
+      on_device(v, SAREK_HIP_LOC_STALE_CPU, dev))
+    return SAREK_HIP_OK;
+  void *buf = nullptr;
+  int st = ensure_buffer(v, dev, &buf);
+  if (st != SAREK_HIP_OK) return st;
+  st = sarek_hip_memcpy_htod(buf, v->host, bytes_of(v));
+  if (st != SAREK_HIP_OK) return st;
+  v->location = SAREK_HIP_LOC_BOTH;
+  v->device = dev;
+  return SAREK_HIP_OK;
+}
+
+// Transfer.to_cpu ?force (Transfer.ml:274-333)
+int to_cpu(sarek_hip_vector_s *v, bool force) {
+  bool needed = false;
+  switch (v->location) {
+    case SAREK_HIP_LOC_BOTH: needed = force; break;
+    case SAREK_HIP_LOC_GPU: case SAREK_HIP_LOC_STALE_CPU: needed = true; break;
+    default: break;                      // CPU: no device copy; Stale_GPU: the host copy is the good one
+  }
+  if (!needed) return SAREK_HIP_OK;
+  auto it = v->buffers.find(v->device);
+  if (it == v->buffers.end()) return fail(SAREK_HIP_E_INVALID_ARG, "to_cpu: no device buffer to transfer from");
+  int st = sarek_hip_memcpy_dtoh(v->host, it->second, bytes_of(v));
+  if (st != SAREK_HIP_OK) return st;
+  v->location = SAREK_HIP_LOC_BOTH;
+  return SAREK_HIP_OK;
+}
+
+// Vector_transfer.ensure_cpu_sync + the callback Transfer registers (Transfer.ml:454-464)
+int ensure_cpu_sync(sarek_hip_vector_s *v) {
+  if (v->auto_sync && v->location == SAREK_HIP_LOC_STALE_CPU && g_auto_mode) return to_cpu(v, false);
+  return SAREK_HIP_OK;
+}
+
+// Vector.set's bookkeeping (Vector.ml:104-109)
+void host_written(sarek_hip_vector_s *v) {
+  if (v->location == SAREK_HIP_LOC_BOTH || v->location == SAREK_HIP_LOC_GPU) v->location = SAREK_HIP_LOC_STALE_GPU;
+}
+
+// Range check of a bulk access, reported like the element accessors report theirs
+// (Vector.ml:80-103).
+int bounds(const sarek_hip_vector_s *v, int64_t first, int64_t count, const char *what) {
+  if (first >= 0 && count >= 0 && first + count <= v->length) return SAREK_HIP_OK;
+  const int64_t bad = first < 0 ? first : (count < 0 ? count : v->length);
+  return fail(SAREK_HIP_E_INVALID_ARG, "Vector.%s: index %lld out of bounds [0, %lld)", what,
+              static_cast<long long>(bad), static_cast<long long>(v->length));
+}
+
+// Execute.transfer_vectors_to_device
+int transfer_args(const sarek_hip_varg *args, int n, int dev) {
+  for (int i = 0; i < n; ++i)
+    if (args[i].kind == SAREK_HIP_VARG_VEC) {
+      if (!args[i].vec) return fail(SAREK_HIP_E_INVALID_ARG, "argument %d: NULL vector", i);
+      int st = to_device(args[i].vec, dev);
+      if (st != SAREK_HIP_OK) return st;
+    }
+  return SAREK_HIP_OK;
+}
+
+// Execute.expand_to_run_source_args
+int expand_args(const sarek_hip_varg *args, int n, int dev, bool inject_lengths, std::vector<sarek_hip_arg> &out) {
+  for (int i = 0; i < n; ++i) {
+    sarek_hip_arg a;
+    std::memset(&a, 0, sizeof(a));
+    switch (args[i].kind) {
+      case SAREK_HIP_VARG_VEC: {
+        sarek_hip_vector_s *v = args[i].vec;
+        auto it = v->buffers.find(dev);
+        if (it == v->buffers.end()) return fail(SAREK_HIP_E_INVALID_ARG, "Vector has no device buffer");
+        a.kind = SAREK_HIP_ARG_BUFFER;
+        a.buffer = it->second;
+        a.length = v->length;
+        out.push_back(a);
+        if (inject_lengths) {
+          sarek_hip_arg l;
+          std::memset(&l, 0, sizeof(l));
+          l.kind = SAREK_HIP_ARG_INT32;
+          l.i32 = static_cast<int32_t>(v->length);
+          out.push_back(l);
+        }
+        continue;
+      }
+      case SAREK_HIP_VARG_INT32: a.kind = SAREK_HIP_ARG_INT32; a.i32 = args[i].i32; break;
+      case SAREK_HIP_VARG_INT64: a.kind = SAREK_HIP_ARG_INT64; a.i64 = args[i].i64; break;
+      case SAREK_HIP_VARG_FLOAT32: a.kind = SAREK_HIP_ARG_FLOAT32; a.f32 = args[i].f32; break;
+      case SAREK_HIP_VARG_FLOAT64: a.kind = SAREK_HIP_ARG_FLOAT64; a.f64 = args[i].f64; break;
+      default: return fail(SAREK_HIP_E_INVALID_ARG, "argument %d: unknown kind %d", i, args[i].kind);
+    }
+    out.push_back(a);
+  }
+  return SAREK_HIP_OK;
+}
+
+// Execute.mark_vectors_stale: only a vector that was in step with the device goes stale.
+void mark_stale(const sarek_hip_varg *args, int n, int dev) {
+  for (int i = 0; i < n; ++i)
+    if (args[i].kind == SAREK_HIP_VARG_VEC && args[i].vec->location == SAREK_HIP_LOC_BOTH) {
+      args[i].vec->location = SAREK_HIP_LOC_STALE_CPU;
+      args[i].vec->device = dev;
+    }
+}
+
+// IR text -> (kernel name, source).  The reference regenerates and re-hashes the source at
+// every launch (Execute.ml:256); here one lowering per distinct IR text is kept.
+struct Lowered {
+  std::string name, source;
+};
+std::mutex g_lowered_mu;
+std::unordered_map<std::string, Lowered> g_lowered;
+
+int lower(const char *ir_text, const int block[3], Lowered &out) {
+  {
+    std::lock_guard<std::mutex> lock(g_lowered_mu);
+    auto it = g_lowered.find(ir_text);
+    if (it != g_lowered.end()) {
+      out = it->second;
+      return SAREK_HIP_OK;
+    }
+  }
+  size_t needed = 0;
+  int st = sarek_hip_generate_source(ir_text, block, nullptr, 0, &needed);
+  if (st != SAREK_HIP_E_BUFFER_TOO_SMALL) {
+    // generate_source returning None: Execute.run raises Compilation_failed (Execute.ml:257-263)
+    const std::string why = sarek_hip_last_error();
+    return fail(st == SAREK_HIP_OK ? SAREK_HIP_E_CODEGEN : st, "Backend failed to generate source: %s", why.c_str());
+  }
+  std::string src(needed, '\0');
+  st = sarek_hip_generate_source(ir_text, block, src.data(), src.size(), &needed);
+  if (st != SAREK_HIP_OK) return st;
+  src.resize(std::strlen(src.c_str()));
+  out.source = src;
+  out.name = ir::parse_kernel(ir_text).name;
+  std::lock_guard<std::mutex> lock(g_lowered_mu);
+  if (g_lowered.size() > 256) g_lowered.clear();
+  g_lowered[ir_text] = out;
+  return SAREK_HIP_OK;
+}
+
+}  // namespace
+}  // namespace sarek_hip
+
+using namespace sarek_hip;
+
+extern "C" {
+
+int sarek_hip_vector_create(int kind, int64_t length, int64_t custom_elem_size, int pinned, sarek_hip_vector *out) {
+  if (!out) return fail(SAREK_HIP_E_INVALID_ARG, "vector_create: NULL out pointer");
+  *out = nullptr;
+  const int64_t es = kind_elem_size(kind, custom_elem_size);
+  if (es <= 0) return fail(SAREK_HIP_E_INVALID_ARG, "vector_create: unknown kind %d or element size %lld", kind,
+                           static_cast<long long>(custom_elem_size));
+  if (length < 0) return fail(SAREK_HIP_E_INVALID_ARG, "vector_create: negative length");
+  auto *v = new sarek_hip_vector_s;
+  v->kind = kind;
+  v->length = length;
+  v->elem_size = es;
+  v->pinned = pinned != 0;
+  const size_t bytes = static_cast<size_t>(length * es);
+  if (v->pinned) {
+    int st = sarek_hip_host_alloc(&v->host, bytes);
+    if (st != SAREK_HIP_OK) {
+      delete v;
+      return st;
+    }
+  } else {
+    v->host = std::malloc(bytes ? bytes : 1);   // like a fresh Bigarray: contents unspecified
+    if (!v->host) {
+      delete v;
+      return fail(SAREK_HIP_E_INVALID_ARG, "vector_create: out of host memory (%zu bytes)", bytes);
+    }
+  }
+  *out = v;
+  return SAREK_HIP_OK;
+}
+
+int sarek_hip_vector_destroy(sarek_hip_vector v) {
+  if (!v) return SAREK_HIP_OK;
+  int first = SAREK_HIP_OK;
+  for (auto &b : v->buffers) {
+    int st = sarek_hip_mem_free(b.second);
+    if (first == SAREK_HIP_OK) first = st;
+  }
+  if (v->pinned) {
+    int st = sarek_hip_host_free(v->host);
+    if (first == SAREK_HIP_OK) first = st;
+  } else {
+    std::free(v->host);
+  }
+  delete v;
+  return first;
+}
+
+int64_t sarek_hip_vector_length(sarek_hip_vector v) { return v ? v->length : -1; }
+int64_t sarek_hip_vector_elem_size(sarek_hip_vector v) { return v ? v->elem_size : -1; }
+int sarek_hip_vector_kind(sarek_hip_vector v) { return v ? v->kind : -1; }
+void *sarek_hip_vector_host_ptr(sarek_hip_vector v) { return v ? v->host : nullptr; }
+
+int sarek_hip_vector_location(sarek_hip_vector v, int *location, int *device) {
+  if (!v || !location) return fail(SAREK_HIP_E_INVALID_ARG, "vector_location: NULL argument");
+  *location = v->location;
+  if (device) *device = v->location == SAREK_HIP_LOC_CPU ? -1 : v->device;
+  return SAREK_HIP_OK;
+}
+
+int sarek_hip_vector_device_ptr(sarek_hip_vector v, void **dptr) {
+  if (!v || !dptr) return fail(SAREK_HIP_E_INVALID_ARG, "vector_device_ptr: NULL argument");
+  int dev = 0;
+  int st = current_device(&dev);
+  if (st != SAREK_HIP_OK) return st;
+  auto it = v->buffers.find(dev);
+  *dptr = it == v->buffers.end() ? nullptr : it->second;
+  return SAREK_HIP_OK;
+}
+
+int sarek_hip_vector_set_auto_sync(sarek_hip_vector v, int enabled) {
+  if (!v) return fail(SAREK_HIP_E_INVALID_ARG, "vector_set_auto_sync: NULL vector");
+  v->auto_sync = enabled != 0;
+  return SAREK_HIP_OK;
+}
+
+int sarek_hip_vector_get(sarek_hip_vector v, int64_t index, void *out_elem) {
+  if (!v || !out_elem) return fail(SAREK_HIP_E_INVALID_ARG, "vector_get: NULL argument");
+  if (index < 0 || index >= v->length)
+    return fail(SAREK_HIP_E_INVALID_ARG, "Vector.get: index %lld out of bounds [0, %lld)",
+                static_cast<long long>(index), static_cast<long long>(v->length));
+  int st = ensure_cpu_sync(v);
+  if (st != SAREK_HIP_OK) return st;
+  std::memcpy(out_elem, static_cast<const char *>(v->host) + index * v->elem_size, v->elem_size);
+  return SAREK_HIP_OK;
+}
+
+int sarek_hip_vector_set(sarek_hip_vector v, int64_t index, const void *elem) {
+  if (!v || !elem) return fail(SAREK_HIP_E_INVALID_ARG, "vector_set: NULL argument");
+  if (index < 0 || index >= v->length)
+    return fail(SAREK_HIP_E_INVALID_ARG, "Vector.set: index %lld out of bounds [0, %lld)",
+                static_cast<long long>(index), static_cast<long long>(v->length));
+  std::memcpy(static_cast<char *>(v->host) + index * v->elem_size, elem, v->elem_size);
+  host_written(v);
+  return SAREK_HIP_OK;
+}
+
+int sarek_hip_vector_read(sarek_hip_vector v, void *dst, int64_t first, int64_t count) {
+  if (!v || (!dst && count > 0)) return fail(SAREK_HIP_E_INVALID_ARG, "vector_read: NULL argument");
+  int st = bounds(v, first, count, "get");
+  if (st != SAREK_HIP_OK) return st;
+  st = ensure_cpu_sync(v);
+  if (st != SAREK_HIP_OK) return st;
+  std::memcpy(dst, static_cast<const char *>(v->host) + first * v->elem_size, static_cast<size_t>(count * v->elem_size));
+  return SAREK_HIP_OK;
+}
+
+int sarek_hip_vector_write(sarek_hip_vector v, const void *src, int64_t first, int64_t count) {
+  if (!v || (!src && count > 0)) return fail(SAREK_HIP_E_INVALID_ARG, "vector_write: NULL argument");
+  int st = bounds(v, first, count, "set");
+  if (st != SAREK_HIP_OK) return st;
+  std::memcpy(static_cast<char *>(v->host) + first * v->elem_size, src, static_cast<size_t>(count * v->elem_size));
+  if (count > 0) host_written(v);
+  return SAREK_HIP_OK;
+}
+
+int sarek_hip_transfer_set_auto(int enabled) {
+  g_auto_mode = enabled != 0;
+  return SAREK_HIP_OK;
+}
+
+int sarek_hip_transfer_to_device(sarek_hip_vector v) {
+  if (!v) return fail(SAREK_HIP_E_INVALID_ARG, "to_device: NULL vector");
+  int dev = 0;
+  int st = current_device(&dev);
+  return st != SAREK_HIP_OK ? st : to_device(v, dev);
+}
+
+int sarek_hip_transfer_to_cpu(sarek_hip_vector v, int force) {
+  if (!v) return fail(SAREK_HIP_E_INVALID_ARG, "to_cpu: NULL vector");
+  return to_cpu(v, force != 0);
+}
+
+// Transfer.sync (Transfer.ml:336-350)
+int sarek_hip_transfer_sync(sarek_hip_vector v) {
+  if (!v) return fail(SAREK_HIP_E_INVALID_ARG, "sync: NULL vector");
+  switch (v->location) {
+    case SAREK_HIP_LOC_GPU: case SAREK_HIP_LOC_STALE_CPU: return to_cpu(v, false);
+    case SAREK_HIP_LOC_STALE_GPU: return to_device(v, v->device);
+    default: return SAREK_HIP_OK;
+  }
+}
+
+// Transfer.free_buffer / free_all_buffers (Transfer.ml:353-381)
+int sarek_hip_transfer_free_buffers(sarek_hip_vector v) {
+  if (!v) return fail(SAREK_HIP_E_INVALID_ARG, "free_buffers: NULL vector");
+  int first = SAREK_HIP_OK;
+  for (auto &b : v->buffers) {
+    int st = sarek_hip_mem_free(b.second);
+    if (first == SAREK_HIP_OK) first = st;
+  }
+  v->buffers.clear();
+  v->location = SAREK_HIP_LOC_CPU;
+  v->device = -1;
+  return first;
+}
+
+int sarek_hip_transfer_flush(void) { return sarek_hip_device_synchronize(); }
+
+int sarek_hip_execute_run_vectors(const char *ir_text, const int block[3], const int grid[3], int shared_mem_bytes,
+                                  const sarek_hip_varg *args, int n_args) {
+  if (!ir_text || !block || !grid || n_args < 0 || (n_args > 0 && !args))
+    return fail(SAREK_HIP_E_INVALID_ARG, "run_vectors: NULL or negative argument");
+  int dev = 0;
+  int st = current_device(&dev);
+  if (st != SAREK_HIP_OK) return st;
+  if ((st = transfer_args(args, n_args, dev)) != SAREK_HIP_OK) return st;
+  Lowered k;
+  try {
+    if ((st = lower(ir_text, block, k)) != SAREK_HIP_OK) return st;
+  } catch (const std::exception &e) {
+    return fail(SAREK_HIP_E_PARSE, "run_vectors: %s", e.what());
+  }
+  std::vector<sarek_hip_arg> rs;
+  if ((st = expand_args(args, n_args, dev, true, rs)) != SAREK_HIP_OK) return st;
+  st = sarek_hip_run_source(k.source.c_str(), SAREK_HIP_LANG_HIP_SOURCE, k.name.c_str(), block, grid,
+                            shared_mem_bytes, rs.data(), static_cast<int>(rs.size()));
+  if (st != SAREK_HIP_OK) return st;
+  mark_stale(args, n_args, dev);
+  return SAREK_HIP_OK;
+}
+
+int sarek_hip_execute_run_source(const char *source, int lang, const char *kernel_name, const int block[3],
+                                 const int grid[3], int shared_mem_bytes, int inject_lengths,
+                                 const sarek_hip_varg *args, int n_args) {
+  if (!source || !kernel_name || !block || !grid || n_args < 0 || (n_args > 0 && !args))
+    return fail(SAREK_HIP_E_INVALID_ARG, "run_source: NULL or negative argument");
+  int dev = 0;
+  int st = current_device(&dev);
+  if (st != SAREK_HIP_OK) return st;
+  if ((st = transfer_args(args, n_args, dev)) != SAREK_HIP_OK) return st;
+  std::vector<sarek_hip_arg> rs;
+  if ((st = expand_args(args, n_args, dev, inject_lengths != 0, rs)) != SAREK_HIP_OK) return st;
+  st = sarek_hip_run_source(source, lang, kernel_name, block, grid, shared_mem_bytes, rs.data(),
+                            static_cast<int>(rs.size()));
+  if (st != SAREK_HIP_OK) return st;
+  mark_stale(args, n_args, dev);
+  return SAREK_HIP_OK;
+}
+
+// Execute.sync_vectors_to_cpu
+int sarek_hip_execute_sync_vectors_to_cpu(const sarek_hip_varg *args, int n_args) {
+  if (n_args < 0 || (n_args > 0 && !args)) return fail(SAREK_HIP_E_INVALID_ARG, "sync_vectors_to_cpu: bad arguments");
+  for (int i = 0; i < n_args; ++i)
+    if (args[i].kind == SAREK_HIP_VARG_VEC && args[i].vec) {
+      int st = to_cpu(args[i].vec, false);
+      if (st != SAREK_HIP_OK) return st;
+    }
+  return SAREK_HIP_OK;
+}
+
+}  // extern "C"

@@ -58,6 +58,12 @@ _vp, _i, _i64, _sz, _f = C.c_void_p, C.c_int, C.c_int64, C.c_size_t, C.c_float
 _int3 = C.POINTER(C.c_int)
 _uint3 = C.POINTER(C.c_uint)
 
+class VArg(C.Structure):
+    """sarek_hip_varg: one Execute.vector_arg."""
+    _fields_ = [("kind", C.c_int), ("vec", C.c_void_p), ("i32", C.c_int32), ("i64", C.c_int64),
+                ("f32", C.c_float), ("f64", C.c_double)]
+
+
 # Every symbol include/sarek_hip.h declares: (restype, argtypes).
 SYMBOLS = {
     "sarek_hip_abi_version": (_i, []),
@@ -88,6 +94,8 @@ SYMBOLS = {
     "sarek_hip_event_record": (_i, [_vp, _vp]),
     "sarek_hip_event_synchronize": (_i, [_vp]),
     "sarek_hip_event_elapsed_ms": (_i, [_vp, _vp, C.POINTER(_f)]),
+    "sarek_hip_profiler_start": (_i, []),
+    "sarek_hip_profiler_stop": (_i, []),
     "sarek_hip_kernel_compile": (_i, [C.c_char_p, C.c_char_p, C.POINTER(_vp), C.c_char_p, _sz]),
     "sarek_hip_kernel_compile_cached": (_i, [C.c_char_p, C.c_char_p, C.POINTER(_vp), C.c_char_p, _sz]),
     "sarek_hip_kernel_clear_cache": (_i, []),
@@ -133,6 +141,28 @@ SYMBOLS = {
                                                C.POINTER(_sz)]),
     "sarek_hip_fusion_detect_reduction": (_i, [C.c_char_p, C.POINTER(_i), C.c_char_p, _sz, C.POINTER(_sz)]),
     "sarek_hip_fusion_is_reduction_kernel": (_i, [C.c_char_p, C.c_char_p, C.POINTER(_i), C.c_char_p]),
+    "sarek_hip_vector_create": (_i, [_i, _i64, _i64, _i, C.POINTER(_vp)]),
+    "sarek_hip_vector_destroy": (_i, [_vp]),
+    "sarek_hip_vector_length": (_i64, [_vp]),
+    "sarek_hip_vector_elem_size": (_i64, [_vp]),
+    "sarek_hip_vector_kind": (_i, [_vp]),
+    "sarek_hip_vector_location": (_i, [_vp, C.POINTER(_i), C.POINTER(_i)]),
+    "sarek_hip_vector_host_ptr": (_vp, [_vp]),
+    "sarek_hip_vector_device_ptr": (_i, [_vp, C.POINTER(_vp)]),
+    "sarek_hip_vector_set_auto_sync": (_i, [_vp, _i]),
+    "sarek_hip_vector_get": (_i, [_vp, _i64, _vp]),
+    "sarek_hip_vector_set": (_i, [_vp, _i64, _vp]),
+    "sarek_hip_vector_read": (_i, [_vp, _vp, _i64, _i64]),
+    "sarek_hip_vector_write": (_i, [_vp, _vp, _i64, _i64]),
+    "sarek_hip_transfer_set_auto": (_i, [_i]),
+    "sarek_hip_transfer_to_device": (_i, [_vp]),
+    "sarek_hip_transfer_to_cpu": (_i, [_vp, _i]),
+    "sarek_hip_transfer_sync": (_i, [_vp]),
+    "sarek_hip_transfer_free_buffers": (_i, [_vp]),
+    "sarek_hip_transfer_flush": (_i, []),
+    "sarek_hip_execute_run_vectors": (_i, [C.c_char_p, _int3, _int3, _i, C.POINTER(VArg), _i]),
+    "sarek_hip_execute_run_source": (_i, [C.c_char_p, _i, C.c_char_p, _int3, _int3, _i, _i, C.POINTER(VArg), _i]),
+    "sarek_hip_execute_sync_vectors_to_cpu": (_i, [C.POINTER(VArg), _i]),
     "sarek_hip_set_tunable": (_i, [C.c_char_p, _i64]),
     "sarek_hip_set_clock_probe": (_i, [_vp, _i64, C.POINTER(_i64)]),
 }

@@ -1,0 +1,238 @@
+"""`Vector`, `Transfer` and `Execute` by the reference's names (sarek/core/Vector.ml,
+sarek/core/Transfer.ml, sarek/sarek/Execute.ml), over the native host layer of libsarek_hip:
+a program written against them reads like the OCaml it mirrors,
+
+    a = Vector.create(Vector.float32, n)
+    for i in range(n): a[i] = ...                      # Vector.set
+    Execute.run_vectors(ir=kernel_ir, args=[Execute.Vec(a), Execute.Int(n)],
+                        block=Execute.dims1d(256), grid=Execute.dims1d((n + 255) // 256))
+    Transfer.flush()
+    result = a.to_array()                              # downloads: the launch left `a` Stale_CPU
+
+Location states, what moves when, and the error texts are the native layer's, which follows
+the reference state by state.
+"""
+import ctypes as C
+
+import numpy as np
+
+from . import hip
+
+CPU, GPU, Both, Stale_CPU, Stale_GPU = "CPU", "GPU", "Both", "Stale_CPU", "Stale_GPU"
+_LOCATIONS = (CPU, GPU, Both, Stale_CPU, Stale_GPU)
+
+
+class _Kind:
+    def __init__(self, code, name, dtype):
+        self.code, self.name, self.dtype = code, name, np.dtype(dtype) if dtype is not None else None
+
+    def __repr__(self):
+        return self.name
+
+
+class Vector:
+    """sarek/core/Vector.ml; a host block, per-device buffers, a location."""
+    float32 = _Kind(0, "Float32", np.float32)
+    float64 = _Kind(1, "Float64", np.float64)
+    int32 = _Kind(2, "Int32", np.int32)
+    int64 = _Kind(3, "Int64", np.int64)
+    char = _Kind(4, "Char", np.uint8)
+    complex32 = _Kind(5, "Complex32", np.complex64)
+
+    def __init__(self, handle, kind):
+        self._h, self._kind = handle, kind
+
+    # -- creation (Vector_storage.create / create_custom / of_array) --
+    @classmethod
+    def create(cls, kind, length, pinned=False):
+        h = C.c_void_p()
+        hip.check(hip.lib.sarek_hip_vector_create(kind.code, length, 0, int(pinned), C.byref(h)))
+        return cls(h, kind)
+
+    @classmethod
+    def create_custom(cls, elem_size, length, pinned=False):
+        h = C.c_void_p()
+        hip.check(hip.lib.sarek_hip_vector_create(6, length, elem_size, int(pinned), C.byref(h)))
+        return cls(h, _Kind(6, f"Custom({elem_size})", np.dtype((np.void, elem_size))))
+
+    @classmethod
+    def of_array(cls, array, kind=None, pinned=False):
+        array = np.ascontiguousarray(array)
+        kind = kind or next(k for k in (cls.float32, cls.float64, cls.int32, cls.int64, cls.char, cls.complex32)
+                            if k.dtype == array.dtype)
+        v = cls.create(kind, array.size, pinned)
+        v.host[:] = array.reshape(-1).astype(kind.dtype, copy=False)      # straight into the host block: stays CPU
+        return v
+
+    def destroy(self):
+        if self._h is not None:
+            hip.check(hip.lib.sarek_hip_vector_destroy(self._h))
+            self._h = None
+
+    def __del__(self):                  # the reference frees device buffers from a GC finaliser
+        try:
+            self.destroy()
+        except Exception:
+            pass
+
+    # -- accessors --
+    @property
+    def length(self):
+        return hip.lib.sarek_hip_vector_length(self._h)
+
+    def __len__(self):
+        return self.length
+
+    @property
+    def kind(self):
+        return self._kind
+
+    @property
+    def location(self):
+        loc = C.c_int(0)
+        hip.check(hip.lib.sarek_hip_vector_location(self._h, C.byref(loc), None))
+        return _LOCATIONS[loc.value]
+
+    @property
+    def host(self):
+        """The raw host block as a numpy view (Vector.host_ptr): no sync, no location update."""
+        n = self.length
+        ptr = hip.lib.sarek_hip_vector_host_ptr(self._h)
+        if n == 0:
+            return np.empty(0, dtype=self._kind.dtype)
+        buf = (C.c_char * (n * self._kind.dtype.itemsize)).from_address(ptr)
+        return np.frombuffer(buf, dtype=self._kind.dtype, count=n)
+
+    @property
+    def device_ptr(self):
+        p = C.c_void_p()
+        hip.check(hip.lib.sarek_hip_vector_device_ptr(self._h, C.byref(p)))
+        return p.value
+
+    def set_auto_sync(self, enabled):
+        hip.check(hip.lib.sarek_hip_vector_set_auto_sync(self._h, int(enabled)))
+
+    # -- element access (Vector.get / Vector.set) --
+    def get(self, index):
+        out = np.empty(1, dtype=self._kind.dtype)
+        st = hip.lib.sarek_hip_vector_get(self._h, index, C.c_void_p(out.ctypes.data))
+        if st == hip.E_INVALID_ARG:
+            raise IndexError(hip.lib.sarek_hip_last_error().decode())      # Invalid_argument in the reference
+        hip.check(st)
+        return out[0]
+
+    def set(self, index, value):
+        elem = np.asarray([value], dtype=self._kind.dtype)
+        st = hip.lib.sarek_hip_vector_set(self._h, index, C.c_void_p(elem.ctypes.data))
+        if st == hip.E_INVALID_ARG:
+            raise IndexError(hip.lib.sarek_hip_last_error().decode())
+        hip.check(st)
+
+    __getitem__ = get
+    __setitem__ = set
+
+    def to_array(self):
+        """Vector.to_array: a fresh array; downloads first when the host copy is stale."""
+        out = np.empty(self.length, dtype=self._kind.dtype)
+        hip.check(hip.lib.sarek_hip_vector_read(self._h, C.c_void_p(out.ctypes.data), 0, out.size))
+        return out
+
+    def fill_from(self, array, first=0):
+        """A loop of Vector.set over a range, in one call."""
+        array = np.ascontiguousarray(array, dtype=self._kind.dtype)
+        st = hip.lib.sarek_hip_vector_write(self._h, C.c_void_p(array.ctypes.data), first, array.size)
+        if st == hip.E_INVALID_ARG:
+            raise IndexError(hip.lib.sarek_hip_last_error().decode())
+        hip.check(st)
+
+
+class Transfer:
+    """sarek/core/Transfer.ml (the device is the current one)."""
+
+    @staticmethod
+    def to_device(vec):
+        hip.check(hip.lib.sarek_hip_transfer_to_device(vec._h))
+
+    @staticmethod
+    def to_cpu(vec, force=False):
+        hip.check(hip.lib.sarek_hip_transfer_to_cpu(vec._h, int(force)))
+
+    @staticmethod
+    def sync(vec):
+        hip.check(hip.lib.sarek_hip_transfer_sync(vec._h))
+
+    @staticmethod
+    def free_all_buffers(vec):
+        hip.check(hip.lib.sarek_hip_transfer_free_buffers(vec._h))
+
+    @staticmethod
+    def flush():
+        hip.check(hip.lib.sarek_hip_transfer_flush())
+
+    @staticmethod
+    def set_auto(enabled):
+        hip.check(hip.lib.sarek_hip_transfer_set_auto(int(enabled)))
+
+
+class Execute:
+    """sarek/sarek/Execute.ml: vector_arg constructors, run_vectors, run_source."""
+
+    @staticmethod
+    def Vec(v): return ("vec", v)
+    @staticmethod
+    def Int(n): return ("i32", int(n))          # expand_to_run_source_args sends Int as Int32
+    @staticmethod
+    def Int32(n): return ("i32", int(n))
+    @staticmethod
+    def Int64(n): return ("i64", int(n))
+    @staticmethod
+    def Float32(x): return ("f32", float(x))
+    @staticmethod
+    def Float64(x): return ("f64", float(x))
+
+    @staticmethod
+    def dims1d(x): return (x, 1, 1)
+    @staticmethod
+    def dims2d(x, y): return (x, y, 1)
+    @staticmethod
+    def dims3d(x, y, z): return (x, y, z)
+
+    @staticmethod
+    def _args(args):
+        out = (hip.VArg * max(len(args), 1))()
+        for a, (kind, v) in zip(out, args):
+            if kind == "vec":
+                a.kind, a.vec = 0, v._h
+            elif kind == "i32":
+                a.kind, a.i32 = 1, v
+            elif kind == "i64":
+                a.kind, a.i64 = 2, v
+            elif kind == "f32":
+                a.kind, a.f32 = 3, v
+            elif kind == "f64":
+                a.kind, a.f64 = 4, v
+            else:
+                raise ValueError(f"unknown vector_arg {kind!r}")
+        return out, len(args)
+
+    @staticmethod
+    def run_vectors(ir, args, block, grid, shared_mem=0):
+        """Execute.run_vectors ~ir ~args ~block ~grid ?shared_mem (); returns the code path that
+        served the launch ("jit" or a hand kernel's tag)."""
+        a, n = Execute._args(args)
+        hip.check(hip.lib.sarek_hip_execute_run_vectors(ir.encode(), (C.c_int * 3)(*block), (C.c_int * 3)(*grid),
+                                                        shared_mem, a, n))
+        return hip.lib.sarek_hip_last_run_path().decode()
+
+    @staticmethod
+    def run_source(source, kernel_name, block, grid, args, lang=hip.LANG_HIP, shared_mem=0, inject_lengths=True):
+        a, n = Execute._args(args)
+        hip.check(hip.lib.sarek_hip_execute_run_source(source.encode(), lang, kernel_name.encode(),
+                                                       (C.c_int * 3)(*block), (C.c_int * 3)(*grid), shared_mem,
+                                                       int(inject_lengths), a, n))
+        return hip.lib.sarek_hip_last_run_path().decode()
+
+    @staticmethod
+    def sync_vectors_to_cpu(args):
+        a, n = Execute._args(args)
+        hip.check(hip.lib.sarek_hip_execute_sync_vectors_to_cpu(a, n))

@@ -77,6 +77,10 @@ def test_runtime_events_and_streams(hip, torch_cuda):
     hip.check(hip.lib.sarek_hip_event_destroy(e0))
     hip.check(hip.lib.sarek_hip_event_destroy(e1))
     hip.check(hip.lib.sarek_hip_stream_destroy(s))
+    # enable_profiling / disable_profiling: never an error, with or without a profiler attached
+    assert hip.lib.sarek_hip_profiler_start() == 0 and hip.lib.sarek_hip_profiler_stop() == 0
+    a = torch_cuda.ones(1024, device="cuda")
+    assert float(hip.triad(a, a, 2.0).sum().item()) == 3072.0     # the runtime is left in working order
 
 
 def test_run_source_external_kernel(hip, torch_cuda):

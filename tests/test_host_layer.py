@@ -1,0 +1,194 @@
+"""Vector / Transfer / Execute above the plugin boundary (sarek/core/Vector.ml,
+sarek/core/Transfer.ml, sarek/sarek/Execute.ml): host-only behaviour on the CPU, the location
+state machine and the dispatcher on the GPU, each step checked against what the reference's
+code does in that state."""
+import numpy as np
+import pytest
+
+from spoc_amd import reference_kernels
+from spoc_amd.sarek import CPU, Both, Execute, Stale_CPU, Stale_GPU, Transfer, Vector
+
+gpu = pytest.mark.gpu
+
+
+# ---- host only --------------------------------------------------------------------------------
+
+def test_create_get_set_and_bounds():
+    v = Vector.create(Vector.float32, 10)
+    assert v.length == 10 and len(v) == 10 and v.kind is Vector.float32 and v.location == CPU
+    for i in range(10):
+        v[i] = i * 0.5                                    # Vector.set
+    assert v.location == CPU                              # a host-only vector stays CPU (Vector.ml:104-109)
+    assert v[3] == np.float32(1.5) and v.get(9) == np.float32(4.5)
+    assert np.array_equal(v.to_array(), np.arange(10, dtype=np.float32) * 0.5)
+    with pytest.raises(IndexError, match=r"Vector.get: index 10 out of bounds \[0, 10\)"):      # Vector.ml:82-88
+        v.get(10)
+    with pytest.raises(IndexError, match=r"Vector.set: index -1 out of bounds \[0, 10\)"):      # Vector.ml:97-103
+        v.set(-1, 0.0)
+    with pytest.raises(IndexError):
+        v.fill_from(np.zeros(4), first=8)
+    v.destroy()
+    v.destroy()                                           # idempotent, like the GC finaliser after an explicit free
+
+
+@pytest.mark.parametrize("kind,size,value", [
+    (Vector.float32, 4, 1.25), (Vector.float64, 8, 1e-300), (Vector.int32, 4, -7), (Vector.int64, 8, 1 << 40),
+    (Vector.char, 1, 200), (Vector.complex32, 8, 1 + 2j)])
+def test_kinds_and_element_sizes(kind, size, value):
+    from spoc_amd import hip
+    v = Vector.create(kind, 3)
+    assert hip.lib.sarek_hip_vector_elem_size(v._h) == size      # Vector_types.scalar_elem_size
+    v[1] = value
+    assert v[1] == kind.dtype.type(value)
+    assert v.host.dtype == kind.dtype and v.host.size == 3
+
+
+def test_custom_and_empty_vectors_and_bad_arguments():
+    from spoc_amd import hip
+    c = Vector.create_custom(12, 5)
+    assert hip.lib.sarek_hip_vector_elem_size(c._h) == 12 and c.host.nbytes == 60
+    e = Vector.create(Vector.int32, 0)
+    assert e.length == 0 and e.to_array().size == 0
+    with pytest.raises(hip.SarekHipError):
+        Vector.create(Vector.float32, -1)
+    with pytest.raises(hip.SarekHipError):
+        Vector.create_custom(0, 4)
+
+
+def test_of_array_writes_the_host_block_directly():
+    x = np.arange(6, dtype=np.int32)
+    v = Vector.of_array(x)
+    assert v.kind is Vector.int32 and v.location == CPU and np.array_equal(v.to_array(), x)
+
+
+# ---- the location state machine on the device ---------------------------------------------------
+
+@gpu
+def test_location_walk(torch_cuda):
+    n = 1000
+    v = Vector.create(Vector.float32, n)
+    v.fill_from(np.arange(n))
+    assert v.location == CPU and v.device_ptr is None
+    Transfer.to_device(v)                                  # CPU -> Both (Transfer.ml:245-268)
+    assert v.location == Both and v.device_ptr is not None
+    ptr = v.device_ptr
+    v.host[0] = -1.0                                       # behind the vector's back: nothing is tracked
+    Transfer.to_device(v)                                  # Both: skipped (Transfer.ml:241-243)
+    assert v.location == Both and v.device_ptr == ptr
+    Transfer.to_cpu(v)                                     # Both without force: nothing moves (:289)
+    assert v.host[0] == -1.0
+    Transfer.to_cpu(v, force=True)                         # forced: the device copy comes back
+    assert v.host[0] == 0.0 and v.location == Both
+    v[5] = 55.0                                            # Vector.set on Both -> Stale_GPU (Vector.ml:106-107)
+    assert v.location == Stale_GPU
+    Transfer.to_cpu(v)                                     # Stale_GPU: the host copy is the good one (:290)
+    assert v[5] == 55.0 and v.location == Stale_GPU
+    Transfer.to_device(v)                                  # Stale_GPU -> upload again -> Both
+    assert v.location == Both
+    Transfer.to_cpu(v, force=True)
+    assert v[5] == 55.0
+    Transfer.free_all_buffers(v)                           # Transfer.ml:371-381
+    assert v.location == CPU and v.device_ptr is None and v[5] == 55.0
+
+
+@gpu
+def test_launch_marks_stale_and_reads_download(torch_cuda):
+    n = 100003
+    b, c = Vector.create(Vector.float32, n), Vector.create(Vector.float32, n)
+    a = Vector.create(Vector.float32, n)
+    b.fill_from(np.arange(n) % 100 / 100.0)
+    c.fill_from((np.arange(n) + 1) % 100 / 100.0)
+    ir = reference_kernels.stream_triad()
+    args = [Execute.Vec(a), Execute.Vec(b), Execute.Vec(c), Execute.Float32(3.0), Execute.Int(n)]
+    block, grid = Execute.dims1d(256), Execute.dims1d((n + 255) // 256)
+    path = Execute.run_vectors(ir=ir, args=args, block=block, grid=grid)
+    assert path == "stream_triad_f32"
+    # every vector argument was uploaded (Both) and is now Stale_CPU, inputs included (Execute.ml:321-335)
+    assert a.location == b.location == c.location == Stale_CPU
+    Transfer.flush()
+    expected = (b.host.astype(np.float64) + 3.0 * c.host.astype(np.float64)).astype(np.float32)
+    assert a[7] == expected[7]                             # Vector.get downloads (ensure_cpu_sync) ...
+    assert a.location == Both                              # ... and leaves Both (Transfer.ml:322)
+    assert np.array_equal(a.to_array(), expected)
+    # second launch: nothing to upload, same buffers
+    pa, pb = a.device_ptr, b.device_ptr
+    Execute.run_vectors(ir=ir, args=args, block=block, grid=grid)
+    assert (a.device_ptr, b.device_ptr) == (pa, pb) and a.location == Stale_CPU
+    assert b.location == Stale_CPU                         # b was never read back, so it was not Both: unchanged
+    # a host write into a Stale_CPU vector is not tracked and is lost at the next download
+    b[0] = 123.0
+    assert b.location == Stale_CPU                         # Vector.ml:108-109
+    Transfer.to_cpu(b)
+    assert b[0] == np.float32(0.0) and b.location == Both
+    # after a tracked write the next launch uploads again
+    c[0] = 0.5
+    assert c.location == Stale_CPU                         # still never synced: Stale_CPU stays
+    Transfer.to_cpu(c)
+    c[0] = 0.5
+    assert c.location == Stale_GPU
+    Execute.run_vectors(ir=ir, args=args, block=block, grid=grid)
+    assert c.location == Stale_CPU and a[0] == np.float32(b[0] + 3.0 * 0.5)
+
+
+@gpu
+def test_auto_sync_switches(torch_cuda):
+    n = 4096
+    x, y = Vector.create(Vector.float32, n), Vector.create(Vector.float32, n)
+    x.fill_from(np.ones(n))
+    y.fill_from(np.zeros(n))
+    args = [Execute.Vec(x), Execute.Vec(y), Execute.Int(n)]
+    Execute.run_vectors(ir=reference_kernels.vector_copy(), args=args, block=(256, 1, 1), grid=(16, 1, 1))
+    Transfer.flush()
+    try:
+        Transfer.set_auto(False)                           # Transfer.auto_mode off: reads see the stale block
+        assert y[0] == 0.0 and y.location == Stale_CPU
+        Transfer.set_auto(True)
+        y.set_auto_sync(False)                             # per-vector switch (Vector_types.auto_sync)
+        assert y[0] == 0.0 and y.location == Stale_CPU
+        y.set_auto_sync(True)
+        assert y[0] == 1.0 and y.location == Both
+    finally:
+        Transfer.set_auto(True)
+    Execute.run_vectors(ir=reference_kernels.vector_copy(), args=args, block=(256, 1, 1), grid=(16, 1, 1))
+    Execute.sync_vectors_to_cpu(args)                      # Execute.ml:546-547
+    assert x.location == Both and y.location == Both
+    Transfer.sync(y)
+    assert y.location == Both
+
+
+@gpu
+def test_run_source_external_kernel_with_and_without_lengths(torch_cuda):
+    """sarek/tests/e2e/test_external_kernel.ml:46-62: a hand-written kernel through Execute.run_source."""
+    n = 1000
+    a, b, c = (Vector.create(Vector.float32, n) for _ in range(3))
+    a.fill_from(np.arange(n))
+    b.fill_from(np.arange(n) * 2)
+    with_len = ('extern "C" __global__ void vadd(const float* a, int al, const float* b, int bl, float* c, int cl, int n) '
+                '{ int i = threadIdx.x + blockIdx.x * blockDim.x; if (i < n && i < cl) c[i] = a[i] + b[i]; }')
+    bare = ('extern "C" __global__ void vadd(const float* a, const float* b, float* c, int n) '
+            '{ int i = threadIdx.x + blockIdx.x * blockDim.x; if (i < n) c[i] = a[i] + b[i] + 1.0f; }')
+    args = [Execute.Vec(a), Execute.Vec(b), Execute.Vec(c), Execute.Int32(n)]
+    assert Execute.run_source(with_len, "vadd", (256, 1, 1), (4, 1, 1), args) == "jit"
+    assert c.location == Stale_CPU and np.array_equal(c.to_array(), np.arange(n, dtype=np.float32) * 3)
+    Execute.run_source(bare, "vadd", (256, 1, 1), (4, 1, 1), args, inject_lengths=False)
+    assert np.array_equal(c.to_array(), np.arange(n, dtype=np.float32) * 3 + 1)
+    from spoc_amd import hip
+    with pytest.raises(hip.SarekHipError, match="does not support PTX"):           # Cuda_plugin.ml:211-220
+        Execute.run_source(bare, "vadd", (256, 1, 1), (4, 1, 1), args, lang=hip.LANG_PTX)
+
+
+@gpu
+def test_lowering_failure_and_pinned_vectors(torch_cuda):
+    from spoc_amd import hip
+    v = Vector.create(Vector.float32, 8, pinned=True)
+    v.fill_from(np.arange(8))
+    with pytest.raises(hip.SarekHipError, match="Backend failed to generate source"):      # Execute.ml:257-263
+        Execute.run_vectors(ir="(kernel k (params) (locals) (body (frob)))", args=[Execute.Vec(v)],
+                            block=(1, 1, 1), grid=(1, 1, 1))
+    assert v.location == Both                              # the upload had happened before the lowering failed
+    big = Vector.create(Vector.float32, 1 << 22, pinned=True)
+    big.fill_from(np.arange(1 << 22) % 977)
+    out = Vector.create(Vector.float32, 1 << 22, pinned=True)
+    Execute.run_vectors(ir=reference_kernels.vector_copy(), args=[Execute.Vec(big), Execute.Vec(out), Execute.Int(1 << 22)],
+                        block=(256, 1, 1), grid=((1 << 22) // 256, 1, 1))
+    assert np.array_equal(out.to_array(), big.host)
