@@ -7,10 +7,11 @@ bench_scan.ml: same inputs, same
 launch geometry, same warmup / timed-iteration protocol (wall clock around the launch plus
 the device flush, one sample per iteration), same verification and tolerance, same
 throughput formula and statistic, and the same per-device result record
-(benchmarks/output.ml:16-28).  Each launch goes the way Execute.run_vectors sends it:
-generate_source on the kernel's IR, then run_source with the vectors expanded to
-(buffer, length) pairs; the plugin decides whether a hand-written kernel or the JIT-compiled
-lowering serves it (reported as `path`).
+(benchmarks/output.ml:16-28).  The programs are written against Vector / Execute / Transfer
+(spoc_amd/sarek.py) as the originals are: Vector.create + Vector.set for the inputs,
+Execute.run_vectors ~ir ~args ~block ~grid per launch, Transfer.flush, Vector.to_array for the
+check; the plugin decides whether a hand-written kernel or the JIT-compiled lowering serves a
+launch (reported as `path`).
 
     python -m spoc_amd.benchmarks matrix_mul_tiled --sizes 1024,4096
     python -m spoc_amd.benchmarks all --json out.json
@@ -23,6 +24,7 @@ import time
 import numpy as np
 
 from . import hip, reference_kernels
+from .sarek import Execute, Transfer, Vector
 
 
 def _stats(times_ms):
@@ -34,17 +36,16 @@ def _stats(times_ms):
 
 def _time_launches(launch, warmup, iterations):
     """benchmarks/bench_stream_triad.ml:76-116: warmup launches, then one wall-clock sample
-    per launch + flush."""
-    sync = hip.lib.sarek_hip_device_synchronize
+    per Execute.run_vectors + Transfer.flush."""
     path = None
     for _ in range(warmup):
         path = launch()
-        hip.check(sync())
+        Transfer.flush()
     times = []
     for _ in range(iterations):
         t0 = time.perf_counter()
         path = launch()
-        hip.check(sync())
+        Transfer.flush()
         times.append((time.perf_counter() - t0) * 1e3)
     return times, path
 
@@ -59,20 +60,12 @@ def _device_record(times, throughput, verified, path, unit):
     return rec
 
 
-def _upload(torch, array):
-    """Transfer.to_device (sarek/core/Transfer.ml:228-268): the vector's host block goes up
-    through Memory.host_ptr_to_device; torch only owns the device block."""
-    host = np.ascontiguousarray(array, dtype=np.float32)
-    dev = torch.empty(host.size, dtype=torch.float32, device="cuda")
-    hip.memcpy_htod(dev.data_ptr(), host)
-    return dev
-
-
-def _download(tensor):
-    """Transfer.to_cpu (sarek/core/Transfer.ml:274-333) through Memory.device_to_host_ptr."""
-    host = np.empty(tensor.numel(), dtype=np.float32)
-    hip.memcpy_dtoh(host, tensor.data_ptr())
-    return host
+def _vector(array, kind=None):
+    """Vector.create + a loop of Vector.set, as the benches fill their inputs (in one call)."""
+    kind = kind or Vector.float32
+    v = Vector.create(kind, len(array))
+    v.fill_from(array)
+    return v
 
 
 def bench_matrix_mul_tiled(size, warmup=5, iterations=20, tile_size=16):
@@ -85,22 +78,20 @@ def bench_matrix_mul_tiled(size, warmup=5, iterations=20, tile_size=16):
     f32 sum add up with one sign (sequential f32 as in the generated kernel, the vendor
     library and this backend all end 4.7e-3 off at 2048 and 1.1e-2 off at 4096, where the
     sums reach 1000)."""
-    import torch
     m = n = k = size
     a = (np.arange(m * k) % 10) / 10.0
     b = ((np.arange(k * n) + 1) % 10) / 10.0
     expected = a.reshape(m, k) @ b.reshape(k, n)              # float64, as ocaml_matmul
-    va, vb = _upload(torch, a), _upload(torch, b)
-    vc = torch.empty(m * n, dtype=torch.float32, device="cuda")   # Vector.create: uninitialised
-    src = hip.generate_source(reference_kernels.matrix_mul_tiled(), block=(tile_size, tile_size, 1))
-    grid = ((n + tile_size - 1) // tile_size, (m + tile_size - 1) // tile_size, 1)
-    args = [va, vb, vc, ("i32", m), ("i32", n), ("i32", k)]
-
-    def launch():
-        return hip.run_source(src, "sarek_kern", (tile_size, tile_size, 1), grid, args,
-                              shared_mem=2 * tile_size * tile_size * 4)
-    times, path = _time_launches(launch, warmup, iterations)
-    verified = bool(np.all(np.abs(_download(vc).astype(np.float64).reshape(m, n) - expected) <= 1e-3))
+    va, vb = _vector(a), _vector(b)
+    vc = Vector.create(Vector.float32, m * n)                 # never zeroed, as in the reference
+    ir = reference_kernels.matrix_mul_tiled()
+    block = Execute.dims2d(tile_size, tile_size)
+    grid = Execute.dims2d((n + tile_size - 1) // tile_size, (m + tile_size - 1) // tile_size)
+    args = [Execute.Vec(va), Execute.Vec(vb), Execute.Vec(vc), Execute.Int(m), Execute.Int(n), Execute.Int(k)]
+    times, path = _time_launches(
+        lambda: Execute.run_vectors(ir=ir, args=args, block=block, grid=grid, shared_mem=2 * tile_size * tile_size * 4),
+        warmup, iterations)
+    verified = bool(np.all(np.abs(vc.to_array().astype(np.float64).reshape(m, n) - expected) <= 1e-3))
     gflops = 2.0 * m * n * k / (statistics.median(times) * 1e6)
     return _device_record(times, gflops, verified, path, "GFLOPS")
 
@@ -108,34 +99,31 @@ def bench_matrix_mul_tiled(size, warmup=5, iterations=20, tile_size=16):
 def bench_stream_triad(size, warmup=5, iterations=20, block_size=256):
     """benchmarks/bench_stream_triad.ml:35-181: b[i] = (i mod 100)/100, c[i] = ((i+1) mod 100)/100,
     scalar 3, every element within 1e-5, GB/s = 12 n / median."""
-    import torch
     n = size
     b = (np.arange(n) % 100) / 100.0
     c = ((np.arange(n) + 1) % 100) / 100.0
     expected = b + c * 3.0
-    va = torch.empty(n, dtype=torch.float32, device="cuda")
-    vb, vc = _upload(torch, b), _upload(torch, c)
-    src = hip.generate_source(reference_kernels.stream_triad(), block=(block_size, 1, 1))
-    grid = ((n + block_size - 1) // block_size, 1, 1)
-    args = [va, vb, vc, ("f32", 3.0), ("i32", n)]
-    times, path = _time_launches(lambda: hip.run_source(src, "sarek_kern", (block_size, 1, 1), grid, args),
+    va, vb, vc = Vector.create(Vector.float32, n), _vector(b), _vector(c)
+    ir = reference_kernels.stream_triad()
+    block, grid = Execute.dims1d(block_size), Execute.dims1d((n + block_size - 1) // block_size)
+    args = [Execute.Vec(va), Execute.Vec(vb), Execute.Vec(vc), Execute.Float32(3.0), Execute.Int(n)]
+    times, path = _time_launches(lambda: Execute.run_vectors(ir=ir, args=args, block=block, grid=grid),
                                  warmup, iterations)
-    verified = bool(np.all(np.abs(_download(va).astype(np.float64) - expected) <= 1e-5))
+    verified = bool(np.all(np.abs(va.to_array().astype(np.float64) - expected) <= 1e-5))
     gbs = 3.0 * n * 4.0 / (statistics.median(times) / 1e3 * 1e9)
     return _device_record(times, gbs, verified, path, "GB/s")
 
 
 def _tree_bench(ir, inputs, n, expected, check, bytes_moved, stat, warmup, iterations, fold=np.sum):
-    import torch
     nblocks = (n + 255) // 256
-    vins = [_upload(torch, x) for x in inputs]
-    vout = torch.zeros(nblocks, dtype=torch.float32, device="cuda")
-    src = hip.generate_source(ir, block=(256, 1, 1))
-    args = vins + [vout, ("i32", n)]
+    vins = [_vector(x) for x in inputs]
+    vout = Vector.create(Vector.float32, nblocks)
+    args = [Execute.Vec(v) for v in vins] + [Execute.Vec(vout), Execute.Int(n)]
     times, path = _time_launches(
-        lambda: hip.run_source(src, "sarek_kern", (256, 1, 1), (nblocks, 1, 1), args, shared_mem=1024),
+        lambda: Execute.run_vectors(ir=ir, args=args, block=Execute.dims1d(256), grid=Execute.dims1d(nblocks),
+                                    shared_mem=1024),
         warmup, iterations)
-    result = float(fold(_download(vout).astype(np.float64)))   # host fold over the partials
+    result = float(fold(vout.to_array().astype(np.float64)))   # host fold over the partials
     verified = check(result, expected)
     t = statistics.mean(times) if stat == "mean" else statistics.median(times)
     return _device_record(times, bytes_moved / (t / 1e3) / 1e9, verified, path, "GB/s")
@@ -168,124 +156,120 @@ def bench_reduction_max(size, warmup=5, iterations=20):
                        lambda r, e: abs(r - e) < 1e-5, 4.0 * n, "median", warmup, iterations, fold=np.max)
 
 
-def _benchmark_gpu(launch, warmup, iterations):
-    """benchmarks/common.ml:200-237 (Common.benchmark_gpu): one launch to compile, `warmup`
-    launches, then `iterations` samples of device-idle -> launch -> device-idle."""
-    sync = hip.lib.sarek_hip_device_synchronize
-    path = launch()
-    hip.check(sync())
+def _benchmark_gpu(init, compute, warmup, iterations):
+    """benchmarks/common.ml:200-237 (Common.benchmark_gpu): vectors from init (), one launch to
+    compile, `warmup` launches, FRESH vectors from init () again, then `iterations` samples of
+    device-idle -> launch -> device-idle.  The fresh vectors are uploaded inside the first timed
+    sample, in the reference as here (its statistics are the mean or the minimum of the samples)."""
+    kernel_args = init()
+    path = compute(kernel_args)
+    Transfer.flush()
     for _ in range(warmup):
-        launch()
-        hip.check(sync())
+        compute(kernel_args)
+        Transfer.flush()
+    kernel_args = init()
     times = []
     for _ in range(iterations):
-        hip.check(sync())
+        Transfer.flush()
         t0 = time.perf_counter()
-        path = launch()
-        hip.check(sync())
+        path = compute(kernel_args)
+        Transfer.flush()
         times.append((time.perf_counter() - t0) * 1e3)
-    return times, path
+    return times, path, kernel_args
 
 
 def bench_vector_add(size, warmup=10, iterations=20):
     """benchmarks/bench_vector_add.ml:53-150: a[i] = 0.001 i, b[i] = 0.002 i, every element within
     1e-3 of the double sum, GB/s = 12 n / MINIMUM time."""
-    import torch
     n = size
     a, b = np.arange(n) * 0.001, np.arange(n) * 0.002
-    va, vb = _upload(torch, a), _upload(torch, b)
-    vc = torch.empty(n, dtype=torch.float32, device="cuda")
-    src = hip.generate_source(reference_kernels.vector_add(), block=(256, 1, 1))
-    grid = ((n + 255) // 256, 1, 1)
-    args = [va, vb, vc, ("i32", n)]
-    times, path = _benchmark_gpu(lambda: hip.run_source(src, "sarek_kern", (256, 1, 1), grid, args),
-                                 warmup, iterations)
-    verified = bool(np.all(np.abs(_download(vc).astype(np.float64) - (a + b)) <= 1e-3))
+    ir = reference_kernels.vector_add()
+    block, grid = Execute.dims1d(256), Execute.dims1d((n + 255) // 256)
+
+    def compute(v):
+        return Execute.run_vectors(ir=ir, args=[Execute.Vec(v[0]), Execute.Vec(v[1]), Execute.Vec(v[2]), Execute.Int(n)],
+                                   block=block, grid=grid)
+    times, path, (_, _, vc) = _benchmark_gpu(lambda: (_vector(a), _vector(b), Vector.create(Vector.float32, n)),
+                                             compute, warmup, iterations)
+    verified = bool(np.all(np.abs(vc.to_array().astype(np.float64) - (a + b)) <= 1e-3))
     return _device_record(times, 12.0 * n / (min(times) / 1e3) / 1e9, verified, path, "GB/s")
 
 
 def bench_vector_copy(size, warmup=5, iterations=20, block_size=256):
     """benchmarks/bench_vector_copy.ml:21-170: a[i] = (i mod 100)/100, every element within 1e-6,
     GB/s = 8 n / median (launch + flush per sample)."""
-    import torch
     n = size
     a = (np.arange(n) % 100) / 100.0
-    va = _upload(torch, a)
-    vb = torch.empty(n, dtype=torch.float32, device="cuda")
-    src = hip.generate_source(reference_kernels.vector_copy(), block=(block_size, 1, 1))
-    grid = ((n + block_size - 1) // block_size, 1, 1)
-    args = [va, vb, ("i32", n)]
-    times, path = _time_launches(lambda: hip.run_source(src, "sarek_kern", (block_size, 1, 1), grid, args),
+    va, vb = _vector(a), Vector.create(Vector.float32, n)
+    ir = reference_kernels.vector_copy()
+    block, grid = Execute.dims1d(block_size), Execute.dims1d((n + block_size - 1) // block_size)
+    args = [Execute.Vec(va), Execute.Vec(vb), Execute.Int(n)]
+    times, path = _time_launches(lambda: Execute.run_vectors(ir=ir, args=args, block=block, grid=grid),
                                  warmup, iterations)
-    verified = bool(np.all(np.abs(_download(vb).astype(np.float64) - a) <= 1e-6))
+    verified = bool(np.all(np.abs(vb.to_array().astype(np.float64) - a) <= 1e-6))
     return _device_record(times, 8.0 * n / (statistics.median(times) / 1e3) / 1e9, verified, path, "GB/s")
 
 
 def bench_matrix_mul(size, warmup=10, iterations=20, block_size=256):
     """benchmarks/bench_matrix_mul.ml:43-165: one thread per element of C, inputs as the tiled
     bench, every element within 1e-3 of the double product, GFLOPS = 2 m n k / MEAN."""
-    import torch
     m = n = k = size
     a = (np.arange(m * k) % 10) / 10.0
     b = ((np.arange(k * n) + 1) % 10) / 10.0
     expected = a.reshape(m, k) @ b.reshape(k, n)
-    va, vb = _upload(torch, a), _upload(torch, b)
-    vc = torch.empty(m * n, dtype=torch.float32, device="cuda")
-    src = hip.generate_source(reference_kernels.matrix_mul(), block=(block_size, 1, 1))
-    grid = ((m * n + block_size - 1) // block_size, 1, 1)
-    args = [va, vb, vc, ("i32", m), ("i32", n), ("i32", k)]
-    times, path = _benchmark_gpu(lambda: hip.run_source(src, "sarek_kern", (block_size, 1, 1), grid, args),
-                                 warmup, iterations)
-    verified = bool(np.all(np.abs(_download(vc).astype(np.float64).reshape(m, n) - expected) <= 1e-3))
+    ir = reference_kernels.matrix_mul()
+    block, grid = Execute.dims1d(block_size), Execute.dims1d((m * n + block_size - 1) // block_size)
+
+    def compute(v):
+        return Execute.run_vectors(ir=ir, args=[Execute.Vec(v[0]), Execute.Vec(v[1]), Execute.Vec(v[2]),
+                                                Execute.Int(m), Execute.Int(n), Execute.Int(k)], block=block, grid=grid)
+    times, path, (_, _, vc) = _benchmark_gpu(lambda: (_vector(a), _vector(b), Vector.create(Vector.float32, m * n)),
+                                             compute, warmup, iterations)
+    verified = bool(np.all(np.abs(vc.to_array().astype(np.float64).reshape(m, n) - expected) <= 1e-3))
     return _device_record(times, 2.0 * m * n * k / (statistics.mean(times) * 1e6), verified, path, "GFLOPS")
 
 
 def _bench_transpose(ir, block, grid_of, size, warmup, iterations):
-    """benchmarks/bench_transpose.ml:100-210 / bench_transpose_tiled.ml:120-240: input[i] = i, square
-    size x size, tolerance 1e-3 (10 beyond 2^24 elements), GB/s = 8 n / MEAN."""
-    import torch
+    """benchmarks/bench_transpose.ml:100-210 / bench_transpose_tiled.ml:120-240: input[i] = i, output
+    zeroed, square size x size, tolerance 1e-3 (10 beyond 2^24 elements), GB/s = 8 n / MEAN."""
     m = size
     n = m * m
     data = np.arange(n, dtype=np.float64)
-    vin = _upload(torch, data)
-    vout = torch.zeros(n, dtype=torch.float32, device="cuda")
-    src = hip.generate_source(ir, block=block)
-    args = [vin, vout, ("i32", m), ("i32", m)]
-    times, path = _benchmark_gpu(lambda: hip.run_source(src, "sarek_kern", block, grid_of(m), args),
-                                 warmup, iterations)
+    grid = grid_of(m)
+
+    def compute(v):
+        return Execute.run_vectors(ir=ir, args=[Execute.Vec(v[0]), Execute.Vec(v[1]), Execute.Int(m), Execute.Int(m)],
+                                   block=block, grid=grid)
+    times, path, (_, vout) = _benchmark_gpu(lambda: (_vector(data), _vector(np.zeros(n))), compute, warmup, iterations)
     tolerance = 10.0 if n > 16_777_216 else 0.001
     expected = data.reshape(m, m).T.reshape(-1)
-    verified = bool(np.all(np.abs(_download(vout).astype(np.float64) - expected) <= tolerance))
+    verified = bool(np.all(np.abs(vout.to_array().astype(np.float64) - expected) <= tolerance))
     return _device_record(times, 8.0 * n / (statistics.mean(times) / 1e3) / 1e9, verified, path, "GB/s")
 
 
 def bench_transpose(size, warmup=10, iterations=20):
-    return _bench_transpose(reference_kernels.transpose_naive(), (256, 1, 1),
-                            lambda m: ((m * m + 255) // 256, 1, 1), size, warmup, iterations)
+    return _bench_transpose(reference_kernels.transpose_naive(), Execute.dims1d(256),
+                            lambda m: Execute.dims1d((m * m + 255) // 256), size, warmup, iterations)
 
 
 def bench_transpose_tiled(size, warmup=10, iterations=20, tile_size=16):
-    return _bench_transpose(reference_kernels.transpose_tiled(), (tile_size, tile_size, 1),
-                            lambda m: ((m + tile_size - 1) // tile_size, (m + tile_size - 1) // tile_size, 1),
+    return _bench_transpose(reference_kernels.transpose_tiled(), Execute.dims2d(tile_size, tile_size),
+                            lambda m: Execute.dims2d((m + tile_size - 1) // tile_size, (m + tile_size - 1) // tile_size),
                             size, warmup, iterations)
 
 
 def bench_scan(size, warmup=5, iterations=20):
     """benchmarks/bench_scan.ml:112-221: inclusive prefix sum of [1..n] in one 256-thread block
     (n = min(size, 256)), every element equal to the serial prefix sum, M elements/s = n / median."""
-    import torch
     n = min(size, 256)
     data = np.arange(1, n + 1, dtype=np.int32)
-    vin = torch.empty(n, dtype=torch.int32, device="cuda")
-    hip.memcpy_htod(vin.data_ptr(), data)
-    vout = torch.zeros(n, dtype=torch.int32, device="cuda")
-    src = hip.generate_source(reference_kernels.inclusive_scan(), block=(256, 1, 1))
-    args = [vin, vout, ("i32", n)]
-    times, path = _time_launches(lambda: hip.run_source(src, "sarek_kern", (256, 1, 1), (1, 1, 1), args),
-                                 warmup, iterations)
-    got = np.empty(n, dtype=np.int32)
-    hip.memcpy_dtoh(got, vout.data_ptr())
-    verified = bool(np.array_equal(got, np.cumsum(data, dtype=np.int32)))
+    vin, vout = _vector(data, Vector.int32), Vector.create(Vector.int32, n)
+    ir = reference_kernels.inclusive_scan()
+    args = [Execute.Vec(vin), Execute.Vec(vout), Execute.Int32(n)]
+    times, path = _time_launches(
+        lambda: Execute.run_vectors(ir=ir, args=args, block=Execute.dims1d(256), grid=Execute.dims1d(1)),
+        warmup, iterations)
+    verified = bool(np.array_equal(vout.to_array(), np.cumsum(data, dtype=np.int32)))
     return _device_record(times, n / (statistics.median(times) / 1e3 * 1e6), verified, path, "Melem/s")
 
 
@@ -295,11 +279,13 @@ def bench_transfer(size, warmup=2, iterations=7):
     loops, timed alone for a float32 vector of `size` elements in ordinary (pageable) host
     memory.  Throughput is the upload rate; the record also carries the download rate and
     both rates of the driver's own copy."""
-    import torch
     host = (np.arange(size) % 100 / 100.0).astype(np.float32)
-    back = np.empty_like(host)
-    dev = torch.empty(size, dtype=torch.float32, device="cuda")
-    sync = hip.lib.sarek_hip_device_synchronize
+    v = _vector(host)
+    Transfer.to_device(v)                 # allocates the device block; later uploads reuse it
+
+    def upload():
+        v[0] = host[0]                    # Vector.set: Both -> Stale_GPU, so to_device copies again
+        Transfer.to_device(v)
 
     def timed(fn):
         for _ in range(warmup):
@@ -308,20 +294,22 @@ def bench_transfer(size, warmup=2, iterations=7):
         for _ in range(iterations):
             t0 = time.perf_counter()
             fn()
-            hip.check(sync())
+            Transfer.flush()
             ts.append((time.perf_counter() - t0) * 1e3)
         return ts
     rates = {}
     for label, threads in (("driver", 0), ("staged", None)):
         if threads is not None:
             hip.set_tunable("transfer.threads", threads)
-        up = timed(lambda: hip.memcpy_htod(dev.data_ptr(), host))
-        down = timed(lambda: hip.memcpy_dtoh(back, dev.data_ptr()))
+        up = timed(upload)
+        v.host[:] = -1.0                  # behind the vector's back: the download has to restore it
+        down = timed(lambda: Transfer.to_cpu(v, force=True))
         hip.set_tunable("transfer.threads", 4)
         rates[label] = (up, down)
+    back = v.host
     gbs = lambda ts: host.nbytes / (statistics.median(ts) / 1e3) / 1e9
     rec = _device_record(rates["staged"][0], gbs(rates["staged"][0]), np.array_equal(back, host),
-                         "memcpy_htod", "GB/s")
+                         "Transfer.to_device", "GB/s")
     rec["download_gbs"] = gbs(rates["staged"][1])
     rec["driver_copy_upload_gbs"] = gbs(rates["driver"][0])
     rec["driver_copy_download_gbs"] = gbs(rates["driver"][1])
