@@ -105,6 +105,13 @@ int sarek_hip_memcpy_dtoh(void *dst_host, const void *src_device, size_t bytes);
  * staging).  `sarek_hip_host_free(NULL)` is accepted.                           */
 int sarek_hip_host_alloc(void **host_ptr, size_t bytes);
 int sarek_hip_host_free(void *host_ptr);
+/* Memory.alloc_zero_copy (spoc/framework/Framework_sig.ml; used by
+ * sarek/core/Transfer.ml:85-126, 185-203): *supported = 1 and *dptr = the device's view
+ * of the host block when `host_ptr` lies in a block from sarek_hip_host_alloc (then
+ * kernels read and write the host block over the link, and the vector's transfers are
+ * no-ops); *supported = 0 (the reference's None) for any other memory, and the caller
+ * allocates and copies.  The view needs no free (sarek_hip_mem_free ignores it).     */
+int sarek_hip_mem_alloc_zero_copy(void *host_ptr, size_t bytes, void **dptr, int *supported);
 int sarek_hip_memcpy_dtod(void *dst_device, const void *src_device, size_t bytes);
 int sarek_hip_memset_d8(void *dst_device, unsigned char value, size_t bytes);
 
@@ -226,7 +233,10 @@ enum {                                  /* Vector_types.location                
   SAREK_HIP_LOC_STALE_GPU = 4           /* the host copy is the good one                 */
 };
 /* Vector.create / create_custom: host block of `length` elements, contents unspecified,
- * location CPU.  pinned != 0 takes the block from sarek_hip_host_alloc.              */
+ * location CPU.  pinned = 1 takes the block from sarek_hip_host_alloc; pinned = 2 does
+ * too and makes the vector zero-copy: its device buffer is the host block itself
+ * (sarek_hip_mem_alloc_zero_copy), uploads and downloads move nothing (a download
+ * waits for the device), the location states change as for any vector.             */
 int sarek_hip_vector_create(int kind, int64_t length, int64_t custom_elem_size, int pinned,
                             sarek_hip_vector *out);
 int sarek_hip_vector_destroy(sarek_hip_vector v);          /* host block and device buffers */

@@ -262,6 +262,22 @@ int sarek_hip_host_alloc(void **host_ptr, size_t bytes) {
   return SAREK_HIP_OK;
 }
 
+int sarek_hip_mem_alloc_zero_copy(void *host_ptr, size_t bytes, void **dptr, int *supported) {
+  if (!dptr || !supported) return fail(SAREK_HIP_E_INVALID_ARG, "alloc_zero_copy: NULL out pointer");
+  *dptr = nullptr;
+  *supported = 0;
+  (void)bytes;
+  if (!host_ptr || !is_pinned(host_ptr)) return SAREK_HIP_OK;      // None: the caller allocates and copies
+  void *alias = nullptr;
+  if (hipHostGetDevicePointer(&alias, host_ptr, 0) != hipSuccess || !alias) {
+    (void)hipGetLastError();
+    return SAREK_HIP_OK;
+  }
+  *dptr = alias;
+  *supported = 1;
+  return SAREK_HIP_OK;
+}
+
 int sarek_hip_host_free(void *host_ptr) {
   if (!host_ptr) return SAREK_HIP_OK;
   SAREK_HIP_TRY(hipHostFree(host_ptr));

@@ -27,6 +27,7 @@ struct sarek_hip_vector_s {
   int64_t length = 0, elem_size = 4;
   void *host = nullptr;
   bool pinned = false;
+  bool zero_copy = false;                // device buffers alias the pinned host block
   bool auto_sync = true;                 // Vector_types.t.auto_sync
   int location = SAREK_HIP_LOC_CPU;
   int device = -1;                       // the device of a non-CPU location
@@ -63,8 +64,17 @@ int ensure_buffer(sarek_hip_vector_s *v, int dev, void **out) {
     return SAREK_HIP_OK;
   }
   void *p = nullptr;
-  int st = sarek_hip_mem_alloc(&p, bytes_of(v));
-  if (st != SAREK_HIP_OK) return st;
+  if (v->zero_copy) {
+    // Memory.alloc_zero_copy returning Some (Transfer.ml:85-126): the buffer is the host block
+    // as the device sees it; its transfers are no-ops.
+    int supported = 0;
+    int st = sarek_hip_mem_alloc_zero_copy(v->host, bytes_of(v), &p, &supported);
+    if (st != SAREK_HIP_OK) return st;
+    if (!supported) return fail(SAREK_HIP_E_UNSUPPORTED, "zero-copy vector: the host block is not device-accessible");
+  } else {
+    int st = sarek_hip_mem_alloc(&p, bytes_of(v));
+    if (st != SAREK_HIP_OK) return st;
+  }
   v->buffers[dev] = p;
   *out = p;
   return SAREK_HIP_OK;
@@ -80,8 +90,10 @@ int to_device(sarek_hip_vector_s *v, int dev) {
   void *buf = nullptr;
   int st = ensure_buffer(v, dev, &buf);
   if (st != SAREK_HIP_OK) return st;
-  st = sarek_hip_memcpy_htod(buf, v->host, bytes_of(v));
-  if (st != SAREK_HIP_OK) return st;
+  if (!v->zero_copy) {
+    st = sarek_hip_memcpy_htod(buf, v->host, bytes_of(v));
+    if (st != SAREK_HIP_OK) return st;
+  }
   v->location = SAREK_HIP_LOC_BOTH;
   v->device = dev;
   return SAREK_HIP_OK;
@@ -98,7 +110,9 @@ int to_cpu(sarek_hip_vector_s *v, bool force) {
   if (!needed) return SAREK_HIP_OK;
   auto it = v->buffers.find(v->device);
   if (it == v->buffers.end()) return fail(SAREK_HIP_E_INVALID_ARG, "to_cpu: no device buffer to transfer from");
-  int st = sarek_hip_memcpy_dtoh(v->host, it->second, bytes_of(v));
+  // A copy waits for the launches before it; a zero-copy vector has nothing to copy, but the
+  // kernel that wrote the host block must have finished before the host reads it.
+  int st = v->zero_copy ? sarek_hip_device_synchronize() : sarek_hip_memcpy_dtoh(v->host, it->second, bytes_of(v));
   if (st != SAREK_HIP_OK) return st;
   v->location = SAREK_HIP_LOC_BOTH;
   return SAREK_HIP_OK;
@@ -233,6 +247,7 @@ int sarek_hip_vector_create(int kind, int64_t length, int64_t custom_elem_size, 
   v->length = length;
   v->elem_size = es;
   v->pinned = pinned != 0;
+  v->zero_copy = pinned == 2;
   const size_t bytes = static_cast<size_t>(length * es);
   if (v->pinned) {
     int st = sarek_hip_host_alloc(&v->host, bytes);

@@ -85,6 +85,7 @@ SYMBOLS = {
     "sarek_hip_memcpy_dtod": (_i, [_vp, _vp, _sz]),
     "sarek_hip_host_alloc": (_i, [C.POINTER(_vp), _sz]),
     "sarek_hip_host_free": (_i, [_vp]),
+    "sarek_hip_mem_alloc_zero_copy": (_i, [_vp, _sz, C.POINTER(_vp), C.POINTER(_i)]),
     "sarek_hip_memset_d8": (_i, [_vp, C.c_ubyte, _sz]),
     "sarek_hip_stream_create": (_i, [C.POINTER(_vp)]),
     "sarek_hip_stream_destroy": (_i, [_vp]),

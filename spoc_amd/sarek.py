@@ -44,9 +44,11 @@ class Vector:
 
     # -- creation (Vector_storage.create / create_custom / of_array) --
     @classmethod
-    def create(cls, kind, length, pinned=False):
+    def create(cls, kind, length, pinned=False, zero_copy=False):
+        """pinned: host block from pinned memory (copies run at the full link rate, no staging).
+        zero_copy: pinned, and the device works on the host block itself: no copies at all."""
         h = C.c_void_p()
-        hip.check(hip.lib.sarek_hip_vector_create(kind.code, length, 0, int(pinned), C.byref(h)))
+        hip.check(hip.lib.sarek_hip_vector_create(kind.code, length, 0, 2 if zero_copy else int(pinned), C.byref(h)))
         return cls(h, kind)
 
     @classmethod

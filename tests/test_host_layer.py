@@ -192,3 +192,43 @@ def test_lowering_failure_and_pinned_vectors(torch_cuda):
     Execute.run_vectors(ir=reference_kernels.vector_copy(), args=[Execute.Vec(big), Execute.Vec(out), Execute.Int(1 << 22)],
                         block=(256, 1, 1), grid=((1 << 22) // 256, 1, 1))
     assert np.array_equal(out.to_array(), big.host)
+
+
+@gpu
+def test_zero_copy_vectors(torch_cuda):
+    """Memory.alloc_zero_copy returning Some (sarek/core/Transfer.ml:85-126, 185-203): the device
+    buffer is the host block; transfers move nothing; the location states change as usual."""
+    from spoc_amd import hip
+    n = 1 << 20
+    b = Vector.create(Vector.float32, n, zero_copy=True)
+    c = Vector.create(Vector.float32, n, zero_copy=True)
+    a = Vector.create(Vector.float32, n, zero_copy=True)
+    b.fill_from(np.arange(n) % 100 / 100.0)
+    c.fill_from((np.arange(n) + 1) % 100 / 100.0)
+    a.host[:] = -1.0
+    args = [Execute.Vec(a), Execute.Vec(b), Execute.Vec(c), Execute.Float32(3.0), Execute.Int(n)]
+    path = Execute.run_vectors(ir=reference_kernels.stream_triad(), args=args, block=(256, 1, 1),
+                               grid=((n + 255) // 256, 1, 1))
+    assert path == "stream_triad_f32" and a.location == Stale_CPU
+    host_addr = a.host.ctypes.data
+    assert a.device_ptr is not None
+    expected = (b.host.astype(np.float64) + 3.0 * c.host.astype(np.float64)).astype(np.float32)
+    assert np.array_equal(a.to_array(), expected)           # to_array waits for the kernel; nothing is copied
+    assert a.location == Both and a.host.ctypes.data == host_addr and np.array_equal(a.host, expected)
+    # a host write is seen by the next launch without an upload
+    b[0] = 10.0
+    assert b.location == Stale_CPU or b.location == Stale_GPU
+    Transfer.to_cpu(b)
+    b[0] = 10.0
+    Execute.run_vectors(ir=reference_kernels.stream_triad(), args=args, block=(256, 1, 1), grid=((n + 255) // 256, 1, 1))
+    assert a[0] == np.float32(10.0 + 3.0 * c.host[0])
+    # alloc_zero_copy itself: None for ordinary memory, a device view for pinned blocks
+    ordinary = np.zeros(16, dtype=np.float32)
+    import ctypes as C
+    dptr, ok = C.c_void_p(), C.c_int(-1)
+    hip.check(hip.lib.sarek_hip_mem_alloc_zero_copy(C.c_void_p(ordinary.ctypes.data), 64, C.byref(dptr), C.byref(ok)))
+    assert ok.value == 0 and dptr.value is None
+    with hip.pinned_array(16, np.float32) as pinned:
+        hip.check(hip.lib.sarek_hip_mem_alloc_zero_copy(C.c_void_p(pinned.ctypes.data), 64, C.byref(dptr), C.byref(ok)))
+        assert ok.value == 1 and dptr.value is not None
+        hip.check(hip.lib.sarek_hip_mem_free(dptr))          # a view needs no free; freeing it is harmless
