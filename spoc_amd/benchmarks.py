@@ -17,6 +17,7 @@ launch (reported as `path`).
     python -m spoc_amd.benchmarks all --json out.json
 """
 import argparse
+import ctypes as C
 import json
 import statistics
 import time
@@ -333,9 +334,70 @@ BENCHMARKS = {
 }
 
 
+def _first_line(cmd, default="unknown"):
+    import subprocess
+    try:
+        out = subprocess.run(cmd, shell=True, capture_output=True, text=True, timeout=10).stdout.splitlines()
+        return out[0].strip() if out and out[0].strip() else default
+    except Exception:
+        return default
+
+
+def system_info():
+    """benchmarks/system_info.ml:22-236: host name, OS, kernel, CPU model / cores / threads, memory
+    and the devices, in the shape its to_json writes."""
+    model = "unknown"
+    try:
+        for line in open("/proc/cpuinfo"):
+            if line.startswith("model name"):
+                model = line.split(":", 1)[1].strip()
+                break
+    except OSError:
+        pass
+    threads = int(_first_line("nproc", "1"))
+    cores = max(1, threads // 2)
+    try:
+        import subprocess
+        cps = sockets = None
+        for line in subprocess.run("lscpu 2>/dev/null", shell=True, capture_output=True, text=True).stdout.splitlines():
+            if line.startswith("Core(s) per socket"):
+                cps = int(line.split(":")[1])
+            elif line.startswith("Socket(s)"):
+                sockets = int(line.split(":")[1])
+        if cps and sockets:
+            cores = cps * sockets
+    except Exception:
+        pass
+    try:
+        memory_gb = float(_first_line("free -b | grep Mem | awk '{print $2}'", "0")) / 2 ** 30
+    except ValueError:
+        memory_gb = 0.0
+    info = hip.device_info(0)
+    version = C.c_int(0)
+    hip.check(hip.lib.sarek_hip_driver_version(C.byref(version)))
+    device = {"driver_version": str(version.value), "compute_capability": f"{info.compute_major}.{info.compute_minor}",
+              "id": 0, "name": info.name.decode(), "framework": "HIP", "memory_gb": info.total_global_mem / 2 ** 30}
+    return {"hostname": _first_line("hostname"), "os": _first_line("uname -s"), "kernel": _first_line("uname -r"),
+            "cpu": {"model": model, "cores": cores, "threads": threads}, "memory_gb": memory_gb, "devices": [device]}
+
+
+def result_record(name, size, block_size, iterations, warmup, device_results, system=None):
+    """benchmarks/output.ml:66-90 (Output.to_json): the file the reference's result tools read."""
+    import subprocess
+    commit = _first_line("git rev-parse HEAD 2>/dev/null", "")
+    return {"benchmark": {"name": name, "timestamp": time.strftime("%Y-%m-%dT%H:%M:%SZ", time.gmtime()),
+                          "git_commit": commit or None,
+                          "parameters": {"size": size, "block_size": block_size, "iterations": iterations,
+                                         "warmup": warmup}},
+            "system": system if system is not None else system_info(),
+            "results": [r for r in device_results                                  # Output.filter_valid_results
+                        if r["iterations"] and not (r["median_ms"] == 0.0 and r["verified"] is False)]}
+
+
 def run(name, sizes=None, warmup=None, iterations=20):
     fn, default_sizes = BENCHMARKS[name]
     out = []
+    system = system_info()
     for size in sizes or default_sizes:
         kw = {} if warmup is None else {"warmup": warmup}
         rec = fn(size, iterations=iterations, **kw)
@@ -347,9 +409,11 @@ def run(name, sizes=None, warmup=None, iterations=20):
             print(f"  Download: {rec['download_gbs']:.3f} GB/s; driver's own copy: "
                   f"{rec['driver_copy_upload_gbs']:.3f} up, {rec['driver_copy_download_gbs']:.3f} down")
         print(f"  Verified: {'✓' if rec['verified'] else '✗'}", flush=True)
-        out.append({"benchmark": {"name": name, "parameters": {"size": size, "iterations": iterations,
-                                                               "warmup": warmup}},
-                    "results": [rec]})
+        import inspect
+        defaults = {k: p.default for k, p in inspect.signature(fn).parameters.items()}
+        block = defaults.get("block_size", defaults.get("tile_size", 256))
+        out.append(result_record(name, size, block * block if "tile_size" in defaults else block, iterations,
+                                 warmup if warmup is not None else defaults.get("warmup"), [rec], system))
     return out
 
 

@@ -201,3 +201,23 @@ def test_reference_benchmarks_run_and_verify(hip, torch_cuda, name, size, path):
     finally:
         hip.check(hip.lib.sarek_hip_set_specialisation(1))
     assert rec["verified"] and rec["path"] == "jit"
+
+
+def test_result_file_has_the_reference_shape(hip, torch_cuda, tmp_path):
+    """benchmarks/output.ml:66-90 and benchmarks/system_info.ml:202-236: what the result tools read."""
+    from spoc_amd import benchmarks
+    (rec,) = benchmarks.run("scan", sizes=[64], iterations=3)
+    assert set(rec) == {"benchmark", "system", "results"}
+    assert set(rec["benchmark"]) == {"name", "timestamp", "git_commit", "parameters"}
+    assert rec["benchmark"]["name"] == "scan" and rec["benchmark"]["timestamp"].endswith("Z")
+    assert rec["benchmark"]["parameters"] == {"size": 64, "block_size": 256, "iterations": 3, "warmup": 5}
+    assert {"hostname", "os", "kernel", "cpu", "memory_gb", "devices"} <= set(rec["system"])
+    assert set(rec["system"]["cpu"]) == {"model", "cores", "threads"}
+    dev = rec["system"]["devices"][0]
+    assert dev["framework"] == "HIP" and dev["memory_gb"] > 100 and dev["id"] == 0
+    (r,) = rec["results"]
+    assert {"device_id", "device_name", "framework", "iterations", "mean_ms", "stddev_ms", "median_ms", "min_ms",
+            "max_ms", "throughput_gflops", "verified"} <= set(r)
+    assert len(r["iterations"]) == 3 and r["verified"] is True
+    (tiled,) = benchmarks.run("matrix_mul_tiled", sizes=[64], iterations=2, warmup=1)
+    assert tiled["benchmark"]["parameters"]["block_size"] == 256          # tile_size squared
