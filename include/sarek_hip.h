@@ -194,8 +194,12 @@ typedef struct {
  * specialisation is enabled, the source carries a leading
  * `// sarek-hip-specialise: <tag>` line that run_source honours; the plain
  * lowering always follows, so the text is valid HIP either way.
- * block: launch block dims or NULL.  Writes at most out_len bytes incl. NUL;
- * *needed gets the full size.                                              */
+ * block: launch block dims or NULL (BACKEND.generate_source ?block).  When given,
+ * the size of a shared array written in terms of the block dimensions (an unsized
+ * let%shared lowers to block_dim_x elements, sarek/ppx/Sarek_lower_ir.ml:496-507) is
+ * emitted as the constant a __shared__ declaration needs; the reference's generators
+ * leave blockDim.x there, which no device compiler accepts.
+ * Writes at most out_len bytes incl. NUL; *needed gets the full size.          */
 int sarek_hip_generate_source(const char *ir_text, const int block[3], char *out, size_t out_len,
                               size_t *needed);
 

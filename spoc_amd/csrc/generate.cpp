@@ -12,14 +12,13 @@ using namespace sarek_hip;
 
 extern "C" int sarek_hip_generate_source(const char *ir_text, const int block[3], char *out,
                                          size_t out_len, size_t *needed) {
-  (void)block;  // the lowering does not depend on the launch shape
   if (!ir_text) return fail(SAREK_HIP_E_INVALID_ARG, "generate_source: NULL IR text");
   std::string src;
   try {
     ir::Kernel k = ir::parse_kernel(ir_text);
     std::string tag = ir::recognise(k);
     if (!tag.empty()) src = std::string(kSpecialiseMarker) + tag + "\n";
-    src += ir::generate(k);
+    src += ir::generate(k, block);
   } catch (const ir::ParseError &e) {
     return fail(SAREK_HIP_E_PARSE, "%s", e.what());
   } catch (const ir::CodegenError &e) {

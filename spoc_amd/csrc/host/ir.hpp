@@ -143,7 +143,11 @@ std::string print_stmt(const StmtP &s);
 // ir_hip.cpp: IR -> HIP C++ for gfx950
 std::string gen_expr(const ExprP &e);
 std::string gen_stmt(const StmtP &s, const std::string &indent);
-std::string generate(const Kernel &k);   // records + variants + helpers + kernel
+// records + variants + helpers + kernel.  `block` (may be null): the launch block, when the
+// caller knows it; sizes of shared arrays written in terms of the block dimensions
+// (`let%shared tile = ()` lowers to block_dim_x elements, sarek/ppx/Sarek_lower_ir.ml:496-507)
+// are then constants, which a __shared__ declaration needs.
+std::string generate(const Kernel &k, const int block[3] = nullptr);
 
 // specialise.cpp: "" or the tag of the hand-written kernel that computes the same thing
 std::string recognise(const Kernel &k);

@@ -24,6 +24,11 @@ namespace {
 
 // Variant definitions of the kernel being generated (for match bindings).
 thread_local const Kernel *t_kernel = nullptr;
+// Launch block known to the caller of generate (0 = unknown) and whether the expression being
+// printed is the size of a shared array: there blockDim.* has to be a constant for the
+// declaration to compile, so the known value is written instead.
+thread_local int t_block[3] = {0, 0, 0};
+thread_local bool t_in_shared_size = false;
 
 std::string mangle(const std::string &name) {
   std::string o = name;
@@ -55,6 +60,14 @@ std::string param_type_str(const TypeP &t) {
 }
 
 const char *thread_intrinsic(const std::string &n) {
+  if (t_in_shared_size && n.size() == 11 && n.compare(0, 10, "block_dim_") == 0) {
+    const int axis = n[10] - 'x';
+    if (axis >= 0 && axis < 3 && t_block[axis] > 0) {
+      static thread_local char num[3][16];
+      std::snprintf(num[axis], sizeof(num[axis]), "%d", t_block[axis]);
+      return num[axis];
+    }
+  }
   static const struct {
     const char *name, *code;
   } table[] = {
@@ -425,8 +438,17 @@ std::string gen_stmt(const StmtP &sp, const std::string &indent) {
     case Stmt::Let:
     case Stmt::LetMut:
       if (s.kind == Stmt::Let && s.e->kind == Expr::ArrayCreate) {
+        t_in_shared_size = s.e->mem == MemSpace::Shared;
+        std::string size;
+        try {
+          size = gen_expr(s.e->args[0]);
+        } catch (...) {
+          t_in_shared_size = false;
+          throw;
+        }
+        t_in_shared_size = false;
         return indent + (s.e->mem == MemSpace::Shared ? "__shared__ " : "") + type_str(s.e->type) + " " +
-               s.var.name + "[" + gen_expr(s.e->args[0]) + "];\n" + gen_stmt(s.stmts[0], indent);
+               s.var.name + "[" + size + "];\n" + gen_stmt(s.stmts[0], indent);
       }
       return indent + type_str(s.var.type) + " " + s.var.name + " = " + gen_expr(s.e) + ";\n" +
              gen_stmt(s.stmts[0], indent);
@@ -440,7 +462,8 @@ std::string gen_stmt(const StmtP &sp, const std::string &indent) {
   return "";
 }
 
-std::string generate(const Kernel &k) {
+std::string generate(const Kernel &k, const int block[3]) {
+  for (int i = 0; i < 3; ++i) t_block[i] = block ? block[i] : 0;
   t_kernel = &k;
   std::string o = "\nextern \"C\" {\n";
   try {

@@ -201,9 +201,12 @@ std::mutex g_lowered_mu;
 std::unordered_map<std::string, Lowered> g_lowered;
 
 int lower(const char *ir_text, const int block[3], Lowered &out) {
+  // the text can depend on the block (sizes of shared arrays): it is part of the key
+  const std::string key = std::to_string(block[0]) + "," + std::to_string(block[1]) + "," +
+                          std::to_string(block[2]) + ";" + ir_text;
   {
     std::lock_guard<std::mutex> lock(g_lowered_mu);
-    auto it = g_lowered.find(ir_text);
+    auto it = g_lowered.find(key);
     if (it != g_lowered.end()) {
       out = it->second;
       return SAREK_HIP_OK;
@@ -224,7 +227,7 @@ int lower(const char *ir_text, const int block[3], Lowered &out) {
   out.name = ir::parse_kernel(ir_text).name;
   std::lock_guard<std::mutex> lock(g_lowered_mu);
   if (g_lowered.size() > 256) g_lowered.clear();
-  g_lowered[ir_text] = out;
+  g_lowered[key] = out;
   return SAREK_HIP_OK;
 }
 
