@@ -73,12 +73,11 @@ def test_superstep_family(hip, torch_cuda, block_size):
     exp[:block_size] = 0.0
     go(shared_n("tile", "f32", BLOCK_DIM, seq(block(cond_load), BARRIER, store)), exp)
     # 7: two shared arrays, one sized by the block and one by a constant
-    if block_size <= 32 or True:
-        two = seq(assign_elem("tile1", TIDX, read("input", GTID)),
-                  assign_elem("tile2", TIDX, add(read("input", GTID), f32("1.0"))))
-        both = assign_elem("output", GTID, add(read("tile1", TIDX), read("tile2", TIDX)))
-        go(shared_n("tile1", "f32", BLOCK_DIM, shared_n("tile2", "f32", i32(max(32, block_size)),
-                                                        seq(block(two), BARRIER, both))), x + (x + 1.0))
+    two = seq(assign_elem("tile1", TIDX, read("input", GTID)),
+              assign_elem("tile2", TIDX, add(read("input", GTID), f32("1.0"))))
+    both = assign_elem("output", GTID, add(read("tile1", TIDX), read("tile2", TIDX)))
+    go(shared_n("tile1", "f32", BLOCK_DIM, shared_n("tile2", "f32", i32(max(32, block_size)),
+                                                    seq(block(two), BARRIER, both))), x + (x + 1.0))
 
 
 def test_unsized_shared_needs_the_block(hip, torch_cuda):
@@ -213,3 +212,48 @@ def test_mandelbrot_two_dimensional_launch(hip, torch_cuda):
     got = out.cpu().numpy().reshape(h, w)
     assert got.min() >= 0 and got.max() == max_iter
     assert (got == it).mean() > 0.995 and np.abs(got - it).max() <= max_iter
+
+
+@pytest.mark.parametrize("elt", ["i32", "f32", "f64", "point3d"])
+def test_transpose_through_a_shared_helper_at_four_types(hip, torch_cuda, elt):
+    """test_transpose.ml:87-138: one module-level helper over 'a vectors, monomorphised at int32,
+    float32, float64 and a three-float record; run with Vector / Execute.run_vectors, the record
+    vector as a custom vector of 12-byte elements."""
+    from spoc_amd.sarek import Execute, Stale_CPU, Vector
+    w, h = 37, 53
+    n = w * h
+    ty = "(record point3d (x f32) (y f32) (z f32))" if elt == "point3d" else elt
+    types = "(types (point3d (x f32) (y f32) (z f32)))" if elt == "point3d" else ""
+    helper = f"""(func do_transpose (params (var input 20 (vec {ty})) (var output 21 (vec {ty})) (var width 22 i32)
+                                          (var height 23 i32) (var tid 24 i32)) unit
+      (let (var n 25 i32) (mul (var width 22 i32) (var height 23 i32))
+       (if (lt (var tid 24 i32) (var n 25 i32))
+        (let (var col 26 i32) (mod (var tid 24 i32) (var width 22 i32))
+        (let (var row 27 i32) (div (var tid 24 i32) (var width 22 i32))
+        (let (var in_idx 28 i32) (add (mul (var row 27 i32) (var width 22 i32)) (var col 26 i32))
+        (let (var out_idx 29 i32) (add (mul (var col 26 i32) (var height 23 i32)) (var row 27 i32))
+         (assign (lelem output (var out_idx 29 i32)) (read input (var in_idx 28 i32))))))))))"""
+    ir = f"""(kernel sarek_kern (params (param (var input 1 (vec {ty}))) (param (var output 2 (vec {ty})))
+                                       (param (var width 3 i32)) (param (var height 4 i32)))
+      (locals) (body (expr (app (var do_transpose 30 unit) (var input 1 (vec {ty})) (var output 2 (vec {ty}))
+                                (var width 3 i32) (var height 4 i32) (intr (Std) global_thread_id))))
+      {types} (funcs {helper}) (native_fn true))"""
+    if elt == "point3d":
+        vin, vout = Vector.create_custom(12, n), Vector.create_custom(12, n)
+        data = np.arange(3 * n, dtype=np.float32).reshape(n, 3)
+        vin.host.view(np.float32).reshape(n, 3)[:] = data
+        vout.host.view(np.uint8)[:] = 0
+    else:
+        kind = {"i32": Vector.int32, "f32": Vector.float32, "f64": Vector.float64}[elt]
+        vin, vout = Vector.create(kind, n), Vector.create(kind, n)
+        data = (np.arange(n) * (1.0 if elt == "i32" else 1.0 + 2.0 ** -30)).astype(kind.dtype)
+        vin.fill_from(data)
+        vout.fill_from(np.zeros(n))
+    path = Execute.run_vectors(ir=ir, args=[Execute.Vec(vin), Execute.Vec(vout), Execute.Int32(w), Execute.Int32(h)],
+                               block=Execute.dims1d(256), grid=Execute.dims1d((n + 255) // 256))
+    assert path == "jit" and vout.location == Stale_CPU
+    if elt == "point3d":
+        got = vout.to_array().view(np.float32).reshape(w, h, 3)
+        assert np.array_equal(got, data.reshape(h, w, 3).transpose(1, 0, 2))
+    else:
+        assert np.array_equal(vout.to_array().reshape(w, h), data.reshape(h, w).T)
