@@ -2,8 +2,9 @@
 
 Host-side mirror of benchmarks/bench_matrix_mul_tiled.ml, bench_stream_triad.ml,
 bench_reduction.ml, bench_dot_product.ml, bench_reduction_max.ml, bench_vector_add.ml,
-bench_vector_copy.ml, bench_matrix_mul.ml, bench_transpose.ml, bench_transpose_tiled.ml and
-bench_scan.ml: same inputs, same
+bench_vector_copy.ml, bench_matrix_mul.ml, bench_transpose.ml, bench_transpose_tiled.ml, bench_scan.ml,
+bench_gather_scatter.ml, bench_histogram.ml, bench_stencil_2d.ml, bench_conv2d.ml, bench_mandelbrot.ml,
+bench_nbody.ml, bench_bitonic_sort.ml and bench_radix_sort.ml (the whole suite): same inputs, same
 launch geometry, same warmup / timed-iteration protocol (wall clock around the launch plus
 the device flush, one sample per iteration), same verification and tolerance, same
 throughput formula and statistic, and the same per-device result record
@@ -274,6 +275,282 @@ def bench_scan(size, warmup=5, iterations=20):
     return _device_record(times, n / (statistics.median(times) / 1e3 * 1e6), verified, path, "Melem/s")
 
 
+def _ocaml_random_ints(n, bound, seed=42):
+    """Stand-in for `Random.init 42; Random.int bound`: OCaml's generator is not available here, so
+    the values differ from the reference's while the distribution (uniform on [0, bound)) is the same."""
+    return np.random.default_rng(seed).integers(0, bound, n).astype(np.int32)
+
+
+def bench_gather(size, warmup=5, iterations=20):
+    """benchmarks/bench_gather_scatter.ml:76-199: input[i] = 2 i, random indices, output[i] =
+    input[indices[i]] exactly, M elements/s = n / median."""
+    n = size
+    data, idx = np.arange(n, dtype=np.int64) * 2, _ocaml_random_ints(n, n)
+    vin, vidx, vout = _vector(data, Vector.int32), _vector(idx, Vector.int32), Vector.create(Vector.int32, n)
+    ir = reference_kernels.gather()
+    args = [Execute.Vec(vin), Execute.Vec(vidx), Execute.Vec(vout), Execute.Int32(n)]
+    times, path = _time_launches(
+        lambda: Execute.run_vectors(ir=ir, args=args, block=Execute.dims1d(256), grid=Execute.dims1d((n + 255) // 256)),
+        warmup, iterations)
+    verified = bool(np.array_equal(vout.to_array(), data.astype(np.int32)[idx]))
+    return _device_record(times, n / (statistics.median(times) / 1e3 * 1e6), verified, path, "Melem/s")
+
+
+def bench_scatter(size, warmup=5, iterations=20):
+    """benchmarks/bench_gather_scatter.ml:202-340: input[i] = 3 i + 1, random (colliding) indices,
+    output zeroed on the host before every launch (so its upload is inside the timed sample, as in
+    the reference); every output element is 0 or one of the inputs."""
+    n = size
+    data, idx = (np.arange(n, dtype=np.int64) * 3 + 1).astype(np.int32), _ocaml_random_ints(n, n)
+    vin, vidx, vout = _vector(data, Vector.int32), _vector(idx, Vector.int32), _vector(np.zeros(n), Vector.int32)
+    ir = reference_kernels.scatter()
+    args = [Execute.Vec(vin), Execute.Vec(vidx), Execute.Vec(vout), Execute.Int32(n)]
+    zeros = np.zeros(n, dtype=np.int32)
+
+    def one():
+        return Execute.run_vectors(ir=ir, args=args, block=Execute.dims1d(256), grid=Execute.dims1d((n + 255) // 256))
+    path = None
+    for _ in range(warmup):
+        vout.fill_from(zeros)
+        path = one()
+        Transfer.flush()
+    times = []
+    for _ in range(iterations):
+        vout.fill_from(zeros)
+        t0 = time.perf_counter()
+        path = one()
+        Transfer.flush()
+        times.append((time.perf_counter() - t0) * 1e3)
+    got = vout.to_array()
+    verified = bool(np.all((got == 0) | ((got % 3 == 1) & (got >= 1) & (got <= 3 * (n - 1) + 1))))
+    # stronger than the reference's membership check: a written slot holds an input that was sent there
+    written = got != 0
+    verified = verified and bool(np.array_equal(idx[(got[written] - 1) // 3], np.nonzero(written)[0]))
+    return _device_record(times, n / (statistics.median(times) / 1e3 * 1e6), verified, path, "Melem/s")
+
+
+def bench_histogram(size, warmup=5, iterations=20):
+    """benchmarks/bench_histogram.ml:86-210: random values in [0, 256), 256 bins, a fresh zeroed
+    histogram vector per timed launch, exact counts, M elements/s = n / median."""
+    n, bins = size, 256
+    data = _ocaml_random_ints(n, bins)
+    vin = _vector(data, Vector.int32)
+    ir = reference_kernels.histogram()
+    block, grid = Execute.dims1d(256), Execute.dims1d((n + 255) // 256)
+
+    def launch(hist):
+        return Execute.run_vectors(ir=ir, args=[Execute.Vec(vin), Execute.Vec(hist), Execute.Int32(n), Execute.Int32(bins)],
+                                   block=block, grid=grid, shared_mem=bins * 4)
+    hist = Vector.create(Vector.int32, bins)
+    for _ in range(warmup):
+        hist.fill_from(np.zeros(bins))
+        path = launch(hist)
+        Transfer.flush()
+    times = []
+    for _ in range(iterations):
+        hist = _vector(np.zeros(bins), Vector.int32)
+        t0 = time.perf_counter()
+        path = launch(hist)
+        Transfer.flush()
+        times.append((time.perf_counter() - t0) * 1e3)
+    verified = bool(np.array_equal(hist.to_array(), np.bincount(data, minlength=bins)))
+    return _device_record(times, n / (statistics.median(times) / 1e3 * 1e6), verified, path, "Melem/s")
+
+
+def _grid_bench(ir, block, grid, size, data, expected, tolerance, warmup, iterations):
+    """The loop of bench_stencil_2d.ml:110-150 / bench_conv2d.ml:133-172: warmup launches without a
+    flush between them, one flush, then launch + flush per sample; interior cells within `tolerance`."""
+    n = size * size
+    vin, vout = _vector(data), _vector(np.zeros(n))
+    args = [Execute.Vec(vin), Execute.Vec(vout), Execute.Int32(size), Execute.Int32(size)]
+    path = None
+    for _ in range(warmup):
+        path = Execute.run_vectors(ir=ir, args=args, block=block, grid=grid)
+    Transfer.flush()
+    times = []
+    for _ in range(iterations):
+        t0 = time.perf_counter()
+        path = Execute.run_vectors(ir=ir, args=args, block=block, grid=grid)
+        Transfer.flush()
+        times.append((time.perf_counter() - t0) * 1e3)
+    got = vout.to_array().astype(np.float64).reshape(size, size)
+    verified = bool(np.all(np.abs(got[1:-1, 1:-1] - expected[1:-1, 1:-1]) <= tolerance))
+    return _device_record(times, n / (statistics.median(times) / 1e3) / 1e6, verified, path, "Mcell/s")
+
+
+def bench_stencil_2d(size, warmup=5, iterations=20):
+    """benchmarks/bench_stencil_2d.ml:60-180: input sin(0.1 x) cos(0.1 y), 16x16 blocks, interior
+    within 1e-4 of the double five-point mean, M cells/s = n / median."""
+    g = np.arange(size, dtype=np.float64)
+    data = (np.sin(g * 0.1)[None, :] * np.cos(g * 0.1)[:, None])
+    f = data.astype(np.float32).astype(np.float64)
+    expected = np.zeros_like(f)
+    expected[1:-1, 1:-1] = (f[:-2, 1:-1] + f[2:, 1:-1] + f[1:-1, :-2] + f[1:-1, 2:] + f[1:-1, 1:-1]) / 5.0
+    tiles = (size + 15) // 16
+    return _grid_bench(reference_kernels.stencil_2d(), Execute.dims2d(16, 16), Execute.dims2d(tiles, tiles), size,
+                       data.reshape(-1), expected, 1e-4, warmup, iterations)
+
+
+def bench_conv2d(size, warmup=5, iterations=20):
+    """benchmarks/bench_conv2d.ml:79-212: input ((x + y) mod 256)/255, 3x3 box filter, one thread per
+    pixel, interior within 1e-3, M pixels/s = n / median."""
+    g = np.arange(size)
+    data = ((g[None, :] + g[:, None]) % 256) / 255.0
+    f = data.astype(np.float32).astype(np.float64)
+    expected = np.zeros_like(f)
+    for dy in (0, 1, 2):
+        for dx in (0, 1, 2):
+            expected[1:-1, 1:-1] += f[dy:size - 2 + dy, dx:size - 2 + dx] / 9.0
+    n = size * size
+    return _grid_bench(reference_kernels.conv2d(), Execute.dims1d(256), Execute.dims1d((n + 255) // 256), size,
+                       data.reshape(-1), expected, 1e-3, warmup, iterations)
+
+
+def bench_mandelbrot(size, warmup=10, iterations=20, max_iterations=256):
+    """benchmarks/bench_mandelbrot.ml:112-225: size x size image, 16x16 blocks, the first 1001 pixels
+    within 10 iterations of the float recurrence, M pixels/s = pixels / MEAN."""
+    width = height = size
+    n = width * height
+    ir = reference_kernels.mandelbrot()
+    tiles = (size + 15) // 16
+    block, grid = Execute.dims2d(16, 16), Execute.dims2d(tiles, tiles)
+
+    def compute(v):
+        return Execute.run_vectors(ir=ir, args=[Execute.Vec(v), Execute.Int(width), Execute.Int(height),
+                                                Execute.Int(max_iterations)], block=block, grid=grid)
+    times, path, vout = _benchmark_gpu(lambda: _vector(np.zeros(n), Vector.int32), compute, warmup, iterations)
+    head = min(1001, n)
+    px = (np.arange(head) % width).astype(np.float64)
+    py = (np.arange(head) // width).astype(np.float64)
+    x0, y0 = 4.0 * (px / width) - 2.5, 3.0 * (py / height) - 1.5
+    x, y, it = np.zeros(head), np.zeros(head), np.zeros(head, dtype=np.int64)
+    for _ in range(max_iterations):
+        live = (x * x + y * y <= 4.0) & (it < max_iterations)
+        x, y = np.where(live, x * x - y * y + x0, x), np.where(live, 2.0 * x * y + y0, y)
+        it += live
+    verified = bool(np.all(np.abs(vout.to_array()[:head].astype(np.int64) - it) <= 10))
+    return _device_record(times, n / (statistics.mean(times) / 1e3) / 1e6, verified, path, "Mpixel/s")
+
+
+def bench_nbody(size, warmup=5, iterations=20):
+    """benchmarks/bench_nbody.ml:107-235: positions (i mod 7, i mod 5, i mod 3)/10, blocks of 64,
+    accelerations against the double all-pairs sum (off by more than 1e-3 both absolutely and
+    relatively counts as an error), G interactions/s = n^2 / median.
+
+    From 4096 bodies on that check fails for any kernel that accumulates in f32 in j order, as the
+    generated code does: the lattice repeats every 105 bodies, single terms reach 1e3 and the net
+    force on some bodies is below 1 after cancellation; a numpy emulation of the f32 loop counts
+    273 such bodies at 4096 (largest difference 0.23 on sums of magnitude 3e4) and none at 2048."""
+    n = size
+    i = np.arange(n)
+    pos = [(i % 7) / 10.0, (i % 5) / 10.0, (i % 3) / 10.0]
+    vpos = [_vector(p) for p in pos]
+    vacc = [_vector(np.zeros(n)) for _ in range(3)]
+    ir = reference_kernels.nbody_accel()
+    args = [Execute.Vec(v) for v in vpos + vacc] + [Execute.Int32(n)]
+    block, grid = Execute.dims1d(64), Execute.dims1d((n + 63) // 64)
+    path = None
+    for _ in range(warmup):
+        path = Execute.run_vectors(ir=ir, args=args, block=block, grid=grid)
+    Transfer.flush()
+    times = []
+    for _ in range(iterations):
+        t0 = time.perf_counter()
+        path = Execute.run_vectors(ir=ir, args=args, block=block, grid=grid)
+        Transfer.flush()
+        times.append((time.perf_counter() - t0) * 1e3)
+    p = np.stack(pos)                                # doubles, as cpu_nbody takes them
+    verified = True
+    for lo in range(0, n, 512):                      # rows of the pair matrix in slabs
+        rows = np.arange(lo, min(lo + 512, n))
+        d = p[:, None, :] - p[:, rows, None]
+        dist2 = (d ** 2).sum(0) + 1e-9
+        w = 1.0 / (np.sqrt(dist2) * dist2)
+        w[rows - lo, rows] = 0.0                     # j <> i
+        exp = (d * w[None]).sum(2)
+        for c in range(3):
+            diff = np.abs(vacc[c].to_array()[rows].astype(np.float64) - exp[c])
+            verified = verified and not bool(np.any((diff > 1e-3) & (diff / (np.abs(exp[c]) + 1e-9) > 1e-3)))
+    return _device_record(times, float(n) * n / (statistics.median(times) / 1e3) / 1e9, verified, path,
+                          "Ginteraction/s")
+
+
+def bench_bitonic_sort(size, warmup=5, iterations=20):
+    """benchmarks/bench_bitonic_sort.ml:58-215: n = the power of two at or below size, random values
+    below 10000 written again before every sort (so the upload is inside the sample), log^2 n
+    launches per sort, result equal to the sorted input, M elements/s = n / median."""
+    n = 1 << int(np.log2(size))
+    data = _ocaml_random_ints(n, 10000)
+    v = _vector(data, Vector.int32)
+    ir = reference_kernels.bitonic_sort_step()
+    block, grid = Execute.dims1d(256), Execute.dims1d((n + 255) // 256)
+
+    def sort():
+        path, k = None, 2
+        while k <= n:
+            j = k // 2
+            while j >= 1:
+                path = Execute.run_vectors(ir=ir, args=[Execute.Vec(v), Execute.Int32(j), Execute.Int32(k),
+                                                        Execute.Int32(n)], block=block, grid=grid)
+                j //= 2
+            k *= 2
+        return path
+    path = None
+    for _ in range(warmup):
+        v.fill_from(data)
+        path = sort()
+        Transfer.flush()
+    times = []
+    for _ in range(iterations):
+        v.fill_from(data)
+        t0 = time.perf_counter()
+        path = sort()
+        Transfer.flush()
+        times.append((time.perf_counter() - t0) * 1e3)
+    verified = bool(np.array_equal(v.to_array(), np.sort(data)))
+    return _device_record(times, n / (statistics.median(times) / 1e3 * 1e6), verified, path, "Melem/s")
+
+
+def bench_radix_sort(size, warmup=5, iterations=20):
+    """benchmarks/bench_radix_sort.ml:118-350: ONE 8-bit pass (the reference's `_num_passes = 1`):
+    per-block histogram kernel, histogram back to the host, exclusive prefix sum there, counters up,
+    scatter kernel with atomic slot allocation; the output must be ordered by its low 8 bits;
+    M elements/s = n / median of the whole pass, uploads included."""
+    n, bins, mask, shift = size, 256, 255, 0
+    data = _ocaml_random_ints(n, 100000)
+    hist_ir, scatter_ir = reference_kernels.radix_sort_histogram(), reference_kernels.radix_sort_scatter()
+    block, grid = Execute.dims1d(256), Execute.dims1d((n + 255) // 256)
+
+    def init():
+        return (_vector(data, Vector.int32), Vector.create(Vector.int32, n), Vector.create(Vector.int32, bins),
+                Vector.create(Vector.int32, bins))
+
+    def compute(vs):
+        vin, vout, hist, counters = vs
+        vin.fill_from(data)
+        Transfer.to_device(vin)
+        hist.fill_from(np.zeros(bins))
+        Transfer.to_device(hist)
+        Execute.run_vectors(ir=hist_ir, args=[Execute.Vec(vin), Execute.Vec(hist), Execute.Int32(n), Execute.Int32(shift),
+                                              Execute.Int32(mask)], block=block, grid=grid)
+        Transfer.flush()
+        Transfer.to_cpu(hist, force=True)
+        h = hist.to_array().astype(np.int64)
+        counters.fill_from(np.concatenate(([0], np.cumsum(h)[:-1])))
+        Transfer.to_device(counters)
+        path = Execute.run_vectors(ir=scatter_ir, args=[Execute.Vec(vin), Execute.Vec(vout), Execute.Vec(counters),
+                                                        Execute.Int32(n), Execute.Int32(shift), Execute.Int32(mask)],
+                                   block=block, grid=grid)
+        Transfer.flush()
+        Transfer.to_cpu(counters, force=True)
+        return path
+    times, path, (_, vout, _, _) = _benchmark_gpu(init, compute, warmup, iterations)
+    Transfer.to_cpu(vout, force=True)
+    out = vout.to_array()
+    verified = bool(np.all(np.diff(out & 255) >= 0)) and bool(np.array_equal(np.sort(out), np.sort(data)))
+    return _device_record(times, n / (statistics.median(times) / 1e3 * 1e6), verified, path, "Melem/s")
+
+
 def bench_transfer(size, warmup=2, iterations=7):
     """Not one of the reference's programs: the Transfer.to_device / Transfer.to_cpu legs
     (sarek/core/Transfer.ml:228-333) that its benches run once before and after their timed
@@ -330,6 +607,15 @@ BENCHMARKS = {
     "transpose": (bench_transpose, [256, 512, 1024, 2048, 4096, 8192]),                     # warmup 10
     "transpose_tiled": (bench_transpose_tiled, [256, 512, 1024, 2048, 4096, 8192]),         # warmup 10
     "scan": (bench_scan, [64, 128, 256]),
+    "gather": (bench_gather, [1_000_000, 10_000_000, 50_000_000]),          # bench_gather_scatter.ml, first half
+    "scatter": (bench_scatter, [1_000_000, 10_000_000, 50_000_000]),        # second half
+    "histogram": (bench_histogram, [1_000_000, 10_000_000, 50_000_000]),
+    "stencil_2d": (bench_stencil_2d, [256, 512, 1024, 2048]),
+    "conv2d": (bench_conv2d, [256, 512, 1024, 2048]),
+    "mandelbrot": (bench_mandelbrot, [512, 1024, 2048, 4096]),              # warmup 10
+    "nbody": (bench_nbody, [512, 1024, 2048, 4096]),
+    "bitonic_sort": (bench_bitonic_sort, [1024, 4096, 16384]),
+    "radix_sort": (bench_radix_sort, [1_000_000, 10_000_000, 50_000_000]),
     "transfer": (bench_transfer, [1_000_000, 10_000_000, 100_000_000, 268_435_456]),   # no such program there
 }
 

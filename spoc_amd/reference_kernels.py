@@ -389,6 +389,138 @@ def inclusive_scan():
     return kernel(params, body)
 
 
+def histogram():
+    """benchmarks/bench_histogram.ml:54-84 (= sarek/tests/e2e/test_histogram.ml:43-69): per-block
+    histogram in shared memory by atomic adds, merged into the global one by atomic adds."""
+    fresh()
+    params = [("input", "(vec i32)"), ("histogram", "(vec i32)"), ("n", "i32"), ("num_bins", "i32")]
+    for p, t in params:
+        var(p, t)
+    nn, nb = var("n"), var("num_bins")
+    lh = var("local_hist", "(array i32 shared)")
+    tid, gid, b = var("tid"), var("gid"), var("bin")
+    old1, old2 = var("_old"), var("_old#2").replace("_old#2", "_old", 1)
+    count = if_(lt(gid, nn), let(b, mod(read("input", gid), nb),
+                                 let(old1, intr("atomic_add_int32", "Gpu", lh, b, i32(1)), "(expr (unit))")))
+    merge = if_(lt(tid, nb), let(old2, intr("atomic_add_global_int32", "Gpu", var("histogram", "(vec i32)"), tid,
+                                            read("local_hist", tid)), "(expr (unit))"))
+    body = shared(lh, "i32", 256, lets(
+        [(tid, intr("thread_idx_x")), (gid, intr("global_thread_id", "Std"))],
+        seq(block(if_(lt(tid, nb), assign_elem("local_hist", tid, i32(0)))), BARRIER,
+            seq(block(count), BARRIER, seq(block(merge), BARRIER, "(expr (unit))")))))
+    return kernel(params, body)
+
+
+def stencil_2d():
+    """benchmarks/bench_stencil_2d.ml:43-58: five-point mean over the interior of a 2-D grid."""
+    fresh()
+    params = [("input", "(vec f32)"), ("output", "(vec f32)"), ("width", "i32"), ("height", "i32")]
+    for p, t in params:
+        var(p, t)
+    w, h = var("width"), var("height")
+    x, y, idx = var("x"), var("y"), var("idx")
+    names = ["up", "down", "left", "right", "center"]
+    up, down, left, right, center = (var(n, "f32") for n in names)
+    inside = land(land(land(gt(x, i32(0)), lt(x, sub(w, i32(1)))), gt(y, i32(0))), lt(y, sub(h, i32(1))))
+    mean = div(add(add(add(add(up, down), left), right), center), f32("5.0"))
+    inner = lets([(idx, add(mul(y, w), x)),
+                  (up, read("input", add(mul(sub(y, i32(1)), w), x))),
+                  (down, read("input", add(mul(add(y, i32(1)), w), x))),
+                  (left, read("input", sub(add(mul(y, w), x), i32(1)))),
+                  (right, read("input", add(add(mul(y, w), x), i32(1)))),
+                  (center, read("input", idx))], assign_elem("output", idx, mean))
+    body = lets([(x, add(intr("thread_idx_x"), mul(intr("block_idx_x"), intr("block_dim_x")))),
+                 (y, add(intr("thread_idx_y"), mul(intr("block_idx_y"), intr("block_dim_y"))))], if_(inside, inner))
+    return kernel(params, body)
+
+
+def conv2d():
+    """benchmarks/bench_conv2d.ml:49-77: 3x3 box filter, one thread per pixel of a 1-D launch,
+    zero on the border."""
+    fresh()
+    params = [("input", "(vec f32)"), ("output", "(vec f32)"), ("width", "i32"), ("height", "i32")]
+    for p, t in params:
+        var(p, t)
+    w, h = var("width"), var("height")
+    tid, n, x, y = var("tid"), var("n"), var("x"), var("y")
+    border = op("or", op("or", op("or", eq(x, i32(0)), eq(x, sub(w, i32(1)))), eq(y, i32(0))), eq(y, sub(h, i32(1))))
+    taps, binds = [], []
+    for r, dy in enumerate((-1, 0, 1)):
+        row = y if dy == 0 else (sub(y, i32(1)) if dy < 0 else add(y, i32(1)))
+        for c, dx in enumerate((-1, 0, 1)):
+            at = add(mul(row, w), x)
+            at = at if dx == 0 else (sub(at, i32(1)) if dx < 0 else add(at, i32(1)))
+            v = var(f"p{r}{c}", "f32")
+            taps.append(v)
+            binds.append((v, read("input", at)))
+    total = taps[0]
+    for t in taps[1:]:
+        total = add(total, t)
+    s = var("sum", "f32")
+    inner = lets(binds, let(s, total, assign_elem("output", tid, div(s, f32("9.0")))))
+    body = lets([(tid, intr("global_thread_id", "Std")), (n, mul(w, h))],
+                if_(lt(tid, n), lets([(x, mod(tid, w)), (y, div(tid, w))],
+                                     if_(border, assign_elem("output", tid, f32("0.0")), inner))))
+    return kernel(params, body)
+
+
+def bitonic_sort_step():
+    """benchmarks/bench_bitonic_sort.ml:39-56: one compare-exchange step of a bitonic network."""
+    fresh()
+    params = [("data", "(vec i32)"), ("j", "i32"), ("k", "i32"), ("n", "i32")]
+    for p, t in params:
+        var(p, t)
+    i, ij, di, dij, asc = var("i"), var("ij"), var("di"), var("dij"), var("ascending", "bool")
+    cond = op("or", land(asc, gt(di, dij)), land(f"(not {asc})", lt(di, dij)))
+    body = let(i, intr("global_thread_id", "Std"), if_(lt(i, var("n")), let(
+        ij, op("bitxor", i, var("j")), if_(gt(ij, i), lets(
+            [(di, read("data", i)), (dij, read("data", ij)), (asc, eq(op("bitand", i, var("k")), i32(0)))],
+            if_(cond, seq(assign_elem("data", i, dij), assign_elem("data", ij, di))))))))
+    return kernel(params, body)
+
+
+def nbody_accel():
+    """benchmarks/bench_nbody.ml:63-105: accelerations of n bodies, all pairs; positions go through
+    a record built by a helper function."""
+    part = "(record particle (x f32) (y f32) (z f32))"
+    P, Q = f"(var p 20 {part})", f"(var q 21 {part})"
+
+    def mk(idx):
+        return f"(app (var make_p 0 {part}) (read xs {idx}) (read ys {idx}) (read zs {idx}))"
+    tid, iv, jv = "(var tid 8 i32)", "(var i 18 i32)", "(var j 9 i32 mut)"
+    fx, fy, fz = ("(var f%s %d f32 mut)" % (c, 10 + k) for k, c in enumerate("xyz"))
+    dx, dy, dz = ("(var d%s %d f32)" % (c, 13 + k) for k, c in enumerate("xyz"))
+    dist2, inv = "(var dist2 16 f32)", "(var inv 17 f32)"
+    return f"""(kernel sarek_kern
+      (params (param (var xs 1 (vec f32))) (param (var ys 2 (vec f32))) (param (var zs 3 (vec f32)))
+              (param (var ax 4 (vec f32))) (param (var ay 5 (vec f32))) (param (var az 6 (vec f32)))
+              (param (var n 7 i32)))
+      (locals)
+      (body (let {tid} (add (intr (Gpu) thread_idx_x) (mul (intr (Gpu) block_idx_x) (intr (Gpu) block_dim_x)))
+        (if (lt {tid} (var n 7 i32))
+          (let {P} {mk(tid)}
+          (letmut {fx} (f32 0.0) (letmut {fy} (f32 0.0) (letmut {fz} (f32 0.0)
+          (let {iv} {tid}
+           (seq
+            (for {jv} (i32 0) (sub (var n 7 i32) (i32 1)) upto
+              (if (ne {jv} {iv})
+                (let {Q} {mk(jv)}
+                (let {dx} (sub (field {Q} x) (field {P} x))
+                (let {dy} (sub (field {Q} y) (field {P} y))
+                (let {dz} (sub (field {Q} z) (field {P} z))
+                (let {dist2} (add (add (add (mul {dx} {dx}) (mul {dy} {dy})) (mul {dz} {dz})) (f32 1e-9))
+                (let {inv} (div (f32 1.0) (mul (intr (Float32) sqrt {dist2}) {dist2}))
+                  (seq (assign (lvar {fx}) (add {fx} (mul {dx} {inv})))
+                       (assign (lvar {fy}) (add {fy} (mul {dy} {inv})))
+                       (assign (lvar {fz}) (add {fz} (mul {dz} {inv}))))))))))))
+            (assign (lelem ax {tid}) {fx}) (assign (lelem ay {tid}) {fy}) (assign (lelem az {tid}) {fz}))))))))))
+      (types (particle (x f32) (y f32) (z f32)))
+      (funcs (func make_p (params (var x 30 f32) (var y 31 f32) (var z 32 f32)) {part}
+               (return (record particle (x (var x 30 f32)) (y (var y 31 f32)) (z (var z 32 f32))))))
+      (native_fn true))
+"""
+
+
 KERNELS = {
     "stream_triad": stream_triad, "vector_add": vector_add, "vector_copy": vector_copy,
     "matrix_mul": matrix_mul, "matrix_mul_tiled": matrix_mul_tiled,
