@@ -341,6 +341,19 @@ int sarek_hip_copy_f32(float *dst, const float *src, int64_t n, sarek_hip_stream
  * of `width` floats).  in and out must not overlap.                                 */
 int sarek_hip_transpose_f32(const float *in, float *out, int width, int height, sarek_hip_stream stream);
 
+/* histogram[b] += #{ i < n : keys[i] mod num_bins == b } for b < num_bins, 1 <= num_bins <= 256:
+ * what a launch of the kernel of benchmarks/bench_histogram.ml:54-84 over n keys adds to the
+ * global histogram (`mod` is the generated code's `%`: a negative key with a non-zero
+ * remainder has no bin and is not counted, where that kernel indexes its shared array with
+ * it).  The histogram is accumulated into, not cleared; keys 16-byte aligned.          */
+int sarek_hip_histogram_i32(int32_t *histogram, const int32_t *keys, int64_t n, int num_bins,
+                            sarek_hip_stream stream);
+/* histogram[d] += #{ i < n : (keys[i] >> shift) & mask == d }, 256 bins, 0 <= mask <= 255,
+ * 0 <= shift <= 31: the counting kernel of one radix-sort pass,
+ * benchmarks/bench_radix_sort.ml:82-116 (`>>` as in the generated code: arithmetic).   */
+int sarek_hip_radix_histogram_i32(int32_t *histogram, const int32_t *keys, int64_t n, int shift, int mask,
+                                  sarek_hip_stream stream);
+
 /* Row-major GEMM  C[m x n] = A[m x k] . B[k x n]  (replaces the generated
  * 16x16 tiled kernel, matrix_mul_tiled_generated.md:9-50; source
  * benchmarks/bench_matrix_mul_tiled.ml:55-95).  Any m,n,k >= 1.            */

@@ -16,7 +16,7 @@ __all__ = [
     "build", "fill_uniform", "round_bf16", "round_f16", "bf16_bits", "f16_bits",
     "triad", "reduce_sum_block256", "reduce_max_block256", "dot_block256", "fold_partials", "triad_sum",
     "gemm", "gemm_rows", "gemm_bias_relu_rowsum", "matmul_tiled_bsp",
-    "vector_add", "vector_copy", "transpose", "matmul_naive",
+    "vector_add", "vector_copy", "transpose", "histogram", "radix_histogram", "matmul_naive",
 ]
 
 
@@ -225,6 +225,32 @@ def vector_copy(a, out, n, threads=None):
     assert out.dtype == np.float32 and out.flags.c_contiguous
     _L().oracle_vector_copy_f32(ap, out.ctypes.data_as(C.POINTER(C.c_float)), n, _launch_size(n, threads))
     return out
+
+
+def _i32(x):
+    x = np.ascontiguousarray(x, dtype=np.int32)
+    return x, x.ctypes.data_as(C.POINTER(C.c_int32))
+
+
+def histogram(keys, hist, n, num_bins, block=256, grid=None, stale=-7):
+    """Adds the launch's counts to `hist` (int32, in place); returns the number of keys without a slot."""
+    keys, kp = _i32(keys)
+    assert hist.dtype == np.int32 and hist.flags.c_contiguous
+    grid = (n + block - 1) // block if grid is None else grid
+    f = _L().oracle_histogram_i32
+    f.restype = C.c_int64
+    return f(kp, hist.ctypes.data_as(C.POINTER(C.c_int32)), C.c_int32(n), C.c_int32(num_bins), C.c_int32(block),
+             C.c_int32(grid), C.c_int32(stale))
+
+
+def radix_histogram(keys, hist, n, shift, mask, block=256, grid=None, stale=-7):
+    keys, kp = _i32(keys)
+    assert hist.dtype == np.int32 and hist.flags.c_contiguous
+    grid = (n + block - 1) // block if grid is None else grid
+    f = _L().oracle_radix_histogram_i32
+    f.restype = C.c_int64
+    return f(kp, hist.ctypes.data_as(C.POINTER(C.c_int32)), C.c_int32(n), C.c_int32(shift), C.c_int32(mask),
+             C.c_int32(block), C.c_int32(grid), C.c_int32(stale))
 
 
 def transpose(x, width, height, out=None, threads=None):

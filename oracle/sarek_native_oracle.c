@@ -445,6 +445,59 @@ void oracle_vector_copy_f32(const float *a, float *b, int64_t n, int64_t threads
     if (tid < n) b[tid] = a[tid];
 }
 
+/* benchmarks/bench_histogram.ml:54-84, block by block: a 256-slot block histogram, the slots below
+ * min(block, num_bins) cleared, one count per thread with gid < n, the same slots added to the global
+ * histogram.  Int32.rem has the sign of the key (sarek/ppx/Sarek_native_gen.ml, Mod on int32); a key whose
+ * slot is outside 0..255 would index the shared array out of bounds: it is skipped and counted in the
+ * return value, so a test can insist on 0.  Slots never cleared start at `stale` (any value: they are
+ * never merged, so it must not show).                                                                    */
+int64_t oracle_histogram_i32(const int32_t *input, int32_t *histogram, int32_t n, int32_t num_bins,
+                             int32_t block, int32_t grid, int32_t stale) {
+  int64_t skipped = 0;
+  for (int32_t b = 0; b < grid; ++b) {
+    int32_t local_hist[256];
+    for (int i = 0; i < 256; ++i) local_hist[i] = stale;
+    for (int32_t tid = 0; tid < block; ++tid)
+      if (tid < num_bins && tid < 256) local_hist[tid] = 0;
+    for (int32_t tid = 0; tid < block; ++tid) {
+      const int64_t gid = (int64_t)b * block + tid;
+      if (gid < n) {
+        const int32_t bin = input[gid] % num_bins;
+        if (bin < 0 || bin > 255) ++skipped;
+        else local_hist[bin] += 1;
+      }
+    }
+    for (int32_t tid = 0; tid < block; ++tid)
+      if (tid < num_bins && tid < 256) histogram[tid] = (int32_t)((uint32_t)histogram[tid] + (uint32_t)local_hist[tid]);
+  }
+  return skipped;
+}
+
+/* The counting kernel of benchmarks/bench_radix_sort.ml:82-116 the same way: digit =
+ * (value lsr shift) land mask, logical shift as the Native backend computes it
+ * (sarek/ppx/Sarek_native_gen.ml:809-815), 256 slots.                                                    */
+int64_t oracle_radix_histogram_i32(const int32_t *input, int32_t *histogram, int32_t n, int32_t shift,
+                                   int32_t mask, int32_t block, int32_t grid, int32_t stale) {
+  int64_t skipped = 0;
+  for (int32_t b = 0; b < grid; ++b) {
+    int32_t local_hist[256];
+    for (int i = 0; i < 256; ++i) local_hist[i] = stale;
+    for (int32_t tid = 0; tid < block; ++tid)
+      if (tid < 256) local_hist[tid] = 0;
+    for (int32_t tid = 0; tid < block; ++tid) {
+      const int64_t gid = (int64_t)b * block + tid;
+      if (gid < n) {
+        const int32_t digit = (int32_t)((uint32_t)input[gid] >> shift) & mask;
+        if (digit < 0 || digit > 255) ++skipped;
+        else local_hist[digit] += 1;
+      }
+    }
+    for (int32_t tid = 0; tid < block; ++tid)
+      if (tid < 256) histogram[tid] = (int32_t)((uint32_t)histogram[tid] + (uint32_t)local_hist[tid]);
+  }
+  return skipped;
+}
+
 void oracle_transpose_f32(const float *input, float *output, int32_t width, int32_t height, int64_t threads) {
   const int32_t n = width * height;
   for (int64_t tid = 0; tid < threads; ++tid)

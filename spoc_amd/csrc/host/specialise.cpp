@@ -6,7 +6,8 @@
 // benchmarks/bench_stream_triad.ml:22-32, benchmarks/bench_reduction.ml:62-96,
 // benchmarks/bench_dot_product.ml:16-54 and benchmarks/bench_reduction_max.ml:18-100 in the
 // reference, the last with any constant as the out-of-range fill; and the vector add, vector
-// copy, one-thread-per-element matmul and the two transposes).  Anything else gets the plain
+// copy, one-thread-per-element matmul, the two transposes, the histogram and the counting
+// kernel of the radix sort).  Anything else gets the plain
 // lowering: a miss costs speed, never correctness.
 //
 // Normalisation removes what the front end is free to vary without changing meaning:
@@ -144,6 +145,15 @@ struct Canon {
     }
   }
 
+  // An expression whose evaluation changes memory (the atomic read-modify-write intrinsics).
+  static bool has_effect(const ExprP &e) {
+    if (!e) return false;
+    if (e->kind == Expr::Intrinsic && e->name.compare(0, 6, "atomic") == 0) return true;
+    for (auto &a : e->args)
+      if (has_effect(a)) return true;
+    return false;
+  }
+
   std::string lvalue(const LValueP &l) {
     switch (l->kind) {
       case LValue::LVar: {
@@ -191,6 +201,11 @@ struct Canon {
           std::string v = bind(s.var);
           out.push_back("(array " + v + " " + type_tag(s.e->type) + " " + sz +
                         (s.e->mem == MemSpace::Shared ? " shared)" : " local)"));
+        } else if (has_effect(s.e)) {
+          // an atomic returns the old value and changes memory: the binding stays a statement
+          std::string val = expr(s.e);
+          std::string v = bind(s.var);
+          out.push_back("(bind " + v + " " + val + ")");
         } else {
           // substitute the value, rendered now so that it is closed over the bindings
           // in force at this point; carried in an Intrinsic node whose name starts
@@ -213,7 +228,9 @@ struct Canon {
       case Stmt::WarpBarrier: out.push_back("(warpbarrier)"); return;
       case Stmt::MemFence: out.push_back("(memfence)"); return;
       case Stmt::Return: out.push_back("(return " + expr(s.e) + ")"); return;
-      case Stmt::ExprS: out.push_back("(do " + expr(s.e) + ")"); return;
+      case Stmt::ExprS:
+        if (s.e->kind != Expr::ConstUnit) out.push_back("(do " + expr(s.e) + ")");   // `()` does nothing
+        return;
       case Stmt::Match: out.push_back("(match?)"); return;
       case Stmt::Native: out.push_back("(native?)"); return;
     }
@@ -341,6 +358,55 @@ const char *kVectorCopy = R"IR(
  (body
  (let (var tid 4 i32) (intr (Std) global_thread_id)
  (if (lt (var tid 4 i32) (var n 3 i32)) (assign (lelem b (var tid 4 i32)) (read a (var tid 4 i32))))))
+ (native_fn true))
+)IR";
+
+// benchmarks/bench_histogram.ml:54-84 and the counting kernel of benchmarks/bench_radix_sort.ml:82-116.
+const char *kHistogram = R"IR(
+(kernel sarek_kern
+ (params (param (var input 1 (vec i32))) (param (var histogram 2 (vec i32))) (param (var n 3 i32)) (param (var num_bins 4 i32)))
+ (locals)
+ (body
+ (let (var local_hist 5 (array i32 shared)) (newarray i32 (i32 256) shared)
+ (let (var tid 6 i32) (intr (Gpu) thread_idx_x)
+ (let (var gid 7 i32) (intr (Std) global_thread_id)
+ (seq
+  (block (if (lt (var tid 6 i32) (var num_bins 4 i32)) (assign (lelem local_hist (var tid 6 i32)) (i32 0))))
+  (barrier)
+  (block (if (lt (var gid 7 i32) (var n 3 i32))
+    (let (var bin 8 i32) (mod (read input (var gid 7 i32)) (var num_bins 4 i32))
+    (let (var _old 9 i32) (intr (Gpu) atomic_add_int32 (var local_hist 5 (array i32 shared)) (var bin 8 i32) (i32 1))
+     (expr (unit))))))
+  (barrier)
+  (block (if (lt (var tid 6 i32) (var num_bins 4 i32))
+    (let (var _old 10 i32) (intr (Gpu) atomic_add_global_int32 (var histogram 2 (vec i32)) (var tid 6 i32) (read local_hist (var tid 6 i32)))
+     (expr (unit)))))
+  (barrier))))))
+ (native_fn true))
+)IR";
+
+const char *kRadixHistogram = R"IR(
+(kernel sarek_kern
+ (params (param (var input 1 (vec i32))) (param (var histogram 2 (vec i32))) (param (var n 3 i32)) (param (var shift 4 i32)) (param (var mask 5 i32)))
+ (locals)
+ (body
+ (let (var local_hist 6 (array i32 shared)) (newarray i32 (i32 256) shared)
+ (let (var tid 7 i32) (intr (Gpu) thread_idx_x)
+ (let (var gid 8 i32) (intr (Std) global_thread_id)
+ (let (var num_bins 9 i32) (i32 256)
+ (seq
+  (block (if (lt (var tid 7 i32) (var num_bins 9 i32)) (assign (lelem local_hist (var tid 7 i32)) (i32 0))))
+  (barrier)
+  (block (if (lt (var gid 8 i32) (var n 3 i32))
+    (let (var value 10 i32) (read input (var gid 8 i32))
+    (let (var digit 11 i32) (bitand (shr (var value 10 i32) (var shift 4 i32)) (var mask 5 i32))
+    (let (var _old 12 i32) (intr (Gpu) atomic_add_int32 (var local_hist 6 (array i32 shared)) (var digit 11 i32) (i32 1))
+     (empty))))))
+  (barrier)
+  (block (if (lt (var tid 7 i32) (var num_bins 9 i32))
+    (let (var _old 13 i32) (intr (Gpu) atomic_add_global_int32 (var histogram 2 (vec i32)) (var tid 7 i32) (read local_hist (var tid 7 i32)))
+     (empty))))
+  (barrier)))))))
  (native_fn true))
 )IR";
 
@@ -500,6 +566,8 @@ std::string recognise(const Kernel &k) {
   static const std::string t_naive = canon_kernel(parse_kernel(kMatmulNaive));
   static const std::string t_tr_naive = canon_kernel(parse_kernel(kTransposeNaive));
   static const std::string t_tr_tiled = strip_trailing_barrier(canon_kernel(parse_kernel(kTransposeTiled)));
+  static const std::string t_hist = strip_trailing_barrier(canon_kernel(parse_kernel(kHistogram)));
+  static const std::string t_radix_hist = strip_trailing_barrier(canon_kernel(parse_kernel(kRadixHistogram)));
   const std::string c = canon_kernel(k);
   if (c == t_matmul) return "matmul_tiled_f32";
   if (c == t_triad) return "stream_triad_f32";
@@ -509,6 +577,8 @@ std::string recognise(const Kernel &k) {
   if (c == t_tr_naive) return "transpose_naive_f32";
   const std::string cs = strip_trailing_barrier(c);
   if (cs == t_tr_tiled) return "transpose_tiled_f32";
+  if (cs == t_hist) return "histogram_i32";
+  if (cs == t_radix_hist) return "radix_histogram_i32";
   if (cs == t_reduce) return "reduce_sum_block256_f32";
   if (cs == t_dot) return "dot_block256_f32";
   const std::string pad = match_max_tree(cs);

@@ -162,6 +162,33 @@ int try_specialised(const std::string &tag, const int block[3], const int grid[3
                                   (int)w, (int)h, nullptr);
     return 1;
   }
+  if (tag == "histogram_i32" || tag == "radix_histogram_i32") {
+    // (input, len, histogram, len, n, num_bins) or (input, len, histogram, len, n, shift, mask).  Each block
+    // clears and merges the bins below its own size, so a block at least as wide as the bin range makes the
+    // launch a plain histogram of the keys its threads reach.
+    const bool radix = tag[0] == 'r';
+    if (n_args != (radix ? 7 : 6) || !vec_at(args, n_args, 0) || !vec_at(args, n_args, 2)) return 0;
+    for (int i = 4; i < n_args; ++i)
+      if (!is_i32(args[i])) return 0;
+    if (block[1] != 1 || block[2] != 1 || grid[1] != 1 || grid[2] != 1) return 0;
+    const int64_t reach = static_cast<int64_t>(block[0]) * grid[0];
+    const int64_t n = args[4].i32 < reach ? args[4].i32 : reach;
+    const int bins = radix ? 256 : args[5].i32;
+    if (n < 0 || bins < 1 || bins > 256 || block[0] < bins) return 0;
+    // up to a shift of 24 the eight digit bits are key bits whichever way `shr` fills from the left
+    // (the reference's GPU code has `>>` on int, its Native backend Int32.shift_right_logical)
+    if (radix && (args[5].i32 < 0 || args[5].i32 > 24 || args[6].i32 < 0 || args[6].i32 > 255)) return 0;
+    if (args[0].length < n || args[2].length < bins) return 0;
+    const uintptr_t in = reinterpret_cast<uintptr_t>(args[0].buffer), hist = reinterpret_cast<uintptr_t>(args[2].buffer);
+    if (in < hist + static_cast<uintptr_t>(bins) * 4 && hist < in + static_cast<uintptr_t>(n) * 4) return 0;
+    if (in & 15) return 0;
+    *rc = radix ? sarek_hip_radix_histogram_i32(static_cast<int32_t *>(args[2].buffer),
+                                                static_cast<const int32_t *>(args[0].buffer), n, args[5].i32,
+                                                args[6].i32, nullptr)
+                : sarek_hip_histogram_i32(static_cast<int32_t *>(args[2].buffer),
+                                          static_cast<const int32_t *>(args[0].buffer), n, bins, nullptr);
+    return 1;
+  }
   if (tag == "reduce_sum_block256_f32" || tag == "dot_block256_f32") {
     const bool dot = tag[0] == 'd';
     const int nv = dot ? 3 : 2;

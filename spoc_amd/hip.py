@@ -115,6 +115,8 @@ SYMBOLS = {
     "sarek_hip_fold_partials_f64": (_i, [_vp, _i64, _vp, _vp]),
     "sarek_hip_copy_f32": (_i, [_vp, _vp, _i64, _vp]),
     "sarek_hip_transpose_f32": (_i, [_vp, _vp, _i, _i, _vp]),
+    "sarek_hip_histogram_i32": (_i, [_vp, _vp, _i64, _i, _vp]),
+    "sarek_hip_radix_histogram_i32": (_i, [_vp, _vp, _i64, _i, _i, _vp]),
     "sarek_hip_gemm_f32": (_i, [_vp, _vp, _vp, _i, _i, _i, _vp]),
     "sarek_hip_gemm_bf16": (_i, [_vp, _vp, _vp, _i, _i, _i, _vp]),
     "sarek_hip_gemm_f16": (_i, [_vp, _vp, _vp, _i, _i, _i, _vp]),
@@ -432,6 +434,28 @@ def transpose(x, out=None):
         raise ValueError("transpose: out has the wrong size")
     check(lib.sarek_hip_transpose_f32(_ptr(x), _ptr(out), w, h, _stream()))
     return out
+
+
+def histogram(keys, hist, num_bins):
+    """hist[b] += #{keys mod num_bins == b} (bench_histogram's kernel over all the keys)."""
+    torch = _torch()
+    _need(keys, torch.int32, "keys")
+    _need(hist, torch.int32, "hist")
+    if hist.numel() < num_bins:
+        raise ValueError("histogram: hist is shorter than num_bins")
+    check(lib.sarek_hip_histogram_i32(_ptr(hist), _ptr(keys), keys.numel(), num_bins, _stream()))
+    return hist
+
+
+def radix_histogram(keys, hist, shift, mask=255):
+    """hist[d] += #{(keys >> shift) & mask == d}, 256 bins (bench_radix_sort's counting kernel)."""
+    torch = _torch()
+    _need(keys, torch.int32, "keys")
+    _need(hist, torch.int32, "hist")
+    if hist.numel() < 256:
+        raise ValueError("radix_histogram: hist has fewer than 256 bins")
+    check(lib.sarek_hip_radix_histogram_i32(_ptr(hist), _ptr(keys), keys.numel(), shift, mask, _stream()))
+    return hist
 
 
 def gemm_f32(a, b, out=None):

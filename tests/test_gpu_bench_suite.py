@@ -11,7 +11,7 @@ pytestmark = pytest.mark.gpu
 
 
 @pytest.mark.parametrize("name,size", [
-    ("gather", 100003), ("scatter", 100003), ("histogram", 100003), ("histogram", 200),
+    ("gather", 100003), ("scatter", 100003),
     ("stencil_2d", 200), ("conv2d", 200), ("conv2d", 37), ("mandelbrot", 100), ("nbody", 300),
     ("bitonic_sort", 1024), ("bitonic_sort", 3000), ("radix_sort", 100003)])
 def test_suite_runs_and_verifies(hip, torch_cuda, name, size):

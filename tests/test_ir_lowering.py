@@ -22,6 +22,7 @@ EXPECTED_TAGS = {
     "reduction": "reduce_sum_block256_f32", "dot_product": "dot_block256_f32",
     "vector_add": "vector_add_f32", "vector_copy": "vector_copy_f32", "matrix_mul": "matmul_naive_f32",
     "transpose_naive": "transpose_naive_f32", "transpose_tiled": "transpose_tiled_f32",
+    "radix_sort_histogram": "radix_histogram_i32",
 }
 
 
@@ -261,6 +262,41 @@ def test_data_movement_and_naive_matmul_near_misses_fall_back(hip):
     assert tag_of("transpose_tiled", "(i32 17)", "(i32 16)") == ""
     assert tag_of("transpose_tiled", "(lt (var write_col 15 i32) (var height 4 i32))",
                   "(lt (var write_col 15 i32) (var width 3 i32))") == ""
+
+
+def test_histogram_recognition_and_near_misses(hip):
+    from spoc_amd import reference_kernels
+    hist = reference_kernels.histogram()
+    assert split_tag(hip.generate_source(hist))[0] == "histogram_i32"
+    # `()` and the empty statement are the same nothing
+    assert split_tag(hip.generate_source(hist.replace("(expr (unit))", "(empty)")))[0] == "histogram_i32"
+    assert split_tag(hip.generate_source(hist.replace("(i32 256)", "(i32 128)")))[0] == ""       # smaller block histogram
+    assert split_tag(hip.generate_source(hist.replace("(mod (read input", "(div (read input")))[0] == ""
+    assert split_tag(hip.generate_source(hist.replace("(i32 1))", "(i32 2))", 1)))[0] == ""       # counts by two
+    assert split_tag(hip.generate_source(hist.replace("(barrier)", "(empty)", 1)))[0] == ""
+    radix = open(os.path.join(IR_DIR, "radix_sort_histogram.ir")).read()
+    assert split_tag(hip.generate_source(radix.replace("(shr ", "(shl ")))[0] == ""
+    assert split_tag(hip.generate_source(radix.replace("(read local_hist (var tid 7 i32)))", "(i32 1))", 1)))[0] == ""
+
+
+def test_an_atomic_in_an_unused_binding_is_part_of_the_program(hip):
+    """`let _old = atomic_add ... in` binds a value nobody reads, and still changes memory: a triad
+    that also counts its calls is not the triad."""
+    expr = f"(add {B} (mul {Cc} {S}))"
+    counted = kernel_with_body(
+        "(let (var tid 6 i32) (intr (Std) global_thread_id) (if (lt (var tid 6 i32) (var n 5 i32)) "
+        "(let (var _old 7 i32) (intr (Gpu) atomic_add_global_int32 (var hits 8 (vec i32)) (i32 0) (i32 1)) "
+        f"(assign (lelem a (var tid 6 i32)) {expr}))))",
+        "(param (var a 1 (vec f32))) (param (var b 2 (vec f32))) (param (var c 3 (vec f32))) "
+        "(param (var scalar 4 f32)) (param (var n 5 i32)) (param (var hits 8 (vec i32)))")
+    tag, src = split_tag(hip.generate_source(counted))
+    assert tag == "" and "atomicAdd" in src
+    # five parameters, the atomic on `a` reinterpreted is still an atomic: not taken either
+    same_params = triad_ir(expr).replace(
+        "(assign (lelem a", "(let (var _old 7 i32) (intr (Gpu) atomic_add_global_int32 (var a 1 (vec f32)) (i32 0) (i32 1)) "
+        "(assign (lelem a", 1).replace(f"{expr})))", f"{expr}))))", 1)
+    assert split_tag(hip.generate_source(triad_ir(expr)))[0] == "stream_triad_f32"
+    assert split_tag(hip.generate_source(same_params))[0] == ""
 
 
 def reduction_max_ir(pad="(f32 -1000000.0)"):

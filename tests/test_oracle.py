@@ -353,3 +353,49 @@ def test_naive_matmul_is_the_same_sum_as_the_tiled_kernel(oracle):
     # row = tid / n, col = tid mod n: a launch of n + 3 threads fills row 0 and three of row 1
     part = oracle.matmul_naive(a, b, m, n, k, out=np.full(m * n, -1, dtype=np.float32), threads=n + 3)
     assert np.array_equal(part[:n + 3], c_full := oracle.matmul_naive(a, b, m, n, k)[:n + 3]) and np.all(part[n + 3:] == -1)
+
+
+# ---- histograms (benchmarks/bench_histogram.ml, bench_radix_sort.ml) -------------------------------
+
+@pytest.mark.parametrize("n,bins,block", [(0, 256, 256), (1, 256, 256), (1000, 256, 256), (100003, 256, 256),
+                                           (5000, 10, 64), (5000, 200, 256), (777, 1, 32), (4096, 256, 1024)])
+def test_histogram_is_numpy_bincount(oracle, n, bins, block):
+    keys = np.random.default_rng(n + bins).integers(0, 1 << 30, n).astype(np.int32)
+    hist = np.full(256, 3, dtype=np.int32)                       # accumulated into, not cleared
+    assert oracle.histogram(keys, hist, n, bins, block=block) == 0
+    expected = np.full(256, 3, dtype=np.int64)
+    expected[:bins] += np.bincount(keys.astype(np.int64) % bins, minlength=bins)
+    assert np.array_equal(hist, expected)
+
+
+def test_histogram_of_a_short_launch_and_of_narrow_blocks(oracle):
+    keys = (np.arange(4000) % 100).astype(np.int32)
+    hist = np.zeros(256, dtype=np.int32)
+    assert oracle.histogram(keys, hist, 4000, 100, block=256, grid=4) == 0      # 1024 threads: the first 1024 keys
+    assert np.array_equal(hist[:100], np.bincount(keys[:1024], minlength=100)) and not hist[100:].any()
+    # a block of 32 threads clears and merges bins 0..31 only; the others hold what the shared
+    # array held before (here -7) and never reach the result
+    hist = np.zeros(256, dtype=np.int32)
+    assert oracle.histogram(keys, hist, 4000, 100, block=32) == 0
+    assert np.array_equal(hist[:32], np.bincount(keys, minlength=100)[:32]) and not hist[32:].any()
+
+
+def test_histogram_remainder_has_the_sign_of_the_key(oracle):
+    keys = np.array([-512, -256, -255, -1, 0, 1, 255, 256, -2**31], dtype=np.int32)
+    hist = np.zeros(256, dtype=np.int32)
+    assert oracle.histogram(keys, hist, len(keys), 256) == 2                     # -255 and -1 have no slot
+    expected = np.zeros(256, dtype=np.int32)
+    expected[0], expected[1], expected[255] = 5, 1, 1
+    assert np.array_equal(hist, expected)
+
+
+@pytest.mark.parametrize("shift,mask", [(0, 255), (8, 255), (16, 255), (24, 255), (3, 15), (0, 0), (31, 1)])
+def test_radix_histogram_counts_digits(oracle, shift, mask):
+    n = 50021
+    keys = np.random.default_rng(shift * 256 + mask).integers(-2**31, 2**31 - 1, n).astype(np.int32)
+    hist = np.zeros(256, dtype=np.int32)
+    assert oracle.radix_histogram(keys, hist, n, shift, mask) == 0
+    digits = (keys.view(np.uint32) >> np.uint32(shift)) & np.uint32(mask)
+    assert np.array_equal(hist, np.bincount(digits, minlength=256))
+    if shift <= 24:   # the eight digit bits are key bits under an arithmetic shift too
+        assert np.array_equal(digits, (keys >> shift) & mask)
