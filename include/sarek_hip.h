@@ -353,6 +353,15 @@ int sarek_hip_histogram_i32(int32_t *histogram, const int32_t *keys, int64_t n, 
  * benchmarks/bench_radix_sort.ml:82-116 (`>>` as in the generated code: arithmetic).   */
 int sarek_hip_radix_histogram_i32(int32_t *histogram, const int32_t *keys, int64_t n, int shift, int mask,
                                   sarek_hip_stream stream);
+/* The scatter kernel of the same pass, benchmarks/bench_radix_sort.ml:120-137: every key i < n takes
+ * the next free position of its digit d = (keys[i] >> shift) & mask,
+ *     pos = counters[d]++;  out[pos] = keys[i].
+ * Afterwards counters[d] has grown by the number of keys with digit d and out holds them in
+ * [old counters[d], new counters[d]), in an order that kernel can produce (it fixes none: its
+ * positions come from global atomics).  A position outside [0, out_len) is skipped, where that
+ * kernel writes out of bounds.  The three vectors must not overlap; keys 16-byte aligned.        */
+int sarek_hip_radix_scatter_i32(int32_t *out, int64_t out_len, int32_t *counters, const int32_t *keys, int64_t n,
+                                int shift, int mask, sarek_hip_stream stream);
 
 /* Row-major GEMM  C[m x n] = A[m x k] . B[k x n]  (replaces the generated
  * 16x16 tiled kernel, matrix_mul_tiled_generated.md:9-50; source

@@ -16,7 +16,7 @@ __all__ = [
     "build", "fill_uniform", "round_bf16", "round_f16", "bf16_bits", "f16_bits",
     "triad", "reduce_sum_block256", "reduce_max_block256", "dot_block256", "fold_partials", "triad_sum",
     "gemm", "gemm_rows", "gemm_bias_relu_rowsum", "matmul_tiled_bsp",
-    "vector_add", "vector_copy", "transpose", "histogram", "radix_histogram", "matmul_naive",
+    "vector_add", "vector_copy", "transpose", "histogram", "radix_histogram", "radix_scatter", "matmul_naive",
 ]
 
 
@@ -251,6 +251,17 @@ def radix_histogram(keys, hist, n, shift, mask, block=256, grid=None, stale=-7):
     f.restype = C.c_int64
     return f(kp, hist.ctypes.data_as(C.POINTER(C.c_int32)), C.c_int32(n), C.c_int32(shift), C.c_int32(mask),
              C.c_int32(block), C.c_int32(grid), C.c_int32(stale))
+
+
+def radix_scatter(keys, out, counters, n, shift, mask, threads=None):
+    """In place on `out` and `counters` (int32); returns the number of positions outside `out`."""
+    keys, kp = _i32(keys)
+    assert out.dtype == np.int32 and out.flags.c_contiguous and counters.dtype == np.int32
+    f = _L().oracle_radix_scatter_i32
+    f.restype = C.c_int64
+    p32 = C.POINTER(C.c_int32)
+    return f(kp, out.ctypes.data_as(p32), C.c_int64(len(out)), counters.ctypes.data_as(p32), C.c_int32(n),
+             C.c_int32(shift), C.c_int32(mask), C.c_int64(_launch_size(n, threads)))
 
 
 def transpose(x, width, height, out=None, threads=None):

@@ -498,6 +498,25 @@ int64_t oracle_radix_histogram_i32(const int32_t *input, int32_t *histogram, int
   return skipped;
 }
 
+/* The scatter kernel of benchmarks/bench_radix_sort.ml:120-137 with its threads run in gid order (the Native
+ * backend runs them one after the other): pos = counters[digit]++, output[pos] = value.  The GPU kernel's
+ * order inside a digit's range is not fixed, so a device result is compared with this one digit by digit as
+ * multisets, and through the counters.  Returns the number of positions outside [0, out_len) (skipped).   */
+int64_t oracle_radix_scatter_i32(const int32_t *input, int32_t *output, int64_t out_len, int32_t *counters,
+                                 int32_t n, int32_t shift, int32_t mask, int64_t threads) {
+  int64_t outside = 0;
+  for (int64_t gid = 0; gid < threads; ++gid)
+    if (gid < n) {
+      const int32_t value = input[gid];
+      const int32_t digit = (int32_t)((uint32_t)value >> shift) & mask;
+      const int32_t pos = counters[digit];
+      counters[digit] = (int32_t)((uint32_t)pos + 1u);
+      if (pos < 0 || pos >= out_len) ++outside;
+      else output[pos] = value;
+    }
+  return outside;
+}
+
 void oracle_transpose_f32(const float *input, float *output, int32_t width, int32_t height, int64_t threads) {
   const int32_t n = width * height;
   for (int64_t tid = 0; tid < threads; ++tid)

@@ -6,8 +6,8 @@
 // benchmarks/bench_stream_triad.ml:22-32, benchmarks/bench_reduction.ml:62-96,
 // benchmarks/bench_dot_product.ml:16-54 and benchmarks/bench_reduction_max.ml:18-100 in the
 // reference, the last with any constant as the out-of-range fill; and the vector add, vector
-// copy, one-thread-per-element matmul, the two transposes, the histogram and the counting
-// kernel of the radix sort).  Anything else gets the plain
+// copy, one-thread-per-element matmul, the two transposes, the histogram and the two kernels
+// of a radix-sort pass).  Anything else gets the plain
 // lowering: a miss costs speed, never correctness.
 //
 // Normalisation removes what the front end is free to vary without changing meaning:
@@ -410,6 +410,21 @@ const char *kRadixHistogram = R"IR(
  (native_fn true))
 )IR";
 
+// The scatter kernel of one radix-sort pass, benchmarks/bench_radix_sort.ml:120-137.
+const char *kRadixScatter = R"IR(
+(kernel sarek_kern
+ (params (param (var input 1 (vec i32))) (param (var output 2 (vec i32))) (param (var counters 3 (vec i32))) (param (var n 4 i32)) (param (var shift 5 i32)) (param (var mask 6 i32)))
+ (locals)
+ (body
+ (let (var gid 7 i32) (intr (Std) global_thread_id)
+ (if (lt (var gid 7 i32) (var n 4 i32))
+  (let (var value 8 i32) (read input (var gid 7 i32))
+  (let (var digit 9 i32) (bitand (shr (var value 8 i32) (var shift 5 i32)) (var mask 6 i32))
+  (let (var pos 10 i32) (intr (Gpu) atomic_add_global_int32 (var counters 3 (vec i32)) (var digit 9 i32) (i32 1))
+   (assign (lelem output (var pos 10 i32)) (var value 8 i32))))))))
+ (native_fn true))
+)IR";
+
 const char *kMatmulNaive = R"IR(
 (kernel sarek_kern
  (params (param (var a 1 (vec f32))) (param (var b 2 (vec f32))) (param (var c 3 (vec f32))) (param (var m 4 i32)) (param (var n 5 i32)) (param (var k 6 i32)))
@@ -568,7 +583,9 @@ std::string recognise(const Kernel &k) {
   static const std::string t_tr_tiled = strip_trailing_barrier(canon_kernel(parse_kernel(kTransposeTiled)));
   static const std::string t_hist = strip_trailing_barrier(canon_kernel(parse_kernel(kHistogram)));
   static const std::string t_radix_hist = strip_trailing_barrier(canon_kernel(parse_kernel(kRadixHistogram)));
+  static const std::string t_radix_scatter = canon_kernel(parse_kernel(kRadixScatter));
   const std::string c = canon_kernel(k);
+  if (c == t_radix_scatter) return "radix_scatter_i32";
   if (c == t_matmul) return "matmul_tiled_f32";
   if (c == t_triad) return "stream_triad_f32";
   if (c == t_add) return "vector_add_f32";

@@ -189,6 +189,30 @@ int try_specialised(const std::string &tag, const int block[3], const int grid[3
                                           static_cast<const int32_t *>(args[0].buffer), n, bins, nullptr);
     return 1;
   }
+  if (tag == "radix_scatter_i32") {
+    // (input, len, output, len, counters, len, n, shift, mask): each key of the threads' reach takes the next
+    // position of its digit
+    if (n_args != 9 || !vec_at(args, n_args, 0) || !vec_at(args, n_args, 2) || !vec_at(args, n_args, 4) ||
+        !is_i32(args[6]) || !is_i32(args[7]) || !is_i32(args[8]))
+      return 0;
+    if (block[1] != 1 || block[2] != 1 || grid[1] != 1 || grid[2] != 1) return 0;
+    const int64_t reach = static_cast<int64_t>(block[0]) * grid[0];
+    const int64_t n = args[6].i32 < reach ? args[6].i32 : reach;
+    const int shift = args[7].i32, mask = args[8].i32;
+    if (n < 0 || shift < 0 || shift > 24 || mask < 0 || mask > 255) return 0;
+    if (args[0].length < n || args[2].length < 0 || args[4].length < mask + 1) return 0;
+    const uintptr_t in = reinterpret_cast<uintptr_t>(args[0].buffer), out = reinterpret_cast<uintptr_t>(args[2].buffer),
+                    cnt = reinterpret_cast<uintptr_t>(args[4].buffer);
+    const uintptr_t in_b = static_cast<uintptr_t>(n) * 4, out_b = static_cast<uintptr_t>(args[2].length) * 4,
+                    cnt_b = static_cast<uintptr_t>(mask + 1) * 4;
+    auto meet = [](uintptr_t a, uintptr_t ab, uintptr_t b, uintptr_t bb) { return a < b + bb && b < a + ab; };
+    if (meet(in, in_b, out, out_b) || meet(in, in_b, cnt, cnt_b) || meet(out, out_b, cnt, cnt_b)) return 0;
+    if (in & 15) return 0;
+    *rc = sarek_hip_radix_scatter_i32(static_cast<int32_t *>(args[2].buffer), args[2].length,
+                                      static_cast<int32_t *>(args[4].buffer),
+                                      static_cast<const int32_t *>(args[0].buffer), n, shift, mask, nullptr);
+    return 1;
+  }
   if (tag == "reduce_sum_block256_f32" || tag == "dot_block256_f32") {
     const bool dot = tag[0] == 'd';
     const int nv = dot ? 3 : 2;

@@ -117,6 +117,7 @@ SYMBOLS = {
     "sarek_hip_transpose_f32": (_i, [_vp, _vp, _i, _i, _vp]),
     "sarek_hip_histogram_i32": (_i, [_vp, _vp, _i64, _i, _vp]),
     "sarek_hip_radix_histogram_i32": (_i, [_vp, _vp, _i64, _i, _i, _vp]),
+    "sarek_hip_radix_scatter_i32": (_i, [_vp, _i64, _vp, _vp, _i64, _i, _i, _vp]),
     "sarek_hip_gemm_f32": (_i, [_vp, _vp, _vp, _i, _i, _i, _vp]),
     "sarek_hip_gemm_bf16": (_i, [_vp, _vp, _vp, _i, _i, _i, _vp]),
     "sarek_hip_gemm_f16": (_i, [_vp, _vp, _vp, _i, _i, _i, _vp]),
@@ -456,6 +457,18 @@ def radix_histogram(keys, hist, shift, mask=255):
         raise ValueError("radix_histogram: hist has fewer than 256 bins")
     check(lib.sarek_hip_radix_histogram_i32(_ptr(hist), _ptr(keys), keys.numel(), shift, mask, _stream()))
     return hist
+
+
+def radix_scatter(keys, out, counters, shift, mask=255):
+    """out[counters[d]++] = key for every key, d = (key >> shift) & mask (bench_radix_sort's scatter kernel)."""
+    torch = _torch()
+    for x, name in ((keys, "keys"), (out, "out"), (counters, "counters")):
+        _need(x, torch.int32, name)
+    if counters.numel() < mask + 1:
+        raise ValueError("radix_scatter: counters shorter than mask + 1")
+    check(lib.sarek_hip_radix_scatter_i32(_ptr(out), out.numel(), _ptr(counters), _ptr(keys), keys.numel(), shift, mask,
+                                          _stream()))
+    return out
 
 
 def gemm_f32(a, b, out=None):

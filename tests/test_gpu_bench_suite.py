@@ -13,7 +13,7 @@ pytestmark = pytest.mark.gpu
 @pytest.mark.parametrize("name,size", [
     ("gather", 100003), ("scatter", 100003),
     ("stencil_2d", 200), ("conv2d", 200), ("conv2d", 37), ("mandelbrot", 100), ("nbody", 300),
-    ("bitonic_sort", 1024), ("bitonic_sort", 3000), ("radix_sort", 100003)])
+    ("bitonic_sort", 1024), ("bitonic_sort", 3000)])
 def test_suite_runs_and_verifies(hip, torch_cuda, name, size):
     from spoc_amd import benchmarks
     rec = benchmarks.BENCHMARKS[name][0](size, warmup=1, iterations=3)

@@ -124,6 +124,78 @@ def test_radix_histogram_ir_dispatch(hip, torch_cuda, oracle, shift):
     assert run_histogram_ir(n, 256, 256, (n + 255) // 256, keys, 1, hip, radix=(25, 255))[0] == "jit"
 
 
+def check_scatter(got, counters_after, keys, n, starts, shift, mask, oracle, out_len=None):
+    """Digit by digit the same keys as the thread-order scatter, whatever their order in the range."""
+    out_len = len(got) if out_len is None else out_len
+    exp, exp_counters = np.full(out_len, -1, dtype=np.int32), starts.copy()
+    outside = oracle.radix_scatter(keys, exp, exp_counters, n, shift, mask)
+    assert np.array_equal(counters_after, exp_counters)
+    if outside == 0:
+        digit = lambda a: (a.view(np.uint32) >> np.uint32(shift)) & np.uint32(mask)     # noqa: E731
+        written = exp != -1
+        assert np.array_equal(got[~written], exp[~written])                    # nothing else touched
+        assert np.array_equal(digit(got[written]), digit(exp[written]))        # every range holds its digit
+        order_g, order_e = np.lexsort((got[written], digit(got[written]))), np.lexsort((exp[written], digit(exp[written])))
+        assert np.array_equal(got[written][order_g], exp[written][order_e])
+    return outside
+
+
+@pytest.mark.parametrize("n", [0, 1, 5, 8191, 8192, 8193, 100_003, 1_000_003])
+@pytest.mark.parametrize("shift,mask", [(0, 255), (8, 255), (4, 15)])
+def test_radix_scatter_sizes(hip, torch_cuda, oracle, n, shift, mask):
+    torch = torch_cuda
+    keys = keys_of(n, n + shift, 1, 2**31 - 1)                    # -1 marks untouched slots below
+    digits = (keys >> shift) & mask
+    counts = np.bincount(digits, minlength=256)
+    starts = np.concatenate(([0], np.cumsum(counts)[:-1])).astype(np.int32)
+    out = torch.full((n + 64,), -1, dtype=torch.int32, device="cuda")
+    counters = torch.from_numpy(starts.copy()).cuda()
+    hip.radix_scatter(torch.from_numpy(keys).cuda(), out, counters, shift, mask)
+    assert check_scatter(out.cpu().numpy(), counters.cpu().numpy(), keys, n, starts, shift, mask, oracle) == 0
+
+
+def test_radix_scatter_skips_positions_outside_the_output(hip, torch_cuda, oracle):
+    """Counters that start 40 too high push the last keys of the last digit past the output: those
+    stores are dropped (the slots behind the output keep their contents), the counters still advance."""
+    torch = torch_cuda
+    n, shift, mask = 50_000, 0, 255
+    keys = keys_of(n, 3, 1, 2**31 - 1)
+    counts = np.bincount(keys & mask, minlength=256)
+    starts = (np.concatenate(([0], np.cumsum(counts)[:-1])) + 40).astype(np.int32)
+    whole = torch.full((n + 4096,), -1, dtype=torch.int32, device="cuda")
+    counters = torch.from_numpy(starts.copy()).cuda()
+    hip.radix_scatter(torch.from_numpy(keys).cuda(), whole[:n], counters, shift, mask)
+    got = whole.cpu().numpy()
+    assert np.all(got[n:] == -1) and np.all(got[:40] == -1) and np.all(got[40:n] != -1)
+    assert np.array_equal(counters.cpu().numpy(), starts + counts)
+    exp, c = np.full(n, -1, dtype=np.int32), starts.copy()
+    assert oracle.radix_scatter(keys, exp, c, n, shift, mask) == 40
+
+
+def test_radix_scatter_ir_dispatch(hip, torch_cuda, oracle):
+    from spoc_amd import reference_kernels
+    from spoc_amd.sarek import Execute, Vector
+    n, shift, mask = 77_777, 8, 255
+    keys = keys_of(n, 9, 1, 2**31 - 1)
+    counts = np.bincount((keys >> shift) & mask, minlength=256)
+    starts = np.concatenate(([0], np.cumsum(counts)[:-1])).astype(np.int32)
+    for specialise, tag, reach in ((1, "radix_scatter_i32", n), (0, "jit", n), (1, "radix_scatter_i32", 25_600)):
+        vk, vo, vc = Vector.create(Vector.int32, n), Vector.create(Vector.int32, n), Vector.create(Vector.int32, 256)
+        vk.fill_from(keys)
+        vo.fill_from(np.full(n, -1))
+        vc.fill_from(starts)
+        hip.check(hip.lib.sarek_hip_set_specialisation(specialise))
+        try:
+            path = Execute.run_vectors(ir=reference_kernels.radix_sort_scatter(),
+                                       args=[Execute.Vec(vk), Execute.Vec(vo), Execute.Vec(vc), Execute.Int32(n),
+                                             Execute.Int32(shift), Execute.Int32(mask)],
+                                       block=Execute.dims1d(256), grid=Execute.dims1d((reach + 255) // 256))
+        finally:
+            hip.check(hip.lib.sarek_hip_set_specialisation(1))
+        assert path == tag
+        assert check_scatter(vo.to_array(), vc.to_array(), keys, min(n, reach), starts, shift, mask, oracle) == 0
+
+
 def test_bench_mirrors_take_the_hand_kernels(hip, torch_cuda):
     from spoc_amd import benchmarks
     rec = benchmarks.bench_histogram(1_000_003, warmup=1, iterations=3)
@@ -134,5 +206,11 @@ def test_bench_mirrors_take_the_hand_kernels(hip, torch_cuda):
     finally:
         hip.check(hip.lib.sarek_hip_set_specialisation(1))
     assert rec["verified"] and rec["path"] == "jit"
+    hip.check(hip.lib.sarek_hip_set_specialisation(0))
+    try:
+        rec = benchmarks.bench_radix_sort(100_003, warmup=1, iterations=2)
+    finally:
+        hip.check(hip.lib.sarek_hip_set_specialisation(1))
+    assert rec["verified"] and rec["path"] == "jit"
     rec = benchmarks.bench_radix_sort(300_001, warmup=1, iterations=2)
-    assert rec["verified"] and rec["path"] == "jit"          # the last launch of a pass is the scatter kernel
+    assert rec["verified"] and rec["path"] == "radix_scatter_i32"      # the last launch of a pass

@@ -22,7 +22,7 @@ EXPECTED_TAGS = {
     "reduction": "reduce_sum_block256_f32", "dot_product": "dot_block256_f32",
     "vector_add": "vector_add_f32", "vector_copy": "vector_copy_f32", "matrix_mul": "matmul_naive_f32",
     "transpose_naive": "transpose_naive_f32", "transpose_tiled": "transpose_tiled_f32",
-    "radix_sort_histogram": "radix_histogram_i32",
+    "radix_sort_histogram": "radix_histogram_i32", "radix_sort_scatter": "radix_scatter_i32",
 }
 
 
@@ -277,6 +277,17 @@ def test_histogram_recognition_and_near_misses(hip):
     radix = open(os.path.join(IR_DIR, "radix_sort_histogram.ir")).read()
     assert split_tag(hip.generate_source(radix.replace("(shr ", "(shl ")))[0] == ""
     assert split_tag(hip.generate_source(radix.replace("(read local_hist (var tid 7 i32)))", "(i32 1))", 1)))[0] == ""
+
+
+def test_radix_scatter_near_misses_fall_back(hip):
+    ir = open(os.path.join(IR_DIR, "radix_sort_scatter.ir")).read()
+    assert split_tag(hip.generate_source(ir))[0] == "radix_scatter_i32"
+    assert split_tag(hip.generate_source(ir.replace("(i32 1))", "(i32 2))", 1)))[0] == ""            # every other slot
+    assert split_tag(hip.generate_source(ir.replace("(lelem output (var pos 10 i32))", "(lelem output (var gid 7 i32))")))[0] == ""
+    assert split_tag(hip.generate_source(ir.replace("(var counters 3 (vec i32)) (var digit 9 i32)",
+                                                    "(var counters 3 (vec i32)) (i32 0)")))[0] == ""
+    assert split_tag(hip.generate_source(ir.replace("(assign (lelem output (var pos 10 i32)) (var value 8 i32))",
+                                                    "(assign (lelem output (var pos 10 i32)) (var digit 9 i32))")))[0] == ""
 
 
 def test_an_atomic_in_an_unused_binding_is_part_of_the_program(hip):

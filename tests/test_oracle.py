@@ -399,3 +399,22 @@ def test_radix_histogram_counts_digits(oracle, shift, mask):
     assert np.array_equal(hist, np.bincount(digits, minlength=256))
     if shift <= 24:   # the eight digit bits are key bits under an arithmetic shift too
         assert np.array_equal(digits, (keys >> shift) & mask)
+
+
+@pytest.mark.parametrize("shift", [0, 8, 24])
+def test_radix_scatter_in_thread_order_is_a_stable_sort_by_digit(oracle, shift):
+    n = 30011
+    keys = np.random.default_rng(shift).integers(-2**31, 2**31 - 1, n).astype(np.int32)
+    digits = ((keys.view(np.uint32) >> np.uint32(shift)) & np.uint32(255)).astype(np.int64)
+    counts = np.bincount(digits, minlength=256)
+    starts = np.concatenate(([0], np.cumsum(counts)[:-1])).astype(np.int32)
+    counters, out = starts.copy(), np.full(n, -1, dtype=np.int32)
+    assert oracle.radix_scatter(keys, out, counters, n, shift, 255) == 0
+    assert np.array_equal(out, keys[np.argsort(digits, kind="stable")])
+    assert np.array_equal(counters, starts + counts)
+    # a launch that reaches only the first 1000 keys; positions past the output are reported, not written
+    counters, out = starts.copy(), np.full(n, -1, dtype=np.int32)
+    assert oracle.radix_scatter(keys, out, counters, n, shift, 255, threads=1000) == 0
+    assert np.array_equal(np.sort(out[out != -1]), np.sort(keys[:1000])) or -1 in keys[:1000]
+    counters, small = starts.copy(), np.full(100, -1, dtype=np.int32)
+    assert oracle.radix_scatter(keys, small, counters, n, shift, 255) == n - 100
