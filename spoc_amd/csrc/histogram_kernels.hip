@@ -150,34 +150,33 @@ __global__ __launch_bounds__(kThreads) void histogram_kernel(int *__restrict__ h
 // the tile by digit in LDS and writes each digit's run to consecutive addresses: an order the
 // reference's kernel can produce too (all keys of a workgroup arriving together), counters left
 // exactly as it leaves them.  8 bytes per key.
-constexpr int kScatterThreads = 512;
-constexpr int kScatterKeys = 16;                                   // per thread
-constexpr int kScatterTile = kScatterThreads * kScatterKeys;       // 8192 keys, 32 KiB of LDS
-
 // out_len guards the stores: a position outside [0, out_len) (counters that do not leave room for the
-// keys) is skipped, where the reference's kernel would write out of bounds.
-__global__ __launch_bounds__(kScatterThreads) void radix_scatter_kernel(int *__restrict__ out, int64_t out_len,
-                                                                        int *__restrict__ counters,
-                                                                        const int *__restrict__ keys, int64_t n,
-                                                                        int shift, int mask) {
-  __shared__ int stage[kScatterTile];
+// keys) is skipped, where the reference's kernel would write out of bounds.  The tile (Threads * Keys
+// keys) is staged in dynamic LDS.
+template <int Threads, int Keys>
+__global__ __launch_bounds__(Threads) void radix_scatter_kernel(int *__restrict__ out, int64_t out_len,
+                                                                int *__restrict__ counters,
+                                                                const int *__restrict__ keys, int64_t n, int shift,
+                                                                int mask) {
+  constexpr int kTile = Threads * Keys;
+  extern __shared__ int stage[];    // kTile keys, ordered by digit
   __shared__ int count[kBins];      // keys of the tile per digit
   __shared__ int start[kBins];      // first slot of the digit in `stage` (exclusive scan of count)
   __shared__ int base[kBins];       // first position of the tile's keys of the digit in `out`
   __shared__ int wave_total[kBins / 64];
   const int t = threadIdx.x, lane = t & 63;
-  const int64_t tile = static_cast<int64_t>(blockIdx.x) * kScatterTile;
-  const int valid = n - tile < kScatterTile ? static_cast<int>(n - tile) : kScatterTile;
+  const int64_t tile = static_cast<int64_t>(blockIdx.x) * kTile;
+  const int valid = n - tile < kTile ? static_cast<int>(n - tile) : kTile;
   if (t < kBins) count[t] = 0;
   __syncthreads();
 
-  // slot j of thread t is key tile + (j / 4 * kScatterThreads + t) * 4 + j % 4: 16-byte loads
-  int key[kScatterKeys], rank[kScatterKeys];
-  if (valid == kScatterTile) {
+  // slot j of thread t is key tile + (j / 4 * Threads + t) * 4 + j % 4: 16-byte loads
+  int key[Keys], rank[Keys];
+  if (valid == kTile) {
     const i32x4_t *k4 = reinterpret_cast<const i32x4_t *>(keys + tile);
 #pragma unroll
-    for (int u = 0; u < kScatterKeys / 4; ++u) {
-      const i32x4_t v = __builtin_nontemporal_load(k4 + u * kScatterThreads + t);
+    for (int u = 0; u < Keys / 4; ++u) {
+      const i32x4_t v = __builtin_nontemporal_load(k4 + u * Threads + t);
       key[4 * u] = v.x;
       key[4 * u + 1] = v.y;
       key[4 * u + 2] = v.z;
@@ -185,14 +184,14 @@ __global__ __launch_bounds__(kScatterThreads) void radix_scatter_kernel(int *__r
     }
   } else {
 #pragma unroll
-    for (int j = 0; j < kScatterKeys; ++j) {
-      const int at = ((j >> 2) * kScatterThreads + t) * 4 + (j & 3);
+    for (int j = 0; j < Keys; ++j) {
+      const int at = ((j >> 2) * Threads + t) * 4 + (j & 3);
       key[j] = at < valid ? keys[tile + at] : 0;
     }
   }
-  auto in_tile = [&](int j) { return ((j >> 2) * kScatterThreads + t) * 4 + (j & 3) < valid; };
+  auto in_tile = [&](int j) { return ((j >> 2) * Threads + t) * 4 + (j & 3) < valid; };
 #pragma unroll
-  for (int j = 0; j < kScatterKeys; ++j)
+  for (int j = 0; j < Keys; ++j)
     rank[j] = in_tile(j) ? atomicAdd(&count[(key[j] >> shift) & mask], 1) : 0;
   __syncthreads();
 
@@ -217,16 +216,38 @@ __global__ __launch_bounds__(kScatterThreads) void radix_scatter_kernel(int *__r
   __syncthreads();
 
 #pragma unroll
-  for (int j = 0; j < kScatterKeys; ++j)
+  for (int j = 0; j < Keys; ++j)
     if (in_tile(j)) stage[start[(key[j] >> shift) & mask] + rank[j]] = key[j];
   __syncthreads();
 
-  for (int s = t; s < valid; s += kScatterThreads) {
+  for (int s = t; s < valid; s += Threads) {
     const int k = stage[s];
     const int d = (k >> shift) & mask;
     const int64_t pos = static_cast<int64_t>(base[d]) + (s - start[d]);
     if (pos >= 0 && pos < out_len) out[pos] = k;
   }
+}
+
+template <int Threads, int Keys>
+int launch_scatter(int *out, int64_t out_len, int *counters, const int *keys, int64_t n, int shift, int mask,
+                   hipStream_t st) {
+  constexpr int kTile = Threads * Keys;
+  constexpr int kLds = kTile * 4;
+  static_assert(Threads >= kBins && Threads % 64 == 0 && Keys % 4 == 0, "tile shape");
+  const int64_t tiles = ceil_div(n, static_cast<int64_t>(kTile));
+  if (tiles > 0x7FFFFFFF) return fail(SAREK_HIP_E_INVALID_ARG, "radix scatter: vector too long for one launch");
+  auto kern = radix_scatter_kernel<Threads, Keys>;
+  static bool attr_done[16] = {};
+  int dev = 0;
+  SAREK_HIP_TRY(hipGetDevice(&dev));
+  if (dev >= 0 && dev < 16 && !attr_done[dev]) {
+    SAREK_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
+                                      hipFuncAttributeMaxDynamicSharedMemorySize, kLds));
+    attr_done[dev] = true;
+  }
+  hipLaunchKernelGGL(kern, dim3(static_cast<unsigned>(tiles)), dim3(Threads), kLds, st, out, out_len, counters,
+                     keys, n, shift, mask);
+  return check_launch("radix scatter kernel launch");
 }
 
 int compute_units() {
@@ -300,11 +321,18 @@ int sarek_hip_radix_scatter_i32(int32_t *out, int64_t out_len, int32_t *counters
   if (mask < 0 || mask >= kBins)
     return fail(SAREK_HIP_E_INVALID_ARG, "radix scatter: mask %d outside 0..%d", mask, kBins - 1);
   if (n == 0) return SAREK_HIP_OK;
-  const int64_t tiles = ceil_div(n, static_cast<int64_t>(kScatterTile));
-  if (tiles > 0x7FFFFFFF) return fail(SAREK_HIP_E_INVALID_ARG, "radix scatter: vector too long for one launch");
-  hipLaunchKernelGGL(radix_scatter_kernel, dim3(static_cast<unsigned>(tiles)), dim3(kScatterThreads), 0,
-                     as_stream(stream), out, out_len, counters, keys, n, shift, mask);
-  return check_launch("radix scatter kernel launch");
+  hipStream_t st = as_stream(stream);
+  // Measured on MI355X: 16384-key tiles from about 4M keys on (half the global atomics of 8192-key tiles:
+  // 95 against 142 us at 50M keys), 8192-key tiles below (more workgroups than CUs sooner).
+  int64_t shape = tunable("radix_scatter.tile", 0);
+  if (shape == 0) shape = n >= (int64_t{1} << 22) ? 2 : 1;
+  switch (shape) {
+    case 1: return launch_scatter<512, 16>(out, out_len, counters, keys, n, shift, mask, st);
+    case 2: return launch_scatter<1024, 16>(out, out_len, counters, keys, n, shift, mask, st);
+    case 3: return launch_scatter<512, 32>(out, out_len, counters, keys, n, shift, mask, st);
+    case 4: return launch_scatter<1024, 32>(out, out_len, counters, keys, n, shift, mask, st);
+    default: return launch_scatter<512, 16>(out, out_len, counters, keys, n, shift, mask, st);
+  }
 }
 
 }  // extern "C"

@@ -154,6 +154,26 @@ def test_radix_scatter_sizes(hip, torch_cuda, oracle, n, shift, mask):
     assert check_scatter(out.cpu().numpy(), counters.cpu().numpy(), keys, n, starts, shift, mask, oracle) == 0
 
 
+@pytest.mark.parametrize("n,shape", [(100_003, 2), (100_003, 3), (100_003, 4), (40_000, 4), ((1 << 22) + 4099, 0)])
+def test_radix_scatter_tile_shapes(hip, torch_cuda, oracle, n, shape):
+    """Every tile shape of the kernel (8192 to 32768 keys; 0 = the library's choice, which from 2^22 keys on
+    is the 16384-key tile), ragged last tiles included."""
+    torch = torch_cuda
+    shift, mask = 8, 255
+    keys = keys_of(n, shape, 1, 2**31 - 1)
+    counts = np.bincount((keys >> shift) & mask, minlength=256)
+    starts = np.concatenate(([0], np.cumsum(counts)[:-1])).astype(np.int32)
+    out = torch.full((n + 64,), -1, dtype=torch.int32, device="cuda")
+    counters = torch.from_numpy(starts.copy()).cuda()
+    hip.set_tunable("radix_scatter.tile", shape)
+    try:
+        hip.radix_scatter(torch.from_numpy(keys).cuda(), out, counters, shift, mask)
+        torch.cuda.synchronize()
+    finally:
+        hip.set_tunable("radix_scatter.tile", 0)
+    assert check_scatter(out.cpu().numpy(), counters.cpu().numpy(), keys, n, starts, shift, mask, oracle) == 0
+
+
 def test_radix_scatter_skips_positions_outside_the_output(hip, torch_cuda, oracle):
     """Counters that start 40 too high push the last keys of the last digit past the output: those
     stores are dropped (the slots behind the output keep their contents), the counters still advance."""
