@@ -243,7 +243,35 @@ enum {                                  /* Vector_types.location                
  * waits for the device), the location states change as for any vector.             */
 int sarek_hip_vector_create(int kind, int64_t length, int64_t custom_elem_size, int pinned,
                             sarek_hip_vector *out);
-int sarek_hip_vector_destroy(sarek_hip_vector v);          /* host block and device buffers */
+int sarek_hip_vector_destroy(sarek_hip_vector v);          /* device buffers; the host block with its last vector */
+/* Vector.id (sarek/core/Vector_storage.ml: next_id; the first vector of a process is #1) and
+ * Vector.to_string (sarek/core/Vector.ml:181-195), "Vector#3<Float32>[1024] @ Both(<device name>)";
+ * a custom vector's kind prints as Custom(<element size>).                                          */
+int64_t sarek_hip_vector_id(sarek_hip_vector v);
+int sarek_hip_vector_to_string(sarek_hip_vector v, char *buf, size_t cap);
+/* Vector.fill (Vector.ml:222-233): every element set to *elem, then as a host write (Both / GPU ->
+ * Stale_GPU; a Stale_CPU vector stays Stale_CPU, its next download overwrites the fill).            */
+int sarek_hip_vector_fill(sarek_hip_vector v, const void *elem);
+/* Vector.copy (Vector.ml:245-249): a new vector on the CPU with the host data, downloaded first
+ * when the host copy is stale and auto-sync is on; no device buffers.                               */
+int sarek_hip_vector_copy(sarek_hip_vector v, sarek_hip_vector *out);
+/* Vector.sub_vector (Vector.ml:259-267, Vector_storage.ml:215-259): `len` elements of v's HOST block
+ * from `start`, shared with v (and kept alive by either); device buffers and location (CPU) are the
+ * sub-vector's own.  ok_range: elements safe to read (negative = len), ko_range: elements not to
+ * write; both are only recorded.  Out of range: SAREK_HIP_E_INVALID_ARG with the reference's text. */
+int sarek_hip_vector_sub(sarek_hip_vector v, int64_t start, int64_t len, int64_t ok_range, int64_t ko_range,
+                         sarek_hip_vector *out);
+/* Vector.is_sub / get_sub_meta / depth / parent_id / sub_start / sub_ok_range / sub_ko_range
+ * (Vector.ml:252-257,300-317); any out pointer but is_sub may be NULL.                              */
+int sarek_hip_vector_sub_meta(sarek_hip_vector v, int *is_sub, int64_t *parent_id, int64_t *start,
+                              int64_t *ok_range, int64_t *ko_range, int *depth);
+/* Vector.partition (Vector.ml:273-281): n_devices sub-vectors covering v, the first length mod n one
+ * element longer; sub-vector i is Stale_GPU of devices[i].  Nothing is copied.                      */
+int sarek_hip_vector_partition(sarek_hip_vector v, int n_devices, const int *devices, sarek_hip_vector *out);
+/* Vector.blit (Vector.ml:500-517): len elements from src[src_off..] to dst[dst_off..] on the host,
+ * in ascending order; src is downloaded first if stale (auto-sync), dst is marked as written.       */
+int sarek_hip_vector_blit(sarek_hip_vector src, int64_t src_off, sarek_hip_vector dst, int64_t dst_off,
+                          int64_t len);
 int64_t sarek_hip_vector_length(sarek_hip_vector v);
 int64_t sarek_hip_vector_elem_size(sarek_hip_vector v);
 int sarek_hip_vector_kind(sarek_hip_vector v);

@@ -12,7 +12,9 @@
 //   - a host read downloads a Stale_CPU vector when auto-sync is on (vector and global).
 #include <cstdlib>
 #include <cstring>
+#include <atomic>
 #include <map>
+#include <memory>
 #include <mutex>
 #include <string>
 #include <unordered_map>
@@ -22,10 +24,28 @@
 #include "host/ir.hpp"
 #include "plugin.hpp"
 
+// The allocation behind a vector's host block; sub-vectors view their parent's, and it lives as
+// long as any of them (a Bigarray.Array1.sub keeps its parent's memory alive the same way).
+struct sarek_hip_host_block {
+  void *base = nullptr;
+  bool pinned = false;
+  ~sarek_hip_host_block() {
+    if (!base) return;
+    if (pinned) sarek_hip_host_free(base);
+    else std::free(base);
+  }
+};
+
 struct sarek_hip_vector_s {
   int kind = SAREK_HIP_KIND_FLOAT32;
   int64_t length = 0, elem_size = 4;
-  void *host = nullptr;
+  int64_t id = 0;                        // Vector_types.t.id (Vector_storage.next_id)
+  std::shared_ptr<sarek_hip_host_block> block;
+  void *host = nullptr;                  // first element: block->base, or inside it for a sub-vector
+  // Vector_storage.sub_meta (Vector_storage.ml:147-175)
+  bool is_sub = false;
+  int64_t parent_id = 0, sub_start = 0, ok_range = 0, ko_range = 0;
+  int depth = 0;
   bool pinned = false;
   bool zero_copy = false;                // device buffers alias the pinned host block
   bool auto_sync = true;                 // Vector_types.t.auto_sync
@@ -38,6 +58,7 @@ namespace sarek_hip {
 namespace {
 
 bool g_auto_mode = true;                 // Transfer.auto_mode (Transfer.ml:20-28)
+std::atomic<int64_t> g_next_id{0};       // Vector_storage.next_id: the first vector is #1
 
 int64_t kind_elem_size(int kind, int64_t custom) {
   switch (kind) {                        // Vector_types.scalar_elem_size
@@ -252,19 +273,23 @@ int sarek_hip_vector_create(int kind, int64_t length, int64_t custom_elem_size, 
   v->pinned = pinned != 0;
   v->zero_copy = pinned == 2;
   const size_t bytes = static_cast<size_t>(length * es);
+  v->block = std::make_shared<sarek_hip_host_block>();
+  v->block->pinned = v->pinned;
   if (v->pinned) {
-    int st = sarek_hip_host_alloc(&v->host, bytes);
+    int st = sarek_hip_host_alloc(&v->block->base, bytes);
     if (st != SAREK_HIP_OK) {
       delete v;
       return st;
     }
   } else {
-    v->host = std::malloc(bytes ? bytes : 1);   // like a fresh Bigarray: contents unspecified
-    if (!v->host) {
+    v->block->base = std::malloc(bytes ? bytes : 1);   // like a fresh Bigarray: contents unspecified
+    if (!v->block->base) {
       delete v;
       return fail(SAREK_HIP_E_INVALID_ARG, "vector_create: out of host memory (%zu bytes)", bytes);
     }
   }
+  v->host = v->block->base;
+  v->id = ++g_next_id;
   *out = v;
   return SAREK_HIP_OK;
 }
@@ -276,14 +301,137 @@ int sarek_hip_vector_destroy(sarek_hip_vector v) {
     int st = sarek_hip_mem_free(b.second);
     if (first == SAREK_HIP_OK) first = st;
   }
-  if (v->pinned) {
-    int st = sarek_hip_host_free(v->host);
-    if (first == SAREK_HIP_OK) first = st;
-  } else {
-    std::free(v->host);
-  }
-  delete v;
+  delete v;        // the host block goes with its last vector
   return first;
+}
+
+int64_t sarek_hip_vector_id(sarek_hip_vector v) { return v ? v->id : -1; }
+
+// Vector.to_string (Vector.ml:189-195): "Vector#<id><<kind>>[<length>] @ <location>"
+int sarek_hip_vector_to_string(sarek_hip_vector v, char *buf, size_t cap) {
+  if (!v || !buf || cap == 0) return fail(SAREK_HIP_E_INVALID_ARG, "vector_to_string: NULL argument");
+  static const char *kinds[] = {"Float32", "Float64", "Int32", "Int64", "Char", "Complex32"};
+  static const char *locs[] = {"CPU", "GPU", "Both", "Stale_CPU", "Stale_GPU"};
+  std::string kind = v->kind == SAREK_HIP_KIND_CUSTOM ? "Custom(" + std::to_string(v->elem_size) + ")"
+                                                      : std::string(kinds[v->kind]);
+  std::string where = locs[v->location];
+  if (v->location != SAREK_HIP_LOC_CPU) {
+    sarek_hip_device_info info;
+    where += sarek_hip_device_get_info(v->device, &info) == SAREK_HIP_OK ? "(" + std::string(info.name) + ")" : "(?)";
+  }
+  std::snprintf(buf, cap, "Vector#%lld<%s>[%lld] @ %s", static_cast<long long>(v->id), kind.c_str(),
+                static_cast<long long>(v->length), where.c_str());
+  return SAREK_HIP_OK;
+}
+
+// Vector.fill (Vector.ml:222-233): every element of the host block, then the bookkeeping of a host write.
+int sarek_hip_vector_fill(sarek_hip_vector v, const void *elem) {
+  if (!v || !elem) return fail(SAREK_HIP_E_INVALID_ARG, "vector_fill: NULL argument");
+  char *p = static_cast<char *>(v->host);
+  for (int64_t i = 0; i < v->length; ++i) std::memcpy(p + i * v->elem_size, elem, static_cast<size_t>(v->elem_size));
+  host_written(v);
+  return SAREK_HIP_OK;
+}
+
+// Vector.copy (Vector.ml:245-249, Vector_storage.copy_host_only): the host data, after a download if
+// the host copy is stale and auto-sync is on; the copy starts on the CPU with no device buffers.
+int sarek_hip_vector_copy(sarek_hip_vector v, sarek_hip_vector *out) {
+  if (!v || !out) return fail(SAREK_HIP_E_INVALID_ARG, "vector_copy: NULL argument");
+  int st = ensure_cpu_sync(v);
+  if (st != SAREK_HIP_OK) return st;
+  st = sarek_hip_vector_create(v->kind, v->length, v->elem_size, 0, out);
+  if (st != SAREK_HIP_OK) return st;
+  std::memcpy((*out)->host, v->host, bytes_of(v));
+  (*out)->auto_sync = v->auto_sync;
+  return SAREK_HIP_OK;
+}
+
+// Vector.sub_vector (Vector.ml:259-267, Vector_storage.ml:215-259): a view of `len` elements of the
+// parent's host block from `start`, with device buffers and a location of its own (CPU).
+// ok_range < 0 stands for the default (len).
+int sarek_hip_vector_sub(sarek_hip_vector v, int64_t start, int64_t len, int64_t ok_range, int64_t ko_range,
+                         sarek_hip_vector *out) {
+  if (!v || !out) return fail(SAREK_HIP_E_INVALID_ARG, "sub_vector: NULL argument");
+  *out = nullptr;
+  if (start < 0 || len < 0 || start + len > v->length)
+    return fail(SAREK_HIP_E_INVALID_ARG, "sub_vector: range [%lld, %lld) out of bounds [0, %lld)",
+                static_cast<long long>(start), static_cast<long long>(start + len),
+                static_cast<long long>(v->length));
+  auto *s = new sarek_hip_vector_s;
+  s->kind = v->kind;
+  s->length = len;
+  s->elem_size = v->elem_size;
+  s->id = ++g_next_id;
+  s->block = v->block;
+  s->host = static_cast<char *>(v->host) + start * v->elem_size;
+  s->pinned = v->pinned;
+  s->zero_copy = v->zero_copy;
+  s->auto_sync = v->auto_sync;
+  s->is_sub = true;
+  s->parent_id = v->id;
+  s->sub_start = start;
+  s->ok_range = ok_range < 0 ? len : ok_range;
+  s->ko_range = ko_range;
+  s->depth = v->depth + 1;
+  *out = s;
+  return SAREK_HIP_OK;
+}
+
+int sarek_hip_vector_sub_meta(sarek_hip_vector v, int *is_sub, int64_t *parent_id, int64_t *start,
+                              int64_t *ok_range, int64_t *ko_range, int *depth) {
+  if (!v || !is_sub) return fail(SAREK_HIP_E_INVALID_ARG, "vector_sub_meta: NULL argument");
+  *is_sub = v->is_sub;
+  if (parent_id) *parent_id = v->parent_id;
+  if (start) *start = v->sub_start;
+  if (ok_range) *ok_range = v->ok_range;
+  if (ko_range) *ko_range = v->ko_range;
+  if (depth) *depth = v->depth;
+  return SAREK_HIP_OK;
+}
+
+// Vector.partition (Vector.ml:273-281, Vector_storage.partition_host): n sub-vectors that cover the
+// vector, the first length mod n one element longer, sub-vector i marked Stale_GPU of devices[i]
+// (host data valid, that device's copy to be made).
+int sarek_hip_vector_partition(sarek_hip_vector v, int n_devices, const int *devices, sarek_hip_vector *out) {
+  if (!v || n_devices < 0 || (n_devices > 0 && (!devices || !out)))
+    return fail(SAREK_HIP_E_INVALID_ARG, "vector_partition: bad arguments");
+  const int64_t base = n_devices ? v->length / n_devices : 0, rem = n_devices ? v->length % n_devices : 0;
+  for (int i = 0; i < n_devices; ++i) out[i] = nullptr;
+  for (int i = 0; i < n_devices; ++i) {
+    const int64_t len = base + (i < rem ? 1 : 0), start = i * base + (i < rem ? i : rem);
+    int st = sarek_hip_vector_sub(v, start, len, len, 0, &out[i]);
+    if (st != SAREK_HIP_OK) {
+      for (int j = 0; j < i; ++j) {
+        sarek_hip_vector_destroy(out[j]);
+        out[j] = nullptr;
+      }
+      return st;
+    }
+    out[i]->location = SAREK_HIP_LOC_STALE_GPU;
+    out[i]->device = devices[i];
+  }
+  return SAREK_HIP_OK;
+}
+
+// Vector.blit (Vector.ml:500-517): source downloaded first if stale (auto-sync), destination written
+// element by element with the bookkeeping of a host write.
+int sarek_hip_vector_blit(sarek_hip_vector src, int64_t src_off, sarek_hip_vector dst, int64_t dst_off, int64_t len) {
+  if (!src || !dst) return fail(SAREK_HIP_E_INVALID_ARG, "vector_blit: NULL argument");
+  if (src->elem_size != dst->elem_size || src->kind != dst->kind)
+    return fail(SAREK_HIP_E_INVALID_ARG, "Vector.blit: vectors of different kinds");
+  if (len < 0 || src_off < 0 || src_off + len > src->length)
+    return fail(SAREK_HIP_E_INVALID_ARG, "Vector.blit: source range out of bounds");
+  if (dst_off < 0 || dst_off + len > dst->length)
+    return fail(SAREK_HIP_E_INVALID_ARG, "Vector.blit: destination range out of bounds");
+  int st = ensure_cpu_sync(src);
+  if (st != SAREK_HIP_OK) return st;
+  // ascending element order, as the reference's loop: overlapping ranges of one block smear forward
+  const char *s = static_cast<const char *>(src->host) + src_off * src->elem_size;
+  char *d = static_cast<char *>(dst->host) + dst_off * dst->elem_size;
+  for (int64_t i = 0; i < len; ++i)
+    std::memmove(d + i * dst->elem_size, s + i * src->elem_size, static_cast<size_t>(src->elem_size));
+  if (len > 0) host_written(dst);
+  return SAREK_HIP_OK;
 }
 
 int64_t sarek_hip_vector_length(sarek_hip_vector v) { return v ? v->length : -1; }

@@ -147,6 +147,15 @@ SYMBOLS = {
     "sarek_hip_fusion_is_reduction_kernel": (_i, [C.c_char_p, C.c_char_p, C.POINTER(_i), C.c_char_p]),
     "sarek_hip_vector_create": (_i, [_i, _i64, _i64, _i, C.POINTER(_vp)]),
     "sarek_hip_vector_destroy": (_i, [_vp]),
+    "sarek_hip_vector_id": (_i64, [_vp]),
+    "sarek_hip_vector_to_string": (_i, [_vp, C.c_char_p, C.c_size_t]),
+    "sarek_hip_vector_fill": (_i, [_vp, _vp]),
+    "sarek_hip_vector_copy": (_i, [_vp, C.POINTER(_vp)]),
+    "sarek_hip_vector_sub": (_i, [_vp, _i64, _i64, _i64, _i64, C.POINTER(_vp)]),
+    "sarek_hip_vector_sub_meta": (_i, [_vp, C.POINTER(_i), C.POINTER(_i64), C.POINTER(_i64), C.POINTER(_i64),
+                                       C.POINTER(_i64), C.POINTER(_i)]),
+    "sarek_hip_vector_partition": (_i, [_vp, _i, C.POINTER(_i), C.POINTER(_vp)]),
+    "sarek_hip_vector_blit": (_i, [_vp, _i64, _vp, _i64, _i64]),
     "sarek_hip_vector_length": (_i64, [_vp]),
     "sarek_hip_vector_elem_size": (_i64, [_vp]),
     "sarek_hip_vector_kind": (_i, [_vp]),

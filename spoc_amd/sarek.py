@@ -66,6 +66,113 @@ class Vector:
         v.host[:] = array.reshape(-1).astype(kind.dtype, copy=False)      # straight into the host block: stays CPU
         return v
 
+    @classmethod
+    def init(cls, kind, length, f):
+        """Vector.init kind n f."""
+        v = cls.create(kind, length)
+        v.host[:] = np.fromiter((f(i) for i in range(length)), dtype=kind.dtype, count=length)
+        return v
+
+    def fill(self, value):
+        """Vector.fill: the host block, then the bookkeeping of a host write."""
+        elem = np.asarray([value], dtype=self._kind.dtype)
+        hip.check(hip.lib.sarek_hip_vector_fill(self._h, C.c_void_p(elem.ctypes.data)))
+
+    def copy(self):
+        """Vector.copy: host data only (downloaded first if stale), location CPU."""
+        h = C.c_void_p()
+        hip.check(hip.lib.sarek_hip_vector_copy(self._h, C.byref(h)))
+        return Vector(h, self._kind)
+
+    def sub_vector(self, start, length, ok_range=None, ko_range=0):
+        """Vector.sub_vector vec ~start ~len ?ok_range ?ko_range (): shares the host block."""
+        h = C.c_void_p()
+        st = hip.lib.sarek_hip_vector_sub(self._h, start, length, -1 if ok_range is None else ok_range, ko_range,
+                                          C.byref(h))
+        if st == hip.E_INVALID_ARG:
+            raise IndexError(hip.lib.sarek_hip_last_error().decode())      # Invalid_argument in the reference
+        hip.check(st)
+        return Vector(h, self._kind)
+
+    def partition(self, devices):
+        """Vector.partition vec devices: one sub-vector per device id, each Stale_GPU of its device."""
+        n = len(devices)
+        out = (C.c_void_p * max(n, 1))()
+        hip.check(hip.lib.sarek_hip_vector_partition(self._h, n, (C.c_int * max(n, 1))(*devices), out))
+        return [Vector(C.c_void_p(out[i]), self._kind) for i in range(n)]
+
+    @staticmethod
+    def blit(src, src_off, dst, dst_off, length):
+        st = hip.lib.sarek_hip_vector_blit(src._h, src_off, dst._h, dst_off, length)
+        if st == hip.E_INVALID_ARG:
+            raise IndexError(hip.lib.sarek_hip_last_error().decode())
+        hip.check(st)
+
+    def _sub_meta(self):
+        is_sub, depth = C.c_int(0), C.c_int(0)
+        parent, start, ok, ko = C.c_int64(0), C.c_int64(0), C.c_int64(0), C.c_int64(0)
+        hip.check(hip.lib.sarek_hip_vector_sub_meta(self._h, C.byref(is_sub), C.byref(parent), C.byref(start),
+                                                    C.byref(ok), C.byref(ko), C.byref(depth)))
+        return bool(is_sub.value), parent.value, start.value, ok.value, ko.value, depth.value
+
+    @property
+    def id(self):
+        return hip.lib.sarek_hip_vector_id(self._h)
+
+    @property
+    def is_sub(self):
+        return self._sub_meta()[0]
+
+    @property
+    def depth(self):
+        return self._sub_meta()[5]
+
+    @property
+    def parent_id(self):
+        m = self._sub_meta()
+        return m[1] if m[0] else None
+
+    @property
+    def sub_start(self):
+        m = self._sub_meta()
+        return m[2] if m[0] else None
+
+    @property
+    def sub_ok_range(self):
+        m = self._sub_meta()
+        return m[3] if m[0] else None
+
+    @property
+    def sub_ko_range(self):
+        m = self._sub_meta()
+        return m[4] if m[0] else None
+
+    # location queries (Vector.ml:154-172)
+    @property
+    def is_on_cpu(self):
+        return self.location in (CPU, Both, Stale_GPU)
+
+    @property
+    def is_on_gpu(self):
+        return self.location in (GPU, Both, Stale_CPU)
+
+    @property
+    def is_synced(self):
+        return self.location == Both
+
+    @property
+    def needs_gpu_update(self):
+        return self.location == Stale_GPU
+
+    @property
+    def needs_cpu_update(self):
+        return self.location in (Stale_CPU, GPU)
+
+    def __str__(self):
+        buf = C.create_string_buffer(256)
+        hip.check(hip.lib.sarek_hip_vector_to_string(self._h, buf, 256))
+        return buf.value.decode()
+
     def destroy(self):
         if self._h is not None:
             hip.check(hip.lib.sarek_hip_vector_destroy(self._h))
@@ -174,6 +281,41 @@ class Transfer:
     @staticmethod
     def set_auto(enabled):
         hip.check(hip.lib.sarek_hip_transfer_set_auto(int(enabled)))
+
+    # batch operations and streams (Transfer.ml:392-452)
+    @staticmethod
+    def to_device_all(vecs):
+        for v in vecs:
+            Transfer.to_device(v)
+
+    @staticmethod
+    def to_cpu_all(vecs):
+        for v in vecs:
+            Transfer.to_cpu(v)
+
+    @staticmethod
+    def sync_all(vecs):
+        for v in vecs:
+            Transfer.sync(v)
+
+    @staticmethod
+    def create_stream():
+        s = C.c_void_p()
+        hip.check(hip.lib.sarek_hip_stream_create(C.byref(s)))
+        return s
+
+    @staticmethod
+    def default_stream():
+        return C.c_void_p(None)
+
+    @staticmethod
+    def synchronize_stream(stream):
+        hip.check(hip.lib.sarek_hip_stream_synchronize(stream))
+
+    @staticmethod
+    def destroy_stream(stream):
+        if stream is not None and stream.value:          # the default stream is never destroyed
+            hip.check(hip.lib.sarek_hip_stream_destroy(stream))
 
 
 class Execute:

@@ -232,3 +232,132 @@ def test_zero_copy_vectors(torch_cuda):
         hip.check(hip.lib.sarek_hip_mem_alloc_zero_copy(C.c_void_p(pinned.ctypes.data), 64, C.byref(dptr), C.byref(ok)))
         assert ok.value == 1 and dptr.value is not None
         hip.check(hip.lib.sarek_hip_mem_free(dptr))          # a view needs no free; freeing it is harmless
+
+
+# ---- the rest of the Vector module: ids, printing, fill / copy / blit, sub-vectors ----------------
+
+def test_ids_printing_fill_copy_init():
+    a, b = Vector.create(Vector.float32, 8), Vector.create(Vector.int64, 3)
+    assert b.id == a.id + 1 and a.id >= 1                  # Vector_storage.next_id
+    assert str(a) == f"Vector#{a.id}<Float32>[8] @ CPU" and str(b) == f"Vector#{b.id}<Int64>[3] @ CPU"
+    assert str(Vector.create_custom(12, 5)).endswith("<Custom(12)>[5] @ CPU")
+    a.fill(2.5)
+    assert a.location == CPU and np.array_equal(a.to_array(), np.full(8, 2.5, dtype=np.float32))
+    c = a.copy()
+    c[0] = 7.0
+    assert a[0] == 2.5 and c.id > b.id and c.location == CPU and len(c) == 8
+    sq = Vector.init(Vector.int32, 6, lambda i: i * i)
+    assert sq.to_array().tolist() == [0, 1, 4, 9, 16, 25]
+    assert a.is_on_cpu and not a.is_on_gpu and not a.is_synced and not a.needs_gpu_update and not a.needs_cpu_update
+
+
+def test_sub_vectors_share_the_host_block():
+    v = Vector.init(Vector.float32, 10, float)
+    s = v.sub_vector(3, 4)
+    assert (len(s), s.is_sub, s.depth, s.parent_id, s.sub_start, s.sub_ok_range, s.sub_ko_range) == (4, True, 1, v.id, 3, 4, 0)
+    assert (v.is_sub, v.depth, v.parent_id, v.sub_start) == (False, 0, None, None)
+    assert s.to_array().tolist() == [3, 4, 5, 6] and s.location == CPU
+    s[1] = -4.0                                            # one block: the parent sees it
+    v[6] = -6.0
+    assert v[4] == -4.0 and s[3] == -6.0
+    g = s.sub_vector(1, 2, ok_range=1, ko_range=1)          # grandchild: start is relative to its parent
+    assert (g.depth, g.parent_id, g.sub_start, g.sub_ok_range, g.sub_ko_range) == (2, s.id, 1, 1, 1)
+    assert g.to_array().tolist() == [-4.0, 5.0]
+    for start, length in ((-1, 2), (8, 3), (0, 11)):
+        with pytest.raises(IndexError, match=r"sub_vector: range \[-?\d+, \d+\) out of bounds \[0, 10\)"):
+            v.sub_vector(start, length)
+    assert len(v.sub_vector(10, 0)) == 0
+    # the block outlives the parent while a view exists
+    v.destroy()
+    s.destroy()
+    assert g.to_array().tolist() == [-4.0, 5.0]
+
+
+def test_partition_and_blit():
+    v = Vector.init(Vector.int32, 10, int)
+    parts = v.partition([0, 0, 0])                          # Vector_storage.partition_host: 4, 3, 3
+    assert [len(p) for p in parts] == [4, 3, 3] and [p.sub_start for p in parts] == [0, 4, 7]
+    assert all(p.location == Stale_GPU and p.needs_gpu_update and p.depth == 1 for p in parts)
+    assert np.concatenate([p.to_array() for p in parts]).tolist() == list(range(10))
+    assert v.partition([]) == []
+    even = Vector.init(Vector.int32, 7, int).partition([0] * 7)
+    assert [len(p) for p in even] == [1] * 7
+    w = Vector.create(Vector.int32, 6)
+    w.fill(0)
+    Vector.blit(v, 2, w, 1, 4)
+    assert w.to_array().tolist() == [0, 2, 3, 4, 5, 0]
+    Vector.blit(v, 0, v, 1, 5)                               # ascending element order smears the first element
+    assert v.to_array().tolist() == [0, 0, 0, 0, 0, 0, 6, 7, 8, 9]
+    with pytest.raises(IndexError, match="Vector.blit: source range out of bounds"):
+        Vector.blit(v, 8, w, 0, 3)
+    with pytest.raises(IndexError, match="Vector.blit: destination range out of bounds"):
+        Vector.blit(v, 0, w, 4, 3)
+
+
+@gpu
+def test_fill_copy_blit_follow_the_location(torch_cuda):
+    n = 5000
+    v = Vector.init(Vector.float32, n, float)
+    Transfer.to_device(v)
+    assert str(v).startswith(f"Vector#{v.id}<Float32>[{n}] @ Both(") and v.is_synced and v.is_on_gpu and v.is_on_cpu
+    v.fill(1.0)                                            # Both -> Stale_GPU (Vector.ml:230-233)
+    assert v.location == Stale_GPU
+    ir = reference_kernels.vector_add()
+    out = Vector.create(Vector.float32, n)
+    Execute.run_vectors(ir=ir, args=[Execute.Vec(v), Execute.Vec(v), Execute.Vec(out), Execute.Int(n)],
+                        block=Execute.dims1d(256), grid=Execute.dims1d((n + 255) // 256))
+    assert out.location == Stale_CPU and out.needs_cpu_update and not out.is_on_cpu
+    c = out.copy()                                         # downloads first (ensure_cpu_sync), host data only
+    assert out.location == Both and c.location == CPU and c.device_ptr is None
+    assert np.array_equal(c.to_array(), np.full(n, 2.0, dtype=np.float32))
+    # a fill of a Stale_CPU vector is not tracked: the download that follows wins
+    Execute.run_vectors(ir=ir, args=[Execute.Vec(v), Execute.Vec(v), Execute.Vec(out), Execute.Int(n)],
+                        block=Execute.dims1d(256), grid=Execute.dims1d((n + 255) // 256))
+    out.fill(9.0)
+    assert out.location == Stale_CPU and out[0] == 2.0
+    # blit: the source is downloaded first, the destination becomes Stale_GPU
+    Execute.run_vectors(ir=ir, args=[Execute.Vec(v), Execute.Vec(out), Execute.Vec(out), Execute.Int(n)],
+                        block=Execute.dims1d(256), grid=Execute.dims1d((n + 255) // 256))
+    assert out.location == Stale_CPU
+    Transfer.to_device(c)
+    Vector.blit(out, 0, c, 10, 5)
+    assert out.location == Both and c.location == Stale_GPU and c.to_array()[8:16].tolist() == [2, 2, 3, 3, 3, 3, 3, 2]
+
+
+@gpu
+@pytest.mark.parametrize("zero_copy", [False, True])
+def test_kernels_on_sub_vectors_and_partitions(torch_cuda, zero_copy):
+    """A launch on a sub-vector uploads, computes and downloads that range only; the parts of a
+    partition together rebuild the parent on the host (the reference's multi-device pattern, here
+    with every part on the one device)."""
+    n = 100_000
+    v = Vector.create(Vector.float32, n, zero_copy=zero_copy)
+    v.fill_from(np.arange(n))
+    mid = v.sub_vector(1000, 50_000)
+    out = Vector.create(Vector.float32, 50_000)
+    ir = reference_kernels.vector_add()
+    Execute.run_vectors(ir=ir, args=[Execute.Vec(mid), Execute.Vec(mid), Execute.Vec(out), Execute.Int(50_000)],
+                        block=Execute.dims1d(256), grid=Execute.dims1d(196))
+    assert v.location == CPU and mid.location == Stale_CPU and v.device_ptr is None
+    assert np.array_equal(out.to_array(), 2 * np.arange(1000, 51_000, dtype=np.float32))
+    parts = v.partition([0, 0, 0])
+    for p in parts:                                        # p <- p + p, in place, part by part
+        Execute.run_vectors(ir=ir, args=[Execute.Vec(p), Execute.Vec(p), Execute.Vec(p), Execute.Int(len(p))],
+                            block=Execute.dims1d(256), grid=Execute.dims1d((len(p) + 255) // 256))
+    assert all(p.location == Stale_CPU for p in parts)
+    Transfer.to_cpu_all(parts)                             # downloads land in the parent's block
+    assert all(p.location == Both for p in parts)
+    assert np.array_equal(v.host, 2 * np.arange(n, dtype=np.float32))
+    Transfer.sync_all(parts)
+    Transfer.to_device_all(parts)
+
+
+@gpu
+def test_streams(torch_cuda):
+    s = Transfer.create_stream()
+    assert s.value
+    Transfer.synchronize_stream(s)
+    Transfer.destroy_stream(s)
+    d = Transfer.default_stream()
+    Transfer.synchronize_stream(d)
+    Transfer.destroy_stream(d)                             # a no-op, as in the reference
