@@ -320,6 +320,18 @@ int sarek_hip_execute_run_source(const char *source, int lang, const char *kerne
                                  const int block[3], const int grid[3], int shared_mem_bytes,
                                  int inject_lengths, const sarek_hip_varg *args, int n_args);
 int sarek_hip_execute_sync_vectors_to_cpu(const sarek_hip_varg *args, int n_args);
+/* Execute.supports_lang for this backend (sarek/sarek/Execute.ml:589-593): 1 for HIP and CUDA source
+ * (CUDA text is compiled as HIP), 0 otherwise.                                                     */
+int sarek_hip_supports_lang(int lang);
+/* Execute.detect_lang (Execute.ml:658-675) by file extension: .cu, .cl, .ptx, .spv, .comp / .glsl
+ * as there, and .hip for this backend's own language; anything else fails with the reference's
+ * "Invalid file <path>: Unknown source file extension ..." text.                                  */
+int sarek_hip_execute_detect_lang(const char *path, int *lang);
+/* Execute.run_source_file (Execute.ml:711-726): the file's text through run_source in the language
+ * its extension names.                                                                             */
+int sarek_hip_execute_run_source_file(const char *path, const char *kernel_name, const int block[3],
+                                      const int grid[3], int shared_mem_bytes, int inject_lengths,
+                                      const sarek_hip_varg *args, int n_args);
 
 /* ---------------------------------------------------------------------- */
 /* Hand-written CDNA4 kernels.  All pointers are device pointers.  These have

@@ -10,6 +10,7 @@
 //   - a host write marks Both / GPU vectors Stale_GPU and does NOT first fetch a stale
 //     host copy (a write into a Stale_CPU vector is overwritten by the next download);
 //   - a host read downloads a Stale_CPU vector when auto-sync is on (vector and global).
+#include <cstdio>
 #include <cstdlib>
 #include <cstring>
 #include <atomic>
@@ -577,6 +578,12 @@ int sarek_hip_execute_run_source(const char *source, int lang, const char *kerne
   int st = current_device(&dev);
   if (st != SAREK_HIP_OK) return st;
   if ((st = transfer_args(args, n_args, dev)) != SAREK_HIP_OK) return st;
+  // Execute.ml:622-633: checked after the uploads, reported as an unsupported argument
+  if (!sarek_hip_supports_lang(lang)) {
+    static const char *names[] = {"CUDA source", "OpenCL source", "PTX", "SPIR-V", "GLSL source", "HIP source"};
+    return fail(SAREK_HIP_E_UNSUPPORTED, "Unsupported argument type %s in HIP backend",
+                lang >= 0 && lang <= 5 ? names[lang] : "of an unknown source language");
+  }
   std::vector<sarek_hip_arg> rs;
   if ((st = expand_args(args, n_args, dev, inject_lengths != 0, rs)) != SAREK_HIP_OK) return st;
   st = sarek_hip_run_source(source, lang, kernel_name, block, grid, shared_mem_bytes, rs.data(),
@@ -584,6 +591,50 @@ int sarek_hip_execute_run_source(const char *source, int lang, const char *kerne
   if (st != SAREK_HIP_OK) return st;
   mark_stale(args, n_args, dev);
   return SAREK_HIP_OK;
+}
+
+// B.supported_source_langs of this backend, as Execute.supports_lang asks it (Execute.ml:589-593)
+int sarek_hip_supports_lang(int lang) {
+  return lang == SAREK_HIP_LANG_HIP_SOURCE || lang == SAREK_HIP_LANG_CUDA_SOURCE;
+}
+
+// Execute.detect_lang (Execute.ml:658-675), with .hip for this backend's own language
+int sarek_hip_execute_detect_lang(const char *path, int *lang) {
+  if (!path || !lang) return fail(SAREK_HIP_E_INVALID_ARG, "detect_lang: NULL argument");
+  const std::string p(path);
+  auto ends = [&](const char *suffix) {
+    const size_t n = std::strlen(suffix);
+    return p.size() >= n && p.compare(p.size() - n, n, suffix) == 0;
+  };
+  if (ends(".cu")) *lang = SAREK_HIP_LANG_CUDA_SOURCE;
+  else if (ends(".hip")) *lang = SAREK_HIP_LANG_HIP_SOURCE;
+  else if (ends(".cl")) *lang = SAREK_HIP_LANG_OPENCL_SOURCE;
+  else if (ends(".ptx")) *lang = SAREK_HIP_LANG_PTX;
+  else if (ends(".spv")) *lang = SAREK_HIP_LANG_SPIR_V;
+  else if (ends(".comp") || ends(".glsl")) *lang = SAREK_HIP_LANG_GLSL_SOURCE;
+  else
+    return fail(SAREK_HIP_E_INVALID_ARG,
+                "Invalid file %s: Unknown source file extension (expected .cu, .cl, .ptx, .spv, .comp, or .glsl)", path);
+  return SAREK_HIP_OK;
+}
+
+// Execute.run_source_file (Execute.ml:711-726): load_source, detect_lang, run_source
+int sarek_hip_execute_run_source_file(const char *path, const char *kernel_name, const int block[3], const int grid[3],
+                                      int shared_mem_bytes, int inject_lengths, const sarek_hip_varg *args,
+                                      int n_args) {
+  if (!path) return fail(SAREK_HIP_E_INVALID_ARG, "run_source_file: NULL path");
+  std::FILE *f = std::fopen(path, "rb");
+  if (!f) return fail(SAREK_HIP_E_INVALID_ARG, "%s: No such file or directory", path);   // Sys_error in the reference
+  std::string source;
+  char chunk[65536];
+  size_t got;
+  while ((got = std::fread(chunk, 1, sizeof(chunk), f)) > 0) source.append(chunk, got);
+  std::fclose(f);
+  int lang = 0;
+  int st = sarek_hip_execute_detect_lang(path, &lang);
+  if (st != SAREK_HIP_OK) return st;
+  return sarek_hip_execute_run_source(source.c_str(), lang, kernel_name, block, grid, shared_mem_bytes, inject_lengths,
+                                      args, n_args);
 }
 
 // Execute.sync_vectors_to_cpu

@@ -176,6 +176,9 @@ SYMBOLS = {
     "sarek_hip_execute_run_vectors": (_i, [C.c_char_p, _int3, _int3, _i, C.POINTER(VArg), _i]),
     "sarek_hip_execute_run_source": (_i, [C.c_char_p, _i, C.c_char_p, _int3, _int3, _i, _i, C.POINTER(VArg), _i]),
     "sarek_hip_execute_sync_vectors_to_cpu": (_i, [C.POINTER(VArg), _i]),
+    "sarek_hip_supports_lang": (_i, [_i]),
+    "sarek_hip_execute_detect_lang": (_i, [C.c_char_p, C.POINTER(_i)]),
+    "sarek_hip_execute_run_source_file": (_i, [C.c_char_p, C.c_char_p, _int3, _int3, _i, _i, C.POINTER(VArg), _i]),
     "sarek_hip_set_tunable": (_i, [C.c_char_p, _i64]),
     "sarek_hip_set_clock_probe": (_i, [_vp, _i64, C.POINTER(_i64)]),
 }

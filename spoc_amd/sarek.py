@@ -342,6 +342,40 @@ class Execute:
     def dims3d(x, y, z): return (x, y, z)
 
     @staticmethod
+    def grid_for_size(problem_size, block_size):
+        return (problem_size + block_size - 1) // block_size
+
+    @staticmethod
+    def grid_for(problem_size, block_size):
+        return Execute.dims1d(Execute.grid_for_size(problem_size, block_size))
+
+    @staticmethod
+    def supports_lang(lang):
+        return bool(hip.lib.sarek_hip_supports_lang(lang))
+
+    @staticmethod
+    def load_source(path):
+        with open(path) as f:
+            return f.read()
+
+    @staticmethod
+    def detect_lang(path):
+        lang = C.c_int(0)
+        st = hip.lib.sarek_hip_execute_detect_lang(str(path).encode(), C.byref(lang))
+        if st == hip.E_INVALID_ARG:
+            raise ValueError(hip.lib.sarek_hip_last_error().decode())      # Execution_error (Invalid_file ...)
+        hip.check(st)
+        return lang.value
+
+    @staticmethod
+    def run_source_file(path, kernel_name, block, grid, args, shared_mem=0, inject_lengths=True):
+        a, n = Execute._args(args)
+        hip.check(hip.lib.sarek_hip_execute_run_source_file(str(path).encode(), kernel_name.encode(),
+                                                            (C.c_int * 3)(*block), (C.c_int * 3)(*grid), shared_mem,
+                                                            int(inject_lengths), a, n))
+        return hip.lib.sarek_hip_last_run_path().decode()
+
+    @staticmethod
     def _args(args):
         out = (hip.VArg * max(len(args), 1))()
         for a, (kind, v) in zip(out, args):

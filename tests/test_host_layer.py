@@ -173,8 +173,12 @@ def test_run_source_external_kernel_with_and_without_lengths(torch_cuda):
     Execute.run_source(bare, "vadd", (256, 1, 1), (4, 1, 1), args, inject_lengths=False)
     assert np.array_equal(c.to_array(), np.arange(n, dtype=np.float32) * 3 + 1)
     from spoc_amd import hip
-    with pytest.raises(hip.SarekHipError, match="does not support PTX"):           # Cuda_plugin.ml:211-220
+    # Execute.run_source refuses the language itself (Execute.ml:622-633); below it, the plugin's
+    # run_source has its own refusal (Cuda_plugin.ml:211-220)
+    with pytest.raises(hip.SarekHipError, match="Unsupported argument type PTX in HIP backend"):
         Execute.run_source(bare, "vadd", (256, 1, 1), (4, 1, 1), args, lang=hip.LANG_PTX)
+    with pytest.raises(hip.SarekHipError, match="does not support PTX"):
+        hip.run_source(bare, "vadd", (256, 1, 1), (4, 1, 1), [], lang=hip.LANG_PTX)
 
 
 @gpu
@@ -361,3 +365,40 @@ def test_streams(torch_cuda):
     d = Transfer.default_stream()
     Transfer.synchronize_stream(d)
     Transfer.destroy_stream(d)                             # a no-op, as in the reference
+
+
+# ---- external kernels from files (Execute.ml:589-593, 654-726) ------------------------------------
+
+def test_detect_lang_and_grid_helpers():
+    from spoc_amd import hip
+    assert Execute.detect_lang("k/optimized.cu") == hip.LANG_CUDA and Execute.detect_lang("a.hip") == hip.LANG_HIP
+    assert [Execute.detect_lang("x" + e) for e in (".cl", ".ptx", ".spv", ".comp", ".glsl")] == \
+        [hip.LANG_OPENCL, hip.LANG_PTX, hip.LANG_SPIRV, hip.LANG_GLSL, hip.LANG_GLSL]
+    with pytest.raises(ValueError, match=r"Invalid file k.txt: Unknown source file extension \(expected .cu, .cl"):
+        Execute.detect_lang("k.txt")
+    assert Execute.supports_lang(hip.LANG_HIP) and Execute.supports_lang(hip.LANG_CUDA)
+    assert not any(Execute.supports_lang(x) for x in (hip.LANG_OPENCL, hip.LANG_PTX, hip.LANG_SPIRV, hip.LANG_GLSL))
+    assert Execute.grid_for_size(1000, 256) == 4 and Execute.grid_for(1024, 256) == (4, 1, 1)
+
+
+@gpu
+def test_run_source_file(torch_cuda, tmp_path):
+    from spoc_amd import hip
+    n = 3000
+    src = 'extern "C" __global__ void scale(float* x, int len, float f) {\n' \
+          '  int i = blockIdx.x * blockDim.x + threadIdx.x;\n  if (i < len) x[i] *= f;\n}\n'
+    for name in ("scale.cu", "scale.hip"):
+        path = tmp_path / name
+        path.write_text(src)
+        v = Vector.init(Vector.float32, n, float)
+        assert Execute.run_source_file(path, "scale", Execute.dims1d(256), Execute.grid_for(n, 256),
+                                       [Execute.Vec(v), Execute.Float32(0.5)]) == "jit"
+        assert v.location == Stale_CPU and np.array_equal(v.to_array(), np.arange(n, dtype=np.float32) * 0.5)
+    cl = tmp_path / "scale.cl"
+    cl.write_text(src)
+    v = Vector.init(Vector.float32, n, float)
+    with pytest.raises(hip.SarekHipError, match="Unsupported argument type OpenCL source in HIP backend"):
+        Execute.run_source_file(cl, "scale", Execute.dims1d(256), Execute.grid_for(n, 256), [Execute.Vec(v)])
+    assert v.location == Both                              # uploaded before the language is checked (Execute.ml:618-633)
+    with pytest.raises(hip.SarekHipError, match="No such file"):
+        Execute.run_source_file(tmp_path / "none.cu", "scale", Execute.dims1d(1), Execute.dims1d(1), [])
