@@ -50,6 +50,24 @@ int sarek_hip_abi_version(void);
 const char *sarek_hip_last_error(void);
 const char *sarek_hip_status_name(int status);
 
+/* BACKEND.name / version / execution_model (spoc/framework/Framework_sig.ml:137-143,285): "HIP",
+ * (1, 0, 0), JIT.  execute_direct does not exist here: a JIT backend refuses it
+ * (sarek-cuda/Cuda_plugin.ml:158-161).                                                         */
+enum { SAREK_HIP_EXECUTION_JIT = 0, SAREK_HIP_EXECUTION_DIRECT = 1, SAREK_HIP_EXECUTION_CUSTOM = 2 };
+const char *sarek_hip_backend_name(void);
+int sarek_hip_backend_version(int *major, int *minor, int *patch);
+int sarek_hip_execution_model(void);
+/* BACKEND.Intrinsics, an INTRINSIC_REGISTRY (Framework_sig.ml:107-119): name -> device code and
+ * convergence.  Preloaded with the thirteen entries of sarek-cuda/Cuda_plugin.ml:47-143 in HIP
+ * spelling (warp_barrier is a wave barrier); register replaces an entry of the same name; list
+ * writes the names sorted, one per line (*needed = bytes incl. NUL, may be asked with out = NULL,
+ * which returns SAREK_HIP_E_BUFFER_TOO_SMALL).                                                  */
+enum { SAREK_HIP_CONVERGENCE_UNIFORM = 0, SAREK_HIP_CONVERGENCE_DIVERGENT = 1, SAREK_HIP_CONVERGENCE_SYNC = 2 };
+int sarek_hip_intrinsic_register(const char *name, const char *codegen, int convergence);
+int sarek_hip_intrinsic_find(const char *name, char *codegen /* may be NULL */, size_t cap,
+                             int *convergence /* may be NULL */, int *found);
+int sarek_hip_intrinsic_list(char *out, size_t cap, size_t *needed);
+
 /* ---------------------------------------------------------------------- */
 /* Device  (replaces the cuInit, cuDeviceGet.. and cuCtx.. groups,
  * sarek-cuda/Cuda_api.ml:35-179)                                            */

@@ -176,6 +176,12 @@ SYMBOLS = {
     "sarek_hip_execute_run_vectors": (_i, [C.c_char_p, _int3, _int3, _i, C.POINTER(VArg), _i]),
     "sarek_hip_execute_run_source": (_i, [C.c_char_p, _i, C.c_char_p, _int3, _int3, _i, _i, C.POINTER(VArg), _i]),
     "sarek_hip_execute_sync_vectors_to_cpu": (_i, [C.POINTER(VArg), _i]),
+    "sarek_hip_backend_name": (C.c_char_p, []),
+    "sarek_hip_backend_version": (_i, [C.POINTER(_i), C.POINTER(_i), C.POINTER(_i)]),
+    "sarek_hip_execution_model": (_i, []),
+    "sarek_hip_intrinsic_register": (_i, [C.c_char_p, C.c_char_p, _i]),
+    "sarek_hip_intrinsic_find": (_i, [C.c_char_p, C.c_char_p, C.c_size_t, C.POINTER(_i), C.POINTER(_i)]),
+    "sarek_hip_intrinsic_list": (_i, [C.c_char_p, C.c_size_t, C.POINTER(C.c_size_t)]),
     "sarek_hip_supports_lang": (_i, [_i]),
     "sarek_hip_execute_detect_lang": (_i, [C.c_char_p, C.POINTER(_i)]),
     "sarek_hip_execute_run_source_file": (_i, [C.c_char_p, C.c_char_p, _int3, _int3, _i, _i, C.POINTER(VArg), _i]),

@@ -32,6 +32,44 @@ def test_abi_version_and_status_names(hip):
     assert hip.lib.sarek_hip_status_name(-5) == b"SAREK_HIP_E_WORKSPACE"
 
 
+def test_backend_identity_and_intrinsic_registry(hip):
+    """BACKEND.name / version / execution_model and BACKEND.Intrinsics (Framework_sig.ml:107-143,285,314):
+    the lookups of sarek/framework/test/test_framework_integration.ml:190-207 against this backend."""
+    import ctypes as C
+    assert hip.lib.sarek_hip_backend_name() == b"HIP" and hip.lib.sarek_hip_execution_model() == 0      # JIT
+    v = [C.c_int(-1) for _ in range(3)]
+    hip.check(hip.lib.sarek_hip_backend_version(*[C.byref(x) for x in v]))
+    assert [x.value for x in v] == [1, 0, 0]
+
+    def find(name):
+        buf, conv, found = C.create_string_buffer(128), C.c_int(-1), C.c_int(-1)
+        hip.check(hip.lib.sarek_hip_intrinsic_find(name.encode(), buf, 128, C.byref(conv), C.byref(found)))
+        return (buf.value.decode(), conv.value) if found.value else None
+
+    def names():
+        need = C.c_size_t(0)
+        assert hip.lib.sarek_hip_intrinsic_list(None, 0, C.byref(need)) == hip.E_BUFFER_TOO_SMALL
+        buf = C.create_string_buffer(need.value)
+        hip.check(hip.lib.sarek_hip_intrinsic_list(buf, need.value, None))
+        return buf.value.decode().split()
+    UNIFORM, DIVERGENT, SYNC = 0, 1, 2
+    assert find("thread_id_x") == ("threadIdx.x", DIVERGENT) and find("block_dim_z") == ("blockDim.z", UNIFORM)
+    assert find("global_thread_id") == ("(threadIdx.x + blockIdx.x * blockDim.x)", DIVERGENT)
+    assert find("block_barrier") == ("__syncthreads()", SYNC) and find("memory_fence") == ("__threadfence()", UNIFORM)
+    assert find("warp_barrier")[1] == SYNC and "wave" in find("warp_barrier")[0]
+    assert find("no_such_intrinsic") is None
+    before = names()
+    assert before == sorted(before) and len(before) >= 13 and "block_id_y" in before
+    hip.check(hip.lib.sarek_hip_intrinsic_register(b"test_thread_id", b"threadIdx.x", DIVERGENT))
+    hip.check(hip.lib.sarek_hip_intrinsic_register(b"test_thread_id", b"__lane_id()", DIVERGENT))       # replaces
+    assert find("test_thread_id") == ("__lane_id()", DIVERGENT) and names().count("test_thread_id") == 1
+    assert hip.lib.sarek_hip_intrinsic_register(b"x", b"y", 7) == hip.E_INVALID_ARG
+    assert hip.lib.sarek_hip_intrinsic_register(b"", b"y", 0) == hip.E_INVALID_ARG
+    small = C.create_string_buffer(4)
+    found = C.c_int(0)
+    assert hip.lib.sarek_hip_intrinsic_find(b"block_barrier", small, 4, None, C.byref(found)) == hip.E_BUFFER_TOO_SMALL
+
+
 def test_is_available_never_raises(hip):
     # Framework_registry wraps is_available in try (sarek/framework/Framework_registry.ml:77-87)
     assert hip.lib.sarek_hip_is_available() in (0, 1)
