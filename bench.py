@@ -35,6 +35,8 @@ MEASURED_TRAFFIC_BYTES = {
     "gemm_bf16_8192": (793626 * 2 + 262153) * 1024,
     "gemm_f32_8192": (1695900 * 2 + 262153) * 1024,
     "gemm_f16_epilogue": (306687 * 2 + 176779) * 1024,
+    "histogram_2p28": (524312 * 2 + 256) * 1024,
+    "radix_scatter_5e7": (97880 * 2 + 215611) * 1024,
 }
 PEAK_MFMA_TFLOPS = {"bf16": 2500.0, "f16": 2500.0, "f32": 157.3}
 
@@ -46,7 +48,8 @@ def parse():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--workload", default="gemm_bf16_8192",
                     choices=["gemm_bf16_8192", "triad_sum_2p28", "gemm_f32_8192", "gemm_f32_1024",
-                             "gemm_f16_epilogue", "copy_1gib", "vendor_gemm_bf16_8192"])
+                             "gemm_f16_epilogue", "copy_1gib", "vendor_gemm_bf16_8192", "histogram_2p28",
+                             "radix_scatter_5e7"])
     ap.add_argument("--no-also", action="store_true", help="measure only the headline workload")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     return ap.parse_args()
@@ -138,6 +141,36 @@ def make_workload(name, torch, hip):
                     peak=PEAK_MFMA_TFLOPS["bf16"], kernel="hipBLASLt (torch.matmul)",
                     config={"workload": "torch.matmul bf16, N(0,0.02)", "m": s, "n": s, "k": s})
         return (lambda: torch.matmul(a, b, out=c)), info
+    if name == "histogram_2p28":
+        n = 1 << 28
+        g.manual_seed(0xC4)
+        keys = torch.randint(0, 256, (n,), device="cuda", generator=g, dtype=torch.int32)
+        hist = torch.zeros(256, device="cuda", dtype=torch.int32)
+        info = dict(metric="256-bin histogram of int32 keys GB/s", unit="GB/s", dtype="i32",
+                    work=4.0 * n, work_unit=1e9, bound="hbm", peak=PEAK_HBM_GBS,
+                    kernel="histogram_kernel<ModPow2Bin>",
+                    config={"workload": "histogram[key mod 256] += 1, uniform keys", "n": n,
+                            "algorithmic_bytes": 4 * n})
+        return (lambda: hip.histogram(keys, hist, 256)), info
+    if name == "radix_scatter_5e7":
+        n = 50_000_000
+        g.manual_seed(0xC5)
+        keys = torch.randint(0, 100000, (n,), device="cuda", generator=g, dtype=torch.int32)
+        hist = torch.zeros(256, device="cuda", dtype=torch.int32)
+        hip.radix_histogram(keys, hist, 0, 255)
+        starts = (torch.cumsum(hist, 0) - hist).to(torch.int32)
+        out = torch.empty(n, device="cuda", dtype=torch.int32)
+        counters = torch.empty(256, device="cuda", dtype=torch.int32)
+        info = dict(metric="radix-sort scatter pass (8-bit digit) GB/s", unit="GB/s", dtype="i32",
+                    work=8.0 * n, work_unit=1e9, bound="hbm", peak=PEAK_HBM_GBS,
+                    kernel="radix_scatter_kernel<1024, 16> (+ a 1 KiB copy that resets the counters)",
+                    config={"workload": "out[counters[key & 255]++] = key, random keys below 100000", "n": n,
+                            "algorithmic_bytes": 8 * n})
+
+        def step():
+            counters.copy_(starts)
+            hip.radix_scatter(keys, out, counters, 0, 255)
+        return step, info
     if name == "gemm_f16_epilogue":
         m, n, k = 4095, 11008, 4096
         g.manual_seed(0xA5)
@@ -340,7 +373,7 @@ def main():
     if not args.no_also:
         also = []
         for name in ["triad_sum_2p28", "gemm_f32_8192", "gemm_f16_epilogue", "gemm_f32_1024",
-                     "gemm_bf16_8192"]:
+                     "gemm_bf16_8192", "histogram_2p28", "radix_scatter_5e7"]:
             if name == args.workload:
                 continue
             torch.cuda.empty_cache()
