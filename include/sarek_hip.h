@@ -29,7 +29,7 @@
 extern "C" {
 #endif
 
-#define SAREK_HIP_ABI_VERSION 1
+#define SAREK_HIP_ABI_VERSION 2
 
 /* Library-level status codes (negative; HIP codes are positive). */
 #define SAREK_HIP_OK 0
@@ -87,6 +87,8 @@ typedef struct {
   int memory_bus_width_bits;
   int l2_cache_size;
   int compute_major, compute_minor;
+  int max_registers_per_block;  /* Framework_sig.capabilities.max_registers_per_block (the CUDA plugin
+                                   puts a constant 65536 there, sarek-cuda/Cuda_plugin_base.ml:190)      */
 } sarek_hip_device_info;
 
 int sarek_hip_init(void);                       /* hipInit(0); idempotent */

@@ -192,6 +192,7 @@ int sarek_hip_device_get_info(int device, sarek_hip_device_info *out) {
   out->l2_cache_size = p.l2CacheSize;
   out->compute_major = p.major;
   out->compute_minor = p.minor;
+  out->max_registers_per_block = p.regsPerBlock;
   return SAREK_HIP_OK;
 }
 

@@ -46,6 +46,7 @@ class DeviceInfo(C.Structure):
         ("multiprocessor_count", C.c_int), ("clock_rate_khz", C.c_int),
         ("memory_clock_rate_khz", C.c_int), ("memory_bus_width_bits", C.c_int),
         ("l2_cache_size", C.c_int), ("compute_major", C.c_int), ("compute_minor", C.c_int),
+        ("max_registers_per_block", C.c_int),
     ]
 
 

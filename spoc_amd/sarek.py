@@ -22,6 +22,101 @@ CPU, GPU, Both, Stale_CPU, Stale_GPU = "CPU", "GPU", "Both", "Stale_CPU", "Stale
 _LOCATIONS = (CPU, GPU, Both, Stale_CPU, Stale_GPU)
 
 
+class Device:
+    """sarek/core/Device.ml for the one framework of this library: enumeration, the capabilities
+    record (spoc/framework/Framework_sig.ml:26-41, filled as sarek-cuda/Cuda_plugin_base.ml:177-195
+    fills it) and the queries over it."""
+    framework = "HIP"
+
+    def __init__(self, dev_id, info):
+        self.id = self.backend_id = dev_id
+        self.name = info.name.decode()
+        self.arch = info.gcn_arch.decode()
+        self.capabilities = dict(
+            max_threads_per_block=info.max_threads_per_block, max_block_dims=tuple(info.max_block_dim),
+            max_grid_dims=tuple(info.max_grid_dim), shared_mem_per_block=info.shared_mem_per_block,
+            total_global_mem=info.total_global_mem, compute_capability=(info.compute_major, info.compute_minor),
+            supports_fp64=True, supports_atomics=True, warp_size=info.warp_size,
+            max_registers_per_block=info.max_registers_per_block, clock_rate_khz=info.clock_rate_khz,
+            multiprocessor_count=info.multiprocessor_count, is_cpu=False)
+
+    _devices = None
+
+    @classmethod
+    def init(cls):
+        """Device.init: enumerate; an unavailable backend gives no devices rather than an error."""
+        cls._devices = []
+        if hip.lib.sarek_hip_is_available():
+            n = C.c_int(0)
+            hip.check(hip.lib.sarek_hip_device_count(C.byref(n)))
+            cls._devices = [cls(i, hip.device_info(i)) for i in range(n.value)]
+        return cls._devices
+
+    @classmethod
+    def all(cls):
+        return cls._devices if cls._devices is not None else cls.init()
+
+    @classmethod
+    def count(cls):
+        return len(cls.all())
+
+    @classmethod
+    def get(cls, dev_id):
+        devs = cls.all()
+        return devs[dev_id] if 0 <= dev_id < len(devs) else None
+
+    @classmethod
+    def first(cls):
+        return cls.get(0)
+
+    best = first
+
+    @classmethod
+    def by_framework(cls, framework):
+        return [d for d in cls.all() if d.framework == framework]
+
+    @classmethod
+    def reset(cls):
+        cls._devices = None
+
+    def to_string(self):
+        major, minor = self.capabilities["compute_capability"]
+        sm = f"SM {major}.{minor}" if major > 0 else self.framework
+        return (f"[{self.id}] {self.name} ({self.framework}) - {sm}, "
+                f"{self.capabilities['total_global_mem'] / 2 ** 30:.1f} GB, {self.capabilities['multiprocessor_count']} MPs")
+
+    __str__ = to_string
+
+    is_gpu, is_cpu = True, False
+
+    def __getattr__(self, name):            # warp_size, max_threads_per_block, multiprocessor_count, ...
+        caps = self.__dict__.get("capabilities", {})
+        if name in caps:
+            return caps[name]
+        raise AttributeError(name)
+
+    @property
+    def total_memory(self):
+        return self.capabilities["total_global_mem"]
+
+    @property
+    def allows_fp64(self):
+        return self.capabilities["supports_fp64"]
+
+    def free_memory(self):
+        self.set_current()
+        free, total = C.c_size_t(0), C.c_size_t(0)
+        hip.check(hip.lib.sarek_hip_mem_get_info(C.byref(free), C.byref(total)))
+        return free.value
+
+    def set_current(self):
+        hip.check(hip.lib.sarek_hip_device_set_current(self.id))
+
+    def synchronize(self):
+        self.set_current()
+        hip.check(hip.lib.sarek_hip_device_synchronize())
+
+
 class _Kind:
     def __init__(self, code, name, dtype):
         self.code, self.name, self.dtype = code, name, np.dtype(dtype) if dtype is not None else None

@@ -26,7 +26,7 @@ def test_python_binding_covers_the_header(hip):
 
 
 def test_abi_version_and_status_names(hip):
-    assert hip.lib.sarek_hip_abi_version() == 1
+    assert hip.lib.sarek_hip_abi_version() == 2
     assert hip.lib.sarek_hip_status_name(0) == b"SAREK_HIP_OK"
     assert hip.lib.sarek_hip_status_name(-2) == b"SAREK_HIP_E_UNSUPPORTED"
     assert hip.lib.sarek_hip_status_name(-5) == b"SAREK_HIP_E_WORKSPACE"

@@ -6,7 +6,7 @@ import numpy as np
 import pytest
 
 from spoc_amd import reference_kernels
-from spoc_amd.sarek import CPU, Both, Execute, Stale_CPU, Stale_GPU, Transfer, Vector
+from spoc_amd.sarek import CPU, Both, Device, Execute, Stale_CPU, Stale_GPU, Transfer, Vector
 
 gpu = pytest.mark.gpu
 
@@ -402,3 +402,27 @@ def test_run_source_file(torch_cuda, tmp_path):
     assert v.location == Both                              # uploaded before the language is checked (Execute.ml:618-633)
     with pytest.raises(hip.SarekHipError, match="No such file"):
         Execute.run_source_file(tmp_path / "none.cu", "scale", Execute.dims1d(1), Execute.dims1d(1), [])
+
+
+# ---- Device (sarek/core/Device.ml) ------------------------------------------------------------------
+
+def test_device_enumeration_without_a_gpu_gives_no_devices():
+    Device.reset()
+    devs = Device.init()                                   # never raises (Framework_registry.ml:77-87)
+    assert Device.count() == len(devs) and Device.get(len(devs)) is None and Device.get(-1) is None
+    assert Device.by_framework("CUDA") == [] and Device.by_framework("HIP") == devs
+    assert (Device.first() is None) == (len(devs) == 0)
+
+
+@gpu
+def test_device_capabilities(torch_cuda):
+    Device.reset()
+    d = Device.best()
+    assert d is not None and d.id == 0 and d.framework == "HIP" and d.is_gpu and not d.is_cpu
+    assert d.warp_size == 64 and d.multiprocessor_count == 256 and d.max_threads_per_block == 1024
+    assert d.allows_fp64 and d.supports_atomics and d.shared_mem_per_block >= 64 * 1024
+    assert d.max_registers_per_block >= 65536 and d.total_memory > 200 * 2 ** 30 and d.arch.startswith("gfx950")
+    assert 0 < d.free_memory() <= d.total_memory
+    text = d.to_string()
+    assert text.startswith(f"[0] {d.name} (HIP) - SM ") and text.endswith("GB, 256 MPs")
+    d.synchronize()
