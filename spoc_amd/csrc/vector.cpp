@@ -13,11 +13,13 @@
 #include <cstdio>
 #include <cstdlib>
 #include <cstring>
+#include <algorithm>
 #include <atomic>
 #include <map>
 #include <memory>
 #include <mutex>
 #include <string>
+#include <thread>
 #include <unordered_map>
 #include <vector>
 
@@ -149,6 +151,34 @@ int ensure_cpu_sync(sarek_hip_vector_s *v) {
 // Vector.set's bookkeeping (Vector.ml:104-109)
 void host_written(sarek_hip_vector_s *v) {
   if (v->location == SAREK_HIP_LOC_BOTH || v->location == SAREK_HIP_LOC_GPU) v->location = SAREK_HIP_LOC_STALE_GPU;
+}
+
+// Bulk copies between a caller's array and a host block.  One core moves about 30 GB/s; from
+// 16 MiB on the copy is cut into four pieces, three of them on threads of their own (a thread
+// costs some tens of microseconds, a 16 MiB copy half a millisecond).
+void host_copy(void *dst, const void *src, size_t bytes) {
+  constexpr size_t kParallelFrom = size_t{16} << 20;
+  constexpr int kPieces = 4;
+  if (bytes < kParallelFrom) {
+    std::memcpy(dst, src, bytes);
+    return;
+  }
+  const size_t piece = (bytes / kPieces + 4095) & ~size_t{4095};
+  std::thread helpers[kPieces - 1];
+  int started = 0;
+  for (int i = 1; i < kPieces; ++i) {
+    const size_t from = piece * i;
+    if (from >= bytes) break;
+    const size_t len = std::min(piece, bytes - from);
+    try {
+      helpers[started] = std::thread([=] { std::memcpy(static_cast<char *>(dst) + from, static_cast<const char *>(src) + from, len); });
+      ++started;
+    } catch (...) {                      // no thread to be had: this one does the piece itself
+      std::memcpy(static_cast<char *>(dst) + from, static_cast<const char *>(src) + from, len);
+    }
+  }
+  std::memcpy(dst, src, std::min(piece, bytes));
+  for (int i = 0; i < started; ++i) helpers[i].join();
 }
 
 // Range check of a bulk access, reported like the element accessors report theirs
@@ -490,7 +520,7 @@ int sarek_hip_vector_read(sarek_hip_vector v, void *dst, int64_t first, int64_t 
   if (st != SAREK_HIP_OK) return st;
   st = ensure_cpu_sync(v);
   if (st != SAREK_HIP_OK) return st;
-  std::memcpy(dst, static_cast<const char *>(v->host) + first * v->elem_size, static_cast<size_t>(count * v->elem_size));
+  host_copy(dst, static_cast<const char *>(v->host) + first * v->elem_size, static_cast<size_t>(count * v->elem_size));
   return SAREK_HIP_OK;
 }
 
@@ -498,7 +528,7 @@ int sarek_hip_vector_write(sarek_hip_vector v, const void *src, int64_t first, i
   if (!v || (!src && count > 0)) return fail(SAREK_HIP_E_INVALID_ARG, "vector_write: NULL argument");
   int st = bounds(v, first, count, "set");
   if (st != SAREK_HIP_OK) return st;
-  std::memcpy(static_cast<char *>(v->host) + first * v->elem_size, src, static_cast<size_t>(count * v->elem_size));
+  host_copy(static_cast<char *>(v->host) + first * v->elem_size, src, static_cast<size_t>(count * v->elem_size));
   if (count > 0) host_written(v);
   return SAREK_HIP_OK;
 }
