@@ -298,8 +298,11 @@ def bench_gather(size, warmup=5, iterations=20):
 
 def bench_scatter(size, warmup=5, iterations=20):
     """benchmarks/bench_gather_scatter.ml:202-340: input[i] = 3 i + 1, random (colliding) indices,
-    output zeroed on the host before every launch (so its upload is inside the timed sample, as in
-    the reference); every output element is 0 or one of the inputs."""
+    output zeroed with Vector.set before every launch; every output element is 0 or one of the
+    inputs.  After the first launch the output vector is Stale_CPU, and a host write into a
+    Stale_CPU vector is not tracked (sarek/core/Vector.ml:104-109): the zeros of the later
+    iterations stay on the host and the device keeps scattering over its earlier results, in the
+    reference as here, so no upload falls into the timed samples."""
     n = size
     data, idx = (np.arange(n, dtype=np.int64) * 3 + 1).astype(np.int32), _ocaml_random_ints(n, n)
     vin, vidx, vout = _vector(data, Vector.int32), _vector(idx, Vector.int32), _vector(np.zeros(n), Vector.int32)
