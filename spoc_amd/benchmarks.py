@@ -480,8 +480,11 @@ def bench_nbody(size, warmup=5, iterations=20):
 
 def bench_bitonic_sort(size, warmup=5, iterations=20):
     """benchmarks/bench_bitonic_sort.ml:58-215: n = the power of two at or below size, random values
-    below 10000 written again before every sort (so the upload is inside the sample), log^2 n
-    launches per sort, result equal to the sorted input, M elements/s = n / median."""
+    below 10000 written again with Vector.set before every sort, log^2 n launches per sort, result
+    equal to the sorted input, M elements/s = n / median.  Only the first sort sees the random
+    values: after it the vector is Stale_CPU and host writes into it are not tracked
+    (sarek/core/Vector.ml:104-109), so the later sorts run over the sorted device copy, in the
+    reference as here (the network does the same work whatever the data)."""
     n = 1 << int(np.log2(size))
     data = _ocaml_random_ints(n, 10000)
     v = _vector(data, Vector.int32)
