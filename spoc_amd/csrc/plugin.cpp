@@ -315,7 +315,7 @@ int sarek_hip_run_source(const char *source, int lang, const char *kernel_name, 
   }
 
   sarek_hip_kernel k = nullptr;
-  std::vector<char> log(16384);
+  thread_local std::vector<char> log(16384);        // compile log, filled on a failed compile only
   int rc = sarek_hip_kernel_compile_cached(source, kernel_name, &k, log.data(), log.size());
   if (rc != SAREK_HIP_OK) return rc;
 
@@ -329,8 +329,19 @@ int sarek_hip_run_source(const char *source, int lang, const char *kernel_name, 
       double f64;
     };
   };
-  std::vector<Slot> slots(n_args);
-  std::vector<void *> params(n_args);
+  constexpr int kInline = 32;                        // launches with more arguments take the heap
+  Slot inline_slots[kInline];
+  void *inline_params[kInline];
+  std::vector<Slot> heap_slots;
+  std::vector<void *> heap_params;
+  Slot *slots = inline_slots;
+  void **params = inline_params;
+  if (n_args > kInline) {
+    heap_slots.resize(n_args);
+    heap_params.resize(n_args);
+    slots = heap_slots.data();
+    params = heap_params.data();
+  }
   for (int i = 0; i < n_args; ++i) {
     switch (args[i].kind) {
       case SAREK_HIP_ARG_BUFFER: slots[i].p = args[i].buffer; break;
@@ -346,7 +357,7 @@ int sarek_hip_run_source(const char *source, int lang, const char *kernel_name, 
   }
   const unsigned g[3] = {(unsigned)grid[0], (unsigned)grid[1], (unsigned)grid[2]};
   const unsigned b[3] = {(unsigned)block[0], (unsigned)block[1], (unsigned)block[2]};
-  rc = sarek_hip_kernel_launch(k, g, b, (unsigned)shared_mem_bytes, nullptr, params.data(), n_args);
+  rc = sarek_hip_kernel_launch(k, g, b, (unsigned)shared_mem_bytes, nullptr, params, n_args);
   if (rc == SAREK_HIP_OK) t_last_path = "jit";
   return rc;
 }

@@ -9,6 +9,7 @@
 
 #include <cstring>
 #include <map>
+#include <unordered_map>
 #include <mutex>
 #include <set>
 #include <string>
@@ -30,20 +31,34 @@ namespace {
 std::mutex g_mu;
 bool g_inited = false;
 std::set<void *> g_live_allocs;  // device pointers handed out and not yet freed
-std::map<std::string, sarek_hip_kernel> g_kernel_cache;
+// Compiled kernels by (device, kernel name, source text): buckets by hash, the text compared on a hit.
+struct CachedKernel {
+  int dev;
+  std::string name, source;
+  sarek_hip_kernel kernel;
+};
+std::unordered_map<uint64_t, std::vector<CachedKernel>> g_kernel_cache;
 
 int rtc_fail(hiprtcResult r, const char *what) {
   return fail(1000 + static_cast<int>(r), "%s: %s", what, hiprtcGetErrorString(r));
 }
 
-// FNV-1a 64-bit of the source text, for the kernel cache key.
-uint64_t fnv1a(const char *s) {
-  uint64_t h = 1469598103934665603ull;
-  for (; *s; ++s) {
-    h ^= static_cast<unsigned char>(*s);
-    h *= 1099511628211ull;
+// 64-bit hash of the source text, eight bytes a step, for the kernel cache (looked up at every
+// launch: a byte-at-a-time hash of a 2 KB source costs as much as the launch call itself).
+uint64_t hash_text(const char *p, size_t n) {
+  uint64_t h = 0x9E3779B97F4A7C15ull ^ n;
+  while (n >= 8) {
+    uint64_t w;
+    std::memcpy(&w, p, 8);
+    h = (h ^ w) * 0xFF51AFD7ED558CCDull;
+    h ^= h >> 32;
+    p += 8;
+    n -= 8;
   }
-  return h;
+  uint64_t w = 0;
+  std::memcpy(&w, p, n);
+  h = (h ^ w) * 0xC4CEB9FE1A85EC53ull;
+  return h ^ (h >> 29);
 }
 
 void copy_log(const std::string &text, char *log, size_t log_len) {
@@ -339,15 +354,21 @@ int sarek_hip_kernel_compile_cached(const char *source, const char *kernel_name,
     return fail(SAREK_HIP_E_INVALID_ARG, "kernel_compile_cached: NULL argument");
   int dev = 0;
   SAREK_HIP_TRY(hipGetDevice(&dev));
-  char key_buf[64];
-  std::snprintf(key_buf, sizeof(key_buf), "%d:%016llx:%zu:", dev,
-                static_cast<unsigned long long>(fnv1a(source)), std::strlen(source));
-  std::string key = std::string(key_buf) + kernel_name;
+  const size_t len = std::strlen(source);
+  const uint64_t key = hash_text(source, len) ^ (static_cast<uint64_t>(dev) << 56);
+  auto find = [&]() -> sarek_hip_kernel {
+    auto it = g_kernel_cache.find(key);
+    if (it == g_kernel_cache.end()) return nullptr;
+    for (const CachedKernel &c : it->second)
+      if (c.dev == dev && c.source.size() == len && c.name == kernel_name &&
+          std::memcmp(c.source.data(), source, len) == 0)
+        return c.kernel;
+    return nullptr;
+  };
   {
     std::lock_guard<std::mutex> lock(g_mu);
-    auto it = g_kernel_cache.find(key);
-    if (it != g_kernel_cache.end()) {
-      *out = it->second;
+    if (sarek_hip_kernel hit = find()) {
+      *out = hit;
       if (log && log_len) log[0] = '\0';
       return SAREK_HIP_OK;
     }
@@ -357,21 +378,24 @@ int sarek_hip_kernel_compile_cached(const char *source, const char *kernel_name,
   if (rc != SAREK_HIP_OK) return rc;
   k->cached = true;
   std::lock_guard<std::mutex> lock(g_mu);
-  auto ins = g_kernel_cache.emplace(key, k);
-  if (!ins.second) {  // another thread compiled the same source meanwhile
+  if (sarek_hip_kernel other = find()) {  // another thread compiled the same source meanwhile
     (void)hipModuleUnload(k->module);
     delete k;
+    *out = other;
+    return SAREK_HIP_OK;
   }
-  *out = ins.first->second;
+  g_kernel_cache[key].push_back({dev, kernel_name, std::string(source, len), k});
+  *out = k;
   return SAREK_HIP_OK;
 }
 
 int sarek_hip_kernel_clear_cache(void) {
   std::lock_guard<std::mutex> lock(g_mu);
-  for (auto &kv : g_kernel_cache) {
-    (void)hipModuleUnload(kv.second->module);
-    delete kv.second;
-  }
+  for (auto &bucket : g_kernel_cache)
+    for (CachedKernel &c : bucket.second) {
+      (void)hipModuleUnload(c.kernel->module);
+      delete c.kernel;
+    }
   g_kernel_cache.clear();
   return SAREK_HIP_OK;
 }

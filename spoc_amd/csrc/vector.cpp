@@ -250,12 +250,17 @@ struct Lowered {
   std::string name, source;
 };
 std::mutex g_lowered_mu;
-std::unordered_map<std::string, Lowered> g_lowered;
+std::unordered_map<std::string, std::shared_ptr<const Lowered>> g_lowered;
 
-int lower(const char *ir_text, const int block[3], Lowered &out) {
+// The lowering of (ir_text, block), made once: a launch loop calls this every time, so a hit
+// hands out the kept text without copying it.
+int lower(const char *ir_text, const int block[3], std::shared_ptr<const Lowered> &out) {
   // the text can depend on the block (sizes of shared arrays): it is part of the key
-  const std::string key = std::to_string(block[0]) + "," + std::to_string(block[1]) + "," +
-                          std::to_string(block[2]) + ";" + ir_text;
+  thread_local std::string key;
+  char head[48];
+  const int head_len = std::snprintf(head, sizeof(head), "%d,%d,%d;", block[0], block[1], block[2]);
+  key.assign(head, static_cast<size_t>(head_len));
+  key.append(ir_text);
   {
     std::lock_guard<std::mutex> lock(g_lowered_mu);
     auto it = g_lowered.find(key);
@@ -275,8 +280,10 @@ int lower(const char *ir_text, const int block[3], Lowered &out) {
   st = sarek_hip_generate_source(ir_text, block, src.data(), src.size(), &needed);
   if (st != SAREK_HIP_OK) return st;
   src.resize(std::strlen(src.c_str()));
-  out.source = src;
-  out.name = ir::parse_kernel(ir_text).name;
+  auto made = std::make_shared<Lowered>();
+  made->source = src;
+  made->name = ir::parse_kernel(ir_text).name;
+  out = made;
   std::lock_guard<std::mutex> lock(g_lowered_mu);
   if (g_lowered.size() > 256) g_lowered.clear();
   g_lowered[key] = out;
@@ -584,7 +591,7 @@ int sarek_hip_execute_run_vectors(const char *ir_text, const int block[3], const
   int st = current_device(&dev);
   if (st != SAREK_HIP_OK) return st;
   if ((st = transfer_args(args, n_args, dev)) != SAREK_HIP_OK) return st;
-  Lowered k;
+  std::shared_ptr<const Lowered> k;
   try {
     if ((st = lower(ir_text, block, k)) != SAREK_HIP_OK) return st;
   } catch (const std::exception &e) {
@@ -592,7 +599,7 @@ int sarek_hip_execute_run_vectors(const char *ir_text, const int block[3], const
   }
   std::vector<sarek_hip_arg> rs;
   if ((st = expand_args(args, n_args, dev, true, rs)) != SAREK_HIP_OK) return st;
-  st = sarek_hip_run_source(k.source.c_str(), SAREK_HIP_LANG_HIP_SOURCE, k.name.c_str(), block, grid,
+  st = sarek_hip_run_source(k->source.c_str(), SAREK_HIP_LANG_HIP_SOURCE, k->name.c_str(), block, grid,
                             shared_mem_bytes, rs.data(), static_cast<int>(rs.size()));
   if (st != SAREK_HIP_OK) return st;
   mark_stale(args, n_args, dev);
