@@ -87,7 +87,7 @@ int compile_impl(const char *source, const char *kernel_name, sarek_hip_kernel *
     (void)hipRuntimeGetVersion(&runtime_version);
     cache_key = cache_compute_key(std::string(prop.name) + "|" + prop.gcnArchName,
                                   "hiprtc " + std::to_string(rtc_major) + "." + std::to_string(rtc_minor) +
-                                      " hip " + std::to_string(runtime_version) + " -O3",
+                                      " hip " + std::to_string(runtime_version) + " -O3 -packed-fp32-ops",
                                   source);
     std::vector<char> cached;
     if (cache_get(cache_key, &cached) && !cached.empty()) {
@@ -110,8 +110,10 @@ int compile_impl(const char *source, const char *kernel_name, sarek_hip_kernel *
   hiprtcProgram prog;
   hiprtcResult r = hiprtcCreateProgram(&prog, source, "sarek_kernel.hip", 0, nullptr, nullptr);
   if (r != HIPRTC_SUCCESS) return rtc_fail(r, "hiprtcCreateProgram");
-  const char *opts[] = {arch.c_str(), "-O3", "-std=c++17"};
-  r = hiprtcCompileProgram(prog, 3, opts);
+  // Packed FP32 instructions are switched off for generated code as for the library's own kernels
+  // (some of their forms have given wrong results on this hardware without any error).
+  const char *opts[] = {arch.c_str(), "-O3", "-std=c++17", "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"};
+  r = hiprtcCompileProgram(prog, static_cast<int>(sizeof(opts) / sizeof(opts[0])), opts);
   std::string build_log;
   size_t log_size = 0;
   if (hiprtcGetProgramLogSize(prog, &log_size) == HIPRTC_SUCCESS && log_size > 1) {
