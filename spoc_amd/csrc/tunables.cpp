@@ -4,6 +4,7 @@
 #include <map>
 #include <mutex>
 #include <string>
+#include <string_view>
 
 #include <hip/hip_runtime.h>
 
@@ -13,8 +14,9 @@
 namespace sarek_hip {
 namespace {
 std::mutex g_mu;
-std::map<std::string, int64_t> &table() {
-  static std::map<std::string, int64_t> t;
+// looked up by the kernels' launch code at every call: no allocation for the key
+std::map<std::string, int64_t, std::less<>> &table() {
+  static std::map<std::string, int64_t, std::less<>> t;
   return t;
 }
 unsigned long long *g_probe = nullptr;
@@ -29,7 +31,7 @@ unsigned long long *clock_probe(int64_t workgroups) {
 int64_t tunable(const char *name, int64_t fallback) {
   std::lock_guard<std::mutex> lock(g_mu);
   auto &t = table();
-  auto it = t.find(name);
+  auto it = t.find(std::string_view(name));
   if (it != t.end()) return it->second;
   std::string env = "SAREK_HIP_TUNE_";
   for (const char *p = name; *p; ++p) env.push_back(*p == '.' ? '_' : *p);
