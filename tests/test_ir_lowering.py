@@ -348,3 +348,43 @@ def test_nesting_depth_is_bounded(hip):
                   f"{('(var x%d %d i32)' % (i - 1, i + 1)) if i else '(i32 0)'}) " for i in range(lets)) +
           f"(assign (lelem o (i32 0)) (var x{lets - 1} {lets + 1} i32))" + ")" * lets + "))")
     assert f"int x{lets - 1} = " in hip.generate_source(ir)
+
+
+def test_damaged_ir_is_refused_not_crashed_on(hip):
+    """Seeded damage to the fixture kernels (atoms swapped for other atoms, pieces cut out, doubled
+    or replaced, texts truncated): the reader and the lowering answer every one of them with a
+    status, the ones that still mean something with a source."""
+    import ctypes as C
+    import random
+    import re
+    rng = random.Random(20240)
+    texts = [open(os.path.join(IR_DIR, k + ".ir")).read() for k in KERNELS]
+    spare = ["i32", "f32", "(var x 1 i32)", "add", "read", "let", "seq", "(i32 0)", "shared", "vec", "-",
+             "999999999999999999999", '"', "template", "match", "case", "record", "variant", "app", "for", "upto", "mut"]
+    seen = {}
+    for it in range(1500):
+        t = rng.choice(texts)
+        if it % 2 == 0:
+            toks = re.findall(r'\(|\)|"[^"]*"|[^\s()]+', t)
+            atoms = [k for k, x in enumerate(toks) if x not in "()"]
+            for _ in range(rng.randint(1, 4)):
+                a, b = rng.choice(atoms), rng.choice(atoms)
+                toks[a] = toks[b] if rng.random() < 0.7 else rng.choice(spare)
+            t = " ".join(toks)
+        else:
+            for _ in range(rng.randint(1, 3)):
+                if not t:
+                    break
+                i = rng.randrange(len(t))
+                j = min(len(t), i + rng.randint(1, 40))
+                kind = rng.randint(0, 4)
+                t = (t[:i] + t[j:], t[:i] + t[i:j] * 2 + t[j:], t[:i] + rng.choice(spare) + t[j:],
+                     t[:i] + rng.choice(spare) + t[i:], t[:i])[kind]
+        buf, need = C.create_string_buffer(1 << 16), C.c_size_t(0)
+        rc = hip.lib.sarek_hip_generate_source(t.encode(), None, buf, len(buf), C.byref(need))
+        seen[rc] = seen.get(rc, 0) + 1
+        if rc == hip.OK:
+            assert b"__global__" in buf.value
+        else:
+            assert hip.lib.sarek_hip_last_error()
+    assert set(seen) <= {hip.OK, hip.E_PARSE, hip.E_CODEGEN} and seen[hip.OK] > 20 and seen[hip.E_PARSE] > 500
