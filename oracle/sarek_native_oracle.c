@@ -1,7 +1,10 @@
 /*
  * TEST INFRASTRUCTURE ONLY.  CPU restatement of what the reference's Native
  * (OCaml-domains) backend computes for the tiled-GEMM, stream-triad and
- * block-256 tree-reduction kernels.  Nothing in the shipped library links,
+ * block-256 tree-reduction kernels, and for the other bench kernels that
+ * have a hand-written counterpart (vector add and copy, transposes, the
+ * one-thread-per-element matmul, the histogram and the two kernels of a
+ * radix-sort pass).  Nothing in the shipped library links,
  * loads or calls this file; only tests/, __graft_entry__.smoke() and the
  * cpu_baseline leg of bench.py may.
  *
@@ -24,7 +27,11 @@
  * benchmarks/bench_reduction.ml:110-111,154-163;
  * benchmarks/bench_dot_product.ml (inputs, 1e-3 rel); a literal
  * block/thread/superstep restatement of the tiled kernel checked against the
- * closed form; float64 library GEMM cross-checks.
+ * closed form; float64 library GEMM cross-checks; for the later kernels the
+ * benches' own inputs, CPU loops and checks (benchmarks/bench_vector_add.ml,
+ * bench_vector_copy.ml, bench_transpose.ml, bench_matrix_mul.ml,
+ * bench_histogram.ml, bench_radix_sort.ml): sums of f32 pairs, identity and
+ * transposition, numpy's bincount, a stable sort by digit.
  *
  * The bf16 / fp16-input GEMMs and the bias+ReLU+row-sum epilogue have NO
  * counterpart in the reference (it has no 16-bit vector kinds and no fused
