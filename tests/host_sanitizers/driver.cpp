@@ -13,14 +13,20 @@
 #include "sarek_hip.h"
 
 static int damaged_ir(const char *path) {
-  (void)path;
   FILE *f = std::fopen(path, "rb");
   if (!f) return 10;
-  std::string all; char buf[65536]; size_t n;
+  std::string all;
+  char buf[65536];
+  size_t n;
   while ((n = std::fread(buf, 1, sizeof(buf), f)) > 0) all.append(buf, n);
   std::fclose(f);
-  std::vector<std::string> recs; size_t at = 0;
-  while (at < all.size()) { size_t e = all.find('\0', at); if (e == std::string::npos) e = all.size(); recs.emplace_back(all.substr(at, e - at)); at = e + 1; }
+  std::vector<std::string> recs;            // NUL-separated records
+  for (size_t at = 0; at < all.size();) {
+    size_t e = all.find('\0', at);
+    if (e == std::string::npos) e = all.size();
+    recs.emplace_back(all.substr(at, e - at));
+    at = e + 1;
+  }
   std::vector<char> out(1 << 18);
   long ok = 0, bad = 0, fused = 0;
   const int block[3] = {256, 1, 1};
