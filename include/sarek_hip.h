@@ -95,6 +95,10 @@ int sarek_hip_init(void);                       /* hipInit(0); idempotent */
 int sarek_hip_is_available(void);               /* 1/0, never fails (Framework_registry.ml:77-87) */
 int sarek_hip_device_count(int *count);
 int sarek_hip_device_get_info(int device, sarek_hip_device_info *out);
+/* sizeof(sarek_hip_device_info) as this library was built: sarek_hip_device_get_info writes that many
+ * bytes, so a binding checks its own struct against it once (no counterpart in the reference, whose
+ * ctypes layer reads one attribute per call, sarek-cuda/Cuda_api.ml:77-129).                         */
+int sarek_hip_device_info_size(void);
 int sarek_hip_device_set_current(int device);
 int sarek_hip_device_get_current(int *device);
 int sarek_hip_device_synchronize(void);         /* Transfer.flush -> Device.synchronize */

@@ -213,6 +213,8 @@ int sarek_hip_device_get_info(int device, sarek_hip_device_info *out) {
   return SAREK_HIP_OK;
 }
 
+int sarek_hip_device_info_size(void) { return static_cast<int>(sizeof(sarek_hip_device_info)); }
+
 int sarek_hip_device_set_current(int device) {
   SAREK_HIP_TRY(hipSetDevice(device));
   return SAREK_HIP_OK;

@@ -68,6 +68,7 @@ class VArg(C.Structure):
 # Every symbol include/sarek_hip.h declares: (restype, argtypes).
 SYMBOLS = {
     "sarek_hip_abi_version": (_i, []),
+    "sarek_hip_device_info_size": (_i, []),
     "sarek_hip_last_error": (C.c_char_p, []),
     "sarek_hip_status_name": (C.c_char_p, [_i]),
     "sarek_hip_init": (_i, []),

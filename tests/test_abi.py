@@ -26,7 +26,9 @@ def test_python_binding_covers_the_header(hip):
 
 
 def test_abi_version_and_status_names(hip):
-    assert hip.lib.sarek_hip_abi_version() == 2
+    import __graft_entry__ as entry
+    assert hip.lib.sarek_hip_abi_version() == entry.header_abi_version() >= 2
+    entry.check_abi_version()       # the check build() ends with: it follows the header, not a literal
     assert hip.lib.sarek_hip_status_name(0) == b"SAREK_HIP_OK"
     assert hip.lib.sarek_hip_status_name(-2) == b"SAREK_HIP_E_UNSUPPORTED"
     assert hip.lib.sarek_hip_status_name(-5) == b"SAREK_HIP_E_WORKSPACE"
@@ -142,3 +144,36 @@ def test_header_is_c_and_a_c_client_links(hip, tmp_path):
     out = subprocess.run([str(exe)], check=True, capture_output=True, text=True).stdout.strip()
     import hashlib
     assert out == hashlib.md5(b"Device11.0kernel code").hexdigest()
+
+
+def header_device_info_fields():
+    """(name, C type text) of every member of sarek_hip_device_info, in order, from the header."""
+    text = open(os.path.join(ROOT, "include", "sarek_hip.h")).read()
+    body = re.search(r"typedef struct \{(.*?)\} sarek_hip_device_info;", text, flags=re.S).group(1)
+    body = re.sub(r"/\*.*?\*/", "", body, flags=re.S)
+    fields = []
+    for decl in body.split(";"):
+        decl = decl.strip()
+        if not decl:
+            continue
+        ctype, names = decl.split(None, 1)
+        for name in names.split(","):
+            m = re.fullmatch(r"\s*(\w+)\s*(?:\[(\d+)\])?\s*", name)
+            fields.append((m.group(1), ctype, int(m.group(2)) if m.group(2) else None))
+    return fields
+
+
+def test_device_info_layout_agrees_between_header_python_and_documented_ocaml_stub(hip):
+    """sarek_hip_device_get_info fills the whole struct: the Python binding and the OCaml ctypes stub a
+    maintainer copies out of the integration notes must declare every member, in the header's order."""
+    fields = header_device_info_fields()
+    assert [f[0] for f in fields][-1] == "max_registers_per_block"
+    assert [name for name, _ in hip.DeviceInfo._fields_] == [f[0] for f in fields]
+    assert hip.lib.sarek_hip_device_info_size() == ctypes.sizeof(hip.DeviceInfo)
+
+    doc = open(os.path.join(ROOT, "INTEGRATION.md")).read()
+    stub = re.findall(r'field device_info "(\w+)" (\(array (\d+) (\w+)\)|\w+)', doc)
+    ocaml = {"char": "char", "uint64_t": "uint64_t", "int": "int"}
+    assert [(s[0], ocaml[s[3] or s[1]], int(s[2]) if s[2] else None) for s in stub] == fields
+    assert doc.index("max_registers_per_block\" int") < doc.index("seal device_info")
+    assert "sarek_hip_device_info_size" in doc
