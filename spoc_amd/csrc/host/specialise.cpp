@@ -11,7 +11,10 @@
 // lowering: a miss costs speed, never correctness.
 //
 // Normalisation removes what the front end is free to vary without changing meaning:
-//   - immutable `let x = e` bindings are substituted into their bodies,
+//   - immutable `let x = e` bindings are substituted into their bodies when that keeps the
+//     meaning: `e` has no atomic and reads no array or mutable variable that the body stores
+//     to (for arrays: nor may the body hold a barrier or fence); any other binding stays a
+//     statement of the normal form, at its place,
 //   - nested sequences are flattened, scoping blocks and empty statements dropped,
 //   - parameters, mutable variables, loop variables and shared arrays are renamed by
 //     order of first binding,
@@ -24,6 +27,7 @@
 #include <cstdlib>
 #include <cstring>
 #include <map>
+#include <set>
 
 #include "ir.hpp"
 
@@ -154,6 +158,99 @@ struct Canon {
     return false;
   }
 
+  // What a let value depends on beyond constants and immutable bindings.
+  struct Reads {
+    std::set<std::string> arrays;   // by name
+    std::set<std::string> vars;     // keys of mutable and loop variables
+    bool unknown = false;           // calls, matches, reads through an array-valued expression
+  };
+  // What the statements in a let's scope may change while the binding is live.
+  struct Writes {
+    std::set<std::string> arrays;
+    std::set<std::string> vars;
+    bool any_array = false;         // a store through an array-valued expression
+    bool sync = false;              // a barrier or fence: other threads' stores become visible
+    bool unknown = false;           // native code, helper calls
+  };
+
+  static void reads_of(const ExprP &ep, Reads &r) {
+    if (!ep) return;
+    const Expr &e = *ep;
+    switch (e.kind) {
+      case Expr::VarRef:
+        if (e.var.is_mutable) r.vars.insert(key(e.var));
+        break;
+      case Expr::ArrayRead: r.arrays.insert(e.name); break;
+      case Expr::ArrayReadExpr:
+      case Expr::App:
+      case Expr::Match: r.unknown = true; break;
+      default: break;
+    }
+    for (auto &a : e.args) reads_of(a, r);
+    for (auto &f : e.fields) reads_of(f.second, r);
+    for (auto &c : e.cases) reads_of(c.second, r);
+  }
+
+  static void writes_of_expr(const ExprP &ep, Writes &w) {
+    if (!ep) return;
+    const Expr &e = *ep;
+    if (e.kind == Expr::App) w.unknown = true;
+    if (e.kind == Expr::Intrinsic && e.name.compare(0, 6, "atomic") == 0) {
+      if (!e.args.empty() && e.args[0]->kind == Expr::VarRef) w.arrays.insert(e.args[0]->var.name);
+      else w.any_array = true;
+    }
+    for (auto &a : e.args) writes_of_expr(a, w);
+    for (auto &f : e.fields) writes_of_expr(f.second, w);
+    for (auto &c : e.cases) writes_of_expr(c.second, w);
+  }
+
+  static void writes_of_lvalue(const LValueP &l, Writes &w) {
+    if (!l) return;
+    switch (l->kind) {
+      case LValue::LVar: w.vars.insert(key(l->var)); break;
+      case LValue::LArrayElem: w.arrays.insert(l->name); writes_of_expr(l->index, w); break;
+      case LValue::LArrayElemExpr: w.any_array = true; writes_of_expr(l->base, w); writes_of_expr(l->index, w); break;
+      case LValue::LRecordField: writes_of_lvalue(l->inner, w); break;
+    }
+  }
+
+  static void writes_of(const StmtP &sp, Writes &w) {
+    if (!sp) return;
+    const Stmt &s = *sp;
+    switch (s.kind) {
+      case Stmt::Assign: writes_of_lvalue(s.lhs, w); break;
+      case Stmt::Barrier:
+      case Stmt::WarpBarrier:
+      case Stmt::MemFence: w.sync = true; break;
+      case Stmt::Native: w.unknown = true; break;
+      default: break;
+    }
+    writes_of_expr(s.e, w);
+    writes_of_expr(s.e2, w);
+    for (auto &c : s.stmts) writes_of(c, w);
+    for (auto &c : s.cases) writes_of(c.second, w);
+  }
+
+  // Whether `let x = value in scope` means the same with every use of x replaced by `value`:
+  // nothing the value reads may change, or become visible from another thread, while x is live.
+  static bool substitutable(const ExprP &value, const StmtP &scope) {
+    Reads r;
+    reads_of(value, r);
+    if (r.unknown) return false;
+    if (r.arrays.empty() && r.vars.empty()) return true;
+    Writes w;
+    writes_of(scope, w);
+    if (w.unknown) return false;
+    for (auto &v : r.vars)
+      if (w.vars.count(v)) return false;
+    if (!r.arrays.empty()) {
+      if (w.any_array || w.sync) return false;
+      for (auto &a : r.arrays)
+        if (w.arrays.count(a)) return false;
+    }
+    return true;
+  }
+
   std::string lvalue(const LValueP &l) {
     switch (l->kind) {
       case LValue::LVar: {
@@ -201,8 +298,9 @@ struct Canon {
           std::string v = bind(s.var);
           out.push_back("(array " + v + " " + type_tag(s.e->type) + " " + sz +
                         (s.e->mem == MemSpace::Shared ? " shared)" : " local)"));
-        } else if (has_effect(s.e)) {
-          // an atomic returns the old value and changes memory: the binding stays a statement
+        } else if (has_effect(s.e) || !substitutable(s.e, s.stmts[0])) {
+          // an atomic returns the old value and changes memory, and a value that reads what the
+          // scope goes on to change is fixed where it is bound: such a binding stays a statement
           std::string val = expr(s.e);
           std::string v = bind(s.var);
           out.push_back("(bind " + v + " " + val + ")");

@@ -388,3 +388,52 @@ def test_damaged_ir_is_refused_not_crashed_on(hip):
         else:
             assert hip.lib.sarek_hip_last_error()
     assert set(seen) <= {hip.OK, hip.E_PARSE, hip.E_CODEGEN} and seen[hip.OK] > 20 and seen[hip.E_PARSE] > 500
+
+
+def test_a_binding_that_reads_what_its_scope_changes_is_not_inlined(hip):
+    """`let x = e in body` keeps x at the value e had when it was bound.  A recogniser that replaces
+    x by e everywhere would take these kernels for the templates they resemble and serve them with
+    a hand kernel that computes something else."""
+    fixture = lambda name: open(os.path.join(IR_DIR, name)).read()     # noqa: E731
+    # block sum whose stored value is the block's first element, read before the tree runs
+    red = fixture("reduction.ir")
+    assert split_tag(hip.generate_source(red))[0] == "reduce_sum_block256_f32"
+    first_barrier = red.index("(barrier)") + len("(barrier)")
+    hoisted = (red[:first_barrier] + "\n (let (var first 99 f32) (read sdata (i32 0)) (seq" + red[first_barrier:])
+    hoisted = hoisted.replace("(assign (lelem output (intr (Gpu) block_idx_x)) (read sdata (i32 0)))",
+                              "(assign (lelem output (intr (Gpu) block_idx_x)) (var first 99 f32))")
+    hoisted = hoisted.replace("(barrier))))))\n (native_fn", "(barrier))))))))\n (native_fn")
+    tag, src = split_tag(hip.generate_source(hoisted))
+    assert tag == "" and "float first = sdata[0];" in src
+    # the same binding placed after the tree reads the finished sum: the template's own program
+    last = red.rindex("(block (if (eq")
+    late = (red[:last] + "(let (var total 99 f32) (read sdata (i32 0)) (seq " +
+            red[last:].replace("(read sdata (i32 0))", "(var total 99 f32)")
+            .replace("(barrier))))))\n (native_fn", "(barrier))))))))\n (native_fn"))
+    assert "float total = sdata[0];" in hip.generate_source(late)
+    assert split_tag(hip.generate_source(late))[0] == ""      # a barrier follows in its scope: kept as written, no match, JIT
+
+    # tiled matmul that stores the accumulator's value from before the loop
+    mm = fixture("matrix_mul_tiled.ir")
+    assert split_tag(hip.generate_source(mm))[0] == "matmul_tiled_f32"
+    stale = mm.replace("(letmut (var sum 15 f32 mut) (f32 0.0)\n (seq",
+                       "(letmut (var sum 15 f32 mut) (f32 0.0)\n (let (var s0 98 f32) (var sum 15 f32 mut) (seq", 1)
+    stale = stale.replace("(var col 12 i32))) (var sum 15 f32 mut))))))))))))))\n (native_fn",
+                          "(var col 12 i32))) (var s0 98 f32)))))))))))))))\n (native_fn", 1)
+    tag, src = split_tag(hip.generate_source(stale))
+    assert tag == "" and "float s0 = sum;" in src
+
+    # a triad whose operand was read before an earlier store to the same vector (in place: a = a + c*s
+    # with the old a[tid] saved, then a[tid] cleared, then the triad stored)
+    saved = kernel_with_body(
+        "(let (var tid 6 i32) (intr (Std) global_thread_id) (if (lt (var tid 6 i32) (var n 5 i32)) "
+        "(let (var old 7 f32) (read b (var tid 6 i32)) (seq "
+        "(assign (lelem b (var tid 6 i32)) (f32 0.0)) "
+        f"(assign (lelem a (var tid 6 i32)) (add (var old 7 f32) (mul {Cc} {S})))))))",
+        "(param (var a 1 (vec f32))) (param (var b 2 (vec f32))) (param (var c 3 (vec f32))) "
+        "(param (var scalar 4 f32)) (param (var n 5 i32))")
+    tag, src = split_tag(hip.generate_source(saved))
+    assert tag == "" and "float old = b[tid];" in src
+    # the same binding with nothing stored to b in its scope is the triad
+    plain = saved.replace("(assign (lelem b (var tid 6 i32)) (f32 0.0)) ", "")
+    assert split_tag(hip.generate_source(plain))[0] == "stream_triad_f32"
