@@ -379,6 +379,21 @@ int sarek_hip_triad_sum_f32(float *a, const float *b, const float *c, float s, i
                             float *partials, int64_t partials_len, double *sum_out,
                             sarek_hip_stream stream);
 
+/* The same operation for callers that cannot allocate device memory or carry a workspace (code
+ * under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc); it has no
+ * counterpart in the reference.  The partials live in an array inside the library's own device
+ * image (2 MiB per device, held until the process ends), so the call makes no hipMalloc / hipFree
+ * and no allocating library call.  n may be at most sarek_hip_triad_sum_static_max_n() = 2^31
+ * elements; a longer vector is refused with SAREK_HIP_E_WORKSPACE before anything is launched.
+ * Results are bit for bit those of sarek_hip_triad_sum_f32.  All calls on one device share that
+ * device's array: calls that overlap in time on one device (different streams, or different host
+ * threads without ordering between their streams) race on it; calls on one stream do not.  The
+ * first call on a device looks the array's address up (hipGetSymbolAddress); make that call
+ * outside a stream capture.                                                                     */
+int64_t sarek_hip_triad_sum_static_max_n(void);
+int sarek_hip_triad_sum_f32_static(float *a, const float *b, const float *c, float s, int64_t n,
+                                   double *sum_out, sarek_hip_stream stream);
+
 /* Block-256 tree reductions: out[j] = sum of in[256j .. 256j+255] (zero
  * padded), j < ceil(n/256)  (benchmarks/bench_reduction.ml:62-96;
  * generated kernel reduction_generated.md:9-75).  dot: sum of a[i]*b[i]

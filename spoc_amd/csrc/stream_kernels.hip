@@ -12,6 +12,8 @@
 // kernel ("last workgroup to arrive") was measured and rejected: on this multi-XCD chip a
 // device-scope fence writes back a whole L2 (7x slower) and publishing the partials with
 // device-scope atomics instead still cost 25 % of the bandwidth.
+#include <atomic>
+
 #include "common.hpp"
 #include "tunables.hpp"
 
@@ -366,6 +368,36 @@ __global__ void store_f64_kernel(double *p, double v) { *p = v; }
 }  // namespace
 }  // namespace sarek_hip
 
+// Partials of sarek_hip_triad_sum_f32_static: one f32 per triad workgroup (4096 elements), room
+// for vectors of up to 2^31 elements; 2 MiB of every device the library runs on, held until the
+// process ends.  In host code this name is only a handle for hipGetSymbolAddress: kernels get the
+// per-device address kept in g_scratch_addr.
+constexpr int64_t kScratchFloats = int64_t{1} << 19;
+static __device__ __align__(256) float scratch[kScratchFloats];
+
+namespace sarek_hip {
+namespace {
+constexpr int kMaxDevices = 64;
+std::atomic<float *> g_scratch_addr[kMaxDevices];
+
+// Device address of `scratch` on the current device, looked up once per device.
+int scratch_on_current_device(float **out) {
+  int dev = 0;
+  SAREK_HIP_TRY(hipGetDevice(&dev));
+  if (dev < 0 || dev >= kMaxDevices)
+    return fail(SAREK_HIP_E_UNSUPPORTED, "triad_sum_static: device ordinal %d beyond %d", dev, kMaxDevices);
+  float *p = g_scratch_addr[dev].load(std::memory_order_acquire);
+  if (!p) {
+    SAREK_HIP_TRY(hipGetSymbolAddress(reinterpret_cast<void **>(&p), HIP_SYMBOL(scratch)));
+    if (!p) return fail(SAREK_HIP_E_UNSUPPORTED, "triad_sum_static: no device address for the partials array");
+    g_scratch_addr[dev].store(p, std::memory_order_release);
+  }
+  *out = p;
+  return SAREK_HIP_OK;
+}
+}  // namespace
+}  // namespace sarek_hip
+
 using namespace sarek_hip;
 
 extern "C" {
@@ -396,6 +428,30 @@ int sarek_hip_triad_sum_f32(float *a, const float *b, const float *c, float s, i
     hipLaunchKernelGGL(store_f64_kernel, dim3(1), dim3(1), 0, st, sum_out, 0.0);
     return check_launch("triad_sum empty launch");
   }
+  return launch_triad(a, b, c, s, n, partials, sum_out, true, st);
+}
+
+int64_t sarek_hip_triad_sum_static_max_n(void) { return kScratchFloats * kChunk * 4; }
+
+int sarek_hip_triad_sum_f32_static(float *a, const float *b, const float *c, float s, int64_t n,
+                                   double *sum_out, sarek_hip_stream stream) {
+  if (n < 0) return fail(SAREK_HIP_E_INVALID_ARG, "triad_sum_static: negative length %lld", (long long)n);
+  if (!sum_out) return fail(SAREK_HIP_E_INVALID_ARG, "triad_sum_static: NULL sum_out");
+  if (n > 0 && (!a || !b || !c)) return fail(SAREK_HIP_E_INVALID_ARG, "triad_sum_static: NULL vector");
+  if (n > sarek_hip_triad_sum_static_max_n())
+    return fail(SAREK_HIP_E_WORKSPACE,
+                "triad_sum_static: %lld elements, the built-in partials array serves at most %lld "
+                "(use sarek_hip_triad_sum_f32 with a workspace)",
+                (long long)n, (long long)sarek_hip_triad_sum_static_max_n());
+  hipStream_t st = as_stream(stream);
+  if (n == 0) {
+    hipLaunchKernelGGL(store_f64_kernel, dim3(1), dim3(1), 0, st, sum_out, 0.0);
+    return check_launch("triad_sum_static empty launch");
+  }
+  // Every workgroup stores its partial before the fold reads exactly those: nothing has to start at zero.
+  float *partials = nullptr;
+  int rc = scratch_on_current_device(&partials);
+  if (rc != SAREK_HIP_OK) return rc;
   return launch_triad(a, b, c, s, n, partials, sum_out, true, st);
 }
 

@@ -111,6 +111,8 @@ SYMBOLS = {
     "sarek_hip_triad_f32": (_i, [_vp, _vp, _vp, _f, _i64, _vp]),
     "sarek_hip_triad_sum_workspace_floats": (_i64, [_i64]),
     "sarek_hip_triad_sum_f32": (_i, [_vp, _vp, _vp, _f, _i64, _vp, _i64, _vp, _vp]),
+    "sarek_hip_triad_sum_static_max_n": (_i64, []),
+    "sarek_hip_triad_sum_f32_static": (_i, [_vp, _vp, _vp, _f, _i64, _vp, _vp]),
     "sarek_hip_reduce_sum_block256_f32": (_i, [_vp, _vp, _i64, _vp]),
     "sarek_hip_dot_block256_f32": (_i, [_vp, _vp, _vp, _i64, _vp]),
     "sarek_hip_reduce_max_block256_f32": (_i, [_vp, _vp, _i64, _f, _vp]),
