@@ -236,6 +236,24 @@ int sarek_hip_run_source(const char *source, int lang, const char *kernel_name,
                          const int block[3], const int grid[3], int shared_mem_bytes,
                          const sarek_hip_arg *args, int n_args);
 
+/* Library kernels: complete HIP sources, each with a specialise tag on its first line, for the
+ * operations that have no kernel in the reference's suite.  A caller passes the text to
+ * sarek_hip_run_source / sarek_hip_execute_run_source (Execute.run_source ~lang:HIP_Source,
+ * sarek/sarek/Execute.ml:613-651, as sarek/tests/e2e/test_external_kernel.ml:46-62 does with its
+ * own text) with lengths injected; with specialisation on and arguments that fit, the hand-written
+ * kernel runs, otherwise the text itself is compiled and gives the same result under the launch
+ * geometry stated in its comment.  Names, arguments (v = device pointer + int32 length) and geometry:
+ *   gemm_bf16, gemm_f16          (a v, b v, c v, m, n, k)   a, b: 2-byte custom elements (bit patterns),
+ *                                c f32; 2-D launch, one thread per element of C
+ *   gemm_f16_bias_relu_rowsum    (a v, b v, bias v, y v, rowsum v, m, n, k)   1-D launch, any size
+ *   triad_sum_f32                (a v, b v, c v, sum v (float64, >= 1 element), scalar f32, n)
+ *                                one 1-D workgroup of a power-of-two size up to 1024
+ * source / entry: buffers for the text and for the kernel_name to launch it under; *source_needed
+ * gets the text's size incl. NUL (SAREK_HIP_E_BUFFER_TOO_SMALL when it does not fit).            */
+int sarek_hip_library_kernel_source(const char *name, char *source, size_t source_cap, size_t *source_needed,
+                                    char *entry /* may be NULL */, size_t entry_cap);
+int sarek_hip_library_kernel_list(char *out, size_t cap, size_t *needed);   /* names, space separated */
+
 /* 1 (default) / 0: honour specialise tags.  Also read once from the
  * environment variable SAREK_HIP_SPECIALISE (0 disables).                  */
 int sarek_hip_set_specialisation(int enabled);
@@ -338,6 +356,24 @@ typedef struct sarek_hip_varg {
  * "Backend failed to generate source" (Execute.ml:257-263).                        */
 int sarek_hip_execute_run_vectors(const char *ir_text, const int block[3], const int grid[3],
                                   int shared_mem_bytes, const sarek_hip_varg *args, int n_args);
+/* A sequence of kernels over shared vectors, each stage what one Execute.run_vectors call takes:
+ * the launches a caller makes for the kernel list Sarek_fusion.auto_fuse_pipeline hands back
+ * (sarek/sarek/Sarek_fusion.ml:1133-1165; that pass cannot fuse a kernel with barriers, :641-661, so
+ * `stream triad, block-256 tree sum` stays two kernels there).  Stages run in order with the
+ * results of separate launches; two consecutive stages that one hand-written kernel computes in
+ * a single pass over the data (stream triad, then the block-256 sum of the vector it wrote) are
+ * launched as that kernel.  *launches (may be NULL) gets the number of device launches made;
+ * sarek_hip_last_run_path() then reads e.g. "stream_triad_f32+reduce_sum_block256_f32", paths of
+ * separate launches joined by ';'.                                                              */
+typedef struct sarek_hip_pipeline_stage {
+  const char *ir_text;
+  int block[3], grid[3];
+  int shared_mem_bytes;
+  const sarek_hip_varg *args;
+  int n_args;
+} sarek_hip_pipeline_stage;
+int sarek_hip_execute_run_pipeline(const sarek_hip_pipeline_stage *stages, int n_stages, int *launches);
+
 /* Execute.run_source (Execute.ml:613-651): an external kernel; inject_lengths = 0 passes
  * bare buffers (sarek/tests/e2e/test_external_kernel.ml:46-62).                      */
 int sarek_hip_execute_run_source(const char *source, int lang, const char *kernel_name,
@@ -379,6 +415,14 @@ int sarek_hip_triad_sum_f32(float *a, const float *b, const float *c, float s, i
                             float *partials, int64_t partials_len, double *sum_out,
                             sarek_hip_stream stream);
 
+/* The pair `stream triad, then block-256 sum of its output` in one pass over the data: writes a as
+ * sarek_hip_triad_f32 does and block_sums[j] = sum of a[256j .. 256j+255] (zero padded),
+ * j < ceil(n/256), with the bits sarek_hip_reduce_sum_block256_f32 would produce from that a
+ * (benchmarks/bench_stream_triad.ml:22-32 followed by benchmarks/bench_reduction.ml:62-96; what
+ * sarek_hip_execute_run_pipeline launches for that pair of kernels).  Vectors 16-byte aligned. */
+int sarek_hip_triad_block256_sum_f32(float *a, const float *b, const float *c, float s, int64_t n,
+                                     float *block_sums, sarek_hip_stream stream);
+
 /* The same operation for callers that cannot allocate device memory or carry a workspace (code
  * under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc); it has no
  * counterpart in the reference.  The partials live in an array inside the library's own device
@@ -407,8 +451,11 @@ int sarek_hip_dot_block256_f32(const float *a, const float *b, float *out, int64
  * (-1000000.0 in that file); same comparison pairs and order as the tree.   */
 int sarek_hip_reduce_max_block256_f32(const float *in, float *out, int64_t n, float pad,
                                       sarek_hip_stream stream);
-/* *sum_out = left-to-right double fold of partials[0..count)
- * (host fold of benchmarks/bench_reduction.ml:154-160, kept on device).    */
+/* *sum_out = double fold of partials[0..count) in an order fixed by count and the pointer's
+ * alignment (host fold of benchmarks/bench_reduction.ml:154-160, kept on device).  From 2^17
+ * partials on, 256 workgroups fold a piece each into a 2 KiB array inside the library's device
+ * image and one more adds those up: such long folds that overlap in time on one device (different
+ * streams) race on that array; folds on one stream do not.                              */
 int sarek_hip_fold_partials_f64(const float *partials, int64_t count, double *sum_out,
                                 sarek_hip_stream stream);
 

@@ -61,6 +61,12 @@ bool shifted_overlap(const void *p, const void *q, int64_t n) {
   return a != b && a < b + bytes && b < a + bytes;
 }
 
+// Byte ranges [p, p + pb) and [q, q + qb) share a byte.
+bool ranges_meet(const void *p, int64_t pb, const void *q, int64_t qb) {
+  const uintptr_t a = reinterpret_cast<uintptr_t>(p), b = reinterpret_cast<uintptr_t>(q);
+  return a < b + static_cast<uintptr_t>(qb) && b < a + static_cast<uintptr_t>(pb);
+}
+
 // A 1-D launch with at least `threads` threads.
 bool covers_1d(const int block[3], const int grid[3], int64_t threads) {
   return block[1] == 1 && block[2] == 1 && grid[1] == 1 && grid[2] == 1 &&
@@ -80,6 +86,10 @@ int try_specialised(const std::string &tag, const int block[3], const int grid[3
     if (block[0] != 16 || block[1] != 16 || block[2] != 1) return 0;
     if (grid[0] < cdiv(n, 16) || grid[1] < cdiv(m, 16) || grid[2] != 1) return 0;
     if (args[0].length < m * k || args[2].length < k * n || args[4].length < m * n) return 0;
+    // C written over A or B is a race in the generated kernel: left to it
+    if (ranges_meet(args[4].buffer, m * n * 4, args[0].buffer, m * k * 4) ||
+        ranges_meet(args[4].buffer, m * n * 4, args[2].buffer, k * n * 4))
+      return 0;
     *rc = sarek_hip_gemm_f32(static_cast<const float *>(args[0].buffer),
                              static_cast<const float *>(args[2].buffer),
                              static_cast<float *>(args[4].buffer), (int)m, (int)n, (int)k, nullptr);
@@ -95,6 +105,9 @@ int try_specialised(const std::string &tag, const int block[3], const int grid[3
     if (block[1] != 1 || block[2] != 1 || grid[1] != 1 || grid[2] != 1) return 0;
     if (static_cast<int64_t>(block[0]) * grid[0] < n) return 0;
     if (args[0].length < n || args[2].length < n || args[4].length < n) return 0;
+    // in place (a is b or c) is element-wise and fine; a shifted overlap is a race in the generated kernel
+    if (shifted_overlap(args[0].buffer, args[2].buffer, n) || shifted_overlap(args[0].buffer, args[4].buffer, n))
+      return 0;
     *rc = sarek_hip_triad_f32(static_cast<float *>(args[0].buffer),
                               static_cast<const float *>(args[2].buffer),
                               static_cast<const float *>(args[4].buffer), args[6].f32, n, nullptr);
@@ -135,6 +148,9 @@ int try_specialised(const std::string &tag, const int block[3], const int grid[3
     if (m <= 0 || n <= 0 || k <= 0 || m * n > 0x7FFFFFFF) return 0;
     if (!covers_1d(block, grid, m * n)) return 0;
     if (args[0].length < m * k || args[2].length < k * n || args[4].length < m * n) return 0;
+    if (ranges_meet(args[4].buffer, m * n * 4, args[0].buffer, m * k * 4) ||
+        ranges_meet(args[4].buffer, m * n * 4, args[2].buffer, k * n * 4))
+      return 0;
     *rc = sarek_hip_gemm_f32(static_cast<const float *>(args[0].buffer),
                              static_cast<const float *>(args[2].buffer),
                              static_cast<float *>(args[4].buffer), (int)m, (int)n, (int)k, nullptr);
@@ -259,10 +275,118 @@ int try_specialised(const std::string &tag, const int block[3], const int grid[3
                                             static_cast<float *>(args[2].buffer), n, pad, nullptr);
     return 1;
   }
+  // ---- the library kernels (texts from sarek_hip_library_kernel_source) -----------------------
+  if (tag == "gemm_bf16" || tag == "gemm_f16") {
+    // (a, len, b, len, c, len, m, n, k); a, b: 2-byte elements; 2-D launch, one thread per element of C
+    if (n_args != 9 || !vec_at(args, n_args, 0) || !vec_at(args, n_args, 2) || !vec_at(args, n_args, 4) ||
+        !is_i32(args[6]) || !is_i32(args[7]) || !is_i32(args[8]))
+      return 0;
+    const int64_t m = args[6].i32, n = args[7].i32, k = args[8].i32;
+    if (m <= 0 || n <= 0 || k <= 0) return 0;
+    if (block[2] != 1 || grid[2] != 1) return 0;
+    if (static_cast<int64_t>(block[0]) * grid[0] < n || static_cast<int64_t>(block[1]) * grid[1] < m) return 0;
+    if (args[0].length < m * k || args[2].length < k * n || args[4].length < m * n) return 0;
+    if (ranges_meet(args[4].buffer, m * n * 4, args[0].buffer, m * k * 2) ||
+        ranges_meet(args[4].buffer, m * n * 4, args[2].buffer, k * n * 2))
+      return 0;
+    auto fn = tag == "gemm_bf16" ? sarek_hip_gemm_bf16 : sarek_hip_gemm_f16;
+    *rc = fn(static_cast<const uint16_t *>(args[0].buffer), static_cast<const uint16_t *>(args[2].buffer),
+             static_cast<float *>(args[4].buffer), (int)m, (int)n, (int)k, nullptr);
+    return 1;
+  }
+  if (tag == "gemm_f16_bias_relu_rowsum") {
+    // (a, len, b, len, bias, len, y, len, rowsum, len, m, n, k); 1-D launch, workgroups take whole rows
+    if (n_args != 13) return 0;
+    for (int v = 0; v < 5; ++v)
+      if (!vec_at(args, n_args, 2 * v)) return 0;
+    if (!is_i32(args[10]) || !is_i32(args[11]) || !is_i32(args[12])) return 0;
+    const int64_t m = args[10].i32, n = args[11].i32, k = args[12].i32;
+    if (m <= 0 || n <= 0 || k <= 0) return 0;
+    if (block[1] != 1 || block[2] != 1 || grid[1] != 1 || grid[2] != 1) return 0;
+    if (args[0].length < m * k || args[2].length < k * n || args[4].length < n || args[6].length < m * n ||
+        args[8].length < m)
+      return 0;
+    const void *ptr[5] = {args[0].buffer, args[2].buffer, args[4].buffer, args[6].buffer, args[8].buffer};
+    const int64_t bytes[5] = {m * k * 2, k * n * 2, n * 4, m * n * 4, m * 4};
+    for (int out = 3; out < 5; ++out)          // y and rowsum against everything else
+      for (int other = 0; other < 5; ++other)
+        if (other != out && ranges_meet(ptr[out], bytes[out], ptr[other], bytes[other])) return 0;
+    *rc = sarek_hip_gemm_f16_bias_relu_rowsum(static_cast<const uint16_t *>(args[0].buffer),
+                                              static_cast<const uint16_t *>(args[2].buffer),
+                                              static_cast<const float *>(args[4].buffer),
+                                              static_cast<float *>(args[6].buffer),
+                                              static_cast<float *>(args[8].buffer), (int)m, (int)n, (int)k, nullptr);
+    return 1;
+  }
+  if (tag == "triad_sum_f32") {
+    // (a, len, b, len, c, len, sum (f64), len, scalar, n); one 1-D workgroup of a power-of-two size
+    if (n_args != 10 || !vec_at(args, n_args, 0) || !vec_at(args, n_args, 2) || !vec_at(args, n_args, 4) ||
+        !vec_at(args, n_args, 6) || !is_f32(args[8]) || !is_i32(args[9]))
+      return 0;
+    const int64_t n = args[9].i32;
+    if (n < 0) return 0;
+    if (grid[0] != 1 || grid[1] != 1 || grid[2] != 1 || block[1] != 1 || block[2] != 1) return 0;
+    if (block[0] > 1024 || (block[0] & (block[0] - 1)) != 0) return 0;
+    if (args[0].length < n || args[2].length < n || args[4].length < n || args[6].length < 1) return 0;
+    if (shifted_overlap(args[0].buffer, args[2].buffer, n) || shifted_overlap(args[0].buffer, args[4].buffer, n))
+      return 0;
+    for (int v = 0; v < 3; ++v)
+      if (ranges_meet(args[6].buffer, 8, args[2 * v].buffer, n * 4)) return 0;
+    if (reinterpret_cast<uintptr_t>(args[6].buffer) % 8 != 0) return 0;
+    // n is an int32: always within what the library's own partials array serves
+    *rc = sarek_hip_triad_sum_f32_static(static_cast<float *>(args[0].buffer),
+                                         static_cast<const float *>(args[2].buffer),
+                                         static_cast<const float *>(args[4].buffer), args[8].f32, n,
+                                         static_cast<double *>(args[6].buffer), nullptr);
+    return 1;
+  }
   return 0;
 }
 
+// The pair `stream triad, then the block-256 sum of the triad's output`, both recognised from IR,
+// served by one pass over the data.  Conditions: each launch alone would be taken over (same
+// checks as above), the sum reads exactly the vector the triad writes, over the same n, and its
+// output lies apart from the triad's three vectors.
+int try_specialised_pair(const std::string &tag0, const int block0[3], const int grid0[3],
+                         const sarek_hip_arg *a0, int n0, const std::string &tag1, const int block1[3],
+                         const int grid1[3], const sarek_hip_arg *a1, int n1, int *rc) {
+  if (tag0 != "stream_triad_f32" || tag1 != "reduce_sum_block256_f32") return 0;
+  if (n0 != 8 || !vec_at(a0, n0, 0) || !vec_at(a0, n0, 2) || !vec_at(a0, n0, 4) || !is_f32(a0[6]) || !is_i32(a0[7]))
+    return 0;
+  if (n1 != 5 || !vec_at(a1, n1, 0) || !vec_at(a1, n1, 2) || !is_i32(a1[4])) return 0;
+  const int64_t n = a0[7].i32;
+  if (n <= 0 || a1[4].i32 != n) return 0;
+  if (!covers_1d(block0, grid0, n)) return 0;
+  if (a0[0].length < n || a0[2].length < n || a0[4].length < n) return 0;
+  if (shifted_overlap(a0[0].buffer, a0[2].buffer, n) || shifted_overlap(a0[0].buffer, a0[4].buffer, n)) return 0;
+  const int64_t nblocks = cdiv(n, 256);
+  if (block1[0] != 256 || block1[1] != 1 || block1[2] != 1 || grid1[1] != 1 || grid1[2] != 1) return 0;
+  if (grid1[0] != nblocks) return 0;
+  if (a1[0].buffer != a0[0].buffer || a1[0].length < n || a1[2].length < nblocks) return 0;
+  for (int v = 0; v < 3; ++v) {
+    if (reinterpret_cast<uintptr_t>(a0[2 * v].buffer) % 16 != 0) return 0;
+    if (ranges_meet(a1[2].buffer, nblocks * 4, a0[2 * v].buffer, n * 4)) return 0;
+  }
+  *rc = sarek_hip_triad_block256_sum_f32(static_cast<float *>(a0[0].buffer), static_cast<const float *>(a0[2].buffer),
+                                         static_cast<const float *>(a0[4].buffer), a0[6].f32, n,
+                                         static_cast<float *>(a1[2].buffer), nullptr);
+  return 1;
+}
+
 }  // namespace
+
+void set_last_run_path(const std::string &path) { t_last_path = path; }
+
+int run_specialised_pair(const char *source0, const int block0[3], const int grid0[3], const sarek_hip_arg *args0,
+                         int n_args0, const char *source1, const int block1[3], const int grid1[3],
+                         const sarek_hip_arg *args1, int n_args1, int *rc) {
+  if (!specialisation_enabled()) return 0;
+  const std::string tag0 = read_tag(source0), tag1 = read_tag(source1);
+  if (tag0.empty() || tag1.empty()) return 0;
+  if (!try_specialised_pair(tag0, block0, grid0, args0, n_args0, tag1, block1, grid1, args1, n_args1, rc)) return 0;
+  t_last_path = tag0 + "+" + tag1;
+  return 1;
+}
 }  // namespace sarek_hip
 
 using namespace sarek_hip;

@@ -80,9 +80,18 @@ __device__ __forceinline__ void stg_nt(float4 *p, float4 v) {
   __builtin_nontemporal_store(w, reinterpret_cast<f32x4_t *>(p));
 }
 
+// What a triad launch leaves besides `a`.
+enum : int {
+  SUM_NONE = 0,
+  SUM_WORKGROUP = 1,   // partials[g] = f32 sum of workgroup g's 4096 elements
+  SUM_BLOCK256 = 2     // partials[j] = f32 sum of a[256j .. 256j+255], the reference's block-256 kernel's output
+};
+
 // a = b + c*s.  Workgroup g owns float4 [g*kChunk, (g+1)*kChunk); the last one also takes
-// the (n & 3) scalar tail.  When WithSum, partials[g] gets the workgroup's f32 sum.
-template <bool WithSum, bool NtLoad = true>
+// the (n & 3) scalar tail.  Float4 slot base + u*256 of a wave is one 256-element block of the
+// reference's tree kernel (64 lanes x 4 elements), so SUM_BLOCK256 needs one wave reduction per
+// load and no LDS; its lane and wave order is block256_kernel's, the results are the same bits.
+template <int Sum, bool NtLoad = true>
 __global__ __launch_bounds__(kBlock) void triad_kernel(float *__restrict__ a,
                                                        const float *__restrict__ b,
                                                        const float *__restrict__ c, float s,
@@ -92,10 +101,10 @@ __global__ __launch_bounds__(kBlock) void triad_kernel(float *__restrict__ a,
   float4 *a4 = reinterpret_cast<float4 *>(a);
   const float4 *b4 = reinterpret_cast<const float4 *>(b);
   const float4 *c4 = reinterpret_cast<const float4 *>(c);
-  float4 acc = make_float4(0.f, 0.f, 0.f, 0.f);
   const int64_t base = static_cast<int64_t>(blockIdx.x) * kChunk + threadIdx.x;
   const bool full = base + (kUnroll - 1) * kBlock < n4;
   float4 r[kUnroll];
+  float extra[kUnroll];   // SUM_BLOCK256: the scalar tail's share of the block that holds it
   if (full) {
     float4 bv[kUnroll], cv[kUnroll];
 #pragma unroll
@@ -103,27 +112,50 @@ __global__ __launch_bounds__(kBlock) void triad_kernel(float *__restrict__ a,
 #pragma unroll
     for (int u = 0; u < kUnroll; ++u) cv[u] = NtLoad ? ldg_nt(c4 + base + u * kBlock) : c4[base + u * kBlock];
 #pragma unroll
-    for (int u = 0; u < kUnroll; ++u) r[u] = triad4(bv[u], cv[u], sd);
+    for (int u = 0; u < kUnroll; ++u) {
+      r[u] = triad4(bv[u], cv[u], sd);
+      extra[u] = 0.f;
+    }
   } else {
 #pragma unroll
     for (int u = 0; u < kUnroll; ++u) {
       const int64_t i = base + u * kBlock;
       r[u] = i < n4 ? triad4(b4[i], c4[i], sd) : make_float4(0.f, 0.f, 0.f, 0.f);
+      extra[u] = 0.f;
+      if (Sum == SUM_BLOCK256 && i == n4) {
+        // the lane whose float4 slot holds the end of the vector takes the one to three elements there
+        for (int64_t e = n4 << 2; e < n; ++e) {
+          const float v = triad1(b[e], c[e], sd);
+          a[e] = v;
+          extra[u] += v;
+        }
+      }
     }
   }
   // scalar tail: at most three elements, taken by the first threads of the last workgroup
   float tail = 0.f;
   const int64_t ti = (n4 << 2) + threadIdx.x;
-  const bool has_tail = blockIdx.x == gridDim.x - 1 && ti < n;
+  const bool has_tail = Sum != SUM_BLOCK256 && blockIdx.x == gridDim.x - 1 && ti < n;
   if (has_tail) tail = triad1(b[ti], c[ti], sd);
 
-  if (WithSum) {
+  if (Sum == SUM_WORKGROUP) {
+    float4 acc = make_float4(0.f, 0.f, 0.f, 0.f);
 #pragma unroll
     for (int u = 0; u < kUnroll; ++u) {
       acc.x += r[u].x; acc.y += r[u].y; acc.z += r[u].z; acc.w += r[u].w;
     }
     float t = block_sum(((acc.x + acc.y) + (acc.z + acc.w)) + tail);
     if (threadIdx.x == 0) partials[blockIdx.x] = t;
+  }
+  if (Sum == SUM_BLOCK256) {
+    const int64_t nblocks = (n + 255) >> 8;
+    const int64_t j0 = static_cast<int64_t>(blockIdx.x) * (kChunk / 64) + (threadIdx.x >> 6);
+#pragma unroll
+    for (int u = 0; u < kUnroll; ++u) {
+      const float t = wave_sum(((r[u].x + r[u].y) + (r[u].z + r[u].w)) + extra[u]);
+      const int64_t j = j0 + u * (kBlock / 64);
+      if ((threadIdx.x & 63) == 0 && j < nblocks) partials[j] = t;
+    }
   }
 
   if (full) {
@@ -160,16 +192,15 @@ __global__ __launch_bounds__(kBlock) void triad_scalar_kernel(float *__restrict_
   }
 }
 
-// *out = sum of partials[0..count) accumulated in double by one block.  Each thread takes
-// float4 pieces at a stride of 1024 pieces, eight loads in flight, then a tree in LDS; the
-// summation order is fixed by (count, thread layout) only.
-__global__ __launch_bounds__(1024) void fold_kernel(const float *__restrict__ partials,
-                                                    int64_t count, double *__restrict__ out) {
+// Double sum of x[0..count) by one 1024-thread block, valid in thread 0.  Each thread takes float4
+// pieces at a stride of 1024 pieces, eight loads in flight, then a tree in LDS; the summation
+// order is fixed by (count, the pointer's alignment, thread layout) only.
+__device__ __forceinline__ double fold_block(const float *__restrict__ x, int64_t count) {
   __shared__ double sh[1024];
   double acc = 0.0;
-  const bool vec = (reinterpret_cast<uintptr_t>(partials) & 15u) == 0;
+  const bool vec = (reinterpret_cast<uintptr_t>(x) & 15u) == 0;
   const int64_t n4 = vec ? count >> 2 : 0;
-  const float4 *p4 = reinterpret_cast<const float4 *>(partials);
+  const float4 *p4 = reinterpret_cast<const float4 *>(x);
   int64_t i = threadIdx.x;
   for (; i + 7 * 1024 < n4; i += 8 * 1024) {
     float4 v[8];
@@ -185,10 +216,41 @@ __global__ __launch_bounds__(1024) void fold_kernel(const float *__restrict__ pa
     acc += (static_cast<double>(v.x) + static_cast<double>(v.y)) +
            (static_cast<double>(v.z) + static_cast<double>(v.w));
   }
-  for (int64_t j = (n4 << 2) + threadIdx.x; j < count; j += 1024) acc += static_cast<double>(partials[j]);
+  for (int64_t j = (n4 << 2) + threadIdx.x; j < count; j += 1024) acc += static_cast<double>(x[j]);
   sh[threadIdx.x] = acc;
   __syncthreads();
   for (int half = 512; half >= 1; half >>= 1) {
+    if (static_cast<int>(threadIdx.x) < half) sh[threadIdx.x] += sh[threadIdx.x + half];
+    __syncthreads();
+  }
+  return sh[0];
+}
+
+// *out = sum of partials[0..count) accumulated in double by one block.
+__global__ __launch_bounds__(1024) void fold_kernel(const float *__restrict__ partials,
+                                                    int64_t count, double *__restrict__ out) {
+  const double t = fold_block(partials, count);
+  if (threadIdx.x == 0) *out = t;
+}
+
+// Long inputs in two steps: workgroup g sums the pieces [g*piece, (g+1)*piece) into stage[g], then
+// one workgroup adds the stage up in index order.  `piece` is a multiple of 4, so every
+// workgroup sees its piece at the alignment of the whole.
+constexpr int kFoldGroups = 256;
+__global__ __launch_bounds__(1024) void fold_pieces_kernel(const float *__restrict__ partials, int64_t count,
+                                                           int64_t piece, double *__restrict__ stage) {
+  const int64_t lo = static_cast<int64_t>(blockIdx.x) * piece;
+  const int64_t len = lo >= count ? 0 : (count - lo < piece ? count - lo : piece);
+  const double t = fold_block(partials + lo, len);
+  if (threadIdx.x == 0) stage[blockIdx.x] = t;
+}
+
+__global__ __launch_bounds__(kFoldGroups) void fold_stage_kernel(const double *__restrict__ stage,
+                                                                 double *__restrict__ out) {
+  __shared__ double sh[kFoldGroups];
+  sh[threadIdx.x] = stage[threadIdx.x];
+  __syncthreads();
+  for (int half = kFoldGroups / 2; half >= 1; half >>= 1) {
     if (static_cast<int>(threadIdx.x) < half) sh[threadIdx.x] += sh[threadIdx.x + half];
     __syncthreads();
   }
@@ -236,9 +298,9 @@ __global__ __launch_bounds__(kBlock) void block256_kernel(const float *__restric
   // the group that holds the end of the input
   for (int u = 0; u < U && j0 + u < nblocks; ++u) {
     const int64_t i = (j0 + u) * 256 + lane * 4;
-    float v = 0.f;
-    for (int e = 0; e < 4; ++e)
-      if (i + e < n) v += Dot ? x[i + e] * y[i + e] : x[i + e];
+    float t[4];
+    for (int e = 0; e < 4; ++e) t[e] = i + e < n ? (Dot ? x[i + e] * y[i + e] : x[i + e]) : 0.f;
+    float v = (t[0] + t[1]) + (t[2] + t[3]);   // the pairing of the full groups above
     v = wave_sum(v);
     if (lane == 0) out[j0 + u] = v;
   }
@@ -330,6 +392,8 @@ inline int64_t triad_blocks(int64_t n) {
   return ceil_div(n > 0 ? n : 1, static_cast<int64_t>(kChunk) * 4);
 }
 
+int launch_fold(const float *partials, int64_t count, double *sum_out, hipStream_t st);
+
 int launch_triad(float *a, const float *b, const float *c, float s, int64_t n, float *partials,
                  double *sum_out, bool with_sum, hipStream_t st) {
   const bool vec = aligned16(a) && aligned16(b) && aligned16(c);
@@ -339,15 +403,14 @@ int launch_triad(float *a, const float *b, const float *c, float s, int64_t n, f
   if (vec) {
     const bool nt = streams_from_hbm(n * 8);
     if (with_sum) {
-      if (nt) hipLaunchKernelGGL((triad_kernel<true, true>), dim3(blocks), dim3(kBlock), 0, st, a, b, c, s, n, partials);
-      else hipLaunchKernelGGL((triad_kernel<true, false>), dim3(blocks), dim3(kBlock), 0, st, a, b, c, s, n, partials);
+      if (nt) hipLaunchKernelGGL((triad_kernel<SUM_WORKGROUP, true>), dim3(blocks), dim3(kBlock), 0, st, a, b, c, s, n, partials);
+      else hipLaunchKernelGGL((triad_kernel<SUM_WORKGROUP, false>), dim3(blocks), dim3(kBlock), 0, st, a, b, c, s, n, partials);
       int rc = check_launch("triad kernel launch");
       if (rc != SAREK_HIP_OK) return rc;
-      hipLaunchKernelGGL(fold_kernel, dim3(1), dim3(1024), 0, st, partials, blocks64, sum_out);
-      return check_launch("fold kernel launch");
+      return launch_fold(partials, blocks64, sum_out, st);
     }
-    if (nt) hipLaunchKernelGGL((triad_kernel<false, true>), dim3(blocks), dim3(kBlock), 0, st, a, b, c, s, n, partials);
-    else hipLaunchKernelGGL((triad_kernel<false, false>), dim3(blocks), dim3(kBlock), 0, st, a, b, c, s, n, partials);
+    if (nt) hipLaunchKernelGGL((triad_kernel<SUM_NONE, true>), dim3(blocks), dim3(kBlock), 0, st, a, b, c, s, n, partials);
+    else hipLaunchKernelGGL((triad_kernel<SUM_NONE, false>), dim3(blocks), dim3(kBlock), 0, st, a, b, c, s, n, partials);
     return check_launch("triad kernel launch");
   }
   // 4-byte aligned vectors: scalar kernel on a capped grid, then a separate fold
@@ -356,8 +419,7 @@ int launch_triad(float *a, const float *b, const float *c, float s, int64_t n, f
     hipLaunchKernelGGL(triad_scalar_kernel<true>, dim3(sblocks), dim3(kBlock), 0, st, a, b, c, s, n, partials);
     int rc = check_launch("triad kernel launch");
     if (rc != SAREK_HIP_OK) return rc;
-    hipLaunchKernelGGL(fold_kernel, dim3(1), dim3(1024), 0, st, partials, (int64_t)sblocks, sum_out);
-    return check_launch("fold kernel launch");
+    return launch_fold(partials, (int64_t)sblocks, sum_out, st);
   }
   hipLaunchKernelGGL(triad_scalar_kernel<false>, dim3(sblocks), dim3(kBlock), 0, st, a, b, c, s, n, partials);
   return check_launch("triad kernel launch");
@@ -375,25 +437,54 @@ __global__ void store_f64_kernel(double *p, double v) { *p = v; }
 constexpr int64_t kScratchFloats = int64_t{1} << 19;
 static __device__ __align__(256) float scratch[kScratchFloats];
 
+// Stage of a long fold: one double per workgroup of fold_pieces_kernel (2 KiB per device).
+static __device__ __align__(256) double fold_stage[sarek_hip::kFoldGroups];
+
 namespace sarek_hip {
 namespace {
 constexpr int kMaxDevices = 64;
 std::atomic<float *> g_scratch_addr[kMaxDevices];
+std::atomic<double *> g_fold_stage_addr[kMaxDevices];
 
-// Device address of `scratch` on the current device, looked up once per device.
-int scratch_on_current_device(float **out) {
+// Device address of a file-scope __device__ array on the current device, looked up once per
+// device: every device holds its own copy of the array at its own address.
+template <typename T>
+int address_on_current_device(std::atomic<T *> *table, const void *symbol, const char *what, T **out) {
   int dev = 0;
   SAREK_HIP_TRY(hipGetDevice(&dev));
   if (dev < 0 || dev >= kMaxDevices)
-    return fail(SAREK_HIP_E_UNSUPPORTED, "triad_sum_static: device ordinal %d beyond %d", dev, kMaxDevices);
-  float *p = g_scratch_addr[dev].load(std::memory_order_acquire);
+    return fail(SAREK_HIP_E_UNSUPPORTED, "%s: device ordinal %d beyond %d", what, dev, kMaxDevices);
+  T *p = table[dev].load(std::memory_order_acquire);
   if (!p) {
-    SAREK_HIP_TRY(hipGetSymbolAddress(reinterpret_cast<void **>(&p), HIP_SYMBOL(scratch)));
-    if (!p) return fail(SAREK_HIP_E_UNSUPPORTED, "triad_sum_static: no device address for the partials array");
-    g_scratch_addr[dev].store(p, std::memory_order_release);
+    SAREK_HIP_TRY(hipGetSymbolAddress(reinterpret_cast<void **>(&p), symbol));
+    if (!p) return fail(SAREK_HIP_E_UNSUPPORTED, "%s: no device address for the library's own array", what);
+    table[dev].store(p, std::memory_order_release);
   }
   *out = p;
   return SAREK_HIP_OK;
+}
+
+int scratch_on_current_device(float **out) {
+  return address_on_current_device(g_scratch_addr, HIP_SYMBOL(scratch), "triad_sum_static", out);
+}
+
+// Folds shorter than this run as one workgroup; longer ones in two steps through fold_stage.
+constexpr int64_t kFoldTwoStepFrom = int64_t{1} << 17;
+
+int launch_fold(const float *partials, int64_t count, double *sum_out, hipStream_t st) {
+  if (count < kFoldTwoStepFrom) {
+    hipLaunchKernelGGL(fold_kernel, dim3(1), dim3(1024), 0, st, partials, count, sum_out);
+    return check_launch("fold kernel launch");
+  }
+  double *stage = nullptr;
+  int rc = address_on_current_device(g_fold_stage_addr, HIP_SYMBOL(fold_stage), "fold_partials", &stage);
+  if (rc != SAREK_HIP_OK) return rc;
+  const int64_t piece = ceil_div(ceil_div(count, kFoldGroups), 4) * 4;
+  hipLaunchKernelGGL(fold_pieces_kernel, dim3(kFoldGroups), dim3(1024), 0, st, partials, count, piece, stage);
+  rc = check_launch("fold pieces kernel launch");
+  if (rc != SAREK_HIP_OK) return rc;
+  hipLaunchKernelGGL(fold_stage_kernel, dim3(1), dim3(kFoldGroups), 0, st, stage, sum_out);
+  return check_launch("fold stage kernel launch");
 }
 }  // namespace
 }  // namespace sarek_hip
@@ -459,8 +550,25 @@ int sarek_hip_fold_partials_f64(const float *partials, int64_t count, double *su
                                 sarek_hip_stream stream) {
   if (count < 0 || !sum_out || (count > 0 && !partials))
     return fail(SAREK_HIP_E_INVALID_ARG, "fold_partials: bad arguments");
-  hipLaunchKernelGGL(fold_kernel, dim3(1), dim3(1024), 0, as_stream(stream), partials, count, sum_out);
-  return check_launch("fold kernel launch");
+  return launch_fold(partials, count, sum_out, as_stream(stream));
+}
+
+int sarek_hip_triad_block256_sum_f32(float *a, const float *b, const float *c, float s, int64_t n,
+                                     float *block_sums, sarek_hip_stream stream) {
+  if (n < 0) return fail(SAREK_HIP_E_INVALID_ARG, "triad_block256_sum: negative length %lld", (long long)n);
+  if (n == 0) return SAREK_HIP_OK;
+  if (!a || !b || !c || !block_sums) return fail(SAREK_HIP_E_INVALID_ARG, "triad_block256_sum: NULL vector");
+  if (!aligned16(a) || !aligned16(b) || !aligned16(c))
+    return fail(SAREK_HIP_E_INVALID_ARG, "triad_block256_sum: vectors must be 16-byte aligned");
+  const int64_t blocks64 = triad_blocks(n);
+  if (blocks64 > 0x7FFFFFFF) return fail(SAREK_HIP_E_INVALID_ARG, "triad_block256_sum: vector too long");
+  const dim3 grid(static_cast<unsigned>(blocks64));
+  hipStream_t st = as_stream(stream);
+  if (streams_from_hbm(n * 8))
+    hipLaunchKernelGGL((triad_kernel<SUM_BLOCK256, true>), grid, dim3(kBlock), 0, st, a, b, c, s, n, block_sums);
+  else
+    hipLaunchKernelGGL((triad_kernel<SUM_BLOCK256, false>), grid, dim3(kBlock), 0, st, a, b, c, s, n, block_sums);
+  return check_launch("triad + block-256 sum kernel launch");
 }
 
 static int launch_block256(const float *x, const float *y, float *out, int64_t n, bool dot,

@@ -215,6 +215,12 @@ int expand_args(const sarek_hip_varg *args, int n, int dev, bool inject_lengths,
         a.buffer = it->second;
         a.length = v->length;
         out.push_back(a);
+        // the length parameter of a kernel is an int32 (sarek-cuda/Sarek_ir_cuda.ml:668-672); a longer
+        // vector would wrap round where the reference passes Int32.of_int of it
+        if (inject_lengths && v->length > 0x7FFFFFFF)
+          return fail(SAREK_HIP_E_INVALID_ARG,
+                      "argument %d: vector of %lld elements, a kernel's length parameter holds at most 2147483647",
+                      i, static_cast<long long>(v->length));
         if (inject_lengths) {
           sarek_hip_arg l;
           std::memset(&l, 0, sizeof(l));
@@ -603,6 +609,60 @@ int sarek_hip_execute_run_vectors(const char *ir_text, const int block[3], const
                             shared_mem_bytes, rs.data(), static_cast<int>(rs.size()));
   if (st != SAREK_HIP_OK) return st;
   mark_stale(args, n_args, dev);
+  return SAREK_HIP_OK;
+}
+
+int sarek_hip_execute_run_pipeline(const sarek_hip_pipeline_stage *stages, int n_stages, int *launches) {
+  if (n_stages < 0 || (n_stages > 0 && !stages)) return fail(SAREK_HIP_E_INVALID_ARG, "run_pipeline: NULL or negative argument");
+  if (launches) *launches = 0;
+  for (int i = 0; i < n_stages; ++i) {
+    const sarek_hip_pipeline_stage &s = stages[i];
+    if (!s.ir_text || s.n_args < 0 || (s.n_args > 0 && !s.args))
+      return fail(SAREK_HIP_E_INVALID_ARG, "run_pipeline: stage %d: NULL or negative argument", i);
+  }
+  int dev = 0;
+  int st = current_device(&dev);
+  if (st != SAREK_HIP_OK) return st;
+  std::string path;
+  for (int i = 0; i < n_stages; ++i) {
+    const sarek_hip_pipeline_stage &s0 = stages[i];
+    if (i + 1 < n_stages) {
+      // two stages one hand kernel can serve: what Execute.run_vectors does for each, with one launch between
+      const sarek_hip_pipeline_stage &s1 = stages[i + 1];
+      std::shared_ptr<const Lowered> k0, k1;
+      try {
+        if ((st = lower(s0.ir_text, s0.block, k0)) != SAREK_HIP_OK) return st;
+        if ((st = lower(s1.ir_text, s1.block, k1)) != SAREK_HIP_OK) return st;
+      } catch (const std::exception &e) {
+        return fail(SAREK_HIP_E_PARSE, "run_pipeline: %s", e.what());
+      }
+      if (std::strncmp(k0->source.c_str(), kSpecialiseMarker, std::strlen(kSpecialiseMarker)) == 0 &&
+          std::strncmp(k1->source.c_str(), kSpecialiseMarker, std::strlen(kSpecialiseMarker)) == 0) {
+        if ((st = transfer_args(s0.args, s0.n_args, dev)) != SAREK_HIP_OK) return st;
+        if ((st = transfer_args(s1.args, s1.n_args, dev)) != SAREK_HIP_OK) return st;
+        std::vector<sarek_hip_arg> rs0, rs1;
+        if ((st = expand_args(s0.args, s0.n_args, dev, true, rs0)) != SAREK_HIP_OK) return st;
+        if ((st = expand_args(s1.args, s1.n_args, dev, true, rs1)) != SAREK_HIP_OK) return st;
+        int rc = SAREK_HIP_OK;
+        if (run_specialised_pair(k0->source.c_str(), s0.block, s0.grid, rs0.data(), static_cast<int>(rs0.size()),
+                                 k1->source.c_str(), s1.block, s1.grid, rs1.data(), static_cast<int>(rs1.size()),
+                                 &rc)) {
+          if (rc != SAREK_HIP_OK) return rc;
+          mark_stale(s0.args, s0.n_args, dev);
+          mark_stale(s1.args, s1.n_args, dev);
+          if (launches) ++*launches;
+          path += (path.empty() ? "" : ";") + std::string(sarek_hip_last_run_path());
+          ++i;
+          continue;
+        }
+      }
+    }
+    st = sarek_hip_execute_run_vectors(s0.ir_text, s0.block, s0.grid, s0.shared_mem_bytes, s0.args, s0.n_args);
+    if (st != SAREK_HIP_OK) return st;
+    if (launches) ++*launches;
+    path += (path.empty() ? "" : ";") + std::string(sarek_hip_last_run_path());
+  }
+  set_last_run_path(path.empty() ? "none" : path);
   return SAREK_HIP_OK;
 }
 

@@ -65,6 +65,12 @@ class VArg(C.Structure):
                 ("f32", C.c_float), ("f64", C.c_double)]
 
 
+class PipelineStage(C.Structure):
+    """sarek_hip_pipeline_stage: one Execute.run_vectors call of a kernel sequence."""
+    _fields_ = [("ir_text", C.c_char_p), ("block", C.c_int * 3), ("grid", C.c_int * 3),
+                ("shared_mem_bytes", C.c_int), ("args", C.POINTER(VArg)), ("n_args", C.c_int)]
+
+
 # Every symbol include/sarek_hip.h declares: (restype, argtypes).
 SYMBOLS = {
     "sarek_hip_abi_version": (_i, []),
@@ -180,6 +186,10 @@ SYMBOLS = {
     "sarek_hip_execute_run_vectors": (_i, [C.c_char_p, _int3, _int3, _i, C.POINTER(VArg), _i]),
     "sarek_hip_execute_run_source": (_i, [C.c_char_p, _i, C.c_char_p, _int3, _int3, _i, _i, C.POINTER(VArg), _i]),
     "sarek_hip_execute_sync_vectors_to_cpu": (_i, [C.POINTER(VArg), _i]),
+    "sarek_hip_execute_run_pipeline": (_i, [C.POINTER(PipelineStage), _i, C.POINTER(_i)]),
+    "sarek_hip_library_kernel_source": (_i, [C.c_char_p, C.c_char_p, _sz, C.POINTER(_sz), C.c_char_p, _sz]),
+    "sarek_hip_library_kernel_list": (_i, [C.c_char_p, _sz, C.POINTER(_sz)]),
+    "sarek_hip_triad_block256_sum_f32": (_i, [_vp, _vp, _vp, _f, _i64, _vp, _vp]),
     "sarek_hip_backend_name": (C.c_char_p, []),
     "sarek_hip_backend_version": (_i, [C.POINTER(_i), C.POINTER(_i), C.POINTER(_i)]),
     "sarek_hip_execution_model": (_i, []),
@@ -399,6 +409,37 @@ def triad_sum(b, c, s, out=None, workspace=None):
     check(lib.sarek_hip_triad_sum_f32(_ptr(a), _ptr(b), _ptr(c), float(s), b.numel(),
                                       _ptr(partials), partials.numel(), _ptr(total), _stream()))
     return a, total
+
+
+def triad_block256_sum(b, c, s, out=None):
+    """a = b + c*s and the block-256 sums of a in one pass.  Returns (a, block_sums)."""
+    torch = _torch()
+    _need(b, torch.float32, "b")
+    _need(c, torch.float32, "c")
+    a = torch.empty_like(b) if out is None else out
+    sums = torch.empty((b.numel() + 255) // 256, dtype=torch.float32, device=b.device)
+    check(lib.sarek_hip_triad_block256_sum_f32(_ptr(a), _ptr(b), _ptr(c), float(s), b.numel(), _ptr(sums), _stream()))
+    return a, sums
+
+
+def library_kernel(name):
+    """(source text, kernel_name) of a library kernel, for Execute.run_source."""
+    need = C.c_size_t(0)
+    entry = C.create_string_buffer(128)
+    rc = lib.sarek_hip_library_kernel_source(name.encode(), None, 0, C.byref(need), None, 0)
+    if rc != E_BUFFER_TOO_SMALL:
+        check(rc)
+    buf = C.create_string_buffer(need.value)
+    check(lib.sarek_hip_library_kernel_source(name.encode(), buf, need.value, None, entry, 128))
+    return buf.value.decode(), entry.value.decode()
+
+
+def library_kernel_names():
+    need = C.c_size_t(0)
+    lib.sarek_hip_library_kernel_list(None, 0, C.byref(need))
+    buf = C.create_string_buffer(need.value)
+    check(lib.sarek_hip_library_kernel_list(buf, need.value, None))
+    return buf.value.decode().split()
 
 
 def reduce_sum_block256(x):

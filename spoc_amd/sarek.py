@@ -498,6 +498,30 @@ class Execute:
         return hip.lib.sarek_hip_last_run_path().decode()
 
     @staticmethod
+    def run_pipeline(stages):
+        """A kernel list run in order: stages = [(ir, args, block, grid)] or [(ir, args, block, grid, shared_mem)],
+        each what one run_vectors call takes.  Returns (code paths, device launches made); consecutive stages
+        that one hand kernel serves count as one launch."""
+        arr = (hip.PipelineStage * max(len(stages), 1))()
+        keep = []
+        for st, stage in zip(arr, stages):
+            ir, args, block, grid = stage[:4]
+            a, n = Execute._args(args)
+            text = ir.encode()
+            keep.append((a, text))
+            st.ir_text, st.block, st.grid = text, (C.c_int * 3)(*block), (C.c_int * 3)(*grid)
+            st.shared_mem_bytes = stage[4] if len(stage) > 4 else 0
+            st.args, st.n_args = a, n
+        launches = C.c_int(0)
+        hip.check(hip.lib.sarek_hip_execute_run_pipeline(arr, len(stages), C.byref(launches)))
+        return hip.lib.sarek_hip_last_run_path().decode(), launches.value
+
+    @staticmethod
+    def library_kernel(name):
+        """(source, kernel_name) of one of the backend's library kernels, to hand to run_source."""
+        return hip.library_kernel(name)
+
+    @staticmethod
     def run_source(source, kernel_name, block, grid, args, lang=hip.LANG_HIP, shared_mem=0, inject_lengths=True):
         a, n = Execute._args(args)
         hip.check(hip.lib.sarek_hip_execute_run_source(source.encode(), lang, kernel_name.encode(),

@@ -52,7 +52,7 @@ def test_host_code_is_clean_under_asan_and_ubsan(tmp_path):
     sources = [os.path.join(HERE, "host_sanitizers", f) for f in ("driver.cpp", "kernel_stubs.cpp")]
     sources += [os.path.join(CSRC, f) for f in (
         "status.cpp", "backend_info.cpp", "tunables.cpp", "runtime.cpp", "transfer.cpp", "vector.cpp",
-        "code_cache.cpp", "plugin.cpp", "generate.cpp", "fusion_abi.cpp", "host/ir_text.cpp", "host/ir_hip.cpp",
+        "code_cache.cpp", "plugin.cpp", "library_kernels.cpp", "generate.cpp", "fusion_abi.cpp", "host/ir_text.cpp", "host/ir_hip.cpp",
         "host/specialise.cpp", "host/fusion.cpp")]
     exe = str(tmp_path / "host_asan")
     flags = ["-std=c++20", "-O1", "-g", "-fsanitize=address,undefined", "-fno-sanitize-recover=undefined",
