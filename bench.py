@@ -9,10 +9,16 @@ the bf16-in / f32-accumulate 8192^3 GEMM; the other configurations of the hot pa
 (fused triad+sum n=2^28, f32 GEMM 8192^3 and 1024^3, fp16 fused-epilogue GEMM) are
 measured the same way and reported under "also", each with its own roofline object.
 
-Timing mirrors the reference's benches (warmup, then timed iterations with the device
-synchronised; benchmarks/bench_stream_triad.ml:76-116) with one difference: the K timed
-steps are bracketed by one synchronise on each side, and the kernel time used for the
-roofline comes from HIP events recorded on the launch stream.
+Every workload goes through the plugin boundary the way a Sarek program reaches it: the
+reference benches' own kernels from their IR through Execute.run_vectors / run_pipeline, the
+16-bit GEMMs and the fused epilogue as library kernel texts through Execute.run_source; the
+record's "served_by" names the hand-written kernel that took the launch.
+
+Timing mirrors the reference's benches (warmup, then timed iterations, each launched and
+waited for; benchmarks/bench_stream_triad.ml:76-116): ms_per_step is the wall time of the K
+timed iterations over K, ms_per_step_stats their min / median / avg / max.  The kernel time
+used for the roofline comes from HIP events recorded round the dominant launch on the launch
+stream; gpu_ms_per_step_back_to_back is the same step launched K times with one wait at the end.
 """
 import argparse
 import ctypes as C
@@ -47,7 +53,7 @@ def parse():
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--workload", default="gemm_bf16_8192",
-                    choices=["gemm_bf16_8192", "triad_sum_2p28", "gemm_f32_8192", "gemm_f32_1024",
+                    choices=["gemm_bf16_8192", "gemm_f16_8192", "triad_sum_2p28", "gemm_f32_8192", "gemm_f32_1024",
                              "gemm_f16_epilogue", "copy_1gib", "vendor_gemm_bf16_8192", "histogram_2p28",
                              "radix_scatter_5e7"])
     ap.add_argument("--no-also", action="store_true", help="measure only the headline workload")
@@ -75,8 +81,41 @@ class Events:
         return float(ms.value)
 
 
+def device_vector(sarek, hip, torch, tensor, kind=None, elem_size=None):
+    """A Vector whose device buffer holds `tensor` (data made on the device by torch): created, given
+    its buffer by Transfer.to_device, then filled device to device.  Location Both, as after an
+    upload; the launches below never read the host block."""
+    V = sarek.Vector
+    v = V.create_custom(elem_size, tensor.numel()) if elem_size else V.create(kind, tensor.numel())
+    sarek.Transfer.to_device(v)
+    hip.check(hip.lib.sarek_hip_memcpy_dtod(v.device_ptr, tensor.data_ptr(), tensor.numel() * tensor.element_size()))
+    return v
+
+
+class Launch:
+    """One prepared call through the plugin boundary: the ctypes argument block is built once."""
+
+    def __init__(self, hip, fn, *args):
+        self.hip, self.fn, self.args = hip, fn, args
+
+    def __call__(self):
+        rc = self.fn(*self.args)
+        if rc != 0:
+            self.hip.check(rc)
+
+
+def dims(*d):
+    return (C.c_int * 3)(*d)
+
+
 def make_workload(name, torch, hip):
-    """Returns (step_fn, info) with inputs resident on the GPU."""
+    """Returns (main, tail, info, keep): main() launches the workload's dominant kernel through the plugin
+    route named in info["route"], tail() (or None) the rest of the step; inputs are resident on the GPU."""
+    from spoc_amd import reference_kernels as rk
+    from spoc_amd import sarek
+    E, V = sarek.Execute, sarek.Vector
+    sarek.Device.init()
+    lib = hip.lib
     g = torch.Generator(device="cuda")
     if name == "copy_1gib":
         # plain device copy of known size: calibrates the FETCH_SIZE / WRITE_SIZE counters
@@ -85,48 +124,86 @@ def make_workload(name, torch, hip):
         dst = torch.empty_like(src)
         info = dict(metric="plain copy GB/s (counter calibration)", unit="GB/s", dtype="f32",
                     work=8.0 * n, work_unit=1e9, bound="hbm", peak=PEAK_HBM_GBS,
-                    kernel="at::native copy kernel",
+                    kernel="at::native copy kernel", route="torch",
                     config={"workload": "dst.copy_(src), 1 GiB read + 1 GiB written", "n": n})
-        return (lambda: dst.copy_(src)), info
+        return (lambda: dst.copy_(src)), None, info, None
     if name == "triad_sum_2p28":
         n = 1 << 28
         g.manual_seed(0xB)
         b = torch.rand(n, device="cuda", generator=g)
+        vb = device_vector(sarek, hip, torch, b, V.float32)
         g.manual_seed(0xC)
-        c = torch.rand(n, device="cuda", generator=g)
-        a = torch.empty_like(b)
-        ws = hip.triad_sum_workspace(n)
+        b.uniform_(0, 1, generator=g)
+        vc = device_vector(sarek, hip, torch, b, V.float32)
+        del b
+        va, vout = V.create(V.float32, n), V.create(V.float32, n // 256)
+        sarek.Transfer.to_device(va)
+        sarek.Transfer.to_device(vout)
+        total = torch.zeros(1, dtype=torch.float64, device="cuda")
+        a0, n0 = E._args([E.Vec(va), E.Vec(vb), E.Vec(vc), E.Float32(3.0), E.Int32(n)])
+        a1, n1 = E._args([E.Vec(va), E.Vec(vout), E.Int32(n)])
+        ir0, ir1 = rk.stream_triad().encode(), rk.tree(False).encode()
+        stages = (hip.PipelineStage * 2)()
+        stages[0].ir_text, stages[0].block, stages[0].grid, stages[0].args, stages[0].n_args = \
+            ir0, dims(256, 1, 1), dims(n // 256, 1, 1), a0, n0
+        stages[1].ir_text, stages[1].block, stages[1].grid, stages[1].args, stages[1].n_args = \
+            ir1, dims(256, 1, 1), dims(n // 256, 1, 1), a1, n1
+        main = Launch(hip, lib.sarek_hip_execute_run_pipeline, stages, 2, None)
+        tail = Launch(hip, lib.sarek_hip_fold_partials_f64, vout.device_ptr, n // 256, total.data_ptr(), None)
         info = dict(metric="fused triad+sum GB/s", unit="GB/s", dtype="f32",
                     work=12.0 * n, work_unit=1e9, bound="hbm", peak=PEAK_HBM_GBS,
-                    kernel="triad_kernel<true, true> (+ fold_kernel, 1 % of the time)",
+                    kernel="triad_kernel<SUM_BLOCK256, nt> (then the fold of the 2^20 block sums: fold_pieces_kernel, "
+                           "fold_stage_kernel)",
+                    route="Execute.run_pipeline [stream_triad IR; block-256 reduction IR], then sarek_hip_fold_partials_f64",
                     config={"workload": "fused stream triad + sum, a=b+3c, sum(a)", "n": n,
                             "algorithmic_bytes": 12 * n})
-        return (lambda: hip.triad_sum(b, c, 3.0, out=a, workspace=ws)), info
+        return main, tail, info, (va, vb, vc, vout, total, a0, a1, ir0, ir1, stages)
     if name in ("gemm_f32_8192", "gemm_f32_1024"):
         s = 8192 if name.endswith("8192") else 1024
         g.manual_seed(0xA11CE)
-        a = torch.rand(s, s, device="cuda", generator=g) * 2 - 1
+        t = torch.rand(s, s, device="cuda", generator=g) * 2 - 1
+        va = device_vector(sarek, hip, torch, t, V.float32)
         g.manual_seed(0xB0B)
-        b = torch.rand(s, s, device="cuda", generator=g) * 2 - 1
-        c = torch.empty(s, s, device="cuda")
+        t = torch.rand(s, s, device="cuda", generator=g) * 2 - 1
+        vb = device_vector(sarek, hip, torch, t, V.float32)
+        del t
+        vc = V.create(V.float32, s * s)
+        sarek.Transfer.to_device(vc)
+        a, n = E._args([E.Vec(va), E.Vec(vb), E.Vec(vc), E.Int32(s), E.Int32(s), E.Int32(s)])
+        ir = rk.matrix_mul_tiled().encode()
+        main = Launch(hip, lib.sarek_hip_execute_run_vectors, ir, dims(16, 16, 1), dims(s // 16, s // 16, 1), 2048, a, n)
         info = dict(metric=f"f32 GEMM {s}^3 TFLOP/s", unit="TFLOP/s", dtype="f32",
                     work=2.0 * s ** 3, work_unit=1e12, bound="mfma", peak=PEAK_MFMA_TFLOPS["f32"],
-                    kernel="gemm_f32_dma_kernel",
-                    config={"workload": f"f32 GEMM C=A.B row-major, U[-1,1)", "m": s, "n": s, "k": s})
-        return (lambda: hip.gemm_f32(a, b, out=c)), info
-    if name == "gemm_bf16_8192":
+                    kernel="gemm_f32_dma_kernel", route="Execute.run_vectors, matrix_mul_tiled IR (bench_matrix_mul_tiled.ml:55-95)",
+                    config={"workload": "f32 GEMM C=A.B row-major, U[-1,1)", "m": s, "n": s, "k": s})
+        return main, None, info, (va, vb, vc, a, ir)
+    if name in ("gemm_bf16_8192", "gemm_f16_8192"):
         s = 8192
+        bf16 = name == "gemm_bf16_8192"
+        dt = torch.bfloat16 if bf16 else torch.float16
         g.manual_seed(0xA4)
-        a = (torch.randn(s, s, device="cuda", generator=g) * 0.02).bfloat16()
+        t = (torch.randn(s, s, device="cuda", generator=g) * 0.02).to(dt)
+        va = device_vector(sarek, hip, torch, t, elem_size=2)
         g.manual_seed(0xB4)
-        b = (torch.randn(s, s, device="cuda", generator=g) * 0.02).bfloat16()
-        c = torch.empty(s, s, device="cuda")
-        info = dict(metric="GEMM TFLOP/s at 8192^3 (bf16-in, f32-accumulate)", unit="TFLOP/s",
-                    dtype="bf16", work=2.0 * s ** 3, work_unit=1e12, bound="mfma",
-                    peak=PEAK_MFMA_TFLOPS["bf16"], kernel="gemm16_dma_kernel<bf16, store, 64, 32, 2, 4, 2>",
-                    config={"workload": "bf16-in f32-acc GEMM C=A.B row-major, N(0,0.02)",
+        t = (torch.randn(s, s, device="cuda", generator=g) * 0.02).to(dt)
+        vb = device_vector(sarek, hip, torch, t, elem_size=2)
+        del t
+        vc = V.create(V.float32, s * s)
+        sarek.Transfer.to_device(vc)
+        lib_name = "gemm_bf16" if bf16 else "gemm_f16"
+        src, entry = hip.library_kernel(lib_name)
+        a, n = E._args([E.Vec(va), E.Vec(vb), E.Vec(vc), E.Int32(s), E.Int32(s), E.Int32(s)])
+        src_b, entry_b = src.encode(), entry.encode()
+        main = Launch(hip, lib.sarek_hip_execute_run_source, src_b, hip.LANG_HIP, entry_b, dims(16, 16, 1),
+                      dims(s // 16, s // 16, 1), 0, 1, a, n)
+        tn = "bf16" if bf16 else "f16"
+        info = dict(metric=f"GEMM TFLOP/s at 8192^3 ({tn}-in, f32-accumulate)", unit="TFLOP/s",
+                    dtype=tn, work=2.0 * s ** 3, work_unit=1e12, bound="mfma",
+                    peak=PEAK_MFMA_TFLOPS[tn], kernel=f"gemm16_dma_kernel<{tn}, store, 64, 32, 2, 4, 2>",
+                    route=f"Execute.run_source ~lang:HIP_Source, library kernel text '{lib_name}'",
+                    config={"workload": f"{tn}-in f32-acc GEMM C=A.B row-major, N(0,0.02)",
                             "m": s, "n": s, "k": s})
-        return (lambda: hip.gemm_bf16(a, b, out=c)), info
+        return main, None, info, (va, vb, vc, a, src_b, entry_b)
     if name == "vendor_gemm_bf16_8192":
         # the vendor library's GEMM (torch.matmul -> hipBLASLt) on the headline inputs, for
         # side-by-side profiles; it writes bf16 C where the kernel here writes f32
@@ -138,20 +215,27 @@ def make_workload(name, torch, hip):
         c = torch.empty(s, s, device="cuda", dtype=torch.bfloat16)
         info = dict(metric="vendor library GEMM TFLOP/s at 8192^3 (bf16 in, bf16 out)", unit="TFLOP/s",
                     dtype="bf16", work=2.0 * s ** 3, work_unit=1e12, bound="mfma",
-                    peak=PEAK_MFMA_TFLOPS["bf16"], kernel="hipBLASLt (torch.matmul)",
+                    peak=PEAK_MFMA_TFLOPS["bf16"], kernel="hipBLASLt (torch.matmul)", route="torch.matmul",
                     config={"workload": "torch.matmul bf16, N(0,0.02)", "m": s, "n": s, "k": s})
-        return (lambda: torch.matmul(a, b, out=c)), info
+        return (lambda: torch.matmul(a, b, out=c)), None, info, None
     if name == "histogram_2p28":
         n = 1 << 28
         g.manual_seed(0xC4)
-        keys = torch.randint(0, 256, (n,), device="cuda", generator=g, dtype=torch.int32)
-        hist = torch.zeros(256, device="cuda", dtype=torch.int32)
+        t = torch.randint(0, 256, (n,), device="cuda", generator=g, dtype=torch.int32)
+        vk = device_vector(sarek, hip, torch, t, V.int32)
+        del t
+        vh = V.create(V.int32, 256)
+        vh.host[:] = 0
+        sarek.Transfer.to_device(vh)
+        a, na = E._args([E.Vec(vk), E.Vec(vh), E.Int32(n), E.Int32(256)])
+        ir = rk.histogram().encode()
+        main = Launch(hip, lib.sarek_hip_execute_run_vectors, ir, dims(256, 1, 1), dims(n // 256, 1, 1), 0, a, na)
         info = dict(metric="256-bin histogram of int32 keys GB/s", unit="GB/s", dtype="i32",
                     work=4.0 * n, work_unit=1e9, bound="hbm", peak=PEAK_HBM_GBS,
-                    kernel="histogram_kernel<ModPow2Bin>",
+                    kernel="histogram_kernel<ModPow2Bin>", route="Execute.run_vectors, histogram IR (bench_histogram.ml:54-84)",
                     config={"workload": "histogram[key mod 256] += 1, uniform keys", "n": n,
                             "algorithmic_bytes": 4 * n})
-        return (lambda: hip.histogram(keys, hist, 256)), info
+        return main, None, info, (vk, vh, a, ir)
     if name == "radix_scatter_5e7":
         n = 50_000_000
         g.manual_seed(0xC5)
@@ -159,79 +243,124 @@ def make_workload(name, torch, hip):
         hist = torch.zeros(256, device="cuda", dtype=torch.int32)
         hip.radix_histogram(keys, hist, 0, 255)
         starts = (torch.cumsum(hist, 0) - hist).to(torch.int32)
-        out = torch.empty(n, device="cuda", dtype=torch.int32)
-        counters = torch.empty(256, device="cuda", dtype=torch.int32)
+        vk = device_vector(sarek, hip, torch, keys, V.int32)
+        del keys
+        vo, vcnt = V.create(V.int32, n), V.create(V.int32, 256)
+        sarek.Transfer.to_device(vo)
+        sarek.Transfer.to_device(vcnt)
+        a, na = E._args([E.Vec(vk), E.Vec(vo), E.Vec(vcnt), E.Int32(n), E.Int32(0), E.Int32(255)])
+        ir = rk.radix_sort_scatter().encode()
+        blocks = (n + 255) // 256
+        reset = Launch(hip, lib.sarek_hip_memcpy_dtod, vcnt.device_ptr, starts.data_ptr(), 1024)
+        scatter = Launch(hip, lib.sarek_hip_execute_run_vectors, ir, dims(256, 1, 1), dims(blocks, 1, 1), 0, a, na)
+
+        def main():
+            reset()
+            scatter()
         info = dict(metric="radix-sort scatter pass (8-bit digit) GB/s", unit="GB/s", dtype="i32",
                     work=8.0 * n, work_unit=1e9, bound="hbm", peak=PEAK_HBM_GBS,
-                    kernel="radix_scatter_kernel<1024, 16> (+ a 1 KiB copy that resets the counters)",
+                    kernel="radix_scatter_kernel (+ a 1 KiB copy that resets the counters)",
+                    route="Execute.run_vectors, radix-sort scatter IR (bench_radix_sort.ml:120-137)",
                     config={"workload": "out[counters[key & 255]++] = key, random keys below 100000", "n": n,
                             "algorithmic_bytes": 8 * n})
-
-        def step():
-            counters.copy_(starts)
-            hip.radix_scatter(keys, out, counters, 0, 255)
-        return step, info
+        return main, None, info, (vk, vo, vcnt, starts, a, ir)
     if name == "gemm_f16_epilogue":
         m, n, k = 4095, 11008, 4096
         g.manual_seed(0xA5)
-        a = (torch.randn(m, k, device="cuda", generator=g) * 0.02).half()
+        t = (torch.randn(m, k, device="cuda", generator=g) * 0.02).half()
+        va = device_vector(sarek, hip, torch, t, elem_size=2)
         g.manual_seed(0xB5)
-        b = (torch.randn(k, n, device="cuda", generator=g) * 0.02).half()
-        bias = torch.rand(n, device="cuda", generator=g) * 0.2 - 0.1
-        y = torch.empty(m, n, device="cuda")
-        rs = torch.empty(m, device="cuda")
+        t = (torch.randn(k, n, device="cuda", generator=g) * 0.02).half()
+        vb = device_vector(sarek, hip, torch, t, elem_size=2)
+        t = torch.rand(n, device="cuda", generator=g) * 0.2 - 0.1
+        vbias = device_vector(sarek, hip, torch, t, V.float32)
+        del t
+        vy, vrs = V.create(V.float32, m * n), V.create(V.float32, m)
+        sarek.Transfer.to_device(vy)
+        sarek.Transfer.to_device(vrs)
+        src, entry = hip.library_kernel("gemm_f16_bias_relu_rowsum")
+        a, na = E._args([E.Vec(va), E.Vec(vb), E.Vec(vbias), E.Vec(vy), E.Vec(vrs), E.Int32(m), E.Int32(n), E.Int32(k)])
+        src_b, entry_b = src.encode(), entry.encode()
+        main = Launch(hip, lib.sarek_hip_execute_run_source, src_b, hip.LANG_HIP, entry_b, dims(256, 1, 1),
+                      dims(1024, 1, 1), 0, 1, a, na)
         info = dict(metric="fp16 GEMM + bias + ReLU + row-sum TFLOP/s", unit="TFLOP/s", dtype="f16",
                     work=2.0 * m * n * k, work_unit=1e12, bound="mfma",
                     peak=PEAK_MFMA_TFLOPS["f16"], kernel="gemm16_dma_kernel<f16, bias_relu_rowsum, 64, 32, 2, 4, 2>",
+                    route="Execute.run_source ~lang:HIP_Source, library kernel text 'gemm_f16_bias_relu_rowsum'",
                     config={"workload": "fp16-in f32-acc Y=relu(A.B+bias), rowsum(Y)",
                             "m": m, "n": n, "k": k})
-        return (lambda: hip.gemm_f16_bias_relu_rowsum(a, b, bias, out=y, rowsum=rs)), info
+        return main, None, info, (va, vb, vbias, vy, vrs, a, src_b, entry_b)
     raise ValueError(name)
 
 
+def stats(xs):
+    xs = sorted(xs)
+    return {"min": round(xs[0], 5), "median": round(xs[len(xs) // 2], 5), "avg": round(sum(xs) / len(xs), 5),
+            "max": round(xs[-1], 5)}
+
+
 def measure(name, torch, hip, steps, warmup):
-    step, info = make_workload(name, torch, hip)
+    """Warmup, then `steps` timed iterations, each launched and waited for, as the reference's benches do
+    (benchmarks/bench_stream_triad.ml:98-115: time around launch + device synchronise, median reported).
+    The dominant kernel's duration comes from HIP events recorded round its launch on the launch stream."""
+    main, tail, info, keep = make_workload(name, torch, hip)
     stream = C.c_void_p(torch.cuda.current_stream().cuda_stream)
     ev = Events(hip, stream)
+    sync = hip.lib.sarek_hip_device_synchronize
     for _ in range(warmup):
-        step()
-    torch.cuda.synchronize()
+        main()
+        if tail:
+            tail()
+    sync()
+    path = None
+    if info["route"].startswith("Execute"):
+        main()                                   # once more, alone, to read which code path served it
+        path = hip.lib.sarek_hip_last_run_path().decode()
+        sync()
+    walls, kerns = [], []
     t0 = time.perf_counter()
+    for _ in range(steps):
+        w0 = time.perf_counter()
+        ev.start()
+        main()
+        hip.check(hip.lib.sarek_hip_event_record(ev.e1, stream))
+        if tail:
+            tail()
+        sync()
+        walls.append((time.perf_counter() - w0) * 1e3)
+        ms = C.c_float(0)
+        hip.check(hip.lib.sarek_hip_event_elapsed_ms(ev.e0, ev.e1, C.byref(ms)))
+        kerns.append(float(ms.value))
+    sync()
+    wall_ms = (time.perf_counter() - t0) * 1e3
+    ms_per_step = wall_ms / steps
+    # second figure: the same launches back to back, one wait at the end (hotter: under the package power
+    # limit the 16-bit GEMMs run slower this way)
     ev.start()
     for _ in range(steps):
-        step()
-    gpu_ms = ev.stop_ms()
-    torch.cuda.synchronize()
-    wall_ms = (time.perf_counter() - t0) * 1e3
-    # roofline: average launch duration from the HIP events around the timed region (the
-    # launches run back to back there, as in a rocprofv3 kernel trace of this command);
-    # for reference also the median of launches timed one at a time with a sync between
-    # them, which run cooler and, under a power cap, faster
-    kernel_ms = gpu_ms / steps
-    per = []
-    for _ in range(min(steps, 20)):
-        ev.start()
-        step()
-        per.append(ev.stop_ms())
-    per.sort()
-    isolated_ms = per[len(per) // 2]
-    ms_per_step = wall_ms / steps
+        main()
+        if tail:
+            tail()
+    back_to_back_ms = ev.stop_ms() / steps
+    kernel_ms = sum(kerns) / len(kerns)
     value = info["work"] / (ms_per_step * 1e-3) / info["work_unit"]
     achieved = info["work"] / (kernel_ms * 1e-3) / info["work_unit"]
     res = {
         "metric": info["metric"], "value": round(value, 2), "unit": info["unit"],
-        "ms_per_step": round(ms_per_step, 5), "gpu_ms_per_step_events": round(gpu_ms / steps, 5),
-        "dtype": info["dtype"], "config": info["config"],
+        "ms_per_step": round(ms_per_step, 5), "ms_per_step_stats": stats(walls),
+        "value_at_median": round(info["work"] / (stats(walls)["median"] * 1e-3) / info["work_unit"], 2),
+        "gpu_ms_per_step_back_to_back": round(back_to_back_ms, 5),
+        "dtype": info["dtype"], "config": info["config"], "route": info["route"], "served_by": path,
         "roofline": {"bound": info["bound"], "achieved": round(achieved, 2), "peak": info["peak"],
                      "unit": "GB/s" if info["bound"] == "hbm" else "TFLOP/s",
                      "frac": round(achieved / info["peak"], 4),
                      "traffic": MEASURED_TRAFFIC_BYTES.get(name),
-                     "kernel": info["kernel"], "kernel_ms": round(kernel_ms, 5),
-                     "isolated_launch_ms": round(isolated_ms, 5)},
+                     "kernel": info["kernel"], "kernel_ms": round(kernel_ms, 5), "kernel_ms_stats": stats(kerns),
+                     "frac_back_to_back": round(info["work"] / (back_to_back_ms * 1e-3) / info["work_unit"] / info["peak"], 4)},
     }
     if name == "triad_sum_2p28":
         res["roofline"]["probe_kernels_GBs"] = hbm_ceiling(torch, hip)
-    if info["bound"] == "mfma":
+    if info["bound"] == "mfma" and info["route"].startswith("Execute"):
         # shader clock the kernel actually ran at (in-kernel cycle counter against the
         # constant-rate wall clock), and the rate of those very launches against the peak
         # scaled to that clock
@@ -240,7 +369,7 @@ def measure(name, torch, hip, steps, warmup):
             for _ in range(min(steps, 10)):
                 probe.buf.zero_()
                 ev.start()
-                step()
+                main()
                 ms = ev.stop_ms()
                 mhz = probe.mhz()
                 if mhz:
@@ -251,6 +380,7 @@ def measure(name, torch, hip, steps, warmup):
             res["roofline"]["shader_clock_mhz"] = round(mhz, 1)
             res["roofline"]["frac_of_peak_at_that_clock"] = round(
                 info["work"] / (ms * 1e-3) / info["work_unit"] / (info["peak"] * mhz / NOMINAL_CLOCK_MHZ), 4)
+    del keep
     return res
 
 
@@ -313,8 +443,8 @@ def cpu_baseline(name):
     import numpy as np
 
     import oracle
-    cores = os.cpu_count() or 1
-    cores = min(cores, 16) if "GRAFT_REPO_ROOT" in os.environ else cores
+    # threads: the cores this process may run on, at most 16 (the share of a one-GPU box)
+    cores = min(len(os.sched_getaffinity(0)) or 1, 16)
     rng = np.random.default_rng(0)
     if name == "triad_sum_2p28":
         n = 1 << 28
@@ -337,6 +467,10 @@ def cpu_baseline(name):
         rows, n, k = 4096, 8192, 8192
     a = rng.normal(0, 0.02, (rows, k)).astype(np.float32)
     b = rng.normal(0, 0.02, (k, n)).astype(np.float32)
+    if name == "gemm_bf16_8192":
+        a, b = oracle.round_bf16(a), oracle.round_bf16(b)
+    elif name == "gemm_f16_epilogue":
+        a, b = oracle.round_f16(a), oracle.round_f16(b)
     idx = np.arange(rows, dtype=np.int32)
     oracle.gemm_rows(a[:8], b, idx[:8], threads=cores)
     t0 = time.perf_counter()
@@ -366,7 +500,9 @@ def main():
         "steps": args.steps, "warmup": args.warmup, "ms_per_step": head["ms_per_step"],
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": head["dtype"],
         "data": "synthetic", "config": head["config"], "roofline": head["roofline"],
-        "gpu_ms_per_step_events": head["gpu_ms_per_step_events"],
+        "route": head["route"], "served_by": head["served_by"], "ms_per_step_stats": head["ms_per_step_stats"],
+        "value_at_median": head["value_at_median"],
+        "gpu_ms_per_step_back_to_back": head["gpu_ms_per_step_back_to_back"],
     }
     if not args.no_cpu_baseline and args.workload not in ("copy_1gib", "vendor_gemm_bf16_8192"):
         out["cpu_baseline"] = cpu_baseline(args.workload)
