@@ -58,6 +58,10 @@ def parse():
                              "radix_scatter_5e7"])
     ap.add_argument("--no-also", action="store_true", help="measure only the headline workload")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--zero-operands", action="store_true",
+                    help="16-bit GEMM workloads: all-zero A and B (what the kernel does when the data costs no power)")
+    ap.add_argument("--tunable", action="append", default=[], metavar="NAME=VALUE",
+                    help="sarek_hip_set_tunable(NAME, VALUE) before measuring (kernel shape and measurement knobs)")
     return ap.parse_args()
 
 
@@ -106,6 +110,9 @@ class Launch:
 
 def dims(*d):
     return (C.c_int * 3)(*d)
+
+
+ZERO_OPERANDS = False
 
 
 def make_workload(name, torch, hip):
@@ -182,10 +189,11 @@ def make_workload(name, torch, hip):
         bf16 = name == "gemm_bf16_8192"
         dt = torch.bfloat16 if bf16 else torch.float16
         g.manual_seed(0xA4)
-        t = (torch.randn(s, s, device="cuda", generator=g) * 0.02).to(dt)
+        scale = 0.0 if ZERO_OPERANDS else 0.02
+        t = (torch.randn(s, s, device="cuda", generator=g) * scale).to(dt)
         va = device_vector(sarek, hip, torch, t, elem_size=2)
         g.manual_seed(0xB4)
-        t = (torch.randn(s, s, device="cuda", generator=g) * 0.02).to(dt)
+        t = (torch.randn(s, s, device="cuda", generator=g) * scale).to(dt)
         vb = device_vector(sarek, hip, torch, t, elem_size=2)
         del t
         vc = V.create(V.float32, s * s)
@@ -493,6 +501,11 @@ def main():
         print("bench.py needs a GPU", file=sys.stderr)
         sys.exit(2)
     torch.cuda.set_device(0)
+    global ZERO_OPERANDS
+    ZERO_OPERANDS = args.zero_operands
+    for item in args.tunable:
+        name, _, value = item.partition("=")
+        hip.check(hip.lib.sarek_hip_set_tunable(name.encode(), int(value)))
 
     head = measure(args.workload, torch, hip, args.steps, args.warmup)
     out = {
@@ -519,6 +532,10 @@ def main():
             also.append(r)
         out["also"] = also
     info = hip.device_info(0)
+    if args.tunable:
+        out["tunables"] = args.tunable
+    if args.zero_operands:
+        out["config"] = dict(out["config"], workload=out["config"]["workload"].replace("N(0,0.02)", "all-zero operands"))
     out["device"] = {"name": info.name.decode(), "arch": info.gcn_arch.decode(),
                      "cus": info.multiprocessor_count, "clock_mhz": info.clock_rate_khz // 1000}
     print(json.dumps(out))

@@ -198,7 +198,11 @@ constexpr int lcm_int(int a, int b) {
   return m;
 }
 
-template <bool Bf16, int Epi, int BKA, int BKB, int NA, int NB, int TJ>
+// Ablate (measurement only, results are wrong by construction; tunable gemm16.ablate): bit 0 leaves the
+// global -> LDS transfers out of the K loop (the ring keeps what the prologue put there), bit 1 the LDS
+// fragment reads (every MFMA reuses the first fragments).  What remains shows what each part of the loop
+// costs in cycles and, under the package power limit, in clock.
+template <bool Bf16, int Epi, int BKA, int BKB, int NA, int NB, int TJ, int Ablate = 0>
 __global__ __launch_bounds__(64 * 2 * (8 / TJ)) void gemm16_dma_kernel(const uint16_t *__restrict__ A,
                                                              const uint16_t *__restrict__ B,
                                                              float *__restrict__ C,
@@ -309,18 +313,22 @@ __global__ __launch_bounds__(64 * 2 * (8 / TJ)) void gemm16_dma_kernel(const uin
   // B: the resource is rebased to the slab's first row (keeps every offset below 2^31).
   const __amdgpu_buffer_rsrc_t a_rsrc = make_rsrc(a_base, 0x80000000u);
   auto issue_a = [&](char *sa, int stage) {
+    if (stage >= NA && (Ablate & 1)) return;
     const uint32_t a_so = static_cast<uint32_t>(min(stage, nstages - 1)) * (BKA * 2);
 #pragma unroll
     for (int i = 0; i < DA; ++i) dma16(a_rsrc, a_off[i], a_so, sa + (wave + NWAVES * i) * 1024);
   };
   auto issue_b = [&](char *sb, int slab) {
+    if (slab >= NB && (Ablate & 1)) return;
     const int sl = min(slab, nslabs - 1);
     const __amdgpu_buffer_rsrc_t b_rsrc = make_rsrc(b_base + sl * b_slab_bytes, 0x80000000u);
 #pragma unroll
     for (int i = 0; i < DB; ++i) dma16(b_rsrc, b_off[i], 0u, sb + (wave + NWAVES * i) * 1024);
   };
   // ka: k-step within the A stage, kb: k-step within the B slab
+  bool frags_loaded = false;
   auto load_frags = [&](const char *sa, const char *sb, int ka, int kb, u32x4 (&af)[4], u32x4 (&bf)[TJ]) {
+    if ((Ablate & 2) && frags_loaded) return;
     const char *pa = sa + (a_addr0 ^ (ka << 5));
 #pragma unroll
     for (int i = 0; i < 4; ++i)
@@ -409,6 +417,10 @@ __global__ __launch_bounds__(64 * 2 * (8 / TJ)) void gemm16_dma_kernel(const uin
   __builtin_amdgcn_s_waitcnt(waitcnt_vm_lgkm0(0));
   barrier_no_fence();
   load_frags(lds_ring<10, A_BYTES_S>, lds_ring<20, B_BYTES_S>, 0, 0, af[0], bf[0]);
+  if (Ablate & 2) {
+    load_frags(lds_ring<10, A_BYTES_S>, lds_ring<20, B_BYTES_S>, 1, 1, af[1], bf[1]);
+    frags_loaded = true;
+  }
   __builtin_amdgcn_sched_barrier(0);
 
   // Whole periods first (no exits inside a period, which keeps the accumulators in
@@ -616,6 +628,22 @@ int launch_gemm16(const uint16_t *a, const uint16_t *b, float *c, const float *b
   hipLaunchKernelGGL((gemm16_dma_kernel<Bf16, Epi, BKA, BKB, NA, NB, TJ>), grid,                      \
                      dim3(64 * 2 * (8 / TJ)), 0, st, a, b, c, bias, rowsum, m, n, k, tiles_m,         \
                      tiles_n, remap, probe)
+      const int ablate = (int)tunable("gemm16.ablate", 0);
+      if (ablate != 0) {
+        // measurement variants of the default shape (bf16, plain store); anything else is refused
+        if (!Bf16 || Epi != EPI_STORE || ring != 0 || tj != 2 || ablate < 1 || ablate > 3)
+          return fail(SAREK_HIP_E_UNSUPPORTED, "gemm16.ablate is for the default bf16 kernel only (1..3)");
+        if constexpr (Bf16 && Epi == EPI_STORE) {
+#define SAREK_LAUNCH_ABLATED(AB)                                                                    \
+  hipLaunchKernelGGL((gemm16_dma_kernel<true, EPI_STORE, 64, 32, 2, 4, 2, AB>), grid, dim3(512), 0, st, a, b, c, \
+                     bias, rowsum, m, n, k, tiles_m, tiles_n, remap, probe)
+          if (ablate == 1) SAREK_LAUNCH_ABLATED(1);
+          else if (ablate == 2) SAREK_LAUNCH_ABLATED(2);
+          else SAREK_LAUNCH_ABLATED(3);
+#undef SAREK_LAUNCH_ABLATED
+        }
+        return check_launch("gemm16 kernel launch");
+      }
       if (ring == 4 && tj == 2) SAREK_LAUNCH_DMA(32, 32, 4, 4, 2);
       else if (ring == 4) SAREK_LAUNCH_DMA(32, 32, 4, 4, 4);
       else if (ring == 2 && tj == 2) SAREK_LAUNCH_DMA(64, 64, 2, 2, 2);
