@@ -99,6 +99,11 @@ int sarek_hip_device_get_info(int device, sarek_hip_device_info *out);
  * bytes, so a binding checks its own struct against it once (no counterpart in the reference, whose
  * ctypes layer reads one attribute per call, sarek-cuda/Cuda_api.ml:77-129).                         */
 int sarek_hip_device_info_size(void);
+/* The text tools/device_info.ml:45-93 prints (banner, "Found N device(s)", one block per device as its
+ * print_device_info :16-43 lays it out, usage lines; or its "No devices found" text) for the devices of this
+ * backend.  *device_count (may be NULL) gets the number of devices: the tool exits 1 when it is 0.
+ * SAREK_HIP_E_BUFFER_TOO_SMALL with *needed set when the text does not fit.  Never fails for lack of a GPU. */
+int sarek_hip_device_report(char *out, size_t cap, size_t *needed, int *device_count);
 int sarek_hip_device_set_current(int device);
 int sarek_hip_device_get_current(int *device);
 int sarek_hip_device_synchronize(void);         /* Transfer.flush -> Device.synchronize */
@@ -109,7 +114,12 @@ int sarek_hip_driver_version(int *version);
 /* Memory  (replaces cuMemAlloc/Free/Memcpy.., sarek-cuda/Cuda_api.ml:183-244).
  * `sarek_hip_mem_free(NULL)` and a double free of the same pointer are
  * accepted: the reference frees buffers both explicitly and from a GC
- * finaliser that may run late (sarek/core/Gpu_memory.ml:163-178).          */
+ * finaliser that may run late (sarek/core/Gpu_memory.ml:163-178).  The library
+ * recognises a freed buffer by its ADDRESS: a second free that arrives after
+ * sarek_hip_mem_alloc has handed the same address out again frees the new
+ * buffer.  A binding therefore keeps its own `freed` flag per buffer record and
+ * calls this once (the reference's finaliser does: Gpu_memory.ml:166-172); the
+ * tolerance here only covers a late free of an address not yet reused.        */
 int sarek_hip_mem_alloc(void **dptr, size_t bytes);
 int sarek_hip_mem_free(void *dptr);
 /* Memory.host_ptr_to_device / device_to_host_ptr (sarek-cuda/Cuda_api.ml:207-230, called

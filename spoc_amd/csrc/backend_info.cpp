@@ -4,6 +4,7 @@
 // the entries the CUDA plugin registers (sarek-cuda/Cuda_plugin.ml:47-143) in their HIP spellings and
 // takes more at run time.  The code generator has its own table: the registry is for callers that ask
 // what a backend offers (sarek/framework/test/test_framework_integration.ml:190-207).
+#include <cstring>
 #include <map>
 #include <mutex>
 #include <string>
@@ -42,6 +43,35 @@ std::map<std::string, Intrinsic> &table() {
   return *t;
 }
 
+// tools/device_info.ml:8-14
+std::string format_memory(uint64_t bytes) {
+  char buf[64];
+  const double gb = static_cast<double>(bytes) / (1024.0 * 1024.0 * 1024.0);
+  if (gb >= 1.0) std::snprintf(buf, sizeof(buf), "%.2f GB", gb);
+  else std::snprintf(buf, sizeof(buf), "%.0f MB", static_cast<double>(bytes) / (1024.0 * 1024.0));
+  return buf;
+}
+
+// tools/device_info.ml:16-43 for a device of this backend (never a CPU device; FP64 and atomics always:
+// the capabilities record of sarek-cuda/Cuda_plugin_base.ml:177-195 with this device's figures)
+std::string device_block(int id, const sarek_hip_device_info &d) {
+  char buf[512];
+  std::string o;
+  std::snprintf(buf, sizeof(buf), "[%d] %s\n    Backend: HIP\n    Memory: %s\n", id, d.name,
+                format_memory(d.total_global_mem).c_str());
+  o += buf;
+  if (d.compute_major > 0) {
+    std::snprintf(buf, sizeof(buf), "    Compute Capability: %d.%d\n", d.compute_major, d.compute_minor);
+    o += buf;
+  }
+  std::snprintf(buf, sizeof(buf),
+                "    Max Threads/Block: %d\n    Compute Units: %d\n    Warp/Wavefront Size: %d\n"
+                "    Features: Atomics, FP64\n",
+                d.max_threads_per_block, d.multiprocessor_count, d.warp_size);
+  o += buf;
+  return o;
+}
+
 }  // namespace
 }  // namespace sarek_hip
 
@@ -60,6 +90,34 @@ int sarek_hip_backend_version(int *major, int *minor, int *patch) {
 }
 
 int sarek_hip_execution_model(void) { return SAREK_HIP_EXECUTION_JIT; }
+
+int sarek_hip_device_report(char *out, size_t cap, size_t *needed, int *device_count) {
+  const std::string rule(70, '=');
+  std::string o = rule + "\nSAREK Device Information Utility\nMulti-Backend GPU/CPU Device Diagnostic Tool\n" + rule + "\n";
+  int count = 0;
+  if (sarek_hip_is_available()) {
+    if (sarek_hip_device_count(&count) != SAREK_HIP_OK) count = 0;
+  }
+  if (device_count) *device_count = count;
+  if (count == 0) {
+    o += "\n\xE2\x9A\xA0 No devices found\nEnsure you have:\n"
+         "  - HIP backend: AMD GPU driver + ROCm runtime (libamdhip64, libhiprtc)\n" + rule + "\n";
+  } else {
+    o += "\nFound " + std::to_string(count) + " device" + (count > 1 ? "s" : "") + ":\n\n";
+    for (int i = 0; i < count; ++i) {
+      sarek_hip_device_info d;
+      if (sarek_hip_device_get_info(i, &d) != SAREK_HIP_OK) continue;     // Device.get i = None: skipped
+      o += device_block(i, d) + "\n";
+    }
+    o += rule + "\nUsage:\n  \xE2\x80\xA2 Device.get N returns device N (0-" + std::to_string(count - 1) + ")\n"
+         "  \xE2\x80\xA2 Device.by_framework \"HIP\" filters by backend\n" + rule + "\n";
+  }
+  if (needed) *needed = o.size() + 1;
+  if (!out || cap < o.size() + 1)
+    return fail(SAREK_HIP_E_BUFFER_TOO_SMALL, "device_report: %zu bytes needed", o.size() + 1);
+  std::memcpy(out, o.c_str(), o.size() + 1);
+  return SAREK_HIP_OK;
+}
 
 int sarek_hip_intrinsic_register(const char *name, const char *codegen, int convergence) {
   if (!name || !codegen || !*name) return fail(SAREK_HIP_E_INVALID_ARG, "intrinsic_register: NULL or empty argument");

@@ -28,7 +28,10 @@ unsigned long long *clock_probe(int64_t workgroups) {
   return (g_probe && workgroups <= g_probe_pairs) ? g_probe : nullptr;
 }
 
-int64_t tunable(const char *name, int64_t fallback) {
+#undef tunable
+std::atomic<uint64_t> g_tunable_generation{1};
+
+int64_t tunable_lookup(const char *name, int64_t fallback) {
   std::lock_guard<std::mutex> lock(g_mu);
   auto &t = table();
   auto it = t.find(std::string_view(name));
@@ -44,6 +47,7 @@ int64_t tunable(const char *name, int64_t fallback) {
 void set_tunable(const char *name, int64_t value) {
   std::lock_guard<std::mutex> lock(g_mu);
   table()[name] = value;
+  g_tunable_generation.fetch_add(1, std::memory_order_release);
 }
 }  // namespace sarek_hip
 

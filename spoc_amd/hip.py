@@ -75,6 +75,7 @@ class PipelineStage(C.Structure):
 SYMBOLS = {
     "sarek_hip_abi_version": (_i, []),
     "sarek_hip_device_info_size": (_i, []),
+    "sarek_hip_device_report": (_i, [C.c_char_p, _sz, C.POINTER(_sz), C.POINTER(_i)]),
     "sarek_hip_last_error": (C.c_char_p, []),
     "sarek_hip_status_name": (C.c_char_p, [_i]),
     "sarek_hip_init": (_i, []),
@@ -374,6 +375,15 @@ class pinned_array:
 
     def __exit__(self, *exc):
         self.close()
+
+
+def device_report():
+    """(text, device count) of the device-information tool (tools/device_info.ml)."""
+    need, count = C.c_size_t(0), C.c_int(0)
+    lib.sarek_hip_device_report(None, 0, C.byref(need), C.byref(count))
+    buf = C.create_string_buffer(need.value)
+    check(lib.sarek_hip_device_report(buf, need.value, None, C.byref(count)))
+    return buf.value.decode(), count.value
 
 
 def device_info(device=0):

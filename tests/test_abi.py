@@ -177,3 +177,16 @@ def test_device_info_layout_agrees_between_header_python_and_documented_ocaml_st
     assert [(s[0], ocaml[s[3] or s[1]], int(s[2]) if s[2] else None) for s in stub] == fields
     assert doc.index("max_registers_per_block\" int") < doc.index("seal device_info")
     assert "sarek_hip_device_info_size" in doc
+
+
+def test_device_report_never_needs_a_gpu(hip):
+    """tools/device_info.ml:45-93: banner first; with no device the tool says so and exits 1."""
+    text, count = hip.device_report()
+    lines = text.split("\n")
+    assert lines[0] == "=" * 70 and lines[1] == "SAREK Device Information Utility" and lines[3] == "=" * 70
+    if count == 0:
+        assert "No devices found" in text and "Found" not in text
+    need = ctypes.c_size_t(0)
+    small = ctypes.create_string_buffer(8)
+    assert hip.lib.sarek_hip_device_report(small, 8, ctypes.byref(need), None) == hip.E_BUFFER_TOO_SMALL
+    assert need.value == len(text.encode()) + 1

@@ -46,6 +46,24 @@ def test_runtime_device_info(hip, torch_cuda):
     assert info.shared_mem_per_block >= 64 * 1024
 
 
+def test_device_report_is_the_reference_tools_text(hip, torch_cuda):
+    """tools/device_info.ml:16-43,66-90: one block per device, laid out as print_device_info does."""
+    import subprocess
+    import sys
+    text, count = hip.device_report()
+    info = hip.device_info(0)
+    gb = info.total_global_mem / 1024 ** 3
+    block = (f"[0] {info.name.decode()}\n    Backend: HIP\n    Memory: {gb:.2f} GB\n"
+             f"    Compute Capability: {info.compute_major}.{info.compute_minor}\n"
+             f"    Max Threads/Block: {info.max_threads_per_block}\n    Compute Units: {info.multiprocessor_count}\n"
+             f"    Warp/Wavefront Size: 64\n    Features: Atomics, FP64\n\n")
+    assert count >= 1 and f"\nFound {count} device{'s' if count > 1 else ''}:\n\n" in text
+    assert block in text and f"Device.get N returns device N (0-{count - 1})" in text
+    root = __import__("os").path.dirname(__import__("os").path.dirname(__import__("os").path.abspath(__file__)))
+    run = subprocess.run([sys.executable, "-m", "spoc_amd.device_info"], cwd=root, capture_output=True, text=True)
+    assert run.returncode == 0 and run.stdout == text
+
+
 def test_runtime_memory_roundtrip_and_double_free(hip, torch_cuda):
     p = C.c_void_p()
     hip.check(hip.lib.sarek_hip_mem_alloc(C.byref(p), 4096))
