@@ -54,7 +54,7 @@ def parse():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--workload", default="gemm_bf16_8192",
                     choices=["gemm_bf16_8192", "gemm_f16_8192", "triad_sum_2p28", "gemm_f32_8192", "gemm_f32_1024",
-                             "gemm_f16_epilogue", "copy_1gib", "vendor_gemm_bf16_8192", "histogram_2p28",
+                             "gemm_f16_epilogue", "gemm_f16_4095x11008x4096", "copy_1gib", "vendor_gemm_bf16_8192", "histogram_2p28",
                              "radix_scatter_5e7"])
     ap.add_argument("--no-also", action="store_true", help="measure only the headline workload")
     ap.add_argument("--no-cpu-baseline", action="store_true")
@@ -272,6 +272,29 @@ def make_workload(name, torch, hip):
                     config={"workload": "out[counters[key & 255]++] = key, random keys below 100000", "n": n,
                             "algorithmic_bytes": 8 * n})
         return main, None, info, (vk, vo, vcnt, starts, a, ir)
+    if name == "gemm_f16_4095x11008x4096":
+        # the epilogue config's product without the epilogue: what the fused chain costs on top
+        m, n, k = 4095, 11008, 4096
+        g.manual_seed(0xA5)
+        t = (torch.randn(m, k, device="cuda", generator=g) * 0.02).half()
+        va = device_vector(sarek, hip, torch, t, elem_size=2)
+        g.manual_seed(0xB5)
+        t = (torch.randn(k, n, device="cuda", generator=g) * 0.02).half()
+        vb = device_vector(sarek, hip, torch, t, elem_size=2)
+        del t
+        vy = V.create(V.float32, m * n)
+        sarek.Transfer.to_device(vy)
+        src, entry = hip.library_kernel("gemm_f16")
+        a, na = E._args([E.Vec(va), E.Vec(vb), E.Vec(vy), E.Int32(m), E.Int32(n), E.Int32(k)])
+        src_b, entry_b = src.encode(), entry.encode()
+        main = Launch(hip, lib.sarek_hip_execute_run_source, src_b, hip.LANG_HIP, entry_b, dims(16, 16, 1),
+                      dims((n + 15) // 16, (m + 15) // 16, 1), 0, 1, a, na)
+        info = dict(metric="fp16 GEMM TFLOP/s at the epilogue config's shape", unit="TFLOP/s", dtype="f16",
+                    work=2.0 * m * n * k, work_unit=1e12, bound="mfma",
+                    peak=PEAK_MFMA_TFLOPS["f16"], kernel="gemm16_dma_kernel<f16, store, 64, 32, 2, 4, 2>",
+                    route="Execute.run_source ~lang:HIP_Source, library kernel text 'gemm_f16'",
+                    config={"workload": "fp16-in f32-acc C=A.B", "m": m, "n": n, "k": k})
+        return main, None, info, (va, vb, vy, a, src_b, entry_b)
     if name == "gemm_f16_epilogue":
         m, n, k = 4095, 11008, 4096
         g.manual_seed(0xA5)
