@@ -37,12 +37,13 @@ NOMINAL_CLOCK_MHZ = 2400.0
 # HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (KiB per dispatch,
 # FETCH_SIZE scaled by 2.0 and WRITE_SIZE by 1.0 after calibration against a plain 1 GiB copy).
 MEASURED_TRAFFIC_BYTES = {
-    "triad_sum_2p28": (1048600 * 2 + 1050630) * 1024,
-    "gemm_bf16_8192": (793626 * 2 + 262153) * 1024,
-    "gemm_f32_8192": (1695900 * 2 + 262153) * 1024,
-    "gemm_f16_epilogue": (306687 * 2 + 176779) * 1024,
-    "histogram_2p28": (524312 * 2 + 256) * 1024,
-    "radix_scatter_5e7": (97880 * 2 + 215611) * 1024,
+    "triad_sum_2p28": (1048610 * 2 + 1052680) * 1024,
+    "gemm_bf16_8192": (793996 * 2 + 262153) * 1024,
+    "gemm_f32_8192": (1698530 * 2 + 262153) * 1024,
+    "gemm_f32_1024": (12333 * 2 + 4098) * 1024,
+    "gemm_f16_epilogue": (307729 * 2 + 176779) * 1024,
+    "histogram_2p28": (493838 * 2 + 256) * 1024,
+    "radix_scatter_5e7": (97870 * 2 + 215643) * 1024,
 }
 PEAK_MFMA_TFLOPS = {"bf16": 2500.0, "f16": 2500.0, "f32": 157.3}
 

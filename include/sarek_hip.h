@@ -264,6 +264,25 @@ int sarek_hip_library_kernel_source(const char *name, char *source, size_t sourc
                                     char *entry /* may be NULL */, size_t entry_cap);
 int sarek_hip_library_kernel_list(char *out, size_t cap, size_t *needed);   /* names, space separated */
 
+/* A sequence of run_source calls made in one: what a plugin does for a list of kernels launched one after the
+ * other on the default stream (no counterpart in BACKEND, whose run_source takes one kernel:
+ * spoc/framework/Framework_sig.ml:324-336).  The results are those of the separate calls; two neighbouring
+ * entries that one hand-written kernel computes in a single pass over the data (a source tagged
+ * stream_triad_f32 followed by one tagged reduce_sum_block256_f32 that reads the vector the first writes,
+ * over the same n) are launched as that kernel.  *device_launches (may be NULL): launches made; *completed
+ * (may be NULL): entries fully served, also when the call fails part of the way.  sarek_hip_last_run_path()
+ * joins the paths with ';', a shared launch reads "<tag>+<tag>".                                              */
+typedef struct sarek_hip_launch {
+  const char *source;
+  int lang;
+  const char *kernel_name;
+  int block[3], grid[3];
+  int shared_mem_bytes;
+  const sarek_hip_arg *args;
+  int n_args;
+} sarek_hip_launch;
+int sarek_hip_run_sources(const sarek_hip_launch *launches, int n_launches, int *device_launches, int *completed);
+
 /* 1 (default) / 0: honour specialise tags.  Also read once from the
  * environment variable SAREK_HIP_SPECIALISE (0 disables).                  */
 int sarek_hip_set_specialisation(int enabled);
@@ -370,9 +389,11 @@ int sarek_hip_execute_run_vectors(const char *ir_text, const int block[3], const
  * the launches a caller makes for the kernel list Sarek_fusion.auto_fuse_pipeline hands back
  * (sarek/sarek/Sarek_fusion.ml:1133-1165; that pass cannot fuse a kernel with barriers, :641-661, so
  * `stream triad, block-256 tree sum` stays two kernels there).  Stages run in order with the
- * results of separate launches; two consecutive stages that one hand-written kernel computes in
- * a single pass over the data (stream triad, then the block-256 sum of the vector it wrote) are
- * launched as that kernel.  *launches (may be NULL) gets the number of device launches made;
+ * results of separate launches: per stage the uploads, the lowering and the argument expansion of
+ * Execute.run_vectors, then all launches through sarek_hip_run_sources (two consecutive stages that
+ * one hand-written kernel computes in a single pass over the data — stream triad, then the block-256
+ * sum of the vector it wrote — are launched as that kernel), then the vectors of the stages that
+ * ran are marked stale.  *launches (may be NULL) gets the number of device launches made;
  * sarek_hip_last_run_path() then reads e.g. "stream_triad_f32+reduce_sum_block256_f32", paths of
  * separate launches joined by ';'.                                                              */
 typedef struct sarek_hip_pipeline_stage {

@@ -375,18 +375,6 @@ int try_specialised_pair(const std::string &tag0, const int block0[3], const int
 
 }  // namespace
 
-void set_last_run_path(const std::string &path) { t_last_path = path; }
-
-int run_specialised_pair(const char *source0, const int block0[3], const int grid0[3], const sarek_hip_arg *args0,
-                         int n_args0, const char *source1, const int block1[3], const int grid1[3],
-                         const sarek_hip_arg *args1, int n_args1, int *rc) {
-  if (!specialisation_enabled()) return 0;
-  const std::string tag0 = read_tag(source0), tag1 = read_tag(source1);
-  if (tag0.empty() || tag1.empty()) return 0;
-  if (!try_specialised_pair(tag0, block0, grid0, args0, n_args0, tag1, block1, grid1, args1, n_args1, rc)) return 0;
-  t_last_path = tag0 + "+" + tag1;
-  return 1;
-}
 }  // namespace sarek_hip
 
 using namespace sarek_hip;
@@ -399,6 +387,46 @@ int sarek_hip_set_specialisation(int enabled) {
 }
 
 const char *sarek_hip_last_run_path(void) { return t_last_path.c_str(); }
+
+int sarek_hip_run_sources(const sarek_hip_launch *launches, int n_launches, int *device_launches, int *completed) {
+  if (device_launches) *device_launches = 0;
+  if (completed) *completed = 0;
+  if (n_launches < 0 || (n_launches > 0 && !launches))
+    return fail(SAREK_HIP_E_INVALID_ARG, "run_sources: NULL or negative argument");
+  std::string path;
+  for (int i = 0; i < n_launches; ++i) {
+    const sarek_hip_launch &l0 = launches[i];
+    int served = 0;
+    if (i + 1 < n_launches && specialisation_enabled() && l0.source && launches[i + 1].source && l0.args &&
+        launches[i + 1].args) {
+      // two launches one hand-written kernel computes in a single pass over the data
+      const sarek_hip_launch &l1 = launches[i + 1];
+      const bool langs_ok = (l0.lang == SAREK_HIP_LANG_HIP_SOURCE || l0.lang == SAREK_HIP_LANG_CUDA_SOURCE) &&
+                            (l1.lang == SAREK_HIP_LANG_HIP_SOURCE || l1.lang == SAREK_HIP_LANG_CUDA_SOURCE);
+      const std::string tag0 = read_tag(l0.source), tag1 = read_tag(l1.source);
+      int rc = SAREK_HIP_OK;
+      if (langs_ok && !tag0.empty() && !tag1.empty() &&
+          try_specialised_pair(tag0, l0.block, l0.grid, l0.args, l0.n_args, tag1, l1.block, l1.grid, l1.args,
+                               l1.n_args, &rc)) {
+        if (rc != SAREK_HIP_OK) return rc;
+        path += (path.empty() ? "" : ";") + tag0 + "+" + tag1;
+        served = 2;
+      }
+    }
+    if (!served) {
+      const int rc = sarek_hip_run_source(l0.source, l0.lang, l0.kernel_name, l0.block, l0.grid, l0.shared_mem_bytes,
+                                          l0.args, l0.n_args);
+      if (rc != SAREK_HIP_OK) return rc;
+      path += (path.empty() ? "" : ";") + t_last_path;
+      served = 1;
+    }
+    i += served - 1;
+    if (device_launches) ++*device_launches;
+    if (completed) *completed += served;
+  }
+  t_last_path = path.empty() ? "none" : path;
+  return SAREK_HIP_OK;
+}
 
 int sarek_hip_run_source(const char *source, int lang, const char *kernel_name, const int block[3],
                          const int grid[3], int shared_mem_bytes, const sarek_hip_arg *args,

@@ -138,6 +138,19 @@ __global__ __launch_bounds__(kBlock) void triad_kernel(float *__restrict__ a,
   const bool has_tail = Sum != SUM_BLOCK256 && blockIdx.x == gridDim.x - 1 && ti < n;
   if (has_tail) tail = triad1(b[ti], c[ti], sd);
 
+  // the stores go out first: the sums below are register work that needs nothing from memory
+  if (full) {
+#pragma unroll
+    for (int u = 0; u < kUnroll; ++u) stg_nt(a4 + base + u * kBlock, r[u]);
+  } else {
+#pragma unroll
+    for (int u = 0; u < kUnroll; ++u) {
+      const int64_t i = base + u * kBlock;
+      if (i < n4) a4[i] = r[u];
+    }
+  }
+  if (has_tail) a[ti] = tail;
+
   if (Sum == SUM_WORKGROUP) {
     float4 acc = make_float4(0.f, 0.f, 0.f, 0.f);
 #pragma unroll
@@ -157,18 +170,6 @@ __global__ __launch_bounds__(kBlock) void triad_kernel(float *__restrict__ a,
       if ((threadIdx.x & 63) == 0 && j < nblocks) partials[j] = t;
     }
   }
-
-  if (full) {
-#pragma unroll
-    for (int u = 0; u < kUnroll; ++u) stg_nt(a4 + base + u * kBlock, r[u]);
-  } else {
-#pragma unroll
-    for (int u = 0; u < kUnroll; ++u) {
-      const int64_t i = base + u * kBlock;
-      if (i < n4) a4[i] = r[u];
-    }
-  }
-  if (has_tail) a[ti] = tail;
 }
 
 // Unaligned-pointer fallback: one element per thread, grid-stride.

@@ -623,47 +623,36 @@ int sarek_hip_execute_run_pipeline(const sarek_hip_pipeline_stage *stages, int n
   int dev = 0;
   int st = current_device(&dev);
   if (st != SAREK_HIP_OK) return st;
-  std::string path;
+  // per stage what Execute.run_vectors does before and after B.run_source (upload, lower, expand ...
+  // mark stale); the launches themselves go to the plugin as one sequence, which may serve neighbours together
+  std::vector<std::shared_ptr<const Lowered>> lowered(n_stages);
+  std::vector<std::vector<sarek_hip_arg>> expanded(n_stages);
+  std::vector<sarek_hip_launch> seq(n_stages);
   for (int i = 0; i < n_stages; ++i) {
-    const sarek_hip_pipeline_stage &s0 = stages[i];
-    if (i + 1 < n_stages) {
-      // two stages one hand kernel can serve: what Execute.run_vectors does for each, with one launch between
-      const sarek_hip_pipeline_stage &s1 = stages[i + 1];
-      std::shared_ptr<const Lowered> k0, k1;
-      try {
-        if ((st = lower(s0.ir_text, s0.block, k0)) != SAREK_HIP_OK) return st;
-        if ((st = lower(s1.ir_text, s1.block, k1)) != SAREK_HIP_OK) return st;
-      } catch (const std::exception &e) {
-        return fail(SAREK_HIP_E_PARSE, "run_pipeline: %s", e.what());
-      }
-      if (std::strncmp(k0->source.c_str(), kSpecialiseMarker, std::strlen(kSpecialiseMarker)) == 0 &&
-          std::strncmp(k1->source.c_str(), kSpecialiseMarker, std::strlen(kSpecialiseMarker)) == 0) {
-        if ((st = transfer_args(s0.args, s0.n_args, dev)) != SAREK_HIP_OK) return st;
-        if ((st = transfer_args(s1.args, s1.n_args, dev)) != SAREK_HIP_OK) return st;
-        std::vector<sarek_hip_arg> rs0, rs1;
-        if ((st = expand_args(s0.args, s0.n_args, dev, true, rs0)) != SAREK_HIP_OK) return st;
-        if ((st = expand_args(s1.args, s1.n_args, dev, true, rs1)) != SAREK_HIP_OK) return st;
-        int rc = SAREK_HIP_OK;
-        if (run_specialised_pair(k0->source.c_str(), s0.block, s0.grid, rs0.data(), static_cast<int>(rs0.size()),
-                                 k1->source.c_str(), s1.block, s1.grid, rs1.data(), static_cast<int>(rs1.size()),
-                                 &rc)) {
-          if (rc != SAREK_HIP_OK) return rc;
-          mark_stale(s0.args, s0.n_args, dev);
-          mark_stale(s1.args, s1.n_args, dev);
-          if (launches) ++*launches;
-          path += (path.empty() ? "" : ";") + std::string(sarek_hip_last_run_path());
-          ++i;
-          continue;
-        }
-      }
+    const sarek_hip_pipeline_stage &s = stages[i];
+    if ((st = transfer_args(s.args, s.n_args, dev)) != SAREK_HIP_OK) return st;
+    try {
+      if ((st = lower(s.ir_text, s.block, lowered[i])) != SAREK_HIP_OK) return st;
+    } catch (const std::exception &e) {
+      return fail(SAREK_HIP_E_PARSE, "run_pipeline: stage %d: %s", i, e.what());
     }
-    st = sarek_hip_execute_run_vectors(s0.ir_text, s0.block, s0.grid, s0.shared_mem_bytes, s0.args, s0.n_args);
-    if (st != SAREK_HIP_OK) return st;
-    if (launches) ++*launches;
-    path += (path.empty() ? "" : ";") + std::string(sarek_hip_last_run_path());
+    if ((st = expand_args(s.args, s.n_args, dev, true, expanded[i])) != SAREK_HIP_OK) return st;
+    sarek_hip_launch &l = seq[i];
+    l.source = lowered[i]->source.c_str();
+    l.lang = SAREK_HIP_LANG_HIP_SOURCE;
+    l.kernel_name = lowered[i]->name.c_str();
+    for (int d = 0; d < 3; ++d) {
+      l.block[d] = s.block[d];
+      l.grid[d] = s.grid[d];
+    }
+    l.shared_mem_bytes = s.shared_mem_bytes;
+    l.args = expanded[i].data();
+    l.n_args = static_cast<int>(expanded[i].size());
   }
-  set_last_run_path(path.empty() ? "none" : path);
-  return SAREK_HIP_OK;
+  int done = 0;
+  st = sarek_hip_run_sources(seq.data(), n_stages, launches, &done);
+  for (int i = 0; i < done; ++i) mark_stale(stages[i].args, stages[i].n_args, dev);
+  return st;
 }
 
 int sarek_hip_execute_run_source(const char *source, int lang, const char *kernel_name, const int block[3],

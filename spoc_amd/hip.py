@@ -65,6 +65,12 @@ class VArg(C.Structure):
                 ("f32", C.c_float), ("f64", C.c_double)]
 
 
+class Launch(C.Structure):
+    """sarek_hip_launch: one run_source call of a sequence."""
+    _fields_ = [("source", C.c_char_p), ("lang", C.c_int), ("kernel_name", C.c_char_p), ("block", C.c_int * 3),
+                ("grid", C.c_int * 3), ("shared_mem_bytes", C.c_int), ("args", C.POINTER(Arg)), ("n_args", C.c_int)]
+
+
 class PipelineStage(C.Structure):
     """sarek_hip_pipeline_stage: one Execute.run_vectors call of a kernel sequence."""
     _fields_ = [("ir_text", C.c_char_p), ("block", C.c_int * 3), ("grid", C.c_int * 3),
@@ -188,6 +194,7 @@ SYMBOLS = {
     "sarek_hip_execute_run_source": (_i, [C.c_char_p, _i, C.c_char_p, _int3, _int3, _i, _i, C.POINTER(VArg), _i]),
     "sarek_hip_execute_sync_vectors_to_cpu": (_i, [C.POINTER(VArg), _i]),
     "sarek_hip_execute_run_pipeline": (_i, [C.POINTER(PipelineStage), _i, C.POINTER(_i)]),
+    "sarek_hip_run_sources": (_i, [C.POINTER(Launch), _i, C.POINTER(_i), C.POINTER(_i)]),
     "sarek_hip_library_kernel_source": (_i, [C.c_char_p, C.c_char_p, _sz, C.POINTER(_sz), C.c_char_p, _sz]),
     "sarek_hip_library_kernel_list": (_i, [C.c_char_p, _sz, C.POINTER(_sz)]),
     "sarek_hip_triad_block256_sum_f32": (_i, [_vp, _vp, _vp, _f, _i64, _vp, _vp]),
@@ -648,6 +655,26 @@ def run_source(source, kernel_name, block, grid, items, shared_mem=0, lang=LANG_
     check(lib.sarek_hip_run_source(source.encode(), lang, kernel_name.encode(), blk, grd,
                                    int(shared_mem), args, n))
     return lib.sarek_hip_last_run_path().decode()
+
+
+def run_sources(launches):
+    """launches: [(source, kernel_name, block, grid, items)] or [(..., shared_mem)]; one call for the
+    sequence.  Returns (code paths, device launches made)."""
+    arr = (Launch * max(len(launches), 1))()
+    keep = []
+    for l, item in zip(arr, launches):
+        source, name, block, grid, items = item[:5]
+        args, n = make_args(items)
+        src, nm = source.encode(), name.encode()
+        keep.append((args, src, nm))
+        l.source, l.lang, l.kernel_name = src, LANG_HIP, nm
+        l.block, l.grid = (C.c_int * 3)(*block), (C.c_int * 3)(*grid)
+        l.shared_mem_bytes = item[5] if len(item) > 5 else 0
+        l.args, l.n_args = args, n
+    made, done = C.c_int(0), C.c_int(0)
+    check(lib.sarek_hip_run_sources(arr, len(launches), C.byref(made), C.byref(done)))
+    assert done.value == len(launches)
+    return lib.sarek_hip_last_run_path().decode(), made.value
 
 
 def generate_source(ir_text, block=None):

@@ -259,6 +259,46 @@ def test_pipeline_pairs_that_are_not_the_fused_operation_run_one_by_one(hip, ora
     assert E.run_pipeline([]) == ("none", 0)
 
 
+def test_run_sources_at_the_plugin_boundary(hip, oracle, torch_cuda):
+    """The sequence entry a plugin calls with raw buffers (what Hip_plugin would marshal from run_source_arg lists):
+    generated triad and block-sum sources one after the other are one launch, anything else one launch each."""
+    torch = torch_cuda
+    n = 300007
+    nb = (n + 255) // 256
+    b = torch.from_numpy(oracle.fill_uniform(n, seed=0xB)).cuda()
+    c = torch.from_numpy(oracle.fill_uniform(n, seed=0xC)).cuda()
+    a = torch.full((n,), float("nan"), device="cuda")
+    sums = torch.full((nb,), float("nan"), device="cuda")
+    tri, red = hip.generate_source(load_ir("stream_triad")), hip.generate_source(load_ir("reduction"), block=(256, 1, 1))
+    l0 = (tri, "sarek_kern", (256, 1, 1), (nb, 1, 1), [a, b, c, ("f32", 3.0), ("i32", n)])
+    l1 = (red, "sarek_kern", (256, 1, 1), (nb, 1, 1), [a, sums, ("i32", n)])
+    assert hip.run_sources([l0, l1]) == ("stream_triad_f32+reduce_sum_block256_f32", 1)
+    torch.cuda.synchronize()
+    a_ref, p_ref, _ = oracle.triad_sum(b.cpu().numpy(), c.cpu().numpy(), 3.0)
+    assert np.array_equal(a.cpu().numpy(), a_ref)
+    assert np.abs(sums.cpu().numpy() - p_ref).max() <= 1e-5 * np.abs(p_ref).max()
+    fused = sums.clone()
+    # the other order, and a single entry, run as they are
+    sums.fill_(0)
+    assert hip.run_sources([l1, l0]) == ("reduce_sum_block256_f32;stream_triad_f32", 2)
+    assert hip.run_sources([l0]) == ("stream_triad_f32", 1)
+    assert hip.run_sources([l1]) == ("reduce_sum_block256_f32", 1)
+    torch.cuda.synchronize()
+    assert torch.equal(sums, fused)
+    assert hip.run_sources([]) == ("none", 0)
+    # a failing entry reports how far the sequence got
+    import ctypes as C
+    arr = (hip.Launch * 2)()
+    args, na = hip.make_args(l0[4])
+    arr[0].source, arr[0].lang, arr[0].kernel_name = tri.encode(), hip.LANG_HIP, b"sarek_kern"
+    arr[0].block, arr[0].grid, arr[0].args, arr[0].n_args = (C.c_int * 3)(256, 1, 1), (C.c_int * 3)(nb, 1, 1), args, na
+    arr[1].source, arr[1].lang, arr[1].kernel_name = b"this is not HIP", hip.LANG_HIP, b"nope"
+    arr[1].block, arr[1].grid, arr[1].args, arr[1].n_args = (C.c_int * 3)(1, 1, 1), (C.c_int * 3)(1, 1, 1), args, 0
+    made, done = C.c_int(-1), C.c_int(-1)
+    assert hip.lib.sarek_hip_run_sources(arr, 2, C.byref(made), C.byref(done)) != 0
+    assert (made.value, done.value) == (1, 1)
+
+
 def test_fused_pair_kernel_at_full_size_properties(hip, torch_cuda):
     """n = 2^28, the size of the bandwidth config: constants make every value exact, so the vector, every
     block sum and the folded total have closed forms."""
@@ -335,3 +375,28 @@ def test_overlapping_outputs_are_left_to_the_generated_code(hip, oracle, sarek):
     assert hip.run_source(tri, "sarek_kern", (256, 1, 1), (16, 1, 1), in_place) == "stream_triad_f32"
     torch.cuda.synchronize()
     assert bool((v[:4096] == 4.0).all())
+
+
+def test_hand_and_generated_triad_agree(hip, oracle, torch_cuda):
+    """The hand triad rounds b + c*s once from double (the Native backend's rule), the generated kernel once from
+    the fused multiply-add: the same f32 unless the double sum itself lands on a rounding boundary."""
+    torch = torch_cuda
+    n = 1 << 22
+    b = torch.from_numpy(oracle.fill_uniform(n, seed=0xB)).cuda()
+    c = torch.from_numpy(oracle.fill_uniform(n, seed=0xC)).cuda()
+    src = hip.generate_source(load_ir("stream_triad"))
+    outs = []
+    for on in (1, 0):
+        a = torch.empty(n, device="cuda")
+        hip.check(hip.lib.sarek_hip_set_specialisation(on))
+        try:
+            path = hip.run_source(src, "sarek_kern", (256, 1, 1), (n // 256, 1, 1), [a, b, c, ("f32", 3.0), ("i32", n)])
+        finally:
+            hip.check(hip.lib.sarek_hip_set_specialisation(1))
+        assert path == ("stream_triad_f32" if on else "jit")
+        outs.append(a)
+    torch.cuda.synchronize()
+    hand, jit = outs
+    differ = (hand != jit)
+    assert int(differ.sum()) <= 2
+    assert bool(((hand - jit).abs() <= torch.finfo(torch.float32).eps * hand.abs()).all())
