@@ -19,6 +19,9 @@
 //   - parameters, mutable variables, loop variables and shared arrays are renamed by
 //     order of first binding,
 //   - operands of commutative operators are ordered, `a > b` becomes `b < a`,
+//   - int32 index arithmetic (+, -, * of int32 values) is brought to a sum of products with its
+//     constants folded, so bracketing, operand order, distribution and named or inlined constants
+//     do not matter (`(k + tile_size) - 1` = `k + 15`, `t * tile_size + tx` = `tx + 16 * t`),
 //   - thread-index intrinsics use one spelling and `global_thread_id` is expanded to
 //     thread_idx_x + block_idx_x * block_dim_x.
 #include <algorithm>
@@ -28,6 +31,8 @@
 #include <cstring>
 #include <map>
 #include <set>
+#include <stdexcept>
+#include <vector>
 
 #include "ir.hpp"
 
@@ -79,9 +84,123 @@ struct Canon {
     return n;
   }
 
+  // ---- integer index arithmetic as polynomials -----------------------------------------------
+  // int32 addition, subtraction and multiplication form a ring (wrap-around included), so an index
+  // expression means the same however it is bracketed, ordered or distributed, and with its constants
+  // folded or not: `(k + ts) - 1`, `k + (ts - 1)` and `k + 15` (ts = 16) are one expression, and so are
+  // `t * ts + tx` and `tx + 16 * t`.  Such expressions are rendered as a sum of terms, each an integer
+  // coefficient times a sorted product of atoms (anything that is not +, -, * of int32 values).
+  using Poly = std::map<std::vector<std::string>, uint32_t>;
+
+  static bool is_index_intrinsic(const std::string &n) {
+    static const char *names[] = {"thread_idx_x", "thread_idx_y", "thread_idx_z", "block_idx_x", "block_idx_y",
+                                  "block_idx_z", "block_dim_x", "block_dim_y", "block_dim_z", "grid_dim_x",
+                                  "grid_dim_y", "grid_dim_z", "global_thread_id", "global_idx", "global_idx_x",
+                                  "global_idx_y", "global_idx_z", "global_size"};
+    for (const char *k : names)
+      if (n == k) return true;
+    return false;
+  }
+
+  bool is_int32(const ExprP &ep) {
+    const Expr &e = *ep;
+    switch (e.kind) {
+      case Expr::ConstInt32: return true;
+      case Expr::VarRef: return e.var.type && e.var.type->kind == Type::Int32;
+      case Expr::Intrinsic: return e.args.empty() && !e.name.empty() && e.name[0] != '\x01' &&
+                                   is_index_intrinsic(intrinsic_name(e.name));
+      case Expr::Cast: return e.type && e.type->kind == Type::Int32;
+      case Expr::UnopE: return e.unop == Unop::Neg && is_int32(e.args[0]);
+      case Expr::BinopE:
+        switch (e.binop) {
+          case Binop::Add: case Binop::Sub: case Binop::Mul: case Binop::Div: case Binop::Mod:
+            return is_int32(e.args[0]) && is_int32(e.args[1]);
+          default: return false;
+        }
+      default: return false;
+    }
+  }
+
+  static void poly_add(Poly &into, const Poly &p, uint32_t scale) {
+    for (auto &t : p) {
+      uint32_t &c = into[t.first];
+      c += t.second * scale;
+    }
+  }
+
+  Poly poly(const ExprP &ep) {
+    const Expr &e = *ep;
+    Poly p;
+    if (e.kind == Expr::ConstInt32) {
+      p[{}] = static_cast<uint32_t>(e.ival);
+      return p;
+    }
+    if (e.kind == Expr::UnopE && e.unop == Unop::Neg && is_int32(e.args[0])) {
+      poly_add(p, poly(e.args[0]), 0xFFFFFFFFu);
+      return p;
+    }
+    if (e.kind == Expr::BinopE && is_int32(ep) &&
+        (e.binop == Binop::Add || e.binop == Binop::Sub || e.binop == Binop::Mul)) {
+      const Poly a = poly(e.args[0]), b = poly(e.args[1]);
+      if (e.binop == Binop::Mul) {
+        if (a.size() * b.size() > 64) throw std::length_error("index expression too large to normalise");
+        for (auto &x : a)
+          for (auto &y : b) {
+            std::vector<std::string> atoms = x.first;
+            atoms.insert(atoms.end(), y.first.begin(), y.first.end());
+            std::sort(atoms.begin(), atoms.end());
+            p[atoms] += x.second * y.second;
+          }
+      } else {
+        poly_add(p, a, 1u);
+        poly_add(p, b, e.binop == Binop::Add ? 1u : 0xFFFFFFFFu);
+      }
+      return p;
+    }
+    if (e.kind == Expr::Intrinsic && e.args.empty()) {
+      const std::string n = intrinsic_name(e.name);
+      if (n == "global_thread_id" || n == "global_idx" || n == "global_idx_x") {
+        p[{"@block_dim_x", "@block_idx_x"}] = 1u;
+        p[{"@thread_idx_x"}] = 1u;
+        return p;
+      }
+    }
+    // a let variable that stands for an integer expression is expanded here, so that its terms join the sum
+    if (e.kind == Expr::VarRef) {
+      auto it = subst_int.find(key(e.var));
+      if (it != subst_int.end()) return it->second;
+    }
+    p[{expr(ep)}] = 1u;
+    return p;
+  }
+
+  static std::string render(const Poly &p) {
+    std::string o = "(poly";
+    int shown = 0;
+    std::string only;
+    for (auto &t : p) {
+      if (t.second == 0) continue;
+      ++shown;
+      std::string term = std::to_string(static_cast<int32_t>(t.second));
+      for (auto &a : t.first) term += "*" + a;
+      if (t.second == 1 && t.first.size() == 1) only = t.first[0];
+      o += " " + term;
+    }
+    if (shown == 0) return "i32:0";
+    if (shown == 1 && !only.empty()) return only;          // a bare atom stays itself
+    if (shown == 1 && p.count({}) && p.at({}) != 0) return "i32:" + std::to_string(static_cast<int32_t>(p.at({})));
+    return o + ")";
+  }
+
+  std::map<std::string, Poly> subst_int;       // immutable int32 let variables -> their value as a polynomial
+
   std::string expr(const ExprP &ep) {
     const Expr &e = *ep;
     char buf[64];
+    if (e.kind == Expr::BinopE && (e.binop == Binop::Add || e.binop == Binop::Sub || e.binop == Binop::Mul) &&
+        is_int32(ep))
+      return render(poly(ep));
+    if (e.kind == Expr::UnopE && e.unop == Unop::Neg && is_int32(ep)) return render(poly(ep));
     switch (e.kind) {
       case Expr::ConstInt32: return "i32:" + std::to_string(e.ival);
       case Expr::ConstInt64: return "i64:" + std::to_string(e.ival);
@@ -94,6 +213,8 @@ struct Canon {
       case Expr::ConstBool: return e.ival ? "true" : "false";
       case Expr::ConstUnit: return "unit";
       case Expr::VarRef: {
+        auto si = subst_int.find(key(e.var));
+        if (si != subst_int.end()) return render(si->second);
         auto s = subst.find(key(e.var));
         if (s != subst.end()) return expr(s->second);
         auto r = rename.find(key(e.var));
@@ -124,11 +245,8 @@ struct Canon {
       case Expr::Intrinsic: {
         if (!e.name.empty() && e.name[0] == '\x01') return e.name.substr(1);  // pre-rendered let value
         const std::string n = intrinsic_name(e.name);
-        if (e.args.empty() && (n == "global_thread_id" || n == "global_idx" || n == "global_idx_x")) {
-          std::string a = "(mul @block_dim_x @block_idx_x)", b = "@thread_idx_x";
-          if (b < a) std::swap(a, b);
-          return "(add " + a + " " + b + ")";
-        }
+        if (e.args.empty() && (n == "global_thread_id" || n == "global_idx" || n == "global_idx_x"))
+          return render(poly(ep));       // thread_idx_x + block_dim_x * block_idx_x
         std::string o = "@" + n;
         if (!e.args.empty()) {
           o = "(" + o;
@@ -308,10 +426,14 @@ struct Canon {
           // substitute the value, rendered now so that it is closed over the bindings
           // in force at this point; carried in an Intrinsic node whose name starts
           // with \x01 (no real intrinsic can)
-          auto closed = std::make_shared<Expr>();
-          closed->kind = Expr::Intrinsic;
-          closed->name = "\x01" + expr(s.e);
-          subst[key(s.var)] = closed;
+          if (s.var.type && s.var.type->kind == Type::Int32 && is_int32(s.e)) {
+            subst_int[key(s.var)] = poly(s.e);
+          } else {
+            auto closed = std::make_shared<Expr>();
+            closed->kind = Expr::Intrinsic;
+            closed->name = "\x01" + expr(s.e);
+            subst[key(s.var)] = closed;
+          }
         }
         stmt(s.stmts[0], out);
         return;
@@ -682,7 +804,12 @@ std::string recognise(const Kernel &k) {
   static const std::string t_hist = strip_trailing_barrier(canon_kernel(parse_kernel(kHistogram)));
   static const std::string t_radix_hist = strip_trailing_barrier(canon_kernel(parse_kernel(kRadixHistogram)));
   static const std::string t_radix_scatter = canon_kernel(parse_kernel(kRadixScatter));
-  const std::string c = canon_kernel(k);
+  std::string c;
+  try {
+    c = canon_kernel(k);
+  } catch (const std::exception &) {
+    return "";                          // nothing a hand kernel serves is that large: plain lowering
+  }
   if (c == t_radix_scatter) return "radix_scatter_i32";
   if (c == t_matmul) return "matmul_tiled_f32";
   if (c == t_triad) return "stream_triad_f32";

@@ -437,3 +437,51 @@ def test_a_binding_that_reads_what_its_scope_changes_is_not_inlined(hip):
     # the same binding with nothing stored to b in its scope is the triad
     plain = saved.replace("(assign (lelem b (var tid 6 i32)) (f32 0.0)) ", "")
     assert split_tag(hip.generate_source(plain))[0] == "stream_triad_f32"
+
+
+def test_recognition_does_not_depend_on_how_index_arithmetic_is_written(hip):
+    """int32 +, -, * form a ring: bracketing, operand order, distribution and named or folded constants do not
+    change an index, so they must not change what a kernel is recognised as.  (No IR printed by the reference's
+    own front end is at hand: the fixtures were derived from its lowering rules, so the recogniser has to take
+    every spelling of the same arithmetic.)"""
+    mm = open(os.path.join(IR_DIR, "matrix_mul_tiled.ir")).read()
+    tag = lambda ir: split_tag(hip.generate_source(ir))[0]                     # noqa: E731
+    assert tag(mm) == "matmul_tiled_f32"
+    ts = "(var tile_size 13 i32)"
+    # the tile size written as a literal everywhere
+    literal = mm.replace(ts, "(i32 16)").replace("(let (i32 16) (i32 16)", f"(let {ts} (i32 16)")
+    assert literal.count(ts) == 1 and tag(literal) == "matmul_tiled_f32"
+    # ceil(k / 16) with the constants folded, or bracketed the other way
+    folded = mm.replace(f"(div (sub (add (var k 6 i32) {ts}) (i32 1)) {ts})", "(div (add (var k 6 i32) (i32 15)) (i32 16))")
+    assert folded != mm and tag(folded) == "matmul_tiled_f32"
+    other = mm.replace(f"(sub (add (var k 6 i32) {ts}) (i32 1))", f"(add (var k 6 i32) (sub {ts} (i32 1)))")
+    assert other != mm and tag(other) == "matmul_tiled_f32"
+    # operands the other way round, a product distributed
+    swapped = mm.replace(f"(add (mul (var t 16 i32 mut) {ts}) (var tx 9 i32))", f"(add (var tx 9 i32) (mul {ts} (var t 16 i32 mut)))")
+    assert swapped != mm and tag(swapped) == "matmul_tiled_f32"
+    rowcol = mm.replace("(add (var ty 10 i32) (mul (intr (Gpu) block_dim_y) (intr (Gpu) block_idx_y)))",
+                        "(add (mul (intr (Gpu) block_idx_y) (intr (Gpu) block_dim_y)) (var ty 10 i32))")
+    assert rowcol != mm and tag(rowcol) == "matmul_tiled_f32"
+    # the loop bound as num_tiles + (-1)
+    bound = mm.replace("(sub (var num_tiles 14 i32) (i32 1))", "(add (var num_tiles 14 i32) (i32 -1))")
+    assert bound != mm and tag(bound) == "matmul_tiled_f32"
+    # ... and what is NOT the same arithmetic stays out
+    assert tag(mm.replace(f"(div (sub (add (var k 6 i32) {ts}) (i32 1)) {ts})", f"(div (add (var k 6 i32) {ts}) {ts})")) == ""
+    assert tag(mm.replace(f"(add (mul (var t 16 i32 mut) {ts}) (var tx 9 i32))", f"(add (mul (var t 16 i32 mut) {ts}) (var ty 10 i32))", 1)) == ""
+    assert tag(mm.replace("(sub (var num_tiles 14 i32) (i32 1))", "(var num_tiles 14 i32)")) == ""
+    # f32 arithmetic is not a ring: (b + c*s) re-bracketed with an extra term is another value
+    assert tag(triad_ir(f"(add (add {B} (mul {Cc} {S})) (f32 0.0))")) == ""
+
+    # thread index spelled out instead of the global_thread_id intrinsic, in either order
+    tri = open(os.path.join(IR_DIR, "stream_triad.ir")).read()
+    assert tag(tri) == "stream_triad_f32"
+    spelled = tri.replace("(intr (Std) global_thread_id)",
+                          "(add (mul (intr (Gpu) block_idx_x) (intr (Gpu) block_dim_x)) (intr (Gpu) thread_idx_x))")
+    assert spelled != tri and tag(spelled) == "stream_triad_f32"
+    red = open(os.path.join(IR_DIR, "reduction.ir")).read()
+    short = red.replace("(add (intr (Gpu) thread_idx_x) (mul (intr (Gpu) block_dim_x) (intr (Gpu) block_idx_x)))",
+                        "(intr (Std) global_thread_id)")
+    assert short != red and tag(short) == "reduce_sum_block256_f32"
+    # the tree's partner index tid + 64 written as 64 + tid
+    assert tag(red.replace("(add (var tid 5 i32) (i32 64))", "(add (i32 64) (var tid 5 i32))")) == "reduce_sum_block256_f32"
+    assert tag(red.replace("(add (var tid 5 i32) (i32 64))", "(add (i32 63) (var tid 5 i32))")) == ""
