@@ -326,9 +326,10 @@ int sarek_hip_radix_scatter_i32(int32_t *out, int64_t out_len, int32_t *counters
   if (n == 0) return SAREK_HIP_OK;
   hipStream_t st = as_stream(stream);
   // Measured on MI355X: 16384-key tiles from about 4M keys on (half the global atomics of 8192-key tiles:
-  // 95 against 142 us at 50M keys), 8192-key tiles below (more workgroups than CUs sooner).
+  // 95 against 142 us at 50M keys), 8192-key tiles below (more workgroups than CUs sooner), 32768-key tiles
+  // from 2^27 keys on (573 against 648 us at 2^28 keys; 111 against 100 us at 50M).
   int64_t shape = tunable("radix_scatter.tile", 0);
-  if (shape == 0) shape = n >= (int64_t{1} << 22) ? 2 : 1;
+  if (shape == 0) shape = n >= (int64_t{1} << 27) ? 4 : n >= (int64_t{1} << 22) ? 2 : 1;
   switch (shape) {
     case 1: return launch_scatter<512, 16>(out, out_len, counters, keys, n, shift, mask, st);
     case 2: return launch_scatter<1024, 16>(out, out_len, counters, keys, n, shift, mask, st);

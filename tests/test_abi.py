@@ -190,3 +190,38 @@ def test_device_report_never_needs_a_gpu(hip):
     small = ctypes.create_string_buffer(8)
     assert hip.lib.sarek_hip_device_report(small, 8, ctypes.byref(need), None) == hip.E_BUFFER_TOO_SMALL
     assert need.value == len(text.encode()) + 1
+
+
+def test_library_kernel_texts_need_no_gpu(hip):
+    """The texts a caller hands to Execute.run_source: complete HIP sources, tag first, found by name."""
+    names = hip.library_kernel_names()
+    assert names == ["gemm_bf16", "gemm_f16", "gemm_f16_bias_relu_rowsum", "triad_sum_f32"]
+    for name in names:
+        src, entry = hip.library_kernel(name)
+        assert src.splitlines()[0] == "// sarek-hip-specialise: " + name
+        assert f'extern "C" __global__ void {entry}(' in src and "Launch:" in src
+        assert src.count("{") == src.count("}")
+    need = ctypes.c_size_t(0)
+    small = ctypes.create_string_buffer(16)
+    assert hip.lib.sarek_hip_library_kernel_source(b"gemm_bf16", small, 16, ctypes.byref(need), None, 0) == hip.E_BUFFER_TOO_SMALL
+    assert need.value > 200
+    assert hip.lib.sarek_hip_library_kernel_source(b"no_such_kernel", None, 0, None, None, 0) == hip.E_INVALID_ARG
+    assert b"no_such_kernel" in hip.lib.sarek_hip_last_error()
+    assert hip.lib.sarek_hip_library_kernel_source(None, None, 0, None, None, 0) == hip.E_INVALID_ARG
+
+
+def test_sequence_entry_points_validate_before_touching_a_device(hip):
+    made, done = ctypes.c_int(7), ctypes.c_int(7)
+    assert hip.lib.sarek_hip_run_sources(None, 0, ctypes.byref(made), ctypes.byref(done)) == 0
+    assert (made.value, done.value) == (0, 0) and hip.lib.sarek_hip_last_run_path() == b"none"
+    assert hip.lib.sarek_hip_run_sources(None, 2, None, None) == hip.E_INVALID_ARG
+    assert hip.lib.sarek_hip_run_sources(None, -1, None, None) == hip.E_INVALID_ARG
+    assert hip.lib.sarek_hip_execute_run_pipeline(None, 1, None) == hip.E_INVALID_ARG
+    stage = (hip.PipelineStage * 1)()
+    assert hip.lib.sarek_hip_execute_run_pipeline(stage, 1, None) == hip.E_INVALID_ARG      # NULL IR text
+    assert b"stage 0" in hip.lib.sarek_hip_last_error()
+    x = ctypes.c_double(0)
+    assert hip.lib.sarek_hip_triad_block256_sum_f32(None, None, None, 3.0, -1, None, None) == hip.E_INVALID_ARG
+    assert hip.lib.sarek_hip_triad_block256_sum_f32(None, None, None, 3.0, 0, None, None) == 0
+    assert hip.lib.sarek_hip_triad_sum_f32_static(None, None, None, 3.0, 8, ctypes.byref(x), None) == hip.E_INVALID_ARG
+    assert hip.lib.sarek_hip_triad_sum_f32_static(None, None, None, 3.0, (1 << 31) + 1, ctypes.byref(x), None) == hip.E_INVALID_ARG
