@@ -55,10 +55,11 @@ def parse():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--workload", default="gemm_bf16_8192",
                     choices=["gemm_bf16_8192", "gemm_f16_8192", "triad_sum_2p28", "gemm_f32_8192", "gemm_f32_1024",
-                             "gemm_f16_epilogue", "gemm_f16_4095x11008x4096", "copy_1gib", "vendor_gemm_bf16_8192", "histogram_2p28",
+                             "gemm_f16_epilogue", "gemm_f16_4095x11008x4096", "gemm_f16_shape", "copy_1gib", "vendor_gemm_bf16_8192", "histogram_2p28",
                              "radix_scatter_5e7"])
     ap.add_argument("--no-also", action="store_true", help="measure only the headline workload")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--shape", default="4096,11264,4096", metavar="M,N,K", help="shape of the gemm_f16_shape workload")
     ap.add_argument("--zero-operands", action="store_true",
                     help="16-bit GEMM workloads: all-zero A and B (what the kernel does when the data costs no power)")
     ap.add_argument("--tunable", action="append", default=[], metavar="NAME=VALUE",
@@ -114,6 +115,7 @@ def dims(*d):
 
 
 ZERO_OPERANDS = False
+GEMM_SHAPE = (4096, 11264, 4096)
 
 
 def make_workload(name, torch, hip):
@@ -273,9 +275,9 @@ def make_workload(name, torch, hip):
                     config={"workload": "out[counters[key & 255]++] = key, random keys below 100000", "n": n,
                             "algorithmic_bytes": 8 * n})
         return main, None, info, (vk, vo, vcnt, starts, a, ir)
-    if name == "gemm_f16_4095x11008x4096":
-        # the epilogue config's product without the epilogue: what the fused chain costs on top
-        m, n, k = 4095, 11008, 4096
+    if name in ("gemm_f16_4095x11008x4096", "gemm_f16_shape"):
+        # the epilogue config's product without the epilogue (what the fused chain costs on top), or any --shape
+        m, n, k = (4095, 11008, 4096) if name != "gemm_f16_shape" else GEMM_SHAPE
         g.manual_seed(0xA5)
         t = (torch.randn(m, k, device="cuda", generator=g) * 0.02).half()
         va = device_vector(sarek, hip, torch, t, elem_size=2)
@@ -290,7 +292,7 @@ def make_workload(name, torch, hip):
         src_b, entry_b = src.encode(), entry.encode()
         main = Launch(hip, lib.sarek_hip_execute_run_source, src_b, hip.LANG_HIP, entry_b, dims(16, 16, 1),
                       dims((n + 15) // 16, (m + 15) // 16, 1), 0, 1, a, na)
-        info = dict(metric="fp16 GEMM TFLOP/s at the epilogue config's shape", unit="TFLOP/s", dtype="f16",
+        info = dict(metric=f"fp16 GEMM TFLOP/s at {m}x{n}x{k}", unit="TFLOP/s", dtype="f16",
                     work=2.0 * m * n * k, work_unit=1e12, bound="mfma",
                     peak=PEAK_MFMA_TFLOPS["f16"], kernel="gemm16_dma_kernel<f16, store, 64, 32, 2, 4, 2>",
                     route="Execute.run_source ~lang:HIP_Source, library kernel text 'gemm_f16'",
@@ -528,8 +530,9 @@ def main():
         print("bench.py needs a GPU", file=sys.stderr)
         sys.exit(2)
     torch.cuda.set_device(0)
-    global ZERO_OPERANDS
+    global ZERO_OPERANDS, GEMM_SHAPE
     ZERO_OPERANDS = args.zero_operands
+    GEMM_SHAPE = tuple(int(x) for x in args.shape.split(","))
     for item in args.tunable:
         name, _, value = item.partition("=")
         hip.check(hip.lib.sarek_hip_set_tunable(name.encode(), int(value)))
