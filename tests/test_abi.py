@@ -225,3 +225,11 @@ def test_sequence_entry_points_validate_before_touching_a_device(hip):
     assert hip.lib.sarek_hip_triad_block256_sum_f32(None, None, None, 3.0, 0, None, None) == 0
     assert hip.lib.sarek_hip_triad_sum_f32_static(None, None, None, 3.0, 8, ctypes.byref(x), None) == hip.E_INVALID_ARG
     assert hip.lib.sarek_hip_triad_sum_f32_static(None, None, None, 3.0, (1 << 31) + 1, ctypes.byref(x), None) == hip.E_INVALID_ARG
+
+
+def test_bench_refuses_more_than_one_gpu_without_touching_one():
+    """bench.py measures one GPU; asked for more it says so and exits before it loads anything."""
+    import subprocess
+    import sys
+    run = subprocess.run([sys.executable, os.path.join(ROOT, "bench.py"), "--gpus", "2"], capture_output=True, text=True)
+    assert run.returncode == 2 and "one GPU" in run.stderr and run.stdout == ""
