@@ -252,7 +252,9 @@ int sarek_hip_run_source(const char *source, int lang, const char *kernel_name,
  * sarek/sarek/Execute.ml:613-651, as sarek/tests/e2e/test_external_kernel.ml:46-62 does with its
  * own text) with lengths injected; with specialisation on and arguments that fit, the hand-written
  * kernel runs, otherwise the text itself is compiled and gives the same result under the launch
- * geometry stated in its comment.  Names, arguments (v = device pointer + int32 length) and geometry:
+ * geometry stated in its comment.  The hand-written kernel stands in for the library's own text only (compared
+ * byte for byte): a caller's text that merely starts with the same tag line is compiled as written.
+ * Names, arguments (v = device pointer + int32 length) and geometry:
  *   gemm_bf16, gemm_f16          (a v, b v, c v, m, n, k)   a, b: 2-byte custom elements (bit patterns),
  *                                c f32; 2-D launch, one thread per element of C
  *   gemm_f16_bias_relu_rowsum    (a v, b v, bias v, y v, rowsum v, m, n, k)   1-D launch, any size

@@ -15,6 +15,7 @@
 #include <string>
 
 #include "common.hpp"
+#include "plugin.hpp"
 
 namespace sarek_hip {
 namespace {
@@ -119,6 +120,19 @@ int copy_out(const std::string &text, char *out, size_t cap, size_t *needed, con
 }
 
 }  // namespace
+
+// Whether `source` is, byte for byte, the library's text of that name: only then does a hand-written
+// kernel stand in for it (a caller's own text that merely starts with the same tag line is compiled).
+bool is_library_kernel_text(const std::string &name, const char *source) {
+  for (const LibraryKernel &k : kKernels)
+    if (name == k.name) return std::strcmp(k.source, source) == 0;
+  return false;
+}
+bool is_library_kernel_name(const std::string &name) {
+  for (const LibraryKernel &k : kKernels)
+    if (name == k.name) return true;
+  return false;
+}
 }  // namespace sarek_hip
 
 using namespace sarek_hip;

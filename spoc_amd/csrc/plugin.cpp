@@ -457,6 +457,8 @@ int sarek_hip_run_source(const char *source, int lang, const char *kernel_name, 
 
   if (specialisation_enabled()) {
     std::string tag = read_tag(source);
+    // a library kernel's tag counts only on the library's own text
+    if (!tag.empty() && is_library_kernel_name(tag) && !is_library_kernel_text(tag, source)) tag.clear();
     if (!tag.empty()) {
       int rc = SAREK_HIP_OK;
       if (try_specialised(tag, block, grid, args, n_args, &rc)) {

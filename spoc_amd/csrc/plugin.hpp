@@ -1,7 +1,12 @@
 // Internal declarations shared by the plugin-level sources.
 #pragma once
+#include <string>
 namespace sarek_hip {
 // First line of a generated source that a hand-written kernel can serve:
 // "// sarek-hip-specialise: <tag>".
 extern const char *const kSpecialiseMarker;
+
+// library_kernels.cpp: the texts sarek_hip_library_kernel_source hands out
+bool is_library_kernel_name(const std::string &name);
+bool is_library_kernel_text(const std::string &name, const char *source);
 }  // namespace sarek_hip

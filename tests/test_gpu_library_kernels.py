@@ -121,6 +121,28 @@ def test_gemm16_run_source_geometry_that_does_not_cover_c_is_left_to_the_text(hi
                           [a16, b16, c32, ("i32", m), ("i32", n), ("i32", k)]) == "jit"
 
 
+def test_a_library_tag_on_somebody_elses_text_is_not_honoured(hip, oracle, sarek):
+    """The hand kernel stands in for the library's own text only: a text that merely starts with the same tag
+    line is compiled and run as it is written."""
+    E, V = sarek.Execute, sarek.Vector
+    m = n = k = 32
+    mine = ("// sarek-hip-specialise: gemm_bf16\n"
+            'extern "C" __global__ void sarek_gemm_bf16(const unsigned short* a, int a_len, const unsigned short* b, '
+            "int b_len, float* c, int c_len, int m, int n, int k) {\n"
+            "  int col = threadIdx.x + blockIdx.x * blockDim.x, row = threadIdx.y + blockIdx.y * blockDim.y;\n"
+            "  if (row < m && col < n) c[row * n + col] = 42.0f;\n}\n")
+    va, vb = custom16(sarek, np.zeros(m * k, np.uint16)), custom16(sarek, np.zeros(k * n, np.uint16))
+    vc = V.create(V.float32, m * n)
+    path = E.run_source(mine, "sarek_gemm_bf16", (16, 16, 1), (2, 2, 1),
+                        [E.Vec(va), E.Vec(vb), E.Vec(vc), E.Int32(m), E.Int32(n), E.Int32(k)])
+    assert path == "jit" and np.all(vc.to_array() == 42.0)
+    # the library's text with trailing whitespace added is no longer the library's text either
+    src, entry = E.library_kernel("gemm_bf16")
+    assert E.run_source(src + "\n", entry, (16, 16, 1), (2, 2, 1),
+                        [E.Vec(va), E.Vec(vb), E.Vec(vc), E.Int32(m), E.Int32(n), E.Int32(k)]) == "jit"
+    assert np.all(vc.to_array() == 0.0)
+
+
 @pytest.mark.parametrize("m,n,k", [(127, 264, 128), (300, 136, 200), (4095 // 8, 1376, 512)])
 def test_epilogue_through_run_source(hip, oracle, sarek, m, n, k):
     E, V = sarek.Execute, sarek.Vector
