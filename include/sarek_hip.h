@@ -240,8 +240,13 @@ int sarek_hip_generate_source(const char *ir_text, const int block[3], char *out
 /* Compile (cached) + bind + launch on the default stream.  Only
  * SAREK_HIP_LANG_HIP_SOURCE and SAREK_HIP_LANG_CUDA_SOURCE (treated as HIP
  * text) are accepted; others return SAREK_HIP_E_UNSUPPORTED.  A specialise
- * tag in the source reroutes the call to the matching hand-written kernel
- * below, ignoring block/grid.                                              */
+ * tag reroutes the call to the matching hand-written kernel when (1) the text
+ * is one this library wrote -- byte for byte a text sarek_hip_generate_source
+ * returned in this process, or a library kernel's text -- and (2) block, grid
+ * and the arguments fit what that kernel assumes (the launch covers the
+ * problem, output buffers do not lie over inputs).  Anything else, a caller's
+ * own program that starts with the same line included, is compiled and
+ * launched as written.                                                      */
 int sarek_hip_run_source(const char *source, int lang, const char *kernel_name,
                          const int block[3], const int grid[3], int shared_mem_bytes,
                          const sarek_hip_arg *args, int n_args);

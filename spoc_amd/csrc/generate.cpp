@@ -2,21 +2,44 @@
 // the kernel is one a hand-written CDNA4 kernel computes (Hip_plugin.generate_source;
 // the reference's counterpart is sarek-cuda/Cuda_plugin.ml:155-157).
 #include <cstring>
+#include <mutex>
 #include <string>
+#include <string_view>
+#include <unordered_set>
 
 #include "common.hpp"
 #include "host/ir.hpp"
 #include "plugin.hpp"
+
+namespace sarek_hip {
+namespace {
+// Every tagged text this process has handed out.  The recogniser matched the whole IR body before it wrote
+// the tag, so exactly these texts may be served by a hand-written kernel; any other text that starts with
+// the same line is somebody else's program.
+struct ViewHash {
+  using is_transparent = void;
+  size_t operator()(std::string_view v) const { return std::hash<std::string_view>{}(v); }
+};
+std::mutex g_tagged_mu;
+std::unordered_set<std::string, ViewHash, std::equal_to<>> g_tagged;
+constexpr size_t kTaggedMax = 4096;     // beyond this the set starts over: forgotten texts run as compiled
+}  // namespace
+
+bool is_generated_tagged_text(const char *source) {
+  std::lock_guard<std::mutex> lock(g_tagged_mu);
+  return g_tagged.find(std::string_view(source)) != g_tagged.end();
+}
+}  // namespace sarek_hip
 
 using namespace sarek_hip;
 
 extern "C" int sarek_hip_generate_source(const char *ir_text, const int block[3], char *out,
                                          size_t out_len, size_t *needed) {
   if (!ir_text) return fail(SAREK_HIP_E_INVALID_ARG, "generate_source: NULL IR text");
-  std::string src;
+  std::string src, tag;
   try {
     ir::Kernel k = ir::parse_kernel(ir_text);
-    std::string tag = ir::recognise(k);
+    tag = ir::recognise(k);
     if (!tag.empty()) src = std::string(kSpecialiseMarker) + tag + "\n";
     src += ir::generate(k, block);
   } catch (const ir::ParseError &e) {
@@ -30,5 +53,10 @@ extern "C" int sarek_hip_generate_source(const char *ir_text, const int block[3]
   if (!out || out_len < src.size() + 1)
     return fail(SAREK_HIP_E_BUFFER_TOO_SMALL, "generate_source: output needs %zu bytes", src.size() + 1);
   std::memcpy(out, src.c_str(), src.size() + 1);
+  if (!tag.empty()) {
+    std::lock_guard<std::mutex> lock(g_tagged_mu);
+    if (g_tagged.size() >= kTaggedMax) g_tagged.clear();
+    g_tagged.insert(std::move(src));
+  }
   return SAREK_HIP_OK;
 }

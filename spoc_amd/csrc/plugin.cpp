@@ -40,6 +40,14 @@ std::string read_tag(const char *source) {
   return std::string(p, e);
 }
 
+// A tag counts only on a text this library wrote: a library kernel's own text, or a text that
+// generate_source produced here after the recogniser matched its IR.  A caller's program that merely
+// starts with the same line is compiled and run as written.
+bool tag_is_ours(const std::string &tag, const char *source) {
+  if (is_library_kernel_name(tag)) return is_library_kernel_text(tag, source);
+  return is_generated_tagged_text(source);
+}
+
 bool is_buf(const sarek_hip_arg &a) { return a.kind == SAREK_HIP_ARG_BUFFER; }
 bool is_i32(const sarek_hip_arg &a) { return a.kind == SAREK_HIP_ARG_INT32; }
 bool is_f32(const sarek_hip_arg &a) { return a.kind == SAREK_HIP_ARG_FLOAT32; }
@@ -405,7 +413,7 @@ int sarek_hip_run_sources(const sarek_hip_launch *launches, int n_launches, int 
                             (l1.lang == SAREK_HIP_LANG_HIP_SOURCE || l1.lang == SAREK_HIP_LANG_CUDA_SOURCE);
       const std::string tag0 = read_tag(l0.source), tag1 = read_tag(l1.source);
       int rc = SAREK_HIP_OK;
-      if (langs_ok && !tag0.empty() && !tag1.empty() &&
+      if (langs_ok && !tag0.empty() && !tag1.empty() && tag_is_ours(tag0, l0.source) && tag_is_ours(tag1, l1.source) &&
           try_specialised_pair(tag0, l0.block, l0.grid, l0.args, l0.n_args, tag1, l1.block, l1.grid, l1.args,
                                l1.n_args, &rc)) {
         if (rc != SAREK_HIP_OK) return rc;
@@ -457,8 +465,7 @@ int sarek_hip_run_source(const char *source, int lang, const char *kernel_name, 
 
   if (specialisation_enabled()) {
     std::string tag = read_tag(source);
-    // a library kernel's tag counts only on the library's own text
-    if (!tag.empty() && is_library_kernel_name(tag) && !is_library_kernel_text(tag, source)) tag.clear();
+    if (!tag.empty() && !tag_is_ours(tag, source)) tag.clear();
     if (!tag.empty()) {
       int rc = SAREK_HIP_OK;
       if (try_specialised(tag, block, grid, args, n_args, &rc)) {

@@ -6,6 +6,9 @@ namespace sarek_hip {
 // "// sarek-hip-specialise: <tag>".
 extern const char *const kSpecialiseMarker;
 
+// generate.cpp: whether sarek_hip_generate_source handed out exactly this tagged text in this process
+bool is_generated_tagged_text(const char *source);
+
 // library_kernels.cpp: the texts sarek_hip_library_kernel_source hands out
 bool is_library_kernel_name(const std::string &name);
 bool is_library_kernel_text(const std::string &name, const char *source);

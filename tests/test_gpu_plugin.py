@@ -150,8 +150,14 @@ def test_specialise_tag_routes_to_hand_kernel(hip, oracle, torch_cuda):
     c = oracle.fill_uniform(n, seed=0xC)
     db, dc = torch.from_numpy(b).cuda(), torch.from_numpy(c).cuda()
     a = torch.zeros(n, device="cuda")
-    tagged = "// sarek-hip-specialise: stream_triad_f32\n" + TRIAD_GENERATED
+    # a tag counts on a text generate_source handed out, not on the same line pasted in front of a program
+    # (a byte-identical copy of a generated text IS that text, so this one differs by a comment)
+    pasted = "// sarek-hip-specialise: stream_triad_f32\n// pasted\n" + TRIAD_GENERATED
     items = [a, db, dc, ("f32", 3.0), ("i32", n)]
+    assert hip.run_source(pasted, "sarek_kern", (256, 1, 1), ((n + 255) // 256, 1, 1), items) == "jit"
+    a.zero_()
+    tagged = hip.generate_source(load_ir("stream_triad"), block=(256, 1, 1))
+    assert tagged.startswith("// sarek-hip-specialise: stream_triad_f32\n")
     path = hip.run_source(tagged, "sarek_kern", (256, 1, 1), ((n + 255) // 256, 1, 1), items)
     torch.cuda.synchronize()
     assert path == "stream_triad_f32"
