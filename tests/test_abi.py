@@ -163,20 +163,15 @@ def header_device_info_fields():
     return fields
 
 
-def test_device_info_layout_agrees_between_header_python_and_documented_ocaml_stub(hip):
-    """sarek_hip_device_get_info fills the whole struct: the Python binding and the OCaml ctypes stub a
-    maintainer copies out of the integration notes must declare every member, in the header's order."""
+def test_device_info_layout_agrees_between_header_and_python(hip):
+    """sarek_hip_device_get_info fills the whole struct: the Python binding must declare every member, in the
+    header's order."""
     fields = header_device_info_fields()
     assert [f[0] for f in fields][-1] == "max_registers_per_block"
     assert [name for name, _ in hip.DeviceInfo._fields_] == [f[0] for f in fields]
     assert hip.lib.sarek_hip_device_info_size() == ctypes.sizeof(hip.DeviceInfo)
 
-    doc = open(os.path.join(ROOT, "INTEGRATION.md")).read()
-    stub = re.findall(r'field device_info "(\w+)" (\(array (\d+) (\w+)\)|\w+)', doc)
-    ocaml = {"char": "char", "uint64_t": "uint64_t", "int": "int"}
-    assert [(s[0], ocaml[s[3] or s[1]], int(s[2]) if s[2] else None) for s in stub] == fields
-    assert doc.index("max_registers_per_block\" int") < doc.index("seal device_info")
-    assert "sarek_hip_device_info_size" in doc
+    # the OCaml stub's member list is checked against the same header in tests/test_ocaml_veneer.py
 
 
 def test_device_report_never_needs_a_gpu(hip):
