@@ -200,8 +200,9 @@ constexpr int lcm_int(int a, int b) {
 
 // Ablate (measurement only, results are wrong by construction; tunable gemm16.ablate): bit 0 leaves the
 // global -> LDS transfers out of the K loop (the ring keeps what the prologue put there), bit 1 the LDS
-// fragment reads (every MFMA reuses the first fragments).  What remains shows what each part of the loop
-// costs in cycles and, under the package power limit, in clock.
+// fragment reads (every MFMA reuses the first fragments), bit 2 makes every workgroup fetch the panels of
+// tile (0, 0) (the same global -> LDS transfers, all served by the L2s: no traffic past them).  What remains
+// shows what each part of the loop costs in cycles and, under the package power limit, in clock.
 template <bool Bf16, int Epi, int BKA, int BKB, int NA, int NB, int TJ, int Ablate = 0>
 __global__ __launch_bounds__(64 * 2 * (8 / TJ)) void gemm16_dma_kernel(const uint16_t *__restrict__ A,
                                                              const uint16_t *__restrict__ B,
@@ -235,6 +236,7 @@ __global__ __launch_bounds__(64 * 2 * (8 / TJ)) void gemm16_dma_kernel(const uin
   int tm, tn;
   tile_of_block(tiles_m, tiles_n, xcd_remap, tm, tn);
   const int m0 = tm * BM, n0 = tn * BN;
+  const int m0_src = (Ablate & 4) ? 0 : m0, n0_src = (Ablate & 4) ? 0 : n0;
   long long probe_c0 = 0, probe_t0 = 0;
   if (probe) {
     probe_c0 = clock64();
@@ -266,7 +268,7 @@ __global__ __launch_bounds__(64 * 2 * (8 / TJ)) void gemm16_dma_kernel(const uin
   for (int i = 0; i < DA; ++i) {
     const int q = wave + NWAVES * i;
     const int arow_t = q * A_ROWS_PER_DMA + lane / A_CHUNKS;
-    const int arow = min(arow_t, M - 1 - m0);
+    const int arow = min(arow_t, M - 1 - m0_src);
     a_off[i] = (static_cast<uint32_t>(arow) * K + (((lane % A_CHUNKS) ^ a_swz(arow_t)) << 3)) * 2u;
   }
 #pragma unroll
@@ -274,10 +276,10 @@ __global__ __launch_bounds__(64 * 2 * (8 / TJ)) void gemm16_dma_kernel(const uin
     const int q = wave + NWAVES * i;
     const int brow = 2 * q + (lane >> 5);
     const int bchunk = (lane & 31) ^ ((brow & 3) << 2);
-    const int bcol = min(n0 + bchunk * 8, N - 8);
+    const int bcol = min(n0_src + bchunk * 8, N - 8);
     b_off[i] = (static_cast<uint32_t>(brow) * N + bcol) * 2u;
   }
-  const char *a_base = reinterpret_cast<const char *>(A + static_cast<int64_t>(m0) * K);
+  const char *a_base = reinterpret_cast<const char *>(A + static_cast<int64_t>(m0_src) * K);
   const char *b_base = reinterpret_cast<const char *>(B);
   const int64_t b_slab_bytes = static_cast<int64_t>(BKB) * N * 2;
   const int nslabs = K / BKB, nstages = K / BKA;
@@ -631,15 +633,16 @@ int launch_gemm16(const uint16_t *a, const uint16_t *b, float *c, const float *b
       const int ablate = (int)tunable("gemm16.ablate", 0);
       if (ablate != 0) {
         // measurement variants of the default shape (bf16, plain store); anything else is refused
-        if (!Bf16 || Epi != EPI_STORE || ring != 0 || tj != 2 || ablate < 1 || ablate > 3)
-          return fail(SAREK_HIP_E_UNSUPPORTED, "gemm16.ablate is for the default bf16 kernel only (1..3)");
+        if (!Bf16 || Epi != EPI_STORE || ring != 0 || tj != 2 || ablate < 1 || ablate > 4)
+          return fail(SAREK_HIP_E_UNSUPPORTED, "gemm16.ablate is for the default bf16 kernel only (1..4)");
         if constexpr (Bf16 && Epi == EPI_STORE) {
 #define SAREK_LAUNCH_ABLATED(AB)                                                                    \
   hipLaunchKernelGGL((gemm16_dma_kernel<true, EPI_STORE, 64, 32, 2, 4, 2, AB>), grid, dim3(512), 0, st, a, b, c, \
                      bias, rowsum, m, n, k, tiles_m, tiles_n, remap, probe)
           if (ablate == 1) SAREK_LAUNCH_ABLATED(1);
           else if (ablate == 2) SAREK_LAUNCH_ABLATED(2);
-          else SAREK_LAUNCH_ABLATED(3);
+          else if (ablate == 3) SAREK_LAUNCH_ABLATED(3);
+          else SAREK_LAUNCH_ABLATED(4);
 #undef SAREK_LAUNCH_ABLATED
         }
         return check_launch("gemm16 kernel launch");
