@@ -249,3 +249,23 @@ def test_plugin_implements_every_member_of_the_backend_signature():
             "clock_rate_khz", "multiprocessor_count", "is_cpu"]
     cap_body = re.search(r"let capabilities.*?\n      \}", base, flags=re.S).group(0)
     assert [c for c in caps if not re.search(r"\b" + c + r" =", cap_body)] == []
+
+
+def test_serialiser_prints_only_forms_the_native_reader_knows():
+    """Every form head and atom Sarek_ir_hip.ml can print ("(read", "(lelemx", "bitxor", "downto", ...) is a
+    literal of the reader (spoc_amd/csrc/host/ir_text.cpp), so the two cannot drift apart unnoticed."""
+    ml = open(os.path.join(OCAML, "Sarek_ir_hip.ml")).read()
+    reader = open(os.path.join(ROOT, "spoc_amd", "csrc", "host", "ir_text.cpp")).read()
+    heads = sorted(set(re.findall(r'"\((\w+)', ml)))
+    atoms = sorted(set(re.findall(r'-> "([a-z_0-9]+)"', ml)))
+    assert len(heads) >= 45 and len(atoms) >= 30
+    assert [w for w in heads + atoms if f'"{w}"' not in reader] == []
+    # one printer per IR type, one case per constructor of spoc/ir/Sarek_ir_types.ml
+    constructors = ["TInt32", "TInt64", "TFloat32", "TFloat64", "TBool", "TUnit", "TRecord", "TVariant", "TArray",
+                    "TVec", "CInt32", "CInt64", "CFloat32", "CFloat64", "CBool", "CUnit", "EConst", "EVar", "EBinop",
+                    "EUnop", "EArrayRead", "EArrayReadExpr", "ERecordField", "EIntrinsic", "ECast", "ETuple", "EApp",
+                    "ERecord", "EVariant", "EArrayLen", "EArrayCreate", "EIf", "EMatch", "LVar", "LArrayElem",
+                    "LArrayElemExpr", "LRecordField", "SAssign", "SSeq", "SIf", "SWhile", "SFor", "SMatch", "SReturn",
+                    "SBarrier", "SWarpBarrier", "SExpr", "SEmpty", "SLet", "SLetMut", "SPragma", "SMemFence", "SBlock",
+                    "SNative", "DParam", "DLocal", "DShared", "PConstr", "PWild"]
+    assert [c for c in constructors if not re.search(r"\b" + c + r"\b", ml)] == []
