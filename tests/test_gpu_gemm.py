@@ -184,6 +184,33 @@ def test_gemm_bf16_full_size_rows(hip, oracle, torch_cuda):
     assert torch.equal(hip.gemm_bf16(a * 2, b), c * 2)
 
 
+def test_measurement_variants_run_and_leave_the_kernel_as_it_was(hip, torch_cuda):
+    """gemm16.ablate (1..4) leaves parts of the K loop out for the power measurements: the results are wrong
+    by construction, but every variant runs within the operands' bounds, other kernels refuse the knob, and
+    with the knob back at 0 the result is the one from before."""
+    torch = torch_cuda
+    m, n, k = 512, 768, 512
+    torch.manual_seed(7)
+    a = (torch.randn(m, k, device="cuda") * 0.1).bfloat16()
+    b = (torch.randn(k, n, device="cuda") * 0.1).bfloat16()
+    good = hip.gemm_bf16(a, b)
+    try:
+        for v in (1, 2, 3, 4):
+            hip.set_tunable("gemm16.ablate", v)
+            c = hip.gemm_bf16(a, b)
+            torch.cuda.synchronize()
+            assert torch.isfinite(c).all()
+        with pytest.raises(hip.SarekHipError) as e:
+            hip.gemm_f16(a.half(), b.half())
+        assert e.value.status == hip.E_UNSUPPORTED
+        hip.set_tunable("gemm16.ablate", 5)
+        with pytest.raises(hip.SarekHipError):
+            hip.gemm_bf16(a, b)
+    finally:
+        hip.set_tunable("gemm16.ablate", 0)
+    assert torch.equal(hip.gemm_bf16(a, b), good)
+
+
 def test_gemm_rejects_bad_arguments(hip, torch_cuda):
     torch = torch_cuda
     a = torch.zeros(4, 4, device="cuda")
