@@ -337,6 +337,42 @@ def test_fused_pair_kernel_at_full_size_properties(hip, torch_cuda):
     assert total.item() == 1.75 * n
 
 
+@pytest.mark.parametrize("n", [1, 255, 1000, 4097, 65536 + 777, (1 << 20) + 3, 5_000_001])
+def test_fused_pair_block_sum_layouts_agree(hip, oracle, torch_cuda, n):
+    """The fused kernel's two layouts (a wave's four blocks neighbours, one 16-byte store; or a workgroup's width
+    apart, four 4-byte stores) and the two hand kernels launched one after the other leave the same bits; block
+    sums that do not start on 16 bytes take the second layout."""
+    torch = torch_cuda
+    b = torch.from_numpy(oracle.fill_uniform(n, seed=n)).cuda()
+    c = torch.from_numpy(oracle.fill_uniform(n, seed=n + 1)).cuda()
+    nb = (n + 255) // 256
+    try:
+        got = []
+        for runs in (1, 0):
+            hip.check(hip.lib.sarek_hip_set_tunable(b"triad.block_sum_runs", runs))
+            a, sums = hip.triad_block256_sum(b, c, 3.0)
+            torch.cuda.synchronize()
+            got.append((a.clone(), sums.clone()))
+    finally:
+        hip.check(hip.lib.sarek_hip_set_tunable(b"triad.block_sum_runs", 1))
+    assert torch.equal(got[0][0], got[1][0]) and torch.equal(got[0][1], got[1][1])
+    a_ref, p_ref, _ = oracle.triad_sum(b.cpu().numpy(), c.cpu().numpy(), 3.0)
+    assert np.array_equal(got[0][0].cpu().numpy(), a_ref)
+    assert np.abs(got[0][1].cpu().numpy() - p_ref).max() <= 1e-5 * np.abs(p_ref).max()
+    # the triad kernel, then the block-256 sum kernel on its output
+    a2 = hip.triad(b, c, 3.0)
+    s2 = torch.empty(nb, device="cuda")
+    hip.check(hip.lib.sarek_hip_reduce_sum_block256_f32(a2.data_ptr(), s2.data_ptr(), n, None))
+    # block sums that start 4 bytes into an allocation
+    pool = torch.full((nb + 1,), float("nan"), device="cuda")
+    a3 = torch.empty_like(b)
+    hip.check(hip.lib.sarek_hip_triad_block256_sum_f32(a3.data_ptr(), b.data_ptr(), c.data_ptr(), 3.0, n,
+                                                       pool.data_ptr() + 4, None))
+    torch.cuda.synchronize()
+    assert torch.equal(a2, got[0][0]) and torch.equal(s2, got[0][1])
+    assert torch.equal(a3, got[0][0]) and torch.equal(pool[1:], got[0][1]) and bool(torch.isnan(pool[0]))
+
+
 @pytest.mark.parametrize("count", [0, 1, 1000, (1 << 17) - 1, 1 << 17, (1 << 17) + 3, (1 << 20) + 77, 3_000_001])
 def test_fold_of_long_partial_vectors(hip, torch_cuda, count):
     """The device fold in one step (short) and in two (from 2^17 partials on) against a float64 sum."""
