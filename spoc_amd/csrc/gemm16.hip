@@ -93,7 +93,7 @@ __device__ __forceinline__ u32x2 lds_read_tr16(const char *lds, int off) {
 //      with the sums of rows q = 2*lm and 2*lm+1;
 //   3. across the WN waves that share the rows through `scratch` (LDS, WN x 256 floats; all
 //      waves must be done with the LDS ring: barriers inside), then one atomicAdd per row.
-template <int Epi, int TJ>
+template <int Epi, int TJ, bool NoStore = false>
 __device__ __forceinline__ void epilogue(f32x16 (&acc)[4][TJ], float *__restrict__ C,
                                          const float *__restrict__ bias,
                                          float *__restrict__ rowsum, int M, int N, int m0,
@@ -124,7 +124,8 @@ __device__ __forceinline__ void epilogue(f32x16 (&acc)[4][TJ], float *__restrict
           v = v > 0.f ? v : 0.f;
           sum += cok[j] ? v : 0.f;
         }
-        if (row < M && cok[j]) C[static_cast<int64_t>(row) * N + col0 + j * 32 + lm] = v;
+        // NoStore (measurement only): the compare keeps the values alive, nothing is written
+        if (row < M && cok[j] && (!NoStore || v == 1.2345e30f)) C[static_cast<int64_t>(row) * N + col0 + j * 32 + lm] = v;
       }
       rs[i * 16 + r] = sum;
     }
@@ -201,7 +202,8 @@ constexpr int lcm_int(int a, int b) {
 // Ablate (measurement only, results are wrong by construction; tunable gemm16.ablate): bit 0 leaves the
 // global -> LDS transfers out of the K loop (the ring keeps what the prologue put there), bit 1 the LDS
 // fragment reads (every MFMA reuses the first fragments), bit 2 makes every workgroup fetch the panels of
-// tile (0, 0) (the same global -> LDS transfers, all served by the L2s: no traffic past them).  What remains
+// tile (0, 0) (the same global -> LDS transfers, all served by the L2s: no traffic past them), bit 3 leaves the
+// stores of C out.  What remains
 // shows what each part of the loop costs in cycles and, under the package power limit, in clock.
 template <bool Bf16, int Epi, int BKA, int BKB, int NA, int NB, int TJ, int Ablate = 0>
 __global__ __launch_bounds__(64 * 2 * (8 / TJ)) void gemm16_dma_kernel(const uint16_t *__restrict__ A,
@@ -438,8 +440,8 @@ __global__ __launch_bounds__(64 * 2 * (8 / TJ)) void gemm16_dma_kernel(const uin
   }(std::make_integer_sequence<int, P - 1>{});
   // drain the (redundant) tail DMA before the LDS is released
   __builtin_amdgcn_s_waitcnt(waitcnt_vm_lgkm0(0));
-  epilogue<Epi, TJ>(acc, C, bias, rowsum, M, N, m0, wm, wn, n0 + wn * (32 * TJ), lm, lh,
-                    reinterpret_cast<float *>(lds_ring<10, A_BYTES_S>));
+  epilogue<Epi, TJ, (Ablate & 8) != 0>(acc, C, bias, rowsum, M, N, m0, wm, wn, n0 + wn * (32 * TJ), lm, lh,
+                                       reinterpret_cast<float *>(lds_ring<10, A_BYTES_S>));
   if (probe && tid == 0) {
     probe[2 * blockIdx.x] = static_cast<unsigned long long>(clock64() - probe_c0);
     probe[2 * blockIdx.x + 1] = static_cast<unsigned long long>(wall_clock64() - probe_t0);
@@ -633,8 +635,8 @@ int launch_gemm16(const uint16_t *a, const uint16_t *b, float *c, const float *b
       const int ablate = (int)tunable("gemm16.ablate", 0);
       if (ablate != 0) {
         // measurement variants of the default shape (bf16, plain store); anything else is refused
-        if (!Bf16 || Epi != EPI_STORE || ring != 0 || tj != 2 || ablate < 1 || ablate > 4)
-          return fail(SAREK_HIP_E_UNSUPPORTED, "gemm16.ablate is for the default bf16 kernel only (1..4)");
+        if (!Bf16 || Epi != EPI_STORE || ring != 0 || tj != 2 || ablate < 1 || (ablate > 4 && ablate != 8))
+          return fail(SAREK_HIP_E_UNSUPPORTED, "gemm16.ablate is for the default bf16 kernel only (1..4, 8)");
         if constexpr (Bf16 && Epi == EPI_STORE) {
 #define SAREK_LAUNCH_ABLATED(AB)                                                                    \
   hipLaunchKernelGGL((gemm16_dma_kernel<true, EPI_STORE, 64, 32, 2, 4, 2, AB>), grid, dim3(512), 0, st, a, b, c, \
@@ -642,6 +644,7 @@ int launch_gemm16(const uint16_t *a, const uint16_t *b, float *c, const float *b
           if (ablate == 1) SAREK_LAUNCH_ABLATED(1);
           else if (ablate == 2) SAREK_LAUNCH_ABLATED(2);
           else if (ablate == 3) SAREK_LAUNCH_ABLATED(3);
+          else if (ablate == 8) SAREK_LAUNCH_ABLATED(8);
           else SAREK_LAUNCH_ABLATED(4);
 #undef SAREK_LAUNCH_ABLATED
         }

@@ -185,9 +185,9 @@ def test_gemm_bf16_full_size_rows(hip, oracle, torch_cuda):
 
 
 def test_measurement_variants_run_and_leave_the_kernel_as_it_was(hip, torch_cuda):
-    """gemm16.ablate (1..4) leaves parts of the K loop out for the power measurements: the results are wrong
-    by construction, but every variant runs within the operands' bounds, other kernels refuse the knob, and
-    with the knob back at 0 the result is the one from before."""
+    """gemm16.ablate (1..4) leaves parts of the K loop out for the power measurements and 8 the stores of C: the
+    results are wrong by construction, but every variant runs within the operands' bounds, other kernels refuse
+    the knob, and with the knob back at 0 the result is the one from before."""
     torch = torch_cuda
     m, n, k = 512, 768, 512
     torch.manual_seed(7)
@@ -200,6 +200,11 @@ def test_measurement_variants_run_and_leave_the_kernel_as_it_was(hip, torch_cuda
             c = hip.gemm_bf16(a, b)
             torch.cuda.synchronize()
             assert torch.isfinite(c).all()
+        hip.set_tunable("gemm16.ablate", 8)
+        untouched = torch.full((m, n), 7.0, device="cuda")
+        hip.gemm_bf16(a, b, out=untouched)
+        torch.cuda.synchronize()
+        assert bool((untouched == 7.0).all())
         with pytest.raises(hip.SarekHipError) as e:
             hip.gemm_f16(a.half(), b.half())
         assert e.value.status == hip.E_UNSUPPORTED
