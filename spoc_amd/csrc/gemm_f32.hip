@@ -229,6 +229,13 @@ __global__ __launch_bounds__(64 * WMW * WNW) void gemm_f32_dma_kernel(
 #pragma unroll
       for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
 
+  // A wave with a single MFMA tile would feed every MFMA the result of the one before; it keeps a second
+  // accumulator for the odd MFMA steps instead (two independent chains), added to the first at the end.
+  constexpr bool kTwoChains = TI * TJ == 1;
+  f32x16 acc_odd;
+#pragma unroll
+  for (int r = 0; r < 16; ++r) acc_odd[r] = 0.f;
+
   const int a_row = wm * 32 * TI + lm;
   int a_addr0 = a_row * A_ROW + ((lh ^ a_swz(a_row)) << 4);           // ^ (kk << 5), + i*32*A_ROW
   int b_addr0 = (4 * lh) * B_ROW + (((wn * 32 * TJ + TJ * lm) * 4) ^ (TJ == 1 ? (lh << 7) : 0));
@@ -260,7 +267,10 @@ __global__ __launch_bounds__(64 * WMW * WNW) void gemm_f32_dma_kernel(
       for (int i = 0; i < TI; ++i)
 #pragma unroll
         for (int jn = 0; jn < TJ; ++jn) {
-          acc[i][jn] = __builtin_amdgcn_mfma_f32_32x32x2f32(af[i][j], bf[j][jn], acc[i][jn], 0, 0, 0);
+          if (kTwoChains && (j & 1))
+            acc_odd = __builtin_amdgcn_mfma_f32_32x32x2f32(af[i][j], bf[j][jn], acc_odd, 0, 0, 0);
+          else
+            acc[i][jn] = __builtin_amdgcn_mfma_f32_32x32x2f32(af[i][j], bf[j][jn], acc[i][jn], 0, 0, 0);
         }
   };
   // Issue order inside one k-step: behind each of the first MFMAs go the DMA instructions
@@ -340,6 +350,10 @@ __global__ __launch_bounds__(64 * WMW * WNW) void gemm_f32_dma_kernel(
     if (full + 2 < nslabs) ring_slab(I2{}, full + 2);
   }
   __builtin_amdgcn_s_waitcnt(waitcnt_vm_lgkm0(0));   // drain the redundant tail DMA
+  if constexpr (kTwoChains) {
+#pragma unroll
+    for (int r = 0; r < 16; ++r) acc[0][0][r] += acc_odd[r];
+  }
 
   // Epilogue: register r of lane l holds row 8*(r/4) + 4*(l/32) + r%4 of its 32-row tile and
   // columns TJ*(l%32) .. +TJ-1 of the wave's span (one per MFMA tile jn).
