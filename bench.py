@@ -56,7 +56,7 @@ def parse():
     ap.add_argument("--workload", default="gemm_bf16_8192",
                     choices=["gemm_bf16_8192", "gemm_f16_8192", "triad_sum_2p28", "gemm_f32_8192", "gemm_f32_1024",
                              "gemm_f16_epilogue", "gemm_f16_4095x11008x4096", "gemm_f16_shape", "copy_1gib", "vendor_gemm_bf16_8192", "histogram_2p28",
-                             "radix_scatter_5e7"])
+                             "radix_scatter_5e7", "mfma_bf16_stream"])
     ap.add_argument("--no-also", action="store_true", help="measure only the headline workload")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--shape", default="4096,11264,4096", metavar="M,N,K", help="shape of the gemm_f16_shape workload")
@@ -215,6 +215,19 @@ def make_workload(name, torch, hip):
                     config={"workload": f"{tn}-in f32-acc GEMM C=A.B row-major, N(0,0.02)",
                             "m": s, "n": s, "k": s})
         return main, None, info, (va, vb, vc, a, src_b, entry_b)
+    if name == "mfma_bf16_stream":
+        # The matrix pipes alone: as many v_mfma_f32_32x32x16_bf16 per wave as the 8192^3 product issues (8 waves per
+        # CU, 8 accumulator tiles per wave, 16384 instructions), on N(0, 0.02)-like operands that stay in registers;
+        # no memory instruction in the loop.  What the package's power limit leaves of the published peak on such data.
+        out = torch.zeros(256 * 512, device="cuda")
+        zero = 1 if ZERO_OPERANDS else 0
+        items = [out, ("i32", 1024), ("i32", zero)]
+        info = dict(metric="bf16 MFMA instruction stream TFLOP/s (no operand traffic)", unit="TFLOP/s", dtype="bf16",
+                    work=256.0 * 8 * 1024 * 16 * 32768, work_unit=1e12, bound="mfma", peak=PEAK_MFMA_TFLOPS["bf16"],
+                    kernel="mfma_stream (JIT)", route="Execute.run_source ~lang:HIP_Source, text in bench.py",
+                    config={"workload": "16384 v_mfma_f32_32x32x16_bf16 per wave, 2048 waves, register operands "
+                                        + ("all zero" if zero else "N(0,0.02)-like")})
+        return (lambda: hip.run_source(MFMA_STREAM_SRC, "mfma_stream", (512, 1, 1), (256, 1, 1), items)), None, info, out
     if name == "vendor_gemm_bf16_8192":
         # the vendor library's GEMM (torch.matmul -> hipBLASLt) on the headline inputs, for
         # side-by-side profiles; it writes bf16 C where the kernel here writes f32
@@ -418,6 +431,44 @@ def measure(name, torch, hip, steps, warmup):
     return res
 
 
+MFMA_STREAM_SRC = r"""
+typedef float f16v __attribute__((ext_vector_type(16)));
+typedef unsigned u4 __attribute__((ext_vector_type(4)));
+#define MF(ACC, A, B) asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, %0" : "+v"(ACC) : "v"(A), "v"(B))
+__device__ inline float rnd(unsigned& s) {   // sum of four uniforms scaled to sigma = 0.02
+  float acc = 0.f;
+  for (int i = 0; i < 4; ++i) { s = s * 1664525u + 1013904223u; acc += (float)(s >> 8) * (1.0f / 16777216.0f) - 0.5f; }
+  return acc * 0.0346f;
+}
+__device__ inline unsigned two_bf16(unsigned& s, int zero) {
+  const float x = zero ? 0.f : rnd(s), y = zero ? 0.f : rnd(s);
+  return (__float_as_uint(x) >> 16) | (__float_as_uint(y) & 0xffff0000u);
+}
+extern "C" __global__ __launch_bounds__(512) void mfma_stream(float* out, int n_out, int iters, int zero) {
+  unsigned s = (blockIdx.x * 512 + threadIdx.x) * 2654435761u + 12345u;
+  u4 A[2][4], B[2][2];
+  _Pragma("unroll") for (int kk = 0; kk < 2; ++kk) {
+    _Pragma("unroll") for (int i = 0; i < 4; ++i)
+      _Pragma("unroll") for (int e = 0; e < 4; ++e) A[kk][i][e] = two_bf16(s, zero);
+    _Pragma("unroll") for (int j = 0; j < 2; ++j)
+      _Pragma("unroll") for (int e = 0; e < 4; ++e) B[kk][j][e] = two_bf16(s, zero);
+  }
+  f16v acc[4][2];
+  _Pragma("unroll") for (int i = 0; i < 4; ++i)
+    _Pragma("unroll") for (int j = 0; j < 2; ++j)
+      _Pragma("unroll") for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
+  for (int it = 0; it < iters; ++it)
+    _Pragma("unroll") for (int kk = 0; kk < 2; ++kk)
+      _Pragma("unroll") for (int i = 0; i < 4; ++i)
+        _Pragma("unroll") for (int j = 0; j < 2; ++j) MF(acc[i][j], A[kk][i], B[kk][j]);
+  float sum = 0.f;
+  _Pragma("unroll") for (int i = 0; i < 4; ++i)
+    _Pragma("unroll") for (int j = 0; j < 2; ++j) sum += acc[i][j][0] + acc[i][j][7];
+  out[blockIdx.x * 512 + threadIdx.x] = sum;
+}
+"""
+
+
 HBM_PROBE_SRC = r"""
 typedef float f4 __attribute__((ext_vector_type(4)));
 #define LOADS(dst, src) _Pragma("unroll") for (int u = 0; u < 4; ++u) dst[u] = __builtin_nontemporal_load(src + base + u * 256)
@@ -547,7 +598,7 @@ def main():
         "value_at_median": head["value_at_median"],
         "gpu_ms_per_step_back_to_back": head["gpu_ms_per_step_back_to_back"],
     }
-    if not args.no_cpu_baseline and args.workload not in ("copy_1gib", "vendor_gemm_bf16_8192"):
+    if not args.no_cpu_baseline and args.workload not in ("copy_1gib", "vendor_gemm_bf16_8192", "mfma_bf16_stream"):
         out["cpu_baseline"] = cpu_baseline(args.workload)
     if not args.no_also:
         also = []
