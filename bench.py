@@ -407,6 +407,12 @@ def measure(name, torch, hip, steps, warmup):
     }
     if name == "triad_sum_2p28":
         res["roofline"]["probe_kernels_GBs"] = hbm_ceiling(torch, hip)
+    if name == "gemm_bf16_8192" and not ZERO_OPERANDS:
+        # the same number of MFMA instructions per wave with nothing round them (register operands of the same
+        # distribution, no memory instruction): what this box's power limit leaves of the peak on such data
+        stream = mfma_stream_rate(torch, hip)
+        res["roofline"]["mfma_stream_only_TFLOPs"] = stream
+        res["roofline"]["frac_of_mfma_stream_only"] = round(achieved / stream, 4)
     if info["bound"] == "mfma" and info["route"].startswith("Execute"):
         # shader clock the kernel actually ran at (in-kernel cycle counter against the
         # constant-rate wall clock), and the rate of those very launches against the peak
@@ -492,6 +498,23 @@ extern "C" __global__ __launch_bounds__(256) void probe_2r1w(f4* w, int nw, cons
   _Pragma("unroll") for (int u = 0; u < 4; ++u) __builtin_nontemporal_store(v[u] + c[u], w + base + u * 256);
 }
 """
+
+
+def mfma_stream_rate(torch, hip, launches=12):
+    """TFLOP/s of the bare v_mfma_f32_32x32x16_bf16 stream (MFMA_STREAM_SRC) at the median of `launches` launches each
+    waited for, JIT-compiled through the plugin path."""
+    out = torch.zeros(256 * 512, device="cuda")
+    stream = C.c_void_p(torch.cuda.current_stream().cuda_stream)
+    ev = Events(hip, stream)
+    times = []
+    for i in range(launches + 2):
+        ev.start()
+        hip.run_source(MFMA_STREAM_SRC, "mfma_stream", (512, 1, 1), (256, 1, 1), [out, ("i32", 1024), ("i32", 0)])
+        ms = ev.stop_ms()
+        if i >= 2:
+            times.append(ms)
+    times.sort()
+    return round(256.0 * 8 * 1024 * 16 * 32768 / (times[len(times) // 2] * 1e-3) / 1e12, 1)
 
 
 def hbm_ceiling(torch, hip, n=1 << 28):
