@@ -517,6 +517,23 @@ def mfma_stream_rate(torch, hip, launches=12):
     return round(256.0 * 8 * 1024 * 16 * 32768 / (times[len(times) // 2] * 1e-3) / 1e12, 1)
 
 
+def event_overhead_ms(torch, hip, launches=20):
+    """Median of what the two events round a launch measure when the kernel does nothing: the part of every
+    `kernel_ms` that is event and dispatch handling, not kernel."""
+    stream = C.c_void_p(torch.cuda.current_stream().cuda_stream)
+    ev = Events(hip, stream)
+    src = 'extern "C" __global__ void nothing(int n) {}'
+    times = []
+    for i in range(launches + 3):
+        ev.start()
+        hip.run_source(src, "nothing", (64, 1, 1), (1, 1, 1), [("i32", 0)])
+        ms = ev.stop_ms()
+        if i >= 3:
+            times.append(ms)
+    times.sort()
+    return round(times[len(times) // 2], 5)
+
+
 def hbm_ceiling(torch, hip, n=1 << 28):
     """What this GPU's HBM delivers to the simplest kernels of three traffic shapes (one
     workgroup per 4096 floats, 128-bit non-temporal accesses), JIT-compiled through the
@@ -635,6 +652,7 @@ def main():
                 r["cpu_baseline"] = cpu_baseline(name)
             also.append(r)
         out["also"] = also
+    out["event_overhead_ms"] = event_overhead_ms(torch, hip)
     info = hip.device_info(0)
     if args.tunable:
         out["tunables"] = args.tunable
