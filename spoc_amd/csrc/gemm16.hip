@@ -48,6 +48,7 @@ typedef __attribute__((ext_vector_type(4))) __bf16 bf16x4;
 typedef __attribute__((ext_vector_type(8))) _Float16 f16x8;
 typedef __attribute__((ext_vector_type(4))) _Float16 f16x4;
 typedef __attribute__((ext_vector_type(16))) float f32x16;
+typedef __attribute__((ext_vector_type(4))) float f32x4_t;
 typedef __attribute__((ext_vector_type(4))) unsigned int u32x4;
 typedef __attribute__((ext_vector_type(2))) unsigned int u32x2;
 
@@ -448,6 +449,297 @@ __global__ __launch_bounds__(64 * 2 * (8 / TJ)) void gemm16_dma_kernel(const uin
   }
 }
 
+// ---- direct-to-LDS kernel on v_mfma_f32_16x16x32 ---------------------------------------
+// The same tile, rings and transfers as gemm16_dma_kernel<.., 64, 32, 2, 4, 2> (256 x 256 per workgroup, 8 waves
+// of 128 x 64, A in 2 stages of K = 64, B in 4 slabs of K = 32, one barrier per B slab), but the products go
+// through the 16 x 16 x 32 instruction: 8 x 4 accumulator tiles of 16 x 16 per wave instead of 4 x 2 of 32 x 32.
+// On N(0, 0.02) data under the package power limit a bare stream of the 16 x 16 x 32 instruction runs 17 % faster
+// than one of the 32 x 32 x 16 instruction (2.09 against 1.79 PFLOP/s; on zeros both reach 2.45): it writes half as
+// many accumulator values per flop.  The LDS bytes read per flop are the same (the wave tile is).
+//
+// Operands: lane (m = lane%16, g = lane/16) supplies k = 8g..8g+7 of row m (A) / column m (B) and receives
+// rows 4g..4g+3 of column m of the 16 x 16 result.
+//   A: one ds_read_b128 per 16-row tile: chunk 4*ks + g of the row (ks = the B slab's place in the A stage).
+//   B: two ds_read_b64_tr_b16 per 16-column tile: rows 8g + {0..3} and 8g + {4..7} of the slab, 16 columns.
+//      A 32-lane phase of that read holds two k groups (rows r and r + 8): the B swizzle of the 32 x 32 kernel
+//      (slot ^= (row & 3) << 2, rows 64 bytes apart) is extended by slot ^= ((row >> 3) & 1) << 1, which puts
+//      the second group on the other 32-byte half of each 64-byte piece.
+// A slab is worked in two units of 16 MFMAs (rows 0-63 of the wave tile, then rows 64-127, same B fragments);
+// the barrier sits between them, and the second unit covers the fragment reads of the next slab.
+template <bool Bf16>
+__device__ __forceinline__ f32x4_t mfma16(u32x4 a, u32x4 b, f32x4_t c) {
+  if constexpr (Bf16)
+    return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b), c,
+                                                   0, 0, 0);
+  else
+    return __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(f16x8, a), __builtin_bit_cast(f16x8, b), c, 0,
+                                                  0, 0);
+}
+
+// Writes one wave's 128 x 64 block held as 8 x 4 tiles of 16 x 16 (register r of lane l: row 4*(l/16) + r, column
+// l%16 of its tile).  Fused form as in `epilogue`: per lane the sum over its four columns for each of its 32 rows,
+// a halving butterfly over the 16 lanes that share those rows (16+8+4+2 exchanges leave lane m with rows 2m, 2m+1
+// of the 32), the four waves along N through LDS, one atomicAdd per row.
+template <int Epi>
+__device__ __forceinline__ void epilogue16(f32x4_t (&acc)[8][4], float *__restrict__ C, const float *__restrict__ bias,
+                                           float *__restrict__ rowsum, int M, int N, int m0, int wm, int wn, int col0,
+                                           int l16, int g, float *scratch) {
+  const int row0 = m0 + wm * 128;
+  float bj[4];
+  bool cok[4];
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    const int col = col0 + j * 16 + l16;
+    cok[j] = col < N;
+    bj[j] = (Epi == EPI_BIAS_RELU_ROWSUM && cok[j]) ? bias[col] : 0.f;
+  }
+  float rs[32];
+#pragma unroll
+  for (int i = 0; i < 8; ++i) {
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+      const int row = row0 + i * 16 + 4 * g + r;
+      float sum = 0.f;
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        float v = acc[i][j][r];
+        if (Epi == EPI_BIAS_RELU_ROWSUM) {
+          v += bj[j];
+          v = v > 0.f ? v : 0.f;
+          sum += cok[j] ? v : 0.f;
+        }
+        if (row < M && cok[j]) C[static_cast<int64_t>(row) * N + col0 + j * 16 + l16] = v;
+      }
+      rs[i * 4 + r] = sum;
+    }
+  }
+  if constexpr (Epi == EPI_BIAS_RELU_ROWSUM) {
+#pragma unroll
+    for (int step = 0; step < 4; ++step) {
+      const int m = 8 >> step, half = 16 >> step;
+      const bool up = (l16 & m) != 0;
+#pragma unroll
+      for (int q = 0; q < half; ++q) {
+        // both values in registers before the selects: otherwise the compiler turns the selects into one
+        // lane-indexed read of rs[] (a compare-and-select chain over all 32 registers per value)
+        float lo = rs[q], hi = rs[q + half];
+        asm volatile("" : "+v"(lo), "+v"(hi));
+        const float send = up ? lo : hi;
+        const float keep = up ? hi : lo;
+        rs[q] = keep + __shfl_xor(send, m, 64);
+      }
+    }
+    // lane l16 now holds rows q = 2*l16 + e (e = 0, 1) of its 16-lane group's 32 rows: tile q/4, register q%4
+    __syncthreads();  // every wave has left the K loop: the LDS ring is free
+#pragma unroll
+    for (int e = 0; e < 2; ++e) {
+      const int q = 2 * l16 + e;
+      scratch[wn * 256 + wm * 128 + (q >> 2) * 16 + 4 * g + (q & 3)] = rs[e];
+    }
+    __syncthreads();
+    const int t = threadIdx.x;
+    if (t < 256 && m0 + t < M) {
+      const float total = (scratch[t] + scratch[256 + t]) + (scratch[512 + t] + scratch[768 + t]);
+      atomicAdd(rowsum + m0 + t, total);
+    }
+  }
+}
+
+template <bool Bf16, int Epi, int Ablate = 0>
+__global__ __launch_bounds__(512) void gemm16_m16_kernel(const uint16_t *__restrict__ A, const uint16_t *__restrict__ B,
+                                                         float *__restrict__ C, const float *__restrict__ bias,
+                                                         float *__restrict__ rowsum, int M, int N, int K, int tiles_m,
+                                                         int tiles_n, int xcd_remap, unsigned long long *probe) {
+  constexpr int BKA = 64, BKB = 32, NA = 2, NB = 4;
+  constexpr int RA = BKA / BKB;                  // B slabs per A stage
+  constexpr int A_ROW = BKA * 2, A_CHUNKS = A_ROW / 16, A_ROWS_PER_DMA = 1024 / A_ROW;
+  constexpr int A_BYTES_S = BM * A_ROW, B_BYTES_S = BKB * BN * 2;
+  constexpr int NWAVES = 8, WN = 4;
+  constexpr int DA = A_BYTES_S / 1024 / NWAVES, DB = B_BYTES_S / 1024 / NWAVES;
+  constexpr int P = lcm_int(NB, RA * NA);
+  static_assert(P % 2 == 0, "the B fragment buffers alternate by slab parity");
+  static_assert((NB - 1) * DB + NA * DA < 64, "vmcnt range");
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int wm = wave / WN, wn = wave % WN;
+  const int l16 = lane & 15, g = lane >> 4;
+  int tm, tn;
+  tile_of_block(tiles_m, tiles_n, xcd_remap, tm, tn);
+  const int m0 = tm * BM, n0 = tn * BN;
+  long long probe_c0 = 0, probe_t0 = 0;
+  if (probe) {
+    probe_c0 = clock64();
+    probe_t0 = wall_clock64();
+  }
+  auto a_swz = [](int row) { return (row >> 1) & 7; };
+  auto b_swz = [](int row) { return ((row & 3) << 2) | (((row >> 3) & 1) << 1); };
+
+  // DMA sources, as in gemm16_dma_kernel (rows past M and columns past N clamped: never stored)
+  uint32_t a_off[DA], b_off[DB];
+#pragma unroll
+  for (int i = 0; i < DA; ++i) {
+    const int q = wave + NWAVES * i;
+    const int arow_t = q * A_ROWS_PER_DMA + lane / A_CHUNKS;
+    const int arow = min(arow_t, M - 1 - m0);
+    a_off[i] = (static_cast<uint32_t>(arow) * K + (((lane % A_CHUNKS) ^ a_swz(arow_t)) << 3)) * 2u;
+  }
+#pragma unroll
+  for (int i = 0; i < DB; ++i) {
+    const int q = wave + NWAVES * i;
+    const int brow = 2 * q + (lane >> 5);
+    const int bchunk = (lane & 31) ^ b_swz(brow);
+    const int bcol = min(n0 + bchunk * 8, N - 8);
+    b_off[i] = (static_cast<uint32_t>(brow) * N + bcol) * 2u;
+  }
+  const char *a_base = reinterpret_cast<const char *>(A + static_cast<int64_t>(m0) * K);
+  const char *b_base = reinterpret_cast<const char *>(B);
+  const int64_t b_slab_bytes = static_cast<int64_t>(BKB) * N * 2;
+  const int nslabs = K / BKB, nstages = K / BKA;
+
+  f32x4_t acc[8][4];
+#pragma unroll
+  for (int i = 0; i < 8; ++i)
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+#pragma unroll
+      for (int r = 0; r < 4; ++r) acc[i][j][r] = 0.f;
+
+  // fragment read offsets.  A: row wm*128 + 16*i + l16, slot (4*ks + g) ^ swz = ((g ^ swz) ^ 4*ks): one base,
+  // XOR (ks << 6), + i * 2 KiB (16 rows leave the swizzle unchanged).  B: row 8g + li/4 (+4), the 8 bytes at
+  // column offset 4*(li%4) of the 16-column tile; tile j is an XOR with j << 5 (32 bytes).
+  const int a_row = wm * 128 + l16;
+  int a_addr0 = a_row * A_ROW + ((g ^ a_swz(a_row)) << 4);
+  const int b_r = l16 >> 2;
+  int b_addr0 = (g * 8 + b_r) * 512 + ((wn * 128 + (l16 & 3) * 8) ^ ((b_r << 6) | ((g & 1) << 5)));
+
+  const __amdgpu_buffer_rsrc_t a_rsrc = make_rsrc(a_base, 0x80000000u);
+  auto issue_a = [&](char *sa, int stage) {
+    if (stage >= NA && (Ablate & 1)) return;
+    const uint32_t a_so = static_cast<uint32_t>(min(stage, nstages - 1)) * (BKA * 2);
+#pragma unroll
+    for (int i = 0; i < DA; ++i) dma16(a_rsrc, a_off[i], a_so, sa + (wave + NWAVES * i) * 1024);
+  };
+  auto issue_b = [&](char *sb, int slab) {
+    if (slab >= NB && (Ablate & 1)) return;
+    const int sl = min(slab, nslabs - 1);
+    const __amdgpu_buffer_rsrc_t b_rsrc = make_rsrc(b_base + sl * b_slab_bytes, 0x80000000u);
+#pragma unroll
+    for (int i = 0; i < DB; ++i) dma16(b_rsrc, b_off[i], 0u, sb + (wave + NWAVES * i) * 1024);
+  };
+  // half: rows 0-63 (0) or 64-127 (1) of the wave tile
+  bool frags_loaded = false;
+  auto load_a = [&](const char *sa, int ks, int half, u32x4 (&af)[4]) {
+    if ((Ablate & 2) && frags_loaded) return;
+    const char *pa = sa + (a_addr0 ^ (ks << 6)) + half * (64 * A_ROW);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) af[i] = *reinterpret_cast<const u32x4 *>(pa + i * 16 * A_ROW);
+  };
+  auto load_b = [&](const char *sb, u32x4 (&bf)[4]) {
+    if ((Ablate & 2) && frags_loaded) return;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int off = b_addr0 ^ (j << 5);
+      u32x2 lo = lds_read_tr16(sb, off);
+      u32x2 hi = lds_read_tr16(sb, off + 4 * 512);
+      bf[j] = u32x4{lo.x, lo.y, hi.x, hi.y};
+    }
+  };
+  auto mfma_unit = [&](auto half_c, u32x4 (&af)[4], u32x4 (&bf)[4]) {
+    constexpr int H = decltype(half_c)::value;
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+      for (int j = 0; j < 4; ++j) acc[H * 4 + i][j] = mfma16<Bf16>(af[i], bf[j], acc[H * 4 + i][j]);
+  };
+  // Issue order of a unit: one LDS read or DMA instruction behind each MFMA, the DMA instructions spread evenly among
+  // the reads.  (A 16 x 16 x 32 MFMA occupies the pipe for 16 cycles: two reads and a DMA instruction behind one MFMA,
+  // the 32 x 32 kernel's pattern, do not fit in its shadow and cost 8 % of the cycle count.)
+  auto spread = [](auto nv_c, auto reads_c) {
+    constexpr int NV = decltype(nv_c)::value, READS = decltype(reads_c)::value, T = NV + READS;
+    static_assert(T <= 16, "one instruction per MFMA");
+    [&]<int... Ks>(std::integer_sequence<int, Ks...>) {
+      (([] {
+         __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+         // item Ks is a DMA instruction when it crosses a multiple of T / NV
+         if constexpr (NV > 0 && (Ks * NV) / T != ((Ks + 1) * NV) / T) __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
+         else __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+       }()),
+       ...);
+    }(std::make_integer_sequence<int, T>{});
+    if (T < 16) __builtin_amdgcn_sched_group_barrier(0x008, 16 - T, 0);
+    __builtin_amdgcn_sched_barrier(0);
+  };
+  auto load_a1 = [&](const char *sa, int ks, int half, int i, u32x4 &af) {
+    if ((Ablate & 2) && frags_loaded) return;
+    af = *reinterpret_cast<const u32x4 *>(sa + (a_addr0 ^ (ks << 6)) + half * (64 * A_ROW) + i * 16 * A_ROW);
+  };
+  using Lo = std::integral_constant<int, 0>;
+  using Hi = std::integral_constant<int, 1>;
+
+  u32x4 af[2][4], bf[2][4];   // af: [half], bf: [slab parity]
+
+  auto slab = [&](auto ic, int s) {
+    constexpr int I = decltype(ic)::value;
+    constexpr int In = (I + 1) % P;
+    constexpr int ia = (I / RA) % NA, ib = I % NB, ibp = (I + NB - 1) % NB;
+    constexpr int ian = (In / RA) % NA, ibn = In % NB;
+    constexpr int ks = I % RA, ksn = In % RA;
+    (void)ib;
+    asm volatile("" : "+v"(a_addr0), "+v"(b_addr0));
+    issue_b(lds_ring<20 + ibp, B_BYTES_S>, s - 1 + NB);
+    load_a(lds_ring<10 + ia, A_BYTES_S>, ks, 1, af[1]);
+    mfma_unit(Lo{}, af[0], bf[I & 1]);
+    spread(std::integral_constant<int, DB>{}, std::integral_constant<int, 4>{});
+    __builtin_amdgcn_s_waitcnt(waitcnt_vm_lgkm0(dma_allowed_in_flight(I, RA, NA, NB, DA, DB)));
+    barrier_no_fence();
+    if constexpr (I % RA == RA - 1) issue_a(lds_ring<10 + ia, A_BYTES_S>, s / RA + NA);
+    // the next slab's fragments in the order its first MFMAs need them: A tile 0, the four B tiles, A tiles 1-3
+    load_a1(lds_ring<10 + ian, A_BYTES_S>, ksn, 0, 0, af[0][0]);
+    load_b(lds_ring<20 + ibn, B_BYTES_S>, bf[In & 1]);
+    load_a1(lds_ring<10 + ian, A_BYTES_S>, ksn, 0, 1, af[0][1]);
+    load_a1(lds_ring<10 + ian, A_BYTES_S>, ksn, 0, 2, af[0][2]);
+    load_a1(lds_ring<10 + ian, A_BYTES_S>, ksn, 0, 3, af[0][3]);
+    mfma_unit(Hi{}, af[1], bf[I & 1]);
+    spread(std::integral_constant<int, (I % RA == RA - 1) ? DA : 0>{}, std::integral_constant<int, 12>{});
+  };
+
+  [&]<int... Is>(std::integer_sequence<int, Is...>) {
+    (issue_a(lds_ring<10 + Is, A_BYTES_S>, Is), ...);
+  }(std::make_integer_sequence<int, NA>{});
+  [&]<int... Is>(std::integer_sequence<int, Is...>) {
+    (issue_b(lds_ring<20 + Is, B_BYTES_S>, Is), ...);
+  }(std::make_integer_sequence<int, NB - 1>{});
+  __builtin_amdgcn_s_waitcnt(waitcnt_vm_lgkm0(0));
+  barrier_no_fence();
+  load_a(lds_ring<10, A_BYTES_S>, 0, 0, af[0]);
+  load_b(lds_ring<20, B_BYTES_S>, bf[0]);
+  if (Ablate & 2) {
+    load_a(lds_ring<10, A_BYTES_S>, 0, 1, af[1]);
+    load_b(lds_ring<20, B_BYTES_S>, bf[1]);
+    frags_loaded = true;
+  }
+  __builtin_amdgcn_sched_barrier(0);
+
+  const int full = nslabs - nslabs % P;
+  for (int s = 0; s < full; s += P) {
+    [&]<int... Is>(std::integer_sequence<int, Is...>) {
+      (slab(std::integral_constant<int, Is>{}, s + Is), ...);
+    }(std::make_integer_sequence<int, P>{});
+  }
+  [&]<int... Is>(std::integer_sequence<int, Is...>) {
+    ((full + Is < nslabs ? slab(std::integral_constant<int, Is>{}, full + Is) : (void)0), ...);
+  }(std::make_integer_sequence<int, P - 1>{});
+  __builtin_amdgcn_s_waitcnt(waitcnt_vm_lgkm0(0));   // drain the (redundant) tail DMA before the LDS is released
+  epilogue16<Epi>(acc, C, bias, rowsum, M, N, m0, wm, wn, n0 + wn * 64, l16, g,
+                  reinterpret_cast<float *>(lds_ring<10, A_BYTES_S>));
+  if (probe && tid == 0) {
+    probe[2 * blockIdx.x] = static_cast<unsigned long long>(clock64() - probe_c0);
+    probe[2 * blockIdx.x + 1] = static_cast<unsigned long long>(wall_clock64() - probe_t0);
+  }
+}
+
 template <bool Bf16, int Epi>
 __global__ __launch_bounds__(THREADS) void gemm16_staged_kernel(const uint16_t *__restrict__ A,
                                                          const uint16_t *__restrict__ B,
@@ -623,6 +915,7 @@ int launch_gemm16(const uint16_t *a, const uint16_t *b, float *c, const float *b
     const bool offsets_ok = static_cast<int64_t>(k) * 256 * 2 < 0x7FFFFFFF &&
                             static_cast<int64_t>(n) * 64 * 2 < 0x7FFFFFFF;
     if (k % BK == 0 && offsets_ok && tunable("gemm16.force_staged", 0) == 0) {
+      // gemm16.mfma: 16 = the kernel on the 16 x 16 x 32 instruction (default; ring 0 and tj 2 only), 32 = 32 x 32 x 16.
       // shape knobs for sweeps: gemm16.ring 0 = A in K=64 stages x2 + B in K=32 slabs x4
       // (default), 4 = both in K=32 slabs x4, 2 = both in K=64 slabs x2; gemm16.tj 2 | 4
       const int ring = (int)tunable("gemm16.ring", 0), tj = (int)tunable("gemm16.tj", 2);
@@ -633,6 +926,22 @@ int launch_gemm16(const uint16_t *a, const uint16_t *b, float *c, const float *b
                      dim3(64 * 2 * (8 / TJ)), 0, st, a, b, c, bias, rowsum, m, n, k, tiles_m,         \
                      tiles_n, remap, probe)
       const int ablate = (int)tunable("gemm16.ablate", 0);
+      const bool m16 = ring == 0 && tj == 2 && tunable("gemm16.mfma", 16) == 16;
+      if (m16 && ablate >= 1 && ablate <= 3 && Bf16 && Epi == EPI_STORE) {
+        // the same measurement variants for the 16 x 16 x 32 kernel (1: no transfers, 2: no fragment reads, 3: neither)
+        if constexpr (Bf16 && Epi == EPI_STORE) {
+#define SAREK_LAUNCH_M16_ABLATED(AB)                                                                        \
+  hipLaunchKernelGGL((gemm16_m16_kernel<true, EPI_STORE, AB>), grid, dim3(512), 0, st, a, b, c, bias, rowsum, m, n, k, \
+                     tiles_m, tiles_n, remap, probe)
+          if (ablate == 1) SAREK_LAUNCH_M16_ABLATED(1);
+          else if (ablate == 2) SAREK_LAUNCH_M16_ABLATED(2);
+          else SAREK_LAUNCH_M16_ABLATED(3);
+#undef SAREK_LAUNCH_M16_ABLATED
+        }
+        return check_launch("gemm16 kernel launch");
+      }
+      if (m16 && ablate != 0)
+        return fail(SAREK_HIP_E_UNSUPPORTED, "gemm16.ablate with the 16 x 16 x 32 kernel: 1..3, bf16 without epilogue (4 and 8: gemm16.mfma=32)");
       if (ablate != 0) {
         // measurement variants of the default shape (bf16, plain store); anything else is refused
         if (!Bf16 || Epi != EPI_STORE || ring != 0 || tj != 2 || ablate < 1 || (ablate > 4 && ablate != 8))
@@ -648,6 +957,11 @@ int launch_gemm16(const uint16_t *a, const uint16_t *b, float *c, const float *b
           else SAREK_LAUNCH_ABLATED(4);
 #undef SAREK_LAUNCH_ABLATED
         }
+        return check_launch("gemm16 kernel launch");
+      }
+      if (m16) {
+        hipLaunchKernelGGL((gemm16_m16_kernel<Bf16, Epi>), grid, dim3(512), 0, st, a, b, c, bias, rowsum, m, n, k,
+                           tiles_m, tiles_n, remap, probe);
         return check_launch("gemm16 kernel launch");
       }
       if (ring == 4 && tj == 2) SAREK_LAUNCH_DMA(32, 32, 4, 4, 2);

@@ -185,9 +185,10 @@ def test_gemm_bf16_full_size_rows(hip, oracle, torch_cuda):
 
 
 def test_measurement_variants_run_and_leave_the_kernel_as_it_was(hip, torch_cuda):
-    """gemm16.ablate (1..4) leaves parts of the K loop out for the power measurements and 8 the stores of C: the
-    results are wrong by construction, but every variant runs within the operands' bounds, other kernels refuse
-    the knob, and with the knob back at 0 the result is the one from before."""
+    """gemm16.ablate leaves parts of the K loop out for the power measurements (1..3 for both MFMA shapes, 4 for the
+    32 x 32 kernel) and 8 the stores of C (32 x 32 kernel): the results are wrong by construction, but every variant
+    runs within the operands' bounds, other kernels refuse the knob, and with the knobs back the result is the one
+    from before."""
     torch = torch_cuda
     m, n, k = 512, 768, 512
     torch.manual_seed(7)
@@ -195,24 +196,34 @@ def test_measurement_variants_run_and_leave_the_kernel_as_it_was(hip, torch_cuda
     b = (torch.randn(k, n, device="cuda") * 0.1).bfloat16()
     good = hip.gemm_bf16(a, b)
     try:
-        for v in (1, 2, 3, 4):
-            hip.set_tunable("gemm16.ablate", v)
-            c = hip.gemm_bf16(a, b)
-            torch.cuda.synchronize()
-            assert torch.isfinite(c).all()
+        for mfma, variants in ((16, (1, 2, 3)), (32, (1, 2, 3, 4))):
+            hip.set_tunable("gemm16.mfma", mfma)
+            for v in variants:
+                hip.set_tunable("gemm16.ablate", v)
+                c = hip.gemm_bf16(a, b)
+                torch.cuda.synchronize()
+                assert torch.isfinite(c).all()
         hip.set_tunable("gemm16.ablate", 8)
         untouched = torch.full((m, n), 7.0, device="cuda")
         hip.gemm_bf16(a, b, out=untouched)
         torch.cuda.synchronize()
         assert bool((untouched == 7.0).all())
-        with pytest.raises(hip.SarekHipError) as e:
-            hip.gemm_f16(a.half(), b.half())
-        assert e.value.status == hip.E_UNSUPPORTED
-        hip.set_tunable("gemm16.ablate", 5)
+        for mfma in (16, 32):
+            hip.set_tunable("gemm16.mfma", mfma)
+            hip.set_tunable("gemm16.ablate", 1)
+            with pytest.raises(hip.SarekHipError) as e:
+                hip.gemm_f16(a.half(), b.half())
+            assert e.value.status == hip.E_UNSUPPORTED
+            hip.set_tunable("gemm16.ablate", 5)
+            with pytest.raises(hip.SarekHipError):
+                hip.gemm_bf16(a, b)
+        hip.set_tunable("gemm16.mfma", 16)
+        hip.set_tunable("gemm16.ablate", 8)
         with pytest.raises(hip.SarekHipError):
             hip.gemm_bf16(a, b)
     finally:
         hip.set_tunable("gemm16.ablate", 0)
+        hip.set_tunable("gemm16.mfma", 16)
     assert torch.equal(hip.gemm_bf16(a, b), good)
 
 
@@ -266,19 +277,51 @@ def test_gemm_f32_every_tile_shape(hip, oracle, torch_cuda, tile, m, n, k):
     assert np.abs(c - oracle.gemm(a, b)).max() <= f32_tol(a, b, k)
 
 
-@pytest.mark.parametrize("ring,tj", [(0, 2), (0, 4), (4, 2), (4, 4), (2, 2), (2, 4)])
+@pytest.mark.parametrize("ring,tj,mfma", [(0, 2, 16), (0, 2, 32), (0, 4, 32), (4, 2, 32), (4, 4, 32), (2, 2, 32), (2, 4, 32)])
 @pytest.mark.parametrize("m,n,k", [(300, 520, 64), (257, 136, 192), (512, 768, 448), (70, 1032, 1216)])
-def test_gemm16_every_ring_shape(hip, oracle, torch_cuda, ring, tj, m, n, k):
-    """Every instantiation of the direct-to-LDS 16-bit kernel (A/B ring shapes, 8 or 4 waves)
-    on ragged M, N and on K values that end the stage pattern at different positions."""
+def test_gemm16_every_ring_shape(hip, oracle, torch_cuda, ring, tj, mfma, m, n, k):
+    """Every instantiation of the direct-to-LDS 16-bit kernels (the 16 x 16 x 32 kernel; the 32 x 32 x 16 kernel's
+    A/B ring shapes with 8 or 4 waves) on ragged M, N and on K values that end the stage pattern at different
+    positions."""
     a = normal16(oracle, (m, k), m + ring, "bf16")
     b = normal16(oracle, (k, n), n + tj, "bf16")
     ref = oracle.gemm(a, b)
     hip.set_tunable("gemm16.ring", ring)
     hip.set_tunable("gemm16.tj", tj)
+    hip.set_tunable("gemm16.mfma", mfma)
     try:
         c = hip.gemm_bf16(dev(torch_cuda, a).bfloat16(), dev(torch_cuda, b).bfloat16()).cpu().numpy()
     finally:
         hip.set_tunable("gemm16.ring", 0)
         hip.set_tunable("gemm16.tj", 2)
+        hip.set_tunable("gemm16.mfma", 16)
     assert np.abs(c - ref).max() / np.abs(ref).max() < 1e-4
+
+
+@pytest.mark.parametrize("kind", ["bf16", "f16"])
+@pytest.mark.parametrize("m,n,k", [(256, 256, 64), (513, 264, 320), (1000, 72, 128)])
+def test_gemm16_both_mfma_shapes_agree_with_the_oracle_and_each_other(hip, oracle, torch_cuda, kind, m, n, k):
+    """The kernel on v_mfma_f32_16x16x32 (default) and the one on v_mfma_f32_32x32x16, plain and with the fused
+    epilogue: both against the oracle; between the two only the order of the f32 additions differs."""
+    torch = torch_cuda
+    a = normal16(oracle, (m, k), m + 5, kind)
+    b = normal16(oracle, (k, n), n + 6, kind)
+    bias = oracle.fill_uniform(n, seed=n, lo=-0.1, hi=0.1)
+    dt = torch.bfloat16 if kind == "bf16" else torch.float16
+    da, db = dev(torch, a).to(dt), dev(torch, b).to(dt)
+    ref = oracle.gemm(a, b)
+    got = {}
+    try:
+        for mfma in (16, 32):
+            hip.set_tunable("gemm16.mfma", mfma)
+            c = (hip.gemm_bf16 if kind == "bf16" else hip.gemm_f16)(da, db).cpu().numpy()
+            assert np.abs(c - ref).max() / np.abs(ref).max() < 1e-4
+            got[mfma] = c
+            if kind == "f16":
+                y, rs = hip.gemm_f16_bias_relu_rowsum(da, db, dev(torch, bias))
+                y_ref, rs_ref = oracle.gemm_bias_relu_rowsum(a, b, bias)
+                assert np.abs(y.cpu().numpy() - y_ref).max() <= 1e-4 * np.abs(y_ref).max()
+                assert np.abs(rs.cpu().numpy() - rs_ref).max() <= 1e-4 * max(np.abs(rs_ref).max(), 1e-30)
+    finally:
+        hip.set_tunable("gemm16.mfma", 16)
+    assert np.abs(got[16] - got[32]).max() <= 1e-5 * np.abs(ref).max()
