@@ -545,7 +545,7 @@ __device__ __forceinline__ void epilogue16(f32x4_t (&acc)[8][4], float *__restri
   }
 }
 
-template <bool Bf16, int Epi, int Ablate = 0>
+template <bool Bf16, int Epi, int Ablate = 0, int Pre = 16>
 __global__ __launch_bounds__(512) void gemm16_m16_kernel(const uint16_t *__restrict__ A, const uint16_t *__restrict__ B,
                                                          float *__restrict__ C, const float *__restrict__ bias,
                                                          float *__restrict__ rowsum, int M, int N, int K, int tiles_m,
@@ -621,12 +621,19 @@ __global__ __launch_bounds__(512) void gemm16_m16_kernel(const uint16_t *__restr
 #pragma unroll
     for (int i = 0; i < DA; ++i) dma16(a_rsrc, a_off[i], a_so, sa + (wave + NWAVES * i) * 1024);
   };
+  // B slabs are issued in order 0, 1, 2, ...: the source of the next one is a running pointer (two scalar adds per
+  // slab instead of a 64-bit multiply) that stops at the last slab, which the tail of the K loop re-issues into
+  // stages nobody reads any more so that the count of outstanding transfers follows the same pattern throughout
+  const char *b_src = b_base;
+  int b_next = 0;
   auto issue_b = [&](char *sb, int slab) {
     if (slab >= NB && (Ablate & 1)) return;
-    const int sl = min(slab, nslabs - 1);
-    const __amdgpu_buffer_rsrc_t b_rsrc = make_rsrc(b_base + sl * b_slab_bytes, 0x80000000u);
+    (void)slab;   // == b_next
+    const __amdgpu_buffer_rsrc_t b_rsrc = make_rsrc(b_src, 0x80000000u);
 #pragma unroll
     for (int i = 0; i < DB; ++i) dma16(b_rsrc, b_off[i], 0u, sb + (wave + NWAVES * i) * 1024);
+    ++b_next;
+    if (b_next < nslabs) b_src += b_slab_bytes;
   };
   // half: rows 0-63 (0) or 64-127 (1) of the wave tile
   bool frags_loaded = false;
@@ -646,38 +653,43 @@ __global__ __launch_bounds__(512) void gemm16_m16_kernel(const uint16_t *__restr
       bf[j] = u32x4{lo.x, lo.y, hi.x, hi.y};
     }
   };
-  auto mfma_unit = [&](auto half_c, u32x4 (&af)[4], u32x4 (&bf)[4]) {
-    constexpr int H = decltype(half_c)::value;
-#pragma unroll
-    for (int i = 0; i < 4; ++i)
-#pragma unroll
-      for (int j = 0; j < 4; ++j) acc[H * 4 + i][j] = mfma16<Bf16>(af[i], bf[j], acc[H * 4 + i][j]);
+  // MFMAs First .. First+Count-1 of a slab's 32, in the order (row tile i, column tile j); row tiles 0-3 take their
+  // A fragments from af[0], 4-7 from af[1]
+  auto mfma_range = [&](auto first_c, auto count_c, u32x4 (&af)[2][4], u32x4 (&bf)[4]) {
+    constexpr int First = decltype(first_c)::value, Count = decltype(count_c)::value;
+    [&]<int... Ts>(std::integer_sequence<int, Ts...>) {
+      ((acc[(First + Ts) / 4][(First + Ts) % 4] = mfma16<Bf16>(af[(First + Ts) / 16][((First + Ts) / 4) % 4],
+                                                              bf[(First + Ts) % 4],
+                                                              acc[(First + Ts) / 4][(First + Ts) % 4])),
+       ...);
+    }(std::make_integer_sequence<int, Count>{});
   };
-  // Issue order of a unit: one LDS read or DMA instruction behind each MFMA, the DMA instructions spread evenly among
-  // the reads.  (A 16 x 16 x 32 MFMA occupies the pipe for 16 cycles: two reads and a DMA instruction behind one MFMA,
-  // the 32 x 32 kernel's pattern, do not fit in its shadow and cost 8 % of the cycle count.)
-  auto spread = [](auto nv_c, auto reads_c) {
-    constexpr int NV = decltype(nv_c)::value, READS = decltype(reads_c)::value, T = NV + READS;
-    static_assert(T <= 16, "one instruction per MFMA");
-    [&]<int... Ks>(std::integer_sequence<int, Ks...>) {
+  // Issue order: the T = NV + READS other instructions (DMA, LDS reads) go one each behind MFMAs spread evenly over
+  // the MFMAS of the section, the DMA instructions evenly among the reads.  (A 16 x 16 x 32 MFMA occupies the pipe for
+  // 16 cycles: two reads and a DMA instruction behind one MFMA, the 32 x 32 kernel's pattern, do not fit in its shadow
+  // and cost 8 % of the cycle count.)
+  auto spread = [](auto nv_c, auto reads_c, auto mfmas_c) {
+    constexpr int NV = decltype(nv_c)::value, READS = decltype(reads_c)::value, MFMAS = decltype(mfmas_c)::value;
+    constexpr int T = NV + READS;
+    static_assert(T <= MFMAS, "one instruction per MFMA at most");
+    [&]<int... Ms>(std::integer_sequence<int, Ms...>) {
       (([] {
          __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-         // item Ks is a DMA instruction when it crosses a multiple of T / NV
-         if constexpr (NV > 0 && (Ks * NV) / T != ((Ks + 1) * NV) / T) __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
-         else __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+         // item k sits behind MFMA (k * MFMAS) / T
+         constexpr int k = (Ms * T + MFMAS - 1) / MFMAS;          // first item at or after this MFMA
+         if constexpr (k < T && (k * MFMAS) / T == Ms) {
+           if constexpr (NV > 0 && (k * NV) / T != ((k + 1) * NV) / T) __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
+           else __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+         }
        }()),
        ...);
-    }(std::make_integer_sequence<int, T>{});
-    if (T < 16) __builtin_amdgcn_sched_group_barrier(0x008, 16 - T, 0);
+    }(std::make_integer_sequence<int, MFMAS>{});
     __builtin_amdgcn_sched_barrier(0);
   };
   auto load_a1 = [&](const char *sa, int ks, int half, int i, u32x4 &af) {
     if ((Ablate & 2) && frags_loaded) return;
     af = *reinterpret_cast<const u32x4 *>(sa + (a_addr0 ^ (ks << 6)) + half * (64 * A_ROW) + i * 16 * A_ROW);
   };
-  using Lo = std::integral_constant<int, 0>;
-  using Hi = std::integral_constant<int, 1>;
-
   u32x4 af[2][4], bf[2][4];   // af: [half], bf: [slab parity]
 
   auto slab = [&](auto ic, int s) {
@@ -690,19 +702,28 @@ __global__ __launch_bounds__(512) void gemm16_m16_kernel(const uint16_t *__restr
     asm volatile("" : "+v"(a_addr0), "+v"(b_addr0));
     issue_b(lds_ring<20 + ibp, B_BYTES_S>, s - 1 + NB);
     load_a(lds_ring<10 + ia, A_BYTES_S>, ks, 1, af[1]);
-    mfma_unit(Lo{}, af[0], bf[I & 1]);
-    spread(std::integral_constant<int, DB>{}, std::integral_constant<int, 4>{});
+    mfma_range(std::integral_constant<int, 0>{}, std::integral_constant<int, Pre>{}, af, bf[I & 1]);
+    spread(std::integral_constant<int, DB>{}, std::integral_constant<int, 4>{}, std::integral_constant<int, Pre>{});
     __builtin_amdgcn_s_waitcnt(waitcnt_vm_lgkm0(dma_allowed_in_flight(I, RA, NA, NB, DA, DB)));
     barrier_no_fence();
     if constexpr (I % RA == RA - 1) issue_a(lds_ring<10 + ia, A_BYTES_S>, s / RA + NA);
     // the next slab's fragments in the order its first MFMAs need them: A tile 0, the four B tiles, A tiles 1-3
+    // (an A register of the low half is reloaded only after the slab's last MFMA that reads it: with the barrier
+    // before MFMA 16 some of those come after the barrier)
+    static_assert(Pre % 4 == 0 && Pre >= 8 && Pre <= 16, "barrier position");
     load_a1(lds_ring<10 + ian, A_BYTES_S>, ksn, 0, 0, af[0][0]);
     load_b(lds_ring<20 + ibn, B_BYTES_S>, bf[In & 1]);
     load_a1(lds_ring<10 + ian, A_BYTES_S>, ksn, 0, 1, af[0][1]);
-    load_a1(lds_ring<10 + ian, A_BYTES_S>, ksn, 0, 2, af[0][2]);
-    load_a1(lds_ring<10 + ian, A_BYTES_S>, ksn, 0, 3, af[0][3]);
-    mfma_unit(Hi{}, af[1], bf[I & 1]);
-    spread(std::integral_constant<int, (I % RA == RA - 1) ? DA : 0>{}, std::integral_constant<int, 12>{});
+    if constexpr (Pre >= 12) load_a1(lds_ring<10 + ian, A_BYTES_S>, ksn, 0, 2, af[0][2]);
+    if constexpr (Pre >= 16) load_a1(lds_ring<10 + ian, A_BYTES_S>, ksn, 0, 3, af[0][3]);
+    if constexpr (Pre < 16) {
+      mfma_range(std::integral_constant<int, Pre>{}, std::integral_constant<int, 16 - Pre>{}, af, bf[I & 1]);
+      if constexpr (Pre < 12) load_a1(lds_ring<10 + ian, A_BYTES_S>, ksn, 0, 2, af[0][2]);
+      load_a1(lds_ring<10 + ian, A_BYTES_S>, ksn, 0, 3, af[0][3]);
+    }
+    mfma_range(std::integral_constant<int, 16>{}, std::integral_constant<int, 16>{}, af, bf[I & 1]);
+    spread(std::integral_constant<int, (I % RA == RA - 1) ? DA : 0>{}, std::integral_constant<int, 12>{},
+           std::integral_constant<int, 32 - Pre>{});
   };
 
   [&]<int... Is>(std::integer_sequence<int, Is...>) {
