@@ -56,7 +56,7 @@ def parse():
     ap.add_argument("--workload", default="gemm_bf16_8192",
                     choices=["gemm_bf16_8192", "gemm_f16_8192", "triad_sum_2p28", "gemm_f32_8192", "gemm_f32_1024",
                              "gemm_f16_epilogue", "gemm_f16_4095x11008x4096", "gemm_f16_shape", "copy_1gib", "vendor_gemm_bf16_8192", "histogram_2p28",
-                             "radix_scatter_5e7", "mfma_bf16_stream"])
+                             "radix_scatter_5e7", "mfma_bf16_stream", "mfma_bf16_stream_32x32x16"])
     ap.add_argument("--no-also", action="store_true", help="measure only the headline workload")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--shape", default="4096,11264,4096", metavar="M,N,K", help="shape of the gemm_f16_shape workload")
@@ -210,24 +210,27 @@ def make_workload(name, torch, hip):
         tn = "bf16" if bf16 else "f16"
         info = dict(metric=f"GEMM TFLOP/s at 8192^3 ({tn}-in, f32-accumulate)", unit="TFLOP/s",
                     dtype=tn, work=2.0 * s ** 3, work_unit=1e12, bound="mfma",
-                    peak=PEAK_MFMA_TFLOPS[tn], kernel=f"gemm16_dma_kernel<{tn}, store, 64, 32, 2, 4, 2>",
+                    peak=PEAK_MFMA_TFLOPS[tn], kernel=f"gemm16_m16_kernel<{tn}, store>",
                     route=f"Execute.run_source ~lang:HIP_Source, library kernel text '{lib_name}'",
                     config={"workload": f"{tn}-in f32-acc GEMM C=A.B row-major, N(0,0.02)",
                             "m": s, "n": s, "k": s})
         return main, None, info, (va, vb, vc, a, src_b, entry_b)
-    if name == "mfma_bf16_stream":
-        # The matrix pipes alone: as many v_mfma_f32_32x32x16_bf16 per wave as the 8192^3 product issues (8 waves per
-        # CU, 8 accumulator tiles per wave, 16384 instructions), on N(0, 0.02)-like operands that stay in registers;
-        # no memory instruction in the loop.  What the package's power limit leaves of the published peak on such data.
+    if name in ("mfma_bf16_stream", "mfma_bf16_stream_32x32x16"):
+        # The matrix pipes alone: the MFMA instructions of the 8192^3 product and nothing else (8 waves per CU,
+        # N(0, 0.02)-like operands that stay in registers, no memory instruction in the loop), with the instruction
+        # the GEMM kernel uses, v_mfma_f32_16x16x32_bf16 (32768 per wave), or with v_mfma_f32_32x32x16_bf16 (16384 per
+        # wave).  What the package's power limit leaves of the published peak on such data.
+        entry = "mfma_stream16" if name == "mfma_bf16_stream" else "mfma_stream"
+        instr = "16x16x32" if name == "mfma_bf16_stream" else "32x32x16"
         out = torch.zeros(256 * 512, device="cuda")
         zero = 1 if ZERO_OPERANDS else 0
         items = [out, ("i32", 1024), ("i32", zero)]
         info = dict(metric="bf16 MFMA instruction stream TFLOP/s (no operand traffic)", unit="TFLOP/s", dtype="bf16",
                     work=256.0 * 8 * 1024 * 16 * 32768, work_unit=1e12, bound="mfma", peak=PEAK_MFMA_TFLOPS["bf16"],
-                    kernel="mfma_stream (JIT)", route="Execute.run_source ~lang:HIP_Source, text in bench.py",
-                    config={"workload": "16384 v_mfma_f32_32x32x16_bf16 per wave, 2048 waves, register operands "
+                    kernel=f"{entry} (JIT)", route="Execute.run_source ~lang:HIP_Source, text in bench.py",
+                    config={"workload": f"v_mfma_f32_{instr}_bf16 stream, 1.0995e12 flop over 2048 waves, register operands "
                                         + ("all zero" if zero else "N(0,0.02)-like")})
-        return (lambda: hip.run_source(MFMA_STREAM_SRC, "mfma_stream", (512, 1, 1), (256, 1, 1), items)), None, info, out
+        return (lambda: hip.run_source(MFMA_STREAM_SRC, entry, (512, 1, 1), (256, 1, 1), items)), None, info, out
     if name == "vendor_gemm_bf16_8192":
         # the vendor library's GEMM (torch.matmul -> hipBLASLt) on the headline inputs, for
         # side-by-side profiles; it writes bf16 C where the kernel here writes f32
@@ -307,7 +310,7 @@ def make_workload(name, torch, hip):
                       dims((n + 15) // 16, (m + 15) // 16, 1), 0, 1, a, na)
         info = dict(metric=f"fp16 GEMM TFLOP/s at {m}x{n}x{k}", unit="TFLOP/s", dtype="f16",
                     work=2.0 * m * n * k, work_unit=1e12, bound="mfma",
-                    peak=PEAK_MFMA_TFLOPS["f16"], kernel="gemm16_dma_kernel<f16, store, 64, 32, 2, 4, 2>",
+                    peak=PEAK_MFMA_TFLOPS["f16"], kernel="gemm16_m16_kernel<f16, store>",
                     route="Execute.run_source ~lang:HIP_Source, library kernel text 'gemm_f16'",
                     config={"workload": "fp16-in f32-acc C=A.B", "m": m, "n": n, "k": k})
         return main, None, info, (va, vb, vy, a, src_b, entry_b)
@@ -332,7 +335,7 @@ def make_workload(name, torch, hip):
                       dims(1024, 1, 1), 0, 1, a, na)
         info = dict(metric="fp16 GEMM + bias + ReLU + row-sum TFLOP/s", unit="TFLOP/s", dtype="f16",
                     work=2.0 * m * n * k, work_unit=1e12, bound="mfma",
-                    peak=PEAK_MFMA_TFLOPS["f16"], kernel="gemm16_dma_kernel<f16, bias_relu_rowsum, 64, 32, 2, 4, 2>",
+                    peak=PEAK_MFMA_TFLOPS["f16"], kernel="gemm16_m16_kernel<f16, bias_relu_rowsum>",
                     route="Execute.run_source ~lang:HIP_Source, library kernel text 'gemm_f16_bias_relu_rowsum'",
                     config={"workload": "fp16-in f32-acc Y=relu(A.B+bias), rowsum(Y)",
                             "m": m, "n": n, "k": k})
@@ -410,9 +413,10 @@ def measure(name, torch, hip, steps, warmup):
     if name == "gemm_bf16_8192" and not ZERO_OPERANDS:
         # the same number of MFMA instructions per wave with nothing round them (register operands of the same
         # distribution, no memory instruction): what this box's power limit leaves of the peak on such data
-        stream = mfma_stream_rate(torch, hip)
+        stream, stream32 = mfma_stream_rates(torch, hip)
         res["roofline"]["mfma_stream_only_TFLOPs"] = stream
         res["roofline"]["frac_of_mfma_stream_only"] = round(achieved / stream, 4)
+        res["roofline"]["mfma_stream_only_32x32x16_TFLOPs"] = stream32
     if info["bound"] == "mfma" and info["route"].startswith("Execute"):
         # shader clock the kernel actually ran at (in-kernel cycle counter against the
         # constant-rate wall clock), and the rate of those very launches against the peak
@@ -472,6 +476,28 @@ extern "C" __global__ __launch_bounds__(512) void mfma_stream(float* out, int n_
     _Pragma("unroll") for (int j = 0; j < 2; ++j) sum += acc[i][j][0] + acc[i][j][7];
   out[blockIdx.x * 512 + threadIdx.x] = sum;
 }
+// the same flops per iteration with v_mfma_f32_16x16x32_bf16: 32 instructions on 16 accumulator tiles of 16 x 16
+typedef float f4v __attribute__((ext_vector_type(4)));
+#define MF16(ACC, A, B) asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, %0" : "+v"(ACC) : "v"(A), "v"(B))
+extern "C" __global__ __launch_bounds__(512) void mfma_stream16(float* out, int n_out, int iters, int zero) {
+  unsigned s = (blockIdx.x * 512 + threadIdx.x) * 2654435761u + 12345u;
+  u4 A[2][4], B[2][4];
+  _Pragma("unroll") for (int kk = 0; kk < 2; ++kk)
+    _Pragma("unroll") for (int i = 0; i < 4; ++i)
+      _Pragma("unroll") for (int e = 0; e < 4; ++e) { A[kk][i][e] = two_bf16(s, zero); B[kk][i][e] = two_bf16(s, zero); }
+  f4v acc[4][4];
+  _Pragma("unroll") for (int i = 0; i < 4; ++i)
+    _Pragma("unroll") for (int j = 0; j < 4; ++j)
+      _Pragma("unroll") for (int r = 0; r < 4; ++r) acc[i][j][r] = 0.f;
+  for (int it = 0; it < iters; ++it)
+    _Pragma("unroll") for (int kk = 0; kk < 2; ++kk)
+      _Pragma("unroll") for (int i = 0; i < 4; ++i)
+        _Pragma("unroll") for (int j = 0; j < 4; ++j) MF16(acc[i][j], A[kk][i], B[kk][j]);
+  float sum = 0.f;
+  _Pragma("unroll") for (int i = 0; i < 4; ++i)
+    _Pragma("unroll") for (int j = 0; j < 4; ++j) sum += acc[i][j][0] + acc[i][j][3];
+  out[blockIdx.x * 512 + threadIdx.x] = sum;
+}
 """
 
 
@@ -500,21 +526,23 @@ extern "C" __global__ __launch_bounds__(256) void probe_2r1w(f4* w, int nw, cons
 """
 
 
-def mfma_stream_rate(torch, hip, launches=12):
-    """TFLOP/s of the bare v_mfma_f32_32x32x16_bf16 stream (MFMA_STREAM_SRC) at the median of `launches` launches each
-    waited for, JIT-compiled through the plugin path."""
+def mfma_stream_rates(torch, hip, launches=15):
+    """TFLOP/s of the bare MFMA streams of MFMA_STREAM_SRC (mfma_stream16 = v_mfma_f32_16x16x32_bf16, the GEMM
+    kernel's instruction; mfma_stream = v_mfma_f32_32x32x16_bf16), JIT-compiled through the plugin path: the two are
+    launched in turn, each launch waited for, and the median launch of each is reported (16x16x32, 32x32x16)."""
     out = torch.zeros(256 * 512, device="cuda")
     stream = C.c_void_p(torch.cuda.current_stream().cuda_stream)
     ev = Events(hip, stream)
-    times = []
-    for i in range(launches + 2):
-        ev.start()
-        hip.run_source(MFMA_STREAM_SRC, "mfma_stream", (512, 1, 1), (256, 1, 1), [out, ("i32", 1024), ("i32", 0)])
-        ms = ev.stop_ms()
-        if i >= 2:
-            times.append(ms)
-    times.sort()
-    return round(256.0 * 8 * 1024 * 16 * 32768 / (times[len(times) // 2] * 1e-3) / 1e12, 1)
+    times = {"mfma_stream16": [], "mfma_stream": []}
+    for i in range(launches + 3):
+        for entry in times:
+            ev.start()
+            hip.run_source(MFMA_STREAM_SRC, entry, (512, 1, 1), (256, 1, 1), [out, ("i32", 1024), ("i32", 0)])
+            ms = ev.stop_ms()
+            if i >= 3:
+                times[entry].append(ms)
+    flop = 256.0 * 8 * 1024 * 16 * 32768
+    return tuple(round(flop / (sorted(t)[len(t) // 2] * 1e-3) / 1e12, 1) for t in times.values())
 
 
 def event_overhead_ms(torch, hip, launches=20):
@@ -638,7 +666,7 @@ def main():
         "value_at_median": head["value_at_median"],
         "gpu_ms_per_step_back_to_back": head["gpu_ms_per_step_back_to_back"],
     }
-    if not args.no_cpu_baseline and args.workload not in ("copy_1gib", "vendor_gemm_bf16_8192", "mfma_bf16_stream"):
+    if not args.no_cpu_baseline and args.workload not in ("copy_1gib", "vendor_gemm_bf16_8192", "mfma_bf16_stream", "mfma_bf16_stream_32x32x16"):
         out["cpu_baseline"] = cpu_baseline(args.workload)
     if not args.no_also:
         also = []
