@@ -545,7 +545,7 @@ __device__ __forceinline__ void epilogue16(f32x4_t (&acc)[8][4], float *__restri
   }
 }
 
-template <bool Bf16, int Epi, int Ablate = 0, int Pre = 16>
+template <bool Bf16, int Epi, int Ablate = 0>
 __global__ __launch_bounds__(512) void gemm16_m16_kernel(const uint16_t *__restrict__ A, const uint16_t *__restrict__ B,
                                                          float *__restrict__ C, const float *__restrict__ bias,
                                                          float *__restrict__ rowsum, int M, int N, int K, int tiles_m,
@@ -702,28 +702,22 @@ __global__ __launch_bounds__(512) void gemm16_m16_kernel(const uint16_t *__restr
     asm volatile("" : "+v"(a_addr0), "+v"(b_addr0));
     issue_b(lds_ring<20 + ibp, B_BYTES_S>, s - 1 + NB);
     load_a(lds_ring<10 + ia, A_BYTES_S>, ks, 1, af[1]);
-    mfma_range(std::integral_constant<int, 0>{}, std::integral_constant<int, Pre>{}, af, bf[I & 1]);
-    spread(std::integral_constant<int, DB>{}, std::integral_constant<int, 4>{}, std::integral_constant<int, Pre>{});
+    mfma_range(std::integral_constant<int, 0>{}, std::integral_constant<int, 16>{}, af, bf[I & 1]);
+    spread(std::integral_constant<int, DB>{}, std::integral_constant<int, 4>{}, std::integral_constant<int, 16>{});
     __builtin_amdgcn_s_waitcnt(waitcnt_vm_lgkm0(dma_allowed_in_flight(I, RA, NA, NB, DA, DB)));
     barrier_no_fence();
     if constexpr (I % RA == RA - 1) issue_a(lds_ring<10 + ia, A_BYTES_S>, s / RA + NA);
-    // the next slab's fragments in the order its first MFMAs need them: A tile 0, the four B tiles, A tiles 1-3
-    // (an A register of the low half is reloaded only after the slab's last MFMA that reads it: with the barrier
-    // before MFMA 16 some of those come after the barrier)
-    static_assert(Pre % 4 == 0 && Pre >= 8 && Pre <= 16, "barrier position");
+    // the next slab's fragments in the order its first MFMAs need them: A tile 0, the four B tiles, A tiles 1-3.
+    // (The barrier was also tried after 8 and after 12 MFMAs, with the low-half A registers reloaded behind their
+    // last readers: 1 % slower.)
     load_a1(lds_ring<10 + ian, A_BYTES_S>, ksn, 0, 0, af[0][0]);
     load_b(lds_ring<20 + ibn, B_BYTES_S>, bf[In & 1]);
     load_a1(lds_ring<10 + ian, A_BYTES_S>, ksn, 0, 1, af[0][1]);
-    if constexpr (Pre >= 12) load_a1(lds_ring<10 + ian, A_BYTES_S>, ksn, 0, 2, af[0][2]);
-    if constexpr (Pre >= 16) load_a1(lds_ring<10 + ian, A_BYTES_S>, ksn, 0, 3, af[0][3]);
-    if constexpr (Pre < 16) {
-      mfma_range(std::integral_constant<int, Pre>{}, std::integral_constant<int, 16 - Pre>{}, af, bf[I & 1]);
-      if constexpr (Pre < 12) load_a1(lds_ring<10 + ian, A_BYTES_S>, ksn, 0, 2, af[0][2]);
-      load_a1(lds_ring<10 + ian, A_BYTES_S>, ksn, 0, 3, af[0][3]);
-    }
+    load_a1(lds_ring<10 + ian, A_BYTES_S>, ksn, 0, 2, af[0][2]);
+    load_a1(lds_ring<10 + ian, A_BYTES_S>, ksn, 0, 3, af[0][3]);
     mfma_range(std::integral_constant<int, 16>{}, std::integral_constant<int, 16>{}, af, bf[I & 1]);
     spread(std::integral_constant<int, (I % RA == RA - 1) ? DA : 0>{}, std::integral_constant<int, 12>{},
-           std::integral_constant<int, 32 - Pre>{});
+           std::integral_constant<int, 16>{});
   };
 
   [&]<int... Is>(std::integer_sequence<int, Is...>) {
