@@ -57,6 +57,11 @@ def parse():
                     choices=["gemm_bf16_8192", "gemm_f16_8192", "triad_sum_2p28", "gemm_f32_8192", "gemm_f32_1024",
                              "gemm_f16_epilogue", "gemm_f16_4095x11008x4096", "gemm_f16_shape", "copy_1gib", "vendor_gemm_bf16_8192", "histogram_2p28",
                              "radix_scatter_5e7", "mfma_bf16_stream", "mfma_bf16_stream_32x32x16"])
+    ap.add_argument("--warmup-ms", type=float, default=60.0,
+                    help="warm up for at least this long (and at least --warmup steps): the clocks of a power-limited "
+                         "kernel take 30-40 ms to settle after a pause")
+    ap.add_argument("--trace-launches", action="store_true",
+                    help="add the timed launches' kernel durations in launch order (kernel_us_by_launch)")
     ap.add_argument("--no-also", action="store_true", help="measure only the headline workload")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--shape", default="4096,11264,4096", metavar="M,N,K", help="shape of the gemm_f16_shape workload")
@@ -349,24 +354,33 @@ def stats(xs):
             "max": round(xs[-1], 5)}
 
 
+WARMUP_MS = 60.0
+TRACE_LAUNCHES = False
+
+
 def measure(name, torch, hip, steps, warmup):
     """Warmup, then `steps` timed iterations, each launched and waited for, as the reference's benches do
     (benchmarks/bench_stream_triad.ml:98-115: time around launch + device synchronise, median reported).
-    The dominant kernel's duration comes from HIP events recorded round its launch on the launch stream."""
+    The dominant kernel's duration comes from HIP events recorded round its launch on the launch stream.
+    The warmup is `warmup` steps and at least WARMUP_MS of them, launched and waited for like the timed ones: the
+    package's power management needs 30-40 ms under a new load before the clocks settle (a power-limited kernel's
+    third to sixth launch after a pause takes up to a third longer than its fiftieth)."""
     main, tail, info, keep = make_workload(name, torch, hip)
     stream = C.c_void_p(torch.cuda.current_stream().cuda_stream)
     ev = Events(hip, stream)
     sync = hip.lib.sarek_hip_device_synchronize
-    for _ in range(warmup):
+    path = None
+    if info["route"].startswith("Execute"):
+        main()                                   # alone, to read which code path served it
+        path = hip.lib.sarek_hip_last_run_path().decode()
+        sync()
+    done, t_warm = 0, time.perf_counter()
+    while done < warmup or (time.perf_counter() - t_warm) * 1e3 < WARMUP_MS:
         main()
         if tail:
             tail()
-    sync()
-    path = None
-    if info["route"].startswith("Execute"):
-        main()                                   # once more, alone, to read which code path served it
-        path = hip.lib.sarek_hip_last_run_path().decode()
         sync()
+        done += 1
     walls, kerns = [], []
     t0 = time.perf_counter()
     for _ in range(steps):
@@ -382,6 +396,7 @@ def measure(name, torch, hip, steps, warmup):
         hip.check(hip.lib.sarek_hip_event_elapsed_ms(ev.e0, ev.e1, C.byref(ms)))
         kerns.append(float(ms.value))
     sync()
+    kerns_in_order = list(kerns)
     wall_ms = (time.perf_counter() - t0) * 1e3
     ms_per_step = wall_ms / steps
     # second figure: the same launches back to back, one wait at the end (hotter: under the package power
@@ -408,6 +423,9 @@ def measure(name, torch, hip, steps, warmup):
                      "kernel": info["kernel"], "kernel_ms": round(kernel_ms, 5), "kernel_ms_stats": stats(kerns),
                      "frac_back_to_back": round(info["work"] / (back_to_back_ms * 1e-3) / info["work_unit"] / info["peak"], 4)},
     }
+    res["warmup_steps_done"] = done
+    if TRACE_LAUNCHES:
+        res["kernel_us_by_launch"] = [round(k * 1e3) for k in kerns_in_order]
     if name == "triad_sum_2p28":
         res["roofline"]["probe_kernels_GBs"] = hbm_ceiling(torch, hip)
     if name == "gemm_bf16_8192" and not ZERO_OPERANDS:
@@ -534,13 +552,16 @@ def mfma_stream_rates(torch, hip, launches=15):
     stream = C.c_void_p(torch.cuda.current_stream().cuda_stream)
     ev = Events(hip, stream)
     times = {"mfma_stream16": [], "mfma_stream": []}
-    for i in range(launches + 3):
+    t_warm, i = time.perf_counter(), 0
+    while len(times["mfma_stream"]) < launches:
+        warm = i < 3 or (time.perf_counter() - t_warm) * 1e3 < WARMUP_MS
         for entry in times:
             ev.start()
             hip.run_source(MFMA_STREAM_SRC, entry, (512, 1, 1), (256, 1, 1), [out, ("i32", 1024), ("i32", 0)])
             ms = ev.stop_ms()
-            if i >= 3:
+            if not warm:
                 times[entry].append(ms)
+        i += 1
     flop = 256.0 * 8 * 1024 * 16 * 32768
     return tuple(round(flop / (sorted(t)[len(t) // 2] * 1e-3) / 1e12, 1) for t in times.values())
 
@@ -649,7 +670,8 @@ def main():
         print("bench.py needs a GPU", file=sys.stderr)
         sys.exit(2)
     torch.cuda.set_device(0)
-    global ZERO_OPERANDS, GEMM_SHAPE
+    global ZERO_OPERANDS, GEMM_SHAPE, WARMUP_MS, TRACE_LAUNCHES
+    WARMUP_MS, TRACE_LAUNCHES = args.warmup_ms, args.trace_launches
     ZERO_OPERANDS = args.zero_operands
     GEMM_SHAPE = tuple(int(x) for x in args.shape.split(","))
     for item in args.tunable:
@@ -665,7 +687,10 @@ def main():
         "route": head["route"], "served_by": head["served_by"], "ms_per_step_stats": head["ms_per_step_stats"],
         "value_at_median": head["value_at_median"],
         "gpu_ms_per_step_back_to_back": head["gpu_ms_per_step_back_to_back"],
+        "warmup_ms": args.warmup_ms, "warmup_steps_done": head["warmup_steps_done"],
     }
+    if args.trace_launches:
+        out["kernel_us_by_launch"] = head["kernel_us_by_launch"]
     if not args.no_cpu_baseline and args.workload not in ("copy_1gib", "vendor_gemm_bf16_8192", "mfma_bf16_stream", "mfma_bf16_stream_32x32x16"):
         out["cpu_baseline"] = cpu_baseline(args.workload)
     if not args.no_also:
