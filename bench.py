@@ -546,24 +546,26 @@ extern "C" __global__ __launch_bounds__(256) void probe_2r1w(f4* w, int nw, cons
 
 def mfma_stream_rates(torch, hip, launches=15):
     """TFLOP/s of the bare MFMA streams of MFMA_STREAM_SRC (mfma_stream16 = v_mfma_f32_16x16x32_bf16, the GEMM
-    kernel's instruction; mfma_stream = v_mfma_f32_32x32x16_bf16), JIT-compiled through the plugin path: the two are
-    launched in turn, each launch waited for, and the median launch of each is reported (16x16x32, 32x32x16)."""
+    kernel's instruction; mfma_stream = v_mfma_f32_32x32x16_bf16), JIT-compiled through the plugin path: each is
+    warmed up like a workload (WARMUP_MS of launches, each waited for, after the launch that compiles it), then the
+    median of `launches` waited launches is reported (16x16x32, 32x32x16)."""
     out = torch.zeros(256 * 512, device="cuda")
     stream = C.c_void_p(torch.cuda.current_stream().cuda_stream)
     ev = Events(hip, stream)
-    times = {"mfma_stream16": [], "mfma_stream": []}
-    t_warm, i = time.perf_counter(), 0
-    while len(times["mfma_stream"]) < launches:
-        warm = i < 3 or (time.perf_counter() - t_warm) * 1e3 < WARMUP_MS
-        for entry in times:
+    flop = 256.0 * 8 * 1024 * 16 * 32768
+    rates = []
+    for entry in ("mfma_stream16", "mfma_stream"):
+        def launch():
             ev.start()
             hip.run_source(MFMA_STREAM_SRC, entry, (512, 1, 1), (256, 1, 1), [out, ("i32", 1024), ("i32", 0)])
-            ms = ev.stop_ms()
-            if not warm:
-                times[entry].append(ms)
-        i += 1
-    flop = 256.0 * 8 * 1024 * 16 * 32768
-    return tuple(round(flop / (sorted(t)[len(t) // 2] * 1e-3) / 1e12, 1) for t in times.values())
+            return ev.stop_ms()
+        launch()
+        t_warm = time.perf_counter()
+        while (time.perf_counter() - t_warm) * 1e3 < WARMUP_MS:
+            launch()
+        times = sorted(launch() for _ in range(launches))
+        rates.append(round(flop / (times[len(times) // 2] * 1e-3) / 1e12, 1))
+    return tuple(rates)
 
 
 def event_overhead_ms(torch, hip, launches=20):
