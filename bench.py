@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the sarek-hip hot path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload NAME] [--no-also]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--warmup-ms T] [--workload NAME] [--no-also]
 
 Prints ONE JSON line.  A "step" is one pass of the workload's hot-path entry point over
 one batch of synthetic input that is already resident in HBM.  The headline workload is
@@ -19,6 +19,8 @@ waited for; benchmarks/bench_stream_triad.ml:76-116): ms_per_step is the wall ti
 timed iterations over K, ms_per_step_stats their min / median / avg / max.  The kernel time
 used for the roofline comes from HIP events recorded round the dominant launch on the launch
 stream; gpu_ms_per_step_back_to_back is the same step launched K times with one wait at the end.
+The warmup is W steps and at least --warmup-ms (60 ms) of them: after a pause the clocks of a
+power-limited kernel need 30-40 ms of load to settle (--trace-launches shows the curve).
 """
 import argparse
 import ctypes as C
