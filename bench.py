@@ -58,7 +58,7 @@ def parse():
     ap.add_argument("--workload", default="gemm_bf16_8192",
                     choices=["gemm_bf16_8192", "gemm_f16_8192", "triad_sum_2p28", "gemm_f32_8192", "gemm_f32_1024",
                              "gemm_f16_epilogue", "gemm_f16_4095x11008x4096", "gemm_f16_shape", "copy_1gib", "vendor_gemm_bf16_8192", "histogram_2p28",
-                             "radix_scatter_5e7", "mfma_bf16_stream", "mfma_bf16_stream_32x32x16"])
+                             "radix_scatter_5e7", "mfma_bf16_stream", "mfma_bf16_stream_32x32x16", "l2_to_lds_stream"])
     ap.add_argument("--warmup-ms", type=float, default=60.0,
                     help="warm up for at least this long (and at least --warmup steps): the clocks of a power-limited "
                          "kernel take 30-40 ms to settle after a pause")
@@ -238,6 +238,21 @@ def make_workload(name, torch, hip):
                     config={"workload": f"v_mfma_f32_{instr}_bf16 stream, 1.0995e12 flop over 2048 waves, register operands "
                                         + ("all zero" if zero else "N(0,0.02)-like")})
         return (lambda: hip.run_source(MFMA_STREAM_SRC, entry, (512, 1, 1), (256, 1, 1), items)), None, info, out
+    if name == "l2_to_lds_stream":
+        # The operand delivery of the 8192^3 16-bit GEMM and nothing else: 1024 workgroups of 8 waves each bring
+        # 8 MiB (a 256 x 256 tile's A and B panels at K = 8192) into LDS with buffer_load_dwordx4 ... lds, 16 transfers
+        # of 1 KiB in flight per wave, all from a 2 MiB window that the L2s hold: what the L2 -> LDS path delivers
+        # when nothing else runs and nothing misses.  peak = 64 B per clock and CU at 2.4 GHz.
+        src = torch.randint(0, 2 ** 31 - 1, ((16 << 20) // 4,), dtype=torch.int32, device="cuda", generator=g)
+        sink = torch.zeros(4, dtype=torch.int32, device="cuda")
+        wgs, per_wg, window = 1024, 8 << 20, 2 << 20
+        items = [src, sink, ("i32", per_wg // (512 * 16)), ("i32", (window // 16 - 1) & ~511), ("i32", (64 << 10) // 16)]
+        info = dict(metric="L2 -> LDS transfer GB/s (no other work, every request an L2 hit)", unit="GB/s", dtype="u8",
+                    work=float(wgs * per_wg), work_unit=1e9, bound="l2", peak=64.0 * 256 * NOMINAL_CLOCK_MHZ * 1e-3,
+                    kernel="l2_to_lds (JIT)", route="Execute.run_source ~lang:HIP_Source, text in bench.py",
+                    config={"workload": "1024 workgroups x 8 MiB by buffer_load_dwordx4 ... lds from a 2 MiB window "
+                                        "(the operand bytes of the 8192^3 16-bit GEMM with 256 x 256 tiles: 8.59 GB)"})
+        return (lambda: hip.run_source(L2_STREAM_SRC, "l2_to_lds", (512, 1, 1), (wgs, 1, 1), items)), None, info, (src, sink)
     if name == "vendor_gemm_bf16_8192":
         # the vendor library's GEMM (torch.matmul -> hipBLASLt) on the headline inputs, for
         # side-by-side profiles; it writes bf16 C where the kernel here writes f32
@@ -419,7 +434,7 @@ def measure(name, torch, hip, steps, warmup):
         "gpu_ms_per_step_back_to_back": round(back_to_back_ms, 5),
         "dtype": info["dtype"], "config": info["config"], "route": info["route"], "served_by": path,
         "roofline": {"bound": info["bound"], "achieved": round(achieved, 2), "peak": info["peak"],
-                     "unit": "GB/s" if info["bound"] == "hbm" else "TFLOP/s",
+                     "unit": "GB/s" if info["bound"] in ("hbm", "l2") else "TFLOP/s",
                      "frac": round(achieved / info["peak"], 4),
                      "traffic": MEASURED_TRAFFIC_BYTES.get(name),
                      "kernel": info["kernel"], "kernel_ms": round(kernel_ms, 5), "kernel_ms_stats": stats(kerns),
@@ -517,6 +532,32 @@ extern "C" __global__ __launch_bounds__(512) void mfma_stream16(float* out, int 
   _Pragma("unroll") for (int i = 0; i < 4; ++i)
     _Pragma("unroll") for (int j = 0; j < 4; ++j) sum += acc[i][j][0] + acc[i][j][3];
   out[blockIdx.x * 512 + threadIdx.x] = sum;
+}
+"""
+
+
+L2_STREAM_SRC = r"""
+typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
+// every workgroup walks its own start in a window of (window_mask + 512) 16-byte pieces and brings 512 x 16 bytes per
+// step into LDS; a wave keeps up to 16 transfers in flight
+extern "C" __global__ __launch_bounds__(512) void l2_to_lds(const u32x4* __restrict__ src, int nsrc, unsigned* __restrict__ sink,
+                                                           int nsink, int steps, int window_mask, int wg_stride) {
+  __shared__ __attribute__((aligned(1024))) char stage[64 * 1024];
+  const int wave = threadIdx.x >> 6;
+  unsigned pos = (blockIdx.x * (unsigned)wg_stride) & window_mask;
+  __amdgpu_buffer_rsrc_t rsrc = __builtin_amdgcn_make_buffer_rsrc((void*)src, 0, nsrc * 4, 0x00020000);
+  for (int i = 0; i < steps; i += 8) {
+    _Pragma("unroll") for (int u = 0; u < 8; ++u) {
+      const unsigned off = (((pos + u * 512) & window_mask) + threadIdx.x) << 4;
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc, (__attribute__((address_space(3))) void*)(stage + (u * 8 + wave) * 1024),
+                                               16, (int)off, 0, 0, 0);
+    }
+    __builtin_amdgcn_s_waitcnt((8 & 15) | ((8 >> 4) << 14) | (7 << 4) | (15 << 8));   // vmcnt <= 8
+    pos = (pos + 8 * 512) & window_mask;
+  }
+  __builtin_amdgcn_s_waitcnt(0);
+  __syncthreads();
+  if (*(volatile unsigned*)(stage + threadIdx.x * 4) == 0x12345678u) sink[0] = 1;
 }
 """
 
@@ -695,7 +736,7 @@ def main():
     }
     if args.trace_launches:
         out["kernel_us_by_launch"] = head["kernel_us_by_launch"]
-    if not args.no_cpu_baseline and args.workload not in ("copy_1gib", "vendor_gemm_bf16_8192", "mfma_bf16_stream", "mfma_bf16_stream_32x32x16"):
+    if not args.no_cpu_baseline and args.workload not in ("copy_1gib", "vendor_gemm_bf16_8192", "mfma_bf16_stream", "mfma_bf16_stream_32x32x16", "l2_to_lds_stream"):
         out["cpu_baseline"] = cpu_baseline(args.workload)
     if not args.no_also:
         also = []
