@@ -57,7 +57,8 @@ def parse():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--workload", default="gemm_bf16_8192",
                     choices=["gemm_bf16_8192", "gemm_f16_8192", "triad_sum_2p28", "gemm_f32_8192", "gemm_f32_1024",
-                             "gemm_f16_epilogue", "gemm_f16_4095x11008x4096", "gemm_f16_shape", "copy_1gib", "vendor_gemm_bf16_8192", "histogram_2p28",
+                             "gemm_f16_epilogue", "gemm_f16_4095x11008x4096", "gemm_f16_shape", "gemm_bf16_shape", "copy_1gib",
+                             "vendor_gemm_bf16_8192", "vendor_gemm_bf16_shape", "histogram_2p28",
                              "radix_scatter_5e7", "mfma_bf16_stream", "mfma_bf16_stream_32x32x16", "l2_to_lds_stream"])
     ap.add_argument("--warmup-ms", type=float, default=60.0,
                     help="warm up for at least this long (and at least --warmup steps): the clocks of a power-limited "
@@ -253,19 +254,19 @@ def make_workload(name, torch, hip):
                     config={"workload": "1024 workgroups x 8 MiB by buffer_load_dwordx4 ... lds from a 2 MiB window "
                                         "(the operand bytes of the 8192^3 16-bit GEMM with 256 x 256 tiles: 8.59 GB)"})
         return (lambda: hip.run_source(L2_STREAM_SRC, "l2_to_lds", (512, 1, 1), (wgs, 1, 1), items)), None, info, (src, sink)
-    if name == "vendor_gemm_bf16_8192":
-        # the vendor library's GEMM (torch.matmul -> hipBLASLt) on the headline inputs, for
+    if name in ("vendor_gemm_bf16_8192", "vendor_gemm_bf16_shape"):
+        # the vendor library's GEMM (torch.matmul -> hipBLASLt) on the headline inputs or on --shape, for
         # side-by-side profiles; it writes bf16 C where the kernel here writes f32
-        s = 8192
+        m, n, k = (8192, 8192, 8192) if name == "vendor_gemm_bf16_8192" else GEMM_SHAPE
         g.manual_seed(0xA4)
-        a = (torch.randn(s, s, device="cuda", generator=g) * 0.02).bfloat16()
+        a = (torch.randn(m, k, device="cuda", generator=g) * 0.02).bfloat16()
         g.manual_seed(0xB4)
-        b = (torch.randn(s, s, device="cuda", generator=g) * 0.02).bfloat16()
-        c = torch.empty(s, s, device="cuda", dtype=torch.bfloat16)
-        info = dict(metric="vendor library GEMM TFLOP/s at 8192^3 (bf16 in, bf16 out)", unit="TFLOP/s",
-                    dtype="bf16", work=2.0 * s ** 3, work_unit=1e12, bound="mfma",
+        b = (torch.randn(k, n, device="cuda", generator=g) * 0.02).bfloat16()
+        c = torch.empty(m, n, device="cuda", dtype=torch.bfloat16)
+        info = dict(metric=f"vendor library GEMM TFLOP/s at {m}x{n}x{k} (bf16 in, bf16 out)", unit="TFLOP/s",
+                    dtype="bf16", work=2.0 * m * n * k, work_unit=1e12, bound="mfma",
                     peak=PEAK_MFMA_TFLOPS["bf16"], kernel="hipBLASLt (torch.matmul)", route="torch.matmul",
-                    config={"workload": "torch.matmul bf16, N(0,0.02)", "m": s, "n": s, "k": s})
+                    config={"workload": "torch.matmul bf16, N(0,0.02)", "m": m, "n": n, "k": k})
         return (lambda: torch.matmul(a, b, out=c)), None, info, None
     if name == "histogram_2p28":
         n = 1 << 28
@@ -313,28 +314,34 @@ def make_workload(name, torch, hip):
                     config={"workload": "out[counters[key & 255]++] = key, random keys below 100000", "n": n,
                             "algorithmic_bytes": 8 * n})
         return main, None, info, (vk, vo, vcnt, starts, a, ir)
-    if name in ("gemm_f16_4095x11008x4096", "gemm_f16_shape"):
+    if name in ("gemm_f16_4095x11008x4096", "gemm_f16_shape", "gemm_bf16_shape"):
         # the epilogue config's product without the epilogue (what the fused chain costs on top), or any --shape
-        m, n, k = (4095, 11008, 4096) if name != "gemm_f16_shape" else GEMM_SHAPE
+        m, n, k = (4095, 11008, 4096) if name == "gemm_f16_4095x11008x4096" else GEMM_SHAPE
+        bf16 = name == "gemm_bf16_shape"
+        dt = torch.bfloat16 if bf16 else torch.float16
         g.manual_seed(0xA5)
-        t = (torch.randn(m, k, device="cuda", generator=g) * 0.02).half()
+        t = (torch.randn(m, k, device="cuda", generator=g) * 0.02).to(dt)
         va = device_vector(sarek, hip, torch, t, elem_size=2)
         g.manual_seed(0xB5)
-        t = (torch.randn(k, n, device="cuda", generator=g) * 0.02).half()
+        t = (torch.randn(k, n, device="cuda", generator=g) * 0.02).to(dt)
         vb = device_vector(sarek, hip, torch, t, elem_size=2)
         del t
         vy = V.create(V.float32, m * n)
         sarek.Transfer.to_device(vy)
-        src, entry = hip.library_kernel("gemm_f16")
+        src, entry = hip.library_kernel("gemm_bf16" if bf16 else "gemm_f16")
         a, na = E._args([E.Vec(va), E.Vec(vb), E.Vec(vy), E.Int32(m), E.Int32(n), E.Int32(k)])
         src_b, entry_b = src.encode(), entry.encode()
         main = Launch(hip, lib.sarek_hip_execute_run_source, src_b, hip.LANG_HIP, entry_b, dims(16, 16, 1),
                       dims((n + 15) // 16, (m + 15) // 16, 1), 0, 1, a, na)
-        info = dict(metric=f"fp16 GEMM TFLOP/s at {m}x{n}x{k}", unit="TFLOP/s", dtype="f16",
+        tn = "bf16" if bf16 else "f16"
+        tile = hip.gemm16_tile(m, n, k)
+        kern = {256: "gemm16_m16_kernel", 128: "gemm16_m16_small_kernel"}.get(tile, "gemm16_staged_kernel")
+        info = dict(metric=f"{tn} GEMM TFLOP/s at {m}x{n}x{k}", unit="TFLOP/s", dtype=tn,
                     work=2.0 * m * n * k, work_unit=1e12, bound="mfma",
-                    peak=PEAK_MFMA_TFLOPS["f16"], kernel="gemm16_m16_kernel<f16, store>",
-                    route="Execute.run_source ~lang:HIP_Source, library kernel text 'gemm_f16'",
-                    config={"workload": "fp16-in f32-acc C=A.B", "m": m, "n": n, "k": k})
+                    peak=PEAK_MFMA_TFLOPS[tn], kernel=f"{kern}<{tn}, store>",
+                    route=f"Execute.run_source ~lang:HIP_Source, library kernel text 'gemm_{tn}'",
+                    config={"workload": f"{tn}-in f32-acc C=A.B, N(0,0.02)", "m": m, "n": n, "k": k,
+                            "workgroup_tile": tile})
         return main, None, info, (va, vb, vy, a, src_b, entry_b)
     if name == "gemm_f16_epilogue":
         m, n, k = 4095, 11008, 4096
@@ -736,7 +743,7 @@ def main():
     }
     if args.trace_launches:
         out["kernel_us_by_launch"] = head["kernel_us_by_launch"]
-    if not args.no_cpu_baseline and args.workload not in ("copy_1gib", "vendor_gemm_bf16_8192", "mfma_bf16_stream", "mfma_bf16_stream_32x32x16", "l2_to_lds_stream"):
+    if not args.no_cpu_baseline and args.workload not in ("copy_1gib", "vendor_gemm_bf16_8192", "vendor_gemm_bf16_shape", "gemm_bf16_shape", "gemm_f16_shape", "mfma_bf16_stream", "mfma_bf16_stream_32x32x16", "l2_to_lds_stream"):
         out["cpu_baseline"] = cpu_baseline(args.workload)
     if not args.no_also:
         also = []

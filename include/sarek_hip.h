@@ -540,6 +540,14 @@ int sarek_hip_gemm_bf16(const uint16_t *a, const uint16_t *b, float *c, int m, i
 int sarek_hip_gemm_f16(const uint16_t *a, const uint16_t *b, float *c, int m, int n, int k,
                        sarek_hip_stream stream);
 
+/* Which kernel the three 16-bit GEMM entry points take for a shape under the
+ * present tunables: 256 or 128 = the workgroup tile of the direct-to-LDS MFMA
+ * kernels (the small tile where large ones would leave CUs idle), 0 = the
+ * staged or the one-thread-per-element kernel (n or k not a multiple of 8, k
+ * not a multiple of 64, ...).  No counterpart in the reference, whose tiled
+ * kernel has one shape (bench_matrix_mul_tiled.ml:55-95); needs no device.  */
+int sarek_hip_gemm16_tile(int m, int n, int k);
+
 /* Fused epilogue chain: y = relu(A.B + bias[col]) (f32, [m x n]) and
  * rowsum[r] = sum_c y[r,c] (f32, [m]).  fp16 inputs.                        */
 int sarek_hip_gemm_f16_bias_relu_rowsum(const uint16_t *a, const uint16_t *b, const float *bias,

@@ -16,7 +16,8 @@
 //      4*(i%4), and receives column i of that 4 x 16 block (its 4 rows).  Two such reads
 //      (rows 0-3 and 4-7 of the lane's k range) give the 8 k values.
 //
-// Three kernels:
+// Kernels (the default fast path is gemm16_m16_kernel on v_mfma_f32_16x16x32 below, with gemm16_m16_small_kernel for
+// products that do not fill the chip; the three described here are the 32 x 32 x 16 kernel and the fallbacks):
 //   gemm16_dma_kernel (K % 64 == 0, the fast path): global -> LDS by
 //     buffer_load_dwordx4 ... lds, which writes the 64 lanes' 16-byte pieces to 1 KiB of
 //     consecutive LDS with no register staging and no ds_write (the buffer form: the
@@ -476,15 +477,19 @@ __device__ __forceinline__ f32x4_t mfma16(u32x4 a, u32x4 b, f32x4_t c) {
                                                   0, 0);
 }
 
-// Writes one wave's 128 x 64 block held as 8 x 4 tiles of 16 x 16 (register r of lane l: row 4*(l/16) + r, column
-// l%16 of its tile).  Fused form as in `epilogue`: per lane the sum over its four columns for each of its 32 rows,
-// a halving butterfly over the 16 lanes that share those rows (16+8+4+2 exchanges leave lane m with rows 2m, 2m+1
-// of the 32), the four waves along N through LDS, one atomicAdd per row.
-template <int Epi>
-__device__ __forceinline__ void epilogue16(f32x4_t (&acc)[8][4], float *__restrict__ C, const float *__restrict__ bias,
+// Writes one wave's (16*TI) x 64 block held as TI x 4 tiles of 16 x 16 (register r of lane l: row 4*(l/16) + r, column
+// l%16 of its tile); TI = 8 in the 256 x 256 workgroup tile (2 x 4 waves), 4 in the 128 x 128 one (2 x 2 waves).
+// Fused form as in `epilogue`: per lane the sum over its four columns for each of its 4*TI rows, a halving butterfly
+// over the 16 lanes that share those rows (with TI = 8: 16+8+4+2 exchanges leave lane m with rows 2m, 2m+1 of the 32;
+// with TI = 4: 8+4+2+1 leave it with row m of the 16), the WNW waves along N through LDS, one atomicAdd per row.
+template <int Epi, int TI = 8, int WNW = 4>
+__device__ __forceinline__ void epilogue16(f32x4_t (&acc)[TI][4], float *__restrict__ C, const float *__restrict__ bias,
                                            float *__restrict__ rowsum, int M, int N, int m0, int wm, int wn, int col0,
                                            int l16, int g, float *scratch) {
-  const int row0 = m0 + wm * 128;
+  constexpr int WROWS = 16 * TI, TROWS = 2 * WROWS, NV = 4 * TI, E = NV / 16;
+  static_assert(TI == 8 || TI == 4, "wave tiles of 128 or 64 rows");
+  static_assert(WNW == 4 || WNW == 2, "four or two waves along N");
+  const int row0 = m0 + wm * WROWS;
   float bj[4];
   bool cok[4];
 #pragma unroll
@@ -493,9 +498,9 @@ __device__ __forceinline__ void epilogue16(f32x4_t (&acc)[8][4], float *__restri
     cok[j] = col < N;
     bj[j] = (Epi == EPI_BIAS_RELU_ROWSUM && cok[j]) ? bias[col] : 0.f;
   }
-  float rs[32];
+  float rs[NV];
 #pragma unroll
-  for (int i = 0; i < 8; ++i) {
+  for (int i = 0; i < TI; ++i) {
 #pragma unroll
     for (int r = 0; r < 4; ++r) {
       const int row = row0 + i * 16 + 4 * g + r;
@@ -516,12 +521,12 @@ __device__ __forceinline__ void epilogue16(f32x4_t (&acc)[8][4], float *__restri
   if constexpr (Epi == EPI_BIAS_RELU_ROWSUM) {
 #pragma unroll
     for (int step = 0; step < 4; ++step) {
-      const int m = 8 >> step, half = 16 >> step;
+      const int m = 8 >> step, half = (NV / 2) >> step;
       const bool up = (l16 & m) != 0;
 #pragma unroll
       for (int q = 0; q < half; ++q) {
         // both values in registers before the selects: otherwise the compiler turns the selects into one
-        // lane-indexed read of rs[] (a compare-and-select chain over all 32 registers per value)
+        // lane-indexed read of rs[] (a compare-and-select chain over all its registers per value)
         float lo = rs[q], hi = rs[q + half];
         asm volatile("" : "+v"(lo), "+v"(hi));
         const float send = up ? lo : hi;
@@ -529,17 +534,19 @@ __device__ __forceinline__ void epilogue16(f32x4_t (&acc)[8][4], float *__restri
         rs[q] = keep + __shfl_xor(send, m, 64);
       }
     }
-    // lane l16 now holds rows q = 2*l16 + e (e = 0, 1) of its 16-lane group's 32 rows: tile q/4, register q%4
+    // lane l16 now holds rows q = E*l16 + e (e < E) of its 16-lane group's 4*TI rows: tile q/4, register q%4
     __syncthreads();  // every wave has left the K loop: the LDS ring is free
 #pragma unroll
-    for (int e = 0; e < 2; ++e) {
-      const int q = 2 * l16 + e;
-      scratch[wn * 256 + wm * 128 + (q >> 2) * 16 + 4 * g + (q & 3)] = rs[e];
+    for (int e = 0; e < E; ++e) {
+      const int q = E * l16 + e;
+      scratch[wn * TROWS + wm * WROWS + (q >> 2) * 16 + 4 * g + (q & 3)] = rs[e];
     }
     __syncthreads();
     const int t = threadIdx.x;
-    if (t < 256 && m0 + t < M) {
-      const float total = (scratch[t] + scratch[256 + t]) + (scratch[512 + t] + scratch[768 + t]);
+    if (t < TROWS && m0 + t < M) {
+      float total;
+      if constexpr (WNW == 4) total = (scratch[t] + scratch[TROWS + t]) + (scratch[2 * TROWS + t] + scratch[3 * TROWS + t]);
+      else total = scratch[t] + scratch[TROWS + t];
       atomicAdd(rowsum + m0 + t, total);
     }
   }
@@ -755,6 +762,200 @@ __global__ __launch_bounds__(512) void gemm16_m16_kernel(const uint16_t *__restr
   }
 }
 
+// The same pipeline on a 128 x 128 workgroup tile, for products whose 256 x 256 tiles would leave most CUs idle:
+// 4 waves (2 x 2) of 64 x 64 = 4 x 4 tiles of v_mfma_f32_16x16x32, A in 3 stages of K = 64 and B in 4 slabs of K = 32
+// (80 KiB of LDS: two workgroups per CU fill its 160 KiB).  A small tile needs twice the operand bytes per flop and has
+// a quarter of the MFMA work per slab to cover their latency with, so the ring depth is what its speed hangs on: the
+// third A stage (transfers 4 slabs ahead instead of 2) is worth 3-7 %, and two resident workgroups run at twice the
+// rate of one.  B rows are 256 bytes here; they start on bank 0 like the 512-byte
+// rows of the large tile, so the same XOR swizzle keeps the transposing reads free of bank conflicts.  A slab is 16 MFMAs:
+// rows 0-31 of the wave tile before the barrier, rows 32-63 after it with the next slab's 12 fragment reads (and, every
+// other slab, the 4 transfers of an A stage) behind them; fragments are double-buffered by slab parity.
+template <bool Bf16, int Epi>
+__global__ __launch_bounds__(256) void gemm16_m16_small_kernel(const uint16_t *__restrict__ A, const uint16_t *__restrict__ B,
+                                                               float *__restrict__ C, const float *__restrict__ bias,
+                                                               float *__restrict__ rowsum, int M, int N, int K, int tiles_m,
+                                                               int tiles_n, int xcd_remap, unsigned long long *probe) {
+  constexpr int SBM = 128, SBN = 128;
+  constexpr int BKA = 64, BKB = 32, NA = 3, NB = 4;
+  constexpr int RA = BKA / BKB;
+  constexpr int A_ROW = BKA * 2, A_CHUNKS = A_ROW / 16, A_ROWS_PER_DMA = 1024 / A_ROW;
+  constexpr int B_ROW = SBN * 2, B_CHUNKS = B_ROW / 16, B_ROWS_PER_DMA = 1024 / B_ROW;
+  constexpr int A_BYTES_S = SBM * A_ROW, B_BYTES_S = BKB * B_ROW;
+  constexpr int NWAVES = 4, WN = 2;
+  constexpr int DA = A_BYTES_S / 1024 / NWAVES, DB = B_BYTES_S / 1024 / NWAVES;
+  constexpr int P = lcm_int(NB, RA * NA);
+  static_assert(P % 2 == 0, "the fragment buffers alternate by slab parity");
+  static_assert(2 * (NA * A_BYTES_S + NB * B_BYTES_S) <= 160 * 1024, "two workgroups per CU");
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int wm = wave / WN, wn = wave % WN;
+  const int l16 = lane & 15, g = lane >> 4;
+  int tm, tn;
+  tile_of_block(tiles_m, tiles_n, xcd_remap, tm, tn);
+  const int m0 = tm * SBM, n0 = tn * SBN;
+  long long probe_c0 = 0, probe_t0 = 0;
+  if (probe) {
+    probe_c0 = clock64();
+    probe_t0 = wall_clock64();
+  }
+  auto a_swz = [](int row) { return (row >> 1) & 7; };
+  auto b_swz = [](int row) { return ((row & 3) << 2) | (((row >> 3) & 1) << 1); };
+
+  // DMA sources (rows past M and columns past N clamped: what they bring is never stored)
+  uint32_t a_off[DA], b_off[DB];
+#pragma unroll
+  for (int i = 0; i < DA; ++i) {
+    const int q = wave + NWAVES * i;
+    const int arow_t = q * A_ROWS_PER_DMA + lane / A_CHUNKS;
+    const int arow = min(arow_t, M - 1 - m0);
+    a_off[i] = (static_cast<uint32_t>(arow) * K + (((lane % A_CHUNKS) ^ a_swz(arow_t)) << 3)) * 2u;
+  }
+#pragma unroll
+  for (int i = 0; i < DB; ++i) {
+    const int q = wave + NWAVES * i;
+    const int brow = q * B_ROWS_PER_DMA + lane / B_CHUNKS;
+    const int bchunk = (lane % B_CHUNKS) ^ b_swz(brow);
+    const int bcol = min(n0 + bchunk * 8, N - 8);
+    b_off[i] = (static_cast<uint32_t>(brow) * N + bcol) * 2u;
+  }
+  const char *a_base = reinterpret_cast<const char *>(A + static_cast<int64_t>(m0) * K);
+  const int64_t b_slab_bytes = static_cast<int64_t>(BKB) * N * 2;
+  const int nslabs = K / BKB, nstages = K / BKA;
+
+  f32x4_t acc[4][4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i)
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+#pragma unroll
+      for (int r = 0; r < 4; ++r) acc[i][j][r] = 0.f;
+
+  const int a_row = wm * 64 + l16;
+  int a_addr0 = a_row * A_ROW + ((g ^ a_swz(a_row)) << 4);
+  const int b_r = l16 >> 2;
+  int b_addr0 = (g * 8 + b_r) * B_ROW + ((wn * 128 + (l16 & 3) * 8) ^ ((b_r << 6) | ((g & 1) << 5)));
+
+  const __amdgpu_buffer_rsrc_t a_rsrc = make_rsrc(a_base, 0x80000000u);
+  auto issue_a = [&](char *sa, int stage) {
+    const uint32_t a_so = static_cast<uint32_t>(min(stage, nstages - 1)) * (BKA * 2);
+#pragma unroll
+    for (int i = 0; i < DA; ++i) dma16(a_rsrc, a_off[i], a_so, sa + (wave + NWAVES * i) * 1024);
+  };
+  // B slabs go out in order; the source is a running pointer that stops at the last slab (the tail of the K loop
+  // re-issues it into stages nobody reads any more, so the count of transfers in flight keeps its pattern)
+  const char *b_src = reinterpret_cast<const char *>(B);
+  int b_next = 0;
+  auto issue_b = [&](char *sb) {
+    const __amdgpu_buffer_rsrc_t b_rsrc = make_rsrc(b_src, 0x80000000u);
+#pragma unroll
+    for (int i = 0; i < DB; ++i) dma16(b_rsrc, b_off[i], 0u, sb + (wave + NWAVES * i) * 1024);
+    ++b_next;
+    if (b_next < nslabs) b_src += b_slab_bytes;
+  };
+  auto load_a1 = [&](const char *sa, int ks, int i, u32x4 &af) {
+    af = *reinterpret_cast<const u32x4 *>(sa + (a_addr0 ^ (ks << 6)) + i * 16 * A_ROW);
+  };
+  auto load_b = [&](const char *sb, u32x4 (&bf)[4]) {
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int off = b_addr0 ^ (j << 5);
+      u32x2 lo = lds_read_tr16(sb, off);
+      u32x2 hi = lds_read_tr16(sb, off + 4 * B_ROW);
+      bf[j] = u32x4{lo.x, lo.y, hi.x, hi.y};
+    }
+  };
+  // MFMAs First .. First+Count-1 of a slab's 16, in the order (row tile i, column tile j)
+  auto mfma_range = [&](auto first_c, auto count_c, u32x4 (&af)[4], u32x4 (&bf)[4]) {
+    constexpr int First = decltype(first_c)::value, Count = decltype(count_c)::value;
+    [&]<int... Ts>(std::integer_sequence<int, Ts...>) {
+      ((acc[(First + Ts) / 4][(First + Ts) % 4] =
+            mfma16<Bf16>(af[(First + Ts) / 4], bf[(First + Ts) % 4], acc[(First + Ts) / 4][(First + Ts) % 4])),
+       ...);
+    }(std::make_integer_sequence<int, Count>{});
+  };
+  // Issue order: the T = NV + READS other instructions (DMA, LDS reads) go behind the MFMAs of the section, item k behind
+  // MFMA (k * MFMAS) / T (two per MFMA where T > MFMAS), the DMA instructions evenly among the reads
+  auto spread = [](auto nv_c, auto reads_c, auto mfmas_c) {
+    constexpr int NV = decltype(nv_c)::value, READS = decltype(reads_c)::value, MFMAS = decltype(mfmas_c)::value;
+    constexpr int T = NV + READS;
+    [&]<int... Ms>(std::integer_sequence<int, Ms...>) {
+      (([] {
+         __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+         constexpr int k0 = (Ms * T + MFMAS - 1) / MFMAS, k1 = ((Ms + 1) * T + MFMAS - 1) / MFMAS;
+         [&]<int... Ks>(std::integer_sequence<int, Ks...>) {
+           (([] {
+              constexpr int k = k0 + Ks;
+              if constexpr (NV > 0 && (k * NV) / T != ((k + 1) * NV) / T) __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
+              else __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+            }()),
+            ...);
+         }(std::make_integer_sequence<int, (k1 < T ? k1 : T) - (k0 < T ? k0 : T)>{});
+       }()),
+       ...);
+    }(std::make_integer_sequence<int, MFMAS>{});
+    __builtin_amdgcn_sched_barrier(0);
+  };
+  u32x4 af[2][4], bf[2][4];   // [slab parity]
+
+  auto slab = [&](auto ic, int s) {
+    constexpr int I = decltype(ic)::value;
+    constexpr int In = (I + 1) % P;
+    constexpr int ia = (I / RA) % NA, ibp = (I + NB - 1) % NB;
+    constexpr int ian = (In / RA) % NA, ibn = In % NB;
+    constexpr int ksn = In % RA;
+    asm volatile("" : "+v"(a_addr0), "+v"(b_addr0));
+    issue_b(lds_ring<40 + ibp, B_BYTES_S>);
+    mfma_range(std::integral_constant<int, 0>{}, std::integral_constant<int, 8>{}, af[I & 1], bf[I & 1]);
+    spread(std::integral_constant<int, DB>{}, std::integral_constant<int, 0>{}, std::integral_constant<int, 8>{});
+    __builtin_amdgcn_s_waitcnt(waitcnt_vm_lgkm0(dma_allowed_in_flight(I, RA, NA, NB, DA, DB)));
+    barrier_no_fence();
+    if constexpr (I % RA == RA - 1) issue_a(lds_ring<30 + ia, A_BYTES_S>, s / RA + NA);
+    // the next slab's fragments in the order its first MFMAs need them
+    load_a1(lds_ring<30 + ian, A_BYTES_S>, ksn, 0, af[In & 1][0]);
+    load_b(lds_ring<40 + ibn, B_BYTES_S>, bf[In & 1]);
+    load_a1(lds_ring<30 + ian, A_BYTES_S>, ksn, 1, af[In & 1][1]);
+    load_a1(lds_ring<30 + ian, A_BYTES_S>, ksn, 2, af[In & 1][2]);
+    load_a1(lds_ring<30 + ian, A_BYTES_S>, ksn, 3, af[In & 1][3]);
+    mfma_range(std::integral_constant<int, 8>{}, std::integral_constant<int, 8>{}, af[I & 1], bf[I & 1]);
+    spread(std::integral_constant<int, (I % RA == RA - 1) ? DA : 0>{}, std::integral_constant<int, 12>{},
+           std::integral_constant<int, 8>{});
+  };
+
+  // prologue: fill both rings except the last B stage (the top of slab 0 issues it) and wait for all of it
+  [&]<int... Is>(std::integer_sequence<int, Is...>) {
+    (issue_a(lds_ring<30 + Is, A_BYTES_S>, Is), ...);
+  }(std::make_integer_sequence<int, NA>{});
+  [&]<int... Is>(std::integer_sequence<int, Is...>) {
+    (issue_b(lds_ring<40 + Is, B_BYTES_S>), ...);
+  }(std::make_integer_sequence<int, NB - 1>{});
+  __builtin_amdgcn_s_waitcnt(waitcnt_vm_lgkm0(0));
+  barrier_no_fence();
+#pragma unroll
+  for (int i = 0; i < 4; ++i) load_a1(lds_ring<30, A_BYTES_S>, 0, i, af[0][i]);
+  load_b(lds_ring<40, B_BYTES_S>, bf[0]);
+  __builtin_amdgcn_sched_barrier(0);
+
+  const int full = nslabs - nslabs % P;
+  for (int s = 0; s < full; s += P) {
+    [&]<int... Is>(std::integer_sequence<int, Is...>) {
+      (slab(std::integral_constant<int, Is>{}, s + Is), ...);
+    }(std::make_integer_sequence<int, P>{});
+  }
+  [&]<int... Is>(std::integer_sequence<int, Is...>) {
+    ((full + Is < nslabs ? slab(std::integral_constant<int, Is>{}, full + Is) : (void)0), ...);
+  }(std::make_integer_sequence<int, P - 1>{});
+  __builtin_amdgcn_s_waitcnt(waitcnt_vm_lgkm0(0));   // drain the (redundant) tail DMA before the LDS is released
+  epilogue16<Epi, 4, WN>(acc, C, bias, rowsum, M, N, m0, wm, wn, n0 + wn * 64, l16, g,
+                         reinterpret_cast<float *>(lds_ring<30, A_BYTES_S>));
+  if (probe && tid == 0) {
+    probe[2 * blockIdx.x] = static_cast<unsigned long long>(clock64() - probe_c0);
+    probe[2 * blockIdx.x + 1] = static_cast<unsigned long long>(wall_clock64() - probe_t0);
+  }
+}
+
 template <bool Bf16, int Epi>
 __global__ __launch_bounds__(THREADS) void gemm16_staged_kernel(const uint16_t *__restrict__ A,
                                                          const uint16_t *__restrict__ B,
@@ -907,6 +1108,41 @@ __global__ void zero_f32_kernel(float *p, int n) {
   if (i < n) p[i] = 0.f;
 }
 
+// Whether the 128 x 128 tile beats the 256 x 256 one.  Measured on MI355X: large tiles run in rounds of one per CU;
+// small tiles in rounds of two per CU, and such a round takes 0.6-0.65 of a large tile's time whether the CUs hold one
+// or two of them (2048^3: 64 large tiles 44.6 us, 256 small ones 28.8; 4096^3: 105 against 127 us).  The small tile is
+// taken when that estimate is at least a tenth ahead (with every CU busy on a long K its extra operand traffic costs
+// clock under the power limit: 4096 x 2048 x 8192 gains 9 % where the estimate says 35 %).
+inline bool small_tile_wins(int m, int n) {
+  static const int cus = [] {
+    int dev = 0, v = 0;
+    if (hipGetDevice(&dev) != hipSuccess ||
+        hipDeviceGetAttribute(&v, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || v <= 0)
+      v = 256;
+    return v;
+  }();
+  const int64_t large = static_cast<int64_t>((m + 255) / 256) * ((n + 255) / 256);
+  const int64_t small = static_cast<int64_t>((m + 127) / 128) * ((n + 127) / 128);
+  const double cost_large = static_cast<double>((large + cus - 1) / cus);
+  const double cost_small = 0.65 * static_cast<double>((small + 2 * cus - 1) / (2 * cus));
+  return cost_small < 0.9 * cost_large;
+}
+
+// The workgroup tile of the direct-to-LDS kernels for this shape under the present tunables (256 or 128), or 0 when
+// the shape goes to the staged or the simple kernel (pointer alignment, which can also send a call there, is not a
+// property of the shape and is not looked at).
+int gemm16_tile_for(int m, int n, int k) {
+  if (m < 1 || n < 1 || k < 1) return 0;
+  if (k % 8 != 0 || n % 8 != 0 || tunable("gemm16.force_simple", 0) != 0) return 0;
+  const bool offsets_ok = static_cast<int64_t>(k) * 256 * 2 < 0x7FFFFFFF && static_cast<int64_t>(n) * 64 * 2 < 0x7FFFFFFF;
+  if (k % BK != 0 || !offsets_ok || tunable("gemm16.force_staged", 0) != 0) return 0;
+  const bool m16 = tunable("gemm16.ring", 0) == 0 && tunable("gemm16.tj", 2) == 2 && tunable("gemm16.mfma", 16) == 16;
+  if (!m16 || tunable("gemm16.ablate", 0) != 0) return 256;
+  // gemm16.tile: 256 | 128 forces the tile, 0 (default) picks by the tile counts
+  const int tile = (int)tunable("gemm16.tile", 0);
+  return (tile == 128 || (tile == 0 && small_tile_wins(m, n))) ? 128 : 256;
+}
+
 template <bool Bf16, int Epi>
 int launch_gemm16(const uint16_t *a, const uint16_t *b, float *c, const float *bias, float *rowsum,
                   int m, int n, int k, hipStream_t st) {
@@ -975,6 +1211,13 @@ int launch_gemm16(const uint16_t *a, const uint16_t *b, float *c, const float *b
         return check_launch("gemm16 kernel launch");
       }
       if (m16) {
+        if (gemm16_tile_for(m, n, k) == 128) {
+          const int sm = (m + 127) / 128, sn = (n + 127) / 128;
+          unsigned long long *sprobe = clock_probe(static_cast<int64_t>(sm) * sn);
+          hipLaunchKernelGGL((gemm16_m16_small_kernel<Bf16, Epi>), dim3(sm * sn), dim3(256), 0, st, a, b, c, bias, rowsum,
+                             m, n, k, sm, sn, remap, sprobe);
+          return check_launch("gemm16 kernel launch");
+        }
         hipLaunchKernelGGL((gemm16_m16_kernel<Bf16, Epi>), grid, dim3(512), 0, st, a, b, c, bias, rowsum, m, n, k,
                            tiles_m, tiles_n, remap, probe);
         return check_launch("gemm16 kernel launch");
@@ -1011,6 +1254,8 @@ int launch_gemm16(const uint16_t *a, const uint16_t *b, float *c, const float *b
 using namespace sarek_hip;
 
 extern "C" {
+
+int sarek_hip_gemm16_tile(int m, int n, int k) { return gemm16_tile_for(m, n, k); }
 
 int sarek_hip_gemm_bf16(const uint16_t *a, const uint16_t *b, float *c, int m, int n, int k,
                         sarek_hip_stream stream) {

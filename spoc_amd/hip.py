@@ -138,6 +138,7 @@ SYMBOLS = {
     "sarek_hip_gemm_f32": (_i, [_vp, _vp, _vp, _i, _i, _i, _vp]),
     "sarek_hip_gemm_bf16": (_i, [_vp, _vp, _vp, _i, _i, _i, _vp]),
     "sarek_hip_gemm_f16": (_i, [_vp, _vp, _vp, _i, _i, _i, _vp]),
+    "sarek_hip_gemm16_tile": (_i, [_i, _i, _i]),
     "sarek_hip_gemm_f16_bias_relu_rowsum": (_i, [_vp, _vp, _vp, _vp, _vp, _i, _i, _i, _vp]),
     "sarek_hip_cast_f32_to_bf16": (_i, [_vp, _vp, _i64, _vp]),
     "sarek_hip_cast_f32_to_f16": (_i, [_vp, _vp, _i64, _vp]),
@@ -579,6 +580,11 @@ def _gemm16(fn, dtype, a, b, out):
 
 def gemm_bf16(a, b, out=None):
     return _gemm16(lib.sarek_hip_gemm_bf16, _torch().bfloat16, a, b, out)
+
+
+def gemm16_tile(m, n, k):
+    """256 / 128: the workgroup tile the 16-bit GEMMs take for this shape now; 0: the staged or simple kernel."""
+    return int(lib.sarek_hip_gemm16_tile(m, n, k))
 
 
 def gemm_f16(a, b, out=None):

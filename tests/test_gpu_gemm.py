@@ -245,9 +245,17 @@ def test_clock_probe_records_cycles_and_ticks(hip, torch_cuda):
     a = torch.randn(m, k, device="cuda").to(torch.bfloat16)
     b = torch.randn(k, n, device="cuda").to(torch.bfloat16)
     with hip.clock_probe(workgroups=64) as probe:
-        hip.gemm_bf16(a, b)                      # 16 workgroups of 256 x 256
+        hip.gemm_bf16(a, b)                      # 64 workgroups of 128 x 128 (16 large tiles would idle most CUs)
         pairs = probe.pairs()
-        assert len(pairs) == 16
+        assert hip.gemm16_tile(m, n, k) == 128 and len(pairs) == 64
+        assert 500 < probe.mhz() < 2600
+        probe.buf.zero_()
+        hip.set_tunable("gemm16.tile", 256)
+        try:
+            hip.gemm_bf16(a, b)                  # 16 workgroups of 256 x 256
+        finally:
+            hip.set_tunable("gemm16.tile", 0)
+        assert len(probe.pairs()) == 16
         assert 500 < probe.mhz() < 2600
         probe.buf.zero_()
         hip.gemm_bf16(torch.zeros(4096, 64, device="cuda", dtype=torch.bfloat16),
@@ -289,12 +297,14 @@ def test_gemm16_every_ring_shape(hip, oracle, torch_cuda, ring, tj, mfma, m, n, 
     hip.set_tunable("gemm16.ring", ring)
     hip.set_tunable("gemm16.tj", tj)
     hip.set_tunable("gemm16.mfma", mfma)
+    hip.set_tunable("gemm16.tile", 256)   # these are shapes of the 256 x 256 kernels
     try:
         c = hip.gemm_bf16(dev(torch_cuda, a).bfloat16(), dev(torch_cuda, b).bfloat16()).cpu().numpy()
     finally:
         hip.set_tunable("gemm16.ring", 0)
         hip.set_tunable("gemm16.tj", 2)
         hip.set_tunable("gemm16.mfma", 16)
+        hip.set_tunable("gemm16.tile", 0)
     assert np.abs(c - ref).max() / np.abs(ref).max() < 1e-4
 
 
@@ -311,6 +321,7 @@ def test_gemm16_both_mfma_shapes_agree_with_the_oracle_and_each_other(hip, oracl
     da, db = dev(torch, a).to(dt), dev(torch, b).to(dt)
     ref = oracle.gemm(a, b)
     got = {}
+    hip.set_tunable("gemm16.tile", 256)
     try:
         for mfma in (16, 32):
             hip.set_tunable("gemm16.mfma", mfma)
@@ -324,4 +335,54 @@ def test_gemm16_both_mfma_shapes_agree_with_the_oracle_and_each_other(hip, oracl
                 assert np.abs(rs.cpu().numpy() - rs_ref).max() <= 1e-4 * max(np.abs(rs_ref).max(), 1e-30)
     finally:
         hip.set_tunable("gemm16.mfma", 16)
+        hip.set_tunable("gemm16.tile", 0)
     assert np.abs(got[16] - got[32]).max() <= 1e-5 * np.abs(ref).max()
+
+
+@pytest.mark.parametrize("kind", ["bf16", "f16"])
+@pytest.mark.parametrize("m,n,k", [(128, 128, 64), (1, 8, 64), (130, 136, 128), (300, 520, 192), (257, 264, 320),
+                                   (512, 768, 448), (70, 1032, 1216), (640, 384, 768)])
+def test_gemm16_both_tile_sizes(hip, oracle, torch_cuda, kind, m, n, k):
+    """The 256 x 256 and the 128 x 128 workgroup tile of the 16 x 16 x 32 kernel, plain and with the fused epilogue,
+    on ragged M and N and on K values that end the stage patterns (periods of 4 and 12 slabs) at different
+    positions: each against the oracle, and the two against each other (same products, same k order per element:
+    the plain results are the same bits)."""
+    torch = torch_cuda
+    a = normal16(oracle, (m, k), m + 11, kind)
+    b = normal16(oracle, (k, n), n + 12, kind)
+    bias = oracle.fill_uniform(n, seed=n + 1, lo=-0.1, hi=0.1)
+    dt = torch.bfloat16 if kind == "bf16" else torch.float16
+    da, db = dev(torch, a).to(dt), dev(torch, b).to(dt)
+    ref = oracle.gemm(a, b)
+    got = {}
+    try:
+        for tile in (128, 256):
+            hip.set_tunable("gemm16.tile", tile)
+            c = (hip.gemm_bf16 if kind == "bf16" else hip.gemm_f16)(da, db)
+            assert hip.gemm16_tile(m, n, k) == tile
+            c = c.cpu().numpy()
+            assert np.abs(c - ref).max() / np.abs(ref).max() < 1e-4
+            got[tile] = c
+            if kind == "f16":
+                y, rs = hip.gemm_f16_bias_relu_rowsum(da, db, dev(torch, bias))
+                y_ref, rs_ref = oracle.gemm_bias_relu_rowsum(a, b, bias)
+                assert np.abs(y.cpu().numpy() - y_ref).max() <= 1e-4 * np.abs(y_ref).max()
+                assert np.abs(rs.cpu().numpy() - rs_ref).max() <= 1e-4 * max(np.abs(rs_ref).max(), 1e-30)
+    finally:
+        hip.set_tunable("gemm16.tile", 0)
+    assert np.array_equal(got[128], got[256])
+
+
+def test_gemm16_tile_choice_by_shape(hip, torch_cuda):
+    """Left to itself the launcher takes the small tile where the large one would leave CUs idle and the large one
+    for products of several rounds; shapes the direct-to-LDS kernels do not take report 0."""
+    for (m, n, k), want in [((1024, 1024, 64), 128), ((2048, 2048, 2048), 128), ((1024, 4096, 4096), 128),
+                            ((4096, 2048, 8192), 128), ((3072, 3072, 3072), 256), ((4096, 4096, 4096), 256),
+                            ((8192, 8192, 8192), 256), ((4095, 11008, 4096), 256), ((512, 512, 72), 0),
+                            ((37, 51, 29), 0)]:
+        assert hip.gemm16_tile(m, n, k) == want, (m, n, k)
+    hip.set_tunable("gemm16.mfma", 32)
+    try:
+        assert hip.gemm16_tile(1024, 1024, 1024) == 256   # the 32 x 32 x 16 kernel has the large tile only
+    finally:
+        hip.set_tunable("gemm16.mfma", 16)
