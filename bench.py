@@ -341,7 +341,7 @@ def make_workload(name, torch, hip):
                     peak=PEAK_MFMA_TFLOPS[tn], kernel=f"{kern}<{tn}, store>",
                     route=f"Execute.run_source ~lang:HIP_Source, library kernel text 'gemm_{tn}'",
                     config={"workload": f"{tn}-in f32-acc C=A.B, N(0,0.02)", "m": m, "n": n, "k": k,
-                            "workgroup_tile": tile})
+                            "workgroup_tile": tile, "k_splits": hip.gemm16_k_splits(m, n, k)})
         return main, None, info, (va, vb, vy, a, src_b, entry_b)
     if name == "gemm_f16_epilogue":
         m, n, k = 4095, 11008, 4096

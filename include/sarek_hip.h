@@ -547,6 +547,13 @@ int sarek_hip_gemm_f16(const uint16_t *a, const uint16_t *b, float *c, int m, in
  * not a multiple of 64, ...).  No counterpart in the reference, whose tiled
  * kernel has one shape (bench_matrix_mul_tiled.ml:55-95); needs no device.  */
 int sarek_hip_gemm16_tile(int m, int n, int k);
+/* Into how many pieces sarek_hip_gemm_bf16 / _f16 cut K for this shape now (1 =
+ * none): products with few 128 x 128 tiles and a long K are spread over the
+ * CUs that way, the partial tiles added up in a fixed order by a second
+ * kernel (device memory for them is kept per stream, at most 64 MiB; a call
+ * under stream capture that would have to allocate it runs unsplit).  The
+ * fused-epilogue entry point never splits.                                  */
+int sarek_hip_gemm16_k_splits(int m, int n, int k);
 
 /* Fused epilogue chain: y = relu(A.B + bias[col]) (f32, [m x n]) and
  * rowsum[r] = sum_c y[r,c] (f32, [m]).  fp16 inputs.                        */

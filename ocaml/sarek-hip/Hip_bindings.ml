@@ -191,6 +191,7 @@ let gemm_f16 =
     (ptr uint16_t @-> ptr uint16_t @-> ptr float @-> int @-> int @-> int @-> ptr void
    @-> returning int)
 let gemm16_tile = bind "sarek_hip_gemm16_tile" (int @-> int @-> int @-> returning int)
+let gemm16_k_splits = bind "sarek_hip_gemm16_k_splits" (int @-> int @-> int @-> returning int)
 let gemm_f16_bias_relu_rowsum =
   bind "sarek_hip_gemm_f16_bias_relu_rowsum"
     (ptr uint16_t @-> ptr uint16_t @-> ptr float @-> ptr float @-> ptr float @-> int @-> int

@@ -34,6 +34,9 @@
 //   gemm16_staged_kernel (any K % 8 == 0): global -> registers -> LDS with zero fill for the
 //     K tail, rows padded (144 / 544 bytes) instead of swizzled, two LDS stages of K = 64.
 //   gemm16_simple_kernel: any shape and alignment, one thread per C element.
+#include <algorithm>
+#include <map>
+#include <mutex>
 #include <type_traits>
 #include <utility>
 
@@ -775,7 +778,8 @@ template <bool Bf16, int Epi>
 __global__ __launch_bounds__(256) void gemm16_m16_small_kernel(const uint16_t *__restrict__ A, const uint16_t *__restrict__ B,
                                                                float *__restrict__ C, const float *__restrict__ bias,
                                                                float *__restrict__ rowsum, int M, int N, int K, int tiles_m,
-                                                               int tiles_n, int xcd_remap, unsigned long long *probe) {
+                                                               int tiles_n, int xcd_remap, unsigned long long *probe,
+                                                               int k_chunk, float *__restrict__ partials) {
   constexpr int SBM = 128, SBN = 128;
   constexpr int BKA = 64, BKB = 32, NA = 3, NB = 4;
   constexpr int RA = BKA / BKB;
@@ -821,9 +825,14 @@ __global__ __launch_bounds__(256) void gemm16_m16_small_kernel(const uint16_t *_
     const int bcol = min(n0 + bchunk * 8, N - 8);
     b_off[i] = (static_cast<uint32_t>(brow) * N + bcol) * 2u;
   }
-  const char *a_base = reinterpret_cast<const char *>(A + static_cast<int64_t>(m0) * K);
+  // K split over gridDim.y workgroups per tile (plain store only): this one takes k0 .. k0 + k_len - 1 and writes its
+  // partial tile to its own M x N plane of `partials`, which a second kernel adds up in a fixed order
+  const int k0 = blockIdx.y * k_chunk;
+  const int k_len = min(k_chunk, K - k0);
+  if (gridDim.y > 1) C = partials + static_cast<int64_t>(blockIdx.y) * M * N;
+  const char *a_base = reinterpret_cast<const char *>(A + static_cast<int64_t>(m0) * K + k0);
   const int64_t b_slab_bytes = static_cast<int64_t>(BKB) * N * 2;
-  const int nslabs = K / BKB, nstages = K / BKA;
+  const int nslabs = k_len / BKB, nstages = k_len / BKA;
 
   f32x4_t acc[4][4];
 #pragma unroll
@@ -846,7 +855,7 @@ __global__ __launch_bounds__(256) void gemm16_m16_small_kernel(const uint16_t *_
   };
   // B slabs go out in order; the source is a running pointer that stops at the last slab (the tail of the K loop
   // re-issues it into stages nobody reads any more, so the count of transfers in flight keeps its pattern)
-  const char *b_src = reinterpret_cast<const char *>(B);
+  const char *b_src = reinterpret_cast<const char *>(B + static_cast<int64_t>(k0) * N);
   int b_next = 0;
   auto issue_b = [&](char *sb) {
     const __amdgpu_buffer_rsrc_t b_rsrc = make_rsrc(b_src, 0x80000000u);
@@ -1128,6 +1137,85 @@ inline bool small_tile_wins(int m, int n) {
   return cost_small < 0.9 * cost_large;
 }
 
+// Adds the `splits` partial M x N planes of a K-split product into C, plane 0 first: a fixed order, so the result does
+// not depend on which workgroup finished when.
+__global__ __launch_bounds__(256) void splitk_reduce_kernel(const float *__restrict__ partials, float *__restrict__ C,
+                                                            int64_t mn, int splits) {
+  const int64_t i = (static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x) * 4;
+  if (i >= mn) return;   // mn is a multiple of 8 (n % 8 == 0)
+  f32x4_t acc = *reinterpret_cast<const f32x4_t *>(partials + i);
+  for (int s = 1; s < splits; ++s) acc += *reinterpret_cast<const f32x4_t *>(partials + s * mn + i);
+  *reinterpret_cast<f32x4_t *>(C + i) = acc;
+}
+
+// Device memory for the partial planes: one block of kSplitWorkspaceBytes per (device, stream), allocated at the first
+// split product on that stream and kept until the process ends (never grown or freed, so a pointer handed out stays
+// good whatever other threads do): calls on different streams never share one, calls on one stream are ordered by it.
+// nullptr (the caller then does not split) for a stream under capture that has none yet, past 16 streams, or when the
+// allocation fails.
+constexpr size_t kSplitWorkspaceBytes = 64u << 20;
+float *splitk_workspace(hipStream_t st) {
+  static std::mutex mu;
+  static std::map<std::pair<int, hipStream_t>, void *> blocks;
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess) return nullptr;
+  std::lock_guard<std::mutex> lock(mu);
+  auto it = blocks.find({dev, st});
+  if (it != blocks.end()) return static_cast<float *>(it->second);
+  if (blocks.size() >= 16) return nullptr;
+  hipStreamCaptureStatus capturing = hipStreamCaptureStatusNone;
+  if (hipStreamIsCapturing(st, &capturing) != hipSuccess || capturing != hipStreamCaptureStatusNone) {
+    (void)hipGetLastError();
+    return nullptr;
+  }
+  void *p = nullptr;
+  if (hipMalloc(&p, kSplitWorkspaceBytes) != hipSuccess) {
+    (void)hipGetLastError();
+    return nullptr;
+  }
+  blocks[{dev, st}] = p;
+  return static_cast<float *>(p);
+}
+
+// K splits of the 128 x 128 kernel for a plain product with few tiles and a long K; 1 = no split.  A tile's K loop is
+// bound by the latency of its transfers (0.19 us per K = 32 slab with one or two workgroups on a CU, measured), so
+// cutting K over idle CUs shortens it; against that stand the second launch (5 us) and the partial planes, which cost
+// 0.65 us per MiB to write and add up.  The count in {2, 4, 8, 16} with the lowest estimate is taken if it is a tenth
+// below the unsplit one; every piece is at least 256 of K and the planes fit kSplitWorkspaceBytes.
+// gemm16.split_k: 0 = this rule, 1 = never, n >= 2 forces n where the shape allows it.
+int splitk_for(int m, int n, int k) {
+  const int64_t tiles = static_cast<int64_t>((m + 127) / 128) * ((n + 127) / 128);
+  const int64_t forced = tunable("gemm16.split_k", 0);
+  if (forced == 1) return 1;
+  static const int cus = [] {
+    int dev = 0, v = 0;
+    if (hipGetDevice(&dev) != hipSuccess ||
+        hipDeviceGetAttribute(&v, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || v <= 0)
+      v = 256;
+    return v;
+  }();
+  const double plane_mib = static_cast<double>(m) * n * 4 / (1 << 20);
+  const int64_t fit = static_cast<int64_t>(static_cast<double>(kSplitWorkspaceBytes >> 20) / plane_mib);
+  int64_t splits = 1;
+  if (forced >= 2) {
+    splits = std::min<int64_t>({forced, static_cast<int64_t>(k / 64), fit});
+  } else {
+    auto estimate = [&](int64_t s) {
+      const double slabs = static_cast<double>(k) / 32 / s;
+      return 8.0 + slabs * 0.19 * (tiles * s > cus ? 1.15 : 1.0) + (s > 1 ? 5.0 + s * plane_mib * 0.65 : 0.0);
+    };
+    double best = estimate(1) * 0.9;
+    for (int64_t s = 2; s <= 16; s *= 2) {
+      if (tiles * s > 2 * cus || k / s < 256 || s > fit) break;
+      if (estimate(s) < best) best = estimate(s), splits = s;
+    }
+  }
+  if (splits < 2) return 1;
+  // whole K = 64 stages per piece; the count follows from the piece so that none is empty
+  const int chunk = static_cast<int>(((k / 64 + splits - 1) / splits) * 64);
+  return (k + chunk - 1) / chunk;
+}
+
 // The workgroup tile of the direct-to-LDS kernels for this shape under the present tunables (256 or 128), or 0 when
 // the shape goes to the staged or the simple kernel (pointer alignment, which can also send a call there, is not a
 // property of the shape and is not looked at).
@@ -1214,8 +1302,25 @@ int launch_gemm16(const uint16_t *a, const uint16_t *b, float *c, const float *b
         if (gemm16_tile_for(m, n, k) == 128) {
           const int sm = (m + 127) / 128, sn = (n + 127) / 128;
           unsigned long long *sprobe = clock_probe(static_cast<int64_t>(sm) * sn);
+          if constexpr (Epi == EPI_STORE) {
+            const int splits = reinterpret_cast<uintptr_t>(c) % 16 == 0 ? splitk_for(m, n, k) : 1;
+            if (splits > 1) {
+              const int64_t mn = static_cast<int64_t>(m) * n;
+              float *partials = splitk_workspace(st);
+              if (partials) {
+                const int chunk = ((k / 64 + splits - 1) / splits) * 64;
+                hipLaunchKernelGGL((gemm16_m16_small_kernel<Bf16, Epi>), dim3(sm * sn, splits), dim3(256), 0, st, a, b, c,
+                                   bias, rowsum, m, n, k, sm, sn, remap, nullptr, chunk, partials);
+                int rc = check_launch("gemm16 kernel launch");
+                if (rc != SAREK_HIP_OK) return rc;
+                hipLaunchKernelGGL(splitk_reduce_kernel, dim3(static_cast<unsigned>((mn / 4 + 255) / 256)), dim3(256), 0, st,
+                                   partials, c, mn, splits);
+                return check_launch("gemm16 split-K reduction launch");
+              }
+            }
+          }
           hipLaunchKernelGGL((gemm16_m16_small_kernel<Bf16, Epi>), dim3(sm * sn), dim3(256), 0, st, a, b, c, bias, rowsum,
-                             m, n, k, sm, sn, remap, sprobe);
+                             m, n, k, sm, sn, remap, sprobe, k, nullptr);
           return check_launch("gemm16 kernel launch");
         }
         hipLaunchKernelGGL((gemm16_m16_kernel<Bf16, Epi>), grid, dim3(512), 0, st, a, b, c, bias, rowsum, m, n, k,
@@ -1256,6 +1361,8 @@ using namespace sarek_hip;
 extern "C" {
 
 int sarek_hip_gemm16_tile(int m, int n, int k) { return gemm16_tile_for(m, n, k); }
+
+int sarek_hip_gemm16_k_splits(int m, int n, int k) { return gemm16_tile_for(m, n, k) == 128 ? splitk_for(m, n, k) : 1; }
 
 int sarek_hip_gemm_bf16(const uint16_t *a, const uint16_t *b, float *c, int m, int n, int k,
                         sarek_hip_stream stream) {

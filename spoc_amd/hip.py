@@ -139,6 +139,7 @@ SYMBOLS = {
     "sarek_hip_gemm_bf16": (_i, [_vp, _vp, _vp, _i, _i, _i, _vp]),
     "sarek_hip_gemm_f16": (_i, [_vp, _vp, _vp, _i, _i, _i, _vp]),
     "sarek_hip_gemm16_tile": (_i, [_i, _i, _i]),
+    "sarek_hip_gemm16_k_splits": (_i, [_i, _i, _i]),
     "sarek_hip_gemm_f16_bias_relu_rowsum": (_i, [_vp, _vp, _vp, _vp, _vp, _i, _i, _i, _vp]),
     "sarek_hip_cast_f32_to_bf16": (_i, [_vp, _vp, _i64, _vp]),
     "sarek_hip_cast_f32_to_f16": (_i, [_vp, _vp, _i64, _vp]),
@@ -585,6 +586,11 @@ def gemm_bf16(a, b, out=None):
 def gemm16_tile(m, n, k):
     """256 / 128: the workgroup tile the 16-bit GEMMs take for this shape now; 0: the staged or simple kernel."""
     return int(lib.sarek_hip_gemm16_tile(m, n, k))
+
+
+def gemm16_k_splits(m, n, k):
+    """Into how many pieces the plain 16-bit GEMMs cut K for this shape now (1 = none)."""
+    return int(lib.sarek_hip_gemm16_k_splits(m, n, k))
 
 
 def gemm_f16(a, b, out=None):

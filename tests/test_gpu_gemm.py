@@ -386,3 +386,93 @@ def test_gemm16_tile_choice_by_shape(hip, torch_cuda):
         assert hip.gemm16_tile(1024, 1024, 1024) == 256   # the 32 x 32 x 16 kernel has the large tile only
     finally:
         hip.set_tunable("gemm16.mfma", 16)
+
+
+@pytest.mark.parametrize("kind", ["bf16", "f16"])
+@pytest.mark.parametrize("m,n,k,splits", [(128, 128, 8192, 0), (256, 256, 4096, 0), (130, 136, 1024, 2),
+                                          (300, 520, 448, 3), (1, 8, 4096, 16), (512, 384, 2048, 5),
+                                          (777, 1000, 320, 2)])
+def test_gemm16_split_k(hip, oracle, torch_cuda, kind, m, n, k, splits):
+    """Products with few tiles and a long K are cut along K over several workgroups per tile and the partial tiles
+    added in a fixed order: against the oracle, the same bits on every run and on another stream, and the count the
+    library reports.  splits = 0 leaves the choice to the launcher (these two shapes split), n forces n pieces
+    (piece sizes that are not equal included: 448 = 192 + 192 + 64)."""
+    torch = torch_cuda
+    a = normal16(oracle, (m, k), m + 21, kind)
+    b = normal16(oracle, (k, n), n + 22, kind)
+    dt = torch.bfloat16 if kind == "bf16" else torch.float16
+    da, db = dev(torch, a).to(dt), dev(torch, b).to(dt)
+    fn = hip.gemm_bf16 if kind == "bf16" else hip.gemm_f16
+    ref = oracle.gemm(a, b)
+    hip.set_tunable("gemm16.split_k", splits)
+    try:
+        reported = hip.gemm16_k_splits(m, n, k)
+        assert reported >= 2 and (splits == 0 or reported <= splits)
+        c1 = fn(da, db)
+        c2 = fn(da, db)
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):
+            c3 = fn(da, db)
+        side.synchronize()
+        # an output that is not 16-byte aligned is computed unsplit
+        odd = torch.empty(m * n + 1, device="cuda")[1:].view(m, n)
+        fn(da, db, out=odd)
+        hip.set_tunable("gemm16.split_k", 1)
+        assert hip.gemm16_k_splits(m, n, k) == 1
+        whole = fn(da, db)
+    finally:
+        hip.set_tunable("gemm16.split_k", 0)
+    assert torch.equal(c1, c2) and torch.equal(c1, c3)
+    assert torch.equal(odd, whole)
+    for c in (c1, whole):
+        assert np.abs(c.cpu().numpy() - ref).max() / np.abs(ref).max() < 1e-4
+    assert (c1 - whole).abs().max().item() <= 1e-5 * float(np.abs(ref).max())
+
+
+def test_gemm16_split_k_rule_and_epilogue(hip, oracle, torch_cuda):
+    """The launcher splits only where it pays (few tiles, long K), never the fused epilogue, and never the large tile."""
+    torch = torch_cuda
+    for (m, n, k), want_split in [((256, 256, 8192), True), ((512, 512, 8192), True), ((128, 4096, 4096), True),
+                                  ((1024, 1024, 1024), False), ((2048, 2048, 2048), False), ((512, 512, 512), False),
+                                  ((8192, 8192, 8192), False), ((4096, 4096, 4096), False)]:
+        assert (hip.gemm16_k_splits(m, n, k) > 1) == want_split, (m, n, k)
+    m, n, k = 128, 256, 4096
+    assert hip.gemm16_k_splits(m, n, k) > 1
+    a = normal16(oracle, (m, k), 31, "f16")
+    b = normal16(oracle, (k, n), 32, "f16")
+    bias = oracle.fill_uniform(n, seed=33, lo=-0.1, hi=0.1)
+    y, rs = hip.gemm_f16_bias_relu_rowsum(dev(torch, a).half(), dev(torch, b).half(), dev(torch, bias))
+    y_ref, rs_ref = oracle.gemm_bias_relu_rowsum(a, b, bias)
+    assert np.abs(y.cpu().numpy() - y_ref).max() <= 1e-4 * np.abs(y_ref).max()
+    assert np.abs(rs.cpu().numpy() - rs_ref).max() <= 1e-4 * np.abs(rs_ref).max()
+
+
+def test_gemm16_split_k_under_graph_capture(hip, torch_cuda):
+    """A split-eligible product captured into a HIP graph on a stream that has no partial-plane block yet runs unsplit
+    (nothing may be allocated under capture); every replay gives the eager result for the inputs of that moment."""
+    torch = torch_cuda
+    m, n, k = 256, 256, 4096
+    assert hip.gemm16_k_splits(m, n, k) > 1
+    a = (torch.randn(m, k, device="cuda") * 0.02).bfloat16()
+    b = (torch.randn(k, n, device="cuda") * 0.02).bfloat16()
+    out = torch.empty(m, n, device="cuda")
+    hip.gemm_bf16(a, b, out=out)          # warm: kernels loaded before the capture
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        hip.gemm_bf16(a, b, out=out)
+    for seed in (1, 2, 3):
+        torch.manual_seed(seed)
+        a.copy_((torch.randn(m, k, device="cuda") * 0.02).bfloat16())
+        out.zero_()
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        got = out.clone()
+        hip.set_tunable("gemm16.split_k", 1)
+        try:
+            want = hip.gemm_bf16(a, b)
+        finally:
+            hip.set_tunable("gemm16.split_k", 0)
+        assert torch.equal(got, want), seed
