@@ -388,6 +388,17 @@ def test_gemm16_tile_choice_by_shape(hip, torch_cuda):
         hip.set_tunable("gemm16.mfma", 16)
 
 
+_SIDE_STREAM = []
+
+
+def side_stream(torch):
+    """One second stream for the whole module: the library keeps a block of device memory per stream it has split a
+    product on (16 streams at most), so the cases share theirs."""
+    if not _SIDE_STREAM:
+        _SIDE_STREAM.append(torch.cuda.Stream())
+    return _SIDE_STREAM[0]
+
+
 @pytest.mark.parametrize("kind", ["bf16", "f16"])
 @pytest.mark.parametrize("m,n,k,splits", [(128, 128, 8192, 0), (256, 256, 4096, 0), (130, 136, 1024, 2),
                                           (300, 520, 448, 3), (1, 8, 4096, 16), (512, 384, 2048, 5),
@@ -410,7 +421,7 @@ def test_gemm16_split_k(hip, oracle, torch_cuda, kind, m, n, k, splits):
         assert reported >= 2 and (splits == 0 or reported <= splits)
         c1 = fn(da, db)
         c2 = fn(da, db)
-        side = torch.cuda.Stream()
+        side = side_stream(torch)
         side.wait_stream(torch.cuda.current_stream())
         with torch.cuda.stream(side):
             c3 = fn(da, db)
