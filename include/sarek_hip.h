@@ -550,9 +550,11 @@ int sarek_hip_gemm16_tile(int m, int n, int k);
 /* Into how many pieces sarek_hip_gemm_bf16 / _f16 cut K for this shape now (1 =
  * none): products with few 128 x 128 tiles and a long K are spread over the
  * CUs that way, the partial tiles added up in a fixed order by a second
- * kernel (device memory for them is kept per stream, at most 64 MiB; a call
- * under stream capture that would have to allocate it runs unsplit).  The
- * fused-epilogue entry point never splits.                                  */
+ * kernel.  Device memory for them: one 64 MiB block per stream, allocated at
+ * the first such call on the stream and kept until the process ends, for up
+ * to 16 streams; calls on further streams, and calls under stream capture on
+ * a stream that has no block yet, run unsplit (same result up to the order of
+ * the f32 additions).  The fused-epilogue entry point never splits.         */
 int sarek_hip_gemm16_k_splits(int m, int n, int k);
 
 /* Fused epilogue chain: y = relu(A.B + bias[col]) (f32, [m x n]) and
