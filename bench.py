@@ -43,6 +43,7 @@ MEASURED_TRAFFIC_BYTES = {
     "gemm_bf16_8192": (801398 * 2 + 262374) * 1024,
     "gemm_f32_8192": (1698530 * 2 + 262153) * 1024,
     "gemm_f32_1024": (12333 * 2 + 4098) * 1024,
+    "gemm_bf16_2048": (24690 * 2 + 16386) * 1024,
     "gemm_f16_epilogue": (311774 * 2 + 176787) * 1024,
     "histogram_2p28": (493838 * 2 + 256) * 1024,
     "radix_scatter_5e7": (97870 * 2 + 215643) * 1024,
@@ -57,7 +58,7 @@ def parse():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--workload", default="gemm_bf16_8192",
                     choices=["gemm_bf16_8192", "gemm_f16_8192", "triad_sum_2p28", "gemm_f32_8192", "gemm_f32_1024",
-                             "gemm_f16_epilogue", "gemm_f16_4095x11008x4096", "gemm_f16_shape", "gemm_bf16_shape", "copy_1gib",
+                             "gemm_f16_epilogue", "gemm_f16_4095x11008x4096", "gemm_f16_shape", "gemm_bf16_shape", "gemm_bf16_2048", "copy_1gib",
                              "vendor_gemm_bf16_8192", "vendor_gemm_bf16_shape", "histogram_2p28",
                              "radix_scatter_5e7", "mfma_bf16_stream", "mfma_bf16_stream_32x32x16", "l2_to_lds_stream"])
     ap.add_argument("--warmup-ms", type=float, default=60.0,
@@ -314,10 +315,11 @@ def make_workload(name, torch, hip):
                     config={"workload": "out[counters[key & 255]++] = key, random keys below 100000", "n": n,
                             "algorithmic_bytes": 8 * n})
         return main, None, info, (vk, vo, vcnt, starts, a, ir)
-    if name in ("gemm_f16_4095x11008x4096", "gemm_f16_shape", "gemm_bf16_shape"):
-        # the epilogue config's product without the epilogue (what the fused chain costs on top), or any --shape
-        m, n, k = (4095, 11008, 4096) if name == "gemm_f16_4095x11008x4096" else GEMM_SHAPE
-        bf16 = name == "gemm_bf16_shape"
+    if name in ("gemm_f16_4095x11008x4096", "gemm_f16_shape", "gemm_bf16_shape", "gemm_bf16_2048"):
+        # the epilogue config's product without the epilogue (what the fused chain costs on top), any --shape, or
+        # 2048^3: a product whose 256 x 256 tiles would occupy a quarter of the CUs (the 128 x 128 tile's case)
+        m, n, k = {"gemm_f16_4095x11008x4096": (4095, 11008, 4096), "gemm_bf16_2048": (2048, 2048, 2048)}.get(name, GEMM_SHAPE)
+        bf16 = name != "gemm_f16_4095x11008x4096" and name != "gemm_f16_shape"
         dt = torch.bfloat16 if bf16 else torch.float16
         g.manual_seed(0xA5)
         t = (torch.randn(m, k, device="cuda", generator=g) * 0.02).to(dt)
