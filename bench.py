@@ -69,6 +69,8 @@ def parse():
     ap.add_argument("--no-also", action="store_true", help="measure only the headline workload")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--shape", default="4096,11264,4096", metavar="M,N,K", help="shape of the gemm_f16_shape workload")
+    ap.add_argument("--l2-stream", default="", metavar="WORKGROUPS,WINDOW_MIB",
+                    help="shape of the l2_to_lds_stream workload (default 1024,2)")
     ap.add_argument("--zero-operands", action="store_true",
                     help="16-bit GEMM workloads: all-zero A and B (what the kernel does when the data costs no power)")
     ap.add_argument("--tunable", action="append", default=[], metavar="NAME=VALUE",
@@ -125,6 +127,7 @@ def dims(*d):
 
 ZERO_OPERANDS = False
 GEMM_SHAPE = (4096, 11264, 4096)
+L2_STREAM_SHAPE = None
 
 
 def make_workload(name, torch, hip):
@@ -248,11 +251,13 @@ def make_workload(name, torch, hip):
         src = torch.randint(0, 2 ** 31 - 1, ((16 << 20) // 4,), dtype=torch.int32, device="cuda", generator=g)
         sink = torch.zeros(4, dtype=torch.int32, device="cuda")
         wgs, per_wg, window = 1024, 8 << 20, 2 << 20
+        if L2_STREAM_SHAPE:       # --l2-stream WORKGROUPS,WINDOW_MIB (window a power of two, at most 16)
+            wgs, window = L2_STREAM_SHAPE[0], L2_STREAM_SHAPE[1] << 20
         items = [src, sink, ("i32", per_wg // (512 * 16)), ("i32", (window // 16 - 1) & ~511), ("i32", (64 << 10) // 16)]
         info = dict(metric="L2 -> LDS transfer GB/s (no other work, every request an L2 hit)", unit="GB/s", dtype="u8",
                     work=float(wgs * per_wg), work_unit=1e9, bound="l2", peak=64.0 * 256 * NOMINAL_CLOCK_MHZ * 1e-3,
                     kernel="l2_to_lds (JIT)", route="Execute.run_source ~lang:HIP_Source, text in bench.py",
-                    config={"workload": "1024 workgroups x 8 MiB by buffer_load_dwordx4 ... lds from a 2 MiB window "
+                    config={"workload": f"{wgs} workgroups x 8 MiB by buffer_load_dwordx4 ... lds from a {window >> 20} MiB window "
                                         "(the operand bytes of the 8192^3 16-bit GEMM with 256 x 256 tiles: 8.59 GB)"})
         return (lambda: hip.run_source(L2_STREAM_SRC, "l2_to_lds", (512, 1, 1), (wgs, 1, 1), items)), None, info, (src, sink)
     if name in ("vendor_gemm_bf16_8192", "vendor_gemm_bf16_shape"):
@@ -724,7 +729,11 @@ def main():
         print("bench.py needs a GPU", file=sys.stderr)
         sys.exit(2)
     torch.cuda.set_device(0)
-    global ZERO_OPERANDS, GEMM_SHAPE, WARMUP_MS, TRACE_LAUNCHES
+    global ZERO_OPERANDS, GEMM_SHAPE, WARMUP_MS, TRACE_LAUNCHES, L2_STREAM_SHAPE
+    if args.l2_stream:
+        L2_STREAM_SHAPE = tuple(int(x) for x in args.l2_stream.split(","))
+        if len(L2_STREAM_SHAPE) != 2 or L2_STREAM_SHAPE[1] not in (1, 2, 4, 8, 16) or L2_STREAM_SHAPE[0] < 1:
+            sys.exit("--l2-stream WORKGROUPS,WINDOW_MIB with a window of 1, 2, 4, 8 or 16 MiB")
     WARMUP_MS, TRACE_LAUNCHES = args.warmup_ms, args.trace_launches
     ZERO_OPERANDS = args.zero_operands
     GEMM_SHAPE = tuple(int(x) for x in args.shape.split(","))
