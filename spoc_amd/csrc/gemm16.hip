@@ -487,8 +487,8 @@ __device__ __forceinline__ f32x4_t mfma16(u32x4 a, u32x4 b, f32x4_t c) {
 // with TI = 4: 8+4+2+1 leave it with row m of the 16), the WNW waves along N through LDS, one atomicAdd per row.
 template <int Epi, int TI = 8, int WNW = 4>
 __device__ __forceinline__ void epilogue16(f32x4_t (&acc)[TI][4], float *__restrict__ C, const float *__restrict__ bias,
-                                           float *__restrict__ rowsum, int M, int N, int m0, int wm, int wn, int col0,
-                                           int l16, int g, float *scratch) {
+                                           float *__restrict__ rowsum, int M, int N, int ld, int m0, int wm, int wn,
+                                           int col0, int l16, int g, float *scratch) {
   constexpr int WROWS = 16 * TI, TROWS = 2 * WROWS, NV = 4 * TI, E = NV / 16;
   static_assert(TI == 8 || TI == 4, "wave tiles of 128 or 64 rows");
   static_assert(WNW == 4 || WNW == 2, "four or two waves along N");
@@ -516,7 +516,7 @@ __device__ __forceinline__ void epilogue16(f32x4_t (&acc)[TI][4], float *__restr
           v = v > 0.f ? v : 0.f;
           sum += cok[j] ? v : 0.f;
         }
-        if (row < M && cok[j]) C[static_cast<int64_t>(row) * N + col0 + j * 16 + l16] = v;
+        if (row < M && cok[j]) C[static_cast<int64_t>(row) * ld + col0 + j * 16 + l16] = v;
       }
       rs[i * 4 + r] = sum;
     }
@@ -555,11 +555,11 @@ __device__ __forceinline__ void epilogue16(f32x4_t (&acc)[TI][4], float *__restr
   }
 }
 
-template <bool Bf16, int Epi, int Ablate = 0>
+template <bool Bf16, int Epi, int Ablate = 0, bool Ragged = false>
 __global__ __launch_bounds__(512) void gemm16_m16_kernel(const uint16_t *__restrict__ A, const uint16_t *__restrict__ B,
                                                          float *__restrict__ C, const float *__restrict__ bias,
                                                          float *__restrict__ rowsum, int M, int N, int K, int tiles_m,
-                                                         int tiles_n, int xcd_remap, unsigned long long *probe) {
+                                                         int tiles_n, int xcd_remap, unsigned long long *probe, int ld) {
   constexpr int BKA = 64, BKB = 32, NA = 2, NB = 4;
   constexpr int RA = BKA / BKB;                  // B slabs per A stage
   constexpr int A_ROW = BKA * 2, A_CHUNKS = A_ROW / 16, A_ROWS_PER_DMA = 1024 / A_ROW;
@@ -586,7 +586,7 @@ __global__ __launch_bounds__(512) void gemm16_m16_kernel(const uint16_t *__restr
   auto a_swz = [](int row) { return (row >> 1) & 7; };
   auto b_swz = [](int row) { return ((row & 3) << 2) | (((row >> 3) & 1) << 1); };
 
-  // DMA sources, as in gemm16_dma_kernel (rows past M and columns past N clamped: never stored)
+  // DMA sources (rows past M clamped: what they bring is never stored)
   uint32_t a_off[DA], b_off[DB];
 #pragma unroll
   for (int i = 0; i < DA; ++i) {
@@ -600,13 +600,26 @@ __global__ __launch_bounds__(512) void gemm16_m16_kernel(const uint16_t *__restr
     const int q = wave + NWAVES * i;
     const int brow = 2 * q + (lane >> 5);
     const int bchunk = (lane & 31) ^ b_swz(brow);
-    const int bcol = min(n0 + bchunk * 8, N - 8);
-    b_off[i] = (static_cast<uint32_t>(brow) * N + bcol) * 2u;
+    // Ragged: columns past N are fetched as they lie (the next row's, or zeros past the end of B: the range of the
+    // buffer resource is exact) and never stored, and rows need no 16-byte alignment (ld may be odd); otherwise
+    // (N % 8 == 0) the pieces past N are clamped onto the last one
+    const int bcol = Ragged ? n0 + bchunk * 8 : min(n0 + bchunk * 8, N - 8);
+    b_off[i] = (static_cast<uint32_t>(brow) * ld + bcol) * 2u;
   }
   const char *a_base = reinterpret_cast<const char *>(A + static_cast<int64_t>(m0) * K);
   const char *b_base = reinterpret_cast<const char *>(B);
-  const int64_t b_slab_bytes = static_cast<int64_t>(BKB) * N * 2;
-  const int nslabs = K / BKB, nstages = K / BKA;
+  const int64_t b_slab_bytes = static_cast<int64_t>(BKB) * ld * 2;
+  const int nslabs = (K + BKB - 1) / BKB, nstages = (K + BKA - 1) / BKA;
+  // K need not fill the last A stage or B slab (K % 8 == 0): there the lanes whose 16-byte piece (A) or row (B) lies
+  // past K give an offset outside the buffer range, which the transfer writes to LDS as zeros.  A lane's k piece is
+  // the same for all its transfers of a stage (rows 16 apart share the swizzle); its B rows are 16 apart.
+  const int k_tail_a = K - (nstages - 1) * BKA, k_tail_b = K - (nslabs - 1) * BKB;
+  const bool a_lane_in_k = !Ragged || (((lane % A_CHUNKS) ^ a_swz(wave * A_ROWS_PER_DMA + lane / A_CHUNKS)) << 3) < k_tail_a;
+  bool b_lane_in_k[DB];
+#pragma unroll
+  for (int i = 0; i < DB; ++i) b_lane_in_k[i] = !Ragged || 2 * (wave + NWAVES * i) + (lane >> 5) < k_tail_b;
+  const char *b_end = b_base + (static_cast<int64_t>(K - 1) * ld + N) * 2;   // the end of row K-1's N columns
+  constexpr uint32_t kOutOfRange = 0x80000000u;
 
   f32x4_t acc[8][4];
 #pragma unroll
@@ -627,9 +640,11 @@ __global__ __launch_bounds__(512) void gemm16_m16_kernel(const uint16_t *__restr
   const __amdgpu_buffer_rsrc_t a_rsrc = make_rsrc(a_base, 0x80000000u);
   auto issue_a = [&](char *sa, int stage) {
     if (stage >= NA && (Ablate & 1)) return;
+    const bool whole = stage < nstages - 1;
     const uint32_t a_so = static_cast<uint32_t>(min(stage, nstages - 1)) * (BKA * 2);
 #pragma unroll
-    for (int i = 0; i < DA; ++i) dma16(a_rsrc, a_off[i], a_so, sa + (wave + NWAVES * i) * 1024);
+    for (int i = 0; i < DA; ++i)
+      dma16(a_rsrc, (!Ragged || whole || a_lane_in_k) ? a_off[i] : kOutOfRange, a_so, sa + (wave + NWAVES * i) * 1024);
   };
   // B slabs are issued in order 0, 1, 2, ...: the source of the next one is a running pointer (two scalar adds per
   // slab instead of a 64-bit multiply) that stops at the last slab, which the tail of the K loop re-issues into
@@ -639,9 +654,13 @@ __global__ __launch_bounds__(512) void gemm16_m16_kernel(const uint16_t *__restr
   auto issue_b = [&](char *sb, int slab) {
     if (slab >= NB && (Ablate & 1)) return;
     (void)slab;   // == b_next
-    const __amdgpu_buffer_rsrc_t b_rsrc = make_rsrc(b_src, 0x80000000u);
+    const bool whole = b_next < nslabs - 1;
+    const int64_t b_left = b_end - b_src;
+    const __amdgpu_buffer_rsrc_t b_rsrc =
+        make_rsrc(b_src, Ragged && b_left < 0x80000000ll ? static_cast<uint32_t>(b_left) : kOutOfRange);
 #pragma unroll
-    for (int i = 0; i < DB; ++i) dma16(b_rsrc, b_off[i], 0u, sb + (wave + NWAVES * i) * 1024);
+    for (int i = 0; i < DB; ++i)
+      dma16(b_rsrc, (!Ragged || whole || b_lane_in_k[i]) ? b_off[i] : kOutOfRange, 0u, sb + (wave + NWAVES * i) * 1024);
     ++b_next;
     if (b_next < nslabs) b_src += b_slab_bytes;
   };
@@ -757,7 +776,7 @@ __global__ __launch_bounds__(512) void gemm16_m16_kernel(const uint16_t *__restr
     ((full + Is < nslabs ? slab(std::integral_constant<int, Is>{}, full + Is) : (void)0), ...);
   }(std::make_integer_sequence<int, P - 1>{});
   __builtin_amdgcn_s_waitcnt(waitcnt_vm_lgkm0(0));   // drain the (redundant) tail DMA before the LDS is released
-  epilogue16<Epi>(acc, C, bias, rowsum, M, N, m0, wm, wn, n0 + wn * 64, l16, g,
+  epilogue16<Epi>(acc, C, bias, rowsum, M, N, ld, m0, wm, wn, n0 + wn * 64, l16, g,
                   reinterpret_cast<float *>(lds_ring<10, A_BYTES_S>));
   if (probe && tid == 0) {
     probe[2 * blockIdx.x] = static_cast<unsigned long long>(clock64() - probe_c0);
@@ -774,12 +793,12 @@ __global__ __launch_bounds__(512) void gemm16_m16_kernel(const uint16_t *__restr
 // rows of the large tile, so the same XOR swizzle keeps the transposing reads free of bank conflicts.  A slab is 16 MFMAs:
 // rows 0-31 of the wave tile before the barrier, rows 32-63 after it with the next slab's 12 fragment reads (and, every
 // other slab, the 4 transfers of an A stage) behind them; fragments are double-buffered by slab parity.
-template <bool Bf16, int Epi>
+template <bool Bf16, int Epi, bool Ragged = false>
 __global__ __launch_bounds__(256) void gemm16_m16_small_kernel(const uint16_t *__restrict__ A, const uint16_t *__restrict__ B,
                                                                float *__restrict__ C, const float *__restrict__ bias,
                                                                float *__restrict__ rowsum, int M, int N, int K, int tiles_m,
                                                                int tiles_n, int xcd_remap, unsigned long long *probe,
-                                                               int k_chunk, float *__restrict__ partials) {
+                                                               int k_chunk, float *__restrict__ partials, int ld) {
   constexpr int SBM = 128, SBN = 128;
   constexpr int BKA = 64, BKB = 32, NA = 3, NB = 4;
   constexpr int RA = BKA / BKB;
@@ -822,17 +841,28 @@ __global__ __launch_bounds__(256) void gemm16_m16_small_kernel(const uint16_t *_
     const int q = wave + NWAVES * i;
     const int brow = q * B_ROWS_PER_DMA + lane / B_CHUNKS;
     const int bchunk = (lane % B_CHUNKS) ^ b_swz(brow);
-    const int bcol = min(n0 + bchunk * 8, N - 8);
-    b_off[i] = (static_cast<uint32_t>(brow) * N + bcol) * 2u;
+    // Ragged: columns past N are fetched as they lie (the next row's, or zeros past the end of B: the range of the
+    // buffer resource is exact) and never stored, and rows need no 16-byte alignment (ld may be odd); otherwise
+    // (N % 8 == 0) the pieces past N are clamped onto the last one
+    const int bcol = Ragged ? n0 + bchunk * 8 : min(n0 + bchunk * 8, N - 8);
+    b_off[i] = (static_cast<uint32_t>(brow) * ld + bcol) * 2u;
   }
   // K split over gridDim.y workgroups per tile (plain store only): this one takes k0 .. k0 + k_len - 1 and writes its
   // partial tile to its own M x N plane of `partials`, which a second kernel adds up in a fixed order
   const int k0 = blockIdx.y * k_chunk;
   const int k_len = min(k_chunk, K - k0);
-  if (gridDim.y > 1) C = partials + static_cast<int64_t>(blockIdx.y) * M * N;
+  if (gridDim.y > 1) C = partials + static_cast<int64_t>(blockIdx.y) * M * ld;
   const char *a_base = reinterpret_cast<const char *>(A + static_cast<int64_t>(m0) * K + k0);
-  const int64_t b_slab_bytes = static_cast<int64_t>(BKB) * N * 2;
-  const int nslabs = k_len / BKB, nstages = k_len / BKA;
+  const int64_t b_slab_bytes = static_cast<int64_t>(BKB) * ld * 2;
+  const int nslabs = (k_len + BKB - 1) / BKB, nstages = (k_len + BKA - 1) / BKA;
+  // the end of K inside the last A stage / B slab, as in the large tile
+  const int k_tail_a = k_len - (nstages - 1) * BKA, k_tail_b = k_len - (nslabs - 1) * BKB;
+  const bool a_lane_in_k = !Ragged || (((lane % A_CHUNKS) ^ a_swz(wave * A_ROWS_PER_DMA + lane / A_CHUNKS)) << 3) < k_tail_a;
+  bool b_lane_in_k[DB];
+#pragma unroll
+  for (int i = 0; i < DB; ++i) b_lane_in_k[i] = !Ragged || (wave + NWAVES * i) * B_ROWS_PER_DMA + lane / B_CHUNKS < k_tail_b;
+  const char *b_end = reinterpret_cast<const char *>(B) + (static_cast<int64_t>(K - 1) * ld + N) * 2;
+  constexpr uint32_t kOutOfRange = 0x80000000u;
 
   f32x4_t acc[4][4];
 #pragma unroll
@@ -849,18 +879,24 @@ __global__ __launch_bounds__(256) void gemm16_m16_small_kernel(const uint16_t *_
 
   const __amdgpu_buffer_rsrc_t a_rsrc = make_rsrc(a_base, 0x80000000u);
   auto issue_a = [&](char *sa, int stage) {
+    const bool whole = stage < nstages - 1;
     const uint32_t a_so = static_cast<uint32_t>(min(stage, nstages - 1)) * (BKA * 2);
 #pragma unroll
-    for (int i = 0; i < DA; ++i) dma16(a_rsrc, a_off[i], a_so, sa + (wave + NWAVES * i) * 1024);
+    for (int i = 0; i < DA; ++i)
+      dma16(a_rsrc, (!Ragged || whole || a_lane_in_k) ? a_off[i] : kOutOfRange, a_so, sa + (wave + NWAVES * i) * 1024);
   };
   // B slabs go out in order; the source is a running pointer that stops at the last slab (the tail of the K loop
   // re-issues it into stages nobody reads any more, so the count of transfers in flight keeps its pattern)
-  const char *b_src = reinterpret_cast<const char *>(B + static_cast<int64_t>(k0) * N);
+  const char *b_src = reinterpret_cast<const char *>(B + static_cast<int64_t>(k0) * ld);
   int b_next = 0;
   auto issue_b = [&](char *sb) {
-    const __amdgpu_buffer_rsrc_t b_rsrc = make_rsrc(b_src, 0x80000000u);
+    const bool whole = b_next < nslabs - 1;
+    const int64_t b_left = b_end - b_src;
+    const __amdgpu_buffer_rsrc_t b_rsrc =
+        make_rsrc(b_src, Ragged && b_left < 0x80000000ll ? static_cast<uint32_t>(b_left) : kOutOfRange);
 #pragma unroll
-    for (int i = 0; i < DB; ++i) dma16(b_rsrc, b_off[i], 0u, sb + (wave + NWAVES * i) * 1024);
+    for (int i = 0; i < DB; ++i)
+      dma16(b_rsrc, (!Ragged || whole || b_lane_in_k[i]) ? b_off[i] : kOutOfRange, 0u, sb + (wave + NWAVES * i) * 1024);
     ++b_next;
     if (b_next < nslabs) b_src += b_slab_bytes;
   };
@@ -957,7 +993,7 @@ __global__ __launch_bounds__(256) void gemm16_m16_small_kernel(const uint16_t *_
     ((full + Is < nslabs ? slab(std::integral_constant<int, Is>{}, full + Is) : (void)0), ...);
   }(std::make_integer_sequence<int, P - 1>{});
   __builtin_amdgcn_s_waitcnt(waitcnt_vm_lgkm0(0));   // drain the (redundant) tail DMA before the LDS is released
-  epilogue16<Epi, 4, WN>(acc, C, bias, rowsum, M, N, m0, wm, wn, n0 + wn * 64, l16, g,
+  epilogue16<Epi, 4, WN>(acc, C, bias, rowsum, M, N, ld, m0, wm, wn, n0 + wn * 64, l16, g,
                          reinterpret_cast<float *>(lds_ring<30, A_BYTES_S>));
   if (probe && tid == 0) {
     probe[2 * blockIdx.x] = static_cast<unsigned long long>(clock64() - probe_c0);
@@ -1137,6 +1173,38 @@ inline bool small_tile_wins(int m, int n) {
   return cost_small < 0.9 * cost_large;
 }
 
+// Column N-1 of C for an odd N, one wave per row: the direct-to-LDS kernels fetch B in pairs of 16-bit elements, and
+// with rows an odd number of elements apart the pair that holds B[K-1][N-1] ends two bytes past B, so they compute
+// the N-1 columns before it (their buffer range ends right in front of that pair) and this kernel the last one, with
+// the same epilogue.  Lane l takes k = l, l + 64, ...; the 64 partial sums are added in a fixed tree.
+template <bool Bf16, int Epi>
+__global__ __launch_bounds__(256) void gemm16_last_column_kernel(const uint16_t *__restrict__ A,
+                                                                 const uint16_t *__restrict__ B, float *__restrict__ C,
+                                                                 const float *__restrict__ bias, float *__restrict__ rowsum,
+                                                                 int M, int N, int K) {
+  const int lane = threadIdx.x & 63;
+  const int row = blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (row >= M) return;   // whole waves leave together
+  auto widen = [](uint16_t bits) {
+    if constexpr (Bf16) return __uint_as_float(static_cast<uint32_t>(bits) << 16);
+    else return static_cast<float>(__builtin_bit_cast(_Float16, bits));
+  };
+  const uint16_t *a = A + static_cast<int64_t>(row) * K;
+  const uint16_t *b = B + (N - 1);
+  float sum = 0.f;
+  for (int k = lane; k < K; k += 64) sum += widen(a[k]) * widen(b[static_cast<int64_t>(k) * N]);
+#pragma unroll
+  for (int m = 32; m >= 1; m >>= 1) sum += __shfl_xor(sum, m, 64);
+  if (lane == 0) {
+    if constexpr (Epi == EPI_BIAS_RELU_ROWSUM) {
+      sum += bias[N - 1];
+      sum = sum > 0.f ? sum : 0.f;
+      atomicAdd(rowsum + row, sum);
+    }
+    C[static_cast<int64_t>(row) * N + N - 1] = sum;
+  }
+}
+
 // Adds the `splits` partial M x N planes of a K-split product into C, plane 0 first: a fixed order, so the result does
 // not depend on which workgroup finished when.
 __global__ __launch_bounds__(256) void splitk_reduce_kernel(const float *__restrict__ partials, float *__restrict__ C,
@@ -1186,7 +1254,7 @@ float *splitk_workspace(hipStream_t st) {
 int splitk_for(int m, int n, int k) {
   const int64_t tiles = static_cast<int64_t>((m + 127) / 128) * ((n + 127) / 128);
   const int64_t forced = tunable("gemm16.split_k", 0);
-  if (forced == 1) return 1;
+  if (forced == 1 || (static_cast<int64_t>(m) * n) % 4 != 0) return 1;   // the planes are added 16 bytes at a time
   static const int cus = [] {
     int dev = 0, v = 0;
     if (hipGetDevice(&dev) != hipSuccess ||
@@ -1212,8 +1280,14 @@ int splitk_for(int m, int n, int k) {
   }
   if (splits < 2) return 1;
   // whole K = 64 stages per piece; the count follows from the piece so that none is empty
-  const int chunk = static_cast<int>(((k / 64 + splits - 1) / splits) * 64);
+  const int chunk = static_cast<int>((((k + 63) / 64 + splits - 1) / splits) * 64);
   return (k + chunk - 1) / chunk;
+}
+
+// The kernel on v_mfma_f32_16x16x32 with nothing switched off: what a call gets unless a sweep knob says otherwise.
+inline bool gemm16_default_kernel() {
+  return tunable("gemm16.ring", 0) == 0 && tunable("gemm16.tj", 2) == 2 && tunable("gemm16.mfma", 16) == 16 &&
+         tunable("gemm16.ablate", 0) == 0;
 }
 
 // The workgroup tile of the direct-to-LDS kernels for this shape under the present tunables (256 or 128), or 0 when
@@ -1221,14 +1295,17 @@ int splitk_for(int m, int n, int k) {
 // property of the shape and is not looked at).
 int gemm16_tile_for(int m, int n, int k) {
   if (m < 1 || n < 1 || k < 1) return 0;
-  if (k % 8 != 0 || n % 8 != 0 || tunable("gemm16.force_simple", 0) != 0) return 0;
+  if (k % 8 != 0 || tunable("gemm16.force_simple", 0) != 0 || tunable("gemm16.force_staged", 0) != 0) return 0;
+  // transfer offsets are 32-bit: 256 rows of A and 64 rows of B must span less than 2 GiB
   const bool offsets_ok = static_cast<int64_t>(k) * 256 * 2 < 0x7FFFFFFF && static_cast<int64_t>(n) * 64 * 2 < 0x7FFFFFFF;
-  if (k % BK != 0 || !offsets_ok || tunable("gemm16.force_staged", 0) != 0) return 0;
-  const bool m16 = tunable("gemm16.ring", 0) == 0 && tunable("gemm16.tj", 2) == 2 && tunable("gemm16.mfma", 16) == 16;
-  if (!m16 || tunable("gemm16.ablate", 0) != 0) return 256;
-  // gemm16.tile: 256 | 128 forces the tile, 0 (default) picks by the tile counts
-  const int tile = (int)tunable("gemm16.tile", 0);
-  return (tile == 128 || (tile == 0 && small_tile_wins(m, n))) ? 128 : 256;
+  if (!offsets_ok) return 0;
+  if (gemm16_default_kernel()) {
+    // any N, any K that is a multiple of 8.  gemm16.tile: 256 | 128 forces the tile, 0 (default) picks by the tile counts
+    const int tile = (int)tunable("gemm16.tile", 0);
+    return (tile == 128 || (tile == 0 && small_tile_wins(m, n))) ? 128 : 256;
+  }
+  // the 32 x 32 x 16 kernel, its ring and wave shapes and the measurement variants: whole K = 64 stages, 16-byte rows of B
+  return (n % 8 == 0 && k % BK == 0) ? 256 : 0;
 }
 
 template <bool Bf16, int Epi>
@@ -1242,6 +1319,66 @@ int launch_gemm16(const uint16_t *a, const uint16_t *b, float *c, const float *b
     hipLaunchKernelGGL(zero_f32_kernel, dim3((m + 255) / 256), dim3(256), 0, st, rowsum, m);
     int rc = check_launch("rowsum clear launch");
     if (rc != SAREK_HIP_OK) return rc;
+  }
+  // The default kernels (v_mfma_f32_16x16x32, 256 x 256 or 128 x 128 tile) take any N and any K that is a multiple of 8:
+  // rows of A then keep the 16-byte alignment of its base, rows of B need none.
+  if (reinterpret_cast<uintptr_t>(a) % 16 == 0 && reinterpret_cast<uintptr_t>(b) % 16 == 0 && gemm16_default_kernel()) {
+    const int tile_choice = gemm16_tile_for(m, n, k);
+    if (tile_choice != 0) {
+      // an odd N: the tiled kernel takes the first N - 1 columns of the N-strided matrices, a matrix-vector kernel the last
+      const int nm = n - (n & 1);
+      const bool ragged = n % 8 != 0 || k % 64 != 0;   // the kernels' template flag: a K tail or B rows that are not 16-byte aligned
+      const int remap = (int)tunable("gemm.xcd_remap", 1);
+      int rc = SAREK_HIP_OK;
+      if (nm > 0 && tile_choice == 128) {
+        const int sm = (m + 127) / 128, sn = (nm + 127) / 128;
+        unsigned long long *sprobe = clock_probe(static_cast<int64_t>(sm) * sn);
+        int splits = 1;
+        float *partials = nullptr;
+        if constexpr (Epi == EPI_STORE) {
+          if (reinterpret_cast<uintptr_t>(c) % 16 == 0) splits = splitk_for(m, n, k);
+          if (splits > 1) partials = splitk_workspace(st);
+          if (!partials) splits = 1;
+        }
+        if (splits > 1) {
+          const int64_t mn = static_cast<int64_t>(m) * n;
+          const int chunk = (((k + 63) / 64 + splits - 1) / splits) * 64;
+          if (ragged)
+            hipLaunchKernelGGL((gemm16_m16_small_kernel<Bf16, Epi, true>), dim3(sm * sn, splits), dim3(256), 0, st, a, b, c,
+                               bias, rowsum, m, nm, k, sm, sn, remap, nullptr, chunk, partials, n);
+          else
+            hipLaunchKernelGGL((gemm16_m16_small_kernel<Bf16, Epi, false>), dim3(sm * sn, splits), dim3(256), 0, st, a, b, c,
+                               bias, rowsum, m, nm, k, sm, sn, remap, nullptr, chunk, partials, n);
+          rc = check_launch("gemm16 kernel launch");
+          if (rc != SAREK_HIP_OK) return rc;
+          hipLaunchKernelGGL(splitk_reduce_kernel, dim3(static_cast<unsigned>((mn / 4 + 255) / 256)), dim3(256), 0, st,
+                             partials, c, mn, splits);
+          rc = check_launch("gemm16 split-K reduction launch");
+        } else {
+          if (ragged)
+            hipLaunchKernelGGL((gemm16_m16_small_kernel<Bf16, Epi, true>), dim3(sm * sn), dim3(256), 0, st, a, b, c, bias,
+                               rowsum, m, nm, k, sm, sn, remap, sprobe, k, nullptr, n);
+          else
+            hipLaunchKernelGGL((gemm16_m16_small_kernel<Bf16, Epi, false>), dim3(sm * sn), dim3(256), 0, st, a, b, c, bias,
+                               rowsum, m, nm, k, sm, sn, remap, sprobe, k, nullptr, n);
+          rc = check_launch("gemm16 kernel launch");
+        }
+      } else if (nm > 0) {
+        const int tiles_m = (m + BM - 1) / BM, tiles_n = (nm + BN - 1) / BN;
+        unsigned long long *probe = clock_probe(static_cast<int64_t>(tiles_m) * tiles_n);
+        if (ragged)
+          hipLaunchKernelGGL((gemm16_m16_kernel<Bf16, Epi, 0, true>), dim3(tiles_m * tiles_n), dim3(512), 0, st, a, b, c, bias,
+                             rowsum, m, nm, k, tiles_m, tiles_n, remap, probe, n);
+        else
+          hipLaunchKernelGGL((gemm16_m16_kernel<Bf16, Epi, 0, false>), dim3(tiles_m * tiles_n), dim3(512), 0, st, a, b, c, bias,
+                             rowsum, m, nm, k, tiles_m, tiles_n, remap, probe, n);
+        rc = check_launch("gemm16 kernel launch");
+      }
+      if (rc != SAREK_HIP_OK || nm == n) return rc;
+      hipLaunchKernelGGL((gemm16_last_column_kernel<Bf16, Epi>), dim3((m + 3) / 4), dim3(256), 0, st, a, b, c, bias, rowsum,
+                         m, n, k);
+      return check_launch("gemm16 last-column launch");
+    }
   }
   // The MFMA kernel issues 16-byte loads: rows of A and B must keep 16-byte alignment.
   const bool vec_ok = (k % 8 == 0) && (n % 8 == 0) &&
@@ -1271,7 +1408,7 @@ int launch_gemm16(const uint16_t *a, const uint16_t *b, float *c, const float *b
         if constexpr (Bf16 && Epi == EPI_STORE) {
 #define SAREK_LAUNCH_M16_ABLATED(AB)                                                                        \
   hipLaunchKernelGGL((gemm16_m16_kernel<true, EPI_STORE, AB>), grid, dim3(512), 0, st, a, b, c, bias, rowsum, m, n, k, \
-                     tiles_m, tiles_n, remap, probe)
+                     tiles_m, tiles_n, remap, probe, n)
           if (ablate == 1) SAREK_LAUNCH_M16_ABLATED(1);
           else if (ablate == 2) SAREK_LAUNCH_M16_ABLATED(2);
           else SAREK_LAUNCH_M16_ABLATED(3);
@@ -1296,35 +1433,6 @@ int launch_gemm16(const uint16_t *a, const uint16_t *b, float *c, const float *b
           else SAREK_LAUNCH_ABLATED(4);
 #undef SAREK_LAUNCH_ABLATED
         }
-        return check_launch("gemm16 kernel launch");
-      }
-      if (m16) {
-        if (gemm16_tile_for(m, n, k) == 128) {
-          const int sm = (m + 127) / 128, sn = (n + 127) / 128;
-          unsigned long long *sprobe = clock_probe(static_cast<int64_t>(sm) * sn);
-          if constexpr (Epi == EPI_STORE) {
-            const int splits = reinterpret_cast<uintptr_t>(c) % 16 == 0 ? splitk_for(m, n, k) : 1;
-            if (splits > 1) {
-              const int64_t mn = static_cast<int64_t>(m) * n;
-              float *partials = splitk_workspace(st);
-              if (partials) {
-                const int chunk = ((k / 64 + splits - 1) / splits) * 64;
-                hipLaunchKernelGGL((gemm16_m16_small_kernel<Bf16, Epi>), dim3(sm * sn, splits), dim3(256), 0, st, a, b, c,
-                                   bias, rowsum, m, n, k, sm, sn, remap, nullptr, chunk, partials);
-                int rc = check_launch("gemm16 kernel launch");
-                if (rc != SAREK_HIP_OK) return rc;
-                hipLaunchKernelGGL(splitk_reduce_kernel, dim3(static_cast<unsigned>((mn / 4 + 255) / 256)), dim3(256), 0, st,
-                                   partials, c, mn, splits);
-                return check_launch("gemm16 split-K reduction launch");
-              }
-            }
-          }
-          hipLaunchKernelGGL((gemm16_m16_small_kernel<Bf16, Epi>), dim3(sm * sn), dim3(256), 0, st, a, b, c, bias, rowsum,
-                             m, n, k, sm, sn, remap, sprobe, k, nullptr);
-          return check_launch("gemm16 kernel launch");
-        }
-        hipLaunchKernelGGL((gemm16_m16_kernel<Bf16, Epi>), grid, dim3(512), 0, st, a, b, c, bias, rowsum, m, n, k,
-                           tiles_m, tiles_n, remap, probe);
         return check_launch("gemm16 kernel launch");
       }
       if (ring == 4 && tj == 2) SAREK_LAUNCH_DMA(32, 32, 4, 4, 2);

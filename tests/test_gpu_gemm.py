@@ -109,7 +109,8 @@ def test_gemm16_vs_oracle(hip, oracle, torch_cuda, kind, m, n, k):
 @pytest.mark.parametrize("kind", ["bf16", "f16"])
 def test_gemm16_unaligned_shapes_use_fallback(hip, oracle, torch_cuda, kind):
     torch = torch_cuda
-    m, n, k = 37, 51, 29   # n, k not multiples of 8
+    m, n, k = 37, 51, 29   # k not a multiple of 8: rows of A are not 16-byte aligned
+    assert hip.gemm16_tile(m, n, k) == 0
     a = normal16(oracle, (m, k), 1, kind)
     b = normal16(oracle, (k, n), 2, kind)
     tdt = torch.bfloat16 if kind == "bf16" else torch.float16
@@ -378,7 +379,8 @@ def test_gemm16_tile_choice_by_shape(hip, torch_cuda):
     for products of several rounds; shapes the direct-to-LDS kernels do not take report 0."""
     for (m, n, k), want in [((1024, 1024, 64), 128), ((2048, 2048, 2048), 128), ((1024, 4096, 4096), 128),
                             ((4096, 2048, 8192), 128), ((3072, 3072, 3072), 256), ((4096, 4096, 4096), 256),
-                            ((8192, 8192, 8192), 256), ((4095, 11008, 4096), 256), ((512, 512, 72), 0),
+                            ((8192, 8192, 8192), 256), ((4095, 11008, 4096), 256), ((512, 512, 72), 128), ((4096, 4100, 4096), 256),
+                            ((1000, 1001, 1000), 128),
                             ((37, 51, 29), 0)]:
         assert hip.gemm16_tile(m, n, k) == want, (m, n, k)
     hip.set_tunable("gemm16.mfma", 32)
@@ -487,3 +489,62 @@ def test_gemm16_split_k_under_graph_capture(hip, torch_cuda):
         finally:
             hip.set_tunable("gemm16.split_k", 0)
         assert torch.equal(got, want), seed
+
+
+RAGGED_SHAPES = [(1, 1, 8), (3, 5, 8), (37, 51, 24), (130, 137, 40), (256, 255, 64), (257, 1001, 1000),
+                 (300, 262, 136), (512, 514, 4104), (777, 1003, 328), (64, 4100, 96), (1000, 3, 2056)]
+
+
+@pytest.mark.parametrize("kind", ["bf16", "f16"])
+@pytest.mark.parametrize("m,n,k", RAGGED_SHAPES)
+def test_gemm16_ragged_shapes_stay_on_the_mfma_kernels(hip, oracle, torch_cuda, kind, m, n, k):
+    """Any N (odd ones included: rows of B and C then have no alignment at all) and any K that is a multiple of 8
+    (a K tail inside the last LDS stage) run on the direct-to-LDS kernels, both tiles, K split or not: against the
+    oracle; nothing is stored outside C; NaNs lying next to A and B in memory (what the transfers fetch past a row's
+    or the matrix's end) do not reach the result."""
+    torch = torch_cuda
+    a = normal16(oracle, (m, k), m + 41, kind)
+    b = normal16(oracle, (k, n), n + 42, kind)
+    dt = torch.bfloat16 if kind == "bf16" else torch.float16
+    fn = hip.gemm_bf16 if kind == "bf16" else hip.gemm_f16
+    ref = oracle.gemm(a, b)
+    # operands as views into NaN-filled buffers, 16-byte aligned as the kernels require of A and B
+    buf_a = torch.full((m * k + 256,), float("nan"), device="cuda").to(dt)
+    buf_b = torch.full((k * n + 256,), float("nan"), device="cuda").to(dt)
+    da, db = buf_a[128:128 + m * k].view(m, k), buf_b[128:128 + k * n].view(k, n)
+    da.copy_(dev(torch, a).to(dt))
+    db.copy_(dev(torch, b).to(dt))
+    try:
+        for tile, split in ((128, 1), (128, 0), (128, 3), (256, 1)):
+            hip.set_tunable("gemm16.tile", tile)
+            hip.set_tunable("gemm16.split_k", split)
+            assert hip.gemm16_tile(m, n, k) == tile
+            guard = torch.full((m * n + 64,), 7.0, device="cuda")
+            c = guard[32:32 + m * n].view(m, n)
+            fn(da, db, out=c)
+            assert bool((guard[:32] == 7).all()) and bool((guard[32 + m * n:] == 7).all())
+            got = c.cpu().numpy()
+            assert np.isfinite(got).all()
+            assert np.abs(got - ref).max() / np.abs(ref).max() < 1e-4, (tile, split)
+    finally:
+        hip.set_tunable("gemm16.tile", 0)
+        hip.set_tunable("gemm16.split_k", 0)
+
+
+@pytest.mark.parametrize("m,n,k", [(130, 137, 40), (257, 1001, 1000), (64, 4100, 96), (4, 1, 64), (300, 263, 136)])
+def test_epilogue_ragged_shapes(hip, oracle, torch_cuda, m, n, k):
+    """The fused epilogue on the same kinds of shape (the last column of an odd N comes from the matrix-vector kernel,
+    which applies bias and ReLU and adds into the row sums like the tiled kernels)."""
+    torch = torch_cuda
+    a = normal16(oracle, (m, k), m + 51, "f16")
+    b = normal16(oracle, (k, n), n + 52, "f16")
+    bias = oracle.fill_uniform(n, seed=n + 53, lo=-0.1, hi=0.1)
+    y_ref, rs_ref = oracle.gemm_bias_relu_rowsum(a, b, bias)
+    try:
+        for tile in (128, 256):
+            hip.set_tunable("gemm16.tile", tile)
+            y, rs = hip.gemm_f16_bias_relu_rowsum(dev(torch, a).half(), dev(torch, b).half(), dev(torch, bias))
+            assert np.abs(y.cpu().numpy() - y_ref).max() <= 1e-4 * max(np.abs(y_ref).max(), 1e-30)
+            assert np.abs(rs.cpu().numpy() - rs_ref).max() <= 1e-4 * max(np.abs(rs_ref).max(), 1e-30)
+    finally:
+        hip.set_tunable("gemm16.tile", 0)
