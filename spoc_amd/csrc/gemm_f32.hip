@@ -164,7 +164,13 @@ __global__ __launch_bounds__(THREADS) void gemm_f32_staged_kernel(const float *_
 // (16-lane phases of ds_read_b128).  B reads are contiguous across lanes; only for TJ = 1
 // the two half-waves (rows r, r+4) would meet modulo 256 B, so rows with bit 2 set are
 // stored with their 128-byte halves swapped.
-template <int TI, int TJ, int WMW, int WNW, int BKT, int NS>
+//
+// Ragged = false: N % 4 == 0, K % BKT == 0, A, B and C 16-byte aligned.  Ragged = true: any N, any K >= BKT (or a multiple of
+// 4 below it), any alignment.  A lane whose offset lies outside the buffer resource's range brings zeros into LDS, the range
+// is checked per dword and the address needs no alignment beyond the element's, so B rows that must not count are a per-lane
+// choice between the usual offset and one past the range, B's range ends with its last element, pieces past column N bring
+// the next row's elements into columns that are never stored, and C is stored element by element.
+template <int TI, int TJ, int WMW, int WNW, int BKT, int NS, bool Ragged = false>
 __global__ __launch_bounds__(64 * WMW * WNW) void gemm_f32_dma_kernel(
     const float *__restrict__ A, const float *__restrict__ B, float *__restrict__ C, int M, int N,
     int K, int tiles_m, int tiles_n, int xcd_remap, unsigned long long *probe) {
@@ -213,13 +219,30 @@ __global__ __launch_bounds__(64 * WMW * WNW) void gemm_f32_dma_kernel(
     const int q = wave + NWAVES * i;
     const int brow = q * B_ROWS_PER_DMA + lane / B_CHUNKS;
     const int chunk = (lane % B_CHUNKS) ^ b_swz(brow);
-    const int col = min(n0 + chunk * 4, N - 4);
+    const int col = Ragged ? n0 + chunk * 4 : min(n0 + chunk * 4, N - 4);
     b_off[i] = (static_cast<uint32_t>(brow) * N + col) * 4u;
   }
   const char *a_base = reinterpret_cast<const char *>(A + static_cast<int64_t>(m0) * K);
   const char *b_base = reinterpret_cast<const char *>(B);
   const int64_t b_slab_bytes = static_cast<int64_t>(BKT) * N * 4;
-  const int nslabs = K / BKT;
+  const int nslabs = (K + BKT - 1) / BKT;
+  // The end of K inside the last slab.  With K >= BKT the last slab is moved back to end at K (its A pieces then hold
+  // nothing but elements of their own row, at whatever alignment) and the B rows it shares with the slab before it
+  // are the ones left out; with a single slab (K < BKT, K % 4 == 0) the A pieces and B rows past K are.  A lane's k
+  // piece is the same for all its A transfers: rows NWAVES * A_ROWS_PER_DMA apart share the swizzle.
+  const int k_tail = K - (nslabs - 1) * BKT;
+  const bool move_last = Ragged && K >= BKT && k_tail != BKT;
+  const int k_last = move_last ? K - BKT : (nslabs - 1) * BKT;   // first k of the last slab
+  const bool a_lane_in_k =
+      !Ragged || move_last || (((lane % A_CHUNKS) ^ a_swz(wave * A_ROWS_PER_DMA + lane / A_CHUNKS)) << 2) < k_tail;
+  bool b_lane_in_k[B_DMA];
+#pragma unroll
+  for (int i = 0; i < B_DMA; ++i) {
+    const int brow = (wave + NWAVES * i) * B_ROWS_PER_DMA + lane / B_CHUNKS;
+    b_lane_in_k[i] = !Ragged || (move_last ? brow >= BKT - k_tail : brow < k_tail);
+  }
+  const char *b_end = b_base + static_cast<int64_t>(K) * N * 4;
+  constexpr uint32_t kOutOfRange = 0x80000000u;
 
   f32x16 acc[TI][TJ];
 #pragma unroll
@@ -245,12 +268,18 @@ __global__ __launch_bounds__(64 * WMW * WNW) void gemm_f32_dma_kernel(
   const __amdgpu_buffer_rsrc_t a_rsrc = make_rsrc(a_base, 0x80000000u);
   auto issue = [&](char *sa, char *sb, int slab) {
     const int sl = min(slab, nslabs - 1);   // the tail re-issues the last slab: constant vmcnt
-    const __amdgpu_buffer_rsrc_t b_rsrc = make_rsrc(b_base + sl * b_slab_bytes, 0x80000000u);
-    const uint32_t a_so = static_cast<uint32_t>(sl) * (BKT * 4);
+    const bool whole = !Ragged || slab < nslabs - 1;
+    const char *b_src = whole ? b_base + sl * b_slab_bytes : b_base + static_cast<int64_t>(k_last) * N * 4;
+    const int64_t b_left = b_end - b_src;
+    const __amdgpu_buffer_rsrc_t b_rsrc =
+        make_rsrc(b_src, Ragged && b_left < 0x80000000ll ? static_cast<uint32_t>(b_left) : kOutOfRange);
+    const uint32_t a_so = static_cast<uint32_t>(whole ? sl * BKT : k_last) * 4u;
 #pragma unroll
-    for (int i = 0; i < A_DMA; ++i) dma16(a_rsrc, a_off[i], a_so, sa + (wave + NWAVES * i) * 1024);
+    for (int i = 0; i < A_DMA; ++i)
+      dma16(a_rsrc, (whole || a_lane_in_k) ? a_off[i] : kOutOfRange, a_so, sa + (wave + NWAVES * i) * 1024);
 #pragma unroll
-    for (int i = 0; i < B_DMA; ++i) dma16(b_rsrc, b_off[i], 0u, sb + (wave + NWAVES * i) * 1024);
+    for (int i = 0; i < B_DMA; ++i)
+      dma16(b_rsrc, (whole || b_lane_in_k[i]) ? b_off[i] : kOutOfRange, 0u, sb + (wave + NWAVES * i) * 1024);
   };
   auto load_frags = [&](const char *sa, const char *sb, int kk, f32x4 (&af)[TI], bvec_t (&bf)[4]) {
     const char *pa = sa + (a_addr0 ^ (kk << 5));
@@ -363,7 +392,11 @@ __global__ __launch_bounds__(64 * WMW * WNW) void gemm_f32_dma_kernel(
     for (int r = 0; r < 16; ++r) {
       const int row = m0 + wm * 32 * TI + i * 32 + 8 * (r >> 2) + 4 * lh + (r & 3);
       const int col = n0 + wn * 32 * TJ + TJ * lm;
-      if (row < M && col < N) {
+      if constexpr (Ragged) {
+#pragma unroll
+        for (int jn = 0; jn < TJ; ++jn)
+          if (row < M && col + jn < N) C[static_cast<int64_t>(row) * N + col + jn] = acc[i][jn][r];
+      } else if (row < M && col < N) {
         bvec_t v;
 #pragma unroll
         for (int jn = 0; jn < TJ; ++jn) v[jn] = acc[i][jn][r];
@@ -401,49 +434,57 @@ extern "C" int sarek_hip_gemm_f32(const float *a, const float *b, float *c, int 
     return fail(SAREK_HIP_E_INVALID_ARG, "gemm_f32: m, n, k must be positive (got %d %d %d)", m, n, k);
   if (!a || !b || !c) return fail(SAREK_HIP_E_INVALID_ARG, "gemm_f32: NULL matrix");
   hipStream_t st = as_stream(stream);
-  const bool vec_ok = (k % 4 == 0) && (n % 4 == 0) &&
-                      (reinterpret_cast<uintptr_t>(a) % 16 == 0) &&
-                      (reinterpret_cast<uintptr_t>(b) % 16 == 0);
-  if (vec_ok && tunable("gemm_f32.force_simple", 0) == 0) {
-    const int remap = (int)tunable("gemm.xcd_remap", 1);
-    // DMA offsets are 32-bit: 256 rows of A and 32 rows of B must span less than 2 GiB
-    const bool offsets_ok = static_cast<int64_t>(k) * 256 * 4 < 0x7FFFFFFF &&
-                            static_cast<int64_t>(n) * 32 * 4 < 0x7FFFFFFF;
-    if (k % 32 == 0 && offsets_ok && reinterpret_cast<uintptr_t>(c) % 16 == 0 &&
-        tunable("gemm_f32.force_staged", 0) == 0) {
-      // Tile choice by a cost model of the launch: a CU holds `occ` workgroups of a tile
-      // shape at once (LDS ring), tiles run in rounds of cus*occ, a workgroup that shares
-      // its CU takes occ times as long, and the tail round runs unshared when it fits one
-      // workgroup per CU.  `eff` is the MFMA issue efficiency measured for each shape.
-      auto ntiles = [&](int t) { return static_cast<int64_t>((m + t - 1) / t) * ((n + t - 1) / t); };
-      static const int cus = [] {
-        int dev = 0, v = 0;
-        if (hipGetDevice(&dev) != hipSuccess ||
-            hipDeviceGetAttribute(&v, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || v <= 0)
-          v = 256;
-        return v;
-      }();
-      auto cost = [&](int t, int occ, double eff) {
-        const int64_t tiles = ntiles(t), slots = static_cast<int64_t>(cus) * occ;
-        const int64_t full = tiles / slots, rest = tiles % slots;
-        const double rounds = static_cast<double>(full) * occ + (rest == 0 ? 0 : rest <= cus ? 1 : occ);
-        return rounds * t * t / eff;
-      };
-      int tile = (int)tunable("gemm_f32.tile", 0);
-      if (tile == 0) {
-        const double c256 = cost(256, 1, 1.0), c128 = cost(128, 2, 0.95), c64 = cost(64, 2, 0.80);
-        tile = (c256 <= c128 && c256 <= c64) ? 256 : (c128 <= c64 ? 128 : 64);
-      }
-#define SAREK_LAUNCH_F32(T, TI, TJ, WMW, WNW, BKT)                                               \
-  hipLaunchKernelGGL((gemm_f32_dma_kernel<TI, TJ, WMW, WNW, BKT, 4>),                             \
+  // The direct-to-LDS kernels take any shape and alignment in their Ragged form, except a K below one slab that is
+  // not a multiple of 4; the aligned form is the faster one where it applies.
+  const bool aligned = (k % 4 == 0) && (reinterpret_cast<uintptr_t>(a) % 16 == 0) &&
+                       (reinterpret_cast<uintptr_t>(b) % 16 == 0);
+  const bool ab_ok = aligned || k >= 32;   // the ragged form needs no alignment once K fills a slab
+  const int remap = (int)tunable("gemm.xcd_remap", 1);
+  // DMA offsets are 32-bit: 256 rows of A and 32 rows of B must span less than 2 GiB
+  const bool offsets_ok = static_cast<int64_t>(k) * 256 * 4 < 0x7FFFFFFF &&
+                          static_cast<int64_t>(n) * 32 * 4 < 0x7FFFFFFF;
+  if (ab_ok && offsets_ok && tunable("gemm_f32.force_simple", 0) == 0 && tunable("gemm_f32.force_staged", 0) == 0) {
+    const bool ragged = !aligned || n % 4 != 0 || k % 32 != 0 || reinterpret_cast<uintptr_t>(c) % 16 != 0;
+    // Tile choice by a cost model of the launch: a CU holds `occ` workgroups of a tile
+    // shape at once (LDS ring), tiles run in rounds of cus*occ, a workgroup that shares
+    // its CU takes occ times as long, and the tail round runs unshared when it fits one
+    // workgroup per CU.  `eff` is the MFMA issue efficiency measured for each shape.
+    auto ntiles = [&](int t) { return static_cast<int64_t>((m + t - 1) / t) * ((n + t - 1) / t); };
+    static const int cus = [] {
+      int dev = 0, v = 0;
+      if (hipGetDevice(&dev) != hipSuccess ||
+          hipDeviceGetAttribute(&v, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || v <= 0)
+        v = 256;
+      return v;
+    }();
+    auto cost = [&](int t, int occ, double eff) {
+      const int64_t tiles = ntiles(t), slots = static_cast<int64_t>(cus) * occ;
+      const int64_t full = tiles / slots, rest = tiles % slots;
+      const double rounds = static_cast<double>(full) * occ + (rest == 0 ? 0 : rest <= cus ? 1 : occ);
+      return rounds * t * t / eff;
+    };
+    int tile = (int)tunable("gemm_f32.tile", 0);
+    if (tile == 0) {
+      const double c256 = cost(256, 1, 1.0), c128 = cost(128, 2, 0.95), c64 = cost(64, 2, 0.80);
+      tile = (c256 <= c128 && c256 <= c64) ? 256 : (c128 <= c64 ? 128 : 64);
+    }
+#define SAREK_LAUNCH_F32(T, TI, TJ, WMW, WNW, BKT, RAGGED)                                         \
+  hipLaunchKernelGGL((gemm_f32_dma_kernel<TI, TJ, WMW, WNW, BKT, 4, RAGGED>),                     \
                      dim3((unsigned)ntiles(T)), dim3(64 * WMW * WNW), 0, st, a, b, c, m, n, k,    \
                      (m + T - 1) / T, (n + T - 1) / T, remap, clock_probe(ntiles(T)))
-      if (tile == 256) SAREK_LAUNCH_F32(256, 4, 2, 2, 4, 16);
-      else if (tile == 128) SAREK_LAUNCH_F32(128, 2, 2, 2, 2, 16);
-      else SAREK_LAUNCH_F32(64, 1, 1, 2, 2, 32);
-#undef SAREK_LAUNCH_F32
-      return check_launch("gemm_f32 kernel launch");
+    if (ragged) {
+      if (tile == 256) SAREK_LAUNCH_F32(256, 4, 2, 2, 4, 16, true);
+      else if (tile == 128) SAREK_LAUNCH_F32(128, 2, 2, 2, 2, 16, true);
+      else SAREK_LAUNCH_F32(64, 1, 1, 2, 2, 32, true);
+    } else {
+      if (tile == 256) SAREK_LAUNCH_F32(256, 4, 2, 2, 4, 16, false);
+      else if (tile == 128) SAREK_LAUNCH_F32(128, 2, 2, 2, 2, 16, false);
+      else SAREK_LAUNCH_F32(64, 1, 1, 2, 2, 32, false);
     }
+#undef SAREK_LAUNCH_F32
+    return check_launch("gemm_f32 kernel launch");
+  }
+  if (aligned && n % 4 == 0 && tunable("gemm_f32.force_simple", 0) == 0) {
     static bool attr_done = false;
     if (!attr_done) {
       SAREK_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(gemm_f32_staged_kernel),

@@ -548,3 +548,34 @@ def test_epilogue_ragged_shapes(hip, oracle, torch_cuda, m, n, k):
             assert np.abs(rs.cpu().numpy() - rs_ref).max() <= 1e-4 * max(np.abs(rs_ref).max(), 1e-30)
     finally:
         hip.set_tunable("gemm16.tile", 0)
+
+
+@pytest.mark.parametrize("tile", [0, 64, 128, 256])
+@pytest.mark.parametrize("m,n,k", [(130, 137, 41), (257, 1001, 1001), (300, 263, 35), (64, 65, 33), (512, 514, 1030),
+                                   (1000, 3, 2051), (1, 1, 4), (37, 51, 24), (256, 255, 64), (70, 1028, 288)])
+def test_gemm_f32_ragged_shapes_stay_on_the_mfma_kernel(hip, oracle, torch_cuda, tile, m, n, k):
+    """Any N, any K of at least a slab (or a multiple of 4 below it) and any alignment of A, B and C run on the
+    direct-to-LDS kernel, every tile shape: against the oracle; nothing is stored outside C; NaNs lying next to A and B
+    in memory (what the transfers fetch past a row's or the matrix's end) do not reach the result."""
+    torch = torch_cuda
+    a = oracle.fill_uniform(m * k, seed=m + 61, lo=-1, hi=1).reshape(m, k)
+    b = oracle.fill_uniform(k * n, seed=n + 62, lo=-1, hi=1).reshape(k, n)
+    ref = oracle.gemm(a, b)
+    off = 129 if k >= 32 else 128          # a base that is only 4-byte aligned where the kernel allows it
+    buf_a = torch.full((m * k + 256,), float("nan"), device="cuda")
+    buf_b = torch.full((k * n + 256,), float("nan"), device="cuda")
+    da, db = buf_a[off:off + m * k].view(m, k), buf_b[off:off + k * n].view(k, n)
+    da.copy_(dev(torch, a))
+    db.copy_(dev(torch, b))
+    hip.set_tunable("gemm_f32.tile", tile)
+    try:
+        for c_off in (32, 33):
+            guard = torch.full((m * n + 80,), 7.0, device="cuda")
+            c = guard[c_off:c_off + m * n].view(m, n)
+            hip.gemm_f32(da, db, out=c)
+            assert bool((guard[:c_off] == 7).all()) and bool((guard[c_off + m * n:] == 7).all())
+            got = c.cpu().numpy()
+            assert np.isfinite(got).all()
+            assert np.abs(got - ref).max() <= f32_tol(a, b, k)
+    finally:
+        hip.set_tunable("gemm_f32.tile", 0)
