@@ -543,9 +543,10 @@ int sarek_hip_gemm_f16(const uint16_t *a, const uint16_t *b, float *c, int m, in
 /* Which kernel the three 16-bit GEMM entry points take for a shape under the
  * present tunables: 256 or 128 = the workgroup tile of the direct-to-LDS MFMA
  * kernels (the small tile where large ones would leave CUs idle; any n, any
- * k that is a multiple of 8), 0 = the one-thread-per-element kernel (k not a
- * multiple of 8: rows of a without 16-byte alignment; a or b itself not 16-byte
- * aligned has the same effect).  No counterpart in the reference, whose tiled
+ * k >= 64 and the multiples of 8 below, any alignment of a and b from k = 64
+ * on), 0 = the one-thread-per-element kernel (k < 64 that is not a multiple
+ * of 8; below 64 an a or b that is not 16-byte aligned has the same effect).
+ * No counterpart in the reference, whose tiled
  * kernel has one shape (bench_matrix_mul_tiled.ml:55-95); needs no device.  */
 int sarek_hip_gemm16_tile(int m, int n, int k);
 /* Into how many pieces sarek_hip_gemm_bf16 / _f16 cut K for this shape now (1 =

@@ -609,15 +609,27 @@ __global__ __launch_bounds__(512) void gemm16_m16_kernel(const uint16_t *__restr
   const char *a_base = reinterpret_cast<const char *>(A + static_cast<int64_t>(m0) * K);
   const char *b_base = reinterpret_cast<const char *>(B);
   const int64_t b_slab_bytes = static_cast<int64_t>(BKB) * ld * 2;
-  const int nslabs = (K + BKB - 1) / BKB, nstages = (K + BKA - 1) / BKA;
-  // K need not fill the last A stage or B slab (K % 8 == 0): there the lanes whose 16-byte piece (A) or row (B) lies
-  // past K give an offset outside the buffer range, which the transfer writes to LDS as zeros.  A lane's k piece is
-  // the same for all its transfers of a stage (rows 16 apart share the swizzle); its B rows are 16 apart.
-  const int k_tail_a = K - (nstages - 1) * BKA, k_tail_b = K - (nslabs - 1) * BKB;
-  const bool a_lane_in_k = !Ragged || (((lane % A_CHUNKS) ^ a_swz(wave * A_ROWS_PER_DMA + lane / A_CHUNKS)) << 3) < k_tail_a;
-  bool b_lane_in_k[DB];
+  // Ragged: K need not fill the last A stage.  A lane whose offset lies outside the buffer resource's range brings
+  // zeros into LDS, so k that must not count are a per-lane choice between the usual offset and one past the range.
+  // From one whole stage on (K >= 64) the last stage is moved back to end at K: its A pieces then hold nothing but
+  // elements of their own rows, at whatever alignment, and the B rows it shares with the stage before it are the
+  // lanes sent out of range, in the first of its two slabs and, past 32 shared rows, in the second.  Below one stage
+  // (K % 8 == 0) the A pieces and B rows past K are.  A lane's k piece is the same for all its transfers of a stage
+  // (rows 16 apart share the swizzle).
+  const int nstages = (K + BKA - 1) / BKA;
+  const bool move_last = Ragged && K >= BKA && K % BKA != 0;
+  const int nslabs = move_last ? RA * nstages : (K + BKB - 1) / BKB;
+  const int k_tail_a = K - (nstages - 1) * BKA, k_tail_b = K - (nslabs - 1) * BKB;   // single stage
+  const int shared_k = nstages * BKA - K;                                               // moved stage
+  const bool a_lane_in_k = !Ragged || move_last ||
+                           (((lane % A_CHUNKS) ^ a_swz(wave * A_ROWS_PER_DMA + lane / A_CHUNKS)) << 3) < k_tail_a;
+  bool b_in_last[DB], b_in_prev[DB];   // the lanes that count in the last slab and in the one before it
 #pragma unroll
-  for (int i = 0; i < DB; ++i) b_lane_in_k[i] = !Ragged || 2 * (wave + NWAVES * i) + (lane >> 5) < k_tail_b;
+  for (int i = 0; i < DB; ++i) {
+    const int brow = 2 * (wave + NWAVES * i) + (lane >> 5);
+    b_in_last[i] = !Ragged || (move_last ? brow + BKB >= shared_k : brow < k_tail_b);
+    b_in_prev[i] = !move_last || brow >= shared_k;
+  }
   const char *b_end = b_base + (static_cast<int64_t>(K - 1) * ld + N) * 2;   // the end of row K-1's N columns
   constexpr uint32_t kOutOfRange = 0x80000000u;
 
@@ -641,7 +653,7 @@ __global__ __launch_bounds__(512) void gemm16_m16_kernel(const uint16_t *__restr
   auto issue_a = [&](char *sa, int stage) {
     if (stage >= NA && (Ablate & 1)) return;
     const bool whole = stage < nstages - 1;
-    const uint32_t a_so = static_cast<uint32_t>(min(stage, nstages - 1)) * (BKA * 2);
+    const uint32_t a_so = static_cast<uint32_t>(!whole && move_last ? K - BKA : min(stage, nstages - 1) * BKA) * 2u;
 #pragma unroll
     for (int i = 0; i < DA; ++i)
       dma16(a_rsrc, (!Ragged || whole || a_lane_in_k) ? a_off[i] : kOutOfRange, a_so, sa + (wave + NWAVES * i) * 1024);
@@ -654,13 +666,15 @@ __global__ __launch_bounds__(512) void gemm16_m16_kernel(const uint16_t *__restr
   auto issue_b = [&](char *sb, int slab) {
     if (slab >= NB && (Ablate & 1)) return;
     (void)slab;   // == b_next
-    const bool whole = b_next < nslabs - 1;
+    const bool last = b_next >= nslabs - 1, prev = b_next == nslabs - 2;
+    if (move_last && prev) b_src = b_base + static_cast<int64_t>(K - BKA) * ld * 2;
     const int64_t b_left = b_end - b_src;
     const __amdgpu_buffer_rsrc_t b_rsrc =
         make_rsrc(b_src, Ragged && b_left < 0x80000000ll ? static_cast<uint32_t>(b_left) : kOutOfRange);
 #pragma unroll
     for (int i = 0; i < DB; ++i)
-      dma16(b_rsrc, (!Ragged || whole || b_lane_in_k[i]) ? b_off[i] : kOutOfRange, 0u, sb + (wave + NWAVES * i) * 1024);
+      dma16(b_rsrc, (!Ragged || (last ? b_in_last[i] : prev ? b_in_prev[i] : true)) ? b_off[i] : kOutOfRange, 0u,
+            sb + (wave + NWAVES * i) * 1024);
     ++b_next;
     if (b_next < nslabs) b_src += b_slab_bytes;
   };
@@ -854,13 +868,27 @@ __global__ __launch_bounds__(256) void gemm16_m16_small_kernel(const uint16_t *_
   if (gridDim.y > 1) C = partials + static_cast<int64_t>(blockIdx.y) * M * ld;
   const char *a_base = reinterpret_cast<const char *>(A + static_cast<int64_t>(m0) * K + k0);
   const int64_t b_slab_bytes = static_cast<int64_t>(BKB) * ld * 2;
-  const int nslabs = (k_len + BKB - 1) / BKB, nstages = (k_len + BKA - 1) / BKA;
-  // the end of K inside the last A stage / B slab, as in the large tile
-  const int k_tail_a = k_len - (nstages - 1) * BKA, k_tail_b = k_len - (nslabs - 1) * BKB;
-  const bool a_lane_in_k = !Ragged || (((lane % A_CHUNKS) ^ a_swz(wave * A_ROWS_PER_DMA + lane / A_CHUNKS)) << 3) < k_tail_a;
-  bool b_lane_in_k[DB];
+  // Ragged: K need not fill the last A stage.  A lane whose offset lies outside the buffer resource's range brings
+  // zeros into LDS, so k that must not count are a per-lane choice between the usual offset and one past the range.
+  // From one whole stage on (K >= 64) the last stage is moved back to end at K: its A pieces then hold nothing but
+  // elements of their own rows, at whatever alignment, and the B rows it shares with the stage before it are the
+  // lanes sent out of range, in the first of its two slabs and, past 32 shared rows, in the second.  Below one stage
+  // (K % 8 == 0) the A pieces and B rows past K are.  A lane's k piece is the same for all its transfers of a stage
+  // (rows 16 apart share the swizzle).
+  const int nstages = (k_len + BKA - 1) / BKA;
+  const bool move_last = Ragged && k_len >= BKA && k_len % BKA != 0;
+  const int nslabs = move_last ? RA * nstages : (k_len + BKB - 1) / BKB;
+  const int k_tail_a = k_len - (nstages - 1) * BKA, k_tail_b = k_len - (nslabs - 1) * BKB;   // single stage
+  const int shared_k = nstages * BKA - k_len;                                               // moved stage
+  const bool a_lane_in_k = !Ragged || move_last ||
+                           (((lane % A_CHUNKS) ^ a_swz(wave * A_ROWS_PER_DMA + lane / A_CHUNKS)) << 3) < k_tail_a;
+  bool b_in_last[DB], b_in_prev[DB];   // the lanes that count in the last slab and in the one before it
 #pragma unroll
-  for (int i = 0; i < DB; ++i) b_lane_in_k[i] = !Ragged || (wave + NWAVES * i) * B_ROWS_PER_DMA + lane / B_CHUNKS < k_tail_b;
+  for (int i = 0; i < DB; ++i) {
+    const int brow = (wave + NWAVES * i) * B_ROWS_PER_DMA + lane / B_CHUNKS;
+    b_in_last[i] = !Ragged || (move_last ? brow + BKB >= shared_k : brow < k_tail_b);
+    b_in_prev[i] = !move_last || brow >= shared_k;
+  }
   const char *b_end = reinterpret_cast<const char *>(B) + (static_cast<int64_t>(K - 1) * ld + N) * 2;
   constexpr uint32_t kOutOfRange = 0x80000000u;
 
@@ -880,7 +908,7 @@ __global__ __launch_bounds__(256) void gemm16_m16_small_kernel(const uint16_t *_
   const __amdgpu_buffer_rsrc_t a_rsrc = make_rsrc(a_base, 0x80000000u);
   auto issue_a = [&](char *sa, int stage) {
     const bool whole = stage < nstages - 1;
-    const uint32_t a_so = static_cast<uint32_t>(min(stage, nstages - 1)) * (BKA * 2);
+    const uint32_t a_so = static_cast<uint32_t>(!whole && move_last ? k_len - BKA : min(stage, nstages - 1) * BKA) * 2u;
 #pragma unroll
     for (int i = 0; i < DA; ++i)
       dma16(a_rsrc, (!Ragged || whole || a_lane_in_k) ? a_off[i] : kOutOfRange, a_so, sa + (wave + NWAVES * i) * 1024);
@@ -890,13 +918,15 @@ __global__ __launch_bounds__(256) void gemm16_m16_small_kernel(const uint16_t *_
   const char *b_src = reinterpret_cast<const char *>(B + static_cast<int64_t>(k0) * ld);
   int b_next = 0;
   auto issue_b = [&](char *sb) {
-    const bool whole = b_next < nslabs - 1;
+    const bool last = b_next >= nslabs - 1, prev = b_next == nslabs - 2;
+    if (move_last && prev) b_src = reinterpret_cast<const char *>(B + static_cast<int64_t>(k0 + k_len - BKA) * ld);
     const int64_t b_left = b_end - b_src;
     const __amdgpu_buffer_rsrc_t b_rsrc =
         make_rsrc(b_src, Ragged && b_left < 0x80000000ll ? static_cast<uint32_t>(b_left) : kOutOfRange);
 #pragma unroll
     for (int i = 0; i < DB; ++i)
-      dma16(b_rsrc, (!Ragged || whole || b_lane_in_k[i]) ? b_off[i] : kOutOfRange, 0u, sb + (wave + NWAVES * i) * 1024);
+      dma16(b_rsrc, (!Ragged || (last ? b_in_last[i] : prev ? b_in_prev[i] : true)) ? b_off[i] : kOutOfRange, 0u,
+            sb + (wave + NWAVES * i) * 1024);
     ++b_next;
     if (b_next < nslabs) b_src += b_slab_bytes;
   };
@@ -1254,7 +1284,8 @@ float *splitk_workspace(hipStream_t st) {
 int splitk_for(int m, int n, int k) {
   const int64_t tiles = static_cast<int64_t>((m + 127) / 128) * ((n + 127) / 128);
   const int64_t forced = tunable("gemm16.split_k", 0);
-  if (forced == 1 || (static_cast<int64_t>(m) * n) % 4 != 0) return 1;   // the planes are added 16 bytes at a time
+  // the planes are added 16 bytes at a time; a last piece below one stage needs K % 8 == 0
+  if (forced == 1 || (static_cast<int64_t>(m) * n) % 4 != 0 || k % 8 != 0) return 1;
   static const int cus = [] {
     int dev = 0, v = 0;
     if (hipGetDevice(&dev) != hipSuccess ||
@@ -1295,17 +1326,19 @@ inline bool gemm16_default_kernel() {
 // property of the shape and is not looked at).
 int gemm16_tile_for(int m, int n, int k) {
   if (m < 1 || n < 1 || k < 1) return 0;
-  if (k % 8 != 0 || tunable("gemm16.force_simple", 0) != 0 || tunable("gemm16.force_staged", 0) != 0) return 0;
+  if (tunable("gemm16.force_simple", 0) != 0 || tunable("gemm16.force_staged", 0) != 0) return 0;
   // transfer offsets are 32-bit: 256 rows of A and 64 rows of B must span less than 2 GiB
   const bool offsets_ok = static_cast<int64_t>(k) * 256 * 2 < 0x7FFFFFFF && static_cast<int64_t>(n) * 64 * 2 < 0x7FFFFFFF;
   if (!offsets_ok) return 0;
   if (gemm16_default_kernel()) {
-    // any N, any K that is a multiple of 8.  gemm16.tile: 256 | 128 forces the tile, 0 (default) picks by the tile counts
+    // any N; any K from one LDS stage (64) on, below that the multiples of 8
+    if (k < 64 && k % 8 != 0) return 0;
+    // gemm16.tile: 256 | 128 forces the tile, 0 (default) picks by the tile counts
     const int tile = (int)tunable("gemm16.tile", 0);
     return (tile == 128 || (tile == 0 && small_tile_wins(m, n))) ? 128 : 256;
   }
   // the 32 x 32 x 16 kernel, its ring and wave shapes and the measurement variants: whole K = 64 stages, 16-byte rows of B
-  return (n % 8 == 0 && k % BK == 0) ? 256 : 0;
+  return (n % 8 == 0 && k % BK == 0) ? 256 : 0;   // (K % 8 == 0 alone: the staged kernel)
 }
 
 template <bool Bf16, int Epi>
@@ -1320,14 +1353,15 @@ int launch_gemm16(const uint16_t *a, const uint16_t *b, float *c, const float *b
     int rc = check_launch("rowsum clear launch");
     if (rc != SAREK_HIP_OK) return rc;
   }
-  // The default kernels (v_mfma_f32_16x16x32, 256 x 256 or 128 x 128 tile) take any N and any K that is a multiple of 8:
-  // rows of A then keep the 16-byte alignment of its base, rows of B need none.
-  if (reinterpret_cast<uintptr_t>(a) % 16 == 0 && reinterpret_cast<uintptr_t>(b) % 16 == 0 && gemm16_default_kernel()) {
+  // The default kernels (v_mfma_f32_16x16x32, 256 x 256 or 128 x 128 tile) take any N, any K of at least one LDS stage and
+  // any alignment of A and B in their Ragged form; below one stage K must be a multiple of 8 and A and B 16-byte aligned.
+  if (gemm16_default_kernel()) {
     const int tile_choice = gemm16_tile_for(m, n, k);
-    if (tile_choice != 0) {
+    const bool ab16 = reinterpret_cast<uintptr_t>(a) % 16 == 0 && reinterpret_cast<uintptr_t>(b) % 16 == 0;
+    if (tile_choice != 0 && (k >= 64 || ab16)) {
       // an odd N: the tiled kernel takes the first N - 1 columns of the N-strided matrices, a matrix-vector kernel the last
       const int nm = n - (n & 1);
-      const bool ragged = n % 8 != 0 || k % 64 != 0;   // the kernels' template flag: a K tail or B rows that are not 16-byte aligned
+      const bool ragged = n % 8 != 0 || k % 64 != 0 || !ab16;   // the kernels' template flag
       const int remap = (int)tunable("gemm.xcd_remap", 1);
       int rc = SAREK_HIP_OK;
       if (nm > 0 && tile_choice == 128) {

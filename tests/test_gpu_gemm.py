@@ -109,7 +109,7 @@ def test_gemm16_vs_oracle(hip, oracle, torch_cuda, kind, m, n, k):
 @pytest.mark.parametrize("kind", ["bf16", "f16"])
 def test_gemm16_unaligned_shapes_use_fallback(hip, oracle, torch_cuda, kind):
     torch = torch_cuda
-    m, n, k = 37, 51, 29   # k not a multiple of 8: rows of A are not 16-byte aligned
+    m, n, k = 37, 51, 29   # k below one LDS stage and not a multiple of 8
     assert hip.gemm16_tile(m, n, k) == 0
     a = normal16(oracle, (m, k), 1, kind)
     b = normal16(oracle, (k, n), 2, kind)
@@ -380,7 +380,7 @@ def test_gemm16_tile_choice_by_shape(hip, torch_cuda):
     for (m, n, k), want in [((1024, 1024, 64), 128), ((2048, 2048, 2048), 128), ((1024, 4096, 4096), 128),
                             ((4096, 2048, 8192), 128), ((3072, 3072, 3072), 256), ((4096, 4096, 4096), 256),
                             ((8192, 8192, 8192), 256), ((4095, 11008, 4096), 256), ((512, 512, 72), 128), ((4096, 4100, 4096), 256),
-                            ((1000, 1001, 1000), 128),
+                            ((1000, 1001, 1000), 128), ((1000, 1001, 1001), 128), ((512, 512, 29), 0),
                             ((37, 51, 29), 0)]:
         assert hip.gemm16_tile(m, n, k) == want, (m, n, k)
     hip.set_tunable("gemm16.mfma", 32)
@@ -492,26 +492,29 @@ def test_gemm16_split_k_under_graph_capture(hip, torch_cuda):
 
 
 RAGGED_SHAPES = [(1, 1, 8), (3, 5, 8), (37, 51, 24), (130, 137, 40), (256, 255, 64), (257, 1001, 1000),
-                 (300, 262, 136), (512, 514, 4104), (777, 1003, 328), (64, 4100, 96), (1000, 3, 2056)]
+                 (300, 262, 136), (512, 514, 4104), (777, 1003, 328), (64, 4100, 96), (1000, 3, 2056),
+                 (130, 137, 65), (257, 1001, 1001), (300, 263, 75), (64, 65, 67), (512, 514, 4107), (33, 40, 127),
+                 (33, 40, 129), (100, 64, 100)]
 
 
 @pytest.mark.parametrize("kind", ["bf16", "f16"])
 @pytest.mark.parametrize("m,n,k", RAGGED_SHAPES)
 def test_gemm16_ragged_shapes_stay_on_the_mfma_kernels(hip, oracle, torch_cuda, kind, m, n, k):
-    """Any N (odd ones included: rows of B and C then have no alignment at all) and any K that is a multiple of 8
-    (a K tail inside the last LDS stage) run on the direct-to-LDS kernels, both tiles, K split or not: against the
-    oracle; nothing is stored outside C; NaNs lying next to A and B in memory (what the transfers fetch past a row's
-    or the matrix's end) do not reach the result."""
+    """Any N (odd ones included: rows of B and C then have no alignment at all), any K from one LDS stage (64) on
+    and the multiples of 8 below it, operands that are only 2-byte aligned (where K reaches a stage): all run on the
+    direct-to-LDS kernels, both tiles, K split or not: against the oracle; nothing is stored outside C; NaNs lying
+    next to A and B in memory (what the transfers fetch past a row's or the matrix's end) do not reach the result."""
     torch = torch_cuda
     a = normal16(oracle, (m, k), m + 41, kind)
     b = normal16(oracle, (k, n), n + 42, kind)
     dt = torch.bfloat16 if kind == "bf16" else torch.float16
     fn = hip.gemm_bf16 if kind == "bf16" else hip.gemm_f16
     ref = oracle.gemm(a, b)
-    # operands as views into NaN-filled buffers, 16-byte aligned as the kernels require of A and B
+    # operands as views into NaN-filled buffers: 16-byte aligned below one stage of K, 2-byte aligned from there on
+    off = 129 if k >= 64 else 128
     buf_a = torch.full((m * k + 256,), float("nan"), device="cuda").to(dt)
     buf_b = torch.full((k * n + 256,), float("nan"), device="cuda").to(dt)
-    da, db = buf_a[128:128 + m * k].view(m, k), buf_b[128:128 + k * n].view(k, n)
+    da, db = buf_a[off:off + m * k].view(m, k), buf_b[off:off + k * n].view(k, n)
     da.copy_(dev(torch, a).to(dt))
     db.copy_(dev(torch, b).to(dt))
     try:
