@@ -534,7 +534,9 @@ int sarek_hip_gemm_f32(const float *a, const float *b, float *c, int m, int n, i
                        sarek_hip_stream stream);
 
 /* 16-bit-input, f32-accumulate GEMMs.  a, b hold bf16 / IEEE fp16 bit
- * patterns, row-major [m x k] and [k x n]; c is f32 row-major.             */
+ * patterns, row-major [m x k] and [k x n]; c is f32 row-major.  Any m, n,
+ * k >= 1 and any alignment of the three (sarek_hip_gemm16_tile below says
+ * which kernel serves a shape).                                             */
 int sarek_hip_gemm_bf16(const uint16_t *a, const uint16_t *b, float *c, int m, int n, int k,
                         sarek_hip_stream stream);
 int sarek_hip_gemm_f16(const uint16_t *a, const uint16_t *b, float *c, int m, int n, int k,
