@@ -582,3 +582,28 @@ def test_gemm_f32_ragged_shapes_stay_on_the_mfma_kernel(hip, oracle, torch_cuda,
             assert np.abs(got - ref).max() <= f32_tol(a, b, k)
     finally:
         hip.set_tunable("gemm_f32.tile", 0)
+
+
+@pytest.mark.parametrize("knob", ["force_staged", "force_simple"])
+@pytest.mark.parametrize("m,n,k", [(264, 520, 72), (100, 64, 200), (8, 8, 8), (300, 264, 192)])
+def test_fallback_kernels_stay_correct(hip, oracle, torch_cuda, knob, m, n, k):
+    """The register-staged and the one-thread-per-element kernels (16-bit and f32) are what is left when a transfer
+    offset would not fit 32 bits or, for the 32 x 32 x 16 variants, when K is not whole stages; the direct-to-LDS
+    kernels now take the shapes that used to reach them, so they are switched on by their knobs here."""
+    torch = torch_cuda
+    a16 = normal16(oracle, (m, k), m + 71, "bf16")
+    b16 = normal16(oracle, (k, n), n + 72, "bf16")
+    a32 = oracle.fill_uniform(m * k, seed=m + 73, lo=-1, hi=1).reshape(m, k)
+    b32 = oracle.fill_uniform(k * n, seed=n + 74, lo=-1, hi=1).reshape(k, n)
+    hip.set_tunable("gemm16." + knob, 1)
+    hip.set_tunable("gemm_f32." + knob, 1)
+    try:
+        assert hip.gemm16_tile(m, n, k) == 0
+        c16 = hip.gemm_bf16(dev(torch, a16).bfloat16(), dev(torch, b16).bfloat16()).cpu().numpy()
+        c32 = hip.gemm_f32(dev(torch, a32), dev(torch, b32)).cpu().numpy()
+    finally:
+        hip.set_tunable("gemm16." + knob, 0)
+        hip.set_tunable("gemm_f32." + knob, 0)
+    ref16 = oracle.gemm(a16, b16)
+    assert np.abs(c16 - ref16).max() / np.abs(ref16).max() < 1e-4
+    assert np.abs(c32 - oracle.gemm(a32, b32)).max() <= f32_tol(a32, b32, k)
