@@ -466,6 +466,8 @@ def measure(name, torch, hip, steps, warmup):
         res["roofline"]["mfma_stream_only_TFLOPs"] = stream
         res["roofline"]["frac_of_mfma_stream_only"] = round(achieved / stream, 4)
         res["roofline"]["mfma_stream_only_32x32x16_TFLOPs"] = stream32
+        # the vendor library on the same inputs, same protocol (torch.matmul -> hipBLASLt; it writes bf16 C)
+        res["roofline"]["vendor_library_TFLOPs"] = vendor_gemm_rate(torch, hip)
     if info["bound"] == "mfma" and info["route"].startswith("Execute"):
         # shader clock the kernel actually ran at (in-kernel cycle counter against the
         # constant-rate wall clock), and the rate of those very launches against the peak
@@ -623,6 +625,30 @@ def mfma_stream_rates(torch, hip, launches=15):
         times = sorted(launch() for _ in range(launches))
         rates.append(round(flop / (times[len(times) // 2] * 1e-3) / 1e12, 1))
     return tuple(rates)
+
+
+def vendor_gemm_rate(torch, hip, launches=20):
+    """TFLOP/s of torch.matmul (hipBLASLt) on the headline's 8192^3 bf16 inputs: WARMUP_MS of launches each waited
+    for, then the average of `launches` waited launches by HIP events on the launch stream, as for the kernel."""
+    s = 8192
+    g = torch.Generator(device="cuda")
+    g.manual_seed(0xA4)
+    a = (torch.randn(s, s, device="cuda", generator=g) * 0.02).bfloat16()
+    g.manual_seed(0xB4)
+    b = (torch.randn(s, s, device="cuda", generator=g) * 0.02).bfloat16()
+    c = torch.empty(s, s, device="cuda", dtype=torch.bfloat16)
+    ev = Events(hip, C.c_void_p(torch.cuda.current_stream().cuda_stream))
+
+    def launch():
+        ev.start()
+        torch.matmul(a, b, out=c)
+        return ev.stop_ms()
+    launch()
+    t_warm = time.perf_counter()
+    while (time.perf_counter() - t_warm) * 1e3 < WARMUP_MS:
+        launch()
+    ms = sum(launch() for _ in range(launches)) / launches
+    return round(2.0 * s ** 3 / (ms * 1e-3) / 1e12, 1)
 
 
 def event_overhead_ms(torch, hip, launches=20):
