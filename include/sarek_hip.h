@@ -532,6 +532,10 @@ int sarek_hip_radix_scatter_i32(int32_t *out, int64_t out_len, int32_t *counters
  * benchmarks/bench_matrix_mul_tiled.ml:55-95).  Any m,n,k >= 1.            */
 int sarek_hip_gemm_f32(const float *a, const float *b, float *c, int m, int n, int k,
                        sarek_hip_stream stream);
+/* Into how many pieces sarek_hip_gemm_f32 cuts K for this shape now (1 = none):
+ * as for the 16-bit products (sarek_hip_gemm16_k_splits below), same per-stream
+ * memory and fixed-order sum; tunable gemm_f32.split_k.                      */
+int sarek_hip_gemm_f32_k_splits(int m, int n, int k);
 
 /* 16-bit-input, f32-accumulate GEMMs.  a, b hold bf16 / IEEE fp16 bit
  * patterns, row-major [m x k] and [k x n]; c is f32 row-major.  Any m, n,

@@ -190,6 +190,7 @@ let gemm_f16 =
   bind "sarek_hip_gemm_f16"
     (ptr uint16_t @-> ptr uint16_t @-> ptr float @-> int @-> int @-> int @-> ptr void
    @-> returning int)
+let gemm_f32_k_splits = bind "sarek_hip_gemm_f32_k_splits" (int @-> int @-> int @-> returning int)
 let gemm16_tile = bind "sarek_hip_gemm16_tile" (int @-> int @-> int @-> returning int)
 let gemm16_k_splits = bind "sarek_hip_gemm16_k_splits" (int @-> int @-> int @-> returning int)
 let gemm_f16_bias_relu_rowsum =

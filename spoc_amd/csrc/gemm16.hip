@@ -1235,46 +1235,6 @@ __global__ __launch_bounds__(256) void gemm16_last_column_kernel(const uint16_t 
   }
 }
 
-// Adds the `splits` partial M x N planes of a K-split product into C, plane 0 first: a fixed order, so the result does
-// not depend on which workgroup finished when.
-__global__ __launch_bounds__(256) void splitk_reduce_kernel(const float *__restrict__ partials, float *__restrict__ C,
-                                                            int64_t mn, int splits) {
-  const int64_t i = (static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x) * 4;
-  if (i >= mn) return;   // mn is a multiple of 8 (n % 8 == 0)
-  f32x4_t acc = *reinterpret_cast<const f32x4_t *>(partials + i);
-  for (int s = 1; s < splits; ++s) acc += *reinterpret_cast<const f32x4_t *>(partials + s * mn + i);
-  *reinterpret_cast<f32x4_t *>(C + i) = acc;
-}
-
-// Device memory for the partial planes: one block of kSplitWorkspaceBytes per (device, stream), allocated at the first
-// split product on that stream and kept until the process ends (never grown or freed, so a pointer handed out stays
-// good whatever other threads do): calls on different streams never share one, calls on one stream are ordered by it.
-// nullptr (the caller then does not split) for a stream under capture that has none yet, past 16 streams, or when the
-// allocation fails.
-constexpr size_t kSplitWorkspaceBytes = 64u << 20;
-float *splitk_workspace(hipStream_t st) {
-  static std::mutex mu;
-  static std::map<std::pair<int, hipStream_t>, void *> blocks;
-  int dev = 0;
-  if (hipGetDevice(&dev) != hipSuccess) return nullptr;
-  std::lock_guard<std::mutex> lock(mu);
-  auto it = blocks.find({dev, st});
-  if (it != blocks.end()) return static_cast<float *>(it->second);
-  if (blocks.size() >= 16) return nullptr;
-  hipStreamCaptureStatus capturing = hipStreamCaptureStatusNone;
-  if (hipStreamIsCapturing(st, &capturing) != hipSuccess || capturing != hipStreamCaptureStatusNone) {
-    (void)hipGetLastError();
-    return nullptr;
-  }
-  void *p = nullptr;
-  if (hipMalloc(&p, kSplitWorkspaceBytes) != hipSuccess) {
-    (void)hipGetLastError();
-    return nullptr;
-  }
-  blocks[{dev, st}] = p;
-  return static_cast<float *>(p);
-}
-
 // K splits of the 128 x 128 kernel for a plain product with few tiles and a long K; 1 = no split.  A tile's K loop is
 // bound by the latency of its transfers (0.19 us per K = 32 slab with one or two workgroups on a CU, measured), so
 // cutting K over idle CUs shortens it; against that stand the second launch (5 us) and the partial planes, which cost
@@ -1385,9 +1345,7 @@ int launch_gemm16(const uint16_t *a, const uint16_t *b, float *c, const float *b
                                bias, rowsum, m, nm, k, sm, sn, remap, nullptr, chunk, partials, n);
           rc = check_launch("gemm16 kernel launch");
           if (rc != SAREK_HIP_OK) return rc;
-          hipLaunchKernelGGL(splitk_reduce_kernel, dim3(static_cast<unsigned>((mn / 4 + 255) / 256)), dim3(256), 0, st,
-                             partials, c, mn, splits);
-          rc = check_launch("gemm16 split-K reduction launch");
+          rc = launch_splitk_reduce(partials, c, mn, splits, st);
         } else {
           if (ragged)
             hipLaunchKernelGGL((gemm16_m16_small_kernel<Bf16, Epi, true>), dim3(sm * sn), dim3(256), 0, st, a, b, c, bias,

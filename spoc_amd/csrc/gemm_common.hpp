@@ -4,6 +4,13 @@
 #include <hip/hip_runtime.h>
 
 namespace sarek_hip {
+
+// K-split products (gemm_splitk.hip): the per-stream block of device memory for the partial planes and the kernel that
+// adds them into C in a fixed order.
+constexpr size_t kSplitWorkspaceBytes = 64u << 20;
+float *splitk_workspace(hipStream_t st);
+int launch_splitk_reduce(const float *partials, float *c, int64_t mn, int splits, hipStream_t st);
+
 namespace {
 
 #define LDS_PTR __attribute__((address_space(3)))

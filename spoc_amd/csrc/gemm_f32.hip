@@ -18,6 +18,8 @@
 #include <type_traits>
 #include <utility>
 
+#include <algorithm>
+
 #include "common.hpp"
 #include "gemm_common.hpp"
 #include "tunables.hpp"
@@ -173,7 +175,8 @@ __global__ __launch_bounds__(THREADS) void gemm_f32_staged_kernel(const float *_
 template <int TI, int TJ, int WMW, int WNW, int BKT, int NS, bool Ragged = false>
 __global__ __launch_bounds__(64 * WMW * WNW) void gemm_f32_dma_kernel(
     const float *__restrict__ A, const float *__restrict__ B, float *__restrict__ C, int M, int N,
-    int K, int tiles_m, int tiles_n, int xcd_remap, unsigned long long *probe) {
+    int K, int tiles_m, int tiles_n, int xcd_remap, unsigned long long *probe, int k_chunk,
+    float *__restrict__ partials) {
   typedef __attribute__((ext_vector_type(TJ))) float bvec_t;
   constexpr int BMT = 32 * TI * WMW, BNT = 32 * TJ * WNW, NWAVES = WMW * WNW;
   constexpr int KK = BKT / 8;
@@ -222,17 +225,22 @@ __global__ __launch_bounds__(64 * WMW * WNW) void gemm_f32_dma_kernel(
     const int col = Ragged ? n0 + chunk * 4 : min(n0 + chunk * 4, N - 4);
     b_off[i] = (static_cast<uint32_t>(brow) * N + col) * 4u;
   }
-  const char *a_base = reinterpret_cast<const char *>(A + static_cast<int64_t>(m0) * K);
-  const char *b_base = reinterpret_cast<const char *>(B);
+  // K cut over gridDim.y workgroups per tile: this one takes k0 .. k0 + k_len - 1 and writes its partial tile to its
+  // own M x N plane of `partials`, which a second kernel adds up in a fixed order
+  const int k0 = blockIdx.y * k_chunk;
+  const int k_len = min(k_chunk, K - k0);
+  if (gridDim.y > 1) C = partials + static_cast<int64_t>(blockIdx.y) * M * N;
+  const char *a_base = reinterpret_cast<const char *>(A + static_cast<int64_t>(m0) * K + k0);
+  const char *b_base = reinterpret_cast<const char *>(B + static_cast<int64_t>(k0) * N);
   const int64_t b_slab_bytes = static_cast<int64_t>(BKT) * N * 4;
-  const int nslabs = (K + BKT - 1) / BKT;
+  const int nslabs = (k_len + BKT - 1) / BKT;
   // The end of K inside the last slab.  With K >= BKT the last slab is moved back to end at K (its A pieces then hold
   // nothing but elements of their own row, at whatever alignment) and the B rows it shares with the slab before it
   // are the ones left out; with a single slab (K < BKT, K % 4 == 0) the A pieces and B rows past K are.  A lane's k
   // piece is the same for all its A transfers: rows NWAVES * A_ROWS_PER_DMA apart share the swizzle.
-  const int k_tail = K - (nslabs - 1) * BKT;
-  const bool move_last = Ragged && K >= BKT && k_tail != BKT;
-  const int k_last = move_last ? K - BKT : (nslabs - 1) * BKT;   // first k of the last slab
+  const int k_tail = k_len - (nslabs - 1) * BKT;
+  const bool move_last = Ragged && k_len >= BKT && k_tail != BKT;
+  const int k_last = move_last ? k_len - BKT : (nslabs - 1) * BKT;   // first k of the last slab, from k0
   const bool a_lane_in_k =
       !Ragged || move_last || (((lane % A_CHUNKS) ^ a_swz(wave * A_ROWS_PER_DMA + lane / A_CHUNKS)) << 2) < k_tail;
   bool b_lane_in_k[B_DMA];
@@ -241,7 +249,7 @@ __global__ __launch_bounds__(64 * WMW * WNW) void gemm_f32_dma_kernel(
     const int brow = (wave + NWAVES * i) * B_ROWS_PER_DMA + lane / B_CHUNKS;
     b_lane_in_k[i] = !Ragged || (move_last ? brow >= BKT - k_tail : brow < k_tail);
   }
-  const char *b_end = b_base + static_cast<int64_t>(K) * N * 4;
+  const char *b_end = reinterpret_cast<const char *>(B) + static_cast<int64_t>(K) * N * 4;
   constexpr uint32_t kOutOfRange = 0x80000000u;
 
   f32x16 acc[TI][TJ];
@@ -428,6 +436,75 @@ __global__ __launch_bounds__(256) void gemm_f32_simple_kernel(const float *__res
 
 using namespace sarek_hip;
 
+namespace {
+// Tile choice by a cost model of the launch: a CU holds `occ` workgroups of a tile shape at once (LDS ring), tiles run
+// in rounds of cus*occ, a workgroup that shares its CU takes occ times as long, and the tail round runs unshared when it
+// fits one workgroup per CU.  `eff` is the MFMA issue efficiency measured for each shape.
+int gemm_f32_tile_for(int m, int n) {
+  auto ntiles = [&](int t) { return static_cast<int64_t>((m + t - 1) / t) * ((n + t - 1) / t); };
+  static const int cus = [] {
+    int dev = 0, v = 0;
+    if (hipGetDevice(&dev) != hipSuccess ||
+        hipDeviceGetAttribute(&v, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || v <= 0)
+      v = 256;
+    return v;
+  }();
+  auto cost = [&](int t, int occ, double eff) {
+    const int64_t tiles = ntiles(t), slots = static_cast<int64_t>(cus) * occ;
+    const int64_t full = tiles / slots, rest = tiles % slots;
+    const double rounds = static_cast<double>(full) * occ + (rest == 0 ? 0 : rest <= cus ? 1 : occ);
+    return rounds * t * t / eff;
+  };
+  const double c256 = cost(256, 1, 1.0), c128 = cost(128, 2, 0.95), c64 = cost(64, 2, 0.80);
+  return (c256 <= c128 && c256 <= c64) ? 256 : (c128 <= c64 ? 128 : 64);
+}
+
+// K pieces for a product on the 64 x 64 tile; 1 = whole.  One such tile per CU runs at the rate of its MFMAs (0.45 us per
+// K = 32 slab, measured; two on a CU share the pipes), so pieces help while CUs are idle; against that stand the second
+// launch (5 us) and the partial planes (0.65 us per MiB).  The count in {2, 4, 8, 16} with the lowest estimate is taken
+// if it is a tenth below the whole product's.  gemm_f32.split_k: 0 = this rule, 1 = never, n >= 2 forces n.
+int splitk_f32_for(int m, int n, int k) {
+  const int64_t forced = tunable("gemm_f32.split_k", 0);
+  if (forced == 1 || (static_cast<int64_t>(m) * n) % 4 != 0 || k % 32 != 0) return 1;
+  static const int cus = [] {
+    int dev = 0, v = 0;
+    if (hipGetDevice(&dev) != hipSuccess ||
+        hipDeviceGetAttribute(&v, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || v <= 0)
+      v = 256;
+    return v;
+  }();
+  const int64_t tiles = static_cast<int64_t>((m + 63) / 64) * ((n + 63) / 64);
+  const double plane_mib = static_cast<double>(m) * n * 4 / (1 << 20);
+  const int64_t fit = static_cast<int64_t>(static_cast<double>(kSplitWorkspaceBytes >> 20) / plane_mib);
+  int64_t splits = 1;
+  if (forced >= 2) {
+    splits = std::min<int64_t>({forced, static_cast<int64_t>(k / 32), fit});
+  } else {
+    auto estimate = [&](int64_t s) {
+      const double rounds = static_cast<double>((tiles * s + cus - 1) / cus);
+      return 8.0 + static_cast<double>(k) / 32 / s * 0.45 * rounds + (s > 1 ? 5.0 + s * plane_mib * 0.65 : 0.0);
+    };
+    double best = estimate(1) * 0.9;
+    for (int64_t s = 2; s <= 16; s *= 2) {
+      if (k / s < 256 || s > fit) break;
+      if (estimate(s) < best) best = estimate(s), splits = s;
+    }
+  }
+  if (splits < 2) return 1;
+  const int chunk = static_cast<int>(((k / 32 + splits - 1) / splits) * 32);
+  return (k + chunk - 1) / chunk;
+}
+}  // namespace
+
+extern "C" int sarek_hip_gemm_f32_k_splits(int m, int n, int k) {
+  if (m < 1 || n < 1 || k < 1) return 1;
+  // the split belongs to the 64 x 64 tile, which the launcher takes where its cost model says so
+  const int64_t forced_tile = tunable("gemm_f32.tile", 0);
+  if (forced_tile != 0 && forced_tile != 64) return 1;
+  if (forced_tile == 0 && gemm_f32_tile_for(m, n) != 64) return 1;
+  return splitk_f32_for(m, n, k);
+}
+
 extern "C" int sarek_hip_gemm_f32(const float *a, const float *b, float *c, int m, int n, int k,
                                   sarek_hip_stream stream) {
   if (m <= 0 || n <= 0 || k <= 0)
@@ -445,33 +522,23 @@ extern "C" int sarek_hip_gemm_f32(const float *a, const float *b, float *c, int 
                           static_cast<int64_t>(n) * 32 * 4 < 0x7FFFFFFF;
   if (ab_ok && offsets_ok && tunable("gemm_f32.force_simple", 0) == 0 && tunable("gemm_f32.force_staged", 0) == 0) {
     const bool ragged = !aligned || n % 4 != 0 || k % 32 != 0 || reinterpret_cast<uintptr_t>(c) % 16 != 0;
-    // Tile choice by a cost model of the launch: a CU holds `occ` workgroups of a tile
-    // shape at once (LDS ring), tiles run in rounds of cus*occ, a workgroup that shares
-    // its CU takes occ times as long, and the tail round runs unshared when it fits one
-    // workgroup per CU.  `eff` is the MFMA issue efficiency measured for each shape.
     auto ntiles = [&](int t) { return static_cast<int64_t>((m + t - 1) / t) * ((n + t - 1) / t); };
-    static const int cus = [] {
-      int dev = 0, v = 0;
-      if (hipGetDevice(&dev) != hipSuccess ||
-          hipDeviceGetAttribute(&v, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || v <= 0)
-        v = 256;
-      return v;
-    }();
-    auto cost = [&](int t, int occ, double eff) {
-      const int64_t tiles = ntiles(t), slots = static_cast<int64_t>(cus) * occ;
-      const int64_t full = tiles / slots, rest = tiles % slots;
-      const double rounds = static_cast<double>(full) * occ + (rest == 0 ? 0 : rest <= cus ? 1 : occ);
-      return rounds * t * t / eff;
-    };
     int tile = (int)tunable("gemm_f32.tile", 0);
-    if (tile == 0) {
-      const double c256 = cost(256, 1, 1.0), c128 = cost(128, 2, 0.95), c64 = cost(64, 2, 0.80);
-      tile = (c256 <= c128 && c256 <= c64) ? 256 : (c128 <= c64 ? 128 : 64);
+    if (tile == 0) tile = gemm_f32_tile_for(m, n);
+    // K cut over idle CUs for the 64 x 64 tile (few tiles, long K): whole slabs per piece, planes added 16 bytes at a time
+    int splits = 1;
+    float *partials = nullptr;
+    if (tile == 64 && k % 32 == 0 && reinterpret_cast<uintptr_t>(c) % 16 == 0) {
+      splits = splitk_f32_for(m, n, k);
+      if (splits > 1) partials = splitk_workspace(st);
+      if (!partials) splits = 1;
     }
+    const int k_chunk = splits > 1 ? ((k / 32 + splits - 1) / splits) * 32 : k;
 #define SAREK_LAUNCH_F32(T, TI, TJ, WMW, WNW, BKT, RAGGED)                                         \
   hipLaunchKernelGGL((gemm_f32_dma_kernel<TI, TJ, WMW, WNW, BKT, 4, RAGGED>),                     \
-                     dim3((unsigned)ntiles(T)), dim3(64 * WMW * WNW), 0, st, a, b, c, m, n, k,    \
-                     (m + T - 1) / T, (n + T - 1) / T, remap, clock_probe(ntiles(T)))
+                     dim3((unsigned)ntiles(T), splits), dim3(64 * WMW * WNW), 0, st, a, b, c, m, n, k, \
+                     (m + T - 1) / T, (n + T - 1) / T, remap, splits > 1 ? nullptr : clock_probe(ntiles(T)), k_chunk, \
+                     partials)
     if (ragged) {
       if (tile == 256) SAREK_LAUNCH_F32(256, 4, 2, 2, 4, 16, true);
       else if (tile == 128) SAREK_LAUNCH_F32(128, 2, 2, 2, 2, 16, true);
@@ -482,7 +549,9 @@ extern "C" int sarek_hip_gemm_f32(const float *a, const float *b, float *c, int 
       else SAREK_LAUNCH_F32(64, 1, 1, 2, 2, 32, false);
     }
 #undef SAREK_LAUNCH_F32
-    return check_launch("gemm_f32 kernel launch");
+    const int rc = check_launch("gemm_f32 kernel launch");
+    if (rc != SAREK_HIP_OK || splits == 1) return rc;
+    return launch_splitk_reduce(partials, c, static_cast<int64_t>(m) * n, splits, st);
   }
   if (aligned && n % 4 == 0 && tunable("gemm_f32.force_simple", 0) == 0) {
     static bool attr_done = false;

@@ -138,6 +138,7 @@ SYMBOLS = {
     "sarek_hip_gemm_f32": (_i, [_vp, _vp, _vp, _i, _i, _i, _vp]),
     "sarek_hip_gemm_bf16": (_i, [_vp, _vp, _vp, _i, _i, _i, _vp]),
     "sarek_hip_gemm_f16": (_i, [_vp, _vp, _vp, _i, _i, _i, _vp]),
+    "sarek_hip_gemm_f32_k_splits": (_i, [_i, _i, _i]),
     "sarek_hip_gemm16_tile": (_i, [_i, _i, _i]),
     "sarek_hip_gemm16_k_splits": (_i, [_i, _i, _i]),
     "sarek_hip_gemm_f16_bias_relu_rowsum": (_i, [_vp, _vp, _vp, _vp, _vp, _i, _i, _i, _vp]),
@@ -564,6 +565,11 @@ def gemm_f32(a, b, out=None):
     c = torch.empty((m, n), dtype=torch.float32, device=a.device) if out is None else out
     check(lib.sarek_hip_gemm_f32(_ptr(a), _ptr(b), _ptr(c), m, n, k, _stream()))
     return c
+
+
+def gemm_f32_k_splits(m, n, k):
+    """Into how many pieces the f32 GEMM cuts K for this shape now (1 = none)."""
+    return int(lib.sarek_hip_gemm_f32_k_splits(m, n, k))
 
 
 def _gemm16(fn, dtype, a, b, out):

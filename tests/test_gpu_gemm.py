@@ -607,3 +607,45 @@ def test_fallback_kernels_stay_correct(hip, oracle, torch_cuda, knob, m, n, k):
     ref16 = oracle.gemm(a16, b16)
     assert np.abs(c16 - ref16).max() / np.abs(ref16).max() < 1e-4
     assert np.abs(c32 - oracle.gemm(a32, b32)).max() <= f32_tol(a32, b32, k)
+
+
+@pytest.mark.parametrize("m,n,k,splits", [(256, 256, 8192, 0), (128, 128, 4096, 0), (130, 136, 1024, 2), (300, 520, 448, 3),
+                                          (1, 8, 4096, 16), (512, 384, 2048, 5), (64, 1001, 2048, 4)])
+def test_gemm_f32_split_k(hip, oracle, torch_cuda, m, n, k, splits):
+    """The f32 product cut along K on the 64 x 64 tile (few tiles, long K): against the oracle, the same bits on every
+    run and on another stream, and the count the library reports.  splits = 0 leaves the choice to the launcher
+    (these two shapes split), n forces n pieces."""
+    torch = torch_cuda
+    a = oracle.fill_uniform(m * k, seed=m + 81, lo=-1, hi=1).reshape(m, k)
+    b = oracle.fill_uniform(k * n, seed=n + 82, lo=-1, hi=1).reshape(k, n)
+    da, db = dev(torch, a), dev(torch, b)
+    ref = oracle.gemm(a, b)
+    hip.set_tunable("gemm_f32.split_k", splits)
+    if splits:
+        hip.set_tunable("gemm_f32.tile", 64)
+    try:
+        reported = hip.gemm_f32_k_splits(m, n, k)
+        assert reported >= 2 and (splits == 0 or reported <= splits)
+        c1 = hip.gemm_f32(da, db)
+        c2 = hip.gemm_f32(da, db)
+        side = side_stream(torch)
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):
+            c3 = hip.gemm_f32(da, db)
+        side.synchronize()
+        hip.set_tunable("gemm_f32.split_k", 1)
+        assert hip.gemm_f32_k_splits(m, n, k) == 1
+        whole = hip.gemm_f32(da, db)
+    finally:
+        hip.set_tunable("gemm_f32.split_k", 0)
+        hip.set_tunable("gemm_f32.tile", 0)
+    assert torch.equal(c1, c2) and torch.equal(c1, c3)
+    for c in (c1, whole):
+        assert np.abs(c.cpu().numpy() - ref).max() <= f32_tol(a, b, k)
+
+
+def test_gemm_f32_split_k_rule(hip, torch_cuda):
+    for (m, n, k), want_split in [((256, 256, 8192), True), ((512, 512, 8192), True), ((128, 4096, 4096), True),
+                                  ((1024, 1024, 1024), False), ((2048, 2048, 2048), False), ((8192, 8192, 8192), False),
+                                  ((1024, 1024, 8192), False), ((512, 512, 100), False)]:
+        assert (hip.gemm_f32_k_splits(m, n, k) > 1) == want_split, (m, n, k)
