@@ -58,7 +58,7 @@ def parse():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--workload", default="gemm_bf16_8192",
                     choices=["gemm_bf16_8192", "gemm_f16_8192", "triad_sum_2p28", "gemm_f32_8192", "gemm_f32_1024",
-                             "gemm_f16_epilogue", "gemm_f16_4095x11008x4096", "gemm_f16_shape", "gemm_bf16_shape", "gemm_bf16_2048", "copy_1gib",
+                             "gemm_f16_epilogue", "gemm_f16_4095x11008x4096", "gemm_f16_shape", "gemm_bf16_shape", "gemm_bf16_2048", "gemm_f32_shape", "vendor_gemm_f32_shape", "copy_1gib",
                              "vendor_gemm_bf16_8192", "vendor_gemm_bf16_shape", "histogram_2p28",
                              "radix_scatter_5e7", "mfma_bf16_stream", "mfma_bf16_stream_32x32x16", "l2_to_lds_stream"])
     ap.add_argument("--warmup-ms", type=float, default=60.0,
@@ -260,6 +260,29 @@ def make_workload(name, torch, hip):
                     config={"workload": f"{wgs} workgroups x 8 MiB by buffer_load_dwordx4 ... lds from a {window >> 20} MiB window "
                                         "(the operand bytes of the 8192^3 16-bit GEMM with 256 x 256 tiles: 8.59 GB)"})
         return (lambda: hip.run_source(L2_STREAM_SRC, "l2_to_lds", (512, 1, 1), (wgs, 1, 1), items)), None, info, (src, sink)
+    if name in ("gemm_f32_shape", "vendor_gemm_f32_shape"):
+        # any --shape of the f32 GEMM through its C-ABI entry point (the IR route fixes 16 x 16 blocks that cover C), and
+        # torch.matmul (no TF32) on the same inputs
+        m, n, k = GEMM_SHAPE
+        g.manual_seed(0xA11CE)
+        a = torch.rand(m, k, device="cuda", generator=g) * 2 - 1
+        g.manual_seed(0xB0B)
+        b = torch.rand(k, n, device="cuda", generator=g) * 2 - 1
+        c = torch.empty(m, n, device="cuda")
+        vendor = name.startswith("vendor")
+        info = dict(metric=("vendor library " if vendor else "") + f"f32 GEMM TFLOP/s at {m}x{n}x{k}", unit="TFLOP/s",
+                    dtype="f32", work=2.0 * m * n * k, work_unit=1e12, bound="mfma", peak=PEAK_MFMA_TFLOPS["f32"],
+                    kernel="hipBLASLt / rocBLAS (torch.matmul)" if vendor else "gemm_f32_dma_kernel",
+                    route="torch.matmul" if vendor else "sarek_hip_gemm_f32 (C ABI)",
+                    config={"workload": "f32 C=A.B row-major, U[-1,1)", "m": m, "n": n, "k": k,
+                            "k_splits": 1 if vendor else hip.gemm_f32_k_splits(m, n, k)})
+        if vendor:
+            torch.backends.cuda.matmul.allow_tf32 = False
+            return (lambda: torch.matmul(a, b, out=c)), None, info, None
+        stream = C.c_void_p(torch.cuda.current_stream().cuda_stream)
+        main = Launch(hip, lib.sarek_hip_gemm_f32, C.c_void_p(a.data_ptr()), C.c_void_p(b.data_ptr()),
+                      C.c_void_p(c.data_ptr()), m, n, k, stream)
+        return main, None, info, (a, b, c)
     if name in ("vendor_gemm_bf16_8192", "vendor_gemm_bf16_shape"):
         # the vendor library's GEMM (torch.matmul -> hipBLASLt) on the headline inputs or on --shape, for
         # side-by-side profiles; it writes bf16 C where the kernel here writes f32
@@ -780,7 +803,7 @@ def main():
     }
     if args.trace_launches:
         out["kernel_us_by_launch"] = head["kernel_us_by_launch"]
-    if not args.no_cpu_baseline and args.workload not in ("copy_1gib", "vendor_gemm_bf16_8192", "vendor_gemm_bf16_shape", "gemm_bf16_shape", "gemm_f16_shape", "mfma_bf16_stream", "mfma_bf16_stream_32x32x16", "l2_to_lds_stream"):
+    if not args.no_cpu_baseline and args.workload not in ("copy_1gib", "vendor_gemm_bf16_8192", "vendor_gemm_bf16_shape", "gemm_bf16_shape", "gemm_f16_shape", "gemm_f32_shape", "vendor_gemm_f32_shape", "mfma_bf16_stream", "mfma_bf16_stream_32x32x16", "l2_to_lds_stream"):
         out["cpu_baseline"] = cpu_baseline(args.workload)
     if not args.no_also:
         also = []
