@@ -460,6 +460,12 @@ int sarek_hip_triad_sum_f32(float *a, const float *b, const float *c, float s, i
  * sarek_hip_execute_run_pipeline launches for that pair of kernels).  Vectors 16-byte aligned. */
 int sarek_hip_triad_block256_sum_f32(float *a, const float *b, const float *c, float s, int64_t n,
                                      float *block_sums, sarek_hip_stream stream);
+/* The same with the block-256 maximum in place of the sum: block_max[j] = what the reference's halving tree
+ * leaves for a[256j .. 256j+255], elements past n counting as `pad` (benchmarks/bench_reduction_max.ml:18-100),
+ * with the bits sarek_hip_reduce_max_block256_f32 would produce from that a.  With s = 1 the triad is the vector
+ * add of benchmarks/bench_vector_add.ml, so the four pairs {triad, add} x {sum, max} of a pipeline are one pass. */
+int sarek_hip_triad_block256_max_f32(float *a, const float *b, const float *c, float s, int64_t n, float pad,
+                                     float *block_max, sarek_hip_stream stream);
 
 /* The same operation for callers that cannot allocate device memory or carry a workspace (code
  * under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc); it has no

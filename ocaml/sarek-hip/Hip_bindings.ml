@@ -216,6 +216,10 @@ let triad_block256_sum =
   bind "sarek_hip_triad_block256_sum_f32"
     (ptr float @-> ptr float @-> ptr float @-> float @-> int64_t @-> ptr float @-> ptr void
    @-> returning int)
+let triad_block256_max =
+  bind "sarek_hip_triad_block256_max_f32"
+    (ptr float @-> ptr float @-> ptr float @-> float @-> int64_t @-> float @-> ptr float @-> ptr void
+   @-> returning int)
 (* the same sum for callers that may not allocate: n <= triad_sum_static_max_n, the partial
    sums live inside the library's device image *)
 let triad_sum_static_max_n =

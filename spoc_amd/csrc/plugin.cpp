@@ -358,26 +358,55 @@ int try_specialised(const std::string &tag, const int block[3], const int grid[3
 int try_specialised_pair(const std::string &tag0, const int block0[3], const int grid0[3],
                          const sarek_hip_arg *a0, int n0, const std::string &tag1, const int block1[3],
                          const int grid1[3], const sarek_hip_arg *a1, int n1, int *rc) {
-  if (tag0 != "stream_triad_f32" || tag1 != "reduce_sum_block256_f32") return 0;
-  if (n0 != 8 || !vec_at(a0, n0, 0) || !vec_at(a0, n0, 2) || !vec_at(a0, n0, 4) || !is_f32(a0[6]) || !is_i32(a0[7]))
+  // the reduction: the block-256 sum (input, len, output, len, n) or the block-256 maximum, same arguments, whose
+  // fill value travels in the tag as f32 bits
+  const bool is_sum = tag1 == "reduce_sum_block256_f32";
+  const bool is_max = tag1.compare(0, 24, "reduce_max_block256_f32:") == 0 && tag1.size() == 32;
+  if (!is_sum && !is_max) return 0;
+  float pad = 0.f;
+  if (is_max) {
+    char *end = nullptr;
+    const unsigned long bits = std::strtoul(tag1.c_str() + 24, &end, 16);
+    if (*end != 0) return 0;
+    const uint32_t b32 = static_cast<uint32_t>(bits);
+    std::memcpy(&pad, &b32, 4);
+  }
+  // the element-wise producer: the stream triad (a, len, b, len, c, len, scalar, n), a = b + scalar * c, or the vector
+  // add (a, len, b, len, c, len, n), c = a + b, which is the triad with scalar 1 (one rounding of the exact sum)
+  int out, in0, in1;
+  float scalar;
+  int64_t n;
+  if (tag0 == "stream_triad_f32") {
+    if (n0 != 8 || !is_f32(a0[6]) || !is_i32(a0[7])) return 0;
+    out = 0, in0 = 2, in1 = 4, scalar = a0[6].f32, n = a0[7].i32;
+  } else if (tag0 == "vector_add_f32") {
+    if (n0 != 7 || !is_i32(a0[6])) return 0;
+    out = 4, in0 = 0, in1 = 2, scalar = 1.0f, n = a0[6].i32;
+  } else {
     return 0;
+  }
+  if (!vec_at(a0, n0, 0) || !vec_at(a0, n0, 2) || !vec_at(a0, n0, 4)) return 0;
   if (n1 != 5 || !vec_at(a1, n1, 0) || !vec_at(a1, n1, 2) || !is_i32(a1[4])) return 0;
-  const int64_t n = a0[7].i32;
   if (n <= 0 || a1[4].i32 != n) return 0;
   if (!covers_1d(block0, grid0, n)) return 0;
   if (a0[0].length < n || a0[2].length < n || a0[4].length < n) return 0;
-  if (shifted_overlap(a0[0].buffer, a0[2].buffer, n) || shifted_overlap(a0[0].buffer, a0[4].buffer, n)) return 0;
+  if (shifted_overlap(a0[out].buffer, a0[in0].buffer, n) || shifted_overlap(a0[out].buffer, a0[in1].buffer, n)) return 0;
   const int64_t nblocks = cdiv(n, 256);
   if (block1[0] != 256 || block1[1] != 1 || block1[2] != 1 || grid1[1] != 1 || grid1[2] != 1) return 0;
   if (grid1[0] != nblocks) return 0;
-  if (a1[0].buffer != a0[0].buffer || a1[0].length < n || a1[2].length < nblocks) return 0;
+  if (a1[0].buffer != a0[out].buffer || a1[0].length < n || a1[2].length < nblocks) return 0;
   for (int v = 0; v < 3; ++v) {
     if (reinterpret_cast<uintptr_t>(a0[2 * v].buffer) % 16 != 0) return 0;
     if (ranges_meet(a1[2].buffer, nblocks * 4, a0[2 * v].buffer, n * 4)) return 0;
   }
-  *rc = sarek_hip_triad_block256_sum_f32(static_cast<float *>(a0[0].buffer), static_cast<const float *>(a0[2].buffer),
-                                         static_cast<const float *>(a0[4].buffer), a0[6].f32, n,
-                                         static_cast<float *>(a1[2].buffer), nullptr);
+  if (is_sum)
+    *rc = sarek_hip_triad_block256_sum_f32(static_cast<float *>(a0[out].buffer), static_cast<const float *>(a0[in0].buffer),
+                                           static_cast<const float *>(a0[in1].buffer), scalar, n,
+                                           static_cast<float *>(a1[2].buffer), nullptr);
+  else
+    *rc = sarek_hip_triad_block256_max_f32(static_cast<float *>(a0[out].buffer), static_cast<const float *>(a0[in0].buffer),
+                                           static_cast<const float *>(a0[in1].buffer), scalar, n, pad,
+                                           static_cast<float *>(a1[2].buffer), nullptr);
   return 1;
 }
 

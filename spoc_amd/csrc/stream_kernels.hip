@@ -357,6 +357,86 @@ __device__ __forceinline__ float tree_max_of_block(float v0, float v1, float v2,
   return m;                        // valid in lane 0
 }
 
+// The stream triad and the block-256 maximum of its output in one pass (the element-wise kernel of bench_stream_triad.ml
+// or bench_vector_add.ml followed by bench_reduction_max.ml's tree).  Layout as triad_kernel's Runs form: a wave owns four
+// consecutive KiB, lane l of a slot holds elements 4l .. 4l+3 of that slot's 256-element block.  The tree's comparisons
+// are made in the tree's order with its strict ">" -- halves 128 .. 4 pair lane l with lanes l+32 .. l+1 component by
+// component, halves 2 and 1 pair the four components of lane 0 -- so NaNs and signed zeros come out as from the tree.
+// Elements past n count as `pad`, as in the reference kernel.
+template <bool NtLoad>
+__global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(8, 8))) void triad_block256_max_kernel(
+    float *__restrict__ a, const float *__restrict__ b, const float *__restrict__ c, float s, int64_t n, float pad,
+    float *__restrict__ block_max) {
+  static_assert(kUnroll == 4, "four block maxima per wave leave as one float4");
+  const double sd = static_cast<double>(s);
+  const int64_t n4 = n >> 2;
+  float4 *a4 = reinterpret_cast<float4 *>(a);
+  const float4 *b4 = reinterpret_cast<const float4 *>(b);
+  const float4 *c4 = reinterpret_cast<const float4 *>(c);
+  constexpr int kStep = 64;
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const int64_t base = static_cast<int64_t>(blockIdx.x) * kChunk + wave * (64 * kUnroll) + lane;
+  const bool full = base + (kUnroll - 1) * kStep < n4;   // the same for all lanes of a wave up to the slot that holds n
+  float4 r[kUnroll];
+  if (full) {
+    float4 bv[kUnroll], cv[kUnroll];
+#pragma unroll
+    for (int u = 0; u < kUnroll; ++u) bv[u] = NtLoad ? ldg_nt(b4 + base + u * kStep) : b4[base + u * kStep];
+#pragma unroll
+    for (int u = 0; u < kUnroll; ++u) cv[u] = NtLoad ? ldg_nt(c4 + base + u * kStep) : c4[base + u * kStep];
+#pragma unroll
+    for (int u = 0; u < kUnroll; ++u) {
+      r[u] = triad4(bv[u], cv[u], sd);
+      stg_nt(a4 + base + u * kStep, r[u]);
+    }
+  } else {
+#pragma unroll
+    for (int u = 0; u < kUnroll; ++u) {
+      const int64_t i = base + u * kStep;
+      if (i < n4) {
+        r[u] = triad4(b4[i], c4[i], sd);
+        a4[i] = r[u];
+      } else {
+        // the slot that holds the end of the vector takes its one to three elements; everything past n is pad
+        float t[4];
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          const int64_t k = (i << 2) + e;
+          t[e] = pad;
+          if (k < n) {
+            t[e] = triad1(b[k], c[k], sd);
+            a[k] = t[e];
+          }
+        }
+        r[u] = make_float4(t[0], t[1], t[2], t[3]);
+      }
+    }
+  }
+  const int64_t nblocks = (n + 255) >> 8;
+  float m[kUnroll];
+#pragma unroll
+  for (int u = 0; u < kUnroll; ++u) {
+    float4 v = r[u];
+#pragma unroll
+    for (int half = 32; half >= 1; half >>= 1) {   // tree halves 128 .. 4: element e against e + 4 * half
+      v.x = take_greater(v.x, __shfl_down(v.x, half, 64));
+      v.y = take_greater(v.y, __shfl_down(v.y, half, 64));
+      v.z = take_greater(v.z, __shfl_down(v.z, half, 64));
+      v.w = take_greater(v.w, __shfl_down(v.w, half, 64));
+    }
+    m[u] = take_greater(take_greater(v.x, v.z), take_greater(v.y, v.w));   // halves 2 and 1 (lane 0)
+  }
+  if (lane != 0) return;
+  const int64_t j0 = static_cast<int64_t>(blockIdx.x) * (kChunk / 64) + wave * kUnroll;
+  if (j0 + kUnroll <= nblocks && (reinterpret_cast<uintptr_t>(block_max) & 15u) == 0) {
+    *reinterpret_cast<float4 *>(block_max + j0) = make_float4(m[0], m[1], m[2], m[3]);
+  } else {
+#pragma unroll
+    for (int u = 0; u < kUnroll; ++u)
+      if (j0 + u < nblocks) block_max[j0 + u] = m[u];
+  }
+}
+
 __global__ __launch_bounds__(kBlock) void block256_max_kernel(const float *__restrict__ x,
                                                               float *__restrict__ out, int64_t n,
                                                               int64_t nblocks, float pad) {
@@ -615,6 +695,24 @@ int sarek_hip_triad_block256_sum_f32(float *a, const float *b, const float *c, f
     hipLaunchKernelGGL((triad_kernel<SUM_BLOCK256, false>), grid, dim3(kBlock), 0, st, a, b, c, s, n, block_sums);
   }
   return check_launch("triad + block-256 sum kernel launch");
+}
+
+int sarek_hip_triad_block256_max_f32(float *a, const float *b, const float *c, float s, int64_t n, float pad,
+                                     float *block_max, sarek_hip_stream stream) {
+  if (n < 0) return fail(SAREK_HIP_E_INVALID_ARG, "triad_block256_max: negative length %lld", (long long)n);
+  if (n == 0) return SAREK_HIP_OK;
+  if (!a || !b || !c || !block_max) return fail(SAREK_HIP_E_INVALID_ARG, "triad_block256_max: NULL vector");
+  if (!aligned16(a) || !aligned16(b) || !aligned16(c))
+    return fail(SAREK_HIP_E_INVALID_ARG, "triad_block256_max: vectors must be 16-byte aligned");
+  const int64_t blocks64 = triad_blocks(n);
+  if (blocks64 > 0x7FFFFFFF) return fail(SAREK_HIP_E_INVALID_ARG, "triad_block256_max: vector too long");
+  const dim3 grid(static_cast<unsigned>(blocks64));
+  hipStream_t st = as_stream(stream);
+  if (streams_from_hbm(n * 8))
+    hipLaunchKernelGGL(triad_block256_max_kernel<true>, grid, dim3(kBlock), 0, st, a, b, c, s, n, pad, block_max);
+  else
+    hipLaunchKernelGGL(triad_block256_max_kernel<false>, grid, dim3(kBlock), 0, st, a, b, c, s, n, pad, block_max);
+  return check_launch("triad + block-256 max kernel launch");
 }
 
 static int launch_block256(const float *x, const float *y, float *out, int64_t n, bool dot,

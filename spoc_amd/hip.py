@@ -201,6 +201,7 @@ SYMBOLS = {
     "sarek_hip_library_kernel_source": (_i, [C.c_char_p, C.c_char_p, _sz, C.POINTER(_sz), C.c_char_p, _sz]),
     "sarek_hip_library_kernel_list": (_i, [C.c_char_p, _sz, C.POINTER(_sz)]),
     "sarek_hip_triad_block256_sum_f32": (_i, [_vp, _vp, _vp, _f, _i64, _vp, _vp]),
+    "sarek_hip_triad_block256_max_f32": (_i, [_vp, _vp, _vp, _f, _i64, _f, _vp, _vp]),
     "sarek_hip_backend_name": (C.c_char_p, []),
     "sarek_hip_backend_version": (_i, [C.POINTER(_i), C.POINTER(_i), C.POINTER(_i)]),
     "sarek_hip_execution_model": (_i, []),
@@ -440,6 +441,19 @@ def triad_block256_sum(b, c, s, out=None):
     sums = torch.empty((b.numel() + 255) // 256, dtype=torch.float32, device=b.device)
     check(lib.sarek_hip_triad_block256_sum_f32(_ptr(a), _ptr(b), _ptr(c), float(s), b.numel(), _ptr(sums), _stream()))
     return a, sums
+
+
+def triad_block256_max(b, c, s, pad, out=None):
+    """a = b + c*s and the block-256 maxima of a (elements past the end count as pad) in one pass.
+    Returns (a, block_max)."""
+    torch = _torch()
+    _need(b, torch.float32, "b")
+    _need(c, torch.float32, "c")
+    a = torch.empty_like(b) if out is None else out
+    mx = torch.empty((b.numel() + 255) // 256, dtype=torch.float32, device=b.device)
+    check(lib.sarek_hip_triad_block256_max_f32(_ptr(a), _ptr(b), _ptr(c), float(s), b.numel(), float(pad), _ptr(mx),
+                                               _stream()))
+    return a, mx
 
 
 def library_kernel(name):

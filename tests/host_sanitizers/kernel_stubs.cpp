@@ -13,6 +13,7 @@ int sarek_hip_reduce_sum_block256_f32(const float *, float *, int64_t, sarek_hip
 int sarek_hip_transpose_f32(const float *, float *, int, int, sarek_hip_stream) { return -1; }
 int sarek_hip_triad_f32(float *, const float *, const float *, float, int64_t, sarek_hip_stream) { return -1; }
 int sarek_hip_triad_block256_sum_f32(float *, const float *, const float *, float, int64_t, float *, sarek_hip_stream) { return -1; }
+int sarek_hip_triad_block256_max_f32(float *, const float *, const float *, float, int64_t, float, float *, sarek_hip_stream) { return -1; }
 int sarek_hip_triad_sum_f32_static(float *, const float *, const float *, float, int64_t, double *, sarek_hip_stream) { return -1; }
 int sarek_hip_gemm_bf16(const uint16_t *, const uint16_t *, float *, int, int, int, sarek_hip_stream) { return -1; }
 int sarek_hip_gemm_f16(const uint16_t *, const uint16_t *, float *, int, int, int, sarek_hip_stream) { return -1; }

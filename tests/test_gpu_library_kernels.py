@@ -257,6 +257,40 @@ def test_triad_then_block_sum_pipeline_is_one_launch(hip, oracle, sarek, n):
     assert np.array_equal(va.to_array(), a_hand) and np.array_equal(vout.to_array(), o_hand)
 
 
+@pytest.mark.parametrize("n", [1, 255, 257, 4099, 1000003])
+def test_vector_add_then_block_sum_pipeline_is_one_launch(hip, oracle, sarek, n):
+    """The other element-wise producer of the reference's benches in front of the block-256 sum
+    (bench_vector_add.ml, bench_reduction.ml): c = a + b and the sums of c in one pass, the same bits as the two hand
+    kernels one after the other, the generated pair within the sum's tolerance."""
+    E, V = sarek.Execute, sarek.Vector
+    a = oracle.fill_uniform(n, seed=0xA)
+    b = oracle.fill_uniform(n, seed=0xB)
+    c_ref, partials_ref, _ = oracle.triad_sum(a, b, 1.0)      # a + 1.0 * b rounded once is the f32 sum
+    assert np.array_equal(c_ref, a + b)
+
+    def stages_and_vectors():
+        va, vb, vc = V.of_array(a), V.of_array(b), V.create(V.float32, n)
+        vout = V.create(V.float32, (n + 255) // 256)
+        vc.host[:] = np.nan
+        vout.host[:] = np.nan
+        grid = ((n + 255) // 256, 1, 1)
+        return [(load_ir("vector_add"), [E.Vec(va), E.Vec(vb), E.Vec(vc), E.Int32(n)], (256, 1, 1), grid),
+                (load_ir("reduction"), [E.Vec(vc), E.Vec(vout), E.Int32(n)], (256, 1, 1), grid)], (vc, vout)
+
+    def run():
+        stages, (vc, vout) = stages_and_vectors()
+        return E.run_pipeline(stages), (vc.to_array().copy(), vout.to_array().copy())
+
+    (hand, (c_hand, o_hand)), (jit, (c_jit, o_jit)) = both_ways(hip, run)
+    assert hand == ("vector_add_f32+reduce_sum_block256_f32", 1) and jit == ("jit;jit", 2)
+    assert np.array_equal(c_hand, c_ref) and np.array_equal(c_jit, c_ref)
+    tol = 1e-5 * np.abs(partials_ref).max()
+    assert np.abs(o_hand - partials_ref).max() <= tol and np.abs(o_jit - partials_ref).max() <= tol
+    stages, (vc, vout) = stages_and_vectors()
+    assert E.run_vectors(*stages[0]) == "vector_add_f32" and E.run_vectors(*stages[1]) == "reduce_sum_block256_f32"
+    assert np.array_equal(vc.to_array(), c_hand) and np.array_equal(vout.to_array(), o_hand)
+
+
 def test_pipeline_pairs_that_are_not_the_fused_operation_run_one_by_one(hip, oracle, sarek):
     E, V = sarek.Execute, sarek.Vector
     n = 70000
@@ -458,3 +492,64 @@ def test_hand_and_generated_triad_agree(hip, oracle, torch_cuda):
     differ = (hand != jit)
     assert int(differ.sum()) <= 2
     assert bool(((hand - jit).abs() <= torch.finfo(torch.float32).eps * hand.abs()).all())
+
+
+@pytest.mark.parametrize("producer", ["stream_triad", "vector_add"])
+@pytest.mark.parametrize("n", [1, 3, 255, 256, 257, 4099, 65537, 1000003])
+def test_elementwise_then_block_max_is_one_launch(hip, oracle, torch_cuda, producer, n):
+    """{stream triad, vector add} followed by the block-256 maximum of its output (bench_reduction_max.ml's tree, fill
+    -1000000.0): one launch at the plugin boundary, the element-wise result and the maxima bit for bit those of the
+    oracle's tree (elements past the end count as the fill), and of the generated pair."""
+    from test_ir_lowering import reduction_max_ir
+    torch = torch_cuda
+    nb = (n + 255) // 256
+    x = (oracle.fill_uniform(n, seed=0x9) * 2000 - 1000).astype(np.float32)
+    y = (oracle.fill_uniform(n, seed=0xA) * 20 - 10).astype(np.float32)
+    s = 3.0 if producer == "stream_triad" else 1.0
+    a_ref = oracle.triad(x, y, s)
+    dx, dy = torch.from_numpy(x).cuda(), torch.from_numpy(y).cuda()
+    red = hip.generate_source(reduction_max_ir(), block=(256, 1, 1))
+    src = hip.generate_source(load_ir(producer))
+    got = {}
+    for specialise in (1, 0):
+        a = torch.full((n,), float("nan"), device="cuda")
+        mx = torch.full((nb,), float("nan"), device="cuda")
+        if producer == "stream_triad":
+            l0 = (src, "sarek_kern", (256, 1, 1), (nb, 1, 1), [a, dx, dy, ("f32", s), ("i32", n)])
+        else:
+            l0 = (src, "sarek_kern", (256, 1, 1), (nb, 1, 1), [dx, dy, a, ("i32", n)])
+        l1 = (red, "sarek_kern", (256, 1, 1), (nb, 1, 1), [a, mx, ("i32", n)], 1024)
+        hip.check(hip.lib.sarek_hip_set_specialisation(specialise))
+        try:
+            got[specialise] = hip.run_sources([l0, l1]), a.cpu().numpy(), mx.cpu().numpy()
+        finally:
+            hip.check(hip.lib.sarek_hip_set_specialisation(1))
+    tag = {"stream_triad": "stream_triad_f32", "vector_add": "vector_add_f32"}[producer]
+    assert got[1][0] == (tag + "+reduce_max_block256_f32:c9742400", 1)
+    assert got[0][0] == ("jit;jit", 2)
+    for _, a, mx in got.values():
+        assert np.array_equal(a, a_ref)
+        assert np.array_equal(mx, oracle.reduce_max_block256(a_ref))
+
+
+def test_fused_block_max_keeps_the_trees_order_for_nans_and_signed_zeros(hip, oracle, torch_cuda):
+    """The tree compares with a strict ">", so which of two equal zeros or which side of a NaN survives depends on
+    the order of the comparisons: the fused kernel's maxima are the bits of the stand-alone tree kernel's and of the
+    oracle's, on inputs full of both."""
+    torch = torch_cuda
+    n = 256 * 37 + 129
+    rng = np.random.default_rng(5)
+    b = rng.choice(np.array([0.0, -0.0, 1.0, -1.0, np.nan, -7.5], np.float32), size=n)
+    c = rng.choice(np.array([0.0, -0.0, 2.0, np.nan], np.float32), size=n)
+    # whole blocks of zeros of both signs, and a block that is all NaN
+    b[:256], c[:256] = rng.choice(np.array([0.0, -0.0], np.float32), size=256), 0.0
+    b[256:512], c[256:512] = np.nan, 0.0
+    db, dc = torch.from_numpy(b).cuda(), torch.from_numpy(c).cuda()
+    for pad in (-1000000.0, 0.0, -0.0):
+        a, mx = hip.triad_block256_max(db, dc, 1.0, pad)
+        a_ref = oracle.triad(b, c, 1.0)
+        assert np.array_equal(a.cpu().numpy().view(np.uint32), a_ref.view(np.uint32))
+        want = oracle.reduce_max_block256(a_ref, pad=pad)
+        alone = hip.reduce_max_block256(a, pad)
+        assert np.array_equal(mx.cpu().numpy().view(np.uint32), want.view(np.uint32))
+        assert np.array_equal(alone.cpu().numpy().view(np.uint32), want.view(np.uint32))
