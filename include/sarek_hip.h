@@ -457,7 +457,8 @@ int sarek_hip_triad_sum_f32(float *a, const float *b, const float *c, float s, i
  * sarek_hip_triad_f32 does and block_sums[j] = sum of a[256j .. 256j+255] (zero padded),
  * j < ceil(n/256), with the bits sarek_hip_reduce_sum_block256_f32 would produce from that a
  * (benchmarks/bench_stream_triad.ml:22-32 followed by benchmarks/bench_reduction.ml:62-96; what
- * sarek_hip_execute_run_pipeline launches for that pair of kernels).  Vectors 16-byte aligned. */
+ * sarek_hip_execute_run_pipeline launches for that pair of kernels).  Vectors at any alignment (16-byte
+ * aligned ones are the fast case: the others cost the pass about 7 %).                                */
 int sarek_hip_triad_block256_sum_f32(float *a, const float *b, const float *c, float s, int64_t n,
                                      float *block_sums, sarek_hip_stream stream);
 /* The same with the block-256 maximum in place of the sum: block_max[j] = what the reference's halving tree

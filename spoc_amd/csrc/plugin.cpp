@@ -254,7 +254,6 @@ int try_specialised(const std::string &tag, const int block[3], const int grid[3
     if (args[2 * (nv - 1)].length < nblocks) return 0;
     for (int v = 0; v < nv - 1; ++v) {
       if (args[2 * v].length < n) return 0;
-      if (reinterpret_cast<uintptr_t>(args[2 * v].buffer) % 16 != 0) return 0;
     }
     if (dot)
       *rc = sarek_hip_dot_block256_f32(static_cast<const float *>(args[0].buffer),
@@ -396,7 +395,6 @@ int try_specialised_pair(const std::string &tag0, const int block0[3], const int
   if (grid1[0] != nblocks) return 0;
   if (a1[0].buffer != a0[out].buffer || a1[0].length < n || a1[2].length < nblocks) return 0;
   for (int v = 0; v < 3; ++v) {
-    if (reinterpret_cast<uintptr_t>(a0[2 * v].buffer) % 16 != 0) return 0;
     if (ranges_meet(a1[2].buffer, nblocks * 4, a0[2 * v].buffer, n * 4)) return 0;
   }
   if (is_sum)

@@ -151,3 +151,47 @@ def test_block256_max_matches_tree_bit_for_bit(hip, oracle, torch_cuda, n):
     # another fill value
     got = hip.reduce_max_block256(torch.from_numpy(x).cuda(), pad=float("-inf")).cpu().numpy()
     assert np.array_equal(got.view(np.uint32), oracle.reduce_max_block256(x, pad=float("-inf")).view(np.uint32))
+
+
+@pytest.mark.parametrize("offsets", [(1, 1, 1), (1, 2, 3), (0, 1, 0), (3, 0, 2)])
+@pytest.mark.parametrize("n", [1, 5, 1023, 4099, 300007])
+def test_stream_kernels_take_vectors_at_any_alignment(hip, oracle, torch_cuda, offsets, n):
+    """Sub-vectors start anywhere (Vector.sub_vector): the triad, the fused triad + block sum / maximum and the block
+    reductions run their 128-bit kernels on vectors that are only 4-byte aligned and give the aligned results; the
+    element-per-thread kernel stays reachable behind stream.force_scalar."""
+    torch = torch_cuda
+    oa, ob, oc = offsets
+    b = oracle.fill_uniform(n, seed=11)
+    c = (oracle.fill_uniform(n, seed=12) * 2000 - 1000).astype(np.float32)
+    db = torch.full((n + 8,), float("nan"), device="cuda")[ob:ob + n]
+    dc = torch.full((n + 8,), float("nan"), device="cuda")[oc:oc + n]
+    db.copy_(dev(torch, b))
+    dc.copy_(dev(torch, c))
+    guard = torch.full((n + 8,), 7.0, device="cuda")
+    out = guard[oa:oa + n]
+    a_ref, partials_ref, sum_ref = oracle.triad_sum(b, c, 3.0)
+    for scalar in (0, 1):
+        hip.set_tunable("stream.force_scalar", scalar)
+        try:
+            guard.fill_(7.0)
+            a, total = hip.triad_sum(db, dc, 3.0, out=out)
+            assert np.array_equal(a.cpu().numpy(), a_ref)
+            assert bool((guard[:oa] == 7).all()) and bool((guard[oa + n:] == 7).all())
+            assert abs(float(total.item()) - sum_ref) <= 1e-5 * abs(sum_ref)
+        finally:
+            hip.set_tunable("stream.force_scalar", 0)
+    guard.fill_(7.0)
+    a, sums = hip.triad_block256_sum(db, dc, 3.0, out=out)
+    assert np.array_equal(a.cpu().numpy(), a_ref) and bool((guard[:oa] == 7).all()) and bool((guard[oa + n:] == 7).all())
+    assert np.abs(sums.cpu().numpy() - partials_ref).max() <= 1e-5 * np.abs(partials_ref).max()
+    a, mx = hip.triad_block256_max(db, dc, 3.0, -1000000.0, out=out)
+    assert np.array_equal(a.cpu().numpy(), a_ref)
+    assert np.array_equal(mx.cpu().numpy(), oracle.reduce_max_block256(a_ref))
+    # the block reductions on an unaligned input
+    assert np.array_equal(hip.reduce_max_block256(dc).cpu().numpy(), oracle.reduce_max_block256(c))
+    got = hip.reduce_sum_block256(db).cpu().numpy()
+    want = oracle.reduce_sum_block256(b)
+    assert np.abs(got - want).max() <= 1e-5 * np.abs(want).max()
+    got = hip.dot_block256(db, dc).cpu().numpy()
+    want = oracle.dot_block256(b, c)
+    assert np.abs(got - want).max() <= 1e-5 * max(np.abs(want).max(), 1e-30)
