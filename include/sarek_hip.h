@@ -516,7 +516,7 @@ int sarek_hip_transpose_f32(const float *in, float *out, int width, int height, 
  * what a launch of the kernel of benchmarks/bench_histogram.ml:54-84 over n keys adds to the
  * global histogram (`mod` is the generated code's `%`: a negative key with a non-zero
  * remainder has no bin and is not counted, where that kernel indexes its shared array with
- * it).  The histogram is accumulated into, not cleared; keys 16-byte aligned.          */
+ * it).  The histogram is accumulated into, not cleared.                                 */
 int sarek_hip_histogram_i32(int32_t *histogram, const int32_t *keys, int64_t n, int num_bins,
                             sarek_hip_stream stream);
 /* histogram[d] += #{ i < n : (keys[i] >> shift) & mask == d }, 256 bins, 0 <= mask <= 255,
@@ -530,7 +530,7 @@ int sarek_hip_radix_histogram_i32(int32_t *histogram, const int32_t *keys, int64
  * Afterwards counters[d] has grown by the number of keys with digit d and out holds them in
  * [old counters[d], new counters[d]), in an order that kernel can produce (it fixes none: its
  * positions come from global atomics).  A position outside [0, out_len) is skipped, where that
- * kernel writes out of bounds.  The three vectors must not overlap; keys 16-byte aligned.        */
+ * kernel writes out of bounds.  The three vectors must not overlap.                              */
 int sarek_hip_radix_scatter_i32(int32_t *out, int64_t out_len, int32_t *counters, const int32_t *keys, int64_t n,
                                 int shift, int mask, sarek_hip_stream stream);
 

@@ -43,7 +43,7 @@ struct DigitBin {     // bench_radix_sort.ml:101: (key >> shift) & mask, `>>` as
 
 // histogram[b] += #{ i < n : bin(keys[i]) == b } for 0 <= b < bins (bins <= 256).  A key whose bin
 // falls outside [0, bins) is not counted (the reference's kernel indexes its shared array with it).
-// keys must be 16-byte aligned; workgroup g takes the 16-byte groups g, g + G, g + 2G, ... in steps
+// keys at any alignment (the 128-bit loads need none beyond the element's); workgroup g takes the 16-byte groups g, g + G, g + 2G, ... in steps
 // of kThreads, the last workgroup also the n & 3 trailing keys.
 template <class Bin>
 __global__ __launch_bounds__(kThreads) void histogram_kernel(int *__restrict__ histogram,
@@ -280,8 +280,6 @@ int launch(int *histogram, const int *keys, int64_t n, int bins, Bin bin, hipStr
 int check_common(const char *what, const int *histogram, const int *keys, int64_t n) {
   if (n < 0) return fail(SAREK_HIP_E_INVALID_ARG, "%s: negative length %lld", what, (long long)n);
   if (n > 0 && (!histogram || !keys)) return fail(SAREK_HIP_E_INVALID_ARG, "%s: NULL vector", what);
-  if (n > 0 && (reinterpret_cast<uintptr_t>(keys) & 15))
-    return fail(SAREK_HIP_E_INVALID_ARG, "%s: the keys must be 16-byte aligned", what);
   return SAREK_HIP_OK;
 }
 

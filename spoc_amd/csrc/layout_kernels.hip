@@ -86,7 +86,7 @@ __device__ __forceinline__ void tile_of(int order, int tiles_c, int tiles_r, int
 // 64 x 64 tile through LDS: 16 lanes read 256 contiguous bytes of an input row, the tile is
 // kept with a row pitch of 65 words (both the row-wise stores and the column-wise loads then
 // touch 64 different banks per wave), and 16 lanes write 256 contiguous bytes of an output
-// row.  Needs width % 4 == height % 4 == 0 and 16-byte aligned matrices.
+// row.  Needs width % 4 == height % 4 == 0 (the matrices themselves may start on any 4-byte boundary).
 template <int TR, bool NtLoad, bool NtStore>
 __global__ __launch_bounds__(kBlock) void transpose_lds_kernel(const float *__restrict__ in,
                                                                float *__restrict__ out, int width, int height,
@@ -170,7 +170,6 @@ __global__ __launch_bounds__(kBlock) void transpose_scalar_kernel(const float *_
   }
 }
 
-inline bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 
 }  // namespace
 }  // namespace sarek_hip
@@ -185,7 +184,8 @@ int sarek_hip_copy_f32(float *dst, const float *src, int64_t n, sarek_hip_stream
   if (!dst || !src) return fail(SAREK_HIP_E_INVALID_ARG, "copy: NULL vector");
   const int64_t blocks = ceil_div(n, static_cast<int64_t>(kCopyChunk));
   if (blocks > 0x7FFFFFFF) return fail(SAREK_HIP_E_INVALID_ARG, "copy: vector too long for one launch");
-  if (aligned16(dst) && aligned16(src)) {
+  // the 128-bit accesses need no alignment beyond the element's; copy.force_scalar keeps the other kernel reachable
+  if (tunable("copy.force_scalar", 0) == 0) {
     int64_t nt = tunable("copy.nt", -1);
     if (nt < 0) nt = n * 4 > kLastLevelCacheBytes;
     if (nt)
@@ -208,7 +208,7 @@ int sarek_hip_transpose_f32(const float *in, float *out, int width, int height, 
   if (!in || !out) return fail(SAREK_HIP_E_INVALID_ARG, "transpose: NULL matrix");
   if (in == out) return fail(SAREK_HIP_E_INVALID_ARG, "transpose: in-place transposition is not supported");
   hipStream_t st = as_stream(stream);
-  if (width % 4 == 0 && height % 4 == 0 && aligned16(in) && aligned16(out)) {
+  if (width % 4 == 0 && height % 4 == 0 && tunable("transpose.force_scalar", 0) == 0) {
     // Measured on MI355X: 128-row tiles; an input that fits the last-level cache is best read
     // with plain loads and with each XCD walking its own run of tiles (order 3), a larger one
     // with non-temporal loads and neighbouring workgroups writing neighbouring pieces (order 1).

@@ -205,7 +205,6 @@ int try_specialised(const std::string &tag, const int block[3], const int grid[3
     if (args[0].length < n || args[2].length < bins) return 0;
     const uintptr_t in = reinterpret_cast<uintptr_t>(args[0].buffer), hist = reinterpret_cast<uintptr_t>(args[2].buffer);
     if (in < hist + static_cast<uintptr_t>(bins) * 4 && hist < in + static_cast<uintptr_t>(n) * 4) return 0;
-    if (in & 15) return 0;
     *rc = radix ? sarek_hip_radix_histogram_i32(static_cast<int32_t *>(args[2].buffer),
                                                 static_cast<const int32_t *>(args[0].buffer), n, args[5].i32,
                                                 args[6].i32, nullptr)
@@ -231,7 +230,6 @@ int try_specialised(const std::string &tag, const int block[3], const int grid[3
                     cnt_b = static_cast<uintptr_t>(mask + 1) * 4;
     auto meet = [](uintptr_t a, uintptr_t ab, uintptr_t b, uintptr_t bb) { return a < b + bb && b < a + ab; };
     if (meet(in, in_b, out, out_b) || meet(in, in_b, cnt, cnt_b) || meet(out, out_b, cnt, cnt_b)) return 0;
-    if (in & 15) return 0;
     *rc = sarek_hip_radix_scatter_i32(static_cast<int32_t *>(args[2].buffer), args[2].length,
                                       static_cast<int32_t *>(args[4].buffer),
                                       static_cast<const int32_t *>(args[0].buffer), n, shift, mask, nullptr);

@@ -44,12 +44,18 @@ def test_copy_unaligned_and_policies(hip, torch_cuda):
     torch = torch_cuda
     n = 70001
     base_s, base_d = torch.rand(n + 16, device="cuda"), torch.zeros(n + 16, device="cuda")
-    for so, do in ((1, 0), (0, 3), (2, 2)):                    # 4-byte aligned only: scalar kernel
-        s, d = base_s[so:so + n], base_d[do:do + n]
-        d.zero_()
-        hip.check(hip.lib.sarek_hip_copy_f32(d.data_ptr(), s.data_ptr(), n, None))
-        torch.cuda.synchronize()
-        assert torch.equal(d, s)
+    for scalar in (0, 1):                                      # the 128-bit kernel and the element-per-thread one
+        hip.set_tunable("copy.force_scalar", scalar)
+        try:
+            for so, do in ((1, 0), (0, 3), (2, 2)):            # 4-byte aligned only
+                s, d = base_s[so:so + n], base_d[do:do + n]
+                base_d.fill_(-1)
+                hip.check(hip.lib.sarek_hip_copy_f32(d.data_ptr(), s.data_ptr(), n, None))
+                torch.cuda.synchronize()
+                assert torch.equal(d, s)
+                assert bool((base_d[:do] == -1).all()) and bool((base_d[do + n:] == -1).all())
+        finally:
+            hip.set_tunable("copy.force_scalar", 0)
     try:
         for nt in (0, 1):                                      # both load policies
             hip.set_tunable("copy.nt", nt)
@@ -91,12 +97,18 @@ def test_transpose_every_variant(hip, torch_cuda):
         hip.set_tunable("transpose.rows", 128)
         hip.set_tunable("transpose.order", -1)
         hip.set_tunable("transpose.nt", -1)
-    # unaligned matrices take the scalar kernel
-    flat = torch.rand(64 * 64 + 1, device="cuda")
-    out = torch.zeros(64 * 64 + 1, device="cuda")
-    hip.check(hip.lib.sarek_hip_transpose_f32(flat[1:].data_ptr(), out[1:].data_ptr(), 64, 64, None))
-    torch.cuda.synchronize()
-    assert torch.equal(out[1:].view(64, 64), flat[1:].view(64, 64).t())
+    # matrices that are only 4-byte aligned: the tiled kernel, and the scalar one behind its knob
+    for scalar in (0, 1):
+        hip.set_tunable("transpose.force_scalar", scalar)
+        try:
+            flat = torch.rand(64 * 128 + 1, device="cuda")
+            out = torch.full((64 * 128 + 3,), -1.0, device="cuda")
+            hip.check(hip.lib.sarek_hip_transpose_f32(flat[1:].data_ptr(), out[1:-2].data_ptr(), 64, 128, None))
+            torch.cuda.synchronize()
+            assert torch.equal(out[1:-2].view(64, 128), flat[1:].view(128, 64).t())
+            assert out[0].item() == -1 and bool((out[-2:] == -1).all())
+        finally:
+            hip.set_tunable("transpose.force_scalar", 0)
     assert hip.lib.sarek_hip_transpose_f32(flat.data_ptr(), flat.data_ptr(), 8, 8, None) == hip.E_INVALID_ARG
     assert hip.lib.sarek_hip_transpose_f32(flat.data_ptr(), out.data_ptr(), -1, 8, None) == hip.E_INVALID_ARG
     assert hip.lib.sarek_hip_transpose_f32(flat.data_ptr(), out.data_ptr(), 0, 8, None) == 0
