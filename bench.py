@@ -60,7 +60,8 @@ def parse():
                     choices=["gemm_bf16_8192", "gemm_f16_8192", "triad_sum_2p28", "gemm_f32_8192", "gemm_f32_1024",
                              "gemm_f16_epilogue", "gemm_f16_4095x11008x4096", "gemm_f16_shape", "gemm_bf16_shape", "gemm_bf16_2048", "gemm_f32_shape", "vendor_gemm_f32_shape", "copy_1gib",
                              "vendor_gemm_bf16_8192", "vendor_gemm_bf16_shape", "histogram_2p28",
-                             "radix_scatter_5e7", "mfma_bf16_stream", "mfma_bf16_stream_32x32x16", "l2_to_lds_stream"])
+                             "radix_scatter_5e7", "stencil_2d_shape", "conv2d_shape", "mfma_bf16_stream", "mfma_bf16_stream_32x32x16",
+                             "l2_to_lds_stream"])
     ap.add_argument("--warmup-ms", type=float, default=60.0,
                     help="warm up for at least this long (and at least --warmup steps): the clocks of a power-limited "
                          "kernel take 30-40 ms to settle after a pause")
@@ -68,7 +69,8 @@ def parse():
                     help="add the timed launches' kernel durations in launch order (kernel_us_by_launch)")
     ap.add_argument("--no-also", action="store_true", help="measure only the headline workload")
     ap.add_argument("--no-cpu-baseline", action="store_true")
-    ap.add_argument("--shape", default="4096,11264,4096", metavar="M,N,K", help="shape of the gemm_f16_shape workload")
+    ap.add_argument("--shape", default="4096,11264,4096", metavar="M,N,K",
+                    help="shape of the *_shape workloads (stencil_2d_shape, conv2d_shape: width,height,ignored)")
     ap.add_argument("--l2-stream", default="", metavar="WORKGROUPS,WINDOW_MIB",
                     help="shape of the l2_to_lds_stream workload (default 1024,2)")
     ap.add_argument("--zero-operands", action="store_true",
@@ -315,6 +317,29 @@ def make_workload(name, torch, hip):
                     config={"workload": "histogram[key mod 256] += 1, uniform keys", "n": n,
                             "algorithmic_bytes": 4 * n})
         return main, None, info, (vk, vh, a, ir)
+    if name in ("stencil_2d_shape", "conv2d_shape"):
+        w, h = GEMM_SHAPE[0], GEMM_SHAPE[1]
+        stencil = name[0] == "s"
+        g.manual_seed(0xC6)
+        t = torch.rand(w * h, device="cuda", generator=g) * 2 - 1
+        vi = device_vector(sarek, hip, torch, t, V.float32)
+        del t
+        vo = V.create(V.float32, w * h)
+        sarek.Transfer.to_device(vo)
+        a, na = E._args([E.Vec(vi), E.Vec(vo), E.Int32(w), E.Int32(h)])
+        if stencil:
+            ir, block, grid = rk.stencil_2d().encode(), dims(16, 16, 1), dims((w + 15) // 16, (h + 15) // 16, 1)
+        else:
+            ir, block, grid = rk.conv2d().encode(), dims(256, 1, 1), dims((w * h + 255) // 256, 1, 1)
+        main = Launch(hip, lib.sarek_hip_execute_run_vectors, ir, block, grid, 0, a, na)
+        what = "five-point mean (bench_stencil_2d.ml:43-58)" if stencil else "3 x 3 box filter (bench_conv2d.ml:49-77)"
+        info = dict(metric=("2-D five-point stencil" if stencil else "3 x 3 box filter") + " GB/s", unit="GB/s",
+                    dtype="f64", work=8.0 * w * h, work_unit=1e9, bound="hbm", peak=PEAK_HBM_GBS,
+                    kernel="neighbourhood_kernel<%s>" % ("true" if not stencil else "false"),
+                    route="Execute.run_vectors, " + what,
+                    config={"workload": what + ", cells uniform[-1,1)", "width": w, "height": h,
+                            "algorithmic_bytes": 8 * w * h})
+        return main, None, info, (vi, vo, a, ir)
     if name == "radix_scatter_5e7":
         n = 50_000_000
         g.manual_seed(0xC5)
@@ -803,7 +828,8 @@ def main():
     }
     if args.trace_launches:
         out["kernel_us_by_launch"] = head["kernel_us_by_launch"]
-    if not args.no_cpu_baseline and args.workload not in ("copy_1gib", "vendor_gemm_bf16_8192", "vendor_gemm_bf16_shape", "gemm_bf16_shape", "gemm_f16_shape", "gemm_f32_shape", "vendor_gemm_f32_shape", "mfma_bf16_stream", "mfma_bf16_stream_32x32x16", "l2_to_lds_stream"):
+    if not args.no_cpu_baseline and args.workload not in ("copy_1gib", "vendor_gemm_bf16_8192", "vendor_gemm_bf16_shape", "gemm_bf16_shape", "gemm_f16_shape", "gemm_f32_shape", "vendor_gemm_f32_shape", "mfma_bf16_stream", "mfma_bf16_stream_32x32x16", "l2_to_lds_stream",
+                                                        "stencil_2d_shape", "conv2d_shape"):
         out["cpu_baseline"] = cpu_baseline(args.workload)
     if not args.no_also:
         also = []

@@ -511,6 +511,16 @@ int sarek_hip_copy_f32(float *dst, const float *src, int64_t n, sarek_hip_stream
  * benchmarks/bench_transpose.ml and bench_transpose_tiled.ml (`in` has `height` rows
  * of `width` floats).  in and out must not overlap.                                 */
 int sarek_hip_transpose_f32(const float *in, float *out, int width, int height, sarek_hip_stream stream);
+/* output[y * width + x] = (up + down + left + right + center) / 5 for 0 < x < width - 1 and
+ * 0 < y < height - 1, the operands widened to double, added in that order and rounded once at
+ * the store; the border keeps what it holds: the kernel of benchmarks/bench_stencil_2d.ml:43-58
+ * launched over the whole grid.  Any width and height (below 3 nothing is written), grids at
+ * any alignment; input and output must not overlap; width * height < 2^31.            */
+int sarek_hip_stencil_2d_f32(const float *input, float *output, int width, int height, sarek_hip_stream stream);
+/* The 3 x 3 box filter of benchmarks/bench_conv2d.ml:49-77 launched over all width * height
+ * cells: 0 on the border, elsewhere the nine cells round (x, y) added row by row, left to
+ * right, in double, divided by 9 and rounded once.  Same conditions as the stencil.    */
+int sarek_hip_conv2d_f32(const float *input, float *output, int width, int height, sarek_hip_stream stream);
 
 /* histogram[b] += #{ i < n : keys[i] mod num_bins == b } for b < num_bins, 1 <= num_bins <= 256:
  * what a launch of the kernel of benchmarks/bench_histogram.ml:54-84 over n keys adds to the

@@ -245,6 +245,12 @@ let copy_f32 =
 let transpose_f32 =
   bind "sarek_hip_transpose_f32"
     (ptr float @-> ptr float @-> int @-> int @-> ptr void @-> returning int)
+let stencil_2d_f32 =
+  bind "sarek_hip_stencil_2d_f32"
+    (ptr float @-> ptr float @-> int @-> int @-> ptr void @-> returning int)
+let conv2d_f32 =
+  bind "sarek_hip_conv2d_f32"
+    (ptr float @-> ptr float @-> int @-> int @-> ptr void @-> returning int)
 let histogram_i32 =
   bind "sarek_hip_histogram_i32"
     (ptr int32_t @-> ptr int32_t @-> int64_t @-> int @-> ptr void @-> returning int)

@@ -17,6 +17,7 @@ __all__ = [
     "triad", "reduce_sum_block256", "reduce_max_block256", "dot_block256", "fold_partials", "triad_sum",
     "gemm", "gemm_rows", "gemm_bias_relu_rowsum", "matmul_tiled_bsp",
     "vector_add", "vector_copy", "transpose", "histogram", "radix_histogram", "radix_scatter", "matmul_naive",
+    "stencil_2d", "conv2d",
 ]
 
 
@@ -60,6 +61,8 @@ def _L():
         lib.oracle_vector_add_f32.argtypes = [f32p, f32p, f32p, i64, i64]
         lib.oracle_vector_copy_f32.argtypes = [f32p, f32p, i64, i64]
         lib.oracle_transpose_f32.argtypes = [f32p, f32p, i32, i32, i64]
+        lib.oracle_stencil_2d_f32.argtypes = [f32p, f32p, i32, i32, i64, i64]
+        lib.oracle_conv2d_f32.argtypes = [f32p, f32p, i32, i32, i64]
         lib.oracle_matmul_naive_f32.argtypes = [f32p, f32p, f32p, i32, i32, i32, i64]
         _lib = lib
     return _lib
@@ -271,6 +274,28 @@ def transpose(x, width, height, out=None, threads=None):
     assert out.dtype == np.float32 and out.flags.c_contiguous
     _L().oracle_transpose_f32(xp, out.ctypes.data_as(C.POINTER(C.c_float)), width, height,
                               _launch_size(width * height, threads))
+    return out
+
+
+def stencil_2d(x, width, height, out=None, threads_xy=None):
+    """In place on `out` (the border and any cell the launch does not reach keep their values; zeros if not given);
+    threads_xy = (threads in x, threads in y) of the 2-D launch, the whole grid by default."""
+    x, xp = _f32(x)
+    if out is None:
+        out = np.zeros(width * height, dtype=np.float32)
+    assert out.dtype == np.float32 and out.flags.c_contiguous
+    tx, ty = (width, height) if threads_xy is None else threads_xy
+    _L().oracle_stencil_2d_f32(xp, out.ctypes.data_as(C.POINTER(C.c_float)), width, height, tx, ty)
+    return out
+
+
+def conv2d(x, width, height, out=None, threads=None):
+    x, xp = _f32(x)
+    if out is None:
+        out = np.zeros(width * height, dtype=np.float32)
+    assert out.dtype == np.float32 and out.flags.c_contiguous
+    _L().oracle_conv2d_f32(xp, out.ctypes.data_as(C.POINTER(C.c_float)), width, height,
+                           _launch_size(width * height, threads))
     return out
 
 

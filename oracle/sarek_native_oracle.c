@@ -545,4 +545,50 @@ void oracle_matmul_naive_f32(const float *a, const float *b, float *c, int32_t m
   }
 }
 
+/* benchmarks/bench_stencil_2d.ml:43-58, thread by thread of a 2-D launch of threads_x x threads_y
+ * threads: x and y are the global thread coordinates; for 0 < x < width - 1 and 0 < y < height - 1 the
+ * five neighbours are read as doubles, added in the order up, down, left, right, center, divided by 5.0
+ * and rounded once at the store (float32 vectors hold OCaml floats on the Native backend); every other
+ * cell of `output` keeps what it holds.                                                                 */
+void oracle_stencil_2d_f32(const float *input, float *output, int32_t width, int32_t height, int64_t threads_x,
+                           int64_t threads_y) {
+  for (int64_t ty = 0; ty < threads_y; ++ty)
+    for (int64_t tx = 0; tx < threads_x; ++tx) {
+      const int32_t x = (int32_t)tx, y = (int32_t)ty;
+      if (x > 0 && x < width - 1 && y > 0 && y < height - 1) {
+        const int32_t idx = y * width + x;
+        const double up = input[(y - 1) * width + x];
+        const double down = input[(y + 1) * width + x];
+        const double left = input[y * width + x - 1];
+        const double right = input[y * width + x + 1];
+        const double center = input[idx];
+        output[idx] = (float)((up + down + left + right + center) / 5.0);
+      }
+    }
+}
+
+/* benchmarks/bench_conv2d.ml:49-77, thread by thread of a 1-D launch: tid < width * height owns cell
+ * x = tid mod width, y = tid / width; a border cell becomes 0, any other the nine cells round it added
+ * p00 + p01 + ... + p22 (rows top to bottom, left to right) in double, divided by 9.0, rounded once.   */
+void oracle_conv2d_f32(const float *input, float *output, int32_t width, int32_t height, int64_t threads) {
+  const int32_t n = width * height;
+  for (int64_t t = 0; t < threads; ++t) {
+    const int32_t tid = (int32_t)t;
+    if (tid < n) {
+      const int32_t x = tid % width, y = tid / width;
+      if (x == 0 || x == width - 1 || y == 0 || y == height - 1) {
+        output[tid] = 0.0f;
+      } else {
+        const double p00 = input[(y - 1) * width + x - 1], p01 = input[(y - 1) * width + x];
+        const double p02 = input[(y - 1) * width + x + 1];
+        const double p10 = input[y * width + x - 1], p11 = input[y * width + x], p12 = input[y * width + x + 1];
+        const double p20 = input[(y + 1) * width + x - 1], p21 = input[(y + 1) * width + x];
+        const double p22 = input[(y + 1) * width + x + 1];
+        const double sum = p00 + p01 + p02 + p10 + p11 + p12 + p20 + p21 + p22;
+        output[tid] = (float)(sum / 9.0);
+      }
+    }
+  }
+}
+
 int oracle_abi_version(void) { return 1; }

@@ -645,6 +645,48 @@ const char *kRadixScatter = R"IR(
  (native_fn true))
 )IR";
 
+// The five-point mean of benchmarks/bench_stencil_2d.ml:43-58 and the 3 x 3 box filter of
+// benchmarks/bench_conv2d.ml:49-77.
+const char *kStencil2d = R"IR(
+(kernel sarek_kern
+ (params (param (var input 1 (vec f32))) (param (var output 2 (vec f32))) (param (var width 3 i32)) (param (var height 4 i32)))
+ (locals)
+ (body
+ (let (var x 5 i32) (add (intr (Gpu) thread_idx_x) (mul (intr (Gpu) block_idx_x) (intr (Gpu) block_dim_x)))
+ (let (var y 6 i32) (add (intr (Gpu) thread_idx_y) (mul (intr (Gpu) block_idx_y) (intr (Gpu) block_dim_y)))
+ (if (and (and (and (gt (var x 5 i32) (i32 0)) (lt (var x 5 i32) (sub (var width 3 i32) (i32 1)))) (gt (var y 6 i32) (i32 0))) (lt (var y 6 i32) (sub (var height 4 i32) (i32 1)))) (let (var idx 7 i32) (add (mul (var y 6 i32) (var width 3 i32)) (var x 5 i32))
+ (let (var up 8 f32) (read input (add (mul (sub (var y 6 i32) (i32 1)) (var width 3 i32)) (var x 5 i32)))
+ (let (var down 9 f32) (read input (add (mul (add (var y 6 i32) (i32 1)) (var width 3 i32)) (var x 5 i32)))
+ (let (var left 10 f32) (read input (sub (add (mul (var y 6 i32) (var width 3 i32)) (var x 5 i32)) (i32 1)))
+ (let (var right 11 f32) (read input (add (add (mul (var y 6 i32) (var width 3 i32)) (var x 5 i32)) (i32 1)))
+ (let (var center 12 f32) (read input (var idx 7 i32))
+ (assign (lelem output (var idx 7 i32)) (div (add (add (add (add (var up 8 f32) (var down 9 f32)) (var left 10 f32)) (var right 11 f32)) (var center 12 f32)) (f32 5.0)))))))))))))
+ (native_fn true))
+)IR";
+
+const char *kConv2d = R"IR(
+(kernel sarek_kern
+ (params (param (var input 1 (vec f32))) (param (var output 2 (vec f32))) (param (var width 3 i32)) (param (var height 4 i32)))
+ (locals)
+ (body
+ (let (var tid 5 i32) (intr (Std) global_thread_id)
+ (let (var n 6 i32) (mul (var width 3 i32) (var height 4 i32))
+ (if (lt (var tid 5 i32) (var n 6 i32)) (let (var x 7 i32) (mod (var tid 5 i32) (var width 3 i32))
+ (let (var y 8 i32) (div (var tid 5 i32) (var width 3 i32))
+ (if (or (or (or (eq (var x 7 i32) (i32 0)) (eq (var x 7 i32) (sub (var width 3 i32) (i32 1)))) (eq (var y 8 i32) (i32 0))) (eq (var y 8 i32) (sub (var height 4 i32) (i32 1)))) (assign (lelem output (var tid 5 i32)) (f32 0.0)) (let (var p00 9 f32) (read input (sub (add (mul (sub (var y 8 i32) (i32 1)) (var width 3 i32)) (var x 7 i32)) (i32 1)))
+ (let (var p01 10 f32) (read input (add (mul (sub (var y 8 i32) (i32 1)) (var width 3 i32)) (var x 7 i32)))
+ (let (var p02 11 f32) (read input (add (add (mul (sub (var y 8 i32) (i32 1)) (var width 3 i32)) (var x 7 i32)) (i32 1)))
+ (let (var p10 12 f32) (read input (sub (add (mul (var y 8 i32) (var width 3 i32)) (var x 7 i32)) (i32 1)))
+ (let (var p11 13 f32) (read input (add (mul (var y 8 i32) (var width 3 i32)) (var x 7 i32)))
+ (let (var p12 14 f32) (read input (add (add (mul (var y 8 i32) (var width 3 i32)) (var x 7 i32)) (i32 1)))
+ (let (var p20 15 f32) (read input (sub (add (mul (add (var y 8 i32) (i32 1)) (var width 3 i32)) (var x 7 i32)) (i32 1)))
+ (let (var p21 16 f32) (read input (add (mul (add (var y 8 i32) (i32 1)) (var width 3 i32)) (var x 7 i32)))
+ (let (var p22 17 f32) (read input (add (add (mul (add (var y 8 i32) (i32 1)) (var width 3 i32)) (var x 7 i32)) (i32 1)))
+ (let (var sum 18 f32) (add (add (add (add (add (add (add (add (var p00 9 f32) (var p01 10 f32)) (var p02 11 f32)) (var p10 12 f32)) (var p11 13 f32)) (var p12 14 f32)) (var p20 15 f32)) (var p21 16 f32)) (var p22 17 f32))
+ (assign (lelem output (var tid 5 i32)) (div (var sum 18 f32) (f32 9.0))))))))))))))))))))
+ (native_fn true))
+)IR";
+
 const char *kMatmulNaive = R"IR(
 (kernel sarek_kern
  (params (param (var a 1 (vec f32))) (param (var b 2 (vec f32))) (param (var c 3 (vec f32))) (param (var m 4 i32)) (param (var n 5 i32)) (param (var k 6 i32)))
@@ -804,6 +846,8 @@ std::string recognise(const Kernel &k) {
   static const std::string t_hist = strip_trailing_barrier(canon_kernel(parse_kernel(kHistogram)));
   static const std::string t_radix_hist = strip_trailing_barrier(canon_kernel(parse_kernel(kRadixHistogram)));
   static const std::string t_radix_scatter = canon_kernel(parse_kernel(kRadixScatter));
+  static const std::string t_stencil = canon_kernel(parse_kernel(kStencil2d));
+  static const std::string t_conv = canon_kernel(parse_kernel(kConv2d));
   std::string c;
   try {
     c = canon_kernel(k);
@@ -817,6 +861,8 @@ std::string recognise(const Kernel &k) {
   if (c == t_copy) return "vector_copy_f32";
   if (c == t_naive) return "matmul_naive_f32";
   if (c == t_tr_naive) return "transpose_naive_f32";
+  if (c == t_stencil) return "stencil_2d_f32";
+  if (c == t_conv) return "conv2d_f32";
   const std::string cs = strip_trailing_barrier(c);
   if (cs == t_tr_tiled) return "transpose_tiled_f32";
   if (cs == t_hist) return "histogram_i32";

@@ -186,6 +186,31 @@ int try_specialised(const std::string &tag, const int block[3], const int grid[3
                                   (int)w, (int)h, nullptr);
     return 1;
   }
+  if (tag == "stencil_2d_f32" || tag == "conv2d_f32") {
+    // (input, len, output, len, width, height).  The stencil's threads are the cells of a 2-D launch, the
+    // filter's the cells in row-major order of a 1-D one; a launch that does not reach every cell computes
+    // only those it reaches and is left to the generated code, like grids that overlap (cells read their
+    // neighbours).
+    if (n_args != 6 || !vec_at(args, n_args, 0) || !vec_at(args, n_args, 2) || !is_i32(args[4]) ||
+        !is_i32(args[5]))
+      return 0;
+    const int64_t w = args[4].i32, h = args[5].i32;
+    if (w <= 0 || h <= 0 || w * h > 0x7FFFFFFF) return 0;
+    const bool stencil = tag[0] == 's';
+    if (stencil) {
+      if (block[2] != 1 || grid[2] != 1) return 0;
+      if (static_cast<int64_t>(block[0]) * grid[0] < w || static_cast<int64_t>(block[1]) * grid[1] < h) return 0;
+    } else if (!covers_1d(block, grid, w * h)) {
+      return 0;
+    }
+    if (args[0].length < w * h || args[2].length < w * h) return 0;
+    if (ranges_meet(args[0].buffer, w * h * 4, args[2].buffer, w * h * 4)) return 0;
+    const float *in = static_cast<const float *>(args[0].buffer);
+    float *out = static_cast<float *>(args[2].buffer);
+    *rc = stencil ? sarek_hip_stencil_2d_f32(in, out, (int)w, (int)h, nullptr)
+                  : sarek_hip_conv2d_f32(in, out, (int)w, (int)h, nullptr);
+    return 1;
+  }
   if (tag == "histogram_i32" || tag == "radix_histogram_i32") {
     // (input, len, histogram, len, n, num_bins) or (input, len, histogram, len, n, shift, mask).  Each block
     // clears and merges the bins below its own size, so a block at least as wide as the bin range makes the

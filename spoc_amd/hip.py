@@ -132,6 +132,8 @@ SYMBOLS = {
     "sarek_hip_fold_partials_f64": (_i, [_vp, _i64, _vp, _vp]),
     "sarek_hip_copy_f32": (_i, [_vp, _vp, _i64, _vp]),
     "sarek_hip_transpose_f32": (_i, [_vp, _vp, _i, _i, _vp]),
+    "sarek_hip_stencil_2d_f32": (_i, [_vp, _vp, _i, _i, _vp]),
+    "sarek_hip_conv2d_f32": (_i, [_vp, _vp, _i, _i, _vp]),
     "sarek_hip_histogram_i32": (_i, [_vp, _vp, _i64, _i, _vp]),
     "sarek_hip_radix_histogram_i32": (_i, [_vp, _vp, _i64, _i, _i, _vp]),
     "sarek_hip_radix_scatter_i32": (_i, [_vp, _i64, _vp, _vp, _i64, _i, _i, _vp]),
@@ -531,6 +533,32 @@ def transpose(x, out=None):
     if out.numel() != x.numel():
         raise ValueError("transpose: out has the wrong size")
     check(lib.sarek_hip_transpose_f32(_ptr(x), _ptr(out), w, h, _stream()))
+    return out
+
+
+def stencil_2d(x, out):
+    """x, out: [height, width] row-major; the interior of out becomes the five-point mean of x
+    (bench_stencil_2d's kernel over the whole grid), its border keeps what it holds."""
+    torch = _torch()
+    _need(x, torch.float32, "x")
+    _need(out, torch.float32, "out")
+    h, w = x.shape
+    if out.numel() != x.numel():
+        raise ValueError("stencil_2d: out has the wrong size")
+    check(lib.sarek_hip_stencil_2d_f32(_ptr(x), _ptr(out), w, h, _stream()))
+    return out
+
+
+def conv2d(x, out=None):
+    """x: [height, width] row-major -> its 3 x 3 box filter, 0 on the border (bench_conv2d's kernel)."""
+    torch = _torch()
+    _need(x, torch.float32, "x")
+    h, w = x.shape
+    out = torch.empty_like(x) if out is None else out
+    _need(out, torch.float32, "out")
+    if out.numel() != x.numel():
+        raise ValueError("conv2d: out has the wrong size")
+    check(lib.sarek_hip_conv2d_f32(_ptr(x), _ptr(out), w, h, _stream()))
     return out
 
 

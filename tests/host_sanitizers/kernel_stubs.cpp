@@ -11,6 +11,8 @@ int sarek_hip_radix_scatter_i32(int32_t *, int64_t, int32_t *, const int32_t *, 
 int sarek_hip_reduce_max_block256_f32(const float *, float *, int64_t, float, sarek_hip_stream) { return -1; }
 int sarek_hip_reduce_sum_block256_f32(const float *, float *, int64_t, sarek_hip_stream) { return -1; }
 int sarek_hip_transpose_f32(const float *, float *, int, int, sarek_hip_stream) { return -1; }
+int sarek_hip_stencil_2d_f32(const float *, float *, int, int, sarek_hip_stream) { return -1; }
+int sarek_hip_conv2d_f32(const float *, float *, int, int, sarek_hip_stream) { return -1; }
 int sarek_hip_triad_f32(float *, const float *, const float *, float, int64_t, sarek_hip_stream) { return -1; }
 int sarek_hip_triad_block256_sum_f32(float *, const float *, const float *, float, int64_t, float *, sarek_hip_stream) { return -1; }
 int sarek_hip_triad_block256_max_f32(float *, const float *, const float *, float, int64_t, float, float *, sarek_hip_stream) { return -1; }

@@ -1,9 +1,10 @@
-"""The rest of the reference's benchmark suite through the plugin's JIT path
+"""The rest of the reference's benchmark suite through the plugin
 (benchmarks/bench_gather_scatter.ml, bench_histogram.ml, bench_stencil_2d.ml, bench_conv2d.ml,
 bench_mandelbrot.ml, bench_nbody.ml, bench_bitonic_sort.ml, bench_radix_sort.ml): each mirror
 builds the reference's inputs, launches with its geometry and applies its own check, so a
 passing run says the lowering computes what the bench expects at sizes with ragged last blocks,
-colliding scatters, atomics in shared and global memory, records and helper functions."""
+colliding scatters, atomics in shared and global memory, records and helper functions; the stencil
+and the box filter run both ways, hand kernel and generated code."""
 import numpy as np
 import pytest
 
@@ -18,7 +19,15 @@ def test_suite_runs_and_verifies(hip, torch_cuda, name, size):
     from spoc_amd import benchmarks
     rec = benchmarks.BENCHMARKS[name][0](size, warmup=1, iterations=3)
     assert rec["verified"], rec
-    assert rec["path"] == "jit" and len(rec["iterations"]) == 3 and rec["throughput_gflops"] > 0
+    hand = {"stencil_2d": "stencil_2d_f32", "conv2d": "conv2d_f32"}
+    assert rec["path"] == hand.get(name, "jit") and len(rec["iterations"]) == 3 and rec["throughput_gflops"] > 0
+    if name in hand:
+        hip.check(hip.lib.sarek_hip_set_specialisation(0))
+        try:
+            rec = benchmarks.BENCHMARKS[name][0](size, warmup=1, iterations=2)
+        finally:
+            hip.check(hip.lib.sarek_hip_set_specialisation(1))
+        assert rec["verified"] and rec["path"] == "jit"
 
 
 def test_suite_is_the_reference_suite():

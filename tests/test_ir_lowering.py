@@ -485,3 +485,21 @@ def test_recognition_does_not_depend_on_how_index_arithmetic_is_written(hip):
     # the tree's partner index tid + 64 written as 64 + tid
     assert tag(red.replace("(add (var tid 5 i32) (i32 64))", "(add (i32 64) (var tid 5 i32))")) == "reduce_sum_block256_f32"
     assert tag(red.replace("(add (var tid 5 i32) (i32 64))", "(add (i32 63) (var tid 5 i32))")) == ""
+
+
+def test_stencil_and_box_filter_are_recognised_and_near_misses_are_not(hip):
+    """A stencil with another divisor, or neighbours added in another association, is another program."""
+    from spoc_amd import reference_kernels
+    st, cv = reference_kernels.stencil_2d(), reference_kernels.conv2d()
+    mark = "// sarek-hip-specialise: "
+    assert hip.generate_source(st).startswith(mark + "stencil_2d_f32")
+    assert hip.generate_source(cv).startswith(mark + "conv2d_f32")
+    for text, old, new in [(st, "(f32 5.0)", "(f32 4.0)"), (cv, "(f32 9.0)", "(f32 8.0)"),
+                           # (a + b is b + a bit for bit; (a + b) + c is not a + (b + c))
+                           (st, "(add (add (var up 8 f32) (var down 9 f32)) (var left 10 f32))",
+                            "(add (var up 8 f32) (add (var down 9 f32) (var left 10 f32)))"),
+                           (st, "(var left 10 f32)) (var right 11 f32)) (var center 12 f32))",
+                            "(var center 12 f32)) (var right 11 f32)) (var left 10 f32))"),
+                           (cv, "(eq (var y 8 i32) (i32 0))", "(eq (var y 8 i32) (i32 1))")]:
+        assert old in text
+        assert not hip.generate_source(text.replace(old, new)).startswith(mark)

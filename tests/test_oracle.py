@@ -355,6 +355,105 @@ def test_naive_matmul_is_the_same_sum_as_the_tiled_kernel(oracle):
     assert np.array_equal(part[:n + 3], c_full := oracle.matmul_naive(a, b, m, n, k)[:n + 3]) and np.all(part[n + 3:] == -1)
 
 
+# ---- the 2-D neighbourhood kernels -------------------------------------------------------------------
+#   benchmarks/bench_stencil_2d.ml:39-51,88-93,158-164 (sin(0.1 x) cos(0.1 y), cpu_stencil_2d, 1e-4)
+#   benchmarks/bench_conv2d.ml:40-60,103-111,179-185 (((x + y) mod 256) / 255, cpu_conv2d with nine 1/9 taps, 1e-3)
+
+def _grid(w, h, f):
+    y, x = np.mgrid[0:h, 0:w]
+    return f(x.astype(np.float64), y.astype(np.float64))
+
+
+def test_stencil_2d_reference_inputs_closed_forms_and_order(oracle):
+    w, h = 37, 29                                                    # a wrong pitch fails on a rectangle
+    data = _grid(w, h, lambda x, y: np.sin(x * 0.1) * np.cos(y * 0.1))
+    out = oracle.stencil_2d(data.reshape(-1), w, h, out=np.full(w * h, -7.0, dtype=np.float32)).reshape(h, w)
+    expected = np.zeros((h, w))
+    for y in range(1, h - 1):                                        # cpu_stencil_2d of the bench
+        for x in range(1, w - 1):
+            expected[y, x] = (data[y - 1, x] + data[y + 1, x] + data[y, x - 1] + data[y, x + 1] + data[y, x]) / 5.0
+    assert np.all(np.abs(out[1:-1, 1:-1] - expected[1:-1, 1:-1]) <= 1e-4)
+    border = np.ones((h, w), dtype=bool)
+    border[1:-1, 1:-1] = False
+    assert np.all(out[border] == -7.0)                               # boundaries unchanged
+    # closed forms on small integers (every step exact): a constant and a plane are fixed points; x^2 gains 2/5 (a
+    # dropped or doubled horizontal neighbour shows), y^2 likewise, x y is a fixed point only with the right pitch
+    for f, g in [(lambda x, y: 0 * x + 3, lambda x, y: 0 * x + 3), (lambda x, y: 3 * x + 7 * y, lambda x, y: 3 * x + 7 * y),
+                 (lambda x, y: x * x, lambda x, y: x * x + 0.4), (lambda x, y: y * y, lambda x, y: y * y + 0.4),
+                 (lambda x, y: x * y, lambda x, y: x * y), (lambda x, y: x * x * y, lambda x, y: x * x * y + 0.4 * y)]:
+        got = oracle.stencil_2d(_grid(w, h, f).reshape(-1), w, h).reshape(h, w)
+        assert np.array_equal(got[1:-1, 1:-1], _grid(w, h, g).astype(np.float32)[1:-1, 1:-1])
+    # the sum runs up, down, left, right, center in double: 2^60 + 1 + 1 + 1 - 2^60 loses the ones, 2^60 - 2^60 first keeps them
+    cell = np.zeros((3, 3), dtype=np.float32)
+    cell[0, 1], cell[2, 1], cell[1, 0], cell[1, 2], cell[1, 1] = 2.0 ** 60, 1, 1, 1, -2.0 ** 60
+    assert oracle.stencil_2d(cell.reshape(-1), 3, 3)[4] == 0.0
+    cell[0, 1], cell[2, 1], cell[1, 0], cell[1, 2], cell[1, 1] = 2.0 ** 60, -2.0 ** 60, 1, 1, 1
+    assert oracle.stencil_2d(cell.reshape(-1), 3, 3)[4] == np.float32(0.6)
+    # one rounding: the double quotient, not a quotient of float32 partial sums
+    rng = np.random.default_rng(11)
+    x = rng.standard_normal((h, w)).astype(np.float32)
+    x64 = x.astype(np.float64)
+    exact = ((((x64[:-2, 1:-1] + x64[2:, 1:-1]) + x64[1:-1, :-2]) + x64[1:-1, 2:]) + x64[1:-1, 1:-1]) / 5.0
+    assert np.array_equal(oracle.stencil_2d(x.reshape(-1), w, h).reshape(h, w)[1:-1, 1:-1], exact.astype(np.float32))
+    # a launch that reaches 10 x 6 threads computes the interior cells among them and nothing else
+    part = oracle.stencil_2d(x.reshape(-1), w, h, out=np.full(w * h, -7.0, dtype=np.float32), threads_xy=(10, 6)).reshape(h, w)
+    assert np.array_equal(part[1:6, 1:10], exact.astype(np.float32)[:5, :9])
+    part[1:6, 1:10] = -7.0
+    assert np.all(part == -7.0)
+    # grids without an interior write nothing
+    for ww, hh in [(1, 1), (2, 5), (5, 2), (1, 9)]:
+        assert np.all(oracle.stencil_2d(np.ones(ww * hh), ww, hh, out=np.full(ww * hh, -7.0, dtype=np.float32)) == -7.0)
+
+
+def test_conv2d_reference_inputs_closed_forms_and_order(oracle):
+    w, h = 41, 23
+    data = _grid(w, h, lambda x, y: ((x + y) % 256) / 255.0)
+    out = oracle.conv2d(data.reshape(-1), w, h, out=np.full(w * h, -7.0, dtype=np.float32)).reshape(h, w)
+    taps = [1.0 / 9.0] * 9
+    expected = np.zeros((h, w))
+    for y in range(1, h - 1):                                        # cpu_conv2d of the bench
+        for x in range(1, w - 1):
+            acc = 0.0
+            for ky in range(3):
+                for kx in range(3):
+                    acc = acc + data[y + ky - 1, x + kx - 1] * taps[ky * 3 + kx]
+            expected[y, x] = acc
+    assert np.all(np.abs(out - expected) <= 1e-3)                    # boundaries are 0 in both
+    assert np.all(out[0] == 0) and np.all(out[-1] == 0) and np.all(out[:, 0] == 0) and np.all(out[:, -1] == 0)
+    for f, g in [(lambda x, y: 0 * x + 3, lambda x, y: 0 * x + 3), (lambda x, y: 3 * x + 7 * y, lambda x, y: 3 * x + 7 * y),
+                 (lambda x, y: x * y, lambda x, y: x * y)]:
+        got = oracle.conv2d(_grid(w, h, f).reshape(-1), w, h).reshape(h, w)
+        assert np.array_equal(got[1:-1, 1:-1], _grid(w, h, g).astype(np.float32)[1:-1, 1:-1])
+    for f, extra in [(lambda x, y: x * x, 6.0), (lambda x, y: y * y, 6.0)]:     # (9 v + 6) / 9, rounded once
+        got = oracle.conv2d(_grid(w, h, f).reshape(-1), w, h).reshape(h, w)
+        assert np.array_equal(got[1:-1, 1:-1], ((9.0 * _grid(w, h, f) + extra) / 9.0).astype(np.float32)[1:-1, 1:-1])
+    # p00 first, p22 last: 2^60 + seven ones - 2^60 is 0 in that order and 7/9 when the two large cells meet first
+    cell = np.ones((3, 3), dtype=np.float32)
+    cell[0, 0], cell[2, 2] = 2.0 ** 60, -2.0 ** 60
+    big = np.zeros((5, 5), dtype=np.float32)
+    big[1:4, 1:4] = cell
+    assert oracle.conv2d(big.reshape(-1), 5, 5)[12] == 0.0
+    big[1, 1], big[1, 2] = 2.0 ** 60, -2.0 ** 60
+    big[3, 3] = 1.0
+    assert oracle.conv2d(big.reshape(-1), 5, 5)[12] == np.float32(7.0 / 9.0)
+    # row-major taps: a single 1 at (y, x) reaches the nine cells round it and no others
+    one = np.zeros((7, 9), dtype=np.float32)
+    one[2, 5] = 9.0
+    got = oracle.conv2d(one.reshape(-1), 9, 7).reshape(7, 9)
+    want = np.zeros((7, 9), dtype=np.float32)
+    want[1:4, 4:7] = 1.0
+    assert np.array_equal(got, want)
+    # tid < n, x = tid mod width, y = tid / width: a short launch fills the first cells in row-major order
+    rng = np.random.default_rng(12)
+    x = rng.standard_normal((h, w)).astype(np.float32)
+    full = oracle.conv2d(x.reshape(-1), w, h)
+    part = oracle.conv2d(x.reshape(-1), w, h, out=np.full(w * h, -7.0, dtype=np.float32), threads=3 * w + 5)
+    assert np.array_equal(part[:3 * w + 5], full[:3 * w + 5]) and np.all(part[3 * w + 5:] == -7.0)
+    # grids that are all border
+    for ww, hh in [(1, 1), (2, 5), (5, 2), (1, 9)]:
+        assert np.all(oracle.conv2d(np.ones(ww * hh), ww, hh, out=np.full(ww * hh, -7.0, dtype=np.float32)) == 0.0)
+
+
 # ---- histograms (benchmarks/bench_histogram.ml, bench_radix_sort.ml) -------------------------------
 
 @pytest.mark.parametrize("n,bins,block", [(0, 256, 256), (1, 256, 256), (1000, 256, 256), (100003, 256, 256),
