@@ -86,8 +86,10 @@ __device__ __forceinline__ void tile_of(int order, int tiles_c, int tiles_r, int
 // 64 x 64 tile through LDS: 16 lanes read 256 contiguous bytes of an input row, the tile is
 // kept with a row pitch of 65 words (both the row-wise stores and the column-wise loads then
 // touch 64 different banks per wave), and 16 lanes write 256 contiguous bytes of an output
-// row.  Needs width % 4 == height % 4 == 0 (the matrices themselves may start on any 4-byte boundary).
-template <int TR, bool NtLoad, bool NtStore>
+// row.  The matrices may start on any 4-byte boundary.  Ragged: width or height is not a multiple of 4, so rows start
+// at any 4-byte offset too (the 128-bit accesses do not mind) and the pieces that straddle the end of a row go
+// element by element.
+template <int TR, bool NtLoad, bool NtStore, bool Ragged>
 __global__ __launch_bounds__(kBlock) void transpose_lds_kernel(const float *__restrict__ in,
                                                                float *__restrict__ out, int width, int height,
                                                                int tiles_c, int tiles_r, int order) {
@@ -102,8 +104,18 @@ __global__ __launch_bounds__(kBlock) void transpose_lds_kernel(const float *__re
   for (int i = 0; i < NL; ++i) {
     const int64_t r = r0 + p + 16 * i, c = c0 + 4 * q;
     const float *src = in + r * width + c;
-    v[i] = (r < height && c < width) ? (NtLoad ? ldg_nt(src) : *reinterpret_cast<const f32x4_t *>(src))
-                                     : f32x4_t{0.f, 0.f, 0.f, 0.f};
+    if (r < height && (Ragged ? c + 3 < width : c < width)) {
+      v[i] = NtLoad ? ldg_nt(src) : *reinterpret_cast<const f32x4_t *>(src);
+    } else {
+      v[i] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+      if constexpr (Ragged) {
+        if (r < height) {
+#pragma unroll
+          for (int j = 0; j < 3; ++j)
+            if (c + j < width) v[i][j] = src[j];
+        }
+      }
+    }
   }
 #pragma unroll
   for (int i = 0; i < NL; ++i)
@@ -120,8 +132,15 @@ __global__ __launch_bounds__(kBlock) void transpose_lds_kernel(const float *__re
     if (orow < width && ocol < height) {
       const f32x4_t w = {tile[4 * oq][oc], tile[4 * oq + 1][oc], tile[4 * oq + 2][oc], tile[4 * oq + 3][oc]};
       float *dst = out + orow * height + ocol;
-      if (NtStore) stg_nt(dst, w);
-      else *reinterpret_cast<f32x4_t *>(dst) = w;
+      if (Ragged && ocol + 3 >= height) {
+#pragma unroll
+        for (int j = 0; j < 3; ++j)
+          if (ocol + j < height) dst[j] = w[j];
+      } else if (NtStore) {
+        stg_nt(dst, w);
+      } else {
+        *reinterpret_cast<f32x4_t *>(dst) = w;
+      }
     }
   }
 }
@@ -208,25 +227,35 @@ int sarek_hip_transpose_f32(const float *in, float *out, int width, int height, 
   if (!in || !out) return fail(SAREK_HIP_E_INVALID_ARG, "transpose: NULL matrix");
   if (in == out) return fail(SAREK_HIP_E_INVALID_ARG, "transpose: in-place transposition is not supported");
   hipStream_t st = as_stream(stream);
-  if (width % 4 == 0 && height % 4 == 0 && tunable("transpose.force_scalar", 0) == 0) {
+  if (tunable("transpose.force_scalar", 0) == 0) {
+    const bool ragged = width % 4 != 0 || height % 4 != 0;
     // Measured on MI355X: 128-row tiles; an input that fits the last-level cache is best read
     // with plain loads and with each XCD walking its own run of tiles (order 3), a larger one
-    // with non-temporal loads and neighbouring workgroups writing neighbouring pieces (order 1).
+    // with non-temporal loads and neighbouring workgroups writing neighbouring pieces (order 1); a larger one whose
+    // rows start off 16 bytes (ragged) with plain accesses and order 3 (4.2 against 3.3-3.6 TB/s at 16383 x 16385 and
+    // 12001 x 20003).
     const bool cached = static_cast<int64_t>(width) * height * 4 <= kLastLevelCacheBytes;
     const int rows = tunable("transpose.rows", 128) == 64 ? 64 : 128;
     const int tiles_c = (width + kTile - 1) / kTile;
     const int64_t variant = tunable("transpose.variant", 0);
     int64_t nt = tunable("transpose.nt", -1);
-    if (nt < 0) nt = cached ? 2 : 3;
-    const int tiles_r = (height + (variant == 0 ? rows : kTile) - 1) / (variant == 0 ? rows : kTile);
+    if (nt < 0) nt = cached ? 2 : ragged ? 0 : 3;
+    const bool lds = variant == 0 || ragged;   // the register-only kernel takes whole 4 x 4 blocks
+    const int tiles_r = (height + (lds ? rows : kTile) - 1) / (lds ? rows : kTile);
     const int64_t tiles = static_cast<int64_t>(tiles_c) * tiles_r;
     if (tiles > 0x7FFFFFFF) return fail(SAREK_HIP_E_INVALID_ARG, "transpose: matrix too large for one launch");
     int order = static_cast<int>(tunable("transpose.order", -1));
-    if (order < 0) order = cached ? 3 : 1;
-#define SAREK_TRANSPOSE(TR, NL, NS)                                                                       \
-  hipLaunchKernelGGL((transpose_lds_kernel<TR, NL, NS>), dim3(static_cast<unsigned>(tiles)), dim3(kBlock), 0, \
-                     st, in, out, width, height, tiles_c, tiles_r, order)
-    if (variant == 0) {
+    if (order < 0) order = cached || ragged ? 3 : 1;
+#define SAREK_TRANSPOSE(TR, NL, NS)                                                                              \
+  do {                                                                                                             \
+    if (ragged)                                                                                                    \
+      hipLaunchKernelGGL((transpose_lds_kernel<TR, NL, NS, true>), dim3(static_cast<unsigned>(tiles)), dim3(kBlock), \
+                         0, st, in, out, width, height, tiles_c, tiles_r, order);                                  \
+    else                                                                                                           \
+      hipLaunchKernelGGL((transpose_lds_kernel<TR, NL, NS, false>), dim3(static_cast<unsigned>(tiles)),            \
+                         dim3(kBlock), 0, st, in, out, width, height, tiles_c, tiles_r, order);                    \
+  } while (0)
+    if (lds) {
       if (rows == 64) {
         if (nt == 3) SAREK_TRANSPOSE(64, true, true);
         else if (nt == 1) SAREK_TRANSPOSE(64, true, false);

@@ -162,7 +162,8 @@ int launch_neighbourhood(const char *what, const float *in, float *out, int widt
                          sarek_hip_stream stream) {
   if (width < 0 || height < 0) return fail(SAREK_HIP_E_INVALID_ARG, "%s: negative shape %d x %d", what, width, height);
   if (width == 0 || height == 0) return SAREK_HIP_OK;
-  if (static_cast<int64_t>(width) * height > 0x7FFFFFFF)
+  // (a strip may reach 1023 columns past the width: those column numbers must still fit an int)
+  if (static_cast<int64_t>(width) * height > 0x7FFFFFFF || width > 0x7FFFFFFF - 1024)
     return fail(SAREK_HIP_E_INVALID_ARG, "%s: %d x %d cells exceed the kernel's int32 indices", what, width, height);
   if (!in || !out) return fail(SAREK_HIP_E_INVALID_ARG, "%s: NULL grid", what);
   const uintptr_t pi = reinterpret_cast<uintptr_t>(in), po = reinterpret_cast<uintptr_t>(out);

@@ -114,6 +114,31 @@ def test_transpose_every_variant(hip, torch_cuda):
     assert hip.lib.sarek_hip_transpose_f32(flat.data_ptr(), out.data_ptr(), 0, 8, None) == 0
 
 
+@pytest.mark.parametrize("h,w", [(519, 1031), (130, 66), (5, 3), (1, 7), (257, 1), (1030, 516), (2, 1029)])
+def test_ragged_transposes_every_policy_and_guards(hip, torch_cuda, h, w):
+    """Widths and heights that are not multiples of 4 run the tiled kernel too (rows then start at any 4-byte offset,
+    the pieces across a row's end go element by element): every tile height, order and cache policy, with guard
+    elements round the output, and the element-per-access kernel behind its knob."""
+    torch = torch_cuda
+    flat = torch.rand(h * w + 3, device="cuda")
+    x = flat[3:].view(h, w)
+    try:
+        for rows, order, nt, scalar in [(r, o, t, 0) for r in (64, 128) for o in (0, 1, 2, 3) for t in (0, 1, 2, 3)] + \
+                                       [(128, -1, -1, 0), (128, -1, -1, 1)]:
+            for name, v in (("rows", rows), ("order", order), ("nt", nt), ("force_scalar", scalar)):
+                hip.set_tunable("transpose." + name, v)
+            out = torch.full((h * w + 9,), -1.0, device="cuda")
+            hip.check(hip.lib.sarek_hip_transpose_f32(x.data_ptr(), out[5:].data_ptr(), w, h, None))
+            torch.cuda.synchronize()
+            assert torch.equal(out[5:5 + h * w].view(w, h), x.t()), (rows, order, nt, scalar)
+            assert bool((out[:5] == -1).all()) and bool((out[5 + h * w:] == -1).all()), (rows, order, nt, scalar)
+    finally:
+        hip.set_tunable("transpose.rows", 128)
+        hip.set_tunable("transpose.order", -1)
+        hip.set_tunable("transpose.nt", -1)
+        hip.set_tunable("transpose.force_scalar", 0)
+
+
 # ---- the reference kernels' IR, hand kernel and JIT lowering side by side ------------------------
 
 @pytest.mark.parametrize("specialise", [1, 0])
