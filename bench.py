@@ -60,7 +60,7 @@ def parse():
                     choices=["gemm_bf16_8192", "gemm_f16_8192", "triad_sum_2p28", "gemm_f32_8192", "gemm_f32_1024",
                              "gemm_f16_epilogue", "gemm_f16_4095x11008x4096", "gemm_f16_shape", "gemm_bf16_shape", "gemm_bf16_2048", "gemm_f32_shape", "vendor_gemm_f32_shape", "copy_1gib",
                              "vendor_gemm_bf16_8192", "vendor_gemm_bf16_shape", "histogram_2p28",
-                             "radix_scatter_5e7", "stencil_2d_shape", "conv2d_shape", "mfma_bf16_stream", "mfma_bf16_stream_32x32x16",
+                             "radix_scatter_5e7", "stencil_2d_shape", "conv2d_shape", "map_sum_2p28", "mfma_bf16_stream", "mfma_bf16_stream_32x32x16",
                              "l2_to_lds_stream"])
     ap.add_argument("--warmup-ms", type=float, default=60.0,
                     help="warm up for at least this long (and at least --warmup steps): the clocks of a power-limited "
@@ -182,6 +182,37 @@ def make_workload(name, torch, hip):
                     config={"workload": "fused stream triad + sum, a=b+3c, sum(a)", "n": n,
                             "algorithmic_bytes": 12 * n})
         return main, tail, info, (va, vb, vc, vout, total, a0, a1, ir0, ir1, stages)
+    if name == "map_sum_2p28":
+        # an element-wise kernel that is not one of the reference's benches (a = b - s * c), then the block-256 sum
+        # of its output: recognised as a map, rebuilt from its own expression and fused with the sum
+        n = 1 << 28
+        g.manual_seed(0xB)
+        b = torch.rand(n, device="cuda", generator=g)
+        vb = device_vector(sarek, hip, torch, b, V.float32)
+        g.manual_seed(0xC)
+        b.uniform_(0, 1, generator=g)
+        vc = device_vector(sarek, hip, torch, b, V.float32)
+        del b
+        va, vout = V.create(V.float32, n), V.create(V.float32, n // 256)
+        sarek.Transfer.to_device(va)
+        sarek.Transfer.to_device(vout)
+        a0, n0 = E._args([E.Vec(va), E.Vec(vb), E.Vec(vc), E.Float32(3.0), E.Int32(n)])
+        a1, n1 = E._args([E.Vec(va), E.Vec(vout), E.Int32(n)])
+        ir0 = rk.stream_triad().replace("(add (read b", "(sub (read b").encode()
+        ir1 = rk.tree(False).encode()
+        stages = (hip.PipelineStage * 2)()
+        stages[0].ir_text, stages[0].block, stages[0].grid, stages[0].args, stages[0].n_args = \
+            ir0, dims(256, 1, 1), dims(n // 256, 1, 1), a0, n0
+        stages[1].ir_text, stages[1].block, stages[1].grid, stages[1].args, stages[1].n_args = \
+            ir1, dims(256, 1, 1), dims(n // 256, 1, 1), a1, n1
+        main = Launch(hip, lib.sarek_hip_execute_run_pipeline, stages, 2, None)
+        info = dict(metric="element-wise map + block-256 sum GB/s", unit="GB/s", dtype="f32",
+                    work=12.0 * n, work_unit=1e9, bound="hbm", peak=PEAK_HBM_GBS,
+                    kernel="sarek_map (the map's own expression in the stream kernels' shape, compiled at run time)",
+                    route="Execute.run_pipeline [a = b - s c IR; block-256 reduction IR]",
+                    config={"workload": "a = b - 3c, then the block-256 sums of a", "n": n,
+                            "algorithmic_bytes": 12 * n})
+        return main, None, info, (va, vb, vc, vout, a0, a1, ir0, ir1, stages)
     if name in ("gemm_f32_8192", "gemm_f32_1024"):
         s = 8192 if name.endswith("8192") else 1024
         g.manual_seed(0xA11CE)
@@ -829,7 +860,7 @@ def main():
     if args.trace_launches:
         out["kernel_us_by_launch"] = head["kernel_us_by_launch"]
     if not args.no_cpu_baseline and args.workload not in ("copy_1gib", "vendor_gemm_bf16_8192", "vendor_gemm_bf16_shape", "gemm_bf16_shape", "gemm_f16_shape", "gemm_f32_shape", "vendor_gemm_f32_shape", "mfma_bf16_stream", "mfma_bf16_stream_32x32x16", "l2_to_lds_stream",
-                                                        "stencil_2d_shape", "conv2d_shape"):
+                                                        "stencil_2d_shape", "conv2d_shape", "map_sum_2p28"):
         out["cpu_baseline"] = cpu_baseline(args.workload)
     if not args.no_also:
         also = []

@@ -5,10 +5,12 @@
 #include <mutex>
 #include <string>
 #include <string_view>
+#include <unordered_map>
 #include <unordered_set>
 
 #include "common.hpp"
 #include "host/ir.hpp"
+#include "host/map_fuse.hpp"
 #include "plugin.hpp"
 
 namespace sarek_hip {
@@ -23,7 +25,17 @@ struct ViewHash {
 std::mutex g_tagged_mu;
 std::unordered_set<std::string, ViewHash, std::equal_to<>> g_tagged;
 constexpr size_t kTaggedMax = 4096;     // beyond this the set starts over: forgotten texts run as compiled
+// The element-wise kernels among them (tag map_f32), by their text: what run_source needs to rebuild them
+std::unordered_map<std::string, ir::MapKernel, ViewHash, std::equal_to<>> g_maps;
 }  // namespace
+
+bool find_generated_map(const char *source, ir::MapKernel *out) {
+  std::lock_guard<std::mutex> lock(g_tagged_mu);
+  const auto it = g_maps.find(std::string_view(source));
+  if (it == g_maps.end()) return false;
+  if (out) *out = it->second;
+  return true;
+}
 
 bool is_generated_tagged_text(const char *source) {
   std::lock_guard<std::mutex> lock(g_tagged_mu);
@@ -37,9 +49,11 @@ extern "C" int sarek_hip_generate_source(const char *ir_text, const int block[3]
                                          size_t out_len, size_t *needed) {
   if (!ir_text) return fail(SAREK_HIP_E_INVALID_ARG, "generate_source: NULL IR text");
   std::string src, tag;
+  std::optional<ir::MapKernel> map;
   try {
     ir::Kernel k = ir::parse_kernel(ir_text);
     tag = ir::recognise(k);
+    if (tag.empty() && (map = ir::match_map(k))) tag = "map_f32";
     if (!tag.empty()) src = std::string(kSpecialiseMarker) + tag + "\n";
     src += ir::generate(k, block);
   } catch (const ir::ParseError &e) {
@@ -55,7 +69,11 @@ extern "C" int sarek_hip_generate_source(const char *ir_text, const int block[3]
   std::memcpy(out, src.c_str(), src.size() + 1);
   if (!tag.empty()) {
     std::lock_guard<std::mutex> lock(g_tagged_mu);
-    if (g_tagged.size() >= kTaggedMax) g_tagged.clear();
+    if (g_tagged.size() >= kTaggedMax) {
+      g_tagged.clear();
+      g_maps.clear();
+    }
+    if (map) g_maps.emplace(src, std::move(*map));
     g_tagged.insert(std::move(src));
   }
   return SAREK_HIP_OK;

@@ -1,0 +1,314 @@
+// Element-wise kernels as a class: `if tid < n then out[tid] <- f(in_1[tid], ..., in_k[tid], scalars, tid)`, the shape
+// of the reference's vector add, stream triad and saxpy kernels (benchmarks/bench_vector_add.ml:53-61,
+// bench_stream_triad.ml:22-32) and of any map a user writes.  The generated kernel for such an IR moves one element per
+// thread; what is built here from the same IR is the stream kernels' shape instead -- four 128-bit loads per input in
+// flight per thread, non-temporal stores, a wave owning four consecutive KiB -- with the kernel's own expression, as
+// the lowering prints it, applied to every element, and optionally the block-256 sums of the result (the reference's
+// tree kernel, benchmarks/bench_reduction.ml:62-96, one wave reduction per 256 elements) in the same pass.
+#include <algorithm>
+#include <optional>
+#include <string>
+#include <vector>
+
+#include "ir.hpp"
+#include "map_fuse.hpp"
+
+namespace sarek_hip {
+namespace ir {
+namespace {
+
+bool is_var(const ExprP &e, const std::string &name) { return e && e->kind == Expr::VarRef && e->var.name == name; }
+
+bool is_intr(const ExprP &e, const char *name) { return e && e->kind == Expr::Intrinsic && e->name == name; }
+
+// threadIdx.x + blockIdx.x * blockDim.x in any of the orders a kernel text writes it
+bool is_global_id(const ExprP &e) {
+  if (is_intr(e, "global_thread_id") || is_intr(e, "global_idx") || is_intr(e, "global_idx_x")) return true;
+  if (!e || e->kind != Expr::BinopE || e->binop != Binop::Add) return false;
+  for (int t = 0; t < 2; ++t) {
+    const ExprP &tx = e->args[t], &prod = e->args[1 - t];
+    if (!(is_intr(tx, "thread_idx_x") || is_intr(tx, "thread_id_x"))) continue;
+    if (!prod || prod->kind != Expr::BinopE || prod->binop != Binop::Mul) continue;
+    for (int u = 0; u < 2; ++u) {
+      const ExprP &bi = prod->args[u], &bd = prod->args[1 - u];
+      if ((is_intr(bi, "block_idx_x") || is_intr(bi, "block_id_x")) && is_intr(bd, "block_dim_x")) return true;
+    }
+  }
+  return false;
+}
+
+struct Matcher {
+  MapKernel m;
+  std::vector<std::string> bound;   // immutable let variables in scope
+
+  int param_index(const std::string &name) const {
+    for (size_t i = 0; i < m.params.size(); ++i)
+      if (m.params[i].name == name) return static_cast<int>(i);
+    return -1;
+  }
+
+  // An expression whose value depends on nothing but the element's inputs, the scalars and tid
+  bool pure(const ExprP &e) {
+    if (!e) return false;
+    switch (e->kind) {
+      case Expr::ConstInt32: case Expr::ConstInt64: case Expr::ConstFloat32: case Expr::ConstFloat64:
+      case Expr::ConstBool:
+        return true;
+      case Expr::VarRef: {
+        if (e->var.is_mutable) return false;
+        if (e->var.name == m.tid) return true;
+        if (std::find(bound.begin(), bound.end(), e->var.name) != bound.end()) return true;
+        const int p = param_index(e->var.name);
+        return p >= 0 && m.params[p].kind != MapKernel::Param::Vec;
+      }
+      case Expr::BinopE: return e->args.size() == 2 && pure(e->args[0]) && pure(e->args[1]);
+      case Expr::UnopE: return e->args.size() == 1 && pure(e->args[0]);
+      case Expr::If: return e->args.size() == 3 && pure(e->args[0]) && pure(e->args[1]) && pure(e->args[2]);
+      case Expr::Cast:
+        if (!e->type || e->args.size() != 1) return false;
+        if (e->type->kind != Type::Int32 && e->type->kind != Type::Int64 && e->type->kind != Type::Float32 &&
+            e->type->kind != Type::Float64)
+          return false;
+        return pure(e->args[0]);
+      case Expr::ArrayRead: {
+        const int p = param_index(e->name);
+        if (p < 0 || m.params[p].kind != MapKernel::Param::Vec || p == m.out) return false;
+        if (e->args.size() != 1 || !is_var(e->args[0], m.tid)) return false;
+        if (std::find(m.inputs.begin(), m.inputs.end(), p) == m.inputs.end()) m.inputs.push_back(p);
+        return true;
+      }
+      case Expr::Intrinsic: {
+        static const char *math[] = {"sin", "cos", "tan", "asin", "acos", "atan", "sinh", "cosh", "tanh", "exp",
+                                     "exp2", "log", "log2", "log10", "sqrt", "rsqrt", "cbrt", "floor", "ceil",
+                                     "round", "trunc", "fabs", "atan2", "pow", "fma", "min", "max"};
+        if (e->has_templ) return false;
+        bool known = false;
+        for (const char *n : math) known = known || e->name == n;
+        if (!known) return false;
+        for (const auto &a : e->args)
+          if (!pure(a)) return false;
+        return true;
+      }
+      default: return false;
+    }
+  }
+
+  // reads of in[tid] become the element's variable in__e
+  ExprP rewrite(const ExprP &e) {
+    if (e->kind == Expr::ArrayRead) {
+      auto v = std::make_shared<Expr>();
+      v->kind = Expr::VarRef;
+      v->var.name = e->name + "__e";
+      return v;
+    }
+    if (e->args.empty()) return e;
+    auto c = std::make_shared<Expr>(*e);
+    for (auto &a : c->args) a = rewrite(a);
+    return c;
+  }
+
+  // S := let x = E in S | out[tid] <- E, through single-statement blocks and sequences
+  std::optional<StmtP> body(const StmtP &s) {
+    if (!s) return std::nullopt;
+    switch (s->kind) {
+      case Stmt::Block:
+      case Stmt::Seq:
+        if (s->stmts.size() != 1) return std::nullopt;
+        return body(s->stmts[0]);
+      case Stmt::Let: {
+        if (s->var.is_mutable || !s->e || s->e->kind == Expr::ArrayCreate || !pure(s->e)) return std::nullopt;
+        if (s->var.name == m.tid || param_index(s->var.name) >= 0 || s->var.name.compare(0, 8, "sarek_f_") == 0)
+          return std::nullopt;
+        if (s->stmts.size() != 1) return std::nullopt;
+        bound.push_back(s->var.name);
+        auto inner = body(s->stmts[0]);
+        bound.pop_back();
+        if (!inner) return std::nullopt;
+        auto c = std::make_shared<Stmt>(*s);
+        c->e = rewrite(s->e);
+        c->stmts[0] = *inner;
+        return StmtP(c);
+      }
+      case Stmt::Assign: {
+        if (!s->lhs || s->lhs->kind != LValue::LArrayElem || param_index(s->lhs->name) != m.out) return std::nullopt;
+        if (!is_var(s->lhs->index, m.tid) || !pure(s->e)) return std::nullopt;
+        auto lhs = std::make_shared<LValue>();
+        lhs->kind = LValue::LVar;
+        lhs->var.name = "sarek_f_res";
+        auto c = std::make_shared<Stmt>(*s);
+        c->lhs = lhs;
+        c->e = rewrite(s->e);
+        return StmtP(c);
+      }
+      default: return std::nullopt;
+    }
+  }
+};
+
+// the first assignment target under the lets: names the output vector before the purity walk needs it
+const Stmt *find_assign(const StmtP &s) {
+  const Stmt *p = s.get();
+  while (p) {
+    if (p->kind == Stmt::Assign) return p;
+    if ((p->kind == Stmt::Block || p->kind == Stmt::Seq || p->kind == Stmt::Let) && p->stmts.size() == 1)
+      p = p->stmts[0].get();
+    else
+      return nullptr;
+  }
+  return nullptr;
+}
+
+}  // namespace
+
+std::optional<MapKernel> match_map(const Kernel &k) {
+  if (!k.funcs.empty() || !k.locals.empty() || !k.types.empty() || !k.variants.empty() || !k.body) return std::nullopt;
+  Matcher mt;
+  MapKernel &m = mt.m;
+  for (const Decl &d : k.params) {
+    if (d.kind != Decl::Param || !d.var.type) return std::nullopt;
+    MapKernel::Param p;
+    p.name = d.var.name;
+    if (p.name.compare(0, 8, "sarek_f_") == 0 || (p.name.size() > 3 && p.name.compare(p.name.size() - 3, 3, "__e") == 0))
+      return std::nullopt;
+    const Type &t = *d.var.type;
+    if (t.kind == Type::Vec && t.elt && t.elt->kind == Type::Float32) p.kind = MapKernel::Param::Vec;
+    else if (t.kind == Type::Float32) p.kind = MapKernel::Param::F32;
+    else if (t.kind == Type::Int32) p.kind = MapKernel::Param::I32;
+    else return std::nullopt;
+    for (const auto &q : m.params)
+      if (q.name == p.name) return std::nullopt;
+    m.params.push_back(p);
+  }
+  // let tid = <global id> in if tid < n then S
+  const Stmt *s = k.body.get();
+  while ((s->kind == Stmt::Block || s->kind == Stmt::Seq) && s->stmts.size() == 1) s = s->stmts[0].get();
+  if (s->kind != Stmt::Let || s->var.is_mutable || !is_global_id(s->e) || s->stmts.size() != 1) return std::nullopt;
+  if (!s->var.type || s->var.type->kind != Type::Int32) return std::nullopt;
+  m.tid = s->var.name;
+  if (mt.param_index(m.tid) >= 0 || m.tid.compare(0, 8, "sarek_f_") == 0) return std::nullopt;
+  const Stmt *guard = s->stmts[0].get();
+  while ((guard->kind == Stmt::Block || guard->kind == Stmt::Seq) && guard->stmts.size() == 1)
+    guard = guard->stmts[0].get();
+  if (guard->kind != Stmt::If || !guard->e || guard->stmts.empty()) return std::nullopt;
+  if (guard->stmts.size() > 1 && guard->stmts[1] && guard->stmts[1]->kind != Stmt::Empty) return std::nullopt;
+  const Expr &c = *guard->e;
+  if (c.kind != Expr::BinopE || c.binop != Binop::Lt || !is_var(c.args[0], m.tid) || !c.args[1] ||
+      c.args[1]->kind != Expr::VarRef)
+    return std::nullopt;
+  m.n = mt.param_index(c.args[1]->var.name);
+  if (m.n < 0 || m.params[m.n].kind != MapKernel::Param::I32) return std::nullopt;
+  const Stmt *assign = find_assign(guard->stmts[0]);
+  if (!assign || !assign->lhs || assign->lhs->kind != LValue::LArrayElem) return std::nullopt;
+  m.out = mt.param_index(assign->lhs->name);
+  if (m.out < 0 || m.params[m.out].kind != MapKernel::Param::Vec) return std::nullopt;
+  auto rewritten = mt.body(guard->stmts[0]);
+  if (!rewritten) return std::nullopt;
+  std::sort(m.inputs.begin(), m.inputs.end());
+  if (m.inputs.size() > 6) return std::nullopt;   // registers: four 128-bit loads per input and thread
+  m.body = gen_stmt(*rewritten, "  ");
+  return m;
+}
+
+std::string map_source(const MapKernel &m, bool with_sums, bool nt_loads) {
+  std::string o;
+  o += "typedef float sarek_f_v4 __attribute__((ext_vector_type(4)));\n";
+  if (with_sums) {
+    // the stream kernels' wave reduction: quad_perm, row_half_mirror, row_mirror, then the four rows
+    o += "template <int Ctrl> __device__ __forceinline__ float sarek_f_dpp_add(float v) {\n"
+         "  int sh = __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), Ctrl, 0xF, 0xF, true);\n"
+         "  return v + __builtin_bit_cast(float, sh);\n}\n"
+         "__device__ __forceinline__ float sarek_f_wave_sum(float v) {\n"
+         "  v = sarek_f_dpp_add<0xB1>(v);\n  v = sarek_f_dpp_add<0x4E>(v);\n  v = sarek_f_dpp_add<0x141>(v);\n"
+         "  v = sarek_f_dpp_add<0x140>(v);\n  int iv = __builtin_bit_cast(int, v);\n"
+         "  float r0 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(iv, 0));\n"
+         "  float r1 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(iv, 16));\n"
+         "  float r2 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(iv, 32));\n"
+         "  float r3 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(iv, 48));\n"
+         "  return (r0 + r1) + (r2 + r3);\n}\n";
+  }
+  // one element: the kernel's own statements on the element's inputs
+  std::string formals, actuals_tail;
+  for (int p : m.inputs) formals += "float " + m.params[p].name + "__e, ";
+  for (const auto &p : m.params) {
+    if (p.kind == MapKernel::Param::Vec) continue;
+    formals += std::string(p.kind == MapKernel::Param::F32 ? "float " : "int ") + p.name + ", ";
+    actuals_tail += p.name + ", ";
+  }
+  o += "__device__ __forceinline__ float sarek_f_apply(" + formals + "int " + m.tid + ") {\n  float sarek_f_res;\n" +
+       m.body + "  return sarek_f_res;\n}\n";
+  // The element's value passes through an empty asm before it is stored and summed: the compiler then cannot fold
+  // the expression's last multiplication into the first addition of the sum (an fma there would add a product that
+  // was never rounded, and the sums would no longer be those of the stored vector).
+  o += "__device__ __forceinline__ float sarek_f_opaque(float v) {\n  asm volatile(\"\" : \"+v\"(v));\n  return v;\n}\n";
+  auto apply = [&](const std::string &value_of, const std::string &index) {
+    std::string a = "sarek_f_opaque(sarek_f_apply(";
+    for (size_t i = 0; i < m.inputs.size(); ++i) {
+      std::string v = value_of;
+      const size_t at = v.find('@');
+      v.replace(at, 1, std::to_string(i));
+      a += v + ", ";
+    }
+    return a + actuals_tail + "(int)(" + index + ")))";
+  };
+  const std::string out = m.params[m.out].name;
+  o += "extern \"C\" __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(8, 8))) void sarek_map(";
+  for (size_t i = 0; i < m.params.size(); ++i) {
+    const auto &p = m.params[i];
+    if (p.kind == MapKernel::Param::Vec)
+      o += (static_cast<int>(i) == m.out ? "float* __restrict__ " : "const float* ") + p.name + ", ";
+    else
+      o += std::string(p.kind == MapKernel::Param::F32 ? "float " : "int ") + p.name + ", ";
+  }
+  o += "float* __restrict__ sarek_f_partials) {\n";
+  o += "  const long long sarek_f_n = " + m.params[m.n].name + ", sarek_f_n4 = sarek_f_n >> 2;\n";
+  // a wave owns four consecutive KiB of every vector: slot u of lane l is float4 number base + 64 u
+  o += "  const long long sarek_f_base = (long long)blockIdx.x * 1024 + (threadIdx.x >> 6) * 256 + (threadIdx.x & 63);\n"
+       "  const bool sarek_f_full = sarek_f_base + 192 < sarek_f_n4;\n"
+       "  sarek_f_v4 sarek_f_r[4];\n  float sarek_f_extra[4] = {0.f, 0.f, 0.f, 0.f};\n";
+  for (size_t i = 0; i < m.inputs.size(); ++i)
+    o += "  const sarek_f_v4* sarek_f_p" + std::to_string(i) + " = reinterpret_cast<const sarek_f_v4*>(" +
+         m.params[m.inputs[i]].name + ");\n";
+  o += "  sarek_f_v4* sarek_f_po = reinterpret_cast<sarek_f_v4*>(" + out + ");\n";
+  o += "  if (sarek_f_full) {\n";
+  for (size_t i = 0; i < m.inputs.size(); ++i) {
+    const std::string is = std::to_string(i);
+    o += "    sarek_f_v4 sarek_f_x" + is + "[4];\n#pragma unroll\n    for (int u = 0; u < 4; ++u) sarek_f_x" + is + "[u] = " +
+         (nt_loads ? "__builtin_nontemporal_load(sarek_f_p" + is + " + sarek_f_base + 64 * u)"
+                   : "sarek_f_p" + is + "[sarek_f_base + 64 * u]") +
+         ";\n";
+  }
+  o += "#pragma unroll\n    for (int u = 0; u < 4; ++u)\n#pragma unroll\n      for (int j = 0; j < 4; ++j)\n"
+       "        sarek_f_r[u][j] = " + apply("sarek_f_x@[u][j]", "(sarek_f_base + 64 * u) * 4 + j") + ";\n";
+  o += "#pragma unroll\n    for (int u = 0; u < 4; ++u) __builtin_nontemporal_store(sarek_f_r[u], sarek_f_po + sarek_f_base + 64 * u);\n";
+  o += "  } else {\n#pragma unroll\n    for (int u = 0; u < 4; ++u) {\n      const long long i = sarek_f_base + 64 * u;\n"
+       "      sarek_f_r[u] = sarek_f_v4{0.f, 0.f, 0.f, 0.f};\n      if (i < sarek_f_n4) {\n";
+  for (size_t i = 0; i < m.inputs.size(); ++i)
+    o += "        const sarek_f_v4 sarek_f_y" + std::to_string(i) + " = sarek_f_p" + std::to_string(i) + "[i];\n";
+  o += "#pragma unroll\n        for (int j = 0; j < 4; ++j) sarek_f_r[u][j] = " + apply("sarek_f_y@[j]", "i * 4 + j") + ";\n"
+       "        sarek_f_po[i] = sarek_f_r[u];\n      }\n";
+  // the lane whose slot holds the end of the vector takes the one to three elements there
+  {
+    std::string a = "sarek_f_opaque(sarek_f_apply(";
+    for (int p : m.inputs) a += m.params[p].name + "[e], ";
+    a += actuals_tail + "(int)e))";
+    o += "      if (i == sarek_f_n4) {\n        for (long long e = sarek_f_n4 << 2; e < sarek_f_n; ++e) {\n"
+         "          const float v = " + a + ";\n          " + out + "[e] = v;\n          sarek_f_extra[u] += v;\n        }\n      }\n";
+  }
+  o += "    }\n  }\n";
+  if (with_sums) {
+    o += "  const long long sarek_f_nblocks = (sarek_f_n + 255) >> 8;\n  float sarek_f_t[4];\n#pragma unroll\n"
+         "  for (int u = 0; u < 4; ++u)\n    sarek_f_t[u] = sarek_f_wave_sum(((sarek_f_r[u][0] + sarek_f_r[u][1]) + "
+         "(sarek_f_r[u][2] + sarek_f_r[u][3])) + sarek_f_extra[u]);\n"
+         "  const long long sarek_f_j0 = (long long)blockIdx.x * 16 + (threadIdx.x >> 6) * 4;\n"
+         "  if ((threadIdx.x & 63) == 0) {\n    if (sarek_f_j0 + 4 <= sarek_f_nblocks) {\n"
+         "      *reinterpret_cast<sarek_f_v4*>(sarek_f_partials + sarek_f_j0) = "
+         "sarek_f_v4{sarek_f_t[0], sarek_f_t[1], sarek_f_t[2], sarek_f_t[3]};\n    } else {\n#pragma unroll\n"
+         "      for (int u = 0; u < 4; ++u)\n        if (sarek_f_j0 + u < sarek_f_nblocks) sarek_f_partials[sarek_f_j0 + u] = sarek_f_t[u];\n"
+         "    }\n  }\n";
+  }
+  o += "}\n";
+  return o;
+}
+
+}  // namespace ir
+}  // namespace sarek_hip

@@ -1,0 +1,35 @@
+// Element-wise kernels recognised as a class and rebuilt in the stream kernels' shape (map_fuse.cpp).
+#pragma once
+#include <optional>
+#include <string>
+#include <vector>
+
+#include "ir.hpp"
+
+namespace sarek_hip {
+namespace ir {
+
+// out[tid] = f(in_1[tid], ..., in_k[tid], scalars, tid) for tid < n
+struct MapKernel {
+  struct Param {
+    std::string name;
+    enum Kind { Vec, F32, I32 } kind = Vec;
+  };
+  std::vector<Param> params;   // the kernel's parameters in order (a vector is a buffer and its length at a launch)
+  int out = -1, n = -1;        // indices into params: the vector written, the bound
+  std::vector<int> inputs;     // the vectors read, ascending
+  std::string tid;             // name of the thread-id variable
+  std::string body;            // HIP statements that set sarek_f_res from <vector>__e, the scalars and tid
+};
+
+// The shape above, or nothing: one guarded store under immutable lets, every read at [tid], no mutable state,
+// helper functions, records, atomics, barriers or launch-geometry intrinsics in the element's expression.
+std::optional<MapKernel> match_map(const Kernel &k);
+
+// HIP source of `sarek_map(<the kernel's parameters without the vector lengths>, float* partials)`: 256-thread
+// workgroups of 4096 elements, ceil(n / 4096) of them; with_sums also stores partials[j] = sum of out[256 j .. 256 j + 255]
+// in the order of the block-256 tree kernels.
+std::string map_source(const MapKernel &m, bool with_sums, bool nt_loads);
+
+}  // namespace ir
+}  // namespace sarek_hip

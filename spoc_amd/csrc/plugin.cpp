@@ -6,10 +6,13 @@
 // way the generated kernel assumes; otherwise the text is JIT-compiled as it stands.
 #include <cstdlib>
 #include <cstring>
+#include <mutex>
 #include <string>
+#include <unordered_map>
 #include <vector>
 
 #include "common.hpp"
+#include "host/map_fuse.hpp"
 #include "plugin.hpp"
 
 namespace sarek_hip {
@@ -79,6 +82,93 @@ bool ranges_meet(const void *p, int64_t pb, const void *q, int64_t qb) {
 bool covers_1d(const int block[3], const int grid[3], int64_t threads) {
   return block[1] == 1 && block[2] == 1 && grid[1] == 1 && grid[2] == 1 &&
          static_cast<int64_t>(block[0]) * grid[0] >= threads;
+}
+
+// An element-wise kernel (tag map_f32) rebuilt in the stream kernels' shape: 128-bit accesses, four loads per input
+// in flight per thread, the kernel's own expression on every element; with `red` (the arguments of a block-256 sum
+// launched right after it on the vector it writes) the sums leave in the same pass.  The text is compiled once per
+// kernel and variant.  Returns 1 when the launch (or the pair) was served, 0 to fall back.
+int try_map(const char *source, const int block[3], const int grid[3], const sarek_hip_arg *a, int na,
+            const sarek_hip_arg *red, int nred, const int rblock[3], const int rgrid[3], int *rc) {
+  ir::MapKernel m;
+  if (!find_generated_map(source, &m)) return 0;
+  struct Slot {
+    union {
+      void *p;
+      int32_t i32;
+      float f32;
+    };
+  };
+  constexpr int kMaxParams = 24;
+  if (m.params.size() + 1 > kMaxParams) return 0;
+  Slot slots[kMaxParams];
+  void *params[kMaxParams];
+  int64_t lengths[kMaxParams];
+  int ai = 0;
+  for (size_t i = 0; i < m.params.size(); ++i) {
+    lengths[i] = 0;
+    switch (m.params[i].kind) {
+      case ir::MapKernel::Param::Vec:
+        if (!vec_at(a, na, ai)) return 0;
+        slots[i].p = a[ai].buffer;
+        lengths[i] = a[ai].length;
+        ai += 2;
+        break;
+      case ir::MapKernel::Param::F32:
+        if (ai >= na || !is_f32(a[ai])) return 0;
+        slots[i].f32 = a[ai++].f32;
+        break;
+      case ir::MapKernel::Param::I32:
+        if (ai >= na || !is_i32(a[ai])) return 0;
+        slots[i].i32 = a[ai++].i32;
+        break;
+    }
+    params[i] = &slots[i];
+  }
+  if (ai != na) return 0;
+  const int64_t n = slots[m.n].i32;
+  if (n <= 0 || n > 0x7FFFFFFF - 4096 || !covers_1d(block, grid, n)) return 0;
+  if (lengths[m.out] < n) return 0;
+  for (int in : m.inputs)
+    if (lengths[in] < n || shifted_overlap(slots[m.out].p, slots[in].p, n)) return 0;
+  const int64_t nblocks = cdiv(n, 256);
+  void *partials = nullptr;
+  if (red) {
+    if (nred != 5 || !vec_at(red, nred, 0) || !vec_at(red, nred, 2) || !is_i32(red[4]) || red[4].i32 != n) return 0;
+    if (rblock[0] != 256 || rblock[1] != 1 || rblock[2] != 1 || rgrid[1] != 1 || rgrid[2] != 1 || rgrid[0] != nblocks)
+      return 0;
+    if (red[0].buffer != slots[m.out].p || red[0].length < n || red[2].length < nblocks) return 0;
+    if (ranges_meet(red[2].buffer, nblocks * 4, slots[m.out].p, n * 4)) return 0;
+    for (int in : m.inputs)
+      if (ranges_meet(red[2].buffer, nblocks * 4, slots[in].p, n * 4)) return 0;
+    partials = red[2].buffer;
+  }
+  // inputs that together fit the 256 MB last-level cache may still be there: plain loads; larger ones go past it
+  const bool nt = static_cast<int64_t>(m.inputs.size()) * n * 4 > (int64_t{256} << 20);
+  static std::mutex mu;
+  static std::unordered_map<std::string, std::string> texts;   // "<variant><generated text>" -> rebuilt text
+  std::string key(1, static_cast<char>('0' + (red ? 2 : 0) + (nt ? 1 : 0)));
+  key += source;
+  std::string text;
+  {
+    std::lock_guard<std::mutex> lock(mu);
+    auto it = texts.find(key);
+    if (it == texts.end()) {
+      if (texts.size() >= 1024) texts.clear();
+      it = texts.emplace(key, ir::map_source(m, red != nullptr, nt)).first;
+    }
+    text = it->second;
+  }
+  sarek_hip_kernel k = nullptr;
+  thread_local std::vector<char> log(16384);
+  *rc = sarek_hip_kernel_compile_cached(text.c_str(), "sarek_map", &k, log.data(), log.size());
+  if (*rc != SAREK_HIP_OK) return 1;
+  Slot part;
+  part.p = partials;
+  params[m.params.size()] = &part;
+  const unsigned g[3] = {static_cast<unsigned>(cdiv(n, 4096)), 1, 1}, b[3] = {256, 1, 1};
+  *rc = sarek_hip_kernel_launch(k, g, b, 0, nullptr, params, static_cast<int>(m.params.size()) + 1);
+  return 1;
 }
 
 // Returns 1 when the call was served by a hand kernel (status in *rc), 0 to fall back.
@@ -464,8 +554,11 @@ int sarek_hip_run_sources(const sarek_hip_launch *launches, int n_launches, int 
       const std::string tag0 = read_tag(l0.source), tag1 = read_tag(l1.source);
       int rc = SAREK_HIP_OK;
       if (langs_ok && !tag0.empty() && !tag1.empty() && tag_is_ours(tag0, l0.source) && tag_is_ours(tag1, l1.source) &&
-          try_specialised_pair(tag0, l0.block, l0.grid, l0.args, l0.n_args, tag1, l1.block, l1.grid, l1.args,
-                               l1.n_args, &rc)) {
+          (tag0 == "map_f32"
+               ? (tag1 == "reduce_sum_block256_f32" && try_map(l0.source, l0.block, l0.grid, l0.args, l0.n_args, l1.args,
+                                                               l1.n_args, l1.block, l1.grid, &rc))
+               : try_specialised_pair(tag0, l0.block, l0.grid, l0.args, l0.n_args, tag1, l1.block, l1.grid, l1.args,
+                                      l1.n_args, &rc))) {
         if (rc != SAREK_HIP_OK) return rc;
         path += (path.empty() ? "" : ";") + tag0 + "+" + tag1;
         served = 2;
@@ -518,7 +611,8 @@ int sarek_hip_run_source(const char *source, int lang, const char *kernel_name, 
     if (!tag.empty() && !tag_is_ours(tag, source)) tag.clear();
     if (!tag.empty()) {
       int rc = SAREK_HIP_OK;
-      if (try_specialised(tag, block, grid, args, n_args, &rc)) {
+      if (tag == "map_f32" ? try_map(source, block, grid, args, n_args, nullptr, 0, nullptr, nullptr, &rc)
+                           : try_specialised(tag, block, grid, args, n_args, &rc)) {
         t_last_path = tag;
         return rc;
       }

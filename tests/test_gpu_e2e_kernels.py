@@ -16,11 +16,11 @@ pytestmark = pytest.mark.gpu
 GID = add(intr("thread_idx_x"), mul(intr("block_dim_x"), intr("block_idx_x")))
 
 
-def launch(hip, ir, n, items, block=256, shared_mem=0):
-    path = hip.run_source(hip.generate_source(ir, block=(block, 1, 1)), "sarek_kern", (block, 1, 1),
+def launch(hip, ir, n, items, block=256, shared_mem=0, path="jit"):
+    took = hip.run_source(hip.generate_source(ir, block=(block, 1, 1)), "sarek_kern", (block, 1, 1),
                           ((n + block - 1) // block, 1, 1), items, shared_mem=shared_mem)
     hip.check(hip.lib.sarek_hip_device_synchronize())
-    assert path == "jit"
+    assert took == path
 
 
 def ints(torch, a):
@@ -99,11 +99,20 @@ def test_math_intrinsics(hip, torch_cuda):
                add(m("sqrt", v), add(m("log", add(v, f32("1.0"))), m("pow", v, f32("1.5")))))
     ir = kernel(params, let(tid, intr("global_thread_id", "Std"),
                             if_(lt(tid, var("n")), let(v, read("x", tid), assign_elem("out", tid, expr)))))
-    out = torch.zeros(n, device="cuda")
-    launch(hip, ir, n, [torch.from_numpy(x).cuda(), out, ("i32", n)])
     x64 = x.astype(np.float64)
     exp = np.sin(x64) * np.cos(x64) + np.exp(-x64) + np.sqrt(x64) + np.log(x64 + 1) + x64 ** 1.5
-    assert np.allclose(out.cpu().numpy(), exp, rtol=2e-6, atol=2e-6)
+    # an element-wise kernel: rebuilt in the stream kernels' shape from the same lowered expression, and as generated
+    results = []
+    for on, path in ((1, "map_f32"), (0, "jit")):
+        out = torch.zeros(n, device="cuda")
+        hip.check(hip.lib.sarek_hip_set_specialisation(on))
+        try:
+            launch(hip, ir, n, [torch.from_numpy(x).cuda(), out, ("i32", n)], path=path)
+        finally:
+            hip.check(hip.lib.sarek_hip_set_specialisation(1))
+        results.append(out.cpu().numpy())
+        assert np.allclose(results[-1], exp, rtol=2e-6, atol=2e-6)
+    assert np.array_equal(results[0], results[1])
 
 
 def test_records_helper_function_and_variant_match(hip, torch_cuda):

@@ -1,0 +1,125 @@
+"""Element-wise kernels rebuilt in the stream kernels' shape (tag map_f32) and fused with the block-256 sum
+(benchmarks/bench_reduction.ml:62-96) in Execute.run_pipeline: the vector they write is the generated kernel's bit
+for bit, the sums are the hand block-256 kernel's on that vector."""
+import os
+
+import numpy as np
+import pytest
+
+from map_kernels import MAPS
+
+pytestmark = pytest.mark.gpu
+
+IR_DIR = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "ir")
+
+
+@pytest.fixture()
+def sarek(hip, torch_cuda):
+    from spoc_amd import sarek as s
+    s.Device.init()
+    yield s
+    hip.check(hip.lib.sarek_hip_set_specialisation(1))
+SIZES = [1, 3, 255, 256, 257, 4095, 4096, 4097, 8191, 100003, (1 << 20) + 5]
+
+
+def arguments(sarek, name, n, rng):
+    """(launch arguments in parameter order, output vector) of MAPS[name] over n elements."""
+    E, V = sarek.Execute, sarek.Vector
+
+    def vec():
+        return V.of_array((rng.standard_normal(n) * 10.0 ** rng.integers(-3, 3, n)).astype(np.float32))
+
+    out = V.create(V.float32, n)
+    out.host[:] = np.nan
+    if name == "scale":
+        return [E.Vec(vec()), E.Vec(out), E.Float32(1.7), E.Int32(n)], out
+    if name == "saxpy_with_let":
+        return [E.Vec(vec()), E.Vec(vec()), E.Vec(out), E.Float32(-0.3), E.Int32(n)], out
+    if name == "norm3":
+        return [E.Vec(out), E.Vec(vec()), E.Vec(vec()), E.Vec(vec()), E.Int32(n)], out
+    if name == "ramp_select":
+        return [E.Vec(vec()), E.Vec(vec()), E.Vec(out), E.Int32(5), E.Int32(n)], out
+    if name == "fill_const":
+        return [E.Vec(out), E.Float32(2.5), E.Int32(n)], out
+    raise KeyError(name)
+
+
+def both_ways(hip, run):
+    res = []
+    for on in (1, 0):
+        hip.check(hip.lib.sarek_hip_set_specialisation(on))
+        try:
+            res.append(run())
+        finally:
+            hip.check(hip.lib.sarek_hip_set_specialisation(1))
+    return res
+
+
+@pytest.mark.parametrize("n", SIZES)
+@pytest.mark.parametrize("name", sorted(MAPS))
+def test_a_map_alone_writes_what_the_generated_kernel_writes(hip, sarek, name, n):
+    E = sarek.Execute
+    ir = MAPS[name]()
+
+    def run():
+        args, out = arguments(sarek, name, n, np.random.default_rng(n))
+        path = E.run_vectors(ir, args, (256, 1, 1), ((n + 255) // 256, 1, 1))
+        return path, out.to_array().copy()
+
+    (p_map, got), (p_jit, want) = both_ways(hip, run)
+    assert (p_map, p_jit) == ("map_f32", "jit")
+    assert not np.isnan(want).any() or name == "norm3"
+    assert np.array_equal(got.view(np.uint32), want.view(np.uint32))
+
+
+@pytest.mark.parametrize("n", SIZES)
+@pytest.mark.parametrize("name", sorted(MAPS))
+def test_map_then_block_sum_is_one_launch(hip, sarek, name, n):
+    E, V = sarek.Execute, sarek.Vector
+    ir = MAPS[name]()
+    reduction = open(os.path.join(IR_DIR, "reduction.ir")).read()
+    nblocks = (n + 255) // 256
+
+    def run():
+        args, out = arguments(sarek, name, n, np.random.default_rng(n))
+        sums = V.create(V.float32, nblocks)
+        sums.host[:] = np.nan
+        stages = [(ir, args, (256, 1, 1), (nblocks, 1, 1)),
+                  (reduction, [E.Vec(out), E.Vec(sums), E.Int32(n)], (256, 1, 1), (nblocks, 1, 1))]
+        return E.run_pipeline(stages), out.to_array().copy(), sums.to_array().copy(), (stages, sums)
+
+    (fused, a_fused, s_fused, (stages, sums)), (jit, a_jit, s_jit, _) = both_ways(hip, run)
+    assert fused == ("map_f32+reduce_sum_block256_f32", 1) and jit == ("jit;jit", 2)
+    assert np.array_equal(a_fused.view(np.uint32), a_jit.view(np.uint32))
+    # the hand block-256 kernel on the same vector gives the same bits; the generated tree kernel is within the
+    # sum's tolerance (it adds the same values in another association)
+    assert E.run_vectors(*stages[1]) == "reduce_sum_block256_f32"
+    assert np.array_equal(sums.to_array().view(np.uint32), s_fused.view(np.uint32))
+    scale = np.abs(a_jit.astype(np.float64)).reshape(-1)
+    bound = np.add.reduceat(scale, np.arange(0, n, 256)) * 1e-5 + 1e-30
+    assert np.all(np.abs(s_fused.astype(np.float64) - s_jit.astype(np.float64)) <= bound)
+
+
+def test_pairs_the_fused_kernel_does_not_serve(hip, sarek):
+    E, V = sarek.Execute, sarek.Vector
+    n = 70000
+    nblocks = (n + 255) // 256
+    reduction = open(os.path.join(IR_DIR, "reduction.ir")).read()
+    rng = np.random.default_rng(1)
+    ir = MAPS["scale"]()
+    args, out = arguments(sarek, "scale", n, rng)
+    sums = V.create(V.float32, nblocks)
+    other = V.of_array(rng.standard_normal(n).astype(np.float32))
+    shape = ((256, 1, 1), (nblocks, 1, 1))
+    # the sum reads another vector, or fewer elements
+    assert E.run_pipeline([(ir, args) + shape, (reduction, [E.Vec(other), E.Vec(sums), E.Int32(n)]) + shape]) == \
+        ("map_f32;reduce_sum_block256_f32", 2)
+    assert E.run_pipeline([(ir, args) + shape, (reduction, [E.Vec(out), E.Vec(sums), E.Int32(n - 256)], (256, 1, 1),
+                                                (nblocks - 1, 1, 1))]) == ("map_f32;reduce_sum_block256_f32", 2)
+    # a launch that does not reach every element runs as generated
+    assert E.run_vectors(ir, args, (256, 1, 1), (nblocks - 1, 1, 1)) == "jit"
+    # a maximum behind a map is two launches (the fused pairs with a maximum are the triad's and the vector add's)
+    from test_ir_lowering import reduction_max_ir
+    reduction_max = reduction_max_ir()
+    path, launches = E.run_pipeline([(ir, args) + shape, (reduction_max, [E.Vec(out), E.Vec(sums), E.Int32(n)]) + shape])
+    assert launches == 2 and path.startswith("map_f32;reduce_max_block256_f32")

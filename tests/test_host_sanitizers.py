@@ -53,7 +53,7 @@ def test_host_code_is_clean_under_asan_and_ubsan(tmp_path):
     sources += [os.path.join(CSRC, f) for f in (
         "status.cpp", "backend_info.cpp", "tunables.cpp", "runtime.cpp", "transfer.cpp", "vector.cpp",
         "code_cache.cpp", "plugin.cpp", "library_kernels.cpp", "generate.cpp", "fusion_abi.cpp", "host/ir_text.cpp", "host/ir_hip.cpp",
-        "host/specialise.cpp", "host/fusion.cpp")]
+        "host/specialise.cpp", "host/fusion.cpp", "host/map_fuse.cpp")]
     exe = str(tmp_path / "host_asan")
     flags = ["-std=c++20", "-O1", "-g", "-fsanitize=address,undefined", "-fno-sanitize-recover=undefined",
              "-fno-omit-frame-pointer", "-D__HIP_PLATFORM_AMD__", "-I/opt/rocm/include",
