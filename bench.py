@@ -865,7 +865,7 @@ def main():
     if not args.no_also:
         also = []
         for name in ["triad_sum_2p28", "gemm_f32_8192", "gemm_f16_epilogue", "gemm_f32_1024",
-                     "gemm_bf16_8192", "histogram_2p28", "radix_scatter_5e7"]:
+                     "gemm_bf16_8192", "histogram_2p28", "radix_scatter_5e7", "map_sum_2p28"]:
             if name == args.workload:
                 continue
             torch.cuda.empty_cache()
