@@ -209,7 +209,12 @@ std::optional<MapKernel> match_map(const Kernel &k) {
   return m;
 }
 
-std::string map_source(const MapKernel &m, bool with_sums, bool nt_loads) {
+namespace {
+
+// What both rebuilt kernels start with: the vector type, the wave reduction (when sums are wanted), the element
+// function sarek_f_apply(<inputs' values>, <scalars>, <index>) holding the kernel's own statements, and
+// sarek_f_opaque.  `actuals_tail` receives the scalar arguments of a call ("alpha, k, ").
+std::string prelude(const MapKernel &m, bool with_sums, std::string *actuals_tail) {
   std::string o;
   o += "typedef float sarek_f_v4 __attribute__((ext_vector_type(4)));\n";
   if (with_sums) {
@@ -227,12 +232,12 @@ std::string map_source(const MapKernel &m, bool with_sums, bool nt_loads) {
          "  return (r0 + r1) + (r2 + r3);\n}\n";
   }
   // one element: the kernel's own statements on the element's inputs
-  std::string formals, actuals_tail;
+  std::string formals;
   for (int p : m.inputs) formals += "float " + m.params[p].name + "__e, ";
   for (const auto &p : m.params) {
     if (p.kind == MapKernel::Param::Vec) continue;
     formals += std::string(p.kind == MapKernel::Param::F32 ? "float " : "int ") + p.name + ", ";
-    actuals_tail += p.name + ", ";
+    *actuals_tail += p.name + ", ";
   }
   o += "__device__ __forceinline__ float sarek_f_apply(" + formals + "int " + m.tid + ") {\n  float sarek_f_res;\n" +
        m.body + "  return sarek_f_res;\n}\n";
@@ -240,18 +245,24 @@ std::string map_source(const MapKernel &m, bool with_sums, bool nt_loads) {
   // the expression's last multiplication into the first addition of the sum (an fma there would add a product that
   // was never rounded, and the sums would no longer be those of the stored vector).
   o += "__device__ __forceinline__ float sarek_f_opaque(float v) {\n  asm volatile(\"\" : \"+v\"(v));\n  return v;\n}\n";
-  auto apply = [&](const std::string &value_of, const std::string &index) {
-    std::string a = "sarek_f_opaque(sarek_f_apply(";
-    for (size_t i = 0; i < m.inputs.size(); ++i) {
-      std::string v = value_of;
-      const size_t at = v.find('@');
-      v.replace(at, 1, std::to_string(i));
-      a += v + ", ";
-    }
-    return a + actuals_tail + "(int)(" + index + ")))";
-  };
-  const std::string out = m.params[m.out].name;
-  o += "extern \"C\" __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(8, 8))) void sarek_map(";
+  return o;
+}
+
+// sarek_f_opaque(sarek_f_apply(...)) with `value_of` ('@' = the input's number) as each input's value
+std::string apply_call(const MapKernel &m, const std::string &actuals_tail, const std::string &value_of,
+                       const std::string &index) {
+  std::string a = "sarek_f_opaque(sarek_f_apply(";
+  for (size_t i = 0; i < m.inputs.size(); ++i) {
+    std::string v = value_of;
+    const size_t at = v.find('@');
+    v.replace(at, 1, std::to_string(i));
+    a += v + ", ";
+  }
+  return a + actuals_tail + "(int)(" + index + ")))";
+}
+
+std::string formal_params(const MapKernel &m) {
+  std::string o;
   for (size_t i = 0; i < m.params.size(); ++i) {
     const auto &p = m.params[i];
     if (p.kind == MapKernel::Param::Vec)
@@ -259,7 +270,20 @@ std::string map_source(const MapKernel &m, bool with_sums, bool nt_loads) {
     else
       o += std::string(p.kind == MapKernel::Param::F32 ? "float " : "int ") + p.name + ", ";
   }
-  o += "float* __restrict__ sarek_f_partials) {\n";
+  return o;
+}
+
+}  // namespace
+
+std::string map_source(const MapKernel &m, bool with_sums, bool nt_loads) {
+  std::string actuals_tail;
+  std::string o = prelude(m, with_sums, &actuals_tail);
+  auto apply = [&](const std::string &value_of, const std::string &index) {
+    return apply_call(m, actuals_tail, value_of, index);
+  };
+  const std::string out = m.params[m.out].name;
+  o += "extern \"C\" __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(8, 8))) void sarek_map(";
+  o += formal_params(m) + "float* __restrict__ sarek_f_partials) {\n";
   o += "  const long long sarek_f_n = " + m.params[m.n].name + ", sarek_f_n4 = sarek_f_n >> 2;\n";
   // a wave owns four consecutive KiB of every vector: slot u of lane l is float4 number base + 64 u
   o += "  const long long sarek_f_base = (long long)blockIdx.x * 1024 + (threadIdx.x >> 6) * 256 + (threadIdx.x & 63);\n"
@@ -307,6 +331,153 @@ std::string map_source(const MapKernel &m, bool with_sums, bool nt_loads) {
          "    }\n  }\n";
   }
   o += "}\n";
+  return o;
+}
+
+// The block-256 tree sum with an element-wise expression in front of it: benchmarks/bench_reduction.ml:62-96 and
+// bench_dot_product.ml:16-54 with any pure f(in_1[gid], ..., scalars, gid) where they have in[gid] and a[gid] * b[gid].
+// The kernel is taken apart (shared array, tid, gid, the guarded first store and its expression), put together again
+// from the tree's text with that expression in its place, and accepted when the two normalise to the same form: so
+// everything but the expression is the tree, to the letter.
+std::optional<MapKernel> match_tree_sum(const Kernel &k) {
+  if (!k.funcs.empty() || !k.locals.empty() || !k.types.empty() || !k.variants.empty() || !k.body) return std::nullopt;
+  Matcher mt;
+  MapKernel &m = mt.m;
+  for (const Decl &d : k.params) {
+    if (d.kind != Decl::Param || !d.var.type) return std::nullopt;
+    MapKernel::Param p;
+    p.name = d.var.name;
+    if (p.name.compare(0, 8, "sarek_f_") == 0 || (p.name.size() > 3 && p.name.compare(p.name.size() - 3, 3, "__e") == 0))
+      return std::nullopt;
+    const Type &t = *d.var.type;
+    if (t.kind == Type::Vec && t.elt && t.elt->kind == Type::Float32) p.kind = MapKernel::Param::Vec;
+    else if (t.kind == Type::Float32) p.kind = MapKernel::Param::F32;
+    else if (t.kind == Type::Int32) p.kind = MapKernel::Param::I32;
+    else return std::nullopt;
+    for (const auto &q : m.params)
+      if (q.name == p.name) return std::nullopt;
+    m.params.push_back(p);
+  }
+  auto unwrap = [](const Stmt *s) {
+    while (s && (s->kind == Stmt::Block || s->kind == Stmt::Seq) && s->stmts.size() == 1) s = s->stmts[0].get();
+    return s;
+  };
+  // let sdata = shared f32[256] in let tid = .. in let gid = .. in seq (block (if gid < n then sdata[tid] <- LEAF else ..)) ..
+  const Stmt *l0 = unwrap(k.body.get());
+  if (!l0 || l0->kind != Stmt::Let || !l0->e || l0->e->kind != Expr::ArrayCreate || l0->stmts.size() != 1) return std::nullopt;
+  const Stmt *l1 = unwrap(l0->stmts[0].get());
+  if (!l1 || l1->kind != Stmt::Let || l1->stmts.size() != 1) return std::nullopt;
+  const Stmt *l2 = unwrap(l1->stmts[0].get());
+  if (!l2 || l2->kind != Stmt::Let || l2->stmts.size() != 1 || !is_global_id(l2->e)) return std::nullopt;
+  const Stmt *sq = l2->stmts[0].get();
+  while (sq && sq->kind == Stmt::Block && sq->stmts.size() == 1) sq = sq->stmts[0].get();
+  if (!sq || sq->kind != Stmt::Seq || sq->stmts.size() < 2) return std::nullopt;
+  const Stmt *first = unwrap(sq->stmts[0].get());
+  if (!first || first->kind != Stmt::If || first->stmts.size() != 2 || !first->e) return std::nullopt;
+  const Expr &c = *first->e;
+  if (c.kind != Expr::BinopE || c.binop != Binop::Lt || !is_var(c.args[0], l2->var.name) || !c.args[1] ||
+      c.args[1]->kind != Expr::VarRef)
+    return std::nullopt;
+  const Stmt *store = unwrap(first->stmts[0].get());
+  if (!store || store->kind != Stmt::Assign || !store->lhs || store->lhs->kind != LValue::LArrayElem ||
+      store->lhs->name != l0->var.name || !store->e)
+    return std::nullopt;
+  m.tid = l2->var.name;
+  m.n = mt.param_index(c.args[1]->var.name);
+  if (m.n < 0 || m.params[m.n].kind != MapKernel::Param::I32) return std::nullopt;
+  if (mt.param_index(m.tid) >= 0 || m.tid.compare(0, 8, "sarek_f_") == 0) return std::nullopt;
+  // the expression first (it names the inputs), then the output: the one vector it does not read
+  m.out = -1;
+  if (!mt.pure(store->e)) return std::nullopt;
+  for (size_t i = 0; i < m.params.size(); ++i) {
+    if (m.params[i].kind != MapKernel::Param::Vec) continue;
+    if (std::find(m.inputs.begin(), m.inputs.end(), static_cast<int>(i)) != m.inputs.end()) continue;
+    if (m.out >= 0) return std::nullopt;   // a vector that is neither read nor the output
+    m.out = static_cast<int>(i);
+  }
+  if (m.out < 0 || m.inputs.empty() || m.inputs.size() > 3) return std::nullopt;
+  std::sort(m.inputs.begin(), m.inputs.end());
+  // the tree round this expression, from the text of the reference's kernel with this kernel's names
+  auto v = [](const Var &x, const char *type) { return "(var " + x.name + " " + std::to_string(x.id) + " " + type + ")"; };
+  const std::string sdata = l0->var.name, tid = v(l1->var, "i32"), gid = v(l2->var, "i32");
+  const std::string n = "(var " + m.params[m.n].name + " " + std::to_string(c.args[1]->var.id) + " i32)";
+  const std::string slot = "(lelem " + sdata + " " + tid + ")";
+  std::string steps = "(block (if (lt " + gid + " " + n + ") (assign " + slot + " " + print_expr(store->e) + ") (assign " +
+                      slot + " (f32 0.0)))) (barrier) ";
+  for (int half = 128; half >= 1; half >>= 1) {
+    const std::string h = "(i32 " + std::to_string(half) + ")";
+    steps += "(block (if (lt " + tid + " " + h + ") (assign " + slot + " (add (read " + sdata + " " + tid + ") (read " +
+             sdata + " (add " + tid + " " + h + ")))))) (barrier) ";
+  }
+  steps += "(block (if (eq " + tid + " (i32 0)) (assign (lelem " + m.params[m.out].name +
+           " (intr (Gpu) block_idx_x)) (read " + sdata + " (i32 0)))))";
+  const std::string want = canonical_form(k);
+  bool same = false;
+  for (int trailing = 0; trailing < 2 && !same; ++trailing) {
+    const std::string body = "(let " + v(l0->var, "(array f32 shared)") + " (newarray f32 (i32 256) shared) (let " + tid +
+                             " (intr (Gpu) thread_idx_x) (let " + gid +
+                             " (add (intr (Gpu) thread_idx_x) (mul (intr (Gpu) block_dim_x) (intr (Gpu) block_idx_x))) (seq " +
+                             steps + (trailing ? " (barrier)" : "") + "))))";
+    Kernel again = k;
+    try {
+      again.body = parse_stmt(body);
+      same = canonical_form(again) == want;
+    } catch (const std::exception &) {
+      return std::nullopt;
+    }
+  }
+  if (!same) return std::nullopt;
+  auto lhs = std::make_shared<LValue>();
+  lhs->kind = LValue::LVar;
+  lhs->var.name = "sarek_f_res";
+  auto st = std::make_shared<Stmt>();
+  st->kind = Stmt::Assign;
+  st->lhs = lhs;
+  st->e = mt.rewrite(store->e);
+  m.body = gen_stmt(StmtP(st), "  ");
+  return m;
+}
+
+// The hand block-256 kernel's shape (a wave takes eight consecutive 256-element blocks, all loads issued before
+// the first use, one DPP wave reduction per block, the eight sums stored as two 16-byte pieces) with the kernel's
+// expression on every element: `sarek_tree(<the kernel's parameters>)`, 256 threads, ceil(ceil(n / 256) / 32) workgroups.
+std::string tree_sum_source(const MapKernel &m, bool nt_loads) {
+  std::string actuals_tail;
+  std::string o = prelude(m, true, &actuals_tail);
+  const std::string out = m.params[m.out].name;
+  o += "extern \"C\" __global__ __launch_bounds__(256) void sarek_tree(" + formal_params(m);
+  o.resize(o.size() - 2);   // the ", " after the last parameter
+  o += ") {\n  const long long sarek_f_n = " + m.params[m.n].name + ", sarek_f_nblocks = (sarek_f_n + 255) >> 8;\n"
+       "  const int sarek_f_lane = threadIdx.x & 63;\n"
+       "  const long long sarek_f_j0 = ((long long)blockIdx.x * 4 + (threadIdx.x >> 6)) * 8;\n"
+       "  if (sarek_f_j0 >= sarek_f_nblocks) return;\n  float sarek_f_r[8];\n"
+       "  if ((sarek_f_j0 + 8) * 256 <= sarek_f_n) {\n";
+  for (size_t i = 0; i < m.inputs.size(); ++i) {
+    const std::string is = std::to_string(i), name = m.params[m.inputs[i]].name;
+    const std::string at = "reinterpret_cast<const sarek_f_v4*>(" + name + " + (sarek_f_j0 + u) * 256) + sarek_f_lane";
+    o += "    sarek_f_v4 sarek_f_x" + is + "[8];\n#pragma unroll\n    for (int u = 0; u < 8; ++u) sarek_f_x" + is + "[u] = " +
+         (nt_loads ? "__builtin_nontemporal_load(" + at + ")" : "*(" + at + ")") + ";\n";
+  }
+  o += "#pragma unroll\n    for (int u = 0; u < 8; ++u) {\n      float v[4];\n#pragma unroll\n      for (int j = 0; j < 4; ++j) v[j] = " +
+       apply_call(m, actuals_tail, "sarek_f_x@[u][j]", "(sarek_f_j0 + u) * 256 + sarek_f_lane * 4 + j") +
+       ";\n      sarek_f_r[u] = sarek_f_wave_sum((v[0] + v[1]) + (v[2] + v[3]));\n    }\n"
+       "    if (sarek_f_lane == 0) {\n      if ((reinterpret_cast<unsigned long long>(" + out + ") & 15ull) == 0) {\n"
+       "        sarek_f_v4* o4 = reinterpret_cast<sarek_f_v4*>(" + out + " + sarek_f_j0);\n"
+       "        o4[0] = sarek_f_v4{sarek_f_r[0], sarek_f_r[1], sarek_f_r[2], sarek_f_r[3]};\n"
+       "        o4[1] = sarek_f_v4{sarek_f_r[4], sarek_f_r[5], sarek_f_r[6], sarek_f_r[7]};\n      } else {\n"
+       "#pragma unroll\n        for (int u = 0; u < 8; ++u) " + out + "[sarek_f_j0 + u] = sarek_f_r[u];\n      }\n    }\n"
+       "    return;\n  }\n";
+  // the group that holds the end of the input
+  {
+    std::string a = "sarek_f_opaque(sarek_f_apply(";
+    for (int p : m.inputs) a += m.params[p].name + "[i + e], ";
+    a += actuals_tail + "(int)(i + e)))";
+    o += "  for (int u = 0; u < 8 && sarek_f_j0 + u < sarek_f_nblocks; ++u) {\n"
+         "    const long long i = (sarek_f_j0 + u) * 256 + sarek_f_lane * 4;\n    float t[4];\n"
+         "    for (int e = 0; e < 4; ++e) t[e] = i + e < sarek_f_n ? " + a + " : 0.f;\n"
+         "    float v = sarek_f_wave_sum((t[0] + t[1]) + (t[2] + t[3]));\n"
+         "    if (sarek_f_lane == 0) " + out + "[sarek_f_j0 + u] = v;\n  }\n}\n";
+  }
   return o;
 }
 

@@ -31,5 +31,15 @@ std::optional<MapKernel> match_map(const Kernel &k);
 // in the order of the block-256 tree kernels.
 std::string map_source(const MapKernel &m, bool with_sums, bool nt_loads);
 
+// The block-256 tree sum (benchmarks/bench_reduction.ml:62-96) with a pure element-wise expression where the
+// reference's kernel reads its input (the dot product of bench_dot_product.ml:16-54 is one such): `out` is then the
+// vector of block sums, `tid` the global index, `body` the expression's statements.  Nothing when the kernel differs
+// from that tree in anything but the expression.
+std::optional<MapKernel> match_tree_sum(const Kernel &k);
+
+// HIP source of `sarek_tree(<the kernel's parameters without the vector lengths>)`: 256-thread workgroups of 32
+// blocks of 256 elements, sums in the order of the hand block-256 kernel.
+std::string tree_sum_source(const MapKernel &m, bool nt_loads);
+
 }  // namespace ir
 }  // namespace sarek_hip

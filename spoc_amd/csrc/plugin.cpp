@@ -171,6 +171,74 @@ int try_map(const char *source, const int block[3], const int grid[3], const sar
   return 1;
 }
 
+// A block-256 tree sum with an element-wise expression in front (tag tree_sum_map_f32), rebuilt in the hand
+// block-256 kernel's shape.  Same conditions as for the plain tree: 256-thread blocks, exactly ceil(n / 256) of them.
+int try_tree_map(const char *source, const int block[3], const int grid[3], const sarek_hip_arg *a, int na, int *rc) {
+  ir::MapKernel m;
+  if (!find_generated_map(source, &m)) return 0;
+  struct Slot {
+    union {
+      void *p;
+      int32_t i32;
+      float f32;
+    };
+  };
+  constexpr int kMaxParams = 24;
+  if (m.params.size() > kMaxParams) return 0;
+  Slot slots[kMaxParams];
+  void *params[kMaxParams];
+  int64_t lengths[kMaxParams];
+  int ai = 0;
+  for (size_t i = 0; i < m.params.size(); ++i) {
+    lengths[i] = 0;
+    switch (m.params[i].kind) {
+      case ir::MapKernel::Param::Vec:
+        if (!vec_at(a, na, ai)) return 0;
+        slots[i].p = a[ai].buffer;
+        lengths[i] = a[ai].length;
+        ai += 2;
+        break;
+      case ir::MapKernel::Param::F32:
+        if (ai >= na || !is_f32(a[ai])) return 0;
+        slots[i].f32 = a[ai++].f32;
+        break;
+      case ir::MapKernel::Param::I32:
+        if (ai >= na || !is_i32(a[ai])) return 0;
+        slots[i].i32 = a[ai++].i32;
+        break;
+    }
+    params[i] = &slots[i];
+  }
+  if (ai != na) return 0;
+  const int64_t n = slots[m.n].i32;
+  if (n <= 0 || n > 0x7FFFFFFF - 8192) return 0;
+  if (block[0] != 256 || block[1] != 1 || block[2] != 1 || grid[1] != 1 || grid[2] != 1) return 0;
+  const int64_t nblocks = cdiv(n, 256);
+  if (grid[0] != nblocks || lengths[m.out] < nblocks) return 0;
+  for (int in : m.inputs)
+    if (lengths[in] < n || ranges_meet(slots[m.out].p, nblocks * 4, slots[in].p, n * 4)) return 0;
+  const bool nt = true;   // the hand block-256 kernels read past the caches at every size
+  static std::mutex mu;
+  static std::unordered_map<std::string, std::string> texts;
+  std::string text;
+  {
+    std::lock_guard<std::mutex> lock(mu);
+    auto it = texts.find(source);
+    if (it == texts.end()) {
+      if (texts.size() >= 1024) texts.clear();
+      it = texts.emplace(source, ir::tree_sum_source(m, nt)).first;
+    }
+    text = it->second;
+  }
+  sarek_hip_kernel k = nullptr;
+  thread_local std::vector<char> log(16384);
+  *rc = sarek_hip_kernel_compile_cached(text.c_str(), "sarek_tree", &k, log.data(), log.size());
+  if (*rc != SAREK_HIP_OK) return 1;
+  const unsigned g[3] = {static_cast<unsigned>(cdiv(nblocks, 32)), 1, 1}, b[3] = {256, 1, 1};
+  *rc = sarek_hip_kernel_launch(k, g, b, 0, nullptr, params, static_cast<int>(m.params.size()));
+  return 1;
+}
+
 // Returns 1 when the call was served by a hand kernel (status in *rc), 0 to fall back.
 int try_specialised(const std::string &tag, const int block[3], const int grid[3],
                     const sarek_hip_arg *args, int n_args, int *rc) {
@@ -611,8 +679,9 @@ int sarek_hip_run_source(const char *source, int lang, const char *kernel_name, 
     if (!tag.empty() && !tag_is_ours(tag, source)) tag.clear();
     if (!tag.empty()) {
       int rc = SAREK_HIP_OK;
-      if (tag == "map_f32" ? try_map(source, block, grid, args, n_args, nullptr, 0, nullptr, nullptr, &rc)
-                           : try_specialised(tag, block, grid, args, n_args, &rc)) {
+      if (tag == "map_f32"            ? try_map(source, block, grid, args, n_args, nullptr, 0, nullptr, nullptr, &rc)
+          : tag == "tree_sum_map_f32" ? try_tree_map(source, block, grid, args, n_args, &rc)
+                                      : try_specialised(tag, block, grid, args, n_args, &rc)) {
         t_last_path = tag;
         return rc;
       }

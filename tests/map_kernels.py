@@ -98,3 +98,52 @@ def near_misses():
                                                        f"(letmut {var('acc', 'f32', mut=True)} {read('x', t)} " +
                                                        assign_elem("out", t, var("acc", "f32", mut=True)) + ")"))))
     return out
+
+
+# ---- block-256 tree sums with an expression in front (benchmarks/bench_reduction.ml:62-96 with a map where it reads) ----
+
+def _tree_with(leaf_of, params):
+    """The reference's tree kernel text with `leaf_of(gid)` where it reads input[gid]."""
+    from spoc_amd import reference_kernels as rk
+    base = rk.tree(False)
+    gid = "(var gid 6 i32)"
+    old = f"(read input {gid})"
+    assert base.count(old) == 1
+    text = base.replace(old, leaf_of(gid))
+    head = "(params (param (var input 1 (vec f32))) (param (var output 2 (vec f32))) (param (var n 3 i32)))"
+    assert head in text
+    return text.replace(head, "(params " + " ".join(f"(param (var {n} {i} {t}))" for n, i, t in params) + ")")
+
+
+def sum_of_squares():
+    """sum of x^2"""
+    return _tree_with(lambda g: f"(mul (read input {g}) (read input {g}))",
+                      [("input", 1, "(vec f32)"), ("output", 2, "(vec f32)"), ("n", 3, "i32")])
+
+
+def weighted_abs_sum():
+    """sum of alpha * |x| * w: two inputs, a scalar, a math intrinsic"""
+    return _tree_with(lambda g: f"(mul (mul (var alpha 31 f32) (intr (Float32) fabs (read input {g}))) (read w {g}))",
+                      [("input", 1, "(vec f32)"), ("w", 30, "(vec f32)"), ("output", 2, "(vec f32)"), ("alpha", 31, "f32"),
+                       ("n", 3, "i32")])
+
+
+def squared_distance():
+    """sum of (x - y)^2"""
+    return _tree_with(lambda g: f"(mul (sub (read input {g}) (read y {g})) (sub (read input {g}) (read y {g})))",
+                      [("input", 1, "(vec f32)"), ("y", 30, "(vec f32)"), ("output", 2, "(vec f32)"), ("n", 3, "i32")])
+
+
+TREES = {"sum_of_squares": sum_of_squares, "weighted_abs_sum": weighted_abs_sum, "squared_distance": squared_distance}
+
+
+def tree_near_misses():
+    sq = sum_of_squares()
+    out = [("a neighbour in the expression", sq.replace("(mul (read input (var gid 6 i32))", "(mul (read input (add (var gid 6 i32) (i32 1)))", 1)),
+           ("a tree of 128", sq.replace("(i32 128)", "(i32 64)", 1)),
+           ("padding with one", sq.replace("(f32 0.0)", "(f32 1.0)", 1)),
+           ("a product tree", sq.replace("(add (read sdata", "(mul (read sdata", 1)),
+           ("the sum stored elsewhere", sq.replace("(lelem output (intr (Gpu) block_idx_x))", "(lelem output (intr (Gpu) thread_idx_x))"))]
+    for _, text in out:
+        assert text != sq
+    return out

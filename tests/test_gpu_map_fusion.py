@@ -6,7 +6,7 @@ import os
 import numpy as np
 import pytest
 
-from map_kernels import MAPS
+from map_kernels import MAPS, TREES
 
 pytestmark = pytest.mark.gpu
 
@@ -123,3 +123,42 @@ def test_pairs_the_fused_kernel_does_not_serve(hip, sarek):
     reduction_max = reduction_max_ir()
     path, launches = E.run_pipeline([(ir, args) + shape, (reduction_max, [E.Vec(out), E.Vec(sums), E.Int32(n)]) + shape])
     assert launches == 2 and path.startswith("map_f32;reduce_max_block256_f32")
+
+
+@pytest.mark.parametrize("n", [1, 255, 256, 257, 2047, 2048, 8191, 8192, 8193, 100003, (1 << 20) + 5])
+@pytest.mark.parametrize("name", sorted(TREES))
+def test_tree_sum_with_an_expression_in_front(hip, sarek, torch_cuda, name, n):
+    """Served in the hand block-256 kernel's shape: the sums are that kernel's on the vector of the expression's
+    values, bit for bit, and the generated tree's within the sum's tolerance."""
+    torch = torch_cuda
+    E, V = sarek.Execute, sarek.Vector
+    rng = np.random.default_rng(n)
+    x = (rng.standard_normal(n) * 10.0 ** rng.integers(-2, 2, n)).astype(np.float32)
+    y = (rng.standard_normal(n) * 10.0 ** rng.integers(-2, 2, n)).astype(np.float32)
+    nblocks = (n + 255) // 256
+    alpha = np.float32(0.37)
+    if name == "sum_of_squares":
+        values, tail = x * x, lambda out: [E.Vec(V.of_array(x)), E.Vec(out), E.Int32(n)]
+    elif name == "weighted_abs_sum":
+        values = (alpha * np.abs(x)) * y
+        tail = lambda out: [E.Vec(V.of_array(x)), E.Vec(V.of_array(y)), E.Vec(out), E.Float32(float(alpha)), E.Int32(n)]  # noqa: E731
+    else:
+        values, tail = (x - y) * (x - y), lambda out: [E.Vec(V.of_array(x)), E.Vec(V.of_array(y)), E.Vec(out), E.Int32(n)]
+    ir = TREES[name]()
+
+    def run():
+        out = V.create(V.float32, nblocks + 3)
+        out.host[:] = -7.0
+        path = E.run_vectors(ir, tail(out), (256, 1, 1), (nblocks, 1, 1))
+        return path, out.to_array().copy()
+
+    (p_hand, got), (p_jit, want) = both_ways(hip, run)
+    assert (p_hand, p_jit) == ("tree_sum_map_f32", "jit")
+    assert np.all(got[nblocks:] == -7.0) and np.all(want[nblocks:] == -7.0)
+    ref = hip.reduce_sum_block256(torch.from_numpy(values).cuda()).cpu().numpy()
+    assert np.array_equal(got[:nblocks].view(np.uint32), ref.view(np.uint32))
+    bound = np.add.reduceat(np.abs(values.astype(np.float64)), np.arange(0, n, 256)) * 1e-5 + 1e-30
+    assert np.all(np.abs(got[:nblocks].astype(np.float64) - want[:nblocks].astype(np.float64)) <= bound)
+    # a grid that is not exactly ceil(n / 256) blocks is left to the generated kernel
+    out = V.create(V.float32, nblocks + 3)
+    assert E.run_vectors(ir, tail(out), (256, 1, 1), (nblocks + 1, 1, 1)) == "jit"

@@ -2,7 +2,7 @@
 the tag never lands on a kernel outside the class.  No GPU needed."""
 import pytest
 
-from map_kernels import MAPS, near_misses
+from map_kernels import MAPS, TREES, near_misses, tree_near_misses
 
 MARK = "// sarek-hip-specialise: "
 
@@ -27,3 +27,19 @@ def test_the_bench_kernels_keep_their_own_tags(hip):
 @pytest.mark.parametrize("name,ir", near_misses(), ids=[n for n, _ in near_misses()])
 def test_near_misses_are_left_alone(hip, name, ir):
     assert not hip.generate_source(ir).startswith(MARK), name
+
+
+@pytest.mark.parametrize("name", sorted(TREES))
+def test_tree_sums_with_an_expression_in_front_are_tagged(hip, name):
+    assert hip.generate_source(TREES[name](), block=(256, 1, 1)).startswith(MARK + "tree_sum_map_f32\n")
+
+
+def test_the_reference_trees_keep_their_tags(hip):
+    from spoc_amd import reference_kernels as rk
+    assert hip.generate_source(rk.tree(False), block=(256, 1, 1)).startswith(MARK + "reduce_sum_block256_f32")
+    assert hip.generate_source(rk.tree(True), block=(256, 1, 1)).startswith(MARK + "dot_block256_f32")
+
+
+@pytest.mark.parametrize("name,ir", tree_near_misses(), ids=[n for n, _ in tree_near_misses()])
+def test_tree_near_misses_are_left_alone(hip, name, ir):
+    assert not hip.generate_source(ir, block=(256, 1, 1)).startswith(MARK), name
