@@ -282,7 +282,10 @@ std::string map_source(const MapKernel &m, bool with_sums, bool nt_loads) {
     return apply_call(m, actuals_tail, value_of, index);
   };
   const std::string out = m.params[m.out].name;
-  o += "extern \"C\" __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(8, 8))) void sarek_map(";
+  // eight waves per SIMD (64 registers) is the triad's measured best and fits four loads of up to two inputs; with
+  // more inputs the loads alone need more registers than that, and the occupancy is left to the compiler
+  o += std::string("extern \"C\" __global__ __launch_bounds__(256) ") +
+       (m.inputs.size() <= 2 ? "__attribute__((amdgpu_waves_per_eu(8, 8))) " : "") + "void sarek_map(";
   o += formal_params(m) + "float* __restrict__ sarek_f_partials) {\n";
   o += "  const long long sarek_f_n = " + m.params[m.n].name + ", sarek_f_n4 = sarek_f_n >> 2;\n";
   // a wave owns four consecutive KiB of every vector: slot u of lane l is float4 number base + 64 u

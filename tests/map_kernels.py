@@ -62,7 +62,17 @@ def fill_const():
                               if_(lt(tid, var("n")), assign_elem("out", tid, var("c", "f32")))))
 
 
-MAPS = {"scale": scale, "saxpy_with_let": saxpy_with_let, "norm3": norm3, "ramp_select": ramp_select,
+def six_inputs():
+    """out = ((v0 + v1) + v2 * v3) + (v4 - v5): the most inputs the class takes"""
+    params = [(f"v{i}", "(vec f32)") for i in range(6)] + [("out", "(vec f32)"), ("n", "i32")]
+    _params(params)
+    tid = var("tid")
+    r = [read(f"v{i}", tid) for i in range(6)]
+    e = add(add(add(r[0], r[1]), mul(r[2], r[3])), sub(r[4], r[5]))
+    return kernel(params, let(tid, intr("global_thread_id", "Std"), if_(lt(tid, var("n")), assign_elem("out", tid, e))))
+
+
+MAPS = {"six_inputs": six_inputs, "scale": scale, "saxpy_with_let": saxpy_with_let, "norm3": norm3, "ramp_select": ramp_select,
         "fill_const": fill_const}
 
 

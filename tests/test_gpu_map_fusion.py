@@ -39,6 +39,8 @@ def arguments(sarek, name, n, rng):
         return [E.Vec(out), E.Vec(vec()), E.Vec(vec()), E.Vec(vec()), E.Int32(n)], out
     if name == "ramp_select":
         return [E.Vec(vec()), E.Vec(vec()), E.Vec(out), E.Int32(5), E.Int32(n)], out
+    if name == "six_inputs":
+        return [E.Vec(vec()) for _ in range(6)] + [E.Vec(out), E.Int32(n)], out
     if name == "fill_const":
         return [E.Vec(out), E.Float32(2.5), E.Int32(n)], out
     raise KeyError(name)
