@@ -37,6 +37,15 @@ bool is_global_id(const ExprP &e) {
   return false;
 }
 
+// Names the rebuilt texts use themselves (their own prefix, the element variables' suffix, the loop variables of the
+// kernel bodies): a parameter of that name would be shadowed there, so such a kernel stays with the generated code.
+bool name_is_free(const std::string &n) {
+  if (n.compare(0, 8, "sarek_f_") == 0 || (n.size() > 3 && n.compare(n.size() - 3, 3, "__e") == 0)) return false;
+  for (const char *own : {"u", "j", "i", "e", "v", "t", "o4"})
+    if (n == own) return false;
+  return true;
+}
+
 struct Matcher {
   MapKernel m;
   std::vector<std::string> bound;   // immutable let variables in scope
@@ -168,8 +177,7 @@ std::optional<MapKernel> match_map(const Kernel &k) {
     if (d.kind != Decl::Param || !d.var.type) return std::nullopt;
     MapKernel::Param p;
     p.name = d.var.name;
-    if (p.name.compare(0, 8, "sarek_f_") == 0 || (p.name.size() > 3 && p.name.compare(p.name.size() - 3, 3, "__e") == 0))
-      return std::nullopt;
+    if (!name_is_free(p.name)) return std::nullopt;
     const Type &t = *d.var.type;
     if (t.kind == Type::Vec && t.elt && t.elt->kind == Type::Float32) p.kind = MapKernel::Param::Vec;
     else if (t.kind == Type::Float32) p.kind = MapKernel::Param::F32;
@@ -350,8 +358,7 @@ std::optional<MapKernel> match_tree_sum(const Kernel &k) {
     if (d.kind != Decl::Param || !d.var.type) return std::nullopt;
     MapKernel::Param p;
     p.name = d.var.name;
-    if (p.name.compare(0, 8, "sarek_f_") == 0 || (p.name.size() > 3 && p.name.compare(p.name.size() - 3, 3, "__e") == 0))
-      return std::nullopt;
+    if (!name_is_free(p.name)) return std::nullopt;
     const Type &t = *d.var.type;
     if (t.kind == Type::Vec && t.elt && t.elt->kind == Type::Float32) p.kind = MapKernel::Param::Vec;
     else if (t.kind == Type::Float32) p.kind = MapKernel::Param::F32;

@@ -97,6 +97,9 @@ def near_misses():
                                       assign_elem("out", t, mul(read("x", t), "(cast f32 " + intr("block_idx_x") + ")"))))))
     out.append(("guard on another bound", k(base, lambda t: if_(lt(t, i32(1000)), assign_elem("out", t, read("x", t))))))
     out.append(("no guard", k(base, lambda t: assign_elem("out", t, read("x", t)))))
+    named_u = [("x", "(vec f32)"), ("out", "(vec f32)"), ("u", "f32"), ("n", "i32")]
+    out.append(("a scalar named like a loop variable of the rebuilt text",
+                k(named_u, lambda t: if_(lt(t, var("n")), assign_elem("out", t, mul(read("x", t), var("u", "f32")))))))
     ints = [("x", "(vec i32)"), ("out", "(vec i32)"), ("n", "i32")]
     out.append(("int32 vectors", k(ints, lambda t: if_(lt(t, var("n")), assign_elem("out", t, read("x", t))))))
     two = [("x", "(vec f32)"), ("out", "(vec f32)"), ("out2", "(vec f32)"), ("n", "i32")]
