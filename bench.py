@@ -864,8 +864,8 @@ def main():
         out["cpu_baseline"] = cpu_baseline(args.workload)
     if not args.no_also:
         also = []
-        for name in ["triad_sum_2p28", "gemm_f32_8192", "gemm_f16_epilogue", "gemm_f32_1024",
-                     "gemm_bf16_8192", "histogram_2p28", "radix_scatter_5e7", "map_sum_2p28"]:
+        for name in ["triad_sum_2p28", "map_sum_2p28", "gemm_f32_8192", "gemm_f16_epilogue", "gemm_f32_1024",
+                     "gemm_bf16_8192", "histogram_2p28", "radix_scatter_5e7"]:
             if name == args.workload:
                 continue
             torch.cuda.empty_cache()

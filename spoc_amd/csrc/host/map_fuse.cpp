@@ -252,7 +252,7 @@ std::string prelude(const MapKernel &m, bool with_sums, std::string *actuals_tai
   // The element's value passes through an empty asm before it is stored and summed: the compiler then cannot fold
   // the expression's last multiplication into the first addition of the sum (an fma there would add a product that
   // was never rounded, and the sums would no longer be those of the stored vector).
-  o += "__device__ __forceinline__ float sarek_f_opaque(float v) {\n  asm volatile(\"\" : \"+v\"(v));\n  return v;\n}\n";
+  o += "__device__ __forceinline__ float sarek_f_opaque(float v) {\n  asm(\"\" : \"+v\"(v));\n  return v;\n}\n";
   return o;
 }
 
