@@ -55,6 +55,7 @@ extern "C" int sarek_hip_generate_source(const char *ir_text, const int block[3]
     tag = ir::recognise(k);
     if (tag.empty() && (map = ir::match_map(k))) tag = "map_f32";
     if (tag.empty() && (map = ir::match_tree_sum(k))) tag = "tree_sum_map_f32";
+    if (tag.empty() && (map = ir::match_tree_max(k))) tag = "tree_max_map_f32";
     if (!tag.empty()) src = std::string(kSpecialiseMarker) + tag + "\n";
     src += ir::generate(k, block);
   } catch (const ir::ParseError &e) {

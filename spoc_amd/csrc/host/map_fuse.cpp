@@ -350,7 +350,8 @@ std::string map_source(const MapKernel &m, bool with_sums, bool nt_loads) {
 // The kernel is taken apart (shared array, tid, gid, the guarded first store and its expression), put together again
 // from the tree's text with that expression in its place, and accepted when the two normalise to the same form: so
 // everything but the expression is the tree, to the letter.
-std::optional<MapKernel> match_tree_sum(const Kernel &k) {
+namespace {
+std::optional<MapKernel> match_tree(const Kernel &k, bool is_max) {
   if (!k.funcs.empty() || !k.locals.empty() || !k.types.empty() || !k.variants.empty() || !k.body) return std::nullopt;
   Matcher mt;
   MapKernel &m = mt.m;
@@ -392,6 +393,10 @@ std::optional<MapKernel> match_tree_sum(const Kernel &k) {
   if (!store || store->kind != Stmt::Assign || !store->lhs || store->lhs->kind != LValue::LArrayElem ||
       store->lhs->name != l0->var.name || !store->e)
     return std::nullopt;
+  const Stmt *fill = unwrap(first->stmts[1].get());
+  if (!fill || fill->kind != Stmt::Assign || !fill->e || fill->e->kind != Expr::ConstFloat32) return std::nullopt;
+  m.is_max = is_max;
+  m.pad = gen_expr(fill->e);
   m.tid = l2->var.name;
   m.n = mt.param_index(c.args[1]->var.name);
   if (m.n < 0 || m.params[m.n].kind != MapKernel::Param::I32) return std::nullopt;
@@ -413,11 +418,20 @@ std::optional<MapKernel> match_tree_sum(const Kernel &k) {
   const std::string n = "(var " + m.params[m.n].name + " " + std::to_string(c.args[1]->var.id) + " i32)";
   const std::string slot = "(lelem " + sdata + " " + tid + ")";
   std::string steps = "(block (if (lt " + gid + " " + n + ") (assign " + slot + " " + print_expr(store->e) + ") (assign " +
-                      slot + " (f32 0.0)))) (barrier) ";
+                      slot + " " + (is_max ? print_expr(fill->e) : std::string("(f32 0.0)")) + "))) (barrier) ";
   for (int half = 128; half >= 1; half >>= 1) {
     const std::string h = "(i32 " + std::to_string(half) + ")";
-    steps += "(block (if (lt " + tid + " " + h + ") (assign " + slot + " (add (read " + sdata + " " + tid + ") (read " +
-             sdata + " (add " + tid + " " + h + ")))))) (barrier) ";
+    if (is_max) {
+      // benchmarks/bench_reduction_max.ml:18-100: let a = sdata[tid], b = sdata[tid + half] in if b > a then sdata[tid] <- b
+      const std::string a = "(var sarek_f_a " + std::to_string(900000 + half) + " f32)";
+      const std::string b = "(var sarek_f_b " + std::to_string(910000 + half) + " f32)";
+      steps += "(block (if (lt " + tid + " " + h + ") (let " + a + " (read " + sdata + " " + tid + ") (let " + b + " (read " +
+               sdata + " (add " + tid + " " + h + ")) (if (gt " + b + " " + a + ") (assign " + slot + " " + b +
+               ")))))) (barrier) ";
+    } else {
+      steps += "(block (if (lt " + tid + " " + h + ") (assign " + slot + " (add (read " + sdata + " " + tid + ") (read " +
+               sdata + " (add " + tid + " " + h + ")))))) (barrier) ";
+    }
   }
   steps += "(block (if (eq " + tid + " (i32 0)) (assign (lelem " + m.params[m.out].name +
            " (intr (Gpu) block_idx_x)) (read " + sdata + " (i32 0)))))";
@@ -446,6 +460,49 @@ std::optional<MapKernel> match_tree_sum(const Kernel &k) {
   st->e = mt.rewrite(store->e);
   m.body = gen_stmt(StmtP(st), "  ");
   return m;
+}
+}  // namespace
+
+std::optional<MapKernel> match_tree_sum(const Kernel &k) { return match_tree(k, false); }
+std::optional<MapKernel> match_tree_max(const Kernel &k) { return match_tree(k, true); }
+
+// The hand block-256 maximum's shape: lane l of a wave holds elements l, l + 64, l + 128, l + 192 of a block, eight
+// blocks per wave, and the comparisons are the tree's in the tree's order with its strict ">" (halves 128 and 64
+// inside the lane, 32 .. 1 across lanes), so NaNs and signed zeros come out as from the tree; slots past n hold the
+// kernel's fill value.
+std::string tree_max_source(const MapKernel &m) {
+  std::string actuals_tail;
+  std::string o = prelude(m, false, &actuals_tail);
+  const std::string out = m.params[m.out].name;
+  o += "__device__ __forceinline__ float sarek_f_greater(float a, float b) { return b > a ? b : a; }\n";
+  o += "extern \"C\" __global__ __launch_bounds__(256) void sarek_tree(" + formal_params(m);
+  o.resize(o.size() - 2);
+  // (comparisons do not contract with anything: the element's value needs no asm in front of them)
+  std::string a = "sarek_f_apply(";
+  for (int p : m.inputs) a += "__builtin_nontemporal_load(" + m.params[p].name + " + i), ";
+  a += actuals_tail + "(int)i)";
+  o += ") {\n  const long long sarek_f_n = " + m.params[m.n].name + ", sarek_f_nblocks = (sarek_f_n + 255) >> 8;\n"
+       "  const int sarek_f_lane = threadIdx.x & 63;\n"
+       "  const long long sarek_f_j0 = ((long long)blockIdx.x * 4 + (threadIdx.x >> 6)) * 8;\n"
+       "  if (sarek_f_j0 >= sarek_f_nblocks) return;\n"
+       "  const bool sarek_f_full = (sarek_f_j0 + 8) * 256 <= sarek_f_n;\n  float sarek_f_m[8];\n"
+       // all 32 loads of a thread are asked for before the first comparison
+       "  float sarek_f_w[8][4];\n  if (sarek_f_full) {\n#pragma unroll\n    for (int u = 0; u < 8; ++u)\n#pragma unroll\n      for (int q = 0; q < 4; ++q) {\n"
+       "        const long long i = (sarek_f_j0 + u) * 256 + sarek_f_lane + 64 * q;\n"
+       "        sarek_f_w[u][q] = " + a + ";\n      }\n  } else {\n"
+       "#pragma unroll\n    for (int u = 0; u < 8; ++u)\n#pragma unroll\n      for (int q = 0; q < 4; ++q) {\n"
+       "        const long long i = (sarek_f_j0 + u) * 256 + sarek_f_lane + 64 * q;\n"
+       "        sarek_f_w[u][q] = " + m.pad + ";\n        if (i < sarek_f_n) sarek_f_w[u][q] = " + a + ";\n      }\n  }\n"
+       "#pragma unroll\n  for (int u = 0; u < 8; ++u) {\n    const float* v = sarek_f_w[u];\n"
+       "    float g = sarek_f_greater(sarek_f_greater(v[0], v[2]), sarek_f_greater(v[1], v[3]));\n"
+       "#pragma unroll\n    for (int half = 32; half >= 1; half >>= 1) g = sarek_f_greater(g, __shfl_down(g, half, 64));\n"
+       "    sarek_f_m[u] = g;\n  }\n  if (sarek_f_lane != 0) return;\n"
+       "  if (sarek_f_j0 + 8 <= sarek_f_nblocks && (reinterpret_cast<unsigned long long>(" + out + ") & 15ull) == 0) {\n"
+       "    sarek_f_v4* o4 = reinterpret_cast<sarek_f_v4*>(" + out + " + sarek_f_j0);\n"
+       "    o4[0] = sarek_f_v4{sarek_f_m[0], sarek_f_m[1], sarek_f_m[2], sarek_f_m[3]};\n"
+       "    o4[1] = sarek_f_v4{sarek_f_m[4], sarek_f_m[5], sarek_f_m[6], sarek_f_m[7]};\n  } else {\n"
+       "#pragma unroll\n    for (int u = 0; u < 8; ++u)\n      if (sarek_f_j0 + u < sarek_f_nblocks) " + out + "[sarek_f_j0 + u] = sarek_f_m[u];\n  }\n}\n";
+  return o;
 }
 
 // The hand block-256 kernel's shape (a wave takes eight consecutive 256-element blocks, all loads issued before

@@ -20,6 +20,8 @@ struct MapKernel {
   std::vector<int> inputs;     // the vectors read, ascending
   std::string tid;             // name of the thread-id variable
   std::string body;            // HIP statements that set sarek_f_res from <vector>__e, the scalars and tid
+  bool is_max = false;         // match_tree: the "take the greater" tree instead of the sum
+  std::string pad;             // match_tree, maximum: the fill value of slots past n, as HIP text
 };
 
 // The shape above, or nothing: one guarded store under immutable lets, every read at [tid], no mutable state,
@@ -36,10 +38,13 @@ std::string map_source(const MapKernel &m, bool with_sums, bool nt_loads);
 // vector of block sums, `tid` the global index, `body` the expression's statements.  Nothing when the kernel differs
 // from that tree in anything but the expression.
 std::optional<MapKernel> match_tree_sum(const Kernel &k);
+// The same for the "take the greater" tree of benchmarks/bench_reduction_max.ml:18-100 (any constant fill value).
+std::optional<MapKernel> match_tree_max(const Kernel &k);
 
 // HIP source of `sarek_tree(<the kernel's parameters without the vector lengths>)`: 256-thread workgroups of 32
-// blocks of 256 elements, sums in the order of the hand block-256 kernel.
+// blocks of 256 elements, sums in the order of the hand block-256 kernel (maxima: the tree's comparisons in the tree's order).
 std::string tree_sum_source(const MapKernel &m, bool nt_loads);
+std::string tree_max_source(const MapKernel &m);
 
 }  // namespace ir
 }  // namespace sarek_hip

@@ -177,8 +177,8 @@ int try_map(const char *source, const int block[3], const int grid[3], const sar
   return 1;
 }
 
-// A block-256 tree sum with an element-wise expression in front (tag tree_sum_map_f32), rebuilt in the hand
-// block-256 kernel's shape.  Same conditions as for the plain tree: 256-thread blocks, exactly ceil(n / 256) of them.
+// A block-256 tree sum or maximum with an element-wise expression in front (tags tree_sum_map_f32, tree_max_map_f32),
+// rebuilt in the hand block-256 kernel's shape.  Same conditions as for the plain tree: 256-thread blocks, exactly ceil(n / 256) of them.
 int try_tree_map(const char *source, const int block[3], const int grid[3], const sarek_hip_arg *a, int na, int *rc) {
   ir::MapKernel m;
   if (!find_generated_map(source, &m)) return 0;
@@ -232,7 +232,7 @@ int try_tree_map(const char *source, const int block[3], const int grid[3], cons
     auto it = texts.find(source);
     if (it == texts.end()) {
       if (texts.size() >= 1024) texts.clear();
-      it = texts.emplace(source, ir::tree_sum_source(m, nt)).first;
+      it = texts.emplace(source, m.is_max ? ir::tree_max_source(m) : ir::tree_sum_source(m, nt)).first;
     }
     text = it->second;
   }
@@ -690,7 +690,7 @@ int sarek_hip_run_source(const char *source, int lang, const char *kernel_name, 
     if (!tag.empty()) {
       int rc = SAREK_HIP_OK;
       if (tag == "map_f32"            ? try_map(source, block, grid, args, n_args, nullptr, 0, nullptr, nullptr, &rc)
-          : tag == "tree_sum_map_f32" ? try_tree_map(source, block, grid, args, n_args, &rc)
+          : tag == "tree_sum_map_f32" || tag == "tree_max_map_f32" ? try_tree_map(source, block, grid, args, n_args, &rc)
                                       : try_specialised(tag, block, grid, args, n_args, &rc)) {
         t_last_path = tag;
         return rc;

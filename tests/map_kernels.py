@@ -160,3 +160,34 @@ def tree_near_misses():
     for _, text in out:
         assert text != sq
     return out
+
+
+def _max_tree_with(leaf_of, params, pad="(f32 -1000000.0)"):
+    """benchmarks/bench_reduction_max.ml:18-100 with `leaf_of(gid)` where it reads input[gid]."""
+    import os
+    ir = open(os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "ir", "reduction_max.ir")).read()
+    free = "(var Float.neg_infinity"
+    i = ir.index(free)
+    j = ir.index(")", i) + 1
+    ir = ir[:i] + pad + ir[j:]
+    gid = "(var gid 6 i32)"
+    old = f"(read input {gid})"
+    assert ir.count(old) == 1, ir
+    ir = ir.replace(old, leaf_of(gid))
+    head = ir[ir.index("(params"):ir.index("(locals)")]
+    return ir.replace(head, "(params " + " ".join(f"(param (var {n} {k} {t}))" for n, k, t in params) + ")\n ")
+
+
+def max_abs():
+    """max |x|: the infinity norm"""
+    return _max_tree_with(lambda g: f"(intr (Float32) fabs (read input {g}))",
+                          [("input", 1, "(vec f32)"), ("output", 2, "(vec f32)"), ("n", 3, "i32")], pad="(f32 0.0)")
+
+
+def max_abs_difference():
+    """max |x - y|"""
+    return _max_tree_with(lambda g: f"(intr (Float32) fabs (sub (read input {g}) (read y {g})))",
+                          [("input", 1, "(vec f32)"), ("y", 30, "(vec f32)"), ("output", 2, "(vec f32)"), ("n", 3, "i32")])
+
+
+MAX_TREES = {"max_abs": max_abs, "max_abs_difference": max_abs_difference}

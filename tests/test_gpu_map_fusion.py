@@ -6,7 +6,7 @@ import os
 import numpy as np
 import pytest
 
-from map_kernels import MAPS, TREES
+from map_kernels import MAPS, MAX_TREES, TREES
 
 pytestmark = pytest.mark.gpu
 
@@ -164,3 +164,36 @@ def test_tree_sum_with_an_expression_in_front(hip, sarek, torch_cuda, name, n):
     # a grid that is not exactly ceil(n / 256) blocks is left to the generated kernel
     out = V.create(V.float32, nblocks + 3)
     assert E.run_vectors(ir, tail(out), (256, 1, 1), (nblocks + 1, 1, 1)) == "jit"
+
+
+@pytest.mark.parametrize("n", [1, 255, 256, 257, 2047, 2048, 8193, 100003, (1 << 20) + 5])
+@pytest.mark.parametrize("name", sorted(MAX_TREES))
+def test_tree_maximum_with_an_expression_in_front(hip, sarek, torch_cuda, name, n):
+    """The tree's comparisons in the tree's order: the maxima are the generated kernel's bit for bit (NaNs and a
+    last block filled with the kernel's own fill value included), and the hand maximum's on the expression's values."""
+    torch = torch_cuda
+    E, V = sarek.Execute, sarek.Vector
+    rng = np.random.default_rng(n)
+    x = (rng.standard_normal(n) * 10.0 ** rng.integers(-2, 2, n)).astype(np.float32)
+    y = (rng.standard_normal(n) * 10.0 ** rng.integers(-2, 2, n)).astype(np.float32)
+    if n > 300:
+        x[17], x[n // 2], y[n - 3] = np.nan, np.inf, -np.inf
+    nblocks = (n + 255) // 256
+    if name == "max_abs":
+        values, pad, tail = np.abs(x), 0.0, lambda out: [E.Vec(V.of_array(x)), E.Vec(out), E.Int32(n)]
+    else:
+        values, pad = np.abs(x - y), -1000000.0
+        tail = lambda out: [E.Vec(V.of_array(x)), E.Vec(V.of_array(y)), E.Vec(out), E.Int32(n)]  # noqa: E731
+    ir = MAX_TREES[name]()
+
+    def run():
+        out = V.create(V.float32, nblocks + 3)
+        out.host[:] = -7.0
+        path = E.run_vectors(ir, tail(out), (256, 1, 1), (nblocks, 1, 1))
+        return path, out.to_array().copy()
+
+    (p_hand, got), (p_jit, want) = both_ways(hip, run)
+    assert (p_hand, p_jit) == ("tree_max_map_f32", "jit")
+    assert np.array_equal(got.view(np.uint32), want.view(np.uint32))
+    ref = hip.reduce_max_block256(torch.from_numpy(values).cuda(), pad=pad).cpu().numpy()
+    assert np.array_equal(got[:nblocks].view(np.uint32), ref.view(np.uint32))

@@ -2,7 +2,7 @@
 the tag never lands on a kernel outside the class.  No GPU needed."""
 import pytest
 
-from map_kernels import MAPS, TREES, near_misses, tree_near_misses
+from map_kernels import MAPS, MAX_TREES, TREES, near_misses, tree_near_misses
 
 MARK = "// sarek-hip-specialise: "
 
@@ -43,3 +43,13 @@ def test_the_reference_trees_keep_their_tags(hip):
 @pytest.mark.parametrize("name,ir", tree_near_misses(), ids=[n for n, _ in tree_near_misses()])
 def test_tree_near_misses_are_left_alone(hip, name, ir):
     assert not hip.generate_source(ir, block=(256, 1, 1)).startswith(MARK), name
+
+
+@pytest.mark.parametrize("name", sorted(MAX_TREES))
+def test_maximum_trees_with_an_expression_in_front_are_tagged(hip, name):
+    ir = MAX_TREES[name]()
+    assert hip.generate_source(ir, block=(256, 1, 1)).startswith(MARK + "tree_max_map_f32\n")
+    # "greater or equal" is another tree (it would pick another of two equal-comparing values, -0 and +0 say)
+    assert "(gt (var b" in ir
+    assert not hip.generate_source(ir.replace("(gt (var b", "(ge (var b", 1), block=(256, 1, 1)).startswith(MARK)
+    assert not hip.generate_source(ir.replace("(i32 32)", "(i32 16)", 1), block=(256, 1, 1)).startswith(MARK)
