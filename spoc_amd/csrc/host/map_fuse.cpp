@@ -6,6 +6,8 @@
 // the lowering prints it, applied to every element, and optionally the block-256 sums of the result (the reference's
 // tree kernel, benchmarks/bench_reduction.ml:62-96, one wave reduction per 256 elements) in the same pass.
 #include <algorithm>
+#include <cstdint>
+#include <cstdio>
 #include <optional>
 #include <string>
 #include <vector>
@@ -41,7 +43,7 @@ bool is_global_id(const ExprP &e) {
 // kernel bodies): a parameter of that name would be shadowed there, so such a kernel stays with the generated code.
 bool name_is_free(const std::string &n) {
   if (n.compare(0, 8, "sarek_f_") == 0 || (n.size() > 3 && n.compare(n.size() - 3, 3, "__e") == 0)) return false;
-  for (const char *own : {"u", "j", "i", "e", "v", "t", "o4"})
+  for (const char *own : {"u", "j", "i", "e", "v", "t", "q", "o4"})
     if (n == own) return false;
   return true;
 }
@@ -283,9 +285,14 @@ std::string formal_params(const MapKernel &m) {
 
 }  // namespace
 
-std::string map_source(const MapKernel &m, bool with_sums, bool nt_loads) {
+std::string map_source(const MapKernel &m, int reduce, bool nt_loads, uint32_t pad_bits) {
+  const bool with_sums = reduce == 1, with_max = reduce == 2;
+  // what slots past n count as: 0 in a sum, the maximum tree's fill value (its exact bits) in a maximum
+  char pad[48] = "0.f";
+  if (with_max) std::snprintf(pad, sizeof(pad), "__uint_as_float(0x%08xu)", static_cast<unsigned>(pad_bits));
   std::string actuals_tail;
   std::string o = prelude(m, with_sums, &actuals_tail);
+  if (with_max) o += "__device__ __forceinline__ float sarek_f_greater(float a, float b) { return b > a ? b : a; }\n";
   auto apply = [&](const std::string &value_of, const std::string &index) {
     return apply_call(m, actuals_tail, value_of, index);
   };
@@ -299,7 +306,7 @@ std::string map_source(const MapKernel &m, bool with_sums, bool nt_loads) {
   // a wave owns four consecutive KiB of every vector: slot u of lane l is float4 number base + 64 u
   o += "  const long long sarek_f_base = (long long)blockIdx.x * 1024 + (threadIdx.x >> 6) * 256 + (threadIdx.x & 63);\n"
        "  const bool sarek_f_full = sarek_f_base + 192 < sarek_f_n4;\n"
-       "  sarek_f_v4 sarek_f_r[4];\n  float sarek_f_extra[4] = {0.f, 0.f, 0.f, 0.f};\n";
+       "  sarek_f_v4 sarek_f_r[4];\n";
   for (size_t i = 0; i < m.inputs.size(); ++i)
     o += "  const sarek_f_v4* sarek_f_p" + std::to_string(i) + " = reinterpret_cast<const sarek_f_v4*>(" +
          m.params[m.inputs[i]].name + ");\n";
@@ -316,26 +323,43 @@ std::string map_source(const MapKernel &m, bool with_sums, bool nt_loads) {
        "        sarek_f_r[u][j] = " + apply("sarek_f_x@[u][j]", "(sarek_f_base + 64 * u) * 4 + j") + ";\n";
   o += "#pragma unroll\n    for (int u = 0; u < 4; ++u) __builtin_nontemporal_store(sarek_f_r[u], sarek_f_po + sarek_f_base + 64 * u);\n";
   o += "  } else {\n#pragma unroll\n    for (int u = 0; u < 4; ++u) {\n      const long long i = sarek_f_base + 64 * u;\n"
-       "      sarek_f_r[u] = sarek_f_v4{0.f, 0.f, 0.f, 0.f};\n      if (i < sarek_f_n4) {\n";
+       "      if (i < sarek_f_n4) {\n";
   for (size_t i = 0; i < m.inputs.size(); ++i)
     o += "        const sarek_f_v4 sarek_f_y" + std::to_string(i) + " = sarek_f_p" + std::to_string(i) + "[i];\n";
   o += "#pragma unroll\n        for (int j = 0; j < 4; ++j) sarek_f_r[u][j] = " + apply("sarek_f_y@[j]", "i * 4 + j") + ";\n"
-       "        sarek_f_po[i] = sarek_f_r[u];\n      }\n";
-  // the lane whose slot holds the end of the vector takes the one to three elements there
+       "        sarek_f_po[i] = sarek_f_r[u];\n      } else {\n";
+  // the slot that holds the end of the vector takes its one to three elements; everything past n is the pad
   {
     std::string a = "sarek_f_opaque(sarek_f_apply(";
-    for (int p : m.inputs) a += m.params[p].name + "[e], ";
-    a += actuals_tail + "(int)e))";
-    o += "      if (i == sarek_f_n4) {\n        for (long long e = sarek_f_n4 << 2; e < sarek_f_n; ++e) {\n"
-         "          const float v = " + a + ";\n          " + out + "[e] = v;\n          sarek_f_extra[u] += v;\n        }\n      }\n";
+    for (int p : m.inputs) a += m.params[p].name + "[sarek_f_k], ";
+    a += actuals_tail + "(int)sarek_f_k))";
+    o += "#pragma unroll\n        for (int e = 0; e < 4; ++e) {\n          const long long sarek_f_k = (i << 2) + e;\n"
+         "          sarek_f_r[u][e] = " + std::string(pad) + ";\n          if (sarek_f_k < sarek_f_n) {\n            sarek_f_r[u][e] = " + a +
+         ";\n            " + out + "[sarek_f_k] = sarek_f_r[u][e];\n          }\n        }\n      }\n";
   }
   o += "    }\n  }\n";
   if (with_sums) {
     o += "  const long long sarek_f_nblocks = (sarek_f_n + 255) >> 8;\n  float sarek_f_t[4];\n#pragma unroll\n"
-         "  for (int u = 0; u < 4; ++u)\n    sarek_f_t[u] = sarek_f_wave_sum(((sarek_f_r[u][0] + sarek_f_r[u][1]) + "
-         "(sarek_f_r[u][2] + sarek_f_r[u][3])) + sarek_f_extra[u]);\n"
+         "  for (int u = 0; u < 4; ++u)\n    sarek_f_t[u] = sarek_f_wave_sum((sarek_f_r[u][0] + sarek_f_r[u][1]) + "
+         "(sarek_f_r[u][2] + sarek_f_r[u][3]));\n"
          "  const long long sarek_f_j0 = (long long)blockIdx.x * 16 + (threadIdx.x >> 6) * 4;\n"
          "  if ((threadIdx.x & 63) == 0) {\n    if (sarek_f_j0 + 4 <= sarek_f_nblocks) {\n"
+         "      *reinterpret_cast<sarek_f_v4*>(sarek_f_partials + sarek_f_j0) = "
+         "sarek_f_v4{sarek_f_t[0], sarek_f_t[1], sarek_f_t[2], sarek_f_t[3]};\n    } else {\n#pragma unroll\n"
+         "      for (int u = 0; u < 4; ++u)\n        if (sarek_f_j0 + u < sarek_f_nblocks) sarek_f_partials[sarek_f_j0 + u] = sarek_f_t[u];\n"
+         "    }\n  }\n";
+  }
+  if (with_max) {
+    // the tree's comparisons in the tree's order: halves 128 .. 4 pair lane l with lanes l + 32 .. l + 1 component by
+    // component, halves 2 and 1 the four components of lane 0
+    o += "  const long long sarek_f_nblocks = (sarek_f_n + 255) >> 8;\n  float sarek_f_t[4];\n#pragma unroll\n"
+         "  for (int u = 0; u < 4; ++u) {\n    sarek_f_v4 sarek_f_w = sarek_f_r[u];\n#pragma unroll\n"
+         "    for (int sarek_f_h = 32; sarek_f_h >= 1; sarek_f_h >>= 1)\n#pragma unroll\n      for (int sarek_f_c = 0; sarek_f_c < 4; ++sarek_f_c) "
+         "sarek_f_w[sarek_f_c] = sarek_f_greater(sarek_f_w[sarek_f_c], __shfl_down(sarek_f_w[sarek_f_c], sarek_f_h, 64));\n"
+         "    sarek_f_t[u] = sarek_f_greater(sarek_f_greater(sarek_f_w[0], sarek_f_w[2]), sarek_f_greater(sarek_f_w[1], sarek_f_w[3]));\n  }\n"
+         "  const long long sarek_f_j0 = (long long)blockIdx.x * 16 + (threadIdx.x >> 6) * 4;\n"
+         "  if ((threadIdx.x & 63) == 0) {\n    if (sarek_f_j0 + 4 <= sarek_f_nblocks && "
+         "(reinterpret_cast<unsigned long long>(sarek_f_partials) & 15ull) == 0) {\n"
          "      *reinterpret_cast<sarek_f_v4*>(sarek_f_partials + sarek_f_j0) = "
          "sarek_f_v4{sarek_f_t[0], sarek_f_t[1], sarek_f_t[2], sarek_f_t[3]};\n    } else {\n#pragma unroll\n"
          "      for (int u = 0; u < 4; ++u)\n        if (sarek_f_j0 + u < sarek_f_nblocks) sarek_f_partials[sarek_f_j0 + u] = sarek_f_t[u];\n"
@@ -494,9 +518,9 @@ std::string tree_max_source(const MapKernel &m) {
        "        const long long i = (sarek_f_j0 + u) * 256 + sarek_f_lane + 64 * q;\n"
        "        sarek_f_w[u][q] = " + m.pad + ";\n        if (i < sarek_f_n) sarek_f_w[u][q] = " + a + ";\n      }\n  }\n"
        "#pragma unroll\n  for (int u = 0; u < 8; ++u) {\n    const float* v = sarek_f_w[u];\n"
-       "    float g = sarek_f_greater(sarek_f_greater(v[0], v[2]), sarek_f_greater(v[1], v[3]));\n"
-       "#pragma unroll\n    for (int half = 32; half >= 1; half >>= 1) g = sarek_f_greater(g, __shfl_down(g, half, 64));\n"
-       "    sarek_f_m[u] = g;\n  }\n  if (sarek_f_lane != 0) return;\n"
+       "    float sarek_f_g = sarek_f_greater(sarek_f_greater(v[0], v[2]), sarek_f_greater(v[1], v[3]));\n"
+       "#pragma unroll\n    for (int sarek_f_h = 32; sarek_f_h >= 1; sarek_f_h >>= 1) sarek_f_g = sarek_f_greater(sarek_f_g, __shfl_down(sarek_f_g, sarek_f_h, 64));\n"
+       "    sarek_f_m[u] = sarek_f_g;\n  }\n  if (sarek_f_lane != 0) return;\n"
        "  if (sarek_f_j0 + 8 <= sarek_f_nblocks && (reinterpret_cast<unsigned long long>(" + out + ") & 15ull) == 0) {\n"
        "    sarek_f_v4* o4 = reinterpret_cast<sarek_f_v4*>(" + out + " + sarek_f_j0);\n"
        "    o4[0] = sarek_f_v4{sarek_f_m[0], sarek_f_m[1], sarek_f_m[2], sarek_f_m[3]};\n"

@@ -1,5 +1,6 @@
 // Element-wise kernels recognised as a class and rebuilt in the stream kernels' shape (map_fuse.cpp).
 #pragma once
+#include <cstdint>
 #include <optional>
 #include <string>
 #include <vector>
@@ -29,9 +30,10 @@ struct MapKernel {
 std::optional<MapKernel> match_map(const Kernel &k);
 
 // HIP source of `sarek_map(<the kernel's parameters without the vector lengths>, float* partials)`: 256-thread
-// workgroups of 4096 elements, ceil(n / 4096) of them; with_sums also stores partials[j] = sum of out[256 j .. 256 j + 255]
-// in the order of the block-256 tree kernels.
-std::string map_source(const MapKernel &m, bool with_sums, bool nt_loads);
+// workgroups of 4096 elements, ceil(n / 4096) of them; reduce = 1 also stores partials[j] = sum of out[256 j .. 256 j + 255]
+// in the order of the hand block-256 sum, reduce = 2 their maximum by the tree's comparisons in the tree's order, slots
+// past n counting as the value with the bits pad_bits; 0 neither.
+std::string map_source(const MapKernel &m, int reduce, bool nt_loads, uint32_t pad_bits = 0);
 
 // The block-256 tree sum (benchmarks/bench_reduction.ml:62-96) with a pure element-wise expression where the
 // reference's kernel reads its input (the dot product of bench_dot_product.ml:16-54 is one such): `out` is then the

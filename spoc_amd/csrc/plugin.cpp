@@ -4,6 +4,7 @@
 // a source that starts with "// sarek-hip-specialise: <tag>" is served by the matching
 // hand-written kernel when the caller's launch geometry covers the whole problem the
 // way the generated kernel assumes; otherwise the text is JIT-compiled as it stands.
+#include <cstdio>
 #include <cstdlib>
 #include <cstring>
 #include <mutex>
@@ -89,7 +90,8 @@ bool covers_1d(const int block[3], const int grid[3], int64_t threads) {
 // launched right after it on the vector it writes) the sums leave in the same pass.  The text is compiled once per
 // kernel and variant.  Returns 1 when the launch (or the pair) was served, 0 to fall back.
 int try_map(const char *source, const int block[3], const int grid[3], const sarek_hip_arg *a, int na,
-            const sarek_hip_arg *red, int nred, const int rblock[3], const int rgrid[3], int *rc) {
+            const sarek_hip_arg *red, int nred, const int rblock[3], const int rgrid[3], int *rc, bool red_is_max = false,
+            uint32_t pad_bits = 0) {
   ir::MapKernel m;
   if (!find_generated_map(source, &m)) return 0;
   struct Slot {
@@ -147,7 +149,10 @@ int try_map(const char *source, const int block[3], const int grid[3], const sar
   const bool nt = static_cast<int64_t>(m.inputs.size()) * n * 4 > (int64_t{256} << 20);
   static std::mutex mu;
   static std::unordered_map<std::string, std::string> texts;   // "<variant><generated text>" -> rebuilt text
-  std::string key(1, static_cast<char>('0' + (red ? 2 : 0) + (nt ? 1 : 0)));
+  const int reduce = !red ? 0 : red_is_max ? 2 : 1;
+  char variant[16];
+  std::snprintf(variant, sizeof(variant), "%d%d%08x", reduce, nt ? 1 : 0, static_cast<unsigned>(red_is_max ? pad_bits : 0));
+  std::string key(variant);
   key += source;
   std::string text;
   {
@@ -155,7 +160,7 @@ int try_map(const char *source, const int block[3], const int grid[3], const sar
     auto it = texts.find(key);
     if (it == texts.end()) {
       if (texts.size() >= 1024) texts.clear();
-      it = texts.emplace(key, ir::map_source(m, red != nullptr, nt)).first;
+      it = texts.emplace(key, ir::map_source(m, reduce, nt, pad_bits)).first;
     }
     text = it->second;
   }
@@ -599,6 +604,20 @@ int try_specialised_pair(const std::string &tag0, const int block0[3], const int
   return 1;
 }
 
+// An element-wise kernel followed by the block-256 sum or maximum (fill value in the tag, as f32 bits) of its output
+int try_map_pair(const sarek_hip_launch &l0, const std::string &tag1, const sarek_hip_launch &l1, int *rc) {
+  if (tag1 == "reduce_sum_block256_f32")
+    return try_map(l0.source, l0.block, l0.grid, l0.args, l0.n_args, l1.args, l1.n_args, l1.block, l1.grid, rc);
+  if (tag1.compare(0, 24, "reduce_max_block256_f32:") == 0 && tag1.size() == 32) {
+    char *end = nullptr;
+    const unsigned long bits = std::strtoul(tag1.c_str() + 24, &end, 16);
+    if (*end != 0) return 0;
+    return try_map(l0.source, l0.block, l0.grid, l0.args, l0.n_args, l1.args, l1.n_args, l1.block, l1.grid, rc, true,
+                   static_cast<uint32_t>(bits));
+  }
+  return 0;
+}
+
 }  // namespace
 
 }  // namespace sarek_hip
@@ -633,8 +652,7 @@ int sarek_hip_run_sources(const sarek_hip_launch *launches, int n_launches, int 
       int rc = SAREK_HIP_OK;
       if (langs_ok && !tag0.empty() && !tag1.empty() && tag_is_ours(tag0, l0.source) && tag_is_ours(tag1, l1.source) &&
           (tag0 == "map_f32"
-               ? (tag1 == "reduce_sum_block256_f32" && try_map(l0.source, l0.block, l0.grid, l0.args, l0.n_args, l1.args,
-                                                               l1.n_args, l1.block, l1.grid, &rc))
+               ? try_map_pair(l0, tag1, l1, &rc)
                : try_specialised_pair(tag0, l0.block, l0.grid, l0.args, l0.n_args, tag1, l1.block, l1.grid, l1.args,
                                       l1.n_args, &rc))) {
         if (rc != SAREK_HIP_OK) return rc;

@@ -120,11 +120,6 @@ def test_pairs_the_fused_kernel_does_not_serve(hip, sarek):
                                                 (nblocks - 1, 1, 1))]) == ("map_f32;reduce_sum_block256_f32", 2)
     # a launch that does not reach every element runs as generated
     assert E.run_vectors(ir, args, (256, 1, 1), (nblocks - 1, 1, 1)) == "jit"
-    # a maximum behind a map is two launches (the fused pairs with a maximum are the triad's and the vector add's)
-    from test_ir_lowering import reduction_max_ir
-    reduction_max = reduction_max_ir()
-    path, launches = E.run_pipeline([(ir, args) + shape, (reduction_max, [E.Vec(out), E.Vec(sums), E.Int32(n)]) + shape])
-    assert launches == 2 and path.startswith("map_f32;reduce_max_block256_f32")
 
 
 @pytest.mark.parametrize("n", [1, 255, 256, 257, 2047, 2048, 8191, 8192, 8193, 100003, (1 << 20) + 5])
@@ -197,3 +192,28 @@ def test_tree_maximum_with_an_expression_in_front(hip, sarek, torch_cuda, name, 
     assert np.array_equal(got.view(np.uint32), want.view(np.uint32))
     ref = hip.reduce_max_block256(torch.from_numpy(values).cuda(), pad=pad).cpu().numpy()
     assert np.array_equal(got[:nblocks].view(np.uint32), ref.view(np.uint32))
+
+
+@pytest.mark.parametrize("n", [1, 255, 257, 4095, 4097, 100003, (1 << 20) + 5])
+@pytest.mark.parametrize("name", ["saxpy_with_let", "norm3", "scale"])
+def test_map_then_block_maximum_is_one_launch(hip, sarek, name, n):
+    """The maximum tree of bench_reduction_max.ml behind a map: the tree's comparisons in the tree's order, so the
+    maxima are the generated pair's bit for bit (NaNs from norm3's 0/0-free but inf-prone division included)."""
+    from test_ir_lowering import reduction_max_ir
+    E, V = sarek.Execute, sarek.Vector
+    ir, reduction_max = MAPS[name](), reduction_max_ir("(f32 -3.5)")
+    nblocks = (n + 255) // 256
+
+    def run():
+        args, out = arguments(sarek, name, n, np.random.default_rng(n))
+        maxima = V.create(V.float32, nblocks + 2)
+        maxima.host[:] = -7.0
+        stages = [(ir, args, (256, 1, 1), (nblocks, 1, 1)),
+                  (reduction_max, [E.Vec(out), E.Vec(maxima), E.Int32(n)], (256, 1, 1), (nblocks, 1, 1))]
+        return E.run_pipeline(stages), out.to_array().copy(), maxima.to_array().copy()
+
+    (fused, a_fused, m_fused), (jit, a_jit, m_jit) = both_ways(hip, run)
+    assert fused[1] == 1 and fused[0].startswith("map_f32+reduce_max_block256_f32:") and jit == ("jit;jit", 2)
+    assert np.array_equal(a_fused.view(np.uint32), a_jit.view(np.uint32))
+    assert np.array_equal(m_fused.view(np.uint32), m_jit.view(np.uint32))
+    assert np.all(m_fused[nblocks:] == -7.0)
