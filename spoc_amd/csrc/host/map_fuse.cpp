@@ -306,7 +306,7 @@ std::string map_source(const MapKernel &m, int reduce, bool nt_loads, uint32_t p
   // a wave owns four consecutive KiB of every vector: slot u of lane l is float4 number base + 64 u
   o += "  const long long sarek_f_base = (long long)blockIdx.x * 1024 + (threadIdx.x >> 6) * 256 + (threadIdx.x & 63);\n"
        "  const bool sarek_f_full = sarek_f_base + 192 < sarek_f_n4;\n"
-       "  sarek_f_v4 sarek_f_r[4];\n";
+       "  sarek_f_v4 sarek_f_r[4];\n  float sarek_f_extra[4] = {0.f, 0.f, 0.f, 0.f};\n";
   for (size_t i = 0; i < m.inputs.size(); ++i)
     o += "  const sarek_f_v4* sarek_f_p" + std::to_string(i) + " = reinterpret_cast<const sarek_f_v4*>(" +
          m.params[m.inputs[i]].name + ");\n";
@@ -323,25 +323,32 @@ std::string map_source(const MapKernel &m, int reduce, bool nt_loads, uint32_t p
        "        sarek_f_r[u][j] = " + apply("sarek_f_x@[u][j]", "(sarek_f_base + 64 * u) * 4 + j") + ";\n";
   o += "#pragma unroll\n    for (int u = 0; u < 4; ++u) __builtin_nontemporal_store(sarek_f_r[u], sarek_f_po + sarek_f_base + 64 * u);\n";
   o += "  } else {\n#pragma unroll\n    for (int u = 0; u < 4; ++u) {\n      const long long i = sarek_f_base + 64 * u;\n"
-       "      if (i < sarek_f_n4) {\n";
+       "      sarek_f_r[u] = sarek_f_v4{0.f, 0.f, 0.f, 0.f};\n      if (i < sarek_f_n4) {\n";
   for (size_t i = 0; i < m.inputs.size(); ++i)
     o += "        const sarek_f_v4 sarek_f_y" + std::to_string(i) + " = sarek_f_p" + std::to_string(i) + "[i];\n";
   o += "#pragma unroll\n        for (int j = 0; j < 4; ++j) sarek_f_r[u][j] = " + apply("sarek_f_y@[j]", "i * 4 + j") + ";\n"
-       "        sarek_f_po[i] = sarek_f_r[u];\n      } else {\n";
-  // the slot that holds the end of the vector takes its one to three elements; everything past n is the pad
+       "        sarek_f_po[i] = sarek_f_r[u];\n      }";
   {
     std::string a = "sarek_f_opaque(sarek_f_apply(";
     for (int p : m.inputs) a += m.params[p].name + "[sarek_f_k], ";
     a += actuals_tail + "(int)sarek_f_k))";
-    o += "#pragma unroll\n        for (int e = 0; e < 4; ++e) {\n          const long long sarek_f_k = (i << 2) + e;\n"
-         "          sarek_f_r[u][e] = " + std::string(pad) + ";\n          if (sarek_f_k < sarek_f_n) {\n            sarek_f_r[u][e] = " + a +
-         ";\n            " + out + "[sarek_f_k] = sarek_f_r[u][e];\n          }\n        }\n      }\n";
+    if (with_max) {
+      // the slot that holds the end of the vector takes its one to three elements; everything past n is the fill value
+      o += " else {\n#pragma unroll\n        for (int e = 0; e < 4; ++e) {\n          const long long sarek_f_k = (i << 2) + e;\n"
+           "          sarek_f_r[u][e] = " + std::string(pad) + ";\n          if (sarek_f_k < sarek_f_n) {\n            sarek_f_r[u][e] = " + a +
+           ";\n            " + out + "[sarek_f_k] = sarek_f_r[u][e];\n          }\n        }\n      }\n";
+    } else {
+      // the lane whose slot holds the end of the vector takes the one to three elements there, summed apart (kept
+      // out of the vector registers: folding them into r measured 2.7 % slower on the whole kernel)
+      o += "\n      if (i == sarek_f_n4) {\n        for (long long sarek_f_k = sarek_f_n4 << 2; sarek_f_k < sarek_f_n; ++sarek_f_k) {\n"
+           "          const float v = " + a + ";\n          " + out + "[sarek_f_k] = v;\n          sarek_f_extra[u] += v;\n        }\n      }\n";
+    }
   }
   o += "    }\n  }\n";
   if (with_sums) {
     o += "  const long long sarek_f_nblocks = (sarek_f_n + 255) >> 8;\n  float sarek_f_t[4];\n#pragma unroll\n"
-         "  for (int u = 0; u < 4; ++u)\n    sarek_f_t[u] = sarek_f_wave_sum((sarek_f_r[u][0] + sarek_f_r[u][1]) + "
-         "(sarek_f_r[u][2] + sarek_f_r[u][3]));\n"
+         "  for (int u = 0; u < 4; ++u)\n    sarek_f_t[u] = sarek_f_wave_sum(((sarek_f_r[u][0] + sarek_f_r[u][1]) + "
+         "(sarek_f_r[u][2] + sarek_f_r[u][3])) + sarek_f_extra[u]);\n"
          "  const long long sarek_f_j0 = (long long)blockIdx.x * 16 + (threadIdx.x >> 6) * 4;\n"
          "  if ((threadIdx.x & 63) == 0) {\n    if (sarek_f_j0 + 4 <= sarek_f_nblocks) {\n"
          "      *reinterpret_cast<sarek_f_v4*>(sarek_f_partials + sarek_f_j0) = "
