@@ -497,11 +497,11 @@ std::optional<MapKernel> match_tree(const Kernel &k, bool is_max) {
 std::optional<MapKernel> match_tree_sum(const Kernel &k) { return match_tree(k, false); }
 std::optional<MapKernel> match_tree_max(const Kernel &k) { return match_tree(k, true); }
 
-// The hand block-256 maximum's shape: lane l of a wave holds elements l, l + 64, l + 128, l + 192 of a block, eight
-// blocks per wave, and the comparisons are the tree's in the tree's order with its strict ">" (halves 128 and 64
-// inside the lane, 32 .. 1 across lanes), so NaNs and signed zeros come out as from the tree; slots past n hold the
-// kernel's fill value.
-std::string tree_max_source(const MapKernel &m) {
+// One input: lane l of a wave holds elements l, l + 64, l + 128, l + 192 of a block (the hand maximum's layout: two
+// comparisons inside the lane, then six across lanes per block; with 128-bit loads the same tree needs 24 cross-lane
+// steps per block, and a 4-byte-per-element kernel is bound by them: 260 against 163 us at n = 2^28).
+namespace {
+std::string tree_max_source_scalar_loads(const MapKernel &m) {
   std::string actuals_tail;
   std::string o = prelude(m, false, &actuals_tail);
   const std::string out = m.params[m.out].name;
@@ -528,6 +528,71 @@ std::string tree_max_source(const MapKernel &m) {
        "    float sarek_f_g = sarek_f_greater(sarek_f_greater(v[0], v[2]), sarek_f_greater(v[1], v[3]));\n"
        "#pragma unroll\n    for (int sarek_f_h = 32; sarek_f_h >= 1; sarek_f_h >>= 1) sarek_f_g = sarek_f_greater(sarek_f_g, __shfl_down(sarek_f_g, sarek_f_h, 64));\n"
        "    sarek_f_m[u] = sarek_f_g;\n  }\n  if (sarek_f_lane != 0) return;\n"
+       "  if (sarek_f_j0 + 8 <= sarek_f_nblocks && (reinterpret_cast<unsigned long long>(" + out + ") & 15ull) == 0) {\n"
+       "    sarek_f_v4* o4 = reinterpret_cast<sarek_f_v4*>(" + out + " + sarek_f_j0);\n"
+       "    o4[0] = sarek_f_v4{sarek_f_m[0], sarek_f_m[1], sarek_f_m[2], sarek_f_m[3]};\n"
+       "    o4[1] = sarek_f_v4{sarek_f_m[4], sarek_f_m[5], sarek_f_m[6], sarek_f_m[7]};\n  } else {\n"
+       "#pragma unroll\n    for (int u = 0; u < 8; ++u)\n      if (sarek_f_j0 + u < sarek_f_nblocks) " + out + "[sarek_f_j0 + u] = sarek_f_m[u];\n  }\n}\n";
+  return o;
+}
+
+}  // namespace
+
+// The maximum tree in the block-256 sum's load shape: lane l of a wave holds elements 4l .. 4l+3 of a block (128-bit
+// loads, eight blocks per wave, all asked for before the first comparison), and the comparisons are the tree's in
+// the tree's order with its strict ">" (halves 128 .. 4 across lanes component by component, 2 and 1 inside lane 0),
+// so NaNs and signed zeros come out as from the tree; slots past n hold the kernel's fill value.  Two or three inputs:
+// the loads are what counts there (339 against 359 us for max |x - y| at n = 2^28).
+std::string tree_max_source(const MapKernel &m) {
+  if (m.inputs.size() == 1) return tree_max_source_scalar_loads(m);
+  std::string actuals_tail;
+  std::string o = prelude(m, false, &actuals_tail);
+  const std::string out = m.params[m.out].name;
+  // (comparisons do not contract with anything: the element's value needs no asm in front of them)
+  auto apply = [&](const std::string &value_of, const std::string &index) {
+    std::string a = "sarek_f_apply(";
+    for (size_t i = 0; i < m.inputs.size(); ++i) {
+      std::string v = value_of;
+      v.replace(v.find('@'), 1, std::to_string(i));
+      a += v + ", ";
+    }
+    return a + actuals_tail + "(int)(" + index + "))";
+  };
+  o += "__device__ __forceinline__ float sarek_f_greater(float a, float b) { return b > a ? b : a; }\n"
+       // lane l holds elements 4l .. 4l+3 of a block: halves 128 .. 4 pair lane l with lanes l + 32 .. l + 1 component
+       // by component, halves 2 and 1 the four components of lane 0
+       "__device__ __forceinline__ float sarek_f_tree_max(sarek_f_v4 w) {\n#pragma unroll\n"
+       "  for (int h = 32; h >= 1; h >>= 1)\n#pragma unroll\n    for (int c = 0; c < 4; ++c) "
+       "w[c] = sarek_f_greater(w[c], __shfl_down(w[c], h, 64));\n"
+       "  return sarek_f_greater(sarek_f_greater(w[0], w[2]), sarek_f_greater(w[1], w[3]));\n}\n";
+  o += "extern \"C\" __global__ __launch_bounds__(256) void sarek_tree(" + formal_params(m);
+  o.resize(o.size() - 2);
+  o += ") {\n  const long long sarek_f_n = " + m.params[m.n].name + ", sarek_f_nblocks = (sarek_f_n + 255) >> 8;\n"
+       "  const int sarek_f_lane = threadIdx.x & 63;\n"
+       "  const long long sarek_f_j0 = ((long long)blockIdx.x * 4 + (threadIdx.x >> 6)) * 8;\n"
+       "  if (sarek_f_j0 >= sarek_f_nblocks) return;\n  float sarek_f_m[8];\n"
+       "  if ((sarek_f_j0 + 8) * 256 <= sarek_f_n) {\n";
+  for (size_t i = 0; i < m.inputs.size(); ++i) {
+    const std::string is = std::to_string(i), name = m.params[m.inputs[i]].name;
+    o += "    sarek_f_v4 sarek_f_x" + is + "[8];\n#pragma unroll\n    for (int u = 0; u < 8; ++u) sarek_f_x" + is +
+         "[u] = __builtin_nontemporal_load(reinterpret_cast<const sarek_f_v4*>(" + name +
+         " + (sarek_f_j0 + u) * 256) + sarek_f_lane);\n";
+  }
+  o += "#pragma unroll\n    for (int u = 0; u < 8; ++u) {\n      sarek_f_v4 sarek_f_w;\n#pragma unroll\n"
+       "      for (int j = 0; j < 4; ++j) sarek_f_w[j] = " +
+       apply("sarek_f_x@[u][j]", "(sarek_f_j0 + u) * 256 + sarek_f_lane * 4 + j") +
+       ";\n      sarek_f_m[u] = sarek_f_tree_max(sarek_f_w);\n    }\n  } else {\n";
+  {
+    // the group that holds the end of the input: slots past n hold the kernel's fill value
+    std::string a = "sarek_f_apply(";
+    for (int p : m.inputs) a += m.params[p].name + "[sarek_f_k], ";
+    a += actuals_tail + "(int)sarek_f_k)";
+    o += "#pragma unroll\n    for (int u = 0; u < 8; ++u) {\n      sarek_f_v4 sarek_f_w;\n#pragma unroll\n"
+         "      for (int j = 0; j < 4; ++j) {\n        const long long sarek_f_k = (sarek_f_j0 + u) * 256 + sarek_f_lane * 4 + j;\n"
+         "        sarek_f_w[j] = " + m.pad + ";\n        if (sarek_f_k < sarek_f_n) sarek_f_w[j] = " + a + ";\n      }\n"
+         "      sarek_f_m[u] = sarek_f_tree_max(sarek_f_w);\n    }\n  }\n";
+  }
+  o += "  if (sarek_f_lane != 0) return;\n"
        "  if (sarek_f_j0 + 8 <= sarek_f_nblocks && (reinterpret_cast<unsigned long long>(" + out + ") & 15ull) == 0) {\n"
        "    sarek_f_v4* o4 = reinterpret_cast<sarek_f_v4*>(" + out + " + sarek_f_j0);\n"
        "    o4[0] = sarek_f_v4{sarek_f_m[0], sarek_f_m[1], sarek_f_m[2], sarek_f_m[3]};\n"
