@@ -236,6 +236,15 @@ typedef struct {
  * Writes at most out_len bytes incl. NUL; *needed gets the full size.          */
 int sarek_hip_generate_source(const char *ir_text, const int block[3], char *out, size_t out_len,
                               size_t *needed);
+/* The text run_source compiles in place of the generated kernel when the IR is of one of the classes
+ * it rebuilds from the kernel's own expression: an element-wise kernel (reduce = 0: alone, 1: with the
+ * block-256 sums of its output, 2: with their maxima, slots past n counting as the f32 with the bits
+ * pad_bits), or a block-256 tree sum / maximum with an expression where the reference's kernels
+ * (benchmarks/bench_reduction.ml:62-96, bench_reduction_max.ml:18-100) read their input (reduce and
+ * pad_bits ignored).  For diagnostics and for compiling the texts ahead of time; no counterpart in the
+ * reference.  SAREK_HIP_E_UNSUPPORTED when the IR is of no such class.  Buffer convention as above.     */
+int sarek_hip_rebuilt_source(const char *ir_text, int reduce, uint32_t pad_bits, char *out, size_t out_len,
+                             size_t *needed);
 
 /* Compile (cached) + bind + launch on the default stream.  Only
  * SAREK_HIP_LANG_HIP_SOURCE and SAREK_HIP_LANG_CUDA_SOURCE (treated as HIP

@@ -145,6 +145,9 @@ let () = seal arg
 let generate_source =
   bind "sarek_hip_generate_source"
     (string @-> ptr int @-> ptr char @-> size_t @-> ptr size_t @-> returning int)
+let rebuilt_source =
+  bind "sarek_hip_rebuilt_source"
+    (string @-> int @-> uint32_t @-> ptr char @-> size_t @-> ptr size_t @-> returning int)
 let run_source =
   bind "sarek_hip_run_source"
     (string @-> int @-> string @-> ptr int @-> ptr int @-> int @-> ptr arg @-> int

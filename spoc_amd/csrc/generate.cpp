@@ -80,3 +80,28 @@ extern "C" int sarek_hip_generate_source(const char *ir_text, const int block[3]
   }
   return SAREK_HIP_OK;
 }
+
+extern "C" int sarek_hip_rebuilt_source(const char *ir_text, int reduce, uint32_t pad_bits, char *out, size_t out_len,
+                                        size_t *needed) {
+  if (!ir_text) return fail(SAREK_HIP_E_INVALID_ARG, "rebuilt_source: NULL IR text");
+  if (reduce < 0 || reduce > 2) return fail(SAREK_HIP_E_INVALID_ARG, "rebuilt_source: reduce must be 0, 1 or 2");
+  std::string src;
+  try {
+    ir::Kernel k = ir::parse_kernel(ir_text);
+    if (!ir::recognise(k).empty())
+      return fail(SAREK_HIP_E_UNSUPPORTED, "rebuilt_source: a hand-written kernel serves this IR");
+    if (auto m = ir::match_map(k)) src = ir::map_source(*m, reduce, true, pad_bits);
+    else if (auto t = ir::match_tree_sum(k)) src = ir::tree_sum_source(*t, true);
+    else if (auto x = ir::match_tree_max(k)) src = ir::tree_max_source(*x);
+    else return fail(SAREK_HIP_E_UNSUPPORTED, "rebuilt_source: the IR is of none of the rebuilt classes");
+  } catch (const ir::ParseError &e) {
+    return fail(SAREK_HIP_E_PARSE, "%s", e.what());
+  } catch (const std::exception &e) {
+    return fail(SAREK_HIP_E_CODEGEN, "rebuilt_source: %s", e.what());
+  }
+  if (needed) *needed = src.size() + 1;
+  if (!out || out_len < src.size() + 1)
+    return fail(SAREK_HIP_E_BUFFER_TOO_SMALL, "rebuilt_source: output needs %zu bytes", src.size() + 1);
+  std::memcpy(out, src.c_str(), src.size() + 1);
+  return SAREK_HIP_OK;
+}

@@ -118,6 +118,7 @@ SYMBOLS = {
     "sarek_hip_kernel_destroy": (_i, [_vp]),
     "sarek_hip_kernel_launch": (_i, [_vp, _uint3, _uint3, C.c_uint, _vp, C.POINTER(_vp), _i]),
     "sarek_hip_generate_source": (_i, [C.c_char_p, _int3, C.c_char_p, _sz, C.POINTER(_sz)]),
+    "sarek_hip_rebuilt_source": (_i, [C.c_char_p, _i, C.c_uint32, C.c_char_p, _sz, C.POINTER(_sz)]),
     "sarek_hip_run_source": (_i, [C.c_char_p, _i, C.c_char_p, _int3, _int3, _i, C.POINTER(Arg), _i]),
     "sarek_hip_set_specialisation": (_i, [_i]),
     "sarek_hip_last_run_path": (C.c_char_p, []),
@@ -735,6 +736,19 @@ def run_sources(launches):
     check(lib.sarek_hip_run_sources(arr, len(launches), C.byref(made), C.byref(done)))
     assert done.value == len(launches)
     return lib.sarek_hip_last_run_path().decode(), made.value
+
+
+def rebuilt_source(ir_text, reduce=0, pad_bits=0):
+    """The text run_source compiles for an IR of one of the rebuilt classes (an element-wise kernel, a tree sum or
+    maximum with an expression in front); raises SarekHipError (unsupported) for any other IR."""
+    needed = C.c_size_t(0)
+    buf = C.create_string_buffer(1 << 16)
+    rc = lib.sarek_hip_rebuilt_source(ir_text.encode(), reduce, pad_bits, buf, len(buf), C.byref(needed))
+    if rc == E_BUFFER_TOO_SMALL:
+        buf = C.create_string_buffer(needed.value + 1)
+        rc = lib.sarek_hip_rebuilt_source(ir_text.encode(), reduce, pad_bits, buf, len(buf), C.byref(needed))
+    check(rc)
+    return buf.value.decode()
 
 
 def generate_source(ir_text, block=None):

@@ -53,3 +53,40 @@ def test_maximum_trees_with_an_expression_in_front_are_tagged(hip, name):
     assert "(gt (var b" in ir
     assert not hip.generate_source(ir.replace("(gt (var b", "(ge (var b", 1), block=(256, 1, 1)).startswith(MARK)
     assert not hip.generate_source(ir.replace("(i32 32)", "(i32 16)", 1), block=(256, 1, 1)).startswith(MARK)
+
+
+def _compiles_for_gfx950(tmp_path, name, text):
+    """hipcc cross-compiles without a GPU: the rebuilt text must be a complete HIP program for the target."""
+    import subprocess
+    src = tmp_path / (name + ".hip")
+    src.write_text("#include <hip/hip_runtime.h>\n" + text)       # what hiprtc provides without being asked
+    res = subprocess.run(["/opt/rocm/bin/hipcc", "--offload-arch=gfx950", "-O3", "-std=c++17", "-Xclang", "-target-feature",
+                          "-Xclang", "-packed-fp32-ops", "--cuda-device-only", "-c", str(src), "-o", str(tmp_path / (name + ".o"))],
+                         capture_output=True, text=True)
+    errors = [line for line in res.stderr.splitlines() if "error" in line and "packed-fp32-ops" not in line]
+    assert res.returncode == 0 and not errors, res.stderr[-2000:]
+
+
+def test_every_rebuilt_text_compiles_for_the_target(hip, tmp_path):
+    """What run_source would hand to hiprtc on the GPU box, compiled here: every map alone, with block sums and with
+    block maxima, every tree sum and maximum."""
+    for name in sorted(MAPS):
+        for reduce, pad in ((0, 0), (1, 0), (2, 0xC0600000)):
+            text = hip.rebuilt_source(MAPS[name](), reduce, pad)
+            assert 'extern "C" __global__' in text and "sarek_map(" in text
+            assert ("sarek_f_wave_sum" in text) == (reduce == 1) and ("0xc0600000u" in text) == (reduce == 2)
+            _compiles_for_gfx950(tmp_path, f"{name}_{reduce}", text)
+    for name, make in sorted({**TREES, **MAX_TREES}.items()):
+        text = hip.rebuilt_source(make())
+        assert "sarek_tree(" in text
+        _compiles_for_gfx950(tmp_path, name, text)
+
+
+def test_rebuilt_source_refuses_everything_else(hip):
+    from spoc_amd import reference_kernels as rk
+    for ir in (rk.stream_triad(), rk.tree(False), near_misses()[0][1], rk.histogram()):
+        with pytest.raises(hip.SarekHipError) as err:
+            hip.rebuilt_source(ir)
+        assert err.value.status == hip.E_UNSUPPORTED
+    with pytest.raises(hip.SarekHipError):
+        hip.rebuilt_source(MAPS["scale"](), reduce=3)

@@ -47,7 +47,7 @@ def header_prototypes():
 
 
 OCAML_SCALARS = {"int": "int", "uint": "unsigned", "uchar": "unsigned char", "size_t": "size_t", "int64_t": "int64_t",
-                 "int32_t": "int32_t", "uint64_t": "uint64_t", "uint16_t": "uint16_t", "float": "float",
+                 "int32_t": "int32_t", "uint64_t": "uint64_t", "uint32_t": "uint32_t", "uint16_t": "uint16_t", "float": "float",
                  "double": "double", "char": "char", "void": "void", "string": "char *",
                  "arg": "sarek_hip_arg", "launch": "sarek_hip_launch", "device_info": "sarek_hip_device_info"}
 
