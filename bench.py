@@ -18,7 +18,9 @@ Timing mirrors the reference's benches (warmup, then timed iterations, each laun
 waited for; benchmarks/bench_stream_triad.ml:76-116): ms_per_step is the wall time of the K
 timed iterations over K, ms_per_step_stats their min / median / avg / max.  The kernel time
 used for the roofline comes from HIP events recorded round the dominant launch on the launch
-stream; gpu_ms_per_step_back_to_back is the same step launched K times with one wait at the end.
+stream, in a second round of K steps right after the timed ones (so that the handling of the events
+is not part of ms_per_step); gpu_ms_per_step_back_to_back is the same step launched K times with one
+wait at the end.
 The warmup is W steps and at least --warmup-ms (60 ms) of them: after a pause the clocks of a
 power-limited kernel need 30-40 ms of load to settle (--trace-launches shows the curve).
 """
@@ -176,8 +178,7 @@ def make_workload(name, torch, hip):
         tail = Launch(hip, lib.sarek_hip_fold_partials_f64, vout.device_ptr, n // 256, total.data_ptr(), None)
         info = dict(metric="fused triad+sum GB/s", unit="GB/s", dtype="f32",
                     work=12.0 * n, work_unit=1e9, bound="hbm", peak=PEAK_HBM_GBS,
-                    kernel="triad_kernel<SUM_BLOCK256, nt> (then the fold of the 2^20 block sums: fold_pieces_kernel, "
-                           "fold_stage_kernel)",
+                    kernel="triad_kernel<SUM_BLOCK256, nt> (then the fold of the 2^20 block sums: fold_onepass_kernel)",
                     route="Execute.run_pipeline [stream_triad IR; block-256 reduction IR], then sarek_hip_fold_partials_f64",
                     config={"workload": "fused stream triad + sum, a=b+3c, sum(a)", "n": n,
                             "algorithmic_bytes": 12 * n})
@@ -492,22 +493,30 @@ def measure(name, torch, hip, steps, warmup):
         sync()
         done += 1
     walls, kerns = [], []
+    region = Events(hip, stream)                 # one pair of events round the whole timed region
     t0 = time.perf_counter()
+    region.start()
     for _ in range(steps):
         w0 = time.perf_counter()
+        main()
+        if tail:
+            tail()
+        sync()
+        walls.append((time.perf_counter() - w0) * 1e3)
+    wall_ms = (time.perf_counter() - t0) * 1e3
+    region_ms = region.stop_ms()
+    # the dominant kernel's own duration: the same steps once more, HIP events round its launch
+    for _ in range(steps):
         ev.start()
         main()
         hip.check(hip.lib.sarek_hip_event_record(ev.e1, stream))
         if tail:
             tail()
         sync()
-        walls.append((time.perf_counter() - w0) * 1e3)
         ms = C.c_float(0)
         hip.check(hip.lib.sarek_hip_event_elapsed_ms(ev.e0, ev.e1, C.byref(ms)))
         kerns.append(float(ms.value))
-    sync()
     kerns_in_order = list(kerns)
-    wall_ms = (time.perf_counter() - t0) * 1e3
     ms_per_step = wall_ms / steps
     # second figure: the same launches back to back, one wait at the end (hotter: under the package power
     # limit the 16-bit GEMMs run slower this way)
@@ -531,6 +540,7 @@ def measure(name, torch, hip, steps, warmup):
                      "frac": round(achieved / info["peak"], 4),
                      "traffic": MEASURED_TRAFFIC_BYTES.get(name),
                      "kernel": info["kernel"], "kernel_ms": round(kernel_ms, 5), "kernel_ms_stats": stats(kerns),
+                     "timed_region_ms_per_step_by_events": round(region_ms / steps, 5),
                      "frac_back_to_back": round(info["work"] / (back_to_back_ms * 1e-3) / info["work_unit"] / info["peak"], 4)},
     }
     res["warmup_steps_done"] = done

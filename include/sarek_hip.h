@@ -487,7 +487,7 @@ int sarek_hip_triad_block256_max_f32(float *a, const float *b, const float *c, f
  * device's array: calls that overlap in time on one device (different streams, or different host
  * threads without ordering between their streams) race on it; calls on one stream do not.  The
  * first call on a device looks the array's address up (hipGetSymbolAddress); make that call
- * outside a stream capture.                                                                     */
+ * outside a stream capture (under one it is refused with SAREK_HIP_E_UNSUPPORTED).              */
 int64_t sarek_hip_triad_sum_static_max_n(void);
 int sarek_hip_triad_sum_f32_static(float *a, const float *b, const float *c, float s, int64_t n,
                                    double *sum_out, sarek_hip_stream stream);
@@ -506,10 +506,11 @@ int sarek_hip_dot_block256_f32(const float *a, const float *b, float *out, int64
 int sarek_hip_reduce_max_block256_f32(const float *in, float *out, int64_t n, float pad,
                                       sarek_hip_stream stream);
 /* *sum_out = double fold of partials[0..count) in an order fixed by count and the pointer's
- * alignment (host fold of benchmarks/bench_reduction.ml:154-160, kept on device).  From 2^17
- * partials on, 256 workgroups fold a piece each into a 2 KiB array inside the library's device
- * image and one more adds those up: such long folds that overlap in time on one device (different
- * streams) race on that array; folds on one stream do not.                              */
+ * alignment (host fold of benchmarks/bench_reduction.ml:154-160, kept on device): one launch.  From
+ * 2^17 partials on, 256 workgroups fold a piece each into a stage inside the library's device image
+ * and the one that finishes last adds those up in index order.  Every (device, stream) gets a stage of
+ * its own (16 per device), so long folds on different streams do not meet; a stream beyond the
+ * sixteenth, and a first long fold on a device made under stream capture, fold with one workgroup.  */
 int sarek_hip_fold_partials_f64(const float *partials, int64_t count, double *sum_out,
                                 sarek_hip_stream stream);
 

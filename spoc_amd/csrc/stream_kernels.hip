@@ -8,11 +8,15 @@
 // grid-stride loop, which measured ~8 % faster on MI355X than any persistent-grid shape
 // (the hardware dispatcher balances the 8 XCDs better than a fixed stride does).  Sums go
 // lane -> DPP wave reduction -> LDS across the waves of a block -> one f32 partial per
-// block -> a one-workgroup fold kernel in double (fixed order).  Folding inside the triad
+// block -> a fold kernel in double (fixed order; long folds: 256 workgroups, the last to finish adds
+// their sums).  Folding inside the triad
 // kernel ("last workgroup to arrive") was measured and rejected: on this multi-XCD chip a
 // device-scope fence writes back a whole L2 (7x slower) and publishing the partials with
 // device-scope atomics instead still cost 25 % of the bandwidth.
 #include <atomic>
+#include <map>
+#include <mutex>
+#include <utility>
 
 #include "common.hpp"
 #include "tunables.hpp"
@@ -257,28 +261,44 @@ __global__ __launch_bounds__(1024) void fold_kernel(const float *__restrict__ pa
   if (threadIdx.x == 0) *out = t;
 }
 
-// Long inputs in two steps: workgroup g sums the pieces [g*piece, (g+1)*piece) into stage[g], then
-// one workgroup adds the stage up in index order.  `piece` is a multiple of 4, so every
-// workgroup sees its piece at the alignment of the whole.
+// Long inputs in one launch: workgroup g sums the piece [g*piece, (g+1)*piece) into slot->stage[g] and takes a
+// ticket; the workgroup that takes the last one adds the stage up in index order (a fixed order whichever
+// workgroup that is) and puts the ticket counter back to zero for the next launch.  `piece` is a multiple of
+// 4, so every workgroup sees its piece at the alignment of the whole.  The stage values cross the device as
+// device-scope atomic stores and loads, ordered by the ticket's release / acquire: in a kernel this small the
+// L2s hold next to nothing that the release has to write back.
 constexpr int kFoldGroups = 256;
-__global__ __launch_bounds__(1024) void fold_pieces_kernel(const float *__restrict__ partials, int64_t count,
-                                                           int64_t piece, double *__restrict__ stage) {
+struct FoldSlot {
+  double stage[kFoldGroups];
+  unsigned ticket;
+  unsigned unused[63];
+};
+__global__ __launch_bounds__(1024) void fold_onepass_kernel(const float *__restrict__ partials, int64_t count,
+                                                            int64_t piece, FoldSlot *__restrict__ slot,
+                                                            double *__restrict__ out) {
   const int64_t lo = static_cast<int64_t>(blockIdx.x) * piece;
   const int64_t len = lo >= count ? 0 : (count - lo < piece ? count - lo : piece);
   const double t = fold_block(partials + lo, len);
-  if (threadIdx.x == 0) stage[blockIdx.x] = t;
-}
-
-__global__ __launch_bounds__(kFoldGroups) void fold_stage_kernel(const double *__restrict__ stage,
-                                                                 double *__restrict__ out) {
+  __shared__ bool last;
+  if (threadIdx.x == 0) {
+    __hip_atomic_store(&slot->stage[blockIdx.x], t, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    const unsigned before = __hip_atomic_fetch_add(&slot->ticket, 1u, __ATOMIC_ACQ_REL, __HIP_MEMORY_SCOPE_AGENT);
+    last = before == gridDim.x - 1;
+  }
+  __syncthreads();
+  if (!last) return;
   __shared__ double sh[kFoldGroups];
-  sh[threadIdx.x] = stage[threadIdx.x];
+  if (threadIdx.x < kFoldGroups)
+    sh[threadIdx.x] = __hip_atomic_load(&slot->stage[threadIdx.x], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
   __syncthreads();
   for (int half = kFoldGroups / 2; half >= 1; half >>= 1) {
     if (static_cast<int>(threadIdx.x) < half) sh[threadIdx.x] += sh[threadIdx.x + half];
     __syncthreads();
   }
-  if (threadIdx.x == 0) *out = sh[0];
+  if (threadIdx.x == 0) {
+    *out = sh[0];
+    __hip_atomic_store(&slot->ticket, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  }
 }
 
 // Per-256-element-block kernels: out[j] = reduction of in[256j .. 256j+255].  A wave takes
@@ -559,25 +579,41 @@ __global__ void store_f64_kernel(double *p, double v) { *p = v; }
 constexpr int64_t kScratchFloats = int64_t{1} << 19;
 static __device__ __align__(256) float scratch[kScratchFloats];
 
-// Stage of a long fold: one double per workgroup of fold_pieces_kernel (2 KiB per device).
-static __device__ __align__(256) double fold_stage[sarek_hip::kFoldGroups];
+// Stages of long folds: kFoldSlots slots of one double per workgroup of fold_onepass_kernel and a ticket counter
+// (36 KiB per device).  The counters start at zero (the image's initial value) and every launch leaves its own at zero.
+constexpr int kFoldSlots = 16;
+static __device__ __align__(256) sarek_hip::FoldSlot fold_slots[kFoldSlots];
 
 namespace sarek_hip {
 namespace {
 constexpr int kMaxDevices = 64;
 std::atomic<float *> g_scratch_addr[kMaxDevices];
-std::atomic<double *> g_fold_stage_addr[kMaxDevices];
+std::atomic<FoldSlot *> g_fold_slots_addr[kMaxDevices];
+
+bool capturing(hipStream_t st) {
+  hipStreamCaptureStatus status = hipStreamCaptureStatusNone;
+  if (hipStreamIsCapturing(st, &status) != hipSuccess) {
+    (void)hipGetLastError();
+    return true;   // treated as the cautious case
+  }
+  return status != hipStreamCaptureStatusNone;
+}
 
 // Device address of a file-scope __device__ array on the current device, looked up once per
-// device: every device holds its own copy of the array at its own address.
+// device: every device holds its own copy of the array at its own address.  The lookup is not
+// allowed while `st` records a graph; a device whose address is not known yet is then refused.
 template <typename T>
-int address_on_current_device(std::atomic<T *> *table, const void *symbol, const char *what, T **out) {
+int address_on_current_device(std::atomic<T *> *table, const void *symbol, const char *what, hipStream_t st, T **out) {
   int dev = 0;
   SAREK_HIP_TRY(hipGetDevice(&dev));
   if (dev < 0 || dev >= kMaxDevices)
     return fail(SAREK_HIP_E_UNSUPPORTED, "%s: device ordinal %d beyond %d", what, dev, kMaxDevices);
   T *p = table[dev].load(std::memory_order_acquire);
   if (!p) {
+    if (capturing(st))
+      return fail(SAREK_HIP_E_UNSUPPORTED,
+                  "%s: first use on device %d under stream capture (call it once outside a capture first)", what,
+                  dev);
     SAREK_HIP_TRY(hipGetSymbolAddress(reinterpret_cast<void **>(&p), symbol));
     if (!p) return fail(SAREK_HIP_E_UNSUPPORTED, "%s: no device address for the library's own array", what);
     table[dev].store(p, std::memory_order_release);
@@ -586,27 +622,46 @@ int address_on_current_device(std::atomic<T *> *table, const void *symbol, const
   return SAREK_HIP_OK;
 }
 
-int scratch_on_current_device(float **out) {
-  return address_on_current_device(g_scratch_addr, HIP_SYMBOL(scratch), "triad_sum_static", out);
+int scratch_on_current_device(hipStream_t st, float **out) {
+  return address_on_current_device(g_scratch_addr, HIP_SYMBOL(scratch), "triad_sum_static", st, out);
 }
 
-// Folds shorter than this run as one workgroup; longer ones in two steps through fold_stage.
-constexpr int64_t kFoldTwoStepFrom = int64_t{1} << 17;
+// The stage slot of (current device, st): a stream keeps the slot it got first, so folds on one stream follow each
+// other through the same slot and folds on different streams never share one.  nullptr when all slots of the device
+// are taken by other streams, or when the device's array cannot be looked up now (first use under capture): the
+// caller then folds with one workgroup, which needs no stage.
+FoldSlot *fold_slot_for(hipStream_t st) {
+  FoldSlot *slots = nullptr;
+  if (address_on_current_device(g_fold_slots_addr, HIP_SYMBOL(fold_slots), "fold_partials", st, &slots) != SAREK_HIP_OK) {
+    last_error_slot().clear();
+    return nullptr;
+  }
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess) return nullptr;
+  static std::mutex mu;
+  static std::map<std::pair<int, hipStream_t>, int> taken;   // (device, stream) -> slot
+  static int used[kMaxDevices] = {};
+  std::lock_guard<std::mutex> lock(mu);
+  auto it = taken.find({dev, st});
+  if (it != taken.end()) return slots + it->second;
+  if (used[dev] >= kFoldSlots) return nullptr;
+  const int slot = used[dev]++;
+  taken[{dev, st}] = slot;
+  return slots + slot;
+}
+
+// Folds shorter than this run as one workgroup; longer ones as 256 workgroups whose last one adds their sums up.
+constexpr int64_t kFoldOnePassFrom = int64_t{1} << 17;
 
 int launch_fold(const float *partials, int64_t count, double *sum_out, hipStream_t st) {
-  if (count < kFoldTwoStepFrom) {
+  FoldSlot *slot = count < kFoldOnePassFrom ? nullptr : fold_slot_for(st);
+  if (!slot) {
     hipLaunchKernelGGL(fold_kernel, dim3(1), dim3(1024), 0, st, partials, count, sum_out);
     return check_launch("fold kernel launch");
   }
-  double *stage = nullptr;
-  int rc = address_on_current_device(g_fold_stage_addr, HIP_SYMBOL(fold_stage), "fold_partials", &stage);
-  if (rc != SAREK_HIP_OK) return rc;
   const int64_t piece = ceil_div(ceil_div(count, kFoldGroups), 4) * 4;
-  hipLaunchKernelGGL(fold_pieces_kernel, dim3(kFoldGroups), dim3(1024), 0, st, partials, count, piece, stage);
-  rc = check_launch("fold pieces kernel launch");
-  if (rc != SAREK_HIP_OK) return rc;
-  hipLaunchKernelGGL(fold_stage_kernel, dim3(1), dim3(kFoldGroups), 0, st, stage, sum_out);
-  return check_launch("fold stage kernel launch");
+  hipLaunchKernelGGL(fold_onepass_kernel, dim3(kFoldGroups), dim3(1024), 0, st, partials, count, piece, slot, sum_out);
+  return check_launch("fold kernel launch");
 }
 }  // namespace
 }  // namespace sarek_hip
@@ -663,7 +718,7 @@ int sarek_hip_triad_sum_f32_static(float *a, const float *b, const float *c, flo
   }
   // Every workgroup stores its partial before the fold reads exactly those: nothing has to start at zero.
   float *partials = nullptr;
-  int rc = scratch_on_current_device(&partials);
+  int rc = scratch_on_current_device(st, &partials);
   if (rc != SAREK_HIP_OK) return rc;
   return launch_triad(a, b, c, s, n, partials, sum_out, true, st);
 }

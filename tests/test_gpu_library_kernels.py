@@ -409,7 +409,8 @@ def test_fused_pair_block_sum_layouts_agree(hip, oracle, torch_cuda, n):
 
 @pytest.mark.parametrize("count", [0, 1, 1000, (1 << 17) - 1, 1 << 17, (1 << 17) + 3, (1 << 20) + 77, 3_000_001])
 def test_fold_of_long_partial_vectors(hip, torch_cuda, count):
-    """The device fold in one step (short) and in two (from 2^17 partials on) against a float64 sum."""
+    """The device fold by one workgroup (short) and by 256 whose last one adds their sums up (from 2^17 partials
+    on) against a float64 sum."""
     torch = torch_cuda
     rng = np.random.default_rng(count)
     x = rng.uniform(0, 500, count).astype(np.float32)
@@ -424,6 +425,29 @@ def test_fold_of_long_partial_vectors(hip, torch_cuda, count):
         torch.cuda.synchronize()
         want = float(x[1:].astype(np.float64).sum())
         assert abs(out.item() - want) <= 1e-12 * max(want, 1.0)
+
+
+def test_long_folds_on_many_streams_do_not_meet(hip, torch_cuda):
+    """Long folds queued on twenty streams at once (sixteen stages per device: the streams past the sixteenth fold
+    with one workgroup), three rounds on the same streams so that every stage's ticket counter is used again:
+    every sum is its own vector's, and a stream's repeated folds give the same bits."""
+    torch = torch_cuda
+    streams = [torch.cuda.Stream() for _ in range(20)]
+    rng = np.random.default_rng(7)
+    xs = [rng.uniform(0, 500, (1 << 17) + 1000 * i + 5).astype(np.float32) for i in range(len(streams))]
+    ds = [torch.from_numpy(x).cuda() for x in xs]
+    outs = torch.full((3, len(streams)), -1.0, dtype=torch.float64, device="cuda")
+    torch.cuda.synchronize()
+    for rnd in range(3):
+        for i, st in enumerate(streams):
+            hip.check(hip.lib.sarek_hip_fold_partials_f64(ds[i].data_ptr(), ds[i].numel(),
+                                                          outs[rnd, i:].data_ptr(), st.cuda_stream))
+    torch.cuda.synchronize()
+    got = outs.cpu().numpy()
+    for i, x in enumerate(xs):
+        want = float(x.astype(np.float64).sum())
+        assert abs(got[0, i] - want) <= 1e-12 * want, i
+        assert got[0, i] == got[1, i] == got[2, i], i
 
 
 def test_tiled_matmul_through_run_vectors_at_1024(hip, oracle, sarek):
