@@ -78,7 +78,11 @@ def parse():
     ap.add_argument("--zero-operands", action="store_true",
                     help="16-bit GEMM workloads: all-zero A and B (what the kernel does when the data costs no power)")
     ap.add_argument("--tunable", action="append", default=[], metavar="NAME=VALUE",
-                    help="sarek_hip_set_tunable(NAME, VALUE) before measuring (kernel shape and measurement knobs)")
+                    help="sarek_hip_set_tunable(NAME, VALUE) before measuring (kernel shape knobs; the measurement knobs "
+                         "gemm16.ablate / ring / tj / mfma need --measure-build)")
+    ap.add_argument("--measure-build", action="store_true",
+                    help="load libsarek_hip_measure.so (make -C spoc_amd/csrc measure): the product's code plus the kernel "
+                         "variants of the ablation studies, some of which compute wrong results on purpose")
     return ap.parse_args()
 
 
@@ -557,20 +561,21 @@ def measure(name, torch, hip, steps, warmup):
         res["roofline"]["mfma_stream_only_32x32x16_TFLOPs"] = stream32
         # the vendor library on the same inputs, same protocol (torch.matmul -> hipBLASLt; it writes bf16 C)
         res["roofline"]["vendor_library_TFLOPs"] = vendor_gemm_rate(torch, hip)
-    if info["bound"] == "mfma" and info["route"].startswith("Execute"):
-        # shader clock the kernel actually ran at (in-kernel cycle counter against the
-        # constant-rate wall clock), and the rate of those very launches against the peak
-        # scaled to that clock
-        with hip.clock_probe() as probe:
-            pairs = []
-            for _ in range(min(steps, 10)):
-                probe.buf.zero_()
-                ev.start()
-                main()
-                ms = ev.stop_ms()
-                mhz = probe.mhz()
-                if mhz:
-                    pairs.append((ms, mhz))
+    if info["bound"] == "mfma" and info["route"].startswith("Execute") and kernel_ms >= 0.2:
+        # shader clock while the kernel runs: eight sleeping waves on a stream of their own count shader cycles against
+        # the constant-rate clock over the first 70 % of the launch (nothing is added to the kernel itself), and the
+        # rate of those very launches against the peak scaled to that clock
+        sampler = hip.shader_clock_sampler()
+        pairs = []
+        for _ in range(min(steps, 10)):
+            sampler.start(0.7 * kernel_ms)
+            ev.start()
+            main()
+            ms = ev.stop_ms()
+            mhz = sampler.mhz()
+            if mhz:
+                pairs.append((ms, mhz))
+        sampler.close()
         if pairs:
             pairs.sort()
             ms, mhz = pairs[len(pairs) // 2]
@@ -838,6 +843,8 @@ def main():
         print("bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1)",
               file=sys.stderr)
         sys.exit(2)
+    if args.measure_build:
+        os.environ["SAREK_HIP_MEASURE_BUILD"] = "1"
     import torch
     from spoc_amd import hip
     if not torch.cuda.is_available():
@@ -888,6 +895,8 @@ def main():
     info = hip.device_info(0)
     if args.tunable:
         out["tunables"] = args.tunable
+    if args.measure_build:
+        out["library"] = "libsarek_hip_measure.so (measurement build)"
     if args.zero_operands:
         out["config"] = dict(out["config"], workload=out["config"]["workload"].replace("N(0,0.02)", "all-zero operands"))
     out["device"] = {"name": info.name.decode(), "arch": info.gcn_arch.decode(),

@@ -679,10 +679,20 @@ int sarek_hip_fusion_detect_reduction(const char *stmt_ir, int *found, char *out
 int sarek_hip_fusion_is_reduction_kernel(const char *kernel_ir, const char *array, int *found, char op[8]);
 
 /* Integer tuning knob (launch shapes, tile variants), for sweeps without a
- * rebuild.  Unknown names are stored and ignored.                           */
+ * rebuild.  Unknown names are stored and ignored.  Every knob of the product
+ * library leaves results as they are; the knobs of the measurement build
+ * (gemm16.ablate, gemm16.ring, gemm16.tj, gemm16.mfma) are refused by the
+ * product library with SAREK_HIP_E_UNSUPPORTED.                              */
 int sarek_hip_set_tunable(const char *name, int64_t value);
 
-/* Diagnostic (no reference counterpart): while a probe buffer is set, every
+/* 1 in libsarek_hip_measure.so (built with -DSAREK_HIP_MEASURE by `make measure`: the
+ * product's code plus retired kernel shapes, variants of the 16-bit GEMMs that leave parts of
+ * the K loop out -- their results are wrong on purpose -- and the in-kernel clock probe; what
+ * the ablation studies are made with), 0 in libsarek_hip.so.                                 */
+int sarek_hip_is_measurement_build(void);
+
+/* Diagnostic of the measurement build (no reference counterpart; the product library
+ * answers SAREK_HIP_E_UNSUPPORTED): while a probe buffer is set, every
  * workgroup of the MFMA GEMM kernels (sarek_hip_gemm_bf16/_f16/_f16_bias_relu_rowsum,
  * direct-to-LDS path) writes two 64-bit counts when it retires:
  * pairs[2*w] = shader-clock cycles it was resident, pairs[2*w+1] = ticks of the

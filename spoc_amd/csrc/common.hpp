@@ -33,4 +33,12 @@ inline hipStream_t as_stream(sarek_hip_stream s) { return reinterpret_cast<hipSt
 
 constexpr int64_t ceil_div(int64_t a, int64_t b) { return (a + b - 1) / b; }
 
+// The measurement build (-DSAREK_HIP_MEASURE, libsarek_hip_measure.so) carries kernel variants and probes that the
+// product library does not have: ablated K loops, retired kernel shapes, the in-kernel clock probe.
+#ifdef SAREK_HIP_MEASURE
+constexpr bool kMeasureBuild = true;
+#else
+constexpr bool kMeasureBuild = false;
+#endif
+
 }  // namespace sarek_hip

@@ -1,39 +1,27 @@
-// 16-bit-input (bf16 / fp16), f32-accumulate GEMM for gfx950 on v_mfma_f32_32x32x16,
-// with an optional fused epilogue  y = relu(acc + bias[col]),  rowsum[row] += y.
+// 16-bit-input (bf16 / fp16), f32-accumulate GEMM for gfx950 on v_mfma_f32_16x16x32,
+// with an optional fused epilogue  y = relu(acc + bias[col]),  rowsum[row] = sum of y over the row.
 //
 // C[M x N] = A[M x K] . B[K x N], all row-major.
 //
-// Tiling: one workgroup owns a 256 x 256 tile of C and walks K in slabs.  Default: 8 waves
-// (2 along M x 4 along N, two per SIMD), each owning 128 x 64 = 4 x 2 MFMA tiles of 32 x 32
-// (128 accumulator registers).  One workgroup per CU (LDS bound), 8192^3 = 1024 tiles =
-// 4 per CU.
-//
-// Operand fetch from LDS:
-//   A: lane (m = lane%32, h = lane/32) needs k = 8h..8h+7 of row m: one ds_read_b128.
-//   B: lane (n = lane%32, h) needs k = 8h..8h+7 of column n.  B is n-contiguous in LDS (as in
-//      global memory), so the column is gathered by ds_read_b64_tr_b16: within each group of
-//      16 lanes, lane i supplies the address of 4 consecutive n of row (i/4) at n-offset
-//      4*(i%4), and receives column i of that 4 x 16 block (its 4 rows).  Two such reads
-//      (rows 0-3 and 4-7 of the lane's k range) give the 8 k values.
-//
-// Kernels (the default fast path is gemm16_m16_kernel on v_mfma_f32_16x16x32 below, with gemm16_m16_small_kernel for
-// products that do not fill the chip; the three described here are the 32 x 32 x 16 kernel and the fallbacks):
-//   gemm16_dma_kernel (K % 64 == 0, the fast path): global -> LDS by
-//     buffer_load_dwordx4 ... lds, which writes the 64 lanes' 16-byte pieces to 1 KiB of
-//     consecutive LDS with no register staging and no ds_write (the buffer form: the
-//     global_load form of the same transfer slows MFMA issue down).  Rows cannot be padded that
-//     way, so bank conflicts are removed by an XOR swizzle applied on the global-address
-//     side (which chunk a lane fetches) and again by the readers.  A streams through a ring
-//     of 2 LDS stages of K = 64 (whole 128-byte lines per request), B through a ring of 4
-//     slabs of K = 32 (128 KiB in all): a stage is refilled as soon as the barrier inside
-//     the slab that read it last has passed, so one to three slabs of MFMA work cover the
-//     latency; the barrier sits before the LAST k-step of a slab, and the first fragments of
-//     the next slab are fetched under that step's MFMAs, so no LDS latency is exposed at
-//     slab boundaries.  Inside a k-step the LDS reads of the next step's fragments are
-//     interleaved behind the first MFMAs (sched_group_barrier).
-//   gemm16_staged_kernel (any K % 8 == 0): global -> registers -> LDS with zero fill for the
-//     K tail, rows padded (144 / 544 bytes) instead of swizzled, two LDS stages of K = 64.
-//   gemm16_simple_kernel: any shape and alignment, one thread per C element.
+// Kernels:
+//   gemm16_m16_kernel: one workgroup owns a 256 x 256 tile of C and walks K in slabs; 8 waves (2 along M x 4 along
+//     N, two per SIMD), each owning 128 x 64 = 8 x 4 MFMA tiles of 16 x 16 (128 accumulator registers).  One
+//     workgroup per CU (LDS bound), 8192^3 = 1024 tiles = 4 per CU.  Global -> LDS by buffer_load_dwordx4 ... lds,
+//     which writes the 64 lanes' 16-byte pieces to 1 KiB of consecutive LDS with no register staging and no ds_write
+//     (the buffer form: the global_load form of the same transfer slows MFMA issue down).  Rows cannot be padded that
+//     way, so bank conflicts are removed by an XOR swizzle applied on the global-address side (which chunk a lane
+//     fetches) and again by the readers.  A streams through a ring of 2 LDS stages of K = 64 (whole 128-byte lines
+//     per request), B through a ring of 4 slabs of K = 32 (128 KiB in all): a stage is refilled as soon as the
+//     barrier inside the slab that read it last has passed.  B is n-contiguous in LDS (as in global memory): a lane's
+//     column fragment is gathered by ds_read_b64_tr_b16.
+//   gemm16_m16_small_kernel: the same pipeline on a 128 x 128 tile (4 waves), two workgroups per CU, for products
+//     that do not fill the chip with large tiles; K split over several workgroups per tile where tiles are few.
+//   gemm16_simple_kernel: any shape and alignment, one thread per C element (K below one LDS stage that is not a
+//     multiple of 8, or operands whose 256-row / 64-row panels span 2 GiB).
+//   gemm16_last_column_kernel: column N-1 of an odd N.
+// A build with -DSAREK_HIP_MEASURE (libsarek_hip_measure.so, for bench.py --measure-build) also holds gemm16_dma_kernel,
+// the same pipeline on v_mfma_f32_32x32x16 in several ring and wave shapes, and variants of both MFMA kernels that leave
+// parts of the K loop out: what the power and ablation studies were measured with.  The product library has none of them.
 #include <algorithm>
 #include <map>
 #include <mutex>
@@ -57,17 +45,57 @@ typedef __attribute__((ext_vector_type(4))) unsigned int u32x4;
 typedef __attribute__((ext_vector_type(2))) unsigned int u32x2;
 
 constexpr int BM = 256, BN = 256, BK = 64;
-constexpr int THREADS = 512;
-constexpr int A_STRIDE = BK * 2 + 16;   // bytes per A row in LDS (144)
-constexpr int B_STRIDE = BN * 2 + 32;   // bytes per B row in LDS (544)
-constexpr int A_BYTES = BM * A_STRIDE;  // 36864
-constexpr int B_BYTES = BK * B_STRIDE;  // 34816
-constexpr int STAGE_BYTES = A_BYTES + B_BYTES;
-constexpr int LDS_BYTES = 2 * STAGE_BYTES;  // 143360
 
 enum { EPI_STORE = 0, EPI_BIAS_RELU_ROWSUM = 1 };
 
 
+// ds_read_b64_tr_b16 at byte offset `off` of the dynamic LDS block.
+__device__ __forceinline__ u32x2 lds_read_tr16(const char *lds, int off) {
+  auto p = (LDS_PTR bf16x4 *)(lds + off);
+  bf16x4 v = __builtin_amdgcn_ds_read_tr16_b64_v4bf16(p);
+  return __builtin_bit_cast(u32x2, v);
+}
+
+// ---- what the direct-to-LDS kernels share -----------------------------------------
+// A moves in stages of BKA k (ring of NA), B in slabs of BKB k (ring of NB); RA = BKA / BKB
+// B slabs consume one A stage.  Default: BKA = 64, NA = 2, BKB = 32, NB = 4.  A rows are
+// K-contiguous in memory, so a 32-wide A slab would touch half of each 128-byte line and
+// the next slab the other half (two L1 -> L2 requests per line: a third more requests
+// over the whole kernel, and the address path stalls on them); with 64-wide A stages
+// every request is a whole line, while B, whose rows are N-contiguous (512 bytes of a row
+// per tile), keeps the finer slabs and the deeper ring.  One barrier per B slab.
+// TJ: 32-column MFMA tiles per wave along N.  TJ = 2: 8 waves (2 x 4) of 128 x 64, two
+// per SIMD; TJ = 4: 4 waves (2 x 2) of 128 x 128, one per SIMD with the 256 accumulator
+// registers in the AGPR half of the register file (fewer LDS bytes read per flop).
+//
+// Order of a wave's transfers (what vmcnt counts): top of slab j: B(j-1+NB), into the stage
+// slab j-1 used; after the barrier of slab j: the A stage that slab j was the last to read.
+constexpr int dma_allowed_in_flight(int I, int RA, int NA, int NB, int DA, int DB) {
+  // Transfers that may still be in flight at the barrier of slab s = I (mod period) once
+  // everything slab s+1 reads has landed: those issued after the later of B(s+1) and the
+  // A stage that slab s+1 starts (if it starts one).  Event 2j = top of slab j, 2j+1 = its
+  // barrier.
+  const int s = I + 64 * RA * NA * NB;
+  int need = 2 * (s + 2 - NB);
+  if ((s + 1) % RA == 0) {
+    const int ev = 2 * (s + RA - RA * NA) + 1;
+    if (ev > need) need = ev;
+  }
+  int count = 0;
+  for (int e = need + 1; e < 2 * s + 1; ++e) {
+    const int j = e / 2;
+    if (e % 2 == 0) count += DB;
+    else if (j % RA == RA - 1) count += DA;
+  }
+  return count;
+}
+constexpr int lcm_int(int a, int b) {
+  int m = a;
+  while (m % b != 0) m += a;
+  return m;
+}
+
+#ifdef SAREK_HIP_MEASURE
 template <bool Bf16>
 __device__ __forceinline__ f32x16 mfma(u32x4 a, u32x4 b, f32x16 c) {
   if constexpr (Bf16)
@@ -76,13 +104,6 @@ __device__ __forceinline__ f32x16 mfma(u32x4 a, u32x4 b, f32x16 c) {
   else
     return __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8, a),
                                                   __builtin_bit_cast(f16x8, b), c, 0, 0, 0);
-}
-
-// ds_read_b64_tr_b16 at byte offset `off` of the dynamic LDS block.
-__device__ __forceinline__ u32x2 lds_read_tr16(const char *lds, int off) {
-  auto p = (LDS_PTR bf16x4 *)(lds + off);
-  bf16x4 v = __builtin_amdgcn_ds_read_tr16_b64_v4bf16(p);
-  return __builtin_bit_cast(u32x2, v);
 }
 
 // Writes one wave's 128 x (32*TJ) accumulator block.  Accumulator layout of the 32x32 MFMA:
@@ -165,45 +186,6 @@ __device__ __forceinline__ void epilogue(f32x16 (&acc)[4][TJ], float *__restrict
   }
 }
 
-// ---- direct-to-LDS kernel ---------------------------------------------------------
-// A moves in stages of BKA k (ring of NA), B in slabs of BKB k (ring of NB); RA = BKA / BKB
-// B slabs consume one A stage.  Default: BKA = 64, NA = 2, BKB = 32, NB = 4.  A rows are
-// K-contiguous in memory, so a 32-wide A slab would touch half of each 128-byte line and
-// the next slab the other half (two L1 -> L2 requests per line: a third more requests
-// over the whole kernel, and the address path stalls on them); with 64-wide A stages
-// every request is a whole line, while B, whose rows are N-contiguous (512 bytes of a row
-// per tile), keeps the finer slabs and the deeper ring.  One barrier per B slab.
-// TJ: 32-column MFMA tiles per wave along N.  TJ = 2: 8 waves (2 x 4) of 128 x 64, two
-// per SIMD; TJ = 4: 4 waves (2 x 2) of 128 x 128, one per SIMD with the 256 accumulator
-// registers in the AGPR half of the register file (fewer LDS bytes read per flop).
-//
-// Order of a wave's transfers (what vmcnt counts): top of slab j: B(j-1+NB), into the stage
-// slab j-1 used; after the barrier of slab j: the A stage that slab j was the last to read.
-constexpr int dma_allowed_in_flight(int I, int RA, int NA, int NB, int DA, int DB) {
-  // Transfers that may still be in flight at the barrier of slab s = I (mod period) once
-  // everything slab s+1 reads has landed: those issued after the later of B(s+1) and the
-  // A stage that slab s+1 starts (if it starts one).  Event 2j = top of slab j, 2j+1 = its
-  // barrier.
-  const int s = I + 64 * RA * NA * NB;
-  int need = 2 * (s + 2 - NB);
-  if ((s + 1) % RA == 0) {
-    const int ev = 2 * (s + RA - RA * NA) + 1;
-    if (ev > need) need = ev;
-  }
-  int count = 0;
-  for (int e = need + 1; e < 2 * s + 1; ++e) {
-    const int j = e / 2;
-    if (e % 2 == 0) count += DB;
-    else if (j % RA == RA - 1) count += DA;
-  }
-  return count;
-}
-constexpr int lcm_int(int a, int b) {
-  int m = a;
-  while (m % b != 0) m += a;
-  return m;
-}
-
 // Ablate (measurement only, results are wrong by construction; tunable gemm16.ablate): bit 0 leaves the
 // global -> LDS transfers out of the K loop (the ring keeps what the prologue put there), bit 1 the LDS
 // fragment reads (every MFMA reuses the first fragments), bit 2 makes every workgroup fetch the panels of
@@ -245,7 +227,7 @@ __global__ __launch_bounds__(64 * 2 * (8 / TJ)) void gemm16_dma_kernel(const uin
   const int m0 = tm * BM, n0 = tn * BN;
   const int m0_src = (Ablate & 4) ? 0 : m0, n0_src = (Ablate & 4) ? 0 : n0;
   long long probe_c0 = 0, probe_t0 = 0;
-  if (probe) {
+  if (kMeasureBuild && probe) {
     probe_c0 = clock64();
     probe_t0 = wall_clock64();
   }
@@ -447,11 +429,13 @@ __global__ __launch_bounds__(64 * 2 * (8 / TJ)) void gemm16_dma_kernel(const uin
   __builtin_amdgcn_s_waitcnt(waitcnt_vm_lgkm0(0));
   epilogue<Epi, TJ, (Ablate & 8) != 0>(acc, C, bias, rowsum, M, N, m0, wm, wn, n0 + wn * (32 * TJ), lm, lh,
                                        reinterpret_cast<float *>(lds_ring<10, A_BYTES_S>));
-  if (probe && tid == 0) {
+  if (kMeasureBuild && probe && tid == 0) {
     probe[2 * blockIdx.x] = static_cast<unsigned long long>(clock64() - probe_c0);
     probe[2 * blockIdx.x + 1] = static_cast<unsigned long long>(wall_clock64() - probe_t0);
   }
 }
+
+#endif  // SAREK_HIP_MEASURE
 
 // ---- direct-to-LDS kernel on v_mfma_f32_16x16x32 ---------------------------------------
 // The same tile, rings and transfers as gemm16_dma_kernel<.., 64, 32, 2, 4, 2> (256 x 256 per workgroup, 8 waves
@@ -484,11 +468,13 @@ __device__ __forceinline__ f32x4_t mfma16(u32x4 a, u32x4 b, f32x4_t c) {
 // l%16 of its tile); TI = 8 in the 256 x 256 workgroup tile (2 x 4 waves), 4 in the 128 x 128 one (2 x 2 waves).
 // Fused form as in `epilogue`: per lane the sum over its four columns for each of its 4*TI rows, a halving butterfly
 // over the 16 lanes that share those rows (with TI = 8: 16+8+4+2 exchanges leave lane m with rows 2m, 2m+1 of the 32;
-// with TI = 4: 8+4+2+1 leave it with row m of the 16), the WNW waves along N through LDS, one atomicAdd per row.
+// with TI = 4: 8+4+2+1 leave it with row m of the 16), the WNW waves along N through LDS.  The tile's sum of row r then
+// goes to rs_plane[r] when the launch has planes (one per tile column, added up in tile order by
+// rowsum_fold_kernel: the same bits on every run), else to rowsum[r] by atomicAdd.
 template <int Epi, int TI = 8, int WNW = 4>
 __device__ __forceinline__ void epilogue16(f32x4_t (&acc)[TI][4], float *__restrict__ C, const float *__restrict__ bias,
-                                           float *__restrict__ rowsum, int M, int N, int ld, int m0, int wm, int wn,
-                                           int col0, int l16, int g, float *scratch) {
+                                           float *__restrict__ rowsum, float *__restrict__ rs_plane, int M, int N, int ld,
+                                           int m0, int wm, int wn, int col0, int l16, int g, float *scratch) {
   constexpr int WROWS = 16 * TI, TROWS = 2 * WROWS, NV = 4 * TI, E = NV / 16;
   static_assert(TI == 8 || TI == 4, "wave tiles of 128 or 64 rows");
   static_assert(WNW == 4 || WNW == 2, "four or two waves along N");
@@ -550,7 +536,8 @@ __device__ __forceinline__ void epilogue16(f32x4_t (&acc)[TI][4], float *__restr
       float total;
       if constexpr (WNW == 4) total = (scratch[t] + scratch[TROWS + t]) + (scratch[2 * TROWS + t] + scratch[3 * TROWS + t]);
       else total = scratch[t] + scratch[TROWS + t];
-      atomicAdd(rowsum + m0 + t, total);
+      if (rs_plane) rs_plane[m0 + t] = total;
+      else atomicAdd(rowsum + m0 + t, total);
     }
   }
 }
@@ -559,7 +546,8 @@ template <bool Bf16, int Epi, int Ablate = 0, bool Ragged = false>
 __global__ __launch_bounds__(512) void gemm16_m16_kernel(const uint16_t *__restrict__ A, const uint16_t *__restrict__ B,
                                                          float *__restrict__ C, const float *__restrict__ bias,
                                                          float *__restrict__ rowsum, int M, int N, int K, int tiles_m,
-                                                         int tiles_n, int xcd_remap, unsigned long long *probe, int ld) {
+                                                         int tiles_n, int xcd_remap, unsigned long long *probe, int ld,
+                                                         float *__restrict__ rs_planes) {
   constexpr int BKA = 64, BKB = 32, NA = 2, NB = 4;
   constexpr int RA = BKA / BKB;                  // B slabs per A stage
   constexpr int A_ROW = BKA * 2, A_CHUNKS = A_ROW / 16, A_ROWS_PER_DMA = 1024 / A_ROW;
@@ -579,7 +567,7 @@ __global__ __launch_bounds__(512) void gemm16_m16_kernel(const uint16_t *__restr
   tile_of_block(tiles_m, tiles_n, xcd_remap, tm, tn);
   const int m0 = tm * BM, n0 = tn * BN;
   long long probe_c0 = 0, probe_t0 = 0;
-  if (probe) {
+  if (kMeasureBuild && probe) {
     probe_c0 = clock64();
     probe_t0 = wall_clock64();
   }
@@ -790,9 +778,9 @@ __global__ __launch_bounds__(512) void gemm16_m16_kernel(const uint16_t *__restr
     ((full + Is < nslabs ? slab(std::integral_constant<int, Is>{}, full + Is) : (void)0), ...);
   }(std::make_integer_sequence<int, P - 1>{});
   __builtin_amdgcn_s_waitcnt(waitcnt_vm_lgkm0(0));   // drain the (redundant) tail DMA before the LDS is released
-  epilogue16<Epi>(acc, C, bias, rowsum, M, N, ld, m0, wm, wn, n0 + wn * 64, l16, g,
-                  reinterpret_cast<float *>(lds_ring<10, A_BYTES_S>));
-  if (probe && tid == 0) {
+  epilogue16<Epi>(acc, C, bias, rowsum, rs_planes ? rs_planes + static_cast<int64_t>(tn) * M : nullptr, M, N, ld, m0, wm, wn,
+                  n0 + wn * 64, l16, g, reinterpret_cast<float *>(lds_ring<10, A_BYTES_S>));
+  if (kMeasureBuild && probe && tid == 0) {
     probe[2 * blockIdx.x] = static_cast<unsigned long long>(clock64() - probe_c0);
     probe[2 * blockIdx.x + 1] = static_cast<unsigned long long>(wall_clock64() - probe_t0);
   }
@@ -812,7 +800,8 @@ __global__ __launch_bounds__(256) void gemm16_m16_small_kernel(const uint16_t *_
                                                                float *__restrict__ C, const float *__restrict__ bias,
                                                                float *__restrict__ rowsum, int M, int N, int K, int tiles_m,
                                                                int tiles_n, int xcd_remap, unsigned long long *probe,
-                                                               int k_chunk, float *__restrict__ partials, int ld) {
+                                                               int k_chunk, float *__restrict__ partials, int ld,
+                                                               float *__restrict__ rs_planes) {
   constexpr int SBM = 128, SBN = 128;
   constexpr int BKA = 64, BKB = 32, NA = 3, NB = 4;
   constexpr int RA = BKA / BKB;
@@ -834,7 +823,7 @@ __global__ __launch_bounds__(256) void gemm16_m16_small_kernel(const uint16_t *_
   tile_of_block(tiles_m, tiles_n, xcd_remap, tm, tn);
   const int m0 = tm * SBM, n0 = tn * SBN;
   long long probe_c0 = 0, probe_t0 = 0;
-  if (probe) {
+  if (kMeasureBuild && probe) {
     probe_c0 = clock64();
     probe_t0 = wall_clock64();
   }
@@ -1023,121 +1012,12 @@ __global__ __launch_bounds__(256) void gemm16_m16_small_kernel(const uint16_t *_
     ((full + Is < nslabs ? slab(std::integral_constant<int, Is>{}, full + Is) : (void)0), ...);
   }(std::make_integer_sequence<int, P - 1>{});
   __builtin_amdgcn_s_waitcnt(waitcnt_vm_lgkm0(0));   // drain the (redundant) tail DMA before the LDS is released
-  epilogue16<Epi, 4, WN>(acc, C, bias, rowsum, M, N, ld, m0, wm, wn, n0 + wn * 64, l16, g,
-                         reinterpret_cast<float *>(lds_ring<30, A_BYTES_S>));
-  if (probe && tid == 0) {
+  epilogue16<Epi, 4, WN>(acc, C, bias, rowsum, rs_planes ? rs_planes + static_cast<int64_t>(tn) * M : nullptr, M, N, ld, m0,
+                         wm, wn, n0 + wn * 64, l16, g, reinterpret_cast<float *>(lds_ring<30, A_BYTES_S>));
+  if (kMeasureBuild && probe && tid == 0) {
     probe[2 * blockIdx.x] = static_cast<unsigned long long>(clock64() - probe_c0);
     probe[2 * blockIdx.x + 1] = static_cast<unsigned long long>(wall_clock64() - probe_t0);
   }
-}
-
-template <bool Bf16, int Epi>
-__global__ __launch_bounds__(THREADS) void gemm16_staged_kernel(const uint16_t *__restrict__ A,
-                                                         const uint16_t *__restrict__ B,
-                                                         float *__restrict__ C,
-                                                         const float *__restrict__ bias,
-                                                         float *__restrict__ rowsum, int M, int N,
-                                                         int K, int tiles_m, int tiles_n, int xcd_remap) {
-  extern __shared__ __attribute__((aligned(16))) char lds[];
-  const int tid = threadIdx.x;
-  const int lane = tid & 63, wave = tid >> 6;
-  const int wm = wave >> 2, wn = wave & 3;  // 2 x 4 waves
-  const int lm = lane & 31, lh = lane >> 5;
-
-  int tm, tn;
-  tile_of_block(tiles_m, tiles_n, xcd_remap, tm, tn);
-  const int m0 = tm * BM, n0 = tn * BN;
-
-  // ---- global -> register staging --------------------------------------------
-  // A slab: 256 rows x 8 chunks of 16 B; chunk c = tid + 512*i -> row c/8, chunk c%8.
-  // B slab: 64 rows x 32 chunks of 16 B; chunk c = tid + 512*i -> row c/32, chunk c%32.
-  u32x4 ra[4], rb[4];
-  const u32x4 zero4 = {0u, 0u, 0u, 0u};
-  auto load_slab = [&](int k0) {
-#pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      const int c = tid + THREADS * i;
-      const int row = c >> 3, kc = (c & 7) * 8;
-      const int gr = m0 + row, gk = k0 + kc;
-      ra[i] = (gr < M && gk < K)
-                  ? *reinterpret_cast<const u32x4 *>(A + static_cast<int64_t>(gr) * K + gk)
-                  : zero4;
-    }
-#pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      const int c = tid + THREADS * i;
-      const int kr = c >> 5, nc = (c & 31) * 8;
-      const int gk = k0 + kr, gn = n0 + nc;
-      rb[i] = (gk < K && gn < N)
-                  ? *reinterpret_cast<const u32x4 *>(B + static_cast<int64_t>(gk) * N + gn)
-                  : zero4;
-    }
-  };
-  auto store_slab = [&](int stage) {
-    char *sa = lds + stage * STAGE_BYTES;
-    char *sb = sa + A_BYTES;
-#pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      const int c = tid + THREADS * i;
-      *reinterpret_cast<u32x4 *>(sa + (c >> 3) * A_STRIDE + (c & 7) * 16) = ra[i];
-    }
-#pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      const int c = tid + THREADS * i;
-      *reinterpret_cast<u32x4 *>(sb + (c >> 5) * B_STRIDE + (c & 31) * 16) = rb[i];
-    }
-  };
-
-  f32x16 acc[4][2];
-#pragma unroll
-  for (int i = 0; i < 4; ++i)
-#pragma unroll
-    for (int j = 0; j < 2; ++j)
-#pragma unroll
-      for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
-
-  // Per-lane LDS offsets that do not depend on the K slab.
-  const int a_off = (wm * 128 + lm) * A_STRIDE + lh * 16;  // + i*32*A_STRIDE + kk*32
-  // transposing read: group of 16 lanes, lane i in group: row i/4, n offset 4*(i%4)
-  const int li = lane & 15;
-  const int b_off = (lh * 8 + (li >> 2)) * B_STRIDE +
-                    (wn * 64 + ((lane >> 4) & 1) * 16 + (li & 3) * 4) * 2;  // + j*64 + kk*16*B_STRIDE
-
-  const int nslabs = (K + BK - 1) / BK;
-  load_slab(0);
-  store_slab(0);
-  __syncthreads();
-
-  for (int s = 0; s < nslabs; ++s) {
-    const int cur = s & 1;
-    if (s + 1 < nslabs) load_slab((s + 1) * BK);
-    const char *sa = lds + cur * STAGE_BYTES;
-    const char *sb = sa + A_BYTES;
-#pragma unroll
-    for (int kk = 0; kk < BK / 16; ++kk) {
-      u32x4 af[4], bf[2];
-#pragma unroll
-      for (int i = 0; i < 4; ++i)
-        af[i] = *reinterpret_cast<const u32x4 *>(sa + a_off + i * 32 * A_STRIDE + kk * 32);
-#pragma unroll
-      for (int j = 0; j < 2; ++j) {
-        const int off = A_BYTES + cur * STAGE_BYTES + b_off + j * 64 + kk * 16 * B_STRIDE;
-        u32x2 lo = lds_read_tr16(lds, off);
-        u32x2 hi = lds_read_tr16(lds, off + 4 * B_STRIDE);
-        bf[j] = u32x4{lo.x, lo.y, hi.x, hi.y};
-      }
-      (void)sb;
-#pragma unroll
-      for (int i = 0; i < 4; ++i)
-#pragma unroll
-        for (int j = 0; j < 2; ++j) acc[i][j] = mfma<Bf16>(af[i], bf[j], acc[i][j]);
-    }
-    if (s + 1 < nslabs) store_slab(cur ^ 1);
-    __syncthreads();
-  }
-
-  epilogue<Epi, 2>(acc, C, bias, rowsum, M, N, m0, wm, wn, n0 + wn * 64, lm, lh,
-                   reinterpret_cast<float *>(lds));
 }
 
 // Any shape, any alignment: one thread per C element, f32 accumulate in k order.
@@ -1147,7 +1027,7 @@ __global__ __launch_bounds__(256) void gemm16_simple_kernel(const uint16_t *__re
                                                             float *__restrict__ C,
                                                             const float *__restrict__ bias,
                                                             float *__restrict__ rowsum, int M,
-                                                            int N, int K) {
+                                                            int N, int K, float *__restrict__ rs_planes) {
   const int col = blockIdx.x * 64 + (threadIdx.x & 63);
   const int row = blockIdx.y * 4 + (threadIdx.x >> 6);
   float acc = 0.f;
@@ -1174,13 +1054,27 @@ __global__ __launch_bounds__(256) void gemm16_simple_kernel(const uint16_t *__re
   if (Epi == EPI_BIAS_RELU_ROWSUM) {
     float rs = (row < M && col < N) ? acc : 0.f;
     for (int off = 32; off >= 1; off >>= 1) rs += __shfl_xor(rs, off, 64);
-    if ((threadIdx.x & 63) == 0 && row < M) atomicAdd(rowsum + row, rs);
+    if ((threadIdx.x & 63) == 0 && row < M) {
+      if (rs_planes) rs_planes[static_cast<int64_t>(blockIdx.x) * M + row] = rs;   // one plane per 64 columns
+      else atomicAdd(rowsum + row, rs);
+    }
   }
 }
 
 __global__ void zero_f32_kernel(float *p, int n) {
   const int i = blockIdx.x * blockDim.x + threadIdx.x;
   if (i < n) p[i] = 0.f;
+}
+
+// rowsum[r] = the per-tile-column sums planes[t * m + r], t = 0 .. count-1, added in that order in double and rounded
+// once: the order is the tiles', not the order they finished in, so a product gives the same row sums on every run.
+__global__ __launch_bounds__(256) void rowsum_fold_kernel(const float *__restrict__ planes, int count, int m,
+                                                          float *__restrict__ rowsum) {
+  const int r = blockIdx.x * 256 + threadIdx.x;
+  if (r >= m) return;
+  double acc = 0.0;
+  for (int t = 0; t < count; ++t) acc += static_cast<double>(planes[static_cast<int64_t>(t) * m + r]);
+  rowsum[r] = static_cast<float>(acc);
 }
 
 // Whether the 128 x 128 tile beats the 256 x 256 one.  Measured on MI355X: large tiles run in rounds of one per CU;
@@ -1211,7 +1105,7 @@ template <bool Bf16, int Epi>
 __global__ __launch_bounds__(256) void gemm16_last_column_kernel(const uint16_t *__restrict__ A,
                                                                  const uint16_t *__restrict__ B, float *__restrict__ C,
                                                                  const float *__restrict__ bias, float *__restrict__ rowsum,
-                                                                 int M, int N, int K) {
+                                                                 int M, int N, int K, float *__restrict__ rs_plane) {
   const int lane = threadIdx.x & 63;
   const int row = blockIdx.x * 4 + (threadIdx.x >> 6);
   if (row >= M) return;   // whole waves leave together
@@ -1229,7 +1123,8 @@ __global__ __launch_bounds__(256) void gemm16_last_column_kernel(const uint16_t 
     if constexpr (Epi == EPI_BIAS_RELU_ROWSUM) {
       sum += bias[N - 1];
       sum = sum > 0.f ? sum : 0.f;
-      atomicAdd(rowsum + row, sum);
+      if (rs_plane) rs_plane[row] = sum;
+      else atomicAdd(rowsum + row, sum);
     }
     C[static_cast<int64_t>(row) * N + N - 1] = sum;
   }
@@ -1275,18 +1170,23 @@ int splitk_for(int m, int n, int k) {
   return (k + chunk - 1) / chunk;
 }
 
-// The kernel on v_mfma_f32_16x16x32 with nothing switched off: what a call gets unless a sweep knob says otherwise.
+// The kernel on v_mfma_f32_16x16x32 with nothing switched off: what a call gets unless, in the measurement build, a sweep
+// knob says otherwise.
 inline bool gemm16_default_kernel() {
+#ifdef SAREK_HIP_MEASURE
   return tunable("gemm16.ring", 0) == 0 && tunable("gemm16.tj", 2) == 2 && tunable("gemm16.mfma", 16) == 16 &&
          tunable("gemm16.ablate", 0) == 0;
+#else
+  return true;
+#endif
 }
 
 // The workgroup tile of the direct-to-LDS kernels for this shape under the present tunables (256 or 128), or 0 when
-// the shape goes to the staged or the simple kernel (pointer alignment, which can also send a call there, is not a
-// property of the shape and is not looked at).
+// the shape goes to the simple kernel (pointer alignment, which can also send a call there, is not a property of the
+// shape and is not looked at).
 int gemm16_tile_for(int m, int n, int k) {
   if (m < 1 || n < 1 || k < 1) return 0;
-  if (tunable("gemm16.force_simple", 0) != 0 || tunable("gemm16.force_staged", 0) != 0) return 0;
+  if (tunable("gemm16.force_simple", 0) != 0) return 0;
   // transfer offsets are 32-bit: 256 rows of A and 64 rows of B must span less than 2 GiB
   const bool offsets_ok = static_cast<int64_t>(k) * 256 * 2 < 0x7FFFFFFF && static_cast<int64_t>(n) * 64 * 2 < 0x7FFFFFFF;
   if (!offsets_ok) return 0;
@@ -1297,9 +1197,76 @@ int gemm16_tile_for(int m, int n, int k) {
     const int tile = (int)tunable("gemm16.tile", 0);
     return (tile == 128 || (tile == 0 && small_tile_wins(m, n))) ? 128 : 256;
   }
-  // the 32 x 32 x 16 kernel, its ring and wave shapes and the measurement variants: whole K = 64 stages, 16-byte rows of B
-  return (n % 8 == 0 && k % BK == 0) ? 256 : 0;   // (K % 8 == 0 alone: the staged kernel)
+  // measurement build: the 32 x 32 x 16 kernel and the ablated variants take whole K = 64 stages and 16-byte rows of B
+  return (n % 8 == 0 && k % BK == 0) ? 256 : 0;
 }
+
+#ifdef SAREK_HIP_MEASURE
+// The measurement build's kernels: the 32 x 32 x 16 pipeline in its ring and wave shapes, and both MFMA kernels with parts
+// of the K loop left out (gemm16.ablate; the results are then wrong by construction).  Plain store, aligned shapes only.
+template <bool Bf16>
+int launch_gemm16_measure(const uint16_t *a, const uint16_t *b, float *c, int m, int n, int k, hipStream_t st) {
+  const bool ok = k % 8 == 0 && n % 8 == 0 && k % BK == 0 && reinterpret_cast<uintptr_t>(a) % 16 == 0 &&
+                  reinterpret_cast<uintptr_t>(b) % 16 == 0 && static_cast<int64_t>(k) * 256 * 2 < 0x7FFFFFFF &&
+                  static_cast<int64_t>(n) * 64 * 2 < 0x7FFFFFFF;
+  if (!ok)
+    return fail(SAREK_HIP_E_UNSUPPORTED, "gemm16 measurement kernels: N %% 8 == 0, K %% 64 == 0 and 16-byte aligned A, B only");
+  const int tiles_m = (m + BM - 1) / BM, tiles_n = (n + BN - 1) / BN;
+  const int remap = (int)tunable("gemm.xcd_remap", 1);
+  // gemm16.mfma: 16 = the kernel on the 16 x 16 x 32 instruction (ring 0 and tj 2 only), 32 = 32 x 32 x 16.
+  // gemm16.ring 0 = A in K=64 stages x2 + B in K=32 slabs x4, 4 = both in K=32 slabs x4, 2 = both in K=64 slabs x2;
+  // gemm16.tj 2 | 4
+  const int ring = (int)tunable("gemm16.ring", 0), tj = (int)tunable("gemm16.tj", 2);
+  const dim3 grid(tiles_m * tiles_n);
+  unsigned long long *probe = clock_probe(static_cast<int64_t>(tiles_m) * tiles_n);
+  float *const none = nullptr;
+#define SAREK_LAUNCH_DMA(BKA, BKB, NA, NB, TJ)                                                      \
+  hipLaunchKernelGGL((gemm16_dma_kernel<Bf16, EPI_STORE, BKA, BKB, NA, NB, TJ>), grid,                \
+                     dim3(64 * 2 * (8 / TJ)), 0, st, a, b, c, none, none, m, n, k, tiles_m,           \
+                     tiles_n, remap, probe)
+  const int ablate = (int)tunable("gemm16.ablate", 0);
+  const bool m16 = ring == 0 && tj == 2 && tunable("gemm16.mfma", 16) == 16;
+  if (m16 && ablate >= 1 && ablate <= 3 && Bf16) {
+    // 1: no transfers in the K loop, 2: no fragment reads, 3: neither
+    if constexpr (Bf16) {
+#define SAREK_LAUNCH_M16_ABLATED(AB)                                                                        \
+  hipLaunchKernelGGL((gemm16_m16_kernel<true, EPI_STORE, AB>), grid, dim3(512), 0, st, a, b, c, none, none, m, n, k, \
+                     tiles_m, tiles_n, remap, probe, n, none)
+      if (ablate == 1) SAREK_LAUNCH_M16_ABLATED(1);
+      else if (ablate == 2) SAREK_LAUNCH_M16_ABLATED(2);
+      else SAREK_LAUNCH_M16_ABLATED(3);
+#undef SAREK_LAUNCH_M16_ABLATED
+    }
+    return check_launch("gemm16 kernel launch");
+  }
+  if (m16)
+    return fail(SAREK_HIP_E_UNSUPPORTED, "gemm16.ablate with the 16 x 16 x 32 kernel: 1..3, bf16 (4 and 8: gemm16.mfma=32)");
+  if (ablate != 0) {
+    if (!Bf16 || ring != 0 || tj != 2 || ablate < 1 || (ablate > 4 && ablate != 8))
+      return fail(SAREK_HIP_E_UNSUPPORTED, "gemm16.ablate is for the default bf16 shape only (1..4, 8)");
+    if constexpr (Bf16) {
+#define SAREK_LAUNCH_ABLATED(AB)                                                                    \
+  hipLaunchKernelGGL((gemm16_dma_kernel<true, EPI_STORE, 64, 32, 2, 4, 2, AB>), grid, dim3(512), 0, st, a, b, c, \
+                     none, none, m, n, k, tiles_m, tiles_n, remap, probe)
+      if (ablate == 1) SAREK_LAUNCH_ABLATED(1);
+      else if (ablate == 2) SAREK_LAUNCH_ABLATED(2);
+      else if (ablate == 3) SAREK_LAUNCH_ABLATED(3);
+      else if (ablate == 8) SAREK_LAUNCH_ABLATED(8);
+      else SAREK_LAUNCH_ABLATED(4);
+#undef SAREK_LAUNCH_ABLATED
+    }
+    return check_launch("gemm16 kernel launch");
+  }
+  if (ring == 4 && tj == 2) SAREK_LAUNCH_DMA(32, 32, 4, 4, 2);
+  else if (ring == 4) SAREK_LAUNCH_DMA(32, 32, 4, 4, 4);
+  else if (ring == 2 && tj == 2) SAREK_LAUNCH_DMA(64, 64, 2, 2, 2);
+  else if (ring == 2) SAREK_LAUNCH_DMA(64, 64, 2, 2, 4);
+  else if (tj == 4) SAREK_LAUNCH_DMA(64, 32, 2, 4, 4);
+  else SAREK_LAUNCH_DMA(64, 32, 2, 4, 2);
+#undef SAREK_LAUNCH_DMA
+  return check_launch("gemm16 kernel launch");
+}
+#endif  // SAREK_HIP_MEASURE
 
 template <bool Bf16, int Epi>
 int launch_gemm16(const uint16_t *a, const uint16_t *b, float *c, const float *bias, float *rowsum,
@@ -1307,150 +1274,102 @@ int launch_gemm16(const uint16_t *a, const uint16_t *b, float *c, const float *b
   if (m <= 0 || n <= 0 || k <= 0)
     return fail(SAREK_HIP_E_INVALID_ARG, "gemm16: m, n, k must be positive (got %d %d %d)", m, n, k);
   if (!a || !b || !c) return fail(SAREK_HIP_E_INVALID_ARG, "gemm16: NULL matrix");
-  if (Epi == EPI_BIAS_RELU_ROWSUM) {
-    if (!bias || !rowsum) return fail(SAREK_HIP_E_INVALID_ARG, "gemm16: NULL bias or rowsum");
-    hipLaunchKernelGGL(zero_f32_kernel, dim3((m + 255) / 256), dim3(256), 0, st, rowsum, m);
-    int rc = check_launch("rowsum clear launch");
-    if (rc != SAREK_HIP_OK) return rc;
+  if (Epi == EPI_BIAS_RELU_ROWSUM && (!bias || !rowsum)) return fail(SAREK_HIP_E_INVALID_ARG, "gemm16: NULL bias or rowsum");
+#ifdef SAREK_HIP_MEASURE
+  if (!gemm16_default_kernel()) {
+    if constexpr (Epi == EPI_STORE) return launch_gemm16_measure<Bf16>(a, b, c, m, n, k, st);
+    else return fail(SAREK_HIP_E_UNSUPPORTED, "gemm16 measurement kernels: plain store only");
   }
-  // The default kernels (v_mfma_f32_16x16x32, 256 x 256 or 128 x 128 tile) take any N, any K of at least one LDS stage and
+#endif
+  // The kernels on v_mfma_f32_16x16x32 (256 x 256 or 128 x 128 tile) take any N, any K of at least one LDS stage and
   // any alignment of A and B in their Ragged form; below one stage K must be a multiple of 8 and A and B 16-byte aligned.
-  if (gemm16_default_kernel()) {
-    const int tile_choice = gemm16_tile_for(m, n, k);
-    const bool ab16 = reinterpret_cast<uintptr_t>(a) % 16 == 0 && reinterpret_cast<uintptr_t>(b) % 16 == 0;
-    if (tile_choice != 0 && (k >= 64 || ab16)) {
-      // an odd N: the tiled kernel takes the first N - 1 columns of the N-strided matrices, a matrix-vector kernel the last
-      const int nm = n - (n & 1);
-      const bool ragged = n % 8 != 0 || k % 64 != 0 || !ab16;   // the kernels' template flag
-      const int remap = (int)tunable("gemm.xcd_remap", 1);
-      int rc = SAREK_HIP_OK;
-      if (nm > 0 && tile_choice == 128) {
-        const int sm = (m + 127) / 128, sn = (nm + 127) / 128;
-        unsigned long long *sprobe = clock_probe(static_cast<int64_t>(sm) * sn);
-        int splits = 1;
-        float *partials = nullptr;
-        if constexpr (Epi == EPI_STORE) {
-          if (reinterpret_cast<uintptr_t>(c) % 16 == 0) splits = splitk_for(m, n, k);
-          if (splits > 1) partials = splitk_workspace(st);
-          if (!partials) splits = 1;
-        }
-        if (splits > 1) {
-          const int64_t mn = static_cast<int64_t>(m) * n;
-          const int chunk = (((k + 63) / 64 + splits - 1) / splits) * 64;
-          if (ragged)
-            hipLaunchKernelGGL((gemm16_m16_small_kernel<Bf16, Epi, true>), dim3(sm * sn, splits), dim3(256), 0, st, a, b, c,
-                               bias, rowsum, m, nm, k, sm, sn, remap, nullptr, chunk, partials, n);
-          else
-            hipLaunchKernelGGL((gemm16_m16_small_kernel<Bf16, Epi, false>), dim3(sm * sn, splits), dim3(256), 0, st, a, b, c,
-                               bias, rowsum, m, nm, k, sm, sn, remap, nullptr, chunk, partials, n);
-          rc = check_launch("gemm16 kernel launch");
-          if (rc != SAREK_HIP_OK) return rc;
-          rc = launch_splitk_reduce(partials, c, mn, splits, st);
-        } else {
-          if (ragged)
-            hipLaunchKernelGGL((gemm16_m16_small_kernel<Bf16, Epi, true>), dim3(sm * sn), dim3(256), 0, st, a, b, c, bias,
-                               rowsum, m, nm, k, sm, sn, remap, sprobe, k, nullptr, n);
-          else
-            hipLaunchKernelGGL((gemm16_m16_small_kernel<Bf16, Epi, false>), dim3(sm * sn), dim3(256), 0, st, a, b, c, bias,
-                               rowsum, m, nm, k, sm, sn, remap, sprobe, k, nullptr, n);
-          rc = check_launch("gemm16 kernel launch");
-        }
-      } else if (nm > 0) {
-        const int tiles_m = (m + BM - 1) / BM, tiles_n = (nm + BN - 1) / BN;
-        unsigned long long *probe = clock_probe(static_cast<int64_t>(tiles_m) * tiles_n);
-        if (ragged)
-          hipLaunchKernelGGL((gemm16_m16_kernel<Bf16, Epi, 0, true>), dim3(tiles_m * tiles_n), dim3(512), 0, st, a, b, c, bias,
-                             rowsum, m, nm, k, tiles_m, tiles_n, remap, probe, n);
-        else
-          hipLaunchKernelGGL((gemm16_m16_kernel<Bf16, Epi, 0, false>), dim3(tiles_m * tiles_n), dim3(512), 0, st, a, b, c, bias,
-                             rowsum, m, nm, k, tiles_m, tiles_n, remap, probe, n);
-        rc = check_launch("gemm16 kernel launch");
-      }
-      if (rc != SAREK_HIP_OK || nm == n) return rc;
-      hipLaunchKernelGGL((gemm16_last_column_kernel<Bf16, Epi>), dim3((m + 3) / 4), dim3(256), 0, st, a, b, c, bias, rowsum,
-                         m, n, k);
-      return check_launch("gemm16 last-column launch");
+  const int tile_choice = gemm16_tile_for(m, n, k);
+  const bool ab16 = reinterpret_cast<uintptr_t>(a) % 16 == 0 && reinterpret_cast<uintptr_t>(b) % 16 == 0;
+  const bool tiled = tile_choice != 0 && (k >= 64 || ab16);
+  // an odd N: the tiled kernel takes the first N - 1 columns of the N-strided matrices, a matrix-vector kernel the last
+  const int nm = n - (n & 1);
+
+  // Row sums: every tile column (every 64 columns of the simple kernel, and the last column of an odd N) leaves its
+  // share of each row in a plane of its own, and rowsum_fold_kernel adds the planes in column order, in double, with one
+  // rounding: the same bits on every run.  The planes live in the stream's workspace block; a call that has none (under
+  // stream capture, past the sixteenth stream, planes beyond the block's size) adds with atomicAdd in arrival order.
+  float *planes = nullptr;
+  int n_planes = 0;
+  if constexpr (Epi == EPI_BIAS_RELU_ROWSUM) {
+    n_planes = !tiled ? (n + 63) / 64 : (nm > 0 ? (nm + tile_choice - 1) / tile_choice : 0) + (n & 1);
+    if (static_cast<int64_t>(n_planes) * m * 4 <= static_cast<int64_t>(kSplitWorkspaceBytes)) planes = splitk_workspace(st);
+    if (!planes) {
+      hipLaunchKernelGGL(zero_f32_kernel, dim3((m + 255) / 256), dim3(256), 0, st, rowsum, m);
+      const int rc = check_launch("rowsum clear launch");
+      if (rc != SAREK_HIP_OK) return rc;
     }
   }
-  // The MFMA kernel issues 16-byte loads: rows of A and B must keep 16-byte alignment.
-  const bool vec_ok = (k % 8 == 0) && (n % 8 == 0) &&
-                      (reinterpret_cast<uintptr_t>(a) % 16 == 0) &&
-                      (reinterpret_cast<uintptr_t>(b) % 16 == 0);
-  if (vec_ok && tunable("gemm16.force_simple", 0) == 0) {
-    const int tiles_m = (m + BM - 1) / BM, tiles_n = (n + BN - 1) / BN;
-    const int remap = (int)tunable("gemm.xcd_remap", 1);
-    // DMA offsets are 32-bit: 256 rows of A and 64 rows of B must span less than 2 GiB
-    const bool offsets_ok = static_cast<int64_t>(k) * 256 * 2 < 0x7FFFFFFF &&
-                            static_cast<int64_t>(n) * 64 * 2 < 0x7FFFFFFF;
-    if (k % BK == 0 && offsets_ok && tunable("gemm16.force_staged", 0) == 0) {
-      // gemm16.mfma: 16 = the kernel on the 16 x 16 x 32 instruction (default; ring 0 and tj 2 only), 32 = 32 x 32 x 16.
-      // shape knobs for sweeps: gemm16.ring 0 = A in K=64 stages x2 + B in K=32 slabs x4
-      // (default), 4 = both in K=32 slabs x4, 2 = both in K=64 slabs x2; gemm16.tj 2 | 4
-      const int ring = (int)tunable("gemm16.ring", 0), tj = (int)tunable("gemm16.tj", 2);
-      const dim3 grid(tiles_m * tiles_n);
-      unsigned long long *probe = clock_probe(static_cast<int64_t>(tiles_m) * tiles_n);
-#define SAREK_LAUNCH_DMA(BKA, BKB, NA, NB, TJ)                                                      \
-  hipLaunchKernelGGL((gemm16_dma_kernel<Bf16, Epi, BKA, BKB, NA, NB, TJ>), grid,                      \
-                     dim3(64 * 2 * (8 / TJ)), 0, st, a, b, c, bias, rowsum, m, n, k, tiles_m,         \
-                     tiles_n, remap, probe)
-      const int ablate = (int)tunable("gemm16.ablate", 0);
-      const bool m16 = ring == 0 && tj == 2 && tunable("gemm16.mfma", 16) == 16;
-      if (m16 && ablate >= 1 && ablate <= 3 && Bf16 && Epi == EPI_STORE) {
-        // the same measurement variants for the 16 x 16 x 32 kernel (1: no transfers, 2: no fragment reads, 3: neither)
-        if constexpr (Bf16 && Epi == EPI_STORE) {
-#define SAREK_LAUNCH_M16_ABLATED(AB)                                                                        \
-  hipLaunchKernelGGL((gemm16_m16_kernel<true, EPI_STORE, AB>), grid, dim3(512), 0, st, a, b, c, bias, rowsum, m, n, k, \
-                     tiles_m, tiles_n, remap, probe, n)
-          if (ablate == 1) SAREK_LAUNCH_M16_ABLATED(1);
-          else if (ablate == 2) SAREK_LAUNCH_M16_ABLATED(2);
-          else SAREK_LAUNCH_M16_ABLATED(3);
-#undef SAREK_LAUNCH_M16_ABLATED
-        }
-        return check_launch("gemm16 kernel launch");
-      }
-      if (m16 && ablate != 0)
-        return fail(SAREK_HIP_E_UNSUPPORTED, "gemm16.ablate with the 16 x 16 x 32 kernel: 1..3, bf16 without epilogue (4 and 8: gemm16.mfma=32)");
-      if (ablate != 0) {
-        // measurement variants of the default shape (bf16, plain store); anything else is refused
-        if (!Bf16 || Epi != EPI_STORE || ring != 0 || tj != 2 || ablate < 1 || (ablate > 4 && ablate != 8))
-          return fail(SAREK_HIP_E_UNSUPPORTED, "gemm16.ablate is for the default bf16 kernel only (1..4, 8)");
-        if constexpr (Bf16 && Epi == EPI_STORE) {
-#define SAREK_LAUNCH_ABLATED(AB)                                                                    \
-  hipLaunchKernelGGL((gemm16_dma_kernel<true, EPI_STORE, 64, 32, 2, 4, 2, AB>), grid, dim3(512), 0, st, a, b, c, \
-                     bias, rowsum, m, n, k, tiles_m, tiles_n, remap, probe)
-          if (ablate == 1) SAREK_LAUNCH_ABLATED(1);
-          else if (ablate == 2) SAREK_LAUNCH_ABLATED(2);
-          else if (ablate == 3) SAREK_LAUNCH_ABLATED(3);
-          else if (ablate == 8) SAREK_LAUNCH_ABLATED(8);
-          else SAREK_LAUNCH_ABLATED(4);
-#undef SAREK_LAUNCH_ABLATED
-        }
-        return check_launch("gemm16 kernel launch");
-      }
-      if (ring == 4 && tj == 2) SAREK_LAUNCH_DMA(32, 32, 4, 4, 2);
-      else if (ring == 4) SAREK_LAUNCH_DMA(32, 32, 4, 4, 4);
-      else if (ring == 2 && tj == 2) SAREK_LAUNCH_DMA(64, 64, 2, 2, 2);
-      else if (ring == 2) SAREK_LAUNCH_DMA(64, 64, 2, 2, 4);
-      else if (tj == 4) SAREK_LAUNCH_DMA(64, 32, 2, 4, 4);
-      else SAREK_LAUNCH_DMA(64, 32, 2, 4, 2);
-#undef SAREK_LAUNCH_DMA
-      return check_launch("gemm16 kernel launch");
-    }
-    static bool attr_done[2][2] = {{false, false}, {false, false}};
-    auto kern = gemm16_staged_kernel<Bf16, Epi>;
-    if (!attr_done[Bf16][Epi]) {
-      SAREK_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
-                                        hipFuncAttributeMaxDynamicSharedMemorySize, LDS_BYTES));
-      attr_done[Bf16][Epi] = true;
-    }
-    hipLaunchKernelGGL(kern, dim3(tiles_m * tiles_n), dim3(THREADS), LDS_BYTES, st, a, b, c, bias,
-                       rowsum, m, n, k, tiles_m, tiles_n, remap);
-  } else {
-    auto kern = gemm16_simple_kernel<Bf16, Epi>;
-    hipLaunchKernelGGL(kern, dim3((n + 63) / 64, (m + 3) / 4), dim3(256), 0, st, a, b, c, bias,
-                       rowsum, m, n, k);
+  auto finish = [&](int rc) {
+    if (rc != SAREK_HIP_OK || !planes) return rc;
+    hipLaunchKernelGGL(rowsum_fold_kernel, dim3((m + 255) / 256), dim3(256), 0, st, planes, n_planes, m, rowsum);
+    return check_launch("rowsum fold launch");
+  };
+
+  if (!tiled) {
+    hipLaunchKernelGGL((gemm16_simple_kernel<Bf16, Epi>), dim3((n + 63) / 64, (m + 3) / 4), dim3(256), 0, st, a, b, c, bias,
+                       rowsum, m, n, k, planes);
+    return finish(check_launch("gemm16 kernel launch"));
   }
-  return check_launch("gemm16 kernel launch");
+  const bool ragged = n % 8 != 0 || k % 64 != 0 || !ab16;   // the kernels' template flag
+  const int remap = (int)tunable("gemm.xcd_remap", 1);
+  int rc = SAREK_HIP_OK;
+  int tile_planes = 0;
+  if (nm > 0 && tile_choice == 128) {
+    const int sm = (m + 127) / 128, sn = (nm + 127) / 128;
+    tile_planes = sn;
+    unsigned long long *sprobe = clock_probe(static_cast<int64_t>(sm) * sn);
+    int splits = 1;
+    float *partials = nullptr;
+    if constexpr (Epi == EPI_STORE) {
+      if (reinterpret_cast<uintptr_t>(c) % 16 == 0) splits = splitk_for(m, n, k);
+      if (splits > 1) partials = splitk_workspace(st);
+      if (!partials) splits = 1;
+    }
+    if (splits > 1) {
+      const int64_t mn = static_cast<int64_t>(m) * n;
+      const int chunk = (((k + 63) / 64 + splits - 1) / splits) * 64;
+      if (ragged)
+        hipLaunchKernelGGL((gemm16_m16_small_kernel<Bf16, Epi, true>), dim3(sm * sn, splits), dim3(256), 0, st, a, b, c,
+                           bias, rowsum, m, nm, k, sm, sn, remap, nullptr, chunk, partials, n, planes);
+      else
+        hipLaunchKernelGGL((gemm16_m16_small_kernel<Bf16, Epi, false>), dim3(sm * sn, splits), dim3(256), 0, st, a, b, c,
+                           bias, rowsum, m, nm, k, sm, sn, remap, nullptr, chunk, partials, n, planes);
+      rc = check_launch("gemm16 kernel launch");
+      if (rc != SAREK_HIP_OK) return rc;
+      rc = launch_splitk_reduce(partials, c, mn, splits, st);
+    } else {
+      if (ragged)
+        hipLaunchKernelGGL((gemm16_m16_small_kernel<Bf16, Epi, true>), dim3(sm * sn), dim3(256), 0, st, a, b, c, bias,
+                           rowsum, m, nm, k, sm, sn, remap, sprobe, k, nullptr, n, planes);
+      else
+        hipLaunchKernelGGL((gemm16_m16_small_kernel<Bf16, Epi, false>), dim3(sm * sn), dim3(256), 0, st, a, b, c, bias,
+                           rowsum, m, nm, k, sm, sn, remap, sprobe, k, nullptr, n, planes);
+      rc = check_launch("gemm16 kernel launch");
+    }
+  } else if (nm > 0) {
+    const int tiles_m = (m + BM - 1) / BM, tiles_n = (nm + BN - 1) / BN;
+    tile_planes = tiles_n;
+    unsigned long long *probe = clock_probe(static_cast<int64_t>(tiles_m) * tiles_n);
+    if (ragged)
+      hipLaunchKernelGGL((gemm16_m16_kernel<Bf16, Epi, 0, true>), dim3(tiles_m * tiles_n), dim3(512), 0, st, a, b, c, bias,
+                         rowsum, m, nm, k, tiles_m, tiles_n, remap, probe, n, planes);
+    else
+      hipLaunchKernelGGL((gemm16_m16_kernel<Bf16, Epi, 0, false>), dim3(tiles_m * tiles_n), dim3(512), 0, st, a, b, c, bias,
+                         rowsum, m, nm, k, tiles_m, tiles_n, remap, probe, n, planes);
+    rc = check_launch("gemm16 kernel launch");
+  }
+  if (rc != SAREK_HIP_OK) return rc;
+  if (nm != n) {
+    hipLaunchKernelGGL((gemm16_last_column_kernel<Bf16, Epi>), dim3((m + 3) / 4), dim3(256), 0, st, a, b, c, bias, rowsum,
+                       m, n, k, planes ? planes + static_cast<int64_t>(tile_planes) * m : nullptr);
+    rc = check_launch("gemm16 last-column launch");
+  }
+  return finish(rc);
 }
 
 }  // namespace

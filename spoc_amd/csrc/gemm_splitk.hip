@@ -25,24 +25,26 @@ __global__ __launch_bounds__(256) void splitk_reduce_kernel(const float *__restr
 
 }  // namespace
 
-// One block of kSplitWorkspaceBytes per (device, stream), allocated at the first split product on that stream and kept
-// until the process ends (never grown or freed, so a pointer handed out stays good whatever other threads do): calls on
-// different streams never share one, calls on one stream are ordered by it.  nullptr (the caller then does not split)
-// for a stream under capture that has none yet, past 16 streams, or when the allocation fails.
+// One block of kSplitWorkspaceBytes per (device, stream), allocated at the first call that wants one on that stream and
+// kept until the process ends (never grown or freed, so a pointer handed out stays good whatever other threads do):
+// calls on different streams never share one, calls on one stream are ordered by it.  nullptr (the caller then works
+// without one: no K split, row sums by atomicAdd) for a stream under capture -- a recorded graph would carry the
+// block's address to wherever it is replayed, next to eager calls or other replays that use the same block --, past 16
+// streams, or when the allocation fails.
 float *splitk_workspace(hipStream_t st) {
   static std::mutex mu;
   static std::map<std::pair<int, hipStream_t>, void *> blocks;
   int dev = 0;
   if (hipGetDevice(&dev) != hipSuccess) return nullptr;
-  std::lock_guard<std::mutex> lock(mu);
-  auto it = blocks.find({dev, st});
-  if (it != blocks.end()) return static_cast<float *>(it->second);
-  if (blocks.size() >= 16) return nullptr;
   hipStreamCaptureStatus capturing = hipStreamCaptureStatusNone;
   if (hipStreamIsCapturing(st, &capturing) != hipSuccess || capturing != hipStreamCaptureStatusNone) {
     (void)hipGetLastError();
     return nullptr;
   }
+  std::lock_guard<std::mutex> lock(mu);
+  auto it = blocks.find({dev, st});
+  if (it != blocks.end()) return static_cast<float *>(it->second);
+  if (blocks.size() >= 16) return nullptr;
   void *p = nullptr;
   if (hipMalloc(&p, kSplitWorkspaceBytes) != hipSuccess) {
     (void)hipGetLastError();

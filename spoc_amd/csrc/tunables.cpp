@@ -53,13 +53,23 @@ void set_tunable(const char *name, int64_t value) {
 
 extern "C" int sarek_hip_set_tunable(const char *name, int64_t value) {
   if (!name) return SAREK_HIP_E_INVALID_ARG;
+  // knobs of kernels that only the measurement build holds (some of them compute wrong results on purpose)
+  if (!sarek_hip::kMeasureBuild)
+    for (const char *measure_only : {"gemm16.ablate", "gemm16.ring", "gemm16.tj", "gemm16.mfma"})
+      if (std::string_view(name) == measure_only)
+        return sarek_hip::fail(SAREK_HIP_E_UNSUPPORTED, "tunable %s exists in the measurement build only (libsarek_hip_measure.so)",
+                               name);
   sarek_hip::set_tunable(name, value);
   return SAREK_HIP_OK;
 }
 
+extern "C" int sarek_hip_is_measurement_build(void) { return sarek_hip::kMeasureBuild ? 1 : 0; }
+
 extern "C" int sarek_hip_set_clock_probe(uint64_t *device_pairs, int64_t capacity_pairs,
                                          int64_t *ticks_per_second) {
   using namespace sarek_hip;
+  if (!kMeasureBuild)
+    return fail(SAREK_HIP_E_UNSUPPORTED, "the in-kernel clock probe exists in the measurement build only (libsarek_hip_measure.so)");
   if (device_pairs && capacity_pairs <= 0)
     return fail(SAREK_HIP_E_INVALID_ARG, "clock probe: capacity must be positive");
   if (ticks_per_second) {

@@ -9,7 +9,10 @@ import ctypes as C
 import os
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
-LIB_PATH = os.path.join(_HERE, "libsarek_hip.so")
+# SAREK_HIP_MEASURE_BUILD=1 (bench.py --measure-build) loads the measurement build instead: the product's code plus the
+# kernel variants of the ablation studies (`make -C spoc_amd/csrc measure`).  Tests and the default bench use the product.
+MEASURE_BUILD = os.environ.get("SAREK_HIP_MEASURE_BUILD", "0") == "1"
+LIB_PATH = os.path.join(_HERE, "libsarek_hip_measure.so" if MEASURE_BUILD else "libsarek_hip.so")
 
 
 class SarekHipError(RuntimeError):
@@ -216,6 +219,7 @@ SYMBOLS = {
     "sarek_hip_execute_run_source_file": (_i, [C.c_char_p, C.c_char_p, _int3, _int3, _i, _i, C.POINTER(VArg), _i]),
     "sarek_hip_set_tunable": (_i, [C.c_char_p, _i64]),
     "sarek_hip_set_clock_probe": (_i, [_vp, _i64, C.POINTER(_i64)]),
+    "sarek_hip_is_measurement_build": (_i, []),
 }
 
 
@@ -291,8 +295,87 @@ def cache_reset_stats():
     check(lib.sarek_hip_cache_reset_stats())
 
 
+SHADER_CLOCK_SRC = r"""
+// One wave per workgroup sleeps for `ticks` of the constant-rate clock and reports how many shader cycles passed.
+extern "C" __global__ void shader_clock_sample(unsigned long long* out, int ticks) {
+  const long long t0 = wall_clock64(), c0 = clock64();
+  long long t1 = t0;
+  while (t1 - t0 < ticks) {           // bounded by the constant-rate clock: the wave always leaves
+    __builtin_amdgcn_s_sleep(64);
+    t1 = wall_clock64();
+  }
+  if (threadIdx.x == 0) {
+    out[2 * blockIdx.x] = (unsigned long long)(clock64() - c0);
+    out[2 * blockIdx.x + 1] = (unsigned long long)(t1 - t0);
+  }
+}
+"""
+
+
+class shader_clock_sampler:
+    """The shader clock while other kernels run, without anything inside those kernels: eight sleeping waves on a stream
+    of their own count shader cycles against the constant-rate clock for `window_ms`, next to whatever the caller
+    launches right after `start()`.  They hold no LDS and eight registers, so they sit beside any resident workgroup."""
+
+    def __init__(self, waves=8):
+        torch = _torch()
+        self.waves = waves
+        self.buf = torch.zeros(2 * waves, dtype=torch.int64, device="cuda")
+        self.stream = C.c_void_p()
+        check(lib.sarek_hip_stream_create(C.byref(self.stream)))
+        self.kernel = C.c_void_p()
+        log = C.create_string_buffer(4096)
+        check(lib.sarek_hip_kernel_compile_cached(SHADER_CLOCK_SRC.encode(), b"shader_clock_sample", C.byref(self.kernel),
+                                                  log, len(log)))
+        self.ticks_per_ms = None
+
+    def _rate(self):
+        """Ticks of the constant-rate clock per millisecond, from one 2 ms sample against HIP events."""
+        if self.ticks_per_ms is None:
+            torch = _torch()
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            st = torch.cuda.ExternalStream(self.stream.value)
+            self.buf.zero_()
+            torch.cuda.synchronize()
+            e0.record(st)
+            self._launch(200_000)     # 2 ms at the usual 100 MHz; only the ratio below is used
+            e1.record(st)
+            torch.cuda.synchronize()
+            ticks = int(self.buf.view(-1, 2)[0, 1].item())
+            self.ticks_per_ms = ticks / e0.elapsed_time(e1)
+        return self.ticks_per_ms
+
+    def _launch(self, ticks):
+        out, t = C.c_void_p(self.buf.data_ptr()), C.c_int(int(ticks))
+        params = (C.c_void_p * 2)(C.cast(C.pointer(out), C.c_void_p), C.cast(C.pointer(t), C.c_void_p))
+        grid, block = (C.c_uint * 3)(self.waves, 1, 1), (C.c_uint * 3)(64, 1, 1)
+        check(lib.sarek_hip_kernel_launch(self.kernel, grid, block, 0, self.stream, params, 2))
+        self._keep = (out, t, params)
+
+    def start(self, window_ms):
+        """Queue the sampling waves; the caller launches its own work next and waits for the device."""
+        rate = self._rate()
+        self.buf.zero_()
+        _torch().cuda.synchronize()
+        self._launch(min(window_ms, 20.0) * rate)
+
+    def mhz(self):
+        _torch().cuda.synchronize()
+        p = self.buf.view(-1, 2).cpu().numpy()
+        p = p[p[:, 1] > 0]
+        if len(p) == 0:
+            return None
+        return float(p[:, 0].sum()) / float(p[:, 1].sum()) * self._rate() / 1e3
+
+    def close(self):
+        if self.stream:
+            _torch().cuda.synchronize()
+            check(lib.sarek_hip_stream_destroy(self.stream))
+            self.stream = C.c_void_p()
+
+
 class clock_probe:
-    """Context manager: MFMA GEMM launches inside it record, per workgroup, the shader-clock
+    """Measurement build only.  Context manager: MFMA GEMM launches inside it record, per workgroup, the shader-clock
     cycles and wall-clock ticks it was resident.  `mhz()` is the shader clock those
     workgroups ran at, averaged over the last launch that fitted the buffer."""
 

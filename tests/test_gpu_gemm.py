@@ -7,10 +7,19 @@ Tolerances (stated by the task for this path):
   bf16/fp16-in  <= 2e-2 relative, measured as max|err| / max|C_ref|
 The 16-bit inputs are rounded once (RNE) and both sides consume the same rounded values,
 so the observed error is f32-accumulation error only and is asserted much tighter."""
+import ctypes as C
+import os
+
 import numpy as np
 import pytest
 
 pytestmark = pytest.mark.gpu
+
+
+def rowsums_ok(rs, rs_ref):
+    """Row sums of non-negative values: every row within 1e-5 of its own reference (the bar for f32 reductions)."""
+    rs, rs_ref = np.asarray(rs, np.float64), np.asarray(rs_ref, np.float64)
+    return bool((np.abs(rs - rs_ref) <= 1e-5 * np.abs(rs_ref) + 1e-30).all())
 
 
 def dev(torch, x):
@@ -147,7 +156,7 @@ def test_epilogue_vs_oracle(hip, oracle, torch_cuda, m, n, k):
     assert np.abs(y - y_ref).max() <= 2e-2 * np.abs(y_ref).max()
     assert np.abs(y - y_ref).max() <= 1e-5 * max(1.0, np.abs(y_ref).max())
     assert (y >= 0).all()
-    assert np.abs(rs - rs_ref).max() <= 1e-4 * np.abs(rs_ref).max()
+    assert rowsums_ok(rs, rs_ref)
 
 
 def test_epilogue_full_size_config(hip, oracle, torch_cuda):
@@ -164,9 +173,61 @@ def test_epilogue_full_size_config(hip, oracle, torch_cuda):
     idx = torch.from_numpy(rows).long().cuda()
     got = y[idx].cpu().numpy()
     assert np.abs(got - y_ref).max() <= 2e-2 * np.abs(y_ref).max()
-    assert np.abs(rs[idx].cpu().numpy() - rs_ref).max() <= 1e-4 * np.abs(rs_ref).max()
-    # size-independent: the fused row sums equal the row sums of the stored Y
-    assert torch.allclose(rs, y.double().sum(dim=1).float(), rtol=1e-4, atol=1e-3)
+    assert rowsums_ok(rs[idx].cpu().numpy(), rs_ref)
+    # size-independent: the fused row sums equal the row sums of the stored Y, row by row, and a second run's bits
+    assert rowsums_ok(rs.cpu().numpy(), y.double().sum(dim=1).cpu().numpy())
+    assert torch.equal(hip.gemm_f16_bias_relu_rowsum(dev(torch, a).half(), dev(torch, b).half(), dev(torch, bias))[1], rs)
+
+
+def test_epilogue_row_sums_are_the_same_bits_on_every_run(hip, oracle, torch_cuda):
+    """The tiles' shares of a row are added in tile order, in double, with one rounding -- not in the order the
+    tiles finish: five runs of a shape with 43 tile columns give the same bits, on the main stream and on another;
+    both tile sizes, an odd N (whose last column comes from a kernel of its own) and the one-thread-per-element kernel
+    each agree with themselves run to run and with the oracle row by row.  Under stream capture no plane block is
+    handed out and the shares are added by atomicAdd: that path is checked against the oracle too."""
+    torch = torch_cuda
+    rng = np.random.default_rng(0xD7)
+    for (m, n, k), tile in [((300, 11008, 128), 256), ((300, 11008, 128), 128), ((259, 1001, 192), 0), ((70, 200, 24), 0),
+                            ((33, 130, 20), 0)]:
+        a = oracle.round_f16(rng.normal(0, 0.02, (m, k)).astype(np.float32))
+        b = oracle.round_f16(rng.normal(0, 0.02, (k, n)).astype(np.float32))
+        bias = oracle.fill_uniform(n, seed=n, lo=-0.1, hi=0.1)
+        da, db, dbias = dev(torch, a).half(), dev(torch, b).half(), dev(torch, bias)
+        _, rs_ref = oracle.gemm_bias_relu_rowsum(a, b, bias)
+        hip.set_tunable("gemm16.tile", tile)
+        try:
+            runs = [hip.gemm_f16_bias_relu_rowsum(da, db, dbias)[1].clone() for _ in range(5)]
+            side = side_stream(torch)
+            side.wait_stream(torch.cuda.current_stream())
+            with torch.cuda.stream(side):
+                runs.append(hip.gemm_f16_bias_relu_rowsum(da, db, dbias)[1].clone())
+            side.synchronize()
+        finally:
+            hip.set_tunable("gemm16.tile", 0)
+        torch.cuda.synchronize()
+        for r in runs[1:]:
+            assert torch.equal(r, runs[0]), (m, n, k, tile)
+        assert rowsums_ok(runs[0].cpu().numpy(), rs_ref), (m, n, k, tile)
+    # captured: atomics
+    m, n, k = 300, 1024, 128
+    a = oracle.round_f16(rng.normal(0, 0.02, (m, k)).astype(np.float32))
+    b = oracle.round_f16(rng.normal(0, 0.02, (k, n)).astype(np.float32))
+    bias = oracle.fill_uniform(n, seed=n, lo=-0.1, hi=0.1)
+    da, db, dbias = dev(torch, a).half(), dev(torch, b).half(), dev(torch, bias)
+    y_ref, rs_ref = oracle.gemm_bias_relu_rowsum(a, b, bias)
+    y, rs = torch.empty(m, n, device="cuda"), torch.empty(m, device="cuda")
+    hip.gemm_f16_bias_relu_rowsum(da, db, dbias, out=y, rowsum=rs)    # warm: kernels loaded before the capture
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        hip.gemm_f16_bias_relu_rowsum(da, db, dbias, out=y, rowsum=rs)
+    for _ in range(3):
+        rs.fill_(float("nan"))
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert rowsums_ok(rs.cpu().numpy(), rs_ref)
+        assert np.abs(y.cpu().numpy() - y_ref).max() <= 1e-4 * np.abs(y_ref).max()
 
 
 def test_gemm_bf16_full_size_rows(hip, oracle, torch_cuda):
@@ -185,47 +246,44 @@ def test_gemm_bf16_full_size_rows(hip, oracle, torch_cuda):
     assert torch.equal(hip.gemm_bf16(a * 2, b), c * 2)
 
 
-def test_measurement_variants_run_and_leave_the_kernel_as_it_was(hip, torch_cuda):
-    """gemm16.ablate leaves parts of the K loop out for the power measurements (1..3 for both MFMA shapes, 4 for the
-    32 x 32 kernel) and 8 the stores of C (32 x 32 kernel): the results are wrong by construction, but every variant
-    runs within the operands' bounds, other kernels refuse the knob, and with the knobs back the result is the one
-    from before."""
+def test_the_product_library_refuses_the_measurement_knobs(hip, torch_cuda):
+    """The knobs of the ablation studies (kernel variants that leave parts of the K loop out and compute wrong
+    results on purpose, retired kernel shapes, the in-kernel clock probe) exist in the measurement build only:
+    the product library answers each with "unsupported", also when it is asked through the environment, and a
+    product computed afterwards is the one from before."""
     torch = torch_cuda
+    assert hip.lib.sarek_hip_is_measurement_build() == 0
     m, n, k = 512, 768, 512
     torch.manual_seed(7)
     a = (torch.randn(m, k, device="cuda") * 0.1).bfloat16()
     b = (torch.randn(k, n, device="cuda") * 0.1).bfloat16()
     good = hip.gemm_bf16(a, b)
-    try:
-        for mfma, variants in ((16, (1, 2, 3)), (32, (1, 2, 3, 4))):
-            hip.set_tunable("gemm16.mfma", mfma)
-            for v in variants:
-                hip.set_tunable("gemm16.ablate", v)
-                c = hip.gemm_bf16(a, b)
-                torch.cuda.synchronize()
-                assert torch.isfinite(c).all()
-        hip.set_tunable("gemm16.ablate", 8)
-        untouched = torch.full((m, n), 7.0, device="cuda")
-        hip.gemm_bf16(a, b, out=untouched)
-        torch.cuda.synchronize()
-        assert bool((untouched == 7.0).all())
-        for mfma in (16, 32):
-            hip.set_tunable("gemm16.mfma", mfma)
-            hip.set_tunable("gemm16.ablate", 1)
-            with pytest.raises(hip.SarekHipError) as e:
-                hip.gemm_f16(a.half(), b.half())
-            assert e.value.status == hip.E_UNSUPPORTED
-            hip.set_tunable("gemm16.ablate", 5)
-            with pytest.raises(hip.SarekHipError):
-                hip.gemm_bf16(a, b)
-        hip.set_tunable("gemm16.mfma", 16)
-        hip.set_tunable("gemm16.ablate", 8)
-        with pytest.raises(hip.SarekHipError):
-            hip.gemm_bf16(a, b)
-    finally:
-        hip.set_tunable("gemm16.ablate", 0)
-        hip.set_tunable("gemm16.mfma", 16)
+    for knob, value in (("gemm16.ablate", 1), ("gemm16.ablate", 8), ("gemm16.mfma", 32), ("gemm16.ring", 4),
+                        ("gemm16.tj", 4)):
+        with pytest.raises(hip.SarekHipError) as e:
+            hip.set_tunable(knob, value)
+        assert e.value.status == hip.E_UNSUPPORTED and "measurement build" in e.value.message
+    buf = torch.zeros(128, dtype=torch.int64, device="cuda")
+    rate = C.c_int64(0)
+    assert hip.lib.sarek_hip_set_clock_probe(C.c_void_p(buf.data_ptr()), 64, C.byref(rate)) == hip.E_UNSUPPORTED
     assert torch.equal(hip.gemm_bf16(a, b), good)
+    torch.cuda.synchronize()
+    assert int(buf.abs().sum().item()) == 0
+
+
+def test_the_measurement_build_in_a_process_of_its_own():
+    """libsarek_hip_measure.so, loaded by a fresh interpreter (a process holds one of the two libraries): it says what it
+    is, takes the knobs, every variant runs within the operands' bounds, the 32 x 32 x 16 kernel's ring and wave
+    shapes agree with the product's kernel, the clock probe records, and with the knobs back the default kernel
+    gives the product's bits."""
+    import subprocess
+    import sys
+    here = os.path.dirname(os.path.abspath(__file__))
+    env = dict(os.environ, SAREK_HIP_MEASURE_BUILD="1")
+    r = subprocess.run([sys.executable, os.path.join(here, "measure_build_checks.py")], env=env, capture_output=True,
+                       text=True, timeout=600)
+    assert r.returncode == 0, r.stdout[-3000:] + r.stderr[-3000:]
+    assert "measurement build ok" in r.stdout
 
 
 def test_gemm_rejects_bad_arguments(hip, torch_cuda):
@@ -236,39 +294,25 @@ def test_gemm_rejects_bad_arguments(hip, torch_cuda):
     assert e.value.status == hip.E_INVALID_ARG
 
 
-def test_clock_probe_records_cycles_and_ticks(hip, torch_cuda):
-    """The diagnostic probe: one (cycles, ticks) pair per workgroup, plausible clock, and
-    nothing written once it is switched off or when the launch has more workgroups than
-    the buffer holds."""
+def test_shader_clock_sampler_reads_a_plausible_clock(hip, torch_cuda):
+    """The sampling waves next to a GEMM: a clock between the idle and the peak engine clock, with nothing added to
+    the GEMM's own kernels (the product library has no probe inside them)."""
     torch = torch_cuda
-    m = n = 1024
-    k = 512
-    a = torch.randn(m, k, device="cuda").to(torch.bfloat16)
-    b = torch.randn(k, n, device="cuda").to(torch.bfloat16)
-    with hip.clock_probe(workgroups=64) as probe:
-        hip.gemm_bf16(a, b)                      # 64 workgroups of 128 x 128 (16 large tiles would idle most CUs)
-        pairs = probe.pairs()
-        assert hip.gemm16_tile(m, n, k) == 128 and len(pairs) == 64
-        assert 500 < probe.mhz() < 2600
-        probe.buf.zero_()
-        hip.set_tunable("gemm16.tile", 256)
-        try:
-            hip.gemm_bf16(a, b)                  # 16 workgroups of 256 x 256
-        finally:
-            hip.set_tunable("gemm16.tile", 0)
-        assert len(probe.pairs()) == 16
-        assert 500 < probe.mhz() < 2600
-        probe.buf.zero_()
-        hip.gemm_bf16(torch.zeros(4096, 64, device="cuda", dtype=torch.bfloat16),
-                      torch.zeros(64, 8192, device="cuda", dtype=torch.bfloat16))   # 512 > 64
-        assert len(probe.pairs()) == 0
-    probe.buf.zero_()
-    hip.gemm_bf16(a, b)
-    assert len(probe.pairs()) == 0
-    x = torch.randn(512, 256, device="cuda")
-    with hip.clock_probe(workgroups=64) as probe:
-        hip.gemm_f32(x, x[:256, :].contiguous())
-        assert len(probe.pairs()) > 0 and 500 < probe.mhz() < 2600
+    m = n = k = 4096
+    a = (torch.randn(m, k, device="cuda") * 0.02).to(torch.bfloat16)
+    b = (torch.randn(k, n, device="cuda") * 0.02).to(torch.bfloat16)
+    c = torch.empty(m, n, device="cuda")
+    for _ in range(20):
+        hip.gemm_bf16(a, b, out=c)
+    torch.cuda.synchronize()
+    sampler = hip.shader_clock_sampler()
+    try:
+        sampler.start(0.08)
+        hip.gemm_bf16(a, b, out=c)
+        mhz = sampler.mhz()
+    finally:
+        sampler.close()
+    assert mhz is not None and 400 < mhz < 2600, mhz
 
 
 @pytest.mark.parametrize("tile", [64, 128, 256])
@@ -284,60 +328,6 @@ def test_gemm_f32_every_tile_shape(hip, oracle, torch_cuda, tile, m, n, k):
     finally:
         hip.set_tunable("gemm_f32.tile", 0)
     assert np.abs(c - oracle.gemm(a, b)).max() <= f32_tol(a, b, k)
-
-
-@pytest.mark.parametrize("ring,tj,mfma", [(0, 2, 16), (0, 2, 32), (0, 4, 32), (4, 2, 32), (4, 4, 32), (2, 2, 32), (2, 4, 32)])
-@pytest.mark.parametrize("m,n,k", [(300, 520, 64), (257, 136, 192), (512, 768, 448), (70, 1032, 1216)])
-def test_gemm16_every_ring_shape(hip, oracle, torch_cuda, ring, tj, mfma, m, n, k):
-    """Every instantiation of the direct-to-LDS 16-bit kernels (the 16 x 16 x 32 kernel; the 32 x 32 x 16 kernel's
-    A/B ring shapes with 8 or 4 waves) on ragged M, N and on K values that end the stage pattern at different
-    positions."""
-    a = normal16(oracle, (m, k), m + ring, "bf16")
-    b = normal16(oracle, (k, n), n + tj, "bf16")
-    ref = oracle.gemm(a, b)
-    hip.set_tunable("gemm16.ring", ring)
-    hip.set_tunable("gemm16.tj", tj)
-    hip.set_tunable("gemm16.mfma", mfma)
-    hip.set_tunable("gemm16.tile", 256)   # these are shapes of the 256 x 256 kernels
-    try:
-        c = hip.gemm_bf16(dev(torch_cuda, a).bfloat16(), dev(torch_cuda, b).bfloat16()).cpu().numpy()
-    finally:
-        hip.set_tunable("gemm16.ring", 0)
-        hip.set_tunable("gemm16.tj", 2)
-        hip.set_tunable("gemm16.mfma", 16)
-        hip.set_tunable("gemm16.tile", 0)
-    assert np.abs(c - ref).max() / np.abs(ref).max() < 1e-4
-
-
-@pytest.mark.parametrize("kind", ["bf16", "f16"])
-@pytest.mark.parametrize("m,n,k", [(256, 256, 64), (513, 264, 320), (1000, 72, 128)])
-def test_gemm16_both_mfma_shapes_agree_with_the_oracle_and_each_other(hip, oracle, torch_cuda, kind, m, n, k):
-    """The kernel on v_mfma_f32_16x16x32 (default) and the one on v_mfma_f32_32x32x16, plain and with the fused
-    epilogue: both against the oracle; between the two only the order of the f32 additions differs."""
-    torch = torch_cuda
-    a = normal16(oracle, (m, k), m + 5, kind)
-    b = normal16(oracle, (k, n), n + 6, kind)
-    bias = oracle.fill_uniform(n, seed=n, lo=-0.1, hi=0.1)
-    dt = torch.bfloat16 if kind == "bf16" else torch.float16
-    da, db = dev(torch, a).to(dt), dev(torch, b).to(dt)
-    ref = oracle.gemm(a, b)
-    got = {}
-    hip.set_tunable("gemm16.tile", 256)
-    try:
-        for mfma in (16, 32):
-            hip.set_tunable("gemm16.mfma", mfma)
-            c = (hip.gemm_bf16 if kind == "bf16" else hip.gemm_f16)(da, db).cpu().numpy()
-            assert np.abs(c - ref).max() / np.abs(ref).max() < 1e-4
-            got[mfma] = c
-            if kind == "f16":
-                y, rs = hip.gemm_f16_bias_relu_rowsum(da, db, dev(torch, bias))
-                y_ref, rs_ref = oracle.gemm_bias_relu_rowsum(a, b, bias)
-                assert np.abs(y.cpu().numpy() - y_ref).max() <= 1e-4 * np.abs(y_ref).max()
-                assert np.abs(rs.cpu().numpy() - rs_ref).max() <= 1e-4 * max(np.abs(rs_ref).max(), 1e-30)
-    finally:
-        hip.set_tunable("gemm16.mfma", 16)
-        hip.set_tunable("gemm16.tile", 0)
-    assert np.abs(got[16] - got[32]).max() <= 1e-5 * np.abs(ref).max()
 
 
 @pytest.mark.parametrize("kind", ["bf16", "f16"])
@@ -368,7 +358,7 @@ def test_gemm16_both_tile_sizes(hip, oracle, torch_cuda, kind, m, n, k):
                 y, rs = hip.gemm_f16_bias_relu_rowsum(da, db, dev(torch, bias))
                 y_ref, rs_ref = oracle.gemm_bias_relu_rowsum(a, b, bias)
                 assert np.abs(y.cpu().numpy() - y_ref).max() <= 1e-4 * np.abs(y_ref).max()
-                assert np.abs(rs.cpu().numpy() - rs_ref).max() <= 1e-4 * max(np.abs(rs_ref).max(), 1e-30)
+                assert rowsums_ok(rs.cpu().numpy(), rs_ref)
     finally:
         hip.set_tunable("gemm16.tile", 0)
     assert np.array_equal(got[128], got[256])
@@ -383,11 +373,6 @@ def test_gemm16_tile_choice_by_shape(hip, torch_cuda):
                             ((1000, 1001, 1000), 128), ((1000, 1001, 1001), 128), ((512, 512, 29), 0),
                             ((37, 51, 29), 0)]:
         assert hip.gemm16_tile(m, n, k) == want, (m, n, k)
-    hip.set_tunable("gemm16.mfma", 32)
-    try:
-        assert hip.gemm16_tile(1024, 1024, 1024) == 256   # the 32 x 32 x 16 kernel has the large tile only
-    finally:
-        hip.set_tunable("gemm16.mfma", 16)
 
 
 _SIDE_STREAM = []
@@ -458,7 +443,7 @@ def test_gemm16_split_k_rule_and_epilogue(hip, oracle, torch_cuda):
     y, rs = hip.gemm_f16_bias_relu_rowsum(dev(torch, a).half(), dev(torch, b).half(), dev(torch, bias))
     y_ref, rs_ref = oracle.gemm_bias_relu_rowsum(a, b, bias)
     assert np.abs(y.cpu().numpy() - y_ref).max() <= 1e-4 * np.abs(y_ref).max()
-    assert np.abs(rs.cpu().numpy() - rs_ref).max() <= 1e-4 * np.abs(rs_ref).max()
+    assert rowsums_ok(rs.cpu().numpy(), rs_ref)
 
 
 def test_gemm16_split_k_under_graph_capture(hip, torch_cuda):
@@ -548,7 +533,7 @@ def test_epilogue_ragged_shapes(hip, oracle, torch_cuda, m, n, k):
             hip.set_tunable("gemm16.tile", tile)
             y, rs = hip.gemm_f16_bias_relu_rowsum(dev(torch, a).half(), dev(torch, b).half(), dev(torch, bias))
             assert np.abs(y.cpu().numpy() - y_ref).max() <= 1e-4 * max(np.abs(y_ref).max(), 1e-30)
-            assert np.abs(rs.cpu().numpy() - rs_ref).max() <= 1e-4 * max(np.abs(rs_ref).max(), 1e-30)
+            assert rowsums_ok(rs.cpu().numpy(), rs_ref)
     finally:
         hip.set_tunable("gemm16.tile", 0)
 
@@ -587,9 +572,10 @@ def test_gemm_f32_ragged_shapes_stay_on_the_mfma_kernel(hip, oracle, torch_cuda,
 @pytest.mark.parametrize("knob", ["force_staged", "force_simple"])
 @pytest.mark.parametrize("m,n,k", [(264, 520, 72), (100, 64, 200), (8, 8, 8), (300, 264, 192)])
 def test_fallback_kernels_stay_correct(hip, oracle, torch_cuda, knob, m, n, k):
-    """The register-staged and the one-thread-per-element kernels (16-bit and f32) are what is left when a transfer
-    offset would not fit 32 bits or, for the 32 x 32 x 16 variants, when K is not whole stages; the direct-to-LDS
-    kernels now take the shapes that used to reach them, so they are switched on by their knobs here."""
+    """The one-thread-per-element kernels (16-bit and f32) and the f32 register-staged kernel are what is left when a
+    transfer offset would not fit 32 bits or K is too short for a slab; the direct-to-LDS kernels take the shapes
+    that used to reach them, so they are switched on by their knobs here (the 16-bit library has no staged kernel:
+    with that knob it runs its usual kernels)."""
     torch = torch_cuda
     a16 = normal16(oracle, (m, k), m + 71, "bf16")
     b16 = normal16(oracle, (k, n), n + 72, "bf16")
@@ -598,7 +584,7 @@ def test_fallback_kernels_stay_correct(hip, oracle, torch_cuda, knob, m, n, k):
     hip.set_tunable("gemm16." + knob, 1)
     hip.set_tunable("gemm_f32." + knob, 1)
     try:
-        assert hip.gemm16_tile(m, n, k) == 0
+        assert (hip.gemm16_tile(m, n, k) == 0) == (knob == "force_simple")
         c16 = hip.gemm_bf16(dev(torch, a16).bfloat16(), dev(torch, b16).bfloat16()).cpu().numpy()
         c32 = hip.gemm_f32(dev(torch, a32), dev(torch, b32)).cpu().numpy()
     finally:

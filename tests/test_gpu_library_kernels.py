@@ -168,7 +168,7 @@ def test_epilogue_through_run_source(hip, oracle, sarek, m, n, k):
     assert p_hand == "gemm_f16_bias_relu_rowsum" and p_jit == "jit"
     assert np.array_equal(y_jit, y_ref) and np.array_equal(rs_jit, rs_ref)
     assert np.abs(y_hand - y_ref).max() <= 1e-4 * np.abs(y_ref).max()
-    assert np.abs(rs_hand - rs_ref).max() <= 1e-4 * np.abs(rs_ref).max()
+    assert (np.abs(rs_hand.astype(np.float64) - rs_ref) <= 1e-5 * np.abs(rs_ref)).all()   # row by row
     assert (y_hand >= 0).all()
 
 
