@@ -26,15 +26,13 @@ std::mutex g_tagged_mu;
 std::unordered_set<std::string, ViewHash, std::equal_to<>> g_tagged;
 constexpr size_t kTaggedMax = 4096;     // beyond this the set starts over: forgotten texts run as compiled
 // The element-wise kernels among them (tag map_f32), by their text: what run_source needs to rebuild them
-std::unordered_map<std::string, ir::MapKernel, ViewHash, std::equal_to<>> g_maps;
+std::unordered_map<std::string, std::shared_ptr<MapEntry>, ViewHash, std::equal_to<>> g_maps;
 }  // namespace
 
-bool find_generated_map(const char *source, ir::MapKernel *out) {
+std::shared_ptr<MapEntry> find_generated_map(const char *source) {
   std::lock_guard<std::mutex> lock(g_tagged_mu);
   const auto it = g_maps.find(std::string_view(source));
-  if (it == g_maps.end()) return false;
-  if (out) *out = it->second;
-  return true;
+  return it == g_maps.end() ? nullptr : it->second;
 }
 
 bool is_generated_tagged_text(const char *source) {
@@ -75,7 +73,11 @@ extern "C" int sarek_hip_generate_source(const char *ir_text, const int block[3]
       g_tagged.clear();
       g_maps.clear();
     }
-    if (map) g_maps.emplace(src, std::move(*map));
+    if (map && g_maps.find(std::string_view(src)) == g_maps.end()) {
+      auto entry = std::make_shared<MapEntry>();
+      entry->m = std::move(*map);
+      g_maps.emplace(src, std::move(entry));
+    }
     g_tagged.insert(std::move(src));
   }
   return SAREK_HIP_OK;

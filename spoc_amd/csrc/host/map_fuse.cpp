@@ -39,13 +39,11 @@ bool is_global_id(const ExprP &e) {
   return false;
 }
 
-// Names the rebuilt texts use themselves (their own prefix, the element variables' suffix, the loop variables of the
-// kernel bodies): a parameter of that name would be shadowed there, so such a kernel stays with the generated code.
+// Names the rebuilt texts use themselves: everything of their own carries the prefix sarek_f_ (the loop variables of
+// the kernel bodies included), the element variables the suffix __e.  A parameter spelled like that would be shadowed
+// there, so such a kernel stays with the generated code; any other name, however short, is the kernel's to use.
 bool name_is_free(const std::string &n) {
-  if (n.compare(0, 8, "sarek_f_") == 0 || (n.size() > 3 && n.compare(n.size() - 3, 3, "__e") == 0)) return false;
-  for (const char *own : {"u", "j", "i", "e", "v", "t", "q", "o4"})
-    if (n == own) return false;
-  return true;
+  return n.compare(0, 8, "sarek_f_") != 0 && !(n.size() > 3 && n.compare(n.size() - 3, 3, "__e") == 0);
 }
 
 struct Matcher {
@@ -314,62 +312,62 @@ std::string map_source(const MapKernel &m, int reduce, bool nt_loads, uint32_t p
   o += "  if (sarek_f_full) {\n";
   for (size_t i = 0; i < m.inputs.size(); ++i) {
     const std::string is = std::to_string(i);
-    o += "    sarek_f_v4 sarek_f_x" + is + "[4];\n#pragma unroll\n    for (int u = 0; u < 4; ++u) sarek_f_x" + is + "[u] = " +
-         (nt_loads ? "__builtin_nontemporal_load(sarek_f_p" + is + " + sarek_f_base + 64 * u)"
-                   : "sarek_f_p" + is + "[sarek_f_base + 64 * u]") +
+    o += "    sarek_f_v4 sarek_f_x" + is + "[4];\n#pragma unroll\n    for (int sarek_f_u = 0; sarek_f_u < 4; ++sarek_f_u) sarek_f_x" + is + "[sarek_f_u] = " +
+         (nt_loads ? "__builtin_nontemporal_load(sarek_f_p" + is + " + sarek_f_base + 64 * sarek_f_u)"
+                   : "sarek_f_p" + is + "[sarek_f_base + 64 * sarek_f_u]") +
          ";\n";
   }
-  o += "#pragma unroll\n    for (int u = 0; u < 4; ++u)\n#pragma unroll\n      for (int j = 0; j < 4; ++j)\n"
-       "        sarek_f_r[u][j] = " + apply("sarek_f_x@[u][j]", "(sarek_f_base + 64 * u) * 4 + j") + ";\n";
-  o += "#pragma unroll\n    for (int u = 0; u < 4; ++u) __builtin_nontemporal_store(sarek_f_r[u], sarek_f_po + sarek_f_base + 64 * u);\n";
-  o += "  } else {\n#pragma unroll\n    for (int u = 0; u < 4; ++u) {\n      const long long i = sarek_f_base + 64 * u;\n"
-       "      sarek_f_r[u] = sarek_f_v4{0.f, 0.f, 0.f, 0.f};\n      if (i < sarek_f_n4) {\n";
+  o += "#pragma unroll\n    for (int sarek_f_u = 0; sarek_f_u < 4; ++sarek_f_u)\n#pragma unroll\n      for (int sarek_f_j = 0; sarek_f_j < 4; ++sarek_f_j)\n"
+       "        sarek_f_r[sarek_f_u][sarek_f_j] = " + apply("sarek_f_x@[sarek_f_u][sarek_f_j]", "(sarek_f_base + 64 * sarek_f_u) * 4 + sarek_f_j") + ";\n";
+  o += "#pragma unroll\n    for (int sarek_f_u = 0; sarek_f_u < 4; ++sarek_f_u) __builtin_nontemporal_store(sarek_f_r[sarek_f_u], sarek_f_po + sarek_f_base + 64 * sarek_f_u);\n";
+  o += "  } else {\n#pragma unroll\n    for (int sarek_f_u = 0; sarek_f_u < 4; ++sarek_f_u) {\n      const long long sarek_f_i = sarek_f_base + 64 * sarek_f_u;\n"
+       "      sarek_f_r[sarek_f_u] = sarek_f_v4{0.f, 0.f, 0.f, 0.f};\n      if (sarek_f_i < sarek_f_n4) {\n";
   for (size_t i = 0; i < m.inputs.size(); ++i)
-    o += "        const sarek_f_v4 sarek_f_y" + std::to_string(i) + " = sarek_f_p" + std::to_string(i) + "[i];\n";
-  o += "#pragma unroll\n        for (int j = 0; j < 4; ++j) sarek_f_r[u][j] = " + apply("sarek_f_y@[j]", "i * 4 + j") + ";\n"
-       "        sarek_f_po[i] = sarek_f_r[u];\n      }";
+    o += "        const sarek_f_v4 sarek_f_y" + std::to_string(i) + " = sarek_f_p" + std::to_string(i) + "[sarek_f_i];\n";
+  o += "#pragma unroll\n        for (int sarek_f_j = 0; sarek_f_j < 4; ++sarek_f_j) sarek_f_r[sarek_f_u][sarek_f_j] = " + apply("sarek_f_y@[sarek_f_j]", "sarek_f_i * 4 + sarek_f_j") + ";\n"
+       "        sarek_f_po[sarek_f_i] = sarek_f_r[sarek_f_u];\n      }";
   {
     std::string a = "sarek_f_opaque(sarek_f_apply(";
     for (int p : m.inputs) a += m.params[p].name + "[sarek_f_k], ";
     a += actuals_tail + "(int)sarek_f_k))";
     if (with_max) {
       // the slot that holds the end of the vector takes its one to three elements; everything past n is the fill value
-      o += " else {\n#pragma unroll\n        for (int e = 0; e < 4; ++e) {\n          const long long sarek_f_k = (i << 2) + e;\n"
-           "          sarek_f_r[u][e] = " + std::string(pad) + ";\n          if (sarek_f_k < sarek_f_n) {\n            sarek_f_r[u][e] = " + a +
-           ";\n            " + out + "[sarek_f_k] = sarek_f_r[u][e];\n          }\n        }\n      }\n";
+      o += " else {\n#pragma unroll\n        for (int sarek_f_e = 0; sarek_f_e < 4; ++sarek_f_e) {\n          const long long sarek_f_k = (sarek_f_i << 2) + sarek_f_e;\n"
+           "          sarek_f_r[sarek_f_u][sarek_f_e] = " + std::string(pad) + ";\n          if (sarek_f_k < sarek_f_n) {\n            sarek_f_r[sarek_f_u][sarek_f_e] = " + a +
+           ";\n            " + out + "[sarek_f_k] = sarek_f_r[sarek_f_u][sarek_f_e];\n          }\n        }\n      }\n";
     } else {
       // the lane whose slot holds the end of the vector takes the one to three elements there, summed apart (kept
       // out of the vector registers: folding them into r measured 2.7 % slower on the whole kernel)
-      o += "\n      if (i == sarek_f_n4) {\n        for (long long sarek_f_k = sarek_f_n4 << 2; sarek_f_k < sarek_f_n; ++sarek_f_k) {\n"
-           "          const float v = " + a + ";\n          " + out + "[sarek_f_k] = v;\n          sarek_f_extra[u] += v;\n        }\n      }\n";
+      o += "\n      if (sarek_f_i == sarek_f_n4) {\n        for (long long sarek_f_k = sarek_f_n4 << 2; sarek_f_k < sarek_f_n; ++sarek_f_k) {\n"
+           "          const float sarek_f_v = " + a + ";\n          " + out + "[sarek_f_k] = sarek_f_v;\n          sarek_f_extra[sarek_f_u] += sarek_f_v;\n        }\n      }\n";
     }
   }
   o += "    }\n  }\n";
   if (with_sums) {
     o += "  const long long sarek_f_nblocks = (sarek_f_n + 255) >> 8;\n  float sarek_f_t[4];\n#pragma unroll\n"
-         "  for (int u = 0; u < 4; ++u)\n    sarek_f_t[u] = sarek_f_wave_sum(((sarek_f_r[u][0] + sarek_f_r[u][1]) + "
-         "(sarek_f_r[u][2] + sarek_f_r[u][3])) + sarek_f_extra[u]);\n"
+         "  for (int sarek_f_u = 0; sarek_f_u < 4; ++sarek_f_u)\n    sarek_f_t[sarek_f_u] = sarek_f_wave_sum(((sarek_f_r[sarek_f_u][0] + sarek_f_r[sarek_f_u][1]) + "
+         "(sarek_f_r[sarek_f_u][2] + sarek_f_r[sarek_f_u][3])) + sarek_f_extra[sarek_f_u]);\n"
          "  const long long sarek_f_j0 = (long long)blockIdx.x * 16 + (threadIdx.x >> 6) * 4;\n"
          "  if ((threadIdx.x & 63) == 0) {\n    if (sarek_f_j0 + 4 <= sarek_f_nblocks) {\n"
          "      *reinterpret_cast<sarek_f_v4*>(sarek_f_partials + sarek_f_j0) = "
          "sarek_f_v4{sarek_f_t[0], sarek_f_t[1], sarek_f_t[2], sarek_f_t[3]};\n    } else {\n#pragma unroll\n"
-         "      for (int u = 0; u < 4; ++u)\n        if (sarek_f_j0 + u < sarek_f_nblocks) sarek_f_partials[sarek_f_j0 + u] = sarek_f_t[u];\n"
+         "      for (int sarek_f_u = 0; sarek_f_u < 4; ++sarek_f_u)\n        if (sarek_f_j0 + sarek_f_u < sarek_f_nblocks) sarek_f_partials[sarek_f_j0 + sarek_f_u] = sarek_f_t[sarek_f_u];\n"
          "    }\n  }\n";
   }
   if (with_max) {
     // the tree's comparisons in the tree's order: halves 128 .. 4 pair lane l with lanes l + 32 .. l + 1 component by
     // component, halves 2 and 1 the four components of lane 0
     o += "  const long long sarek_f_nblocks = (sarek_f_n + 255) >> 8;\n  float sarek_f_t[4];\n#pragma unroll\n"
-         "  for (int u = 0; u < 4; ++u) {\n    sarek_f_v4 sarek_f_w = sarek_f_r[u];\n#pragma unroll\n"
+         "  for (int sarek_f_u = 0; sarek_f_u < 4; ++sarek_f_u) {\n    sarek_f_v4 sarek_f_w = sarek_f_r[sarek_f_u];\n#pragma unroll\n"
          "    for (int sarek_f_h = 32; sarek_f_h >= 1; sarek_f_h >>= 1)\n#pragma unroll\n      for (int sarek_f_c = 0; sarek_f_c < 4; ++sarek_f_c) "
          "sarek_f_w[sarek_f_c] = sarek_f_greater(sarek_f_w[sarek_f_c], __shfl_down(sarek_f_w[sarek_f_c], sarek_f_h, 64));\n"
-         "    sarek_f_t[u] = sarek_f_greater(sarek_f_greater(sarek_f_w[0], sarek_f_w[2]), sarek_f_greater(sarek_f_w[1], sarek_f_w[3]));\n  }\n"
+         "    sarek_f_t[sarek_f_u] = sarek_f_greater(sarek_f_greater(sarek_f_w[0], sarek_f_w[2]), sarek_f_greater(sarek_f_w[1], sarek_f_w[3]));\n  }\n"
          "  const long long sarek_f_j0 = (long long)blockIdx.x * 16 + (threadIdx.x >> 6) * 4;\n"
          "  if ((threadIdx.x & 63) == 0) {\n    if (sarek_f_j0 + 4 <= sarek_f_nblocks && "
          "(reinterpret_cast<unsigned long long>(sarek_f_partials) & 15ull) == 0) {\n"
          "      *reinterpret_cast<sarek_f_v4*>(sarek_f_partials + sarek_f_j0) = "
          "sarek_f_v4{sarek_f_t[0], sarek_f_t[1], sarek_f_t[2], sarek_f_t[3]};\n    } else {\n#pragma unroll\n"
-         "      for (int u = 0; u < 4; ++u)\n        if (sarek_f_j0 + u < sarek_f_nblocks) sarek_f_partials[sarek_f_j0 + u] = sarek_f_t[u];\n"
+         "      for (int sarek_f_u = 0; sarek_f_u < 4; ++sarek_f_u)\n        if (sarek_f_j0 + sarek_f_u < sarek_f_nblocks) sarek_f_partials[sarek_f_j0 + sarek_f_u] = sarek_f_t[sarek_f_u];\n"
          "    }\n  }\n";
   }
   o += "}\n";
@@ -510,29 +508,29 @@ std::string tree_max_source_scalar_loads(const MapKernel &m) {
   o.resize(o.size() - 2);
   // (comparisons do not contract with anything: the element's value needs no asm in front of them)
   std::string a = "sarek_f_apply(";
-  for (int p : m.inputs) a += "__builtin_nontemporal_load(" + m.params[p].name + " + i), ";
-  a += actuals_tail + "(int)i)";
+  for (int p : m.inputs) a += "__builtin_nontemporal_load(" + m.params[p].name + " + sarek_f_i), ";
+  a += actuals_tail + "(int)sarek_f_i)";
   o += ") {\n  const long long sarek_f_n = " + m.params[m.n].name + ", sarek_f_nblocks = (sarek_f_n + 255) >> 8;\n"
        "  const int sarek_f_lane = threadIdx.x & 63;\n"
        "  const long long sarek_f_j0 = ((long long)blockIdx.x * 4 + (threadIdx.x >> 6)) * 8;\n"
        "  if (sarek_f_j0 >= sarek_f_nblocks) return;\n"
        "  const bool sarek_f_full = (sarek_f_j0 + 8) * 256 <= sarek_f_n;\n  float sarek_f_m[8];\n"
        // all 32 loads of a thread are asked for before the first comparison
-       "  float sarek_f_w[8][4];\n  if (sarek_f_full) {\n#pragma unroll\n    for (int u = 0; u < 8; ++u)\n#pragma unroll\n      for (int q = 0; q < 4; ++q) {\n"
-       "        const long long i = (sarek_f_j0 + u) * 256 + sarek_f_lane + 64 * q;\n"
-       "        sarek_f_w[u][q] = " + a + ";\n      }\n  } else {\n"
-       "#pragma unroll\n    for (int u = 0; u < 8; ++u)\n#pragma unroll\n      for (int q = 0; q < 4; ++q) {\n"
-       "        const long long i = (sarek_f_j0 + u) * 256 + sarek_f_lane + 64 * q;\n"
-       "        sarek_f_w[u][q] = " + m.pad + ";\n        if (i < sarek_f_n) sarek_f_w[u][q] = " + a + ";\n      }\n  }\n"
-       "#pragma unroll\n  for (int u = 0; u < 8; ++u) {\n    const float* v = sarek_f_w[u];\n"
-       "    float sarek_f_g = sarek_f_greater(sarek_f_greater(v[0], v[2]), sarek_f_greater(v[1], v[3]));\n"
+       "  float sarek_f_w[8][4];\n  if (sarek_f_full) {\n#pragma unroll\n    for (int sarek_f_u = 0; sarek_f_u < 8; ++sarek_f_u)\n#pragma unroll\n      for (int sarek_f_q = 0; sarek_f_q < 4; ++sarek_f_q) {\n"
+       "        const long long sarek_f_i = (sarek_f_j0 + sarek_f_u) * 256 + sarek_f_lane + 64 * sarek_f_q;\n"
+       "        sarek_f_w[sarek_f_u][sarek_f_q] = " + a + ";\n      }\n  } else {\n"
+       "#pragma unroll\n    for (int sarek_f_u = 0; sarek_f_u < 8; ++sarek_f_u)\n#pragma unroll\n      for (int sarek_f_q = 0; sarek_f_q < 4; ++sarek_f_q) {\n"
+       "        const long long sarek_f_i = (sarek_f_j0 + sarek_f_u) * 256 + sarek_f_lane + 64 * sarek_f_q;\n"
+       "        sarek_f_w[sarek_f_u][sarek_f_q] = " + m.pad + ";\n        if (sarek_f_i < sarek_f_n) sarek_f_w[sarek_f_u][sarek_f_q] = " + a + ";\n      }\n  }\n"
+       "#pragma unroll\n  for (int sarek_f_u = 0; sarek_f_u < 8; ++sarek_f_u) {\n    const float* sarek_f_v = sarek_f_w[sarek_f_u];\n"
+       "    float sarek_f_g = sarek_f_greater(sarek_f_greater(sarek_f_v[0], sarek_f_v[2]), sarek_f_greater(sarek_f_v[1], sarek_f_v[3]));\n"
        "#pragma unroll\n    for (int sarek_f_h = 32; sarek_f_h >= 1; sarek_f_h >>= 1) sarek_f_g = sarek_f_greater(sarek_f_g, __shfl_down(sarek_f_g, sarek_f_h, 64));\n"
-       "    sarek_f_m[u] = sarek_f_g;\n  }\n  if (sarek_f_lane != 0) return;\n"
+       "    sarek_f_m[sarek_f_u] = sarek_f_g;\n  }\n  if (sarek_f_lane != 0) return;\n"
        "  if (sarek_f_j0 + 8 <= sarek_f_nblocks && (reinterpret_cast<unsigned long long>(" + out + ") & 15ull) == 0) {\n"
-       "    sarek_f_v4* o4 = reinterpret_cast<sarek_f_v4*>(" + out + " + sarek_f_j0);\n"
-       "    o4[0] = sarek_f_v4{sarek_f_m[0], sarek_f_m[1], sarek_f_m[2], sarek_f_m[3]};\n"
-       "    o4[1] = sarek_f_v4{sarek_f_m[4], sarek_f_m[5], sarek_f_m[6], sarek_f_m[7]};\n  } else {\n"
-       "#pragma unroll\n    for (int u = 0; u < 8; ++u)\n      if (sarek_f_j0 + u < sarek_f_nblocks) " + out + "[sarek_f_j0 + u] = sarek_f_m[u];\n  }\n}\n";
+       "    sarek_f_v4* sarek_f_o4 = reinterpret_cast<sarek_f_v4*>(" + out + " + sarek_f_j0);\n"
+       "    sarek_f_o4[0] = sarek_f_v4{sarek_f_m[0], sarek_f_m[1], sarek_f_m[2], sarek_f_m[3]};\n"
+       "    sarek_f_o4[1] = sarek_f_v4{sarek_f_m[4], sarek_f_m[5], sarek_f_m[6], sarek_f_m[7]};\n  } else {\n"
+       "#pragma unroll\n    for (int sarek_f_u = 0; sarek_f_u < 8; ++sarek_f_u)\n      if (sarek_f_j0 + sarek_f_u < sarek_f_nblocks) " + out + "[sarek_f_j0 + sarek_f_u] = sarek_f_m[sarek_f_u];\n  }\n}\n";
   return o;
 }
 
@@ -574,30 +572,30 @@ std::string tree_max_source(const MapKernel &m) {
        "  if ((sarek_f_j0 + 8) * 256 <= sarek_f_n) {\n";
   for (size_t i = 0; i < m.inputs.size(); ++i) {
     const std::string is = std::to_string(i), name = m.params[m.inputs[i]].name;
-    o += "    sarek_f_v4 sarek_f_x" + is + "[8];\n#pragma unroll\n    for (int u = 0; u < 8; ++u) sarek_f_x" + is +
-         "[u] = __builtin_nontemporal_load(reinterpret_cast<const sarek_f_v4*>(" + name +
-         " + (sarek_f_j0 + u) * 256) + sarek_f_lane);\n";
+    o += "    sarek_f_v4 sarek_f_x" + is + "[8];\n#pragma unroll\n    for (int sarek_f_u = 0; sarek_f_u < 8; ++sarek_f_u) sarek_f_x" + is +
+         "[sarek_f_u] = __builtin_nontemporal_load(reinterpret_cast<const sarek_f_v4*>(" + name +
+         " + (sarek_f_j0 + sarek_f_u) * 256) + sarek_f_lane);\n";
   }
-  o += "#pragma unroll\n    for (int u = 0; u < 8; ++u) {\n      sarek_f_v4 sarek_f_w;\n#pragma unroll\n"
-       "      for (int j = 0; j < 4; ++j) sarek_f_w[j] = " +
-       apply("sarek_f_x@[u][j]", "(sarek_f_j0 + u) * 256 + sarek_f_lane * 4 + j") +
-       ";\n      sarek_f_m[u] = sarek_f_tree_max(sarek_f_w);\n    }\n  } else {\n";
+  o += "#pragma unroll\n    for (int sarek_f_u = 0; sarek_f_u < 8; ++sarek_f_u) {\n      sarek_f_v4 sarek_f_w;\n#pragma unroll\n"
+       "      for (int sarek_f_j = 0; sarek_f_j < 4; ++sarek_f_j) sarek_f_w[sarek_f_j] = " +
+       apply("sarek_f_x@[sarek_f_u][sarek_f_j]", "(sarek_f_j0 + sarek_f_u) * 256 + sarek_f_lane * 4 + sarek_f_j") +
+       ";\n      sarek_f_m[sarek_f_u] = sarek_f_tree_max(sarek_f_w);\n    }\n  } else {\n";
   {
     // the group that holds the end of the input: slots past n hold the kernel's fill value
     std::string a = "sarek_f_apply(";
     for (int p : m.inputs) a += m.params[p].name + "[sarek_f_k], ";
     a += actuals_tail + "(int)sarek_f_k)";
-    o += "#pragma unroll\n    for (int u = 0; u < 8; ++u) {\n      sarek_f_v4 sarek_f_w;\n#pragma unroll\n"
-         "      for (int j = 0; j < 4; ++j) {\n        const long long sarek_f_k = (sarek_f_j0 + u) * 256 + sarek_f_lane * 4 + j;\n"
-         "        sarek_f_w[j] = " + m.pad + ";\n        if (sarek_f_k < sarek_f_n) sarek_f_w[j] = " + a + ";\n      }\n"
-         "      sarek_f_m[u] = sarek_f_tree_max(sarek_f_w);\n    }\n  }\n";
+    o += "#pragma unroll\n    for (int sarek_f_u = 0; sarek_f_u < 8; ++sarek_f_u) {\n      sarek_f_v4 sarek_f_w;\n#pragma unroll\n"
+         "      for (int sarek_f_j = 0; sarek_f_j < 4; ++sarek_f_j) {\n        const long long sarek_f_k = (sarek_f_j0 + sarek_f_u) * 256 + sarek_f_lane * 4 + sarek_f_j;\n"
+         "        sarek_f_w[sarek_f_j] = " + m.pad + ";\n        if (sarek_f_k < sarek_f_n) sarek_f_w[sarek_f_j] = " + a + ";\n      }\n"
+         "      sarek_f_m[sarek_f_u] = sarek_f_tree_max(sarek_f_w);\n    }\n  }\n";
   }
   o += "  if (sarek_f_lane != 0) return;\n"
        "  if (sarek_f_j0 + 8 <= sarek_f_nblocks && (reinterpret_cast<unsigned long long>(" + out + ") & 15ull) == 0) {\n"
-       "    sarek_f_v4* o4 = reinterpret_cast<sarek_f_v4*>(" + out + " + sarek_f_j0);\n"
-       "    o4[0] = sarek_f_v4{sarek_f_m[0], sarek_f_m[1], sarek_f_m[2], sarek_f_m[3]};\n"
-       "    o4[1] = sarek_f_v4{sarek_f_m[4], sarek_f_m[5], sarek_f_m[6], sarek_f_m[7]};\n  } else {\n"
-       "#pragma unroll\n    for (int u = 0; u < 8; ++u)\n      if (sarek_f_j0 + u < sarek_f_nblocks) " + out + "[sarek_f_j0 + u] = sarek_f_m[u];\n  }\n}\n";
+       "    sarek_f_v4* sarek_f_o4 = reinterpret_cast<sarek_f_v4*>(" + out + " + sarek_f_j0);\n"
+       "    sarek_f_o4[0] = sarek_f_v4{sarek_f_m[0], sarek_f_m[1], sarek_f_m[2], sarek_f_m[3]};\n"
+       "    sarek_f_o4[1] = sarek_f_v4{sarek_f_m[4], sarek_f_m[5], sarek_f_m[6], sarek_f_m[7]};\n  } else {\n"
+       "#pragma unroll\n    for (int sarek_f_u = 0; sarek_f_u < 8; ++sarek_f_u)\n      if (sarek_f_j0 + sarek_f_u < sarek_f_nblocks) " + out + "[sarek_f_j0 + sarek_f_u] = sarek_f_m[sarek_f_u];\n  }\n}\n";
   return o;
 }
 
@@ -617,29 +615,29 @@ std::string tree_sum_source(const MapKernel &m, bool nt_loads) {
        "  if ((sarek_f_j0 + 8) * 256 <= sarek_f_n) {\n";
   for (size_t i = 0; i < m.inputs.size(); ++i) {
     const std::string is = std::to_string(i), name = m.params[m.inputs[i]].name;
-    const std::string at = "reinterpret_cast<const sarek_f_v4*>(" + name + " + (sarek_f_j0 + u) * 256) + sarek_f_lane";
-    o += "    sarek_f_v4 sarek_f_x" + is + "[8];\n#pragma unroll\n    for (int u = 0; u < 8; ++u) sarek_f_x" + is + "[u] = " +
+    const std::string at = "reinterpret_cast<const sarek_f_v4*>(" + name + " + (sarek_f_j0 + sarek_f_u) * 256) + sarek_f_lane";
+    o += "    sarek_f_v4 sarek_f_x" + is + "[8];\n#pragma unroll\n    for (int sarek_f_u = 0; sarek_f_u < 8; ++sarek_f_u) sarek_f_x" + is + "[sarek_f_u] = " +
          (nt_loads ? "__builtin_nontemporal_load(" + at + ")" : "*(" + at + ")") + ";\n";
   }
-  o += "#pragma unroll\n    for (int u = 0; u < 8; ++u) {\n      float v[4];\n#pragma unroll\n      for (int j = 0; j < 4; ++j) v[j] = " +
-       apply_call(m, actuals_tail, "sarek_f_x@[u][j]", "(sarek_f_j0 + u) * 256 + sarek_f_lane * 4 + j") +
-       ";\n      sarek_f_r[u] = sarek_f_wave_sum((v[0] + v[1]) + (v[2] + v[3]));\n    }\n"
+  o += "#pragma unroll\n    for (int sarek_f_u = 0; sarek_f_u < 8; ++sarek_f_u) {\n      float sarek_f_v[4];\n#pragma unroll\n      for (int sarek_f_j = 0; sarek_f_j < 4; ++sarek_f_j) sarek_f_v[sarek_f_j] = " +
+       apply_call(m, actuals_tail, "sarek_f_x@[sarek_f_u][sarek_f_j]", "(sarek_f_j0 + sarek_f_u) * 256 + sarek_f_lane * 4 + sarek_f_j") +
+       ";\n      sarek_f_r[sarek_f_u] = sarek_f_wave_sum((sarek_f_v[0] + sarek_f_v[1]) + (sarek_f_v[2] + sarek_f_v[3]));\n    }\n"
        "    if (sarek_f_lane == 0) {\n      if ((reinterpret_cast<unsigned long long>(" + out + ") & 15ull) == 0) {\n"
-       "        sarek_f_v4* o4 = reinterpret_cast<sarek_f_v4*>(" + out + " + sarek_f_j0);\n"
-       "        o4[0] = sarek_f_v4{sarek_f_r[0], sarek_f_r[1], sarek_f_r[2], sarek_f_r[3]};\n"
-       "        o4[1] = sarek_f_v4{sarek_f_r[4], sarek_f_r[5], sarek_f_r[6], sarek_f_r[7]};\n      } else {\n"
-       "#pragma unroll\n        for (int u = 0; u < 8; ++u) " + out + "[sarek_f_j0 + u] = sarek_f_r[u];\n      }\n    }\n"
+       "        sarek_f_v4* sarek_f_o4 = reinterpret_cast<sarek_f_v4*>(" + out + " + sarek_f_j0);\n"
+       "        sarek_f_o4[0] = sarek_f_v4{sarek_f_r[0], sarek_f_r[1], sarek_f_r[2], sarek_f_r[3]};\n"
+       "        sarek_f_o4[1] = sarek_f_v4{sarek_f_r[4], sarek_f_r[5], sarek_f_r[6], sarek_f_r[7]};\n      } else {\n"
+       "#pragma unroll\n        for (int sarek_f_u = 0; sarek_f_u < 8; ++sarek_f_u) " + out + "[sarek_f_j0 + sarek_f_u] = sarek_f_r[sarek_f_u];\n      }\n    }\n"
        "    return;\n  }\n";
   // the group that holds the end of the input
   {
     std::string a = "sarek_f_opaque(sarek_f_apply(";
-    for (int p : m.inputs) a += m.params[p].name + "[i + e], ";
-    a += actuals_tail + "(int)(i + e)))";
-    o += "  for (int u = 0; u < 8 && sarek_f_j0 + u < sarek_f_nblocks; ++u) {\n"
-         "    const long long i = (sarek_f_j0 + u) * 256 + sarek_f_lane * 4;\n    float t[4];\n"
-         "    for (int e = 0; e < 4; ++e) t[e] = i + e < sarek_f_n ? " + a + " : 0.f;\n"
-         "    float v = sarek_f_wave_sum((t[0] + t[1]) + (t[2] + t[3]));\n"
-         "    if (sarek_f_lane == 0) " + out + "[sarek_f_j0 + u] = v;\n  }\n}\n";
+    for (int p : m.inputs) a += m.params[p].name + "[sarek_f_i + sarek_f_e], ";
+    a += actuals_tail + "(int)(sarek_f_i + sarek_f_e)))";
+    o += "  for (int sarek_f_u = 0; sarek_f_u < 8 && sarek_f_j0 + sarek_f_u < sarek_f_nblocks; ++sarek_f_u) {\n"
+         "    const long long sarek_f_i = (sarek_f_j0 + sarek_f_u) * 256 + sarek_f_lane * 4;\n    float sarek_f_t[4];\n"
+         "    for (int sarek_f_e = 0; sarek_f_e < 4; ++sarek_f_e) sarek_f_t[sarek_f_e] = sarek_f_i + sarek_f_e < sarek_f_n ? " + a + " : 0.f;\n"
+         "    float sarek_f_v = sarek_f_wave_sum((sarek_f_t[0] + sarek_f_t[1]) + (sarek_f_t[2] + sarek_f_t[3]));\n"
+         "    if (sarek_f_lane == 0) " + out + "[sarek_f_j0 + sarek_f_u] = sarek_f_v;\n  }\n}\n";
   }
   return o;
 }

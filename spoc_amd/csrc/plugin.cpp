@@ -89,11 +89,36 @@ bool covers_1d(const int block[3], const int grid[3], int64_t threads) {
 // in flight per thread, the kernel's own expression on every element; with `red` (the arguments of a block-256 sum
 // launched right after it on the vector it writes) the sums leave in the same pass.  The text is compiled once per
 // kernel and variant.  Returns 1 when the launch (or the pair) was served, 0 to fall back.
+// The compiled kernel of one variant of a rebuilt text, built at the first launch that wants it and kept in the
+// kernel's entry; nullptr when the text does not compile (a name of the kernel's that means something else in HIP, say:
+// no reason to fail the launch, the generated kernel is still there).
+sarek_hip_kernel rebuilt_kernel(MapEntry &e, int reduce, bool nt, uint32_t pad_bits, const char *entry_point) {
+  std::lock_guard<std::mutex> lock(e.mu);
+  const uint64_t generation = kernel_cache_generation();
+  if (e.cache_generation != generation) {   // the compile cache was emptied: the handles kept here are gone
+    e.built.clear();
+    e.cache_generation = generation;
+  }
+  for (const MapEntry::Built &b : e.built)
+    if (b.reduce == reduce && b.nt == nt && b.pad_bits == pad_bits) return static_cast<sarek_hip_kernel>(b.kernel);
+  const std::string text = reduce < 0 ? (e.m.is_max ? ir::tree_max_source(e.m) : ir::tree_sum_source(e.m, nt))
+                                      : ir::map_source(e.m, reduce, nt, pad_bits);
+  sarek_hip_kernel k = nullptr;
+  thread_local std::vector<char> log(16384);
+  if (text.empty() || sarek_hip_kernel_compile_cached(text.c_str(), entry_point, &k, log.data(), log.size()) != SAREK_HIP_OK) {
+    k = nullptr;
+    last_error_slot().clear();   // the launch goes on with the generated text: the compiler's message is not its error
+  }
+  if (e.built.size() < 64) e.built.push_back({reduce, nt, pad_bits, k});
+  return k;
+}
+
 int try_map(const char *source, const int block[3], const int grid[3], const sarek_hip_arg *a, int na,
             const sarek_hip_arg *red, int nred, const int rblock[3], const int rgrid[3], int *rc, bool red_is_max = false,
             uint32_t pad_bits = 0) {
-  ir::MapKernel m;
-  if (!find_generated_map(source, &m)) return 0;
+  const std::shared_ptr<MapEntry> entry = find_generated_map(source);
+  if (!entry) return 0;
+  const ir::MapKernel &m = entry->m;
   struct Slot {
     union {
       void *p;
@@ -147,33 +172,9 @@ int try_map(const char *source, const int block[3], const int grid[3], const sar
   }
   // inputs that together fit the 256 MB last-level cache may still be there: plain loads; larger ones go past it
   const bool nt = static_cast<int64_t>(m.inputs.size()) * n * 4 > (int64_t{256} << 20);
-  static std::mutex mu;
-  static std::unordered_map<std::string, std::string> texts;   // "<variant><generated text>" -> rebuilt text
   const int reduce = !red ? 0 : red_is_max ? 2 : 1;
-  char variant[16];
-  std::snprintf(variant, sizeof(variant), "%d%d%08x", reduce, nt ? 1 : 0, static_cast<unsigned>(red_is_max ? pad_bits : 0));
-  std::string key(variant);
-  key += source;
-  std::string text;
-  {
-    std::lock_guard<std::mutex> lock(mu);
-    auto it = texts.find(key);
-    if (it == texts.end()) {
-      if (texts.size() >= 1024) texts.clear();
-      it = texts.emplace(key, ir::map_source(m, reduce, nt, pad_bits)).first;
-    }
-    text = it->second;
-  }
-  sarek_hip_kernel k = nullptr;
-  thread_local std::vector<char> log(16384);
-  // a rebuilt text that does not compile (a name of the kernel's that means something else in HIP, say) is no reason
-  // to fail the launch: the generated kernel is still there
-  if (text.empty()) return 0;   // did not compile the first time
-  if (sarek_hip_kernel_compile_cached(text.c_str(), "sarek_map", &k, log.data(), log.size()) != SAREK_HIP_OK) {
-    std::lock_guard<std::mutex> lock(mu);
-    texts[key].clear();
-    return 0;
-  }
+  sarek_hip_kernel k = rebuilt_kernel(*entry, reduce, nt, red_is_max ? pad_bits : 0, "sarek_map");
+  if (!k) return 0;
   Slot part;
   part.p = partials;
   params[m.params.size()] = &part;
@@ -185,8 +186,9 @@ int try_map(const char *source, const int block[3], const int grid[3], const sar
 // A block-256 tree sum or maximum with an element-wise expression in front (tags tree_sum_map_f32, tree_max_map_f32),
 // rebuilt in the hand block-256 kernel's shape.  Same conditions as for the plain tree: 256-thread blocks, exactly ceil(n / 256) of them.
 int try_tree_map(const char *source, const int block[3], const int grid[3], const sarek_hip_arg *a, int na, int *rc) {
-  ir::MapKernel m;
-  if (!find_generated_map(source, &m)) return 0;
+  const std::shared_ptr<MapEntry> entry = find_generated_map(source);
+  if (!entry) return 0;
+  const ir::MapKernel &m = entry->m;
   struct Slot {
     union {
       void *p;
@@ -228,27 +230,9 @@ int try_tree_map(const char *source, const int block[3], const int grid[3], cons
   if (grid[0] != nblocks || lengths[m.out] < nblocks) return 0;
   for (int in : m.inputs)
     if (lengths[in] < n || ranges_meet(slots[m.out].p, nblocks * 4, slots[in].p, n * 4)) return 0;
-  const bool nt = true;   // the hand block-256 kernels read past the caches at every size
-  static std::mutex mu;
-  static std::unordered_map<std::string, std::string> texts;
-  std::string text;
-  {
-    std::lock_guard<std::mutex> lock(mu);
-    auto it = texts.find(source);
-    if (it == texts.end()) {
-      if (texts.size() >= 1024) texts.clear();
-      it = texts.emplace(source, m.is_max ? ir::tree_max_source(m) : ir::tree_sum_source(m, nt)).first;
-    }
-    text = it->second;
-  }
-  sarek_hip_kernel k = nullptr;
-  thread_local std::vector<char> log(16384);
-  if (text.empty()) return 0;   // did not compile the first time: the generated kernel serves
-  if (sarek_hip_kernel_compile_cached(text.c_str(), "sarek_tree", &k, log.data(), log.size()) != SAREK_HIP_OK) {
-    std::lock_guard<std::mutex> lock(mu);
-    texts[source].clear();
-    return 0;
-  }
+  // the hand block-256 kernels read past the caches at every size
+  sarek_hip_kernel k = rebuilt_kernel(*entry, -1, true, 0, "sarek_tree");
+  if (!k) return 0;
   const unsigned g[3] = {static_cast<unsigned>(cdiv(nblocks, 32)), 1, 1}, b[3] = {256, 1, 1};
   *rc = sarek_hip_kernel_launch(k, g, b, 0, nullptr, params, static_cast<int>(m.params.size()));
   return 1;

@@ -7,6 +7,7 @@
 
 #include "code_cache.hpp"
 
+#include <atomic>
 #include <cstring>
 #include <map>
 #include <unordered_map>
@@ -157,6 +158,10 @@ int compile_impl(const char *source, const char *kernel_name, sarek_hip_kernel *
 }
 
 }  // namespace
+
+// Bumped whenever the compile cache is emptied: handles of cached kernels kept elsewhere are stale from then on.
+std::atomic<uint64_t> g_kernel_cache_generation{1};
+uint64_t kernel_cache_generation() { return g_kernel_cache_generation.load(std::memory_order_acquire); }
 }  // namespace sarek_hip
 
 using namespace sarek_hip;
@@ -395,6 +400,7 @@ int sarek_hip_kernel_compile_cached(const char *source, const char *kernel_name,
 
 int sarek_hip_kernel_clear_cache(void) {
   std::lock_guard<std::mutex> lock(g_mu);
+  g_kernel_cache_generation.fetch_add(1, std::memory_order_release);
   for (auto &bucket : g_kernel_cache)
     for (CachedKernel &c : bucket.second) {
       (void)hipModuleUnload(c.kernel->module);

@@ -72,7 +72,19 @@ def six_inputs():
     return kernel(params, let(tid, intr("global_thread_id", "Std"), if_(lt(tid, var("n")), assign_elem("out", tid, e))))
 
 
-MAPS = {"six_inputs": six_inputs, "scale": scale, "saxpy_with_let": saxpy_with_let, "norm3": norm3, "ramp_select": ramp_select,
+def short_names():
+    """e = u * i + v * t + float(tid mod j), over q elements: every parameter carries one of the short names a kernel
+    text likes for its own loop variables (the rebuilt texts keep theirs under a prefix, so these are the kernel's)"""
+    params = [("i", "(vec f32)"), ("t", "(vec f32)"), ("e", "(vec f32)"), ("u", "f32"), ("v", "f32"), ("j", "i32"),
+              ("q", "i32")]
+    _params(params)
+    tid = var("tid")
+    ex = add(add(mul(var("u", "f32"), read("i", tid)), mul(var("v", "f32"), read("t", tid))),
+             "(cast f32 " + mod(tid, var("j")) + ")")
+    return kernel(params, let(tid, intr("global_thread_id", "Std"), if_(lt(tid, var("q")), assign_elem("e", tid, ex))))
+
+
+MAPS = {"short_names": short_names, "six_inputs": six_inputs, "scale": scale, "saxpy_with_let": saxpy_with_let, "norm3": norm3, "ramp_select": ramp_select,
         "fill_const": fill_const}
 
 
@@ -97,9 +109,9 @@ def near_misses():
                                       assign_elem("out", t, mul(read("x", t), "(cast f32 " + intr("block_idx_x") + ")"))))))
     out.append(("guard on another bound", k(base, lambda t: if_(lt(t, i32(1000)), assign_elem("out", t, read("x", t))))))
     out.append(("no guard", k(base, lambda t: assign_elem("out", t, read("x", t)))))
-    named_u = [("x", "(vec f32)"), ("out", "(vec f32)"), ("u", "f32"), ("n", "i32")]
-    out.append(("a scalar named like a loop variable of the rebuilt text",
-                k(named_u, lambda t: if_(lt(t, var("n")), assign_elem("out", t, mul(read("x", t), var("u", "f32")))))))
+    own = [("x", "(vec f32)"), ("out", "(vec f32)"), ("sarek_f_n", "f32"), ("n", "i32")]
+    out.append(("a scalar that carries the rebuilt texts' own prefix",
+                k(own, lambda t: if_(lt(t, var("n")), assign_elem("out", t, mul(read("x", t), var("sarek_f_n", "f32")))))))
     ints = [("x", "(vec i32)"), ("out", "(vec i32)"), ("n", "i32")]
     out.append(("int32 vectors", k(ints, lambda t: if_(lt(t, var("n")), assign_elem("out", t, read("x", t))))))
     two = [("x", "(vec f32)"), ("out", "(vec f32)"), ("out2", "(vec f32)"), ("n", "i32")]
@@ -147,7 +159,15 @@ def squared_distance():
                       [("input", 1, "(vec f32)"), ("y", 30, "(vec f32)"), ("output", 2, "(vec f32)"), ("n", 3, "i32")])
 
 
-TREES = {"sum_of_squares": sum_of_squares, "weighted_abs_sum": weighted_abs_sum, "squared_distance": squared_distance}
+def short_named_tree():
+    """sum of u * i * t with the vectors named i and t, the output e, the scalar u, the length q"""
+    text = _tree_with(lambda g: f"(mul (mul (var u 31 f32) (read input {g})) (read t {g}))",
+                      [("input", 1, "(vec f32)"), ("t", 30, "(vec f32)"), ("output", 2, "(vec f32)"), ("u", 31, "f32"),
+                       ("n", 3, "i32")])
+    return text.replace("input", "i").replace("(var n 3 i32)", "(var q 3 i32)").replace("output", "e")
+
+
+TREES = {"short_named_tree": short_named_tree, "sum_of_squares": sum_of_squares, "weighted_abs_sum": weighted_abs_sum, "squared_distance": squared_distance}
 
 
 def tree_near_misses():

@@ -43,6 +43,8 @@ def arguments(sarek, name, n, rng):
         return [E.Vec(vec()) for _ in range(6)] + [E.Vec(out), E.Int32(n)], out
     if name == "fill_const":
         return [E.Vec(out), E.Float32(2.5), E.Int32(n)], out
+    if name == "short_names":
+        return [E.Vec(vec()), E.Vec(vec()), E.Vec(out), E.Float32(0.75), E.Float32(-1.25), E.Int32(9), E.Int32(n)], out
     raise KeyError(name)
 
 
@@ -136,6 +138,9 @@ def test_tree_sum_with_an_expression_in_front(hip, sarek, torch_cuda, name, n):
     alpha = np.float32(0.37)
     if name == "sum_of_squares":
         values, tail = x * x, lambda out: [E.Vec(V.of_array(x)), E.Vec(out), E.Int32(n)]
+    elif name == "short_named_tree":
+        values = (alpha * x) * y
+        tail = lambda out: [E.Vec(V.of_array(x)), E.Vec(V.of_array(y)), E.Vec(out), E.Float32(float(alpha)), E.Int32(n)]  # noqa: E731
     elif name == "weighted_abs_sum":
         values = (alpha * np.abs(x)) * y
         tail = lambda out: [E.Vec(V.of_array(x)), E.Vec(V.of_array(y)), E.Vec(out), E.Float32(float(alpha)), E.Int32(n)]  # noqa: E731
