@@ -363,8 +363,11 @@ std::string gen_expr(const ExprP &ep) {
       return o + "}";
     }
     case Expr::Variant:
-      if (e.args.empty()) return e.name2;
-      return "make_" + e.name + "_" + e.name2 + "(" + join_args(e.args) + ")";
+      // A constructor without payload goes through its make_ function like the others.  (The reference prints the bare
+      // tag there, sarek-cuda/Sarek_ir_cuda.ml:155: an enum constant where a value of the variant's struct type is
+      // wanted, which no C++ compiler takes in `c = cond ? make_t_A(x) : B` or `t c = B`; none of its golden texts
+      // has such a constructor.)
+      return "make_" + mangle(e.name) + "_" + e.name2 + "(" + join_args(e.args) + ")";
     case Expr::ArrayLen: return "sarek_" + e.name + "_length";
     case Expr::ArrayCreate:
       throw CodegenError("HIP codegen: array creation is only valid as the value of a let binding");
@@ -467,11 +470,59 @@ std::string generate(const Kernel &k, const int block[3]) {
   t_kernel = &k;
   std::string o = "\nextern \"C\" {\n";
   try {
-    for (const auto &v : k.variants) o += gen_variant_def(v.first, v.second);
-    for (const auto &t : k.types) {
-      o += "typedef struct {\n";
-      for (const auto &f : t.second) o += "  " + type_str(f.second) + " " + f.first + ";\n";
-      o += "} " + mangle(t.first) + ";\n\n";
+    // Type definitions: the variants, then the records, each in the order the kernel lists them (the reference's
+    // order, sarek-cuda/Sarek_ir_cuda.ml:880-898) -- except that a type whose fields or payloads are of another of
+    // the kernel's types waits until that one is defined (a record inside a record, a record as a variant's payload:
+    // the reference's lists come out of a hash table and carry no such order).
+    struct Def {
+      bool is_variant;
+      size_t index;
+      const std::string *name;
+    };
+    std::vector<Def> defs;
+    for (size_t i = 0; i < k.variants.size(); ++i) defs.push_back({true, i, &k.variants[i].first});
+    for (size_t i = 0; i < k.types.size(); ++i) defs.push_back({false, i, &k.types[i].first});
+    auto defined_here = [&](const std::string &n) {
+      for (const Def &d : defs)
+        if (*d.name == n) return true;
+      return false;
+    };
+    auto needs = [&](const Def &d, const std::vector<bool> &done) {
+      auto waits_for = [&](const TypeP &t) {
+        if (!t || (t->kind != Type::Record && t->kind != Type::Variant) || t->name == *d.name || !defined_here(t->name))
+          return false;
+        for (size_t j = 0; j < defs.size(); ++j)
+          if (*defs[j].name == t->name && !done[j]) return true;
+        return false;
+      };
+      if (d.is_variant) {
+        for (const auto &c : k.variants[d.index].second)
+          for (const TypeP &t : c.second)
+            if (waits_for(t)) return true;
+      } else {
+        for (const auto &f : k.types[d.index].second)
+          if (waits_for(f.second)) return true;
+      }
+      return false;
+    };
+    std::vector<bool> done(defs.size(), false);
+    for (size_t emitted = 0; emitted < defs.size(); ++emitted) {
+      size_t pick = defs.size();
+      for (size_t j = 0; j < defs.size() && pick == defs.size(); ++j)
+        if (!done[j] && !needs(defs[j], done)) pick = j;
+      if (pick == defs.size())   // types that contain each other: no order exists, the compiler will say so
+        for (size_t j = 0; j < defs.size() && pick == defs.size(); ++j)
+          if (!done[j]) pick = j;
+      done[pick] = true;
+      const Def &d = defs[pick];
+      if (d.is_variant) {
+        o += gen_variant_def(k.variants[d.index].first, k.variants[d.index].second);
+      } else {
+        const auto &t = k.types[d.index];
+        o += "typedef struct {\n";
+        for (const auto &f : t.second) o += "  " + type_str(f.second) + " " + f.first + ";\n";
+        o += "} " + mangle(t.first) + ";\n\n";
+      }
     }
     for (const auto &f : k.funcs) o += gen_helper(f);
     o += "__global__ void " + k.name + "(";
