@@ -29,7 +29,10 @@
 extern "C" {
 #endif
 
-#define SAREK_HIP_ABI_VERSION 2
+/* 3: entry points added since 2 (sarek_hip_run_sources, sarek_hip_execute_run_pipeline, sarek_hip_rebuilt_source,
+ * the library kernels, the stencil, layout and histogram kernels, sarek_hip_is_measurement_build); the measurement
+ * knobs and the in-kernel clock probe left the product library; nothing that version 2 declared changed its meaning. */
+#define SAREK_HIP_ABI_VERSION 3
 
 /* Library-level status codes (negative; HIP codes are positive). */
 #define SAREK_HIP_OK 0

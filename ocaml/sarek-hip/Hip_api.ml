@@ -16,7 +16,7 @@ let check (operation : string) (rc : int) : unit =
 
 (* The ABI the library was built to and the struct layout this file declares must agree before
    the first call that fills a struct. *)
-let expected_abi_version = 2
+let expected_abi_version = 3
 
 let verified =
   lazy
