@@ -786,6 +786,195 @@ __global__ __launch_bounds__(512) void gemm16_m16_kernel(const uint16_t *__restr
   }
 }
 
+#ifdef SAREK_HIP_MEASURE
+// The 256 x 256 tile with 4 waves (2 x 2) of 128 x 128 = 8 x 8 MFMA tiles, one wave per SIMD with its 256 accumulator
+// registers in the AGPR half of the register file: the same rings, transfers and LDS layout as gemm16_m16_kernel, two
+// thirds of its LDS fragment bytes (a wave reads 128 rows of A and 128 columns of B per k where two waves of 128 x 64
+// read 256 and 128).  Left to the compiler, the 64 accumulator tiles do not stay in place (the MFMA builtin came out
+// with different source and destination registers and two AGPR <-> VGPR copies per MFMA), so the MFMAs are written
+// as asm with the accumulator tied to itself, and with them the issue order: memory instructions do not move across a
+// volatile asm, so each LDS read and each transfer sits behind the MFMA it is written after.  A slab is 64 MFMAs per
+// wave: row tiles 0-3 before the barrier with the slab's last four A fragments and its 4 B transfers behind every
+// fourth MFMA, row tiles 4-7 after it with the next slab's 20 fragment reads (and, every other slab, the 8 transfers of
+// an A stage) one behind each MFMA.  Aligned shapes, plain store.  Measurement build only (tunable gemm16.waves = 4):
+// with every instruction where it was meant to be it takes 0.766 ms for the bf16 8192^3 product where the 8-wave kernel
+// takes 0.744 in the same run -- a higher clock (1.68 against 1.59 GHz), fewer of its cycles used: with one wave per SIMD
+// nothing fills the pipe while that wave waits at the slab's barrier.
+template <bool Bf16>
+__device__ __forceinline__ void mfma16_in_place(u32x4 a, u32x4 b, f32x4_t &c) {
+  if constexpr (Bf16) asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, %0" : "+a"(c) : "v"(a), "v"(b));
+  else asm volatile("v_mfma_f32_16x16x32_f16 %0, %1, %2, %0" : "+a"(c) : "v"(a), "v"(b));
+}
+
+template <bool Bf16>
+__global__ __launch_bounds__(256) void gemm16_m16w4_kernel(const uint16_t *__restrict__ A, const uint16_t *__restrict__ B,
+                                                           float *__restrict__ C, int M, int N, int K, int tiles_m,
+                                                           int tiles_n, int xcd_remap, int ld) {
+  constexpr int BKA = 64, BKB = 32, NA = 2, NB = 4;
+  constexpr int RA = BKA / BKB;
+  constexpr int A_ROW = BKA * 2, A_CHUNKS = A_ROW / 16, A_ROWS_PER_DMA = 1024 / A_ROW;
+  constexpr int A_BYTES_S = BM * A_ROW, B_BYTES_S = BKB * BN * 2;
+  constexpr int NWAVES = 4, WN = 2;
+  constexpr int DA = A_BYTES_S / 1024 / NWAVES, DB = B_BYTES_S / 1024 / NWAVES;   // 8, 4
+  constexpr int P = lcm_int(NB, RA * NA);
+  static_assert(P % 2 == 0 && DA == 8 && DB == 4, "the issue tables below are written for these counts");
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int wm = wave / WN, wn = wave % WN;
+  const int l16 = lane & 15, g = lane >> 4;
+  int tm, tn;
+  tile_of_block(tiles_m, tiles_n, xcd_remap, tm, tn);
+  const int m0 = tm * BM, n0 = tn * BN;
+  auto a_swz = [](int row) { return (row >> 1) & 7; };
+  auto b_swz = [](int row) { return ((row & 3) << 2) | (((row >> 3) & 1) << 1); };
+
+  uint32_t a_off[DA], b_off[DB];
+#pragma unroll
+  for (int i = 0; i < DA; ++i) {
+    const int q = wave + NWAVES * i;
+    const int arow_t = q * A_ROWS_PER_DMA + lane / A_CHUNKS;
+    const int arow = min(arow_t, M - 1 - m0);
+    a_off[i] = (static_cast<uint32_t>(arow) * K + (((lane % A_CHUNKS) ^ a_swz(arow_t)) << 3)) * 2u;
+  }
+#pragma unroll
+  for (int i = 0; i < DB; ++i) {
+    const int q = wave + NWAVES * i;
+    const int brow = 2 * q + (lane >> 5);
+    const int bchunk = (lane & 31) ^ b_swz(brow);
+    b_off[i] = (static_cast<uint32_t>(brow) * ld + min(n0 + bchunk * 8, N - 8)) * 2u;
+  }
+  const char *a_base = reinterpret_cast<const char *>(A + static_cast<int64_t>(m0) * K);
+  const int64_t b_slab_bytes = static_cast<int64_t>(BKB) * ld * 2;
+  const int nstages = K / BKA, nslabs = K / BKB;
+
+  f32x4_t acc[8][8];
+#pragma unroll
+  for (int i = 0; i < 8; ++i)
+#pragma unroll
+    for (int j = 0; j < 8; ++j)
+#pragma unroll
+      for (int r = 0; r < 4; ++r) acc[i][j][r] = 0.f;
+
+  const int a_row = wm * 128 + l16;
+  int a_addr0 = a_row * A_ROW + ((g ^ a_swz(a_row)) << 4);
+  const int b_r = l16 >> 2;
+  int b_addr0 = (g * 8 + b_r) * 512 + ((wn * 256 + (l16 & 3) * 8) ^ ((b_r << 6) | ((g & 1) << 5)));
+
+  const __amdgpu_buffer_rsrc_t a_rsrc = make_rsrc(a_base, 0x80000000u);
+  // transfer i of A stage `stage` / of the next B slab (the tail of the K loop re-issues the last ones into stages
+  // nobody reads any more, so the count of transfers in flight keeps its pattern)
+  auto dma_a = [&](char *sa, int stage, int i) __attribute__((always_inline)) {
+    dma16(a_rsrc, a_off[i], static_cast<uint32_t>(min(stage, nstages - 1) * BKA) * 2u, sa + (wave + NWAVES * i) * 1024);
+  };
+  const char *b_src = reinterpret_cast<const char *>(B);
+  int b_next = 0;
+  auto dma_b = [&](char *sb, int i) __attribute__((always_inline)) {
+    dma16(make_rsrc(b_src, 0x80000000u), b_off[i], 0u, sb + (wave + NWAVES * i) * 1024);
+  };
+  auto b_advance = [&]() __attribute__((always_inline)) {
+    ++b_next;
+    if (b_next < nslabs) b_src += b_slab_bytes;
+  };
+  auto read_a = [&](const char *sa, int ks, int half, int i, u32x4 &af) __attribute__((always_inline)) {
+    af = *reinterpret_cast<const u32x4 *>(sa + (a_addr0 ^ (ks << 6)) + half * (64 * A_ROW) + i * 16 * A_ROW);
+  };
+  // half h (0: rows 8g+0..3, 1: rows 8g+4..7) of column tile j
+  auto read_b = [&](const char *sb, int j, int h, u32x2 &out) __attribute__((always_inline)) { out = lds_read_tr16(sb, (b_addr0 ^ (j << 5)) + h * 4 * 512); };
+
+  u32x4 af[2][4];    // [half of the wave tile's rows]
+  u32x2 bh[2][8][2]; // [slab parity][column tile][k half]
+  auto bfrag = [&](int par, int j) __attribute__((always_inline)) { return u32x4{bh[par][j][0].x, bh[par][j][0].y, bh[par][j][1].x, bh[par][j][1].y}; };
+
+  auto slab = [&](auto ic, int s) __attribute__((always_inline)) {
+    constexpr int I = decltype(ic)::value;
+    constexpr int In = (I + 1) % P;
+    constexpr int ia = (I / RA) % NA, ibp = (I + NB - 1) % NB;
+    constexpr int ian = (In / RA) % NA, ibn = In % NB;
+    constexpr int ks = I % RA, ksn = In % RA;
+    constexpr bool refill_a = I % RA == RA - 1;
+    asm volatile("" : "+v"(a_addr0), "+v"(b_addr0));
+    // rows 0-63: MFMA t = 8 i + j; behind every fourth one of the slab's last four A fragments or one of the four
+    // transfers of B slab s - 1 + NB
+    [&]<int... Ts>(std::integer_sequence<int, Ts...>) {
+      (([&]() __attribute__((always_inline)) {
+         mfma16_in_place<Bf16>(af[0][Ts / 8], bfrag(I & 1, Ts % 8), acc[Ts / 8][Ts % 8]);
+         if constexpr (Ts % 8 == 0) read_a(lds_ring<10 + ia, A_BYTES_S>, ks, 1, Ts / 8, af[1][Ts / 8]);
+         if constexpr (Ts % 8 == 4) dma_b(lds_ring<20 + ibp, B_BYTES_S>, Ts / 8);
+       }()),
+       ...);
+    }(std::make_integer_sequence<int, 32>{});
+    b_advance();
+    __builtin_amdgcn_s_waitcnt(waitcnt_vm_lgkm0(dma_allowed_in_flight(I, RA, NA, NB, DA, DB)));
+    barrier_no_fence();
+    // rows 64-127, and behind them the next slab's fragments in the order its first MFMAs need them (A tile 0, the
+    // eight B tiles, A tiles 1-3: 20 reads) and, after the last slab of an A stage, the 8 transfers that refill it
+    [&]<int... Ts>(std::integer_sequence<int, Ts...>) {
+      (([&]() __attribute__((always_inline)) {
+         mfma16_in_place<Bf16>(af[1][Ts / 8], bfrag(I & 1, Ts % 8), acc[4 + Ts / 8][Ts % 8]);
+         if constexpr (Ts == 0) read_a(lds_ring<10 + ian, A_BYTES_S>, ksn, 0, 0, af[0][0]);
+         else if constexpr (Ts <= 16) read_b(lds_ring<20 + ibn, B_BYTES_S>, (Ts - 1) / 2, (Ts - 1) % 2, bh[In & 1][(Ts - 1) / 2][(Ts - 1) % 2]);
+         else if constexpr (Ts <= 19) read_a(lds_ring<10 + ian, A_BYTES_S>, ksn, 0, Ts - 16, af[0][Ts - 16]);
+         if constexpr (refill_a && Ts >= 20 && Ts < 28) dma_a(lds_ring<10 + ia, A_BYTES_S>, s / RA + NA, Ts - 20);
+       }()),
+       ...);
+    }(std::make_integer_sequence<int, 32>{});
+  };
+
+  // prologue: fill both rings except the last B stage (the top of slab 0 issues it) and wait for all of it
+  [&]<int... Is>(std::integer_sequence<int, Is...>) {
+    (([&] {
+       _Pragma("unroll") for (int i = 0; i < DA; ++i) dma_a(lds_ring<10 + Is, A_BYTES_S>, Is, i);
+     }()),
+     ...);
+  }(std::make_integer_sequence<int, NA>{});
+  [&]<int... Is>(std::integer_sequence<int, Is...>) {
+    (([&] {
+       _Pragma("unroll") for (int i = 0; i < DB; ++i) dma_b(lds_ring<20 + Is, B_BYTES_S>, i);
+       b_advance();
+     }()),
+     ...);
+  }(std::make_integer_sequence<int, NB - 1>{});
+  __builtin_amdgcn_s_waitcnt(waitcnt_vm_lgkm0(0));
+  barrier_no_fence();
+#pragma unroll
+  for (int i = 0; i < 4; ++i) read_a(lds_ring<10, A_BYTES_S>, 0, 0, i, af[0][i]);
+#pragma unroll
+  for (int j = 0; j < 8; ++j) {
+    read_b(lds_ring<20, B_BYTES_S>, j, 0, bh[0][j][0]);
+    read_b(lds_ring<20, B_BYTES_S>, j, 1, bh[0][j][1]);
+  }
+  __builtin_amdgcn_sched_barrier(0);
+
+  const int full = nslabs - nslabs % P;
+  for (int s = 0; s < full; s += P) {
+    [&]<int... Is>(std::integer_sequence<int, Is...>) {
+      (slab(std::integral_constant<int, Is>{}, s + Is), ...);
+    }(std::make_integer_sequence<int, P>{});
+  }
+  [&]<int... Is>(std::integer_sequence<int, Is...>) {
+    ((full + Is < nslabs ? slab(std::integral_constant<int, Is>{}, full + Is) : (void)0), ...);
+  }(std::make_integer_sequence<int, P - 1>{});
+  __builtin_amdgcn_s_waitcnt(waitcnt_vm_lgkm0(0));   // drain the (redundant) tail DMA before the LDS is released
+  // the compiler does not know that the asm above are matrix instructions whose results land some cycles after issue
+  asm volatile("s_nop 7\n\ts_nop 7\n\ts_nop 7\n\ts_nop 7" ::: "memory");
+  // register r of lane (l16, g) of tile (i, j): row 16 i + 4 g + r, column 16 j + l16 of the wave's 128 x 128
+#pragma unroll
+  for (int i = 0; i < 8; ++i)
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+      const int row = m0 + wm * 128 + i * 16 + 4 * g + r;
+      if (row >= M) continue;
+      float *crow = C + static_cast<int64_t>(row) * ld + n0 + wn * 128 + l16;
+#pragma unroll
+      for (int j = 0; j < 8; ++j)
+        if (n0 + wn * 128 + j * 16 + l16 < N) crow[j * 16] = acc[i][j][r];
+    }
+}
+
+#endif  // SAREK_HIP_MEASURE
+
 // The same pipeline on a 128 x 128 workgroup tile, for products whose 256 x 256 tiles would leave most CUs idle:
 // 4 waves (2 x 2) of 64 x 64 = 4 x 4 tiles of v_mfma_f32_16x16x32, A in 3 stages of K = 64 and B in 4 slabs of K = 32
 // (80 KiB of LDS: two workgroups per CU fill its 160 KiB).  A small tile needs twice the operand bytes per flop and has
@@ -1355,6 +1544,12 @@ int launch_gemm16(const uint16_t *a, const uint16_t *b, float *c, const float *b
     const int tiles_m = (m + BM - 1) / BM, tiles_n = (nm + BN - 1) / BN;
     tile_planes = tiles_n;
     unsigned long long *probe = clock_probe(static_cast<int64_t>(tiles_m) * tiles_n);
+#ifdef SAREK_HIP_MEASURE
+    if (Epi == EPI_STORE && !ragged && tunable("gemm16.waves", 8) == 4) {
+      hipLaunchKernelGGL((gemm16_m16w4_kernel<Bf16>), dim3(tiles_m * tiles_n), dim3(256), 0, st, a, b, c, m, nm, k, tiles_m,
+                         tiles_n, remap, n);
+    } else
+#endif
     if (ragged)
       hipLaunchKernelGGL((gemm16_m16_kernel<Bf16, Epi, 0, true>), dim3(tiles_m * tiles_n), dim3(512), 0, st, a, b, c, bias,
                          rowsum, m, nm, k, tiles_m, tiles_n, remap, probe, n, planes);

@@ -20,11 +20,16 @@ constexpr int NUM_XCD = 8;   // XCDs of an MI355X; workgroup ids are dealt to th
 // Workgroup -> tile.  The hardware deals consecutive workgroup ids round-robin to the
 // 8 XCDs (each with its own L2), so ids are first regrouped to give every XCD one
 // contiguous run of tiles, and the run is walked in bands of GROUP tile-rows, column by
-// column: the ~32 tiles an XCD has in flight then form a compact GROUP x 4 patch that
+// column: the ~32 tiles an XCD has in flight then form a compact GROUP x (32 / GROUP) patch that
 // moves through K together and shares A row-panels and B column-panels in that L2.
+// GROUP = 4 (xcd_remap = 1; a larger xcd_remap sets another height): with 32 x 32 tiles every XCD then owns one
+// band of four tile-rows and all eight walk the same column panels of B at the same time, so what one of them
+// brings past its L2 the others find in the memory-side cache.  Measured on bf16 products against bands of 8:
+// 8192^3 0.729 against 0.740 ms, 8192 x 4096 x 8192 0.365 against 0.374, 16384 x 8192 x 2048 0.442 against 0.474,
+// nothing lost on 3072^3, 4096^3, the fp16 epilogue shape and the f32 8192^3 product; bands of 2, 16 or 32 are slower.
 __device__ __forceinline__ void tile_of_block(int tiles_m, int tiles_n, int xcd_remap, int &tm,
                                               int &tn) {
-  const int GROUP = xcd_remap > 1 ? xcd_remap : 8;   // tile-rows per raster band
+  const int GROUP = xcd_remap > 1 ? xcd_remap : 4;   // tile-rows per raster band
   const int nblocks = tiles_m * tiles_n;
   const int xcd = blockIdx.x % NUM_XCD, slot = blockIdx.x / NUM_XCD;
   int tile = xcd * (nblocks / NUM_XCD) + min(xcd, nblocks % NUM_XCD) + slot;

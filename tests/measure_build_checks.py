@@ -50,6 +50,23 @@ def main():
             assert np.abs(c - ref).max() / np.abs(ref).max() < 1e-4, (m, n, k, ring, tj, mfma)
     print("ring shapes ok", flush=True)
 
+    # the 4-wave kernel (128 x 128 per wave, asm MFMAs on AGPR accumulators): the 8-wave kernel's bits
+    for (m, n, k) in [(256, 256, 64), (512, 768, 448), (300, 520, 192), (1024, 1024, 1216), (70, 1032, 128)]:
+        a, b = normal16((m, k), m + 1), normal16((k, n), n + 1)
+        da, db = dev(a).bfloat16(), dev(b).bfloat16()
+        hip.set_tunable("gemm16.tile", 256)
+        try:
+            ref = hip.gemm_bf16(da, db)
+            ref16 = hip.gemm_f16(da.half(), db.half())
+            hip.set_tunable("gemm16.waves", 4)
+            got = hip.gemm_bf16(da, db)
+            got16 = hip.gemm_f16(da.half(), db.half())
+        finally:
+            hip.set_tunable("gemm16.waves", 8)
+            hip.set_tunable("gemm16.tile", 0)
+        assert torch.equal(got, ref) and torch.equal(got16, ref16), (m, n, k)
+    print("4-wave kernel ok", flush=True)
+
     # the ablated variants: wrong by construction, but within bounds; other kernels refuse the knob
     m, n, k = 512, 768, 512
     torch.manual_seed(7)
