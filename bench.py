@@ -41,14 +41,15 @@ NOMINAL_CLOCK_MHZ = 2400.0
 # HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (KiB per dispatch,
 # FETCH_SIZE scaled by 2.0 and WRITE_SIZE by 1.0 after calibration against a plain 1 GiB copy).
 MEASURED_TRAFFIC_BYTES = {
-    "triad_sum_2p28": (1048610 * 2 + 1052680) * 1024,
-    "gemm_bf16_8192": (801398 * 2 + 262374) * 1024,
-    "gemm_f32_8192": (1698530 * 2 + 262153) * 1024,
-    "gemm_f32_1024": (12333 * 2 + 4098) * 1024,
+    "triad_sum_2p28": (1048600 * 2 + 1052680) * 1024,
+    "map_sum_2p28": (1048590 * 2 + 1052710) * 1024,
+    "gemm_bf16_8192": (791065 * 2 + 262151) * 1024,
+    "gemm_f32_8192": (1572980 * 2 + 262144) * 1024,
+    "gemm_f32_1024": (12345 * 2 + 4096) * 1024,
     "gemm_bf16_2048": (24690 * 2 + 16386) * 1024,
-    "gemm_f16_epilogue": (311774 * 2 + 176787) * 1024,
-    "histogram_2p28": (493838 * 2 + 256) * 1024,
-    "radix_scatter_5e7": (97870 * 2 + 215643) * 1024,
+    "gemm_f16_epilogue": (287023 * 2 + 176781) * 1024,
+    "histogram_2p28": (522415 * 2 + 256) * 1024,
+    "radix_scatter_5e7": (97861 * 2 + 215796) * 1024,
 }
 PEAK_MFMA_TFLOPS = {"bf16": 2500.0, "f16": 2500.0, "f32": 157.3}
 
@@ -63,7 +64,7 @@ def parse():
                              "gemm_f16_epilogue", "gemm_f16_4095x11008x4096", "gemm_f16_shape", "gemm_bf16_shape", "gemm_bf16_2048", "gemm_f32_shape", "vendor_gemm_f32_shape", "copy_1gib",
                              "vendor_gemm_bf16_8192", "vendor_gemm_bf16_shape", "histogram_2p28",
                              "radix_scatter_5e7", "stencil_2d_shape", "conv2d_shape", "map_sum_2p28", "mfma_bf16_stream", "mfma_bf16_stream_32x32x16",
-                             "l2_to_lds_stream"])
+                             "l2_to_lds_stream", "radix_scatter_chain_probe"])
     ap.add_argument("--warmup-ms", type=float, default=60.0,
                     help="warm up for at least this long (and at least --warmup steps): the clocks of a power-limited "
                          "kernel take 30-40 ms to settle after a pause")
@@ -75,6 +76,9 @@ def parse():
                     help="shape of the *_shape workloads (stencil_2d_shape, conv2d_shape: width,height,ignored)")
     ap.add_argument("--l2-stream", default="", metavar="WORKGROUPS,WINDOW_MIB",
                     help="shape of the l2_to_lds_stream workload (default 1024,2)")
+    ap.add_argument("--chain", default="0,1", metavar="PREDECESSORS,ROUNDS",
+                    help="radix_scatter_chain_probe: status words of how many earlier tiles every tile reads, in how many "
+                         "dependent rounds (0,1: no status traffic at all)")
     ap.add_argument("--zero-operands", action="store_true",
                     help="16-bit GEMM workloads: all-zero A and B (what the kernel does when the data costs no power)")
     ap.add_argument("--tunable", action="append", default=[], metavar="NAME=VALUE",
@@ -134,6 +138,7 @@ def dims(*d):
 
 
 ZERO_OPERANDS = False
+CHAIN = (0, 1)
 GEMM_SHAPE = (4096, 11264, 4096)
 L2_STREAM_SHAPE = None
 
@@ -404,6 +409,28 @@ def make_workload(name, torch, hip):
                     config={"workload": "out[counters[key & 255]++] = key, random keys below 100000", "n": n,
                             "algorithmic_bytes": 8 * n})
         return main, None, info, (vk, vo, vcnt, starts, a, ir)
+    if name == "radix_scatter_chain_probe":
+        # What a chained scan over the tiles (each tile publishes its 256 digit counts, later tiles add up what their
+        # predecessors published) could cost at best in the scatter pass: the hand kernel's phases on 16384-key tiles with
+        # the 256 returning atomics of a tile replaced by the scan's traffic alone -- 256 status words stored twice with
+        # device scope, the words of CHAIN[0] earlier tiles loaded with device scope in CHAIN[1] dependent rounds -- and
+        # no waiting for anybody (positions are wrong: timing only).  CHAIN = (0, 1): neither atomics nor status traffic.
+        n = 3051 * 16384
+        look, rounds = CHAIN
+        g.manual_seed(0xC5)
+        keys = torch.randint(0, 100000, (n,), device="cuda", generator=g, dtype=torch.int32)
+        out = torch.empty_like(keys)
+        counters = torch.zeros(256, device="cuda", dtype=torch.int32)
+        status = torch.zeros(3051 * 256, device="cuda", dtype=torch.int32)
+        src = SCATTER_CHAIN_SRC.replace("LOOK_N", str(look)).replace("ROUNDS_N", str(max(rounds, 1)))
+        items = [out, keys, counters, status, ("i32", 0), ("i32", 255)]
+        info = dict(metric="radix scatter pass with a chained scan's traffic in place of its atomics, GB/s (timing only)",
+                    unit="GB/s", dtype="i32", work=8.0 * n, work_unit=1e9, bound="hbm", peak=PEAK_HBM_GBS,
+                    kernel="scatter_chain_probe (JIT)", route="Execute.run_source ~lang:HIP_Source, text in bench.py",
+                    config={"workload": f"16384-key tiles, every tile reads the status of {look} predecessors in {rounds} "
+                                        "dependent rounds", "n": n, "algorithmic_bytes": 8 * n})
+        return (lambda: hip.run_source(src, "scatter_chain_probe", (1024, 1, 1), (3051, 1, 1), items, shared_mem=65536)), \
+            None, info, (keys, out, counters, status)
     if name in ("gemm_f16_4095x11008x4096", "gemm_f16_shape", "gemm_bf16_shape", "gemm_bf16_2048"):
         # the epilogue config's product without the epilogue (what the fused chain costs on top), any --shape, or
         # 2048^3: a product whose 256 x 256 tiles would occupy a quarter of the CUs (the 128 x 128 tile's case)
@@ -672,6 +699,79 @@ extern "C" __global__ __launch_bounds__(512) void l2_to_lds(const u32x4* __restr
 """
 
 
+SCATTER_CHAIN_SRC = r"""
+typedef int i32x4 __attribute__((ext_vector_type(4)));
+#define LOOK LOOK_N
+#define ROUNDS ROUNDS_N
+// The phases of the library's scatter kernel on a tile of 1024 x 16 keys; where that kernel takes the tile's range of
+// every digit with a returning atomic, this one publishes and reads status words as a chained scan would.
+extern "C" __global__ __launch_bounds__(1024) void scatter_chain_probe(int* __restrict__ out, int n_out, const int* __restrict__ keys,
+                                                                      int n_keys, int* __restrict__ counters, int n_counters,
+                                                                      unsigned* __restrict__ status, int n_status, int shift, int mask) {
+  extern __shared__ int stage[];
+  __shared__ int count[256], start[256], base[256], wave_total[4];
+  __shared__ unsigned look[1024];
+  const int t = threadIdx.x, lane = t & 63;
+  const long tile = (long)blockIdx.x * 16384;
+  if (t < 256) count[t] = 0;
+  __syncthreads();
+  int key[16], rank[16];
+  const i32x4* k4 = (const i32x4*)(keys + tile);
+  _Pragma("unroll") for (int u = 0; u < 4; ++u) {
+    const i32x4 v = __builtin_nontemporal_load(k4 + u * 1024 + t);
+    key[4 * u] = v.x; key[4 * u + 1] = v.y; key[4 * u + 2] = v.z; key[4 * u + 3] = v.w;
+  }
+  _Pragma("unroll") for (int j = 0; j < 16; ++j) rank[j] = atomicAdd(&count[(key[j] >> shift) & mask], 1);
+  __syncthreads();
+  unsigned seen = 0;
+  if (LOOK > 0) {
+    const int d = t & 255, q = t >> 8;
+    if (t < 256) __hip_atomic_store(status + (long)blockIdx.x * 256 + t, 0x40000000u | (unsigned)count[t], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    long first = (long)blockIdx.x - 1;
+    _Pragma("unroll 1") for (int r = 0; r < ROUNDS; ++r) {
+      unsigned part = seen & 1;                       // the next round's addresses wait for this round's words
+      _Pragma("unroll") for (int j = 0; j < (LOOK / ROUNDS + 3) / 4; ++j) {
+        long p = first - part - (j * 4 + q);
+        if (p < 0) p = 0;
+        part += __hip_atomic_load(status + p * 256 + d, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) & 0x3fffffffu;
+      }
+      seen += part;
+      first -= LOOK / ROUNDS;
+    }
+    look[t] = seen;
+    __syncthreads();
+    if (t < 256) {
+      seen = look[t] + look[256 + t] + look[512 + t] + look[768 + t];
+      __hip_atomic_store(status + (long)blockIdx.x * 256 + t, 0x80000000u | (seen & 0x3fffffffu), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+  }
+  if (t < 256) {
+    const int c = count[t];
+    int incl = c;
+    _Pragma("unroll") for (int o = 1; o < 64; o <<= 1) { const int up = __shfl_up(incl, o); if (lane >= o) incl += up; }
+    if (lane == 63) wave_total[t >> 6] = incl;
+    start[t] = incl - c;
+    base[t] = counters[t] + (int)(blockIdx.x % 7) * c + (seen == 0xffffffffu ? 1 : 0);   // somewhere inside the output
+  }
+  __syncthreads();
+  if (t < 256) {
+    int before = 0;
+    for (int w = 0; w < (t >> 6); ++w) before += wave_total[w];
+    start[t] += before;
+    base[t] -= start[t];
+  }
+  __syncthreads();
+  _Pragma("unroll") for (int j = 0; j < 16; ++j) stage[start[(key[j] >> shift) & mask] + rank[j]] = key[j];
+  __syncthreads();
+  for (int s = t; s < 16384; s += 1024) {
+    const int k = stage[s];
+    const long pos = (long)base[(k >> shift) & mask] + s;
+    if (pos >= 0 && pos < n_out) out[pos] = k;
+  }
+}
+"""
+
+
 HBM_PROBE_SRC = r"""
 typedef float f4 __attribute__((ext_vector_type(4)));
 #define LOADS(dst, src) _Pragma("unroll") for (int u = 0; u < 4; ++u) dst[u] = __builtin_nontemporal_load(src + base + u * 256)
@@ -851,7 +951,10 @@ def main():
         print("bench.py needs a GPU", file=sys.stderr)
         sys.exit(2)
     torch.cuda.set_device(0)
-    global ZERO_OPERANDS, GEMM_SHAPE, WARMUP_MS, TRACE_LAUNCHES, L2_STREAM_SHAPE
+    global ZERO_OPERANDS, GEMM_SHAPE, WARMUP_MS, TRACE_LAUNCHES, L2_STREAM_SHAPE, CHAIN
+    CHAIN = tuple(int(x) for x in args.chain.split(","))
+    if len(CHAIN) != 2 or CHAIN[0] < 0 or CHAIN[0] > 1024 or CHAIN[1] < 1 or CHAIN[1] > 16:
+        sys.exit("--chain PREDECESSORS,ROUNDS with 0..1024 predecessors in 1..16 rounds")
     if args.l2_stream:
         L2_STREAM_SHAPE = tuple(int(x) for x in args.l2_stream.split(","))
         if len(L2_STREAM_SHAPE) != 2 or L2_STREAM_SHAPE[1] not in (1, 2, 4, 8, 16) or L2_STREAM_SHAPE[0] < 1:
@@ -877,7 +980,7 @@ def main():
     if args.trace_launches:
         out["kernel_us_by_launch"] = head["kernel_us_by_launch"]
     if not args.no_cpu_baseline and args.workload not in ("copy_1gib", "vendor_gemm_bf16_8192", "vendor_gemm_bf16_shape", "gemm_bf16_shape", "gemm_f16_shape", "gemm_f32_shape", "vendor_gemm_f32_shape", "mfma_bf16_stream", "mfma_bf16_stream_32x32x16", "l2_to_lds_stream",
-                                                        "stencil_2d_shape", "conv2d_shape", "map_sum_2p28"):
+                                                        "stencil_2d_shape", "conv2d_shape", "map_sum_2p28", "radix_scatter_chain_probe"):
         out["cpu_baseline"] = cpu_baseline(args.workload)
     if not args.no_also:
         also = []

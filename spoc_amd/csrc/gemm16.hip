@@ -1257,12 +1257,22 @@ __global__ void zero_f32_kernel(float *p, int n) {
 
 // rowsum[r] = the per-tile-column sums planes[t * m + r], t = 0 .. count-1, added in that order in double and rounded
 // once: the order is the tiles', not the order they finished in, so a product gives the same row sums on every run.
-__global__ __launch_bounds__(256) void rowsum_fold_kernel(const float *__restrict__ planes, int count, int m,
-                                                          float *__restrict__ rowsum) {
-  const int r = blockIdx.x * 256 + threadIdx.x;
+__global__ __launch_bounds__(64) void rowsum_fold_kernel(const float *__restrict__ planes, int count, int m,
+                                                         float *__restrict__ rowsum) {
+  const int r = blockIdx.x * 64 + threadIdx.x;
   if (r >= m) return;
   double acc = 0.0;
-  for (int t = 0; t < count; ++t) acc += static_cast<double>(planes[static_cast<int64_t>(t) * m + r]);
+  // sixteen planes' values are asked for before the first is added (the loads are what takes the time: a row has one
+  // thread), the additions keep the planes' order
+  int t = 0;
+  for (; t + 16 <= count; t += 16) {
+    float v[16];
+#pragma unroll
+    for (int u = 0; u < 16; ++u) v[u] = planes[static_cast<int64_t>(t + u) * m + r];
+#pragma unroll
+    for (int u = 0; u < 16; ++u) acc += static_cast<double>(v[u]);
+  }
+  for (; t < count; ++t) acc += static_cast<double>(planes[static_cast<int64_t>(t) * m + r]);
   rowsum[r] = static_cast<float>(acc);
 }
 
@@ -1495,7 +1505,7 @@ int launch_gemm16(const uint16_t *a, const uint16_t *b, float *c, const float *b
   }
   auto finish = [&](int rc) {
     if (rc != SAREK_HIP_OK || !planes) return rc;
-    hipLaunchKernelGGL(rowsum_fold_kernel, dim3((m + 255) / 256), dim3(256), 0, st, planes, n_planes, m, rowsum);
+    hipLaunchKernelGGL(rowsum_fold_kernel, dim3((m + 63) / 64), dim3(64), 0, st, planes, n_planes, m, rowsum);
     return check_launch("rowsum fold launch");
   };
 

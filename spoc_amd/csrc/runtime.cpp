@@ -24,6 +24,7 @@ struct sarek_hip_kernel_s {
   std::string name;
   int device = -1;
   bool cached = false;
+  std::atomic<unsigned> dynamic_lds_allowed{48u << 10};   // raised on demand, see sarek_hip_kernel_launch
 };
 
 namespace sarek_hip {
@@ -425,6 +426,13 @@ int sarek_hip_kernel_launch(sarek_hip_kernel k, const unsigned grid[3], const un
   for (int i = 0; i < 3; ++i)
     if (grid[i] == 0 || block[i] == 0)
       return fail(SAREK_HIP_E_INVALID_ARG, "kernel_launch: zero grid or block dimension");
+  // A launch that asks for more dynamic LDS than a kernel gets by default (?shared_mem of Execute.run_vectors above
+  // 48 KiB; a CU has 160 KiB) needs the kernel's limit raised first, once per kernel and size.
+  if (shared_mem_bytes > k->dynamic_lds_allowed.load(std::memory_order_acquire)) {
+    SAREK_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(k->function),
+                                      hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(shared_mem_bytes)));
+    k->dynamic_lds_allowed.store(shared_mem_bytes, std::memory_order_release);
+  }
   SAREK_HIP_TRY(hipModuleLaunchKernel(k->function, grid[0], grid[1], grid[2], block[0], block[1],
                                       block[2], shared_mem_bytes, as_stream(stream), params,
                                       nullptr));

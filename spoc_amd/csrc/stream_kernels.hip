@@ -220,11 +220,12 @@ __global__ __launch_bounds__(kBlock) void triad_scalar_kernel(float *__restrict_
   }
 }
 
-// Double sum of x[0..count) by one 1024-thread block, valid in thread 0.  Each thread takes float4
-// pieces at a stride of 1024 pieces, eight loads in flight, then a tree in LDS; the summation
-// order is fixed by (count, the pointer's alignment, thread layout) only.
+// Double sum of x[0..count) by one 1024-thread block, valid in every thread.  Each thread takes float4
+// pieces at a stride of 1024 pieces, eight loads in flight, then the wave's lanes are added by exchanges
+// and the sixteen waves' sums through LDS; the summation order is fixed by (count, the pointer's
+// alignment, thread layout) only.
 __device__ __forceinline__ double fold_block(const float *__restrict__ x, int64_t count) {
-  __shared__ double sh[1024];
+  __shared__ double sh[16];
   double acc = 0.0;
   const bool vec = (reinterpret_cast<uintptr_t>(x) & 15u) == 0;
   const int64_t n4 = vec ? count >> 2 : 0;
@@ -245,13 +246,15 @@ __device__ __forceinline__ double fold_block(const float *__restrict__ x, int64_
            (static_cast<double>(v.z) + static_cast<double>(v.w));
   }
   for (int64_t j = (n4 << 2) + threadIdx.x; j < count; j += 1024) acc += static_cast<double>(x[j]);
-  sh[threadIdx.x] = acc;
+  // across the lanes of a wave by exchanges (no LDS, no barrier), then the sixteen waves' sums in wave order
+#pragma unroll
+  for (int m = 32; m >= 1; m >>= 1) acc += __shfl_xor(acc, m, 64);
+  if ((threadIdx.x & 63) == 0) sh[threadIdx.x >> 6] = acc;
   __syncthreads();
-  for (int half = 512; half >= 1; half >>= 1) {
-    if (static_cast<int>(threadIdx.x) < half) sh[threadIdx.x] += sh[threadIdx.x + half];
-    __syncthreads();
-  }
-  return sh[0];
+  double total = 0.0;
+#pragma unroll
+  for (int w = 0; w < 16; ++w) total += sh[w];
+  return total;
 }
 
 // *out = sum of partials[0..count) accumulated in double by one block.
@@ -287,16 +290,17 @@ __global__ __launch_bounds__(1024) void fold_onepass_kernel(const float *__restr
   }
   __syncthreads();
   if (!last) return;
-  __shared__ double sh[kFoldGroups];
-  if (threadIdx.x < kFoldGroups)
-    sh[threadIdx.x] = __hip_atomic_load(&slot->stage[threadIdx.x], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-  __syncthreads();
-  for (int half = kFoldGroups / 2; half >= 1; half >>= 1) {
-    if (static_cast<int>(threadIdx.x) < half) sh[threadIdx.x] += sh[threadIdx.x + half];
-    __syncthreads();
+  // the 256 stage values: four waves add theirs by exchanges, thread 0 the four sums in wave order
+  __shared__ double last_sums[kFoldGroups / 64];
+  if (threadIdx.x < kFoldGroups) {
+    double v = __hip_atomic_load(&slot->stage[threadIdx.x], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+#pragma unroll
+    for (int m = 32; m >= 1; m >>= 1) v += __shfl_xor(v, m, 64);
+    if ((threadIdx.x & 63) == 0) last_sums[threadIdx.x >> 6] = v;
   }
+  __syncthreads();
   if (threadIdx.x == 0) {
-    *out = sh[0];
+    *out = (last_sums[0] + last_sums[1]) + (last_sums[2] + last_sums[3]);
     __hip_atomic_store(&slot->ticket, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
   }
 }
