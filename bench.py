@@ -64,7 +64,7 @@ def parse():
                              "gemm_f16_epilogue", "gemm_f16_4095x11008x4096", "gemm_f16_shape", "gemm_bf16_shape", "gemm_bf16_2048", "gemm_f32_shape", "vendor_gemm_f32_shape", "copy_1gib",
                              "vendor_gemm_bf16_8192", "vendor_gemm_bf16_shape", "histogram_2p28",
                              "radix_scatter_5e7", "stencil_2d_shape", "conv2d_shape", "map_sum_2p28", "mfma_bf16_stream", "mfma_bf16_stream_32x32x16",
-                             "l2_to_lds_stream", "radix_scatter_chain_probe"])
+                             "l2_to_lds_stream", "radix_scatter_chain_probe", "triad_shape_probe"])
     ap.add_argument("--warmup-ms", type=float, default=60.0,
                     help="warm up for at least this long (and at least --warmup steps): the clocks of a power-limited "
                          "kernel take 30-40 ms to settle after a pause")
@@ -76,6 +76,9 @@ def parse():
                     help="shape of the *_shape workloads (stencil_2d_shape, conv2d_shape: width,height,ignored)")
     ap.add_argument("--l2-stream", default="", metavar="WORKGROUPS,WINDOW_MIB",
                     help="shape of the l2_to_lds_stream workload (default 1024,2)")
+    ap.add_argument("--triad-shape", default="256,4,0", metavar="THREADS,FLOAT4_PER_THREAD,PHASES",
+                    help="triad_shape_probe: workgroup size, 128-bit pieces per thread and input, and whether a barrier "
+                         "separates the workgroup's loads from its stores (1) or not (0)")
     ap.add_argument("--chain", default="0,1", metavar="PREDECESSORS,ROUNDS",
                     help="radix_scatter_chain_probe: status words of how many earlier tiles every tile reads, in how many "
                          "dependent rounds (0,1: no status traffic at all)")
@@ -139,6 +142,7 @@ def dims(*d):
 
 ZERO_OPERANDS = False
 CHAIN = (0, 1)
+TRIAD_SHAPE = (256, 4, 0)
 GEMM_SHAPE = (4096, 11264, 4096)
 L2_STREAM_SHAPE = None
 
@@ -409,6 +413,23 @@ def make_workload(name, torch, hip):
                     config={"workload": "out[counters[key & 255]++] = key, random keys below 100000", "n": n,
                             "algorithmic_bytes": 8 * n})
         return main, None, info, (vk, vo, vcnt, starts, a, ir)
+    if name == "triad_shape_probe":
+        # The plain triad (a = b + 3 c, the library kernel's arithmetic) in other launch shapes: THREADS x FLOAT4 pieces of
+        # 16 bytes per workgroup and vector, all loads of a workgroup issued before its first store, optionally with a
+        # barrier between the two phases so that a whole workgroup reads, then writes ("direction batching").
+        threads, per_thread, phases = TRIAD_SHAPE
+        n = 1 << 28
+        b = torch.rand(n, device="cuda", generator=g)
+        c = torch.rand(n, device="cuda", generator=g)
+        a = torch.empty(n, device="cuda")
+        src = TRIAD_SHAPE_SRC.replace("THREADS_N", str(threads)).replace("PIECES_N", str(per_thread)).replace("PHASES_N", str(phases))
+        grid = n // 4 // (threads * per_thread)
+        info = dict(metric="stream triad GB/s in a given launch shape", unit="GB/s", dtype="f32", work=12.0 * n, work_unit=1e9,
+                    bound="hbm", peak=PEAK_HBM_GBS, kernel="triad_shape_probe (JIT)",
+                    route="Execute.run_source ~lang:HIP_Source, text in bench.py",
+                    config={"workload": f"a = b + 3c, {threads} threads x {per_thread} float4 per vector and workgroup"
+                                        + (", loads | barrier | stores" if phases else ""), "n": n, "algorithmic_bytes": 12 * n})
+        return (lambda: hip.run_source(src, "triad_shape_probe", (threads, 1, 1), (grid, 1, 1), [a, b, c])), None, info, (a, b, c)
     if name == "radix_scatter_chain_probe":
         # What a chained scan over the tiles (each tile publishes its 256 digit counts, later tiles add up what their
         # predecessors published) could cost at best in the scatter pass: the hand kernel's phases on 16384-key tiles with
@@ -699,6 +720,25 @@ extern "C" __global__ __launch_bounds__(512) void l2_to_lds(const u32x4* __restr
 """
 
 
+TRIAD_SHAPE_SRC = r"""
+typedef float f4 __attribute__((ext_vector_type(4)));
+#define THREADS THREADS_N
+#define PIECES PIECES_N
+__device__ inline float t1(float b, float c) { return (float)((double)b + (double)c * 3.0); }
+extern "C" __global__ __launch_bounds__(THREADS) void triad_shape_probe(f4* __restrict__ a, int na, const f4* __restrict__ b, int nb,
+                                                                       const f4* __restrict__ c, int nc) {
+  const long base = (long)blockIdx.x * THREADS * PIECES + threadIdx.x;
+  f4 bv[PIECES], cv[PIECES], r[PIECES];
+  _Pragma("unroll") for (int u = 0; u < PIECES; ++u) bv[u] = __builtin_nontemporal_load(b + base + u * THREADS);
+  _Pragma("unroll") for (int u = 0; u < PIECES; ++u) cv[u] = __builtin_nontemporal_load(c + base + u * THREADS);
+  _Pragma("unroll") for (int u = 0; u < PIECES; ++u)
+    r[u] = f4{t1(bv[u].x, cv[u].x), t1(bv[u].y, cv[u].y), t1(bv[u].z, cv[u].z), t1(bv[u].w, cv[u].w)};
+  if (PHASES_N) __syncthreads();
+  _Pragma("unroll") for (int u = 0; u < PIECES; ++u) __builtin_nontemporal_store(r[u], a + base + u * THREADS);
+}
+"""
+
+
 SCATTER_CHAIN_SRC = r"""
 typedef int i32x4 __attribute__((ext_vector_type(4)));
 #define LOOK LOOK_N
@@ -951,7 +991,11 @@ def main():
         print("bench.py needs a GPU", file=sys.stderr)
         sys.exit(2)
     torch.cuda.set_device(0)
-    global ZERO_OPERANDS, GEMM_SHAPE, WARMUP_MS, TRACE_LAUNCHES, L2_STREAM_SHAPE, CHAIN
+    global ZERO_OPERANDS, GEMM_SHAPE, WARMUP_MS, TRACE_LAUNCHES, L2_STREAM_SHAPE, CHAIN, TRIAD_SHAPE
+    TRIAD_SHAPE = tuple(int(x) for x in args.triad_shape.split(","))
+    if len(TRIAD_SHAPE) != 3 or TRIAD_SHAPE[0] not in (64, 128, 256, 512, 1024) or TRIAD_SHAPE[1] not in (1, 2, 4, 6, 8) or \
+            TRIAD_SHAPE[0] * TRIAD_SHAPE[1] > 6144:
+        sys.exit("--triad-shape THREADS,FLOAT4_PER_THREAD,PHASES: 64..1024 threads, 1, 2, 4, 6 or 8 pieces, at most 6144 per workgroup")
     CHAIN = tuple(int(x) for x in args.chain.split(","))
     if len(CHAIN) != 2 or CHAIN[0] < 0 or CHAIN[0] > 1024 or CHAIN[1] < 1 or CHAIN[1] > 16:
         sys.exit("--chain PREDECESSORS,ROUNDS with 0..1024 predecessors in 1..16 rounds")
@@ -980,7 +1024,7 @@ def main():
     if args.trace_launches:
         out["kernel_us_by_launch"] = head["kernel_us_by_launch"]
     if not args.no_cpu_baseline and args.workload not in ("copy_1gib", "vendor_gemm_bf16_8192", "vendor_gemm_bf16_shape", "gemm_bf16_shape", "gemm_f16_shape", "gemm_f32_shape", "vendor_gemm_f32_shape", "mfma_bf16_stream", "mfma_bf16_stream_32x32x16", "l2_to_lds_stream",
-                                                        "stencil_2d_shape", "conv2d_shape", "map_sum_2p28", "radix_scatter_chain_probe"):
+                                                        "stencil_2d_shape", "conv2d_shape", "map_sum_2p28", "radix_scatter_chain_probe", "triad_shape_probe"):
         out["cpu_baseline"] = cpu_baseline(args.workload)
     if not args.no_also:
         also = []

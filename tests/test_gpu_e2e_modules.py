@@ -371,3 +371,25 @@ def test_nested_types_inside_kernels(hip, torch_cuda):
     kk = np.arange(n) % 4
     want = np.where(kk == 0, i, np.where(kk == 1, y, np.where(kk == 2, i * y, -1.0))).astype(np.float32)
     assert np.array_equal(dst.to_array(), want)
+
+
+def test_the_two_smallest_kernels(hip, torch_cuda):
+    """test_debug_native.ml:19-32 (there run on the Native device to debug its runtime): a constant fill and the
+    thread id as a float, 1024 elements in blocks of 256 -- both element-wise maps without an input vector."""
+    from spoc_amd.sarek import Execute, Transfer, Vector
+    n = 1024
+    tid = "(var tid 3 i32)"
+
+    def kernel(value):
+        return (f"(kernel sarek_kern (params (param (var output 1 (vec f32))) (param (var n 2 i32))) (locals) (body "
+                f"(let {tid} (intr (Std) global_thread_id) (if (lt {tid} (var n 2 i32)) "
+                f"(assign (lelem output {tid}) {value})))) (native_fn true))")
+
+    for value, want in (("(f32 42.0)", np.full(n, 42.0, np.float32)),
+                        (f"(cast f32 {tid})", np.arange(n, dtype=np.float32))):
+        out = Vector.create(Vector.float32, n)
+        path = Execute.run_vectors(ir=kernel(value), args=[Execute.Vec(out), Execute.Int32(n)],
+                                   block=Execute.dims1d(256), grid=Execute.dims1d(n // 256))
+        Transfer.flush()
+        assert path == "map_f32"
+        assert np.array_equal(out.to_array(), want)
