@@ -43,13 +43,13 @@ NOMINAL_CLOCK_MHZ = 2400.0
 MEASURED_TRAFFIC_BYTES = {
     "triad_sum_2p28": (1048600 * 2 + 1052680) * 1024,
     "map_sum_2p28": (1048590 * 2 + 1052710) * 1024,
-    "gemm_bf16_8192": (791065 * 2 + 262151) * 1024,
-    "gemm_f32_8192": (1572980 * 2 + 262144) * 1024,
+    "gemm_bf16_8192": (788983 * 2 + 262171) * 1024,
+    "gemm_f32_8192": (1572990 * 2 + 262144) * 1024,
     "gemm_f32_1024": (12345 * 2 + 4096) * 1024,
     "gemm_bf16_2048": (24690 * 2 + 16386) * 1024,
-    "gemm_f16_epilogue": (287023 * 2 + 176781) * 1024,
-    "histogram_2p28": (522415 * 2 + 256) * 1024,
-    "radix_scatter_5e7": (97861 * 2 + 215796) * 1024,
+    "gemm_f16_epilogue": (287017 * 2 + 176780) * 1024,
+    "histogram_2p28": (522398 * 2 + 256) * 1024,
+    "radix_scatter_5e7": (97857 * 2 + 215917) * 1024,
 }
 PEAK_MFMA_TFLOPS = {"bf16": 2500.0, "f16": 2500.0, "f32": 157.3}
 
