@@ -369,6 +369,7 @@ int sarek_hip_vector_location(sarek_hip_vector v, int *location, int *device /* 
 void *sarek_hip_vector_host_ptr(sarek_hip_vector v);       /* Vector.host_ptr: raw, no sync  */
 int sarek_hip_vector_device_ptr(sarek_hip_vector v, void **dptr);   /* NULL: no buffer yet */
 int sarek_hip_vector_set_auto_sync(sarek_hip_vector v, int enabled);
+int sarek_hip_vector_auto_sync(sarek_hip_vector v);         /* Vector.auto_sync: 1 / 0; NULL vector: 0 */
 /* Vector.get / Vector.set (Vector.ml:80-109): bounds-checked ("Vector.get: index I out
  * of bounds [0, N)" with SAREK_HIP_E_INVALID_ARG); get first downloads a Stale_CPU
  * vector when auto-sync is on; set marks a Both / GPU vector Stale_GPU and does not
@@ -386,6 +387,34 @@ int sarek_hip_transfer_to_cpu(sarek_hip_vector v, int force);
 int sarek_hip_transfer_sync(sarek_hip_vector v);
 int sarek_hip_transfer_free_buffers(sarek_hip_vector v);
 int sarek_hip_transfer_flush(void);
+/* Gpu_memory (sarek/core/Gpu_memory.ml:20-141): bookkeeping of the device memory that vectors
+ * hold, kept by the native Vector layer as the reference keeps it from Transfer.ensure_buffer
+ * (track_alloc, Transfer.ml:218), free_buffer / free_all_buffers (track_free, :359,375) and the
+ * vector's finaliser (gc_free_count, gc_freed_bytes; here sarek_hip_vector_destroy, which is what a
+ * host language's finaliser calls).  with_retry is the reference's retry of a failed allocation
+ * after a collection (Gpu_memory.ml:123-141): up to three attempts, the reclaim callback between
+ * them (attempt 1 where the reference runs Gc.full_major, 2 where it runs Gc.compact), the first
+ * failure's status and message returned when all three fail, one attempt when auto_gc is off.
+ * The native Vector layer allocates its device buffers through it.  A host with a garbage collector
+ * registers the callback; without one the retries find nothing new and the first error comes back.
+ * With the OCaml veneer the reference's own Gpu_memory module does all of this and these entry
+ * points stay unused.                                                                          */
+typedef struct sarek_hip_gpu_memory_stats_t {
+  int64_t current_bytes, peak_bytes, alloc_count, free_count, gc_free_count, gc_freed_bytes, retry_count;
+} sarek_hip_gpu_memory_stats_t;
+typedef void (*sarek_hip_reclaim_fn)(void *ctx, int attempt);
+typedef int (*sarek_hip_attempt_fn)(void *ctx);          /* a status: 0 = success */
+void sarek_hip_gpu_memory_set_auto_gc(int enabled);
+int sarek_hip_gpu_memory_get_auto_gc(void);
+void sarek_hip_gpu_memory_track_alloc(int64_t bytes);
+void sarek_hip_gpu_memory_track_free(int64_t bytes);
+int64_t sarek_hip_gpu_memory_usage(void);
+int64_t sarek_hip_gpu_memory_peak_usage(void);
+int sarek_hip_gpu_memory_stats(sarek_hip_gpu_memory_stats_t *out);
+void sarek_hip_gpu_memory_reset_stats(void);
+void sarek_hip_gpu_memory_set_reclaim(sarek_hip_reclaim_fn fn, void *ctx);
+void sarek_hip_gpu_memory_trigger_gc(void);                /* Gpu_memory.trigger_gc: the callback, attempt 1 */
+int sarek_hip_gpu_memory_with_retry(sarek_hip_attempt_fn attempt, void *ctx);
 /* Execute.vector_arg (Execute.ml:28-35; Int goes as INT32, as expand_to_run_source_args sends it). */
 enum { SAREK_HIP_VARG_VEC = 0, SAREK_HIP_VARG_INT32 = 1, SAREK_HIP_VARG_INT64 = 2,
        SAREK_HIP_VARG_FLOAT32 = 3, SAREK_HIP_VARG_FLOAT64 = 4 };

@@ -24,6 +24,7 @@
 #include <vector>
 
 #include "common.hpp"
+#include "gpu_memory.hpp"
 #include "host/ir.hpp"
 #include "plugin.hpp"
 
@@ -87,20 +88,31 @@ int ensure_buffer(sarek_hip_vector_s *v, int dev, void **out) {
     *out = it->second;
     return SAREK_HIP_OK;
   }
-  void *p = nullptr;
-  if (v->zero_copy) {
-    // Memory.alloc_zero_copy returning Some (Transfer.ml:85-126): the buffer is the host block
-    // as the device sees it; its transfers are no-ops.
-    int supported = 0;
-    int st = sarek_hip_mem_alloc_zero_copy(v->host, bytes_of(v), &p, &supported);
-    if (st != SAREK_HIP_OK) return st;
-    if (!supported) return fail(SAREK_HIP_E_UNSUPPORTED, "zero-copy vector: the host block is not device-accessible");
-  } else {
-    int st = sarek_hip_mem_alloc(&p, bytes_of(v));
-    if (st != SAREK_HIP_OK) return st;
-  }
-  v->buffers[dev] = p;
-  *out = p;
+  // Gpu_memory.with_retry round the allocation, track_alloc after it (Transfer.ml:184-218)
+  struct Attempt {
+    sarek_hip_vector_s *v;
+    void *p;
+  } attempt{v, nullptr};
+  int st = sarek_hip_gpu_memory_with_retry(
+      [](void *ctx) -> int {
+        auto *a = static_cast<Attempt *>(ctx);
+        if (a->v->zero_copy) {
+          // Memory.alloc_zero_copy returning Some (Transfer.ml:85-126): the buffer is the host block
+          // as the device sees it; its transfers are no-ops.
+          int supported = 0;
+          int st = sarek_hip_mem_alloc_zero_copy(a->v->host, bytes_of(a->v), &a->p, &supported);
+          if (st != SAREK_HIP_OK) return st;
+          if (!supported)
+            return fail(SAREK_HIP_E_UNSUPPORTED, "zero-copy vector: the host block is not device-accessible");
+          return SAREK_HIP_OK;
+        }
+        return sarek_hip_mem_alloc(&a->p, bytes_of(a->v));
+      },
+      &attempt);
+  if (st != SAREK_HIP_OK) return st;
+  v->buffers[dev] = attempt.p;
+  sarek_hip_gpu_memory_track_alloc(static_cast<int64_t>(bytes_of(v)));
+  *out = attempt.p;
   return SAREK_HIP_OK;
 }
 
@@ -341,8 +353,9 @@ int sarek_hip_vector_create(int kind, int64_t length, int64_t custom_elem_size, 
 int sarek_hip_vector_destroy(sarek_hip_vector v) {
   if (!v) return SAREK_HIP_OK;
   int first = SAREK_HIP_OK;
-  for (auto &b : v->buffers) {
+  for (auto &b : v->buffers) {      // what the reference's finaliser does (Gpu_memory.ml:163-178)
     int st = sarek_hip_mem_free(b.second);
+    if (st == SAREK_HIP_OK) sarek_hip::track_gc_free(static_cast<int64_t>(v->length * v->elem_size));
     if (first == SAREK_HIP_OK) first = st;
   }
   delete v;        // the host block goes with its last vector
@@ -500,6 +513,8 @@ int sarek_hip_vector_device_ptr(sarek_hip_vector v, void **dptr) {
   return SAREK_HIP_OK;
 }
 
+int sarek_hip_vector_auto_sync(sarek_hip_vector v) { return v && v->auto_sync ? 1 : 0; }
+
 int sarek_hip_vector_set_auto_sync(sarek_hip_vector v, int enabled) {
   if (!v) return fail(SAREK_HIP_E_INVALID_ARG, "vector_set_auto_sync: NULL vector");
   v->auto_sync = enabled != 0;
@@ -579,6 +594,7 @@ int sarek_hip_transfer_free_buffers(sarek_hip_vector v) {
   int first = SAREK_HIP_OK;
   for (auto &b : v->buffers) {
     int st = sarek_hip_mem_free(b.second);
+    sarek_hip_gpu_memory_track_free(static_cast<int64_t>(v->length * v->elem_size));
     if (first == SAREK_HIP_OK) first = st;
   }
   v->buffers.clear();

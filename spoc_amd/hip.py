@@ -189,6 +189,18 @@ SYMBOLS = {
     "sarek_hip_vector_host_ptr": (_vp, [_vp]),
     "sarek_hip_vector_device_ptr": (_i, [_vp, C.POINTER(_vp)]),
     "sarek_hip_vector_set_auto_sync": (_i, [_vp, _i]),
+    "sarek_hip_vector_auto_sync": (_i, [_vp]),
+    "sarek_hip_gpu_memory_set_auto_gc": (None, [_i]),
+    "sarek_hip_gpu_memory_get_auto_gc": (_i, []),
+    "sarek_hip_gpu_memory_track_alloc": (None, [_i64]),
+    "sarek_hip_gpu_memory_track_free": (None, [_i64]),
+    "sarek_hip_gpu_memory_usage": (_i64, []),
+    "sarek_hip_gpu_memory_peak_usage": (_i64, []),
+    "sarek_hip_gpu_memory_stats": (_i, [_vp]),
+    "sarek_hip_gpu_memory_reset_stats": (None, []),
+    "sarek_hip_gpu_memory_set_reclaim": (None, [_vp, _vp]),
+    "sarek_hip_gpu_memory_trigger_gc": (None, []),
+    "sarek_hip_gpu_memory_with_retry": (_i, [_vp, _vp]),
     "sarek_hip_vector_get": (_i, [_vp, _i64, _vp]),
     "sarek_hip_vector_set": (_i, [_vp, _i64, _vp]),
     "sarek_hip_vector_read": (_i, [_vp, _vp, _i64, _i64]),

@@ -137,6 +137,27 @@ class Vector:
     def __init__(self, handle, kind):
         self._h, self._kind = handle, kind
 
+    # -- kinds (Vector_types.elem_size / kind_name) --
+    @staticmethod
+    def elem_size(kind):
+        return kind.dtype.itemsize
+
+    @staticmethod
+    def kind_name(kind):
+        return kind.name
+
+    @classmethod
+    def create_float32(cls, length): return cls.create(cls.float32, length)
+
+    @classmethod
+    def create_float64(cls, length): return cls.create(cls.float64, length)
+
+    @classmethod
+    def create_int32(cls, length): return cls.create(cls.int32, length)
+
+    @classmethod
+    def create_int64(cls, length): return cls.create(cls.int64, length)
+
     # -- creation (Vector_storage.create / create_custom / of_array) --
     @classmethod
     def create(cls, kind, length, pinned=False, zero_copy=False):
@@ -160,6 +181,22 @@ class Vector:
         v = cls.create(kind, array.size, pinned)
         v.host[:] = array.reshape(-1).astype(kind.dtype, copy=False)      # straight into the host block: stays CPU
         return v
+
+    @classmethod
+    def of_list(cls, kind, values):
+        """Vector.of_list kind l."""
+        return cls.of_array(np.asarray(list(values), dtype=kind.dtype), kind)
+
+    @classmethod
+    def of_bigarray(cls, kind, array):
+        """Vector.of_bigarray: a numpy array stands in for the Bigarray; the vector gets a block of its own."""
+        return cls.of_array(array, kind)
+
+    def to_bigarray(self):
+        """Vector.to_bigarray: the host block itself, no sync (Vector.ml:57-62)."""
+        if self._kind.code == 6:
+            raise ValueError("to_bigarray: vector uses custom storage")
+        return self.host
 
     @classmethod
     def init(cls, kind, length, f):
@@ -316,6 +353,10 @@ class Vector:
     def set_auto_sync(self, enabled):
         hip.check(hip.lib.sarek_hip_vector_set_auto_sync(self._h, int(enabled)))
 
+    @property
+    def auto_sync(self):
+        return bool(hip.lib.sarek_hip_vector_auto_sync(self._h))
+
     # -- element access (Vector.get / Vector.set) --
     def get(self, index):
         out = np.empty(1, dtype=self._kind.dtype)
@@ -335,6 +376,82 @@ class Vector:
     __getitem__ = get
     __setitem__ = set
 
+    def unsafe_get(self, index):
+        """Vector.unsafe_get: the host block as it is -- no bounds check, no sync (Vector.ml:118-122)."""
+        return self.host[index]
+
+    def unsafe_set(self, index, value):
+        """Vector.unsafe_set: no bounds check; the location follows as for set (Vector.ml:124-133)."""
+        self.set(index, value)
+
+    # -- the element-wise conveniences (Vector.ml:318-470): each syncs the host copy first, then works on it --
+    def iter(self, f):
+        for x in self.to_array():
+            f(x)
+
+    def iteri(self, f):
+        for i, x in enumerate(self.to_array()):
+            f(i, x)
+
+    def map(self, f, kind):
+        return Vector.of_array(np.asarray([f(x) for x in self.to_array()], dtype=kind.dtype), kind)
+
+    def mapi(self, f, kind):
+        return Vector.of_array(np.asarray([f(i, x) for i, x in enumerate(self.to_array())], dtype=kind.dtype), kind)
+
+    def map_inplace(self, f):
+        self.fill_from(np.asarray([f(x) for x in self.to_array()], dtype=self._kind.dtype))
+
+    def fold_left(self, f, init):
+        acc = init
+        for x in self.to_array():
+            acc = f(acc, x)
+        return acc
+
+    def fold_right(self, f, init):
+        acc = init
+        for x in self.to_array()[::-1]:
+            acc = f(x, acc)
+        return acc
+
+    def for_all(self, p):
+        return all(p(x) for x in self.to_array())
+
+    def exists(self, p):
+        return any(p(x) for x in self.to_array())
+
+    def find(self, p):
+        return next((x for x in self.to_array() if p(x)), None)
+
+    def find_index(self, p):
+        return next((i for i, x in enumerate(self.to_array()) if p(x)), None)
+
+    def sum(self, zero, add):
+        return self.fold_left(add, zero)
+
+    def min_elt(self, compare):
+        a = self.to_array()
+        if a.size == 0:
+            return None
+        m = a[0]
+        for x in a[1:]:
+            if compare(x, m) < 0:
+                m = x
+        return m
+
+    def max_elt(self, compare):
+        a = self.to_array()
+        if a.size == 0:
+            return None
+        m = a[0]
+        for x in a[1:]:
+            if compare(x, m) > 0:
+                m = x
+        return m
+
+    def to_list(self):
+        return list(self.to_array())
+
     def to_array(self):
         """Vector.to_array: a fresh array; downloads first when the host copy is stale."""
         out = np.empty(self.length, dtype=self._kind.dtype)
@@ -348,6 +465,73 @@ class Vector:
         if st == hip.E_INVALID_ARG:
             raise IndexError(hip.lib.sarek_hip_last_error().decode())
         hip.check(st)
+
+
+class GpuMemory:
+    """sarek/core/Gpu_memory.ml over the library's counters: the native Vector layer tracks every device buffer it
+    allocates and frees, and allocates through with_retry; Python's collector is the reclaim callback."""
+
+    class Stats(C.Structure):
+        _fields_ = [(n, C.c_int64) for n in ("current_bytes", "peak_bytes", "alloc_count", "free_count",
+                                              "gc_free_count", "gc_freed_bytes", "retry_count")]
+
+    _ATTEMPT = C.CFUNCTYPE(C.c_int, C.c_void_p)
+    _RECLAIM = C.CFUNCTYPE(None, C.c_void_p, C.c_int)
+    _reclaim = None
+
+    @staticmethod
+    def set_auto_gc(enabled): hip.lib.sarek_hip_gpu_memory_set_auto_gc(int(enabled))
+
+    @staticmethod
+    def get_auto_gc(): return bool(hip.lib.sarek_hip_gpu_memory_get_auto_gc())
+
+    @staticmethod
+    def track_alloc(nbytes): hip.lib.sarek_hip_gpu_memory_track_alloc(nbytes)
+
+    @staticmethod
+    def track_free(nbytes): hip.lib.sarek_hip_gpu_memory_track_free(nbytes)
+
+    @staticmethod
+    def usage(): return hip.lib.sarek_hip_gpu_memory_usage()
+
+    @staticmethod
+    def peak_usage(): return hip.lib.sarek_hip_gpu_memory_peak_usage()
+
+    @classmethod
+    def stats(cls):
+        s = cls.Stats()
+        hip.check(hip.lib.sarek_hip_gpu_memory_stats(C.byref(s)))
+        return s
+
+    @staticmethod
+    def reset_stats(): hip.lib.sarek_hip_gpu_memory_reset_stats()
+
+    @staticmethod
+    def trigger_gc(): hip.lib.sarek_hip_gpu_memory_trigger_gc()
+
+    @classmethod
+    def use_python_collector(cls):
+        """Registers gc.collect() as what a retry runs between two attempts (Gc.full_major / Gc.compact there)."""
+        import gc
+        cls._reclaim = cls._RECLAIM(lambda ctx, attempt: gc.collect() and None)
+        hip.lib.sarek_hip_gpu_memory_set_reclaim(C.cast(cls._reclaim, C.c_void_p), None)
+
+    @classmethod
+    def with_retry(cls, f):
+        """Gpu_memory.with_retry f: f raises to fail; the first failure is the one re-raised after three."""
+        box = {}
+
+        def attempt(ctx):
+            try:
+                box["value"] = f()
+                return 0
+            except Exception as e:          # noqa: BLE001 -- any failure counts, as `with exn1` there
+                box.setdefault("first", e)
+                return hip.E_INVALID_ARG
+        cb = cls._ATTEMPT(attempt)
+        if hip.lib.sarek_hip_gpu_memory_with_retry(C.cast(cb, C.c_void_p), None) != 0:
+            raise box["first"]
+        return box["value"]
 
 
 class Transfer:

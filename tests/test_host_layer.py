@@ -92,6 +92,38 @@ def test_location_walk(torch_cuda):
 
 
 @gpu
+def test_device_buffers_are_tracked_as_the_reference_tracks_them(torch_cuda):
+    """Transfer.ensure_buffer -> Gpu_memory.track_alloc (Transfer.ml:218); free_all_buffers -> track_free (:375); a
+    vector that goes away with a buffer -> the finaliser's gc_free_count / gc_freed_bytes (Gpu_memory.ml:163-178)."""
+    import gc
+    from spoc_amd.sarek import GpuMemory
+    gc.collect()                                           # vectors of earlier tests go now, not in the middle of this one
+    GpuMemory.reset_stats()
+    v = Vector.create(Vector.float32, 1000)
+    w = Vector.create(Vector.int64, 500)
+    Transfer.to_device(v)
+    Transfer.to_device(v)                                  # the buffer is there: nothing new
+    Transfer.to_device(w)
+    s = GpuMemory.stats()
+    assert (s.current_bytes, s.peak_bytes, s.alloc_count, s.free_count) == (8000, 8000, 2, 0)
+    Transfer.free_all_buffers(v)
+    s = GpuMemory.stats()
+    assert (s.current_bytes, s.peak_bytes, s.alloc_count, s.free_count, s.gc_free_count) == (4000, 8000, 2, 1, 0)
+    w.destroy()                                            # what a finaliser does
+    s = GpuMemory.stats()
+    assert (s.current_bytes, s.free_count, s.gc_free_count, s.gc_freed_bytes) == (0, 1, 1, 4000)
+    v.destroy()                                            # no buffer left: nothing to count
+    assert GpuMemory.stats().gc_free_count == 1 and GpuMemory.usage() == 0
+    # a sub-vector's buffer is its own share
+    parent = Vector.create(Vector.float32, 100)
+    sub = parent.sub_vector(10, 20)
+    Transfer.to_device(sub)
+    assert GpuMemory.usage() == 80
+    Transfer.free_all_buffers(sub)
+    assert GpuMemory.usage() == 0
+
+
+@gpu
 def test_launch_marks_stale_and_reads_download(torch_cuda):
     n = 100003
     b, c = Vector.create(Vector.float32, n), Vector.create(Vector.float32, n)

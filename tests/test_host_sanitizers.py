@@ -51,7 +51,7 @@ def damaged_texts(count, seed):
 def test_host_code_is_clean_under_asan_and_ubsan(tmp_path):
     sources = [os.path.join(HERE, "host_sanitizers", f) for f in ("driver.cpp", "kernel_stubs.cpp")]
     sources += [os.path.join(CSRC, f) for f in (
-        "status.cpp", "backend_info.cpp", "tunables.cpp", "runtime.cpp", "transfer.cpp", "vector.cpp",
+        "status.cpp", "backend_info.cpp", "tunables.cpp", "runtime.cpp", "transfer.cpp", "vector.cpp", "gpu_memory.cpp",
         "code_cache.cpp", "plugin.cpp", "library_kernels.cpp", "generate.cpp", "fusion_abi.cpp", "host/ir_text.cpp", "host/ir_hip.cpp",
         "host/specialise.cpp", "host/fusion.cpp", "host/map_fuse.cpp")]
     exe = str(tmp_path / "host_asan")
