@@ -542,7 +542,8 @@ int sarek_hip_reduce_max_block256_f32(const float *in, float *out, int64_t n, fl
  * 2^17 partials on, 256 workgroups fold a piece each into a stage inside the library's device image
  * and the one that finishes last adds those up in index order.  Every (device, stream) gets a stage of
  * its own (16 per device), so long folds on different streams do not meet; a stream beyond the
- * sixteenth, and a first long fold on a device made under stream capture, fold with one workgroup.  */
+ * sixteenth, and any fold recorded under stream capture (a graph may be replayed on any stream, next
+ * to anything), fold with one workgroup and no shared stage.                                        */
 int sarek_hip_fold_partials_f64(const float *partials, int64_t count, double *sum_out,
                                 sarek_hip_stream stream);
 

@@ -632,8 +632,8 @@ int scratch_on_current_device(hipStream_t st, float **out) {
 
 // The stage slot of (current device, st): a stream keeps the slot it got first, so folds on one stream follow each
 // other through the same slot and folds on different streams never share one.  nullptr when all slots of the device
-// are taken by other streams, or when the device's array cannot be looked up now (first use under capture): the
-// caller then folds with one workgroup, which needs no stage.
+// are taken by other streams (a slot stays with its stream's handle for the life of the process): the caller then
+// folds with one workgroup, which needs no stage.
 FoldSlot *fold_slot_for(hipStream_t st) {
   FoldSlot *slots = nullptr;
   if (address_on_current_device(g_fold_slots_addr, HIP_SYMBOL(fold_slots), "fold_partials", st, &slots) != SAREK_HIP_OK) {
@@ -658,7 +658,8 @@ FoldSlot *fold_slot_for(hipStream_t st) {
 constexpr int64_t kFoldOnePassFrom = int64_t{1} << 17;
 
 int launch_fold(const float *partials, int64_t count, double *sum_out, hipStream_t st) {
-  FoldSlot *slot = count < kFoldOnePassFrom ? nullptr : fold_slot_for(st);
+  // a launch recorded into a graph may be replayed on any stream, next to anything: it gets no shared stage
+  FoldSlot *slot = count < kFoldOnePassFrom || capturing(st) ? nullptr : fold_slot_for(st);
   if (!slot) {
     hipLaunchKernelGGL(fold_kernel, dim3(1), dim3(1024), 0, st, partials, count, sum_out);
     return check_launch("fold kernel launch");

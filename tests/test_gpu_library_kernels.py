@@ -450,6 +450,33 @@ def test_long_folds_on_many_streams_do_not_meet(hip, torch_cuda):
         assert got[0, i] == got[1, i] == got[2, i], i
 
 
+def test_a_long_fold_recorded_into_a_graph_keeps_no_shared_state(hip, torch_cuda):
+    """A fold of 2^20 partials recorded under stream capture takes the one-workgroup kernel (a graph may be replayed
+    on any stream, next to anything, so it gets no stage of the library's): four replays with eager long folds on the
+    same stream and new data between them, each checked against numpy's double sum of what the vector held then."""
+    torch = torch_cuda
+    n = 1 << 20
+    rng = np.random.default_rng(11)
+    x = torch.from_numpy(rng.uniform(0, 4, n).astype(np.float32)).cuda()
+    out = torch.zeros(1, dtype=torch.float64, device="cuda")
+    eager = torch.zeros(1, dtype=torch.float64, device="cuda")
+    stream = torch.cuda.Stream()
+    hip.check(hip.lib.sarek_hip_fold_partials_f64(x.data_ptr(), n, eager.data_ptr(), stream.cuda_stream))
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph, stream=stream):
+        hip.check(hip.lib.sarek_hip_fold_partials_f64(x.data_ptr(), n, out.data_ptr(), torch.cuda.current_stream().cuda_stream))
+    for replay in range(4):
+        x.mul_(0.5 + 0.25 * replay)
+        torch.cuda.synchronize()
+        want = float(x.cpu().numpy().astype(np.float64).sum())
+        hip.check(hip.lib.sarek_hip_fold_partials_f64(x.data_ptr(), n, eager.data_ptr(), stream.cuda_stream))
+        graph.replay()
+        torch.cuda.synchronize()
+        assert abs(out.item() - want) <= 1e-12 * want, replay
+        assert abs(eager.item() - want) <= 1e-12 * want, replay
+
+
 def test_tiled_matmul_through_run_vectors_at_1024(hip, oracle, sarek):
     """bench_matrix_mul_tiled's kernel from IR through Execute.run_vectors at the size of the first config."""
     E, V = sarek.Execute, sarek.Vector
