@@ -269,3 +269,61 @@ def test_serialiser_prints_only_forms_the_native_reader_knows():
                     "SBarrier", "SWarpBarrier", "SExpr", "SEmpty", "SLet", "SLetMut", "SPragma", "SMemFence", "SBlock",
                     "SNative", "DParam", "DLocal", "DShared", "PConstr", "PWild"]
     assert [c for c in constructors if not re.search(r"\b" + c + r"\b", ml)] == []
+
+
+def test_the_forms_the_ocaml_unit_test_expects_are_forms_the_native_reader_takes():
+    """ocaml/sarek-hip/test/test_sarek_ir_hip.ml pins the text Sarek_ir_hip prints per IR constructor.  No compiler
+    here can run it, so the other half of the contract is checked from this side: every expected string of that file
+    goes through the library's reader and lowering inside a kernel."""
+    from spoc_amd import hip
+    ml = open(os.path.join(OCAML, "test", "test_sarek_ir_hip.ml")).read()
+
+    def unescape(s):
+        s = re.sub(r"\\\n\s*", "", s)                     # OCaml's line continuation inside a string
+        return s.replace('\\"', '"').replace("\\\\", "\\")
+
+    def table(name):
+        body = re.search(r"let " + name + r" =\n(.*?)\n\n", ml, flags=re.S).group(1)
+        return [unescape(s) for s in re.findall(r'"(\((?:[^"\\]|\\.)*)"\)', body)]
+
+    def kernel(params="", body="(empty)"):
+        return f"(kernel k (params{params}) (locals) (body {body}) (native_fn true))"
+
+    types, consts = table("types"), table("constants_and_variables")
+    exprs, stmts = table("expressions"), table("statements")
+    assert (len(types), len(consts), len(exprs), len(stmts)) == (6, 7, 15, 18)
+    for t in types:
+        hip.generate_source(kernel(params=f" (param (var p 9 {t}))"))
+    for e in consts + exprs:
+        if e.startswith("(newarray"):                     # an array is created as the value of a let only
+            hip.generate_source(kernel(body=f"(let (var tile 9 (array f32 shared)) {e} (empty))"))
+        else:
+            hip.generate_source(kernel(body=f"(expr {e})"))
+    for s in stmts:
+        hip.generate_source(kernel(body=s))
+    whole = unescape(re.search(r'"(\(kernel sarek_kern (?:[^"\\]|\\.)*)"', ml, flags=re.S).group(1))
+    src = hip.generate_source(whole)
+    assert "void sarek_kern(float* __restrict__ a, int sarek_a_length, int n)" in src and "} point;" in src
+    bare = re.search(r'"(\(intr \(Gpu\) [a-z_]+\))"', ml).group(1)
+    # a name neither side knows goes out as a call of that name, for the device compiler to judge
+    assert "no_such_intrinsic_for_this_test()" in hip.generate_source(kernel(body=f"(expr {bare})"))
+
+
+def test_the_ocaml_test_directory_builds_against_the_plugin_library():
+    dune = open(os.path.join(OCAML, "test", "dune")).read()
+    tests = re.findall(r"\(name (\w+)\)", dune)
+    assert sorted(tests) == ["test_hip_error", "test_sarek_ir_hip"]
+    for t in tests:
+        assert os.path.exists(os.path.join(OCAML, "test", t + ".ml")) and f"(modules {t})" in dune
+    assert dune.count("sarek_hip") >= 2                   # the plugin library's dune name (ocaml/sarek-hip/dune)
+    # every Hip_error constructor the error test builds is one the shared functor provides and the veneer raises
+    # or could raise (spoc/framework/Backend_error.ml:291-347)
+    err = open(os.path.join(OCAML, "test", "test_hip_error.ml")).read()
+    functor = {"unknown_intrinsic", "invalid_arg_count", "unsupported_construct", "type_error", "invalid_memory_space",
+               "unsupported_type", "no_device_selected", "device_not_found", "compilation_failed", "module_load_failed",
+               "kernel_launch_failed", "memory_allocation_failed", "memory_copy_failed", "context_error",
+               "synchronization_failed", "unsupported_source_lang", "backend_unavailable", "library_not_found",
+               "initialization_failed", "feature_not_supported", "to_string", "raise_error", "with_default", "to_result",
+               "Hip_error"}
+    used = set(re.findall(r"Hip_error\.(\w+)", err))
+    assert used and used <= functor, used - functor
