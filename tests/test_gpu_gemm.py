@@ -230,6 +230,27 @@ def test_epilogue_row_sums_are_the_same_bits_on_every_run(hip, oracle, torch_cud
         assert np.abs(y.cpu().numpy() - y_ref).max() <= 1e-4 * np.abs(y_ref).max()
 
 
+def test_epilogue_row_sums_beyond_the_plane_block_are_added_by_atomics(hip, torch_cuda):
+    """More row-sum shares than the per-stream block holds (rows x planes x 4 bytes > 64 MiB; here the
+    one-thread-per-element kernel's plane per 64 columns on an 8192 x 131136 product with K = 20): the shares go to the
+    zeroed vector by atomicAdd, in no fixed order -- every row within 1e-4 of the double sum of the stored row."""
+    torch = torch_cuda
+    m, n, k = 8192, 131136, 20
+    assert m * ((n + 63) // 64) * 4 > 64 << 20
+    g = torch.Generator(device="cuda")
+    g.manual_seed(0xE9)
+    a = (torch.randn(m, k, device="cuda", generator=g) * 0.2).half()
+    b = (torch.randn(k, n, device="cuda", generator=g) * 0.2).half()
+    bias = torch.rand(n, device="cuda", generator=g) * 0.2 - 0.1
+    y, rs = hip.gemm_f16_bias_relu_rowsum(a, b, bias)
+    sums = torch.sum(y, dim=1, dtype=torch.float64)
+    assert bool((sums > 0).all()) and bool(((rs.double() - sums).abs() <= 1e-4 * sums).all())
+    # sampled elements against the definition
+    rows = torch.tensor([0, 4097, 8191], device="cuda")
+    want = torch.relu(a[rows].double() @ b.double() + bias.double())
+    assert bool(((y[rows].double() - want).abs() <= 1e-5 * want.abs().max()).all())
+
+
 def test_gemm_bf16_full_size_rows(hip, oracle, torch_cuda):
     torch = torch_cuda
     m = n = k = 8192
