@@ -55,6 +55,12 @@ extern "C" int sarek_hip_generate_source(const char *ir_text, const int block[3]
     if (tag.empty() && (map = ir::match_tree_sum(k))) tag = "tree_sum_map_f32";
     if (tag.empty() && (map = ir::match_tree_max(k))) tag = "tree_max_map_f32";
     if (!tag.empty()) src = std::string(kSpecialiseMarker) + tag + "\n";
+    // A kernel of one of the three rebuilt classes has two texts, this one and the one rebuilt from its expression
+    // (host/map_fuse.cpp), and either may serve a launch.  Both evaluate the expression as it is written, every
+    // operation rounded once: where the compiler may contract a product into a sum, which products it contracts
+    // depends on the code round the expression (an arm of an `if` turned into a branch or a select, a
+    // scalar-only product shared by the sixteen elements of a thread), and the two texts would differ in last bits.
+    if (map) src += "#pragma clang fp contract(off)\n";
     src += ir::generate(k, block);
   } catch (const ir::ParseError &e) {
     return fail(SAREK_HIP_E_PARSE, "%s", e.what());

@@ -343,9 +343,15 @@ std::string gen_expr(const ExprP &ep) {
     case Expr::ConstUnit: return "(void)0";
     case Expr::VarRef: return e.var.name;
     case Expr::BinopE: return "(" + gen_expr(e.args[0]) + binop_str(e.binop) + gen_expr(e.args[1]) + ")";
-    case Expr::UnopE:
-      return std::string("(") + (e.unop == Unop::Neg ? "-" : e.unop == Unop::Not ? "!" : "~") +
-             gen_expr(e.args[0]) + ")";
+    case Expr::UnopE: {
+      // As the reference prints it, "(" op operand ")" -- except that the minus of a negation keeps a space from an
+      // operand that itself begins with a minus (a negative literal): "(--3.5f)" is a decrement of a literal and does
+      // not compile, there or here.
+      const std::string operand = gen_expr(e.args[0]);
+      const char *sign = e.unop == Unop::Neg ? (!operand.empty() && operand[0] == '-' ? "- " : "-")
+                         : e.unop == Unop::Not ? "!" : "~";
+      return std::string("(") + sign + operand + ")";
+    }
     case Expr::ArrayRead: return e.name + "[" + gen_expr(e.args[0]) + "]";
     case Expr::ArrayReadExpr: return "(" + gen_expr(e.args[0]) + ")[" + gen_expr(e.args[1]) + "]";
     case Expr::RecordField: return gen_expr(e.args[0]) + "." + e.name;

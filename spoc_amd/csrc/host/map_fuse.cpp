@@ -224,6 +224,9 @@ namespace {
 // sarek_f_opaque.  `actuals_tail` receives the scalar arguments of a call ("alpha, k, ").
 std::string prelude(const MapKernel &m, bool with_sums, std::string *actuals_tail) {
   std::string o;
+  // no contraction of products into sums, here as in the generated text of the same kernel: the two texts then
+  // round the expression's operations alike whatever code surrounds them
+  o += "#pragma clang fp contract(off)\n";
   o += "typedef float sarek_f_v4 __attribute__((ext_vector_type(4)));\n";
   if (with_sums) {
     // the stream kernels' wave reduction: quad_perm, row_half_mirror, row_mirror, then the four rows
@@ -301,10 +304,11 @@ std::string map_source(const MapKernel &m, int reduce, bool nt_loads, uint32_t p
        (m.inputs.size() <= 2 ? "__attribute__((amdgpu_waves_per_eu(8, 8))) " : "") + "void sarek_map(";
   o += formal_params(m) + "float* __restrict__ sarek_f_partials) {\n";
   o += "  const long long sarek_f_n = " + m.params[m.n].name + ", sarek_f_n4 = sarek_f_n >> 2;\n";
-  // a wave owns four consecutive KiB of every vector: slot u of lane l is float4 number base + 64 u
+  // a wave owns four consecutive KiB of every vector: slot u of lane l is float4 number base + 64 u; the tail's share
+  // of a block sum starts at -0, whose addition changes nothing (a block of elements that are all -0 sums to -0)
   o += "  const long long sarek_f_base = (long long)blockIdx.x * 1024 + (threadIdx.x >> 6) * 256 + (threadIdx.x & 63);\n"
        "  const bool sarek_f_full = sarek_f_base + 192 < sarek_f_n4;\n"
-       "  sarek_f_v4 sarek_f_r[4];\n  float sarek_f_extra[4] = {0.f, 0.f, 0.f, 0.f};\n";
+       "  sarek_f_v4 sarek_f_r[4];\n  float sarek_f_extra[4] = {-0.f, -0.f, -0.f, -0.f};\n";
   for (size_t i = 0; i < m.inputs.size(); ++i)
     o += "  const sarek_f_v4* sarek_f_p" + std::to_string(i) + " = reinterpret_cast<const sarek_f_v4*>(" +
          m.params[m.inputs[i]].name + ");\n";

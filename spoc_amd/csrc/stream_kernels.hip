@@ -113,7 +113,9 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(8, 8))) 
                        (Runs ? (threadIdx.x >> 6) * (64 * kUnroll) + (threadIdx.x & 63) : threadIdx.x);
   const bool full = base + (kUnroll - 1) * kStep < n4;
   float4 r[kUnroll];
-  float extra[kUnroll];   // SUM_BLOCK256: the scalar tail's share of the block that holds it
+  // SUM_BLOCK256: the scalar tail's share of the block that holds it.  It starts at -0, the one value whose addition
+  // changes nothing: a block of 256 elements that are all -0 sums to -0, as in block256_kernel.
+  float extra[kUnroll];
   if (full) {
     float4 bv[kUnroll], cv[kUnroll];
 #pragma unroll
@@ -123,14 +125,14 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(8, 8))) 
 #pragma unroll
     for (int u = 0; u < kUnroll; ++u) {
       r[u] = triad4(bv[u], cv[u], sd);
-      extra[u] = 0.f;
+      extra[u] = -0.f;
     }
   } else {
 #pragma unroll
     for (int u = 0; u < kUnroll; ++u) {
       const int64_t i = base + u * kStep;
       r[u] = i < n4 ? triad4(b4[i], c4[i], sd) : make_float4(0.f, 0.f, 0.f, 0.f);
-      extra[u] = 0.f;
+      extra[u] = -0.f;
       if (Sum == SUM_BLOCK256 && i == n4) {
         // the lane whose float4 slot holds the end of the vector takes the one to three elements there
         for (int64_t e = n4 << 2; e < n; ++e) {

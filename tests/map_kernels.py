@@ -211,3 +211,113 @@ def max_abs_difference():
 
 
 MAX_TREES = {"max_abs": max_abs, "max_abs_difference": max_abs_difference}
+
+
+def _random_expression(rng, reads, index, scalars=("a", "b"), lets_made=(), depth=None):
+    """A seeded f32 expression tree over the element's inputs (`reads`: the read forms), the f32 scalars, the int
+    scalar k and the element's index: arithmetic, a guarded division, one-argument math intrinsics, `if` expressions
+    on values and on the index, casts of index arithmetic, negation."""
+    def int_expr(d):
+        pick = rng.randint(0, 3 if d > 0 else 1)
+        if pick == 0:
+            return index
+        if pick == 1:
+            return i32(rng.randint(1, 9))
+        if pick == 2:
+            return mod(int_expr(d - 1), add(var("k"), i32(rng.randint(1, 5))))     # k >= 0 at the call sites
+        return add(int_expr(d - 1), mul(int_expr(d - 1), i32(rng.randint(1, 3))))
+
+    def leaf():
+        pick = rng.randint(0, 5)
+        if pick <= 2:
+            return rng.choice(reads)
+        if pick == 3:
+            return var(rng.choice(scalars), "f32")
+        if pick == 4 and lets_made:
+            return rng.choice(lets_made)
+        return f32(repr(round(rng.uniform(-4, 4), 3)))
+
+    def expr(d):
+        if d == 0:
+            return leaf()
+        pick = rng.randint(0, 9)
+        if pick <= 3:
+            return op(rng.choice(["add", "sub", "mul"]), expr(d - 1), expr(d - 1))
+        if pick == 4:
+            return div(expr(d - 1), add(intr("fabs", "Float32", expr(d - 1)), f32("1.5")))
+        if pick == 5:
+            return intr(rng.choice(["sqrt", "exp", "log", "sin", "cos", "tanh", "floor", "fabs"]), "Float32", expr(d - 1))
+        if pick == 6:
+            cond = op(rng.choice(["lt", "le", "gt"]), expr(d - 1), expr(d - 1))
+            return f"(if {cond} {expr(d - 1)} {expr(d - 1)})"
+        if pick == 7:
+            cond = op(rng.choice(["lt", "eq"]), mod(index, i32(rng.randint(2, 7))), i32(rng.randint(0, 3)))
+            return f"(if {cond} {expr(d - 1)} {expr(d - 1)})"
+        if pick == 8:
+            return f"(cast f32 {int_expr(2)})"
+        return f"(neg {expr(d - 1)})"
+
+    return expr(rng.randint(2, 4) if depth is None else depth)
+
+
+def random_map(seed):
+    """A seeded element-wise kernel of the shape the map class takes: one to four input vectors, two f32 scalars, an
+    int scalar, immutable lets in front of the store.  Returns (ir, number of input vectors)."""
+    import random
+    rng = random.Random(seed)
+    n_in = rng.randint(1, 4)
+    params = [(f"x{i}", "(vec f32)") for i in range(n_in)] + [("out", "(vec f32)"), ("a", "f32"), ("b", "f32"),
+                                                               ("k", "i32"), ("n", "i32")]
+    _params(params)
+    tid = var("tid")
+    reads = [read(f"x{i}", tid) for i in range(n_in)]
+    lets_made, bindings = [], []
+    for j in range(rng.randint(0, 3)):
+        e = _random_expression(rng, reads, tid, lets_made=tuple(lets_made), depth=rng.randint(1, 3))
+        v = var(f"t{j}", "f32")
+        bindings.append((v, e))
+        lets_made.append(v)
+    body = assign_elem("out", tid, _random_expression(rng, reads, tid, lets_made=tuple(lets_made)))
+    for v, e in reversed(bindings):
+        body = let(v, e, body)
+    return kernel(params, let(tid, intr("global_thread_id", "Std"), if_(lt(tid, var("n")), body))), n_in
+
+
+def random_tree(seed, maximum=False):
+    """The reference's block-256 sum (or maximum) tree with a seeded expression of one to three inputs, two f32
+    scalars and an int scalar where it reads input[gid].  Returns (tree ir, map ir, number of inputs): the map
+    kernel stores the same expression element by element, for the values the tree adds up or compares."""
+    import random
+    rng = random.Random(seed * 2 + int(maximum))
+    n_in = rng.randint(1, 3)
+    names = ["input", "y", "z"][:n_in]
+    fresh()
+    for name in ("a", "b"):
+        var(name, "f32")
+    var("k")
+    tree_params = [("input", 1, "(vec f32)")] + [(nm, 30 + 2 * i, "(vec f32)") for i, nm in enumerate(names[1:])] + \
+        [("output", 2, "(vec f32)"), ("a", 41, "f32"), ("b", 42, "f32"), ("k", 43, "i32"), ("n", 3, "i32")]
+    # the tree classes want every input vector read: draw until the expression reads them all
+    while True:
+        state = rng.getstate()
+        probe = _random_expression(rng, [read(nm, "@") for nm in names], "@", depth=rng.randint(1, 3))
+        if all(f"(read {nm} @)" in probe for nm in names):
+            break
+
+    def leaf_of(index):
+        rng.setstate(state)                       # the same tree for the tree kernel and for the map kernel
+        return _random_expression(rng, [read(nm, index) for nm in names], index, depth=rng.randint(1, 3))
+
+    def with_ids(text):                            # the builders number a, b, k as they like: the parameters' ids
+        for name, ident, ty in (("a", 41, "f32"), ("b", 42, "f32"), ("k", 43, "i32")):
+            import re
+            text = re.sub(r"\(var " + name + r" \d+ " + ty + r"\)", f"(var {name} {ident} {ty})", text)
+        return text
+
+    build = _max_tree_with if maximum else _tree_with
+    tree_ir = with_ids(build(leaf_of, tree_params))
+    tid = "(var tid 50 i32)"
+    map_params = " ".join(f"(param (var {nm} {i} {t}))" for nm, i, t in tree_params)
+    map_ir = (f"(kernel sarek_kern (params {map_params}) (locals) (body (let {tid} (intr (Std) global_thread_id) "
+              f"(if (lt {tid} (var n 3 i32)) (assign (lelem output {tid}) {with_ids(leaf_of(tid))})))) (native_fn true))")
+    return tree_ir, map_ir, n_in

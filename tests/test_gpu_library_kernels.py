@@ -371,6 +371,28 @@ def test_fused_pair_kernel_at_full_size_properties(hip, torch_cuda):
     assert total.item() == 1.75 * n
 
 
+@pytest.mark.parametrize("n", [256, 4097, 100003])
+def test_fused_pair_keeps_the_sign_of_a_zero_sum(hip, torch_cuda, n):
+    """Blocks whose 256 elements are all -0 sum to -0 in the block-256 kernel (-0 + -0 = -0); the fused kernel adds
+    the scalar tail's share to every block and must not turn that into +0.  Bits, not values."""
+    torch = torch_cuda
+    b = torch.full((n,), -0.0, device="cuda")
+    c = torch.full((n,), -0.0, device="cuda")
+    for runs in (1, 0):
+        hip.check(hip.lib.sarek_hip_set_tunable(b"triad.block_sum_runs", runs))
+        try:
+            a, sums = hip.triad_block256_sum(b, c, 3.0)
+        finally:
+            hip.check(hip.lib.sarek_hip_set_tunable(b"triad.block_sum_runs", 1))
+        a2 = hip.triad(b, c, 3.0)
+        s2 = torch.empty((n + 255) // 256, device="cuda")
+        hip.check(hip.lib.sarek_hip_reduce_sum_block256_f32(a2.data_ptr(), s2.data_ptr(), n, None))
+        torch.cuda.synchronize()
+        assert bool(torch.signbit(a).all()) and torch.equal(a.view(torch.int32), a2.view(torch.int32))
+        assert torch.equal(sums.view(torch.int32), s2.view(torch.int32)), runs
+        assert bool(torch.signbit(s2[: n // 256]).all())          # the full blocks: -0; a padded last block: +0
+
+
 @pytest.mark.parametrize("n", [1, 255, 1000, 4097, 65536 + 777, (1 << 20) + 3, 5_000_001])
 def test_fused_pair_block_sum_layouts_agree(hip, oracle, torch_cuda, n):
     """The fused kernel's two layouts (a wave's four blocks neighbours, one 16-byte store; or a workgroup's width

@@ -104,6 +104,95 @@ def test_map_then_block_sum_is_one_launch(hip, sarek, name, n):
     assert np.all(np.abs(s_fused.astype(np.float64) - s_jit.astype(np.float64)) <= bound)
 
 
+@pytest.mark.parametrize("seed", range(int(os.environ.get("SAREK_HIP_TEST_MAP_SEEDS", "32"))))
+def test_seeded_random_maps_alone_and_in_front_of_the_sum(hip, sarek, seed):
+    """Kernels nobody wrote by hand: seeded expression trees (arithmetic, divisions, math intrinsics, `if`
+    expressions on values and on the index, casts of index arithmetic, lets) over one to four inputs.  The rebuilt
+    kernel writes the generated kernel's bits, alone and fused with the block sums, whose bits are the hand
+    block-256 kernel's on that vector."""
+    from map_kernels import random_map
+    E, V = sarek.Execute, sarek.Vector
+    ir, n_in = random_map(seed)
+    reduction = open(os.path.join(IR_DIR, "reduction.ir")).read()
+    for n in (4097, 100003):
+        nblocks = (n + 255) // 256
+        rng = np.random.default_rng(seed * 7 + n)
+        inputs = [(rng.standard_normal(n) * 10.0 ** rng.integers(-2, 2, n)).astype(np.float32) for _ in range(n_in)]
+
+        def run(pipeline):
+            out = V.create(V.float32, n)
+            out.host[:] = np.nan
+            args = [E.Vec(V.of_array(x)) for x in inputs] + [E.Vec(out), E.Float32(0.75), E.Float32(-1.25), E.Int32(3),
+                                                            E.Int32(n)]
+            shape = ((256, 1, 1), (nblocks, 1, 1))
+            if not pipeline:
+                return E.run_vectors(ir, args, *shape), out.to_array().copy(), None
+            sums = V.create(V.float32, nblocks)
+            path = E.run_pipeline([(ir, args) + shape, (reduction, [E.Vec(out), E.Vec(sums), E.Int32(n)]) + shape])
+            fused_sums = sums.to_array().copy()
+            assert E.run_vectors(reduction, [E.Vec(out), E.Vec(sums), E.Int32(n)], *shape) == \
+                ("reduce_sum_block256_f32" if pipeline == "on" else "jit")
+            return path, out.to_array().copy(), (fused_sums, sums.to_array().copy())
+
+        (p_map, got, _), (p_jit, want, _) = both_ways(hip, lambda: run(None))
+        assert (p_map, p_jit) == ("map_f32", "jit"), (seed, n)
+        same = got.view(np.uint32) == want.view(np.uint32)
+        assert bool((same | (np.isnan(got) & np.isnan(want))).all()), (seed, n, int((~same).sum()))
+        hip.check(hip.lib.sarek_hip_set_specialisation(1))
+        path, fused, (fused_sums, hand_sums) = run("on")
+        assert path == ("map_f32+reduce_sum_block256_f32", 1), (seed, n)
+        same = fused.view(np.uint32) == want.view(np.uint32)
+        assert bool((same | (np.isnan(fused) & np.isnan(want))).all()), (seed, n)
+        same = fused_sums.view(np.uint32) == hand_sums.view(np.uint32)
+        assert bool((same | (np.isnan(fused_sums) & np.isnan(hand_sums))).all()), (seed, n)
+
+
+@pytest.mark.parametrize("maximum", [False, True])
+@pytest.mark.parametrize("seed", range(int(os.environ.get("SAREK_HIP_TEST_MAP_SEEDS", "32")) // 2))
+def test_seeded_random_trees(hip, sarek, torch_cuda, seed, maximum):
+    """The block-256 sum and maximum trees with seeded expressions where they read their input.  Sum: the hand
+    block-256 kernel's sums of the expression's values (the values the map kernel of the same expression stores), bit
+    for bit, and the generated tree's within the sum's tolerance.  Maximum: the generated tree's maxima, bit for bit."""
+    from map_kernels import random_tree
+    torch = torch_cuda
+    E, V = sarek.Execute, sarek.Vector
+    tree_ir, map_ir, n_in = random_tree(seed, maximum)
+    for n in (4097, 100003):
+        nblocks = (n + 255) // 256
+        rng = np.random.default_rng(seed * 11 + n)
+        inputs = [(rng.standard_normal(n) * 10.0 ** rng.integers(-2, 2, n)).astype(np.float32) for _ in range(n_in)]
+        scalars = [E.Float32(0.75), E.Float32(-1.25), E.Int32(3), E.Int32(n)]
+
+        def run_tree():
+            out = V.create(V.float32, nblocks)
+            out.host[:] = -7.0
+            args = [E.Vec(V.of_array(x)) for x in inputs] + [E.Vec(out)] + scalars
+            return E.run_vectors(tree_ir, args, (256, 1, 1), (nblocks, 1, 1)), out.to_array().copy()
+
+        (p_hand, got), (p_jit, want) = both_ways(hip, run_tree)
+        assert (p_hand, p_jit) == ("tree_max_map_f32" if maximum else "tree_sum_map_f32", "jit"), (seed, n)
+        same = got.view(np.uint32) == want.view(np.uint32)
+        if maximum:
+            assert bool((same | (np.isnan(got) & np.isnan(want))).all()), (seed, n, int((~same).sum()))
+            continue
+        values = V.create(V.float32, n)
+        hip.check(hip.lib.sarek_hip_set_specialisation(0))
+        try:
+            args = [E.Vec(V.of_array(x)) for x in inputs] + [E.Vec(values)] + scalars
+            assert E.run_vectors(map_ir, args, (256, 1, 1), (nblocks, 1, 1)) == "jit"
+        finally:
+            hip.check(hip.lib.sarek_hip_set_specialisation(1))
+        vals = values.to_array().copy()
+        ref = hip.reduce_sum_block256(torch.from_numpy(vals).cuda()).cpu().numpy()
+        same = got.view(np.uint32) == ref.view(np.uint32)
+        assert bool((same | (np.isnan(got) & np.isnan(ref))).all()), (seed, n, int((~same).sum()))
+        finite = np.isfinite(vals)
+        bound = np.add.reduceat(np.where(finite, np.abs(vals.astype(np.float64)), 0.0), np.arange(0, n, 256)) * 1e-5 + 1e-30
+        ok = np.abs(got.astype(np.float64) - want.astype(np.float64)) <= bound
+        blocks_finite = np.logical_and.reduceat(finite, np.arange(0, n, 256))
+        assert bool((ok | ~blocks_finite).all()), (seed, n)
+
+
 def test_pairs_the_fused_kernel_does_not_serve(hip, sarek):
     E, V = sarek.Execute, sarek.Vector
     n = 70000

@@ -82,6 +82,11 @@ def test_operations(hip):
     assert expr_text(hip, "(add (i32 1) (i32 2))") == "(1 + 2)"
     assert expr_text(hip, "(mul (var x 1 i32) (i32 3))") == "(x * 3)"
     assert expr_text(hip, "(neg (var x 1 i32))") == "(-x)"
+    assert expr_text(hip, "(neg (neg (var x 1 i32)))") == "(-(-x))"
+    # the minus of a negation and the minus of a negative literal never meet ("--3.5f" decrements a literal)
+    assert expr_text(hip, "(neg (f32 -3.5))") == "(- -3.5f)"
+    assert expr_text(hip, "(neg (i32 -5))") == "(- -5)"
+    assert expr_text(hip, "(sub (var x 1 i32) (i32 -5))") == "(x - -5)"
     assert expr_text(hip, "(shl (var x 1 i32) (i32 2))") == "(x << 2)"
     assert expr_text(hip, "(if (lt (var x 1 i32) (i32 0)) (i32 1) (i32 2))") == "((x < 0) ? 1 : 2)"
     assert expr_text(hip, "(cast f32 (var x 1 i32))") == "(float)x"
