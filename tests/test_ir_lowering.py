@@ -511,3 +511,83 @@ def test_stencil_and_box_filter_are_recognised_and_near_misses_are_not(hip):
                            (cv, "(eq (var y 8 i32) (i32 0))", "(eq (var y 8 i32) (i32 1))")]:
         assert old in text
         assert not hip.generate_source(text.replace(old, new)).startswith(mark)
+
+
+# ---- mutation tests of the recognisers: a kernel that differs from a template in one token is another program ----
+
+_MUTATIONS = {"add": ["sub", "mul"], "sub": ["add"], "mul": ["add", "div"], "div": ["mul"], "mod": ["div"],
+              "lt": ["le", "gt"], "le": ["lt"], "gt": ["ge", "lt"], "ge": ["gt"], "eq": ["ne"], "ne": ["eq"],
+              "and": ["or"], "or": ["and"], "shl": ["shr"], "shr": ["shl"], "bitand": ["bitor"], "bitor": ["bitand"],
+              "bitxor": ["bitor"]}
+
+
+def _single_token_mutants(ir):
+    """(position, mutant text) for every operator swapped for a neighbour, every int32 constant moved by one either
+    way, every f32 constant moved by one, every loop turned round."""
+    import re
+    for m in re.finditer(r"\(([a-z_]+)\b|\((i32|f32) (-?[0-9.e+]+)\)|\b(upto)\b", ir):
+        if m.group(1) in _MUTATIONS:
+            for alt in _MUTATIONS[m.group(1)]:
+                yield m.start(1), ir[:m.start(1)] + alt + ir[m.end(1):]
+        elif m.group(2) == "i32":
+            for d in (1, -1):
+                yield m.start(3), ir[:m.start(3)] + str(int(m.group(3)) + d) + ir[m.end(3):]
+        elif m.group(2) == "f32":
+            yield m.start(3), ir[:m.start(3)] + repr(float(m.group(3)) + 1.0) + ir[m.end(3):]
+        elif m.group(4):
+            yield m.start(4), ir[:m.start(4)] + "downto" + ir[m.end(4):]
+
+
+def _tag_or_none(hip, ir):
+    try:
+        return split_tag(hip.generate_source(ir, block=(256, 1, 1)))[0]
+    except hip.SarekHipError:
+        return None
+
+
+@pytest.mark.parametrize("name", sorted(EXPECTED_TAGS))
+def test_no_single_token_mutant_of_a_template_keeps_its_tag(hip, name):
+    """The hand kernels stand in for fifteen exact programs.  Every operator of a recognised kernel swapped for a
+    neighbour (+ for -, < for <=, ...), every integer constant moved by one, every float constant changed, every
+    loop turned round gives a kernel that computes something else -- none of them may keep the template's tag."""
+    ir = open(os.path.join(IR_DIR, name + ".ir")).read()
+    tag = EXPECTED_TAGS[name]
+    mutants = list(_single_token_mutants(ir))
+    assert len(mutants) >= 2
+    assert [m for _, m in mutants if _tag_or_none(hip, m) == tag] == []
+
+
+def test_tree_class_mutants_keep_their_tag_only_inside_the_expression(hip):
+    """The tree classes take any expression where the reference's tree reads its input (and any fill constant in the
+    maximum tree); everything else is the tree to the letter.  A single-token mutant keeps the class tag exactly when
+    the token lies in the expression or is the fill value."""
+    import sys
+    sys.path.insert(0, HERE)
+    import map_kernels
+
+    def span_after(ir, head, start=0):
+        at = ir.index(head, start) + len(head)
+        depth, i = 0, at
+        while True:
+            depth += {"(": 1, ")": -1}.get(ir[i], 0)
+            i += 1
+            if depth == 0:
+                return at, i
+
+    store = "(assign (lelem sdata (var tid 5 i32)) "
+    for name, make in list(map_kernels.TREES.items()) + list(map_kernels.MAX_TREES.items()):
+        ir = make()
+        tag = _tag_or_none(hip, ir)
+        assert tag in ("tree_sum_map_f32", "tree_max_map_f32"), name
+        leaf = span_after(ir, store)
+        fill = span_after(ir, store, leaf[1])          # the guard's else branch: the padding value
+        kept = outside = 0
+        for at, mutant in _single_token_mutants(ir):
+            free = leaf[0] <= at < leaf[1] or (tag == "tree_max_map_f32" and fill[0] <= at < fill[1])
+            same = _tag_or_none(hip, mutant) == tag
+            if free:
+                kept += same
+            else:
+                outside += 1
+                assert not same, (name, ir[max(0, at - 60):at + 30])
+        assert kept >= 1 and outside >= 40, (name, kept, outside)
