@@ -540,6 +540,65 @@ def test_gemm16_ragged_shapes_stay_on_the_mfma_kernels(hip, oracle, torch_cuda, 
         hip.set_tunable("gemm16.split_k", 0)
 
 
+@pytest.mark.parametrize("seed", [1, 2, 3])
+def test_seeded_random_shapes_through_every_gemm_entry_point(hip, torch_cuda, seed):
+    """150 seeded shapes per seed (dimensions at and next to 1, 8, 16, 32, 64, 128, 256, 512 and at random up to
+    700 x 1100 x 900), an entry point (bf16, fp16, f32, fused epilogue), a tile choice and a K split drawn for each;
+    A, B and C at element offsets 0 to 129 inside buffers that are NaN (operands) or a guard value (results) everywhere
+    else.  Against the float64 product of the same rounded operands, computed on the device (it differs from the
+    oracle's k-ordered double sum by 1e-16 relative, far inside the bars): 1e-4 of max|C| for 16-bit operands, 1e-5 for
+    f32, row sums 1e-5 per row; nothing stored outside C or the row sums, nothing non-finite."""
+    import random
+    torch = torch_cuda
+    rng = random.Random(seed)
+
+    def dim(hi):
+        base = rng.choice([1, 2, 7, 8, 15, 16, 17, 31, 32, 33, 63, 64, 65, 127, 128, 129, 255, 256, 257, 300, 511, 512,
+                           513, hi])
+        return max(1, min(hi, base + rng.choice([0, 0, 0, 1, -1, 3, rng.randint(0, 40)])))
+
+    knobs = ("gemm16.tile", "gemm16.split_k", "gemm_f32.tile", "gemm_f32.split_k")
+    for it in range(150):
+        m, n, k = dim(700), dim(1100), dim(900)
+        kind = rng.choice(["bf16", "f16", "f32", "epi"])
+        tile = rng.choice([0, 0, 128, 256]) if kind != "f32" else rng.choice([0, 0, 64, 128, 256])
+        split = rng.choice([0, 0, 1, 2, 3])
+        case = (seed, it, kind, m, n, k, tile, split)
+        g = torch.Generator(device="cuda")
+        g.manual_seed(seed * 1000 + it)
+        dt = {"bf16": torch.bfloat16, "f16": torch.float16, "f32": torch.float32, "epi": torch.float16}[kind]
+        offa, offb, offc = rng.choice([0, 1, 3, 8, 129]), rng.choice([0, 1, 5, 8, 129]), rng.choice([32, 33, 35])
+        buf_a = torch.full((m * k + 300,), float("nan"), device="cuda").to(dt)
+        buf_b = torch.full((k * n + 300,), float("nan"), device="cuda").to(dt)
+        da, db = buf_a[offa:offa + m * k].view(m, k), buf_b[offb:offb + k * n].view(k, n)
+        da.copy_((torch.randn(m, k, device="cuda", generator=g) * 0.1).to(dt))
+        db.copy_((torch.randn(k, n, device="cuda", generator=g) * 0.1).to(dt))
+        ref = da.double() @ db.double()
+        guard = torch.full((m * n + 64,), 7.0, device="cuda")
+        c = guard[offc:offc + m * n].view(m, n)
+        try:
+            hip.set_tunable("gemm_f32.tile" if kind == "f32" else "gemm16.tile", tile)
+            hip.set_tunable("gemm_f32.split_k" if kind == "f32" else "gemm16.split_k", split)
+            if kind == "epi":
+                bias = torch.rand(n, device="cuda", generator=g) * 0.2 - 0.1
+                rs = torch.full((m + 16,), 7.0, device="cuda")
+                hip.gemm_f16_bias_relu_rowsum(da, db, bias, out=c, rowsum=rs[8:8 + m])
+                ref = torch.relu(ref + bias.double())
+                sums = ref.sum(dim=1)
+                assert bool((rs[:8] == 7).all()) and bool((rs[8 + m:] == 7).all()), case
+                assert bool(((rs[8:8 + m].double() - sums).abs() <= 1e-5 * sums.abs() + 1e-6 * sums.abs().max()).all()), case
+            else:
+                {"bf16": hip.gemm_bf16, "f16": hip.gemm_f16, "f32": hip.gemm_f32}[kind](da, db, out=c)
+        finally:
+            for t in knobs:
+                hip.set_tunable(t, 0)
+        torch.cuda.synchronize()
+        assert bool((guard[:offc] == 7).all()) and bool((guard[offc + m * n:] == 7).all()), case
+        assert bool(torch.isfinite(c).all()), case
+        err = (c.double() - ref).abs().max().item() / max(ref.abs().max().item(), 1e-30)
+        assert err <= (1e-5 if kind == "f32" else 1e-4), (case, err)
+
+
 @pytest.mark.parametrize("m,n,k", [(130, 137, 40), (257, 1001, 1000), (64, 4100, 96), (4, 1, 64), (300, 263, 136)])
 def test_epilogue_ragged_shapes(hip, oracle, torch_cuda, m, n, k):
     """The fused epilogue on the same kinds of shape (the last column of an odd N comes from the matrix-vector kernel,
