@@ -142,3 +142,77 @@ def test_hand_and_generated_routes_agree_under_any_geometry(hip, sarek, seed):
     assert failures == []
     assert all("hand" in r for r in routes.values()), routes
     assert sum("jit" in r for r in routes.values()) >= 6, routes
+
+
+@pytest.mark.parametrize("seed", [1, 2])
+def test_pipelines_agree_with_their_stages_run_as_generated(hip, sarek, seed):
+    """Execute.run_pipeline on [producer; block reduction] pairs drawn at random: the stream triad, the vector add or a
+    seeded random map in front of the block-256 sum or maximum; geometries that fit or are off by a block, the
+    reduction over the producer's vector or another one, over all of it or fewer elements.  One launch serves a pair
+    only when the pair is the fused operation; whatever route is taken, the vector and the block results are what the
+    two generated kernels leave (triad: one ulp, the hand kernel rounds the double result; sums: 1e-5 x 256 x scale,
+    another association; everything else bit for bit)."""
+    import os
+    import sys
+    sys.path.insert(0, os.path.dirname(os.path.abspath(__file__)))
+    from map_kernels import random_map
+    from spoc_amd import reference_kernels as rk
+    E, V = sarek.Execute, sarek.Vector
+    rng = random.Random(seed)
+    routes, failures = {}, []
+
+    def fvec(x):
+        return V.of_array(np.ascontiguousarray(x, dtype=np.float32))
+
+    for it in range(150):
+        n = rng.choice([1, 255, 256, 257, 1000, 4096, 4097, 70001, 300000])
+        first, second = rng.choice(["triad", "add", "map"]), rng.choice(["sum", "max"])
+        blocks = (n + 255) // 256
+        n_red = n if rng.random() < 0.8 else max(1, n - rng.choice([1, 256, 300]))
+        blocks_red = (n_red + 255) // 256
+        g1 = max(1, blocks + rng.choice([0, 0, 0, 1, -1]))
+        g2 = max(1, blocks_red + rng.choice([0, 0, 0, 1, -1]))
+        another_vector = rng.random() < 0.1
+        map_seed = rng.randrange(100)
+
+        def run():
+            nrng = np.random.default_rng(seed * 1000 + it)
+            out, res = fvec(np.full(n, 7.0)), fvec(np.full(max(g2, blocks_red) + 2, 7.0))
+            b, c = fvec(nrng.standard_normal(n)), fvec(nrng.standard_normal(n))
+            if first == "triad":
+                ir, args = rk.stream_triad(), [E.Vec(out), E.Vec(b), E.Vec(c), E.Float32(3.0), E.Int32(n)]
+            elif first == "add":
+                ir, args = rk.vector_add(), [E.Vec(b), E.Vec(c), E.Vec(out), E.Int32(n)]
+            else:
+                ir, n_in = random_map(map_seed)
+                args = [E.Vec(fvec(nrng.standard_normal(n))) for _ in range(n_in)] + \
+                    [E.Vec(out), E.Float32(0.75), E.Float32(-1.25), E.Int32(3), E.Int32(n)]
+            source = fvec(np.arange(n) % 7) if another_vector else out
+            reduction = rk.tree(False) if second == "sum" else rk.reduction_max(-1000000.0)
+            path = E.run_pipeline([(ir, args, (256, 1, 1), (g1, 1, 1)),
+                                   (reduction, [E.Vec(source), E.Vec(res), E.Int32(n_red)], (256, 1, 1), (g2, 1, 1))])
+            return path, out.to_array().copy(), res.to_array().copy()
+
+        results = []
+        for on in (1, 0):
+            hip.check(hip.lib.sarek_hip_set_specialisation(on))
+            try:
+                results.append(run())
+            finally:
+                hip.check(hip.lib.sarek_hip_set_specialisation(1))
+        (path, vec, red), (p_jit, vec_jit, red_jit) = results
+        assert p_jit == ("jit;jit", 2)
+        routes[path[0]] = routes.get(path[0], 0) + 1
+        ulps = np.abs(vec.view(np.int32).astype(np.int64) - vec_jit.view(np.int32).astype(np.int64))
+        vec_ok = (ulps <= (1 if first == "triad" else 0)) | (np.isnan(vec) & np.isnan(vec_jit))
+        if second == "max":
+            red_ok = (red == red_jit) | (np.isnan(red) & np.isnan(red_jit))
+        else:
+            scale = max(1.0, float(np.abs(np.nan_to_num(vec_jit, nan=0.0, posinf=0.0, neginf=0.0)).max()))
+            with np.errstate(invalid="ignore"):              # inf - inf where a random map overflowed
+                red_ok = (np.abs(red - red_jit) <= 1e-5 * 256 * scale) | ~np.isfinite(red_jit)
+        if not (vec_ok.all() and red_ok.all()):
+            failures.append((seed, it, first, second, n, n_red, g1, g2, another_vector, path))
+    assert failures == []
+    fused = [r for r in routes if "+" in r]
+    assert len(fused) >= 5 and "jit;jit" in routes and any(";" in r and r != "jit;jit" for r in routes), routes
