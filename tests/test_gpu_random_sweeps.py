@@ -11,6 +11,8 @@ kernels are tests/test_gpu_stream.py, test_gpu_layout.py, test_gpu_histogram.py)
   maximum exact
   fold 1e-12
   copy, transpose                                                           exact, nothing stored outside the result
+  five-point stencil, 3 x 3 box filter                                      bit for bit the double sums in the benches' order, one
+                                                                            rounding; borders kept (stencil) or zero (filter)
   histogram (mod bins), radix histogram (shift, mask), radix scatter        exact counts on top of what the bins held
   output
                                                                             ordered by digit, the same keys per digit, counters
@@ -56,7 +58,7 @@ def test_seeded_random_cases(hip, torch_cuda, seed):
                 failures.append((seed, it, kind, n, what))
 
         kind = rng.choice(["triad", "triad_bsum", "triad_bmax", "triad_sum", "bsum", "bmax", "dot", "fold", "copy",
-                           "transpose", "hist", "rhist", "scatter"])
+                           "transpose", "hist", "rhist", "scatter", "stencil", "conv2d"])
         n = size()
         g = torch.Generator(device="cuda")
         g.manual_seed(it)
@@ -135,6 +137,27 @@ def test_seeded_random_cases(hip, torch_cuda, seed):
             hip.transpose(x.view(h, w), out=out.view(w, h))
             torch.cuda.synchronize()
             expect(torch.equal(out.view(w, h), x.view(h, w).t()) and guard_ok(obuf, off, h * w, 7.0), "transpose")
+        elif kind in ("stencil", "conv2d"):
+            h = rng.choice([1, 2, 3, 4, 5, 17, 64, 65, 200, 777])
+            w = rng.choice([1, 2, 3, 4, 5, 8, 63, 64, 65, 129, 256, 500, 1031])
+            _, x, _ = view(h * w)
+            x.copy_(torch.randn(h * w, device="cuda", generator=g) * 10.0 ** rng.randint(-3, 3))
+            obuf, out, off = view(h * w, fill=7.0)
+            g2, d = x.view(h, w), x.view(h, w).double()
+            want = torch.full((h, w), 7.0 if kind == "stencil" else 0.0, device="cuda")
+            if h > 2 and w > 2:
+                if kind == "stencil":          # up + down + left + right + center, in double, / 5.0, one rounding
+                    inner = (d[:-2, 1:-1] + d[2:, 1:-1] + d[1:-1, :-2] + d[1:-1, 2:] + d[1:-1, 1:-1]) / 5.0
+                else:                          # the nine cells row by row, in double, / 9.0, one rounding
+                    inner = d[:-2, :-2] + d[:-2, 1:-1] + d[:-2, 2:]
+                    inner = inner + d[1:-1, :-2] + d[1:-1, 1:-1] + d[1:-1, 2:]
+                    inner = (inner + d[2:, :-2] + d[2:, 1:-1] + d[2:, 2:]) / 9.0
+                want[1:-1, 1:-1] = inner.float()
+            (hip.stencil_2d if kind == "stencil" else hip.conv2d)(g2, out=out.view(h, w))
+            torch.cuda.synchronize()
+            n = (h, w)
+            expect(torch.equal(out.view(h, w).view(torch.int32), want.view(torch.int32)), "grid bits")
+            expect(guard_ok(obuf, off, h * w, 7.0), "guard")
         elif kind in ("hist", "rhist"):
             bins = rng.choice([1, 2, 7, 16, 100, 255, 256])
             _, keys, _ = view(n, torch.int32, 0)
