@@ -591,3 +591,63 @@ def test_tree_class_mutants_keep_their_tag_only_inside_the_expression(hip):
                 outside += 1
                 assert not same, (name, ir[max(0, at - 60):at + 30])
         assert kept >= 1 and outside >= 40, (name, kept, outside)
+
+
+def test_random_expressions_lower_to_text_the_device_compiler_takes(hip, tmp_path):
+    """150 seeded integer kernels (arithmetic, bit operations, shifts, negations of negative literals, casts through
+    float, `if` expressions, `not` / `and` / `or` in the guard) and 150 seeded float maps, lowered and handed to the
+    device compiler's front end in one translation unit: the text must parse, whatever the operands of a unary
+    minus or a cast begin with."""
+    import random
+    import shutil
+    import subprocess
+    import sys
+    sys.path.insert(0, HERE)
+    import map_kernels
+    from spoc_amd import reference_kernels as rk
+    hipcc = shutil.which("hipcc") or "/opt/rocm/bin/hipcc"
+    if not os.path.exists(hipcc):
+        pytest.skip("no hipcc to parse the text with")
+
+    def int_expr(rng, depth, leaves):
+        if depth == 0:
+            return rng.choice(leaves + [rk.i32(rng.randint(-9, 12))])
+        a, b = int_expr(rng, depth - 1, leaves), int_expr(rng, depth - 1, leaves)
+        pick = rng.randint(0, 7)
+        if pick == 0:
+            return rk.op(rng.choice(["add", "sub", "mul"]), a, b)
+        if pick == 1:
+            return rk.op(rng.choice(["bitand", "bitor", "bitxor"]), a, b)
+        if pick == 2:
+            return rk.op(rng.choice(["shl", "shr"]), a, rk.i32(rng.randint(0, 5)))
+        if pick == 3:
+            return f"(neg {a})"
+        if pick == 4:
+            return f"(bitnot {a})"
+        if pick == 5:
+            return f"(if {rk.op(rng.choice(['lt', 'le', 'gt', 'ge', 'eq', 'ne']), a, b)} {a} {b})"
+        if pick == 6:
+            return rk.op("mod", a, rk.add(rk.op("bitand", b, rk.i32(7)), rk.i32(1)))
+        return f"(cast i32 (cast f32 {a}))"
+
+    texts = ["#include <hip/hip_runtime.h>\n"]
+    for seed in range(150):
+        rng = random.Random(seed)
+        rk.fresh()
+        params = [("x", "(vec i32)"), ("out", "(vec i32)"), ("k", "i32"), ("n", "i32")]
+        for p, t in params:
+            rk.var(p, t)
+        tid = rk.var("tid")
+        value = int_expr(rng, rng.randint(2, 4), [tid, rk.var("k"), rk.read("x", tid)])
+        guard = rng.choice([f"(not {rk.lt(tid, rk.var('k'))})",
+                            f"(and {rk.lt(tid, rk.var('n'))} (or {rk.op('ge', tid, rk.i32(0))} {rk.op('ne', rk.var('k'), rk.i32(-2))}))"])
+        body = rk.let(tid, rk.intr("global_thread_id", "Std"),
+                      rk.if_(rk.lt(tid, rk.var("n")),
+                             rk.if_(guard, rk.assign_elem("out", tid, value), rk.assign_elem("out", tid, f"(neg {rk.i32(-7)})"))))
+        texts.append(hip.generate_source(rk.kernel(params, body)).replace("sarek_kern", f"ints_{seed}"))
+        texts.append(hip.generate_source(map_kernels.random_map(1000 + seed)[0]).replace("sarek_kern", f"floats_{seed}"))
+    path = tmp_path / "random_kernels.hip"
+    path.write_text("\n".join(texts))
+    done = subprocess.run([hipcc, "--offload-arch=gfx950", "--cuda-device-only", "-fsyntax-only", "-w", str(path)],
+                          capture_output=True, text=True, timeout=300)
+    assert done.returncode == 0, done.stderr[-3000:]
