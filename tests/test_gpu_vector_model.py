@@ -16,6 +16,7 @@ a Stale_CPU vector is not tracked and is overwritten by the next download, a wri
 Stale_GPU although the host copy was never fetched, a sub-vector writes through to its parent's host block without
 touching the parent's location."""
 import ctypes as C
+import os
 import random
 
 import numpy as np
@@ -98,7 +99,7 @@ def device_contents(hip, v):
     return out
 
 
-@pytest.mark.parametrize("seed", range(12))
+@pytest.mark.parametrize("seed", range(int(os.environ.get("SAREK_HIP_TEST_WALK_SEEDS", "12"))))
 def test_random_walks_follow_the_reference_state_machine(hip, sarek, seed):
     E, V, T = sarek.Execute, sarek.Vector, sarek.Transfer
     rng = random.Random(seed)
