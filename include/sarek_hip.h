@@ -714,8 +714,9 @@ int sarek_hip_fusion_is_reduction_kernel(const char *kernel_ir, const char *arra
 /* Integer tuning knob (launch shapes, tile variants), for sweeps without a
  * rebuild.  Unknown names are stored and ignored.  Every knob of the product
  * library leaves results as they are; the knobs of the measurement build
- * (gemm16.ablate, gemm16.ring, gemm16.tj, gemm16.mfma, gemm16.waves) are refused by the
- * product library with SAREK_HIP_E_UNSUPPORTED.                              */
+ * (gemm16.ablate, gemm16.ring, gemm16.tj, gemm16.mfma, gemm16.waves,
+ * gemm16.barriers) are refused by the product library with
+ * SAREK_HIP_E_UNSUPPORTED.                                                   */
 int sarek_hip_set_tunable(const char *name, int64_t value);
 
 /* 1 in libsarek_hip_measure.so (built with -DSAREK_HIP_MEASURE by `make measure`: the

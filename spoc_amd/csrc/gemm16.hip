@@ -70,13 +70,15 @@ __device__ __forceinline__ u32x2 lds_read_tr16(const char *lds, int off) {
 //
 // Order of a wave's transfers (what vmcnt counts): top of slab j: B(j-1+NB), into the stage
 // slab j-1 used; after the barrier of slab j: the A stage that slab j was the last to read.
-constexpr int dma_allowed_in_flight(int I, int RA, int NA, int NB, int DA, int DB) {
+constexpr int dma_allowed_in_flight(int I, int RA, int NA, int NB, int DA, int DB, int slabs_per_barrier = 1) {
   // Transfers that may still be in flight at the barrier of slab s = I (mod period) once
   // everything slab s+1 reads has landed: those issued after the later of B(s+1) and the
   // A stage that slab s+1 starts (if it starts one).  Event 2j = top of slab j, 2j+1 = its
-  // barrier.
+  // barrier.  With a barrier in every other slab only (slabs_per_barrier = 2: the top of slab j
+  // issues B(j-2+NB), and the barrier of an odd slab s covers what slabs s+1 and s+2 read) the
+  // later B slab is B(s+2), issued at the top of slab s+4-NB.
   const int s = I + 64 * RA * NA * NB;
-  int need = 2 * (s + 2 - NB);
+  int need = slabs_per_barrier == 2 ? 2 * (s + 4 - NB) : 2 * (s + 2 - NB);
   if ((s + 1) % RA == 0) {
     const int ev = 2 * (s + RA - RA * NA) + 1;
     if (ev > need) need = ev;
@@ -542,14 +544,19 @@ __device__ __forceinline__ void epilogue16(f32x4_t (&acc)[TI][4], float *__restr
   }
 }
 
-template <bool Bf16, int Epi, int Ablate = 0, bool Ragged = false>
+template <bool Bf16, int Epi, int Ablate = 0, bool Ragged = false, bool HalfBarriers = false>
 __global__ __launch_bounds__(512) void gemm16_m16_kernel(const uint16_t *__restrict__ A, const uint16_t *__restrict__ B,
                                                          float *__restrict__ C, const float *__restrict__ bias,
                                                          float *__restrict__ rowsum, int M, int N, int K, int tiles_m,
                                                          int tiles_n, int xcd_remap, unsigned long long *probe, int ld,
                                                          float *__restrict__ rs_planes) {
-  constexpr int BKA = 64, BKB = 32, NA = 2, NB = 4;
+  // HalfBarriers: one barrier per A stage (K = 64) instead of one per B slab (K = 32).  A transfer may then only
+  // overwrite the slab before the previous one (the waves are a whole stage apart at most), so the top of slab j
+  // issues B(j - 2 + NB) and the ring is two slabs deeper, 160 KiB of LDS in all.
+  constexpr int BKA = 64, BKB = 32, NA = 2, NB = HalfBarriers ? 6 : 4;
+  constexpr int BEHIND = HalfBarriers ? 2 : 1;   // the slab whose stage the top of a slab refills lies this far back
   constexpr int RA = BKA / BKB;                  // B slabs per A stage
+  static_assert(!HalfBarriers || RA == 2, "the barrier sits in the second slab of an A stage");
   constexpr int A_ROW = BKA * 2, A_CHUNKS = A_ROW / 16, A_ROWS_PER_DMA = 1024 / A_ROW;
   constexpr int A_BYTES_S = BM * A_ROW, B_BYTES_S = BKB * BN * 2;
   constexpr int NWAVES = 8, WN = 4;
@@ -726,17 +733,20 @@ __global__ __launch_bounds__(512) void gemm16_m16_kernel(const uint16_t *__restr
   auto slab = [&](auto ic, int s) {
     constexpr int I = decltype(ic)::value;
     constexpr int In = (I + 1) % P;
-    constexpr int ia = (I / RA) % NA, ib = I % NB, ibp = (I + NB - 1) % NB;
+    constexpr int ia = (I / RA) % NA, ib = I % NB, ibp = (I + NB - BEHIND) % NB;
     constexpr int ian = (In / RA) % NA, ibn = In % NB;
     constexpr int ks = I % RA, ksn = In % RA;
     (void)ib;
     asm volatile("" : "+v"(a_addr0), "+v"(b_addr0));
-    issue_b(lds_ring<20 + ibp, B_BYTES_S>, s - 1 + NB);
+    issue_b(lds_ring<20 + ibp, B_BYTES_S>, s - BEHIND + NB);
     load_a(lds_ring<10 + ia, A_BYTES_S>, ks, 1, af[1]);
     mfma_range(std::integral_constant<int, 0>{}, std::integral_constant<int, 16>{}, af, bf[I & 1]);
     spread(std::integral_constant<int, DB>{}, std::integral_constant<int, 4>{}, std::integral_constant<int, 16>{});
-    __builtin_amdgcn_s_waitcnt(waitcnt_vm_lgkm0(dma_allowed_in_flight(I, RA, NA, NB, DA, DB)));
-    barrier_no_fence();
+    if constexpr (!HalfBarriers || I % RA == RA - 1) {
+      __builtin_amdgcn_s_waitcnt(
+          waitcnt_vm_lgkm0(dma_allowed_in_flight(I, RA, NA, NB, DA, DB, HalfBarriers ? 2 : 1)));
+      barrier_no_fence();
+    }
     if constexpr (I % RA == RA - 1) issue_a(lds_ring<10 + ia, A_BYTES_S>, s / RA + NA);
     // the next slab's fragments in the order its first MFMAs need them: A tile 0, the four B tiles, A tiles 1-3.
     // (The barrier was also tried after 8 and after 12 MFMAs, with the low-half A registers reloaded behind their
@@ -756,7 +766,7 @@ __global__ __launch_bounds__(512) void gemm16_m16_kernel(const uint16_t *__restr
   }(std::make_integer_sequence<int, NA>{});
   [&]<int... Is>(std::integer_sequence<int, Is...>) {
     (issue_b(lds_ring<20 + Is, B_BYTES_S>, Is), ...);
-  }(std::make_integer_sequence<int, NB - 1>{});
+  }(std::make_integer_sequence<int, NB - BEHIND>{});
   __builtin_amdgcn_s_waitcnt(waitcnt_vm_lgkm0(0));
   barrier_no_fence();
   load_a(lds_ring<10, A_BYTES_S>, 0, 0, af[0]);
@@ -1558,6 +1568,9 @@ int launch_gemm16(const uint16_t *a, const uint16_t *b, float *c, const float *b
     if (Epi == EPI_STORE && !ragged && tunable("gemm16.waves", 8) == 4) {
       hipLaunchKernelGGL((gemm16_m16w4_kernel<Bf16>), dim3(tiles_m * tiles_n), dim3(256), 0, st, a, b, c, m, nm, k, tiles_m,
                          tiles_n, remap, n);
+    } else if (!ragged && tunable("gemm16.barriers", 2) == 1) {
+      hipLaunchKernelGGL((gemm16_m16_kernel<Bf16, Epi, 0, false, true>), dim3(tiles_m * tiles_n), dim3(512), 0, st, a, b, c,
+                         bias, rowsum, m, nm, k, tiles_m, tiles_n, remap, probe, n, planes);
     } else
 #endif
     if (ragged)

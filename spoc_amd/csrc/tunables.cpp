@@ -55,7 +55,7 @@ extern "C" int sarek_hip_set_tunable(const char *name, int64_t value) {
   if (!name) return SAREK_HIP_E_INVALID_ARG;
   // knobs of kernels that only the measurement build holds (some of them compute wrong results on purpose)
   if (!sarek_hip::kMeasureBuild)
-    for (const char *measure_only : {"gemm16.ablate", "gemm16.ring", "gemm16.tj", "gemm16.mfma", "gemm16.waves"})
+    for (const char *measure_only : {"gemm16.ablate", "gemm16.ring", "gemm16.tj", "gemm16.mfma", "gemm16.waves", "gemm16.barriers"})
       if (std::string_view(name) == measure_only)
         return sarek_hip::fail(SAREK_HIP_E_UNSUPPORTED, "tunable %s exists in the measurement build only (libsarek_hip_measure.so)",
                                name);

@@ -67,6 +67,25 @@ def main():
         assert torch.equal(got, ref) and torch.equal(got16, ref16), (m, n, k)
     print("4-wave kernel ok", flush=True)
 
+    # one barrier per K = 64 instead of per K = 32 (a deeper B ring): the 8-wave kernel's bits, run after run
+    for (m, n, k) in [(256, 256, 64), (256, 256, 192), (512, 768, 448), (300, 520, 256), (1024, 1024, 1216)]:
+        a, b = normal16((m, k), m + 2), normal16((k, n), n + 2)
+        da, db = dev(a).bfloat16(), dev(b).bfloat16()
+        bias = dev(np.linspace(-0.1, 0.1, n, dtype=np.float32))
+        hip.set_tunable("gemm16.tile", 256)
+        try:
+            ref, ref16 = hip.gemm_bf16(da, db), hip.gemm_f16(da.half(), db.half())
+            y_ref, rs_ref = hip.gemm_f16_bias_relu_rowsum(da.half(), db.half(), bias)
+            hip.set_tunable("gemm16.barriers", 1)
+            for _ in range(3):
+                assert torch.equal(hip.gemm_bf16(da, db), ref) and torch.equal(hip.gemm_f16(da.half(), db.half()), ref16)
+            y, rs = hip.gemm_f16_bias_relu_rowsum(da.half(), db.half(), bias)
+            assert torch.equal(y, y_ref) and torch.equal(rs, rs_ref), (m, n, k)
+        finally:
+            hip.set_tunable("gemm16.barriers", 2)
+            hip.set_tunable("gemm16.tile", 0)
+    print("half-barrier kernel ok", flush=True)
+
     # the ablated variants: wrong by construction, but within bounds; other kernels refuse the knob
     m, n, k = 512, 768, 512
     torch.manual_seed(7)

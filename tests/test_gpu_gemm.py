@@ -280,7 +280,7 @@ def test_the_product_library_refuses_the_measurement_knobs(hip, torch_cuda):
     b = (torch.randn(k, n, device="cuda") * 0.1).bfloat16()
     good = hip.gemm_bf16(a, b)
     for knob, value in (("gemm16.ablate", 1), ("gemm16.ablate", 8), ("gemm16.mfma", 32), ("gemm16.ring", 4),
-                        ("gemm16.tj", 4), ("gemm16.waves", 4)):
+                        ("gemm16.tj", 4), ("gemm16.waves", 4), ("gemm16.barriers", 1)):
         with pytest.raises(hip.SarekHipError) as e:
             hip.set_tunable(knob, value)
         assert e.value.status == hip.E_UNSUPPORTED and "measurement build" in e.value.message
