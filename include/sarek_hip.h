@@ -543,7 +543,8 @@ int sarek_hip_reduce_max_block256_f32(const float *in, float *out, int64_t n, fl
  * and the one that finishes last adds those up in index order.  Every (device, stream) gets a stage of
  * its own (16 per device), so long folds on different streams do not meet; a stream beyond the
  * sixteenth, and any fold recorded under stream capture (a graph may be replayed on any stream, next
- * to anything), fold with one workgroup and no shared stage.                                        */
+ * to anything), fold with one workgroup that takes the 256 pieces in turn and needs no shared stage:
+ * slower, and the same bits, since it adds what the 256 add in the same order.                       */
 int sarek_hip_fold_partials_f64(const float *partials, int64_t count, double *sum_out,
                                 sarek_hip_stream stream);
 

@@ -278,6 +278,18 @@ struct FoldSlot {
   unsigned ticket;
   unsigned unused[63];
 };
+// The 256 stage values, one in each of the first 256 threads: four waves add theirs by exchanges, then the four sums
+// in wave order.  Valid in thread 0.
+__device__ __forceinline__ double fold_stage(double v) {
+  __shared__ double last_sums[kFoldGroups / 64];
+  if (threadIdx.x < kFoldGroups) {
+#pragma unroll
+    for (int m = 32; m >= 1; m >>= 1) v += __shfl_xor(v, m, 64);
+    if ((threadIdx.x & 63) == 0) last_sums[threadIdx.x >> 6] = v;
+  }
+  __syncthreads();
+  return (last_sums[0] + last_sums[1]) + (last_sums[2] + last_sums[3]);
+}
 __global__ __launch_bounds__(1024) void fold_onepass_kernel(const float *__restrict__ partials, int64_t count,
                                                             int64_t piece, FoldSlot *__restrict__ slot,
                                                             double *__restrict__ out) {
@@ -292,19 +304,32 @@ __global__ __launch_bounds__(1024) void fold_onepass_kernel(const float *__restr
   }
   __syncthreads();
   if (!last) return;
-  // the 256 stage values: four waves add theirs by exchanges, thread 0 the four sums in wave order
-  __shared__ double last_sums[kFoldGroups / 64];
-  if (threadIdx.x < kFoldGroups) {
-    double v = __hip_atomic_load(&slot->stage[threadIdx.x], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-#pragma unroll
-    for (int m = 32; m >= 1; m >>= 1) v += __shfl_xor(v, m, 64);
-    if ((threadIdx.x & 63) == 0) last_sums[threadIdx.x >> 6] = v;
-  }
-  __syncthreads();
+  const double v = threadIdx.x < kFoldGroups
+                       ? __hip_atomic_load(&slot->stage[threadIdx.x], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)
+                       : 0.0;
+  const double total = fold_stage(v);
   if (threadIdx.x == 0) {
-    *out = (last_sums[0] + last_sums[1]) + (last_sums[2] + last_sums[3]);
+    *out = total;
     __hip_atomic_store(&slot->ticket, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
   }
+}
+
+// The same sum with no stage outside the workgroup: one workgroup takes the 256 pieces one after the other and keeps
+// their sums in LDS.  Piece by piece and in the last step it adds what fold_onepass_kernel adds, in that order, so
+// a long fold gives the same bits whether or not it had a stage (a launch recorded into a graph, or a stream that
+// came when every slot was taken, has none).
+__global__ __launch_bounds__(1024) void fold_pieces_kernel(const float *__restrict__ partials, int64_t count,
+                                                           int64_t piece, double *__restrict__ out) {
+  __shared__ double stage[kFoldGroups];
+  for (int g = 0; g < kFoldGroups; ++g) {
+    const int64_t lo = static_cast<int64_t>(g) * piece;
+    const int64_t len = lo >= count ? 0 : (count - lo < piece ? count - lo : piece);
+    const double t = fold_block(partials + lo, len);
+    if (threadIdx.x == 0) stage[g] = t;
+    __syncthreads();   // fold_block's own LDS is free again, stage[g] is written
+  }
+  const double total = fold_stage(threadIdx.x < kFoldGroups ? stage[threadIdx.x] : 0.0);
+  if (threadIdx.x == 0) *out = total;
 }
 
 // Per-256-element-block kernels: out[j] = reduction of in[256j .. 256j+255].  A wave takes
@@ -661,12 +686,16 @@ constexpr int64_t kFoldOnePassFrom = int64_t{1} << 17;
 
 int launch_fold(const float *partials, int64_t count, double *sum_out, hipStream_t st) {
   // a launch recorded into a graph may be replayed on any stream, next to anything: it gets no shared stage
-  FoldSlot *slot = count < kFoldOnePassFrom || capturing(st) ? nullptr : fold_slot_for(st);
-  if (!slot) {
+  if (count < kFoldOnePassFrom) {
     hipLaunchKernelGGL(fold_kernel, dim3(1), dim3(1024), 0, st, partials, count, sum_out);
     return check_launch("fold kernel launch");
   }
   const int64_t piece = ceil_div(ceil_div(count, kFoldGroups), 4) * 4;
+  FoldSlot *slot = capturing(st) ? nullptr : fold_slot_for(st);
+  if (!slot) {
+    hipLaunchKernelGGL(fold_pieces_kernel, dim3(1), dim3(1024), 0, st, partials, count, piece, sum_out);
+    return check_launch("fold kernel launch");
+  }
   hipLaunchKernelGGL(fold_onepass_kernel, dim3(kFoldGroups), dim3(1024), 0, st, partials, count, piece, slot, sum_out);
   return check_launch("fold kernel launch");
 }

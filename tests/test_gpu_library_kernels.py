@@ -473,9 +473,10 @@ def test_long_folds_on_many_streams_do_not_meet(hip, torch_cuda):
 
 
 def test_a_long_fold_recorded_into_a_graph_keeps_no_shared_state(hip, torch_cuda):
-    """A fold of 2^20 partials recorded under stream capture takes the one-workgroup kernel (a graph may be replayed
+    """A fold of 2^20 partials recorded under stream capture takes a one-workgroup kernel (a graph may be replayed
     on any stream, next to anything, so it gets no stage of the library's): four replays with eager long folds on the
-    same stream and new data between them, each checked against numpy's double sum of what the vector held then."""
+    same stream and new data between them, each checked against numpy's double sum of what the vector held then, and
+    against the eager fold bit for bit -- the one workgroup adds piece by piece what the 256 add."""
     torch = torch_cuda
     n = 1 << 20
     rng = np.random.default_rng(11)
@@ -497,6 +498,7 @@ def test_a_long_fold_recorded_into_a_graph_keeps_no_shared_state(hip, torch_cuda
         torch.cuda.synchronize()
         assert abs(out.item() - want) <= 1e-12 * want, replay
         assert abs(eager.item() - want) <= 1e-12 * want, replay
+        assert out.item() == eager.item(), replay
 
 
 def test_tiled_matmul_through_run_vectors_at_1024(hip, oracle, sarek):
