@@ -143,6 +143,15 @@ std::string print_stmt(const StmtP &s);
 // ir_hip.cpp: IR -> HIP C++ for gfx950
 std::string gen_expr(const ExprP &e);
 std::string gen_stmt(const StmtP &s, const std::string &indent);
+// For statements printed on their own (the body of a function some other text declares): the names that function
+// already holds -- its parameters and locals -- so that a binding of one of them in the statements gets a name of
+// its own, as inside generate().
+struct FunctionScope {
+  explicit FunctionScope(const std::vector<std::string> &names);
+  ~FunctionScope();
+  FunctionScope(const FunctionScope &) = delete;
+  FunctionScope &operator=(const FunctionScope &) = delete;
+};
 // records + variants + helpers + kernel.  `block` (may be null): the launch block, when the
 // caller knows it; sizes of shared arrays written in terms of the block dimensions
 // (`let%shared tile = ()` lowers to block_dim_x elements, sarek/ppx/Sarek_lower_ir.ml:496-507)

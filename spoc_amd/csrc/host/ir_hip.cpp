@@ -12,9 +12,12 @@
 // HIP-specific spellings: `__syncwarp()` does not exist for AMD targets, a wave-level
 // barrier is `__builtin_amdgcn_wave_barrier()`; the source is compiled by hiprtc, which
 // pre-includes the HIP device runtime, so no #include lines are emitted.
+#include <algorithm>
 #include <cmath>
 #include <cstdio>
 #include <cstring>
+#include <memory>
+#include <utility>
 
 #include "ir.hpp"
 
@@ -29,6 +32,79 @@ thread_local const Kernel *t_kernel = nullptr;
 // declaration to compile, so the known value is written instead.
 thread_local int t_block[3] = {0, 0, 0};
 thread_local bool t_in_shared_size = false;
+
+// Names and C scopes.  The reference prints a let as `type name = value;` followed by its body in the same C block
+// (sarek-cuda/Sarek_ir_cuda.ml:437-578), so a kernel that binds a name again -- `let x = f x in ...`, ordinary OCaml --
+// comes out as a redefinition (or, in an inner block, as `int x = (x + 1);`, whose right-hand side is the new,
+// uninitialised x) and does not compile there.  Here a binding whose name is already declared in an open C block of
+// the function, or is one of its parameters, is printed under a name of its own (x_2, x_3, ...) for the length of its
+// body; the value is printed first, with the outer meaning of the name.  A kernel without such a binding -- every
+// golden text -- comes out as the reference prints it.
+struct Rename {
+  std::string name;
+  int id;   // the binding's id in the IR, -1 where the IR gives none (a pattern's variables)
+  std::string printed;
+};
+thread_local std::vector<std::vector<std::string>> t_c_blocks;   // declared names per open C block
+thread_local std::vector<Rename> t_renames;                      // innermost binding last
+
+bool name_declared(const std::string &n) {
+  for (const auto &block : t_c_blocks)
+    for (const auto &d : block)
+      if (d == n) return true;
+  return false;
+}
+
+// What a use of the name prints: the binding of that name and id (the front end numbers every binding, so a use
+// carries the id of the binding it means, sarek/ppx/Sarek_lower_ir.ml:237); where no binding in force has the id --
+// an array use, which carries a name alone, or IR written by hand -- the innermost binding of the name.
+const std::string &printed_name(const std::string &n, int id = -1) {
+  if (id >= 0)
+    for (auto it = t_renames.rbegin(); it != t_renames.rend(); ++it)
+      if (it->id == id && it->name == n) return it->printed;
+  for (auto it = t_renames.rbegin(); it != t_renames.rend(); ++it)
+    if (it->name == n) return it->printed;
+  return n;
+}
+const std::string &printed_name(const Var &v) { return printed_name(v.name, v.id); }
+
+struct CBlock {   // an opening brace of the generated text
+  size_t renames;
+  CBlock() : renames(t_renames.size()) { t_c_blocks.emplace_back(); }
+  ~CBlock() {
+    t_c_blocks.pop_back();
+    t_renames.erase(t_renames.begin() + static_cast<std::ptrdiff_t>(std::min(renames, t_renames.size())), t_renames.end());
+  }
+};
+
+struct Binding {  // a declaration in the current C block; its name means the new variable while this object lives
+  std::string printed;
+  size_t at = 0;
+  bool pushed = false;
+  explicit Binding(const Var &v) : Binding(v.name, v.id) {}
+  explicit Binding(const std::string &name, int id = -1) : printed(name) {
+    if (t_c_blocks.empty()) return;   // a statement printed outside any function: nothing to compare with
+    if (name_declared(name)) {
+      int k = 2;
+      do printed = name + "_" + std::to_string(k++);
+      while (name_declared(printed));
+    }
+    t_c_blocks.back().push_back(printed);
+    // the name stands for this variable in the body even when it is printed as it is: an outer rename of the same
+    // name must not reach into it
+    at = t_renames.size();
+    t_renames.push_back({name, id, printed});
+    pushed = true;
+  }
+  // A let without a body, in sequence with what uses it (a module's constant in front of the kernel function,
+  // sarek/ppx/Sarek_lower_ir.ml:634-671): the name keeps this meaning until the C block closes.
+  void keep() { pushed = false; }
+  ~Binding() {
+    if (pushed && at < t_renames.size()) t_renames.erase(t_renames.begin() + static_cast<std::ptrdiff_t>(at), t_renames.end());
+  }
+  Binding(const Binding &) = delete;
+  Binding &operator=(const Binding &) = delete;
+};
 
 std::string mangle(const std::string &name) {
   std::string o = name;
@@ -206,8 +282,8 @@ std::string fmt17(double v) {
 
 std::string gen_lvalue(const LValueP &l) {
   switch (l->kind) {
-    case LValue::LVar: return l->var.name;
-    case LValue::LArrayElem: return l->name + "[" + gen_expr(l->index) + "]";
+    case LValue::LVar: return printed_name(l->var);
+    case LValue::LArrayElem: return printed_name(l->name) + "[" + gen_expr(l->index) + "]";
     case LValue::LArrayElemExpr: return "(" + gen_expr(l->base) + ")[" + gen_expr(l->index) + "]";
     case LValue::LRecordField: return gen_lvalue(l->inner) + "." + l->name;
   }
@@ -229,15 +305,22 @@ std::string gen_match_case(const std::string &indent, const std::string &scrutin
     o += "  default: {\n";
   } else {
     o += "  case " + p.constr + ": {\n";
+  }
+  CBlock braces;
+  std::vector<std::unique_ptr<Binding>> bound;
+  if (!p.wildcard) {
     const std::vector<TypeP> *types = constructor_types(p.constr);
     if (!p.vars.empty() && types && !types->empty()) {
       if (p.vars.size() == 1 && types->size() == 1) {
-        o += indent + "    " + type_str((*types)[0]) + " " + p.vars[0] + " = " + scrutinee + ".data." +
+        bound.push_back(std::make_unique<Binding>(p.vars[0]));
+        o += indent + "    " + type_str((*types)[0]) + " " + bound.back()->printed + " = " + scrutinee + ".data." +
              p.constr + "_v;\n";
       } else if (p.vars.size() == types->size()) {
-        for (size_t i = 0; i < p.vars.size(); ++i)
-          o += indent + "    " + type_str((*types)[i]) + " " + p.vars[i] + " = " + scrutinee +
+        for (size_t i = 0; i < p.vars.size(); ++i) {
+          bound.push_back(std::make_unique<Binding>(p.vars[i]));
+          o += indent + "    " + type_str((*types)[i]) + " " + bound.back()->printed + " = " + scrutinee +
                ".data." + p.constr + "_v._" + std::to_string(i) + ";\n";
+        }
       } else {
         throw CodegenError("HIP codegen: pattern '" + p.constr + "' binds " +
                            std::to_string(p.vars.size()) + " variables, constructor has " +
@@ -247,6 +330,7 @@ std::string gen_match_case(const std::string &indent, const std::string &scrutin
   }
   o += gen_stmt(body, indent + "    ");
   o += indent + "    break;\n" + indent + "  }\n";
+  while (!bound.empty()) bound.pop_back();   // innermost first
   return o;
 }
 
@@ -274,6 +358,11 @@ std::string gen_helper(const HelperFunc &f) {
   std::string o = "__device__ " + type_str(f.ret) + " " + f.name + "(";
   for (size_t i = 0; i < f.params.size(); ++i)
     o += (i ? ", " : "") + type_str(f.params[i].type) + " " + f.params[i].name;
+  CBlock function;
+  for (const auto &p : f.params) {
+    t_c_blocks.back().push_back(p.name);
+    t_renames.push_back({p.name, p.id, p.name});
+  }
   o += ") {\n" + gen_stmt(f.body, "  ") + "}\n\n";
   return o;
 }
@@ -341,7 +430,7 @@ std::string gen_expr(const ExprP &ep) {
     case Expr::ConstFloat64: return fmt17(e.fval);
     case Expr::ConstBool: return e.ival ? "1" : "0";
     case Expr::ConstUnit: return "(void)0";
-    case Expr::VarRef: return e.var.name;
+    case Expr::VarRef: return printed_name(e.var);
     case Expr::BinopE: return "(" + gen_expr(e.args[0]) + binop_str(e.binop) + gen_expr(e.args[1]) + ")";
     case Expr::UnopE: {
       // As the reference prints it, "(" op operand ")" -- except that the minus of a negation keeps a space from an
@@ -352,7 +441,7 @@ std::string gen_expr(const ExprP &ep) {
                          : e.unop == Unop::Not ? "!" : "~";
       return std::string("(") + sign + operand + ")";
     }
-    case Expr::ArrayRead: return e.name + "[" + gen_expr(e.args[0]) + "]";
+    case Expr::ArrayRead: return printed_name(e.name) + "[" + gen_expr(e.args[0]) + "]";
     case Expr::ArrayReadExpr: return "(" + gen_expr(e.args[0]) + ")[" + gen_expr(e.args[1]) + "]";
     case Expr::RecordField: return gen_expr(e.args[0]) + "." + e.name;
     case Expr::Intrinsic: return gen_intrinsic(e);
@@ -414,18 +503,33 @@ std::string gen_stmt(const StmtP &sp, const std::string &indent) {
       }
       return indent + gen_lvalue(s.lhs) + " = " + gen_expr(s.e) + ";\n";
     case Stmt::If: {
-      std::string o = indent + "if (" + gen_expr(s.e) + ") {\n" + gen_stmt(s.stmts[0], in2) + indent + "}";
-      if (s.stmts.size() > 1) o += " else {\n" + gen_stmt(s.stmts[1], in2) + indent + "}\n";
-      else o += "\n";
+      std::string o = indent + "if (" + gen_expr(s.e) + ") {\n";
+      {
+        CBlock braces;
+        o += gen_stmt(s.stmts[0], in2) + indent + "}";
+      }
+      if (s.stmts.size() > 1) {
+        CBlock braces;
+        o += " else {\n" + gen_stmt(s.stmts[1], in2) + indent + "}\n";
+      } else {
+        o += "\n";
+      }
       return o;
     }
-    case Stmt::While:
-      return indent + "while (" + gen_expr(s.e) + ") {\n" + gen_stmt(s.stmts[0], in2) + indent + "}\n";
+    case Stmt::While: {
+      const std::string cond = gen_expr(s.e);
+      CBlock braces;
+      return indent + "while (" + cond + ") {\n" + gen_stmt(s.stmts[0], in2) + indent + "}\n";
+    }
     case Stmt::For: {
       const char *op = s.downto ? ">=" : "<=";
       const char *inc = s.downto ? "--" : "++";
-      return indent + "for (" + type_str(s.var.type) + " " + s.var.name + " = " + gen_expr(s.e) + "; " +
-             s.var.name + " " + op + " " + gen_expr(s.e2) + "; " + s.var.name + inc + ") {\n" +
+      const std::string from = gen_expr(s.e), to = gen_expr(s.e2);   // both with the outer meaning of the name
+      CBlock scope;                                                  // the statement's own scope holds the counter
+      Binding counter(s.var);
+      CBlock braces;
+      return indent + "for (" + type_str(s.var.type) + " " + counter.printed + " = " + from + "; " +
+             counter.printed + " " + op + " " + to + "; " + counter.printed + inc + ") {\n" +
              gen_stmt(s.stmts[0], in2) + indent + "}\n";
     }
     case Stmt::Match: {
@@ -456,24 +560,45 @@ std::string gen_stmt(const StmtP &sp, const std::string &indent) {
           throw;
         }
         t_in_shared_size = false;
+        Binding array(s.var);
         return indent + (s.e->mem == MemSpace::Shared ? "__shared__ " : "") + type_str(s.e->type) + " " +
-               s.var.name + "[" + size + "];\n" + gen_stmt(s.stmts[0], indent);
+               array.printed + "[" + size + "];\n" + gen_stmt(s.stmts[0], indent);
       }
-      return indent + type_str(s.var.type) + " " + s.var.name + " = " + gen_expr(s.e) + ";\n" +
-             gen_stmt(s.stmts[0], indent);
+      {
+        const std::string value = gen_expr(s.e);   // before the name changes its meaning
+        Binding bound(s.var);
+        if (s.stmts[0]->kind == Stmt::Empty) bound.keep();
+        return indent + type_str(s.var.type) + " " + bound.printed + " = " + value + ";\n" +
+               gen_stmt(s.stmts[0], indent);
+      }
     case Stmt::Pragma: {
       std::string o = indent + "#pragma ";
       for (size_t i = 0; i < s.hints.size(); ++i) o += (i ? " " : "") + s.hints[i];
       return o + "\n" + gen_stmt(s.stmts[0], indent);
     }
-    case Stmt::Block: return indent + "{\n" + gen_stmt(s.stmts[0], in2) + indent + "}\n";
+    case Stmt::Block: {
+      CBlock braces;
+      return indent + "{\n" + gen_stmt(s.stmts[0], in2) + indent + "}\n";
+    }
   }
   return "";
+}
+
+FunctionScope::FunctionScope(const std::vector<std::string> &names) {
+  t_c_blocks.clear();
+  t_renames.clear();
+  t_c_blocks.push_back(names);
+}
+FunctionScope::~FunctionScope() {
+  t_c_blocks.clear();
+  t_renames.clear();
 }
 
 std::string generate(const Kernel &k, const int block[3]) {
   for (int i = 0; i < 3; ++i) t_block[i] = block ? block[i] : 0;
   t_kernel = &k;
+  t_c_blocks.clear();
+  t_renames.clear();
   std::string o = "\nextern \"C\" {\n";
   try {
     // Type definitions: the variants, then the records, each in the order the kernel lists them (the reference's
@@ -534,7 +659,17 @@ std::string generate(const Kernel &k, const int block[3]) {
     o += "__global__ void " + k.name + "(";
     for (size_t i = 0; i < k.params.size(); ++i) o += (i ? ", " : "") + gen_param(k.params[i]);
     o += ") {\n";
-    for (const auto &l : k.locals) o += gen_local(l, "  ");
+    CBlock function;
+    for (const auto &d : k.params) {
+      t_c_blocks.back().push_back(d.var.name);
+      t_c_blocks.back().push_back("sarek_" + d.var.name + "_length");
+      t_renames.push_back({d.var.name, d.var.id, d.var.name});
+    }
+    for (const auto &l : k.locals) {
+      o += gen_local(l, "  ");
+      t_c_blocks.back().push_back(l.kind == Decl::Shared ? l.name : l.var.name);
+      if (l.kind != Decl::Shared) t_renames.push_back({l.var.name, l.var.id, l.var.name});
+    }
     o += gen_stmt(k.body, "  ");
     o += "}\n}\n";
   } catch (...) {

@@ -42,6 +42,14 @@ bool is_global_id(const ExprP &e) {
 // Names the rebuilt texts use themselves: everything of their own carries the prefix sarek_f_ (the loop variables of
 // the kernel bodies included), the element variables the suffix __e.  A parameter spelled like that would be shadowed
 // there, so such a kernel stays with the generated code; any other name, however short, is the kernel's to use.
+// What sarek_f_apply declares before the kernel's own statements: the inputs' element values, the scalars, the
+// element's index and the result.
+std::vector<std::string> element_function_names(const MapKernel &m) {
+  std::vector<std::string> names{m.tid, "sarek_f_res"};
+  for (const auto &p : m.params) names.push_back(p.kind == MapKernel::Param::Vec ? p.name + "__e" : p.name);
+  return names;
+}
+
 bool name_is_free(const std::string &n) {
   return n.compare(0, 8, "sarek_f_") != 0 && !(n.size() > 3 && n.compare(n.size() - 3, 3, "__e") == 0);
 }
@@ -126,7 +134,11 @@ struct Matcher {
         return body(s->stmts[0]);
       case Stmt::Let: {
         if (s->var.is_mutable || !s->e || s->e->kind == Expr::ArrayCreate || !pure(s->e)) return std::nullopt;
-        if (s->var.name == m.tid || param_index(s->var.name) >= 0 || s->var.name.compare(0, 8, "sarek_f_") == 0)
+        // A let may take a scalar parameter's name (the lowering gives the new variable a name of its own); one that
+        // hides the index or a vector would change what the reads and the store mean.
+        const int hidden = param_index(s->var.name);
+        if (s->var.name == m.tid || !name_is_free(s->var.name) ||
+            (hidden >= 0 && m.params[hidden].kind == MapKernel::Param::Vec))
           return std::nullopt;
         if (s->stmts.size() != 1) return std::nullopt;
         bound.push_back(s->var.name);
@@ -193,7 +205,7 @@ std::optional<MapKernel> match_map(const Kernel &k) {
   if (s->kind != Stmt::Let || s->var.is_mutable || !is_global_id(s->e) || s->stmts.size() != 1) return std::nullopt;
   if (!s->var.type || s->var.type->kind != Type::Int32) return std::nullopt;
   m.tid = s->var.name;
-  if (mt.param_index(m.tid) >= 0 || m.tid.compare(0, 8, "sarek_f_") == 0) return std::nullopt;
+  if (mt.param_index(m.tid) >= 0 || !name_is_free(m.tid)) return std::nullopt;
   const Stmt *guard = s->stmts[0].get();
   while ((guard->kind == Stmt::Block || guard->kind == Stmt::Seq) && guard->stmts.size() == 1)
     guard = guard->stmts[0].get();
@@ -213,6 +225,7 @@ std::optional<MapKernel> match_map(const Kernel &k) {
   if (!rewritten) return std::nullopt;
   std::sort(m.inputs.begin(), m.inputs.end());
   if (m.inputs.size() > 6) return std::nullopt;   // registers: four 128-bit loads per input and thread
+  FunctionScope element_function(element_function_names(m));
   m.body = gen_stmt(*rewritten, "  ");
   return m;
 }
@@ -433,7 +446,7 @@ std::optional<MapKernel> match_tree(const Kernel &k, bool is_max) {
   m.tid = l2->var.name;
   m.n = mt.param_index(c.args[1]->var.name);
   if (m.n < 0 || m.params[m.n].kind != MapKernel::Param::I32) return std::nullopt;
-  if (mt.param_index(m.tid) >= 0 || m.tid.compare(0, 8, "sarek_f_") == 0) return std::nullopt;
+  if (mt.param_index(m.tid) >= 0 || !name_is_free(m.tid)) return std::nullopt;
   // the expression first (it names the inputs), then the output: the one vector it does not read
   m.out = -1;
   if (!mt.pure(store->e)) return std::nullopt;
@@ -491,6 +504,7 @@ std::optional<MapKernel> match_tree(const Kernel &k, bool is_max) {
   st->kind = Stmt::Assign;
   st->lhs = lhs;
   st->e = mt.rewrite(store->e);
+  FunctionScope element_function(element_function_names(m));
   m.body = gen_stmt(StmtP(st), "  ");
   return m;
 }

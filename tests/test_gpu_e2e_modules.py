@@ -393,3 +393,22 @@ def test_the_two_smallest_kernels(hip, torch_cuda):
         Transfer.flush()
         assert path == "map_f32"
         assert np.array_equal(out.to_array(), want)
+
+
+def test_names_bound_again_mean_what_ocaml_says(hip, torch_cuda):
+    """`let x = 1 in let x = x + 1 in ...`, two sibling lets of one name, a let named like a parameter, a loop counter
+    named like a visible let: each run by one thread, the vector then holds what OCaml's scoping gives.  The bodies
+    and expected values are those the lowering tests pin the text of."""
+    from test_ir_lowering import REBOUND, REBOUND_PARAMS, kernel_with_body
+    from spoc_amd.sarek import Execute, Transfer, Vector
+    for name, (body, _, want) in REBOUND.items():
+        v = Vector.of_array(np.full(8, -1, np.int32))
+        path = Execute.run_vectors(ir=kernel_with_body(body, REBOUND_PARAMS), args=[Execute.Vec(v), Execute.Int32(3)],
+                                   block=Execute.dims1d(1), grid=Execute.dims1d(1))
+        Transfer.flush()
+        assert path == "jit", name
+        expected = np.full(8, -1, np.int32)
+        for at, value in want.items():
+            expected[at] = value
+        assert np.array_equal(v.to_array(), expected), name
+

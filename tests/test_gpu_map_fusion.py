@@ -147,6 +147,51 @@ def test_seeded_random_maps_alone_and_in_front_of_the_sum(hip, sarek, seed):
         assert bool((same | (np.isnan(fused_sums) & np.isnan(hand_sums))).all()), (seed, n)
 
 
+def test_a_map_that_binds_a_name_again(hip, sarek):
+    """out[i] = let t = x[i] * a in let t = t + x[i] in let a = t * t in a - b: lets that reuse a name and then a
+    parameter's, which the lowering prints as t_2 and a_2.  Rebuilt or generated, alone or compiled into the block
+    sums' kernel, the map writes the bits of the expression evaluated in OCaml's scoping."""
+    E, V = sarek.Execute, sarek.Vector
+    n = 4096 + 37
+    nblocks = (n + 255) // 256
+    tid = "(var tid 9 i32)"
+    xi = f"(read x {tid})"
+    body = (f"(let (var t 10 f32) (mul {xi} (var a 3 f32)) (let (var t 11 f32) (add (var t 10 f32) {xi}) "
+            f"(let (var a 12 f32) (mul (var t 11 f32) (var t 11 f32)) "
+            f"(assign (lelem out {tid}) (sub (var a 12 f32) (var b 4 f32))))))")
+    ir = ("(kernel sarek_kern (params (param (var x 1 (vec f32))) (param (var out 2 (vec f32))) (param (var a 3 f32)) "
+          f"(param (var b 4 f32)) (param (var n 5 i32))) (locals) (body (let {tid} (intr (Std) global_thread_id) "
+          f"(if (lt {tid} (var n 5 i32)) {body}))) (native_fn true))")
+    text = hip.generate_source(ir)
+    assert "float t_2 = (t + x[tid]);" in text and "float a_2 = (t_2 * t_2);" in text
+    reduction = open(os.path.join(IR_DIR, "reduction.ir")).read()
+    x = np.random.default_rng(5).standard_normal(n).astype(np.float32)
+    a, b = np.float32(1.25), np.float32(-0.375)
+    t2 = x * a + x
+    want = t2 * t2 - b
+    shape = ((256, 1, 1), (nblocks, 1, 1))
+
+    def run(pipeline):
+        out = V.create(V.float32, n)
+        out.host[:] = np.nan
+        args = [E.Vec(V.of_array(x)), E.Vec(out), E.Float32(a), E.Float32(b), E.Int32(n)]
+        if not pipeline:
+            return E.run_vectors(ir, args, *shape), out.to_array().copy()
+        sums = V.create(V.float32, nblocks)
+        path = E.run_pipeline([(ir, args) + shape, (reduction, [E.Vec(out), E.Vec(sums), E.Int32(n)]) + shape])
+        fused_sums = sums.to_array().copy()
+        E.run_vectors(reduction, [E.Vec(out), E.Vec(sums), E.Int32(n)], *shape)
+        return path, out.to_array().copy(), fused_sums, sums.to_array().copy()
+
+    (p_map, got), (p_jit, generated) = both_ways(hip, lambda: run(False))
+    assert (p_map, p_jit) == ("map_f32", "jit")
+    assert np.array_equal(got, want) and np.array_equal(generated, want)
+    hip.check(hip.lib.sarek_hip_set_specialisation(1))
+    path, fused, fused_sums, hand_sums = run(True)
+    assert path == ("map_f32+reduce_sum_block256_f32", 1)
+    assert np.array_equal(fused, want) and np.array_equal(fused_sums, hand_sums)
+
+
 @pytest.mark.parametrize("maximum", [False, True])
 @pytest.mark.parametrize("seed", range(int(os.environ.get("SAREK_HIP_TEST_MAP_SEEDS", "32")) // 2))
 def test_seeded_random_trees(hip, sarek, torch_cuda, seed, maximum):

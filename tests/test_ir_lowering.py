@@ -651,3 +651,83 @@ def test_random_expressions_lower_to_text_the_device_compiler_takes(hip, tmp_pat
     done = subprocess.run([hipcc, "--offload-arch=gfx950", "--cuda-device-only", "-fsyntax-only", "-w", str(path)],
                           capture_output=True, text=True, timeout=300)
     assert done.returncode == 0, done.stderr[-3000:]
+
+
+REBOUND = {
+    # name: (body, the text it lowers to, what v holds after one thread has run it, from OCaml's scoping)
+    "nested": ("(let (var x 1 i32) (i32 1) (let (var x 2 i32) (add (var x 1 i32) (i32 1)) "
+               "(assign (lelem v (i32 0)) (var x 2 i32))))",
+               "  int x = 1;\n  int x_2 = (x + 1);\n  v[0] = x_2;\n", {0: 2}),
+    "siblings": ("(seq (let (var x 1 i32) (i32 1) (assign (lelem v (i32 0)) (var x 1 i32))) "
+                 "(let (var x 2 i32) (i32 2) (assign (lelem v (i32 1)) (var x 2 i32))))",
+                 "  int x = 1;\n  v[0] = x;\n  int x_2 = 2;\n  v[1] = x_2;\n", {0: 1, 1: 2}),
+    "a parameter": ("(let (var n 5 i32) (add (var n 2 i32) (i32 1)) (assign (lelem v (i32 0)) (var n 5 i32)))",
+                    "  int n_2 = (n + 1);\n  v[0] = n_2;\n", {0: 4}),
+    "a loop counter": ("(let (var i 1 i32) (i32 2) (seq (for (var i 2 i32 mut) (i32 0) (var i 1 i32) upto "
+                       "(assign (lelem v (var i 2 i32)) (add (var i 2 i32) (i32 10)))) "
+                       "(assign (lelem v (i32 3)) (var i 1 i32))))",
+                       "  int i = 2;\n  for (int i_2 = 0; i_2 <= i; i_2++) {\n    v[i_2] = (i_2 + 10);\n  }\n  v[3] = i;\n",
+                       {0: 10, 1: 11, 2: 12, 3: 2}),
+    "inside a branch": ("(let (var x 1 i32) (i32 1) (seq (if (bool true) (let (var x 2 i32) (mul (var x 1 i32) (i32 3)) "
+                        "(assign (lelem v (i32 0)) (var x 2 i32)))) (assign (lelem v (i32 1)) (var x 1 i32))))",
+                        "  int x = 1;\n  if (1) {\n    int x_2 = (x * 3);\n    v[0] = x_2;\n  }\n  v[1] = x;\n", {0: 3, 1: 1}),
+    "three deep": ("(let (var x 1 i32) (i32 1) (let (var x 2 i32) (add (var x 1 i32) (i32 1)) (let (var x 3 i32) "
+                   "(add (var x 2 i32) (i32 1)) (assign (lelem v (i32 0)) (var x 3 i32)))))",
+                   "  int x = 1;\n  int x_2 = (x + 1);\n  int x_3 = (x_2 + 1);\n  v[0] = x_3;\n", {0: 3}),
+    "a name already of that form": ("(let (var x_2 1 i32) (i32 5) (let (var x 2 i32) (i32 1) (let (var x 3 i32) "
+                                    "(add (var x 2 i32) (var x_2 1 i32)) (assign (lelem v (i32 0)) (var x 3 i32)))))",
+                                    "  int x_2 = 5;\n  int x = 1;\n  int x_3 = (x + x_2);\n  v[0] = x_3;\n", {0: 6}),
+    # a let without a body in sequence with what follows is how a module's constant reaches the kernel
+    # (Sarek_lower_ir.ml:634-671); the use's id says which binding it means
+    "a constant named like a parameter": ("(seq (let (var n 7 i32) (i32 9) (empty)) (assign (lelem v (i32 0)) (var n 2 i32)))",
+                                          "  int n_2 = 9;\n  v[0] = n;\n", {0: 3}),
+    "two constants of one name": ("(seq (let (var s 7 i32) (i32 1) (empty)) (let (var s 8 i32) (i32 2) (empty)) "
+                                  "(assign (lelem v (i32 0)) (var s 8 i32)))",
+                                  "  int s = 1;\n  int s_2 = 2;\n  v[0] = s_2;\n", {0: 2}),
+}
+REBOUND_PARAMS = "(param (var v 1 (vec i32))) (param (var n 2 i32))"
+
+
+@pytest.mark.parametrize("name", REBOUND)
+def test_a_name_bound_again_gets_a_variable_of_its_own(hip, name):
+    """OCaml lets a kernel bind a name again (`let x = 1 in let x = x + 1 in ...`), and the IR keeps the source's
+    names (sarek/ppx/Sarek_lower_ir.ml:237 prints `v.var_name`).  Printed as they are, `int x = 1; int x = (x + 1);`
+    is a redefinition in one C block and reads its own uninitialised self in a nested one, so the reference's text for
+    such a kernel (Sarek_ir_cuda.ml:367-376, the same names) does not compile or computes something else.  Here the
+    value is printed with the outer meaning and the new variable is called x_2, x_3, ... for the length of its body;
+    a kernel that binds no name twice comes out as before (the golden texts above)."""
+    body, text, _ = REBOUND[name]
+    assert body_text(hip, body, REBOUND_PARAMS) == text
+
+
+def test_rebound_names_in_helpers_and_match_cases(hip):
+    ir = """
+    (kernel k (params (param (var out 1 (vec f32))) (param (var r 2 f32)))
+      (locals)
+      (body (match (var s 3 (variant shape (Circle f32) (Rect f32 f32)))
+              (case (Circle r) (assign (lelem out (i32 0)) (add (var r 4 f32) (var r 4 f32))))
+              (case (Rect r h) (let (var h 7 f32) (mul (var r 5 f32) (var h 6 f32)) (assign (lelem out (i32 1)) (var h 7 f32))))))
+      (variants (shape (Circle f32) (Rect f32 f32)))
+      (funcs (func sq (params (var a 8 f32)) f32 (let (var a 9 f32) (mul (var a 8 f32) (var a 8 f32)) (return (var a 9 f32)))))
+      (native_fn false))"""
+    src = hip.generate_source(ir)
+    assert "__device__ float sq(float a) {\n  float a_2 = (a * a);\n  return a_2;\n}" in src
+    assert "float r_2 = s.data.Circle_v;" in src and "out[0] = (r_2 + r_2);" in src
+    assert "float r_2 = s.data.Rect_v._0;" in src and "float h = s.data.Rect_v._1;" in src
+    assert "float h_2 = (r_2 * h);" in src and "out[1] = h_2;" in src
+
+
+def test_rebound_names_parse_as_device_code(hip, tmp_path):
+    import shutil
+    import subprocess
+    hipcc = shutil.which("hipcc") or "/opt/rocm/bin/hipcc"
+    if not os.path.exists(hipcc):
+        pytest.skip("no hipcc to parse the text with")
+    texts = ["#include <hip/hip_runtime.h>\n"]
+    for k, (body, _, _) in enumerate(REBOUND.values()):
+        texts.append(hip.generate_source(kernel_with_body(body, REBOUND_PARAMS)).replace("sarek_kern", f"rebound_{k}"))
+    path = tmp_path / "rebound.hip"
+    path.write_text("\n".join(texts))
+    done = subprocess.run([hipcc, "--offload-arch=gfx950", "--cuda-device-only", "-fsyntax-only", "-Wall", "-Werror=uninitialized",
+                           "-Wno-unused-variable", str(path)], capture_output=True, text=True, timeout=300)
+    assert done.returncode == 0, done.stderr[-3000:]

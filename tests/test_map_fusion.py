@@ -90,3 +90,36 @@ def test_rebuilt_source_refuses_everything_else(hip):
         assert err.value.status == hip.E_UNSUPPORTED
     with pytest.raises(hip.SarekHipError):
         hip.rebuilt_source(MAPS["scale"](), reduce=3)
+
+
+def _map_with_lets(lets, value, tid_name="tid"):
+    """out[tid] <- VALUE under the given (name, expression) lets, over x, scalars a and b, and n."""
+    tid = f"(var {tid_name} 9 i32)"
+    body = f"(assign (lelem out {tid}) {value})"
+    for k, (name, e) in reversed(list(enumerate(lets))):
+        body = f"(let (var {name} {20 + k} f32) {e} {body})"
+    return ("(kernel sarek_kern (params (param (var x 1 (vec f32))) (param (var out 2 (vec f32))) (param (var a 3 f32)) "
+            f"(param (var b 4 f32)) (param (var n 5 i32))) (locals) (body (let {tid} (intr (Std) global_thread_id) "
+            f"(if (lt {tid} (var n 5 i32)) {body}))) (native_fn true))")
+
+
+def test_lets_that_take_a_name_again_in_a_map(hip, tmp_path):
+    """A let may reuse a let's name or a scalar parameter's: the element function then holds the lowering's renamed
+    variables.  A let that would hide the element's index, a vector, or one of the rebuilt text's own names keeps the
+    kernel with the generated code."""
+    xi, a = "(read x (var tid 9 i32))", "(var a 3 f32)"
+    ir = _map_with_lets([("t", f"(mul {xi} {a})"), ("t", f"(add (var t 20 f32) {xi})"), ("a", "(mul (var t 21 f32) (var t 21 f32))")],
+                        "(sub (var a 22 f32) (var b 4 f32))")
+    assert hip.generate_source(ir).startswith(MARK + "map_f32\n")
+    text = hip.rebuilt_source(ir, 1, 0)
+    assert ("  float t = (x__e * a);\n  float t_2 = (t + x__e);\n  float a_2 = (t_2 * t_2);\n"
+            "  sarek_f_res = (a_2 - b);\n") in text
+    _compiles_for_gfx950(tmp_path, "rebound", text)
+    for lets, value, tid_name in (
+            ([("tid", "(f32 1.0)")], xi, "tid"),                       # out[tid] would mean another element
+            ([("x", "(f32 1.0)")], "(var x 20 f32)", "tid"),           # hides the input vector
+            ([("out", "(f32 1.0)")], xi, "tid"),                       # hides the output vector
+            ([("x__e", "(f32 1.0)")], f"(add {xi} (var x__e 20 f32))", "tid"),
+            ([("sarek_f_res", "(f32 1.0)")], xi, "tid"),
+            ([], "(read x (var x__e 9 i32))", "x__e")):
+        assert not hip.generate_source(_map_with_lets(lets, value, tid_name)).startswith(MARK), lets
