@@ -44,6 +44,7 @@ struct Rename {
   std::string name;
   int id;   // the binding's id in the IR, -1 where the IR gives none (a pattern's variables)
   std::string printed;
+  bool is_mutable;   // a loop's own counter is not: only its loop changes it, between turns
 };
 thread_local std::vector<std::vector<std::string>> t_c_blocks;   // declared names per open C block
 thread_local std::vector<Rename> t_renames;                      // innermost binding last
@@ -58,13 +59,17 @@ bool name_declared(const std::string &n) {
 // What a use of the name prints: the binding of that name and id (the front end numbers every binding, so a use
 // carries the id of the binding it means, sarek/ppx/Sarek_lower_ir.ml:237); where no binding in force has the id --
 // an array use, which carries a name alone, or IR written by hand -- the innermost binding of the name.
-const std::string &printed_name(const std::string &n, int id = -1) {
+const Rename *binding_of(const std::string &n, int id) {
   if (id >= 0)
     for (auto it = t_renames.rbegin(); it != t_renames.rend(); ++it)
-      if (it->id == id && it->name == n) return it->printed;
+      if (it->id == id && it->name == n) return &*it;
   for (auto it = t_renames.rbegin(); it != t_renames.rend(); ++it)
-    if (it->name == n) return it->printed;
-  return n;
+    if (it->name == n) return &*it;
+  return nullptr;
+}
+const std::string &printed_name(const std::string &n, int id = -1) {
+  const Rename *b = binding_of(n, id);
+  return b ? b->printed : n;
 }
 const std::string &printed_name(const Var &v) { return printed_name(v.name, v.id); }
 
@@ -81,8 +86,8 @@ struct Binding {  // a declaration in the current C block; its name means the ne
   std::string printed;
   size_t at = 0;
   bool pushed = false;
-  explicit Binding(const Var &v) : Binding(v.name, v.id) {}
-  explicit Binding(const std::string &name, int id = -1) : printed(name) {
+  explicit Binding(const Var &v, bool is_mutable = false) : Binding(v.name, v.id, is_mutable || v.is_mutable) {}
+  explicit Binding(const std::string &name, int id = -1, bool is_mutable = false) : printed(name) {
     if (t_c_blocks.empty()) return;   // a statement printed outside any function: nothing to compare with
     if (name_declared(name)) {
       int k = 2;
@@ -93,7 +98,7 @@ struct Binding {  // a declaration in the current C block; its name means the ne
     // the name stands for this variable in the body even when it is printed as it is: an outer rename of the same
     // name must not reach into it
     at = t_renames.size();
-    t_renames.push_back({name, id, printed});
+    t_renames.push_back({name, id, printed, is_mutable});
     pushed = true;
   }
   // A let without a body, in sequence with what uses it (a module's constant in front of the kernel function,
@@ -361,7 +366,7 @@ std::string gen_helper(const HelperFunc &f) {
   CBlock function;
   for (const auto &p : f.params) {
     t_c_blocks.back().push_back(p.name);
-    t_renames.push_back({p.name, p.id, p.name});
+    t_renames.push_back({p.name, p.id, p.name, p.is_mutable});
   }
   o += ") {\n" + gen_stmt(f.body, "  ") + "}\n\n";
   return o;
@@ -484,6 +489,30 @@ std::string gen_expr(const ExprP &ep) {
   return "";
 }
 
+// Whether nothing a loop's body does can change the expression's value: constants, immutable variables, the thread's
+// indices and operators over those.
+bool fixed_during_a_loop(const ExprP &ep) {
+  if (!ep) return true;
+  const Expr &e = *ep;
+  switch (e.kind) {
+    case Expr::ConstInt32: case Expr::ConstInt64: case Expr::ConstFloat32: case Expr::ConstFloat64:
+    case Expr::ConstBool: case Expr::ConstUnit: case Expr::ArrayLen:
+      return true;
+    case Expr::VarRef: {
+      const Rename *b = binding_of(e.var.name, e.var.id);
+      return b ? !b->is_mutable : !e.var.is_mutable;
+    }
+    case Expr::Intrinsic:
+      if (!e.args.empty() || !thread_intrinsic(e.name)) return false;
+      return true;
+    case Expr::BinopE: case Expr::UnopE: case Expr::Cast: case Expr::If: case Expr::RecordField:
+      for (const auto &a : e.args)
+        if (!fixed_during_a_loop(a)) return false;
+      return true;
+    default: return false;
+  }
+}
+
 std::string gen_stmt(const StmtP &sp, const std::string &indent) {
   const Stmt &s = *sp;
   const std::string in2 = indent + "  ";
@@ -526,10 +555,21 @@ std::string gen_stmt(const StmtP &sp, const std::string &indent) {
       const char *inc = s.downto ? "--" : "++";
       const std::string from = gen_expr(s.e), to = gen_expr(s.e2);   // both with the outer meaning of the name
       CBlock scope;                                                  // the statement's own scope holds the counter
-      Binding counter(s.var);
+      Binding counter(s.var.name, s.var.id, false);
+      // A bound that the body cannot change is printed in the condition, as the reference prints every bound
+      // (Sarek_ir_cuda.ml:391-409).  One that reads a mutable variable, memory or a call would be evaluated again
+      // in front of every turn there, where OCaml, the Native backend's loop and the reference's own walker
+      // (Sarek_ir_interp.ml:858-872) evaluate it once: it is kept in a variable of the statement's scope.
+      std::string stop = to, keep;
+      std::unique_ptr<Binding> kept;
+      if (!fixed_during_a_loop(s.e2)) {
+        kept = std::make_unique<Binding>("sarek_to_" + counter.printed);
+        stop = kept->printed;
+        keep = ", " + stop + " = " + to;
+      }
       CBlock braces;
-      return indent + "for (" + type_str(s.var.type) + " " + counter.printed + " = " + from + "; " +
-             counter.printed + " " + op + " " + to + "; " + counter.printed + inc + ") {\n" +
+      return indent + "for (" + type_str(s.var.type) + " " + counter.printed + " = " + from + keep + "; " +
+             counter.printed + " " + op + " " + stop + "; " + counter.printed + inc + ") {\n" +
              gen_stmt(s.stmts[0], in2) + indent + "}\n";
     }
     case Stmt::Match: {
@@ -566,7 +606,7 @@ std::string gen_stmt(const StmtP &sp, const std::string &indent) {
       }
       {
         const std::string value = gen_expr(s.e);   // before the name changes its meaning
-        Binding bound(s.var);
+        Binding bound(s.var, s.kind == Stmt::LetMut);
         if (s.stmts[0]->kind == Stmt::Empty) bound.keep();
         return indent + type_str(s.var.type) + " " + bound.printed + " = " + value + ";\n" +
                gen_stmt(s.stmts[0], indent);
@@ -663,12 +703,12 @@ std::string generate(const Kernel &k, const int block[3]) {
     for (const auto &d : k.params) {
       t_c_blocks.back().push_back(d.var.name);
       t_c_blocks.back().push_back("sarek_" + d.var.name + "_length");
-      t_renames.push_back({d.var.name, d.var.id, d.var.name});
+      t_renames.push_back({d.var.name, d.var.id, d.var.name, d.var.is_mutable});
     }
     for (const auto &l : k.locals) {
       o += gen_local(l, "  ");
       t_c_blocks.back().push_back(l.kind == Decl::Shared ? l.name : l.var.name);
-      if (l.kind != Decl::Shared) t_renames.push_back({l.var.name, l.var.id, l.var.name});
+      if (l.kind != Decl::Shared) t_renames.push_back({l.var.name, l.var.id, l.var.name, true});
     }
     o += gen_stmt(k.body, "  ");
     o += "}\n}\n";

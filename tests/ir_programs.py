@@ -1,0 +1,342 @@
+"""Seeded integer programs in the IR, and what one thread of them computes.
+
+`evaluate` walks the IR text the way the reference's own walker does (sarek/sarek/Sarek_ir_interp.ml: variables by
+binding id, then by name :76-91; Int32 operators :171-266 -- `shr` on non-negative operands only, where filling with
+zeros and with the sign agree; statements :844-941 -- a `for` evaluates both bounds once and is inclusive :858-872).
+It is a model for tests, over the integer subset the generator below emits: no floats, no records, no barriers, one
+thread at a time (the programs touch no memory another thread writes).
+
+`random_program(seed)` builds a kernel over (x : int32 vector, out : int32 vector, k : int32, n : int32) in which
+thread tid < n computes with lets, mutable variables, assignments, `if` statements and expressions, `for` loops in
+both directions (bounds that read mutable variables the body changes among them), counted `while` loops and blocks, and
+stores into out[tid * SLOTS + j].  Names come from a small pool, parameters' names included, so bindings hide each
+other all the time; every use carries the id of the binding OCaml's scoping gives it.  A program in which an int32
+operation would overflow (undefined in the generated C) is not returned: the next candidate of the seed is."""
+import random
+
+SLOTS = 4
+INT_MIN, INT_MAX = -(1 << 31), (1 << 31) - 1
+
+
+class Overflow(Exception):
+    pass
+
+
+def parse(text):
+    """IR text -> nested lists of atoms."""
+    tokens = text.replace("(", " ( ").replace(")", " ) ").split()
+    pos = 0
+
+    def node():
+        nonlocal pos
+        tok = tokens[pos]
+        pos += 1
+        if tok != "(":
+            return tok
+        items = []
+        while tokens[pos] != ")":
+            items.append(node())
+        pos += 1
+        return items
+
+    tree = node()
+    assert pos == len(tokens)
+    return tree
+
+
+def _fit(v):
+    if not INT_MIN <= v <= INT_MAX:
+        raise Overflow()
+    return v
+
+
+def _trunc_div(a, b):
+    q = abs(a) // abs(b)
+    return q if (a < 0) == (b < 0) else -q
+
+
+class Thread:
+    """One thread's state: bindings by id and by name (the innermost binding of a name is the last one made), the
+    vectors by name."""
+
+    def __init__(self, arrays, index):
+        self.by_id, self.by_name, self.arrays, self.index, self.steps = {}, {}, arrays, index, 0
+
+    def bind(self, var, value):
+        self.by_id[int(var[2])] = value
+        self.by_name[var[1]] = value
+
+    def lookup(self, var):
+        vid = int(var[2])
+        return self.by_id[vid] if vid in self.by_id else self.by_name[var[1]]
+
+    def expr(self, e):
+        head = e[0]
+        if head == "i32":
+            return int(e[1])
+        if head == "bool":
+            return e[1] == "true"
+        if head == "var":
+            return self.lookup(e)
+        if head == "read":
+            return int(self.arrays[e[1]][self.expr(e[2])])
+        if head == "intr":
+            assert e[2] in ("global_thread_id", "global_idx_x", "global_idx"), e
+            return self.index
+        if head == "if":
+            return self.expr(e[2]) if self.expr(e[1]) else self.expr(e[3])
+        if head == "neg":
+            return _fit(-self.expr(e[1]))
+        if head == "bitnot":
+            return ~self.expr(e[1])
+        if head == "not":
+            return not self.expr(e[1])
+        a, b = self.expr(e[1]), self.expr(e[2])
+        if head == "add": return _fit(a + b)
+        if head == "sub": return _fit(a - b)
+        if head == "mul": return _fit(a * b)
+        if head == "div": return _fit(_trunc_div(a, b))
+        if head == "mod": return a - b * _trunc_div(a, b)
+        if head == "bitand": return a & b
+        if head == "bitor": return a | b
+        if head == "bitxor": return a ^ b
+        if head == "shl":
+            assert 0 <= b < 32
+            return _fit(a << b)
+        if head == "shr":
+            assert a >= 0 and 0 <= b < 32
+            return a >> b
+        if head == "lt": return a < b
+        if head == "le": return a <= b
+        if head == "gt": return a > b
+        if head == "ge": return a >= b
+        if head == "eq": return a == b
+        if head == "ne": return a != b
+        if head == "and": return bool(a) and bool(b)
+        if head == "or": return bool(a) or bool(b)
+        raise KeyError(head)
+
+    def stmt(self, s):
+        head = s[0]
+        self.steps += 1
+        if self.steps > 2_000_000:
+            raise RuntimeError("the program does not end")
+        if head == "empty":
+            return
+        if head == "seq":
+            for c in s[1:]:
+                self.stmt(c)
+        elif head == "block":
+            self.stmt(s[1])
+        elif head in ("let", "letmut"):
+            self.bind(s[1], self.expr(s[2]))
+            self.stmt(s[3])
+        elif head == "assign":
+            value, target = self.expr(s[2]), s[1]
+            if target[0] == "lvar":
+                self.bind(target[1], value)
+            else:
+                assert target[0] == "lelem"
+                self.arrays[target[1]][self.expr(target[2])] = value
+        elif head == "if":
+            if self.expr(s[1]):
+                self.stmt(s[2])
+            elif len(s) > 3:
+                self.stmt(s[3])
+        elif head == "while":
+            while self.expr(s[1]):
+                self.stmt(s[2])
+        elif head == "for":
+            i, stop = self.expr(s[2]), self.expr(s[3])
+            step = 1 if s[4] == "upto" else -1
+            while (i <= stop) if step == 1 else (i >= stop):
+                self.bind(s[1], i)
+                self.stmt(s[5])
+                i += step
+        else:
+            raise KeyError(head)
+
+
+def evaluate(ir, arrays, threads):
+    """Runs threads 0 .. threads-1 of the kernel's body, one after the other, on `arrays` (name -> numpy int32
+    array, changed in place) and the scalar arguments given in `arrays` under their names."""
+    kernel = parse(ir)
+    sections = {item[0]: item for item in kernel[2:] if isinstance(item, list)}
+    params = [p[1] for p in sections["params"][1:]]
+    body = sections["body"][1]
+    vectors = {p[1]: arrays[p[1]] for p in params if isinstance(p[3], list)}
+    for index in range(threads):
+        t = Thread(vectors, index)
+        for p in params:
+            if not isinstance(p[3], list):
+                t.bind(p, int(arrays[p[1]]))
+        t.stmt(body)
+
+
+class _Builder:
+    POOL = ["a", "b", "c", "k", "i", "j"]          # k is a parameter's name too
+
+    def __init__(self, rng):
+        self.rng, self.next_id = rng, 10
+        # name -> (id, mutable) of the binding in force; the parameters first
+        self.scope = {"x": (1, False), "out": (2, False), "k": (3, False), "n": (4, False), "tid": (5, False)}
+        self.vectors = {"x", "out"}
+        self.counters = set()      # ids of loop counters: mutable in the IR, assigned by their loop alone
+
+    def var(self, name, vid, mutable):
+        return f"(var {name} {vid} i32{' mut' if mutable else ''})"
+
+    def use(self, name):
+        vid, mutable = self.scope[name]
+        return self.var(name, vid, mutable)
+
+    def ints_in_scope(self):
+        return [n for n in self.scope if n not in self.vectors]
+
+    def small(self, e, bits=7):
+        return f"(bitand {e} (i32 {(1 << bits) - 1}))"
+
+    def expr(self, depth):
+        r = self.rng
+        if depth == 0:
+            pick = r.randint(0, 5)
+            if pick == 0:
+                return f"(i32 {r.randint(-9, 12)})"
+            if pick == 1:
+                return f"(read x {self.use('tid')})"
+            return self.use(r.choice(self.ints_in_scope()))
+        a, b = self.expr(depth - 1), self.expr(depth - 1)
+        pick = r.randint(0, 9)
+        if pick == 0:
+            return f"({r.choice(['add', 'sub'])} {a} {b})"
+        if pick == 1:
+            return f"(mul {self.small(a, 5)} {self.small(b, 5)})"
+        if pick == 2:
+            return f"({r.choice(['bitand', 'bitor', 'bitxor'])} {a} {b})"
+        if pick == 3:
+            return f"(shl {self.small(a, 10)} (i32 {r.randint(0, 5)}))"
+        if pick == 4:
+            return f"(shr {self.small(a, 15)} (i32 {r.randint(0, 5)}))"
+        if pick == 5:
+            return f"(neg {a})"
+        if pick == 6:
+            return f"(bitnot {a})"
+        if pick == 7:
+            return f"(if {self.cond(0)} {a} {b})"
+        if pick == 8:
+            return f"({r.choice(['div', 'mod'])} {a} (add {self.small(b, 3)} (i32 1)))"
+        return f"(sub {a} {b})"
+
+    def cond(self, depth):
+        r = self.rng
+        if depth > 0 and r.random() < 0.4:
+            pick = r.randint(0, 2)
+            if pick == 0:
+                return f"(not {self.cond(depth - 1)})"
+            return f"({'and' if pick == 1 else 'or'} {self.cond(depth - 1)} {self.cond(depth - 1)})"
+        return f"({r.choice(['lt', 'le', 'gt', 'ge', 'eq', 'ne'])} {self.expr(1)} {self.expr(1)})"
+
+    def bound_body(self, name, mutable, make_body, counter=False):
+        """Text of a binding's declaration and the body built with the name meaning the new variable."""
+        vid = self.next_id
+        self.next_id += 1
+        if counter:
+            self.counters.add(vid)
+        hidden = self.scope.get(name)
+        self.scope[name] = (vid, mutable)
+        body = make_body()
+        if hidden is None:
+            del self.scope[name]
+        else:
+            self.scope[name] = hidden
+        return self.var(name, vid, mutable), body
+
+    def store(self):
+        slot = self.rng.randrange(SLOTS)
+        return f"(assign (lelem out (add (mul {self.use('tid')} (i32 {SLOTS})) (i32 {slot}))) {self.expr(self.rng.randint(0, 2))})"
+
+    def stmts(self, depth, count):
+        return "(seq " + " ".join(self.stmt(depth) for _ in range(count)) + ")" if count != 1 else self.stmt(depth)
+
+    def stmt(self, depth):
+        r = self.rng
+        mutables = [n for n, (vid, m) in self.scope.items() if m and vid not in self.counters]
+        if depth == 0:
+            if mutables and r.random() < 0.5:
+                return f"(assign (lvar {self.use(r.choice(mutables))}) {self.expr(r.randint(0, 2))})"
+            return self.store()
+        pick = r.randint(0, 9)
+        if pick in (0, 1):                                   # let NAME = e in S (the value reads the outer NAME)
+            value = self.expr(r.randint(0, 2))
+            v, body = self.bound_body(r.choice(self.POOL), False, lambda: self.stmts(depth - 1, r.randint(1, 3)))
+            return f"(let {v} {value} {body})"
+        if pick in (2, 3):
+            value = self.expr(r.randint(0, 2))
+            v, body = self.bound_body(r.choice(self.POOL), True, lambda: self.stmts(depth - 1, r.randint(1, 3)))
+            return f"(letmut {v} {value} {body})"
+        if pick == 4:
+            other = f" {self.stmts(depth - 1, r.randint(1, 2))}" if r.random() < 0.6 else ""
+            return f"(if {self.cond(1)} {self.stmts(depth - 1, r.randint(1, 2))}{other})"
+        if pick in (5, 6):                                   # for NAME = lo to / downto hi
+            lo, hi = self.small(self.expr(1), 2), self.small(self.expr(1), 3)
+            down = r.random() < 0.4
+            moving = r.choice(mutables) if mutables and r.random() < 0.5 else None
+            if moving:                                       # the far bound reads what the body goes on to change
+                bound = self.small(self.use(moving), 3)
+                lo, hi = (bound, hi) if down else (lo, bound)
+            first, last = (hi, lo) if down else (lo, hi)
+            counter = r.choice(self.POOL)
+
+            def turns():
+                body = self.stmts(depth - 1, r.randint(1, 2))
+                if moving and self.scope.get(moving, (None, False))[1] and counter != moving:
+                    slot = f"(add (mul {self.use('tid')} (i32 {SLOTS})) (i32 {r.randrange(SLOTS)}))"
+                    body = (f"(seq {body} (assign (lelem out {slot}) (add {self.use(counter)} {self.use(moving)})) "
+                            f"(assign (lvar {self.use(moving)}) {self.expr(1)}))")
+                return body
+            # the counter is declared mutable in the IR (Sarek_lower_ir.ml:476-484) though no kernel assigns it
+            v, body = self.bound_body(counter, True, turns, counter=True)
+            return f"(for {v} {first} {last} {'downto' if down else 'upto'} {body})"
+        if pick == 7:                                        # let lim = e in letmut turn = 0 in while turn < lim do S; turn++
+            limit = self.small(self.expr(1), 3)
+
+            def counter():
+                def loop():
+                    turn = self.use("turn")
+                    inner = self.stmts(depth - 1, r.randint(1, 2))
+                    return (f"(while (lt {turn} {self.use('lim')}) (seq {inner} "
+                            f"(assign (lvar {turn}) (add {turn} (i32 1)))))")
+                v, body = self.bound_body("turn", True, loop, counter=True)
+                return f"(letmut {v} (i32 0) {body})"
+            lim, body = self.bound_body("lim", False, counter)
+            return f"(let {lim} {limit} {body})"
+        if pick == 8:
+            return f"(block {self.stmts(depth - 1, r.randint(1, 3))})"
+        return self.store()
+
+
+def random_program(seed, threads=24):
+    """(ir, x, k): a program of the seed in which no thread overflows; out is to be SLOTS * threads elements."""
+    import numpy as np
+    for attempt in range(200):
+        rng = random.Random(seed * 1000 + attempt)
+        b = _Builder(rng)
+        body = b.stmts(rng.randint(2, 4), rng.randint(2, 4))
+        ir = ("(kernel sarek_kern (params (param (var x 1 (vec i32))) (param (var out 2 (vec i32))) "
+              "(param (var k 3 i32)) (param (var n 4 i32))) (locals) (body (let (var tid 5 i32) "
+              f"(intr (Std) global_thread_id) (if (lt (var tid 5 i32) (var n 4 i32)) {body}))) (native_fn true))")
+        x = np.array([rng.randint(-100, 100) for _ in range(threads)], np.int32)
+        k = rng.randint(-5, 9)
+        try:
+            expected(ir, x, k, threads)
+        except Overflow:
+            continue
+        return ir, x, k
+    raise RuntimeError(f"seed {seed}: no candidate without overflow")
+
+
+def expected(ir, x, k, threads):
+    import numpy as np
+    out = np.full(SLOTS * threads, -1, np.int32)
+    evaluate(ir, {"x": x.copy(), "out": out, "k": k, "n": threads}, threads)
+    return out

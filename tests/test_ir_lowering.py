@@ -731,3 +731,76 @@ def test_rebound_names_parse_as_device_code(hip, tmp_path):
     done = subprocess.run([hipcc, "--offload-arch=gfx950", "--cuda-device-only", "-fsyntax-only", "-Wall", "-Werror=uninitialized",
                            "-Wno-unused-variable", str(path)], capture_output=True, text=True, timeout=300)
     assert done.returncode == 0, done.stderr[-3000:]
+
+
+def test_the_program_model_on_known_cases(hip):
+    """The tests' walker of integer IR (ir_programs.evaluate) against the results the re-binding cases above fix by
+    hand, and against loops whose bounds the body changes: OCaml evaluates a `for`'s bounds once."""
+    import numpy as np
+    import ir_programs
+    for name, (body, _, want) in REBOUND.items():
+        v = np.full(8, -1, np.int32)
+        ir_programs.evaluate(kernel_with_body(body, REBOUND_PARAMS), {"v": v, "n": 3}, 1)
+        expected = np.full(8, -1, np.int32)
+        for at, value in want.items():
+            expected[at] = value
+        assert np.array_equal(v, expected), name
+    for name, (body, _, want) in LOOP_BOUNDS.items():
+        v = np.full(8, -1, np.int32)
+        ir_programs.evaluate(kernel_with_body(body, REBOUND_PARAMS), {"v": v, "n": 3}, 1)
+        assert v.tolist() == want, name
+
+
+M = "(var m 7 i32 mut)"
+LOOP_BOUNDS = {
+    # name: (body, lowered text, v after one thread with n = 3)
+    "a bound the body lowers": (
+        f"(letmut {M} (i32 5) (for (var i 8 i32 mut) (i32 0) {M} upto (seq (assign (lelem v (var i 8 i32 mut)) {M}) "
+        f"(assign (lvar {M}) (sub {M} (i32 1))))))",
+        "  int m = 5;\n  for (int i = 0, sarek_to_i = m; i <= sarek_to_i; i++) {\n    v[i] = m;\n    m = (m - 1);\n  }\n",
+        [5, 4, 3, 2, 1, 0, -1, -1]),
+    "downwards, to an element the body overwrites": (
+        "(seq (assign (lelem v (i32 7)) (i32 2)) (for (var i 8 i32 mut) (i32 5) (read v (i32 7)) downto "
+        "(seq (assign (lelem v (var i 8 i32 mut)) (i32 9)) (assign (lelem v (i32 7)) (i32 4)))))",
+        "  v[7] = 2;\n  for (int i = 5, sarek_to_i = v[7]; i >= sarek_to_i; i--) {\n    v[i] = 9;\n    v[7] = 4;\n  }\n",
+        [-1, -1, 9, 9, 9, 9, -1, 4]),
+    "fixed bounds stay in the condition": (
+        "(let (var a 9 i32) (i32 2) (for (var i 8 i32 mut) (var a 9 i32) (add (var n 2 i32) (var a 9 i32)) upto "
+        "(for (var j 10 i32 mut) (i32 0) (var i 8 i32 mut) upto (assign (lelem v (var j 10 i32 mut)) (var i 8 i32 mut)))))",
+        "  int a = 2;\n  for (int i = a; i <= (n + a); i++) {\n    for (int j = 0; j <= i; j++) {\n      v[j] = i;\n    }\n  }\n",
+        [5, 5, 5, 5, 5, 5, -1, -1]),
+}
+
+
+@pytest.mark.parametrize("name", LOOP_BOUNDS)
+def test_a_loop_bound_the_body_may_change_is_evaluated_once(hip, name):
+    """`for i = 0 to !m do ... m := !m - 1 done` runs to the value m had at the start in OCaml, on the Native backend
+    and in the reference's IR walker (Sarek_ir_interp.ml:858-872: stop_val is computed before the loop); the
+    reference's device text repeats the bound in the condition (Sarek_ir_cuda.ml:391-409), which evaluates it before
+    every turn.  Here such a bound is kept in a variable of the statement's scope; a bound of constants, immutable
+    variables, thread indices and loop counters is printed in the condition as before."""
+    body, text, _ = LOOP_BOUNDS[name]
+    assert body_text(hip, body, REBOUND_PARAMS) == text
+
+
+def test_seeded_integer_programs_parse_as_device_code(hip, tmp_path):
+    """120 seeded programs of lets, mutable variables, loops and branches whose names hide each other all the time
+    (ir_programs.random_program), lowered and handed to the device compiler's front end: no redefinition, no use of
+    a variable in its own initialiser."""
+    import shutil
+    import subprocess
+    import ir_programs
+    hipcc = shutil.which("hipcc") or "/opt/rocm/bin/hipcc"
+    if not os.path.exists(hipcc):
+        pytest.skip("no hipcc to parse the text with")
+    texts = ["#include <hip/hip_runtime.h>\n"]
+    for seed in range(120):
+        ir, _, _ = ir_programs.random_program(seed)
+        texts.append(hip.generate_source(ir).replace("sarek_kern", f"program_{seed}"))
+    path = tmp_path / "programs.hip"
+    path.write_text("\n".join(texts))
+    done = subprocess.run([hipcc, "--offload-arch=gfx950", "--cuda-device-only", "-fsyntax-only", "-Wall",
+                           "-Werror=uninitialized", "-Wno-unused-variable", "-Wno-unused-but-set-variable",
+                           "-Wno-self-assign", "-Wno-tautological-compare", "-Wno-parentheses-equality", str(path)],
+                          capture_output=True, text=True, timeout=600)
+    assert done.returncode == 0, done.stderr[-3000:]
