@@ -283,6 +283,33 @@ def random_map(seed):
     return kernel(params, let(tid, intr("global_thread_id", "Std"), if_(lt(tid, var("n")), body))), n_in
 
 
+def random_map_rebinding(seed):
+    """Like random_map, with two to five lets whose names come from (t, u, a): lets hide earlier lets of the same
+    name and the scalar parameter a, every binding under an id of its own, every use with the id of the binding
+    OCaml's scoping gives it.  Returns (ir, number of input vectors)."""
+    import random
+    rng = random.Random(77000 + seed)
+    n_in = rng.randint(1, 3)
+    params = [(f"x{i}", "(vec f32)") for i in range(n_in)] + [("out", "(vec f32)"), ("a", "f32"), ("b", "f32"),
+                                                               ("k", "i32"), ("n", "i32")]
+    _params(params)
+    tid = var("tid")
+    reads = [read(f"x{i}", tid) for i in range(n_in)]
+    in_force, bindings, scalars = {}, [], ("a", "b")
+    for j in range(rng.randint(2, 5)):
+        e = _random_expression(rng, reads, tid, scalars=scalars, lets_made=tuple(in_force.values()), depth=rng.randint(1, 2))
+        name = rng.choice(["t", "u", "a"])
+        v = f"(var {name} {100 + j} f32)"
+        bindings.append((v, e))
+        in_force[name] = v
+        if name == "a":
+            scalars = ("b",)
+    body = assign_elem("out", tid, _random_expression(rng, reads, tid, scalars=scalars, lets_made=tuple(in_force.values())))
+    for v, e in reversed(bindings):
+        body = let(v, e, body)
+    return kernel(params, let(tid, intr("global_thread_id", "Std"), if_(lt(tid, var("n")), body))), n_in
+
+
 def random_tree(seed, maximum=False):
     """The reference's block-256 sum (or maximum) tree with a seeded expression of one to three inputs, two f32
     scalars and an int scalar where it reads input[gid].  Returns (tree ir, map ir, number of inputs): the map

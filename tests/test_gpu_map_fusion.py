@@ -111,8 +111,19 @@ def test_seeded_random_maps_alone_and_in_front_of_the_sum(hip, sarek, seed):
     kernel writes the generated kernel's bits, alone and fused with the block sums, whose bits are the hand
     block-256 kernel's on that vector."""
     from map_kernels import random_map
+    _rebuilt_map_against_generated(hip, sarek, *random_map(seed), seed)
+
+
+@pytest.mark.parametrize("seed", range(int(os.environ.get("SAREK_HIP_TEST_MAP_SEEDS", "32")) // 2))
+def test_seeded_random_maps_whose_lets_hide_each_other(hip, sarek, seed):
+    """The same check for maps whose lets reuse names -- an earlier let's, the scalar parameter a's --, which the
+    lowering prints under names of their own in both texts."""
+    from map_kernels import random_map_rebinding
+    _rebuilt_map_against_generated(hip, sarek, *random_map_rebinding(seed), seed)
+
+
+def _rebuilt_map_against_generated(hip, sarek, ir, n_in, seed):
     E, V = sarek.Execute, sarek.Vector
-    ir, n_in = random_map(seed)
     reduction = open(os.path.join(IR_DIR, "reduction.ir")).read()
     for n in (4097, 100003):
         nblocks = (n + 255) // 256
