@@ -7,7 +7,8 @@ It is a model for tests, over the integer subset the generator below emits: no f
 thread at a time (the programs touch no memory another thread writes).
 
 `random_program(seed)` builds a kernel over (x : int32 vector, out : int32 vector, k : int32, n : int32) in which
-thread tid < n computes with lets, mutable variables, assignments, `if` statements and expressions, `for` loops in
+thread tid < n computes with lets, mutable variables, assignments, `if` statements and expressions, calls of up to
+two helper functions (their own lets, loops and branches, a return at every end), `for` loops in
 both directions (bounds that read mutable variables the body changes among them), counted `while` loops and blocks, and
 stores into out[tid * SLOTS + j].  Names come from a small pool, parameters' names included, so bindings hide each
 other all the time; every use carries the id of the binding OCaml's scoping gives it.  A program in which an int32
@@ -20,6 +21,11 @@ INT_MIN, INT_MAX = -(1 << 31), (1 << 31) - 1
 
 class Overflow(Exception):
     pass
+
+
+class _Return(Exception):
+    def __init__(self, value):
+        self.value = value
 
 
 def parse(text):
@@ -59,8 +65,9 @@ class Thread:
     """One thread's state: bindings by id and by name (the innermost binding of a name is the last one made), the
     vectors by name."""
 
-    def __init__(self, arrays, index):
+    def __init__(self, arrays, index, funcs=None):
         self.by_id, self.by_name, self.arrays, self.index, self.steps = {}, {}, arrays, index, 0
+        self.funcs = funcs or {}
 
     def bind(self, var, value):
         self.by_id[int(var[2])] = value
@@ -85,6 +92,18 @@ class Thread:
             return self.index
         if head == "if":
             return self.expr(e[2]) if self.expr(e[1]) else self.expr(e[3])
+        if head == "app":                                  # a helper: its own bindings, the value its return gives
+            params, body = self.funcs[e[1][1]]
+            callee = Thread(self.arrays, self.index, self.funcs)
+            for p, a in zip(params, [self.expr(a) for a in e[2:]]):
+                callee.bind(p, a)
+            try:
+                callee.stmt(body)
+            except _Return as r:
+                return r.value
+            finally:
+                self.steps += callee.steps
+            raise AssertionError("a helper ended without a return")
         if head == "neg":
             return _fit(-self.expr(e[1]))
         if head == "bitnot":
@@ -123,6 +142,8 @@ class Thread:
             raise RuntimeError("the program does not end")
         if head == "empty":
             return
+        if head == "return":
+            raise _Return(self.expr(s[1]))
         if head == "seq":
             for c in s[1:]:
                 self.stmt(c)
@@ -165,8 +186,9 @@ def evaluate(ir, arrays, threads):
     params = [p[1] for p in sections["params"][1:]]
     body = sections["body"][1]
     vectors = {p[1]: arrays[p[1]] for p in params if isinstance(p[3], list)}
+    funcs = {f[1]: (f[2][1:], f[4]) for f in sections.get("funcs", ["funcs"])[1:]}
     for index in range(threads):
-        t = Thread(vectors, index)
+        t = Thread(vectors, index, funcs)
         for p in params:
             if not isinstance(p[3], list):
                 t.bind(p, int(arrays[p[1]]))
@@ -182,6 +204,41 @@ class _Builder:
         self.scope = {"x": (1, False), "out": (2, False), "k": (3, False), "n": (4, False), "tid": (5, False)}
         self.vectors = {"x", "out"}
         self.counters = set()      # ids of loop counters: mutable in the IR, assigned by their loop alone
+        self.helpers = []          # (name, number of parameters) of the helper functions made so far
+        self.in_helper = False     # a helper sees its parameters alone: no vector, no thread index
+
+    def helper(self, name):
+        """Text of a helper function over one or two int32 parameters whose names come from the pool: lets and
+        mutable variables that hide them, loops, and a return at every end."""
+        r = self.rng
+        outer, self.scope, self.in_helper = self.scope, {}, True
+        params = []
+        for pname in r.sample(self.POOL, r.randint(1, 2)):
+            self.scope[pname] = (self.next_id, False)
+            params.append(self.var(pname, self.next_id, False))
+            self.next_id += 1
+        body = self.returning(r.randint(1, 3))
+        self.scope, self.in_helper = outer, False
+        self.helpers.append((name, len(params)))
+        return f"(func {name} (params {' '.join(params)}) i32 {body})"
+
+    def returning(self, depth):
+        r = self.rng
+        if depth == 0:
+            return f"(return {self.expr(r.randint(0, 2))})"
+        pick = r.randint(0, 3)
+        if pick == 0:
+            value = self.expr(r.randint(0, 2))
+            v, body = self.bound_body(r.choice(self.POOL), False, lambda: self.returning(depth - 1))
+            return f"(let {v} {value} {body})"
+        if pick == 1:
+            value = self.expr(r.randint(0, 2))
+            v, body = self.bound_body(r.choice(self.POOL), True,
+                                      lambda: f"(seq {self.stmts(min(depth, 2), r.randint(1, 2))} {self.returning(depth - 1)})")
+            return f"(letmut {v} {value} {body})"
+        if pick == 2:
+            return f"(if {self.cond(1)} {self.returning(depth - 1)} {self.returning(depth - 1)})"
+        return f"(return {self.expr(r.randint(0, 2))})"
 
     def var(self, name, vid, mutable):
         return f"(var {name} {vid} i32{' mut' if mutable else ''})"
@@ -202,9 +259,12 @@ class _Builder:
             pick = r.randint(0, 5)
             if pick == 0:
                 return f"(i32 {r.randint(-9, 12)})"
-            if pick == 1:
+            if pick == 1 and not self.in_helper:
                 return f"(read x {self.use('tid')})"
             return self.use(r.choice(self.ints_in_scope()))
+        if self.helpers and not self.in_helper and r.random() < 0.15:
+            name, arity = r.choice(self.helpers)
+            return f"(app (var {name} 0 i32) {' '.join(self.small(self.expr(depth - 1), 6) for _ in range(arity))})"
         a, b = self.expr(depth - 1), self.expr(depth - 1)
         pick = r.randint(0, 9)
         if pick == 0:
@@ -252,6 +312,11 @@ class _Builder:
         return self.var(name, vid, mutable), body
 
     def store(self):
+        if self.in_helper:                                  # no memory there: an assignment, or nothing
+            mutables = [n for n, (vid, m) in self.scope.items() if m and vid not in self.counters]
+            if not mutables:
+                return "(empty)"
+            return f"(assign (lvar {self.use(self.rng.choice(mutables))}) {self.expr(self.rng.randint(0, 2))})"
         slot = self.rng.randrange(SLOTS)
         return f"(assign (lelem out (add (mul {self.use('tid')} (i32 {SLOTS})) (i32 {slot}))) {self.expr(self.rng.randint(0, 2))})"
 
@@ -290,9 +355,11 @@ class _Builder:
             def turns():
                 body = self.stmts(depth - 1, r.randint(1, 2))
                 if moving and self.scope.get(moving, (None, False))[1] and counter != moving:
-                    slot = f"(add (mul {self.use('tid')} (i32 {SLOTS})) (i32 {r.randrange(SLOTS)}))"
-                    body = (f"(seq {body} (assign (lelem out {slot}) (add {self.use(counter)} {self.use(moving)})) "
-                            f"(assign (lvar {self.use(moving)}) {self.expr(1)}))")
+                    shown = ""
+                    if not self.in_helper:
+                        slot = f"(add (mul {self.use('tid')} (i32 {SLOTS})) (i32 {r.randrange(SLOTS)}))"
+                        shown = f"(assign (lelem out {slot}) (add {self.use(counter)} {self.use(moving)})) "
+                    body = f"(seq {body} {shown}(assign (lvar {self.use(moving)}) {self.expr(1)}))"
                 return body
             # the counter is declared mutable in the IR (Sarek_lower_ir.ml:476-484) though no kernel assigns it
             v, body = self.bound_body(counter, True, turns, counter=True)
@@ -321,10 +388,12 @@ def random_program(seed, threads=24):
     for attempt in range(200):
         rng = random.Random(seed * 1000 + attempt)
         b = _Builder(rng)
+        funcs = " ".join(b.helper(f"helper{h}") for h in range(rng.randint(0, 2)))
         body = b.stmts(rng.randint(2, 4), rng.randint(2, 4))
         ir = ("(kernel sarek_kern (params (param (var x 1 (vec i32))) (param (var out 2 (vec i32))) "
               "(param (var k 3 i32)) (param (var n 4 i32))) (locals) (body (let (var tid 5 i32) "
-              f"(intr (Std) global_thread_id) (if (lt (var tid 5 i32) (var n 4 i32)) {body}))) (native_fn true))")
+              f"(intr (Std) global_thread_id) (if (lt (var tid 5 i32) (var n 4 i32)) {body}))) "
+              f"(funcs {funcs}) (native_fn true))")
         x = np.array([rng.randint(-100, 100) for _ in range(threads)], np.int32)
         k = rng.randint(-5, 9)
         try:

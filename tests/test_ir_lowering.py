@@ -796,7 +796,8 @@ def test_seeded_integer_programs_parse_as_device_code(hip, tmp_path):
     texts = ["#include <hip/hip_runtime.h>\n"]
     for seed in range(120):
         ir, _, _ = ir_programs.random_program(seed)
-        texts.append(hip.generate_source(ir).replace("sarek_kern", f"program_{seed}"))
+        text = hip.generate_source(ir).replace("sarek_kern", f"program_{seed}")
+        texts.append(text.replace("helper0(", f"helper0_{seed}(").replace("helper1(", f"helper1_{seed}("))
     path = tmp_path / "programs.hip"
     path.write_text("\n".join(texts))
     done = subprocess.run([hipcc, "--offload-arch=gfx950", "--cuda-device-only", "-fsyntax-only", "-Wall",
