@@ -89,7 +89,7 @@ int compile_impl(const char *source, const char *kernel_name, sarek_hip_kernel *
     (void)hipRuntimeGetVersion(&runtime_version);
     cache_key = cache_compute_key(std::string(prop.name) + "|" + prop.gcnArchName,
                                   "hiprtc " + std::to_string(rtc_major) + "." + std::to_string(rtc_minor) +
-                                      " hip " + std::to_string(runtime_version) + " -O3 -packed-fp32-ops",
+                                      " hip " + std::to_string(runtime_version) + " -O3 -packed-fp32-ops -fwrapv",
                                   source);
     std::vector<char> cached;
     if (cache_get(cache_key, &cached) && !cached.empty()) {
@@ -114,7 +114,11 @@ int compile_impl(const char *source, const char *kernel_name, sarek_hip_kernel *
   if (r != HIPRTC_SUCCESS) return rtc_fail(r, "hiprtcCreateProgram");
   // Packed FP32 instructions are switched off for generated code as for the library's own kernels
   // (some of their forms have given wrong results on this hardware without any error).
-  const char *opts[] = {arch.c_str(), "-O3", "-std=c++17", "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"};
+  // -fwrapv: int32 / int64 arithmetic of a kernel wraps modulo 2^32 / 2^64 on the Native backend (OCaml's Int32 and
+  // Int64 are defined that way), so an overflow in the device text -- a hash, a linear congruential generator -- must
+  // not be something the optimiser may assume away.
+  const char *opts[] = {arch.c_str(), "-O3",    "-std=c++17",       "-fwrapv",
+                        "-Xclang",    "-target-feature", "-Xclang", "-packed-fp32-ops"};
   r = hiprtcCompileProgram(prog, static_cast<int>(sizeof(opts) / sizeof(opts[0])), opts);
   std::string build_log;
   size_t log_size = 0;

@@ -11,16 +11,12 @@ thread tid < n computes with lets, mutable variables, assignments, `if` statemen
 two helper functions (their own lets, loops and branches, a return at every end), `for` loops in
 both directions (bounds that read mutable variables the body changes among them), counted `while` loops and blocks, and
 stores into out[tid * SLOTS + j].  Names come from a small pool, parameters' names included, so bindings hide each
-other all the time; every use carries the id of the binding OCaml's scoping gives it.  A program in which an int32
-operation would overflow (undefined in the generated C) is not returned: the next candidate of the seed is."""
+other all the time; every use carries the id of the binding OCaml's scoping gives it.  Sums, products and negations
+overflow now and then (a linear congruential step is one of the expression forms): Int32 arithmetic wraps."""
 import random
 
 SLOTS = 4
 INT_MIN, INT_MAX = -(1 << 31), (1 << 31) - 1
-
-
-class Overflow(Exception):
-    pass
 
 
 class _Return(Exception):
@@ -51,9 +47,8 @@ def parse(text):
 
 
 def _fit(v):
-    if not INT_MIN <= v <= INT_MAX:
-        raise Overflow()
-    return v
+    """Int32 arithmetic is modulo 2^32 (OCaml's Int32; the device text is compiled with wrapping signed arithmetic)."""
+    return (v - INT_MIN) % (1 << 32) + INT_MIN
 
 
 def _trunc_div(a, b):
@@ -266,7 +261,11 @@ class _Builder:
             name, arity = r.choice(self.helpers)
             return f"(app (var {name} 0 i32) {' '.join(self.small(self.expr(depth - 1), 6) for _ in range(arity))})"
         a, b = self.expr(depth - 1), self.expr(depth - 1)
-        pick = r.randint(0, 9)
+        pick = r.randint(0, 11)
+        if pick == 10:                                       # a linear congruential step: overflows at once
+            return f"(add (mul {a} (i32 1103515245)) (i32 12345))"
+        if pick == 11:
+            return f"(mul {a} {b})"
         if pick == 0:
             return f"({r.choice(['add', 'sub'])} {a} {b})"
         if pick == 1:
@@ -383,25 +382,18 @@ class _Builder:
 
 
 def random_program(seed, threads=24):
-    """(ir, x, k): a program of the seed in which no thread overflows; out is to be SLOTS * threads elements."""
+    """(ir, x, k) of the seed; out is to be SLOTS * threads elements."""
     import numpy as np
-    for attempt in range(200):
-        rng = random.Random(seed * 1000 + attempt)
-        b = _Builder(rng)
-        funcs = " ".join(b.helper(f"helper{h}") for h in range(rng.randint(0, 2)))
-        body = b.stmts(rng.randint(2, 4), rng.randint(2, 4))
-        ir = ("(kernel sarek_kern (params (param (var x 1 (vec i32))) (param (var out 2 (vec i32))) "
-              "(param (var k 3 i32)) (param (var n 4 i32))) (locals) (body (let (var tid 5 i32) "
-              f"(intr (Std) global_thread_id) (if (lt (var tid 5 i32) (var n 4 i32)) {body}))) "
-              f"(funcs {funcs}) (native_fn true))")
-        x = np.array([rng.randint(-100, 100) for _ in range(threads)], np.int32)
-        k = rng.randint(-5, 9)
-        try:
-            expected(ir, x, k, threads)
-        except Overflow:
-            continue
-        return ir, x, k
-    raise RuntimeError(f"seed {seed}: no candidate without overflow")
+    rng = random.Random(seed * 1000)
+    b = _Builder(rng)
+    funcs = " ".join(b.helper(f"helper{h}") for h in range(rng.randint(0, 2)))
+    body = b.stmts(rng.randint(2, 4), rng.randint(2, 4))
+    ir = ("(kernel sarek_kern (params (param (var x 1 (vec i32))) (param (var out 2 (vec i32))) "
+          "(param (var k 3 i32)) (param (var n 4 i32))) (locals) (body (let (var tid 5 i32) "
+          f"(intr (Std) global_thread_id) (if (lt (var tid 5 i32) (var n 4 i32)) {body}))) "
+          f"(funcs {funcs}) (native_fn true))")
+    x = np.array([rng.randint(-100, 100) for _ in range(threads)], np.int32)
+    return ir, x, rng.randint(-5, 9)
 
 
 def expected(ir, x, k, threads):
