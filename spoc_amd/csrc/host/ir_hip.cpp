@@ -14,6 +14,7 @@
 // pre-includes the HIP device runtime, so no #include lines are emitted.
 #include <algorithm>
 #include <cmath>
+#include <cstdint>
 #include <cstdio>
 #include <cstring>
 #include <memory>
@@ -277,10 +278,16 @@ const char *binop_str(Binop op) {
   return s[static_cast<int>(op)];
 }
 
-std::string fmt17(double v) {
+// A floating constant: "%.17g" as the reference prints it (Sarek_ir_cuda.ml:83-89), which reads back as the same
+// double.  Infinities and NaN come out of that format as "inf" / "nan", no C at all: they are written as the
+// compiler's builtins, which need no header (the run-time compiler includes none that defines INFINITY or NAN).
+std::string fmt17(double v, bool single) {
   char buf[64];
-  if (std::isnan(v)) return "NAN";
-  if (std::isinf(v)) return v > 0 ? "INFINITY" : "(-INFINITY)";
+  if (std::isnan(v)) return single ? "__builtin_nanf(\"\")" : "__builtin_nan(\"\")";
+  if (std::isinf(v)) {
+    const char *inf = single ? "__builtin_inff()" : "__builtin_inf()";
+    return v > 0 ? inf : std::string("(-") + inf + ")";
+  }
   std::snprintf(buf, sizeof(buf), "%.17g", v);
   return buf;
 }
@@ -422,17 +429,29 @@ std::string gen_variant_def(const std::string &name,
 std::string gen_expr(const ExprP &ep) {
   const Expr &e = *ep;
   switch (e.kind) {
-    case Expr::ConstInt32: return std::to_string(static_cast<int32_t>(e.ival));
-    case Expr::ConstInt64: return std::to_string(e.ival) + "LL";
+    // The least value of a type has no literal of that type in C: 2147483648 is a long long and 9223372036854775808LL
+    // does not fit, so "-2147483648" would make the arithmetic around it 64-bit.
+    case Expr::ConstInt32:
+      if (static_cast<int32_t>(e.ival) == INT32_MIN) return "(-2147483647 - 1)";
+      return std::to_string(static_cast<int32_t>(e.ival));
+    case Expr::ConstInt64:
+      if (e.ival == INT64_MIN) return "(-9223372036854775807LL - 1)";
+      return std::to_string(e.ival) + "LL";
     case Expr::ConstFloat32: {
-      std::string s = fmt17(e.fval);
+      std::string s = fmt17(e.fval, true);
       if (std::isfinite(e.fval)) {
         if (s.find('.') == std::string::npos && s.find('e') == std::string::npos) s += ".0";
         s += "f";
       }
       return s;
     }
-    case Expr::ConstFloat64: return fmt17(e.fval);
+    case Expr::ConstFloat64: {
+      // The reference prints "%.17g" as it is (Sarek_ir_cuda.ml:90), so 2.0 comes out as `2`, an int in C: `1.0 /. 2.0`
+      // would be the integer division (1 / 2) and -0.0 the integer 0.  A whole value gets its decimal point here.
+      std::string s = fmt17(e.fval, false);
+      if (std::isfinite(e.fval) && s.find('.') == std::string::npos && s.find('e') == std::string::npos) s += ".0";
+      return s;
+    }
     case Expr::ConstBool: return e.ival ? "1" : "0";
     case Expr::ConstUnit: return "(void)0";
     case Expr::VarRef: return printed_name(e.var);

@@ -201,3 +201,53 @@ def test_ray_helpers_that_call_helpers(hip, torch_cuda):
                         np.stack([1 - tt + tt * 0.5, 1 - tt + tt * 0.7, np.ones(n)], axis=1))
     assert 0 < int((disc > 0).sum()) < n                        # both branches are taken
     assert np.all(np.abs(out.to_array().reshape(n, 3) - expected) <= 1e-3)
+
+
+def test_literals_at_the_edges_of_their_types(hip, torch_cuda):
+    """Constants a kernel may hold and the text must carry to the bit: infinities, a NaN, the signed zero, the
+    largest float and the smallest denormals of both float types, the ends of int32 and int64, and the negation of
+    each negative one (`(- -5LL)`, not a decrement).  One thread stores them; the host compares bit patterns."""
+    from spoc_amd.sarek import Execute, Transfer, Vector
+    f32s = ["inf", "-inf", "nan", "-0.0", "3.4028234663852886e+38", "1.401298464324817e-45", "-1.1754942106924411e-38",
+            "0.1", "16777217.0"]
+    f64s = ["inf", "-inf", "nan", "-0.0", "1.7976931348623157e+308", "5e-324", "0.1", "1e-320"]
+    i32s = [-2147483648, 2147483647, -1, 0]
+    i64s = [-9223372036854775808, 9223372036854775807, -5, 4294967301]
+    stores = []
+    for k, v in enumerate(f32s):
+        stores.append(f"(assign (lelem a (i32 {k})) (f32 {v}))")
+    stores.append(f"(assign (lelem a (i32 {len(f32s)})) (neg (f32 -2.5)))")
+    for k, v in enumerate(f64s):
+        stores.append(f"(assign (lelem b (i32 {k})) (f64 {v}))")
+    stores.append(f"(assign (lelem b (i32 {len(f64s)})) (neg (f64 -2.5)))")
+    stores.append(f"(assign (lelem b (i32 {len(f64s) + 1})) (div (f64 1.0) (f64 2.0)))")     # not the integer 1 / 2
+    stores.append(f"(assign (lelem c (i32 6)) (if (lt (sub (i32 -2147483648) (i32 1)) (i32 0)) (i32 1) (i32 2)))")
+    for k, v in enumerate(i32s):
+        stores.append(f"(assign (lelem c (i32 {k})) (i32 {v}))")
+    stores.append(f"(assign (lelem c (i32 {len(i32s)})) (neg (i32 -7)))")
+    for k, v in enumerate(i64s):
+        stores.append(f"(assign (lelem d (i32 {k})) (i64 {v}))")
+    stores.append(f"(assign (lelem d (i32 {len(i64s)})) (neg (i64 -5)))")
+    stores.append(f"(assign (lelem d (i32 {len(i64s) + 1})) (cast i64 (i32 -3)))")
+    stores.append(f"(assign (lelem c (i32 {len(i32s) + 1})) (cast i32 (i64 4294967301)))")
+    ir = ("(kernel sarek_kern (params (param (var a 1 (vec f32))) (param (var b 2 (vec f64))) (param (var c 3 (vec i32))) "
+          "(param (var d 4 (vec i64)))) (locals) (body (if (eq (intr (Std) global_thread_id) (i32 0)) "
+          f"(seq {' '.join(stores)}))) (native_fn true))")
+    a, b = Vector.create(Vector.float32, 16), Vector.create(Vector.float64, 16)
+    c, d = Vector.create(Vector.int32, 8), Vector.create(Vector.int64, 8)
+    path = Execute.run_vectors(ir=ir, args=[Execute.Vec(a), Execute.Vec(b), Execute.Vec(c), Execute.Vec(d)],
+                               block=Execute.dims1d(64), grid=Execute.dims1d(1))
+    Transfer.flush()
+    assert path == "jit"
+    want_a = np.array([float(v) for v in f32s] + [2.5], np.float32)
+    got_a = a.to_array()[:len(want_a)]
+    assert np.isnan(got_a[2]) and np.isnan(want_a[2])
+    keep = np.arange(len(want_a)) != 2
+    assert np.array_equal(got_a.view(np.uint32)[keep], want_a.view(np.uint32)[keep]), got_a
+    want_b = np.array([float(v) for v in f64s] + [2.5, 0.5], np.float64)
+    got_b = b.to_array()[:len(want_b)]
+    assert np.isnan(got_b[2])
+    assert np.array_equal(got_b.view(np.uint64)[keep[:len(want_b)]], want_b.view(np.uint64)[keep[:len(want_b)]]), got_b
+    # min_int - 1 wraps to max_int in int32 arithmetic (a `-2147483648` in the text would be a 64-bit operand)
+    assert c.to_array()[:len(i32s) + 3].tolist() == i32s + [7, 5, 2]
+    assert d.to_array()[:len(i64s) + 2].tolist() == i64s + [5, -3]

@@ -75,6 +75,18 @@ def test_literals(hip):
     assert expr_text(hip, "(f32 2.5)") == "2.5f"
     assert expr_text(hip, "(f32 0.1)") == "0.10000000000000001f"   # "%.17g" + f
     assert expr_text(hip, "(f32 1e30)") == "1e+30f"
+    # what "%.17g" prints as inf / nan (no C: the reference's text for such a constant does not compile) is written
+    # with builtins, which the run-time compiler knows without a header
+    assert expr_text(hip, "(f32 inf)") == "__builtin_inff()" and expr_text(hip, "(f64 -inf)") == "(-__builtin_inf())"
+    assert expr_text(hip, "(f32 nan)") == '__builtin_nanf("")' and expr_text(hip, "(f64 nan)") == '__builtin_nan("")'
+    # a whole-valued double keeps a decimal point: `2` is an int in C, (1 / 2) the integer division, -0 the integer 0
+    assert expr_text(hip, "(f64 2.0)") == "2.0" and expr_text(hip, "(f64 -0.0)") == "-0.0"
+    assert expr_text(hip, "(div (f64 1.0) (f64 2.0))") == "(1.0 / 2.0)" and expr_text(hip, "(f64 1e22)") == "1e+22"
+    # the least int32 / int64 have no literal of their own type
+    assert expr_text(hip, "(i32 -2147483648)") == "(-2147483647 - 1)"
+    assert expr_text(hip, "(i32 -2147483647)") == "-2147483647"
+    assert expr_text(hip, "(i64 -9223372036854775808)") == "(-9223372036854775807LL - 1)"
+    assert expr_text(hip, "(i64 9223372036854775807)") == "9223372036854775807LL"
 
 
 def test_operations(hip):
