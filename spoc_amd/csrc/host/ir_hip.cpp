@@ -493,16 +493,39 @@ std::string gen_expr(const ExprP &ep) {
     case Expr::If:
       return "(" + gen_expr(e.args[0]) + " ? " + gen_expr(e.args[1]) + " : " + gen_expr(e.args[2]) + ")";
     case Expr::Match: {
+      // Nested conditionals on the tag, as the reference prints them (Sarek_ir_cuda.ml:179-208).  There a case's
+      // variables stay undeclared (`match s with Circle r -> r *. r | ...` as a value does not compile); here each
+      // stands for the payload it names, `s.data.Circle_v`, for the length of its case.
       if (e.cases.empty()) throw CodegenError("HIP codegen: empty match expression");
-      if (e.cases.size() == 1) return gen_expr(e.cases[0].second);
+      const std::string scrutinee = gen_expr(e.args[0]);
+      auto value_of = [&](const Pattern &p, const ExprP &body) {
+        const size_t mark = t_renames.size();
+        const std::vector<TypeP> *types = p.wildcard || p.vars.empty() ? nullptr : constructor_types(p.constr);
+        if (types && types->size() == p.vars.size())
+          for (size_t i = 0; i < p.vars.size(); ++i)
+            t_renames.push_back({p.vars[i], -1,
+                                 scrutinee + ".data." + p.constr + "_v" +
+                                     (p.vars.size() == 1 ? std::string() : "._" + std::to_string(i)),
+                                 false});
+        std::string text;
+        try {
+          text = gen_expr(body);
+        } catch (...) {
+          t_renames.erase(t_renames.begin() + static_cast<std::ptrdiff_t>(mark), t_renames.end());
+          throw;
+        }
+        t_renames.erase(t_renames.begin() + static_cast<std::ptrdiff_t>(mark), t_renames.end());
+        return text;
+      };
+      if (e.cases.size() == 1) return value_of(e.cases[0].first, e.cases[0].second);
       std::string o, close;
       for (size_t i = 0; i + 1 < e.cases.size(); ++i) {
         const Pattern &p = e.cases[i].first;
-        o += "(" + (p.wildcard ? std::string("1") : "(" + gen_expr(e.args[0]) + ".tag == " + p.constr + ")") +
-             " ? " + gen_expr(e.cases[i].second) + " : ";
+        o += "(" + (p.wildcard ? std::string("1") : "(" + scrutinee + ".tag == " + p.constr + ")") + " ? " +
+             value_of(p, e.cases[i].second) + " : ";
         close += ")";
       }
-      return o + gen_expr(e.cases.back().second) + close;
+      return o + value_of(e.cases.back().first, e.cases.back().second) + close;
     }
   }
   return "";
@@ -622,6 +645,11 @@ std::string gen_stmt(const StmtP &sp, const std::string &indent) {
         Binding array(s.var);
         return indent + (s.e->mem == MemSpace::Shared ? "__shared__ " : "") + type_str(s.e->type) + " " +
                array.printed + "[" + size + "];\n" + gen_stmt(s.stmts[0], indent);
+      }
+      if (s.var.type && s.var.type->kind == Type::Unit) {
+        // `let () = e in body` (Sarek_lower_ir.ml:448-470 lowers it like any let): nothing to declare -- the
+        // reference's `void u = e;` does not compile --, the value is evaluated for what it does
+        return indent + gen_expr(s.e) + ";\n" + gen_stmt(s.stmts[0], indent);
       }
       {
         const std::string value = gen_expr(s.e);   // before the name changes its meaning

@@ -251,3 +251,19 @@ def test_literals_at_the_edges_of_their_types(hip, torch_cuda):
     # min_int - 1 wraps to max_int in int32 arithmetic (a `-2147483648` in the text would be a 64-bit operand)
     assert c.to_array()[:len(i32s) + 3].tolist() == i32s + [7, 5, 2]
     assert d.to_array()[:len(i64s) + 2].tolist() == i64s + [5, -3]
+
+
+def test_a_match_used_as_a_value(hip, torch_cuda):
+    """A variant built by nested `if`s and taken apart by a match in expression position, payload variables and all
+    (the kernel whose text tests/test_ir_lowering.py pins)."""
+    from test_ir_lowering import MATCH_AS_A_VALUE
+    from spoc_amd.sarek import Execute, Transfer, Vector
+    n = 1000
+    x = np.random.default_rng(2).uniform(-3, 3, n).astype(np.float32)
+    dst = Vector.create(Vector.float32, n)
+    path = Execute.run_vectors(ir=MATCH_AS_A_VALUE, args=[Execute.Vec(Vector.of_array(x)), Execute.Vec(dst), Execute.Int32(n)],
+                               block=Execute.dims1d(128), grid=Execute.dims1d((n + 127) // 128))
+    Transfer.flush()
+    assert path == "jit"
+    want = np.where(x > 1, x * x, np.where(x < -1, x * np.float32(2), x))
+    assert np.array_equal(dst.to_array(), want)

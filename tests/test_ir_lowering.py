@@ -123,6 +123,8 @@ def test_statements(hip):
     assert down == "  for (int i = 9; i >= 0; i--) {\n  }\n"
     assert body_text(hip, "(let (var x 1 i32) (i32 42) (empty))") == "  int x = 42;\n"
     assert "double y = 3.14" in body_text(hip, "(letmut (var y 1 f64 mut) (f64 3.14) (empty))")
+    # a let of type unit declares nothing (`void u = ...;` is no C): the value is evaluated for what it does
+    assert body_text(hip, "(let (var u 1 unit) (unit) (assign (lvar (var r 2 i32 mut)) (i32 1)))") == "  (void)0;\n  r = 1;\n"
     assert body_text(hip, "(block (empty))") == "  {\n  }\n"
     assert body_text(hip, "(pragma (unroll) (empty))") == "  #pragma unroll\n"
     assert body_text(hip, '(native "asm volatile(\\"\\");")') == '  asm volatile("");\n'
@@ -817,3 +819,25 @@ def test_seeded_integer_programs_parse_as_device_code(hip, tmp_path):
                            "-Wno-self-assign", "-Wno-tautological-compare", "-Wno-parentheses-equality", str(path)],
                           capture_output=True, text=True, timeout=600)
     assert done.returncode == 0, done.stderr[-3000:]
+
+
+SHAPE = "(variant shape (Circle f32) (Rect f32 f32) (Empty))"
+MATCH_AS_A_VALUE = f"""(kernel sarek_kern (params (param (var xs 1 (vec f32))) (param (var dst 2 (vec f32))) (param (var n 3 i32))) (locals)
+ (body (let (var tid 4 i32) (intr (Std) global_thread_id) (if (lt (var tid 4 i32) (var n 3 i32))
+   (let (var x 5 f32) (read xs (var tid 4 i32))
+   (let (var s 6 {SHAPE}) (if (gt (var x 5 f32) (f32 1.0)) (variant shape Circle (var x 5 f32))
+                             (if (lt (var x 5 f32) (f32 -1.0)) (variant shape Rect (var x 5 f32) (f32 2.0)) (variant shape Empty)))
+     (assign (lelem dst (var tid 4 i32))
+             (match (var s 6 {SHAPE}) (case (Circle x) (mul (var x 7 f32) (var x 7 f32)))
+                                      (case (Rect w h) (mul (var w 8 f32) (var h 9 f32)))
+                                      (case _ (var x 5 f32)))))))))
+ (variants (shape (Circle f32) (Rect f32 f32) (Empty))) (native_fn true))"""
+
+
+def test_a_match_used_as_a_value_binds_its_patterns(hip):
+    """`dst.(tid) <- (match s with Circle x -> x *. x | Rect (w, h) -> w *. h | _ -> x)`: nested conditionals on the
+    tag as the reference prints them (Sarek_ir_cuda.ml:179-208), with each case's variables standing for the payload
+    they name -- the reference leaves them undeclared.  The Circle case's x hides the let's x inside that case only."""
+    text = hip.generate_source(MATCH_AS_A_VALUE)
+    assert ("dst[tid] = ((s.tag == Circle) ? (s.data.Circle_v * s.data.Circle_v) : "
+            "((s.tag == Rect) ? (s.data.Rect_v._0 * s.data.Rect_v._1) : x));") in text
