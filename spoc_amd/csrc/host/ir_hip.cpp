@@ -201,6 +201,26 @@ const char *stdlib_template(const std::vector<std::string> &path, const std::str
     if (f64 && n == "of_float32") return "(double)(%s)";
     if (f32 && n == "of_float64") return "(float)(%s)";
   }
+  const bool i32 = mod == "Int32", i64 = mod == "Int64";
+  if (i32 || i64) {
+    // sarek/Sarek_stdlib/Int32.ml:30-88 and Int64.ml:31-88
+    static const char *ops[][2] = {{"add", "(%s + %s)"}, {"sub", "(%s - %s)"}, {"mul", "(%s * %s)"},
+                                   {"div", "(%s / %s)"}, {"mod", "(%s %% %s)"}};
+    for (auto &o : ops)
+      if (n == o[0] || n == std::string(o[0]) + (i32 ? "_int32" : "_int64")) return o[1];
+    static const char *same[][2] = {{"logand", "(%s & %s)"}, {"logor", "(%s | %s)"}, {"logxor", "(%s ^ %s)"},
+                                    {"lognot", "(~%s)"}, {"shift_left", "(%s << %s)"}, {"shift_right", "(%s >> %s)"},
+                                    {"neg", "(-%s)"}};
+    for (auto &o : same)
+      if (n == o[0]) return o[1];
+    if (n == "shift_right_logical") return i32 ? "((unsigned int)%s >> %s)" : "((unsigned long)%s >> %s)";
+    if (n == "abs") return i32 ? "abs(%s)" : "llabs(%s)";
+    if (n == "of_float" || n == "of_int") return i32 ? "(int)(%s)" : "(long long)(%s)";
+    if (n == "to_float") return "(double)(%s)";
+    if (n == "to_int") return "(int)(%s)";
+    if (i64 && n == "of_int32") return "(long long)(%s)";
+    if (i64 && n == "to_int32") return "(int)(%s)";
+  }
   if (n == "float" || n == "float_of_int") return "(float)(%s)";
   if (n == "int_of_float") return "(int)(%s)";
   return nullptr;
@@ -230,12 +250,22 @@ std::string apply_template(const std::string &templ, const std::vector<ExprP> &a
   size_t a = 0;
   for (size_t i = 0; i < templ.size(); ++i) {
     if (templ[i] == '%' && i + 1 < templ.size() && templ[i + 1] == 's') {
-      o += gen_expr(args[a++]);
+      const std::string arg = gen_expr(args[a++]);
+      // "(-%s)" round "-5": a minus keeps a space from an operand that begins with one, here as in a negation
+      if (!o.empty() && o.back() == '-' && !arg.empty() && arg[0] == '-') o.push_back(' ');
+      o += arg;
+      ++i;
+    } else if (templ[i] == '%' && i + 1 < templ.size() && templ[i + 1] == '%') {
+      o.push_back('%');   // the registry's templates are format strings: "%%" is the remainder operator
       ++i;
     } else {
       o.push_back(templ[i]);
     }
   }
+  // The logical shifts are spelled with an unsigned operand (Int32.ml:68-72, Int64.ml:68-72), which leaves the whole
+  // expression unsigned: `(x lsr 1) - 5 < 0` would never hold.  OCaml's result is the signed type again.
+  if (templ == "((unsigned int)%s >> %s)") return "(int)" + o;
+  if (templ == "((unsigned long)%s >> %s)") return "(long long)" + o;
   return o;
 }
 

@@ -7,7 +7,8 @@ It is a model for tests, over the integer subset the generator below emits: no f
 thread at a time (the programs touch no memory another thread writes).
 
 `random_program(seed)` builds a kernel over (x : int32 vector, out : int32 vector, k : int32, n : int32) in which
-thread tid < n computes with lets, mutable variables, assignments, `if` statements and expressions, calls of up to
+thread tid < n computes with lets, mutable variables, assignments, `if` statements and expressions, Stdlib.Int32's
+functions (by name, and with the registry's device templates as the front end attaches them), calls of up to
 two helper functions (their own lets, loops and branches, a return at every end), `for` loops in
 both directions (bounds that read mutable variables the body changes among them), counted `while` loops and blocks, and
 stores into out[tid * SLOTS + j].  Names come from a small pool, parameters' names included, so bindings hide each
@@ -26,7 +27,8 @@ class _Return(Exception):
 
 def parse(text):
     """IR text -> nested lists of atoms."""
-    tokens = text.replace("(", " ( ").replace(")", " ) ").split()
+    import re
+    tokens = re.findall(r'"[^"]*"|[()]|[^\s()"]+', text)
     pos = 0
 
     def node():
@@ -83,8 +85,22 @@ class Thread:
         if head == "read":
             return int(self.arrays[e[1]][self.expr(e[2])])
         if head == "intr":
-            assert e[2] in ("global_thread_id", "global_idx_x", "global_idx"), e
-            return self.index
+            name = e[2]
+            if name in ("global_thread_id", "global_idx_x", "global_idx"):
+                return self.index
+            assert e[1][-1] == "Int32", e                   # Stdlib.Int32's functions (sarek/Sarek_stdlib/Int32.ml:30-88)
+            args = [self.expr(a) for a in e[3:] if not (isinstance(a, list) and a and a[0] == "template")]
+            if name == "abs": return _fit(abs(args[0]))
+            if name == "neg": return _fit(-args[0])
+            if name == "lognot": return ~args[0]
+            if name == "min": return min(args)
+            if name == "max": return max(args)
+            if name == "logxor": return args[0] ^ args[1]
+            if name == "mod_int32": return args[0] - args[1] * _trunc_div(args[0], args[1])
+            if name == "shift_right_logical":
+                assert 0 <= args[1] < 32
+                return _fit((args[0] % (1 << 32)) >> args[1])
+            raise KeyError(name)
         if head == "if":
             return self.expr(e[2]) if self.expr(e[1]) else self.expr(e[3])
         if head == "app":                                  # a helper: its own bindings, the value its return gives
@@ -262,6 +278,21 @@ class _Builder:
             return f"(app (var {name} 0 i32) {' '.join(self.small(self.expr(depth - 1), 6) for _ in range(arity))})"
         a, b = self.expr(depth - 1), self.expr(depth - 1)
         pick = r.randint(0, 11)
+        if r.random() < 0.12:                                # Stdlib.Int32's functions, by name or with the registry's template
+            pick = r.randint(0, 6)
+            if pick == 0:
+                return f"(intr (Int32) abs {a})"
+            if pick == 1:
+                return f'(intr (Int32) neg (template "(-%s)") {a})'
+            if pick == 2:
+                return f"(intr (Int32) {r.choice(['min', 'max'])} {a} {b})"
+            if pick == 3:                                    # of a negative operand too: zeros come in from the left
+                return f"(sub (intr (Int32) shift_right_logical {a} (i32 {r.randint(0, 31)})) (i32 5))"
+            if pick == 4:
+                return f'(intr (Sarek_stdlib Int32) mod_int32 (template "(%s %% %s)") {a} (add {self.small(b, 3)} (i32 1)))'
+            if pick == 5:
+                return f"(intr (Int32) lognot {a})"
+            return f'(intr (Int32) shift_right_logical (template "((unsigned int)%s >> %s)") {a} (i32 {r.randint(1, 31)}))'
         if pick == 10:                                       # a linear congruential step: overflows at once
             return f"(add (mul {a} (i32 1103515245)) (i32 12345))"
         if pick == 11:

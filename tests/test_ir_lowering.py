@@ -151,6 +151,19 @@ def test_intrinsics(hip):
     assert expr_text(hip, "(intr (Mod Sub) unknown_fn (i32 1))") == "Mod.Sub.unknown_fn(1)"
     assert expr_text(hip, "(intr (Gpu) atomic_add (read h (i32 0)) (i32 1))") == "atomicAdd(&h[0], 1)"
     assert expr_text(hip, "(intr (Gpu) atomic_add (var h 1 (vec i32)) (i32 3) (i32 1))") == "atomicAdd(&h[3], 1)"
+    # Stdlib.Int32 / Int64 by name (sarek/Sarek_stdlib/Int32.ml:30-88, Int64.ml:31-88)
+    assert expr_text(hip, "(intr (Int32) abs (var a 1 i32))") == "abs(a)"
+    assert expr_text(hip, "(intr (Int64) abs (var a 1 i64))") == "llabs(a)"
+    assert expr_text(hip, "(intr (Sarek_stdlib Int32) logxor (var a 1 i32) (i32 3))") == "(a ^ 3)"
+    assert expr_text(hip, "(intr (Int32) min (var a 1 i32) (i32 3))") == "min(a, 3)"
+    # the registry's templates are format strings (applied with Printf there, Sarek_ir_cuda.ml:360-396): %% is a %
+    assert expr_text(hip, '(intr (Int32) mod_int32 (template "(%s %% %s)") (var a 1 i32) (i32 3))') == "(a % 3)"
+    # a minus in a template keeps a space from an operand that begins with one
+    assert expr_text(hip, '(intr (Int32) neg (template "(-%s)") (i32 -5))') == "(- -5)"
+    # the logical shifts' templates leave an unsigned value: OCaml's result is signed again
+    assert expr_text(hip, "(intr (Int32) shift_right_logical (var a 1 i32) (i32 3))") == "(int)((unsigned int)a >> 3)"
+    assert expr_text(hip, '(intr (Int64) shift_right_logical (template "((unsigned long)%s >> %s)") (var a 1 i64) (i32 3))') \
+        == "(long long)((unsigned long)a >> 3)"
 
 
 def test_vector_params_get_length_arguments(hip):
