@@ -430,7 +430,11 @@ typedef struct sarek_hip_varg {
  * lowers the IR (one lowering per distinct text is kept), expands vectors to
  * (buffer, int32 length), launches through sarek_hip_run_source under the kernel's own
  * name, then marks the Both vectors Stale_CPU.  A kernel the lowering refuses is
- * "Backend failed to generate source" (Execute.ml:257-263).                        */
+ * "Backend failed to generate source" (Execute.ml:257-263).  The arguments are held to the
+ * kernel's parameter list first -- their number, vector or scalar, int32 / int64 / float32 /
+ * float64, a vector's element size -- and a mismatch is SAREK_HIP_E_INVALID_ARG naming the
+ * argument, with nothing launched (the reference passes on what it is given, Execute.ml:197-216,
+ * and the kernel then reads a parameter block of another layout).                  */
 int sarek_hip_execute_run_vectors(const char *ir_text, const int block[3], const int grid[3],
                                   int shared_mem_bytes, const sarek_hip_varg *args, int n_args);
 /* A sequence of kernels over shared vectors, each stage what one Execute.run_vectors call takes:

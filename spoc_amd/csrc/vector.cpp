@@ -266,7 +266,57 @@ void mark_stale(const sarek_hip_varg *args, int n, int dev) {
 // every launch (Execute.ml:256); here one lowering per distinct IR text is kept.
 struct Lowered {
   std::string name, source;
+  // What each parameter takes: 'v' a vector (element size in bytes, 0 when the IR does not fix it: records), 'i' / 'l'
+  // / 'f' / 'd' an int32 / int64 / float32 / float64 scalar, '?' anything (a record passed by value).
+  struct Param {
+    std::string name;
+    char kind;
+    int elem_size;
+  };
+  std::vector<Param> params;
 };
+
+int scalar_size(const ir::Type &t) {
+  switch (t.kind) {
+    case ir::Type::Int32: case ir::Type::Float32: case ir::Type::Bool: return 4;
+    case ir::Type::Int64: case ir::Type::Float64: return 8;
+    default: return 0;
+  }
+}
+
+// A launch with the wrong number or kinds of arguments would hand the kernel a parameter block of another layout:
+// lengths read as pointers, a float's bits as an element count.  The reference passes on what it is given
+// (Execute.ml:197-216); here the mismatch is an error before anything is launched.
+int check_args(const Lowered &k, const sarek_hip_varg *args, int n, const char *what) {
+  if (static_cast<size_t>(n) != k.params.size())
+    return fail(SAREK_HIP_E_INVALID_ARG, "%s: kernel %s takes %zu arguments, %d given", what, k.name.c_str(),
+                k.params.size(), n);
+  static const char *given[] = {"a vector", "an int32", "an int64", "a float32", "a float64"};
+  for (int i = 0; i < n; ++i) {
+    const Lowered::Param &p = k.params[static_cast<size_t>(i)];
+    const int kind = args[i].kind;
+    const char *is = kind >= 0 && kind <= 4 ? given[kind] : "of an unknown kind";
+    const char *wants = nullptr;
+    switch (p.kind) {
+      case 'v':
+        if (kind != SAREK_HIP_VARG_VEC) wants = "a vector";
+        else if (args[i].vec && p.elem_size > 0 && static_cast<int64_t>(p.elem_size) != args[i].vec->elem_size)
+          return fail(SAREK_HIP_E_INVALID_ARG,
+                      "%s: argument %d (%s) of kernel %s is a vector of %d-byte elements, the vector given has %lld-byte elements",
+                      what, i, p.name.c_str(), k.name.c_str(), p.elem_size, static_cast<long long>(args[i].vec->elem_size));
+        break;
+      case 'i': if (kind != SAREK_HIP_VARG_INT32) wants = "an int32"; break;
+      case 'l': if (kind != SAREK_HIP_VARG_INT64) wants = "an int64"; break;
+      case 'f': if (kind != SAREK_HIP_VARG_FLOAT32) wants = "a float32"; break;
+      case 'd': if (kind != SAREK_HIP_VARG_FLOAT64) wants = "a float64"; break;
+      default: break;
+    }
+    if (wants)
+      return fail(SAREK_HIP_E_INVALID_ARG, "%s: argument %d (%s) of kernel %s is %s, %s given", what, i, p.name.c_str(),
+                  k.name.c_str(), wants, is);
+  }
+  return SAREK_HIP_OK;
+}
 std::mutex g_lowered_mu;
 std::unordered_map<std::string, std::shared_ptr<const Lowered>> g_lowered;
 
@@ -300,7 +350,26 @@ int lower(const char *ir_text, const int block[3], std::shared_ptr<const Lowered
   src.resize(std::strlen(src.c_str()));
   auto made = std::make_shared<Lowered>();
   made->source = src;
-  made->name = ir::parse_kernel(ir_text).name;
+  const ir::Kernel parsed = ir::parse_kernel(ir_text);
+  made->name = parsed.name;
+  for (const ir::Decl &d : parsed.params) {
+    Lowered::Param p{d.var.name, '?', 0};
+    if (d.var.type) {
+      const ir::Type &t = *d.var.type;
+      switch (t.kind) {
+        case ir::Type::Vec: case ir::Type::Array:
+          p.kind = 'v';
+          p.elem_size = t.elt ? scalar_size(*t.elt) : 0;
+          break;
+        case ir::Type::Int32: case ir::Type::Bool: p.kind = 'i'; break;
+        case ir::Type::Int64: p.kind = 'l'; break;
+        case ir::Type::Float32: p.kind = 'f'; break;
+        case ir::Type::Float64: p.kind = 'd'; break;
+        default: break;
+      }
+    }
+    made->params.push_back(p);
+  }
   out = made;
   std::lock_guard<std::mutex> lock(g_lowered_mu);
   if (g_lowered.size() > 256) g_lowered.clear();
@@ -619,6 +688,7 @@ int sarek_hip_execute_run_vectors(const char *ir_text, const int block[3], const
   } catch (const std::exception &e) {
     return fail(SAREK_HIP_E_PARSE, "run_vectors: %s", e.what());
   }
+  if ((st = check_args(*k, args, n_args, "run_vectors")) != SAREK_HIP_OK) return st;
   std::vector<sarek_hip_arg> rs;
   if ((st = expand_args(args, n_args, dev, true, rs)) != SAREK_HIP_OK) return st;
   st = sarek_hip_run_source(k->source.c_str(), SAREK_HIP_LANG_HIP_SOURCE, k->name.c_str(), block, grid,
@@ -652,6 +722,7 @@ int sarek_hip_execute_run_pipeline(const sarek_hip_pipeline_stage *stages, int n
     } catch (const std::exception &e) {
       return fail(SAREK_HIP_E_PARSE, "run_pipeline: stage %d: %s", i, e.what());
     }
+    if ((st = check_args(*lowered[i], s.args, s.n_args, "run_pipeline")) != SAREK_HIP_OK) return st;
     if ((st = expand_args(s.args, s.n_args, dev, true, expanded[i])) != SAREK_HIP_OK) return st;
     sarek_hip_launch &l = seq[i];
     l.source = lowered[i]->source.c_str();

@@ -412,3 +412,41 @@ def test_names_bound_again_mean_what_ocaml_says(hip, torch_cuda):
             expected[at] = value
         assert np.array_equal(v.to_array(), expected), name
 
+
+
+def test_arguments_that_do_not_fit_the_kernel_are_refused_before_the_launch(hip, torch_cuda):
+    """A launch with too few arguments, a scalar where a vector goes, an int for a float or a vector of another
+    element size would give the kernel a parameter block of another layout (a length read as a pointer).  The
+    reference passes on what it is given (Execute.ml:197-216); here each is an error that names the argument, and
+    nothing runs: the output vector keeps what it held."""
+    from spoc_amd.sarek import Execute, Transfer, Vector
+    ir = ("(kernel scale_kernel (params (param (var x 1 (vec f32))) (param (var out 2 (vec f32))) (param (var a 3 f32)) "
+          "(param (var n 4 i32))) (locals) (body (let (var tid 5 i32) (intr (Std) global_thread_id) "
+          "(if (lt (var tid 5 i32) (var n 4 i32)) (assign (lelem out (var tid 5 i32)) "
+          "(add (mul (read x (var tid 5 i32)) (var a 3 f32)) (f32 1.0)))))) (native_fn true))")
+    n = 256
+    x = Vector.of_array(np.arange(n, dtype=np.float32))
+    out = Vector.of_array(np.full(n, -7, np.float32))
+    wide = Vector.of_array(np.zeros(n, np.float64))
+    good = [Execute.Vec(x), Execute.Vec(out), Execute.Float32(2.0), Execute.Int32(n)]
+    cases = [
+        (good[:3], "takes 4 arguments, 3 given"),
+        (good + [Execute.Int32(1)], "takes 4 arguments, 5 given"),
+        ([Execute.Vec(x), Execute.Float32(2.0), Execute.Vec(out), Execute.Int32(n)], "argument 1 (out) of kernel scale_kernel is a vector, a float32 given"),
+        ([Execute.Vec(x), Execute.Vec(out), Execute.Int32(2), Execute.Int32(n)], "argument 2 (a) of kernel scale_kernel is a float32, an int32 given"),
+        ([Execute.Vec(x), Execute.Vec(out), Execute.Float64(2.0), Execute.Int32(n)], "is a float32, a float64 given"),
+        ([Execute.Vec(x), Execute.Vec(out), Execute.Float32(2.0), Execute.Int64(n)], "argument 3 (n) of kernel scale_kernel is an int32, an int64 given"),
+        ([Execute.Vec(wide), Execute.Vec(out), Execute.Float32(2.0), Execute.Int32(n)], "is a vector of 4-byte elements, the vector given has 8-byte elements"),
+    ]
+    for args, message in cases:
+        with pytest.raises(hip.SarekHipError) as err:
+            Execute.run_vectors(ir=ir, args=args, block=Execute.dims1d(64), grid=Execute.dims1d(4))
+        assert err.value.status == hip.E_INVALID_ARG and message in str(err.value), (message, str(err.value))
+        with pytest.raises(hip.SarekHipError) as err:
+            Execute.run_pipeline([(ir, args, (64, 1, 1), (4, 1, 1))])
+        assert err.value.status == hip.E_INVALID_ARG and message in str(err.value), (message, str(err.value))
+    Transfer.flush()
+    assert np.array_equal(out.to_array(), np.full(n, -7, np.float32))
+    assert Execute.run_vectors(ir=ir, args=good, block=Execute.dims1d(64), grid=Execute.dims1d(4)) in ("map_f32", "jit")
+    Transfer.flush()
+    assert np.array_equal(out.to_array(), np.arange(n, dtype=np.float32) * 2 + 1)
