@@ -22,7 +22,10 @@ let binop = function
   | Le -> "le" | Gt -> "gt" | Ge -> "ge" | And -> "and" | Or -> "or" | Shl -> "shl" | Shr -> "shr"
   | BitAnd -> "bitand" | BitOr -> "bitor" | BitXor -> "bitxor"
 let unop = function Neg -> "neg" | Not -> "not" | BitNot -> "bitnot"
-let pat = function PWild -> "_" | PConstr (c, vs) -> Printf.sprintf "(%s%s)" c (cat Fun.id vs)
+let pat = function
+  | PWild -> "_"
+  | PConstr ("", vs) -> Printf.sprintf "(?%s)" (cat Fun.id vs)   (* a variable pattern, Sarek_lower_ir.ml:559 *)
+  | PConstr (c, vs) -> Printf.sprintf "(%s%s)" c (cat Fun.id vs)
 let const = function
   | CInt32 n -> Printf.sprintf "(i32 %ld)" n | CInt64 n -> Printf.sprintf "(i64 %Ld)" n
   | CFloat32 f -> Printf.sprintf "(f32 %.17g)" f | CFloat64 f -> Printf.sprintf "(f64 %.17g)" f   (* nan, inf, -inf pass *)

@@ -51,6 +51,9 @@ let expressions =
     ("match expression",
      EMatch (EVar (v ~id:3 "s" (TVariant ("shape", []))), [(PConstr ("Circle", ["r"]), i 1); (PWild, i 0)]),
      "(match (var s 3 (variant shape)) (case (Circle r) (i32 1)) (case _ (i32 0)))");
+    ("match with a variable pattern",
+     EMatch (EVar (v ~id:3 "s" (TVariant ("shape", []))), [(PConstr ("Circle", ["r"]), i 1); (PConstr ("", ["rest"]), i 0)]),
+     "(match (var s 3 (variant shape)) (case (Circle r) (i32 1)) (case (? rest) (i32 0)))");
     ("helper call", EApp (EVar (v "square" TFloat32), [EVar acc]), "(app (var square 0 f32) (var acc 2 f32 mut))") ]
 
 let statements =

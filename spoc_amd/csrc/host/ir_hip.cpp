@@ -343,14 +343,19 @@ const std::vector<TypeP> *constructor_types(const std::string &cname) {
 std::string gen_match_case(const std::string &indent, const std::string &scrutinee,
                            const Pattern &p, const StmtP &body) {
   std::string o = indent;
-  if (p.wildcard) {
+  const bool names_the_value = !p.wildcard && p.constr.empty();   // `| x -> ...`
+  if (p.wildcard || names_the_value) {
     o += "  default: {\n";
   } else {
     o += "  case " + p.constr + ": {\n";
   }
   CBlock braces;
   std::vector<std::unique_ptr<Binding>> bound;
-  if (!p.wildcard) {
+  if (names_the_value) {
+    // the reference prints `case : {` for it (Sarek_ir_cuda.ml:594-640 takes the empty name for a constructor)
+    bound.push_back(std::make_unique<Binding>(p.vars.at(0)));
+    o += indent + "    auto " + bound.back()->printed + " = " + scrutinee + ";\n";
+  } else if (!p.wildcard) {
     const std::vector<TypeP> *types = constructor_types(p.constr);
     if (!p.vars.empty() && types && !types->empty()) {
       if (p.vars.size() == 1 && types->size() == 1) {
@@ -530,7 +535,10 @@ std::string gen_expr(const ExprP &ep) {
       const std::string scrutinee = gen_expr(e.args[0]);
       auto value_of = [&](const Pattern &p, const ExprP &body) {
         const size_t mark = t_renames.size();
-        const std::vector<TypeP> *types = p.wildcard || p.vars.empty() ? nullptr : constructor_types(p.constr);
+        const std::vector<TypeP> *types =
+            p.wildcard || p.vars.empty() || p.constr.empty() ? nullptr : constructor_types(p.constr);
+        if (!p.wildcard && p.constr.empty() && p.vars.size() == 1)   // `| x -> ...`: x is the value itself
+          t_renames.push_back({p.vars[0], -1, scrutinee, false});
         if (types && types->size() == p.vars.size())
           for (size_t i = 0; i < p.vars.size(); ++i)
             t_renames.push_back({p.vars[i], -1,
@@ -551,7 +559,7 @@ std::string gen_expr(const ExprP &ep) {
       std::string o, close;
       for (size_t i = 0; i + 1 < e.cases.size(); ++i) {
         const Pattern &p = e.cases[i].first;
-        o += "(" + (p.wildcard ? std::string("1") : "(" + scrutinee + ".tag == " + p.constr + ")") + " ? " +
+        o += "(" + (p.wildcard || p.constr.empty() ? std::string("1") : "(" + scrutinee + ".tag == " + p.constr + ")") + " ? " +
              value_of(p, e.cases[i].second) + " : ";
         close += ")";
       }

@@ -247,6 +247,12 @@ Pattern to_pattern(const SExp &e) {
   p.wildcard = false;
   p.constr = atom(e.items[0], "a constructor name");
   for (size_t i = 1; i < e.items.size(); ++i) p.vars.push_back(atom(e.items[i], "a variable name"));
+  // `| x -> ...`: the front end lowers a variable pattern to a constructor pattern with an empty name and the one
+  // variable (Sarek_lower_ir.ml:556-559); written (? x) here
+  if (p.constr == "?") {
+    if (p.vars.size() != 1) perr(e, "expected (? VAR)");
+    p.constr.clear();
+  }
   return p;
 }
 
@@ -657,7 +663,7 @@ std::string pr_var(const Var &v) {
 
 std::string pr_pat(const Pattern &p) {
   if (p.wildcard) return "_";
-  std::string s = "(" + p.constr;
+  std::string s = "(" + (p.constr.empty() ? std::string("?") : p.constr);
   for (auto &v : p.vars) s += " " + v;
   return s + ")";
 }

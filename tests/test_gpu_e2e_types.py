@@ -267,3 +267,17 @@ def test_a_match_used_as_a_value(hip, torch_cuda):
     assert path == "jit"
     want = np.where(x > 1, x * x, np.where(x < -1, x * np.float32(2), x))
     assert np.array_equal(dst.to_array(), want)
+
+
+def test_a_pattern_that_names_the_value(hip, torch_cuda):
+    """`match s with Circle r -> r | other -> (match other with Rect (w, h) -> w *. h | rest -> -1.)`."""
+    from test_ir_lowering import MATCH_WITH_A_VARIABLE_PATTERN
+    from spoc_amd.sarek import Execute, Transfer, Vector
+    n = 500
+    x = np.random.default_rng(4).uniform(-3, 3, n).astype(np.float32)
+    dst = Vector.create(Vector.float32, n)
+    path = Execute.run_vectors(ir=MATCH_WITH_A_VARIABLE_PATTERN, args=[Execute.Vec(Vector.of_array(x)), Execute.Vec(dst), Execute.Int32(n)],
+                               block=Execute.dims1d(64), grid=Execute.dims1d((n + 63) // 64))
+    Transfer.flush()
+    assert path == "jit"
+    assert np.array_equal(dst.to_array(), np.where(x > 1, x, x * np.float32(3)))

@@ -854,3 +854,26 @@ def test_a_match_used_as_a_value_binds_its_patterns(hip):
     text = hip.generate_source(MATCH_AS_A_VALUE)
     assert ("dst[tid] = ((s.tag == Circle) ? (s.data.Circle_v * s.data.Circle_v) : "
             "((s.tag == Rect) ? (s.data.Rect_v._0 * s.data.Rect_v._1) : x));") in text
+
+
+MATCH_WITH_A_VARIABLE_PATTERN = f"""(kernel sarek_kern (params (param (var xs 1 (vec f32))) (param (var dst 2 (vec f32))) (param (var n 3 i32))) (locals)
+ (body (let (var tid 4 i32) (intr (Std) global_thread_id) (if (lt (var tid 4 i32) (var n 3 i32))
+   (let (var x 5 f32) (read xs (var tid 4 i32))
+   (let (var s 6 {SHAPE}) (if (gt (var x 5 f32) (f32 1.0)) (variant shape Circle (var x 5 f32)) (variant shape Rect (var x 5 f32) (f32 3.0)))
+     (seq (match (var s 6 {SHAPE})
+            (case (Circle r) (assign (lelem dst (var tid 4 i32)) (var r 7 f32)))
+            (case (? other) (assign (lelem dst (var tid 4 i32))
+                                    (match (var other 8 {SHAPE}) (case (Rect w h) (mul (var w 9 f32) (var h 10 f32)))
+                                                                 (case (? rest) (f32 -1.0))))))))))))
+ (variants (shape (Circle f32) (Rect f32 f32) (Empty))) (native_fn true))"""
+
+
+def test_a_pattern_that_names_the_value(hip):
+    """`| other -> ...`: the front end lowers a variable pattern to a constructor pattern with an empty name
+    (Sarek_lower_ir.ml:556-559), for which the reference prints `case : {`.  Here it is the default case with the
+    variable bound to the value matched, as a statement and -- the variable standing for the value -- as a value."""
+    text = hip.generate_source(MATCH_WITH_A_VARIABLE_PATTERN)
+    assert "      default: {\n        auto other = s;\n" in text
+    assert "dst[tid] = ((other.tag == Rect) ? (other.data.Rect_v._0 * other.data.Rect_v._1) : -1.0f);" in text
+    with pytest.raises(hip.SarekHipError):
+        hip.generate_source(MATCH_WITH_A_VARIABLE_PATTERN.replace("(? other)", "(? other more)"))

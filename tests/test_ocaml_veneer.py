@@ -291,7 +291,7 @@ def test_the_forms_the_ocaml_unit_test_expects_are_forms_the_native_reader_takes
 
     types, consts = table("types"), table("constants_and_variables")
     exprs, stmts = table("expressions"), table("statements")
-    assert (len(types), len(consts), len(exprs), len(stmts)) == (6, 7, 15, 18)
+    assert (len(types), len(consts), len(exprs), len(stmts)) == (6, 7, 16, 18)
     for t in types:
         hip.generate_source(kernel(params=f" (param (var p 9 {t}))"))
     for e in consts + exprs:
