@@ -175,8 +175,14 @@ int sarek_hip_profiler_stop(void);
 /* Kernel JIT + launch  (replaces the nvrtc.., cuModule.. groups and cuLaunchKernel,
  * sarek-cuda/Cuda_nvrtc.ml:263-389, sarek-cuda/Cuda_api.ml:315-486).
  * `source` is HIP C++ text; it is compiled by hiprtc for the current
- * device's architecture (--offload-arch=<gcnArchName>).  On failure the
- * compiler log is copied into `log` (truncated to log_len-1 bytes).        */
+ * device's architecture (--offload-arch=<gcnArchName>), -O3, with wrapping
+ * signed arithmetic (-fwrapv: OCaml's Int32 / Int64 wrap) and without packed
+ * FP32 instructions.  A text that names Float.x, Int32.x or Int64.x without
+ * declaring an object of that name is given OCaml's constants of those modules
+ * in front (a value outside the kernel lowers to a variable of its name,
+ * sarek/ppx/Sarek_lower_ir.ml:378-380; line numbers in the log then count
+ * those lines).  On failure the compiler log is copied into `log` (truncated
+ * to log_len-1 bytes).                                                      */
 int sarek_hip_kernel_compile(const char *source, const char *kernel_name,
                              sarek_hip_kernel *out, char *log, size_t log_len);
 /* Same, memoised on (device, hash(source), kernel_name)

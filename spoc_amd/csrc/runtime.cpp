@@ -8,6 +8,7 @@
 #include "code_cache.hpp"
 
 #include <atomic>
+#include <cctype>
 #include <cstring>
 #include <map>
 #include <unordered_map>
@@ -70,11 +71,55 @@ void copy_log(const std::string &text, char *log, size_t log_len) {
   log[n] = '\0';
 }
 
-int compile_impl(const char *source, const char *kernel_name, sarek_hip_kernel *out, char *log,
+// Whether `text` uses the module-qualified name MODULE.something without declaring MODULE itself.
+bool uses_module(const std::string &text, const char *module) {
+  const std::string name = module;
+  bool used = false;
+  for (size_t at = text.find(name); at != std::string::npos; at = text.find(name, at + 1)) {
+    const bool starts = at == 0 || !(std::isalnum(static_cast<unsigned char>(text[at - 1])) || text[at - 1] == '_');
+    if (!starts) continue;
+    const char after = at + name.size() < text.size() ? text[at + name.size()] : '\0';
+    if (after == '.') used = true;
+    else if (!(std::isalnum(static_cast<unsigned char>(after)) || after == '_')) return false;   // the text's own Float
+  }
+  return used;
+}
+
+// OCaml's constants that a kernel may name.  A reference to a value outside the kernel lowers to a variable of that
+// name (sarek/ppx/Sarek_lower_ir.ml:378-380), so the text says `sdata[tid] = Float.neg_infinity;` -- as the reference's
+// own generated reduction does (benchmarks/generate_backend_code.ml:164) -- which is no C without an object called
+// Float.  The Native backend evaluates the OCaml value, a double; these are the same values.
+std::string ocaml_constants_for(const std::string &text) {
+  std::string o;
+  if (uses_module(text, "Float"))
+    o += "struct sarek_hip_ocaml_float { double infinity, neg_infinity, nan, pi, epsilon, max_float, min_float, zero, one, "
+         "minus_one; };\nstatic constexpr sarek_hip_ocaml_float Float = {__builtin_inf(), -__builtin_inf(), "
+         "__builtin_nan(\"\"), 3.141592653589793116, 2.220446049250313081e-16, 1.797693134862315708e+308, "
+         "2.225073858507201383e-308, 0.0, 1.0, -1.0};\n";
+  if (uses_module(text, "Int32"))
+    o += "struct sarek_hip_ocaml_int32 { int max_int, min_int, zero, one, minus_one; };\n"
+         "static constexpr sarek_hip_ocaml_int32 Int32 = {2147483647, -2147483647 - 1, 0, 1, -1};\n";
+  if (uses_module(text, "Int64"))
+    o += "struct sarek_hip_ocaml_int64 { long long max_int, min_int, zero, one, minus_one; };\n"
+         "static constexpr sarek_hip_ocaml_int64 Int64 = {9223372036854775807LL, -9223372036854775807LL - 1, 0, 1, -1};\n";
+  return o;
+}
+
+int compile_impl(const char *source_given, const char *kernel_name, sarek_hip_kernel *out, char *log,
                  size_t log_len) {
-  if (!source || !kernel_name || !out)
+  if (!source_given || !kernel_name || !out)
     return fail(SAREK_HIP_E_INVALID_ARG, "kernel_compile: NULL argument");
   if (log && log_len) log[0] = '\0';
+  std::string with_constants;
+  const char *source = source_given;
+  {
+    const std::string text = source_given;
+    const std::string constants = ocaml_constants_for(text);
+    if (!constants.empty()) {
+      with_constants = constants + text;
+      source = with_constants.c_str();
+    }
+  }
   int dev = 0;
   SAREK_HIP_TRY(hipGetDevice(&dev));
   hipDeviceProp_t prop;

@@ -281,3 +281,39 @@ def test_a_pattern_that_names_the_value(hip, torch_cuda):
     Transfer.flush()
     assert path == "jit"
     assert np.array_equal(dst.to_array(), np.where(x > 1, x, x * np.float32(3)))
+
+
+def test_ocaml_constants_a_kernel_names(hip, torch_cuda):
+    """A reference to a value outside the kernel lowers to a variable of that name (Sarek_lower_ir.ml:378-380): the
+    reference's own generated maximum reduction says `sdata[tid] = Float.neg_infinity;`
+    (benchmarks/generate_backend_code.ml:164, the golden text of reduction_max).  The run-time compiler is given
+    OCaml's values for Float.*, Int32.* and Int64.* when a text names them: the golden kernel runs as generated,
+    block maxima bit for bit, and a kernel that stores a few of the others holds OCaml's values."""
+    from spoc_amd import reference_kernels as rk
+    from spoc_amd.sarek import Execute, Transfer, Vector
+    n = 1000
+    x = np.random.default_rng(8).standard_normal(n).astype(np.float32) - 5
+    out = Vector.create(Vector.float32, 4)
+    ir = rk.reduction_max()
+    assert "Float.neg_infinity" in hip.generate_source(ir, block=(256, 1, 1))
+    path = Execute.run_vectors(ir=ir, args=[Execute.Vec(Vector.of_array(x)), Execute.Vec(out), Execute.Int32(n)],
+                               block=Execute.dims1d(256), grid=Execute.dims1d(4))
+    Transfer.flush()
+    assert path == "jit"
+    assert np.array_equal(out.to_array(), [x[b * 256:(b + 1) * 256].max() for b in range(4)])
+
+    stores = [("(var Float.pi 10 f64)", "d", np.pi), ("(var Float.epsilon 11 f64)", "d", np.finfo(np.float64).eps),
+              ("(var Float.infinity 12 f64)", "d", np.inf), ("(var Float.max_float 13 f64)", "d", np.finfo(np.float64).max),
+              ("(var Int32.max_int 14 i32)", "i", 2**31 - 1), ("(var Int32.min_int 15 i32)", "i", -2**31),
+              ("(var Int64.max_int 16 i64)", "l", 2**63 - 1), ("(var Int64.min_int 17 i64)", "l", -2**63),
+              ("(add (var Int32.max_int 14 i32) (var Int32.one 18 i32))", "i", -2**31)]
+    body = " ".join(f"(assign (lelem {v} (i32 {k})) {e})" for k, (e, v, _) in enumerate(stores))
+    ir = ("(kernel sarek_kern (params (param (var d 1 (vec f64))) (param (var i 2 (vec i32))) (param (var l 3 (vec i64)))) "
+          f"(locals) (body (if (eq (intr (Std) global_thread_id) (i32 0)) (seq {body}))) (native_fn true))")
+    d, i, l = Vector.create(Vector.float64, 16), Vector.create(Vector.int32, 16), Vector.create(Vector.int64, 16)
+    Execute.run_vectors(ir=ir, args=[Execute.Vec(d), Execute.Vec(i), Execute.Vec(l)], block=Execute.dims1d(64),
+                        grid=Execute.dims1d(1))
+    Transfer.flush()
+    got = {"d": d.to_array(), "i": i.to_array(), "l": l.to_array()}
+    for k, (e, v, want) in enumerate(stores):
+        assert got[v][k] == want, (e, got[v][k], want)

@@ -355,3 +355,19 @@ def test_reference_benchmarks_run_and_verify(hip, torch_cuda, name, size, path):
     finally:
         hip.check(hip.lib.sarek_hip_set_specialisation(1))
     assert rec["verified"] and rec["path"] == "jit"
+
+
+def test_a_text_with_a_float_of_its_own_is_left_as_written(hip, torch_cuda):
+    """Texts that name OCaml's Float.* / Int32.* / Int64.* constants are compiled with their values in front; a text
+    that declares an object called Float itself gets nothing added (the two definitions would clash)."""
+    torch = torch_cuda
+    own = ("struct mine { float neg_infinity; };\n__device__ mine Float = {42.0f};\n"
+           "extern \"C\" __global__ void k(float* out, int out_len) { out[0] = Float.neg_infinity; }\n")
+    out = torch.zeros(4, device="cuda")
+    assert hip.run_source(own, "k", (1, 1, 1), (1, 1, 1), [out]) == "jit"
+    torch.cuda.synchronize()
+    assert out[0].item() == 42.0
+    named = "extern \"C\" __global__ void k2(float* out, int out_len) { out[1] = Float.neg_infinity; out[2] = (float)Int32.max_int; }\n"
+    hip.run_source(named, "k2", (1, 1, 1), (1, 1, 1), [out])
+    torch.cuda.synchronize()
+    assert out[1].item() == float("-inf") and out[2].item() == 2147483648.0
