@@ -296,11 +296,17 @@ def test_ocaml_constants_a_kernel_names(hip, torch_cuda):
     out = Vector.create(Vector.float32, 4)
     ir = rk.reduction_max()
     assert "Float.neg_infinity" in hip.generate_source(ir, block=(256, 1, 1))
-    path = Execute.run_vectors(ir=ir, args=[Execute.Vec(Vector.of_array(x)), Execute.Vec(out), Execute.Int32(n)],
-                               block=Execute.dims1d(256), grid=Execute.dims1d(4))
-    Transfer.flush()
-    assert path == "jit"
-    assert np.array_equal(out.to_array(), [x[b * 256:(b + 1) * 256].max() for b in range(4)])
+    for specialise, served_by in ((0, "jit"), (1, "reduce_max_block256_f32:ff800000")):   # as generated, then by the hand kernel
+        hip.check(hip.lib.sarek_hip_set_specialisation(specialise))
+        try:
+            out.fill(np.float32(7))
+            path = Execute.run_vectors(ir=ir, args=[Execute.Vec(Vector.of_array(x)), Execute.Vec(out), Execute.Int32(n)],
+                                       block=Execute.dims1d(256), grid=Execute.dims1d(4))
+            Transfer.flush()
+        finally:
+            hip.check(hip.lib.sarek_hip_set_specialisation(1))
+        assert path == served_by
+        assert np.array_equal(out.to_array(), [x[b * 256:(b + 1) * 256].max() for b in range(4)])
 
     stores = [("(var Float.pi 10 f64)", "d", np.pi), ("(var Float.epsilon 11 f64)", "d", np.finfo(np.float64).eps),
               ("(var Float.infinity 12 f64)", "d", np.inf), ("(var Float.max_float 13 f64)", "d", np.finfo(np.float64).max),
