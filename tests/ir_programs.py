@@ -7,7 +7,7 @@ It is a model for tests, over the integer subset the generator below emits: no f
 thread at a time (the programs touch no memory another thread writes).
 
 `random_program(seed)` builds a kernel over (x : int32 vector, out : int32 vector, k : int32, n : int32) in which
-thread tid < n computes with lets, mutable variables, assignments, `if` statements and expressions, Stdlib.Int32's
+thread tid < n computes with int32 and int64 lets, mutable variables, assignments, casts between the two, `if` statements and expressions, Stdlib.Int32's
 functions (by name, and with the registry's device templates as the front end attaches them), calls of up to
 two helper functions (their own lets, loops and branches, a return at every end), `for` loops in
 both directions (bounds that read mutable variables the body changes among them), counted `while` loops and blocks, and
@@ -48,9 +48,29 @@ def parse(text):
     return tree
 
 
-def _fit(v):
-    """Int32 arithmetic is modulo 2^32 (OCaml's Int32; the device text is compiled with wrapping signed arithmetic)."""
-    return (v - INT_MIN) % (1 << 32) + INT_MIN
+def _fit(v, bits=32):
+    """Int32 / Int64 arithmetic is modulo 2^32 / 2^64 (OCaml's Int32 and Int64; the device text is compiled with
+    wrapping signed arithmetic)."""
+    half = 1 << (bits - 1)
+    return (v + half) % (1 << bits) - half
+
+
+def width(e):
+    """32 or 64: the integer type of an expression, from its leaves (OCaml's operators take operands of one type)."""
+    head = e[0]
+    if head == "i64":
+        return 64
+    if head == "var":
+        return 64 if e[3] == "i64" else 32
+    if head == "cast":
+        return 64 if e[1] == "i64" else 32
+    if head == "intr":
+        return 64 if e[1][-1] == "Int64" else 32
+    if head == "if":
+        return width(e[2])
+    if head in ("neg", "bitnot", "add", "sub", "mul", "div", "mod", "bitand", "bitor", "bitxor", "shl", "shr"):
+        return width(e[1])
+    return 32
 
 
 def _trunc_div(a, b):
@@ -76,8 +96,10 @@ class Thread:
 
     def expr(self, e):
         head = e[0]
-        if head == "i32":
+        if head in ("i32", "i64"):
             return int(e[1])
+        if head == "cast":                                  # Int64.of_int32 keeps the value, Int64.to_int32 its low 32 bits
+            return _fit(self.expr(e[2]), 64 if e[1] == "i64" else 32)
         if head == "bool":
             return e[1] == "true"
         if head == "var":
@@ -88,18 +110,19 @@ class Thread:
             name = e[2]
             if name in ("global_thread_id", "global_idx_x", "global_idx"):
                 return self.index
-            assert e[1][-1] == "Int32", e                   # Stdlib.Int32's functions (sarek/Sarek_stdlib/Int32.ml:30-88)
+            assert e[1][-1] in ("Int32", "Int64"), e        # Stdlib.Int32 / Int64 (sarek/Sarek_stdlib/Int32.ml:30-88, Int64.ml)
+            bits = 64 if e[1][-1] == "Int64" else 32
             args = [self.expr(a) for a in e[3:] if not (isinstance(a, list) and a and a[0] == "template")]
-            if name == "abs": return _fit(abs(args[0]))
-            if name == "neg": return _fit(-args[0])
+            if name == "abs": return _fit(abs(args[0]), bits)
+            if name == "neg": return _fit(-args[0], bits)
             if name == "lognot": return ~args[0]
             if name == "min": return min(args)
             if name == "max": return max(args)
             if name == "logxor": return args[0] ^ args[1]
             if name == "mod_int32": return args[0] - args[1] * _trunc_div(args[0], args[1])
             if name == "shift_right_logical":
-                assert 0 <= args[1] < 32
-                return _fit((args[0] % (1 << 32)) >> args[1])
+                assert 0 <= args[1] < bits
+                return _fit((args[0] % (1 << bits)) >> args[1], bits)
             raise KeyError(name)
         if head == "if":
             return self.expr(e[2]) if self.expr(e[1]) else self.expr(e[3])
@@ -115,26 +138,27 @@ class Thread:
             finally:
                 self.steps += callee.steps
             raise AssertionError("a helper ended without a return")
+        bits = width(e)
         if head == "neg":
-            return _fit(-self.expr(e[1]))
+            return _fit(-self.expr(e[1]), bits)
         if head == "bitnot":
             return ~self.expr(e[1])
         if head == "not":
             return not self.expr(e[1])
         a, b = self.expr(e[1]), self.expr(e[2])
-        if head == "add": return _fit(a + b)
-        if head == "sub": return _fit(a - b)
-        if head == "mul": return _fit(a * b)
-        if head == "div": return _fit(_trunc_div(a, b))
+        if head == "add": return _fit(a + b, bits)
+        if head == "sub": return _fit(a - b, bits)
+        if head == "mul": return _fit(a * b, bits)
+        if head == "div": return _fit(_trunc_div(a, b), bits)
         if head == "mod": return a - b * _trunc_div(a, b)
         if head == "bitand": return a & b
         if head == "bitor": return a | b
         if head == "bitxor": return a ^ b
         if head == "shl":
-            assert 0 <= b < 32
-            return _fit(a << b)
+            assert 0 <= b < bits
+            return _fit(a << b, bits)
         if head == "shr":
-            assert a >= 0 and 0 <= b < 32
+            assert a >= 0 and 0 <= b < bits
             return a >> b
         if head == "lt": return a < b
         if head == "le": return a <= b
@@ -215,6 +239,7 @@ class _Builder:
         self.scope = {"x": (1, False), "out": (2, False), "k": (3, False), "n": (4, False), "tid": (5, False)}
         self.vectors = {"x", "out"}
         self.counters = set()      # ids of loop counters: mutable in the IR, assigned by their loop alone
+        self.wide = set()          # ids of the int64 variables
         self.helpers = []          # (name, number of parameters) of the helper functions made so far
         self.in_helper = False     # a helper sees its parameters alone: no vector, no thread index
 
@@ -252,14 +277,51 @@ class _Builder:
         return f"(return {self.expr(r.randint(0, 2))})"
 
     def var(self, name, vid, mutable):
-        return f"(var {name} {vid} i32{' mut' if mutable else ''})"
+        return f"(var {name} {vid} {'i64' if vid in self.wide else 'i32'}{' mut' if mutable else ''})"
 
     def use(self, name):
         vid, mutable = self.scope[name]
         return self.var(name, vid, mutable)
 
     def ints_in_scope(self):
-        return [n for n in self.scope if n not in self.vectors]
+        return [n for n, (vid, _) in self.scope.items() if n not in self.vectors and vid not in self.wide]
+
+    def longs_in_scope(self):
+        return [n for n, (vid, _) in self.scope.items() if vid in self.wide]
+
+    def expr64(self, depth):
+        """An int64 expression: Int64's operators and functions over constants of all sizes, the int64 variables in
+        scope and widened int32 expressions."""
+        r = self.rng
+        if depth == 0:
+            longs = self.longs_in_scope()
+            pick = r.randint(0, 3)
+            if pick == 0 or (pick == 1 and not longs):
+                return f"(i64 {r.choice([0, 1, -1, 5, -7, 4294967296, -4294967297, 1 << 40, 9223372036854775807, -9223372036854775808, r.randint(-1 << 62, 1 << 62)])})"
+            if pick == 1:
+                return self.use(r.choice(longs))
+            return f"(cast i64 {self.expr(r.randint(0, 1))})"
+        a, b = self.expr64(depth - 1), self.expr64(depth - 1)
+        pick = r.randint(0, 9)
+        if pick == 0:
+            return f"({r.choice(['add', 'sub', 'mul'])} {a} {b})"
+        if pick == 1:
+            return f"({r.choice(['bitand', 'bitor', 'bitxor'])} {a} {b})"
+        if pick == 2:
+            return f"(shl (bitand {a} (i64 1048575)) (i32 {r.randint(0, 40)}))"
+        if pick == 3:
+            return f"(shr (bitand {a} (i64 {(1 << 50) - 1})) (i32 {r.randint(0, 45)}))"
+        if pick == 4:
+            return f"({r.choice(['neg', 'bitnot'])} {a})"
+        if pick == 5:
+            return f"(if {self.cond(0)} {a} {b})"
+        if pick == 6:
+            return f"(intr (Int64) {r.choice(['min', 'max'])} {a} {b})"
+        if pick == 7:
+            return f"(intr (Int64) shift_right_logical {a} (i32 {r.randint(0, 63)}))"
+        if pick == 8:
+            return f"(add (mul {a} (i64 6364136223846793005)) (i64 1442695040888963407))"
+        return f"({r.choice(['div', 'mod'])} {a} (add (bitand {b} (i64 7)) (i64 1)))"
 
     def small(self, e, bits=7):
         return f"(bitand {e} (i32 {(1 << bits) - 1}))"
@@ -273,6 +335,9 @@ class _Builder:
             if pick == 1 and not self.in_helper:
                 return f"(read x {self.use('tid')})"
             return self.use(r.choice(self.ints_in_scope()))
+        if r.random() < 0.1:                                 # the low or the high half of an int64 value
+            wide = self.expr64(depth - 1)
+            return r.choice([f"(cast i32 {wide})", f"(cast i32 (intr (Int64) shift_right_logical {wide} (i32 32)))"])
         if self.helpers and not self.in_helper and r.random() < 0.15:
             name, arity = r.choice(self.helpers)
             return f"(app (var {name} 0 i32) {' '.join(self.small(self.expr(depth - 1), 6) for _ in range(arity))})"
@@ -324,14 +389,18 @@ class _Builder:
             if pick == 0:
                 return f"(not {self.cond(depth - 1)})"
             return f"({'and' if pick == 1 else 'or'} {self.cond(depth - 1)} {self.cond(depth - 1)})"
+        if r.random() < 0.15:
+            return f"({r.choice(['lt', 'le', 'gt', 'ge', 'eq', 'ne'])} {self.expr64(1)} {self.expr64(1)})"
         return f"({r.choice(['lt', 'le', 'gt', 'ge', 'eq', 'ne'])} {self.expr(1)} {self.expr(1)})"
 
-    def bound_body(self, name, mutable, make_body, counter=False):
+    def bound_body(self, name, mutable, make_body, counter=False, wide=False):
         """Text of a binding's declaration and the body built with the name meaning the new variable."""
         vid = self.next_id
         self.next_id += 1
         if counter:
             self.counters.add(vid)
+        if wide:
+            self.wide.add(vid)
         hidden = self.scope.get(name)
         self.scope[name] = (vid, mutable)
         body = make_body()
@@ -341,12 +410,16 @@ class _Builder:
             self.scope[name] = hidden
         return self.var(name, vid, mutable), body
 
+    def assign(self, name):
+        value = self.expr64(self.rng.randint(0, 2)) if self.scope[name][0] in self.wide else self.expr(self.rng.randint(0, 2))
+        return f"(assign (lvar {self.use(name)}) {value})"
+
     def store(self):
         if self.in_helper:                                  # no memory there: an assignment, or nothing
             mutables = [n for n, (vid, m) in self.scope.items() if m and vid not in self.counters]
             if not mutables:
                 return "(empty)"
-            return f"(assign (lvar {self.use(self.rng.choice(mutables))}) {self.expr(self.rng.randint(0, 2))})"
+            return self.assign(self.rng.choice(mutables))
         slot = self.rng.randrange(SLOTS)
         return f"(assign (lelem out (add (mul {self.use('tid')} (i32 {SLOTS})) (i32 {slot}))) {self.expr(self.rng.randint(0, 2))})"
 
@@ -358,24 +431,22 @@ class _Builder:
         mutables = [n for n, (vid, m) in self.scope.items() if m and vid not in self.counters]
         if depth == 0:
             if mutables and r.random() < 0.5:
-                return f"(assign (lvar {self.use(r.choice(mutables))}) {self.expr(r.randint(0, 2))})"
+                return self.assign(r.choice(mutables))
             return self.store()
         pick = r.randint(0, 9)
-        if pick in (0, 1):                                   # let NAME = e in S (the value reads the outer NAME)
-            value = self.expr(r.randint(0, 2))
-            v, body = self.bound_body(r.choice(self.POOL), False, lambda: self.stmts(depth - 1, r.randint(1, 3)))
-            return f"(let {v} {value} {body})"
-        if pick in (2, 3):
-            value = self.expr(r.randint(0, 2))
-            v, body = self.bound_body(r.choice(self.POOL), True, lambda: self.stmts(depth - 1, r.randint(1, 3)))
-            return f"(letmut {v} {value} {body})"
+        if pick in (0, 1, 2, 3):                             # let [mutable] NAME = e in S (the value reads the outer NAME)
+            wide = r.random() < 0.25
+            value = self.expr64(r.randint(0, 2)) if wide else self.expr(r.randint(0, 2))
+            v, body = self.bound_body(r.choice(self.POOL), pick >= 2, lambda: self.stmts(depth - 1, r.randint(1, 3)), wide=wide)
+            return f"({'letmut' if pick >= 2 else 'let'} {v} {value} {body})"
         if pick == 4:
             other = f" {self.stmts(depth - 1, r.randint(1, 2))}" if r.random() < 0.6 else ""
             return f"(if {self.cond(1)} {self.stmts(depth - 1, r.randint(1, 2))}{other})"
         if pick in (5, 6):                                   # for NAME = lo to / downto hi
             lo, hi = self.small(self.expr(1), 2), self.small(self.expr(1), 3)
             down = r.random() < 0.4
-            moving = r.choice(mutables) if mutables and r.random() < 0.5 else None
+            narrow = [n for n in mutables if self.scope[n][0] not in self.wide]
+            moving = r.choice(narrow) if narrow and r.random() < 0.5 else None
             if moving:                                       # the far bound reads what the body goes on to change
                 bound = self.small(self.use(moving), 3)
                 lo, hi = (bound, hi) if down else (lo, bound)
