@@ -50,6 +50,30 @@ __device__ __forceinline__ float wave_sum(float v) {
   return (r0 + r1) + (r2 + r3);
 }
 
+// The same for a double: both halves moved by the same lane pattern.
+template <int Ctrl>
+__device__ __forceinline__ double dpp_add(double v) {
+  const long long bits = __builtin_bit_cast(long long, v);
+  const int lo = __builtin_amdgcn_update_dpp(0, static_cast<int>(bits), Ctrl, 0xF, 0xF, true);
+  const int hi = __builtin_amdgcn_update_dpp(0, static_cast<int>(bits >> 32), Ctrl, 0xF, 0xF, true);
+  const long long moved = (static_cast<long long>(hi) << 32) | static_cast<unsigned int>(lo);
+  return v + __builtin_bit_cast(double, moved);
+}
+__device__ __forceinline__ double readlane(double v, int lane) {
+  const long long bits = __builtin_bit_cast(long long, v);
+  const int lo = __builtin_amdgcn_readlane(static_cast<int>(bits), lane);
+  const int hi = __builtin_amdgcn_readlane(static_cast<int>(bits >> 32), lane);
+  return __builtin_bit_cast(double, (static_cast<long long>(hi) << 32) | static_cast<unsigned int>(lo));
+}
+// Sum over the 64 lanes of a wave in a fixed order; every lane of the wave takes part, the result is valid in all.
+__device__ __forceinline__ double wave_sum(double v) {
+  v = dpp_add<0xB1>(v);
+  v = dpp_add<0x4E>(v);
+  v = dpp_add<0x141>(v);
+  v = dpp_add<0x140>(v);
+  return (readlane(v, 0) + readlane(v, 16)) + (readlane(v, 32) + readlane(v, 48));
+}
+
 // Sum over a 256-thread block; valid in thread 0.
 __device__ __forceinline__ float block_sum(float v) {
   __shared__ float wave_part[kBlock / 64];
@@ -223,7 +247,7 @@ __global__ __launch_bounds__(kBlock) void triad_scalar_kernel(float *__restrict_
 }
 
 // Double sum of x[0..count) by one 1024-thread block, valid in every thread.  Each thread takes float4
-// pieces at a stride of 1024 pieces, eight loads in flight, then the wave's lanes are added by exchanges
+// pieces at a stride of 1024 pieces, eight loads in flight, then the wave's lanes are added by lane moves
 // and the sixteen waves' sums through LDS; the summation order is fixed by (count, the pointer's
 // alignment, thread layout) only.
 __device__ __forceinline__ double fold_block(const float *__restrict__ x, int64_t count) {
@@ -248,9 +272,8 @@ __device__ __forceinline__ double fold_block(const float *__restrict__ x, int64_
            (static_cast<double>(v.z) + static_cast<double>(v.w));
   }
   for (int64_t j = (n4 << 2) + threadIdx.x; j < count; j += 1024) acc += static_cast<double>(x[j]);
-  // across the lanes of a wave by exchanges (no LDS, no barrier), then the sixteen waves' sums in wave order
-#pragma unroll
-  for (int m = 32; m >= 1; m >>= 1) acc += __shfl_xor(acc, m, 64);
+  // across the lanes of a wave by lane moves (no LDS, no barrier), then the sixteen waves' sums in wave order
+  acc = wave_sum(acc);
   if ((threadIdx.x & 63) == 0) sh[threadIdx.x >> 6] = acc;
   __syncthreads();
   double total = 0.0;
@@ -278,13 +301,12 @@ struct FoldSlot {
   unsigned ticket;
   unsigned unused[63];
 };
-// The 256 stage values, one in each of the first 256 threads: four waves add theirs by exchanges, then the four sums
+// The 256 stage values, one in each of the first 256 threads: four waves add theirs by lane moves, then the four sums
 // in wave order.  Valid in thread 0.
 __device__ __forceinline__ double fold_stage(double v) {
   __shared__ double last_sums[kFoldGroups / 64];
-  if (threadIdx.x < kFoldGroups) {
-#pragma unroll
-    for (int m = 32; m >= 1; m >>= 1) v += __shfl_xor(v, m, 64);
+  if (threadIdx.x < kFoldGroups) {   // four whole waves
+    v = wave_sum(v);
     if ((threadIdx.x & 63) == 0) last_sums[threadIdx.x >> 6] = v;
   }
   __syncthreads();
@@ -314,19 +336,90 @@ __global__ __launch_bounds__(1024) void fold_onepass_kernel(const float *__restr
   }
 }
 
-// The same sum with no stage outside the workgroup: one workgroup takes the 256 pieces one after the other and keeps
-// their sums in LDS.  Piece by piece and in the last step it adds what fold_onepass_kernel adds, in that order, so
-// a long fold gives the same bits whether or not it had a stage (a launch recorded into a graph, or a stream that
-// came when every slot was taken, has none).
+// The 256 pieces of a long fold through one workgroup, for aligned pieces of at most K * 4096 elements (K 128-bit
+// loads per thread and piece): 8 / K pieces at a time, their loads asked for while the pieces before them are added
+// up, one barrier for the lot.  Thread t adds what fold_block's thread t adds to its running sum, in its order; the
+// wave's lanes and the sixteen waves' sums are added as there: stage[g] gets fold_block's bits for piece g.
+template <int K>
+__device__ __forceinline__ void fold_pieces_batched(const float *__restrict__ partials, int64_t count, int64_t piece,
+                                                    double *stage) {
+  constexpr int B = 8 / K;    // pieces per batch: eight 128-bit loads per thread in flight, which 128 registers hold
+  __shared__ double wave_sums[2][B][16];
+  const int t = threadIdx.x, lane = t & 63, wave = t >> 6;
+  auto length_of = [&](int g) {
+    const int64_t lo = static_cast<int64_t>(g) * piece;
+    return lo >= count ? int64_t{0} : (count - lo < piece ? count - lo : piece);
+  };
+  float4 next[B * K];
+  auto load_batch = [&](int b) {
+#pragma unroll
+    for (int q = 0; q < B; ++q) {
+      const int g = b * B + q;
+      const int64_t n4 = length_of(g) >> 2;
+      const float4 *p4 = reinterpret_cast<const float4 *>(partials + static_cast<int64_t>(g) * piece);
+#pragma unroll
+      for (int k = 0; k < K; ++k) next[q * K + k] = t + k * 1024 < n4 ? p4[t + k * 1024] : make_float4(0.f, 0.f, 0.f, 0.f);
+    }
+  };
+  load_batch(0);
+  for (int b = 0; b < kFoldGroups / B; ++b) {
+    double acc[B];
+#pragma unroll
+    for (int q = 0; q < B; ++q) {
+      const int g = b * B + q;
+      const int64_t len = length_of(g), n4 = len >> 2;
+      acc[q] = 0.0;
+#pragma unroll
+      for (int k = 0; k < K; ++k)
+        if (t + k * 1024 < n4) {
+          const float4 v = next[q * K + k];
+          acc[q] += (static_cast<double>(v.x) + static_cast<double>(v.y)) + (static_cast<double>(v.z) + static_cast<double>(v.w));
+        }
+      // the last, short four of the whole input
+      if ((n4 << 2) + t < len) acc[q] += static_cast<double>(partials[static_cast<int64_t>(g) * piece + (n4 << 2) + t]);
+    }
+    if (b + 1 < kFoldGroups / B) load_batch(b + 1);
+#pragma unroll
+    for (int q = 0; q < B; ++q) {
+      const double s = wave_sum(acc[q]);
+      if (lane == 0) wave_sums[b & 1][q][wave] = s;
+    }
+    __syncthreads();
+    if (t < B) {
+      double total = 0.0;
+#pragma unroll
+      for (int w = 0; w < 16; ++w) total += wave_sums[b & 1][t][w];
+      stage[b * B + t] = total;
+    }
+    // no second barrier: the next batch writes the other half of wave_sums, and the one after it comes after the
+    // next barrier, which these readers reach only when they have read
+  }
+  __syncthreads();
+}
+
+// The same sum with no stage outside the workgroup: one workgroup takes the 256 pieces itself and keeps their sums
+// in LDS.  Piece by piece and in the last step it adds what fold_onepass_kernel adds, in that order, so a long fold
+// gives the same bits whether or not it had a stage (a launch recorded into a graph, or a stream that came when every
+// slot was taken, has none).  Aligned folds of up to 2^22 partials take the batched walk above; longer or unaligned
+// ones go through fold_block piece by piece.
 __global__ __launch_bounds__(1024) void fold_pieces_kernel(const float *__restrict__ partials, int64_t count,
                                                            int64_t piece, double *__restrict__ out) {
   __shared__ double stage[kFoldGroups];
-  for (int g = 0; g < kFoldGroups; ++g) {
-    const int64_t lo = static_cast<int64_t>(g) * piece;
-    const int64_t len = lo >= count ? 0 : (count - lo < piece ? count - lo : piece);
-    const double t = fold_block(partials + lo, len);
-    if (threadIdx.x == 0) stage[g] = t;
-    __syncthreads();   // fold_block's own LDS is free again, stage[g] is written
+  const bool aligned = (reinterpret_cast<uintptr_t>(partials) & 15u) == 0;
+  if (aligned && piece <= 4096) {
+    fold_pieces_batched<1>(partials, count, piece, stage);
+  } else if (aligned && piece <= 8192) {
+    fold_pieces_batched<2>(partials, count, piece, stage);
+  } else if (aligned && piece <= 16384) {
+    fold_pieces_batched<4>(partials, count, piece, stage);
+  } else {
+    for (int g = 0; g < kFoldGroups; ++g) {
+      const int64_t lo = static_cast<int64_t>(g) * piece;
+      const int64_t len = lo >= count ? 0 : (count - lo < piece ? count - lo : piece);
+      const double t = fold_block(partials + lo, len);
+      if (threadIdx.x == 0) stage[g] = t;
+      __syncthreads();   // fold_block's own LDS is free again, stage[g] is written
+    }
   }
   const double total = fold_stage(threadIdx.x < kFoldGroups ? stage[threadIdx.x] : 0.0);
   if (threadIdx.x == 0) *out = total;

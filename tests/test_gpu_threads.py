@@ -81,15 +81,17 @@ def test_four_threads_on_four_streams(hip, torch_cuda):
 
 def test_long_folds_on_more_streams_than_the_library_has_stages(hip, torch_cuda):
     """Long folds keep their per-workgroup sums in one of sixteen stages a device holds, one per stream; a stream
-    that comes when all are taken folds with one workgroup.  Twenty-four streams, three lengths (an unaligned one
-    among them): every sum is, bit for bit, the one the default stream gives."""
+    that comes when all are taken folds with one workgroup.  Twenty-four streams, seven lengths (one, two, four and
+    more loads per thread and piece, unaligned ones among them): every sum is, bit for bit, the one the default
+    stream gives."""
     torch = torch_cuda
     g = torch.Generator(device="cuda")
     g.manual_seed(3)
     streams = {torch.cuda.Stream().cuda_stream: None for _ in range(64)}
     streams = [torch.cuda.ExternalStream(s) for s in streams][:24]
     assert len(streams) == 24
-    for n, offset in (((1 << 17) + 0, 0), ((1 << 20) + 77, 0), ((1 << 19) + 5, 1)):
+    for n, offset in (((1 << 17) + 0, 0), ((1 << 20) - 3, 0), ((1 << 19) + 5, 1), ((1 << 21) - 77, 0), ((1 << 22) - 3, 0),
+                      ((1 << 22) + 4096, 0), ((1 << 21) + 1, 3)):
         x = (torch.rand(n + offset, device="cuda", generator=g) * 100)[offset:]
         want = torch.zeros(1, dtype=torch.float64, device="cuda")
         hip.check(hip.lib.sarek_hip_fold_partials_f64(x.data_ptr(), n, want.data_ptr(), None))
