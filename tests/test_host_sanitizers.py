@@ -21,6 +21,10 @@ def damaged_texts(count, seed):
     rng = random.Random(seed)
     texts = [open(f).read() for f in sorted(glob.glob(os.path.join(HERE, "golden", "ir", "*.ir")))]
     texts += [rk.histogram(), rk.nbody_accel(), rk.conv2d(), rk.inclusive_scan(), rk.stencil_2d()]
+    # names bound again, loops with moving bounds, helper functions, int64, matches with payloads and variable patterns
+    import ir_programs
+    from test_ir_lowering import MATCH_AS_A_VALUE, MATCH_WITH_A_VARIABLE_PATTERN
+    texts += [ir_programs.random_program(s)[0] for s in range(10)] + [MATCH_AS_A_VALUE, MATCH_WITH_A_VARIABLE_PATTERN]
     spare = ["i32", "f32", "(var x 1 i32)", "add", "read", "let", "seq", "(i32 0)", "shared", "vec", "-",
              "99999999999999999999", '"', "template", "match", "case", "record", "variant", "app", "for", "upto",
              "mut", "output", "a"]
