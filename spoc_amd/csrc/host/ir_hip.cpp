@@ -681,8 +681,12 @@ std::string gen_stmt(const StmtP &sp, const std::string &indent) {
         }
         t_in_shared_size = false;
         Binding array(s.var);
-        return indent + (s.e->mem == MemSpace::Shared ? "__shared__ " : "") + type_str(s.e->type) + " " +
-               array.printed + "[" + size + "];\n" + gen_stmt(s.stmts[0], indent);
+        // An array a thread creates for itself starts at zero on the CPU backends (`Array.make size default`,
+        // Sarek_native_gen.ml:466-469; the reference's IR walker likewise): `= {}` here, where the reference's text
+        // leaves it uninitialised.  Shared arrays stay as declared: every kernel writes them before it reads.
+        const bool shared = s.e->mem == MemSpace::Shared;
+        return indent + (shared ? "__shared__ " : "") + type_str(s.e->type) + " " + array.printed + "[" + size + "]" +
+               (shared ? "" : " = {}") + ";\n" + gen_stmt(s.stmts[0], indent);
       }
       if (s.var.type && s.var.type->kind == Type::Unit) {
         // `let () = e in body` (Sarek_lower_ir.ml:448-470 lowers it like any let): nothing to declare -- the

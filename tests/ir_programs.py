@@ -106,6 +106,8 @@ class Thread:
             return self.lookup(e)
         if head == "read":
             return int(self.arrays[e[1]][self.expr(e[2])])
+        if head == "len":
+            return len(self.arrays[e[1]])
         if head == "intr":
             name = e[2]
             if name in ("global_thread_id", "global_idx_x", "global_idx"):
@@ -185,7 +187,11 @@ class Thread:
         elif head == "block":
             self.stmt(s[1])
         elif head in ("let", "letmut"):
-            self.bind(s[1], self.expr(s[2]))
+            if s[2][0] == "newarray":                       # an array of the thread's own: zeros (Sarek_ir_interp.ml:908-931)
+                self.arrays = dict(self.arrays)
+                self.arrays[s[1][1]] = [0] * self.expr(s[2][2])
+            else:
+                self.bind(s[1], self.expr(s[2]))
             self.stmt(s[3])
         elif head == "assign":
             value, target = self.expr(s[2]), s[1]

@@ -323,3 +323,21 @@ def test_ocaml_constants_a_kernel_names(hip, torch_cuda):
     got = {"d": d.to_array(), "i": i.to_array(), "l": l.to_array()}
     for k, (e, v, want) in enumerate(stores):
         assert got[v][k] == want, (e, got[v][k], want)
+
+
+def test_the_references_known_answers_for_ir_semantics(hip, torch_cuda):
+    """The cases of sarek/tests/unit/test_ir_interp.ml (array read, length and creation, a record's field, a
+    variant's payload, conditionals, casts, operators, assignment, let, while, for, the conversions to int32 and to
+    bool), lowered, compiled and run by one thread: every result is the one the reference's test asserts."""
+    import interp_cases
+    from spoc_amd.sarek import Execute, Transfer, Vector
+    data, seven = Vector.of_array(np.array([10, 20, 30], np.int32)), Vector.of_array(np.zeros(7, np.int32))
+    out, fout = Vector.of_array(np.full(32, -7, np.int32)), Vector.of_array(np.full(4, -7, np.float32))
+    path = Execute.run_vectors(ir=interp_cases.kernel(), args=[Execute.Vec(data), Execute.Vec(seven), Execute.Vec(out), Execute.Vec(fout)],
+                               block=Execute.dims1d(64), grid=Execute.dims1d(1))
+    Transfer.flush()
+    assert path == "jit"
+    got = out.to_array()
+    for k, want in interp_cases.EXPECTED.items():
+        assert got[k] == want, (k, got[k], want)
+    assert fout.to_array()[0] == 42.0

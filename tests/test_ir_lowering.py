@@ -882,3 +882,21 @@ def test_a_pattern_that_names_the_value(hip):
     assert "dst[tid] = ((other.tag == Rect) ? (other.data.Rect_v._0 * other.data.Rect_v._1) : -1.0f);" in text
     with pytest.raises(hip.SarekHipError):
         hip.generate_source(MATCH_WITH_A_VARIABLE_PATTERN.replace("(? other)", "(? other more)"))
+
+
+def test_the_program_model_on_the_references_known_answers(hip):
+    """The integer cases of the reference's own unit tests for its IR walker (tests/interp_cases.py), through the
+    tests' walker: the model the seeded programs are held to gives the reference's answers."""
+    import numpy as np
+    import interp_cases
+    import ir_programs
+    out = np.full(32, -7, np.int32)
+    arrays = {"data": np.array([10, 20, 30], np.int32), "seven": np.zeros(7, np.int32), "out": out,
+              "fout": np.zeros(1, np.float32)}
+    ir_programs.evaluate(interp_cases.kernel(only_integers=True), arrays, 1)
+    for k, want in interp_cases.EXPECTED.items():
+        if k not in (3, 4, 7, 18):
+            assert out[k] == want, k
+    # and the whole kernel lowers to text the device compiler takes
+    text = hip.generate_source(interp_cases.kernel())
+    assert "int a[5] = {};" in text and "out[7] = (int)42.700000000000003f;" in text
