@@ -242,6 +242,14 @@ typedef struct {
  * let%shared lowers to block_dim_x elements, sarek/ppx/Sarek_lower_ir.ml:496-507) is
  * emitted as the constant a __shared__ declaration needs; the reference's generators
  * leave blockDim.x there, which no device compiler accepts.
+ * The text is what sarek-cuda/Sarek_ir_cuda.ml:751-786 prints for the same IR -- byte for
+ * byte on the reference's golden kernels -- except where that text does not compile or
+ * computes something else than the CPU backends do: a name bound again gets a variable of
+ * its own (x_2, ...), a `for` bound the body may change is evaluated once, a match used as
+ * a value binds its cases' variables, variable patterns and lets of type unit are taken,
+ * infinities / NaN / the least integers / whole-valued doubles are spelled so that they
+ * keep their value and type, a thread's own arrays start at zero, the standard library's
+ * logical shifts give a signed value.
  * Writes at most out_len bytes incl. NUL; *needed gets the full size.          */
 int sarek_hip_generate_source(const char *ir_text, const int block[3], char *out, size_t out_len,
                               size_t *needed);
