@@ -340,7 +340,8 @@ class _Builder:
                 return f"(i32 {r.randint(-9, 12)})"
             if pick == 1 and not self.in_helper:
                 return f"(read x {self.use('tid')})"
-            return self.use(r.choice(self.ints_in_scope()))
+            ints = self.ints_in_scope()                      # none when int64 lets hide a helper's every parameter
+            return self.use(r.choice(ints)) if ints else f"(i32 {r.randint(-9, 12)})"
         if r.random() < 0.1:                                 # the low or the high half of an int64 value
             wide = self.expr64(depth - 1)
             return r.choice([f"(cast i32 {wide})", f"(cast i32 (intr (Int64) shift_right_logical {wide} (i32 32)))"])
