@@ -48,3 +48,54 @@ def test_loop_bounds_the_body_changes(hip, sarek):
     for name, (body, _, want) in LOOP_BOUNDS.items():
         (got,) = run(sarek, kernel_with_body(body, REBOUND_PARAMS), [np.full(8, -1, np.int32)], [3], block=1)
         assert got.tolist() == want, name
+
+
+@pytest.mark.parametrize("seed", range(12))
+def test_seeded_parameter_lists_arrive_as_given(hip, sarek, seed):
+    """Kernels with four to twelve parameters in a seeded order -- int32, int64, float32 and float64 scalars between
+    the four output vectors, each vector followed by its injected length -- store every scalar and every length
+    into the output of its type: what arrives is what was passed, whatever the mix does to the alignment of the
+    parameter block."""
+    import random
+    rng = random.Random(9000 + seed)
+    E, T, V = sarek.Execute, sarek.Transfer, sarek.Vector
+    kinds = {"i32": (V.int32, np.int32, E.Int32), "i64": (V.int64, np.int64, E.Int64),
+             "f32": (V.float32, np.float32, E.Float32), "f64": (V.float64, np.float64, E.Float64)}
+    outs = {t: (f"o_{t}", rng.randint(5, 40)) for t in kinds}                      # output vector of each type, its length
+    params = [("vec", t) for t in kinds] + [("scalar", rng.choice(list(kinds))) for _ in range(rng.randint(0, 8))]
+    rng.shuffle(params)
+    decls, args, stores, want, slot, vid = [], [], [], {t: {} for t in kinds}, {t: 0 for t in kinds}, 1
+    vectors = {}
+    for what, t in params:
+        if what == "vec":
+            name, length = outs[t]
+            decls.append(f"(param (var {name} {vid} (vec {t})))")
+            vectors[t] = V.of_array(np.full(length, 77, kinds[t][1]))
+            args.append(E.Vec(vectors[t]))
+        else:
+            name = f"s{vid}"
+            value = {"i32": rng.randint(-2**31, 2**31 - 1), "i64": rng.randint(-2**63, 2**63 - 1),
+                     "f32": float(np.float32(rng.uniform(-1e6, 1e6))), "f64": rng.uniform(-1e300, 1e300)}[t]
+            decls.append(f"(param (var {name} {vid} {t}))")
+            args.append(kinds[t][2](value))
+            stores.append(f"(assign (lelem {outs[t][0]} (i32 {slot[t]})) (var {name} {vid} {t}))")
+            want[t][slot[t]] = value
+            slot[t] += 1
+        vid += 1
+    for t in kinds:                                         # every vector's injected length, into the int32 output
+        stores.append(f"(assign (lelem o_i32 (i32 {slot['i32']})) (len {outs[t][0]}))")
+        want["i32"][slot["i32"]] = outs[t][1]
+        slot["i32"] += 1
+    assert max(slot.values()) <= 5 + 8
+    outs_len_ok = all(slot[t] <= outs[t][1] for t in kinds)
+    if not outs_len_ok:
+        pytest.skip("more scalars of a type than its output holds")
+    ir = (f"(kernel sarek_kern (params {' '.join(decls)}) (locals) (body (if (eq (intr (Std) global_thread_id) (i32 0)) "
+          f"(seq {' '.join(stores)}))) (native_fn true))")
+    assert E.run_vectors(ir, args, (64, 1, 1), (1, 1, 1)) == "jit"
+    T.flush()
+    for t in kinds:
+        got = vectors[t].to_array()
+        for k, value in want[t].items():
+            assert got[k] == kinds[t][1](value), (seed, t, k, got[k], value)
+        assert (got[slot[t]:] == 77).all(), (seed, t)
