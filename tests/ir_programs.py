@@ -20,6 +20,17 @@ SLOTS = 4
 INT_MIN, INT_MAX = -(1 << 31), (1 << 31) - 1
 
 
+class Inexact(Exception):
+    """A float program left the values float32 holds exactly."""
+
+
+def _exact(v):
+    import struct
+    if struct.unpack("f", struct.pack("f", v))[0] != v:
+        raise Inexact()
+    return v
+
+
 class _Return(Exception):
     def __init__(self, value):
         self.value = value
@@ -98,20 +109,40 @@ class Thread:
         head = e[0]
         if head in ("i32", "i64"):
             return int(e[1])
-        if head == "cast":                                  # Int64.of_int32 keeps the value, Int64.to_int32 its low 32 bits
-            return _fit(self.expr(e[2]), 64 if e[1] == "i64" else 32)
+        if head in ("f32", "f64"):
+            return float(e[1])
+        if head == "cast":
+            v = self.expr(e[2])
+            if e[1] in ("f32", "f64"):                      # the float programs keep to values both float types hold
+                return float(v)
+            if isinstance(v, float):                        # Int32.of_float: towards zero
+                v = int(v)
+            return _fit(v, 64 if e[1] == "i64" else 32)     # Int64.of_int32 keeps the value, to_int32 its low 32 bits
         if head == "bool":
             return e[1] == "true"
         if head == "var":
             return self.lookup(e)
         if head == "read":
-            return int(self.arrays[e[1]][self.expr(e[2])])
+            v = self.arrays[e[1]][self.expr(e[2])]
+            return float(v) if isinstance(v, float) or getattr(v, "dtype", None) is not None and v.dtype.kind == "f" else int(v)
         if head == "len":
             return len(self.arrays[e[1]])
         if head == "intr":
             name = e[2]
             if name in ("global_thread_id", "global_idx_x", "global_idx"):
                 return self.index
+            if e[1][-1] in ("Float32", "Float64"):          # sarek/Sarek_stdlib/Float32.ml:41-157, Sarek_float64/Float64.ml
+                import math
+                args = [self.expr(a) for a in e[3:] if not (isinstance(a, list) and a and a[0] == "template")]
+                if name == "floor": return math.copysign(float(math.floor(args[0])), args[0]) if math.floor(args[0]) == 0 else float(math.floor(args[0]))
+                if name == "ceil": return math.copysign(float(math.ceil(args[0])), args[0]) if math.ceil(args[0]) == 0 else float(math.ceil(args[0]))
+                if name == "abs_float": return abs(args[0])
+                if name in ("min", "max"): return min(args) if name == "min" else max(args)
+                if name in ("of_int", "of_float32", "of_float64"): return float(args[0])
+                if name == "to_int": return _fit(int(args[0]))
+                if name in ("add", "minus", "mul"):
+                    return _exact({"add": args[0] + args[1], "minus": args[0] - args[1], "mul": args[0] * args[1]}[name])
+                raise KeyError(name)
             assert e[1][-1] in ("Int32", "Int64"), e        # Stdlib.Int32 / Int64 (sarek/Sarek_stdlib/Int32.ml:30-88, Int64.ml)
             bits = 64 if e[1][-1] == "Int64" else 32
             args = [self.expr(a) for a in e[3:] if not (isinstance(a, list) and a and a[0] == "template")]
@@ -142,12 +173,15 @@ class Thread:
             raise AssertionError("a helper ended without a return")
         bits = width(e)
         if head == "neg":
-            return _fit(-self.expr(e[1]), bits)
+            v = self.expr(e[1])
+            return -v if isinstance(v, float) else _fit(-v, bits)
         if head == "bitnot":
             return ~self.expr(e[1])
         if head == "not":
             return not self.expr(e[1])
         a, b = self.expr(e[1]), self.expr(e[2])
+        if isinstance(a, float) and head in ("add", "sub", "mul", "div"):
+            return _exact({"add": a + b, "sub": a - b, "mul": a * b, "div": a / b if head == "div" else 0.0}[head])
         if head == "add": return _fit(a + b, bits)
         if head == "sub": return _fit(a - b, bits)
         if head == "mul": return _fit(a * b, bits)
@@ -232,7 +266,7 @@ def evaluate(ir, arrays, threads):
         t = Thread(vectors, index, funcs)
         for p in params:
             if not isinstance(p[3], list):
-                t.bind(p, int(arrays[p[1]]))
+                t.bind(p, float(arrays[p[1]]) if p[3] in ("f32", "f64") else int(arrays[p[1]]))
         t.stmt(body)
 
 
@@ -510,3 +544,113 @@ def expected(ir, x, k, threads):
     out = np.full(SLOTS * threads, -1, np.int32)
     evaluate(ir, {"x": x.copy(), "out": out, "k": k, "n": threads}, threads)
     return out
+
+
+class _Floats:
+    """Float programs whose every value is a multiple of 1/8 below 2^15 in size, so that float32 and float64 hold it
+    exactly and a fused multiply-add gives what a multiplication and an addition give: sums and differences of
+    leaves, products with powers of two, negations, conditionals, floor / ceil / abs, conversions
+    between int32, float32 and float64.  Lets of both float types hide each other as in the integer programs."""
+    POOL = ["a", "b", "c", "s"]            # s is a parameter's name too
+
+    def __init__(self, rng):
+        self.rng, self.next_id = rng, 10
+        self.scope = {"s": (3, "f32")}     # name -> (id, type); the vectors and n are used by name below
+
+    def use(self, name):
+        vid, ty = self.scope[name]
+        return f"(var {name} {vid} {ty})", ty
+
+    def leaf(self, ty):
+        r = self.rng
+        names = [n for n, (_, t) in self.scope.items() if t == ty]
+        pick = r.randint(0, 4)
+        if pick == 0 and names:
+            return self.use(r.choice(names))[0]
+        if pick == 1:
+            read = "(read x (var tid 5 i32))"
+            return read if ty == "f32" else f"(intr (Float64) of_float32 {read})"
+        if pick == 2:
+            return f"(cast {ty} (bitand (var tid 5 i32) (i32 31)))"
+        if pick == 3:
+            other = "f64" if ty == "f32" else "f32"
+            names = [n for n, (_, t) in self.scope.items() if t == other]
+            if names:
+                return f"(cast {ty} {self.use(r.choice(names))[0]})"
+        return f"({ty} {r.randint(-64, 64) / 8})"
+
+    def expr(self, ty, depth):
+        r = self.rng
+        if depth == 0:
+            return self.leaf(ty)
+        a, b = self.expr(ty, depth - 1), self.expr(ty, depth - 1)
+        module = "Float32" if ty == "f32" else "Float64"
+        pick = r.randint(0, 9)
+        if pick <= 1:
+            return f"({r.choice(['add', 'sub'])} {a} {b})"
+        if pick == 2:
+            return f"(mul {a} ({ty} {r.choice([0.5, 2.0, -1.0, 0.25, 4.0, 1.0, -2.0])}))"
+        if pick == 3:
+            return f"(neg {a})"
+        if pick == 4:
+            return f"(if ({r.choice(['lt', 'le', 'gt', 'ge', 'eq', 'ne'])} {a} {b}) {a} {b})"
+        if pick == 5:
+            return f"(intr ({module}) {r.choice(['floor', 'ceil', 'abs_float'])} {a})"
+        if pick == 6:                                        # (no min / max: which of -0 and +0 is the smaller is nobody's law)
+            return f"(if (lt {a} {b}) {b} {a})"
+        if pick == 7:                                        # through int32 and back: towards zero
+            return f"(intr ({module}) of_int (cast i32 {a}))"
+        if pick == 8:
+            return f"(div {a} ({ty} {r.choice([2.0, 4.0, -2.0, 0.5])}))"
+        return f'(intr ({module}) add (template "(%s + %s)") {a} {b})'
+
+    def body(self, lets):
+        r = self.rng
+        if lets == 0:
+            stores = []
+            for slot in range(SLOTS):
+                ty = r.choice(["f32", "f64"])
+                value = self.expr(ty, r.randint(0, 2))
+                target = "out" if ty == "f32" else "wide"
+                stores.append(f"(assign (lelem {target} (add (mul (var tid 5 i32) (i32 {SLOTS})) (i32 {slot}))) {value})")
+            return "(seq " + " ".join(stores) + ")"
+        ty = r.choice(["f32", "f64"])
+        value = self.expr(ty, r.randint(0, 2))
+        name, vid = r.choice(self.POOL), self.next_id
+        self.next_id += 1
+        hidden = self.scope.get(name)
+        self.scope[name] = (vid, ty)
+        inner = self.body(lets - 1)
+        if hidden is None:
+            del self.scope[name]
+        else:
+            self.scope[name] = hidden
+        return f"(let (var {name} {vid} {ty}) {value} {inner})"
+
+
+def random_float_program(seed, threads=24):
+    """(ir, x, s) over (x : float32 vector, out : float32 vector, s : float32, wide : float64 vector, n : int32):
+    thread tid < n stores SLOTS values into out or wide (a slot left alone keeps what the vector held)."""
+    import numpy as np
+    for attempt in range(100):                              # the first candidate whose every value float32 holds exactly
+        rng = random.Random(500000 + seed * 100 + attempt)
+        b = _Floats(rng)
+        body = b.body(rng.randint(2, 6))
+        ir = ("(kernel sarek_kern (params (param (var x 1 (vec f32))) (param (var out 2 (vec f32))) (param (var s 3 f32)) "
+              "(param (var wide 6 (vec f64))) (param (var n 4 i32))) (locals) (body (let (var tid 5 i32) "
+              f"(intr (Std) global_thread_id) (if (lt (var tid 5 i32) (var n 4 i32)) {body}))) (native_fn true))")
+        x = np.array([rng.randint(-64, 64) / 8 for _ in range(threads)], np.float32)
+        s = rng.randint(-32, 32) / 8
+        try:
+            expected_floats(ir, x, s, threads)
+        except Inexact:
+            continue
+        return ir, x, s
+    raise RuntimeError(f"seed {seed}: no exact candidate")
+
+
+def expected_floats(ir, x, s, threads):
+    import numpy as np
+    out, wide = np.full(SLOTS * threads, -1, np.float32), np.full(SLOTS * threads, -1, np.float64)
+    evaluate(ir, {"x": x.copy(), "out": out, "wide": wide, "s": s, "n": threads}, threads)
+    return out, wide

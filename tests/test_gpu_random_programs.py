@@ -99,3 +99,22 @@ def test_seeded_parameter_lists_arrive_as_given(hip, sarek, seed):
         for k, value in want[t].items():
             assert got[k] == kinds[t][1](value), (seed, t, k, got[k], value)
         assert (got[slot[t]:] == 77).all(), (seed, t)
+
+
+@pytest.mark.parametrize("seed", range(int(os.environ.get("SAREK_HIP_TEST_PROGRAM_SEEDS", "48")) // 2))
+def test_seeded_float_programs_compute_what_the_walker_computes(hip, sarek, seed):
+    """Float programs whose every value both float types hold exactly (multiples of 1/8 and of powers of two, small):
+    sums, products with powers of two, conditionals, floor / ceil / abs, conversions between int32,
+    float32 and float64, lets of both types that hide each other.  Nothing is rounded anywhere, so the device's
+    float32 and float64 arithmetic, fused or not, gives the walker's values bit for bit."""
+    E, T, V = sarek.Execute, sarek.Transfer, sarek.Vector
+    ir, x, s = ir_programs.random_float_program(seed, THREADS)
+    want, want_wide = ir_programs.expected_floats(ir, x, s, THREADS)
+    out = V.of_array(np.full(ir_programs.SLOTS * THREADS, -1, np.float32))
+    wide = V.of_array(np.full(ir_programs.SLOTS * THREADS, -1, np.float64))
+    path = E.run_vectors(ir, [E.Vec(V.of_array(x)), E.Vec(out), E.Float32(s), E.Vec(wide), E.Int32(THREADS)], (32, 1, 1), (1, 1, 1))
+    T.flush()
+    assert path in ("jit", "map_f32")
+    got, got_wide = out.to_array(), wide.to_array()
+    assert np.array_equal(got.view(np.uint32), want.view(np.uint32)), (seed, np.flatnonzero(got != want)[:8].tolist())
+    assert np.array_equal(got_wide.view(np.uint64), want_wide.view(np.uint64)), (seed, np.flatnonzero(got_wide != want_wide)[:8].tolist())
