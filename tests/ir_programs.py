@@ -96,6 +96,7 @@ class Thread:
     def __init__(self, arrays, index, funcs=None):
         self.by_id, self.by_name, self.arrays, self.index, self.steps = {}, {}, arrays, index, 0
         self.funcs = funcs or {}
+        self.geometry = {}
 
     def bind(self, var, value):
         self.by_id[int(var[2])] = value
@@ -131,6 +132,8 @@ class Thread:
             name = e[2]
             if name in ("global_thread_id", "global_idx_x", "global_idx"):
                 return self.index
+            if name in ("thread_idx_x", "block_idx_x", "block_dim_x", "grid_dim_x"):
+                return self.geometry[name]
             if e[1][-1] in ("Float32", "Float64"):          # sarek/Sarek_stdlib/Float32.ml:41-157, Sarek_float64/Float64.ml
                 import math
                 args = [self.expr(a) for a in e[3:] if not (isinstance(a, list) and a and a[0] == "template")]
@@ -654,3 +657,92 @@ def expected_floats(ir, x, s, threads):
     out, wide = np.full(SLOTS * threads, -1, np.float32), np.full(SLOTS * threads, -1, np.float64)
     evaluate(ir, {"x": x.copy(), "out": out, "wide": wide, "s": s, "n": threads}, threads)
     return out, wide
+
+
+def evaluate_blocks(ir, arrays, block, grid):
+    """Runs a kernel of the shape `let <shared arrays and thread-private bindings> in (seq S1 (barrier) S2 ...)` block
+    by block: the bindings in front of the sequence per thread, then the statements between two barriers for every
+    thread of the block in turn (a superstep: the programs below read only what an earlier superstep wrote and
+    write only their own slots, so the order of the threads inside one does not matter -- Sarek_cpu_runtime.ml:686-782
+    runs them in that order too)."""
+    kernel = parse(ir)
+    sections = {item[0]: item for item in kernel[2:] if isinstance(item, list)}
+    params = [p[1] for p in sections["params"][1:]]
+    vectors = {p[1]: arrays[p[1]] for p in params if isinstance(p[3], list)}
+    for b in range(grid):
+        shared = dict(vectors)
+        threads = []
+        for t in range(block):
+            th = Thread(shared, b * block + t)
+            th.geometry = {"thread_idx_x": t, "block_idx_x": b, "block_dim_x": block, "grid_dim_x": grid}
+            for p in params:
+                if not isinstance(p[3], list):
+                    th.bind(p, int(arrays[p[1]]))
+            threads.append(th)
+        # the bindings in front of the sequence: shared arrays once per block, the rest per thread
+        node = sections["body"][1]
+        while node[0] in ("let", "letmut"):
+            if node[2][0] == "newarray":
+                assert node[2][3] == "shared"
+                shared[node[1][1]] = [0] * threads[0].expr(node[2][2])
+            else:
+                for th in threads:
+                    th.bind(node[1], th.expr(node[2]))
+            node = node[3]
+        assert node[0] == "seq"
+        for statement in node[1:]:
+            if statement[0] == "barrier":
+                continue
+            for th in threads:
+                th.stmt(statement)
+
+
+def random_block_program(seed, block=64, grid=3):
+    """(ir, x, k): supersteps over two shared int32 arrays of one element per thread.  A superstep writes the
+    thread's own slot of one array (and, now and then, its running value) from its running value, its indices and
+    slots of the arrays written in earlier supersteps, at seeded offsets and strides round the block; the last one
+    stores the running value to out[global id]."""
+    import numpy as np
+    rng = random.Random(900000 + seed)
+    tid, gid = "(var tid 10 i32)", "(var gid 11 i32)"
+    acc = "(var acc 12 i32 mut)"
+    arrays = ["tile", "other"]
+    written = set()
+
+    def slot_of(other_thread):
+        return f"(mod (add (mul {tid} (i32 {rng.choice([1, 1, 3, 5, 7])})) (i32 {other_thread})) (intr (Gpu) block_dim_x))"
+
+    def value(depth):
+        if depth == 0:
+            pick = rng.randint(0, 5)
+            if pick == 0 and written:
+                return f"(read {rng.choice(sorted(written))} {slot_of(rng.randint(0, 63))})"
+            return [acc, tid, gid, f"(i32 {rng.randint(-9, 9)})", "(var k 3 i32)", "(intr (Gpu) block_idx_x)"][pick]
+        a, b = value(depth - 1), value(depth - 1)
+        op = rng.choice(["add", "sub", "mul", "bitxor", "bitand", "bitor"])
+        return f"({op} {a} {b})" if op != "mul" else f"(mul (bitand {a} (i32 255)) (bitand {b} (i32 255)))"
+
+    steps = []
+    for _ in range(rng.randint(2, 6)):
+        target = rng.choice(arrays)
+        # a superstep may read the array it is about to overwrite only through the running value it took before
+        readable = written - {target}
+        saved, written_now = written, readable
+        written = readable
+        body = [f"(assign (lelem {target} {tid}) {value(rng.randint(1, 2))})"]
+        if rng.random() < 0.6:
+            body.append(f"(assign (lvar {acc}) {value(rng.randint(1, 2))})")
+        written = saved | {target}
+        rng.shuffle(body)
+        steps.append(f"(block (seq {' '.join(body)}))" if rng.random() < 0.5 else " ".join(body))
+        steps.append("(barrier)")
+    final = value(2)
+    steps.append(f"(assign (lelem out {gid}) {final})")
+    body = (f"(let (var tile 20 (array i32 shared)) (newarray i32 (intr (Gpu) block_dim_x) shared) "
+            f"(let (var other 21 (array i32 shared)) (newarray i32 (i32 {block}) shared) "
+            f"(let {tid} (intr (Gpu) thread_idx_x) (let {gid} (intr (Std) global_thread_id) "
+            f"(letmut {acc} (read x {gid}) (seq {' '.join(steps)}))))))")
+    ir = ("(kernel sarek_kern (params (param (var x 1 (vec i32))) (param (var out 2 (vec i32))) (param (var k 3 i32))) "
+          f"(locals) (body {body}) (native_fn true))")
+    x = np.array([rng.randint(-100, 100) for _ in range(block * grid)], np.int32)
+    return ir, x, rng.randint(-5, 9)

@@ -118,3 +118,21 @@ def test_seeded_float_programs_compute_what_the_walker_computes(hip, sarek, seed
     got, got_wide = out.to_array(), wide.to_array()
     assert np.array_equal(got.view(np.uint32), want.view(np.uint32)), (seed, np.flatnonzero(got != want)[:8].tolist())
     assert np.array_equal(got_wide.view(np.uint64), want_wide.view(np.uint64)), (seed, np.flatnonzero(got_wide != want_wide)[:8].tolist())
+
+
+@pytest.mark.parametrize("seed", range(int(os.environ.get("SAREK_HIP_TEST_PROGRAM_SEEDS", "48")) // 2))
+def test_seeded_supersteps_over_shared_arrays(hip, sarek, seed):
+    """Block-level programs: two shared arrays (one sized by the block dimension), two to six supersteps separated by
+    barriers, each writing the thread's own slot from slots other threads wrote in earlier supersteps (seeded strides
+    and offsets round the block), three blocks of 64 threads.  The walker runs a block superstep by superstep; every
+    element of the output is its."""
+    E, T, V = sarek.Execute, sarek.Transfer, sarek.Vector
+    block, grid = 64, 3
+    ir, x, k = ir_programs.random_block_program(seed, block, grid)
+    want = np.full(x.size, -1, np.int32)
+    ir_programs.evaluate_blocks(ir, {"x": x.copy(), "out": want, "k": k}, block, grid)
+    out = V.of_array(np.full(x.size, -1, np.int32))
+    assert E.run_vectors(ir, [E.Vec(V.of_array(x)), E.Vec(out), E.Int32(k)], (block, 1, 1), (grid, 1, 1)) == "jit"
+    T.flush()
+    got = out.to_array()
+    assert np.array_equal(got, want), (seed, np.flatnonzero(got != want)[:8].tolist())
