@@ -1,19 +1,23 @@
-"""Seeded integer programs in the IR, and what one thread of them computes.
+"""Seeded programs in the IR, and what they compute.
 
 `evaluate` walks the IR text the way the reference's own walker does (sarek/sarek/Sarek_ir_interp.ml: variables by
 binding id, then by name :76-91; Int32 operators :171-266 -- `shr` on non-negative operands only, where filling with
-zeros and with the sign agree; statements :844-941 -- a `for` evaluates both bounds once and is inclusive :858-872).
-It is a model for tests, over the integer subset the generator below emits: no floats, no records, no barriers, one
-thread at a time (the programs touch no memory another thread writes).
+zeros and with the sign agree; statements :844-941 -- a `for` evaluates both bounds once and is inclusive :858-872),
+one thread after the other; `evaluate_blocks` runs a kernel with barriers superstep by superstep.  It is a model
+for tests, over the subset the generators below emit: int32 and int64 arithmetic modulo 2^32 / 2^64, floats only
+where nothing is rounded, no records.
 
 `random_program(seed)` builds a kernel over (x : int32 vector, out : int32 vector, k : int32, n : int32) in which
-thread tid < n computes with int32 and int64 lets, mutable variables, assignments, casts between the two, `if` statements and expressions, Stdlib.Int32's
-functions (by name, and with the registry's device templates as the front end attaches them), calls of up to
-two helper functions (their own lets, loops and branches, a return at every end), `for` loops in
-both directions (bounds that read mutable variables the body changes among them), counted `while` loops and blocks, and
-stores into out[tid * SLOTS + j].  Names come from a small pool, parameters' names included, so bindings hide each
-other all the time; every use carries the id of the binding OCaml's scoping gives it.  Sums, products and negations
-overflow now and then (a linear congruential step is one of the expression forms): Int32 arithmetic wraps."""
+thread tid < n computes with int32 and int64 lets, mutable variables, assignments, casts between the two, `if`
+statements and expressions, Stdlib.Int32's and Int64's functions (by name, and with the registry's device templates as
+the front end attaches them), calls of up to two helper functions (their own lets, loops and branches, a return at
+every end), `for` loops in both directions (bounds that read mutable variables the body changes among them), counted
+`while` loops and blocks, and stores into out[tid * SLOTS + j].  Names come from a small pool, parameters' names
+included, so bindings hide each other all the time; every use carries the id of the binding OCaml's scoping gives
+it.  Sums, products and negations overflow now and then (a linear congruential step is one of the expression forms).
+
+`random_float_program(seed)`: float32 and float64 lets and stores whose every value both types hold exactly.
+`random_block_program(seed)`: supersteps over two shared arrays."""
 import random
 
 SLOTS = 4
