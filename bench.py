@@ -64,7 +64,10 @@ def parse():
                              "gemm_f16_epilogue", "gemm_f16_4095x11008x4096", "gemm_f16_shape", "gemm_bf16_shape", "gemm_bf16_2048", "gemm_f32_shape", "vendor_gemm_f32_shape", "copy_1gib",
                              "vendor_gemm_bf16_8192", "vendor_gemm_bf16_shape", "histogram_2p28",
                              "radix_scatter_5e7", "stencil_2d_shape", "conv2d_shape", "map_sum_2p28", "mfma_bf16_stream", "mfma_bf16_stream_32x32x16",
-                             "l2_to_lds_stream", "radix_scatter_chain_probe", "triad_shape_probe"])
+                             "l2_to_lds_stream", "radix_scatter_chain_probe", "triad_shape_probe", "fold_partials"])
+    ap.add_argument("--fold", default="1048576,0", metavar="PARTIALS,TAKE_STAGES",
+                    help="fold_partials: how many float32 partials, and 1 to give the library's sixteen fold stages "
+                         "to other streams first, so that the measured fold runs without one")
     ap.add_argument("--warmup-ms", type=float, default=60.0,
                     help="warm up for at least this long (and at least --warmup steps): the clocks of a power-limited "
                          "kernel take 30-40 ms to settle after a pause")
@@ -141,6 +144,7 @@ def dims(*d):
 
 
 ZERO_OPERANDS = False
+FOLD = (1 << 20, 0)
 CHAIN = (0, 1)
 TRIAD_SHAPE = (256, 4, 0)
 GEMM_SHAPE = (4096, 11264, 4096)
@@ -344,6 +348,34 @@ def make_workload(name, torch, hip):
                     peak=PEAK_MFMA_TFLOPS["bf16"], kernel="hipBLASLt (torch.matmul)", route="torch.matmul",
                     config={"workload": "torch.matmul bf16, N(0,0.02)", "m": m, "n": n, "k": k})
         return (lambda: torch.matmul(a, b, out=c)), None, info, None
+    if name == "fold_partials":
+        # the double fold of float32 partials (the host fold of bench_reduction.ml:154-160 kept on the device), with
+        # one of the library's stages or, when other streams hold all sixteen, as one workgroup
+        n, take = FOLD
+        g.manual_seed(0xF0)
+        parts = torch.rand(n, device="cuda", generator=g) * 4
+        total = torch.zeros(1, dtype=torch.float64, device="cuda")
+        held = []
+        if take:
+            seen = {}
+            while len(seen) < 16:
+                st = torch.cuda.Stream()
+                seen[st.cuda_stream] = st
+            small = torch.rand(1 << 17, device="cuda", generator=g)
+            for st in seen.values():
+                hip.check(lib.sarek_hip_fold_partials_f64(C.c_void_p(small.data_ptr()), small.numel(),
+                                                          C.c_void_p(total.data_ptr()), C.c_void_p(st.cuda_stream)))
+            torch.cuda.synchronize()
+            held = [seen, small]
+        main = Launch(hip, lib.sarek_hip_fold_partials_f64, C.c_void_p(parts.data_ptr()), n,
+                      C.c_void_p(total.data_ptr()), C.c_void_p(torch.cuda.current_stream().cuda_stream))
+        info = dict(metric="double fold of float32 partials GB/s", unit="GB/s", dtype="f64",
+                    work=4.0 * n, work_unit=1e9, bound="hbm", peak=PEAK_HBM_GBS,
+                    kernel="fold_pieces_kernel" if take else "fold_onepass_kernel",
+                    route="sarek_hip_fold_partials_f64",
+                    config={"workload": "sum of float32 partials in double, fixed order", "n": n,
+                            "without_a_stage": bool(take), "algorithmic_bytes": 4 * n})
+        return main, None, info, (parts, total, held)
     if name == "histogram_2p28":
         n = 1 << 28
         g.manual_seed(0xC4)
@@ -991,7 +1023,10 @@ def main():
         print("bench.py needs a GPU", file=sys.stderr)
         sys.exit(2)
     torch.cuda.set_device(0)
-    global ZERO_OPERANDS, GEMM_SHAPE, WARMUP_MS, TRACE_LAUNCHES, L2_STREAM_SHAPE, CHAIN, TRIAD_SHAPE
+    global ZERO_OPERANDS, GEMM_SHAPE, WARMUP_MS, TRACE_LAUNCHES, L2_STREAM_SHAPE, CHAIN, TRIAD_SHAPE, FOLD
+    FOLD = tuple(int(x) for x in args.fold.split(","))
+    if len(FOLD) != 2 or not 1 <= FOLD[0] <= 1 << 28 or FOLD[1] not in (0, 1):
+        sys.exit("--fold PARTIALS,TAKE_STAGES: 1 .. 2^28 partials, 0 or 1")
     TRIAD_SHAPE = tuple(int(x) for x in args.triad_shape.split(","))
     if len(TRIAD_SHAPE) != 3 or TRIAD_SHAPE[0] not in (64, 128, 256, 512, 1024) or TRIAD_SHAPE[1] not in (1, 2, 4, 6, 8) or \
             TRIAD_SHAPE[0] * TRIAD_SHAPE[1] > 6144:
