@@ -200,6 +200,22 @@ const char *stdlib_template(const std::vector<std::string> &path, const std::str
     if (n == "to_int") return "(int)(%s)";
     if (f64 && n == "of_float32") return "(double)(%s)";
     if (f32 && n == "of_float64") return "(float)(%s)";
+    // sarek/Sarek_float64/Float64.ml:133-146
+    if (f64 && n == "of_int32") return "(double)(%s)";
+    if (f64 && n == "to_int32") return "(int)(%s)";
+    if (f64 && n == "to_float32") return "(float)(%s)";
+  }
+  if (mod == "Math") {   // sarek/Sarek_stdlib/Math.ml:19-35
+    if (n == "xor") return "(%s ^ %s)";
+    if (n == "logical_and") return "(%s & %s)";
+    if (n == "pow") return "(int)powf((float)%s, (float)%s)";
+  }
+  if (mod == "Gpu" || mod == "Std") {   // sarek/Sarek_stdlib/Gpu.ml:117-247
+    if (n == "float64_of_int") return "(double)(%s)";
+    if (n == "int_of_float64") return "(int)(%s)";
+    if (n == "spoc_powint") return "spoc_powint";
+    if (n == "atomic_add_int32") return "atomicAdd(%s + %s, %s)";
+    if (n == "atomic_inc_int32" || n == "atomic_inc_global_int32") return "atomicAdd(%s + %s, 1)";
   }
   const bool i32 = mod == "Int32", i64 = mod == "Int64";
   if (i32 || i64) {

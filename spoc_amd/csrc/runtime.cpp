@@ -102,6 +102,11 @@ std::string ocaml_constants_for(const std::string &text) {
   if (uses_module(text, "Int64"))
     o += "struct sarek_hip_ocaml_int64 { long long max_int, min_int, zero, one, minus_one; };\n"
          "static constexpr sarek_hip_ocaml_int64 Int64 = {9223372036854775807LL, -9223372036854775807LL - 1, 0, 1, -1};\n";
+  // Gpu.spoc_powint's device text is a call of that name (sarek/Sarek_stdlib/Gpu.ml:235-247), which nothing in the
+  // reference's device headers defines; its OCaml side multiplies `exp` times.
+  if (text.find("spoc_powint(") != std::string::npos && text.find("int spoc_powint(") == std::string::npos)
+    o += "__device__ __forceinline__ int spoc_powint(int base, int exp) {\n  int acc = 1;\n"
+         "  for (; exp > 0; --exp) acc *= base;\n  return acc;\n}\n";
   return o;
 }
 

@@ -312,7 +312,10 @@ def test_ocaml_constants_a_kernel_names(hip, torch_cuda):
               ("(var Float.infinity 12 f64)", "d", np.inf), ("(var Float.max_float 13 f64)", "d", np.finfo(np.float64).max),
               ("(var Int32.max_int 14 i32)", "i", 2**31 - 1), ("(var Int32.min_int 15 i32)", "i", -2**31),
               ("(var Int64.max_int 16 i64)", "l", 2**63 - 1), ("(var Int64.min_int 17 i64)", "l", -2**63),
-              ("(add (var Int32.max_int 14 i32) (var Int32.one 18 i32))", "i", -2**31)]
+              ("(add (var Int32.max_int 14 i32) (var Int32.one 18 i32))", "i", -2**31),
+              # Gpu.spoc_powint's device text is a call of that name (Gpu.ml:235-247), which the compile step defines
+              ("(intr (Gpu) spoc_powint (i32 3) (i32 4))", "i", 81), ("(intr (Gpu) spoc_powint (i32 -2) (i32 31))", "i", -2**31),
+              ("(intr (Gpu) spoc_powint (i32 7) (i32 0))", "i", 1)]
     body = " ".join(f"(assign (lelem {v} (i32 {k})) {e})" for k, (e, v, _) in enumerate(stores))
     ir = ("(kernel sarek_kern (params (param (var d 1 (vec f64))) (param (var i 2 (vec i32))) (param (var l 3 (vec i64)))) "
           f"(locals) (body (if (eq (intr (Std) global_thread_id) (i32 0)) (seq {body}))) (native_fn true))")

@@ -157,6 +157,12 @@ def test_intrinsics(hip):
     assert expr_text(hip, "(intr (Int64) abs (var a 1 i64))") == "llabs(a)"
     assert expr_text(hip, "(intr (Sarek_stdlib Int32) logxor (var a 1 i32) (i32 3))") == "(a ^ 3)"
     assert expr_text(hip, "(intr (Int32) min (var a 1 i32) (i32 3))") == "min(a, 3)"
+    # the rest of the standard library by name (Sarek_float64/Float64.ml:133-146, Math.ml:19-35, Gpu.ml:117-247)
+    assert expr_text(hip, "(intr (Float64) of_int32 (var a 1 i32))") == "(double)(a)"
+    assert expr_text(hip, "(intr (Float64) to_float32 (var d 1 f64))") == "(float)(d)"
+    assert expr_text(hip, "(intr (Math) xor (var a 1 i32) (i32 3))") == "(a ^ 3)"
+    assert expr_text(hip, "(intr (Gpu) spoc_powint (var a 1 i32) (i32 3))") == "spoc_powint(a, 3)"
+    assert expr_text(hip, '(intr (Gpu) float64_of_int (template "(double)") (var a 1 i32))') == "(double)(a)"
     # the registry's templates are format strings (applied with Printf there, Sarek_ir_cuda.ml:360-396): %% is a %
     assert expr_text(hip, '(intr (Int32) mod_int32 (template "(%s %% %s)") (var a 1 i32) (i32 3))') == "(a % 3)"
     # a minus in a template keeps a space from an operand that begins with one
