@@ -338,13 +338,14 @@ __global__ __launch_bounds__(1024) void fold_onepass_kernel(const float *__restr
 
 // The 256 pieces of a long fold through one workgroup, for aligned pieces of at most K * 4096 elements (K 128-bit
 // loads per thread and piece): 8 / K pieces at a time, their loads asked for while the pieces before them are added
-// up, one barrier for the lot.  Thread t adds what fold_block's thread t adds to its running sum, in its order; the
-// wave's lanes and the sixteen waves' sums are added as there: stage[g] gets fold_block's bits for piece g.
+// up.  Thread t adds what fold_block's thread t adds to its running sum, in its order, and the wave's lanes are
+// added as there; the sixteen wave sums of every piece wait in LDS (32 KiB) for one barrier at the end, so no wave
+// waits for another on the way, and thread g then adds piece g's sixteen in wave order: stage[g] gets fold_block's
+// bits for piece g.
 template <int K>
 __device__ __forceinline__ void fold_pieces_batched(const float *__restrict__ partials, int64_t count, int64_t piece,
-                                                    double *stage) {
+                                                    double (*wave_sums)[16], double *stage) {
   constexpr int B = 8 / K;    // pieces per batch: eight 128-bit loads per thread in flight, which 128 registers hold
-  __shared__ double wave_sums[2][B][16];
   const int t = threadIdx.x, lane = t & 63, wave = t >> 6;
   auto length_of = [&](int g) {
     const int64_t lo = static_cast<int64_t>(g) * piece;
@@ -382,17 +383,15 @@ __device__ __forceinline__ void fold_pieces_batched(const float *__restrict__ pa
 #pragma unroll
     for (int q = 0; q < B; ++q) {
       const double s = wave_sum(acc[q]);
-      if (lane == 0) wave_sums[b & 1][q][wave] = s;
+      if (lane == 0) wave_sums[b * B + q][wave] = s;
     }
-    __syncthreads();
-    if (t < B) {
-      double total = 0.0;
+  }
+  __syncthreads();
+  if (t < kFoldGroups) {
+    double total = 0.0;
 #pragma unroll
-      for (int w = 0; w < 16; ++w) total += wave_sums[b & 1][t][w];
-      stage[b * B + t] = total;
-    }
-    // no second barrier: the next batch writes the other half of wave_sums, and the one after it comes after the
-    // next barrier, which these readers reach only when they have read
+    for (int w = 0; w < 16; ++w) total += wave_sums[t][w];
+    stage[t] = total;
   }
   __syncthreads();
 }
@@ -405,13 +404,14 @@ __device__ __forceinline__ void fold_pieces_batched(const float *__restrict__ pa
 __global__ __launch_bounds__(1024) void fold_pieces_kernel(const float *__restrict__ partials, int64_t count,
                                                            int64_t piece, double *__restrict__ out) {
   __shared__ double stage[kFoldGroups];
+  __shared__ double wave_sums[kFoldGroups][16];
   const bool aligned = (reinterpret_cast<uintptr_t>(partials) & 15u) == 0;
   if (aligned && piece <= 4096) {
-    fold_pieces_batched<1>(partials, count, piece, stage);
+    fold_pieces_batched<1>(partials, count, piece, wave_sums, stage);
   } else if (aligned && piece <= 8192) {
-    fold_pieces_batched<2>(partials, count, piece, stage);
+    fold_pieces_batched<2>(partials, count, piece, wave_sums, stage);
   } else if (aligned && piece <= 16384) {
-    fold_pieces_batched<4>(partials, count, piece, stage);
+    fold_pieces_batched<4>(partials, count, piece, wave_sums, stage);
   } else {
     for (int g = 0; g < kFoldGroups; ++g) {
       const int64_t lo = static_cast<int64_t>(g) * piece;
