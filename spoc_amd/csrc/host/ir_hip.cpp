@@ -13,6 +13,7 @@
 // barrier is `__builtin_amdgcn_wave_barrier()`; the source is compiled by hiprtc, which
 // pre-includes the HIP device runtime, so no #include lines are emitted.
 #include <algorithm>
+#include <cctype>
 #include <cmath>
 #include <cstdint>
 #include <cstdio>
@@ -620,11 +621,46 @@ std::string gen_stmt(const StmtP &sp, const std::string &indent) {
       return o;
     }
     case Stmt::Assign:
-      if (s.e->kind == Expr::Record) {  // field-by-field: no compound literals in assignments
+      if (s.e->kind == Expr::Record) {
+        // Field by field, as the reference prints it (Sarek_ir_cuda.ml:440-444).  When a field's value reads the
+        // record being assigned -- `p <- {x = p.y; y = p.x}` -- the later fields would see the earlier stores, where
+        // OCaml builds the whole record first: the values are then taken into temporaries before the first store.
+        const std::string target = gen_lvalue(s.lhs);
+        std::string root;   // the variable or vector the target lives in; none for a computed base
+        for (const LValue *l = s.lhs.get(); l;) {
+          if (l->kind == LValue::LRecordField) {
+            l = l->inner.get();
+          } else {
+            if (l->kind == LValue::LVar) root = printed_name(l->var);
+            else if (l->kind == LValue::LArrayElem) root = printed_name(l->name);
+            break;
+          }
+        }
+        std::vector<std::string> values;
+        bool reads_target = root.empty();
+        for (const auto &f : s.e->fields) {
+          values.push_back(gen_expr(f.second));
+          for (size_t at = values.back().find(root); !reads_target && at != std::string::npos;
+               at = values.back().find(root, at + 1)) {
+            auto part_of_a_name = [](char c) { return std::isalnum(static_cast<unsigned char>(c)) || c == '_'; };
+            const std::string &v = values.back();
+            const bool starts = at == 0 || !part_of_a_name(v[at - 1]);
+            const bool ends = at + root.size() >= v.size() || !part_of_a_name(v[at + root.size()]);
+            reads_target = starts && ends;
+          }
+        }
         std::string o;
-        for (const auto &f : s.e->fields)
-          o += indent + gen_lvalue(s.lhs) + "." + f.first + " = " + gen_expr(f.second) + ";\n";
-        return o;
+        if (!reads_target) {
+          for (size_t i = 0; i < values.size(); ++i)
+            o += indent + target + "." + s.e->fields[i].first + " = " + values[i] + ";\n";
+          return o;
+        }
+        o = indent + "{\n";
+        for (size_t i = 0; i < values.size(); ++i)
+          o += in2 + "const auto sarek_field_" + std::to_string(i) + " = " + values[i] + ";\n";
+        for (size_t i = 0; i < values.size(); ++i)
+          o += in2 + target + "." + s.e->fields[i].first + " = sarek_field_" + std::to_string(i) + ";\n";
+        return o + indent + "}\n";
       }
       return indent + gen_lvalue(s.lhs) + " = " + gen_expr(s.e) + ";\n";
     case Stmt::If: {

@@ -5,7 +5,7 @@ binding id, then by name :76-91; Int32 operators :171-266 -- `shr` on non-negati
 zeros and with the sign agree; statements :844-941 -- a `for` evaluates both bounds once and is inclusive :858-872),
 one thread after the other; `evaluate_blocks` runs a kernel with barriers superstep by superstep.  It is a model
 for tests, over the subset the generators below emit: int32 and int64 arithmetic modulo 2^32 / 2^64, floats only
-where nothing is rounded, no records.
+where nothing is rounded, records of integers as values.
 
 `random_program(seed)` builds a kernel over (x : int32 vector, out : int32 vector, k : int32, n : int32) in which
 thread tid < n computes with int32 and int64 lets, mutable variables, assignments, casts between the two, `if`
@@ -17,7 +17,8 @@ included, so bindings hide each other all the time; every use carries the id of 
 it.  Sums, products and negations overflow now and then (a linear congruential step is one of the expression forms).
 
 `random_float_program(seed)`: float32 and float64 lets and stores whose every value both types hold exactly.
-`random_block_program(seed)`: supersteps over two shared arrays."""
+`random_block_program(seed)`: supersteps over two shared arrays.
+`random_record_program(seed)`: two record types, one nested in the other, as values, in vectors and through a helper."""
 import random
 
 SLOTS = 4
@@ -33,6 +34,10 @@ def _exact(v):
     if struct.unpack("f", struct.pack("f", v))[0] != v:
         raise Inexact()
     return v
+
+
+def _copy(v):
+    return {k: _copy(x) if isinstance(x, dict) else x for k, x in v.items()}
 
 
 class _Return(Exception):
@@ -126,12 +131,19 @@ class Thread:
         if head == "bool":
             return e[1] == "true"
         if head == "var":
-            return self.lookup(e)
+            v = self.lookup(e)
+            return _copy(v) if isinstance(v, dict) else v
         if head == "read":
             v = self.arrays[e[1]][self.expr(e[2])]
+            if isinstance(v, dict):
+                return _copy(v)
             return float(v) if isinstance(v, float) or getattr(v, "dtype", None) is not None and v.dtype.kind == "f" else int(v)
         if head == "len":
             return len(self.arrays[e[1]])
+        if head == "record":                                # a value: a fresh one wherever it is bound or stored
+            return {f[0]: self.expr(f[1]) for f in e[2:]}
+        if head == "field":
+            return self.expr(e[1])[e[2]]
         if head == "intr":
             name = e[2]
             if name in ("global_thread_id", "global_idx_x", "global_idx"):
@@ -238,6 +250,15 @@ class Thread:
             value, target = self.expr(s[2]), s[1]
             if target[0] == "lvar":
                 self.bind(target[1], value)
+            elif target[0] == "lfield":                     # a field of a mutable record variable or of a vector's element
+                path = []
+                while target[0] == "lfield":
+                    path.append(target[2])
+                    target = target[1]
+                holder = self.lookup(target[1]) if target[0] == "lvar" else self.arrays[target[1]][self.expr(target[2])]
+                for name in reversed(path[1:]):
+                    holder = holder[name]
+                holder[path[0]] = value
             else:
                 assert target[0] == "lelem"
                 self.arrays[target[1]][self.expr(target[2])] = value
@@ -750,3 +771,144 @@ def random_block_program(seed, block=64, grid=3):
           f"(locals) (body {body}) (native_fn true))")
     x = np.array([rng.randint(-100, 100) for _ in range(block * grid)], np.int32)
     return ir, x, rng.randint(-5, 9)
+
+
+POINT = "(record point (x i32) (y i32))"
+SEG = f"(record seg (a {POINT}) (b {POINT}) (w i32))"
+
+
+class _Records:
+    """Programs over two record types, point {x; y} and seg {a : point; b : point; w}: record literals, elements of
+    record vectors, fields and fields of fields, conditionals between records, a helper that takes a seg and returns a
+    point, mutable record variables whose fields are assigned, stores of whole records and of single fields into the
+    vectors.  Records are values here as in the device text; no variable is bound to another mutable record (an
+    alias in OCaml, a copy in C)."""
+
+    def __init__(self, rng):
+        self.rng, self.next_id = rng, 40
+        self.points, self.segs, self.mutable = [], [], set()      # variables in scope, as IR text
+
+    def fresh(self, name, ty, mutable=False):
+        vid = self.next_id
+        self.next_id += 1
+        text = f"(var {name}{vid} {vid} {ty}{' mut' if mutable else ''})"
+        if mutable:
+            self.mutable.add(text)
+        return text
+
+    def integer(self, depth):
+        r = self.rng
+        if depth == 0:
+            pick = r.randint(0, 5)
+            if pick == 0:
+                return f"(i32 {r.randint(-20, 20)})"
+            if pick == 1:
+                return "(var tid 5 i32)"
+            if pick == 2 and self.segs:
+                return f"(field {r.choice(self.segs)} w)"
+            if pick == 3 and self.segs:
+                return f"(field (field {r.choice(self.segs)} {r.choice('ab')}) {r.choice('xy')})"
+            if pick == 4:
+                return f"(field (read ps (var tid 5 i32)) {r.choice('xy')})"
+            return f"(field {self.point(0)} {r.choice('xy')})"
+        a, b = self.integer(depth - 1), self.integer(depth - 1)
+        return f"({r.choice(['add', 'sub', 'bitxor', 'bitand'])} {a} {b})"
+
+    def point(self, depth):
+        r = self.rng
+        pick = r.randint(0, 6)
+        if pick == 0 and self.points:
+            return r.choice(self.points)
+        if pick == 1:
+            return "(read ps (var tid 5 i32))"
+        if pick == 2 and self.segs:
+            return f"(field {r.choice(self.segs)} {r.choice('ab')})"
+        if pick == 3:
+            return f"(field (read ss (var tid 5 i32)) {r.choice('ab')})"
+        if pick == 4 and depth > 0:
+            return f"(if (lt {self.integer(1)} {self.integer(1)}) {self.point(depth - 1)} {self.point(depth - 1)})"
+        if pick == 5 and depth > 0:
+            return f"(app (var mid 0 {POINT}) {self.seg(depth - 1)})"
+        return f"(record point (x {self.integer(min(depth, 1))}) (y {self.integer(min(depth, 1))}))"
+
+    def seg(self, depth):
+        r = self.rng
+        pick = r.randint(0, 3)
+        if pick == 0 and self.segs:
+            return r.choice(self.segs)
+        if pick == 1:
+            return "(read ss (var tid 5 i32))"
+        if pick == 2 and depth > 0:
+            return f"(if (ge {self.integer(1)} {self.integer(1)}) {self.seg(depth - 1)} {self.seg(depth - 1)})"
+        return f"(record seg (a {self.point(depth)}) (b {self.point(depth)}) (w {self.integer(1)}))"
+
+    def body(self, steps):
+        r = self.rng
+        if steps == 0:
+            stores = [f"(assign (lelem out (add (mul (var tid 5 i32) (i32 {SLOTS})) (i32 {slot}))) {self.integer(2)})" for slot in range(SLOTS)]
+            stores.append(f"(assign (lelem ps (var tid 5 i32)) {self.point(2)})")
+            stores.append(r.choice([f"(assign (lelem ss (var tid 5 i32)) {self.seg(1)})",
+                                    f"(assign (lfield (lelem ss (var tid 5 i32)) w) {self.integer(2)})",
+                                    f"(assign (lfield (lfield (lelem ss (var tid 5 i32)) {r.choice('ab')}) {r.choice('xy')}) {self.integer(2)})"]))
+            r.shuffle(stores)
+            return "(seq " + " ".join(stores) + ")"
+        pick = r.randint(0, 4)
+        if pick <= 1:                                        # let p = <point> in ...
+            value, v = self.point(2), self.fresh("p", POINT)
+            self.points.append(v)
+            inner = self.body(steps - 1)
+            self.points.remove(v)
+            return f"(let {v} {value} {inner})"
+        if pick == 2:
+            value, v = self.seg(1), self.fresh("s", SEG)
+            self.segs.append(v)
+            inner = self.body(steps - 1)
+            self.segs.remove(v)
+            return f"(let {v} {value} {inner})"
+        # let mutable q = <literal or element> in q.f <- e; ...   (never another variable: no aliases)
+        wide = pick == 4
+        saved_points, saved_segs = self.points, self.segs
+        self.points, self.segs = [], []                       # the initial value names no variable
+        value = (self.seg(0) if wide else self.point(0))
+        self.points, self.segs = saved_points, saved_segs
+        v = self.fresh("q", SEG if wide else POINT, mutable=True)
+        target = f"(lvar {v})"
+        if wide:
+            assign = r.choice([f"(assign (lfield {target} w) {self.integer(1)})",
+                               f"(assign (lfield (lfield {target} {r.choice('ab')}) {r.choice('xy')}) {self.integer(1)})",
+                               f"(assign (lfield {target} {r.choice('ab')}) {self.point(1)})"])
+            self.segs.append(v)
+        else:
+            assign = f"(assign (lfield {target} {r.choice('xy')}) {self.integer(1)})"
+            self.points.append(v)
+        inner = self.body(steps - 1)
+        (self.segs if wide else self.points).remove(v)
+        return f"(letmut {v} {value} (seq {assign} {inner}))"
+
+
+def random_record_program(seed, threads=24):
+    """(ir, ps, ss): ps an int32 array [threads, 2], ss one [threads, 5] (a.x a.y b.x b.y w)."""
+    import numpy as np
+    rng = random.Random(700000 + seed)
+    b = _Records(rng)
+    body = b.body(rng.randint(2, 5))
+    s = f"(var s 30 {SEG})"
+    mid = (f"(func mid (params {s}) {POINT} (return (record point (x (add (field (field {s} a) x) (field (field {s} b) x))) "
+           f"(y (sub (field (field {s} a) y) (field {s} w))))))")
+    ir = (f"(kernel sarek_kern (params (param (var ps 1 (vec {POINT}))) (param (var ss 2 (vec {SEG}))) "
+          "(param (var out 3 (vec i32))) (param (var n 4 i32))) (locals) (body (let (var tid 5 i32) "
+          f"(intr (Std) global_thread_id) (if (lt (var tid 5 i32) (var n 4 i32)) {body}))) "
+          f"(types (point (x i32) (y i32)) (seg (a {POINT}) (b {POINT}) (w i32))) (funcs {mid}) (native_fn true))")
+    ps = np.array([[rng.randint(-50, 50) for _ in range(2)] for _ in range(threads)], np.int32)
+    ss = np.array([[rng.randint(-50, 50) for _ in range(5)] for _ in range(threads)], np.int32)
+    return ir, ps, ss
+
+
+def expected_records(ir, ps, ss, threads):
+    import numpy as np
+    points = [{"x": int(p[0]), "y": int(p[1])} for p in ps]
+    segs = [{"a": {"x": int(q[0]), "y": int(q[1])}, "b": {"x": int(q[2]), "y": int(q[3])}, "w": int(q[4])} for q in ss]
+    out = np.full(SLOTS * threads, -1, np.int32)
+    evaluate(ir, {"ps": points, "ss": segs, "out": out, "n": threads}, threads)
+    return (np.array([[p["x"], p["y"]] for p in points], np.int32),
+            np.array([[q["a"]["x"], q["a"]["y"], q["b"]["x"], q["b"]["y"], q["w"]] for q in segs], np.int32), out)

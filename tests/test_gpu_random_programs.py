@@ -136,3 +136,23 @@ def test_seeded_supersteps_over_shared_arrays(hip, sarek, seed):
     T.flush()
     got = out.to_array()
     assert np.array_equal(got, want), (seed, np.flatnonzero(got != want)[:8].tolist())
+
+
+@pytest.mark.parametrize("seed", range(int(os.environ.get("SAREK_HIP_TEST_PROGRAM_SEEDS", "48")) // 2))
+def test_seeded_record_programs_compute_what_the_walker_computes(hip, sarek, seed):
+    """Programs over point {x; y} and seg {a : point; b : point; w}: literals, elements of record vectors, fields of
+    fields, conditionals between records, a helper from seg to point, mutable records whose fields are assigned,
+    stores of whole records and of single fields.  The two record vectors and the int32 output end as the walker
+    leaves them."""
+    E, T, V = sarek.Execute, sarek.Transfer, sarek.Vector
+    ir, ps, ss = ir_programs.random_record_program(seed, THREADS)
+    want_ps, want_ss, want_out = ir_programs.expected_records(ir, ps, ss, THREADS)
+    vps, vss = V.create_custom(8, THREADS), V.create_custom(20, THREADS)
+    vps.host.view(np.int32).reshape(THREADS, 2)[:] = ps
+    vss.host.view(np.int32).reshape(THREADS, 5)[:] = ss
+    out = V.of_array(np.full(ir_programs.SLOTS * THREADS, -1, np.int32))
+    assert E.run_vectors(ir, [E.Vec(vps), E.Vec(vss), E.Vec(out), E.Int32(THREADS)], (32, 1, 1), (1, 1, 1)) == "jit"
+    T.flush()
+    assert np.array_equal(out.to_array(), want_out), (seed, "out")
+    assert np.array_equal(vps.to_array().view(np.int32).reshape(THREADS, 2), want_ps), (seed, "ps")
+    assert np.array_equal(vss.to_array().view(np.int32).reshape(THREADS, 5), want_ss), (seed, "ss")

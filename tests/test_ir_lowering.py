@@ -906,3 +906,23 @@ def test_the_program_model_on_the_references_known_answers(hip):
     # and the whole kernel lowers to text the device compiler takes
     text = hip.generate_source(interp_cases.kernel())
     assert "int a[5] = {};" in text and "out[7] = (int)42.700000000000003f;" in text
+
+
+def test_a_record_literal_that_reads_what_it_is_assigned_to(hip):
+    """`ps.(i) <- {x = ps.(i).y; y = ps.(i).x}`: the reference stores field by field (Sarek_ir_cuda.ml:440-444), so
+    the second field would read the first one's new value; OCaml builds the record first.  The values are taken
+    before the first store when one of them names the target's vector or variable; otherwise the text is the
+    reference's."""
+    pt = "(record point (x i32) (y i32))"
+    read = "(read ps (var i 2 i32))"
+    swap = f"(assign (lelem ps (var i 2 i32)) (record point (x (field {read} y)) (y (field {read} x))))"
+    params = f"(param (var ps 1 (vec {pt}))) (param (var i 2 i32)) (param (var qs 3 (vec {pt})))"
+    ir = f"(kernel k (params {params}) (locals) (body {swap}) (types (point (x i32) (y i32))) (native_fn true))"
+    text = hip.generate_source(ir)
+    assert ("  {\n    const auto sarek_field_0 = ps[i].y;\n    const auto sarek_field_1 = ps[i].x;\n"
+            "    ps[i].x = sarek_field_0;\n    ps[i].y = sarek_field_1;\n  }\n") in text
+    other = ir.replace("(assign (lelem ps ", "(assign (lelem qs ")
+    assert "  qs[i].x = ps[i].y;\n  qs[i].y = ps[i].x;\n" in hip.generate_source(other)
+    # a variable whose name only contains the target's is not the target
+    longer = other.replace("(var qs 3", "(var s 3").replace("(lelem qs ", "(lelem s ")
+    assert "  s[i].x = ps[i].y;\n  s[i].y = ps[i].x;\n" in hip.generate_source(longer)
