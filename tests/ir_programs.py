@@ -37,7 +37,9 @@ def _exact(v):
 
 
 def _copy(v):
-    return {k: _copy(x) if isinstance(x, dict) else x for k, x in v.items()}
+    if isinstance(v, tuple):
+        return (v[0], [_copy(x) if isinstance(x, (dict, tuple)) else x for x in v[1]])
+    return {k: _copy(x) if isinstance(x, (dict, tuple)) else x for k, x in v.items()}
 
 
 class _Return(Exception):
@@ -132,7 +134,7 @@ class Thread:
             return e[1] == "true"
         if head == "var":
             v = self.lookup(e)
-            return _copy(v) if isinstance(v, dict) else v
+            return _copy(v) if isinstance(v, (dict, tuple)) else v
         if head == "read":
             v = self.arrays[e[1]][self.expr(e[2])]
             if isinstance(v, dict):
@@ -144,6 +146,11 @@ class Thread:
             return {f[0]: self.expr(f[1]) for f in e[2:]}
         if head == "field":
             return self.expr(e[1])[e[2]]
+        if head == "variant":                               # (constructor, payload values)
+            return (e[2], [self.expr(a) for a in e[3:]])
+        if head == "match":
+            body = self.matching_case(self.expr(e[1]), e[2:])
+            return self.expr(body)
         if head == "intr":
             name = e[2]
             if name in ("global_thread_id", "global_idx_x", "global_idx"):
@@ -225,6 +232,23 @@ class Thread:
         if head == "or": return bool(a) or bool(b)
         raise KeyError(head)
 
+    def matching_case(self, value, cases):
+        """The body of the first case that takes `value`, its pattern's variables bound by name (a pattern carries no
+        ids, Sarek_ir_interp.ml:873-899)."""
+        constructor, payload = value
+        for case in cases:
+            pattern, body = case[1], case[2]
+            if pattern == "_":
+                return body
+            if pattern[0] == "?":
+                self.by_name[pattern[1]] = value
+                return body
+            if pattern[0] == constructor:
+                for name, v in zip(pattern[1:], payload):
+                    self.by_name[name] = v
+                return body
+        raise AssertionError("no case matches")
+
     def stmt(self, s):
         head = s[0]
         self.steps += 1
@@ -267,6 +291,8 @@ class Thread:
                 self.stmt(s[2])
             elif len(s) > 3:
                 self.stmt(s[3])
+        elif head == "match":
+            self.stmt(self.matching_case(self.expr(s[1]), s[2:]))
         elif head == "while":
             while self.expr(s[1]):
                 self.stmt(s[2])
@@ -775,18 +801,78 @@ def random_block_program(seed, block=64, grid=3):
 
 POINT = "(record point (x i32) (y i32))"
 SEG = f"(record seg (a {POINT}) (b {POINT}) (w i32))"
+SHAPE = f"(variant shape (Dot {POINT}) (Line {SEG}) (Scaled i32 i32) (Nothing))"
 
 
 class _Records:
     """Programs over two record types, point {x; y} and seg {a : point; b : point; w}: record literals, elements of
     record vectors, fields and fields of fields, conditionals between records, a helper that takes a seg and returns a
     point, mutable record variables whose fields are assigned, stores of whole records and of single fields into the
-    vectors.  Records are values here as in the device text; no variable is bound to another mutable record (an
+    vectors; and a variant over them (Dot of point | Line of seg | Scaled of int32 * int32 | Nothing) built by
+    constructors and conditionals and taken apart by matches, as statements and as values, with wildcard and variable
+    patterns.  Records are values here as in the device text; no variable is bound to another mutable record (an
     alias in OCaml, a copy in C)."""
 
     def __init__(self, rng):
         self.rng, self.next_id = rng, 40
         self.points, self.segs, self.mutable = [], [], set()      # variables in scope, as IR text
+        self.shapes, self.ints = [], []
+
+    def shape(self, depth):
+        """A value of shape = Dot of point | Line of seg | Scaled of int32 * int32 | Nothing."""
+        r = self.rng
+        pick = r.randint(0, 5)
+        if pick == 0 and self.shapes:
+            return r.choice(self.shapes)
+        if pick == 1:
+            return f"(variant shape Dot {self.point(depth)})"
+        if pick == 2:
+            return f"(variant shape Line {self.seg(max(depth - 1, 0))})"
+        if pick == 3:
+            return f"(variant shape Scaled {self.integer(1)} {self.integer(1)})"
+        if pick == 4 and depth > 0:
+            return f"(if (ne {self.integer(1)} {self.integer(1)}) {self.shape(depth - 1)} {self.shape(depth - 1)})"
+        return "(variant shape Nothing)"
+
+    def cases(self, make_body):
+        """Cases over shape in a seeded order, the last one a wildcard, a variable pattern or the constructor left;
+        `make_body` builds a case's body with the pattern's variables in scope."""
+        r = self.rng
+        constructors = ["Dot", "Line", "Scaled", "Nothing"]
+        r.shuffle(constructors)
+        texts = []
+        for c in constructors[:r.randint(2, 4)]:
+            n = self.next_id
+            self.next_id += 4
+            if c == "Dot":
+                v = f"(var pat{n} {n} {POINT})"
+                self.points.append(v)
+                texts.append(f"(case (Dot pat{n}) {make_body()})")
+                self.points.remove(v)
+            elif c == "Line":
+                v = f"(var pat{n} {n} {SEG})"
+                self.segs.append(v)
+                texts.append(f"(case (Line pat{n}) {make_body()})")
+                self.segs.remove(v)
+            elif c == "Scaled":
+                a, b = f"(var pat{n} {n} i32)", f"(var pat{n + 1} {n + 1} i32)"
+                self.ints += [a, b]
+                texts.append(f"(case (Scaled pat{n} pat{n + 1}) {make_body()})")
+                self.ints.remove(a)
+                self.ints.remove(b)
+            else:
+                texts.append(f"(case (Nothing) {make_body()})")
+        if len(texts) < 4:
+            if r.random() < 0.5:
+                texts.append(f"(case _ {make_body()})")
+            else:
+                n = self.next_id
+                self.next_id += 1
+                v = f"(var rest{n} {n} {SHAPE})"
+                self.shapes.append(v)
+                texts.append(f"(case (? rest{n}) {make_body()})")
+                self.shapes.remove(v)
+        return " ".join(texts)
 
     def fresh(self, name, ty, mutable=False):
         vid = self.next_id
@@ -798,8 +884,13 @@ class _Records:
 
     def integer(self, depth):
         r = self.rng
+        if depth > 0 and r.random() < 0.2:                   # a match used as a value
+            scrutinee = self.shape(1)
+            return f"(match {scrutinee} {self.cases(lambda: self.integer(depth - 1))})"
         if depth == 0:
             pick = r.randint(0, 5)
+            if self.ints and r.random() < 0.3:
+                return r.choice(self.ints)
             if pick == 0:
                 return f"(i32 {r.randint(-20, 20)})"
             if pick == 1:
@@ -852,7 +943,18 @@ class _Records:
                                     f"(assign (lfield (lfield (lelem ss (var tid 5 i32)) {r.choice('ab')}) {r.choice('xy')}) {self.integer(2)})"]))
             r.shuffle(stores)
             return "(seq " + " ".join(stores) + ")"
-        pick = r.randint(0, 4)
+        pick = r.randint(0, 6)
+        if pick == 5:                                        # let v = <shape> in ...
+            value, v = self.shape(2), self.fresh("v", SHAPE)
+            self.shapes.append(v)
+            inner = self.body(steps - 1)
+            self.shapes.remove(v)
+            return f"(let {v} {value} {inner})"
+        if pick == 6:                                        # match <shape> with cases that store, then the rest
+            slot = r.randrange(SLOTS)
+            store = lambda: f"(assign (lelem out (add (mul (var tid 5 i32) (i32 {SLOTS})) (i32 {slot}))) {self.integer(1)})"
+            scrutinee = self.shape(1)
+            return f"(seq (match {scrutinee} {self.cases(store)}) {self.body(steps - 1)})"
         if pick <= 1:                                        # let p = <point> in ...
             value, v = self.point(2), self.fresh("p", POINT)
             self.points.append(v)
@@ -898,7 +1000,8 @@ def random_record_program(seed, threads=24):
     ir = (f"(kernel sarek_kern (params (param (var ps 1 (vec {POINT}))) (param (var ss 2 (vec {SEG}))) "
           "(param (var out 3 (vec i32))) (param (var n 4 i32))) (locals) (body (let (var tid 5 i32) "
           f"(intr (Std) global_thread_id) (if (lt (var tid 5 i32) (var n 4 i32)) {body}))) "
-          f"(types (point (x i32) (y i32)) (seg (a {POINT}) (b {POINT}) (w i32))) (funcs {mid}) (native_fn true))")
+          f"(types (point (x i32) (y i32)) (seg (a {POINT}) (b {POINT}) (w i32))) "
+          f"(variants (shape (Dot {POINT}) (Line {SEG}) (Scaled i32 i32) (Nothing))) (funcs {mid}) (native_fn true))")
     ps = np.array([[rng.randint(-50, 50) for _ in range(2)] for _ in range(threads)], np.int32)
     ss = np.array([[rng.randint(-50, 50) for _ in range(5)] for _ in range(threads)], np.int32)
     return ir, ps, ss
