@@ -12,7 +12,7 @@ thread tid < n computes with int32 and int64 lets, mutable variables, assignment
 statements and expressions, Stdlib.Int32's and Int64's functions (by name, and with the registry's device templates as
 the front end attaches them), calls of up to two helper functions (their own lets, loops and branches, a return at
 every end), `for` loops in both directions (bounds that read mutable variables the body changes among them), counted
-`while` loops and blocks, and stores into out[tid * SLOTS + j].  Names come from a small pool, parameters' names
+`while` loops, blocks and arrays of the thread's own (zero to begin with), and stores into out[tid * SLOTS + j].  Names come from a small pool, parameters' names
 included, so bindings hide each other all the time; every use carries the id of the binding OCaml's scoping gives
 it.  Sums, products and negations overflow now and then (a linear congruential step is one of the expression forms).
 
@@ -334,6 +334,7 @@ class _Builder:
         self.vectors = {"x", "out"}
         self.counters = set()      # ids of loop counters: mutable in the IR, assigned by their loop alone
         self.wide = set()          # ids of the int64 variables
+        self.local_arrays = []     # names of the thread's own arrays in scope (eight int32 each)
         self.helpers = []          # (name, number of parameters) of the helper functions made so far
         self.in_helper = False     # a helper sees its parameters alone: no vector, no thread index
 
@@ -428,6 +429,8 @@ class _Builder:
                 return f"(i32 {r.randint(-9, 12)})"
             if pick == 1 and not self.in_helper:
                 return f"(read x {self.use('tid')})"
+            if pick == 2 and self.local_arrays:
+                return f"(read {r.choice(self.local_arrays)} {self.small(self.expr(0), 3)})"
             ints = self.ints_in_scope()                      # none when int64 lets hide a helper's every parameter
             return self.use(r.choice(ints)) if ints else f"(i32 {r.randint(-9, 12)})"
         if r.random() < 0.1:                                 # the low or the high half of an int64 value
@@ -510,6 +513,9 @@ class _Builder:
         return f"(assign (lvar {self.use(name)}) {value})"
 
     def store(self):
+        if self.local_arrays and self.rng.random() < 0.4:
+            return (f"(assign (lelem {self.rng.choice(self.local_arrays)} {self.small(self.expr(1), 3)}) "
+                    f"{self.expr(self.rng.randint(0, 2))})")
         if self.in_helper:                                  # no memory there: an assignment, or nothing
             mutables = [n for n, (vid, m) in self.scope.items() if m and vid not in self.counters]
             if not mutables:
@@ -575,6 +581,14 @@ class _Builder:
             return f"(let {lim} {limit} {body})"
         if pick == 8:
             return f"(block {self.stmts(depth - 1, r.randint(1, 3))})"
+        if pick == 9 and r.random() < 0.6:                   # an array of the thread's own: eight zeros to begin with
+            vid = self.next_id
+            self.next_id += 1
+            name = f"arr{vid}"
+            self.local_arrays.append(name)
+            body = self.stmts(depth - 1, r.randint(2, 4))
+            self.local_arrays.remove(name)
+            return f"(let (var {name} {vid} (array i32 local)) (newarray i32 (i32 8) local) {body})"
         return self.store()
 
 
