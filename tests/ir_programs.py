@@ -8,7 +8,7 @@ for tests, over the subset the generators below emit: int32 and int64 arithmetic
 where nothing is rounded, records of integers as values.
 
 `random_program(seed)` builds a kernel over (x : int32 vector, out : int32 vector, k : int32, n : int32) in which
-thread tid < n computes with int32 and int64 lets, mutable variables, assignments, casts between the two, `if`
+thread tid < n computes with int32, int64 and bool lets, mutable variables, assignments, casts between the two, `if`
 statements and expressions, Stdlib.Int32's and Int64's functions (by name, and with the registry's device templates as
 the front end attaches them), calls of up to two helper functions (their own lets, loops and branches, a return at
 every end), `for` loops in both directions (bounds that read mutable variables the body changes among them), counted
@@ -335,6 +335,7 @@ class _Builder:
         self.counters = set()      # ids of loop counters: mutable in the IR, assigned by their loop alone
         self.wide = set()          # ids of the int64 variables
         self.local_arrays = []     # names of the thread's own arrays in scope (eight int32 each)
+        self.flags = set()         # ids of the bool variables
         self.helpers = []          # (name, number of parameters) of the helper functions made so far
         self.in_helper = False     # a helper sees its parameters alone: no vector, no thread index
 
@@ -372,14 +373,16 @@ class _Builder:
         return f"(return {self.expr(r.randint(0, 2))})"
 
     def var(self, name, vid, mutable):
-        return f"(var {name} {vid} {'i64' if vid in self.wide else 'i32'}{' mut' if mutable else ''})"
+        ty = "bool" if vid in self.flags else "i64" if vid in self.wide else "i32"
+        return f"(var {name} {vid} {ty}{' mut' if mutable else ''})"
 
     def use(self, name):
         vid, mutable = self.scope[name]
         return self.var(name, vid, mutable)
 
     def ints_in_scope(self):
-        return [n for n, (vid, _) in self.scope.items() if n not in self.vectors and vid not in self.wide]
+        return [n for n, (vid, _) in self.scope.items()
+                if n not in self.vectors and vid not in self.wide and vid not in self.flags]
 
     def longs_in_scope(self):
         return [n for n, (vid, _) in self.scope.items() if vid in self.wide]
@@ -436,7 +439,7 @@ class _Builder:
         if r.random() < 0.1:                                 # the low or the high half of an int64 value
             wide = self.expr64(depth - 1)
             return r.choice([f"(cast i32 {wide})", f"(cast i32 (intr (Int64) shift_right_logical {wide} (i32 32)))"])
-        if self.helpers and not self.in_helper and r.random() < 0.15:
+        if self.helpers and r.random() < 0.15:              # (a helper calls the helpers made before it)
             name, arity = r.choice(self.helpers)
             return f"(app (var {name} 0 i32) {' '.join(self.small(self.expr(depth - 1), 6) for _ in range(arity))})"
         a, b = self.expr(depth - 1), self.expr(depth - 1)
@@ -487,6 +490,9 @@ class _Builder:
             if pick == 0:
                 return f"(not {self.cond(depth - 1)})"
             return f"({'and' if pick == 1 else 'or'} {self.cond(depth - 1)} {self.cond(depth - 1)})"
+        flags = [n for n, (vid, _) in self.scope.items() if vid in self.flags]
+        if flags and r.random() < 0.3:
+            return self.use(r.choice(flags))
         if r.random() < 0.15:
             return f"({r.choice(['lt', 'le', 'gt', 'ge', 'eq', 'ne'])} {self.expr64(1)} {self.expr64(1)})"
         return f"({r.choice(['lt', 'le', 'gt', 'ge', 'eq', 'ne'])} {self.expr(1)} {self.expr(1)})"
@@ -509,7 +515,9 @@ class _Builder:
         return self.var(name, vid, mutable), body
 
     def assign(self, name):
-        value = self.expr64(self.rng.randint(0, 2)) if self.scope[name][0] in self.wide else self.expr(self.rng.randint(0, 2))
+        vid = self.scope[name][0]
+        value = self.cond(1) if vid in self.flags else self.expr64(self.rng.randint(0, 2)) if vid in self.wide \
+            else self.expr(self.rng.randint(0, 2))
         return f"(assign (lvar {self.use(name)}) {value})"
 
     def store(self):
@@ -536,6 +544,13 @@ class _Builder:
             return self.store()
         pick = r.randint(0, 9)
         if pick in (0, 1, 2, 3):                             # let [mutable] NAME = e in S (the value reads the outer NAME)
+            if r.random() < 0.12:                            # a bool: the name stands for a condition from here on
+                value = self.cond(1)
+                vid = self.next_id
+                self.flags.add(vid)
+                v, body = self.bound_body(r.choice(self.POOL), pick >= 2, lambda: self.stmts(depth - 1, r.randint(1, 3)))
+                assert f" {vid} bool" in v
+                return f"({'letmut' if pick >= 2 else 'let'} {v} {value} {body})"
             wide = r.random() < 0.25
             value = self.expr64(r.randint(0, 2)) if wide else self.expr(r.randint(0, 2))
             v, body = self.bound_body(r.choice(self.POOL), pick >= 2, lambda: self.stmts(depth - 1, r.randint(1, 3)), wide=wide)
@@ -546,7 +561,7 @@ class _Builder:
         if pick in (5, 6):                                   # for NAME = lo to / downto hi
             lo, hi = self.small(self.expr(1), 2), self.small(self.expr(1), 3)
             down = r.random() < 0.4
-            narrow = [n for n in mutables if self.scope[n][0] not in self.wide]
+            narrow = [n for n in mutables if self.scope[n][0] not in self.wide and self.scope[n][0] not in self.flags]
             moving = r.choice(narrow) if narrow and r.random() < 0.5 else None
             if moving:                                       # the far bound reads what the body goes on to change
                 bound = self.small(self.use(moving), 3)
