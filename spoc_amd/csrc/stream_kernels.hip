@@ -352,7 +352,20 @@ __device__ __forceinline__ void fold_pieces_batched(const float *__restrict__ pa
     return lo >= count ? int64_t{0} : (count - lo < piece ? count - lo : piece);
   };
   float4 next[B * K];
+  // all pieces but the last ones are whole: a batch that lies inside the input has one length, known beforehand
+  const int64_t whole_n4 = piece >> 2;
+  const float4 *const base4 = reinterpret_cast<const float4 *>(partials);
+  auto whole = [&](int b) { return static_cast<int64_t>(b + 1) * B * piece <= count; };
   auto load_batch = [&](int b) {
+    if (whole(b)) {
+      const float4 *p4 = base4 + static_cast<int64_t>(b) * B * whole_n4 + t;
+#pragma unroll
+      for (int q = 0; q < B; ++q)
+#pragma unroll
+        for (int k = 0; k < K; ++k)
+          next[q * K + k] = t + k * 1024 < whole_n4 ? p4[q * whole_n4 + k * 1024] : make_float4(0.f, 0.f, 0.f, 0.f);
+      return;
+    }
 #pragma unroll
     for (int q = 0; q < B; ++q) {
       const int g = b * B + q;
@@ -365,10 +378,11 @@ __device__ __forceinline__ void fold_pieces_batched(const float *__restrict__ pa
   load_batch(0);
   for (int b = 0; b < kFoldGroups / B; ++b) {
     double acc[B];
+    const bool all_whole = whole(b);
 #pragma unroll
     for (int q = 0; q < B; ++q) {
       const int g = b * B + q;
-      const int64_t len = length_of(g), n4 = len >> 2;
+      const int64_t len = all_whole ? piece : length_of(g), n4 = len >> 2;
       acc[q] = 0.0;
 #pragma unroll
       for (int k = 0; k < K; ++k)
@@ -377,7 +391,8 @@ __device__ __forceinline__ void fold_pieces_batched(const float *__restrict__ pa
           acc[q] += (static_cast<double>(v.x) + static_cast<double>(v.y)) + (static_cast<double>(v.z) + static_cast<double>(v.w));
         }
       // the last, short four of the whole input
-      if ((n4 << 2) + t < len) acc[q] += static_cast<double>(partials[static_cast<int64_t>(g) * piece + (n4 << 2) + t]);
+      if (!all_whole && (n4 << 2) + t < len)
+        acc[q] += static_cast<double>(partials[static_cast<int64_t>(g) * piece + (n4 << 2) + t]);
     }
     if (b + 1 < kFoldGroups / B) load_batch(b + 1);
 #pragma unroll
