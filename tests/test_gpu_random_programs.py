@@ -156,3 +156,45 @@ def test_seeded_record_programs_compute_what_the_walker_computes(hip, sarek, see
     assert np.array_equal(out.to_array(), want_out), (seed, "out")
     assert np.array_equal(vps.to_array().view(np.int32).reshape(THREADS, 2), want_ps), (seed, "ps")
     assert np.array_equal(vss.to_array().view(np.int32).reshape(THREADS, 5), want_ss), (seed, "ss")
+
+
+@pytest.mark.parametrize("seed", range(6))
+def test_every_geometry_intrinsic_under_seeded_three_dimensional_launches(hip, sarek, seed):
+    """thread_idx / block_idx / block_dim / grid_dim in x, y and z (both spellings of the indices), the global indices
+    and global_size, stored by every thread of a seeded three-dimensional launch at its linear position: what the
+    reference's walker computes for them (sarek/sarek/Sarek_ir_interp.ml:296-375: global_idx_a = block_idx_a *
+    block_dim_a + thread_idx_a)."""
+    import random
+    rng = random.Random(4242 + seed)
+    E, T, V = sarek.Execute, sarek.Transfer, sarek.Vector
+    block = (rng.choice([1, 3, 8, 16]), rng.choice([1, 2, 4]), rng.choice([1, 2, 3]))
+    grid = (rng.randint(1, 5), rng.randint(1, 4), rng.randint(1, 3))
+    names = ["thread_idx_x", "thread_idx_y", "thread_idx_z", "block_idx_x", "block_idx_y", "block_idx_z",
+             "block_dim_x", "block_dim_y", "block_dim_z", "grid_dim_x", "grid_dim_y", "grid_dim_z",
+             "global_idx_x", "global_idx_y", "global_idx_z", "global_thread_id", "global_size",
+             "thread_id_x", "block_id_y"]
+    g = lambda n: f"(intr (Gpu) {n})"
+    gx, gy, gz = g("global_idx_x"), g("global_idx_y"), g("global_idx_z")
+    wx = f"(mul {g('block_dim_x')} {g('grid_dim_x')})"
+    wy = f"(mul {g('block_dim_y')} {g('grid_dim_y')})"
+    linear = f"(add {gx} (mul {wx} (add {gy} (mul {wy} {gz}))))"
+    stores = " ".join(f"(assign (lelem out (add (mul (var at 9 i32) (i32 {len(names)})) (i32 {k}))) {g(n)})"
+                      for k, n in enumerate(names))
+    ir = (f"(kernel sarek_kern (params (param (var out 1 (vec i32)))) (locals) (body (let (var at 9 i32) {linear} "
+          f"(seq {stores}))) (native_fn true))")
+    total = block[0] * block[1] * block[2] * grid[0] * grid[1] * grid[2]
+    out = V.of_array(np.full(total * len(names), -1, np.int32))
+    assert E.run_vectors(ir, [E.Vec(out)], block, grid) == "jit"
+    T.flush()
+    got = out.to_array().reshape(total, len(names))
+    width = (block[0] * grid[0], block[1] * grid[1])
+    for bz in range(grid[2]):
+        for by in range(grid[1]):
+            for bx in range(grid[0]):
+                for tz in range(block[2]):
+                    for ty in range(block[1]):
+                        for tx in range(block[0]):
+                            ix, iy, iz = bx * block[0] + tx, by * block[1] + ty, bz * block[2] + tz
+                            want = [tx, ty, tz, bx, by, bz, *block, *grid, ix, iy, iz, ix, block[0] * grid[0], tx, by]
+                            at = ix + width[0] * (iy + width[1] * iz)
+                            assert got[at].tolist() == want, (seed, block, grid, at)
