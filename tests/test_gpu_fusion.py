@@ -140,3 +140,72 @@ def test_map_into_serial_reduction_runs_as_written(env):
     launch(hip, r, "reduce", threads, [out2, temp])
     torch.cuda.synchronize()
     assert torch.equal(out2, torch.full_like(out2, int((inp[:count] * 2).sum())))
+
+
+@pytest.mark.parametrize("seed", range(24))
+def test_seeded_integer_pipelines_fused_and_unfused(env, seed):
+    """Pipelines of two to four element-wise int32 stages with seeded expressions (the intermediate read once or
+    several times, a second input vector or a scalar here and there), fused by fuse_pipeline and by
+    auto_fuse_pipeline: the fused kernel's output is the last stage's after the launches one by one, element for
+    element (Int32 arithmetic wraps on both sides).  The fused kernel's arguments are given in the order of its own
+    parameter list."""
+    import random
+    import re
+    torch, hip, F = env
+    rng = random.Random(31000 + seed)
+    n, vec = 4096, "(vec i32)"
+    tensors = {"input": torch.randint(-2**20, 2**20, (n,), dtype=torch.int32, device="cuda")}
+    scalars = {}
+
+    def expr(depth, leaves):
+        if depth == 0:
+            return rng.choice(leaves)
+        a, b = expr(depth - 1, leaves), expr(depth - 1, leaves)
+        pick = rng.randint(0, 5)
+        if pick == 0:
+            return op(rng.choice(["add", "sub", "mul"]), a, b)
+        if pick == 1:
+            return op(rng.choice(["bitand", "bitor", "bitxor"]), a, b)
+        if pick == 2:
+            return op("shl", op("bitand", a, i32(1023)), i32(rng.randint(0, 5)))
+        if pick == 3:
+            return f"(neg {a})"
+        if pick == 4:
+            return f"(if (lt {a} {b}) {b} {a})"
+        return op("add", op("mul", a, i32(1103515245)), i32(12345))
+
+    stages, prev = [], "input"
+    for k in range(rng.randint(2, 4)):
+        out = f"v{k}"
+        tensors[out] = torch.zeros(n, dtype=torch.int32, device="cuda")
+        params, leaves = [(out, vec), (prev, vec)], [read(prev, GID), read(prev, GID), i32(rng.randint(-9, 9)), GID]
+        if rng.random() < 0.5:
+            extra = f"e{k}"
+            tensors[extra] = torch.randint(-1000, 1000, (n,), dtype=torch.int32, device="cuda")
+            params.append((extra, vec))
+            leaves.append(read(extra, GID))
+        if rng.random() < 0.5:
+            s = f"s{k}"
+            scalars[s] = rng.randint(-50, 50)
+            params.append((s, "i32"))
+            leaves.append(f"(var {s} {len(params)} i32)")
+        stages.append((f"stage{k}", params, kernel(f"stage{k}", params, store(out, GID, expr(rng.randint(1, 3), leaves)))))
+        prev = out
+
+    def arguments(ir):
+        head = ir[ir.index("(params"):ir.index("(locals")]
+        names = re.findall(r"\(param \(var ([A-Za-z0-9_]+) ", head)
+        return [tensors[m] if m in tensors else ("i32", scalars[m]) for m in names]
+
+    for name, params, ir in stages:
+        launch(hip, ir, name, n, arguments(ir))
+    torch.cuda.synchronize()
+    want = tensors[prev].clone()
+    last = stages[-1][0]
+    for fused_ir in (F.fuse_pipeline([ir for _, _, ir in stages])[0], F.auto_fuse_pipeline([ir for _, _, ir in stages])[0]):
+        tensors[prev].zero_()
+        fused_name = re.search(r"\(kernel ([A-Za-z0-9_]+)", fused_ir).group(1)
+        assert fused_name == last + "_fused" or fused_name == last
+        launch(hip, fused_ir, fused_name, n, arguments(fused_ir))
+        torch.cuda.synchronize()
+        assert torch.equal(tensors[prev], want), (seed, fused_name)
