@@ -145,7 +145,7 @@ def test_map_into_serial_reduction_runs_as_written(env):
 @pytest.mark.parametrize("seed", range(24))
 def test_seeded_integer_pipelines_fused_and_unfused(env, seed):
     """Pipelines of two to four element-wise int32 stages with seeded expressions (the intermediate read once or
-    several times, a second input vector or a scalar here and there), fused by fuse_pipeline and by
+    several times, a second input vector or a scalar here and there, some of them shared by name between stages), fused by fuse_pipeline and by
     auto_fuse_pipeline: the fused kernel's output is the last stage's after the launches one by one, element for
     element (Int32 arithmetic wraps on both sides).  The fused kernel's arguments are given in the order of its own
     parameter list."""
@@ -180,13 +180,14 @@ def test_seeded_integer_pipelines_fused_and_unfused(env, seed):
         tensors[out] = torch.zeros(n, dtype=torch.int32, device="cuda")
         params, leaves = [(out, vec), (prev, vec)], [read(prev, GID), read(prev, GID), i32(rng.randint(-9, 9)), GID]
         if rng.random() < 0.5:
-            extra = f"e{k}"
-            tensors[extra] = torch.randint(-1000, 1000, (n,), dtype=torch.int32, device="cuda")
+            extra = rng.choice([f"e{k}", "e"])                  # `e` may belong to several stages: one argument by name
+            if extra not in tensors:
+                tensors[extra] = torch.randint(-1000, 1000, (n,), dtype=torch.int32, device="cuda")
             params.append((extra, vec))
             leaves.append(read(extra, GID))
         if rng.random() < 0.5:
-            s = f"s{k}"
-            scalars[s] = rng.randint(-50, 50)
+            s = rng.choice([f"s{k}", "k"])                      # likewise (Sarek_fusion.ml:502-527 merges parameters by name)
+            scalars.setdefault(s, rng.randint(-50, 50))
             params.append((s, "i32"))
             leaves.append(f"(var {s} {len(params)} i32)")
         stages.append((f"stage{k}", params, kernel(f"stage{k}", params, store(out, GID, expr(rng.randint(1, 3), leaves)))))
