@@ -52,15 +52,20 @@ def test_four_threads_on_four_streams(hip, torch_cuda):
         torch.cuda.synchronize()
 
     assert hip.gemm16_k_splits(256, 256, 4096) > 1
+    # each thread's share runs on one stream both times: what a stream's calls may use (a block for K-split partials,
+    # a stage for long folds) is the same alone and together, however many streams the process has seen before
+    streams = [torch.cuda.Stream() for _ in range(4)]
+    assert len({st.cuda_stream for st in streams}) == 4
     alone = []
     for t in range(4):
         alone.append([])
-        work(t, alone[t])
+        with torch.cuda.stream(streams[t]):
+            work(t, alone[t])
     together, errors = [[] for _ in range(4)], []
 
     def threaded(t):
         try:
-            with torch.cuda.stream(torch.cuda.Stream()):
+            with torch.cuda.stream(streams[t]):
                 work(t, together[t])
         except Exception as e:              # noqa: BLE001 -- reported by the main thread
             errors.append((t, repr(e)))
